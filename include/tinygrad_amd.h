@@ -1,0 +1,78 @@
+/* C-ABI of libtinygrad_amd.so: hand-written gfx950 kernels for the quantized-weight linear path.
+ *
+ * Plain pointers and sizes only.  Every device pointer is memory the CALLER owns (allocated with tga_malloc or any HIP
+ * allocation of the same process); no entry point allocates or frees an output.  All work is enqueued on `stream`
+ * (a hipStream_t passed as void*, NULL = the null stream) and is asynchronous unless stated.
+ * Return value: 0 on success, non-zero on failure with the message available from tga_last_error() (per thread).
+ *
+ * Citations name the reference interface each entry point replaces (paths relative to the tinygrad tree).
+ */
+#ifndef TINYGRAD_AMD_H
+#define TINYGRAD_AMD_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids, as in tinygrad/llm/gguf.py:20-21 */
+#define TGA_F32 0
+#define TGA_F16 1
+#define TGA_Q4_0 2
+#define TGA_Q8_0 8
+#define TGA_Q6_K 14
+#define TGA_MXFP4 39
+
+/* ---- runtime: replaces HIPDevice / HIPAllocator / HIPProgram timing in tinygrad/runtime/ops_hip.py:12-70 ---- */
+const char* tga_last_error(void);
+int tga_init(int device);                                  /* hipSetDevice + kernel attribute set-up; ops_hip.py:14-20 */
+int tga_device_name(char* buf, size_t len);
+int tga_malloc(void** ptr, size_t nbytes);                 /* ops_hip.py:60-62 */
+int tga_free(void* ptr);                                   /* ops_hip.py:63 */
+int tga_memcpy_h2d(void* dst, const void* src, size_t n);  /* ops_hip.py:64-66, synchronous */
+int tga_memcpy_d2h(void* dst, const void* src, size_t n);  /* ops_hip.py:67-69, synchronous */
+int tga_memcpy_d2d(void* dst, const void* src, size_t n, void* stream);
+int tga_memset(void* dst, int value, size_t n, void* stream);
+int tga_sync(void);                                        /* ops_hip.py:22-24 hipDeviceSynchronize */
+int tga_stream_create(void** stream);
+int tga_stream_destroy(void* stream);
+int tga_stream_sync(void* stream);
+int tga_event_create(void** ev);                           /* ops_hip.py:49-57 wait=True timing */
+int tga_event_destroy(void* ev);
+int tga_event_record(void* ev, void* stream);
+int tga_event_sync(void* ev);
+int tga_event_elapsed_ms(void* start, void* stop, float* ms);
+/* Replay support (the reference replays a captured kernel list per token: tinygrad/engine/jit.py:163-198). */
+int tga_graph_begin(void* stream);
+int tga_graph_end(void* stream, void** graph_exec);
+int tga_graph_launch(void* graph_exec, void* stream);
+int tga_graph_destroy(void* graph_exec);
+
+/* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 8, 14, 39) ----
+ * blocks: device pointer to the raw GGUF tensor bytes; n: number of elements (multiple of the block size).
+ * out_dtype TGA_F32: bit-exact ggml_data_to_tensor result.  TGA_F16: that result cast to fp16 round-to-nearest-even,
+ * i.e. the weight the model path holds after tinygrad/llm/model.py:376. */
+int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out_dtype, void* stream);
+
+/* ---- fused dequant + linear: nn.Linear.__call__ over a lazily dequantized GGUF weight,
+ * tinygrad/nn/__init__.py:177 -> Tensor.dot tinygrad/mixin/op.py:367-392 (float32 accumulation, dtype.py:212-216).
+ *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
+ * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
+ * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  K must be a multiple of the type's block size.
+ * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K (GGUF aligns tensor data to 32 bytes, gguf.py:144-148). */
+int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
+                int M, int64_t N, int64_t K, void* stream);
+
+/* Several weights sharing one activation in ONE launch (attn_q/k/v at tinygrad/llm/model.py:168; ffn_gate/ffn_up at :137).
+ * nseg <= 3; segment i is an (n[i], K) weight of type ggml_type written to y[i] as (M, n[i]).
+ * epilogue: 0 = plain store; 1 = y[i] = resid[i] + x W^T in float32 (the residual adds at model.py:149-150; requires
+ * y_dtype TGA_F32; resid[i] may alias y[i]); 2 = SwiGLU: nseg must be 2 with n[0] == n[1], and the single output
+ * y[0] = silu(x Wgate^T) * (x Wup^T) (model.py:137), resid ignored. */
+int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                      const void* x, int x_dtype, int y_dtype, int M, int64_t K,
+                      int epilogue, const void* const* resid, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

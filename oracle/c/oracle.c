@@ -1,0 +1,144 @@
+/* Scalar C restatement of the reference's quantized-weight linear path.  TEST INFRASTRUCTURE ONLY: the checker and the
+ * timed CPU baseline; never linked into the shipped library.
+ *
+ * Dequant loops restate the published ggml reference routines (ggml-quants.c dequantize_row_q4_0 / q8_0 / q6_K /
+ * mxfp4; gguf-py >= 0.18 is what the reference's tests call, pyproject.toml:79) element by element, independently of
+ * the vectorised numpy restatement of tinygrad/llm/gguf.py:46,56,68-72,105-114 in oracle/ggml.py: the two must agree
+ * bit for bit (tests/test_oracle_ggml.py).
+ * The linear restates Tensor.dot (tinygrad/mixin/op.py:367-392) with sum_acc_dtype = float32 (tinygrad/dtype.py:212-216).
+ */
+#include <stdint.h>
+#include <string.h>
+#include <math.h>
+#include <stdlib.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static inline float h2f(uint16_t h) {
+  uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1f, m = h & 0x3ffu, u;
+  if (e == 0) {
+    if (m == 0) u = s;
+    else { int sh = 0; while (!(m & 0x400u)) { m <<= 1; sh++; } m &= 0x3ffu; u = s | ((uint32_t)(113 - sh) << 23) | (m << 13); }
+  } else if (e == 31) u = s | 0x7f800000u | (m << 13);
+  else u = s | ((e + 112) << 23) | (m << 13);
+  float f; memcpy(&f, &u, 4); return f;
+}
+/* round-to-nearest-even float32 -> float16 bits (the cast at tinygrad/llm/model.py:376) */
+static inline uint16_t f2h(float f) {
+  uint32_t x; memcpy(&x, &f, 4);
+  uint32_t s = (x >> 16) & 0x8000u, a = x & 0x7fffffffu;
+  if (a >= 0x7f800000u) return (uint16_t)(s | 0x7c00u | ((a > 0x7f800000u) ? 0x200u : 0));
+  if (a >= 0x477ff000u) return (uint16_t)(s | 0x7c00u);           /* >= 65520 rounds to inf */
+  if (a < 0x33000001u) return (uint16_t)s;                         /* <= 2^-25 rounds to zero */
+  int e = (int)(a >> 23) - 127;
+  uint32_t m = (a & 0x7fffffu) | 0x800000u;
+  int shift = (e < -14) ? (13 + (-14 - e)) : 13;
+  uint32_t r = m >> shift, rem = m & ((1u << shift) - 1), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (r & 1))) r++;
+  if (e < -14) return (uint16_t)(s | r);                           /* subnormal (r may carry into exponent 1: fine) */
+  return (uint16_t)(s | (((uint32_t)(e + 15) << 10) + (r - 0x400u)));
+}
+float orc_h2f(uint16_t h) { return h2f(h); }
+uint16_t orc_f2h(float f) { return f2h(f); }
+
+/* ---- block dequant: y gets nb * nel floats ---- */
+static void deq_q4_0(const uint8_t* b, float* y) {            /* block_q4_0: ggml_common.py:21 */
+  uint16_t dh; memcpy(&dh, b, 2); const float d = h2f(dh);
+  for (int j = 0; j < 16; j++) {
+    y[j]      = (float)((int)(b[2 + j] & 0x0F) - 8) * d;
+    y[j + 16] = (float)((int)(b[2 + j] >> 4) - 8) * d;
+  }
+}
+static void deq_q8_0(const uint8_t* b, float* y) {            /* block_q8_0: ggml_common.py:59-64 */
+  uint16_t dh; memcpy(&dh, b, 2); const float d = h2f(dh);
+  for (int j = 0; j < 32; j++) y[j] = (float)(int8_t)b[2 + j] * d;
+}
+static void deq_q6_k(const uint8_t* b, float* y) {            /* block_q6_K: ggml_common.py:123-129 */
+  uint16_t dh; memcpy(&dh, b + 208, 2); const float d = h2f(dh);
+  const uint8_t *ql = b, *qh = b + 128; const int8_t* sc = (const int8_t*)(b + 192);
+  for (int n = 0; n < 256; n += 128) {
+    for (int l = 0; l < 32; l++) {
+      int is = l / 16;
+      int q1 = (int)((ql[l]      & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+      int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+      int q3 = (int)((ql[l]      >> 4)  | (((qh[l] >> 4) & 3) << 4)) - 32;
+      int q4 = (int)((ql[l + 32] >> 4)  | (((qh[l] >> 6) & 3) << 4)) - 32;
+      y[l]      = d * sc[is + 0] * q1;
+      y[l + 32] = d * sc[is + 2] * q2;
+      y[l + 64] = d * sc[is + 4] * q3;
+      y[l + 96] = d * sc[is + 6] * q4;
+    }
+    y += 128; ql += 64; qh += 32; sc += 8;
+  }
+}
+/* ggml's kvalues_mxfp4 is an int8 table (code 8 -> +0); the reference's float LUT (tinygrad/llm/gguf.py:108-110) holds -0.0
+ * for code 8, and bit-exactness is owed to the reference, so the table here is the reference's. */
+static const float kvalues_mxfp4[16] = {0.0f, 1.0f, 2.0f, 3.0f, 4.0f, 6.0f, 8.0f, 12.0f, -0.0f, -1.0f, -2.0f, -3.0f, -4.0f, -6.0f, -8.0f, -12.0f};
+static void deq_mxfp4(const uint8_t* b, float* y) {           /* block_mxfp4: ggml_common.py:35 */
+  /* ggml: d = GGML_E8M0_TO_FP32_HALF(e) = 2^(e-128), built from bits so e = 0, 1 give fp32 subnormals */
+  uint32_t e = b[0], bits = (e < 2) ? (0x00200000u << e) : ((e - 1) << 23);
+  float d; memcpy(&d, &bits, 4);
+  for (int j = 0; j < 16; j++) {
+    y[j]      = kvalues_mxfp4[b[1 + j] & 0x0F] * d;
+    y[j + 16] = kvalues_mxfp4[b[1 + j] >> 4] * d;
+  }
+}
+
+static int type_geom(int t, int* nel, int* nby) {
+  switch (t) { case 2: *nel = 32; *nby = 18; return 0; case 8: *nel = 32; *nby = 34; return 0;
+               case 14: *nel = 256; *nby = 210; return 0; case 39: *nel = 32; *nby = 17; return 0; }
+  return -1;
+}
+static void deq_block(int t, const uint8_t* b, float* y) {
+  switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break; }
+}
+
+/* ggml_data_to_tensor (tinygrad/llm/gguf.py:23): n_blocks blocks -> float32 */
+int orc_dequant(int ggml_type, const uint8_t* blocks, int64_t n_blocks, float* out, int threads) {
+  int nel, nby; if (type_geom(ggml_type, &nel, &nby)) return -1;
+  (void)threads;
+  #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t i = 0; i < n_blocks; i++) deq_block(ggml_type, blocks + i * nby, out + i * nel);
+  return 0;
+}
+
+/* y[m,n] = sum_k x[m,k] * W[n,k], float32 accumulate in k order.
+ * w_round_f16 = 1 applies the model path's fp16 cast of the dequantized weight (tinygrad/llm/model.py:376).
+ * x_f16 = 1: x holds fp16 bits (config-1 style standalone matmul); products are then formed in float32 from the exact
+ *            fp16 values (prod_round_f16 = 1 additionally rounds each product to fp16 as an fp16*fp16 Tensor multiply does,
+ *            tinygrad/mixin/op.py:392). */
+int orc_linear(int ggml_type, const uint8_t* w, const void* x, float* y, int M, int64_t N, int64_t K,
+               int x_f16, int w_round_f16, int prod_round_f16, int threads) {
+  int nel, nby; if (type_geom(ggml_type, &nel, &nby)) return -1;
+  if (K % nel) return -2;
+  const int64_t bpr = K / nel;
+  float* xf = (float*)malloc(sizeof(float) * (size_t)M * K);
+  for (int64_t i = 0; i < (int64_t)M * K; i++) xf[i] = x_f16 ? h2f(((const uint16_t*)x)[i]) : ((const float*)x)[i];
+  #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)
+  for (int64_t n = 0; n < N; n++) {
+    float acc[8] = {0}; float wb[256];
+    const uint8_t* row = w + n * bpr * nby;
+    for (int64_t b = 0; b < bpr; b++) {
+      deq_block(ggml_type, row + b * nby, wb);
+      if (w_round_f16) for (int j = 0; j < nel; j++) wb[j] = h2f(f2h(wb[j]));
+      for (int m = 0; m < M; m++) {
+        const float* xr = xf + (int64_t)m * K + b * nel; float a = acc[m];
+        if (prod_round_f16) for (int j = 0; j < nel; j++) a += h2f(f2h(xr[j] * wb[j]));
+        else for (int j = 0; j < nel; j++) a += xr[j] * wb[j];
+        acc[m] = a;
+      }
+    }
+    for (int m = 0; m < M; m++) y[(int64_t)m * N + n] = acc[m];
+  }
+  free(xf);
+  return 0;
+}
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

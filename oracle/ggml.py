@@ -1,0 +1,117 @@
+"""numpy restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for the four block layouts on the path,
+plus the ggml reference quantizers used only to build synthetic models.  Test infrastructure only."""
+import numpy as np
+
+Q4_0, Q8_0, Q6_K, MXFP4, F32, F16 = 2, 8, 14, 39, 0, 1
+# {ggml_type: (elements per block, bytes per block)}  tinygrad/llm/gguf.py:20-21
+GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q6_K: (256, 210), MXFP4: (32, 17)}
+# tinygrad/llm/gguf.py:108-110 (== 2 * E2M1 values; ggml_common.py:218 kvalues_mxfp4)
+FP4_LUT = np.array([0.0, 1.0, 2.0, 3.0, 4.0, 6.0, 8.0, 12.0, -0.0, -1.0, -2.0, -3.0, -4.0, -6.0, -8.0, -12.0], dtype=np.float32)
+
+def q_to_uint8(t: np.ndarray, b: int) -> np.ndarray:
+  """gguf.py:38-41: unpack 8//b b-bit fields per byte, FIELD-MAJOR over the last axis
+  (all field-0 values of the row first, then all field-1 values, ...)."""
+  shifts = np.arange(8 // b, dtype=np.uint8) * b
+  fields = (t[..., None] >> shifts) & (0xff >> (8 - b))          # (..., nbytes, 8//b)
+  return np.swapaxes(fields, -1, -2).reshape(*t.shape[:-1], -1)   # (..., 8//b * nbytes)
+
+def _blocks(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
+  nel, nby = GGML_QUANT[ggml_type]
+  data = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+  return data[:(n // nel) * nby].reshape(-1, nby)                  # gguf.py:45
+
+def _f16(b: np.ndarray) -> np.ndarray: return np.ascontiguousarray(b).view(np.float16).astype(np.float32)
+
+def dequant_q4_0(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:46  (q_to_uint8(qs,4).bitcast(int8) - 8) * float32(fp16 d)"""
+  return (q_to_uint8(blocks[:, 2:], 4).view(np.int8) - np.int8(8)).astype(np.float32) * _f16(blocks[:, :2])
+
+def dequant_q8_0(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:56  float32(fp16 d) * int8 qs"""
+  return _f16(blocks[:, :2]) * np.ascontiguousarray(blocks[:, 2:]).view(np.int8).astype(np.float32)
+
+def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:68-72  d * (int8(xl | xh) - 32) * scales, in that association order"""
+  nb = blocks.shape[0]
+  xl = q_to_uint8(blocks[:, :128].reshape(nb, 2, 64), 4)
+  xh = q_to_uint8(blocks[:, 128:192].reshape(nb, 2, 32), 2) << 4
+  scales = np.repeat(np.ascontiguousarray(blocks[:, 192:208]).view(np.int8), 16, axis=1).astype(np.float32)
+  d = _f16(blocks[:, 208:210])
+  q = ((xl | xh).view(np.int8) - np.int8(32)).reshape(nb, 256).astype(np.float32)
+  return (d * q) * scales
+
+def dequant_mxfp4(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:105-114  d = bitcast_f32((e-1)<<23) (e>=2), 2^-127 (e==1), 2^-128 (e==0); value = LUT[code] * d"""
+  e = blocks[:, 0].astype(np.uint32)
+  small = np.array([0x00200000, 0x00400000], dtype=np.uint32)[np.clip(e, 0, 1)]
+  d = np.where(e < 2, small, (e - 1) * np.uint32(0x00800000)).astype(np.uint32).view(np.float32)[:, None]
+  return FP4_LUT[q_to_uint8(blocks[:, 1:17], 4)] * d
+
+_DEQ = {Q4_0: dequant_q4_0, Q8_0: dequant_q8_0, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
+
+def ggml_data_to_tensor(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
+  """gguf.py:23-119 restricted to the types on the path; returns flat float32 of n elements."""
+  if ggml_type == F32: return np.ascontiguousarray(data).view(np.uint8)[:4 * n].view(np.float32).copy()
+  if ggml_type == F16: return np.ascontiguousarray(data).view(np.uint8)[:2 * n].view(np.float16).copy()
+  if ggml_type not in _DEQ: raise ValueError(f"GGML type '{ggml_type}' is not supported!")   # gguf.py:119
+  return _DEQ[ggml_type](_blocks(data, n, ggml_type)).reshape(-1)[:n]
+
+def row_bytes(ggml_type: int, k: int) -> int:
+  nel, nby = GGML_QUANT[ggml_type]
+  assert k % nel == 0
+  return k // nel * nby
+
+# ---------------------------------------------------------------------------------------------------------------
+# Quantizers.  The reference has none (weights arrive quantized inside GGUF files); these restate ggml's published
+# reference quantizers (ggml-quants.c quantize_row_q4_0_ref / q8_0_ref / q6_K_ref is NOT restated: Q6_K synthetic
+# weights use the simpler rule documented below) and exist only to build synthetic models.
+# ---------------------------------------------------------------------------------------------------------------
+def quantize_q4_0(w: np.ndarray) -> np.ndarray:
+  """ggml rule: per 32 block, max = signed value of largest magnitude, d = max / -8, id = 1/d (0 if d == 0),
+  q = min(15, int8(x*id + 8.5)); byte j = q[j] | q[j+16] << 4; d stored as fp16."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 32)
+  idx = np.argmax(np.abs(x), axis=1)
+  mx = x[np.arange(x.shape[0]), idx]
+  d = mx / np.float32(-8.0)
+  with np.errstate(divide="ignore"): idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+  q = np.minimum(15, (x * idv[:, None] + np.float32(8.5)).astype(np.int8)).astype(np.uint8)
+  out = np.empty((x.shape[0], 18), dtype=np.uint8)
+  out[:, :2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:] = q[:, :16] | (q[:, 16:] << 4)
+  return out.reshape(-1)
+
+def quantize_q8_0(w: np.ndarray) -> np.ndarray:
+  """ggml rule: d = amax / 127, q = round(x / d) (round half away from zero, as roundf)."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 32)
+  d = np.abs(x).max(axis=1) / np.float32(127.0)
+  with np.errstate(divide="ignore"): idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+  v = x * idv[:, None]
+  q = (np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))).astype(np.int8)
+  out = np.empty((x.shape[0], 34), dtype=np.uint8)
+  out[:, :2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:] = q.view(np.uint8)
+  return out.reshape(-1)
+
+def quantize_q6_k(w: np.ndarray) -> np.ndarray:
+  """Simple absmax rule (NOT ggml's iterative make_qx_quants search): per 16-group scale s_g = amax_g / 31,
+  d = max_g |s_g| / 127, sc_g = round(s_g / d) in int8, q = clamp(round(x / (d*sc_g)), -32, 31) + 32.
+  The byte packing is exactly the layout dequant_q6_k / gguf.py:68-72 decodes."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 16, 16)
+  nb = x.shape[0]
+  s = np.abs(x).max(axis=2) / np.float32(31.0)
+  d = (s.max(axis=1) / np.float32(127.0)).astype(np.float16).astype(np.float32)
+  with np.errstate(divide="ignore", invalid="ignore"):
+    sc = np.where(d[:, None] > 0, np.rint(s / d[:, None]), 0).clip(-128, 127).astype(np.int8)
+    eff = d[:, None] * sc.astype(np.float32)
+    q = np.where(eff[:, :, None] != 0, np.rint(x / eff[:, :, None]), 0).clip(-32, 31).astype(np.int8)
+  u = (q.reshape(nb, 256).astype(np.int16) + 32).astype(np.uint8)               # 0..63
+  lo, hi = (u & 0xF).reshape(nb, 2, 4, 32), (u >> 4).reshape(nb, 2, 4, 32)       # [half][32-group j][l]
+  out = np.empty((nb, 210), dtype=np.uint8)
+  ql = np.empty((nb, 2, 64), dtype=np.uint8)
+  ql[:, :, :32] = lo[:, :, 0] | (lo[:, :, 2] << 4)
+  ql[:, :, 32:] = lo[:, :, 1] | (lo[:, :, 3] << 4)
+  out[:, :128] = ql.reshape(nb, 128)
+  out[:, 128:192] = (hi[:, :, 0] | (hi[:, :, 1] << 2) | (hi[:, :, 2] << 4) | (hi[:, :, 3] << 6)).reshape(nb, 64)
+  out[:, 192:208] = sc.view(np.uint8)
+  out[:, 208:210] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  return out.reshape(-1)

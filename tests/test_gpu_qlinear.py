@@ -1,0 +1,120 @@
+"""Fused dequant-GEMV / small-batch GEMM on the GPU vs the oracle.
+
+Bar: rel-err = max|y - ref| / max|ref| <= 1e-3 against the float64 textbook product of the exact dequantized weights, and the
+same bound against the restatement of the reference's own numerics (model path: fp16-rounded weights; standalone: fp16 products).
+fp16 outputs must equal the RNE cast of the float32 output of the same kernel."""
+import numpy as np, pytest
+from oracle import ggml as og, linear as ol, cref
+from tinygrad_amd import synth
+from tinygrad_amd.runtime import GGML_QUANT
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+def _run(gpu, t, w, x, n, k, ydt=np.float32):
+  from tinygrad_amd.nn import QuantLinear
+  lin = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  return lin(gpu.Buffer.from_numpy(x), out_dtype=ydt).numpy()
+
+def _check(y, x, W):
+  ref64 = ol.linear_f64(x.astype(np.float32), W)
+  e = ol.rel_err(y, ref64)
+  assert e <= TOL, f"rel-err {e:.3e} vs float64 anchor"
+  # elementwise: allclose in the sense of the reference's VALIDATE_WITH_CPU harness (engine/realize.py:192-201), atol scaled to the output rms
+  np.testing.assert_allclose(y, ref64, rtol=TOL, atol=TOL * float(np.sqrt(np.mean(ref64 ** 2))))
+  return e
+
+@pytest.mark.parametrize("t", [2, 8, 14, 39])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_small_shapes_all_batches(gpu, t, m):
+  rng = np.random.default_rng(1000 * t + m)
+  n, k = 257, 1024                       # odd row count: the last row group is ragged
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  W = ol.weight_f32(w, n, k, t)
+  y = _run(gpu, t, w, x, n, k)
+  _check(y, x, W)
+  # against the C restatement of the reference's model path (fp16-rounded weights, float32 accumulate)
+  ym = cref.linear(t, w, x, n, k, w_round_f16=True)
+  assert ol.rel_err(y, ym) <= TOL
+
+@pytest.mark.parametrize("t,k", [(2, 32), (2, 96), (2, 4096 + 32), (8, 32), (8, 160), (39, 32), (39, 2048 + 64), (14, 256), (14, 768), (14, 4096 + 256)])
+def test_ragged_k(gpu, t, k):
+  """K that is not a multiple of 64 units per row: partially filled waves."""
+  rng = np.random.default_rng(k + t)
+  n = 130
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, 2, k, np.float16)
+  _check(_run(gpu, t, w, x, n, k), x, ol.weight_f32(w, n, k, t))
+
+@pytest.mark.parametrize("t", [2, 8, 14, 39])
+def test_f32_activations_and_f16_output(gpu, t):
+  rng = np.random.default_rng(31 + t)
+  n, k = 512, 2048
+  w = synth.random_blocks(rng, t, n, k)
+  x32 = synth.activations(rng, 1, k, np.float32)
+  W = ol.weight_f32(w, n, k, t)
+  y32 = _run(gpu, t, w, x32, n, k, np.float32)
+  _check(y32, x32, W)                       # fp32 x is rounded to fp16 inside the kernel: still inside the 1e-3 bar
+  assert ol.rel_err(y32, ol.linear_model(x32, W)) <= TOL
+  y16 = _run(gpu, t, w, x32, n, k, np.float16)
+  assert y16.tobytes() == y32.astype(np.float16).tobytes()
+
+def test_config1_q4_0_4096(gpu):
+  """BASELINE config 1 at full size: W 4096x4096 Q4_0, x fp16 [1,4096], fp32 accumulate, fp16 out (seed 1001)."""
+  w, x, (n, k) = synth.config1()
+  W = ol.weight_f32(w, n, k, 2)
+  y32 = _run(gpu, 2, w, x, n, k, np.float32)
+  e = _check(y32, x, W)
+  y16 = _run(gpu, 2, w, x, n, k, np.float16)
+  assert y16.tobytes() == y32.astype(np.float16).tobytes()
+  # the reference's own standalone numerics (fp16 products, fp32 accumulate, fp16 out): within 1e-3 + one fp16 ulp of the output
+  ref16 = ol.linear_standalone_f16(x, W).astype(np.float32)
+  tol = TOL * np.abs(ref16).max() + np.spacing(np.abs(ref16).astype(np.float16)).astype(np.float32)
+  assert (np.abs(y16.astype(np.float32) - ref16) <= tol).all()
+  print(f"config1 rel-err vs f64 anchor {e:.2e}")
+
+@pytest.mark.parametrize("t,n,k,m", [(8, 4096, 14336, 8), (8, 512, 14336, 5), (2, 300, 14336, 8), (14, 200, 8192, 8)])
+def test_chunked_k_large_batch(gpu, t, n, k, m):
+  """M*K activations beyond the LDS budget: the kernel walks K in chunks."""
+  rng = np.random.default_rng(n + k + m)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  y = _run(gpu, t, w, x, n, k)
+  ref = cref.linear(t, w, x, n, k, threads=8)
+  assert ol.rel_err(y, ref) <= TOL
+
+def test_multi_segment_and_epilogues(gpu):
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(77)
+  k = 1024
+  ns = [512, 128, 130]
+  ws = [synth.random_blocks(rng, 2, n, k) for n in ns]
+  x = synth.activations(rng, 1, k, np.float16)
+  layers = [QuantLinear(gpu.Buffer.from_numpy(w), 2, n, k) for w, n in zip(ws, ns)]
+  xb = gpu.Buffer.from_numpy(x)
+  outs = [gpu.Buffer((1, n), np.float32) for n in ns]
+  qlinear_multi(layers, xb, outs)
+  refs = [ol.linear_f64(x.astype(np.float32), ol.weight_f32(w, n, k, 2)) for w, n in zip(ws, ns)]
+  for o, r in zip(outs, refs): assert ol.rel_err(o.numpy(), r) <= TOL
+  # residual epilogue, in place
+  res = [rng.standard_normal((1, n)).astype(np.float32) for n in ns]
+  rb = [gpu.Buffer.from_numpy(r) for r in res]
+  qlinear_multi(layers, xb, rb, epilogue=1, resid=rb)
+  for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL
+  # SwiGLU epilogue: silu(gate) * up (tinygrad/llm/model.py:137)
+  g = [QuantLinear(gpu.Buffer.from_numpy(ws[1]), 2, 128, k), QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, 2, 128, k)), 2, 128, k)]
+  out = gpu.Buffer((1, 128), np.float32)
+  qlinear_multi(g, xb, [out], epilogue=2)
+  a = ol.linear_f64(x.astype(np.float32), ol.weight_f32(g[0].blocks.numpy(), 128, k, 2))
+  b = ol.linear_f64(x.astype(np.float32), ol.weight_f32(g[1].blocks.numpy(), 128, k, 2))
+  ref = a / (1 + np.exp(-a)) * b
+  assert ol.rel_err(out.numpy(), ref) <= TOL
+
+def test_argument_errors(gpu):
+  from tinygrad_amd.nn import QuantLinear
+  w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))
+  with pytest.raises(ValueError): QuantLinear(w, 1337, 4, 32)
+  lin = QuantLinear(w, 2, 4, 32)
+  with pytest.raises(AssertionError): lin(gpu.Buffer((9, 32), np.float16))
+  with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))

@@ -1,0 +1,75 @@
+// C-ABI runtime shim: device, memory, streams, events, graph replay.  Mirrors what the reference's HIP device does through
+// libamdhip64 (tinygrad/runtime/ops_hip.py:12-70): every HIP status != 0 becomes an error string the Python wrapper raises
+// as RuntimeError("HIP Error n, <string>") (ops_hip.py:9-10).
+#include "host.h"
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+int tga_set_error(const char* fmt, ...) {
+  va_list ap; va_start(ap, fmt); vsnprintf(g_err, sizeof(g_err), fmt, ap); va_end(ap);
+  return 1;
+}
+
+extern "C" {
+
+const char* tga_last_error(void) { return g_err; }
+
+int tga_init(int device) {
+  int n = 0;
+  TGA_HIP(hipGetDeviceCount(&n));
+  TGA_REQUIRE(device >= 0 && device < n, "tga_init: device %d out of range (have %d)", device, n);
+  TGA_HIP(hipSetDevice(device));
+  hipDeviceProp_t p;
+  TGA_HIP(hipGetDeviceProperties(&p, device));
+  TGA_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, "tga_init: kernels are built for gfx950 only, device is %s", p.gcnArchName);
+  return 0;
+}
+
+int tga_device_name(char* buf, size_t len) {
+  int dev = 0; hipDeviceProp_t p;
+  TGA_HIP(hipGetDevice(&dev));
+  TGA_HIP(hipGetDeviceProperties(&p, dev));
+  snprintf(buf, len, "%s (%s, %d CUs, %.0f MHz)", p.name, p.gcnArchName, p.multiProcessorCount, p.clockRate / 1000.0);
+  return 0;
+}
+
+int tga_malloc(void** ptr, size_t nbytes) { TGA_REQUIRE(ptr, "tga_malloc: null out pointer"); TGA_HIP(hipMalloc(ptr, nbytes ? nbytes : 1)); return 0; }
+int tga_free(void* ptr) { TGA_HIP(hipFree(ptr)); return 0; }
+int tga_memcpy_h2d(void* dst, const void* src, size_t n) { TGA_HIP(hipMemcpy(dst, src, n, hipMemcpyHostToDevice)); return 0; }
+int tga_memcpy_d2h(void* dst, const void* src, size_t n) { TGA_HIP(hipMemcpy(dst, src, n, hipMemcpyDeviceToHost)); return 0; }
+int tga_memcpy_d2d(void* dst, const void* src, size_t n, void* stream) {
+  TGA_HIP(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, (hipStream_t)stream)); return 0;
+}
+int tga_memset(void* dst, int value, size_t n, void* stream) { TGA_HIP(hipMemsetAsync(dst, value, n, (hipStream_t)stream)); return 0; }
+int tga_sync(void) { TGA_HIP(hipDeviceSynchronize()); return 0; }
+
+int tga_stream_create(void** stream) { TGA_HIP(hipStreamCreate((hipStream_t*)stream)); return 0; }   // default priority only
+int tga_stream_destroy(void* stream) { TGA_HIP(hipStreamDestroy((hipStream_t)stream)); return 0; }
+int tga_stream_sync(void* stream) { TGA_HIP(hipStreamSynchronize((hipStream_t)stream)); return 0; }
+
+int tga_event_create(void** ev) { TGA_HIP(hipEventCreate((hipEvent_t*)ev)); return 0; }
+int tga_event_destroy(void* ev) { TGA_HIP(hipEventDestroy((hipEvent_t)ev)); return 0; }
+int tga_event_record(void* ev, void* stream) { TGA_HIP(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream)); return 0; }
+int tga_event_sync(void* ev) { TGA_HIP(hipEventSynchronize((hipEvent_t)ev)); return 0; }
+int tga_event_elapsed_ms(void* start, void* stop, float* ms) { TGA_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop)); return 0; }
+
+int tga_graph_begin(void* stream) {
+  TGA_REQUIRE(stream, "tga_graph_begin: capture needs a non-null stream");
+  TGA_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return 0;
+}
+int tga_graph_end(void* stream, void** graph_exec) {
+  hipGraph_t g = nullptr;
+  TGA_HIP(hipStreamEndCapture((hipStream_t)stream, &g));
+  hipGraphExec_t ge = nullptr;
+  hipError_t e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  TGA_HIP(e);
+  *graph_exec = ge;
+  return 0;
+}
+int tga_graph_launch(void* graph_exec, void* stream) { TGA_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream)); return 0; }
+int tga_graph_destroy(void* graph_exec) { TGA_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec)); return 0; }
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+"""ctypes binding of libtinygrad_amd.so: the only way Python reaches the GPU in this package (no torch, no Triton).
+
+Mirrors the reference's HIP device glue (tinygrad/runtime/ops_hip.py:9-70): a non-zero status becomes RuntimeError with the
+library's message, buffers are explicit device allocations owned by the Python side."""
+from __future__ import annotations
+import ctypes, pathlib
+import numpy as np
+
+F32, F16, Q4_0, Q8_0, Q6_K, MXFP4 = 0, 1, 2, 8, 14, 39
+# {ggml_type: (elements per block, bytes per block)}: tinygrad/llm/gguf.py:20-21
+GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q6_K: (256, 210), MXFP4: (32, 17)}
+_NP_DTYPE = {F32: np.float32, F16: np.float16}
+
+_LIB_PATH = pathlib.Path(__file__).resolve().parent / "libtinygrad_amd.so"
+_lib = None
+_initialised = False
+
+c_void_pp = ctypes.POINTER(ctypes.c_void_p)
+
+def _declare(lib):
+  vp, i, i64, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
+  sig = {
+    "tga_init": [i], "tga_device_name": [ctypes.c_char_p, sz], "tga_malloc": [c_void_pp, sz], "tga_free": [vp],
+    "tga_memcpy_h2d": [vp, vp, sz], "tga_memcpy_d2h": [vp, vp, sz], "tga_memcpy_d2d": [vp, vp, sz, vp], "tga_memset": [vp, i, sz, vp],
+    "tga_sync": [], "tga_stream_create": [c_void_pp], "tga_stream_destroy": [vp], "tga_stream_sync": [vp],
+    "tga_event_create": [c_void_pp], "tga_event_destroy": [vp], "tga_event_record": [vp, vp], "tga_event_sync": [vp],
+    "tga_event_elapsed_ms": [vp, vp, ctypes.POINTER(ctypes.c_float)],
+    "tga_graph_begin": [vp], "tga_graph_end": [vp, c_void_pp], "tga_graph_launch": [vp, vp], "tga_graph_destroy": [vp],
+    "tga_dequant": [i, vp, i64, vp, i, vp],
+    "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
+    "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, vp],
+  }
+  for name, args in sig.items():
+    fn = getattr(lib, name)
+    fn.argtypes, fn.restype = args, ctypes.c_int
+  lib.tga_last_error.restype, lib.tga_last_error.argtypes = ctypes.c_char_p, []
+  return lib
+
+def load_library() -> ctypes.CDLL:
+  """Loads the built library.  Fails loudly when it is missing: there is no CPU fallback."""
+  global _lib
+  if _lib is None:
+    if not _LIB_PATH.exists():
+      raise RuntimeError(f"{_LIB_PATH} is missing: build it with `python -m tinygrad_amd.build` (needs hipcc); there is no fallback path")
+    _lib = _declare(ctypes.CDLL(str(_LIB_PATH)))
+  return _lib
+
+def check(status: int) -> None:
+  if status != 0: raise RuntimeError(load_library().tga_last_error().decode())
+
+def init(device: int = 0) -> None:
+  global _initialised
+  check(load_library().tga_init(device))
+  _initialised = True
+
+def lib() -> ctypes.CDLL:
+  if not _initialised: init(0)
+  return _lib
+
+def device_name() -> str:
+  buf = ctypes.create_string_buffer(256)
+  check(lib().tga_device_name(buf, 256))
+  return buf.value.decode()
+
+def synchronize() -> None: check(lib().tga_sync())
+
+class Buffer:
+  """A device allocation plus the (shape, dtype) the host side attaches to it.  dtype is a numpy dtype."""
+  def __init__(self, shape, dtype=np.uint8, ptr: int | None = None, owner=None):
+    self.shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+    self.dtype = np.dtype(dtype)
+    self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+    self._owner = owner
+    if ptr is None:
+      p = ctypes.c_void_p()
+      check(lib().tga_malloc(ctypes.byref(p), self.nbytes))
+      self.ptr, self._owned = p.value, True
+    else: self.ptr, self._owned = ptr, False
+
+  def __del__(self):
+    if getattr(self, "_owned", False) and self.ptr and _lib is not None:
+      _lib.tga_free(ctypes.c_void_p(self.ptr)); self.ptr = None
+
+  @staticmethod
+  def from_numpy(a: np.ndarray) -> "Buffer":
+    a = np.ascontiguousarray(a)
+    b = Buffer(a.shape, a.dtype)
+    if a.nbytes: check(lib().tga_memcpy_h2d(b.ptr, a.ctypes.data, a.nbytes))
+    return b
+
+  def copyin(self, a: np.ndarray) -> "Buffer":
+    a = np.ascontiguousarray(a)
+    assert a.nbytes == self.nbytes, (a.nbytes, self.nbytes)
+    if a.nbytes: check(lib().tga_memcpy_h2d(self.ptr, a.ctypes.data, a.nbytes))
+    return self
+
+  def numpy(self) -> np.ndarray:
+    out = np.empty(self.shape, dtype=self.dtype)
+    if self.nbytes: check(lib().tga_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
+    return out
+
+  def view(self, byte_offset: int, shape, dtype) -> "Buffer":
+    """A non-owning window into this allocation (e.g. one tensor's byte range inside a GGUF file buffer)."""
+    v = Buffer(shape, dtype, ptr=self.ptr + byte_offset, owner=self)
+    assert byte_offset + v.nbytes <= self.nbytes
+    return v
+
+  def zero_(self, stream=None) -> "Buffer":
+    if self.nbytes: check(lib().tga_memset(self.ptr, 0, self.nbytes, stream))
+    return self
+
+class Stream:
+  def __init__(self):
+    p = ctypes.c_void_p(); check(lib().tga_stream_create(ctypes.byref(p))); self.handle = p.value
+  def synchronize(self): check(lib().tga_stream_sync(self.handle))
+  def __del__(self):
+    if getattr(self, "handle", None) and _lib is not None: _lib.tga_stream_destroy(ctypes.c_void_p(self.handle)); self.handle = None
+
+class Event:
+  def __init__(self):
+    p = ctypes.c_void_p(); check(lib().tga_event_create(ctypes.byref(p))); self.handle = p.value
+  def record(self, stream=None): check(lib().tga_event_record(self.handle, stream))
+  def synchronize(self): check(lib().tga_event_sync(self.handle))
+  def elapsed_ms(self, end: "Event") -> float:
+    ms = ctypes.c_float(); check(lib().tga_event_elapsed_ms(self.handle, end.handle, ctypes.byref(ms))); return ms.value
+  def __del__(self):
+    if getattr(self, "handle", None) and _lib is not None: _lib.tga_event_destroy(ctypes.c_void_p(self.handle)); self.handle = None
+
+class Graph:
+  """Captured launch sequence replayed per decode step (the reference's TinyJit replay, tinygrad/engine/jit.py:163-198)."""
+  def __init__(self, stream: Stream): self.stream, self.handle = stream, None
+  def __enter__(self): check(lib().tga_graph_begin(self.stream.handle)); return self
+  def __exit__(self, et, ev, tb):
+    p = ctypes.c_void_p(); st = lib().tga_graph_end(self.stream.handle, ctypes.byref(p))
+    if et is None: check(st); self.handle = p.value
+    return False
+  def launch(self): check(lib().tga_graph_launch(self.handle, self.stream.handle))
+  def __del__(self):
+    if getattr(self, "handle", None) and _lib is not None: _lib.tga_graph_destroy(ctypes.c_void_p(self.handle)); self.handle = None
+
+def dtype_code(dt) -> int:
+  dt = np.dtype(dt)
+  if dt == np.float32: return F32
+  if dt == np.float16: return F16
+  raise TypeError(f"unsupported activation dtype {dt}")
