@@ -4,9 +4,14 @@
 // when W is the lazy ggml_data_to_tensor expression over raw GGUF bytes (tinygrad/llm/gguf.py:46,56,68-72,105-114).
 //
 // Design (bandwidth-bound, no MFMA):
-//  * a "unit" is the slice of one weight row a lane owns per step: one 32-weight block (Q4_0 18 B, Q8_0 34 B, MXFP4 17 B) or a
-//    quarter of a Q6_K superblock (64 weights).  Lane l of a wave takes unit l, l+64, ... of a row, so a wave's loads cover a
-//    contiguous span of the row; each lane issues 128-bit loads straight from the packed GGUF bytes (no repacking).
+//  * a "unit" is the slice of one weight row a lane owns per step: a PAIR of 32-weight blocks for Q4_0 (36 B) and Q8_0 (68 B),
+//    one MXFP4 block (17 B), or a quarter of a Q6_K superblock (64 weights).  Lane l of a wave takes unit l, l+64, ... of a row,
+//    so a wave's loads cover a contiguous span of the row; each lane issues 128-bit loads straight from the packed GGUF
+//    bytes (no repacking).  Measured on MI355X, dwordx4 loads that are only 2-byte aligned run ~25 % slower than 4-byte
+//    aligned ones, so every hot load is 4-byte aligned: block pairs start on 4-byte boundaries, and the 17/210-byte layouts load
+//    the enclosing aligned dwords and realign in registers (v_alignbit_b32 / 64-bit shift).  An aligned dword that holds at
+//    least one byte of the tensor never leaves that byte's page, so the realigned loads cannot fault past the buffer.
+//    Shapes whose rows are not pair-aligned (odd K/32, or a 2-byte aligned base) take a single-block fallback format.
 //  * nibbles / bytes are turned into fp16 with biased-exponent tricks in registers (v_and_or_b32, v_perm_b32,
 //    v_cvt_scalef32_pk_f16_fp4) and multiplied with v_dot2_f32_f16 (two fp16 products, float32 accumulate).  The integer offset
 //    (-8, -32, +128 bias, plus the 1024/64 exponent bias) is removed with a per-unit correction  c = -bias * sum(x)  that is
@@ -41,6 +46,10 @@ __device__ __forceinline__ uint32_t pack_odd(uint32_t a, uint32_t b) { return (a
 
 template <int T> struct Fmt;
 
+// A constant the compiler must keep in a VGPR: VOP3 forms such as v_and_or_b32 / v_perm_b32 accept a single scalar
+// operand and no literal on this ISA, so (x & MASK) | BIAS only becomes one instruction when BIAS already lives in a VGPR.
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t c) { asm("" : "+v"(c)); return c; }
+
 // ------------------------------------------------------------------------------------------------ Q4_0 (gguf.py:46)
 template <> struct Fmt<GGML_Q4_0> {
   static constexpr int UW = 32, UPB = 1, BW = 32, BB = 18;   // weights per unit, units per block, block weights / bytes
@@ -52,14 +61,16 @@ template <> struct Fmt<GGML_Q4_0> {
   // element index (within the row) of natural pair k (elements 2k, 2k+1) of unit u
   static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
   // wv[4t+c] multiplies x pair xs[t][c].  low nibble -> 1024+n (0x6400), high nibble in place -> 64+n (0x5400)
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv) {
+  static constexpr int NKC = 2;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       const uint32_t w = r.q[t], w8 = w >> 8;
-      wv[4 * t + 0] = and_or(w, 0x000F000Fu, 0x64006400u);    // weights 4t, 4t+2
-      wv[4 * t + 1] = and_or(w, 0x00F000F0u, 0x54005400u);    // weights 4t+16, 4t+18
-      wv[4 * t + 2] = and_or(w8, 0x000F000Fu, 0x64006400u);   // weights 4t+1, 4t+3
-      wv[4 * t + 3] = and_or(w8, 0x00F000F0u, 0x54005400u);   // weights 4t+17, 4t+19
+      wv[4 * t + 0] = and_or(w, 0x000F000Fu, kc[0]);    // weights 4t, 4t+2
+      wv[4 * t + 1] = and_or(w, 0x00F000F0u, kc[1]);    // weights 4t+16, 4t+18
+      wv[4 * t + 2] = and_or(w8, 0x000F000Fu, kc[0]);   // weights 4t+1, 4t+3
+      wv[4 * t + 3] = and_or(w8, 0x00F000F0u, kc[1]);   // weights 4t+17, 4t+19
     }
   }
   static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
@@ -86,12 +97,14 @@ template <> struct Fmt<GGML_Q8_0> {
   }
   static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
   // int8 q -> byte q^0x80 = q+128 placed under exponent byte 0x64: fp16 value 1024 + 128 + q
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv) {
+  static constexpr int NKC = 1;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64646464u); }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       const uint32_t u = (t < 4 ? r.q0[t] : r.q1[t - 4]) ^ 0x80808080u;
-      wv[2 * t + 0] = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);   // bytes (u0,0x64,u1,0x64): weights 4t, 4t+1
-      wv[2 * t + 1] = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);   // weights 4t+2, 4t+3
+      wv[2 * t + 0] = __builtin_amdgcn_perm(kc[0], u, 0x04010400u);   // bytes (u0,0x64,u1,0x64): weights 4t, 4t+1
+      wv[2 * t + 1] = __builtin_amdgcn_perm(kc[0], u, 0x04030402u);   // weights 4t+2, 4t+3
     }
   }
   static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
@@ -105,17 +118,136 @@ template <> struct Fmt<GGML_Q8_0> {
   static __device__ __forceinline__ float finish(const Raw& r, const float* a) { return h2f_bits(r.d) * a[0]; }
 };
 
+
+enum { F_Q4_0P = 1002, F_Q8_0P = 1008 };   // block-pair formats (4-byte aligned 36 / 68 byte units)
+
+__device__ __forceinline__ u32x4 ld16_a4(const uint8_t* p) {   // 4-byte aligned 16-byte load
+  u32x4 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16); return v;
+}
+__device__ __forceinline__ uint32_t ld4_a4(const uint8_t* p) { return *(const uint32_t*)p; }
+// 16 bytes at a 2-byte aligned address: the five enclosing aligned dwords, funnel-shifted by 0 or 16 bits per lane
+__device__ __forceinline__ u32x4 ld16_a2(const uint8_t* p, uint32_t& tail_dword, uint32_t& sh) {
+  const uintptr_t a = (uintptr_t)p; sh = (uint32_t)(a & 2) * 8;
+  const uint8_t* q = (const uint8_t*)(a & ~(uintptr_t)3);
+  const u32x4 v = ld16_a4(q); const uint32_t e = ld4_a4(q + 16);
+  tail_dword = e;
+  u32x4 r = {__builtin_amdgcn_alignbit(v.y, v.x, sh), __builtin_amdgcn_alignbit(v.z, v.y, sh),
+             __builtin_amdgcn_alignbit(v.w, v.z, sh), __builtin_amdgcn_alignbit(e, v.w, sh)};
+  return r;
+}
+
+// ------------------------------------------------------------------------------------------------ Q4_0 block pair
+// unit u = blocks 2u, 2u+1 of the row = 9 dwords D0..D8 at a 4-byte aligned address:
+//   D0 = d0 | q0[0..1] << 16,  D1..D3 = q0[2..13],  D4 = q0[14..15] | d1 << 16,  D5..D8 = q1[0..15].
+// Quant dwords: Q0 = (D0 >> 16) | (D4 << 16) = bytes q0[0], q0[1], q0[14], q0[15];  Q1..Q3 = D1..D3;  Q4..Q7 = D5..D8.
+// The byte order inside Q0..Q3 differs from the block order; the activations are staged in the matching order instead.
+template <> struct Fmt<F_Q4_0P> {
+  static constexpr int UW = 64, UPB = 1, BW = 64, BB = 36;
+  static constexpr int XV = 8, NG = 2, NWV = 32;
+  struct Raw { u32x4 a, b; uint32_t c; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* p = row + 36 * u; Raw r; r.a = ld16_a4(p); r.b = ld16_a4(p + 16); r.c = ld4_a4(p + 32); return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 2;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+    const uint32_t q[8] = {__builtin_amdgcn_alignbit(r.b.x, r.a.x, 16), r.a.y, r.a.z, r.a.w, r.b.y, r.b.z, r.b.w, r.c};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t w = q[i], w8 = w >> 8;
+      wv[4 * i + 0] = and_or(w, 0x000F000Fu, kc[0]);    // low nibbles of bytes 0, 2
+      wv[4 * i + 1] = and_or(w, 0x00F000F0u, kc[1]);    // high nibbles of bytes 0, 2 (weights +16)
+      wv[4 * i + 2] = and_or(w8, 0x000F000Fu, kc[0]);   // low nibbles of bytes 1, 3
+      wv[4 * i + 3] = and_or(w8, 0x00F000F0u, kc[1]);   // high nibbles of bytes 1, 3
+    }
+  }
+  // nx[k] = (x[2k], x[2k+1]) of the unit's 64 activations.  Quant dword i holds bytes (b0, b0+1, b2, b2+1) of its block with
+  // (b0, b2)/2 = (0,7), (1,2), (3,4), (5,6) for block 0 and (2t, 2t+1) for block 1.
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+    constexpr int P0[8] = {0, 1, 3, 5, 16, 18, 20, 22}, P2[8] = {7, 2, 4, 6, 17, 19, 21, 23};
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      xv[i].x = pack_even(nx[P0[i]], nx[P2[i]]);     xv[i].y = pack_even(nx[P0[i] + 8], nx[P2[i] + 8]);
+      xv[i].z = pack_odd(nx[P0[i]], nx[P2[i]]);      xv[i].w = pack_odd(nx[P0[i] + 8], nx[P2[i] + 8]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float lo = 0.f, hi = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; k++) { lo = dot2(nx[16 * j + k], 0x64086408u, lo); hi = dot2(nx[16 * j + k + 8], 0x54805480u, hi); }   // 1032, 72
+      c[j] = -(lo + hi);
+    }
+  }
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+    return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
+  }
+};
+
+// ------------------------------------------------------------------------------------------------ Q8_0 block pair
+// unit u = 17 dwords D0..D16:  D0 = d0 | q0[0..1] << 16,  D1..D7 = q0[2..29],  D8 = q0[30..31] | d1 << 16,  D9..D16 = q1[0..31].
+// Quant dwords: Q0 = (D0 >> 16) | (D8 << 16) = q0[0], q0[1], q0[30], q0[31];  Q1..Q7 = D1..D7;  Q8..Q15 = D9..D16.
+template <> struct Fmt<F_Q8_0P> {
+  static constexpr int UW = 64, UPB = 1, BW = 64, BB = 68;
+  static constexpr int XV = 8, NG = 2, NWV = 32;
+  struct Raw { u32x4 a, b, c, d; uint32_t e; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* p = row + 68 * u; Raw r; r.a = ld16_a4(p); r.b = ld16_a4(p + 16); r.c = ld16_a4(p + 32); r.d = ld16_a4(p + 48); r.e = ld4_a4(p + 64); return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 1;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64646464u); }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+    const uint32_t q[16] = {__builtin_amdgcn_alignbit(r.c.x, r.a.x, 16), r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w,
+                            r.c.y, r.c.z, r.c.w, r.d.x, r.d.y, r.d.z, r.d.w, r.e};
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const uint32_t u = q[i] ^ 0x80808080u;
+      wv[2 * i + 0] = __builtin_amdgcn_perm(kc[0], u, 0x04010400u);   // bytes 0, 1 -> fp16 1152 + q
+      wv[2 * i + 1] = __builtin_amdgcn_perm(kc[0], u, 0x04030402u);   // bytes 2, 3
+    }
+  }
+  // pairs in decode order: block 0: N0, N15, N1, N2, ..., N14;  block 1: natural
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+    constexpr int ORD[16] = {0, 15, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14};
+#pragma unroll
+    for (int v = 0; v < 4; v++) { xv[v].x = nx[ORD[4 * v]]; xv[v].y = nx[ORD[4 * v + 1]]; xv[v].z = nx[ORD[4 * v + 2]]; xv[v].w = nx[ORD[4 * v + 3]]; }
+#pragma unroll
+    for (int v = 4; v < 8; v++) { xv[v].x = nx[4 * v]; xv[v].y = nx[4 * v + 1]; xv[v].z = nx[4 * v + 2]; xv[v].w = nx[4 * v + 3]; }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; k++) t = dot2(nx[16 * j + k], 0x64806480u, t);   // 1152
+      c[j] = -t;
+    }
+  }
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+    return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
+  }
+};
+
 // ------------------------------------------------------------------------------------------------ MXFP4 (gguf.py:105-114)
 template <> struct Fmt<GGML_MXFP4> {
   static constexpr int UW = 32, UPB = 1, BW = 32, BB = 17;
   static constexpr int XV = 4, NG = 1, NWV = 16;
   struct Raw { u32x4 q; uint32_t e; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    const uint8_t* p = row + 17 * u; Raw r; r.e = p[0]; r.q = ld16(p + 1); return r;
+    // the 17-byte block starts at any byte offset o of an aligned dword: load the five enclosing dwords and shift
+    const uintptr_t a = (uintptr_t)(row + 17 * u); const uint32_t o = (uint32_t)(a & 3);
+    const uint8_t* q = (const uint8_t*)(a & ~(uintptr_t)3);
+    const u32x4 v = ld16_a4(q); const uint32_t t = ld4_a4(q + 16);
+    const uint32_t sh = 8 * (o + 1);   // 8..32
+    Raw r; r.e = (v.x >> (8 * o)) & 0xFFu;
+    r.q.x = (uint32_t)((((uint64_t)v.y << 32) | v.x) >> sh); r.q.y = (uint32_t)((((uint64_t)v.z << 32) | v.y) >> sh);
+    r.q.z = (uint32_t)((((uint64_t)v.w << 32) | v.z) >> sh); r.q.w = (uint32_t)((((uint64_t)t << 32) | v.w) >> sh);
+    return r;
   }
   static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
   // hardware E2M1 -> fp16 (true values 0..6); byte s of dword t holds weights 4t+s (low nibble) and 4t+s+16 (high nibble)
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv) {
+  static constexpr int NKC = 1;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = 0; }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t*) {
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       wv[4 * t + 0] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], 1.0f, 0));
@@ -147,27 +279,34 @@ template <> struct Fmt<GGML_Q6_K> {
   static constexpr int XV = 8, NG = 4, NWV = 32;
   struct Raw { u32x4 a, b, h; uint32_t sc0, sc1, d; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    // superblocks are 2-byte aligned: every piece is loaded as its enclosing aligned dwords and funnel-shifted per lane
     const uint8_t* p = row + 210 * (u >> 2); const int h = (u >> 1) & 1, g = u & 1;
-    Raw r; r.a = ld16(p + 64 * h + 16 * g); r.b = ld16(p + 64 * h + 32 + 16 * g); r.h = ld16(p + 128 + 32 * h + 16 * g);
-    r.sc0 = ld4(p + 192 + 8 * h); r.sc1 = ld4(p + 196 + 8 * h); r.d = (uint32_t)g | (ld2(p + 208) << 16);
+    uint32_t tail, sh;
+    Raw r; r.a = ld16_a2(p + 64 * h + 16 * g, tail, sh); r.b = ld16_a2(p + 64 * h + 32 + 16 * g, tail, sh); r.h = ld16_a2(p + 128 + 32 * h + 16 * g, tail, sh);
+    const u32x4 sc = ld16_a2(p + 192, tail, sh);                         // sc[0..15]; tail dword holds d (bytes 208, 209)
+    r.sc0 = h ? sc.z : sc.x; r.sc1 = h ? sc.w : sc.y;
+    r.d = (uint32_t)g | (__builtin_amdgcn_alignbit(0u, tail, sh) << 16);
     return r;
   }
   static __device__ __forceinline__ int xoff(int u, int k) {   // k = 0..31: natural pair k of the unit's 64 x values (j = k/8)
     return 256 * (u >> 2) + 128 * ((u >> 1) & 1) + 32 * (k >> 3) + 16 * (u & 1) + 2 * (k & 7);
   }
   // wv[8j + 2t + {0,1}] = even / odd pairs of dword t of group j; value 1024 + 6-bit q
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv) {
+  static constexpr int NKC = 1;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+    const uint32_t K64 = kc[0];
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       const uint32_t A = r.a[t], B = r.b[t], H = r.h[t];
-      wv[0 + 2 * t]      = and_or(H << 4, 0x00300030u, and_or(A, 0x000F000Fu, 0x64006400u));
-      wv[0 + 2 * t + 1]  = and_or(H >> 4, 0x00300030u, and_or(A >> 8, 0x000F000Fu, 0x64006400u));
-      wv[8 + 2 * t]      = and_or(H << 2, 0x00300030u, and_or(B, 0x000F000Fu, 0x64006400u));
-      wv[8 + 2 * t + 1]  = and_or(H >> 6, 0x00300030u, and_or(B >> 8, 0x000F000Fu, 0x64006400u));
-      wv[16 + 2 * t]     = and_or(H, 0x00300030u, and_or(A >> 4, 0x000F000Fu, 0x64006400u));
-      wv[16 + 2 * t + 1] = and_or(H >> 8, 0x00300030u, and_or(A >> 12, 0x000F000Fu, 0x64006400u));
-      wv[24 + 2 * t]     = and_or(H >> 2, 0x00300030u, and_or(B >> 4, 0x000F000Fu, 0x64006400u));
-      wv[24 + 2 * t + 1] = and_or(H >> 10, 0x00300030u, and_or(B >> 12, 0x000F000Fu, 0x64006400u));
+      wv[0 + 2 * t]      = and_or(H << 4, 0x00300030u, and_or(A, 0x000F000Fu, K64));
+      wv[0 + 2 * t + 1]  = and_or(H >> 4, 0x00300030u, and_or(A >> 8, 0x000F000Fu, K64));
+      wv[8 + 2 * t]      = and_or(H << 2, 0x00300030u, and_or(B, 0x000F000Fu, K64));
+      wv[8 + 2 * t + 1]  = and_or(H >> 6, 0x00300030u, and_or(B >> 8, 0x000F000Fu, K64));
+      wv[16 + 2 * t]     = and_or(H, 0x00300030u, and_or(A >> 4, 0x000F000Fu, K64));
+      wv[16 + 2 * t + 1] = and_or(H >> 8, 0x00300030u, and_or(A >> 12, 0x000F000Fu, K64));
+      wv[24 + 2 * t]     = and_or(H >> 2, 0x00300030u, and_or(B >> 4, 0x000F000Fu, K64));
+      wv[24 + 2 * t + 1] = and_or(H >> 10, 0x00300030u, and_or(B >> 12, 0x000F000Fu, K64));
     }
   }
   // xv[2j + t/2] = {E(t), O(t), E(t+1), O(t+1)} (t even), E/O = even/odd element pairs of dword t of group j
@@ -219,10 +358,10 @@ __device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs
 }
 
 template <int T, int M>
-__device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const u32x4* xs, const float* cs, int cu, int ul, float* acc) {
+__device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const u32x4* xs, const float* cs, int cu, int ul, float* acc, const uint32_t* kc) {
   using F = Fmt<T>;
   uint32_t wv[F::NWV];
-  F::decode(raw, wv);
+  F::decode(raw, wv, kc);
   constexpr int VPG = F::XV / F::NG;   // x vectors per accumulator group
 #pragma unroll
   for (int m = 0; m < M; m++) {
@@ -292,33 +431,66 @@ __device__ __forceinline__ void store_rows(const QArgs& a, long long rg, float (
 template <int T, int M, int R>
 __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
   using F = Fmt<T>;
+  typedef typename F::Raw Raw;
   extern __shared__ u32x4 lds[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: row pointers stay in SGPRs
   const long long gw = (long long)blockIdx.x * QG_WAVES + wave, nw = (long long)gridDim.x * QG_WAVES;
   const long long ngroups = (a.epilogue == 2) ? a.ntot : (a.ntot + R - 1) / R;
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  float acc[R][M];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int m = 0; m < M; m++) acc[r][m] = 0.f;
 
   if (a.nchunks == 1) {
-    const int cu = a.nu;
+    // Software pipeline over "steps" (row group, 64-unit slice of K): the loads of step s+1 are in flight while step s is
+    // multiplied, and the first step's loads are issued before the activations are staged.
+    const int cu = a.nu, iters = (cu + 63) >> 6;
+    const long long mine = gw < ngroups ? (ngroups - gw + nw - 1) / nw : 0, nsteps = mine * iters;
     u32x4* xs = lds; float* cs = (float*)(lds + M * F::XV * cu);
+    long long l_rg = gw, c_rg = gw; int l_it = 0, c_it = 0;
+    const uint8_t* l_rp[R];
+    auto l_setup = [&]() {
+#pragma unroll
+      for (int r = 0; r < R; r++) { int seg; long long lr; bool valid; map_row<R>(a, l_rg, r, seg, lr, valid); l_rp[r] = a.w[seg] + lr * a.row_bytes; }
+    };
+    auto issue = [&](Raw* buf) {
+      const int u = l_it * 64 + lane;
+      if (u < cu) {
+#pragma unroll
+        for (int r = 0; r < R; r++) buf[r] = F::load(l_rp[r], u);
+      }
+      if (++l_it == iters) { l_it = 0; l_rg += nw; if (l_rg < ngroups) l_setup(); }
+    };
+    auto compute = [&](const Raw* buf) {
+      const int u = c_it * 64 + lane;
+      if (u < cu) {
+#pragma unroll
+        for (int r = 0; r < R; r++) unit_dot<T, M>(buf[r], xs, cs, cu, u, acc[r], kc);
+      }
+      if (++c_it == iters) {
+        store_rows<T, M, R>(a, c_rg, acc);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+          for (int m = 0; m < M; m++) acc[r][m] = 0.f;
+        c_it = 0; c_rg += nw;
+      }
+    };
+    Raw b0[R], b1[R];
+    if (mine) { l_setup(); issue(b0); }
     stage_chunk<T, M>(a, xs, cs, 0, cu);
     __syncthreads();
-    for (long long rg = gw; rg < ngroups; rg += nw) {
-      const uint8_t* rp[R];
-#pragma unroll
-      for (int r = 0; r < R; r++) { int seg; long long lr; bool valid; map_row<R>(a, rg, r, seg, lr, valid); rp[r] = a.w[seg] + lr * a.row_bytes; }
-      float acc[R][M];
-#pragma unroll
-      for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int m = 0; m < M; m++) acc[r][m] = 0.f;
-      for (int u = lane; u < cu; u += 64) {
-        typename F::Raw raw[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) raw[r] = F::load(rp[r], u);
-#pragma unroll
-        for (int r = 0; r < R; r++) unit_dot<T, M>(raw[r], xs, cs, cu, u, acc[r]);
+    for (long long s = 0; s < nsteps; s += 2) {
+      if (s + 1 < nsteps) issue(b1);
+      compute(b0);
+      if (s + 1 < nsteps) {
+        if (s + 2 < nsteps) issue(b0);
+        compute(b1);
       }
-      store_rows<T, M, R>(a, rg, acc);
     }
   } else {
     // K walked in LDS-sized chunks; one row group per wave (the host sizes the grid so that gw covers every group)
@@ -327,11 +499,6 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
     const uint8_t* rp[R];
 #pragma unroll
     for (int r = 0; r < R; r++) { int seg; long long lr; bool valid; map_row<R>(a, active ? rg : 0, r, seg, lr, valid); rp[r] = a.w[seg] + lr * a.row_bytes; }
-    float acc[R][M];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-      for (int m = 0; m < M; m++) acc[r][m] = 0.f;
     for (int ch = 0; ch < a.nchunks; ch++) {
       const int u0 = ch * a.chunk_u, cu = min(a.chunk_u, a.nu - u0);
       u32x4* xs = lds; float* cs = (float*)(lds + M * F::XV * cu);
@@ -340,11 +507,11 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
       __syncthreads();
       if (active) {
         for (int ul = lane; ul < cu; ul += 64) {
-          typename F::Raw raw[R];
+          Raw raw[R];
 #pragma unroll
           for (int r = 0; r < R; r++) raw[r] = F::load(rp[r], u0 + ul);
 #pragma unroll
-          for (int r = 0; r < R; r++) unit_dot<T, M>(raw[r], xs, cs, cu, ul, acc[r]);
+          for (int r = 0; r < R; r++) unit_dot<T, M>(raw[r], xs, cs, cu, ul, acc[r], kc);
         }
       }
     }
@@ -401,7 +568,7 @@ static int launch_qgemv_r(const QArgs& a, hipStream_t s) {
   // SwiGLU pairs gate/up rows: exactly two rows per group.  Otherwise two rows per wave step as well (more loads in flight
   // per lane); a single row per group when there are too few rows to fill the chip.
   if (a.epilogue == 2) return launch_qgemv<T, M, 2>(a, s);
-  if (a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
+  if (M > 1 || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
   return launch_qgemv<T, M, 2>(a, s);
 }
 
@@ -447,9 +614,12 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
   }
   a.ntot = (epilogue == 2) ? n[0] : ntot;
   hipStream_t s = (hipStream_t)stream;
+  // block-pair units need an even number of blocks per row and 4-byte aligned rows
+  bool pair = (K / 32) % 2 == 0;
+  for (int i = 0; i < nseg; i++) pair = pair && ((uintptr_t)w[i] & 3) == 0;
   switch (ggml_type) {
-    case GGML_Q4_0: return launch_qgemv_m<GGML_Q4_0>(a, M, s);
-    case GGML_Q8_0: return launch_qgemv_m<GGML_Q8_0>(a, M, s);
+    case GGML_Q4_0: return pair ? launch_qgemv_m<F_Q4_0P>(a, M, s) : launch_qgemv_m<GGML_Q4_0>(a, M, s);
+    case GGML_Q8_0: return pair ? launch_qgemv_m<F_Q8_0P>(a, M, s) : launch_qgemv_m<GGML_Q8_0>(a, M, s);
     case GGML_Q6_K: return launch_qgemv_m<GGML_Q6_K>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
   }
