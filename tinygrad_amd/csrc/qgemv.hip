@@ -21,314 +21,7 @@
 //  * a wave owns whole rows: K is reduced inside the lane, then across the wave with DPP adds (no LDS, no atomics).
 //  * when M*K activations do not fit LDS the kernel walks K in chunks with one row group per wave (accumulators stay in
 //    registers across chunks).
-#include "common.h"
-#include "host.h"
-
-#define QG_THREADS 256
-#define QG_WAVES 4
-#define QG_MAX_SEG 3
-
-struct QArgs {
-  const uint8_t* w[QG_MAX_SEG];
-  void* y[QG_MAX_SEG];
-  const float* resid[QG_MAX_SEG];
-  long long n[QG_MAX_SEG];
-  const void* x;
-  long long ntot;       // rows over all segments (epilogue 2: rows of one segment)
-  long long row_bytes;  // bytes per weight row
-  int nseg, x_f32, y_f32, epilogue;
-  int K, nu;            // units per row
-  int chunk_u, nchunks; // units per LDS chunk
-};
-
-__device__ __forceinline__ uint32_t pack_even(uint32_t a, uint32_t b) { return (a & 0xFFFFu) | (b << 16); }        // (a.lo, b.lo)
-__device__ __forceinline__ uint32_t pack_odd(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xFFFF0000u); }     // (a.hi, b.hi)
-
-template <int T> struct Fmt;
-
-// A constant the compiler must keep in a VGPR: VOP3 forms such as v_and_or_b32 / v_perm_b32 accept a single scalar
-// operand and no literal on this ISA, so (x & MASK) | BIAS only becomes one instruction when BIAS already lives in a VGPR.
-__device__ __forceinline__ uint32_t vgpr_const(uint32_t c) { asm("" : "+v"(c)); return c; }
-
-// ------------------------------------------------------------------------------------------------ Q4_0 (gguf.py:46)
-template <> struct Fmt<GGML_Q4_0> {
-  static constexpr int UW = 32, UPB = 1, BW = 32, BB = 18;   // weights per unit, units per block, block weights / bytes
-  static constexpr int XV = 4, NG = 1, NWV = 16;
-  struct Raw { u32x4 q; uint32_t d; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    const uint8_t* p = row + 18 * u; Raw r; r.d = ld2(p); r.q = ld16(p + 2); return r;
-  }
-  // element index (within the row) of natural pair k (elements 2k, 2k+1) of unit u
-  static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
-  // wv[4t+c] multiplies x pair xs[t][c].  low nibble -> 1024+n (0x6400), high nibble in place -> 64+n (0x5400)
-  static constexpr int NKC = 2;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      const uint32_t w = r.q[t], w8 = w >> 8;
-      wv[4 * t + 0] = and_or(w, 0x000F000Fu, kc[0]);    // weights 4t, 4t+2
-      wv[4 * t + 1] = and_or(w, 0x00F000F0u, kc[1]);    // weights 4t+16, 4t+18
-      wv[4 * t + 2] = and_or(w8, 0x000F000Fu, kc[0]);   // weights 4t+1, 4t+3
-      wv[4 * t + 3] = and_or(w8, 0x00F000F0u, kc[1]);   // weights 4t+17, 4t+19
-    }
-  }
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      xv[t].x = pack_even(nx[2 * t], nx[2 * t + 1]);       xv[t].y = pack_even(nx[2 * t + 8], nx[2 * t + 9]);
-      xv[t].z = pack_odd(nx[2 * t], nx[2 * t + 1]);        xv[t].w = pack_odd(nx[2 * t + 8], nx[2 * t + 9]);
-    }
-    float lo = 0.f, hi = 0.f;
-#pragma unroll
-    for (int k = 0; k < 8; k++) { lo = dot2(nx[k], 0x64086408u, lo); hi = dot2(nx[k + 8], 0x54805480u, hi); }   // 1032, 72
-    c[0] = -(lo + hi);
-  }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) { return h2f_bits(r.d) * a[0]; }
-};
-
-// ------------------------------------------------------------------------------------------------ Q8_0 (gguf.py:56)
-template <> struct Fmt<GGML_Q8_0> {
-  static constexpr int UW = 32, UPB = 1, BW = 32, BB = 34;
-  static constexpr int XV = 4, NG = 1, NWV = 16;
-  struct Raw { u32x4 q0, q1; uint32_t d; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    const uint8_t* p = row + 34 * u; Raw r; r.d = ld2(p); r.q0 = ld16(p + 2); r.q1 = ld16(p + 18); return r;
-  }
-  static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
-  // int8 q -> byte q^0x80 = q+128 placed under exponent byte 0x64: fp16 value 1024 + 128 + q
-  static constexpr int NKC = 1;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64646464u); }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
-#pragma unroll
-    for (int t = 0; t < 8; t++) {
-      const uint32_t u = (t < 4 ? r.q0[t] : r.q1[t - 4]) ^ 0x80808080u;
-      wv[2 * t + 0] = __builtin_amdgcn_perm(kc[0], u, 0x04010400u);   // bytes (u0,0x64,u1,0x64): weights 4t, 4t+1
-      wv[2 * t + 1] = __builtin_amdgcn_perm(kc[0], u, 0x04030402u);   // weights 4t+2, 4t+3
-    }
-  }
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-    float s = 0.f;
-#pragma unroll
-    for (int t = 0; t < 4; t++) { xv[t].x = nx[4 * t]; xv[t].y = nx[4 * t + 1]; xv[t].z = nx[4 * t + 2]; xv[t].w = nx[4 * t + 3]; }
-#pragma unroll
-    for (int k = 0; k < 16; k++) s = dot2(nx[k], 0x64806480u, s);   // 1152
-    c[0] = -s;
-  }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) { return h2f_bits(r.d) * a[0]; }
-};
-
-
-enum { F_Q4_0P = 1002, F_Q8_0P = 1008 };   // block-pair formats (4-byte aligned 36 / 68 byte units)
-
-__device__ __forceinline__ u32x4 ld16_a4(const uint8_t* p) {   // 4-byte aligned 16-byte load
-  u32x4 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16); return v;
-}
-__device__ __forceinline__ uint32_t ld4_a4(const uint8_t* p) { return *(const uint32_t*)p; }
-// 16 bytes at a 2-byte aligned address: the five enclosing aligned dwords, funnel-shifted by 0 or 16 bits per lane
-__device__ __forceinline__ u32x4 ld16_a2(const uint8_t* p, uint32_t& tail_dword, uint32_t& sh) {
-  const uintptr_t a = (uintptr_t)p; sh = (uint32_t)(a & 2) * 8;
-  const uint8_t* q = (const uint8_t*)(a & ~(uintptr_t)3);
-  const u32x4 v = ld16_a4(q); const uint32_t e = ld4_a4(q + 16);
-  tail_dword = e;
-  u32x4 r = {__builtin_amdgcn_alignbit(v.y, v.x, sh), __builtin_amdgcn_alignbit(v.z, v.y, sh),
-             __builtin_amdgcn_alignbit(v.w, v.z, sh), __builtin_amdgcn_alignbit(e, v.w, sh)};
-  return r;
-}
-
-// ------------------------------------------------------------------------------------------------ Q4_0 block pair
-// unit u = blocks 2u, 2u+1 of the row = 9 dwords D0..D8 at a 4-byte aligned address:
-//   D0 = d0 | q0[0..1] << 16,  D1..D3 = q0[2..13],  D4 = q0[14..15] | d1 << 16,  D5..D8 = q1[0..15].
-// Quant dwords: Q0 = (D0 >> 16) | (D4 << 16) = bytes q0[0], q0[1], q0[14], q0[15];  Q1..Q3 = D1..D3;  Q4..Q7 = D5..D8.
-// The byte order inside Q0..Q3 differs from the block order; the activations are staged in the matching order instead.
-template <> struct Fmt<F_Q4_0P> {
-  static constexpr int UW = 64, UPB = 1, BW = 64, BB = 36;
-  static constexpr int XV = 8, NG = 2, NWV = 32;
-  struct Raw { u32x4 a, b; uint32_t c; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    const uint8_t* p = row + 36 * u; Raw r; r.a = ld16_a4(p); r.b = ld16_a4(p + 16); r.c = ld4_a4(p + 32); return r;
-  }
-  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
-  static constexpr int NKC = 2;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
-    const uint32_t q[8] = {__builtin_amdgcn_alignbit(r.b.x, r.a.x, 16), r.a.y, r.a.z, r.a.w, r.b.y, r.b.z, r.b.w, r.c};
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const uint32_t w = q[i], w8 = w >> 8;
-      wv[4 * i + 0] = and_or(w, 0x000F000Fu, kc[0]);    // low nibbles of bytes 0, 2
-      wv[4 * i + 1] = and_or(w, 0x00F000F0u, kc[1]);    // high nibbles of bytes 0, 2 (weights +16)
-      wv[4 * i + 2] = and_or(w8, 0x000F000Fu, kc[0]);   // low nibbles of bytes 1, 3
-      wv[4 * i + 3] = and_or(w8, 0x00F000F0u, kc[1]);   // high nibbles of bytes 1, 3
-    }
-  }
-  // nx[k] = (x[2k], x[2k+1]) of the unit's 64 activations.  Quant dword i holds bytes (b0, b0+1, b2, b2+1) of its block with
-  // (b0, b2)/2 = (0,7), (1,2), (3,4), (5,6) for block 0 and (2t, 2t+1) for block 1.
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-    constexpr int P0[8] = {0, 1, 3, 5, 16, 18, 20, 22}, P2[8] = {7, 2, 4, 6, 17, 19, 21, 23};
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      xv[i].x = pack_even(nx[P0[i]], nx[P2[i]]);     xv[i].y = pack_even(nx[P0[i] + 8], nx[P2[i] + 8]);
-      xv[i].z = pack_odd(nx[P0[i]], nx[P2[i]]);      xv[i].w = pack_odd(nx[P0[i] + 8], nx[P2[i] + 8]);
-    }
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-      float lo = 0.f, hi = 0.f;
-#pragma unroll
-      for (int k = 0; k < 8; k++) { lo = dot2(nx[16 * j + k], 0x64086408u, lo); hi = dot2(nx[16 * j + k + 8], 0x54805480u, hi); }   // 1032, 72
-      c[j] = -(lo + hi);
-    }
-  }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
-    return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
-  }
-};
-
-// ------------------------------------------------------------------------------------------------ Q8_0 block pair
-// unit u = 17 dwords D0..D16:  D0 = d0 | q0[0..1] << 16,  D1..D7 = q0[2..29],  D8 = q0[30..31] | d1 << 16,  D9..D16 = q1[0..31].
-// Quant dwords: Q0 = (D0 >> 16) | (D8 << 16) = q0[0], q0[1], q0[30], q0[31];  Q1..Q7 = D1..D7;  Q8..Q15 = D9..D16.
-template <> struct Fmt<F_Q8_0P> {
-  static constexpr int UW = 64, UPB = 1, BW = 64, BB = 68;
-  static constexpr int XV = 8, NG = 2, NWV = 32;
-  struct Raw { u32x4 a, b, c, d; uint32_t e; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    const uint8_t* p = row + 68 * u; Raw r; r.a = ld16_a4(p); r.b = ld16_a4(p + 16); r.c = ld16_a4(p + 32); r.d = ld16_a4(p + 48); r.e = ld4_a4(p + 64); return r;
-  }
-  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
-  static constexpr int NKC = 1;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64646464u); }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
-    const uint32_t q[16] = {__builtin_amdgcn_alignbit(r.c.x, r.a.x, 16), r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w,
-                            r.c.y, r.c.z, r.c.w, r.d.x, r.d.y, r.d.z, r.d.w, r.e};
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const uint32_t u = q[i] ^ 0x80808080u;
-      wv[2 * i + 0] = __builtin_amdgcn_perm(kc[0], u, 0x04010400u);   // bytes 0, 1 -> fp16 1152 + q
-      wv[2 * i + 1] = __builtin_amdgcn_perm(kc[0], u, 0x04030402u);   // bytes 2, 3
-    }
-  }
-  // pairs in decode order: block 0: N0, N15, N1, N2, ..., N14;  block 1: natural
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-    constexpr int ORD[16] = {0, 15, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14};
-#pragma unroll
-    for (int v = 0; v < 4; v++) { xv[v].x = nx[ORD[4 * v]]; xv[v].y = nx[ORD[4 * v + 1]]; xv[v].z = nx[ORD[4 * v + 2]]; xv[v].w = nx[ORD[4 * v + 3]]; }
-#pragma unroll
-    for (int v = 4; v < 8; v++) { xv[v].x = nx[4 * v]; xv[v].y = nx[4 * v + 1]; xv[v].z = nx[4 * v + 2]; xv[v].w = nx[4 * v + 3]; }
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-      float t = 0.f;
-#pragma unroll
-      for (int k = 0; k < 16; k++) t = dot2(nx[16 * j + k], 0x64806480u, t);   // 1152
-      c[j] = -t;
-    }
-  }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
-    return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
-  }
-};
-
-// ------------------------------------------------------------------------------------------------ MXFP4 (gguf.py:105-114)
-template <> struct Fmt<GGML_MXFP4> {
-  static constexpr int UW = 32, UPB = 1, BW = 32, BB = 17;
-  static constexpr int XV = 4, NG = 1, NWV = 16;
-  struct Raw { u32x4 q; uint32_t e; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    // the 17-byte block starts at any byte offset o of an aligned dword: load the five enclosing dwords and shift
-    const uintptr_t a = (uintptr_t)(row + 17 * u); const uint32_t o = (uint32_t)(a & 3);
-    const uint8_t* q = (const uint8_t*)(a & ~(uintptr_t)3);
-    const u32x4 v = ld16_a4(q); const uint32_t t = ld4_a4(q + 16);
-    const uint32_t sh = 8 * (o + 1);   // 8..32
-    Raw r; r.e = (v.x >> (8 * o)) & 0xFFu;
-    r.q.x = (uint32_t)((((uint64_t)v.y << 32) | v.x) >> sh); r.q.y = (uint32_t)((((uint64_t)v.z << 32) | v.y) >> sh);
-    r.q.z = (uint32_t)((((uint64_t)v.w << 32) | v.z) >> sh); r.q.w = (uint32_t)((((uint64_t)t << 32) | v.w) >> sh);
-    return r;
-  }
-  static __device__ __forceinline__ int xoff(int u, int k) { return 32 * u + 2 * k; }
-  // hardware E2M1 -> fp16 (true values 0..6); byte s of dword t holds weights 4t+s (low nibble) and 4t+s+16 (high nibble)
-  static constexpr int NKC = 1;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = 0; }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t*) {
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      wv[4 * t + 0] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], 1.0f, 0));
-      wv[4 * t + 1] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], 1.0f, 1));
-      wv[4 * t + 2] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], 1.0f, 2));
-      wv[4 * t + 3] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], 1.0f, 3));
-    }
-  }
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-#pragma unroll
-    for (int t = 0; t < 4; t++) {   // pairs (x[j], x[j+16]), j = 4t..4t+3
-      xv[t].x = pack_even(nx[2 * t], nx[2 * t + 8]);         xv[t].y = pack_odd(nx[2 * t], nx[2 * t + 8]);
-      xv[t].z = pack_even(nx[2 * t + 1], nx[2 * t + 9]);     xv[t].w = pack_odd(nx[2 * t + 1], nx[2 * t + 9]);
-    }
-    c[0] = 0.f;
-  }
-  // reference value = (2 * e2m1) * 2^(e-128) = e2m1 * 2^(e-127); e = 0 is the fp32 subnormal 2^-127
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
-    return __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u) * a[0];
-  }
-};
-
-// ------------------------------------------------------------------------------------------------ Q6_K (gguf.py:68-72)
-// unit u of a row: superblock u>>2, half h=(u>>1)&1, sixteen-run g=u&1.  Its 64 weights are, for j = 0..3 and i = 0..15,
-// element 256*sb + 128*h + 32*j + 16*g + i, decoded from ql[64h+16g+i] (j even) / ql[64h+32+16g+i] (j odd), low nibble for
-// j < 2 and high nibble for j >= 2, and bits 2j..2j+1 of qh[32h+16g+i]; all sixteen share scale sc[8h + 2j + g].
-template <> struct Fmt<GGML_Q6_K> {
-  static constexpr int UW = 64, UPB = 4, BW = 256, BB = 210;
-  static constexpr int XV = 8, NG = 4, NWV = 32;
-  struct Raw { u32x4 a, b, h; uint32_t sc0, sc1, d; };
-  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
-    // superblocks are 2-byte aligned: every piece is loaded as its enclosing aligned dwords and funnel-shifted per lane
-    const uint8_t* p = row + 210 * (u >> 2); const int h = (u >> 1) & 1, g = u & 1;
-    uint32_t tail, sh;
-    Raw r; r.a = ld16_a2(p + 64 * h + 16 * g, tail, sh); r.b = ld16_a2(p + 64 * h + 32 + 16 * g, tail, sh); r.h = ld16_a2(p + 128 + 32 * h + 16 * g, tail, sh);
-    const u32x4 sc = ld16_a2(p + 192, tail, sh);                         // sc[0..15]; tail dword holds d (bytes 208, 209)
-    r.sc0 = h ? sc.z : sc.x; r.sc1 = h ? sc.w : sc.y;
-    r.d = (uint32_t)g | (__builtin_amdgcn_alignbit(0u, tail, sh) << 16);
-    return r;
-  }
-  static __device__ __forceinline__ int xoff(int u, int k) {   // k = 0..31: natural pair k of the unit's 64 x values (j = k/8)
-    return 256 * (u >> 2) + 128 * ((u >> 1) & 1) + 32 * (k >> 3) + 16 * (u & 1) + 2 * (k & 7);
-  }
-  // wv[8j + 2t + {0,1}] = even / odd pairs of dword t of group j; value 1024 + 6-bit q
-  static constexpr int NKC = 1;
-  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); }
-  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
-    const uint32_t K64 = kc[0];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      const uint32_t A = r.a[t], B = r.b[t], H = r.h[t];
-      wv[0 + 2 * t]      = and_or(H << 4, 0x00300030u, and_or(A, 0x000F000Fu, K64));
-      wv[0 + 2 * t + 1]  = and_or(H >> 4, 0x00300030u, and_or(A >> 8, 0x000F000Fu, K64));
-      wv[8 + 2 * t]      = and_or(H << 2, 0x00300030u, and_or(B, 0x000F000Fu, K64));
-      wv[8 + 2 * t + 1]  = and_or(H >> 6, 0x00300030u, and_or(B >> 8, 0x000F000Fu, K64));
-      wv[16 + 2 * t]     = and_or(H, 0x00300030u, and_or(A >> 4, 0x000F000Fu, K64));
-      wv[16 + 2 * t + 1] = and_or(H >> 8, 0x00300030u, and_or(A >> 12, 0x000F000Fu, K64));
-      wv[24 + 2 * t]     = and_or(H >> 2, 0x00300030u, and_or(B >> 4, 0x000F000Fu, K64));
-      wv[24 + 2 * t + 1] = and_or(H >> 10, 0x00300030u, and_or(B >> 12, 0x000F000Fu, K64));
-    }
-  }
-  // xv[2j + t/2] = {E(t), O(t), E(t+1), O(t+1)} (t even), E/O = even/odd element pairs of dword t of group j
-  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const uint32_t* n = nx + 8 * j;
-      xv[2 * j].x = pack_even(n[0], n[1]); xv[2 * j].y = pack_odd(n[0], n[1]); xv[2 * j].z = pack_even(n[2], n[3]); xv[2 * j].w = pack_odd(n[2], n[3]);
-      xv[2 * j + 1].x = pack_even(n[4], n[5]); xv[2 * j + 1].y = pack_odd(n[4], n[5]); xv[2 * j + 1].z = pack_even(n[6], n[7]); xv[2 * j + 1].w = pack_odd(n[6], n[7]);
-      float s = 0.f;
-#pragma unroll
-      for (int k = 0; k < 8; k++) s = dot2(n[k], 0x64206420u, s);   // 1056 = 1024 + 32
-      c[j] = -s;
-    }
-  }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
-    const int g8 = (r.d & 1) * 8;   // scales 8h + 2j + g live in bytes g, g+2 of sc0 (j = 0, 1) and sc1 (j = 2, 3)
-    const float s0 = (float)(int)(int8_t)(r.sc0 >> g8), s1 = (float)(int)(int8_t)(r.sc0 >> (16 + g8));
-    const float s2 = (float)(int)(int8_t)(r.sc1 >> g8), s3 = (float)(int)(int8_t)(r.sc1 >> (16 + g8));
-    return h2f_bits(r.d >> 16) * (s0 * a[0] + s1 * a[1] + s2 * a[2] + s3 * a[3]);
-  }
-};
+#include "qfmt.h"
 
 // ------------------------------------------------------------------------------------------------ kernel
 // LDS layout for units [u0, u0+cu): xs[(m*XV + t) * cu + (u-u0)] (u32x4), then cs[(m*NG + j) * cu + (u-u0)] (float)
@@ -381,52 +74,64 @@ __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const 
   }
 }
 
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + __expf(-v)); }
-
-// row r (0..R-1) of row group rg -> segment and local row.  epilogue 2 pairs gate row rg with up row rg.
-template <int R>
-__device__ __forceinline__ void map_row(const QArgs& a, long long rg, int r, int& seg, long long& lr, bool& valid) {
-  if (a.epilogue == 2) { seg = r; lr = rg; valid = true; return; }
-  long long row = rg * R + r;
-  valid = row < a.ntot;
-  if (!valid) row = a.ntot - 1;
-  seg = 0;
-  if (a.nseg > 1 && row >= a.n[0]) { row -= a.n[0]; seg = 1; if (a.nseg > 2 && row >= a.n[1]) { row -= a.n[1]; seg = 2; } }
-  lr = row;
-}
-
-template <int T, int M, int R>
-__device__ __forceinline__ void store_rows(const QArgs& a, long long rg, float (&acc)[R][M]) {
-  const int lane = threadIdx.x & 63;
+// Reduce R x M partial sums across the wave and let lane 63 write rows row0 .. row0+R-1 of segment `seg` (rows >= row_end are
+// skipped; ld = rows of the segment = leading dimension of y).  Epilogue 2 (SwiGLU) treats the two accumulator rows as
+// (gate, up) of output row row0.
+template <int M, int R>
+__device__ __forceinline__ void store_rows(const QArgs& a, int seg, long long row0, long long row_end, long long ld, float (&acc)[R][M]) {
 #pragma unroll
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int m = 0; m < M; m++) acc[r][m] = wave_sum_lane63(acc[r][m]);
-  if (lane != 63) return;
+  if ((threadIdx.x & 63) != 63) return;
   if (a.epilogue == 2) {
     if constexpr (R == 2) {
 #pragma unroll
       for (int m = 0; m < M; m++) {
         const float v = silu_f(acc[0][m]) * acc[1][m];
-        if (a.y_f32) ((float*)a.y[0])[(long long)m * a.n[0] + rg] = v; else ((_Float16*)a.y[0])[(long long)m * a.n[0] + rg] = (_Float16)v;
+        const long long o = (long long)m * ld + row0;
+        if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
       }
     }
     return;
   }
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    int seg; long long lr; bool valid;
-    map_row<R>(a, rg, r, seg, lr, valid);
-    if (!valid) continue;
+    if (row0 + r >= row_end) continue;
 #pragma unroll
     for (int m = 0; m < M; m++) {
-      const long long o = (long long)m * a.n[seg] + lr;
+      const long long o = (long long)m * ld + row0 + r;
       float v = acc[r][m];
       if (a.epilogue == 1) v += a.resid[seg][o];
       if (a.y_f32) ((float*)a.y[seg])[o] = v; else ((_Float16*)a.y[seg])[o] = (_Float16)v;
     }
   }
 }
+
+// The wave's slice [lo, hi) of a segment's rows (SwiGLU: of the paired gate/up rows), walked as a software pipeline over
+// "steps" (R rows x one 64-unit slice of K): the loads of step s+1 are in flight while step s is multiplied.
+// PRIMED: the first step's loads were already issued into b0 before the activations were staged.
+template <int T, int M, int R>
+struct RowWalker {
+  using F = Fmt<T>;
+  typedef typename F::Raw Raw;
+  const QArgs& a; const u32x4* xs; const float* cs; const uint32_t* kc;
+  int cu, iters, lane;
+  // load stream
+  const uint8_t* base[R]; long long l_row, hi; int l_it;
+  __device__ __forceinline__ void issue(Raw* buf) {
+    const int u = l_it * 64 + lane;
+    if (u < cu) {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        long long row = (a.epilogue == 2) ? l_row : l_row + r;
+        if (row > hi - 1) row = hi - 1;                      // ragged last group: reload a valid row, the result is dropped
+        buf[r] = F::load(base[(a.epilogue == 2) ? r : 0] + row * a.row_bytes, u);
+      }
+    }
+    if (++l_it == iters) { l_it = 0; l_row += (a.epilogue == 2) ? 1 : R; }
+  }
+};
 
 template <int T, int M, int R>
 __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
@@ -436,7 +141,8 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: row pointers stay in SGPRs
   const long long gw = (long long)blockIdx.x * QG_WAVES + wave, nw = (long long)gridDim.x * QG_WAVES;
-  const long long ngroups = (a.epilogue == 2) ? a.ntot : (a.ntot + R - 1) / R;
+  const int RS = (a.epilogue == 2) ? 1 : R;                            // output rows per row group
+  const long long ngroups = (a.ntot + RS - 1) / RS;
   uint32_t kc[F::NKC];
   F::consts(kc);
   float acc[R][M];
@@ -446,59 +152,68 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
     for (int m = 0; m < M; m++) acc[r][m] = 0.f;
 
   if (a.nchunks == 1) {
-    // Software pipeline over "steps" (row group, 64-unit slice of K): the loads of step s+1 are in flight while step s is
-    // multiplied, and the first step's loads are issued before the activations are staged.
+    // contiguous share of the row groups for this wave: groups [g0, g1), sizes differing by at most one
+    const long long gbase = ngroups / nw, grem = ngroups % nw;
+    const long long g0 = gw * gbase + (gw < grem ? gw : grem), g1 = g0 + gbase + (gw < grem ? 1 : 0);
+    const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
     const int cu = a.nu, iters = (cu + 63) >> 6;
-    const long long mine = gw < ngroups ? (ngroups - gw + nw - 1) / nw : 0, nsteps = mine * iters;
     u32x4* xs = lds; float* cs = (float*)(lds + M * F::XV * cu);
-    long long l_rg = gw, c_rg = gw; int l_it = 0, c_it = 0;
-    const uint8_t* l_rp[R];
-    auto l_setup = [&]() {
-#pragma unroll
-      for (int r = 0; r < R; r++) { int seg; long long lr; bool valid; map_row<R>(a, l_rg, r, seg, lr, valid); l_rp[r] = a.w[seg] + lr * a.row_bytes; }
-    };
-    auto issue = [&](Raw* buf) {
-      const int u = l_it * 64 + lane;
-      if (u < cu) {
-#pragma unroll
-        for (int r = 0; r < R; r++) buf[r] = F::load(l_rp[r], u);
-      }
-      if (++l_it == iters) { l_it = 0; l_rg += nw; if (l_rg < ngroups) l_setup(); }
-    };
-    auto compute = [&](const Raw* buf) {
-      const int u = c_it * 64 + lane;
-      if (u < cu) {
-#pragma unroll
-        for (int r = 0; r < R; r++) unit_dot<T, M>(buf[r], xs, cs, cu, u, acc[r], kc);
-      }
-      if (++c_it == iters) {
-        store_rows<T, M, R>(a, c_rg, acc);
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-          for (int m = 0; m < M; m++) acc[r][m] = 0.f;
-        c_it = 0; c_rg += nw;
-      }
-    };
+    RowWalker<T, M, R> wk{a, xs, cs, kc, cu, iters, lane};
     Raw b0[R], b1[R];
-    if (mine) { l_setup(); issue(b0); }
-    stage_chunk<T, M>(a, xs, cs, 0, cu);
-    __syncthreads();
-    for (long long s = 0; s < nsteps; s += 2) {
-      if (s + 1 < nsteps) issue(b1);
-      compute(b0);
-      if (s + 1 < nsteps) {
-        if (s + 2 < nsteps) issue(b0);
-        compute(b1);
+    bool staged = false;
+    long long seg_start = 0;
+    const int nseg = (a.epilogue == 2) ? 1 : a.nseg;
+    for (int seg = 0; seg < nseg; seg++) {
+      const long long seg_rows = a.n[seg];
+      // this wave's rows inside the segment, as local row indices [lo, hi)
+      long long lo = row_lo - seg_start, hi = row_hi - seg_start;
+      if (lo < 0) lo = 0;
+      if (hi > seg_rows) hi = seg_rows;
+      seg_start += seg_rows;
+      const long long nrg = hi > lo ? (hi - lo + RS - 1) / RS : 0, nsteps = nrg * iters;
+      wk.base[0] = a.w[seg]; if constexpr (R > 1) { if (a.epilogue == 2) wk.base[1] = a.w[1]; }
+      wk.l_row = lo; wk.hi = hi; wk.l_it = 0;
+      if (nsteps) wk.issue(b0);
+      if (!staged) { stage_chunk<T, M>(a, xs, cs, 0, cu); __syncthreads(); staged = true; }
+      long long c_row = lo; int c_it = 0;
+      auto compute = [&](const Raw* buf) {
+        const int u = c_it * 64 + lane;
+        if (u < cu) {
+#pragma unroll
+          for (int r = 0; r < R; r++) unit_dot<T, M>(buf[r], xs, cs, cu, u, acc[r], kc);
+        }
+        if (++c_it == iters) {
+          store_rows<M, R>(a, seg, c_row, hi, seg_rows, acc);
+#pragma unroll
+          for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int m = 0; m < M; m++) acc[r][m] = 0.f;
+          c_it = 0; c_row += RS;
+        }
+      };
+      for (long long s = 0; s < nsteps; s += 2) {
+        if (s + 1 < nsteps) wk.issue(b1);
+        compute(b0);
+        if (s + 1 < nsteps) {
+          if (s + 2 < nsteps) wk.issue(b0);
+          compute(b1);
+        }
       }
     }
+    if (!staged) { stage_chunk<T, M>(a, xs, cs, 0, cu); __syncthreads(); }   // keep the barrier count uniform across waves
   } else {
     // K walked in LDS-sized chunks; one row group per wave (the host sizes the grid so that gw covers every group)
-    const long long rg = gw;
-    const bool active = rg < ngroups;
+    const bool active = gw < ngroups;
+    // locate the group's segment and local row (rows of a group never straddle a segment: host enforces R == 1 or nseg == 1)
+    long long row = (active ? gw : 0) * RS; int seg = 0;
+    if (a.epilogue != 2) while (seg + 1 < a.nseg && row >= a.n[seg]) { row -= a.n[seg]; seg++; }
+    const long long seg_rows = a.n[seg];
     const uint8_t* rp[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) { int seg; long long lr; bool valid; map_row<R>(a, active ? rg : 0, r, seg, lr, valid); rp[r] = a.w[seg] + lr * a.row_bytes; }
+    for (int r = 0; r < R; r++) {
+      long long rr = (a.epilogue == 2) ? row : (row + r < seg_rows ? row + r : seg_rows - 1);
+      rp[r] = a.w[(a.epilogue == 2) ? r : seg] + rr * a.row_bytes;
+    }
     for (int ch = 0; ch < a.nchunks; ch++) {
       const int u0 = ch * a.chunk_u, cu = min(a.chunk_u, a.nu - u0);
       u32x4* xs = lds; float* cs = (float*)(lds + M * F::XV * cu);
@@ -515,7 +230,7 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
         }
       }
     }
-    if (active) store_rows<T, M, R>(a, rg, acc);
+    if (active) store_rows<M, R>(a, seg, row, seg_rows, seg_rows, acc);
   }
 }
 
@@ -568,7 +283,8 @@ static int launch_qgemv_r(const QArgs& a, hipStream_t s) {
   // SwiGLU pairs gate/up rows: exactly two rows per group.  Otherwise two rows per wave step as well (more loads in flight
   // per lane); a single row per group when there are too few rows to fill the chip.
   if (a.epilogue == 2) return launch_qgemv<T, M, 2>(a, s);
-  if (M > 1 || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
+  const bool chunked = (long long)M * (16 * Fmt<T>::XV + 4 * Fmt<T>::NG) * (a.K / Fmt<T>::UW) > QG_LDS_BUDGET;
+  if (M > 1 || chunked || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
   return launch_qgemv<T, M, 2>(a, s);
 }
 
@@ -586,6 +302,8 @@ static int launch_qgemv_m(const QArgs& a, int M, hipStream_t s) {
   }
   return tga_set_error("tga_qlinear: M=%d out of range 1..8", M);
 }
+
+int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 
 extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                  const void* x, int x_dtype, int y_dtype, int M, int64_t K,
@@ -617,6 +335,10 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
   // block-pair units need an even number of blocks per row and 4-byte aligned rows
   bool pair = (K / 32) % 2 == 0;
   for (int i = 0; i < nseg; i++) pair = pair && ((uintptr_t)w[i] & 3) == 0;
+  if (M == 1) {
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+    if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
+  }
   switch (ggml_type) {
     case GGML_Q4_0: return pair ? launch_qgemv_m<F_Q4_0P>(a, M, s) : launch_qgemv_m<GGML_Q4_0>(a, M, s);
     case GGML_Q8_0: return pair ? launch_qgemv_m<F_Q8_0P>(a, M, s) : launch_qgemv_m<GGML_Q8_0>(a, M, s);

@@ -1,0 +1,201 @@
+// M = 1 dequant-GEMV fast path (decode): see qgemv.hip for the overall design.
+#include "qfmt.h"
+
+// ------------------------------------------------------------------------------------------------ M = 1 fast path
+// One activation row: each lane keeps the activations of ITS unit in registers for the whole kernel (no LDS traffic in the
+// loop).  A workgroup is WR x WK waves: the WK waves of a row team split K (wave wk owns units 64wk .. 64wk+63) and their
+// partial sums meet in LDS once per row group (the only LDS use in the loop: split-K partials); the WR teams own disjoint
+// row ranges.  Each team walks a contiguous range of row groups with a two-deep register pipeline: the loads of group g+1
+// are in flight while group g is multiplied and reduced.
+// Activations reach the registers through one LDS transpose per workgroup: coalesced 16-byte global loads of the plain row,
+// then each lane reads back the 64 (or 32) values of its unit (unit stride padded to spread LDS banks).
+template <int T, int R, int WK, int WR, int EPI>
+__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
+  using F = Fmt<T>;
+  typedef typename F::Raw Raw;
+  static_assert(WK == 1 || WR == 1, "row teams and K split are not combined");
+  constexpr int NT = WK * WR * 64;
+  constexpr int NP = F::UW / 2;                                  // dwords (fp16 pairs) per unit
+  constexpr int USTRIDE = NP + 4;                                // padded unit stride in dwords
+  extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
+  __shared__ float part[2][WK][R];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wk = (WK > 1) ? wave : 0, wr = (WK > 1) ? 0 : wave;
+  const int u = wk * 64 + lane;
+  const bool uvalid = u < a.nu;
+  constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
+  const long long ngroups = (a.ntot + RS - 1) / RS;
+  const long long nteams = (long long)gridDim.x * WR, team = (long long)blockIdx.x * WR + wr;
+  const long long gbase = ngroups / nteams, grem = ngroups % nteams;
+  const long long g0 = team * gbase + (team < grem ? team : grem), g1 = g0 + gbase + (team < grem ? 1 : 0);
+  const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  u32x4 xv[F::XV]; float cv[F::NG];
+  bool staged = false;
+  long long seg_start = 0;
+  const int nseg = (EPI == 2) ? 1 : a.nseg;
+  int parity = 0;
+  for (int seg = 0; seg < nseg; seg++) {
+    const long long seg_rows = a.n[seg];
+    long long lo = row_lo - seg_start, hi = row_hi - seg_start;
+    if (lo < 0) lo = 0;
+    if (hi > seg_rows) hi = seg_rows;
+    seg_start += seg_rows;
+    const long long cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;   // row groups of this team inside the segment
+    const uint8_t* base0 = a.w[seg];
+    const uint8_t* base1 = (EPI == 2) ? a.w[1] : a.w[seg];
+    auto issue = [&](Raw* buf, long long row) {
+      if (uvalid) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          long long rr = (EPI == 2) ? row : row + r;
+          if (rr > hi - 1) rr = hi - 1;                            // ragged last group: reload a valid row, result dropped
+          buf[r] = F::load(((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes, u);
+        }
+      }
+    };
+    auto finish_group = [&](const Raw* buf, long long row) {
+      float acc[R];
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        if (uvalid) unit_dot_reg<T>(buf[r], xv, cv, acc[r], kc);
+        acc[r] = wave_sum_lane63(acc[r]);
+      }
+      if constexpr (WK > 1) {
+        if (lane == 63) {
+#pragma unroll
+          for (int r = 0; r < R; r++) part[parity][wave][r] = acc[r];
+        }
+        __syncthreads();
+        if (wave == 0) {
+          float t = 0.f;
+          if (lane < R) {
+#pragma unroll
+            for (int j = 0; j < WK; j++) t += part[parity][j][lane];
+          }
+          if constexpr (EPI == 2) {
+            const float up = __shfl(t, 1, 64);
+            if (lane == 0) store_swiglu(a, row, t, up);
+          } else {
+            if (lane < R && row + lane < hi) store_one<EPI>(a, seg, row + lane, t);
+          }
+        }
+        parity ^= 1;
+      } else {
+        if (lane == 63) {
+          if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1]);
+          else {
+#pragma unroll
+            for (int r = 0; r < R; r++) if (row + r < hi) store_one<EPI>(a, seg, row + r, acc[r]);
+          }
+        }
+      }
+    };
+    Raw b0[R], b1[R];
+    if (cnt) issue(b0, lo);
+    if (!staged) {
+      // activations: coalesced global -> LDS (natural order, padded unit stride) -> this lane's unit -> staged registers
+      const int nq = a.K / 8;                                      // 16-byte fp16 pieces in the row
+      for (int i = threadIdx.x; i < nq; i += NT) {
+        u32x4 v;
+        if (a.x_f32) {
+          const f32x4 lo4 = ((const f32x4*)a.x)[2 * i], hi4 = ((const f32x4*)a.x)[2 * i + 1];
+          v.x = f2h_bits(lo4.x) | (f2h_bits(lo4.y) << 16); v.y = f2h_bits(lo4.z) | (f2h_bits(lo4.w) << 16);
+          v.z = f2h_bits(hi4.x) | (f2h_bits(hi4.y) << 16); v.w = f2h_bits(hi4.z) | (f2h_bits(hi4.w) << 16);
+        } else v = ((const u32x4*)a.x)[i];
+        // element 8i lives in unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
+        *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
+      }
+      __syncthreads();
+      if (uvalid) {
+        uint32_t nx[NP];
+#pragma unroll
+        for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + u * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+        F::stage(nx, xv, cv);
+      }
+      staged = true;
+    }
+    long long row = lo;
+    for (long long g = 0; g < cnt; g += 2) {
+      if (g + 1 < cnt) issue(b1, row + RS);
+      finish_group(b0, row);
+      row += RS;
+      if (g + 1 < cnt) {
+        if (g + 2 < cnt) issue(b0, row + RS);
+        finish_group(b1, row);
+        row += RS;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ host side
+static int fast_cu_count() {
+  static int n = 0;
+  if (!n) { int dev = 0; hipDeviceProp_t p; n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) ? p.multiProcessorCount : 256; }
+  return n;
+}
+
+template <int T, int R, int WK, int WR, int EPI>
+static int launch_fast(QArgs a, hipStream_t s) {
+  using F = Fmt<T>;
+  constexpr int RS = (EPI == 2) ? 1 : R;
+  const long long ngroups = (a.ntot + RS - 1) / RS;
+  const size_t lds = (size_t)a.nu * (F::UW / 2 + 4) * 4;
+  // resident row teams per CU: 16 waves (<= 128 VGPRs) unless the staged activations in LDS (160 KB per CU) allow fewer
+  int wg_per_cu = 16 / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;
+  const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
+  const long long max_teams = (long long)fast_cu_count() * wg_per_cu * WR;
+  const long long per = (ngroups + max_teams - 1) / max_teams;     // row groups per team
+  const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
+  long long grid = (teams + WR - 1) / WR;
+  if (grid < 1) grid = 1;
+  auto kern = qgemv1_kernel<T, R, WK, WR, EPI>;
+  if (lds > 48 * 1024) {
+    static bool configured = false;
+    if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); configured = true; }
+  }
+  kern<<<dim3((unsigned)grid), dim3(WK * WR * 64), lds, s>>>(a);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int T, int WK, int WR>
+static int launch_fast_e(const QArgs& a, hipStream_t s) {
+  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2>(a, s);
+  // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice
+  // (the wide Q8_0 / Q6_K units would need > 128 VGPRs with two rows in flight twice: one row there)
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4) && a.ntot >= (long long)fast_cu_count() * 16 * 2 / WK;
+  if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1>(a, s) : launch_fast<T, 1, WK, WR, 1>(a, s);
+  return r2 ? launch_fast<T, 2, WK, WR, 0>(a, s) : launch_fast<T, 1, WK, WR, 0>(a, s);
+}
+
+template <int T>
+static int launch_fast_w(QArgs a, hipStream_t s) {
+  using F = Fmt<T>;
+  a.nu = a.K / F::UW;
+  a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+  const int waves = (a.nu + 63) / 64;
+  if (waves <= 1) return launch_fast_e<T, 1, 4>(a, s);
+  if (waves <= 2) return launch_fast_e<T, 2, 1>(a, s);
+  if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);
+  if (waves <= 8) return launch_fast_e<T, 8, 1>(a, s);
+  return launch_fast_e<T, 16, 1>(a, s);
+}
+
+// Returns -1 when the shape is outside the fast path (caller falls back to the LDS-staged kernel).
+int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
+  const int uw = (fmt == GGML_MXFP4) ? 32 : 64;
+  if ((a.K / uw + 63) / 64 > 16 || a.K % 8) return -1;
+  if (((uintptr_t)a.x & 15) != 0) return -1;                       // coalesced 16-byte activation loads
+  switch (fmt) {
+    case F_Q4_0P: return launch_fast_w<F_Q4_0P>(a, s);
+    case F_Q8_0P: return launch_fast_w<F_Q8_0P>(a, s);
+    case GGML_Q6_K: return launch_fast_w<GGML_Q6_K>(a, s);
+    case GGML_MXFP4: return launch_fast_w<GGML_MXFP4>(a, s);
+  }
+  return -1;
+}
