@@ -72,6 +72,35 @@ int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const
                       const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                       int epilogue, const void* const* resid, void* stream);
 
+/* ---- decode-step neighbours of the linears (batch 1), tinygrad/llm/model.py:144-204, 358-364 ----
+ * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, pad[12]} so that one captured launch sequence serves
+ * every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484). */
+
+/* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q8_0 / F16 / F32 table. */
+int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream);
+
+/* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL). */
+int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, void* stream);
+
+/* One token of TransformerBlock._attention after the q/k/v projections (model.py:180-197): half-split RoPE of q and k with the
+ * freqs_cis table rope_table[max_ctx][head_dim] = cos half | sin half (model.py:16-19, 29-33), fp16 KV append at state.pos
+ * (cache layout [n_kv_heads][max_ctx][head_dim]), GQA scaled-dot-product attention over positions 0..pos with softmax in
+ * float32 (tinygrad/mixin/rand.py:298-327).  partials: float workspace of n_heads * ceil(max_ctx/64) * (head_dim + 2). */
+int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+
+/* argmax(-1) with first-max tie rule (tinygrad/mixin/op.py:866-891) + the bookkeeping of Transformer.generate (model.py:475-484):
+ * while state.pos + 1 < state.n_prompt the next input token is prompt[pos + 1]; otherwise the argmax token is stored at
+ * out_tokens[state.step] and fed back.  scratch_v / scratch_i: 256 floats / 256 int32. */
+int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i, void* state, const int* prompt, int* out_tokens, int max_tokens, void* stream);
+/* prompt step that skips the output projection: token = prompt[pos + 1], pos += 1. */
+int tga_advance_prompt(void* state, const int* prompt, void* stream);
+
+/* ---- synthetic-model writer (no counterpart in the reference, whose weights always come from GGUF files): fills `out` with
+ * n_elements random-init weights U(-amp, amp) (nn.Linear's init range, tinygrad/nn/__init__.py:173-174) already quantized to
+ * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule); TGA_F32 fills the constant `amp`. */
+int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, uint32_t seed, float amp, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,295 @@
+// Decode-step neighbours of the quantized linears (batch 1): embedding row dequant, RMSNorm, RoPE + KV append + GQA attention
+// (flash-decoding over 64-position splits), split combine, argmax / token bookkeeping.
+// They restate, for one token, what tinygrad/llm/model.py:167-204 (_attention), :144-151 (block), :358-364 (forward) compute.
+// The position and token live in device memory so that one captured launch sequence can be replayed for every token
+// (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
+#include "common.h"
+#include "host.h"
+
+struct DecodeState {   // device-resident, 16 int32
+  int pos;             // position of the token being processed
+  int token;           // current input token id
+  int step;            // tokens generated so far
+  int n_prompt;        // prompt length: while pos + 1 < n_prompt the next input token comes from the prompt, not from argmax
+  int pad[12];
+};
+
+// ---------------------------------------------------------------------------------------------- embedding (Q4_0 / F16 / F32 row)
+// token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized.
+__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, const DecodeState* st, float* __restrict__ out) {
+  const int tok = st->token;
+  if (ggml_type == GGML_Q4_0) {
+    const uint8_t* row = table + (size_t)tok * (dim / 32) * 18;
+    for (int e = threadIdx.x; e < dim; e += 256) {
+      const uint8_t* b = row + (e >> 5) * 18; const int j = e & 31;
+      const float d = h2f_bits(ld2(b));
+      const int q = (j < 16) ? (b[2 + j] & 0xF) : (b[2 + j - 16] >> 4);
+      out[e] = (float)(q - 8) * d;
+    }
+  } else if (ggml_type == GGML_Q8_0) {
+    const uint8_t* row = table + (size_t)tok * (dim / 32) * 34;
+    for (int e = threadIdx.x; e < dim; e += 256) {
+      const uint8_t* b = row + (e >> 5) * 34;
+      out[e] = h2f_bits(ld2(b)) * (float)(int8_t)b[2 + (e & 31)];
+    }
+  } else if (ggml_type == GGML_F16) {
+    const uint16_t* row = (const uint16_t*)table + (size_t)tok * dim;
+    for (int e = threadIdx.x; e < dim; e += 256) out[e] = h2f_bits(row[e]);
+  } else {
+    const float* row = (const float*)table + (size_t)tok * dim;
+    for (int e = threadIdx.x; e < dim; e += 256) out[e] = row[e];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------- RMSNorm
+// nn.RMSNorm (tinygrad/nn/__init__.py:296-304): x * rsqrt(mean(x^2) + eps), then * weight.  Output fp16 (the activation the
+// dequant-GEMV multiplies) and optionally fp32.
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, int dim, float eps,
+                                                       _Float16* __restrict__ out16, float* __restrict__ out32) {
+  __shared__ float red[16];
+  float s = 0.f;
+  for (int e = threadIdx.x; e < dim; e += blockDim.x) { const float v = x[e]; s += v * v; }
+  s = wave_sum(s);
+  const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[wave] = s;
+  __syncthreads();
+  float tot = 0.f;
+  for (int i = 0; i < nw; i++) tot += red[i];
+  const float scale = 1.0f / sqrtf(tot / (float)dim + eps);
+  for (int e = threadIdx.x; e < dim; e += blockDim.x) {
+    const float v = (x[e] * scale) * w[e];
+    if (out16) out16[e] = (_Float16)v;
+    if (out32) out32[e] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------- RoPE + KV append + attention
+// One workgroup per (kv head, 64-position split); wave w of the workgroup serves query head kvh * group + w (group <= 4 waves
+// per pass).  q, k are rotated with the half-split rule of apply_rope (tinygrad/llm/model.py:29-33) using the caller's
+// freqs_cis table [max_ctx][hd] = cos half | sin half (precompute_freqs_cis, model.py:16-19); the split that contains `pos` writes the rotated k and v into the fp16 cache.
+// Scores: lane <-> position, softmax partials per split (max, sum, weighted V) go to `part` for the combine kernel.
+struct AttnArgs {
+  const float* q; const float* k; const float* v;     // this token's projections: [n_heads*hd], [n_kv*hd], [n_kv*hd]
+  _Float16* cache_k; _Float16* cache_v;                // [n_kv][max_ctx][hd]
+  float* part;                                         // [n_heads][nsplit][hd + 2]
+  const DecodeState* st;
+  int n_heads, n_kv, hd, max_ctx, nsplit;
+  const float* rope;                                   // [max_ctx][hd]: cos(pos * f_i) for i < hd/2, then sin(pos * f_i)
+  float scale;
+};
+
+__global__ __launch_bounds__(256) void attn_split_kernel(const AttnArgs a) {
+  const int kvh = blockIdx.x, split = blockIdx.y;
+  const int pos = a.st->pos;
+  const int p0 = split * 64;
+  if (p0 > pos) return;                                 // nothing cached in this split yet
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int hd = a.hd, half = hd >> 1, group = a.n_heads / a.n_kv;
+  __shared__ float qs[4][256];                          // rotated queries of up to 4 heads (hd <= 256)
+  __shared__ float ks[256];                             // rotated key of this token
+  // rotate this token's key (all threads cooperate) and, in the owning split, append k/v to the cache
+  for (int i = threadIdx.x; i < half; i += 256) {
+    const float c = a.rope[(size_t)pos * hd + i], s = a.rope[(size_t)pos * hd + half + i];
+    const float x1 = a.k[kvh * hd + i], x2 = a.k[kvh * hd + half + i];
+    ks[i] = x1 * c - x2 * s; ks[half + i] = x2 * c + x1 * s;
+  }
+  __syncthreads();
+  const bool owner = (pos >> 6) == split;
+  if (owner) {
+    for (int i = threadIdx.x; i < hd; i += 256) {
+      a.cache_k[((size_t)kvh * a.max_ctx + pos) * hd + i] = (_Float16)ks[i];
+      a.cache_v[((size_t)kvh * a.max_ctx + pos) * hd + i] = (_Float16)a.v[kvh * hd + i];
+    }
+  }
+  for (int h0 = 0; h0 < group; h0 += 4) {
+    const int gh = h0 + wave;                           // head within the group served by this wave
+    const bool hvalid = gh < group;
+    const int head = kvh * group + gh;
+    if (hvalid) {
+      for (int i = lane; i < half; i += 64) {
+        const float c = a.rope[(size_t)pos * hd + i], s = a.rope[(size_t)pos * hd + half + i];
+        const float x1 = a.q[head * hd + i], x2 = a.q[head * hd + half + i];
+        qs[wave][i] = x1 * c - x2 * s; qs[wave][half + i] = x2 * c + x1 * s;
+      }
+    }
+    __syncthreads();
+    if (hvalid) {
+      // scores: lane <-> position p0 + lane.  The current position's key comes from LDS (fp16-rounded like the cache copy).
+      const int p = p0 + lane;
+      const bool pvalid = p <= pos;
+      float sc = -INFINITY;
+      if (pvalid) {
+        float acc = 0.f;
+        if (p == pos) {
+          for (int i = 0; i < hd; i++) acc += qs[wave][i] * (float)(_Float16)ks[i];
+        } else {
+          const u32x4* kr = (const u32x4*)(a.cache_k + ((size_t)kvh * a.max_ctx + p) * hd);
+          for (int i8 = 0; i8 < hd / 8; i8++) {
+            const u32x4 kk = kr[i8];
+            const float* qq = &qs[wave][i8 * 8];
+            acc += qq[0] * h2f_bits(kk.x & 0xFFFF) + qq[1] * h2f_bits(kk.x >> 16) + qq[2] * h2f_bits(kk.y & 0xFFFF) + qq[3] * h2f_bits(kk.y >> 16)
+                 + qq[4] * h2f_bits(kk.z & 0xFFFF) + qq[5] * h2f_bits(kk.z >> 16) + qq[6] * h2f_bits(kk.w & 0xFFFF) + qq[7] * h2f_bits(kk.w >> 16);
+          }
+        }
+        sc = acc * a.scale;
+      }
+      const float m = wave_max(sc);
+      const float e = pvalid ? __expf(sc - m) : 0.f;
+      const float l = wave_sum(e);
+      // weighted V: lane <-> dims (lane, lane + 64, ...); positions broadcast with readlane
+      const int np = min(64, pos - p0 + 1);
+      for (int d0 = 0; d0 < hd; d0 += 64) {
+        const int d = d0 + lane;
+        float o = 0.f;
+        if (d < hd) {
+          for (int j = 0; j < np; j++) {
+            const float pj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, e), j));
+            const int pp = p0 + j;
+            const float vv = (pp == pos) ? (float)(_Float16)a.v[kvh * hd + d] : (float)a.cache_v[((size_t)kvh * a.max_ctx + pp) * hd + d];
+            o += pj * vv;
+          }
+          a.part[((size_t)head * a.nsplit + split) * (hd + 2) + d] = o;
+        }
+      }
+      if (lane == 0) {
+        a.part[((size_t)head * a.nsplit + split) * (hd + 2) + hd] = m;
+        a.part[((size_t)head * a.nsplit + split) * (hd + 2) + hd + 1] = l;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// softmax-weighted merge of the per-split partials -> attention output (fp16 activation of attn_output, optionally fp32)
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part, const DecodeState* st, int n_heads, int hd, int nsplit,
+                                                           _Float16* __restrict__ out16, float* __restrict__ out32) {
+  const int head = blockIdx.x;
+  const int ns = (st->pos >> 6) + 1;
+  const float* ph = part + (size_t)head * nsplit * (hd + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < ns; s++) m = fmaxf(m, ph[s * (hd + 2) + hd]);
+  float l = 0.f;
+  for (int s = 0; s < ns; s++) l += ph[s * (hd + 2) + hd + 1] * __expf(ph[s * (hd + 2) + hd] - m);
+  const float inv = 1.0f / l;
+  for (int d = threadIdx.x; d < hd; d += 256) {
+    float o = 0.f;
+    for (int s = 0; s < ns; s++) o += ph[s * (hd + 2) + d] * __expf(ph[s * (hd + 2) + hd] - m);
+    o *= inv;
+    if (out16) out16[head * hd + d] = (_Float16)o;
+    if (out32) out32[head * hd + d] = o;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------- argmax + token bookkeeping
+// argmax(-1) with the reference's tie rule: the first index of the maximum (tinygrad/mixin/op.py:866-891).
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int n, float* __restrict__ pv, int* __restrict__ pi) {
+  float best = -INFINITY; int bi = 0x7fffffff;
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+    const float v = logits[i];
+    if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+  }
+  __shared__ float sv[256]; __shared__ int si[256];
+  sv[threadIdx.x] = best; si[threadIdx.x] = bi;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (threadIdx.x < o) {
+      const float v = sv[threadIdx.x + o]; const int i = si[threadIdx.x + o];
+      if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && i < si[threadIdx.x])) { sv[threadIdx.x] = v; si[threadIdx.x] = i; }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) { pv[blockIdx.x] = sv[0]; pi[blockIdx.x] = si[0]; }
+}
+// Final reduce and the loop bookkeeping of Transformer.generate (tinygrad/llm/model.py:475-484) kept on the device: while
+// prompt tokens remain the next input is prompt[pos + 1]; afterwards the argmax token is appended to out_tokens and fed back.
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi, int np, DecodeState* st,
+                                                           const int* __restrict__ prompt, int* __restrict__ out_tokens, int max_tokens) {
+  __shared__ float sv[256]; __shared__ int si[256];
+  float best = -INFINITY; int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < np; i += 256) {
+    const float v = pv[i]; const int ix = pi[i];
+    if (v > best || (v == best && ix < bi)) { best = v; bi = ix; }
+  }
+  sv[threadIdx.x] = best; si[threadIdx.x] = bi;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (threadIdx.x < o) {
+      const float v = sv[threadIdx.x + o]; const int i = si[threadIdx.x + o];
+      if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && i < si[threadIdx.x])) { sv[threadIdx.x] = v; si[threadIdx.x] = i; }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const int next = st->pos + 1;
+    if (next < st->n_prompt) st->token = prompt[next];
+    else {
+      const int tok = si[0];
+      if (out_tokens && st->step < max_tokens) out_tokens[st->step] = tok;
+      st->token = tok; st->step += 1;
+    }
+    st->pos = next;
+  }
+}
+// Prompt step without sampling (no lm-head was run): feed prompt[pos + 1] and advance.
+__global__ void advance_prompt_kernel(DecodeState* st, const int* __restrict__ prompt) {
+  const int next = st->pos + 1;
+  if (next < st->n_prompt) st->token = prompt[next];
+  st->pos = next;
+}
+
+// ---------------------------------------------------------------------------------------------- C-ABI
+extern "C" {
+
+int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream) {
+  TGA_REQUIRE(table && state && out, "tga_embed_row: null pointer");
+  TGA_REQUIRE(ggml_type == GGML_Q4_0 || ggml_type == GGML_Q8_0 || ggml_type == GGML_F16 || ggml_type == GGML_F32, "tga_embed_row: unsupported table type %d", ggml_type);
+  TGA_REQUIRE(dim > 0 && dim % 32 == 0, "tga_embed_row: dim=%d must be a positive multiple of 32", dim);
+  embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (const DecodeState*)state, out);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, void* stream) {
+  TGA_REQUIRE(x && weight && (out_f16 || out_f32), "tga_rmsnorm: null pointer");
+  TGA_REQUIRE(dim > 0, "tga_rmsnorm: dim=%d", dim);
+  rmsnorm_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
+  TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
+  TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
+  TGA_REQUIRE(head_dim % 8 == 0 && head_dim >= 8 && head_dim <= 256, "tga_attention_decode: head_dim=%d must be a multiple of 8 in 8..256", head_dim);
+  TGA_REQUIRE(max_ctx > 0, "tga_attention_decode: max_ctx=%d", max_ctx);
+  AttnArgs a;
+  a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (const DecodeState*)state;
+  a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
+  a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
+  attn_split_kernel<<<dim3(n_kv_heads, a.nsplit), 256, 0, (hipStream_t)stream>>>(a);
+  TGA_LAUNCH_CHECK();
+  attn_combine_kernel<<<n_heads, 256, 0, (hipStream_t)stream>>>(partials, a.st, n_heads, head_dim, a.nsplit, (_Float16*)out_f16, out_f32);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i, void* state, const int* prompt, int* out_tokens, int max_tokens, void* stream) {
+  TGA_REQUIRE(logits && scratch_v && scratch_i && state && prompt, "tga_argmax_step: null pointer");
+  TGA_REQUIRE(n > 0, "tga_argmax_step: n=%d", n);
+  const int np = 256;
+  argmax_partial_kernel<<<np, 256, 0, (hipStream_t)stream>>>(logits, n, scratch_v, scratch_i);
+  TGA_LAUNCH_CHECK();
+  argmax_final_kernel<<<1, 256, 0, (hipStream_t)stream>>>(scratch_v, scratch_i, np, (DecodeState*)state, prompt, out_tokens, max_tokens);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_advance_prompt(void* state, const int* prompt, void* stream) {
+  TGA_REQUIRE(state && prompt, "tga_advance_prompt: null pointer");
+  advance_prompt_kernel<<<1, 1, 0, (hipStream_t)stream>>>((DecodeState*)state, prompt);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,183 @@
+"""Batch-1 decode of a llama-architecture Transformer whose linears stay in GGUF blocks (mirror of tinygrad/llm/model.py).
+
+Transformer mirrors the reference's class for the dense (non-MoE) path: token_embd -> blocks -> output_norm -> output ->
+greedy argmax (model.py:358-364).  Every Linear call site of the reference (model.py:168,198,137,362) is a fused dequant-GEMV
+over the raw GGUF bytes; per block the launches are
+  rmsnorm -> q/k/v (one launch) -> RoPE + KV append + attention -> attn_output (+ residual) -> rmsnorm -> gate/up + SwiGLU -> down (+ residual)
+and one token step is captured once and replayed (the reference's TinyJit replay), with position/token kept in device memory.
+Numerics that differ from the reference's defaults, stated once: activations entering a linear are rounded to fp16
+(reference: fp32 activations x fp16 weights), the KV cache is fp16 (config 3; reference default is fp32)."""
+from __future__ import annotations
+import ctypes
+from dataclasses import dataclass
+import numpy as np
+from tinygrad_amd import runtime as rt
+from tinygrad_amd.runtime import Buffer, GGML_QUANT
+from tinygrad_amd.nn import QuantLinear, qlinear_multi
+
+@dataclass(frozen=True)
+class TransformerConfig:
+  """Subset of the reference's TransformerConfig (tinygrad/llm/model.py:52-82) the dense path reads."""
+  num_blocks: int
+  dim: int
+  hidden_dim: int
+  n_heads: int
+  n_kv_heads: int
+  norm_eps: float
+  vocab_size: int
+  head_dim: int
+  rope_theta: float
+  max_context: int
+
+LLAMA3_8B = dict(num_blocks=32, dim=4096, hidden_dim=14336, n_heads=32, n_kv_heads=8, norm_eps=1e-5, vocab_size=128256,
+                 head_dim=128, rope_theta=500000.0)
+
+def precompute_freqs_cis(dim: int, end: int, theta: float) -> np.ndarray:
+  """tinygrad/llm/model.py:16-19 in float32: cat(cos(pos * f), sin(pos * f)), f = 1 / theta^(2i/dim)."""
+  freqs = (np.float32(1.0) / (np.float32(theta) ** (np.arange(0, dim, 2, dtype=np.float32)[:dim // 2] / np.float32(dim)))).astype(np.float32)
+  ang = (np.arange(end, dtype=np.float32)[:, None] * freqs[None, :]).astype(np.float32)
+  return np.concatenate([np.cos(ang), np.sin(ang)], axis=-1).astype(np.float32)
+
+def quant_nbytes(ggml_type: int, n: int) -> int:
+  if ggml_type == rt.F32: return 4 * n
+  if ggml_type == rt.F16: return 2 * n
+  nel, nby = GGML_QUANT[ggml_type]
+  return n // nel * nby
+
+def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = rt.Q4_0, head_type: int = rt.Q6_K, stream=None) -> dict:
+  """Random-init model written straight into HBM as GGUF blocks: {gguf tensor name: (Buffer, ggml_type, (rows, cols))}.
+  Linear and embedding weights ~ U(-1/sqrt(in), 1/sqrt(in)) quantized to linear_type, lm-head to head_type, norm weights 1."""
+  c, sd, tid = config, {}, [0]
+  def mk(name, rows, cols, t, amp):
+    buf = Buffer((quant_nbytes(t, rows * cols),), np.uint8)
+    tid[0] += 1
+    rt.check(rt.lib().tga_synth_weights(t, buf.ptr, rows * cols, (seed * 7919 + tid[0]) & 0xFFFFFFFF, amp, stream))
+    sd[name] = (buf, t, (rows, cols))
+  mk("token_embd.weight", c.vocab_size, c.dim, linear_type, 1.0)
+  for i in range(c.num_blocks):
+    p = f"blk.{i}."
+    mk(p + "attn_norm.weight", 1, c.dim, rt.F32, 1.0)
+    mk(p + "attn_q.weight", c.n_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
+    mk(p + "attn_k.weight", c.n_kv_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
+    mk(p + "attn_v.weight", c.n_kv_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
+    mk(p + "attn_output.weight", c.dim, c.n_heads * c.head_dim, linear_type, (c.n_heads * c.head_dim) ** -0.5)
+    mk(p + "ffn_norm.weight", 1, c.dim, rt.F32, 1.0)
+    mk(p + "ffn_gate.weight", c.hidden_dim, c.dim, linear_type, c.dim ** -0.5)
+    mk(p + "ffn_up.weight", c.hidden_dim, c.dim, linear_type, c.dim ** -0.5)
+    mk(p + "ffn_down.weight", c.dim, c.hidden_dim, linear_type, c.hidden_dim ** -0.5)
+  mk("output_norm.weight", 1, c.dim, rt.F32, 1.0)
+  mk("output.weight", c.vocab_size, c.dim, head_type, c.dim ** -0.5)
+  return sd
+
+class TransformerBlock:
+  """One decode step of the reference's TransformerBlock/FFNBlock (tinygrad/llm/model.py:144-204) for batch 1."""
+  def __init__(self, config: TransformerConfig, sd: dict, i: int, shared):
+    c, p = config, f"blk.{i}."
+    lin = lambda name: QuantLinear(sd[p + name][0], sd[p + name][1], *sd[p + name][2])
+    self.attn_norm, self.ffn_norm = sd[p + "attn_norm.weight"][0], sd[p + "ffn_norm.weight"][0]
+    self.attn_q, self.attn_k, self.attn_v, self.attn_output = lin("attn_q.weight"), lin("attn_k.weight"), lin("attn_v.weight"), lin("attn_output.weight")
+    self.ffn_gate, self.ffn_up, self.ffn_down = lin("ffn_gate.weight"), lin("ffn_up.weight"), lin("ffn_down.weight")
+    # KV cache: fp16 [n_kv_heads][max_context][head_dim] each (reference: one [2,B,KvH,ctx,Hd] tensor, model.py:202)
+    self.cache_k = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
+    self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
+    self.config, self.s = c, shared
+
+  def __call__(self, x: Buffer, stream):
+    c, s, L = self.config, self.s, rt.lib()
+    # h = x + attention(attn_norm(x))                                                     model.py:149
+    rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
+    qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream)
+    rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
+                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, stream))
+    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream)
+    # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
+    rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
+    qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream)
+    qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream)
+
+class _Shared:
+  """Activation buffers shared by all blocks (batch 1)."""
+  def __init__(self, c: TransformerConfig, max_new: int):
+    f32, f16 = np.float32, np.float16
+    self.state = Buffer((16,), np.int32).zero_()
+    self.x = Buffer((1, c.dim), f32)
+    self.xn = Buffer((1, c.dim), f16)
+    self.q, self.k, self.v = Buffer((1, c.n_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32)
+    self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
+    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32)
+    self.act = Buffer((1, c.hidden_dim), f16)
+    self.logits = Buffer((1, c.vocab_size), f32)
+    self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)
+    self.rope = Buffer.from_numpy(precompute_freqs_cis(c.head_dim, c.max_context, c.rope_theta))
+    self.prompt = Buffer((c.max_context,), np.int32).zero_()
+    self.out_tokens = Buffer((max(1, max_new),), np.int32).zero_()
+
+class Transformer:
+  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096):
+    self.config = c = config
+    self.s = _Shared(c, max_new)
+    self.max_new = max_new
+    emb = state_dict["token_embd.weight"]
+    self.token_embd, self.embd_type = emb[0], emb[1]
+    self.blk = [TransformerBlock(c, state_dict, i, self.s) for i in range(c.num_blocks)]
+    self.output_norm = state_dict["output_norm.weight"][0]
+    out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
+    self.output = QuantLinear(out[0], out[1], *out[2])
+    self.stream = rt.Stream()
+    self._graphs = {}
+
+  # one token through all blocks; with_head adds output_norm + output + argmax (model.py:358-364)
+  def _step(self, with_head: bool):
+    c, s, L, st = self.config, self.s, rt.lib(), self.stream.handle
+    rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
+    for b in self.blk: b(s.x, st)
+    if with_head:
+      rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, st))
+      self.output(s.xn, out=s.logits, stream=st)
+      rt.check(L.tga_argmax_step(s.logits.ptr, c.vocab_size, s.am_v.ptr, s.am_i.ptr, s.state.ptr, s.prompt.ptr, s.out_tokens.ptr, self.max_new, st))
+    else:
+      rt.check(L.tga_advance_prompt(s.state.ptr, s.prompt.ptr, st))
+
+  def _graph(self, with_head: bool) -> rt.Graph:
+    if with_head not in self._graphs:
+      g = rt.Graph(self.stream)
+      with g: self._step(with_head)
+      self._graphs[with_head] = g
+    return self._graphs[with_head]
+
+  def reset(self, tokens: list[int]):
+    """Start a new sequence: position 0, first prompt token loaded, nothing cached (no KV-prefix reuse)."""
+    c, s = self.config, self.s
+    assert 1 <= len(tokens) < c.max_context
+    prompt = np.zeros(c.max_context, dtype=np.int32); prompt[:len(tokens)] = tokens
+    s.prompt.copyin(prompt)
+    st = np.zeros(16, dtype=np.int32); st[1], st[3] = tokens[0], len(tokens)
+    s.state.copyin(st)
+
+  def prefill(self, tokens: list[int], use_graph: bool = True):
+    """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step."""
+    self.reset(tokens)
+    for _ in range(len(tokens) - 1):
+      if use_graph: self._graph(False).launch()
+      else: self._step(False)
+    self.stream.synchronize()
+
+  def decode_step(self, use_graph: bool = True, sync: bool = True):
+    if use_graph: self._graph(True).launch()
+    else: self._step(True)
+    if sync: self.stream.synchronize()
+
+  def generate(self, tokens: list[int], max_new_tokens: int, use_graph: bool = True):
+    """Greedy decoding (temperature 0): yields one token id per step, like Transformer.generate (model.py:464-484)."""
+    self.prefill(tokens, use_graph)
+    for i in range(max_new_tokens):
+      self.decode_step(use_graph, sync=True)                          # the reference syncs once per token too (out.item(), model.py:482)
+      yield int(self.s.out_tokens.view(4 * i, (1,), np.int32).numpy()[0])
+
+  def logits(self) -> np.ndarray: return self.s.logits.numpy().reshape(-1)
+
+  def weight_bytes_per_token(self) -> int:
+    """Packed weight bytes one decode step streams (all block linears + lm-head), the reference's GB/s accounting (cli.py:179-181)."""
+    n = self.output.nbytes
+    for b in self.blk: n += sum(l.nbytes for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down))
+    return n

@@ -29,6 +29,12 @@ def _declare(lib):
     "tga_dequant": [i, vp, i64, vp, i, vp],
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
     "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, vp],
+    "tga_embed_row": [vp, i, i, vp, vp, vp],
+    "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, vp],
+    "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
+    "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
+    "tga_advance_prompt": [vp, vp, vp],
+    "tga_synth_weights": [i, vp, i64, ctypes.c_uint32, ctypes.c_float, vp],
   }
   for name, args in sig.items():
     fn = getattr(lib, name)
