@@ -55,6 +55,7 @@ def main():
   ap.add_argument("--prefill", type=int, default=1024)
   ap.add_argument("--layers", type=int, default=32, help="reduce only for smoke runs; the reported config then says so")
   ap.add_argument("--no-cpu", action="store_true")
+  ap.add_argument("--no-graph", action="store_true", help="eager launches instead of graph replay (for kernel-trace profiling)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py: this build measures one GPU only (no collectives, no sharding in this run); use --gpus 1", file=sys.stderr)
@@ -73,11 +74,12 @@ def main():
 
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=args.prefill)]
-  model.prefill(prompt)                                    # fills positions 0..prefill-2; the last prompt token is the first decode input
-  for _ in range(args.warmup): model.decode_step()
+  ug = not args.no_graph
+  model.prefill(prompt, ug)                                    # fills positions 0..prefill-2; the last prompt token is the first decode input
+  for _ in range(args.warmup): model.decode_step(ug)
   rt.synchronize()
   t0 = time.perf_counter()
-  for _ in range(args.steps): model.decode_step()          # graph launch + stream sync per token
+  for _ in range(args.steps): model.decode_step(ug)          # graph launch + stream sync per token
   rt.synchronize()
   dt = time.perf_counter() - t0
   ms_per_step = dt / args.steps * 1e3

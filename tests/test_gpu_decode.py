@@ -59,7 +59,7 @@ def test_attention_decode_kernel_vs_numpy(gpu):
   rng = np.random.default_rng(5)
   rope = precompute_freqs_cis(hd, ctx, 10000.0)
   ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
-  part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2),), np.float32)
+  part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2) + KV,), np.float32).zero_()
   ropeb = gpu.Buffer.from_numpy(rope)
   out = gpu.Buffer((H * hd,), np.float32)
   rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)

@@ -71,112 +71,160 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
 struct AttnArgs {
   const float* q; const float* k; const float* v;     // this token's projections: [n_heads*hd], [n_kv*hd], [n_kv*hd]
   _Float16* cache_k; _Float16* cache_v;                // [n_kv][max_ctx][hd]
-  float* part;                                         // [n_heads][nsplit][hd + 2]
+  float* part;                                         // [n_heads][nsplit][hd + 2], then n_kv int32 arrival counters (zero between launches)
   const DecodeState* st;
   int n_heads, n_kv, hd, max_ctx, nsplit;
   const float* rope;                                   // [max_ctx][hd]: cos(pos * f_i) for i < hd/2, then sin(pos * f_i)
   float scale;
+  _Float16* out16; float* out32;                       // attention output [n_heads*hd]
 };
 
-__global__ __launch_bounds__(256) void attn_split_kernel(const AttnArgs a) {
+// 8 fp16 values (one 16-byte piece) of row `p` of a cache plane; the row of the token being processed comes from LDS (fp32
+// values rounded to fp16 exactly like the copy that goes into the cache)
+__device__ __forceinline__ u32x4 kv_piece(const _Float16* plane_row0, int hd, int p, int pos, int piece, const float* cur) {
+  if (p == pos) {
+    const float* c = cur + piece * 8;
+    u32x4 r = {f2h_bits(c[0]) | (f2h_bits(c[1]) << 16), f2h_bits(c[2]) | (f2h_bits(c[3]) << 16),
+               f2h_bits(c[4]) | (f2h_bits(c[5]) << 16), f2h_bits(c[6]) | (f2h_bits(c[7]) << 16)};
+    return r;
+  }
+  return *(const u32x4*)(plane_row0 + (size_t)p * hd + piece * 8);
+}
+
+// HD8 = head_dim / 8 (16-byte pieces per row).  Workgroup = (kv head, 64-position split), wave w serves query heads w, w+4, ...
+// of the group.  K: lane <-> position (whole row in registers).  V: RPI = 64 / HD8 rows per load instruction, lane = (row-in-
+// instruction, piece); both tiles are requested before any arithmetic so their latencies overlap.
+// The last workgroup of a kv head to finish (device-scope arrival counter) merges that head group's split partials.
+template <int HD8>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
+  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 64 / RPI;   // rows per V instruction, V instructions per 64 rows
   const int kvh = blockIdx.x, split = blockIdx.y;
   const int pos = a.st->pos;
   const int p0 = split * 64;
   if (p0 > pos) return;                                 // nothing cached in this split yet
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int hd = a.hd, half = hd >> 1, group = a.n_heads / a.n_kv;
-  __shared__ float qs[4][256];                          // rotated queries of up to 4 heads (hd <= 256)
-  __shared__ float ks[256];                             // rotated key of this token
-  // rotate this token's key (all threads cooperate) and, in the owning split, append k/v to the cache
+  const int half = HD >> 1, group = a.n_heads / a.n_kv;
+  __shared__ float qs[4][HD];                           // rotated queries of the 4 heads in flight
+  __shared__ float ks[HD], vs[HD];                      // rotated key / value of this token
+  __shared__ int last_flag;
   for (int i = threadIdx.x; i < half; i += 256) {
-    const float c = a.rope[(size_t)pos * hd + i], s = a.rope[(size_t)pos * hd + half + i];
-    const float x1 = a.k[kvh * hd + i], x2 = a.k[kvh * hd + half + i];
+    const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
+    const float x1 = a.k[kvh * HD + i], x2 = a.k[kvh * HD + half + i];
     ks[i] = x1 * c - x2 * s; ks[half + i] = x2 * c + x1 * s;
   }
+  for (int i = threadIdx.x; i < HD; i += 256) vs[i] = a.v[kvh * HD + i];
   __syncthreads();
-  const bool owner = (pos >> 6) == split;
-  if (owner) {
-    for (int i = threadIdx.x; i < hd; i += 256) {
-      a.cache_k[((size_t)kvh * a.max_ctx + pos) * hd + i] = (_Float16)ks[i];
-      a.cache_v[((size_t)kvh * a.max_ctx + pos) * hd + i] = (_Float16)a.v[kvh * hd + i];
+  const _Float16* krow0 = a.cache_k + (size_t)kvh * a.max_ctx * HD;
+  const _Float16* vrow0 = a.cache_v + (size_t)kvh * a.max_ctx * HD;
+  if ((pos >> 6) == split) {                            // owner split appends this token to the cache
+    for (int i = threadIdx.x; i < HD; i += 256) {
+      a.cache_k[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)ks[i];
+      a.cache_v[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)vs[i];
     }
   }
+  // K tile: lane <-> position p0 + lane;  V tile: instruction i covers rows p0 + i*RPI + lane / HD8, piece lane % HD8
+  const int p = p0 + lane;
+  const bool pvalid = p <= pos;
+  const int pc = pvalid ? p : pos;                      // clamp to a valid row, result masked
+  u32x4 kt[HD8], vt[NVI];
+#pragma unroll
+  for (int i = 0; i < HD8; i++) kt[i] = kv_piece(krow0, HD, pc, pos, i, ks);
+  const int vr = lane / HD8, vp = lane % HD8;
+#pragma unroll
+  for (int i = 0; i < NVI; i++) { const int r = p0 + i * RPI + vr; vt[i] = kv_piece(vrow0, HD, r <= pos ? r : pos, pos, vp, vs); }
+
   for (int h0 = 0; h0 < group; h0 += 4) {
-    const int gh = h0 + wave;                           // head within the group served by this wave
+    const int gh = h0 + wave;
     const bool hvalid = gh < group;
     const int head = kvh * group + gh;
     if (hvalid) {
       for (int i = lane; i < half; i += 64) {
-        const float c = a.rope[(size_t)pos * hd + i], s = a.rope[(size_t)pos * hd + half + i];
-        const float x1 = a.q[head * hd + i], x2 = a.q[head * hd + half + i];
+        const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
+        const float x1 = a.q[head * HD + i], x2 = a.q[head * HD + half + i];
         qs[wave][i] = x1 * c - x2 * s; qs[wave][half + i] = x2 * c + x1 * s;
       }
     }
     __syncthreads();
     if (hvalid) {
-      // scores: lane <-> position p0 + lane.  The current position's key comes from LDS (fp16-rounded like the cache copy).
-      const int p = p0 + lane;
-      const bool pvalid = p <= pos;
-      float sc = -INFINITY;
-      if (pvalid) {
-        float acc = 0.f;
-        if (p == pos) {
-          for (int i = 0; i < hd; i++) acc += qs[wave][i] * (float)(_Float16)ks[i];
-        } else {
-          const u32x4* kr = (const u32x4*)(a.cache_k + ((size_t)kvh * a.max_ctx + p) * hd);
-          for (int i8 = 0; i8 < hd / 8; i8++) {
-            const u32x4 kk = kr[i8];
-            const float* qq = &qs[wave][i8 * 8];
-            acc += qq[0] * h2f_bits(kk.x & 0xFFFF) + qq[1] * h2f_bits(kk.x >> 16) + qq[2] * h2f_bits(kk.y & 0xFFFF) + qq[3] * h2f_bits(kk.y >> 16)
-                 + qq[4] * h2f_bits(kk.z & 0xFFFF) + qq[5] * h2f_bits(kk.z >> 16) + qq[6] * h2f_bits(kk.w & 0xFFFF) + qq[7] * h2f_bits(kk.w >> 16);
-          }
-        }
-        sc = acc * a.scale;
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < HD8; i++) {
+        const float* qq = &qs[wave][i * 8];
+        const u32x4 kk = kt[i];
+        acc += qq[0] * h2f_bits(kk.x & 0xFFFF) + qq[1] * h2f_bits(kk.x >> 16) + qq[2] * h2f_bits(kk.y & 0xFFFF) + qq[3] * h2f_bits(kk.y >> 16)
+             + qq[4] * h2f_bits(kk.z & 0xFFFF) + qq[5] * h2f_bits(kk.z >> 16) + qq[6] * h2f_bits(kk.w & 0xFFFF) + qq[7] * h2f_bits(kk.w >> 16);
       }
+      const float sc = pvalid ? acc * a.scale : -INFINITY;
       const float m = wave_max(sc);
       const float e = pvalid ? __expf(sc - m) : 0.f;
       const float l = wave_sum(e);
-      // weighted V: lane <-> dims (lane, lane + 64, ...); positions broadcast with readlane
-      const int np = min(64, pos - p0 + 1);
-      for (int d0 = 0; d0 < hd; d0 += 64) {
-        const int d = d0 + lane;
-        float o = 0.f;
-        if (d < hd) {
-          for (int j = 0; j < np; j++) {
-            const float pj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, e), j));
-            const int pp = p0 + j;
-            const float vv = (pp == pos) ? (float)(_Float16)a.v[kvh * hd + d] : (float)a.cache_v[((size_t)kvh * a.max_ctx + pp) * hd + d];
-            o += pj * vv;
-          }
-          a.part[((size_t)head * a.nsplit + split) * (hd + 2) + d] = o;
-        }
+      float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < NVI; i++) {
+        const float pj = __shfl(e, i * RPI + vr, 64);          // weight of the row this lane holds in instruction i (0 beyond pos)
+        const u32x4 vv = vt[i];
+        o[0] += pj * h2f_bits(vv.x & 0xFFFF); o[1] += pj * h2f_bits(vv.x >> 16); o[2] += pj * h2f_bits(vv.y & 0xFFFF); o[3] += pj * h2f_bits(vv.y >> 16);
+        o[4] += pj * h2f_bits(vv.z & 0xFFFF); o[5] += pj * h2f_bits(vv.z >> 16); o[6] += pj * h2f_bits(vv.w & 0xFFFF); o[7] += pj * h2f_bits(vv.w >> 16);
       }
-      if (lane == 0) {
-        a.part[((size_t)head * a.nsplit + split) * (hd + 2) + hd] = m;
-        a.part[((size_t)head * a.nsplit + split) * (hd + 2) + hd + 1] = l;
+      // sum the RPI lane groups that hold the same piece
+#pragma unroll
+      for (int off = HD8; off < 64; off <<= 1)
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] += __shfl_xor(o[j], off, 64);
+      float* po = a.part + ((size_t)head * a.nsplit + split) * (HD + 2);
+      if (lane < HD8) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) po[lane * 8 + j] = o[j];
       }
+      if (lane == 0) { po[HD] = m; po[HD + 1] = l; }
     }
     __syncthreads();
   }
-}
-
-// softmax-weighted merge of the per-split partials -> attention output (fp16 activation of attn_output, optionally fp32)
-__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part, const DecodeState* st, int n_heads, int hd, int nsplit,
-                                                           _Float16* __restrict__ out16, float* __restrict__ out32) {
-  const int head = blockIdx.x;
-  const int ns = (st->pos >> 6) + 1;
-  const float* ph = part + (size_t)head * nsplit * (hd + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < ns; s++) m = fmaxf(m, ph[s * (hd + 2) + hd]);
-  float l = 0.f;
-  for (int s = 0; s < ns; s++) l += ph[s * (hd + 2) + hd + 1] * __expf(ph[s * (hd + 2) + hd] - m);
-  const float inv = 1.0f / l;
-  for (int d = threadIdx.x; d < hd; d += 256) {
+  // ---- merge: the last split of this kv head to arrive combines all its heads' partials ----
+  int* counters = (int*)(a.part + (size_t)a.n_heads * a.nsplit * (HD + 2));
+  const int ns = (pos >> 6) + 1;
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int prev = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    last_flag = (prev == ns - 1);
+    if (prev == ns - 1) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __threadfence();
+  // softmax weights of every (head, split) first (parallel loads), then the weighted sum with 8 partial rows in flight per thread
+  __shared__ float sw[2048];                            // exp(m_s - m) / l per (head in group, split); host guarantees group * nsplit <= 2048
+  for (int idx = threadIdx.x; idx < group * ns; idx += 256) {
+    const int gh = idx / ns, sp = idx - gh * ns;
+    const float* ph = a.part + ((size_t)(kvh * group + gh) * a.nsplit + sp) * (HD + 2);
+    sw[gh * a.nsplit + sp] = __builtin_nontemporal_load(&ph[HD]);
+    sw[1024 + gh * a.nsplit + sp] = __builtin_nontemporal_load(&ph[HD + 1]);
+  }
+  __syncthreads();
+  for (int gh = wave; gh < group; gh += 4) {            // one wave per head: m, l, then normalised weights in place
+    float m = -INFINITY;
+    for (int sp = lane; sp < ns; sp += 64) m = fmaxf(m, sw[gh * a.nsplit + sp]);
+    m = wave_max(m);
+    float l = 0.f;
+    for (int sp = lane; sp < ns; sp += 64) l += sw[1024 + gh * a.nsplit + sp] * __expf(sw[gh * a.nsplit + sp] - m);
+    l = wave_sum(l);
+    for (int sp = lane; sp < ns; sp += 64) sw[gh * a.nsplit + sp] = __expf(sw[gh * a.nsplit + sp] - m) / l;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < group * HD; idx += 256) {
+    const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
+    const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
     float o = 0.f;
-    for (int s = 0; s < ns; s++) o += ph[s * (hd + 2) + d] * __expf(ph[s * (hd + 2) + hd] - m);
-    o *= inv;
-    if (out16) out16[head * hd + d] = (_Float16)o;
-    if (out32) out32[head * hd + d] = o;
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
+#pragma unroll
+      for (int j = 0; j < 8; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
+    }
+    if (a.out16) a.out16[head * HD + d] = (_Float16)o;
+    if (a.out32) a.out32[head * HD + d] = o;
   }
 }
 
@@ -261,15 +309,18 @@ int tga_attention_decode(const float* q, const float* k, const float* v, void* c
                          int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
-  TGA_REQUIRE(head_dim % 8 == 0 && head_dim >= 8 && head_dim <= 256, "tga_attention_decode: head_dim=%d must be a multiple of 8 in 8..256", head_dim);
-  TGA_REQUIRE(max_ctx > 0, "tga_attention_decode: max_ctx=%d", max_ctx);
+  TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode: head_dim=%d must be 64, 128 or 256", head_dim);
+  TGA_REQUIRE(max_ctx > 0 && (n_heads / n_kv_heads) * ((max_ctx + 63) / 64) <= 1024, "tga_attention_decode: max_ctx=%d too long for the merge table ((n_heads/n_kv_heads) * ceil(max_ctx/64) <= 1024)", max_ctx);
   AttnArgs a;
   a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (const DecodeState*)state;
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
-  attn_split_kernel<<<dim3(n_kv_heads, a.nsplit), 256, 0, (hipStream_t)stream>>>(a);
-  TGA_LAUNCH_CHECK();
-  attn_combine_kernel<<<n_heads, 256, 0, (hipStream_t)stream>>>(partials, a.st, n_heads, head_dim, a.nsplit, (_Float16*)out_f16, out_f32);
+  a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
+  const dim3 grid(n_kv_heads, a.nsplit);
+  hipStream_t s = (hipStream_t)stream;
+  if (head_dim == 64) attn_decode_kernel<8><<<grid, 256, 0, s>>>(a);
+  else if (head_dim == 128) attn_decode_kernel<16><<<grid, 256, 0, s>>>(a);
+  else attn_decode_kernel<32><<<grid, 256, 0, s>>>(a);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -104,7 +104,7 @@ class _Shared:
     self.xn = Buffer((1, c.dim), f16)
     self.q, self.k, self.v = Buffer((1, c.n_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32)
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
-    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32)
+    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters
     self.act = Buffer((1, c.hidden_dim), f16)
     self.logits = Buffer((1, c.vocab_size), f32)
     self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)
