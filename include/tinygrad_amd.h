@@ -72,6 +72,21 @@ int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const
                       const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                       int epilogue, const void* const* resid, void* stream);
 
+/* ExpertWeights.__call__ (tinygrad/llm/model.py:21-27) over a stacked (n_experts, N, K) weight kept in GGUF blocks: for job j
+ * (one (token, slot) pair) y[j, :] = x[j / jobs_per_x_row, :] @ W[sel[j]]^T; only the selected experts' bytes are read.
+ * With w_up != NULL the output is silu(x Wgate[e]^T) * (x Wup[e]^T) (model.py:129), w being the gate stack.
+ * sel: n_jobs int32 expert ids in device memory.  x: (ceil(n_jobs / jobs_per_x_row), K); y: (n_jobs, N). */
+int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* sel, int n_jobs,
+                        int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
+
+/* Expert gating of FFNBlock._feed_forward (model.py:112-128): scores by ExpertGating (1 SOFTMAX, 2 SIGMOID, 3 SOFTMAX_WEIGHT,
+ * 4 SQRT_SOFTPLUS; model.py:9-13), pairwise_topk selection (model.py:35-41: ascending, lower index wins ties), probabilities
+ * gathered / renormalised / scaled.  logits (n_tokens, n_experts) float32 -> sel (n_tokens, k) int32, probs (n_tokens, k). */
+int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int gating, int norm_topk_prob, float scale,
+                 int32_t* sel, float* probs, void* stream);
+/* out[t] = resid[t] + sum_s probs[t, s] * y[t, s, :]  (model.py:130 and the residual add :150); resid may be NULL or alias out. */
+int tga_moe_combine(const float* y, const float* probs, const float* resid, int n_tokens, int k, int dim, float* out, void* stream);
+
 /* ---- decode-step neighbours of the linears (batch 1), tinygrad/llm/model.py:144-204, 358-364 ----
  * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, pad[12]} so that one captured launch sequence serves
  * every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484). */
@@ -100,7 +115,8 @@ int tga_advance_prompt(void* state, const int* prompt, void* stream);
 
 /* ---- synthetic-model writer (no counterpart in the reference, whose weights always come from GGUF files): fills `out` with
  * n_elements random-init weights U(-amp, amp) (nn.Linear's init range, tinygrad/nn/__init__.py:173-174) already quantized to
- * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule); TGA_F32 fills the constant `amp`. */
+ * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule; TGA_F16: plain fp16 cast); TGA_F32 fills the
+ * constant `amp`; TGA_MXFP4 ignores amp: uniform E2M1 codes with E8M0 bytes uniform in [119, 123] (block scales 2^-8 .. 2^-4). */
 int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, uint32_t seed, float amp, void* stream);
 
 #ifdef __cplusplus

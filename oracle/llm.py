@@ -6,7 +6,7 @@ tinygrad/mixin/elementwise.py:682-690; argmax tinygrad/mixin/op.py:866-891 (firs
 Weights are the float32 dequantization of the same GGUF bytes, cast to fp16 like model.py:376 (w_round_f16) - the model path.
 kv_dtype: the reference's cache is float32 by default (model.py:202); BASELINE config 3 asks for fp16, which is what the build runs."""
 import numpy as np
-from oracle import ggml
+from oracle import ggml, moe as omoe
 
 def precompute_freqs_cis(dim, end, theta):
   freqs = (np.float32(1.0) / (np.float32(theta) ** (np.arange(0, dim, 2, dtype=np.float32)[:dim // 2] / np.float32(dim)))).astype(np.float32)
@@ -32,8 +32,8 @@ class Model:
     each linear to fp16 (what the GPU build does) - used only to separate that known deviation from real discrepancies."""
     self.c, self.max_context, self.kv_dtype, self.act16 = cfg, max_context, kv_dtype, act_round_f16
     def deq(name):
-      raw, t, (r, k) = tensors[name]
-      w = ggml.ggml_data_to_tensor(raw, r * k, t).reshape(r, k)
+      raw, t, shp = tensors[name]
+      w = ggml.ggml_data_to_tensor(raw, int(np.prod(shp)), t).reshape(shp)
       return w.astype(np.float16).astype(np.float32) if (w_round_f16 and t not in (0,)) else w.astype(np.float32)
     self.w = {name: deq(name) for name in tensors}
     if "output.weight" not in self.w: self.w["output.weight"] = self.w["token_embd.weight"]
@@ -54,8 +54,10 @@ class Model:
     for i in range(c["num_blocks"]):
       p = f"blk.{i}."
       n = rmsnorm(x, self.w[p + "attn_norm.weight"].reshape(-1), eps)
-      q = apply_rope(self._lin(p + "attn_q.weight", n).reshape(H, hd), self.fc[pos])
-      k = apply_rope(self._lin(p + "attn_k.weight", n).reshape(KV, hd), self.fc[pos])
+      q, k = self._lin(p + "attn_q.weight", n), self._lin(p + "attn_k.weight", n)
+      if c.get("qk_norm", 0) and c["qk_norm"] != hd:                        # model.py:169: full-width q/k norm before the head split
+        q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
+      q, k = apply_rope(q.reshape(H, hd), self.fc[pos]), apply_rope(k.reshape(KV, hd), self.fc[pos])
       v = self._lin(p + "attn_v.weight", n).reshape(KV, hd)
       self.ck[i, :, pos], self.cv[i, :, pos] = k.astype(self.kv_dtype), v.astype(self.kv_dtype)
       K = np.repeat(self.ck[i, :, :pos + 1].astype(np.float32), H // KV, axis=0)      # (H, T, hd)  GQA repeat_interleave
@@ -65,7 +67,23 @@ class Model:
       attn = np.einsum("ht,htd->hd", pr, V).astype(np.float32).reshape(-1)
       h = x + self._lin(p + "attn_output.weight", attn)
       n2 = rmsnorm(h, self.w[p + "ffn_norm.weight"].reshape(-1), eps)
-      x = h + self._lin(p + "ffn_down.weight", silu(self._lin(p + "ffn_gate.weight", n2)) * self._lin(p + "ffn_up.weight", n2))
+      if c.get("num_experts", 0):                                           # model.py:110-135
+        kx = c["num_experts_per_tok"]
+        logits = self._lin(p + "ffn_gate_inp.weight", n2)
+        sel, probs = omoe.gate_probs(logits[None, :], kx, c.get("expert_gating_func", 1), c.get("norm_topk_prob", False), c.get("routed_scaling_factor", 1.0))
+        n2l = n2.astype(np.float16).astype(np.float32) if self.act16 else n2
+        acc = np.zeros_like(x, dtype=np.float64)
+        for sl in range(kx):
+          e = int(sel[0, sl])
+          g = (n2l.astype(np.float64) @ self.w[p + "ffn_gate_exps.weight"][e].astype(np.float64).T).astype(np.float32)
+          u = (n2l.astype(np.float64) @ self.w[p + "ffn_up_exps.weight"][e].astype(np.float64).T).astype(np.float32)
+          a = silu(g) * u
+          if self.act16: a = a.astype(np.float16).astype(np.float32)
+          acc += np.float64(probs[0, sl]) * (a.astype(np.float64) @ self.w[p + "ffn_down_exps.weight"][e].astype(np.float64).T).astype(np.float32)
+        x = h + acc.astype(np.float32)
+        self.last_sel = sel[0]
+      else:
+        x = h + self._lin(p + "ffn_down.weight", silu(self._lin(p + "ffn_gate.weight", n2)) * self._lin(p + "ffn_up.weight", n2))
     return self._lin("output.weight", rmsnorm(x, self.w["output_norm.weight"].reshape(-1), eps))
 
   def generate(self, tokens, max_new):

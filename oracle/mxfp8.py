@@ -1,0 +1,85 @@
+"""numpy restatement of the MXFP8 operand format of the MoE grouped GEMM.  Test infrastructure only.
+
+quantize_mxfp8 / mx_pack / _mx_block_scale: extra/gemm/cdna_asm_gemm.py:149-173 (test twin test/backend/test_asm_gemm.py:278-292).
+E4M3 conversion: tinygrad/dtype.py:237-260 (round-to-nearest-even, finite saturation to 448, no infinities, NaN = 0x7f/0xff)."""
+import numpy as np
+
+def float_to_e4m3(x: np.ndarray) -> np.ndarray:
+  """float -> E4M3 (fn) bits, RNE, saturating: |x| > 464 -> 448 (dtype.py:238-252: ovf_threshold 464, max_norm 0x7E)."""
+  x = np.asarray(x, dtype=np.float64)
+  sign = (np.signbit(x)).astype(np.uint8) << 7
+  a = np.abs(x)
+  nan = ~np.isfinite(x)
+  a = np.where(nan, 0.0, a)
+  with np.errstate(divide="ignore"):
+    e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+  e = np.clip(e, -6, 8)
+  quantum = np.exp2(e - 3)
+  q = np.rint(a / quantum) * quantum                      # RNE on the 3-bit mantissa grid (subnormal grid 2^-9 below 2^-6)
+  q = np.where(a > 464.0, 448.0, np.minimum(q, 480.0))
+  q = np.where(q > 448.0, 448.0, q)                        # (448, 464] rounds (ties-to-even) down to 448
+  with np.errstate(divide="ignore"):
+    e2 = np.floor(np.log2(np.where(q > 0, q, 1.0)))
+  sub = q < 2.0 ** -6
+  expf = np.where(sub, 0, e2 + 7).astype(np.int64)
+  mant = np.where(sub, q / 2.0 ** -9, (q / np.exp2(e2) - 1.0) * 8).astype(np.int64)
+  bits = (expf << 3 | mant).astype(np.uint8)
+  bits = np.where(q == 0, 0, bits).astype(np.uint8)
+  return np.where(nan, np.uint8(0x7f), bits) | sign
+
+def e4m3_to_float(b: np.ndarray) -> np.ndarray:
+  b = np.asarray(b, dtype=np.uint8)
+  s = np.where(b & 0x80, -1.0, 1.0)
+  e = ((b >> 3) & 0xF).astype(np.int64); m = (b & 7).astype(np.float64)
+  v = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e - 7.0))
+  v = np.where((b & 0x7f) == 0x7f, np.nan, v)
+  return (s * v).astype(np.float32)
+
+def quantize_mxfp8(x: np.ndarray):
+  """cdna_asm_gemm.py:149-159: per 32 block along the last axis, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254),
+  q = e4m3(clamp(x * 2^(127 - e8), +-448)).  Returns (q bits uint8 (.., K), e8 uint8 (.., K/32))."""
+  x = np.asarray(x, dtype=np.float32)
+  *batch, K = x.shape
+  xb = x.reshape(*batch, K // 32, 32)
+  amax = np.abs(xb).max(axis=-1)
+  e8 = np.clip(np.floor(np.log2(np.maximum(amax, np.float32(1e-38)).astype(np.float32))) + 127, 0, 254).astype(np.uint8)
+  qscale = np.exp2(127.0 - e8.astype(np.float32)).astype(np.float32)[..., None]
+  xs = np.clip(xb * qscale, -448.0, 448.0)
+  return float_to_e4m3(xs).reshape(*batch, K), e8
+
+def block_scale(e8: np.ndarray) -> np.ndarray:
+  """cdna_asm_gemm.py:165-173: dequant scale 2^(e8-127) broadcast to element shape."""
+  return np.repeat(np.exp2(e8.astype(np.float32) - 127.0).astype(np.float32), 32, axis=-1)
+
+def dequant_mxfp8(q: np.ndarray, e8: np.ndarray) -> np.ndarray:
+  return e4m3_to_float(q) * block_scale(e8)
+
+def mx_pack(e8: np.ndarray) -> np.ndarray:
+  """cdna_asm_gemm.py:161-163: (rows, K/32) u8 -> (K/128, rows) u32, 4 consecutive block scales little-endian, transposed."""
+  rows, sk = e8.shape
+  return np.ascontiguousarray(np.ascontiguousarray(e8).reshape(rows, sk // 4, 4).view(np.uint32).reshape(rows, sk // 4).T)
+
+def mx_pack_3d(e8: np.ndarray) -> np.ndarray:
+  """extra/gemm/moe_gemm.py:87-89: (E, rows, K/32) -> (E, K/128, rows) u32."""
+  return np.stack([mx_pack(e) for e in e8])
+
+def to_bf16(x: np.ndarray) -> np.ndarray:
+  """float32 -> bfloat16 (RNE) kept as float32 values (tinygrad/dtype.py:224-226)."""
+  u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+  u = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+  return u.view(np.float32)
+
+def grouped_mx_gemm_ref(x_q, x_e8, w_q, w_e8, expert_off):
+  """Semantic definition of grouped_mx_gemm (extra/gemm/moe_gemm.py:112-134) through the reference's non-grouped fallback
+  matmul_mx (examples/mlperf/models/gpt_oss.py:64-83): bf16(dequant x) @ bf16(dequant w[e])^T accumulated in float, stored as
+  bf16, where rows [off[e], off[e+1]) belong to expert e.  Returned as float32 holding bf16 values; rows outside any expert's
+  range stay 0 here (the kernel's result there is unspecified padding)."""
+  xd = to_bf16(dequant_mxfp8(x_q, x_e8)).astype(np.float64)
+  M, N = x_q.shape[0], w_q.shape[1]
+  out = np.zeros((M, N), dtype=np.float32)
+  for e in range(w_q.shape[0]):
+    lo, hi = int(expert_off[e]), int(expert_off[e + 1])
+    if hi > lo:
+      wd = to_bf16(dequant_mxfp8(w_q[e], w_e8[e])).astype(np.float64)
+      out[lo:hi] = to_bf16((xd[lo:hi] @ wd.T).astype(np.float32))
+  return out

@@ -1,0 +1,93 @@
+"""MoE decode pieces on the GPU vs the oracle: expert gating/top-k (reference vectors test/unit/test_attention.py:249-270),
+MXFP4 expert GEMVs with expert indirection (ExpertWeights, tinygrad/llm/model.py:21-27), the reference's MoE closed form
+(test/unit/test_llm_moe.py:15-34) and a small OLMoE-architecture greedy decode."""
+import numpy as np, pytest
+from oracle import ggml as og, linear as ol, moe as omoe, llm as ollm
+from tinygrad_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+def _gate(gpu, logits, k, gating=1, norm=False, scale=1.0):
+  from tinygrad_amd.nn import moe_gate
+  T, E = logits.shape
+  lb = gpu.Buffer.from_numpy(logits.astype(np.float32)); sel = gpu.Buffer((T, k), np.int32); pr = gpu.Buffer((T, k), np.float32)
+  moe_gate(lb, T, E, k, sel, pr, gating, norm, scale)
+  return sel.numpy(), pr.numpy()
+
+def test_pairwise_topk_reference_vectors(gpu):
+  sel, p = _gate(gpu, np.array([[1.0, 3.0, 2.0, 5.0, 4.0]]), 3, gating=3)          # SOFTMAX_WEIGHT: scores are the logits themselves
+  assert sel.tolist() == [[1, 4, 3]]
+  np.testing.assert_allclose(p[0], omoe.softmax(np.array([3.0, 4.0, 5.0])), rtol=1e-6)
+  sel, _ = _gate(gpu, np.array([[5.0, 5.0, 3.0, 5.0]]), 2, gating=3)               # duplicates: the lower index ranks higher, output ascending
+  assert sel.tolist() == [[1, 0]]
+
+@pytest.mark.parametrize("gating", [1, 2, 3, 4])
+@pytest.mark.parametrize("norm", [False, True])
+def test_gating_modes_vs_oracle(gpu, gating, norm):
+  rng = np.random.default_rng(10 * gating + norm)
+  lg = rng.standard_normal((7, 64)).astype(np.float32) * 2
+  lg[3, 10] = lg[3, 20] = lg[3].max() + 1                                          # an exact tie among the selected
+  sel, p = _gate(gpu, lg, 8, gating, norm, 2.5)
+  rs, rp = omoe.gate_probs(lg, 8, gating, norm, 2.5)
+  np.testing.assert_array_equal(sel, rs)
+  np.testing.assert_allclose(p, rp, rtol=2e-5, atol=1e-7)
+
+@pytest.mark.parametrize("t,kdim,n", [(39, 2048, 1024), (39, 1024, 2048), (2, 512, 256), (8, 256, 192), (14, 512, 96)])
+def test_expert_gemv_with_indirection(gpu, t, kdim, n):
+  from tinygrad_amd.nn import ExpertWeights
+  rng = np.random.default_rng(n + t)
+  E, T, k = 6, 3, 4
+  w = synth.random_blocks(rng, t, E * n, kdim)
+  wu = synth.random_blocks(rng, t, E * n, kdim)
+  W, WU = ol.weight_f32(w, E * n, kdim, t).reshape(E, n, kdim), ol.weight_f32(wu, E * n, kdim, t).reshape(E, n, kdim)
+  x = synth.activations(rng, T, kdim, np.float16)
+  sel = rng.integers(0, E, size=(T, k)).astype(np.int32)
+  ew, eu = ExpertWeights(gpu.Buffer.from_numpy(w), t, E, n, kdim), ExpertWeights(gpu.Buffer.from_numpy(wu), t, E, n, kdim)
+  selb, xb = gpu.Buffer.from_numpy(sel), gpu.Buffer.from_numpy(x)
+  y = gpu.Buffer((T * k, n), np.float32)
+  ew(selb, xb, y, jobs_per_x_row=k)
+  ref = np.stack([ol.linear_f64(x[j // k][None].astype(np.float32), W[sel.reshape(-1)[j]])[0] for j in range(T * k)])
+  assert ol.rel_err(y.numpy(), ref) <= 1e-3
+  # SwiGLU pair: silu(gate_e x) * (up_e x)
+  ew(selb, xb, y, jobs_per_x_row=k, up=eu)
+  refu = np.stack([ol.linear_f64(x[j // k][None].astype(np.float32), WU[sel.reshape(-1)[j]])[0] for j in range(T * k)])
+  assert ol.rel_err(y.numpy(), ref / (1 + np.exp(-ref)) * refu) <= 1e-3
+  # one activation row per job (the down projection's case)
+  xj = synth.activations(rng, T * k, kdim, np.float16)
+  ew(selb, gpu.Buffer.from_numpy(xj), y, jobs_per_x_row=1)
+  refj = np.stack([ol.linear_f64(xj[j][None].astype(np.float32), W[sel.reshape(-1)[j]])[0] for j in range(T * k)])
+  assert ol.rel_err(y.numpy(), refj) <= 1e-3
+
+def test_moe_combine(gpu):
+  from tinygrad_amd.nn import moe_combine
+  rng = np.random.default_rng(3)
+  T, k, D = 3, 8, 2048
+  y, p, r = rng.standard_normal((T, k, D)).astype(np.float32), rng.random((T, k)).astype(np.float32), rng.standard_normal((T, D)).astype(np.float32)
+  out = gpu.Buffer((T, D), np.float32)
+  moe_combine(gpu.Buffer.from_numpy(y), gpu.Buffer.from_numpy(p), gpu.Buffer.from_numpy(r), T, k, D, out)
+  np.testing.assert_allclose(out.numpy(), r + (y * p[:, :, None]).sum(1), rtol=1e-5, atol=1e-5)
+
+SMALL_MOE = dict(num_blocks=2, dim=256, hidden_dim=128, n_heads=4, n_kv_heads=4, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,
+                 qk_norm=256, num_experts=8, num_experts_per_tok=2, norm_topk_prob=False, expert_gating_func=1)
+
+def test_small_olmoe_decode(gpu):
+  """OLMoE-architecture (fp16 attention/router, MXFP4 experts, full-width qk norm) greedy decode vs the numpy restatement."""
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe
+  c = TransformerConfig(max_context=128, **SMALL_MOE)
+  sd = synth_state_moe(c, seed=1004)
+  gpu.synchronize()
+  host = {k: (b.numpy(), t, shp) for k, (b, t, shp) in sd.items()}
+  model = Transformer(c, sd, max_new=64)
+  rng = np.random.default_rng(1004)
+  prompt = [int(t) for t in rng.integers(0, 512, size=20)]
+  got = list(model.generate(prompt, 16))
+  lg_gpu = model.logits()
+  o = ollm.Model(SMALL_MOE, host, 128, act_round_f16=True)
+  ref, margins = o.generate(prompt, 16)
+  print(f"oracle min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(SMALL_MOE, host, 128, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(16): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(lg_gpu, lg) <= 1e-3

@@ -18,6 +18,9 @@ struct QArgs {
   int nseg, x_f32, y_f32, epilogue;
   int K, nu;            // units per row
   int chunk_u, nchunks; // units per LDS chunk
+  // job indirection (MoE expert GEMVs): blockIdx.y = job; expert = sel[job]; weights shifted by expert * estride bytes;
+  // activation row = job / xdiv; outputs shifted by job * ystride elements.  sel == nullptr: a single job.
+  const int* sel; long long estride, ystride; int xdiv, xdiv_jobs;   // xdiv_jobs: number of jobs (grid.y)
 };
 
 __device__ __forceinline__ uint32_t pack_even(uint32_t a, uint32_t b) { return (a & 0xFFFFu) | (b << 16); }        // (a.lo, b.lo)
@@ -214,6 +217,36 @@ template <> struct Fmt<F_Q8_0P> {
   }
 };
 
+
+// ------------------------------------------------------------------------------------------------ F16 (dense fp16 rows, gguf.py:35-36)
+// unit = 64 consecutive fp16 weights (128 bytes); no decode: the weight dwords are the fp16 pairs.
+template <> struct Fmt<GGML_F16> {
+  static constexpr int UW = 64, UPB = 1, BW = 64, BB = 128;
+  static __device__ __forceinline__ int unit_of(int e) { return e / UW; }
+  static __device__ __forceinline__ int pair_of(int e) { return (e % UW) >> 1; }
+  static constexpr int XV = 8, NG = 1, NWV = 32;
+  struct Raw { u32x4 q[8]; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* p = row + 128 * u; Raw r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.q[i] = ld16_a4(p + 16 * i);
+    return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 1;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = 0; }
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t*) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) { wv[4 * i] = r.q[i].x; wv[4 * i + 1] = r.q[i].y; wv[4 * i + 2] = r.q[i].z; wv[4 * i + 3] = r.q[i].w; }
+  }
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+#pragma unroll
+    for (int v = 0; v < 8; v++) { xv[v].x = nx[4 * v]; xv[v].y = nx[4 * v + 1]; xv[v].z = nx[4 * v + 2]; xv[v].w = nx[4 * v + 3]; }
+    c[0] = 0.f;
+  }
+  static __device__ __forceinline__ float finish(const Raw&, const float* a) { return a[0]; }
+};
+
 // ------------------------------------------------------------------------------------------------ MXFP4 (gguf.py:105-114)
 template <> struct Fmt<GGML_MXFP4> {
   static constexpr int UW = 32, UPB = 1, BW = 32, BB = 17;
@@ -348,12 +381,12 @@ __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, co
 
 // M = 1 stores.  EPI 0: plain, EPI 1: + residual, EPI 2: silu(gate) * up into output row `row` of segment 0.
 template <int EPI>
-__device__ __forceinline__ void store_one(const QArgs& a, int seg, long long row, float v) {
-  if constexpr (EPI == 1) v += a.resid[seg][row];
-  if (a.y_f32) ((float*)a.y[seg])[row] = v; else ((_Float16*)a.y[seg])[row] = (_Float16)v;
+__device__ __forceinline__ void store_one(const QArgs& a, int seg, long long row, float v, long long yofs = 0) {
+  if constexpr (EPI == 1) v += a.resid[seg][yofs + row];
+  if (a.y_f32) ((float*)a.y[seg])[yofs + row] = v; else ((_Float16*)a.y[seg])[yofs + row] = (_Float16)v;
 }
-__device__ __forceinline__ void store_swiglu(const QArgs& a, long long row, float gate, float up) {
+__device__ __forceinline__ void store_swiglu(const QArgs& a, long long row, float gate, float up, long long yofs = 0) {
   const float o = silu_f(gate) * up;
-  if (a.y_f32) ((float*)a.y[0])[row] = o; else ((_Float16*)a.y[0])[row] = (_Float16)o;
+  if (a.y_f32) ((float*)a.y[0])[yofs + row] = o; else ((_Float16*)a.y[0])[yofs + row] = (_Float16)o;
 }
 

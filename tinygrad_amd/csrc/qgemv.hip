@@ -316,8 +316,9 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
   TGA_REQUIRE(epilogue != 1 || (y_dtype == TGA_F32 && resid), "tga_qlinear: the residual epilogue needs float32 y and resid pointers");
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: bw = 256; break;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: bw = 256; break; case GGML_F16: bw = 64; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
+  TGA_REQUIRE(ggml_type != GGML_F16 || M == 1, "tga_qlinear: dense fp16 weights are served for M = 1 only");
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
   TGA_REQUIRE(x, "tga_qlinear: null x");
   QArgs a = {};
@@ -345,11 +346,37 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     case GGML_Q6_K: return launch_qgemv_m<GGML_Q6_K>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
   }
-  return 1;
+  return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
 }
 
 extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                            int M, int64_t N, int64_t K, void* stream) {
   const void* ws[1] = {w}; void* ys[1] = {y}; int64_t ns[1] = {N};
   return tga_qlinear_multi(ggml_type, 1, ws, ys, ns, x, x_dtype, y_dtype, M, K, 0, nullptr, stream);
+}
+
+// ExpertWeights.__call__ (tinygrad/llm/model.py:21-27): per (token, slot) job j, y[j] = x[j / jobs_per_x_row] @ W[sel[j]]^T over a
+// stacked (n_experts, N, K) weight; with w_up the output is silu(x Wgate[e]^T) * (x Wup[e]^T) (model.py:129).  Only the
+// selected experts' bytes are read (the indexed load the reference's codegen produces from weight[sel]).
+extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* sel, int n_jobs,
+                                   int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
+  TGA_REQUIRE(w && sel && x && y, "tga_qlinear_experts: null pointer");
+  TGA_REQUIRE(n_jobs >= 1 && n_jobs <= 65535 && jobs_per_x_row >= 1 && n_experts >= 1, "tga_qlinear_experts: bad job geometry");
+  TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32, "tga_qlinear_experts: x_dtype must be TGA_F16 or TGA_F32");
+  TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear_experts: y_dtype must be TGA_F16 or TGA_F32");
+  int bw, bb;
+  switch (ggml_type) { case GGML_Q4_0: bw = 32; bb = 18; break; case GGML_Q8_0: bw = 32; bb = 34; break; case GGML_MXFP4: bw = 32; bb = 17; break;
+    case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_F16: bw = 64; bb = 128; break;
+    default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
+  TGA_REQUIRE(K > 0 && K % bw == 0 && N > 0, "tga_qlinear_experts: K=%lld must be a positive multiple of %d", (long long)K, bw);
+  QArgs a = {};
+  a.nseg = w_up ? 2 : 1; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = w_up ? 2 : 0; a.K = (int)K;
+  a.w[0] = (const uint8_t*)w; a.w[1] = (const uint8_t*)w_up; a.y[0] = y; a.n[0] = N; a.n[1] = N; a.ntot = N;
+  a.sel = sel; a.estride = (long long)N * (K / bw) * bb; a.ystride = N; a.xdiv = jobs_per_x_row; a.xdiv_jobs = n_jobs;
+  const bool pair = (K / 32) % 2 == 0 && ((uintptr_t)w & 3) == 0 && (!w_up || ((uintptr_t)w_up & 3) == 0) && a.estride % 4 == 0;
+  const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+  TGA_REQUIRE(fmt >= 0, "tga_qlinear_experts: Q4_0/Q8_0 expert weights need K %% 64 == 0 and 4-byte aligned experts");
+  const int rc = tga_qgemv1_dispatch(fmt, a, (hipStream_t)stream);
+  TGA_REQUIRE(rc >= 0, "tga_qlinear_experts: shape K=%lld outside the expert GEMV path", (long long)K);
+  return rc;
 }

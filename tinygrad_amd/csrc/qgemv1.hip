@@ -24,6 +24,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
   const int wk = (WK > 1) ? wave : 0, wr = (WK > 1) ? 0 : wave;
   const int u = wk * 64 + lane;
   const bool uvalid = u < a.nu;
+  const int job = blockIdx.y;
+  const long long eoff = a.sel ? (long long)a.sel[job] * a.estride : 0, yofs = (long long)job * a.ystride;
+  const long long xrow = a.sel ? job / a.xdiv : 0;
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
   const long long ngroups = (a.ntot + RS - 1) / RS;
   const long long nteams = (long long)gridDim.x * WR, team = (long long)blockIdx.x * WR + wr;
@@ -44,8 +47,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
     if (hi > seg_rows) hi = seg_rows;
     seg_start += seg_rows;
     const long long cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;   // row groups of this team inside the segment
-    const uint8_t* base0 = a.w[seg];
-    const uint8_t* base1 = (EPI == 2) ? a.w[1] : a.w[seg];
+    const uint8_t* base0 = a.w[seg] + eoff;
+    const uint8_t* base1 = ((EPI == 2) ? a.w[1] : a.w[seg]) + eoff;
     auto issue = [&](Raw* buf, long long row) {
       if (uvalid) {
 #pragma unroll
@@ -78,18 +81,18 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
           }
           if constexpr (EPI == 2) {
             const float up = __shfl(t, 1, 64);
-            if (lane == 0) store_swiglu(a, row, t, up);
+            if (lane == 0) store_swiglu(a, row, t, up, yofs);
           } else {
-            if (lane < R && row + lane < hi) store_one<EPI>(a, seg, row + lane, t);
+            if (lane < R && row + lane < hi) store_one<EPI>(a, seg, row + lane, t, yofs);
           }
         }
         parity ^= 1;
       } else {
         if (lane == 63) {
-          if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1]);
+          if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1], yofs);
           else {
 #pragma unroll
-            for (int r = 0; r < R; r++) if (row + r < hi) store_one<EPI>(a, seg, row + r, acc[r]);
+            for (int r = 0; r < R; r++) if (row + r < hi) store_one<EPI>(a, seg, row + r, acc[r], yofs);
           }
         }
       }
@@ -102,10 +105,11 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
       for (int i = threadIdx.x; i < nq; i += NT) {
         u32x4 v;
         if (a.x_f32) {
-          const f32x4 lo4 = ((const f32x4*)a.x)[2 * i], hi4 = ((const f32x4*)a.x)[2 * i + 1];
+          const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
+          const f32x4 lo4 = xr[2 * i], hi4 = xr[2 * i + 1];
           v.x = f2h_bits(lo4.x) | (f2h_bits(lo4.y) << 16); v.y = f2h_bits(lo4.z) | (f2h_bits(lo4.w) << 16);
           v.z = f2h_bits(hi4.x) | (f2h_bits(hi4.y) << 16); v.w = f2h_bits(hi4.z) | (f2h_bits(hi4.w) << 16);
-        } else v = ((const u32x4*)a.x)[i];
+        } else v = ((const u32x4*)((const uint16_t*)a.x + xrow * a.K))[i];
         // element 8i lives in unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
         *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
       }
@@ -148,7 +152,8 @@ static int launch_fast(QArgs a, hipStream_t s) {
   // resident row teams per CU: 16 waves (<= 128 VGPRs) unless the staged activations in LDS (160 KB per CU) allow fewer
   int wg_per_cu = 16 / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;
   const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
-  const long long max_teams = (long long)fast_cu_count() * wg_per_cu * WR;
+  long long max_teams = (long long)fast_cu_count() * wg_per_cu * WR;
+  if (a.sel && a.xdiv_jobs > 1) { max_teams = (max_teams + a.xdiv_jobs - 1) / a.xdiv_jobs; if (max_teams < 1) max_teams = 1; }
   const long long per = (ngroups + max_teams - 1) / max_teams;     // row groups per team
   const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
   long long grid = (teams + WR - 1) / WR;
@@ -158,7 +163,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
     static bool configured = false;
     if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); configured = true; }
   }
-  kern<<<dim3((unsigned)grid), dim3(WK * WR * 64), lds, s>>>(a);
+  kern<<<dim3((unsigned)grid, (unsigned)(a.sel ? a.xdiv_jobs : 1)), dim3(WK * WR * 64), lds, s>>>(a);
   TGA_LAUNCH_CHECK();
   return 0;
 }
@@ -189,6 +194,7 @@ static int launch_fast_w(QArgs a, hipStream_t s) {
 // Returns -1 when the shape is outside the fast path (caller falls back to the LDS-staged kernel).
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
   const int uw = (fmt == GGML_MXFP4) ? 32 : 64;
+  if (fmt == GGML_F16 && a.K % 64) return -1;
   if ((a.K / uw + 63) / 64 > 16 || a.K % 8) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;                       // coalesced 16-byte activation loads
   switch (fmt) {
@@ -196,6 +202,7 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
     case F_Q8_0P: return launch_fast_w<F_Q8_0P>(a, s);
     case GGML_Q6_K: return launch_fast_w<GGML_Q6_K>(a, s);
     case GGML_MXFP4: return launch_fast_w<GGML_MXFP4>(a, s);
+    case GGML_F16: return launch_fast_w<GGML_F16>(a, s);
   }
   return -1;
 }

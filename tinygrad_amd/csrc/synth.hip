@@ -62,6 +62,23 @@ __global__ __launch_bounds__(256) void synth_q6_k_kernel(uint8_t* __restrict__ o
   }
 }
 
+__global__ __launch_bounds__(256) void synth_f16_kernel(_Float16* __restrict__ out, int64_t n, uint32_t seed, float amp) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) out[i] = (_Float16)rnd_uniform(seed, (uint64_t)i, amp);
+}
+// MXFP4 blocks: E2M1 nibbles uniform in 0..15, E8M0 byte uniform in [127 + lo, 127 + hi] (effective block scale 2^lo..2^hi on
+// the true E2M1 values; under the reference's decode that is 2^(e-128) times the doubled table: the same number)
+__global__ __launch_bounds__(256) void synth_mxfp4_kernel(uint8_t* __restrict__ out, int64_t nblocks, uint32_t seed, int lo, int hi) {
+  for (int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x; b < nblocks; b += (int64_t)gridDim.x * 256) {
+    uint8_t* o = out + b * 17;
+    const uint32_t h = fmix32((uint32_t)b * 0x9E3779B1u + fmix32(seed ^ (uint32_t)(b >> 32) ^ 0x5bd1e995u));
+    o[0] = (uint8_t)(127 + lo + (int)(h % (uint32_t)(hi - lo + 1)));
+    for (int j = 0; j < 4; j++) {
+      const uint32_t r = fmix32(h + 0x9E3779B9u * (j + 1));
+      o[1 + 4 * j] = r & 0xFF; o[2 + 4 * j] = (r >> 8) & 0xFF; o[3 + 4 * j] = (r >> 16) & 0xFF; o[4 + 4 * j] = r >> 24;
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ out, int64_t n, float value) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) out[i] = value;
 }
@@ -78,6 +95,13 @@ extern "C" int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, u
     TGA_REQUIRE(n_elements % 256 == 0, "tga_synth_weights: Q6_K needs a multiple of 256 elements");
     const int64_t nb = n_elements / 256; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
     synth_q6_k_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, amp);
+  } else if (ggml_type == GGML_F16) {
+    const int grid = (int)((n_elements + 255) / 256 < 65536 ? (n_elements + 255) / 256 : 65536);
+    synth_f16_kernel<<<grid, 256, 0, s>>>((_Float16*)out, n_elements, seed, amp);
+  } else if (ggml_type == GGML_MXFP4) {
+    TGA_REQUIRE(n_elements % 32 == 0, "tga_synth_weights: MXFP4 needs a multiple of 32 elements");
+    const int64_t nb = n_elements / 32; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
+    synth_mxfp4_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, -8, -4);   // amp unused: exponents ~ U[-8, -4] (BASELINE config 4)
   } else if (ggml_type == GGML_F32) {
     const int grid = (int)((n_elements + 255) / 256 < 65536 ? (n_elements + 255) / 256 : 65536);
     fill_f32_kernel<<<grid, 256, 0, s>>>((float*)out, n_elements, amp);   // constant fill (norm weights = 1)

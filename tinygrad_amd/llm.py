@@ -13,7 +13,7 @@ from dataclasses import dataclass
 import numpy as np
 from tinygrad_amd import runtime as rt
 from tinygrad_amd.runtime import Buffer, GGML_QUANT
-from tinygrad_amd.nn import QuantLinear, qlinear_multi
+from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine
 
 @dataclass(frozen=True)
 class TransformerConfig:
@@ -28,9 +28,19 @@ class TransformerConfig:
   head_dim: int
   rope_theta: float
   max_context: int
+  qk_norm: int = 0                 # width of attn_q_norm / attn_k_norm (OLMoE: the full projection width, model.py:169)
+  num_experts: int = 0
+  num_experts_per_tok: int = 0
+  norm_topk_prob: bool = False
+  expert_gating_func: int = 1      # ExpertGating.SOFTMAX (model.py:9-13)
+  routed_scaling_factor: float = 1.0
 
 LLAMA3_8B = dict(num_blocks=32, dim=4096, hidden_dim=14336, n_heads=32, n_kv_heads=8, norm_eps=1e-5, vocab_size=128256,
                  head_dim=128, rope_theta=500000.0)
+
+# OLMoE architecture of BASELINE config 4 (hidden_dim is the expert FFN width, as expert_feed_forward_length maps in model.py:422)
+OLMOE = dict(num_blocks=16, dim=2048, hidden_dim=1024, n_heads=16, n_kv_heads=16, norm_eps=1e-5, vocab_size=50304, head_dim=128,
+             rope_theta=10000.0, qk_norm=2048, num_experts=64, num_experts_per_tok=8, norm_topk_prob=False, expert_gating_func=1)
 
 def precompute_freqs_cis(dim: int, end: int, theta: float) -> np.ndarray:
   """tinygrad/llm/model.py:16-19 in float32: cat(cos(pos * f), sin(pos * f)), f = 1 / theta^(2i/dim)."""
@@ -43,6 +53,35 @@ def quant_nbytes(ggml_type: int, n: int) -> int:
   if ggml_type == rt.F16: return 2 * n
   nel, nby = GGML_QUANT[ggml_type]
   return n // nel * nby
+
+def synth_state_moe(config: TransformerConfig, seed: int = 1004, dense_type: int = rt.F16, expert_type: int = rt.MXFP4, stream=None) -> dict:
+  """OLMoE-architecture random model: fp16 attention / router / embedding / lm-head, MXFP4 expert stacks (E, out, in), norms 1."""
+  c, sd, tid = config, {}, [0]
+  def mk(name, shape, t, amp):
+    n = int(np.prod(shape))
+    buf = Buffer((quant_nbytes(t, n),), np.uint8)
+    tid[0] += 1
+    rt.check(rt.lib().tga_synth_weights(t, buf.ptr, n, (seed * 7919 + tid[0]) & 0xFFFFFFFF, amp, stream))
+    sd[name] = (buf, t, tuple(shape))
+  E, H, D = c.num_experts, c.hidden_dim, c.dim
+  mk("token_embd.weight", (c.vocab_size, D), dense_type, 1.0)
+  for i in range(c.num_blocks):
+    p = f"blk.{i}."
+    mk(p + "attn_norm.weight", (1, D), rt.F32, 1.0)
+    for nm, rows in (("attn_q", c.n_heads * c.head_dim), ("attn_k", c.n_kv_heads * c.head_dim), ("attn_v", c.n_kv_heads * c.head_dim)):
+      mk(p + nm + ".weight", (rows, D), dense_type, D ** -0.5)
+    mk(p + "attn_output.weight", (D, c.n_heads * c.head_dim), dense_type, (c.n_heads * c.head_dim) ** -0.5)
+    if c.qk_norm:
+      mk(p + "attn_q_norm.weight", (1, c.n_heads * c.head_dim), rt.F32, 1.0)
+      mk(p + "attn_k_norm.weight", (1, c.n_kv_heads * c.head_dim), rt.F32, 1.0)
+    mk(p + "ffn_norm.weight", (1, D), rt.F32, 1.0)
+    mk(p + "ffn_gate_inp.weight", (E, D), dense_type, D ** -0.5)
+    mk(p + "ffn_gate_exps.weight", (E, H, D), expert_type, D ** -0.5)
+    mk(p + "ffn_up_exps.weight", (E, H, D), expert_type, D ** -0.5)
+    mk(p + "ffn_down_exps.weight", (E, D, H), expert_type, H ** -0.5)
+  mk("output_norm.weight", (1, D), rt.F32, 1.0)
+  mk("output.weight", (c.vocab_size, D), dense_type, D ** -0.5)
+  return sd
 
 def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = rt.Q4_0, head_type: int = rt.Q6_K, stream=None) -> dict:
   """Random-init model written straight into HBM as GGUF blocks: {gguf tensor name: (Buffer, ggml_type, (rows, cols))}.
@@ -76,7 +115,15 @@ class TransformerBlock:
     lin = lambda name: QuantLinear(sd[p + name][0], sd[p + name][1], *sd[p + name][2])
     self.attn_norm, self.ffn_norm = sd[p + "attn_norm.weight"][0], sd[p + "ffn_norm.weight"][0]
     self.attn_q, self.attn_k, self.attn_v, self.attn_output = lin("attn_q.weight"), lin("attn_k.weight"), lin("attn_v.weight"), lin("attn_output.weight")
-    self.ffn_gate, self.ffn_up, self.ffn_down = lin("ffn_gate.weight"), lin("ffn_up.weight"), lin("ffn_down.weight")
+    self.moe = c.num_experts > 0
+    if self.moe:
+      ex = lambda name: ExpertWeights(sd[p + name][0], sd[p + name][1], *sd[p + name][2])
+      self.ffn_gate_inp = lin("ffn_gate_inp.weight")                      # router
+      self.ffn_gate_exps, self.ffn_up_exps, self.ffn_down_exps = ex("ffn_gate_exps.weight"), ex("ffn_up_exps.weight"), ex("ffn_down_exps.weight")
+    else:
+      self.ffn_gate, self.ffn_up, self.ffn_down = lin("ffn_gate.weight"), lin("ffn_up.weight"), lin("ffn_down.weight")
+    self.q_norm = sd[p + "attn_q_norm.weight"][0] if c.qk_norm else None
+    self.k_norm = sd[p + "attn_k_norm.weight"][0] if c.qk_norm else None
     # KV cache: fp16 [n_kv_heads][max_context][head_dim] each (reference: one [2,B,KvH,ctx,Hd] tensor, model.py:202)
     self.cache_k = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
@@ -87,13 +134,26 @@ class TransformerBlock:
     # h = x + attention(attn_norm(x))                                                     model.py:149
     rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
     qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream)
+    if c.qk_norm:                                                        # full-width q/k RMSNorm before the head split (model.py:169)
+      assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
+      rt.check(L.tga_rmsnorm(s.q.ptr, self.q_norm.ptr, c.n_heads * c.head_dim, c.norm_eps, None, s.q.ptr, stream))
+      rt.check(L.tga_rmsnorm(s.k.ptr, self.k_norm.ptr, c.n_kv_heads * c.head_dim, c.norm_eps, None, s.k.ptr, stream))
     rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
                                     c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, stream))
     qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
-    qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream)
-    qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream)
+    if not self.moe:
+      qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream)
+      qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream)
+      return
+    # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
+    k = c.num_experts_per_tok
+    self.ffn_gate_inp(s.xn, out=s.router, stream=stream)
+    moe_gate(s.router, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
+    self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
+    self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
+    moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)
 
 class _Shared:
   """Activation buffers shared by all blocks (batch 1)."""
@@ -106,6 +166,10 @@ class _Shared:
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
     self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters
     self.act = Buffer((1, c.hidden_dim), f16)
+    if c.num_experts:
+      k = c.num_experts_per_tok
+      self.router, self.sel, self.probs = Buffer((1, c.num_experts), f32), Buffer((k,), np.int32), Buffer((k,), f32)
+      self.act_e, self.y_e = Buffer((k, c.hidden_dim), f16), Buffer((k, c.dim), f32)
     self.logits = Buffer((1, c.vocab_size), f32)
     self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)
     self.rope = Buffer.from_numpy(precompute_freqs_cis(c.head_dim, c.max_context, c.rope_theta))
@@ -179,5 +243,8 @@ class Transformer:
   def weight_bytes_per_token(self) -> int:
     """Packed weight bytes one decode step streams (all block linears + lm-head), the reference's GB/s accounting (cli.py:179-181)."""
     n = self.output.nbytes
-    for b in self.blk: n += sum(l.nbytes for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down))
+    for b in self.blk:
+      n += sum(l.nbytes for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output))
+      if b.moe: n += b.ffn_gate_inp.nbytes + self.config.num_experts_per_tok * sum(e.expert_nbytes for e in (b.ffn_gate_exps, b.ffn_up_exps, b.ffn_down_exps))
+      else: n += sum(l.nbytes for l in (b.ffn_gate, b.ffn_up, b.ffn_down))
     return n

@@ -9,15 +9,15 @@ from tinygrad_amd.runtime import Buffer, GGML_QUANT
 
 class QuantLinear:
   def __init__(self, blocks: Buffer, ggml_type: int, out_features: int, in_features: int):
-    if ggml_type not in GGML_QUANT: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
-    nel, nby = GGML_QUANT[ggml_type]
+    if ggml_type != rt.F16 and ggml_type not in GGML_QUANT: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
+    nel, nby = GGML_QUANT.get(ggml_type, (64, 128))                     # dense fp16 rows go in 64-element units
     assert in_features % nel == 0, f"in_features {in_features} must be a multiple of the block size {nel}"
     assert blocks.nbytes >= out_features * (in_features // nel) * nby, "weight buffer too small"
     self.blocks, self.ggml_type, self.out_features, self.in_features = blocks, ggml_type, out_features, in_features
 
   @property
   def nbytes(self) -> int:
-    nel, nby = GGML_QUANT[self.ggml_type]
+    nel, nby = GGML_QUANT.get(self.ggml_type, (64, 128))
     return self.out_features * (self.in_features // nel) * nby
 
   def __call__(self, x: Buffer, out: Buffer | None = None, out_dtype=None, stream=None) -> Buffer:
@@ -46,3 +46,29 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   ydt = rt.dtype_code(outs[0].dtype)
   rt.check(rt.lib().tga_qlinear_multi(t, nseg, w, y, n, x.ptr, rt.dtype_code(x.dtype), ydt, m, k, epilogue, r, stream))
   return outs
+
+class ExpertWeights:
+  """Like QuantLinear but with a num_experts dimension: weight (num_experts, out_features, in_features) kept in GGUF blocks
+  (mirror of ExpertWeights, tinygrad/llm/model.py:21-27).  __call__(sel, x): sel (n_jobs,) int32 device buffer of expert ids,
+  x (n_jobs // jobs_per_x_row, in) -> (n_jobs, out)."""
+  def __init__(self, blocks: Buffer, ggml_type: int, num_experts: int, out_features: int, in_features: int):
+    if ggml_type != rt.F16 and ggml_type not in GGML_QUANT: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
+    self.blocks, self.ggml_type, self.num_experts, self.out_features, self.in_features = blocks, ggml_type, num_experts, out_features, in_features
+
+  @property
+  def expert_nbytes(self) -> int:
+    if self.ggml_type == rt.F16: return 2 * self.out_features * self.in_features
+    nel, nby = GGML_QUANT[self.ggml_type]
+    return self.out_features * (self.in_features // nel) * nby
+
+  def __call__(self, sel: Buffer, x: Buffer, out: Buffer, jobs_per_x_row: int = 1, up: "ExpertWeights | None" = None, stream=None) -> Buffer:
+    n_jobs = int(np.prod(sel.shape))
+    rt.check(rt.lib().tga_qlinear_experts(self.ggml_type, self.blocks.ptr, up.blocks.ptr if up is not None else None, self.num_experts, sel.ptr, n_jobs,
+                                          jobs_per_x_row, x.ptr, rt.dtype_code(x.dtype), out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
+    return out
+
+def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer, probs: Buffer, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
+  rt.check(rt.lib().tga_moe_gate(logits.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
+
+def moe_combine(y: Buffer, probs: Buffer, resid: Buffer | None, n_tokens: int, k: int, dim: int, out: Buffer, stream=None):
+  rt.check(rt.lib().tga_moe_combine(y.ptr, probs.ptr, resid.ptr if resid is not None else None, n_tokens, k, dim, out.ptr, stream))

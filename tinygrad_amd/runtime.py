@@ -29,6 +29,9 @@ def _declare(lib):
     "tga_dequant": [i, vp, i64, vp, i, vp],
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
     "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, vp],
+    "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
+    "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
+    "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
