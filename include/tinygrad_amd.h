@@ -113,6 +113,33 @@ int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i
 /* prompt step that skips the output projection: token = prompt[pos + 1], pos += 1. */
 int tga_advance_prompt(void* state, const int* prompt, void* stream);
 
+/* ---- MXFP8 MoE prefill path: extra/gemm/cdna_asm_gemm.py, extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py ---- */
+
+/* quantize_mxfp8 (cdna_asm_gemm.py:149-159): per 32 block along K, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254),
+ * q = E4M3(clamp(x * 2^(127 - e8), +-448)) (RNE, tinygrad/dtype.py:237-260).  x: (rows, K) bf16 (x_is_bf16) or float32.
+ * q: (rows, K) bytes; e8: (rows, K/32) bytes; packed (may be NULL): mx_pack layout (K/128, rows) uint32 (cdna_asm_gemm.py:161-163). */
+int tga_quantize_mxfp8(const void* x, int x_is_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream);
+
+/* route (moe_routing.py:109-122) for one device group: top-k (descending, lower index first among equals), weights =
+ * softmax(top values), per-expert counts padded to 256 -> off (E+1), dest_row[j] = off[e_j] + stable rank of assignment j among
+ * those of expert e_j in flattened (token, slot) order.  scratch: int32[n_tokens*k + ceil(n_tokens*k/1024)*n_experts]. */
+int tga_moe_route(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
+                  int32_t* counts, int32_t* scratch, void* stream);
+/* dispatch (moe_routing.py:124-126): xg[dest_row[j], :] = x[j / k, :] (bf16 rows); rows no assignment maps to are zero-filled. */
+int tga_moe_dispatch(const void* x_bf16, const int32_t* dest_row, const int32_t* off, const int32_t* counts, int n_tokens, int k, int n_experts,
+                     int64_t m_l, int D, void* xg_bf16, void* stream);
+/* combine (moe_routing.py:128-131): out[t] = sum_s bf16(weights[t,s]) * z[dest_row[t*k+s]] in bf16 products, float32 sum, bf16 out. */
+int tga_moe_combine_rows(const void* z_bf16, const int32_t* dest_row, const float* weights, int n_tokens, int k, int D, void* out_bf16, void* stream);
+
+/* grouped_mx_gemm's kernel (moe_gemm.py:31-48, 112-134), same operand list and order as the reference's custom kernel:
+ * C (M,N) bf16 = A (M,K) e4m3 . B[e(tile)] (E,N,K) e4m3 ^T with E8M0 1x32 scales x_e8 (M,K/32), w_e8 (E,N,K/32); e(tile) from
+ * expert_off (E+1) as Routing.rows_e (moe_routing.py:98-104).  x_si / w_si (the mx_pack copies) are accepted and unused.
+ * Requires M % 256 == 0, N % 256 == 0, K % 128 == 0 (moe_gemm.py:120).  Rows at or beyond expert_off[E] are left untouched. */
+int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
+                           const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
+/* clamped interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98), bf16 (rows, 2I) -> (rows, I). */
+int tga_swiglu_interleaved(const void* h_bf16, int64_t rows, int two_inter, float limit, float alpha, void* y_bf16, void* stream);
+
 /* ---- synthetic-model writer (no counterpart in the reference, whose weights always come from GGUF files): fills `out` with
  * n_elements random-init weights U(-amp, amp) (nn.Linear's init range, tinygrad/nn/__init__.py:173-174) already quantized to
  * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule; TGA_F16: plain fp16 cast); TGA_F32 fills the

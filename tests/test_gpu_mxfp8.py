@@ -1,0 +1,75 @@
+"""MXFP8 MoE prefill path on the GPU vs the oracle: quantize_mxfp8 bit-exact, route/dispatch/combine exact (integer / byte work),
+grouped GEMM within the reference's own error bars (test/backend/test_asm_gemm.py:310-313: mean-rel-err < 1e-2 vs dequant-matmul)."""
+import numpy as np, pytest
+from oracle import mxfp8 as omx, moe as omoe
+
+pytestmark = pytest.mark.gpu
+
+def test_quantize_mxfp8_bit_exact(gpu):
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(1)
+  x = (rng.standard_normal((300, 512)) * np.exp2(rng.integers(-20, 12, size=(300, 1)))).astype(np.float32)
+  x[0, :32] = 0; x[1, :64] = 2.0 ** -3; x[2, 5] = 448.0; x[3, :32] = 1e-30
+  q, e8, packed = moe.quantize_mxfp8(gpu.Buffer.from_numpy(x))
+  rq, re8 = omx.quantize_mxfp8(x)
+  np.testing.assert_array_equal(e8.numpy(), re8)
+  np.testing.assert_array_equal(q.numpy(), rq)
+  np.testing.assert_array_equal(packed.numpy(), omx.mx_pack(re8))
+  # bf16 input
+  xb = moe.to_bf16_bits(x)
+  q2, e82, _ = moe.quantize_mxfp8(gpu.Buffer.from_numpy(xb))
+  rq2, re82 = omx.quantize_mxfp8(moe.from_bf16_bits(xb))
+  np.testing.assert_array_equal(e82.numpy(), re82); np.testing.assert_array_equal(q2.numpy(), rq2)
+
+@pytest.mark.parametrize("T,E,k", [(300, 16, 4), (4096, 128, 8), (7, 5, 5)])
+def test_route_dispatch_combine(gpu, T, E, k):
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(T + E)
+  logits = rng.standard_normal((T, E)).astype(np.float32)
+  if T > 10: logits[3, 2] = logits[3, 7] = 9.0                                   # a tie inside the top-k
+  if E == 128: logits[:, :64] -= 3.0                                             # skewed load, some experts (nearly) empty
+  r = moe.route(gpu.Buffer.from_numpy(logits), k, E)
+  ref = omoe.route(logits, k, E)
+  np.testing.assert_array_equal(r.topi.numpy(), ref["topi"])
+  np.testing.assert_array_equal(r.off.numpy(), ref["off"])
+  np.testing.assert_array_equal(r.dest_row.numpy(), ref["dest_row"])
+  np.testing.assert_allclose(r.weights.numpy(), ref["weights"], rtol=2e-6, atol=1e-8)
+  assert r.m_l == ref["m_l"]
+  # invariants: dest_row is injective into expert-contiguous 256-padded ranges
+  d = r.dest_row.numpy(); off = r.off.numpy(); e = r.topi.numpy().reshape(-1)
+  assert len(set(d.tolist())) == T * k and (off % 256 == 0).all() and ((d >= off[e]) & (d < off[e + 1])).all()
+  D = 64
+  x = moe.to_bf16_bits(rng.standard_normal((T, D)).astype(np.float32))
+  xg = moe.dispatch(gpu.Buffer.from_numpy(x), r)
+  np.testing.assert_array_equal(xg.numpy(), omoe.dispatch(x, ref, k))
+  # identity experts: combine(dispatch(x)) = x * sum(weights) = x (up to bf16 rounding of the products)
+  out = moe.combine(xg, r, T, k)
+  xf = moe.from_bf16_bits(x)
+  wb = moe.from_bf16_bits(moe.to_bf16_bits(ref["weights"]))
+  exp = moe.to_bf16_bits(moe.from_bf16_bits(moe.to_bf16_bits(xf[:, None, :] * wb[:, :, None])).sum(1))
+  np.testing.assert_array_equal(out.numpy(), exp)
+
+@pytest.mark.parametrize("E,N,K,rows", [(4, 256, 128, [256, 0, 512, 256]), (8, 512, 2048, [256] * 8), (3, 256, 768, [512, 256, 0])])
+def test_grouped_mxfp8_gemm(gpu, E, N, K, rows):
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(N + K)
+  off = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+  M = int(off[-1]) + 256                                                          # one unrouted tile at the end
+  x = (rng.standard_normal((M, K)) * 0.5).astype(np.float32)
+  w = (rng.standard_normal((E, N, K)) * 0.5).astype(np.float32)
+  xq, xe8 = omx.quantize_mxfp8(x); wq, we8 = omx.quantize_mxfp8(w)
+  C = gpu.Buffer((M, N), np.uint16).zero_()
+  bufs = [gpu.Buffer.from_numpy(a) for a in (xq, wq, xe8, we8, off)]
+  gpu.check(gpu.lib().tga_grouped_mxfp8_gemm(C.ptr, bufs[0].ptr, bufs[1].ptr, None, None, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr, M, N, K, E, None))
+  got = moe.from_bf16_bits(C.numpy())
+  ref = omx.grouped_mx_gemm_ref(xq, xe8, wq, we8, off)
+  used = int(off[-1])
+  err_mx = np.abs(got[:used] - ref[:used]).mean() / np.abs(ref[:used]).mean()
+  assert err_mx < 1e-2, err_mx                                                    # the reference's bar
+  # tighter: bf16 output of a float32 accumulation of exactly representable products: within one bf16 ulp of the oracle
+  np.testing.assert_allclose(got[:used], ref[:used], rtol=2 ** -7, atol=1e-3 * np.abs(ref).max())
+  assert (got[used:] == 0).all()                                                  # unrouted tile untouched
+  # against the unquantized product: the reference's second bar (< 6e-2)
+  full = np.zeros_like(ref)
+  for e in range(E): full[off[e]:off[e + 1]] = x[off[e]:off[e + 1]] @ w[e].T
+  assert np.abs(got[:used] - full[:used]).mean() / np.abs(full[:used]).mean() < 6e-2

@@ -1,0 +1,84 @@
+"""MXFP8 MoE grouped-GEMM path behind the reference's names (extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py,
+extra/gemm/cdna_asm_gemm.py): route / dispatch / combine, quantize_mxfp8, grouped_mx_gemm.  bf16 and E4M3 tensors are device
+Buffers of uint16 / uint8 (numpy has neither type); shapes follow the reference."""
+from __future__ import annotations
+from dataclasses import dataclass
+import numpy as np
+from tinygrad_amd import runtime as rt
+from tinygrad_amd.runtime import Buffer
+
+BLOCK_ROW = 256
+
+def m_max_for(t_local: int, experts_per_tok: int, n_experts: int) -> int:          # moe_routing.py:89-90
+  return (-(-t_local * experts_per_tok // BLOCK_ROW) + n_experts) * BLOCK_ROW
+
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+  u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+  return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+def from_bf16_bits(b: np.ndarray) -> np.ndarray:
+  return (np.ascontiguousarray(b).astype(np.uint32) << 16).view(np.float32)
+
+@dataclass
+class Routing:
+  """moe_routing.py:92-96 (one device group)."""
+  weights: Buffer      # (T, k) float32
+  dest_row: Buffer     # (T*k,) int32
+  off: Buffer          # (E+1,) int32
+  m_l: int
+  t_local: int
+  topi: Buffer         # (T, k) int32
+  counts: Buffer       # (E,) int32
+
+def route(logits: Buffer, experts_per_tok: int, n_experts: int, stream=None) -> Routing:
+  T, E = logits.shape
+  assert E == n_experts
+  k = experts_per_tok
+  w, topi, dest, off, cnt = Buffer((T, k), np.float32), Buffer((T, k), np.int32), Buffer((T * k,), np.int32), Buffer((E + 1,), np.int32), Buffer((E,), np.int32)
+  scratch = Buffer((T * k + ((T * k + 1023) // 1024) * E,), np.int32)
+  rt.check(rt.lib().tga_moe_route(logits.ptr, T, E, k, w.ptr, topi.ptr, dest.ptr, off.ptr, cnt.ptr, scratch.ptr, stream))
+  r = Routing(w, dest, off, m_max_for(T, k, E), T, topi, cnt)
+  r._scratch = scratch                                                            # keep alive until the stream has run
+  return r
+
+def dispatch(x: Buffer, r: Routing, stream=None, out: Buffer | None = None) -> Buffer:
+  """x (T, D) bf16 bits -> xg (m_l, D) bf16 bits."""
+  T, D = x.shape
+  k = r.dest_row.shape[0] // T
+  xg = out if out is not None else Buffer((r.m_l, D), np.uint16)
+  rt.check(rt.lib().tga_moe_dispatch(x.ptr, r.dest_row.ptr, r.off.ptr, r.counts.ptr, T, k, r.off.shape[0] - 1, r.m_l, D, xg.ptr, stream))
+  return xg
+
+def combine(y: Buffer, r: Routing, n_tokens: int, experts_per_tok: int, stream=None, out: Buffer | None = None) -> Buffer:
+  D = y.shape[-1]
+  o = out if out is not None else Buffer((n_tokens, D), np.uint16)
+  rt.check(rt.lib().tga_moe_combine_rows(y.ptr, r.dest_row.ptr, r.weights.ptr, n_tokens, experts_per_tok, D, o.ptr, stream))
+  return o
+
+def quantize_mxfp8(x: Buffer, stream=None):
+  """cdna_asm_gemm.py:149-159: x (rows, K) bf16 bits (uint16) or float32 -> (q uint8 (rows,K), e8 uint8 (rows,K/32), packed uint32 (K/128, rows) or None)."""
+  rows, K = x.shape
+  q, e8 = Buffer((rows, K), np.uint8), Buffer((rows, K // 32), np.uint8)
+  packed = Buffer((K // 128, rows), np.uint32) if K % 128 == 0 else None
+  rt.check(rt.lib().tga_quantize_mxfp8(x.ptr, int(x.dtype == np.uint16), rows, K, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
+  return q, e8, packed
+
+def grouped_mx_gemm(x: Buffer, w: tuple[Buffer, Buffer], expert_off: Buffer, stream=None, out: Buffer | None = None) -> Buffer:
+  """moe_gemm.py:112-134 with pre-quantized weights w = (w_q (E,N,K) e4m3 bits, w_e8 (E,N,K/32)): quantizes x (M,K) bf16 to MXFP8 and
+  runs the grouped GEMM; returns (M, N) bf16 bits."""
+  w_q, w_e8 = w
+  E, N, K2 = w_q.shape
+  M, K = x.shape
+  assert K == K2, f"shape mismatch {x.shape} {w_q.shape}"
+  assert M % 256 == 0 and N % 256 == 0 and K % 128 == 0, f"grouped mxfp8 needs M%256,N%256,K%128, got {x.shape} {w_q.shape}"   # moe_gemm.py:120
+  x_q, x_e8, x_si = quantize_mxfp8(x, stream)
+  o = out if out is not None else Buffer((M, N), np.uint16)
+  rt.check(rt.lib().tga_grouped_mxfp8_gemm(o.ptr, x_q.ptr, w_q.ptr, x_si.ptr, None, x_e8.ptr, w_e8.ptr, expert_off.ptr, M, N, K, E, stream))
+  o._keep = (x_q, x_e8, x_si)
+  return o
+
+def swiglu(h: Buffer, limit: float = 7.0, alpha: float = 1.702, stream=None) -> Buffer:
+  rows, two_i = h.shape
+  y = Buffer((rows, two_i // 2), np.uint16)
+  rt.check(rt.lib().tga_swiglu_interleaved(h.ptr, rows, two_i, limit, alpha, y.ptr, stream))
+  return y

@@ -32,6 +32,12 @@ def _declare(lib):
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
+    "tga_quantize_mxfp8": [vp, i, i64, i64, vp, vp, vp, vp],
+    "tga_moe_route": [vp, i, i, i, vp, vp, vp, vp, vp, vp, vp],
+    "tga_moe_dispatch": [vp, vp, vp, vp, i, i, i, i64, i, vp, vp],
+    "tga_moe_combine_rows": [vp, vp, vp, i, i, i, vp, vp],
+    "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
+    "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
