@@ -1,0 +1,115 @@
+"""Pins the oracle's block dequant (no GPU): the reference's own known-answer vectors, the independent scalar C restatement of
+the published ggml loops, brute force on the bit layout, and closed forms."""
+import numpy as np, pytest
+from oracle import ggml as og, cref
+
+def test_q8_0_reference_kat():
+  # test/unit/test_gguf.py:36-40
+  block = np.frombuffer(np.float16(2.0).tobytes() + np.arange(1, 33, dtype=np.int8).tobytes(), dtype=np.uint8).copy()
+  np.testing.assert_array_equal(og.ggml_data_to_tensor(block, 32, 8), np.arange(1, 33, dtype=np.float32) * 2.0)
+
+def test_mxfp4_reference_kat_hardcoded():
+  # test/unit/test_gguf.py:42-48: pins low-nibbles-first order, scale 2^(E-128) and the doubled table
+  block = np.array([0x80] + list(range(16)), dtype=np.uint8)
+  exp = np.array([0., 1., 2., 3., 4., 6., 8., 12., -0., -1., -2., -3., -4., -6., -8., -12.] + [0.] * 16, dtype=np.float32)
+  np.testing.assert_array_equal(og.ggml_data_to_tensor(block, 32, 39), exp)
+
+def test_mxfp4_reference_closed_form_seed42():
+  # test/unit/test_gguf.py:65-87: independent E2M1 x E8M0 formula incl. E < 2 subnormal scales
+  def decode(code, E):
+    sign = -1.0 if (code & 0b1000) else 1.0
+    exp, mant = (code >> 1) & 0b11, code & 0b1
+    val = 2 * ((1.0 + 0.5 * mant) * np.exp2(exp - 1) if exp else 0.5 * mant)
+    return sign * val * (np.exp2(E - 128) if E >= 2 else np.exp2(-127 if E == 1 else -128))
+  blocks, expected = [], []
+  rng = np.random.default_rng(42)
+  for _ in range(4):
+    E = rng.integers(0, 256)
+    codes = rng.integers(0, 16, size=32, dtype=np.uint8)
+    blocks.append(np.array([E] + [(lo & 0xF) | ((hi & 0xF) << 4) for lo, hi in zip(codes[:16], codes[16:])], dtype=np.uint8))
+    expected.extend(decode(int(c), int(E)) for c in codes)
+  with np.errstate(over="ignore"):
+    out = og.ggml_data_to_tensor(np.concatenate(blocks), len(expected), 39)
+    np.testing.assert_array_equal(out, np.array(expected, dtype=np.float32))
+  for E in (0, 1, 2):                                        # the two fp32-subnormal scales explicitly
+    b = np.array([E] + [0x21] * 16, dtype=np.uint8)
+    np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 32, 39), np.array([decode(1, E)] * 16 + [decode(2, E)] * 16, dtype=np.float32))
+
+def test_mxfp4_reference_real_block():
+  # test/unit/test_gguf.py:89-105 (first block of GLM-4.7-Flash blk.0.attn_k_b.weight)
+  block = np.array([0x7a, 0x29, 0xab, 0x61, 0x10, 0x21, 0x02, 0x4a, 0x15, 0xca, 0x05, 0x01, 0x9b, 0x39, 0x0b, 0x0b, 0x1c], dtype=np.uint8)
+  exp = np.array([-0.015625, -0.046875, 0.015625, 0.0, 0.015625, 0.03125, -0.03125, 0.09375, -0.03125, 0.09375, 0.015625, -0.046875,
+                  -0.015625, -0.046875, -0.046875, -0.0625, 0.03125, -0.03125, 0.125, 0.015625, 0.03125, 0.0, 0.0625, 0.015625,
+                  -0.0625, 0.0, 0.0, -0.015625, 0.046875, 0.0, 0.0, 0.015625], dtype=np.float32)
+  np.testing.assert_array_equal(og.ggml_data_to_tensor(block, 32, 39), exp)
+
+def test_q4_0_brute_force_layout():
+  """Every nibble position: w[j] = (low nibble of qs[j]) - 8, w[j+16] = (high nibble of qs[j]) - 8, times d (ggml_common.py:21)."""
+  for j in range(16):
+    for nib, hi in ((0x0, False), (0xF, False), (0x5, True), (0xF, True)):
+      b = np.zeros(18, dtype=np.uint8); b[:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+      b[2:] = 0x88                                            # all weights 0
+      b[2 + j] = (0x80 | nib) if not hi else (0x08 | (nib << 4))
+      exp = np.zeros(32, dtype=np.float32); exp[j + (16 if hi else 0)] = (nib - 8) * 0.5
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 32, 2), exp)
+
+def test_q6_k_brute_force_layout():
+  """One weight at a time: ggml's dequantize_row_q6_K index map (ql/qh/scale position of element e)."""
+  for e in [0, 1, 15, 16, 31, 32, 63, 64, 95, 96, 127, 128, 129, 160, 200, 255]:
+    b = np.zeros(210, dtype=np.uint8)
+    b[208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    b[192:208] = 1                                            # all sub-scales 1
+    # all quants = 32 (-> 0): low nibble 0, high bits 2
+    b[:128] = 0x00; b[128:192] = 0xAA
+    half, j, l = e >> 7, (e >> 5) & 3, e & 31
+    q = 63                                                    # -> +31
+    qi = 64 * half + (32 if j & 1 else 0) + l
+    b[qi] = (int(b[qi]) & (0x0F if j & 2 else 0xF0)) | ((q & 0xF) << (4 if j & 2 else 0))
+    hi_i = 128 + 32 * half + l
+    b[hi_i] = (int(b[hi_i]) & (0xFF ^ (3 << (2 * j)))) | ((q >> 4) << (2 * j))
+    b[192 + e // 16] = 0xFD                                   # int8 -3
+    exp = np.zeros(256, dtype=np.float32); exp[e] = 31 * -3.0
+    out = og.ggml_data_to_tensor(b, 256, 14)
+    np.testing.assert_array_equal(out, exp, err_msg=f"element {e}")
+
+@pytest.mark.parametrize("t", [2, 8, 14, 39])
+def test_numpy_restatement_equals_scalar_c_loops(t):
+  """Vectorised restatement of tinygrad/llm/gguf.py (field-major q_to_uint8) == independent scalar loops of the published ggml
+  routines, bit for bit, on fully random bytes (NaN/Inf/subnormal scales included)."""
+  rng = np.random.default_rng(t)
+  nel, nby = og.GGML_QUANT[t]
+  data = rng.integers(0, 256, size=(2048, nby), dtype=np.uint8)
+  if t == 39: data[:6, 0] = [0, 1, 2, 254, 255, 127]
+  with np.errstate(all="ignore"): a = og.ggml_data_to_tensor(data, 2048 * nel, t)
+  c = cref.dequant(t, data)
+  same = (a.view(np.uint32) == c.view(np.uint32)) | (np.isnan(a) & np.isnan(c))
+  assert same.all()
+
+def test_q6_k_association_order_is_exact():
+  """(d*q)*sc == d*(sc*q) == (d*sc)*q in float32: 11 + 6 + 8 significant bits fit in 24."""
+  rng = np.random.default_rng(3)
+  d = np.float16(rng.standard_normal(4096)).astype(np.float32); q = rng.integers(-32, 32, 4096).astype(np.float32); sc = rng.integers(-128, 128, 4096).astype(np.float32)
+  np.testing.assert_array_equal((d * q) * sc, (d * sc) * q)
+
+def test_quantizers_round_trip():
+  rng = np.random.default_rng(0)
+  w = rng.standard_normal(256 * 64).astype(np.float32)
+  for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0)):
+    dq = og.ggml_data_to_tensor(qf(w), w.size, t)
+    nel = og.GGML_QUANT[t][0] if t != 14 else 16
+    amax = np.abs(w.reshape(-1, nel)).max(1, keepdims=True)
+    assert (np.abs(dq.reshape(-1, nel) - w.reshape(-1, nel)) <= tol * amax + 1e-6).all(), t
+
+def test_unknown_type_raises():
+  with pytest.raises(ValueError): og.ggml_data_to_tensor(np.zeros(512, np.uint8), 256, 1337)   # test/unit/test_gguf.py:114-116
+
+def test_fp16_conversions_exhaustive():
+  L = cref.lib()
+  f = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+  for h in range(0, 65536, 3):
+    v = np.float32(L.orc_h2f(h))
+    assert v.tobytes() == f[h].tobytes() or (np.isnan(v) and np.isnan(f[h]))
+  rng = np.random.default_rng(5)
+  xs = (rng.standard_normal(5000) * np.float32(10.0) ** rng.integers(-9, 6, 5000)).astype(np.float32)
+  with np.errstate(over="ignore"): exp = xs.astype(np.float16).view(np.uint16)
+  assert all(L.orc_f2h(float(v)) == int(e) for v, e in zip(xs, exp))
