@@ -35,7 +35,7 @@ class Model:
       raw, t, shp = tensors[name]
       w = ggml.ggml_data_to_tensor(raw, int(np.prod(shp)), t).reshape(shp)
       return w.astype(np.float16).astype(np.float32) if (w_round_f16 and t not in (0,)) else w.astype(np.float32)
-    self.w = {name: deq(name) for name in tensors}
+    self.w = {name: (deq(name) if isinstance(tensors[name], tuple) else np.asarray(tensors[name], dtype=np.float32)) for name in tensors}
     if "output.weight" not in self.w: self.w["output.weight"] = self.w["token_embd.weight"]
     self.fc = precompute_freqs_cis(cfg["head_dim"], max_context, cfg["rope_theta"])
     L, kv, hd = cfg["num_blocks"], cfg["n_kv_heads"], cfg["head_dim"]

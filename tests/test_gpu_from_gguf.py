@@ -1,0 +1,51 @@
+"""End to end through a GGUF file: write a small llama-architecture model (Q4_0 linears, Q8_0 embedding, Q6_K lm-head, F32 norms),
+load it with Transformer.from_gguf (byte-level q/k row permutation, tied-embedding rule) and compare greedy tokens with the numpy
+restatement of the reference's from_gguf + forward."""
+import numpy as np, pytest
+from oracle import ggml as og, gguf as ogguf, llm as ollm, linear as ol
+
+pytestmark = pytest.mark.gpu
+
+def _make_file(tmp_path, tied: bool):
+  rng = np.random.default_rng(11)
+  c = dict(dim=256, hidden=512, H=4, KV=2, hd=64, L=2, vocab=512)
+  def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
+  tensors = [("token_embd.weight", (c["vocab"], c["dim"]), 8, og.quantize_q8_0(lin(c["vocab"], c["dim"]) * 16))]
+  for i in range(c["L"]):
+    p = f"blk.{i}."
+    tensors += [(p + "attn_norm.weight", (c["dim"],), 0, (1 + 0.1 * rng.standard_normal(c["dim"])).astype(np.float32)),
+                (p + "attn_q.weight", (c["H"] * c["hd"], c["dim"]), 2, og.quantize_q4_0(lin(c["H"] * c["hd"], c["dim"]))),
+                (p + "attn_k.weight", (c["KV"] * c["hd"], c["dim"]), 2, og.quantize_q4_0(lin(c["KV"] * c["hd"], c["dim"]))),
+                (p + "attn_v.weight", (c["KV"] * c["hd"], c["dim"]), 2, og.quantize_q4_0(lin(c["KV"] * c["hd"], c["dim"]))),
+                (p + "attn_output.weight", (c["dim"], c["H"] * c["hd"]), 2, og.quantize_q4_0(lin(c["dim"], c["H"] * c["hd"]))),
+                (p + "ffn_norm.weight", (c["dim"],), 0, (1 + 0.1 * rng.standard_normal(c["dim"])).astype(np.float32)),
+                (p + "ffn_gate.weight", (c["hidden"], c["dim"]), 2, og.quantize_q4_0(lin(c["hidden"], c["dim"]))),
+                (p + "ffn_up.weight", (c["hidden"], c["dim"]), 2, og.quantize_q4_0(lin(c["hidden"], c["dim"]))),
+                (p + "ffn_down.weight", (c["dim"], c["hidden"]), 2, og.quantize_q4_0(lin(c["dim"], c["hidden"])))]
+  tensors.append(("output_norm.weight", (c["dim"],), 0, np.ones(c["dim"], np.float32)))
+  if not tied: tensors.append(("output.weight", (c["vocab"], c["dim"]), 14, og.quantize_q6_k(lin(c["vocab"], c["dim"]))))
+  kvs = [("general.architecture", "llama"), ("llama.context_length", 96), ("llama.attention.head_count", c["H"]), ("llama.attention.head_count_kv", c["KV"]),
+         ("llama.block_count", c["L"]), ("llama.embedding_length", c["dim"]), ("llama.feed_forward_length", c["hidden"]),
+         ("llama.attention.layer_norm_rms_epsilon", 1e-5), ("llama.rope.freq_base", 10000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(c["vocab"])])]
+  from tinygrad_amd.gguf import gguf_write
+  path = tmp_path / ("tied.gguf" if tied else "model.gguf")
+  return path, gguf_write(path, kvs, tensors)
+
+@pytest.mark.parametrize("tied", [False, True])
+def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
+  from tinygrad_amd.llm import Transformer
+  path, raw = _make_file(tmp_path, tied)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  assert model.config.max_context == 64 and model.config.vocab_size == 512 and kv["general.architecture"] == "llama"
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  prompt = [1, 77, 300, 9, 410, 3]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)         # weights already prepared (fp16-rounded, permuted)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3

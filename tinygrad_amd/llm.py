@@ -108,6 +108,13 @@ def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = 
   mk("output.weight", c.vocab_size, c.dim, head_type, c.dim ** -0.5)
   return sd
 
+def _to_f32(data: np.ndarray, typ: int) -> np.ndarray:
+  raw = np.ascontiguousarray(data).view(np.uint8)
+  if typ == rt.F32: return raw.view(np.float32)
+  if typ == rt.F16: return raw.view(np.float16).astype(np.float32)
+  if typ == 30: return (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32)      # bfloat16
+  raise NotImplementedError(f"ggml type {typ} for a norm / dense tensor")
+
 class TransformerBlock:
   """One decode step of the reference's TransformerBlock/FFNBlock (tinygrad/llm/model.py:144-204) for batch 1."""
   def __init__(self, config: TransformerConfig, sd: dict, i: int, shared):
@@ -208,6 +215,53 @@ class Transformer:
       with g: self._step(with_head)
       self._graphs[with_head] = g
     return self._graphs[with_head]
+
+  @staticmethod
+  def from_gguf(gguf, max_context: int | None = None, max_new: int = 4096) -> tuple["Transformer", dict]:
+    """Transformer.from_gguf (tinygrad/llm/model.py:370-451) for the architectures on the path (dense llama-family and MoE with
+    qk-norm).  Weights stay in their GGUF blocks on the device; F32 / BF16 matrices are cast to fp16 on the host (the reference
+    casts every weight to fp16, model.py:376); for arch == 'llama' the rows of attn_q / attn_k are permuted from the interleaved
+    to the half-split RoPE layout (model.py:409-419) by moving whole block rows."""
+    from tinygrad_amd.gguf import gguf_load, GGUF_F32_LIKE
+    kv, ts = gguf_load(gguf)
+    arch = kv["general.architecture"]
+    ctx = kv[f"{arch}.context_length"]
+    max_context = min(max_context, ctx) if max_context is not None else ctx
+    n_heads, n_kv = kv[f"{arch}.attention.head_count"], kv[f"{arch}.attention.head_count_kv"]
+    dim = kv[f"{arch}.embedding_length"]
+    head_dim = kv.get(f"{arch}.attention.key_length", dim // n_heads)
+    rope_dim = kv.get(f"{arch}.rope.dimension_count", head_dim)
+    if rope_dim != head_dim: raise NotImplementedError("partial rotary embeddings are not built")
+    if kv.get(f"{arch}.attention.kv_lora_rank", 0) or arch in ("qwen35", "qwen35moe", "kimi-linear"): raise NotImplementedError(f"architecture {arch} is outside the built path")
+    sd = {}
+    for name, t in ts.items():
+      if name == "rope_freqs.weight": continue                         # unused by the reference too (model.py:446)
+      rows, cols = (int(np.prod(t.shape[:-1])), t.shape[-1]) if len(t.shape) > 1 else (1, t.shape[0])
+      typ, buf, data = t.ggml_type, t.buffer, t.data
+      is_norm = name.endswith("_norm.weight")
+      if is_norm:
+        if typ != rt.F32: data = _to_f32(data, typ); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F32
+      elif typ in GGUF_F32_LIKE:                                       # F32 / BF16 matrices -> fp16 (model.py:376)
+        data = _to_f32(data, typ).astype(np.float16); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F16
+      if arch == "llama" and (name.endswith("attn_q.weight") or name.endswith("attn_k.weight")):
+        h = n_heads if name.endswith("attn_q.weight") else n_kv
+        raw = np.ascontiguousarray(data).view(np.uint8).reshape(rows, -1)
+        per = rows // h
+        idx = np.arange(rows).reshape(h, per // 2, 2).transpose(0, 2, 1).reshape(-1)   # "n (h two) d -> n (two h) d"
+        buf = Buffer.from_numpy(np.ascontiguousarray(raw[idx]).reshape(-1))
+      shape = (rows, cols) if len(t.shape) <= 2 else tuple(t.shape)
+      sd[name] = (buf, typ, shape)
+    if "output.weight" not in sd: sd["output.weight"] = sd["token_embd.weight"]        # tied embeddings, model.py:379
+    config = TransformerConfig(
+      num_blocks=kv[f"{arch}.block_count"], dim=dim,
+      hidden_dim=kv.get(f"{arch}.expert_feed_forward_length", kv.get(f"{arch}.feed_forward_length", 0)),
+      n_heads=n_heads, n_kv_heads=n_kv, norm_eps=kv[f"{arch}.attention.layer_norm_rms_epsilon"], vocab_size=len(kv["tokenizer.ggml.tokens"]),
+      head_dim=head_dim, rope_theta=kv[f"{arch}.rope.freq_base"], max_context=max_context,
+      qk_norm=int(sd["blk.0.attn_q_norm.weight"][2][-1]) if "blk.0.attn_q_norm.weight" in sd else 0,
+      num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
+      norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe",)),
+      expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0))
+    return Transformer(config, sd, max_new=max_new), kv
 
   def reset(self, tokens: list[int]):
     """Start a new sequence: position 0, first prompt token loaded, nothing cached (no KV-prefix reuse)."""
