@@ -97,21 +97,21 @@ def main():
     per = {k: [] for k in durs}
     for b in model.blk:
       s = model.s
-      rt.check(L.tga_rmsnorm(s.x.ptr, b.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, st))
+      rt.check(L.tga_rmsnorm(s.x.ptr, b.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, b.attn_q.ggml_type if b.staged else 0, st))
       e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.xn, [s.q, s.k, s.v], stream=st)
+      qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.xn, [s.q, s.k, s.v], stream=st, x_staged=b.staged)
       e[1].record(st); per["qkv"].append(e)
       rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                      c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, st))
+                                      c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if b.staged else 0, st))
       e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st)
+      qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.staged)
       e[1].record(st); per["attn_output"].append(e)
-      rt.check(L.tga_rmsnorm(s.x.ptr, b.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, st))
+      rt.check(L.tga_rmsnorm(s.x.ptr, b.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, b.ffn_gate.ggml_type if b.staged else 0, st))
       e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.ffn_gate, b.ffn_up], s.xn, [s.act], epilogue=2, stream=st)
+      qlinear_multi([b.ffn_gate, b.ffn_up], s.xn, [s.act], epilogue=2, stream=st, x_staged=b.staged, stage_out_for=b.ffn_down if b.staged else None)
       e[1].record(st); per["gate_up"].append(e)
       e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st)
+      qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.staged)
       e[1].record(st); per["down"].append(e)
     rt.check(L.tga_advance_prompt(model.s.state.ptr, model.s.prompt.ptr, st))
     model.stream.synchronize()

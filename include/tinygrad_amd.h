@@ -22,6 +22,8 @@ extern "C" {
 #define TGA_Q8_0 8
 #define TGA_Q6_K 14
 #define TGA_MXFP4 39
+/* activation dtype code: fp16 values in the staged order of the consuming weight (see tga_stage_activation) */
+#define TGA_F16_STAGED 101
 
 /* ---- runtime: replaces HIPDevice / HIPAllocator / HIPProgram timing in tinygrad/runtime/ops_hip.py:12-70 ---- */
 const char* tga_last_error(void);
@@ -70,7 +72,15 @@ int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* 
  * y[0] = silu(x Wgate^T) * (x Wup^T) (model.py:137), resid ignored. */
 int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                       const void* x, int x_dtype, int y_dtype, int M, int64_t K,
-                      int epilogue, const void* const* resid, void* stream);
+                      int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
+
+/* Staged activations (no counterpart in the reference; an M = 1 fast path): the decode GEMV keeps each lane's activations in
+ * registers in the order its in-register decode produces weights, which is a fixed permutation of the row that depends on the
+ * weight's (ggml_type, K).  tga_stage_activation writes that permutation as fp16 (K values); a linear then takes it with
+ * x_dtype = TGA_F16_STAGED and skips its own staging.  Producers can emit the order directly: tga_rmsnorm / tga_attention_decode
+ * (stage_type, stage_K) and tga_qlinear_multi (y_stage_type != 0: the single fp16 output, of length y_stage_K, is written in the
+ * staged order of a consumer weight of that type whose K = y_stage_K).  Requires K % 64 == 0 (Q6_K: % 256). */
+int tga_stage_activation(int ggml_type, const void* x, int x_dtype, int64_t K, void* out_f16, void* stream);
 
 /* ExpertWeights.__call__ (tinygrad/llm/model.py:21-27) over a stacked (n_experts, N, K) weight kept in GGUF blocks: for job j
  * (one (token, slot) pair) y[j, :] = x[j / jobs_per_x_row, :] @ W[sel[j]]^T; only the selected experts' bytes are read.
@@ -94,17 +104,19 @@ int tga_moe_combine(const float* y, const float* probs, const float* resid, int 
 /* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q8_0 / F16 / F32 table. */
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream);
 
-/* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL). */
-int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, void* stream);
+/* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL).
+ * stage_type != 0: the fp16 output is written in the staged order of a consumer weight of that ggml type with K = dim. */
+int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream);
 
 /* One token of TransformerBlock._attention after the q/k/v projections (model.py:180-197): half-split RoPE of q and k with the
  * freqs_cis table rope_table[max_ctx][head_dim] = cos half | sin half (model.py:16-19, 29-33), fp16 KV append at state.pos
  * (cache layout [n_kv_heads][max_ctx][head_dim]), GQA scaled-dot-product attention over positions 0..pos with softmax in
  * float32 (tinygrad/mixin/rand.py:298-327).  head_dim is 64, 128 or 256.  partials: workspace of
  * n_heads * ceil(max_ctx/64) * (head_dim + 2) floats followed by n_kv_heads int32 arrival counters that must be ZERO before the
- * first call (each call leaves them zero again); calls sharing one workspace must not overlap. */
+ * first call (each call leaves them zero again); calls sharing one workspace must not overlap.
+ * stage_type != 0: out_f16 is written in the staged order of a consumer weight of that type with K = n_heads * head_dim. */
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
-                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
 /* argmax(-1) with first-max tie rule (tinygrad/mixin/op.py:866-891) + the bookkeeping of Transformer.generate (model.py:475-484):
  * while state.pos + 1 < state.n_prompt the next input token is prompt[pos + 1]; otherwise the argmax token is stored at

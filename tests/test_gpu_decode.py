@@ -67,7 +67,7 @@ def test_attention_decode_kernel_vs_numpy(gpu):
     q, k, v = (rng.standard_normal(n).astype(np.float32) for n in (H * hd, KV * hd, KV * hd))
     st = np.zeros(16, np.int32); st[0] = pos
     qb, kb, vb, stb = (gpu.Buffer.from_numpy(t) for t in (q, k, v, st))       # keep the device buffers alive across the launch
-    gpu.check(gpu.lib().tga_attention_decode(qb.ptr, kb.ptr, vb.ptr, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None, out.ptr, None))
+    gpu.check(gpu.lib().tga_attention_decode(qb.ptr, kb.ptr, vb.ptr, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None, out.ptr, 0, None))
     gpu.synchronize()
     qr = ollm.apply_rope(q.reshape(H, hd), rope[pos]); kr = ollm.apply_rope(k.reshape(KV, hd), rope[pos])
     rk[:, pos], rv[:, pos] = kr.astype(np.float16), v.reshape(KV, hd).astype(np.float16)
@@ -84,7 +84,7 @@ def test_rmsnorm_argmax_embed(gpu):
   x = rng.standard_normal(4096).astype(np.float32) * 3; w = rng.standard_normal(4096).astype(np.float32)
   o32 = gpu.Buffer((4096,), np.float32); o16 = gpu.Buffer((4096,), np.float16)
   xb, wb = gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(w)
-  gpu.check(gpu.lib().tga_rmsnorm(xb.ptr, wb.ptr, 4096, 1e-5, o16.ptr, o32.ptr, None))
+  gpu.check(gpu.lib().tga_rmsnorm(xb.ptr, wb.ptr, 4096, 1e-5, o16.ptr, o32.ptr, 0, None))
   ref = ollm.rmsnorm(x, w, 1e-5)
   np.testing.assert_allclose(o32.numpy(), ref, rtol=2e-6, atol=1e-6)
   assert o16.numpy().tobytes() == o32.numpy().astype(np.float16).tobytes()

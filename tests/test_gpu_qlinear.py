@@ -118,3 +118,38 @@ def test_argument_errors(gpu):
   lin = QuantLinear(w, 2, 4, 32)
   with pytest.raises(AssertionError): lin(gpu.Buffer((9, 32), np.float16))
   with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))
+
+@pytest.mark.parametrize("t,k", [(2, 4096), (2, 14336), (8, 4096), (14, 4096), (39, 2048), (1, 2048)])
+def test_staged_activations_equal_plain_path(gpu, t, k):
+  """tga_stage_activation + TGA_F16_STAGED gives the plain path's result (same products; only the order the per-block offset
+  correction is summed in differs), and a SwiGLU output staged for a consumer feeds that consumer correctly."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi, stage_activation
+  rng = np.random.default_rng(k + t)
+  n = 384
+  w = synth.random_blocks(rng, t, n, k) if t != 1 else (rng.standard_normal((n, k)) * 0.02).astype(np.float16).view(np.uint8).reshape(-1)
+  lin = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  x = synth.activations(rng, 1, k, np.float16)
+  xb = gpu.Buffer.from_numpy(x)
+  plain = lin(xb, out_dtype=np.float32).numpy()
+  xs = stage_activation(lin, xb)
+  assert sorted(xs.numpy().reshape(-1).view(np.uint16).tolist()) == sorted(x.reshape(-1).view(np.uint16).tolist())   # a permutation of the row
+  out = gpu.Buffer((1, n), np.float32)
+  qlinear_multi([lin], xs, [out], x_staged=True)
+  assert ol.rel_err(out.numpy(), plain) <= 1e-5
+  # fp32 input staged (rounded to fp16 on the way)
+  xs32 = stage_activation(lin, gpu.Buffer.from_numpy(x.astype(np.float32)))
+  assert xs32.numpy().tobytes() == xs.numpy().tobytes()
+
+def test_swiglu_output_staged_for_the_down_projection(gpu):
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(8)
+  d, hdim = 512, 1024
+  g, u, dn = (QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, 2, r, c)), 2, r, c) for r, c in ((hdim, d), (hdim, d), (d, hdim)))
+  x = gpu.Buffer.from_numpy(synth.activations(rng, 1, d, np.float16))
+  act_n, act_s = gpu.Buffer((1, hdim), np.float16), gpu.Buffer((1, hdim), np.float16)
+  y_n, y_s = gpu.Buffer((1, d), np.float32), gpu.Buffer((1, d), np.float32)
+  qlinear_multi([g, u], x, [act_n], epilogue=2)
+  qlinear_multi([dn], act_n, [y_n])
+  qlinear_multi([g, u], x, [act_s], epilogue=2, stage_out_for=dn)
+  qlinear_multi([dn], act_s, [y_s], x_staged=True)
+  assert ol.rel_err(y_s.numpy(), y_n.numpy()) <= 1e-5

@@ -3,8 +3,7 @@
 // They restate, for one token, what tinygrad/llm/model.py:167-204 (_attention), :144-151 (block), :358-364 (forward) compute.
 // The position and token live in device memory so that one captured launch sequence can be replayed for every token
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
-#include "common.h"
-#include "host.h"
+#include "qfmt.h"
 
 struct DecodeState {   // device-resident, 16 int32
   int pos;             // position of the token being processed
@@ -45,7 +44,7 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 // nn.RMSNorm (tinygrad/nn/__init__.py:296-304): x * rsqrt(mean(x^2) + eps), then * weight.  Output fp16 (the activation the
 // dequant-GEMV multiplies) and optionally fp32.
 __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, int dim, float eps,
-                                                       _Float16* __restrict__ out16, float* __restrict__ out32) {
+                                                       _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu) {
   __shared__ float red[16];
   float s = 0.f;
   for (int e = threadIdx.x; e < dim; e += blockDim.x) { const float v = x[e]; s += v * v; }
@@ -58,7 +57,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
   const float scale = 1.0f / sqrtf(tot / (float)dim + eps);
   for (int e = threadIdx.x; e < dim; e += blockDim.x) {
     const float v = (x[e] * scale) * w[e];
-    if (out16) out16[e] = (_Float16)v;
+    if (out16) out16[stage_fmt ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
     if (out32) out32[e] = v;
   }
 }
@@ -77,6 +76,7 @@ struct AttnArgs {
   const float* rope;                                   // [max_ctx][hd]: cos(pos * f_i) for i < hd/2, then sin(pos * f_i)
   float scale;
   _Float16* out16; float* out32;                       // attention output [n_heads*hd]
+  int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
 };
 
 // 8 fp16 values (one 16-byte piece) of row `p` of a cache plane; the row of the token being processed comes from LDS (fp32
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
 #pragma unroll
       for (int j = 0; j < 8; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
     }
-    if (a.out16) a.out16[head * HD + d] = (_Float16)o;
+    if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, head * HD + d, a.stage_nu) : head * HD + d] = (_Float16)o;
     if (a.out32) a.out32[head * HD + d] = o;
   }
 }
@@ -297,16 +297,30 @@ int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, 
   return 0;
 }
 
-int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, void* stream) {
+// staged layout lookup shared with the GEMV host side (qgemv.hip)
+static int decode_staged_fmt(int ggml_type, long long K, int* nu) {
+  int fmt = -1, uw = 64;
+  switch (ggml_type) {
+    case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
+    case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
+  }
+  if (fmt < 0 || K <= 0 || K % (ggml_type == GGML_Q6_K ? 256 : 64) != 0) return -1;
+  *nu = (int)(K / uw);
+  return fmt;
+}
+
+int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(x && weight && (out_f16 || out_f32), "tga_rmsnorm: null pointer");
   TGA_REQUIRE(dim > 0, "tga_rmsnorm: dim=%d", dim);
-  rmsnorm_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32);
+  int sfmt = 0, snu = 0;
+  if (stage_type) { sfmt = decode_staged_fmt(stage_type, dim, &snu); TGA_REQUIRE(sfmt >= 0, "tga_rmsnorm: no staged layout for type %d with K=%d", stage_type, dim); }
+  rmsnorm_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu);
   TGA_LAUNCH_CHECK();
   return 0;
 }
 
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
-                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
+                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
   TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode: head_dim=%d must be 64, 128 or 256", head_dim);
@@ -316,6 +330,8 @@ int tga_attention_decode(const float* q, const float* k, const float* v, void* c
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
+  a.stage_fmt = 0; a.stage_nu = 0;
+  if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
   const dim3 grid(n_kv_heads, a.nsplit);
   hipStream_t s = (hipStream_t)stream;
   if (head_dim == 64) attn_decode_kernel<8><<<grid, 256, 0, s>>>(a);

@@ -21,7 +21,13 @@ struct QArgs {
   // job indirection (MoE expert GEMVs): blockIdx.y = job; expert = sel[job]; weights shifted by expert * estride bytes;
   // activation row = job / xdiv; outputs shifted by job * ystride elements.  sel == nullptr: a single job.
   const int* sel; long long estride, ystride; int xdiv, xdiv_jobs;   // xdiv_jobs: number of jobs (grid.y)
+  // x_staged: x already holds fp16 activations in the consumer format's staged order (Fmt::spos).
+  // y_stage_fmt / y_stage_nu: when y_stage_fmt != 0 the fp16 outputs are written in the staged order of THAT consumer format.
+  int x_staged, y_stage_fmt, y_stage_nu;
 };
+
+// staged position of element e for a consumer of format `fmt` (row length K = UW * nu)
+__device__ __forceinline__ int staged_pos(int fmt, int e, int nu);
 
 __device__ __forceinline__ uint32_t pack_even(uint32_t a, uint32_t b) { return (a & 0xFFFFu) | (b << 16); }        // (a.lo, b.lo)
 __device__ __forceinline__ uint32_t pack_odd(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xFFFF0000u); }     // (a.hi, b.hi)
@@ -170,6 +176,26 @@ template <> struct Fmt<F_Q4_0P> {
   static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
   }
+  // halfword index of row element e inside the staged activation buffer ([XV][nu] vectors of 4 fp16 pairs)
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = e >> 6, w = e & 63, blk = w >> 5, b = w & 31, hi = b >> 4, q = b & 15;
+    int i, p;
+    if (blk) { i = 4 + (q >> 2); p = q & 3; }
+    else if (q < 2) { i = 0; p = q; }
+    else if (q >= 14) { i = 0; p = q - 12; }
+    else { i = 1 + ((q - 2) >> 2); p = (q - 2) & 3; }
+    return ((i * nu + u) * 4 + (p & 1) * 2 + hi) * 2 + (p >> 1);
+  }
+  // the accumulator start values recomputed from staged vectors (x,z: low-nibble weights, bias 1032; y,w: high-nibble, bias 72)
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float lo = 0.f, hi = 0.f;
+#pragma unroll
+      for (int i = 4 * j; i < 4 * j + 4; i++) { lo = dot2(xv[i].x, 0x64086408u, lo); lo = dot2(xv[i].z, 0x64086408u, lo); hi = dot2(xv[i].y, 0x54805480u, hi); hi = dot2(xv[i].w, 0x54805480u, hi); }
+      c[j] = -(lo + hi);
+    }
+  }
 };
 
 // ------------------------------------------------------------------------------------------------ Q8_0 block pair
@@ -215,6 +241,20 @@ template <> struct Fmt<F_Q8_0P> {
   static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
   }
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = e >> 6, w = e & 63, blk = w >> 5, b = w & 31, n = b >> 1;
+    const int s = blk ? 16 + n : (n == 0 ? 0 : (n == 15 ? 1 : n + 1));
+    return (((s >> 2) * nu + u) * 4 + (s & 3)) * 2 + (b & 1);
+  }
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float t = 0.f;
+#pragma unroll
+      for (int i = 4 * j; i < 4 * j + 4; i++) { t = dot2(xv[i].x, 0x64806480u, t); t = dot2(xv[i].y, 0x64806480u, t); t = dot2(xv[i].z, 0x64806480u, t); t = dot2(xv[i].w, 0x64806480u, t); }
+      c[j] = -t;
+    }
+  }
 };
 
 
@@ -245,6 +285,8 @@ template <> struct Fmt<GGML_F16> {
     c[0] = 0.f;
   }
   static __device__ __forceinline__ float finish(const Raw&, const float* a) { return a[0]; }
+  static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 6, w = e & 63; return (((w >> 3) * nu + u) * 4 + ((w >> 1) & 3)) * 2 + (w & 1); }
+  static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
 
 // ------------------------------------------------------------------------------------------------ MXFP4 (gguf.py:105-114)
@@ -290,6 +332,8 @@ template <> struct Fmt<GGML_MXFP4> {
   static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
     return __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u) * a[0];
   }
+  static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 5, b = e & 31, q = b & 15; return (((q >> 2) * nu + u) * 4 + (q & 3)) * 2 + (b >> 4); }
+  static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
 
 // ------------------------------------------------------------------------------------------------ Q6_K (gguf.py:68-72)
@@ -352,6 +396,19 @@ template <> struct Fmt<GGML_Q6_K> {
     const float s2 = (float)(int)(int8_t)(r.sc1 >> g8), s3 = (float)(int)(int8_t)(r.sc1 >> (16 + g8));
     return h2f_bits(r.d >> 16) * (s0 * a[0] + s1 * a[1] + s2 * a[2] + s3 * a[3]);
   }
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = unit_of(e), j = (e >> 5) & 3, i = e & 15, td = i >> 2, p = i & 3;
+    return (((2 * j + (td >> 1)) * nu + u) * 4 + (td & 1) * 2 + (p & 1)) * 2 + (p >> 1);
+  }
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      float t = 0.f;
+#pragma unroll
+      for (int i = 2 * j; i < 2 * j + 2; i++) { t = dot2(xv[i].x, 0x64206420u, t); t = dot2(xv[i].y, 0x64206420u, t); t = dot2(xv[i].z, 0x64206420u, t); t = dot2(xv[i].w, 0x64206420u, t); }
+      c[j] = -t;
+    }
+  }
 };
 
 
@@ -383,10 +440,23 @@ __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, co
 template <int EPI>
 __device__ __forceinline__ void store_one(const QArgs& a, int seg, long long row, float v, long long yofs = 0) {
   if constexpr (EPI == 1) v += a.resid[seg][yofs + row];
-  if (a.y_f32) ((float*)a.y[seg])[yofs + row] = v; else ((_Float16*)a.y[seg])[yofs + row] = (_Float16)v;
+  if (a.y_f32) ((float*)a.y[seg])[yofs + row] = v;
+  else ((_Float16*)a.y[seg])[yofs + (a.y_stage_fmt ? staged_pos(a.y_stage_fmt, (int)row, a.y_stage_nu) : row)] = (_Float16)v;
 }
 __device__ __forceinline__ void store_swiglu(const QArgs& a, long long row, float gate, float up, long long yofs = 0) {
   const float o = silu_f(gate) * up;
-  if (a.y_f32) ((float*)a.y[0])[yofs + row] = o; else ((_Float16*)a.y[0])[yofs + row] = (_Float16)o;
+  if (a.y_f32) ((float*)a.y[0])[yofs + row] = o;
+  else ((_Float16*)a.y[0])[yofs + (a.y_stage_fmt ? staged_pos(a.y_stage_fmt, (int)row, a.y_stage_nu) : row)] = (_Float16)o;
 }
 
+
+__device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
+  switch (fmt) {
+    case F_Q4_0P: return Fmt<F_Q4_0P>::spos(e, nu);
+    case F_Q8_0P: return Fmt<F_Q8_0P>::spos(e, nu);
+    case GGML_Q6_K: return Fmt<GGML_Q6_K>::spos(e, nu);
+    case GGML_MXFP4: return Fmt<GGML_MXFP4>::spos(e, nu);
+    case GGML_F16: return Fmt<GGML_F16>::spos(e, nu);
+  }
+  return e;
+}

@@ -305,14 +305,45 @@ static int launch_qgemv_m(const QArgs& a, int M, hipStream_t s) {
 
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 
+// internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
+static int staged_fmt(int ggml_type, long long K, int* nu) {
+  int fmt = -1, uw = 64;
+  switch (ggml_type) {
+    case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
+    case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
+  }
+  if (fmt < 0 || K <= 0 || K % (ggml_type == GGML_Q6_K ? 256 : 64) != 0) return -1;
+  *nu = (int)(K / uw);
+  return fmt;
+}
+
+__global__ __launch_bounds__(256) void stage_activation_kernel(const void* __restrict__ x, int x_f32, int K, int fmt, int nu, _Float16* __restrict__ out) {
+  for (int e = blockIdx.x * 256 + threadIdx.x; e < K; e += gridDim.x * 256) {
+    const _Float16 v = x_f32 ? (_Float16)((const float*)x)[e] : ((const _Float16*)x)[e];
+    out[staged_pos(fmt, e, nu)] = v;
+  }
+}
+
+// fp16 copy of one activation row in the order the M = 1 GEMV of a (ggml_type, K) weight consumes (a permutation of the row)
+extern "C" int tga_stage_activation(int ggml_type, const void* x, int x_dtype, int64_t K, void* out_f16, void* stream) {
+  TGA_REQUIRE(x && out_f16, "tga_stage_activation: null pointer");
+  TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32, "tga_stage_activation: x_dtype must be TGA_F16 or TGA_F32");
+  int nu; const int fmt = staged_fmt(ggml_type, K, &nu);
+  TGA_REQUIRE(fmt >= 0, "tga_stage_activation: no staged layout for type %d with K=%lld", ggml_type, (long long)K);
+  stage_activation_kernel<<<(unsigned)((K + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, x_dtype == TGA_F32, (int)K, fmt, nu, (_Float16*)out_f16);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                  const void* x, int x_dtype, int y_dtype, int M, int64_t K,
-                                 int epilogue, const void* const* resid, void* stream) {
+                                 int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
   TGA_REQUIRE(M >= 1 && M <= 8, "tga_qlinear: M=%d out of range 1..8", M);
-  TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32, "tga_qlinear: x_dtype must be TGA_F16 or TGA_F32");
+  TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
   TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
   TGA_REQUIRE(epilogue >= 0 && epilogue <= 2, "tga_qlinear: epilogue=%d unknown", epilogue);
+  TGA_REQUIRE(x_dtype != TGA_F16_STAGED || M == 1, "tga_qlinear: staged activations are an M = 1 format");
   TGA_REQUIRE(epilogue != 1 || (y_dtype == TGA_F32 && resid), "tga_qlinear: the residual epilogue needs float32 y and resid pointers");
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
@@ -322,7 +353,7 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
   TGA_REQUIRE(x, "tga_qlinear: null x");
   QArgs a = {};
-  a.nseg = nseg; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = epilogue; a.K = (int)K;
+  a.nseg = nseg; a.x = x; a.x_staged = x_dtype == TGA_F16_STAGED; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = epilogue; a.K = (int)K;
   long long ntot = 0;
   for (int i = 0; i < nseg; i++) {
     TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)), "tga_qlinear: segment %d has a null pointer or no rows", i);
@@ -332,6 +363,12 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     ntot += n[i];
   }
   a.ntot = (epilogue == 2) ? n[0] : ntot;
+  if (y_stage_type) {
+    TGA_REQUIRE(M == 1 && y_dtype == TGA_F16 && (nseg == 1 || epilogue == 2), "tga_qlinear: staged output needs M = 1, fp16 y and a single output");
+    TGA_REQUIRE(y_stage_K == a.ntot, "tga_qlinear: staged output length %lld must equal the output rows %lld", (long long)y_stage_K, (long long)a.ntot);
+    a.y_stage_fmt = staged_fmt(y_stage_type, y_stage_K, &a.y_stage_nu);
+    TGA_REQUIRE(a.y_stage_fmt >= 0, "tga_qlinear: no staged layout for consumer type %d with K=%lld", y_stage_type, (long long)y_stage_K);
+  }
   hipStream_t s = (hipStream_t)stream;
   // block-pair units need an even number of blocks per row and 4-byte aligned rows
   bool pair = (K / 32) % 2 == 0;
@@ -340,6 +377,7 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
   }
+  TGA_REQUIRE(!a.x_staged && !a.y_stage_fmt, "tga_qlinear: staged activations need the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, K <= 65536)");
   switch (ggml_type) {
     case GGML_Q4_0: return pair ? launch_qgemv_m<F_Q4_0P>(a, M, s) : launch_qgemv_m<GGML_Q4_0>(a, M, s);
     case GGML_Q8_0: return pair ? launch_qgemv_m<F_Q8_0P>(a, M, s) : launch_qgemv_m<GGML_Q8_0>(a, M, s);
@@ -352,7 +390,7 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
 extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                            int M, int64_t N, int64_t K, void* stream) {
   const void* ws[1] = {w}; void* ys[1] = {y}; int64_t ns[1] = {N};
-  return tga_qlinear_multi(ggml_type, 1, ws, ys, ns, x, x_dtype, y_dtype, M, K, 0, nullptr, stream);
+  return tga_qlinear_multi(ggml_type, 1, ws, ys, ns, x, x_dtype, y_dtype, M, K, 0, nullptr, 0, 0, stream);
 }
 
 // ExpertWeights.__call__ (tinygrad/llm/model.py:21-27): per (token, slot) job j, y[j] = x[j / jobs_per_x_row] @ W[sel[j]]^T over a

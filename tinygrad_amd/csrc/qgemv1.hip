@@ -49,14 +49,15 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
     const long long cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;   // row groups of this team inside the segment
     const uint8_t* base0 = a.w[seg] + eoff;
     const uint8_t* base1 = ((EPI == 2) ? a.w[1] : a.w[seg]) + eoff;
+    // Loads are issued UNCONDITIONALLY (row and unit clamped to valid ones, surplus results dropped): a branch around a load
+    // makes the compiler's s_waitcnt placement conservative (vmcnt(0) at the join), which would serialise the pipeline.
+    const int uc = uvalid ? u : a.nu - 1;
     auto issue = [&](Raw* buf, long long row) {
-      if (uvalid) {
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-          long long rr = (EPI == 2) ? row : row + r;
-          if (rr > hi - 1) rr = hi - 1;                            // ragged last group: reload a valid row, result dropped
-          buf[r] = F::load(((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes, u);
-        }
+      for (int r = 0; r < R; r++) {
+        long long rr = (EPI == 2) ? row : row + r;
+        rr = rr < hi - 1 ? rr : hi - 1;                            // beyond the range: reload the last valid row
+        buf[r] = F::load(((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes, uc);
       }
     };
     auto finish_group = [&](const Raw* buf, long long row) {
@@ -64,8 +65,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
 #pragma unroll
       for (int r = 0; r < R; r++) {
         acc[r] = 0.f;
-        if (uvalid) unit_dot_reg<T>(buf[r], xv, cv, acc[r], kc);
-        acc[r] = wave_sum_lane63(acc[r]);
+        unit_dot_reg<T>(buf[r], xv, cv, acc[r], kc);
+        acc[r] = wave_sum_lane63(uvalid ? acc[r] : 0.f);
       }
       if constexpr (WK > 1) {
         if (lane == 63) {
@@ -98,7 +99,18 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
       }
     };
     Raw b0[R], b1[R];
-    if (cnt) issue(b0, lo);
+    if (!staged && a.x_staged) {
+      // producer-staged activations: XV coalesced 16-byte loads per lane, issued ahead of the first weight loads (loads return in
+      // issue order, so the small activation reads must not queue behind the weight stream)
+      {
+        const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
+#pragma unroll
+        for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
+      }
+      if (cnt) issue(b0, lo);
+      F::cfromx(xv, cv);
+      staged = true;
+    } else if (cnt) issue(b0, lo);
     if (!staged) {
       // activations: coalesced global -> LDS (natural order, padded unit stride) -> this lane's unit -> staged registers
       const int nq = a.K / 8;                                      // 16-byte fp16 pieces in the row
@@ -114,24 +126,23 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
         *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
       }
       __syncthreads();
-      if (uvalid) {
+      {
         uint32_t nx[NP];
 #pragma unroll
-        for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + u * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+        for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + uc * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
         F::stage(nx, xv, cv);
       }
       staged = true;
     }
     long long row = lo;
     for (long long g = 0; g < cnt; g += 2) {
-      if (g + 1 < cnt) issue(b1, row + RS);
+      issue(b1, row + RS);                                       // prefetch (clamped past the end)
       finish_group(b0, row);
       row += RS;
-      if (g + 1 < cnt) {
-        if (g + 2 < cnt) issue(b0, row + RS);
-        finish_group(b1, row);
-        row += RS;
-      }
+      if (g + 1 >= cnt) break;
+      issue(b0, row + RS);
+      finish_group(b1, row);
+      row += RS;
     }
   }
 }
@@ -196,7 +207,7 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
   const int uw = (fmt == GGML_MXFP4) ? 32 : 64;
   if (fmt == GGML_F16 && a.K % 64) return -1;
   if ((a.K / uw + 63) / 64 > 16 || a.K % 8) return -1;
-  if (((uintptr_t)a.x & 15) != 0) return -1;                       // coalesced 16-byte activation loads
+  if (((uintptr_t)a.x & 15) != 0) return a.x_staged ? tga_set_error("tga_qlinear: staged activations must be 16-byte aligned") : -1;   // 16-byte activation loads
   switch (fmt) {
     case F_Q4_0P: return launch_fast_w<F_Q4_0P>(a, s);
     case F_Q8_0P: return launch_fast_w<F_Q8_0P>(a, s);

@@ -135,25 +135,31 @@ class TransformerBlock:
     self.cache_k = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.config, self.s = c, shared
+    # staged activations need every consumer of one activation to share a type and a staged layout (K % 64, Q6_K: % 256)
+    self.staged = (not self.moe) and all(l.ggml_type in (rt.Q4_0, rt.Q8_0, rt.F16) and l.in_features % 64 == 0 and l.in_features <= 65536
+                                         for l in (self.attn_q, self.attn_output, self.ffn_gate, self.ffn_down)) \
+                  and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
 
   def __call__(self, x: Buffer, stream):
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
-    rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
-    qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream)
+    st = self.staged                                                     # producers write the consumer's staged order directly
+    rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.attn_q.ggml_type if st else 0, stream))
+    qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream, x_staged=st)
     if c.qk_norm:                                                        # full-width q/k RMSNorm before the head split (model.py:169)
       assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
-      rt.check(L.tga_rmsnorm(s.q.ptr, self.q_norm.ptr, c.n_heads * c.head_dim, c.norm_eps, None, s.q.ptr, stream))
-      rt.check(L.tga_rmsnorm(s.k.ptr, self.k_norm.ptr, c.n_kv_heads * c.head_dim, c.norm_eps, None, s.k.ptr, stream))
+      rt.check(L.tga_rmsnorm(s.q.ptr, self.q_norm.ptr, c.n_heads * c.head_dim, c.norm_eps, None, s.q.ptr, 0, stream))
+      rt.check(L.tga_rmsnorm(s.k.ptr, self.k_norm.ptr, c.n_kv_heads * c.head_dim, c.norm_eps, None, s.k.ptr, 0, stream))
     rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, stream))
-    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream)
+                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if st else 0, stream))
+    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
-    rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, stream))
     if not self.moe:
-      qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream)
-      qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream)
+      rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if st else 0, stream))
+      qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=st, stage_out_for=self.ffn_down if st else None)
+      qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
       return
+    rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
     self.ffn_gate_inp(s.xn, out=s.router, stream=stream)
@@ -203,7 +209,7 @@ class Transformer:
     rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
     for b in self.blk: b(s.x, st)
     if with_head:
-      rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, st))
+      rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
       self.output(s.xn, out=s.logits, stream=st)
       rt.check(L.tga_argmax_step(s.logits.ptr, c.vocab_size, s.am_v.ptr, s.am_i.ptr, s.state.ptr, s.prompt.ptr, s.out_tokens.ptr, self.max_new, st))
     else:

@@ -31,9 +31,12 @@ class QuantLinear:
                                   m, self.out_features, self.in_features, stream))
     return out
 
-def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None):
+def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None,
+                  x_staged: bool = False, stage_out_for: QuantLinear | None = None):
   """Several QuantLinear layers over the same activation in one launch (attn_q/k/v, ffn_gate/ffn_up).
-  epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x)."""
+  epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x).
+  x_staged: x is already in the staged order of these weights (stage_activation or a staging producer).
+  stage_out_for: write the single fp16 output in the staged order of that consumer layer."""
   nseg = len(layers)
   t, k = layers[0].ggml_type, layers[0].in_features
   assert all(l.ggml_type == t and l.in_features == k for l in layers)
@@ -44,7 +47,9 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   n = (ctypes.c_int64 * nseg)(*[l.out_features for l in layers])
   r = VP(*[b.ptr for b in resid]) if resid is not None else None
   ydt = rt.dtype_code(outs[0].dtype)
-  rt.check(rt.lib().tga_qlinear_multi(t, nseg, w, y, n, x.ptr, rt.dtype_code(x.dtype), ydt, m, k, epilogue, r, stream))
+  so = stage_out_for
+  rt.check(rt.lib().tga_qlinear_multi(t, nseg, w, y, n, x.ptr, rt.F16_STAGED if x_staged else rt.dtype_code(x.dtype), ydt, m, k, epilogue, r,
+                                      so.ggml_type if so is not None else 0, so.in_features if so is not None else 0, stream))
   return outs
 
 class ExpertWeights:
@@ -72,3 +77,9 @@ def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer,
 
 def moe_combine(y: Buffer, probs: Buffer, resid: Buffer | None, n_tokens: int, k: int, dim: int, out: Buffer, stream=None):
   rt.check(rt.lib().tga_moe_combine(y.ptr, probs.ptr, resid.ptr if resid is not None else None, n_tokens, k, dim, out.ptr, stream))
+
+def stage_activation(layer: QuantLinear, x: Buffer, out: Buffer | None = None, stream=None) -> Buffer:
+  """fp16 copy of one activation row in the order `layer`'s M = 1 GEMV consumes (a permutation of the row)."""
+  out = out if out is not None else Buffer((1, layer.in_features), np.float16)
+  rt.check(rt.lib().tga_stage_activation(layer.ggml_type, x.ptr, rt.dtype_code(x.dtype), layer.in_features, out.ptr, stream))
+  return out

@@ -7,6 +7,7 @@ import ctypes, pathlib
 import numpy as np
 
 F32, F16, Q4_0, Q8_0, Q6_K, MXFP4 = 0, 1, 2, 8, 14, 39
+F16_STAGED = 101          # activation dtype code: fp16 in the staged order of the consuming weight (tga_stage_activation)
 # {ggml_type: (elements per block, bytes per block)}: tinygrad/llm/gguf.py:20-21
 GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q6_K: (256, 210), MXFP4: (32, 17)}
 _NP_DTYPE = {F32: np.float32, F16: np.float16}
@@ -28,7 +29,8 @@ def _declare(lib):
     "tga_graph_begin": [vp], "tga_graph_end": [vp, c_void_pp], "tga_graph_launch": [vp, vp], "tga_graph_destroy": [vp],
     "tga_dequant": [i, vp, i64, vp, i, vp],
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
-    "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, vp],
+    "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, i, i64, vp],
+    "tga_stage_activation": [i, vp, i, i64, vp, vp],
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
@@ -39,8 +41,8 @@ def _declare(lib):
     "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
     "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
-    "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, vp],
-    "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
+    "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
+    "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
     "tga_advance_prompt": [vp, vp, vp],
     "tga_synth_weights": [i, vp, i64, ctypes.c_uint32, ctypes.c_float, vp],
