@@ -125,6 +125,22 @@ int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i
 /* prompt step that skips the output projection: token = prompt[pos + 1], pos += 1. */
 int tga_advance_prompt(void* state, const int* prompt, void* stream);
 
+/* All transformer blocks of one batch-1 decode step in one persistent launch (dense llama-family blocks whose seven linears share
+ * one type, Q4_0 or Q8_0): per block attn_norm -> q/k/v -> RoPE + KV append + attention -> attn_output + residual -> ffn_norm ->
+ * silu(gate) * up -> down + residual (tinygrad/llm/model.py:144-204), the same arithmetic as the per-op entry points above.
+ * layer_table: device array of n_layers records of 11 pointers {attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down
+ * (GGUF block bytes, 4-byte aligned), attn_norm, ffn_norm (float32), cache_k, cache_v (fp16 [n_kv_heads][max_ctx][head_dim])}.
+ * x: residual stream, float32 [dim], updated in place.  Workspaces: qkv float32 [(n_heads + 2 n_kv_heads) * head_dim],
+ * attn_f16 fp16 [dim], act_f16 fp16 [hidden], partials as for tga_attention_decode, sync: 1280 bytes, zero at first use (uint32
+ * arrival counters, error flag at [2]; a launch leaves the counters at zero).  The launch is sized to be resident as a
+ * whole and synchronises its workgroups through `sync`; run one such launch at a time per device.  A barrier wait that does not
+ * complete within a bounded number of polls sets the uint32 sync[2] to 1 and ends the launch with incomplete results and dirty
+ * counters (zero all 1280 bytes before the next launch).
+ * Constraints: n_heads * head_dim == dim, head_dim 64 or 128, dim and hidden multiples of 64 and <= 16384. */
+int tga_decode_layers(const void* layer_table, int n_layers, int weight_type, float* x, float* qkv, void* attn_f16, void* act_f16,
+                      float* partials, const void* state, const float* rope_table, void* sync, int dim, int hidden, int n_heads,
+                      int n_kv_heads, int head_dim, int max_ctx, float eps, void* stream);
+
 /* ---- MXFP8 MoE prefill path: extra/gemm/cdna_asm_gemm.py, extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py ---- */
 
 /* quantize_mxfp8 (cdna_asm_gemm.py:149-159): per 32 block along K, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254),

@@ -10,16 +10,20 @@ pytestmark = pytest.mark.gpu
 
 SMALL = dict(num_blocks=2, dim=256, hidden_dim=512, n_heads=4, n_kv_heads=2, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=500000.0)
 
-def _build(gpu, cfg, max_context, seed=1003):
+def _build(gpu, cfg, max_context, seed=1003, fused=True, linear_type=None):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state
+  from tinygrad_amd import runtime as rt
   c = TransformerConfig(max_context=max_context, **cfg)
-  sd = synth_state(c, seed=seed)
+  sd = synth_state(c, seed=seed, linear_type=rt.Q4_0 if linear_type is None else linear_type)
   gpu.synchronize()
   host = {k: (b.numpy(), t, shp) for k, (b, t, shp) in sd.items()}
-  return Transformer(c, sd, max_new=64), host
+  m = Transformer(c, sd, max_new=64, fused=fused)
+  assert (m.layer_table is not None) == fused
+  return m, host
 
-def test_small_model_logits_and_tokens(gpu):
-  model, host = _build(gpu, SMALL, 128)
+@pytest.mark.parametrize("fused", [True, False], ids=["one-launch", "per-op"])
+def test_small_model_logits_and_tokens(gpu, fused):
+  model, host = _build(gpu, SMALL, 128, fused=fused)
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=70)]      # spans two 64-position attention splits
   got = list(model.generate(prompt, 32, use_graph=True))
@@ -51,6 +55,30 @@ def test_graph_replay_equals_eager(gpu):
   b = list(model.generate(prompt, 16, use_graph=True))
   assert a == b
   np.testing.assert_array_equal(la, model.logits())
+
+# shapes that take the other template paths of the one-launch kernel: head_dim 128, K split over four waves (K > 4096), Q8_0
+WIDE = dict(num_blocks=2, dim=1024, hidden_dim=4608, n_heads=8, n_kv_heads=1, norm_eps=1e-5, vocab_size=512, head_dim=128, rope_theta=10000.0)
+WIDE_D = dict(num_blocks=2, dim=4352, hidden_dim=256, n_heads=34, n_kv_heads=17, norm_eps=1e-5, vocab_size=256, head_dim=128, rope_theta=10000.0)
+
+@pytest.mark.parametrize("cfg,ltype", [(WIDE, "Q4_0"), (WIDE, "Q8_0"), (WIDE_D, "Q4_0"), (SMALL, "Q8_0")], ids=["wide-hidden-q4", "wide-hidden-q8", "wide-dim-q4", "small-q8"])
+def test_one_launch_blocks_equal_per_op_path(gpu, cfg, ltype):
+  """tga_decode_layers against the per-op launches on the same weights: same greedy tokens, logits within 1e-3 (both paths
+  round activations to fp16 at the same points; fp32 summation order differs and flips a few of those roundings), KV cache contents equal to fp16 rounding of nearly equal values."""
+  from tinygrad_amd import runtime as rt
+  lt = getattr(rt, ltype)
+  a, _ = _build(gpu, cfg, 192, seed=11, fused=True, linear_type=lt)
+  b, _ = _build(gpu, cfg, 192, seed=11, fused=False, linear_type=lt)
+  rng = np.random.default_rng(3)
+  prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=67)]
+  ta = list(a.generate(prompt, 12, use_graph=True))
+  tb = list(b.generate(prompt, 12, use_graph=True))
+  la, lb = a.logits(), b.logits()
+  assert np.isfinite(la).all()
+  assert ta == tb
+  assert ol.rel_err(la, lb) <= 1e-3
+  ka, kb = a.blk[1].cache_k.numpy().astype(np.float32), b.blk[1].cache_k.numpy().astype(np.float32)
+  assert ol.rel_err(ka[:, :78], kb[:, :78]) <= 2e-3
+  assert not a.s.sync.numpy().any()                                # barrier counters back at zero, no error flag
 
 def test_attention_decode_kernel_vs_numpy(gpu):
   """tga_attention_decode alone: RoPE + fp16 KV append + GQA softmax attention at several positions."""

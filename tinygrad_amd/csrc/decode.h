@@ -1,0 +1,11 @@
+// Device-resident decode bookkeeping shared by the decode-step kernels.
+#pragma once
+#include <stdint.h>
+
+struct DecodeState {   // 16 int32
+  int pos;             // position of the token being processed
+  int token;           // current input token id
+  int step;            // tokens generated so far
+  int n_prompt;        // prompt length: while pos + 1 < n_prompt the next input token comes from the prompt, not from argmax
+  int pad[12];
+};

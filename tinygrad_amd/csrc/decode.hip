@@ -4,14 +4,7 @@
 // The position and token live in device memory so that one captured launch sequence can be replayed for every token
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
 #include "qfmt.h"
-
-struct DecodeState {   // device-resident, 16 int32
-  int pos;             // position of the token being processed
-  int token;           // current input token id
-  int step;            // tokens generated so far
-  int n_prompt;        // prompt length: while pos + 1 < n_prompt the next input token comes from the prompt, not from argmax
-  int pad[12];
-};
+#include "decode.h"
 
 // ---------------------------------------------------------------------------------------------- embedding (Q4_0 / F16 / F32 row)
 // token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized.

@@ -113,10 +113,14 @@ template <> struct Fmt<GGML_Q8_0> {
 
 enum { F_Q4_0P = 1002, F_Q8_0P = 1008 };   // block-pair formats (4-byte aligned 36 / 68 byte units)
 
-__device__ __forceinline__ u32x4 ld16_a4(const uint8_t* p) {   // 4-byte aligned 16-byte load
-  u32x4 v; __builtin_memcpy(&v, __builtin_assume_aligned(p, 4), 16); return v;
-}
-__device__ __forceinline__ uint32_t ld4_a4(const uint8_t* p) { return *(const uint32_t*)p; }
+// Weight bytes always live in global memory: the loads name that address space, so that pointers which reach a kernel through
+// a table in memory (and carry no address space of their own) still become global_load instead of FLAT instructions.
+#define TGA_GLOBAL __attribute__((address_space(1)))
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+__device__ __forceinline__ u32x4 ld16_a4(const uint8_t* p) { return *(const TGA_GLOBAL u32x4_a4*)p; }   // 4-byte aligned 16-byte load
+__device__ __forceinline__ uint32_t ld4_a4(const uint8_t* p) { return *(const TGA_GLOBAL uint32_t*)p; }
+__device__ __forceinline__ u32x4 gld16(const void* p) { return *(const TGA_GLOBAL u32x4*)p; }            // 16-byte aligned
+__device__ __forceinline__ f32x4 gld16f(const void* p) { return *(const TGA_GLOBAL f32x4*)p; }
 // 16 bytes at a 2-byte aligned address: the five enclosing aligned dwords, funnel-shifted by 0 or 16 bits per lane
 __device__ __forceinline__ u32x4 ld16_a2(const uint8_t* p, uint32_t& tail_dword, uint32_t& sh) {
   const uintptr_t a = (uintptr_t)p; sh = (uint32_t)(a & 2) * 8;

@@ -32,6 +32,21 @@ __global__ __launch_bounds__(256) void synth_q4_0_kernel(uint8_t* __restrict__ o
   }
 }
 
+// Q8_0: d = amax / 127, q = round(x / d) (ggml's reference rule)
+__global__ __launch_bounds__(256) void synth_q8_0_kernel(uint8_t* __restrict__ out, int64_t nblocks, uint32_t seed, float amp) {
+  for (int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x; b < nblocks; b += (int64_t)gridDim.x * 256) {
+    float x[32]; float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 32; j++) { x[j] = rnd_uniform(seed, (uint64_t)b * 32 + j, amp); amax = fmaxf(amax, fabsf(x[j])); }
+    const float d = amax / 127.0f, id = d != 0.f ? 1.0f / d : 0.f;
+    uint8_t* o = out + b * 34;
+    const uint32_t dh = f2h_bits(d);
+    o[0] = dh & 0xFF; o[1] = dh >> 8;
+#pragma unroll
+    for (int j = 0; j < 32; j++) o[2 + j] = (uint8_t)(int8_t)max(-127, min(127, (int)rintf(x[j] * id)));
+  }
+}
+
 __global__ __launch_bounds__(256) void synth_q6_k_kernel(uint8_t* __restrict__ out, int64_t nblocks, uint32_t seed, float amp) {
   for (int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x; b < nblocks; b += (int64_t)gridDim.x * 256) {
     uint8_t* o = out + b * 210;
@@ -91,6 +106,10 @@ extern "C" int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, u
     TGA_REQUIRE(n_elements % 32 == 0, "tga_synth_weights: Q4_0 needs a multiple of 32 elements");
     const int64_t nb = n_elements / 32; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
     synth_q4_0_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, amp);
+  } else if (ggml_type == GGML_Q8_0) {
+    TGA_REQUIRE(n_elements % 32 == 0, "tga_synth_weights: Q8_0 needs a multiple of 32 elements");
+    const int64_t nb = n_elements / 32; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
+    synth_q8_0_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, amp);
   } else if (ggml_type == GGML_Q6_K) {
     TGA_REQUIRE(n_elements % 256 == 0, "tga_synth_weights: Q6_K needs a multiple of 256 elements");
     const int64_t nb = n_elements / 256; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);

@@ -175,7 +175,10 @@ class _Shared:
     self.state = Buffer((16,), np.int32).zero_()
     self.x = Buffer((1, c.dim), f32)
     self.xn = Buffer((1, c.dim), f16)
-    self.q, self.k, self.v = Buffer((1, c.n_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32), Buffer((1, c.n_kv_heads * c.head_dim), f32)
+    nq, nkv = c.n_heads * c.head_dim, c.n_kv_heads * c.head_dim
+    self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v, contiguous for the fused block launch
+    self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
+    self.sync = Buffer((320,), np.uint32).zero_()                        # device-wide barrier counters + error flag of the fused launch
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
     self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters
     self.act = Buffer((1, c.hidden_dim), f16)
@@ -190,7 +193,7 @@ class _Shared:
     self.out_tokens = Buffer((max(1, max_new),), np.int32).zero_()
 
 class Transformer:
-  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096):
+  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096, fused: bool = True):
     self.config = c = config
     self.s = _Shared(c, max_new)
     self.max_new = max_new
@@ -202,12 +205,39 @@ class Transformer:
     self.output = QuantLinear(out[0], out[1], *out[2])
     self.stream = rt.Stream()
     self._graphs = {}
+    # one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
+    self.layer_table = self._build_layer_table() if fused else None
+
+  def _build_layer_table(self):
+    c = self.config
+    if c.num_experts or c.qk_norm or c.head_dim not in (64, 128) or c.n_heads * c.head_dim != c.dim: return None
+    if c.dim % 64 or c.hidden_dim % 64 or max(c.dim, c.hidden_dim) > 16384: return None
+    if c.n_heads // c.n_kv_heads * ((c.max_context + 63) // 64) > 1024: return None
+    t0 = self.blk[0].attn_q.ggml_type
+    if t0 not in (rt.Q4_0, rt.Q8_0): return None
+    rows = []
+    for b in self.blk:
+      lins = (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down)
+      if any(l.ggml_type != t0 or l.blocks.ptr % 4 for l in lins): return None
+      rows.append([l.blocks.ptr for l in lins] + [b.attn_norm.ptr, b.ffn_norm.ptr, b.cache_k.ptr, b.cache_v.ptr])
+    self.layer_type = t0
+    return Buffer.from_numpy(np.array(rows, dtype=np.uint64))
+
+  def check_fused(self):
+    """Raises when a fused block launch gave up on its device-wide barrier (results of that step are incomplete)."""
+    if self.layer_table is not None and int(self.s.sync.numpy()[2]) != 0:
+      self.s.sync.zero_()
+      raise RuntimeError("tga_decode_layers: a barrier wait timed out (launch not resident as a whole?)")
 
   # one token through all blocks; with_head adds output_norm + output + argmax (model.py:358-364)
   def _step(self, with_head: bool):
     c, s, L, st = self.config, self.s, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
-    for b in self.blk: b(s.x, st)
+    if self.layer_table is not None:
+      rt.check(L.tga_decode_layers(self.layer_table.ptr, c.num_blocks, self.layer_type, s.x.ptr, s.qkv.ptr, s.attn.ptr, s.act.ptr, s.attn_part.ptr,
+                                   s.state.ptr, s.rope.ptr, s.sync.ptr, c.dim, c.hidden_dim, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, c.norm_eps, st))
+    else:
+      for b in self.blk: b(s.x, st)
     if with_head:
       rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
       self.output(s.xn, out=s.logits, stream=st)
@@ -285,6 +315,7 @@ class Transformer:
       if use_graph: self._graph(False).launch()
       else: self._step(False)
     self.stream.synchronize()
+    self.check_fused()
 
   def decode_step(self, use_graph: bool = True, sync: bool = True):
     if use_graph: self._graph(True).launch()
@@ -296,6 +327,7 @@ class Transformer:
     self.prefill(tokens, use_graph)
     for i in range(max_new_tokens):
       self.decode_step(use_graph, sync=True)                          # the reference syncs once per token too (out.item(), model.py:482)
+      self.check_fused()
       yield int(self.s.out_tokens.view(4 * i, (1,), np.int32).numpy()[0])
 
   def logits(self) -> np.ndarray: return self.s.logits.numpy().reshape(-1)
