@@ -141,6 +141,11 @@ int tga_decode_layers(const void* layer_table, int n_layers, int weight_type, fl
                       float* partials, const void* state, const float* rope_table, void* sync, int dim, int hidden, int n_heads,
                       int n_kv_heads, int head_dim, int max_ctx, float eps, void* stream);
 
+/* Profiling aid for tga_decode_layers (no counterpart in the reference): buf = device buffer of >= 8 * 11 * n_layers uint64 that
+ * later launches fill with 100 MHz wall-clock stamps, [w][block][11], taken by workgroups 73 * w (w < 8) at the phase
+ * boundaries of every block; NULL = off. */
+int tga_decode_layers_trace(void* buf);
+
 /* ---- MXFP8 MoE prefill path: extra/gemm/cdna_asm_gemm.py, extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py ---- */
 
 /* quantize_mxfp8 (cdna_asm_gemm.py:149-159): per 32 block along K, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254),

@@ -28,10 +28,11 @@ struct LayersArgs {
   float* part;                    // attention split partials [n_heads][nsplit][hd + 2] + n_kv int32 arrival counters
   const DecodeState* st;
   const float* rope;              // [max_ctx][hd]
-  unsigned* sync;                 // 1280 bytes: [0] groups arrived, [1] workgroups done, [2] error flag, [32 * (1 + g)] arrivals of group g
+  unsigned* sync;                 // 320 uint32: [0] groups arrived, [1] workgroups done, [2] error flag, [32 * (1 + g)] arrivals of group g
   int dim, hidden, n_heads, n_kv, hd, max_ctx, nsplit;
   float eps, scale;
   unsigned spin_limit;
+  unsigned long long* trace;      // optional: a few workgroups record the 100 MHz wall clock at every phase boundary
 };
 
 #define LY_THREADS 256
@@ -120,7 +121,8 @@ struct GridSync {
 // ------------------------------------------------------------------------------------------------ GEMV phase pieces
 // A phase multiplies `ngroups` row groups (R rows each) by one activation row held in registers (lane <-> unit).  WK = 1: a wave
 // is a team and owns whole rows; WK = 4: the workgroup is a team, wave w owns units 64w..64w+63 and partial sums meet in LDS.
-// Each team owns a contiguous range of groups and keeps D groups of raw weight bytes in flight.
+// Each team owns a contiguous range of groups and keeps D groups of raw weight bytes in flight.  store(group, sums, owner) is
+// called by every lane of the wave that holds the sums; only the owner lane writes.
 template <int T, int R, int D, class PF>
 __device__ __forceinline__ void gemv_prefetch(typename Fmt<T>::Raw (&buf)[D * R], int g0, int g1, int uc, PF ptr) {
 #pragma unroll
@@ -163,11 +165,11 @@ __device__ __forceinline__ void gemv_run(typename Fmt<T>::Raw (&buf)[D * R], int
             float o[R];
 #pragma unroll
             for (int r = 0; r < R; r++) o[r] = __shfl(t, r, 64);
-            if (lane == 0) store(gg, o);
+            store(gg, o, lane == 0);
           }
           parity ^= 1;
         } else {
-          if (lane == 63) store(gg, acc);
+          store(gg, acc, lane == 63);
         }
       }
       int gn = gg + D; gn = gn < g1 ? gn : g1 - 1;                       // refill (clamped past the end)
@@ -175,6 +177,19 @@ __device__ __forceinline__ void gemv_run(typename Fmt<T>::Raw (&buf)[D * R], int
       for (int r = 0; r < R; r++) buf[d * R + r] = Fmt<T>::load(ptr(gn, r), uc);
     }
   }
+}
+
+// Residual rows of a team (two per group, contiguous): lane j fetches x[2 g0 + j] once at the start of the phase, so the GEMV loop
+// holds no load whose result it must wait for (a wait there would also wait for every weight row in flight).
+__device__ __forceinline__ float resid_load(const float* x, int g0, int g1, int dim, int lane) {
+  int i = 2 * g0 + (lane < 2 * (g1 - g0) ? lane : 0);
+  return cld(&x[i < dim ? i : dim - 1]);
+}
+__device__ __forceinline__ void resid_store(float* x, int g, int g0, int g1, float resid, const float* v, bool own) {
+  float r0, r1;
+  if (2 * (g1 - g0) <= 64) { r0 = __shfl(resid, 2 * (g - g0), 64); r1 = __shfl(resid, 2 * (g - g0) + 1, 64); }
+  else { r0 = cld(&x[2 * g]); r1 = cld(&x[2 * g + 1]); }
+  if (own) { cst(&x[2 * g], r0 + v[0]); cst(&x[2 * g + 1], r1 + v[1]); }
 }
 
 // contiguous share of `n` groups for team `t` of `nt`
@@ -196,12 +211,16 @@ __device__ __forceinline__ u32x4 pack8(const f32x4 lo, const f32x4 hi) {
              f2h_bits(hi.x) | (f2h_bits(hi.y) << 16), f2h_bits(hi.z) | (f2h_bits(hi.w) << 16)};
   return v;
 }
-// fp16 source, no norm
-template <int T>
+// fp16 source, no norm.  NIT = pieces per thread (K <= 2048 * NIT): all loads go out before the first LDS write.
+template <int T, int NIT>
 __device__ __forceinline__ void stage_f16(int tid, const _Float16* src, int K, int uc, uint32_t* xl, u32x4* xv, float* cv) {
   using F = Fmt<T>; constexpr int US = F::UW / 2 + 4;
   const int nq = K >> 3;
-  for (int i = tid; i < nq; i += LY_THREADS) *(u32x4*)(xl + F::unit_of(8 * i) * US + F::pair_of(8 * i)) = cld16((const u32x4*)src + i);
+  u32x4 v[NIT];
+#pragma unroll
+  for (int j = 0; j < NIT; j++) { const int i = tid + LY_THREADS * j; v[j] = cld16((const u32x4*)src + (i < nq ? i : nq - 1)); }
+#pragma unroll
+  for (int j = 0; j < NIT; j++) { const int i = tid + LY_THREADS * j; if (i < nq) *(u32x4*)(xl + F::unit_of(8 * i) * US + F::pair_of(8 * i)) = v[j]; }
   __syncthreads();
   stage_read<T>(xl, uc, xv, cv);
 }
@@ -394,14 +413,35 @@ __device__ __forceinline__ void attn_task(const LayersArgs& a, const LayerPtrs& 
   }
   __syncthreads();
   if (*last_flag) {
-    for (int idx = tid; idx < group * ns; idx += LY_THREADS) {
+    // All loads of the merge go out in one batch: (m, l) of every (head, split), then the first 2 x 16 partial values of this
+    // thread's outputs, and only then are the softmax weights formed (loads return in issue order).
+    constexpr int SC = 16;                              // splits in flight per output
+    const int nml = group * ns, nout = group * HD;
+    const int e0 = tid < nml ? tid : nml - 1;
+    const int e0h = e0 / ns, e0s = e0 - e0h * ns;
+    const float* ph0 = a.part + ((size_t)(kvh * group + e0h) * a.nsplit + e0s) * (HD + 2);
+    const float mv = cld(&ph0[HD]), lv = cld(&ph0[HD + 1]);
+    float vv[2][SC];
+    auto load_chunk = [&](int ib, int sb) {
+#pragma unroll
+      for (int k = 0; k < 2; k++) {
+        const int c = ib + LY_THREADS * k < nout ? ib + LY_THREADS * k : nout - 1;
+        const int gh = c / HD, d = c - gh * HD;
+        const float* p = a.part + (size_t)(kvh * group + gh) * a.nsplit * (HD + 2) + d;
+#pragma unroll
+        for (int j = 0; j < SC; j++) vv[k][j] = cld(&p[(size_t)min(sb + j, ns - 1) * (HD + 2)]);
+      }
+    };
+    load_chunk(tid, 0);
+    if (tid < nml) { sw[e0h * a.nsplit + e0s] = mv; sw[1024 + e0h * a.nsplit + e0s] = lv; }
+    for (int idx = tid + LY_THREADS; idx < nml; idx += LY_THREADS) {
       const int gh = idx / ns, sp = idx - gh * ns;
       const float* ph = a.part + ((size_t)(kvh * group + gh) * a.nsplit + sp) * (HD + 2);
       sw[gh * a.nsplit + sp] = cld(&ph[HD]);
       sw[1024 + gh * a.nsplit + sp] = cld(&ph[HD + 1]);
     }
     __syncthreads();
-    for (int gh = wave; gh < group; gh += 4) {
+    for (int gh = wave; gh < group; gh += 4) {            // one wave per head: m, l, then normalised weights in place
       float m = -INFINITY;
       for (int sp = lane; sp < ns; sp += 64) m = fmaxf(m, sw[gh * a.nsplit + sp]);
       m = wave_max(m);
@@ -411,18 +451,20 @@ __device__ __forceinline__ void attn_task(const LayersArgs& a, const LayerPtrs& 
       for (int sp = lane; sp < ns; sp += 64) sw[gh * a.nsplit + sp] = __expf(sw[gh * a.nsplit + sp] - m) / l;
     }
     __syncthreads();
-    for (int idx = tid; idx < group * HD; idx += LY_THREADS) {
-      const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
-      const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
-      float o = 0.f;
-      for (int s0 = 0; s0 < ns; s0 += 8) {
-        float vv[8];
+    for (int ib = tid; ib < nout; ib += 2 * LY_THREADS) {
+      float o[2] = {0.f, 0.f};
+      for (int sb = 0; sb < ns; sb += SC) {
+        if (ib != tid || sb != 0) load_chunk(ib, sb);
 #pragma unroll
-        for (int j = 0; j < 8; j++) vv[j] = cld(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
+        for (int k = 0; k < 2; k++) {
+          const int c = ib + LY_THREADS * k < nout ? ib + LY_THREADS * k : nout - 1;
+          const float* wrow = sw + (c / HD) * a.nsplit + sb;
 #pragma unroll
-        for (int j = 0; j < 8; j++) if (s0 + j < ns) o += vv[j] * sw[gh * a.nsplit + s0 + j];
+          for (int j = 0; j < SC; j++) if (sb + j < ns) o[k] += vv[k][j] * wrow[j];
+        }
       }
-      cst_h(&a.attn[head * HD + d], o);
+#pragma unroll
+      for (int k = 0; k < 2; k++) if (ib + LY_THREADS * k < nout) cst_h(&a.attn[kvh * group * HD + ib + LY_THREADS * k], o[k]);
     }
   }
   __syncthreads();                                      // LDS is reused by the next task / phase
@@ -456,6 +498,8 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
 
   GridSync gs;
   gs.init(a.sync, (unsigned)G, a.spin_limit, &flag_sync);
+  int tr_i = 0;
+#define LY_TRACE() do { if (a.trace && blockIdx.x % 73 == 0 && threadIdx.x == 0) a.trace[(blockIdx.x / 73) * 11 * a.n_layers + tr_i] = wall_clock64(); tr_i++; } while (0)
 #define LY_WAIT() do { if (!gs.wait()) { if (threadIdx.x == 0) a.sync[2] = 1u; return; } } while (0)
 
   // row ranges (identical for every block)
@@ -484,7 +528,9 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       const int tid = opaque_i(threadIdx.x), lane = tid & 63; bool uv; const int uc = unit_d(lane, uv);
       auto ptrA = [&](int g, int) { return g < nq ? L.wq + (size_t)((unsigned)g * rb_d) : (g < nq + nkv ? L.wk + (size_t)((unsigned)(g - nq) * rb_d) : L.wv + (size_t)((unsigned)(g - nq - nkv) * rb_d)); };
       stage_norm<T, WKD == 1>(tid, a.x, L.attn_norm, a.eps, a.dim, uc, dyn, red, xv, cv);
-      gemv_run<T, WKD, 1, 4>(buf, ga0, ga1, uc, uv, xv, cv, kc, ptrA, [&](int g, const float* v) { cst(&a.qkv[g], v[0]); }, part, lane, wave);
+      LY_TRACE();
+      gemv_run<T, WKD, 1, 4>(buf, ga0, ga1, uc, uv, xv, cv, kc, ptrA, [&](int g, const float* v, bool own) { if (own) cst(&a.qkv[g], v[0]); }, part, lane, wave);
+      LY_TRACE();
     }
     gs.arrive();
     // ---------------- phase B: RoPE + KV append + attention ----------------
@@ -494,12 +540,14 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       int task = blockIdx.x;
       if (task < ntasks) attn_load_tiles<HD8>(a, L, task % a.n_kv, task / a.n_kv, pos, tid, kt, vt);
       LY_WAIT();
+      LY_TRACE();
       bool first = true;
       for (; task < ntasks; task += G) {
         if (!first) attn_load_tiles<HD8>(a, L, task % a.n_kv, task / a.n_kv, pos, tid, kt, vt);
         attn_task<HD8>(a, L, task % a.n_kv, task / a.n_kv, pos, tid, kt, vt, (float*)dyn, &flag_last);
         first = false;
       }
+      LY_TRACE();
     }
     gs.arrive();
     // ---------------- phase C: x += W_o * attn ----------------
@@ -508,9 +556,12 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       auto ptrC = [&](int g, int r) { return L.wo + (size_t)((unsigned)(2 * g + r) * rb_d); };
       gemv_prefetch<T, 2, 2>(buf, gc0, gc1, uc, ptrC);
       LY_WAIT();
-      stage_f16<T>(tid, a.attn, a.dim, uc, dyn, xv, cv);
+      LY_TRACE();
+      const float resid = resid_load(a.x, gc0, gc1, a.dim, lane);
+      stage_f16<T, WKD == 1 ? 2 : 8>(tid, a.attn, a.dim, uc, dyn, xv, cv);
       gemv_run<T, WKD, 2, 2>(buf, gc0, gc1, uc, uv, xv, cv, kc, ptrC,
-                             [&](int g, const float* v) { const float r0 = cld(&a.x[2 * g]), r1 = cld(&a.x[2 * g + 1]); cst(&a.x[2 * g], r0 + v[0]); cst(&a.x[2 * g + 1], r1 + v[1]); }, part, lane, wave);
+                             [&](int g, const float* v, bool own) { resid_store(a.x, g, gc0, gc1, resid, v, own); }, part, lane, wave);
+      LY_TRACE();
     }
     gs.arrive();
     // ---------------- phase D: act = silu(W_gate * n) * (W_up * n), n = ffn_norm(x) ----------------
@@ -519,9 +570,11 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       auto ptrD = [&](int g, int r) { return (r ? L.wu : L.wg) + (size_t)((unsigned)g * rb_d); };
       gemv_prefetch<T, 2, 2>(buf, gd0, gd1, uc, ptrD);
       LY_WAIT();
+      LY_TRACE();
       stage_norm<T, WKD == 1>(tid, a.x, L.ffn_norm, a.eps, a.dim, uc, dyn, red, xv, cv);
       gemv_run<T, WKD, 2, 2>(buf, gd0, gd1, uc, uv, xv, cv, kc, ptrD,
-                             [&](int g, const float* v) { cst_h(&a.act[g], silu_f(v[0]) * v[1]); }, part, lane, wave);
+                             [&](int g, const float* v, bool own) { if (own) cst_h(&a.act[g], silu_f(v[0]) * v[1]); }, part, lane, wave);
+      LY_TRACE();
     }
     gs.arrive();
     // ---------------- phase E: x += W_down * act ----------------
@@ -530,9 +583,12 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       auto ptrE = [&](int g, int r) { return L.wd + (size_t)((unsigned)(2 * g + r) * rb_h); };
       gemv_prefetch<T, 2, 2>(buf, ge0, ge1, uc, ptrE);
       LY_WAIT();
-      stage_f16<T>(tid, a.act, a.hidden, uc, dyn, xv, cv);
+      LY_TRACE();
+      const float resid = resid_load(a.x, ge0, ge1, a.dim, lane);
+      stage_f16<T, WKH == 1 ? 2 : 8>(tid, a.act, a.hidden, uc, dyn, xv, cv);
       gemv_run<T, WKH, 2, 2>(buf, ge0, ge1, uc, uv, xv, cv, kc, ptrE,
-                             [&](int g, const float* v) { const float r0 = cld(&a.x[2 * g]), r1 = cld(&a.x[2 * g + 1]); cst(&a.x[2 * g], r0 + v[0]); cst(&a.x[2 * g + 1], r1 + v[1]); }, part, lane, wave);
+                             [&](int g, const float* v, bool own) { resid_store(a.x, g, ge0, ge1, resid, v, own); }, part, lane, wave);
+      LY_TRACE();
     }
     if (l + 1 < a.n_layers) {
       gs.arrive();
@@ -542,9 +598,11 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       gemv_prefetch<T, 1, 4>(buf, ga0, ga1, uc, ptrA);
       LY_WAIT();
     }
+    LY_TRACE();
   }
   gs.finish();
 #undef LY_WAIT
+#undef LY_TRACE
 }
 
 // ------------------------------------------------------------------------------------------------ host side
@@ -573,6 +631,12 @@ static int launch_layers_w(const LayersArgs& a, size_t lds, hipStream_t s) {
   return nu_h <= 64 ? launch_layers<T, 4, 1, HD8>(a, lds, s) : launch_layers<T, 4, 4, HD8>(a, lds, s);
 }
 
+static unsigned long long* g_layers_trace = nullptr;
+// Profiling aid: a device buffer of at least 8 * 11 * n_layers uint64 that workgroups 0, 73, 146, ... (at most 8) of later
+// tga_decode_layers launches fill with 100 MHz wall-clock stamps, [workgroup / 73][block][11]: [stage A done, A done, B start, B done, C start, C done, D start, D done, E start, E done,
+// next block ready].  NULL switches it off.
+extern "C" int tga_decode_layers_trace(void* buf) { g_layers_trace = (unsigned long long*)buf; return 0; }
+
 extern "C" int tga_decode_layers(const void* layer_table, int n_layers, int weight_type, float* x, float* qkv, void* attn_f16, void* act_f16,
                                  float* partials, const void* state, const float* rope_table, void* sync, int dim, int hidden, int n_heads,
                                  int n_kv_heads, int head_dim, int max_ctx, float eps, void* stream) {
@@ -592,6 +656,7 @@ extern "C" int tga_decode_layers(const void* layer_table, int n_layers, int weig
   a.st = (const DecodeState*)state; a.rope = rope_table; a.sync = (unsigned*)sync;
   a.dim = dim; a.hidden = hidden; a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.eps = eps; a.scale = 1.0f / sqrtf((float)head_dim);
+  a.trace = g_layers_trace;
   a.spin_limit = 1u << 20;                                             // polls before a barrier wait gives up (seconds)
   const int numax = (dim > hidden ? dim : hidden) / 64;
   const long long rb_max = (long long)numax * (weight_type == GGML_Q4_0 ? 36 : 68);
