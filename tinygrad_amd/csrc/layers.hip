@@ -12,6 +12,7 @@
 // hanging; the counters then stay dirty and the caller has to zero them.
 #include "qfmt.h"
 #include "decode.h"
+#include <stdlib.h>
 
 struct LayerPtrs {     // one record per block, in device memory (11 pointers)
   const uint8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
@@ -272,10 +273,11 @@ __device__ __forceinline__ void stage_norm(int tid, const float* x, const float*
 // waves (16 each) and every wave serving all query heads of the group: a wave's K and V tiles are 16 rows (HD8 / 4 load
 // instructions each: instruction i covers rows i*RPI + lane / HD8, RPI = 64 / HD8, and lane % HD8 picks the 16-byte piece), so
 // a lane only ever needs the 8 query values of ITS piece.  Scores: 8 FMAs per instruction, then a DPP sum over the HD8 lanes
-// of a row.  Per-wave softmax partials meet in LDS and leave as one partial per (head, split).
+// of a row.  Each run of HD8 lanes keeps its own softmax partial (its rows only); the partials meet in LDS and leave as one
+// partial per (head, split).
 // The tiles of a workgroup's first task are requested before the barrier that publishes q/k/v; the row of the current token
 // (and the clamped rows behind it) is patched in from LDS afterwards.
-#define LY_ATTN_LDS_FLOATS(HD) (6 * (HD) + 16 * ((HD) + 2) + 2048)
+#define LY_ATTN_LDS_FLOATS(HD) (6 * (HD) + 16 * (512 / (HD)) * ((HD) + 4) + 2048)
 template <int HD8>
 __device__ __forceinline__ void attn_load_tiles(const LayersArgs& a, const LayerPtrs& L, int kvh, int split, int pos, int tid, u32x4* kt, u32x4* vt) {
   constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI;
@@ -310,10 +312,15 @@ __device__ __forceinline__ void attn_task(const LayersArgs& a, const LayerPtrs& 
   const int half = HD >> 1, group = a.n_heads / a.n_kv;
   float (*qs)[HD] = (float (*)[HD])lds;                 // rotated queries of the 4 heads in flight
   float* ks = lds + 4 * HD; float* vs = ks + HD;        // rotated key / value of this token
-  float (*comb)[4][HD + 2] = (float (*)[4][HD + 2])(vs + HD);   // [head in flight][wave]: o[HD], m, l
-  float* sw = vs + HD + 16 * (HD + 2);                  // [2048] merge weights
+  constexpr int NGRP = 4 * RPI, CSTR = HD + 4;          // row runs per workgroup (wave, lane / HD8); floats per partial (16-byte multiple)
+  float* comb = vs + HD;                                // [head in flight][run]: o[HD], m, l
+  float* sw = comb + 4 * NGRP * CSTR;                   // [2048] merge weights
   const float* q = a.qkv; const float* k = a.qkv + a.n_heads * HD; const float* v = k + a.n_kv * HD;
   const int p0 = split * 64 + wave * 16;                // first position of this wave
+  // the query of the first head pass is requested together with k and v (one round trip instead of two); half <= 64 lanes
+  const int qi = lane < half ? lane : half - 1, qh = kvh * group + (wave < group ? wave : 0);
+  const float qx1 = cld(&q[qh * HD + qi]), qx2 = cld(&q[qh * HD + half + qi]);
+  const float qc = a.rope[(size_t)pos * HD + qi], qsn = a.rope[(size_t)pos * HD + half + qi];
   for (int i = tid; i < half; i += LY_THREADS) {
     const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
     const float x1 = cld(&k[kvh * HD + i]), x2 = cld(&k[kvh * HD + half + i]);
@@ -334,7 +341,9 @@ __device__ __forceinline__ void attn_task(const LayersArgs& a, const LayerPtrs& 
     for (int i = 0; i < NVI; i++) if (p0 + i * RPI + vr >= pos) { kt[i] = kcur; vt[i] = vcur; }
   }
   for (int h0 = 0; h0 < group; h0 += 4) {
-    if (h0 + wave < group) {                            // wave w rotates the query of head h0 + w
+    if (h0 == 0) {
+      if (wave < group && lane < half) { qs[wave][lane] = qx1 * qc - qx2 * qsn; qs[wave][half + lane] = qx2 * qc + qx1 * qsn; }
+    } else if (h0 + wave < group) {                     // wave w rotates the query of head h0 + w
       const int head = kvh * group + h0 + wave;
       for (int i = lane; i < half; i += 64) {
         const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
@@ -361,43 +370,44 @@ __device__ __forceinline__ void attn_task(const LayersArgs& a, const LayerPtrs& 
           sc[i] = (p0 + i * RPI + vr <= pos) ? t * a.scale : -INFINITY;
           m = fmaxf(m, sc[i]);
         }
-#pragma unroll
-        for (int off = HD8; off < 64; off <<= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        // softmax partial of this lane run (rows i * RPI + vr of the wave): no cross-lane traffic, the fold below sums the runs
         float l = 0.f;
-        float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        f32x4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < NVI; i++) {
           const float pj = (p0 + i * RPI + vr <= pos) ? __expf(sc[i] - m) : 0.f;
           l += pj;
           const u32x4 vv = vt[i];
           const half2_t v0 = as_h2(vv.x), v1 = as_h2(vv.y), v2 = as_h2(vv.z), v3 = as_h2(vv.w);
-          o[0] += pj * (float)v0.x; o[1] += pj * (float)v0.y; o[2] += pj * (float)v1.x; o[3] += pj * (float)v1.y;
-          o[4] += pj * (float)v2.x; o[5] += pj * (float)v2.y; o[6] += pj * (float)v3.x; o[7] += pj * (float)v3.y;
+          o0.x += pj * (float)v0.x; o0.y += pj * (float)v0.y; o0.z += pj * (float)v1.x; o0.w += pj * (float)v1.y;
+          o1.x += pj * (float)v2.x; o1.y += pj * (float)v2.y; o1.z += pj * (float)v3.x; o1.w += pj * (float)v3.y;
         }
-        // sum the RPI lane groups (rows) that hold the same piece; l counts every row once
-#pragma unroll
-        for (int off = HD8; off < 64; off <<= 1) {
-          l += __shfl_xor(l, off, 64);
-#pragma unroll
-          for (int j = 0; j < 8; j++) o[j] += __shfl_xor(o[j], off, 64);
-        }
-        float* cw = comb[hh][wave];
-        if (lane < HD8) {
-#pragma unroll
-          for (int j = 0; j < 8; j++) cw[lane * 8 + j] = o[j];
-        }
-        if (lane == 0) { cw[HD] = m; cw[HD + 1] = l; }
+        float* cw = comb + (size_t)(hh * NGRP + wave * RPI + vr) * CSTR;
+        *(f32x4*)(cw + vp * 8) = o0; *(f32x4*)(cw + vp * 8 + 4) = o1;
+        if (vp == 0) { cw[HD] = m; cw[HD + 1] = l; }
       }
     }
     __syncthreads();
-    if (h0 + wave < group) {                            // wave w folds the four wave partials of head h0 + w into the split partial
+    if (h0 + wave < group) {                            // wave w folds the row-run partials of head h0 + w into the split partial
       const int head = kvh * group + h0 + wave;
-      const float m0 = comb[wave][0][HD], m1 = comb[wave][1][HD], m2 = comb[wave][2][HD], m3 = comb[wave][3][HD];
-      const float m = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));            // wave 0 always holds a valid position: m is finite
-      const float w0 = __expf(m0 - m), w1 = __expf(m1 - m), w2 = __expf(m2 - m), w3 = __expf(m3 - m);
+      const float* cb = comb + (size_t)wave * NGRP * CSTR;
+      float m = -INFINITY;                              // the first run of wave 0 always holds a valid position: m is finite
+#pragma unroll
+      for (int g = 0; g < NGRP; g++) m = fmaxf(m, cb[g * CSTR + HD]);
+      float l = 0.f, od[HD / 64];
+#pragma unroll
+      for (int j = 0; j < HD / 64; j++) od[j] = 0.f;
+#pragma unroll
+      for (int g = 0; g < NGRP; g++) {
+        const float wg = __expf(cb[g * CSTR + HD] - m);
+        l += wg * cb[g * CSTR + HD + 1];
+#pragma unroll
+        for (int j = 0; j < HD / 64; j++) od[j] += wg * cb[g * CSTR + lane + 64 * j];
+      }
       float* po = a.part + ((size_t)head * a.nsplit + split) * (HD + 2);
-      for (int d = lane; d < HD; d += 64) cst(&po[d], comb[wave][0][d] * w0 + comb[wave][1][d] * w1 + comb[wave][2][d] * w2 + comb[wave][3][d] * w3);
-      if (lane == 0) { cst(&po[HD], m); cst(&po[HD + 1], comb[wave][0][HD + 1] * w0 + comb[wave][1][HD + 1] * w1 + comb[wave][2][HD + 1] * w2 + comb[wave][3][HD + 1] * w3); }
+#pragma unroll
+      for (int j = 0; j < HD / 64; j++) cst(&po[lane + 64 * j], od[j]);
+      if (lane == 0) { cst(&po[HD], m); cst(&po[HD + 1], l); }
     }
     __syncthreads();
   }
@@ -499,7 +509,7 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
   GridSync gs;
   gs.init(a.sync, (unsigned)G, a.spin_limit, &flag_sync);
   int tr_i = 0;
-#define LY_TRACE() do { if (a.trace && blockIdx.x % 73 == 0 && threadIdx.x == 0) a.trace[(blockIdx.x / 73) * 11 * a.n_layers + tr_i] = wall_clock64(); tr_i++; } while (0)
+#define LY_TRACE() do { if (a.trace && threadIdx.x == 0) { if (blockIdx.x % 73 == 0) a.trace[(blockIdx.x / 73) * 11 * a.n_layers + tr_i] = wall_clock64(); } tr_i++; } while (0)
 #define LY_WAIT() do { if (!gs.wait()) { if (threadIdx.x == 0) a.sync[2] = 1u; return; } } while (0)
 
   // row ranges (identical for every block)
@@ -510,7 +520,8 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
   team_range(a.dim / 2, team_h, nteam_h, ge0, ge1);      // down: two rows per group
   const int ns = (pos >> 6) + 1, ntasks = a.n_kv * ns;
 
-  Raw buf[4];
+  constexpr int NB = 4, NB2 = NB / 2;                   // weight rows in flight per wave (six measured no faster)
+  Raw buf[NB];
   u32x4 xv[F::XV]; float cv[F::NG];
   // this lane's unit (clamped) for K = dim / K = hidden, from a per-phase opaque lane id
   auto unit_d = [&](int lane, bool& valid) { const int u = (WKD == 1) ? lane : wave * 64 + lane; valid = u < nu_d; return valid ? u : nu_d - 1; };
@@ -519,7 +530,7 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
     const LayerPtrs L0 = load_layer(a.layers, 0);
     bool uv; const int uc = unit_d(lane0, uv);
     auto ptrA = [&](int g, int) { return g < nq ? L0.wq + (size_t)((unsigned)g * rb_d) : (g < nq + nkv ? L0.wk + (size_t)((unsigned)(g - nq) * rb_d) : L0.wv + (size_t)((unsigned)(g - nq - nkv) * rb_d)); };
-    gemv_prefetch<T, 1, 4>(buf, ga0, ga1, uc, ptrA);
+    gemv_prefetch<T, 1, NB>(buf, ga0, ga1, uc, ptrA);
   }
   for (int l = 0; l < a.n_layers; l++) {
     const LayerPtrs L = load_layer(a.layers, l);
@@ -529,7 +540,7 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       auto ptrA = [&](int g, int) { return g < nq ? L.wq + (size_t)((unsigned)g * rb_d) : (g < nq + nkv ? L.wk + (size_t)((unsigned)(g - nq) * rb_d) : L.wv + (size_t)((unsigned)(g - nq - nkv) * rb_d)); };
       stage_norm<T, WKD == 1>(tid, a.x, L.attn_norm, a.eps, a.dim, uc, dyn, red, xv, cv);
       LY_TRACE();
-      gemv_run<T, WKD, 1, 4>(buf, ga0, ga1, uc, uv, xv, cv, kc, ptrA, [&](int g, const float* v, bool own) { if (own) cst(&a.qkv[g], v[0]); }, part, lane, wave);
+      gemv_run<T, WKD, 1, NB>(buf, ga0, ga1, uc, uv, xv, cv, kc, ptrA, [&](int g, const float* v, bool own) { if (own) cst(&a.qkv[g], v[0]); }, part, lane, wave);
       LY_TRACE();
     }
     gs.arrive();
@@ -554,12 +565,12 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
     {
       const int tid = opaque_i(threadIdx.x), lane = tid & 63; bool uv; const int uc = unit_d(lane, uv);
       auto ptrC = [&](int g, int r) { return L.wo + (size_t)((unsigned)(2 * g + r) * rb_d); };
-      gemv_prefetch<T, 2, 2>(buf, gc0, gc1, uc, ptrC);
+      gemv_prefetch<T, 2, NB2>(buf, gc0, gc1, uc, ptrC);
       LY_WAIT();
       LY_TRACE();
       const float resid = resid_load(a.x, gc0, gc1, a.dim, lane);
       stage_f16<T, WKD == 1 ? 2 : 8>(tid, a.attn, a.dim, uc, dyn, xv, cv);
-      gemv_run<T, WKD, 2, 2>(buf, gc0, gc1, uc, uv, xv, cv, kc, ptrC,
+      gemv_run<T, WKD, 2, NB2>(buf, gc0, gc1, uc, uv, xv, cv, kc, ptrC,
                              [&](int g, const float* v, bool own) { resid_store(a.x, g, gc0, gc1, resid, v, own); }, part, lane, wave);
       LY_TRACE();
     }
@@ -568,11 +579,11 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
     {
       const int tid = opaque_i(threadIdx.x), lane = tid & 63; bool uv; const int uc = unit_d(lane, uv);
       auto ptrD = [&](int g, int r) { return (r ? L.wu : L.wg) + (size_t)((unsigned)g * rb_d); };
-      gemv_prefetch<T, 2, 2>(buf, gd0, gd1, uc, ptrD);
+      gemv_prefetch<T, 2, NB2>(buf, gd0, gd1, uc, ptrD);
       LY_WAIT();
       LY_TRACE();
       stage_norm<T, WKD == 1>(tid, a.x, L.ffn_norm, a.eps, a.dim, uc, dyn, red, xv, cv);
-      gemv_run<T, WKD, 2, 2>(buf, gd0, gd1, uc, uv, xv, cv, kc, ptrD,
+      gemv_run<T, WKD, 2, NB2>(buf, gd0, gd1, uc, uv, xv, cv, kc, ptrD,
                              [&](int g, const float* v, bool own) { if (own) cst_h(&a.act[g], silu_f(v[0]) * v[1]); }, part, lane, wave);
       LY_TRACE();
     }
@@ -581,12 +592,12 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
     {
       const int tid = opaque_i(threadIdx.x), lane = tid & 63; bool uv; const int uc = unit_h(lane, uv);
       auto ptrE = [&](int g, int r) { return L.wd + (size_t)((unsigned)(2 * g + r) * rb_h); };
-      gemv_prefetch<T, 2, 2>(buf, ge0, ge1, uc, ptrE);
+      gemv_prefetch<T, 2, NB2>(buf, ge0, ge1, uc, ptrE);
       LY_WAIT();
       LY_TRACE();
       const float resid = resid_load(a.x, ge0, ge1, a.dim, lane);
       stage_f16<T, WKH == 1 ? 2 : 8>(tid, a.act, a.hidden, uc, dyn, xv, cv);
-      gemv_run<T, WKH, 2, 2>(buf, ge0, ge1, uc, uv, xv, cv, kc, ptrE,
+      gemv_run<T, WKH, 2, NB2>(buf, ge0, ge1, uc, uv, xv, cv, kc, ptrE,
                              [&](int g, const float* v, bool own) { resid_store(a.x, g, ge0, ge1, resid, v, own); }, part, lane, wave);
       LY_TRACE();
     }
@@ -595,7 +606,7 @@ __global__ __launch_bounds__(LY_THREADS, 2) void decode_layers_kernel(const Laye
       const int lane = opaque_i(lane0); bool uv; const int uc = unit_d(lane, uv);
       const LayerPtrs Ln = load_layer(a.layers, l + 1);
       auto ptrA = [&](int g, int) { return g < nq ? Ln.wq + (size_t)((unsigned)g * rb_d) : (g < nq + nkv ? Ln.wk + (size_t)((unsigned)(g - nq) * rb_d) : Ln.wv + (size_t)((unsigned)(g - nq - nkv) * rb_d)); };
-      gemv_prefetch<T, 1, 4>(buf, ga0, ga1, uc, ptrA);
+      gemv_prefetch<T, 1, NB>(buf, ga0, ga1, uc, ptrA);
       LY_WAIT();
     }
     LY_TRACE();
@@ -617,7 +628,8 @@ static int launch_layers(const LayersArgs& a, size_t lds, hipStream_t s) {
     TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
     TGA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, LY_THREADS, 64 * 1024));
     TGA_REQUIRE(per_cu >= 1, "tga_decode_layers: the kernel does not fit on a CU");
-    grid = p.multiProcessorCount * (per_cu >= 2 ? 2 : 1);              // every workgroup resident at once
+    const char* e = getenv("TGA_LAYERS_WGPC");
+    grid = p.multiProcessorCount * ((per_cu >= 2 && !(e && e[0] == '1')) ? 2 : 1);              // every workgroup resident at once
   }
   kern<<<grid, LY_THREADS, lds, s>>>(a);
   TGA_LAUNCH_CHECK();
