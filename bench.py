@@ -4,8 +4,10 @@
 A step is one decoded token.  Random-init weights are written on the GPU as GGUF blocks (Q4_0 linears and embedding, Q6_K
 lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the model itself, then --warmup + --steps tokens
 are decoded greedily, one captured launch sequence per token with a host sync per token (as the reference's generate loop does).
-Prints ONE JSON line: tok/s, the roofline of the dominant kernel (the fused ffn_gate/ffn_up dequant-GEMV) from HIP-event
-timings taken live, and a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the same weights)."""
+Prints ONE JSON line: tok/s, the roofline of the dominant kernel (the one-launch kernel that runs all 32 blocks of a token:
+every Q4_0 dequant-GEMV, RMSNorm, RoPE + KV append + attention) from HIP-event timings taken live, the same figures for the
+per-op dequant-GEMV kernels on the same weights, and a CPU baseline (C restatement of the reference arithmetic on a bounded
+sample of the same weights)."""
 import argparse, json, os, sys, time
 import numpy as np
 
@@ -56,6 +58,7 @@ def main():
   ap.add_argument("--layers", type=int, default=32, help="reduce only for smoke runs; the reported config then says so")
   ap.add_argument("--no-cpu", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="eager launches instead of graph replay (for kernel-trace profiling)")
+  ap.add_argument("--per-op", action="store_true", help="one launch per op instead of the one-launch block kernel")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py: this build measures one GPU only (no collectives, no sharding in this run); use --gpus 1", file=sys.stderr)
@@ -65,11 +68,11 @@ def main():
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
   rt.init(0)
   cfg = dict(LLAMA3_8B); cfg["num_blocks"] = args.layers
-  max_new = args.steps + args.warmup + 8
+  max_new = args.steps + args.warmup + 16                    # + the eager steps of the per-kernel timing below
   max_ctx = ((args.prefill + max_new + 63) // 64) * 64
   c = TransformerConfig(max_context=max_ctx, **cfg)
   sd = synth_state(c, seed=1003)
-  model = Transformer(c, sd, max_new=max_new)
+  model = Transformer(c, sd, max_new=max_new, fused=not args.per_op)
   rt.synchronize()
 
   rng = np.random.default_rng(1003)
@@ -85,14 +88,37 @@ def main():
   ms_per_step = dt / args.steps * 1e3
   tok_s = args.steps / dt
 
-  # ---- live per-kernel timing of the dominant kernel: HIP events around every fused gate/up launch of a few eager steps ----
-  from tinygrad_amd.nn import qlinear_multi
+  # ---- live timing of the dominant kernel: HIP events (on the model's stream) around the one-launch block kernel of eager steps ----
   st = model.stream.handle
   L = rt.lib()
-  evs = [(rt.Event(), rt.Event()) for _ in range(len(model.blk))]
+  fused_us, phase = [], None
+  if model.layer_table is not None:
+    s_ = model.s
+    tb = rt.Buffer((8 * 11 * c.num_blocks,), np.uint64).zero_()
+    for it in range(8):
+      rt.check(L.tga_embed_row(model.token_embd.ptr, model.embd_type, c.dim, s_.state.ptr, s_.x.ptr, st))
+      if it == 7: rt.check(L.tga_decode_layers_trace(tb.ptr))
+      e0, e1 = rt.Event(), rt.Event(); e0.record(st)
+      rt.check(L.tga_decode_layers(model.layer_table.ptr, c.num_blocks, model.layer_type, s_.x.ptr, s_.qkv.ptr, s_.attn.ptr, s_.act.ptr, s_.attn_part.ptr,
+                                   s_.state.ptr, s_.rope.ptr, s_.sync.ptr, c.dim, c.hidden_dim, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, c.norm_eps, st))
+      e1.record(st)
+      rt.check(L.tga_advance_prompt(s_.state.ptr, s_.prompt.ptr, st))
+      model.stream.synchronize()
+      fused_us.append(e0.elapsed_ms(e1) * 1e3)
+    rt.check(L.tga_decode_layers_trace(None))
+    model.check_fused()
+    if c.num_blocks > 2:
+      # wall-clock stamps (100 MHz) of workgroups 0, 73, ... at the phase boundaries of every block: time from the start of a
+      # phase (all workgroups past the barrier) to the last sampled workgroup finishing it, median over the inner blocks
+      T = tb.numpy().astype(np.int64).reshape(8, c.num_blocks, 11)[:, 1:-1]
+      span = lambda i0, i1: float(np.median(T[:, :, i1].max(0) - T[:, :, i0].min(0)) * 0.01)
+      phase = {"qkv_after_staging_us": round(span(0, 1), 2),
+               "attention_us": round(span(2, 3), 2), "attn_output_us": round(span(4, 5), 2), "gate_up_us": round(span(6, 7), 2), "down_us": round(span(8, 9), 2),
+               "block_us": round(float(np.median(np.diff(T[0, :, 0])) * 0.01), 2)}
+  # ---- the per-op dequant-GEMV kernels on the same weights: HIP events around each launch of a few eager per-op steps ----
+  from tinygrad_amd.nn import qlinear_multi
   durs = {"gate_up": [], "down": [], "qkv": [], "attn_output": []}
   for _ in range(3):
-    # a plain eager token step, with event pairs around the kernels of interest
     rt.check(L.tga_embed_row(model.token_embd.ptr, model.embd_type, c.dim, model.s.state.ptr, model.s.x.ptr, st))
     per = {k: [] for k in durs}
     for b in model.blk:
@@ -123,9 +149,9 @@ def main():
          "attn_output": b0.attn_output.nbytes + c.dim * 2 + c.dim * 8}
   kern = {k: {"avg_us": round(float(np.mean(v)), 3), "alg_bytes": int(alg[k]), "GBps": round(alg[k] / np.mean(v) / 1e3, 1),
               "frac_hbm": round(alg[k] / np.mean(v) / 1e3 / HBM_PEAK_GBS, 4)} for k, v in durs.items()}
-  dom = kern["gate_up"]
   wbytes = model.weight_bytes_per_token()
-  kv_bytes = 2 * c.num_blocks * c.n_kv_heads * c.head_dim * (args.prefill + args.warmup + args.steps // 2) * 2
+  ctx_mid = args.prefill + args.warmup + args.steps // 2
+  kv_bytes = 2 * c.num_blocks * c.n_kv_heads * c.head_dim * ctx_mid * 2
   out = {
     "metric": "Q4_0 8B-arch decode tok/s @bs1; dequant-GEMV GB/s as % of HBM peak", "value": round(tok_s, 2), "unit": "tok/s",
     "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
@@ -134,10 +160,25 @@ def main():
                            f"fp16 KV prefilled with {args.prefill} random ids, greedy decode", "device": rt.device_name(),
                "weight_bytes_per_token": int(wbytes), "stream_GBps_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
                "frac_hbm_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
-    "roofline": {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU> (fused ffn_gate+ffn_up, 2x14336x4096)",
-                 "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"], "traffic": None,
-                 "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"], "other_kernels": {k: v for k, v in kern.items() if k != "gate_up"}},
   }
+  if fused_us:
+    # algorithmic bytes of one launch: the seven Q4_0 matrices of every block + the fp16 K/V rows read at this context length
+    blk_w = sum(l.nbytes for b in model.blk for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down))
+    ctx_now = args.prefill + args.warmup + args.steps
+    alg_f = blk_w + 2 * c.num_blocks * c.n_kv_heads * c.head_dim * ctx_now * 2
+    avg = float(np.mean(fused_us[1:]))
+    out["roofline"] = {"bound": "hbm", "kernel": f"decode_layers_kernel<Q4_0 pair> (all {c.num_blocks} blocks of one token in one persistent launch: 4 dequant-GEMV phases + attention per block)",
+                       "achieved": round(alg_f / avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_f / avg / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                       "avg_launch_us": round(avg, 2), "alg_bytes_per_launch": int(alg_f), "phase_us_inside_launch": phase,
+                       "per_op_kernels": kern}
+    if phase:
+      out["roofline"]["gate_up_phase_GBps"] = round(alg["gate_up"] / phase["gate_up_us"] / 1e3, 1)
+      out["roofline"]["down_phase_GBps"] = round(alg["down"] / phase["down_us"] / 1e3, 1)
+  else:
+    dom = kern["gate_up"]
+    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU> (fused ffn_gate+ffn_up, 2x14336x4096)",
+                       "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"], "traffic": None,
+                       "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"], "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
   if not args.no_cpu:
     out["cpu_baseline"] = cpu_baseline(model, cfg)
   print(json.dumps(out))

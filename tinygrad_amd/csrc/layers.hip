@@ -12,7 +12,6 @@
 // hanging; the counters then stay dirty and the caller has to zero them.
 #include "qfmt.h"
 #include "decode.h"
-#include <stdlib.h>
 
 struct LayerPtrs {     // one record per block, in device memory (11 pointers)
   const uint8_t *wq, *wk, *wv, *wo, *wg, *wu, *wd;
@@ -628,8 +627,7 @@ static int launch_layers(const LayersArgs& a, size_t lds, hipStream_t s) {
     TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
     TGA_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, LY_THREADS, 64 * 1024));
     TGA_REQUIRE(per_cu >= 1, "tga_decode_layers: the kernel does not fit on a CU");
-    const char* e = getenv("TGA_LAYERS_WGPC");
-    grid = p.multiProcessorCount * ((per_cu >= 2 && !(e && e[0] == '1')) ? 2 : 1);              // every workgroup resident at once
+    grid = p.multiProcessorCount * (per_cu >= 2 ? 2 : 1);              // every workgroup resident at once
   }
   kern<<<grid, LY_THREADS, lds, s>>>(a);
   TGA_LAUNCH_CHECK();
