@@ -173,6 +173,10 @@ int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_
 /* clamped interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98), bf16 (rows, 2I) -> (rows, I). */
 int tga_swiglu_interleaved(const void* h_bf16, int64_t rows, int two_inter, float limit, float alpha, void* y_bf16, void* stream);
 
+/* Measured peak of the scaled FP8 MFMA (method of extra/mmapeak/mmapeak.py:16-52,97-109): n_workgroups x 4 waves each issue
+ * loops x 200 register-only v_mfma_scale_f32_16x16x128_f8f6f4; FLOPs = n_workgroups * 4 * loops * 200 * 65536; the caller times it. */
+int tga_mfma_peak(int n_workgroups, int loops, float* scratch, void* stream);
+
 /* ---- synthetic-model writer (no counterpart in the reference, whose weights always come from GGUF files): fills `out` with
  * n_elements random-init weights U(-amp, amp) (nn.Linear's init range, tinygrad/nn/__init__.py:173-174) already quantized to
  * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule; TGA_F16: plain fp16 cast); TGA_F32 fills the

@@ -1,0 +1,155 @@
+"""Kernel-level measurements on one MI355X for the configurations that are not the headline benchmark:
+  config 1  Q4_0 4096x4096 GEMV, batch 1
+  config 2  Q8_0 / Q6_K small-batch sweep, M in {1, 2, 4, 8}
+  config 4  OLMoE-architecture MXFP4 expert decode, batch 1 (tok/s and expert-GEMV GB/s)
+  config 5  MXFP8 grouped GEMM at T = 4096, E = 128, k = 8 with Zipf routing (MFMA utilisation and GB/s), plus the measured
+            register-only peak of the scaled FP8 MFMA
+
+    python -m tinygrad_amd.benchmarks [--config N ...]        prints one JSON object per measurement
+
+Timing: HIP events around >= 100 back-to-back launches; weights are rotated over enough distinct copies to exceed the 256 MB
+Infinity Cache (a single matrix that is re-read every launch would be served from that cache, not from HBM).  Weights for
+configs 1 / 2 / 4 are written on the GPU as valid GGUF blocks by tga_synth_weights; timing does not depend on their values (the
+parity tests use the seeded host generators)."""
+from __future__ import annotations
+import argparse, json, sys
+import numpy as np
+from tinygrad_amd import runtime as rt
+from tinygrad_amd.runtime import Buffer
+from tinygrad_amd.nn import QuantLinear, ExpertWeights
+
+HBM_PEAK_GBS = 8000.0
+MFMA_FP8_PEAK_TFLOPS = 5000.0
+MALL_BYTES = 256 << 20
+
+def _time_launches(fn, n_variants: int, iters: int, stream: rt.Stream) -> float:
+  """Average microseconds per call of fn(i % n_variants) over `iters` back-to-back launches (one warm-up pass first)."""
+  for i in range(n_variants): fn(i)
+  stream.synchronize()
+  e0, e1 = rt.Event(), rt.Event()
+  e0.record(stream.handle)
+  for i in range(iters): fn(i % n_variants)
+  e1.record(stream.handle); e1.synchronize()
+  return e0.elapsed_ms(e1) * 1e3 / iters
+
+def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
+  nel, nby = rt.GGML_QUANT[ggml_type]
+  wbytes = n * (k // nel) * nby
+  copies = max(2, -(-int(1.25 * MALL_BYTES) // wbytes))
+  big = Buffer((copies * wbytes,), np.uint8)
+  for c in range(copies): rt.check(rt.lib().tga_synth_weights(ggml_type, big.ptr + c * wbytes, n * k, 1000 + c, k ** -0.5, None))
+  rt.synchronize()
+  lins = [QuantLinear(big.view(c * wbytes, (wbytes,), np.uint8), ggml_type, n, k) for c in range(copies)]
+  rng = np.random.default_rng(1002)
+  x = Buffer.from_numpy(rng.standard_normal((m, k)).astype(np.float16)); y = Buffer((m, n), np.float16)
+  s = rt.Stream()
+  us = _time_launches(lambda i: lins[i](x, out=y, stream=s.handle), copies, iters, s)
+  alg = wbytes + m * k * 2 + m * n * 2
+  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
+  return {"case": f"{name} {n}x{k} M={m}", "avg_us": round(us, 2), "alg_bytes": alg, "GBps": round(alg / us / 1e3, 1),
+          "frac_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_rotated": copies, "launches": iters}
+
+def config1(): return [dict(config=1, **gemv_case(rt.Q4_0, 4096, 4096, 1, iters=400))]
+
+def config2():
+  out = []
+  for t, n, k in ((rt.Q8_0, 4096, 4096), (rt.Q8_0, 14336, 4096), (rt.Q8_0, 4096, 14336), (rt.Q6_K, 128256, 4096)):
+    for m in (1, 2, 4, 8): out.append(dict(config=2, **gemv_case(t, n, k, m, iters=100 if n > 100000 else 200)))
+  return out
+
+def config4(steps: int = 64, ctx: int = 512):
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
+  import time
+  c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **OLMOE)
+  model = Transformer(c, synth_state_moe(c, seed=1004), max_new=steps + 16)
+  rt.synchronize()
+  rng = np.random.default_rng(1004)
+  model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)], True)
+  for _ in range(8): model.decode_step(True)
+  rt.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps): model.decode_step(True)
+  rt.synchronize()
+  dt = (time.perf_counter() - t0) / steps
+  expert_bytes = c.num_blocks * c.num_experts_per_tok * sum(e.expert_nbytes for e in (model.blk[0].ffn_gate_exps, model.blk[0].ffn_up_exps, model.blk[0].ffn_down_exps))
+  res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, graph replay + sync per token)",
+          "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "expert_bytes_per_token": expert_bytes, "weight_bytes_per_token": model.weight_bytes_per_token(),
+          "weight_GBps_over_step": round(model.weight_bytes_per_token() / dt / 1e9, 1)}]
+  # the expert GEMVs alone: B tokens x 8 experts, gate/up fused then down, distinct experts per slot, layers rotated
+  k, s = c.num_experts_per_tok, rt.Stream()
+  for B in (1, 2, 4, 8):
+    sel_host = np.stack([rng.permutation(c.num_experts)[:k] for _ in range(B)]).astype(np.int32).reshape(-1)
+    sel = Buffer.from_numpy(sel_host)
+    x = Buffer.from_numpy(rng.standard_normal((B, c.dim)).astype(np.float16))
+    act, y = Buffer((B * k, c.hidden_dim), np.float16), Buffer((B * k, c.dim), np.float32)
+    blks = model.blk
+    def run(i):
+      b = blks[i]
+      b.ffn_gate_exps(sel, x, act, jobs_per_x_row=k, up=b.ffn_up_exps, stream=s.handle)
+      b.ffn_down_exps(sel, act, y, jobs_per_x_row=1, stream=s.handle)
+    us = _time_launches(run, len(blks), 320, s)
+    per_e = sum(e.expert_nbytes for e in (blks[0].ffn_gate_exps, blks[0].ffn_up_exps, blks[0].ffn_down_exps))
+    nbytes = B * k * per_e                                                  # every (token, slot) job streams its expert once
+    res.append({"config": 4, "case": f"expert GEMVs of one layer, B={B} ({B * k} jobs, {len(np.unique(sel_host))} distinct experts)", "avg_us": round(us, 2),
+                "alg_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+  return res
+
+def mfma_peak() -> dict:
+  L, s = rt.lib(), rt.Stream()
+  scratch = Buffer((64,), np.float32).zero_()
+  wgs, loops = 256 * 4, 2000
+  rt.check(L.tga_mfma_peak(wgs, 10, scratch.ptr, s.handle)); s.synchronize()
+  e0, e1 = rt.Event(), rt.Event(); e0.record(s.handle)
+  rt.check(L.tga_mfma_peak(wgs, loops, scratch.ptr, s.handle))
+  e1.record(s.handle); e1.synchronize()
+  ms = e0.elapsed_ms(e1)
+  flops = wgs * 4 * loops * 200 * 65536
+  return {"config": 5, "case": "register-only v_mfma_scale_f32_16x16x128_f8f6f4 (1024 workgroups x 4 waves x 2000 x 200)", "ms": round(ms, 3),
+          "TFLOPs": round(flops / ms / 1e9, 1), "frac_of_5_PFLOPs": round(flops / ms / 1e9 / MFMA_FP8_PEAK_TFLOPS, 4)}
+
+def config5():
+  """Grouped MXFP8 GEMM of the MoE prefill: T = 4096 tokens, E = 128, k = 8, d = 2048, gate/up (128, 1536, 2048), down (128, 2048, 768)."""
+  from tinygrad_amd import moe
+  L = rt.lib()
+  T, E, k, D, I2, I = 4096, 128, 8, 2048, 1536, 768
+  rng = np.random.default_rng(1005)
+  # Zipf(1.1) expert popularity over a fixed random permutation, no duplicate expert within a token: logits = log(popularity) + Gumbel
+  pop = 1.0 / np.arange(1, E + 1) ** 1.1
+  logits = (np.log(pop[rng.permutation(E)])[None, :] + rng.gumbel(size=(T, E))).astype(np.float32)
+  s = rt.Stream()
+  r = moe.route(Buffer.from_numpy(logits), k, E, stream=s.handle)
+  s.synchronize()
+  off = r.off.numpy(); counts = r.counts.numpy()
+  m_used = int(off[-1])
+  def rand_mx(shape_rows, K):
+    q = rng.integers(0, 256, size=(shape_rows, K), dtype=np.uint8); q[(q & 0x7F) == 0x7F] = 0x38      # no E4M3 NaN codes
+    e8 = rng.integers(121, 126, size=(shape_rows, K // 32), dtype=np.uint8)
+    return Buffer.from_numpy(q), Buffer.from_numpy(e8)
+  res = [mfma_peak()]
+  for name, N, K in (("gate/up", I2, D), ("down", D, I)):
+    wq, we = rand_mx(E * N, K)
+    xq, xe = rand_mx(r.m_l, K)
+    out = Buffer((r.m_l, N), np.uint16)
+    fn = lambda i: rt.check(L.tga_grouped_mxfp8_gemm(out.ptr, xq.ptr, wq.ptr, None, None, xe.ptr, we.ptr, r.off.ptr, r.m_l, N, K, E, s.handle))
+    us = _time_launches(fn, 1, 50, s)
+    flops_unpadded = 2 * T * k * N * K
+    flops_padded = 2 * m_used * N * K
+    nbytes = E * N * K + E * N * K // 32 + T * k * K + T * k * K // 32 + T * k * N * 2
+    res.append({"config": 5, "case": f"grouped MXFP8 GEMM {name}: {T * k} routed rows ({m_used} after 256-row padding), N={N}, K={K}, E={E}, Zipf(1.1) routing "
+                f"(busiest expert {int(counts.max())} rows, idlest {int(counts.min())})", "avg_us": round(us, 1),
+                "TFLOPs_unpadded": round(flops_unpadded / us / 1e6, 1), "mfma_utilisation_vs_5_PFLOPs": round(flops_unpadded / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 4),
+                "TFLOPs_with_padding_rows": round(flops_padded / us / 1e6, 1), "alg_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+  return res
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5])
+  args = ap.parse_args()
+  rt.init(0)
+  print(json.dumps({"device": rt.device_name()}), flush=True)
+  for cfg in args.config:
+    for row in {1: config1, 2: config2, 4: config4, 5: config5}[cfg](): print(json.dumps(row), flush=True)
+
+if __name__ == "__main__":
+  main()

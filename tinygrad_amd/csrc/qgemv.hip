@@ -31,15 +31,20 @@ __device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs
   constexpr int NP = F::UW / 2;
   for (int i = threadIdx.x; i < M * cu; i += QG_THREADS) {
     const int m = i / cu, ul = i - m * cu, u = u0 + ul;
+    // four consecutive pairs (8 activations) of a unit are contiguous in every format: 16-byte (fp16) / 2 x 16-byte (fp32) loads
     uint32_t nx[NP];
     if (a.x_f32) {
       const float* x = (const float*)a.x + (long long)m * a.K;
 #pragma unroll
-      for (int k = 0; k < NP; k++) { const float2 v = *(const float2*)(x + F::xoff(u, k)); nx[k] = f2h_bits(v.x) | (f2h_bits(v.y) << 16); }
+      for (int k = 0; k < NP; k += 4) {
+        const f32x4 lo = *(const f32x4*)(x + F::xoff(u, k)), hi = *(const f32x4*)(x + F::xoff(u, k) + 4);
+        nx[k] = f2h_bits(lo.x) | (f2h_bits(lo.y) << 16); nx[k + 1] = f2h_bits(lo.z) | (f2h_bits(lo.w) << 16);
+        nx[k + 2] = f2h_bits(hi.x) | (f2h_bits(hi.y) << 16); nx[k + 3] = f2h_bits(hi.z) | (f2h_bits(hi.w) << 16);
+      }
     } else {
       const uint16_t* x = (const uint16_t*)a.x + (long long)m * a.K;
 #pragma unroll
-      for (int k = 0; k < NP; k++) nx[k] = *(const uint32_t*)(x + F::xoff(u, k));
+      for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(x + F::xoff(u, k)); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
     }
     u32x4 xv[F::XV]; float c[F::NG];
     F::stage(nx, xv, c);
