@@ -168,7 +168,10 @@ def main():
     alg_f = blk_w + 2 * c.num_blocks * c.n_kv_heads * c.head_dim * ctx_now * 2
     avg = float(np.mean(fused_us[1:]))
     out["roofline"] = {"bound": "hbm", "kernel": f"decode_layers_kernel<Q4_0 pair> (all {c.num_blocks} blocks of one token in one persistent launch: 4 dequant-GEMV phases + attention per block)",
-                       "achieved": round(alg_f / avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_f / avg / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                       "achieved": round(alg_f / avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_f / avg / 1e3 / HBM_PEAK_GBS, 4),
+                       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py at context 1024
+                       # (counters scaled by a 1 GiB copy kernel: x2.0000 and x1.0000): 4 100.5 MB fetched + 43.0 MB written
+                       "traffic": 4143500000 if c.num_blocks == 32 else None,
                        "avg_launch_us": round(avg, 2), "alg_bytes_per_launch": int(alg_f), "phase_us_inside_launch": phase,
                        "per_op_kernels": kern}
     if phase:

@@ -34,6 +34,8 @@ int tga_free(void* ptr);                                   /* ops_hip.py:63 */
 int tga_memcpy_h2d(void* dst, const void* src, size_t n);  /* ops_hip.py:64-66, synchronous */
 int tga_memcpy_d2h(void* dst, const void* src, size_t n);  /* ops_hip.py:67-69, synchronous */
 int tga_memcpy_d2d(void* dst, const void* src, size_t n, void* stream);
+/* device-to-device copy done by a plain kernel (n bytes, 16-byte aligned): a known-size yardstick for hardware traffic counters. */
+int tga_copy_kernel(void* dst, const void* src, size_t n, void* stream);
 int tga_memset(void* dst, int value, size_t n, void* stream);
 int tga_sync(void);                                        /* ops_hip.py:22-24 hipDeviceSynchronize */
 int tga_stream_create(void** stream);

@@ -41,6 +41,18 @@ int tga_memcpy_d2h(void* dst, const void* src, size_t n) { TGA_HIP(hipMemcpy(dst
 int tga_memcpy_d2d(void* dst, const void* src, size_t n, void* stream) {
   TGA_HIP(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, (hipStream_t)stream)); return 0;
 }
+// Plain 16-byte-per-thread copy kernel of a known size: the yardstick the HBM traffic counters (FETCH_SIZE / WRITE_SIZE) of other
+// kernels are scaled by.
+__global__ __launch_bounds__(256) void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+int tga_copy_kernel(void* dst, const void* src, size_t n, void* stream) {
+  TGA_REQUIRE(dst && src && n % 16 == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0, "tga_copy_kernel: pointers and size must be multiples of 16");
+  if (n == 0) return 0;
+  copy_kernel<<<2048, 256, 0, (hipStream_t)stream>>>((uint4*)dst, (const uint4*)src, n / 16);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
 int tga_memset(void* dst, int value, size_t n, void* stream) { TGA_HIP(hipMemsetAsync(dst, value, n, (hipStream_t)stream)); return 0; }
 int tga_sync(void) { TGA_HIP(hipDeviceSynchronize()); return 0; }
 

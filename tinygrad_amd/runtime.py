@@ -47,6 +47,7 @@ def _declare(lib):
     "tga_decode_layers_trace": [vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
     "tga_advance_prompt": [vp, vp, vp],
+    "tga_copy_kernel": [vp, vp, ctypes.c_size_t, vp],
     "tga_mfma_peak": [i, i, vp, vp],
     "tga_synth_weights": [i, vp, i64, ctypes.c_uint32, ctypes.c_float, vp],
   }
