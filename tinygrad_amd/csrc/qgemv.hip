@@ -79,6 +79,44 @@ __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const 
   }
 }
 
+// R rows of one unit against the M staged activation rows: the R weight slices are decoded first, then each activation's
+// vectors are read from LDS ONCE and used for all R rows (the LDS traffic per weight byte falls with R; at M = 8 it is what
+// bounds the kernel).
+template <int T, int M, int R>
+__device__ __forceinline__ void unit_dot_rows(const typename Fmt<T>::Raw* raw, const u32x4* xs, const float* cs, int cu, int ul, float (&acc)[R][M], const uint32_t* kc) {
+  using F = Fmt<T>;
+  uint32_t wv[R][F::NWV];
+#pragma unroll
+  for (int r = 0; r < R; r++) F::decode(raw[r], wv[r], kc);
+  constexpr int VPG = F::XV / F::NG;   // x vectors per accumulator group
+#pragma unroll
+  for (int m = 0; m < M; m++) {
+    float g[R][F::NG];
+#pragma unroll
+    for (int j = 0; j < F::NG; j++) {
+      const float c0 = cs[(m * F::NG + j) * cu + ul];
+      float s[R];
+#pragma unroll
+      for (int r = 0; r < R; r++) s[r] = c0;
+#pragma unroll
+      for (int v = 0; v < VPG; v++) {
+        const u32x4 xv = xs[(m * F::XV + j * VPG + v) * cu + ul];
+        const int wi = 4 * (j * VPG + v);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          s[r] = dot2(wv[r][wi + 0], xv.x, s[r]); s[r] = dot2(wv[r][wi + 1], xv.y, s[r]); s[r] = dot2(wv[r][wi + 2], xv.z, s[r]); s[r] = dot2(wv[r][wi + 3], xv.w, s[r]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++) g[r][j] = s[r];
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r][m] += F::finish(raw[r], g[r]);
+    // one activation row's vectors live at a time: without this the scheduler hoists the LDS reads of all M rows (M x 32 VGPRs)
+    if constexpr (M * R > 4) __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 // Reduce R x M partial sums across the wave and let lane 63 write rows row0 .. row0+R-1 of segment `seg` (rows >= row_end are
 // skipped; ld = rows of the segment = leading dimension of y).  Epilogue 2 (SwiGLU) treats the two accumulator rows as
 // (gate, up) of output row row0.
@@ -183,10 +221,7 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
       long long c_row = lo; int c_it = 0;
       auto compute = [&](const Raw* buf) {
         const int u = c_it * 64 + lane;
-        if (u < cu) {
-#pragma unroll
-          for (int r = 0; r < R; r++) unit_dot<T, M>(buf[r], xs, cs, cu, u, acc[r], kc);
-        }
+        if (u < cu) unit_dot_rows<T, M, R>(buf, xs, cs, cu, u, acc, kc);
         if (++c_it == iters) {
           store_rows<M, R>(a, seg, c_row, hi, seg_rows, acc);
 #pragma unroll
@@ -230,8 +265,7 @@ __global__ __launch_bounds__(QG_THREADS) void qgemv_kernel(const QArgs a) {
           Raw raw[R];
 #pragma unroll
           for (int r = 0; r < R; r++) raw[r] = F::load(rp[r], u0 + ul);
-#pragma unroll
-          for (int r = 0; r < R; r++) unit_dot<T, M>(raw[r], xs, cs, cu, ul, acc[r], kc);
+          unit_dot_rows<T, M, R>(raw, xs, cs, cu, ul, acc, kc);
         }
       }
     }
@@ -289,7 +323,8 @@ static int launch_qgemv_r(const QArgs& a, hipStream_t s) {
   // per lane); a single row per group when there are too few rows to fill the chip.
   if (a.epilogue == 2) return launch_qgemv<T, M, 2>(a, s);
   const bool chunked = (long long)M * (16 * Fmt<T>::XV + 4 * Fmt<T>::NG) * (a.K / Fmt<T>::UW) > QG_LDS_BUDGET;
-  if (M > 1 || chunked || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
+  // (chunked K with several segments needs one row per group: a group must not straddle a segment)
+  if ((chunked && a.nseg > 1) || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
   return launch_qgemv<T, M, 2>(a, s);
 }
 
