@@ -123,3 +123,34 @@ def test_rmsnorm_argmax_embed(gpu):
   lgb, sv, si = gpu.Buffer.from_numpy(lg), gpu.Buffer((256,), np.float32), gpu.Buffer((256,), np.int32)
   gpu.check(gpu.lib().tga_argmax_step(lgb.ptr, lg.size, sv.ptr, si.ptr, stb.ptr, pr.ptr, outt.ptr, 4, None))
   assert outt.numpy()[0] == 777 and list(stb.numpy()[:3]) == [1, 777, 1]
+
+def test_decode_layers_argument_checks_and_trace(gpu):
+  """tga_decode_layers rejects shapes outside its contract with a message (no launch), and the phase trace fills its buffer."""
+  from tinygrad_amd import runtime as rt
+  L = rt.lib()
+  m, _ = _build(gpu, SMALL, 128, seed=5)
+  s, c = m.s, m.config
+  call = lambda **kw: L.tga_decode_layers(m.layer_table.ptr, kw.get("n_layers", c.num_blocks), kw.get("wtype", m.layer_type), s.x.ptr, s.qkv.ptr, s.attn.ptr, s.act.ptr,
+                                          s.attn_part.ptr, s.state.ptr, s.rope.ptr, s.sync.ptr, kw.get("dim", c.dim), kw.get("hidden", c.hidden_dim), c.n_heads, c.n_kv_heads,
+                                          kw.get("hd", c.head_dim), c.max_context, c.norm_eps, m.stream.handle)
+  for bad in (dict(wtype=rt.Q6_K), dict(hd=32), dict(dim=c.dim + 64), dict(hidden=c.hidden_dim + 32), dict(n_layers=0)):
+    assert call(**bad) != 0
+    assert b"tga_decode_layers" in L.tga_last_error()
+  tb = rt.Buffer((8 * 11 * c.num_blocks,), np.uint64).zero_()
+  rt.check(L.tga_decode_layers_trace(tb.ptr))
+  try:
+    out = list(m.generate([1, 2, 3], 2, use_graph=False))
+  finally:
+    rt.check(L.tga_decode_layers_trace(None))
+  t = tb.numpy().reshape(8, c.num_blocks, 11)[0].astype(np.int64)
+  assert len(out) == 2 and (t > 0).all() and (np.diff(t.reshape(-1)) >= 0).all()      # workgroup 0's stamps are in program order
+
+def test_copy_kernel_and_mfma_peak_run(gpu):
+  from tinygrad_amd import runtime as rt
+  L = rt.lib()
+  a = rt.Buffer.from_numpy(np.arange(1 << 16, dtype=np.uint32)); b = rt.Buffer((1 << 16,), np.uint32).zero_()
+  rt.check(L.tga_copy_kernel(b.ptr, a.ptr, a.nbytes, None))
+  np.testing.assert_array_equal(b.numpy(), a.numpy())
+  assert L.tga_copy_kernel(b.ptr, a.ptr, 24, None) != 0
+  scratch = rt.Buffer((64,), np.float32).zero_()
+  rt.check(L.tga_mfma_peak(8, 2, scratch.ptr, None)); rt.synchronize()
