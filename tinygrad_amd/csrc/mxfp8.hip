@@ -241,20 +241,20 @@ __global__ __launch_bounds__(256) void grouped_mxfp8_gemm_kernel(const GemmArgs 
 // sub-tile lives in LDS in the order the MFMA consumes it: plane p (the lane's first / second 16 bytes), slot 16g + r <- row r,
 // bytes [64p + 16g, 64p + 16g + 16), with the slot's low three bits XORed by (g + 4p): the 8 threads that copy one row's 128
 // bytes then hit 8 different 16-byte bank groups, and so do the 8 consecutive lanes of every ds_read_b128.  While step s is
-// multiplied, the global loads of step s + 1 (8 x 16 bytes per thread) and its scale bytes are in flight (a scheduling barrier
+// multiplied, the global loads of step s + 1 (8 x 16 bytes + one scale dword per thread) are in flight (a scheduling barrier
 // keeps them ahead of the MFMAs); they are written to the other stage after the MFMAs, one workgroup barrier per step.
 // Operands are swapped in the MFMA (weights as A, activations as B), so a lane ends up with four consecutive output columns
 // of one row: 8-byte bf16 stores.
 #define GG_TILE 256
 #define GG_THREADS 512
-#define GG_STAGE_BYTES (2 * GG_TILE * 128)
+#define GG_STAGE_BYTES (2 * GG_TILE * 128 + 2 * GG_TILE * 4)   // operand tiles + one scale dword per row
 __device__ __forceinline__ int gg_slot_off(int R, int c) {       // byte offset inside a 256-row operand region of (row R, 16-byte chunk c)
   const int sub = R >> 4, r = R & 15, p = c >> 2, g = c & 3;
   return sub * 2048 + p * 1024 + ((16 * g + (r ^ (g + 4 * p))) << 4);
 }
 
 __global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(const GemmArgs g) {
-  extern __shared__ uint8_t smem[];                          // [stage][A 32 KB | B 32 KB]
+  extern __shared__ uint8_t smem[];                          // [stage][A 32 KB | B 32 KB | 512 scale dwords]
   const int tiles_n = g.N / GG_TILE, ntiles = gridDim.x;
   // consecutive workgroups go to different XCDs: give each XCD a contiguous run of tiles so that the N tiles of one row block
   // (which share the activation tile) and the row blocks of one expert (which share the weight tile) meet in one L2
@@ -282,9 +282,9 @@ __global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(cons
   for (int j = 0; j < 4; j++) cpy_off[j] = gg_slot_off(cpy_r + 64 * j, cpy_c);
   const uint8_t* a_src = Ag + (size_t)cpy_r * g.K + cpy_c * 16;
   const uint8_t* b_src = Bg + (size_t)cpy_r * g.K + cpy_c * 16;
-  // scale bytes: lane (g, r) of sub-tile i needs the E8M0 of (row 16 i + r, K block 4 s + g)
-  const uint8_t* a_sc = g.a_e8 + (size_t)(row0 + wm * 128 + r16) * KB + kg;
-  const uint8_t* b_sc = g.b_e8 + ((size_t)e * g.N + (size_t)tn * GG_TILE + wn * 64 + r16) * KB + kg;
+  // scale dwords (the four E8M0 bytes of K blocks 4s .. 4s+3 of one row) travel through LDS too: thread t < 256 copies activation
+  // row t's, thread t >= 256 weight row t - 256's; lane (g, r) of sub-tile i then takes byte g of row 16 i + r
+  const uint8_t* sc_src = tid < GG_TILE ? g.a_e8 + (size_t)(row0 + tid) * KB : g.b_e8 + ((size_t)e * g.N + (size_t)tn * GG_TILE + (tid - GG_TILE)) * KB;
   // fragment read offsets of this lane inside a sub-tile (plane 0 / plane 1)
   const int f0 = ((16 * kg + (r16 ^ kg)) << 4), f1 = 1024 + ((16 * kg + (r16 ^ (kg + 4))) << 4);
 
@@ -294,55 +294,47 @@ __global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(cons
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
 
-  u32x4 stg_a[4], stg_b[4];
-  int sa[8], sb[4], sa_n[8], sb_n[4];
+  u32x4 stg_a[4], stg_b[4]; uint32_t stg_sc;
   auto load_step = [&](int s) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       stg_a[j] = *(const u32x4*)(a_src + (size_t)(64 * j) * g.K + (size_t)s * 128);
       stg_b[j] = *(const u32x4*)(b_src + (size_t)(64 * j) * g.K + (size_t)s * 128);
     }
-#pragma unroll
-    for (int i = 0; i < 8; i++) sa_n[i] = a_sc[(size_t)(16 * i) * KB + 4 * s];
-#pragma unroll
-    for (int j = 0; j < 4; j++) sb_n[j] = b_sc[(size_t)(16 * j) * KB + 4 * s];
+    stg_sc = *(const uint32_t*)(sc_src + 4 * s);
   };
   auto store_step = [&](int stage) {
     uint8_t* base = smem + stage * GG_STAGE_BYTES;
 #pragma unroll
     for (int j = 0; j < 4; j++) { *(u32x4*)(base + cpy_off[j]) = stg_a[j]; *(u32x4*)(base + GG_TILE * 128 + cpy_off[j]) = stg_b[j]; }
-#pragma unroll
-    for (int i = 0; i < 8; i++) sa[i] = sa_n[i];
-#pragma unroll
-    for (int j = 0; j < 4; j++) sb[j] = sb_n[j];
+    ((uint32_t*)(base + 2 * GG_TILE * 128))[tid] = stg_sc;
   };
   load_step(0);
   store_step(0);
   __syncthreads();
   for (int s = 0; s < nsteps; s++) {
-    const int sn = s + 1 < nsteps ? s + 1 : s;                 // the last step reloads itself (dropped)
-    int sa_c[8], sb_c[4];
-#pragma unroll
-    for (int i = 0; i < 8; i++) sa_c[i] = sa[i];
-#pragma unroll
-    for (int j = 0; j < 4; j++) sb_c[j] = sb[j];
-    load_step(sn);
+    load_step(s + 1 < nsteps ? s + 1 : s);                    // the last step reloads itself (dropped)
     __builtin_amdgcn_sched_barrier(0);                        // the loads of the next step stay ahead of this step's MFMAs
-    const uint8_t* As = smem + (s & 1) * GG_STAGE_BYTES + wm * 8 * 2048;
-    const uint8_t* Bs = smem + (s & 1) * GG_STAGE_BYTES + GG_TILE * 128 + wn * 4 * 2048;
-    v8i32 bf[4];
+    const uint8_t* base = smem + (s & 1) * GG_STAGE_BYTES;
+    const uint8_t* As = base + wm * 8 * 2048;
+    const uint8_t* Bs = base + GG_TILE * 128 + wn * 4 * 2048;
+    const uint32_t* sA = (const uint32_t*)(base + 2 * GG_TILE * 128) + wm * 128 + r16;
+    const uint32_t* sB = (const uint32_t*)(base + 2 * GG_TILE * 128) + GG_TILE + wn * 64 + r16;
+    v8i32 bf[4]; int sb[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const u32x4 y0 = *(const u32x4*)(Bs + j * 2048 + f0), y1 = *(const u32x4*)(Bs + j * 2048 + f1);
       bf[j] = v8i32{(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+      sb[j] = (int)(sB[16 * j] >> (8 * kg));
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const u32x4 x0 = *(const u32x4*)(As + i * 2048 + f0), x1 = *(const u32x4*)(As + i * 2048 + f1);
       const v8i32 af = v8i32{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+      const int sa = (int)(sA[16 * i] >> (8 * kg));
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af, acc[i][j], 0, 0, 0, sb_c[j], 0, sa_c[i]);
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af, acc[i][j], 0, 0, 0, sb[j], 0, sa);
     }
     __builtin_amdgcn_sched_barrier(0);
     store_step((s + 1) & 1);
