@@ -76,6 +76,14 @@ int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const
                       const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                       int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
 
+/* tga_qlinear_multi at M = 1 with the RMSNorm that precedes it folded in (attn_norm -> attn_q/k/v and ffn_norm -> ffn_gate/up,
+ * tinygrad/llm/model.py:149-150; output_norm -> output, :362; nn.RMSNorm tinygrad/nn/__init__.py:296-304): x is the float32
+ * row BEFORE the norm, the kernel multiplies W by fp16((x * rsqrt(mean(x^2) + norm_eps)) * norm_weight).  Needs the M = 1 fast
+ * path (K % 64 == 0, K <= 65536, 16-byte aligned x and norm_weight, 4-byte aligned weights); other arguments as above. */
+int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                              const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
+                              int y_stage_type, int64_t y_stage_K, void* stream);
+
 /* Staged activations (no counterpart in the reference; an M = 1 fast path): the decode GEMV keeps each lane's activations in
  * registers in the order its in-register decode produces weights, which is a fixed permutation of the row that depends on the
  * weight's (ggml_type, K).  tga_stage_activation writes that permutation as fp16 (K values); a linear then takes it with
@@ -96,6 +104,12 @@ int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t 
  * gathered / renormalised / scaled.  logits (n_tokens, n_experts) float32 -> sel (n_tokens, k) int32, probs (n_tokens, k). */
 int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int gating, int norm_topk_prob, float scale,
                  int32_t* sel, float* probs, void* stream);
+/* Router of ONE token in one launch (model.py:112-128 with the block's ffn_norm, :150): h = fp16(RMSNorm(x) * norm_weight) (norm_weight
+ * NULL: h = fp16(x)), logits = h @ Wr^T for a dense fp16 router weight (n_experts, dim), then gating + top-k as tga_moe_gate.
+ * xn_out_f16 (dim fp16, the activation of the expert GEMVs) and logits_out (n_experts floats) may be NULL.
+ * dim % 8 == 0, dim <= 16384, n_experts <= 1024, k <= 64. */
+int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
+                   int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_out, int32_t* sel, float* probs, void* stream);
 /* out[t] = resid[t] + sum_s probs[t, s] * y[t, s, :]  (model.py:130 and the residual add :150); resid may be NULL or alias out. */
 int tga_moe_combine(const float* y, const float* probs, const float* resid, int n_tokens, int k, int dim, float* out, void* stream);
 
@@ -119,6 +133,13 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
  * stage_type != 0: out_f16 is written in the staged order of a consumer weight of that type with K = n_heads * head_dim. */
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
                          int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
+
+/* tga_attention_decode with the full-width q / k RMSNorm of model.py:169 (attn_q_norm over all n_heads * head_dim values, attn_k_norm
+ * over all n_kv_heads * head_dim) applied before RoPE: q_norm_weight [n_heads * head_dim], k_norm_weight [n_kv_heads * head_dim]
+ * float32, both NULL for no norm; q and k must be 16-byte aligned when the norm is on. */
+int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                void* cache_k, void* cache_v, float* partials, const void* state,
+                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
 /* argmax(-1) with first-max tie rule (tinygrad/mixin/op.py:866-891) + the bookkeeping of Transformer.generate (model.py:475-484):
  * while state.pos + 1 < state.n_prompt the next input token is prompt[pos + 1]; otherwise the argmax token is stored at

@@ -80,32 +80,42 @@ def test_one_launch_blocks_equal_per_op_path(gpu, cfg, ltype):
   assert ol.rel_err(ka[:, :78], kb[:, :78]) <= 2e-3
   assert not a.s.sync.numpy().any()                                # barrier counters back at zero, no error flag
 
-def test_attention_decode_kernel_vs_numpy(gpu):
-  """tga_attention_decode alone: RoPE + fp16 KV append + GQA softmax attention at several positions."""
+@pytest.mark.parametrize("H,KV,hd,normed", [(8, 2, 128, False), (4, 4, 64, True), (12, 2, 128, True), (4, 2, 256, False), (16, 16, 128, True)],
+                         ids=["gqa4-hd128", "mha-hd64-qknorm", "gqa6-hd128-qknorm", "gqa2-hd256", "mha16-hd128-qknorm"])
+def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
+  """tga_attention_decode(_normed) alone: (full-width q/k RMSNorm,) RoPE + fp16 KV append + GQA softmax attention at several positions."""
   from tinygrad_amd.llm import precompute_freqs_cis
-  H, KV, hd, ctx = 8, 2, 128, 256
-  rng = np.random.default_rng(5)
+  ctx = 256
+  rng = np.random.default_rng(5 + H)
   rope = precompute_freqs_cis(hd, ctx, 10000.0)
   ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
   part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2) + KV,), np.float32).zero_()
   ropeb = gpu.Buffer.from_numpy(rope)
   out = gpu.Buffer((H * hd,), np.float32)
+  qw, kw = (rng.standard_normal(n).astype(np.float32) for n in (H * hd, KV * hd))
+  qwb, kwb = gpu.Buffer.from_numpy(qw), gpu.Buffer.from_numpy(kw)
   rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)
   for pos in range(0, 140):
-    q, k, v = (rng.standard_normal(n).astype(np.float32) for n in (H * hd, KV * hd, KV * hd))
+    q, k, v = (rng.standard_normal(n).astype(np.float32) * 1.5 for n in (H * hd, KV * hd, KV * hd))
     st = np.zeros(16, np.int32); st[0] = pos
     qb, kb, vb, stb = (gpu.Buffer.from_numpy(t) for t in (q, k, v, st))       # keep the device buffers alive across the launch
-    gpu.check(gpu.lib().tga_attention_decode(qb.ptr, kb.ptr, vb.ptr, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None, out.ptr, 0, None))
+    if normed:
+      gpu.check(gpu.lib().tga_attention_decode_normed(qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, 1e-5, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx,
+                                                      ropeb.ptr, None, out.ptr, 0, None))
+      q, k = ollm.rmsnorm(q, qw, 1e-5), ollm.rmsnorm(k, kw, 1e-5)
+    else:
+      gpu.check(gpu.lib().tga_attention_decode(qb.ptr, kb.ptr, vb.ptr, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None, out.ptr, 0, None))
     gpu.synchronize()
     qr = ollm.apply_rope(q.reshape(H, hd), rope[pos]); kr = ollm.apply_rope(k.reshape(KV, hd), rope[pos])
     rk[:, pos], rv[:, pos] = kr.astype(np.float16), v.reshape(KV, hd).astype(np.float16)
-    if pos in (0, 1, 63, 64, 65, 127, 128, 139):
+    if pos in (0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 139):
       K = np.repeat(rk[:, :pos + 1].astype(np.float32), H // KV, axis=0); V = np.repeat(rv[:, :pos + 1].astype(np.float32), H // KV, axis=0)
       sc = np.einsum("hd,htd->ht", qr, K) / np.sqrt(hd)
       e = np.exp(sc - sc.max(-1, keepdims=True)); p = e / e.sum(-1, keepdims=True)
       ref = np.einsum("ht,htd->hd", p, V).reshape(-1)
       assert ol.rel_err(out.numpy(), ref) <= 1e-4, pos
   assert ck.numpy().tobytes() == rk.tobytes() or ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
+  assert not part.numpy()[-KV:].view(np.int32).any()                 # arrival counters back at zero
 
 def test_rmsnorm_argmax_embed(gpu):
   rng = np.random.default_rng(9)

@@ -58,6 +58,27 @@ def test_expert_gemv_with_indirection(gpu, t, kdim, n):
   refj = np.stack([ol.linear_f64(xj[j][None].astype(np.float32), W[sel.reshape(-1)[j]])[0] for j in range(T * k)])
   assert ol.rel_err(y.numpy(), refj) <= 1e-3
 
+@pytest.mark.parametrize("dim,E,k,gating,normw", [(2048, 64, 8, 1, True), (256, 8, 2, 3, True), (1024, 130, 6, 2, False)])
+def test_router_in_one_launch(gpu, dim, E, k, gating, normw):
+  """tga_moe_router (ffn_norm + router logits + gating + top-k) against the oracle fed with the float64 logits of the fp16-rounded row."""
+  from tinygrad_amd.nn import QuantLinear, moe_router
+  from tinygrad_amd import runtime as rt
+  rng = np.random.default_rng(dim + E)
+  x = (rng.standard_normal(dim) * 2).astype(np.float32); nw = rng.standard_normal(dim).astype(np.float32)
+  wr = (rng.standard_normal((E, dim)) * dim ** -0.5).astype(np.float16)
+  router = QuantLinear(gpu.Buffer.from_numpy(wr.view(np.uint8).reshape(-1)), rt.F16, E, dim)
+  xn, lg = gpu.Buffer((dim,), np.float16), gpu.Buffer((E,), np.float32)
+  sel, pr = gpu.Buffer((k,), np.int32), gpu.Buffer((k,), np.float32)
+  moe_router(gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw) if normw else None, 1e-5, router, k, sel, pr, xn_out=xn, logits_out=lg, gating=gating,
+             norm_topk_prob=True, scale=1.5)
+  h = (ollm.rmsnorm(x, nw, 1e-5) if normw else x).astype(np.float16)
+  assert np.mean(xn.numpy() != h) < 0.01 and ol.rel_err(xn.numpy().astype(np.float32), h.astype(np.float32)) < 1e-3   # fp16 ties may round either way
+  ref_lg = (h.astype(np.float64) @ wr.astype(np.float64).T).astype(np.float32)
+  assert ol.rel_err(lg.numpy(), ref_lg) <= 1e-3
+  rs, rp = omoe.gate_probs(lg.numpy()[None], k, gating, True, 1.5)        # selection on the kernel's own logits: exact
+  np.testing.assert_array_equal(sel.numpy(), rs[0])
+  np.testing.assert_allclose(pr.numpy(), rp[0], rtol=2e-5, atol=1e-7)
+
 def test_moe_combine(gpu):
   from tinygrad_amd.nn import moe_combine
   rng = np.random.default_rng(3)

@@ -153,3 +153,40 @@ def test_swiglu_output_staged_for_the_down_projection(gpu):
   qlinear_multi([g, u], x, [act_s], epilogue=2, stage_out_for=dn)
   qlinear_multi([dn], act_s, [y_s], x_staged=True)
   assert ol.rel_err(y_s.numpy(), y_n.numpy()) <= 1e-5
+
+@pytest.mark.parametrize("t,k", [(2, 2048), (8, 512), (14, 1024), (39, 2048), (1, 2048), (2, 8192)], ids=["q4_0", "q8_0", "q6_k", "mxfp4", "f16", "q4_0-k8192"])
+def test_rmsnorm_folded_into_the_linear(gpu, t, k):
+  """tga_rmsnorm_qlinear_multi against tga_rmsnorm followed by tga_qlinear_multi (same fp16 activation up to the summation order of
+  the mean square) and against the float64 anchor on the fp16-rounded normalised row."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  from tinygrad_amd import runtime as rt
+  from oracle import llm as ollm
+  rng = np.random.default_rng(t * 1000 + k)
+  ns = [192, 64]
+  if t == 1: ws = [rng.standard_normal((n, k)).astype(np.float16).view(np.uint8).reshape(-1) * 1 for n in ns]
+  else: ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+  layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+  x = (rng.standard_normal((1, k)) * 3).astype(np.float32); nw = rng.standard_normal(k).astype(np.float32)
+  xb, nwb = gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw)
+  fused = [gpu.Buffer((1, n), np.float32) for n in ns]
+  qlinear_multi(layers, xb, fused, norm=(nwb, 1e-5))
+  xn = gpu.Buffer((1, k), np.float16)
+  gpu.check(gpu.lib().tga_rmsnorm(xb.ptr, nwb.ptr, k, 1e-5, xn.ptr, None, 0, None))
+  plain = [gpu.Buffer((1, n), np.float32) for n in ns]
+  qlinear_multi(layers, xn, plain)
+  h = ollm.rmsnorm(x[0], nw, 1e-5).astype(np.float16).astype(np.float32)[None]
+  for f, p, w, n in zip(fused, plain, ws, ns):
+    W = w.view(np.float16).astype(np.float32).reshape(n, k) if t == 1 else ol.weight_f32(w, n, k, t)
+    assert ol.rel_err(f.numpy(), p.numpy()) <= 2e-4
+    assert ol.rel_err(f.numpy(), ol.linear_f64(h, W)) <= TOL
+  # SwiGLU epilogue with the folded norm (ffn_norm -> ffn_gate / ffn_up)
+  pair = [QuantLinear(layers[1].blocks, t, 64, k), QuantLinear(gpu.Buffer.from_numpy(ws[0][: len(ws[0]) // 3]), t, 64, k)]
+  o1, o2 = gpu.Buffer((1, 64), np.float32), gpu.Buffer((1, 64), np.float32)
+  qlinear_multi(pair, xb, [o1], epilogue=2, norm=(nwb, 1e-5))
+  qlinear_multi(pair, xn, [o2], epilogue=2)
+  assert ol.rel_err(o1.numpy(), o2.numpy()) <= 1e-3
+  # outside the fast path the call is refused with a message
+  bad = QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, 2, 8, 96)), 2, 8, 96)
+  with pytest.raises(RuntimeError, match="fast path"):
+    qlinear_multi([bad], gpu.Buffer.from_numpy(x[:, :96].copy()), [gpu.Buffer((1, 8), np.float32)], norm=(nwb, 1e-5))
+

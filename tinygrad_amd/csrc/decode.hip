@@ -5,6 +5,7 @@
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
 #include "qfmt.h"
 #include "decode.h"
+#include "coherent.h"
 
 // ---------------------------------------------------------------------------------------------- embedding (Q4_0 / F16 / F32 row)
 // token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized.
@@ -56,10 +57,11 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------- RoPE + KV append + attention
-// One workgroup per (kv head, 64-position split); wave w of the workgroup serves query head kvh * group + w (group <= 4 waves
-// per pass).  q, k are rotated with the half-split rule of apply_rope (tinygrad/llm/model.py:29-33) using the caller's
-// freqs_cis table [max_ctx][hd] = cos half | sin half (precompute_freqs_cis, model.py:16-19); the split that contains `pos` writes the rotated k and v into the fp16 cache.
-// Scores: lane <-> position, softmax partials per split (max, sum, weighted V) go to `part` for the combine kernel.
+// One workgroup per (kv head, 64-position split).  q, k are rotated with the half-split rule of apply_rope
+// (tinygrad/llm/model.py:29-33) using the caller's freqs_cis table [max_ctx][hd] = cos half | sin half (precompute_freqs_cis,
+// model.py:16-19); the split that contains `pos` writes the rotated k and v into the fp16 cache.  With q_norm / k_norm the
+// full-width RMSNorm of model.py:169 (attn_q_norm / attn_k_norm over all heads at once) is applied to q and k first.
+// Softmax partials per split (max, sum, weighted V) go to `part`; the last split of a kv head to finish merges them.
 struct AttnArgs {
   const float* q; const float* k; const float* v;     // this token's projections: [n_heads*hd], [n_kv*hd], [n_kv*hd]
   _Float16* cache_k; _Float16* cache_v;                // [n_kv][max_ctx][hd]
@@ -70,132 +72,184 @@ struct AttnArgs {
   float scale;
   _Float16* out16; float* out32;                       // attention output [n_heads*hd]
   int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
+  const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights over the whole q / k vectors
 };
 
-// 8 fp16 values (one 16-byte piece) of row `p` of a cache plane; the row of the token being processed comes from LDS (fp32
-// values rounded to fp16 exactly like the copy that goes into the cache)
-__device__ __forceinline__ u32x4 kv_piece(const _Float16* plane_row0, int hd, int p, int pos, int piece, const float* cur) {
-  if (p == pos) {
-    const float* c = cur + piece * 8;
-    u32x4 r = {f2h_bits(c[0]) | (f2h_bits(c[1]) << 16), f2h_bits(c[2]) | (f2h_bits(c[3]) << 16),
-               f2h_bits(c[4]) | (f2h_bits(c[5]) << 16), f2h_bits(c[6]) | (f2h_bits(c[7]) << 16)};
-    return r;
-  }
-  return *(const u32x4*)(plane_row0 + (size_t)p * hd + piece * 8);
+__device__ __forceinline__ u32x4 pack8_f16(const float* c) {
+  u32x4 r = {f2h_bits(c[0]) | (f2h_bits(c[1]) << 16), f2h_bits(c[2]) | (f2h_bits(c[3]) << 16),
+             f2h_bits(c[4]) | (f2h_bits(c[5]) << 16), f2h_bits(c[6]) | (f2h_bits(c[7]) << 16)};
+  return r;
+}
+// sum over the HD8 (8, 16 or 32) consecutive lanes that hold one row; every lane of the run gets the sum
+template <int HD8>
+__device__ __forceinline__ float run_sum(float v) {
+  v = dpp_add<0xB1>(v); v = dpp_add<0x4E>(v); v = dpp_add<0x141>(v);
+  if constexpr (HD8 >= 16) v = dpp_add<0x140>(v);
+  if constexpr (HD8 == 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+// sum of squares of n floats (n % 4 == 0, 16-byte aligned) over the whole workgroup of 256 threads; red: 4 floats of LDS
+__device__ __forceinline__ float block_sumsq(const float* x, int n, float* red) {
+  float s = 0.f;
+  for (int i = threadIdx.x * 4; i < n; i += 1024) { const f32x4 v = *(const f32x4*)(x + i); s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
 }
 
-// HD8 = head_dim / 8 (16-byte pieces per row).  Workgroup = (kv head, 64-position split), wave w serves query heads w, w+4, ...
-// of the group.  K: lane <-> position (whole row in registers).  V: RPI = 64 / HD8 rows per load instruction, lane = (row-in-
-// instruction, piece); both tiles are requested before any arithmetic so their latencies overlap.
-// The last workgroup of a kv head to finish (device-scope arrival counter) merges that head group's split partials.
+// HD8 = head_dim / 8 (16-byte pieces per row).  The four waves split the 64 positions (16 each) and every wave serves all
+// query heads of the group.  A wave's K and V tiles are 16 rows in one shared register layout: load instruction i covers rows
+// i*RPI + lane / HD8 (RPI = 64 / HD8) and lane % HD8 picks the 16-byte piece, so a lane only needs the 8 query values of its
+// piece.  Scores: 8 FMAs per instruction, then a DPP sum over the HD8 lanes of a row.  Each run of HD8 lanes keeps its own
+// softmax partial (its rows only); the partials meet in LDS and leave as one partial per (head, split).  Both tiles are
+// requested before anything else; the row of the current token (not in the cache yet) is patched in from LDS.
+// Partials cross workgroups inside the launch, so they move through write-through stores and cache-bypassing loads, and the
+// arrival counter is a relaxed device-scope atomic after the stores have completed (no cache write-back / invalidate).
 template <int HD8>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
-  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 64 / RPI;   // rows per V instruction, V instructions per 64 rows
+  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = 4 * RPI, CSTR = HD + 4;
   const int kvh = blockIdx.x, split = blockIdx.y;
   const int pos = a.st->pos;
-  const int p0 = split * 64;
-  if (p0 > pos) return;                                 // nothing cached in this split yet
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (split * 64 > pos) return;                         // nothing cached in this split yet
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = HD >> 1, group = a.n_heads / a.n_kv;
   __shared__ float qs[4][HD];                           // rotated queries of the 4 heads in flight
   __shared__ float ks[HD], vs[HD];                      // rotated key / value of this token
+  __shared__ float comb[4 * NGRP * CSTR];               // [head in flight][run]: o[HD], m, l
+  __shared__ float sw[2048];                            // merge weights; host guarantees group * nsplit <= 1024
+  __shared__ float red[8];
   __shared__ int last_flag;
-  for (int i = threadIdx.x; i < half; i += 256) {
+  const int vr = lane / HD8, vp = lane % HD8;
+  const int p0 = split * 64 + wave * 16;                // first position of this wave
+  u32x4 kt[NVI], vt[NVI];
+  {
+    const _Float16* kbase = a.cache_k + (size_t)kvh * a.max_ctx * HD + vp * 8;
+    const _Float16* vbase = a.cache_v + (size_t)kvh * a.max_ctx * HD + vp * 8;
+#pragma unroll
+    for (int i = 0; i < NVI; i++) {
+      const int r = p0 + i * RPI + vr, rc = r < pos ? r : pos;   // rows >= pos are replaced below
+      kt[i] = *(const u32x4*)(kbase + (size_t)rc * HD);
+      vt[i] = *(const u32x4*)(vbase + (size_t)rc * HD);
+    }
+  }
+  float qscale = 1.f, kscale = 1.f;
+  if (a.q_norm) {
+    qscale = 1.0f / sqrtf(block_sumsq(a.q, a.n_heads * HD, red) / (float)(a.n_heads * HD) + a.norm_eps);
+    kscale = 1.0f / sqrtf(block_sumsq(a.k, a.n_kv * HD, red + 4) / (float)(a.n_kv * HD) + a.norm_eps);
+  }
+  auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[i] : a.q[i]; };
+  auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[i] : a.k[i]; };
+  for (int i = tid; i < half; i += 256) {
     const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
-    const float x1 = a.k[kvh * HD + i], x2 = a.k[kvh * HD + half + i];
+    const float x1 = kval(kvh * HD + i), x2 = kval(kvh * HD + half + i);
     ks[i] = x1 * c - x2 * s; ks[half + i] = x2 * c + x1 * s;
   }
-  for (int i = threadIdx.x; i < HD; i += 256) vs[i] = a.v[kvh * HD + i];
+  for (int i = tid; i < HD; i += 256) vs[i] = a.v[kvh * HD + i];
   __syncthreads();
-  const _Float16* krow0 = a.cache_k + (size_t)kvh * a.max_ctx * HD;
-  const _Float16* vrow0 = a.cache_v + (size_t)kvh * a.max_ctx * HD;
   if ((pos >> 6) == split) {                            // owner split appends this token to the cache
-    for (int i = threadIdx.x; i < HD; i += 256) {
+    for (int i = tid; i < HD; i += 256) {
       a.cache_k[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)ks[i];
       a.cache_v[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)vs[i];
     }
   }
-  // K tile: lane <-> position p0 + lane;  V tile: instruction i covers rows p0 + i*RPI + lane / HD8, piece lane % HD8
-  const int p = p0 + lane;
-  const bool pvalid = p <= pos;
-  const int pc = pvalid ? p : pos;                      // clamp to a valid row, result masked
-  u32x4 kt[HD8], vt[NVI];
+  {
+    const u32x4 kcur = pack8_f16(ks + vp * 8), vcur = pack8_f16(vs + vp * 8);   // rounded to fp16 exactly like the cached copy
 #pragma unroll
-  for (int i = 0; i < HD8; i++) kt[i] = kv_piece(krow0, HD, pc, pos, i, ks);
-  const int vr = lane / HD8, vp = lane % HD8;
-#pragma unroll
-  for (int i = 0; i < NVI; i++) { const int r = p0 + i * RPI + vr; vt[i] = kv_piece(vrow0, HD, r <= pos ? r : pos, pos, vp, vs); }
-
+    for (int i = 0; i < NVI; i++) if (p0 + i * RPI + vr >= pos) { kt[i] = kcur; vt[i] = vcur; }
+  }
   for (int h0 = 0; h0 < group; h0 += 4) {
-    const int gh = h0 + wave;
-    const bool hvalid = gh < group;
-    const int head = kvh * group + gh;
-    if (hvalid) {
+    if (h0 + wave < group) {                            // wave w rotates the query of head h0 + w
+      const int head = kvh * group + h0 + wave;
       for (int i = lane; i < half; i += 64) {
         const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
-        const float x1 = a.q[head * HD + i], x2 = a.q[head * HD + half + i];
+        const float x1 = qval(head * HD + i), x2 = qval(head * HD + half + i);
         qs[wave][i] = x1 * c - x2 * s; qs[wave][half + i] = x2 * c + x1 * s;
       }
     }
     __syncthreads();
-    if (hvalid) {
-      float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < HD8; i++) {
-        const float* qq = &qs[wave][i * 8];
-        const u32x4 kk = kt[i];
-        acc += qq[0] * h2f_bits(kk.x & 0xFFFF) + qq[1] * h2f_bits(kk.x >> 16) + qq[2] * h2f_bits(kk.y & 0xFFFF) + qq[3] * h2f_bits(kk.y >> 16)
-             + qq[4] * h2f_bits(kk.z & 0xFFFF) + qq[5] * h2f_bits(kk.z >> 16) + qq[6] * h2f_bits(kk.w & 0xFFFF) + qq[7] * h2f_bits(kk.w >> 16);
+    for (int hh = 0; hh < 4; hh++) {
+      if (h0 + hh < group) {
+        float qq[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) qq[j] = qs[hh][vp * 8 + j];
+        float sc[NVI];
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < NVI; i++) {
+          const u32x4 kk = kt[i];
+          const half2_t k0 = as_h2(kk.x), k1 = as_h2(kk.y), k2 = as_h2(kk.z), k3 = as_h2(kk.w);
+          float t = qq[0] * (float)k0.x; t += qq[1] * (float)k0.y; t += qq[2] * (float)k1.x; t += qq[3] * (float)k1.y;
+          t += qq[4] * (float)k2.x; t += qq[5] * (float)k2.y; t += qq[6] * (float)k3.x; t += qq[7] * (float)k3.y;
+          t = run_sum<HD8>(t);
+          sc[i] = (p0 + i * RPI + vr <= pos) ? t * a.scale : -INFINITY;
+          m = fmaxf(m, sc[i]);
+        }
+        // softmax partial of this lane run (rows i * RPI + vr of the wave): no cross-lane traffic, the fold below sums the runs
+        float l = 0.f;
+        f32x4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NVI; i++) {
+          const float pj = (p0 + i * RPI + vr <= pos) ? __expf(sc[i] - m) : 0.f;
+          l += pj;
+          const u32x4 vv = vt[i];
+          const half2_t v0 = as_h2(vv.x), v1 = as_h2(vv.y), v2 = as_h2(vv.z), v3 = as_h2(vv.w);
+          o0.x += pj * (float)v0.x; o0.y += pj * (float)v0.y; o0.z += pj * (float)v1.x; o0.w += pj * (float)v1.y;
+          o1.x += pj * (float)v2.x; o1.y += pj * (float)v2.y; o1.z += pj * (float)v3.x; o1.w += pj * (float)v3.y;
+        }
+        float* cw = comb + (size_t)(hh * NGRP + wave * RPI + vr) * CSTR;
+        *(f32x4*)(cw + vp * 8) = o0; *(f32x4*)(cw + vp * 8 + 4) = o1;
+        if (vp == 0) { cw[HD] = m; cw[HD + 1] = l; }
       }
-      const float sc = pvalid ? acc * a.scale : -INFINITY;
-      const float m = wave_max(sc);
-      const float e = pvalid ? __expf(sc - m) : 0.f;
-      const float l = wave_sum(e);
-      float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();
+    if (h0 + wave < group) {                            // wave w folds the row-run partials of head h0 + w into the split partial
+      const int head = kvh * group + h0 + wave;
+      const float* cb = comb + (size_t)wave * NGRP * CSTR;
+      float m = -INFINITY;                              // the first run of wave 0 always holds a valid position: m is finite
 #pragma unroll
-      for (int i = 0; i < NVI; i++) {
-        const float pj = __shfl(e, i * RPI + vr, 64);          // weight of the row this lane holds in instruction i (0 beyond pos)
-        const u32x4 vv = vt[i];
-        o[0] += pj * h2f_bits(vv.x & 0xFFFF); o[1] += pj * h2f_bits(vv.x >> 16); o[2] += pj * h2f_bits(vv.y & 0xFFFF); o[3] += pj * h2f_bits(vv.y >> 16);
-        o[4] += pj * h2f_bits(vv.z & 0xFFFF); o[5] += pj * h2f_bits(vv.z >> 16); o[6] += pj * h2f_bits(vv.w & 0xFFFF); o[7] += pj * h2f_bits(vv.w >> 16);
+      for (int g = 0; g < NGRP; g++) m = fmaxf(m, cb[g * CSTR + HD]);
+      float l = 0.f, od[HD / 64];
+#pragma unroll
+      for (int j = 0; j < HD / 64; j++) od[j] = 0.f;
+#pragma unroll
+      for (int g = 0; g < NGRP; g++) {
+        const float mg = cb[g * CSTR + HD];
+        const float wg = mg == -INFINITY ? 0.f : __expf(mg - m);   // a run without valid rows contributes nothing
+        l += wg * cb[g * CSTR + HD + 1];
+#pragma unroll
+        for (int j = 0; j < HD / 64; j++) od[j] += wg * cb[g * CSTR + lane + 64 * j];
       }
-      // sum the RPI lane groups that hold the same piece
-#pragma unroll
-      for (int off = HD8; off < 64; off <<= 1)
-#pragma unroll
-        for (int j = 0; j < 8; j++) o[j] += __shfl_xor(o[j], off, 64);
       float* po = a.part + ((size_t)head * a.nsplit + split) * (HD + 2);
-      if (lane < HD8) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) po[lane * 8 + j] = o[j];
-      }
-      if (lane == 0) { po[HD] = m; po[HD + 1] = l; }
+      for (int j = 0; j < HD / 64; j++) cst(&po[lane + 64 * j], od[j]);
+      if (lane == 0) { cst(&po[HD], m); cst(&po[HD + 1], l); }
     }
     __syncthreads();
   }
-  // ---- merge: the last split of this kv head to arrive combines all its heads' partials ----
+  // ---- merge: the last split of this kv head to arrive combines its heads' partials ----
   int* counters = (int*)(a.part + (size_t)a.n_heads * a.nsplit * (HD + 2));
   const int ns = (pos >> 6) + 1;
-  __threadfence();
+  stores_done();
   __syncthreads();
-  if (threadIdx.x == 0) {
-    const int prev = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) {
+    const int prev = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     last_flag = (prev == ns - 1);
     if (prev == ns - 1) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
   }
   __syncthreads();
   if (!last_flag) return;
-  __threadfence();
-  // softmax weights of every (head, split) first (parallel loads), then the weighted sum with 8 partial rows in flight per thread
-  __shared__ float sw[2048];                            // exp(m_s - m) / l per (head in group, split); host guarantees group * nsplit <= 2048
-  for (int idx = threadIdx.x; idx < group * ns; idx += 256) {
+  // (m, l) of every (head, split), then one wave per head forms the normalised weights, then the weighted sum with 16 splits in
+  // flight per output
+  for (int idx = tid; idx < group * ns; idx += 256) {
     const int gh = idx / ns, sp = idx - gh * ns;
     const float* ph = a.part + ((size_t)(kvh * group + gh) * a.nsplit + sp) * (HD + 2);
-    sw[gh * a.nsplit + sp] = __builtin_nontemporal_load(&ph[HD]);
-    sw[1024 + gh * a.nsplit + sp] = __builtin_nontemporal_load(&ph[HD + 1]);
+    sw[gh * a.nsplit + sp] = cld(&ph[HD]);
+    sw[1024 + gh * a.nsplit + sp] = cld(&ph[HD + 1]);
   }
   __syncthreads();
-  for (int gh = wave; gh < group; gh += 4) {            // one wave per head: m, l, then normalised weights in place
+  for (int gh = wave; gh < group; gh += 4) {
     float m = -INFINITY;
     for (int sp = lane; sp < ns; sp += 64) m = fmaxf(m, sw[gh * a.nsplit + sp]);
     m = wave_max(m);
@@ -205,16 +259,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
     for (int sp = lane; sp < ns; sp += 64) sw[gh * a.nsplit + sp] = __expf(sw[gh * a.nsplit + sp] - m) / l;
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < group * HD; idx += 256) {
+  constexpr int SC = 16;
+  for (int idx = tid; idx < group * HD; idx += 256) {
     const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
     const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
     float o = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += 8) {
-      float v[8];
+    for (int s0 = 0; s0 < ns; s0 += SC) {
+      float v[SC];
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = __builtin_nontemporal_load(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
+      for (int j = 0; j < SC; j++) v[j] = cld(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
 #pragma unroll
-      for (int j = 0; j < 8; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
+      for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
     }
     if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, head * HD + d, a.stage_nu) : head * HD + d] = (_Float16)o;
     if (a.out32) a.out32[head * HD + d] = o;
@@ -312,18 +367,22 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
   return 0;
 }
 
-int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
-                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
+int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                void* cache_k, void* cache_v, float* partials, const void* state,
+                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
   TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode: head_dim=%d must be 64, 128 or 256", head_dim);
   TGA_REQUIRE(max_ctx > 0 && (n_heads / n_kv_heads) * ((max_ctx + 63) / 64) <= 1024, "tga_attention_decode: max_ctx=%d too long for the merge table ((n_heads/n_kv_heads) * ceil(max_ctx/64) <= 1024)", max_ctx);
+  TGA_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr), "tga_attention_decode: q and k norm weights come together");
+  TGA_REQUIRE(!q_norm_weight || ((((uintptr_t)q | (uintptr_t)k) & 15) == 0), "tga_attention_decode: q and k must be 16-byte aligned for the fused norm");
   AttnArgs a;
   a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (const DecodeState*)state;
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
   a.stage_fmt = 0; a.stage_nu = 0;
+  a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps;
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
   const dim3 grid(n_kv_heads, a.nsplit);
   hipStream_t s = (hipStream_t)stream;
@@ -332,6 +391,12 @@ int tga_attention_decode(const float* q, const float* k, const float* v, void* c
   else attn_decode_kernel<32><<<grid, 256, 0, s>>>(a);
   TGA_LAUNCH_CHECK();
   return 0;
+}
+
+int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                         int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
+  return tga_attention_decode_normed(q, k, v, nullptr, nullptr, 0.f, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx, rope_table,
+                                     out_f16, out_f32, stage_type, stream);
 }
 
 int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i, void* state, const int* prompt, int* out_tokens, int max_tokens, void* stream) {

@@ -3,15 +3,14 @@
 #include "common.h"
 #include "host.h"
 
-// One workgroup (64 threads) per token.  scores per ExpertGating (model.py:9-13, 116-121): 1 SOFTMAX, 2 SIGMOID,
-// 3 SOFTMAX_WEIGHT (softmax over the selected logits), 4 SQRT_SOFTPLUS.  Top-k by pairwise rank exactly as pairwise_topk
-// (model.py:35-41): rank_i = #{j: s_i > s_j or (s_i == s_j and i < j)}; the k highest ranks are emitted in ASCENDING rank
-// order (the largest last), so among equal scores the lower index ranks higher.
-__global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ logits, int n_experts, int k, int gating, int norm_topk,
-                                                      float scale, int* __restrict__ sel, float* __restrict__ probs) {
-  extern __shared__ float sc[];                         // n_experts scores
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const float* lg = logits + (size_t)t * n_experts;
+// scores per ExpertGating (model.py:9-13, 116-121): 1 SOFTMAX, 2 SIGMOID, 3 SOFTMAX_WEIGHT (softmax over the selected logits),
+// 4 SQRT_SOFTPLUS.  Top-k by pairwise rank exactly as pairwise_topk (model.py:35-41): rank_i = #{j: s_i > s_j or (s_i == s_j and
+// i < j)}; the k highest ranks are emitted in ASCENDING rank order (the largest last), so among equal scores the lower index
+// ranks higher.  Runs on ONE wave (lane = threadIdx.x & 63 of the calling wave); lg may live in LDS or global memory, sc is
+// n_experts floats of LDS, tmp 192 floats of LDS.  The caller separates the call from earlier LDS writes with a barrier.
+__device__ __forceinline__ void gate_topk_wave(const float* lg, int n_experts, int k, int gating, int norm_topk, float scale,
+                                               int* __restrict__ sel, float* __restrict__ probs, float* sc, float* tmp, int lane) {
+  int* s_sel = (int*)tmp; float* s_p = tmp + 64; float* s_q = tmp + 128;
   if (gating == 1 && norm_topk) { gating = 3; norm_topk = 0; }   // model.py:116-117 fast path (no selection bias)
   float mx = -INFINITY;
   for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, lg[i]);
@@ -27,8 +26,7 @@ __global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ 
     else s = sqrtf(log1pf(expf(v)));
     sc[i] = s;
   }
-  __syncthreads();
-  __shared__ int s_sel[64]; __shared__ float s_p[64];
+  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's LDS writes are visible to its own lanes
   for (int i = lane; i < n_experts; i += 64) {
     const float si = sc[i];
     int rank = 0;
@@ -36,8 +34,7 @@ __global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ 
     const int slot = rank - (n_experts - k);
     if (slot >= 0) { s_sel[slot] = i; s_p[slot] = si; }
   }
-  __syncthreads();
-  __shared__ float s_q[64];
+  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);
   float p = lane < k ? s_p[lane] : 0.f;
   if (gating == 3 && lane < k) {                          // softmax over the selected logits
     float m2 = -INFINITY; for (int j = 0; j < k; j++) m2 = fmaxf(m2, s_p[j]);
@@ -45,12 +42,69 @@ __global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ 
     p = expf(p - m2) * (1.0f / z);
   }
   s_q[lane] = p;
-  __syncthreads();
+  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);
   if (lane < k) {
     if (norm_topk) { float z = 0.f; for (int j = 0; j < k; j++) z += s_q[j]; p = p / z; }
-    sel[(size_t)t * k + lane] = s_sel[lane];
-    probs[(size_t)t * k + lane] = p * scale;
+    sel[lane] = s_sel[lane];
+    probs[lane] = p * scale;
   }
+}
+
+// One workgroup (64 threads) per token.
+__global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ logits, int n_experts, int k, int gating, int norm_topk,
+                                                      float scale, int* __restrict__ sel, float* __restrict__ probs) {
+  extern __shared__ float sc[];                         // n_experts scores
+  __shared__ float tmp[192];
+  const int t = blockIdx.x;
+  gate_topk_wave(logits + (size_t)t * n_experts, n_experts, k, gating, norm_topk, scale, sel + (size_t)t * k, probs + (size_t)t * k, sc, tmp, threadIdx.x);
+}
+
+// Router of one token in one launch (tinygrad/llm/model.py:112-121 with the block's ffn_norm, :150): h = RMSNorm(x) * weight rounded
+// to fp16 (also written to xn_out for the expert GEMVs that follow), logits = h @ Wr^T for a dense fp16 router weight (n_experts,
+// dim), then gating + top-k as above.  One workgroup of 1024 threads: the normalised row lives in LDS, wave w takes rows w, w + 16, ...
+#define ROUTER_THREADS 1024
+__global__ __launch_bounds__(ROUTER_THREADS) void moe_router_kernel(const float* __restrict__ x, const float* __restrict__ norm_w, float eps, const _Float16* __restrict__ wr,
+                                                                    int dim, int n_experts, int k, int gating, int norm_topk, float scale,
+                                                                    _Float16* __restrict__ xn_out, float* __restrict__ logits_out, int* __restrict__ sel, float* __restrict__ probs) {
+  extern __shared__ float dyn[];                        // logits[n_experts] | scores[n_experts] | fp16 row [dim]
+  float* lg = dyn; float* sc = dyn + n_experts;
+  _Float16* xn = (_Float16*)(dyn + 2 * n_experts);
+  __shared__ float red[ROUTER_THREADS / 64];
+  __shared__ float tmp[192];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float s = 0.f;
+  for (int e = tid; e < dim; e += ROUTER_THREADS) { const float v = x[e]; s += v * v; }
+  s = wave_sum(s);
+  if (lane == 0) red[wave] = s;
+  __syncthreads();
+  float tot = 0.f;
+  for (int i = 0; i < ROUTER_THREADS / 64; i++) tot += red[i];
+  const float nscale = norm_w ? 1.0f / sqrtf(tot / (float)dim + eps) : 1.f;
+  for (int e = tid; e < dim; e += ROUTER_THREADS) {
+    const _Float16 h = (_Float16)(norm_w ? (x[e] * nscale) * norm_w[e] : x[e]);
+    xn[e] = h;
+    if (xn_out) xn_out[e] = h;
+  }
+  __syncthreads();
+  const int np = dim / 8;                               // 16-byte pieces per row
+  for (int r0 = wave * 4; r0 < n_experts; r0 += (ROUTER_THREADS / 64) * 4) {   // four rows per wave pass, loads of all four in flight
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int p = lane; p < np; p += 64) {
+      const u32x4 xv = *(const u32x4*)(xn + 8 * p);
+      u32x4 wv[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) { const int r = r0 + j < n_experts ? r0 + j : n_experts - 1; wv[j] = *(const u32x4*)(wr + (size_t)r * dim + 8 * p); }
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[j] = dot2(wv[j].w, xv.w, dot2(wv[j].z, xv.z, dot2(wv[j].y, xv.y, dot2(wv[j].x, xv.x, acc[j]))));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float t = wave_sum(acc[j]);
+      if (lane == 0 && r0 + j < n_experts) { lg[r0 + j] = t; if (logits_out) logits_out[r0 + j] = t; }
+    }
+  }
+  __syncthreads();
+  if (wave == 0) gate_topk_wave(lg, n_experts, k, gating, norm_topk, scale, sel, probs, sc, tmp, lane);
 }
 
 // out[t, :] = resid[t, :] + sum_s probs[t, s] * y[t, s, :]     ((x_down * probs).sum(axis=2), model.py:130, plus the block residual :150)
@@ -72,6 +126,18 @@ int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int ga
   TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 4096 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_gate: bad geometry (k <= 64, n_experts <= 4096)");
   TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_gate: unknown ExpertGating %d", gating);
   moe_gate_kernel<<<n_tokens, 64, n_experts * sizeof(float), (hipStream_t)stream>>>(logits, n_experts, k, gating, norm_topk_prob, scale, sel, probs);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
+                   int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_out, int32_t* sel, float* probs, void* stream) {
+  TGA_REQUIRE(x && router_w_f16 && sel && probs, "tga_moe_router: null pointer");
+  TGA_REQUIRE(dim >= 8 && dim % 8 == 0 && dim <= 16384 && ((uintptr_t)router_w_f16 & 15) == 0, "tga_moe_router: dim=%d must be a multiple of 8, at most 16384, with a 16-byte aligned weight", dim);
+  TGA_REQUIRE(n_experts >= 1 && n_experts <= 1024 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_router: bad geometry (k <= 64, n_experts <= 1024)");
+  TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_router: unknown ExpertGating %d", gating);
+  moe_router_kernel<<<1, ROUTER_THREADS, 2 * n_experts * sizeof(float) + (size_t)dim * 2, (hipStream_t)stream>>>(
+      x, norm_weight, norm_eps, (const _Float16*)router_w_f16, dim, n_experts, k, gating, norm_topk_prob, scale, (_Float16*)xn_out_f16, logits_out, sel, probs);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -24,6 +24,9 @@ struct QArgs {
   // x_staged: x already holds fp16 activations in the consumer format's staged order (Fmt::spos).
   // y_stage_fmt / y_stage_nu: when y_stage_fmt != 0 the fp16 outputs are written in the staged order of THAT consumer format.
   int x_staged, y_stage_fmt, y_stage_nu;
+  // norm_w != nullptr (M = 1 fast path, fp32 x): the activation row is RMS-normalised while it is staged,
+  // x * rsqrt(mean(x^2) + norm_eps) * norm_w (nn.RMSNorm, tinygrad/nn/__init__.py:296-304), then rounded to fp16.
+  const float* norm_w; float norm_eps;
 };
 
 // staged position of element e for a consumer of format `fmt` (row length K = UW * nu)

@@ -375,9 +375,9 @@ extern "C" int tga_stage_activation(int ggml_type, const void* x, int x_dtype, i
   return 0;
 }
 
-extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
-                                 const void* x, int x_dtype, int y_dtype, int M, int64_t K,
-                                 int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
+static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                              const void* x, int x_dtype, int y_dtype, int M, int64_t K,
+                              int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
   TGA_REQUIRE(M >= 1 && M <= 8, "tga_qlinear: M=%d out of range 1..8", M);
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
@@ -409,6 +409,10 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     a.y_stage_fmt = staged_fmt(y_stage_type, y_stage_K, &a.y_stage_nu);
     TGA_REQUIRE(a.y_stage_fmt >= 0, "tga_qlinear: no staged layout for consumer type %d with K=%lld", y_stage_type, (long long)y_stage_K);
   }
+  if (norm_w) {
+    TGA_REQUIRE(M == 1 && x_dtype == TGA_F32 && ((uintptr_t)norm_w & 15) == 0, "tga_rmsnorm_qlinear: needs M = 1, float32 x and a 16-byte aligned norm weight");
+    a.norm_w = norm_w; a.norm_eps = norm_eps;
+  }
   hipStream_t s = (hipStream_t)stream;
   // block-pair units need an even number of blocks per row and 4-byte aligned rows
   bool pair = (K / 32) % 2 == 0;
@@ -417,6 +421,7 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
   }
+  TGA_REQUIRE(!norm_w, "tga_rmsnorm_qlinear: the fused norm needs the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, 16-byte aligned x, K <= 65536)");
   TGA_REQUIRE(!a.x_staged && !a.y_stage_fmt, "tga_qlinear: staged activations need the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, K <= 65536)");
   switch (ggml_type) {
     case GGML_Q4_0: return pair ? launch_qgemv_m<F_Q4_0P>(a, M, s) : launch_qgemv_m<GGML_Q4_0>(a, M, s);
@@ -425,6 +430,22 @@ extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, 
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
   }
   return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
+}
+
+extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                                 const void* x, int x_dtype, int y_dtype, int M, int64_t K,
+                                 int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
+  return qlinear_multi_impl(nullptr, 0.f, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+}
+
+// RMSNorm (nn.RMSNorm, tinygrad/nn/__init__.py:296-304) of the float32 activation row folded into the M = 1 linear that consumes it
+// (attn_norm -> attn_q/k/v, ffn_norm -> ffn_gate/up, output_norm -> output: tinygrad/llm/model.py:149-150, 362): no normalised copy
+// of the row goes through memory.
+extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                                         const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
+                                         int y_stage_type, int64_t y_stage_K, void* stream) {
+  TGA_REQUIRE(norm_weight, "tga_rmsnorm_qlinear_multi: null norm weight");
+  return qlinear_multi_impl(norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
 }
 
 extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,

@@ -19,6 +19,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
   constexpr int USTRIDE = NP + 4;                                // padded unit stride in dwords
   extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
   __shared__ float part[2][WK][R];
+  __shared__ float nred[NT / 64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wk = (WK > 1) ? wave : 0, wr = (WK > 1) ? 0 : wave;
@@ -114,11 +115,29 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
     if (!staged) {
       // activations: coalesced global -> LDS (natural order, padded unit stride) -> this lane's unit -> staged registers
       const int nq = a.K / 8;                                      // 16-byte fp16 pieces in the row
+      float nscale = 1.f;
+      if (a.norm_w) {                                              // fused RMSNorm: sum of squares over the workgroup first
+        const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < 2 * nq; i += NT) { const f32x4 v = xr[i]; ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+        ss = wave_sum(ss);
+        if (lane == 0) nred[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < NT / 64; j++) tot += nred[j];
+        nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+      }
       for (int i = threadIdx.x; i < nq; i += NT) {
         u32x4 v;
         if (a.x_f32) {
           const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
-          const f32x4 lo4 = xr[2 * i], hi4 = xr[2 * i + 1];
+          f32x4 lo4 = xr[2 * i], hi4 = xr[2 * i + 1];
+          if (a.norm_w) {
+            const f32x4 w0 = ((const f32x4*)a.norm_w)[2 * i], w1 = ((const f32x4*)a.norm_w)[2 * i + 1];
+            lo4.x = (lo4.x * nscale) * w0.x; lo4.y = (lo4.y * nscale) * w0.y; lo4.z = (lo4.z * nscale) * w0.z; lo4.w = (lo4.w * nscale) * w0.w;
+            hi4.x = (hi4.x * nscale) * w1.x; hi4.y = (hi4.y * nscale) * w1.y; hi4.z = (hi4.z * nscale) * w1.z; hi4.w = (hi4.w * nscale) * w1.w;
+          }
           v.x = f2h_bits(lo4.x) | (f2h_bits(lo4.y) << 16); v.y = f2h_bits(lo4.z) | (f2h_bits(lo4.w) << 16);
           v.z = f2h_bits(hi4.x) | (f2h_bits(hi4.y) << 16); v.w = f2h_bits(hi4.z) | (f2h_bits(hi4.w) << 16);
         } else v = ((const u32x4*)((const uint16_t*)a.x + xrow * a.K))[i];

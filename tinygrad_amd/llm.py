@@ -13,7 +13,7 @@ from dataclasses import dataclass
 import numpy as np
 from tinygrad_amd import runtime as rt
 from tinygrad_amd.runtime import Buffer, GGML_QUANT
-from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine
+from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine, moe_router
 
 @dataclass(frozen=True)
 class TransformerConfig:
@@ -139,31 +139,46 @@ class TransformerBlock:
     self.staged = (not self.moe) and all(l.ggml_type in (rt.Q4_0, rt.Q8_0, rt.F16) and l.in_features % 64 == 0 and l.in_features <= 65536
                                          for l in (self.attn_q, self.attn_output, self.ffn_gate, self.ffn_down)) \
                   and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
+    # RMSNorm folded into the consuming M = 1 linear (needs its register-resident fast path: K % 64, 4-byte aligned weights)
+    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type != rt.Q6_K or l.in_features % 256 == 0)
+    self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
 
   def __call__(self, x: Buffer, stream):
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     st = self.staged                                                     # producers write the consumer's staged order directly
-    rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.attn_q.ggml_type if st else 0, stream))
-    qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream, x_staged=st)
-    if c.qk_norm:                                                        # full-width q/k RMSNorm before the head split (model.py:169)
-      assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
-      rt.check(L.tga_rmsnorm(s.q.ptr, self.q_norm.ptr, c.n_heads * c.head_dim, c.norm_eps, None, s.q.ptr, 0, stream))
-      rt.check(L.tga_rmsnorm(s.k.ptr, self.k_norm.ptr, c.n_kv_heads * c.head_dim, c.norm_eps, None, s.k.ptr, 0, stream))
-    rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if st else 0, stream))
+    if st:
+      rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.attn_q.ggml_type, stream))
+      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream, x_staged=True)
+    elif self.fuse_norm:                                                 # the q/k/v launch normalises the row while staging it
+      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], x, [s.q, s.k, s.v], stream=stream, norm=(self.attn_norm, c.norm_eps))
+    else:
+      rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
+      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream)
+    if c.qk_norm: assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
+    # full-width q/k RMSNorm before the head split (model.py:169) inside the attention launch
+    rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
+                                           self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
+                                           s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if st else 0, stream))
     qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     if not self.moe:
-      rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if st else 0, stream))
-      qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=st, stage_out_for=self.ffn_down if st else None)
+      if not st and self.fuse_norm:
+        qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps))
+      else:
+        rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if st else 0, stream))
+        qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=st, stage_out_for=self.ffn_down if st else None)
       qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
       return
-    rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
-    self.ffn_gate_inp(s.xn, out=s.router, stream=stream)
-    moe_gate(s.router, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
+    if self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024:
+      moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, xn_out=s.xn, logits_out=s.router, gating=c.expert_gating_func,
+                 norm_topk_prob=c.norm_topk_prob, scale=c.routed_scaling_factor, stream=stream)
+    else:
+      rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
+      self.ffn_gate_inp(s.xn, out=s.router, stream=stream)
+      moe_gate(s.router, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
     self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
     self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
     moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)
@@ -203,6 +218,7 @@ class Transformer:
     self.output_norm = state_dict["output_norm.weight"][0]
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
+    self.fuse_head_norm = c.dim % (256 if out[1] == rt.Q6_K else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
     self.stream = rt.Stream()
     self._graphs = {}
     # one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
@@ -239,8 +255,11 @@ class Transformer:
     else:
       for b in self.blk: b(s.x, st)
     if with_head:
-      rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
-      self.output(s.xn, out=s.logits, stream=st)
+      if self.fuse_head_norm:                                          # output_norm inside the lm-head launch (model.py:362)
+        qlinear_multi([self.output], s.x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps))
+      else:
+        rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
+        self.output(s.xn, out=s.logits, stream=st)
       rt.check(L.tga_argmax_step(s.logits.ptr, c.vocab_size, s.am_v.ptr, s.am_i.ptr, s.state.ptr, s.prompt.ptr, s.out_tokens.ptr, self.max_new, st))
     else:
       rt.check(L.tga_advance_prompt(s.state.ptr, s.prompt.ptr, st))

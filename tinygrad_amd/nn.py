@@ -32,11 +32,12 @@ class QuantLinear:
     return out
 
 def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None,
-                  x_staged: bool = False, stage_out_for: QuantLinear | None = None):
+                  x_staged: bool = False, stage_out_for: QuantLinear | None = None, norm: tuple[Buffer, float] | None = None):
   """Several QuantLinear layers over the same activation in one launch (attn_q/k/v, ffn_gate/ffn_up).
   epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x).
   x_staged: x is already in the staged order of these weights (stage_activation or a staging producer).
-  stage_out_for: write the single fp16 output in the staged order of that consumer layer."""
+  stage_out_for: write the single fp16 output in the staged order of that consumer layer.
+  norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it."""
   nseg = len(layers)
   t, k = layers[0].ggml_type, layers[0].in_features
   assert all(l.ggml_type == t and l.in_features == k for l in layers)
@@ -48,6 +49,11 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   r = VP(*[b.ptr for b in resid]) if resid is not None else None
   ydt = rt.dtype_code(outs[0].dtype)
   so = stage_out_for
+  if norm is not None:
+    assert m == 1 and x.dtype == np.float32 and not x_staged
+    rt.check(rt.lib().tga_rmsnorm_qlinear_multi(norm[0].ptr, norm[1], t, nseg, w, y, n, x.ptr, ydt, k, epilogue, r,
+                                                so.ggml_type if so is not None else 0, so.in_features if so is not None else 0, stream))
+    return outs
   rt.check(rt.lib().tga_qlinear_multi(t, nseg, w, y, n, x.ptr, rt.F16_STAGED if x_staged else rt.dtype_code(x.dtype), ydt, m, k, epilogue, r,
                                       so.ggml_type if so is not None else 0, so.in_features if so is not None else 0, stream))
   return outs
@@ -74,6 +80,14 @@ class ExpertWeights:
 
 def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer, probs: Buffer, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
   rt.check(rt.lib().tga_moe_gate(logits.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
+
+def moe_router(x: Buffer, norm_weight: Buffer | None, eps: float, router: QuantLinear, k: int, sel: Buffer, probs: Buffer, xn_out: Buffer | None = None,
+               logits_out: Buffer | None = None, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
+  """ffn_norm + router logits + gating + top-k of one token in one launch (dense fp16 router weight)."""
+  assert router.ggml_type == rt.F16
+  rt.check(rt.lib().tga_moe_router(x.ptr, norm_weight.ptr if norm_weight is not None else None, eps, router.blocks.ptr, router.in_features, router.out_features, k,
+                                   gating, int(norm_topk_prob), scale, xn_out.ptr if xn_out is not None else None,
+                                   logits_out.ptr if logits_out is not None else None, sel.ptr, probs.ptr, stream))
 
 def moe_combine(y: Buffer, probs: Buffer, resid: Buffer | None, n_tokens: int, k: int, dim: int, out: Buffer, stream=None):
   rt.check(rt.lib().tga_moe_combine(y.ptr, probs.ptr, resid.ptr if resid is not None else None, n_tokens, k, dim, out.ptr, stream))

@@ -30,10 +30,12 @@ def _declare(lib):
     "tga_dequant": [i, vp, i64, vp, i, vp],
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
     "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, i, i64, vp],
+    "tga_rmsnorm_qlinear_multi": [vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i64, i, c_void_pp, i, i64, vp],
     "tga_stage_activation": [i, vp, i, i64, vp, vp],
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
+    "tga_moe_router": [vp, vp, ctypes.c_float, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp, vp, vp],
     "tga_quantize_mxfp8": [vp, i, i64, i64, vp, vp, vp, vp],
     "tga_moe_route": [vp, i, i, i, vp, vp, vp, vp, vp, vp, vp],
     "tga_moe_dispatch": [vp, vp, vp, vp, i, i, i, i64, i, vp, vp],
@@ -43,6 +45,7 @@ def _declare(lib):
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
+    "tga_attention_decode_normed": [vp, vp, vp, vp, vp, ctypes.c_float, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
     "tga_decode_layers": [vp, i, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, ctypes.c_float, vp],
     "tga_decode_layers_trace": [vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
