@@ -106,10 +106,11 @@ int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int ga
                  int32_t* sel, float* probs, void* stream);
 /* Router of ONE token in one launch (model.py:112-128 with the block's ffn_norm, :150): h = fp16(RMSNorm(x) * norm_weight) (norm_weight
  * NULL: h = fp16(x)), logits = h @ Wr^T for a dense fp16 router weight (n_experts, dim), then gating + top-k as tga_moe_gate.
- * xn_out_f16 (dim fp16, the activation of the expert GEMVs) and logits_out (n_experts floats) may be NULL.
- * dim % 8 == 0, dim <= 16384, n_experts <= 1024, k <= 64. */
+ * xn_out_f16 (dim fp16, the activation of the expert GEMVs) may be NULL.  logits_ws: n_experts floats (the logits, readable
+ * afterwards) followed by one int32 arrival counter that must be ZERO before the first call (each call leaves it zero); calls
+ * sharing one workspace must not overlap.  dim % 8 == 0, dim <= 16384, n_experts <= 1024, k <= 64. */
 int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
-                   int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_out, int32_t* sel, float* probs, void* stream);
+                   int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_ws, int32_t* sel, float* probs, void* stream);
 /* out[t] = resid[t] + sum_s probs[t, s] * y[t, s, :]  (model.py:130 and the residual add :150); resid may be NULL or alias out. */
 int tga_moe_combine(const float* y, const float* probs, const float* resid, int n_tokens, int k, int dim, float* out, void* stream);
 

@@ -67,15 +67,18 @@ def test_router_in_one_launch(gpu, dim, E, k, gating, normw):
   x = (rng.standard_normal(dim) * 2).astype(np.float32); nw = rng.standard_normal(dim).astype(np.float32)
   wr = (rng.standard_normal((E, dim)) * dim ** -0.5).astype(np.float16)
   router = QuantLinear(gpu.Buffer.from_numpy(wr.view(np.uint8).reshape(-1)), rt.F16, E, dim)
-  xn, lg = gpu.Buffer((dim,), np.float16), gpu.Buffer((E,), np.float32)
+  xn, lg = gpu.Buffer((dim,), np.float16), gpu.Buffer((E + 1,), np.float32).zero_()
   sel, pr = gpu.Buffer((k,), np.int32), gpu.Buffer((k,), np.float32)
-  moe_router(gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw) if normw else None, 1e-5, router, k, sel, pr, xn_out=xn, logits_out=lg, gating=gating,
-             norm_topk_prob=True, scale=1.5)
+  for _ in range(2):                                                     # twice: the arrival counter is left at zero
+    moe_router(gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw) if normw else None, 1e-5, router, k, sel, pr, lg, xn_out=xn, gating=gating,
+               norm_topk_prob=True, scale=1.5)
+  assert lg.numpy()[E:].view(np.int32)[0] == 0
+  lgv = lg.numpy()[:E]
   h = (ollm.rmsnorm(x, nw, 1e-5) if normw else x).astype(np.float16)
   assert np.mean(xn.numpy() != h) < 0.01 and ol.rel_err(xn.numpy().astype(np.float32), h.astype(np.float32)) < 1e-3   # fp16 ties may round either way
   ref_lg = (h.astype(np.float64) @ wr.astype(np.float64).T).astype(np.float32)
-  assert ol.rel_err(lg.numpy(), ref_lg) <= 1e-3
-  rs, rp = omoe.gate_probs(lg.numpy()[None], k, gating, True, 1.5)        # selection on the kernel's own logits: exact
+  assert ol.rel_err(lgv, ref_lg) <= 1e-3
+  rs, rp = omoe.gate_probs(lgv[None], k, gating, True, 1.5)        # selection on the kernel's own logits: exact
   np.testing.assert_array_equal(sel.numpy(), rs[0])
   np.testing.assert_allclose(pr.numpy(), rp[0], rtol=2e-5, atol=1e-7)
 

@@ -44,6 +44,15 @@ __device__ __forceinline__ float wave_sum_lane63(float v) {
   v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2,3
   return v;
 }
+// Sums over lanes 0-31 and over lanes 32-63 separately.  Results valid in lanes 31 and 63.
+__device__ __forceinline__ float half_sum_lane31(float v) {
+  v = dpp_add<0xB1>(v);
+  v = dpp_add<0x4E>(v);
+  v = dpp_add<0x141>(v);
+  v = dpp_add<0x140>(v);
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1,3: lane 31 = rows 0+1, lane 63 = rows 2+3
+  return v;
+}
 __device__ __forceinline__ float wave_sum(float v) {
   v = wave_sum_lane63(v);
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));

@@ -268,15 +268,27 @@ template <> struct Fmt<F_Q8_0P> {
 // ------------------------------------------------------------------------------------------------ F16 (dense fp16 rows, gguf.py:35-36)
 // unit = 64 consecutive fp16 weights (128 bytes); no decode: the weight dwords are the fp16 pairs.
 template <> struct Fmt<GGML_F16> {
+  // A unit is 64 weights, but NOT 64 consecutive ones: the row is cut into 16-byte pieces (8 weights) and unit u owns pieces
+  // u, u + nu, ..., u + 7 nu (nu = units per row), so that load instruction j of a wave covers pieces j*nu .. j*nu + 63, one
+  // contiguous span (a lane stride of 128 bytes would touch 64 cache lines per instruction).  The fast M = 1 kernel uses
+  // load_nu / unit_of_nu / pair_of_nu; the staged order of a row is therefore the natural order.
   static constexpr int UW = 64, UPB = 1, BW = 64, BB = 128;
   static __device__ __forceinline__ int unit_of(int e) { return e / UW; }
   static __device__ __forceinline__ int pair_of(int e) { return (e % UW) >> 1; }
+  static __device__ __forceinline__ int unit_of_nu(int e, int nu) { return (e >> 3) % nu; }
+  static __device__ __forceinline__ int pair_of_nu(int e, int nu) { return ((e >> 3) / nu) * 4 + ((e & 7) >> 1); }
   static constexpr int XV = 8, NG = 1, NWV = 32;
   struct Raw { u32x4 q[8]; };
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
     const uint8_t* p = row + 128 * u; Raw r;
 #pragma unroll
     for (int i = 0; i < 8; i++) r.q[i] = ld16_a4(p + 16 * i);
+    return r;
+  }
+  static __device__ __forceinline__ Raw load_nu(const uint8_t* row, int u, int nu) {
+    const uint8_t* p = row + 16 * u; Raw r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.q[i] = ld16_a4(p + (size_t)16 * nu * i);
     return r;
   }
   static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
@@ -292,7 +304,7 @@ template <> struct Fmt<GGML_F16> {
     c[0] = 0.f;
   }
   static __device__ __forceinline__ float finish(const Raw&, const float* a) { return a[0]; }
-  static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 6, w = e & 63; return (((w >> 3) * nu + u) * 4 + ((w >> 1) & 3)) * 2 + (w & 1); }
+  static __device__ __forceinline__ int spos(int e, int nu) { return e; }
   static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
 

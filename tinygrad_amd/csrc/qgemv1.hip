@@ -9,11 +9,15 @@
 // are in flight while group g is multiplied and reduced.
 // Activations reach the registers through one LDS transpose per workgroup: coalesced 16-byte global loads of the plain row,
 // then each lane reads back the 64 (or 32) values of its unit (unit stride padded to spread LDS banks).
-template <int T, int R, int WK, int WR, int EPI>
+// H (rows of at most 32 units, WK = 1): a row occupies half a wave, so each half-wave is a row team of its own (lanes 0-31 and
+// 32-63 walk different row ranges; the DPP sum stops at 32 lanes) instead of leaving half of the lanes without loads.
+template <int T, int R, int WK, int WR, int EPI, bool H>
 __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
   using F = Fmt<T>;
   typedef typename F::Raw Raw;
   static_assert(WK == 1 || WR == 1, "row teams and K split are not combined");
+  static_assert(!H || WK == 1, "half-wave rows need the whole row inside one wave");
+  constexpr int HM = H ? 2 : 1;
   constexpr int NT = WK * WR * 64;
   constexpr int NP = F::UW / 2;                                  // dwords (fp16 pairs) per unit
   constexpr int USTRIDE = NP + 4;                                // padded unit stride in dwords
@@ -23,14 +27,15 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wk = (WK > 1) ? wave : 0, wr = (WK > 1) ? 0 : wave;
-  const int u = wk * 64 + lane;
+  const int hl = H ? (lane & 31) : lane, hrow = H ? (lane >> 5) : 0;
+  const int u = wk * 64 + hl;
   const bool uvalid = u < a.nu;
   const int job = blockIdx.y;
   const long long eoff = a.sel ? (long long)a.sel[job] * a.estride : 0, yofs = (long long)job * a.ystride;
   const long long xrow = a.sel ? job / a.xdiv : 0;
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
   const long long ngroups = (a.ntot + RS - 1) / RS;
-  const long long nteams = (long long)gridDim.x * WR, team = (long long)blockIdx.x * WR + wr;
+  const long long nteams = (long long)gridDim.x * WR * HM, team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
   const long long gbase = ngroups / nteams, grem = ngroups % nteams;
   const long long g0 = team * gbase + (team < grem ? team : grem), g1 = g0 + gbase + (team < grem ? 1 : 0);
   const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
@@ -58,7 +63,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
       for (int r = 0; r < R; r++) {
         long long rr = (EPI == 2) ? row : row + r;
         rr = rr < hi - 1 ? rr : hi - 1;                            // beyond the range: reload the last valid row
-        buf[r] = F::load(((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes, uc);
+        const uint8_t* rp = ((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes;
+        if constexpr (T == GGML_F16) buf[r] = F::load_nu(rp, uc, a.nu); else buf[r] = F::load(rp, uc);
       }
     };
     auto finish_group = [&](const Raw* buf, long long row) {
@@ -67,7 +73,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
       for (int r = 0; r < R; r++) {
         acc[r] = 0.f;
         unit_dot_reg<T>(buf[r], xv, cv, acc[r], kc);
-        acc[r] = wave_sum_lane63(uvalid ? acc[r] : 0.f);
+        acc[r] = H ? half_sum_lane31(uvalid ? acc[r] : 0.f) : wave_sum_lane63(uvalid ? acc[r] : 0.f);
       }
       if constexpr (WK > 1) {
         if (lane == 63) {
@@ -90,7 +96,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
         }
         parity ^= 1;
       } else {
-        if (lane == 63) {
+        if (hl == (H ? 31 : 63)) {
           if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1], yofs);
           else {
 #pragma unroll
@@ -142,7 +148,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
           v.z = f2h_bits(hi4.x) | (f2h_bits(hi4.y) << 16); v.w = f2h_bits(hi4.z) | (f2h_bits(hi4.w) << 16);
         } else v = ((const u32x4*)((const uint16_t*)a.x + xrow * a.K))[i];
         // element 8i lives in unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
-        *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
+        if constexpr (T == GGML_F16) *(u32x4*)(xlds + F::unit_of_nu(8 * i, a.nu) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v;
+        else *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
       }
       __syncthreads();
       {
@@ -173,7 +180,7 @@ static int fast_cu_count() {
   return n;
 }
 
-template <int T, int R, int WK, int WR, int EPI>
+template <int T, int R, int WK, int WR, int EPI, bool H = false>
 static int launch_fast(QArgs a, hipStream_t s) {
   using F = Fmt<T>;
   constexpr int RS = (EPI == 2) ? 1 : R;
@@ -182,13 +189,18 @@ static int launch_fast(QArgs a, hipStream_t s) {
   // resident row teams per CU: 16 waves (<= 128 VGPRs) unless the staged activations in LDS (160 KB per CU) allow fewer
   int wg_per_cu = 16 / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;
   const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
-  long long max_teams = (long long)fast_cu_count() * wg_per_cu * WR;
+  constexpr int TPW = WR * (H ? 2 : 1);                           // row teams per workgroup
+  long long max_teams = (long long)fast_cu_count() * wg_per_cu * TPW;
   if (a.sel && a.xdiv_jobs > 1) { max_teams = (max_teams + a.xdiv_jobs - 1) / a.xdiv_jobs; if (max_teams < 1) max_teams = 1; }
-  const long long per = (ngroups + max_teams - 1) / max_teams;     // row groups per team
+  long long per = (ngroups + max_teams - 1) / max_teams;           // row groups per team
+  // short rows: a team should own a few row groups, so that the activation staging of its workgroup is paid once per several
+  // rows, as long as every CU still gets a workgroup
+  long long per_min = ngroups / ((long long)fast_cu_count() * TPW); per_min = per_min < 1 ? 1 : per_min > 4 ? 4 : per_min;
+  if (!a.sel && per < per_min) per = per_min;
   const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
-  long long grid = (teams + WR - 1) / WR;
+  long long grid = (teams + TPW - 1) / TPW;
   if (grid < 1) grid = 1;
-  auto kern = qgemv1_kernel<T, R, WK, WR, EPI>;
+  auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H>;
   if (lds > 48 * 1024) {
     static bool configured = false;
     if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); configured = true; }
@@ -198,14 +210,14 @@ static int launch_fast(QArgs a, hipStream_t s) {
   return 0;
 }
 
-template <int T, int WK, int WR>
+template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
-  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2>(a, s);
+  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice
   // (the wide Q8_0 / Q6_K units would need > 128 VGPRs with two rows in flight twice: one row there)
   const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4) && a.ntot >= (long long)fast_cu_count() * 16 * 2 / WK;
-  if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1>(a, s) : launch_fast<T, 1, WK, WR, 1>(a, s);
-  return r2 ? launch_fast<T, 2, WK, WR, 0>(a, s) : launch_fast<T, 1, WK, WR, 0>(a, s);
+  if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
+  return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);
 }
 
 template <int T>
@@ -214,6 +226,7 @@ static int launch_fast_w(QArgs a, hipStream_t s) {
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const int waves = (a.nu + 63) / 64;
+  if (a.nu <= 32) return launch_fast_e<T, 1, 4, true>(a, s);
   if (waves <= 1) return launch_fast_e<T, 1, 4>(a, s);
   if (waves <= 2) return launch_fast_e<T, 2, 1>(a, s);
   if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);

@@ -173,12 +173,13 @@ class TransformerBlock:
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
     if self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024:
-      moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, xn_out=s.xn, logits_out=s.router, gating=c.expert_gating_func,
+      moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, s.router, xn_out=s.xn, gating=c.expert_gating_func,
                  norm_topk_prob=c.norm_topk_prob, scale=c.routed_scaling_factor, stream=stream)
     else:
       rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
-      self.ffn_gate_inp(s.xn, out=s.router, stream=stream)
-      moe_gate(s.router, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
+      lg = s.router.view(0, (1, c.num_experts), np.float32)
+      self.ffn_gate_inp(s.xn, out=lg, stream=stream)
+      moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
     self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
     self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
     moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)
@@ -199,7 +200,7 @@ class _Shared:
     self.act = Buffer((1, c.hidden_dim), f16)
     if c.num_experts:
       k = c.num_experts_per_tok
-      self.router, self.sel, self.probs = Buffer((1, c.num_experts), f32), Buffer((k,), np.int32), Buffer((k,), f32)
+      self.router, self.sel, self.probs = Buffer((1, c.num_experts + 1), f32).zero_(), Buffer((k,), np.int32), Buffer((k,), f32)   # logits + arrival counter
       self.act_e, self.y_e = Buffer((k, c.hidden_dim), f16), Buffer((k, c.dim), f32)
     self.logits = Buffer((1, c.vocab_size), f32)
     self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)

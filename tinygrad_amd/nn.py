@@ -81,13 +81,13 @@ class ExpertWeights:
 def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer, probs: Buffer, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
   rt.check(rt.lib().tga_moe_gate(logits.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
 
-def moe_router(x: Buffer, norm_weight: Buffer | None, eps: float, router: QuantLinear, k: int, sel: Buffer, probs: Buffer, xn_out: Buffer | None = None,
-               logits_out: Buffer | None = None, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
-  """ffn_norm + router logits + gating + top-k of one token in one launch (dense fp16 router weight)."""
-  assert router.ggml_type == rt.F16
+def moe_router(x: Buffer, norm_weight: Buffer | None, eps: float, router: QuantLinear, k: int, sel: Buffer, probs: Buffer, logits_ws: Buffer,
+               xn_out: Buffer | None = None, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
+  """ffn_norm + router logits + gating + top-k of one token in one launch (dense fp16 router weight).
+  logits_ws: n_experts + 1 float32, zero before the first use (the last word is an arrival counter)."""
+  assert router.ggml_type == rt.F16 and logits_ws.nbytes >= 4 * (router.out_features + 1)
   rt.check(rt.lib().tga_moe_router(x.ptr, norm_weight.ptr if norm_weight is not None else None, eps, router.blocks.ptr, router.in_features, router.out_features, k,
-                                   gating, int(norm_topk_prob), scale, xn_out.ptr if xn_out is not None else None,
-                                   logits_out.ptr if logits_out is not None else None, sel.ptr, probs.ptr, stream))
+                                   gating, int(norm_topk_prob), scale, xn_out.ptr if xn_out is not None else None, logits_ws.ptr, sel.ptr, probs.ptr, stream))
 
 def moe_combine(y: Buffer, probs: Buffer, resid: Buffer | None, n_tokens: int, k: int, dim: int, out: Buffer, stream=None):
   rt.check(rt.lib().tga_moe_combine(y.ptr, probs.ptr, resid.ptr if resid is not None else None, n_tokens, k, dim, out.ptr, stream))
