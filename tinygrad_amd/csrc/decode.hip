@@ -40,8 +40,19 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, int dim, float eps,
                                                        _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu) {
   __shared__ float red[16];
-  float s = 0.f;
-  for (int e = threadIdx.x; e < dim; e += blockDim.x) { const float v = x[e]; s += v * v; }
+  // two elements per thread and loop pass are requested together and kept for the second pass (rows up to 2048 values never reload)
+  float s = 0.f, v0 = 0.f, v1 = 0.f, w0 = 0.f, w1 = 0.f;
+  const int e0 = threadIdx.x, e1 = threadIdx.x + 1024;
+  if (e0 < dim) { v0 = x[e0]; w0 = w[e0]; }
+  if (e1 < dim) { v1 = x[e1]; w1 = w[e1]; }
+  s = v0 * v0 + v1 * v1;
+  for (int b = threadIdx.x + 2048; b < dim; b += 4096) {
+    float t[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) t[j] = x[b + 1024 * j < dim ? b + 1024 * j : dim - 1];
+#pragma unroll
+    for (int j = 0; j < 4; j++) if (b + 1024 * j < dim) s += t[j] * t[j];
+  }
   s = wave_sum(s);
   const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   if ((threadIdx.x & 63) == 0) red[wave] = s;
@@ -49,10 +60,18 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
   float tot = 0.f;
   for (int i = 0; i < nw; i++) tot += red[i];
   const float scale = 1.0f / sqrtf(tot / (float)dim + eps);
-  for (int e = threadIdx.x; e < dim; e += blockDim.x) {
-    const float v = (x[e] * scale) * w[e];
+  auto emit = [&](int e, float v) {
     if (out16) out16[stage_fmt ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
     if (out32) out32[e] = v;
+  };
+  if (e0 < dim) emit(e0, (v0 * scale) * w0);
+  if (e1 < dim) emit(e1, (v1 * scale) * w1);
+  for (int b = threadIdx.x + 2048; b < dim; b += 4096) {
+    float t[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) { const int e = b + 1024 * j < dim ? b + 1024 * j : dim - 1; t[j] = x[e]; u[j] = w[e]; }
+#pragma unroll
+    for (int j = 0; j < 4; j++) if (b + 1024 * j < dim) emit(b + 1024 * j, (t[j] * scale) * u[j]);
   }
 }
 
@@ -88,14 +107,26 @@ __device__ __forceinline__ float run_sum(float v) {
   if constexpr (HD8 == 32) v += __shfl_xor(v, 16, 64);
   return v;
 }
-// sum of squares of n floats (n % 4 == 0, 16-byte aligned) over the whole workgroup of 256 threads; red: 4 floats of LDS
-__device__ __forceinline__ float block_sumsq(const float* x, int n, float* red) {
-  float s = 0.f;
-  for (int i = threadIdx.x * 4; i < n; i += 1024) { const f32x4 v = *(const f32x4*)(x + i); s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
-  s = wave_sum(s);
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+// sums of squares of two float vectors (lengths % 4 == 0, 16-byte aligned) over the whole workgroup of 256 threads; red: 8 floats
+// of LDS.  The loads of four loop iterations of both vectors go out as one batch.
+__device__ __forceinline__ void block_sumsq2(const float* q, int nq, const float* k, int nk, float* red, float& sq, float& sk) {
+  float s0 = 0.f, s1 = 0.f;
+  const int n4q = nq >> 2, n4k = nk >> 2, nmax = n4q > n4k ? n4q : n4k;
+  for (int b = threadIdx.x; b < nmax; b += 1024) {
+    f32x4 vq[4], vk[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) { const int i = b + 256 * t; vq[t] = ((const f32x4*)q)[i < n4q ? i : n4q - 1]; vk[t] = ((const f32x4*)k)[i < n4k ? i : n4k - 1]; }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int i = b + 256 * t;
+      if (i < n4q) s0 += vq[t].x * vq[t].x + vq[t].y * vq[t].y + vq[t].z * vq[t].z + vq[t].w * vq[t].w;
+      if (i < n4k) s1 += vk[t].x * vk[t].x + vk[t].y * vk[t].y + vk[t].z * vk[t].z + vk[t].w * vk[t].w;
+    }
+  }
+  s0 = wave_sum(s0); s1 = wave_sum(s1);
+  if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = s0; red[4 + (threadIdx.x >> 6)] = s1; }
   __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
+  sq = red[0] + red[1] + red[2] + red[3]; sk = red[4] + red[5] + red[6] + red[7];
 }
 
 // HD8 = head_dim / 8 (16-byte pieces per row).  The four waves split the 64 positions (16 each) and every wave serves all
@@ -135,8 +166,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
   }
   float qscale = 1.f, kscale = 1.f;
   if (a.q_norm) {
-    qscale = 1.0f / sqrtf(block_sumsq(a.q, a.n_heads * HD, red) / (float)(a.n_heads * HD) + a.norm_eps);
-    kscale = 1.0f / sqrtf(block_sumsq(a.k, a.n_kv * HD, red + 4) / (float)(a.n_kv * HD) + a.norm_eps);
+    float sq, sk;
+    block_sumsq2(a.q, a.n_heads * HD, a.k, a.n_kv * HD, red, sq, sk);
+    qscale = 1.0f / sqrtf(sq / (float)(a.n_heads * HD) + a.norm_eps);
+    kscale = 1.0f / sqrtf(sk / (float)(a.n_kv * HD) + a.norm_eps);
   }
   auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[i] : a.q[i]; };
   auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[i] : a.k[i]; };

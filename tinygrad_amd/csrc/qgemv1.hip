@@ -120,12 +120,19 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
     } else if (cnt) issue(b0, lo);
     if (!staged) {
       // activations: coalesced global -> LDS (natural order, padded unit stride) -> this lane's unit -> staged registers
+      // Loads of up to four (two) loop iterations are issued as one batch: a load per iteration would cost a memory round trip each.
       const int nq = a.K / 8;                                      // 16-byte fp16 pieces in the row
+      const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
       float nscale = 1.f;
       if (a.norm_w) {                                              // fused RMSNorm: sum of squares over the workgroup first
-        const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
         float ss = 0.f;
-        for (int i = threadIdx.x; i < 2 * nq; i += NT) { const f32x4 v = xr[i]; ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+        for (int b = threadIdx.x; b < 2 * nq; b += NT * 4) {
+          f32x4 v[4];
+#pragma unroll
+          for (int t = 0; t < 4; t++) { const int i = b + NT * t; v[t] = xr[i < 2 * nq ? i : 2 * nq - 1]; }
+#pragma unroll
+          for (int t = 0; t < 4; t++) if (b + NT * t < 2 * nq) ss += v[t].x * v[t].x + v[t].y * v[t].y + v[t].z * v[t].z + v[t].w * v[t].w;
+        }
         ss = wave_sum(ss);
         if (lane == 0) nred[wave] = ss;
         __syncthreads();
@@ -134,22 +141,33 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
         for (int j = 0; j < NT / 64; j++) tot += nred[j];
         nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
       }
-      for (int i = threadIdx.x; i < nq; i += NT) {
-        u32x4 v;
-        if (a.x_f32) {
-          const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
-          f32x4 lo4 = xr[2 * i], hi4 = xr[2 * i + 1];
-          if (a.norm_w) {
-            const f32x4 w0 = ((const f32x4*)a.norm_w)[2 * i], w1 = ((const f32x4*)a.norm_w)[2 * i + 1];
-            lo4.x = (lo4.x * nscale) * w0.x; lo4.y = (lo4.y * nscale) * w0.y; lo4.z = (lo4.z * nscale) * w0.z; lo4.w = (lo4.w * nscale) * w0.w;
-            hi4.x = (hi4.x * nscale) * w1.x; hi4.y = (hi4.y * nscale) * w1.y; hi4.z = (hi4.z * nscale) * w1.z; hi4.w = (hi4.w * nscale) * w1.w;
+      for (int b = threadIdx.x; b < nq; b += NT * 2) {
+        u32x4 v[2]; f32x4 lo4[2], hi4[2], w0[2], w1[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int i = b + NT * t < nq ? b + NT * t : nq - 1;
+          if (a.x_f32) {
+            lo4[t] = xr[2 * i]; hi4[t] = xr[2 * i + 1];
+            if (a.norm_w) { w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1]; }
+          } else v[t] = ((const u32x4*)((const uint16_t*)a.x + xrow * a.K))[i];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int i = b + NT * t;
+          if (i >= nq) break;
+          if (a.x_f32) {
+            f32x4 l = lo4[t], h = hi4[t];
+            if (a.norm_w) {
+              l.x = (l.x * nscale) * w0[t].x; l.y = (l.y * nscale) * w0[t].y; l.z = (l.z * nscale) * w0[t].z; l.w = (l.w * nscale) * w0[t].w;
+              h.x = (h.x * nscale) * w1[t].x; h.y = (h.y * nscale) * w1[t].y; h.z = (h.z * nscale) * w1[t].z; h.w = (h.w * nscale) * w1[t].w;
+            }
+            v[t].x = f2h_bits(l.x) | (f2h_bits(l.y) << 16); v[t].y = f2h_bits(l.z) | (f2h_bits(l.w) << 16);
+            v[t].z = f2h_bits(h.x) | (f2h_bits(h.y) << 16); v[t].w = f2h_bits(h.z) | (f2h_bits(h.w) << 16);
           }
-          v.x = f2h_bits(lo4.x) | (f2h_bits(lo4.y) << 16); v.y = f2h_bits(lo4.z) | (f2h_bits(lo4.w) << 16);
-          v.z = f2h_bits(hi4.x) | (f2h_bits(hi4.y) << 16); v.w = f2h_bits(hi4.z) | (f2h_bits(hi4.w) << 16);
-        } else v = ((const u32x4*)((const uint16_t*)a.x + xrow * a.K))[i];
-        // element 8i lives in unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
-        if constexpr (T == GGML_F16) *(u32x4*)(xlds + F::unit_of_nu(8 * i, a.nu) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v;
-        else *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
+          // element 8i lives in unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
+          if constexpr (T == GGML_F16) *(u32x4*)(xlds + F::unit_of_nu(8 * i, a.nu) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v[t];
+          else *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v[t];
+        }
       }
       __syncthreads();
       {
