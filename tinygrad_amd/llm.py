@@ -147,10 +147,7 @@ class TransformerBlock:
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     st = self.staged                                                     # producers write the consumer's staged order directly
-    if st:
-      rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.attn_q.ggml_type, stream))
-      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream, x_staged=True)
-    elif self.fuse_norm:                                                 # the q/k/v launch normalises the row while staging it
+    if self.fuse_norm:                                                   # the q/k/v launch normalises the row while staging it
       qlinear_multi([self.attn_q, self.attn_k, self.attn_v], x, [s.q, s.k, s.v], stream=stream, norm=(self.attn_norm, c.norm_eps))
     else:
       rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
@@ -163,8 +160,8 @@ class TransformerBlock:
     qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     if not self.moe:
-      if not st and self.fuse_norm:
-        qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps))
+      if self.fuse_norm:
+        qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps), stage_out_for=self.ffn_down if st else None)
       else:
         rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if st else 0, stream))
         qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=st, stage_out_for=self.ffn_down if st else None)
