@@ -20,6 +20,8 @@ extern "C" {
 #define TGA_F16 1
 #define TGA_Q4_0 2
 #define TGA_Q8_0 8
+#define TGA_Q4_K 12
+#define TGA_Q5_K 13
 #define TGA_Q6_K 14
 #define TGA_MXFP4 39
 /* activation dtype code: fp16 values in the staged order of the consuming weight (see tga_stage_activation) */
@@ -63,7 +65,7 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
  * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  K must be a multiple of the type's block size.
- * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K (GGUF aligns tensor data to 32 bytes, gguf.py:144-148). */
+ * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K (GGUF aligns tensor data to 32 bytes, gguf.py:144-148). */
 int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                 int M, int64_t N, int64_t K, void* stream);
 
@@ -89,7 +91,7 @@ int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml
  * weight's (ggml_type, K).  tga_stage_activation writes that permutation as fp16 (K values); a linear then takes it with
  * x_dtype = TGA_F16_STAGED and skips its own staging.  Producers can emit the order directly: tga_rmsnorm / tga_attention_decode
  * (stage_type, stage_K) and tga_qlinear_multi (y_stage_type != 0: the single fp16 output, of length y_stage_K, is written in the
- * staged order of a consumer weight of that type whose K = y_stage_K).  Requires K % 64 == 0 (Q6_K: % 256). */
+ * staged order of a consumer weight of that type whose K = y_stage_K).  Requires K % 64 == 0 (Q4_K / Q5_K / Q6_K: % 256). */
 int tga_stage_activation(int ggml_type, const void* x, int x_dtype, int64_t K, void* out_f16, void* stream);
 
 /* ExpertWeights.__call__ (tinygrad/llm/model.py:21-27) over a stacked (n_experts, N, K) weight kept in GGUF blocks: for job j

@@ -1,8 +1,8 @@
 /* Scalar C restatement of the reference's quantized-weight linear path.  TEST INFRASTRUCTURE ONLY: the checker and the
  * timed CPU baseline; never linked into the shipped library.
  *
- * Dequant loops restate the published ggml reference routines (ggml-quants.c dequantize_row_q4_0 / q8_0 / q6_K /
- * mxfp4; gguf-py >= 0.18 is what the reference's tests call, pyproject.toml:79) element by element, independently of
+ * Dequant loops restate the published ggml reference routines (ggml-quants.c dequantize_row_q4_0 / q8_0 / q4_K / q5_K /
+ * q6_K / mxfp4; gguf-py >= 0.18 is what the reference's tests call, pyproject.toml:79) element by element, independently of
  * the vectorised numpy restatement of tinygrad/llm/gguf.py:46,56,68-72,105-114 in oracle/ggml.py: the two must agree
  * bit for bit (tests/test_oracle_ggml.py).
  * The linear restates Tensor.dot (tinygrad/mixin/op.py:367-392) with sum_acc_dtype = float32 (tinygrad/dtype.py:212-216).
@@ -72,6 +72,37 @@ static void deq_q6_k(const uint8_t* b, float* y) {            /* block_q6_K: ggm
     y += 128; ql += 64; qh += 32; sc += 8;
   }
 }
+/* get_scale_min_k4 of ggml-quants.c: 6-bit scale and min of sub-block j from the 12 packed bytes */
+static void scale_min_k4(int j, const uint8_t* q, uint8_t* d, uint8_t* m) {
+  if (j < 4) { *d = q[j] & 63; *m = q[j + 4] & 63; }
+  else { *d = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4)); *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4)); }
+}
+static void deq_q4_k(const uint8_t* b, float* y) {            /* block_q4_K: d, dmin, scales[12], qs[128]  (dequantize_row_q4_K) */
+  uint16_t dh, mh; memcpy(&dh, b, 2); memcpy(&mh, b + 2, 2);
+  const float d = h2f(dh), min = h2f(mh);
+  const uint8_t* q = b + 16; int is = 0;
+  for (int j = 0; j < 256; j += 64) {
+    uint8_t sc, m;
+    scale_min_k4(is + 0, b + 4, &sc, &m); const float d1 = d * sc, m1 = min * m;
+    scale_min_k4(is + 1, b + 4, &sc, &m); const float d2 = d * sc, m2 = min * m;
+    for (int l = 0; l < 32; l++) *y++ = d1 * (q[l] & 0xF) - m1;
+    for (int l = 0; l < 32; l++) *y++ = d2 * (q[l] >> 4) - m2;
+    q += 32; is += 2;
+  }
+}
+static void deq_q5_k(const uint8_t* b, float* y) {            /* block_q5_K: d, dmin, scales[12], qh[32], qs[128]  (dequantize_row_q5_K) */
+  uint16_t dh, mh; memcpy(&dh, b, 2); memcpy(&mh, b + 2, 2);
+  const float d = h2f(dh), min = h2f(mh);
+  const uint8_t *qh = b + 16, *ql = b + 48; int is = 0; uint8_t u1 = 1, u2 = 2;
+  for (int j = 0; j < 256; j += 64) {
+    uint8_t sc, m;
+    scale_min_k4(is + 0, b + 4, &sc, &m); const float d1 = d * sc, m1 = min * m;
+    scale_min_k4(is + 1, b + 4, &sc, &m); const float d2 = d * sc, m2 = min * m;
+    for (int l = 0; l < 32; l++) *y++ = d1 * ((ql[l] & 0xF) + (qh[l] & u1 ? 16 : 0)) - m1;
+    for (int l = 0; l < 32; l++) *y++ = d2 * ((ql[l] >> 4) + (qh[l] & u2 ? 16 : 0)) - m2;
+    ql += 32; is += 2; u1 <<= 2; u2 <<= 2;
+  }
+}
 /* ggml's kvalues_mxfp4 is an int8 table (code 8 -> +0); the reference's float LUT (tinygrad/llm/gguf.py:108-110) holds -0.0
  * for code 8, and bit-exactness is owed to the reference, so the table here is the reference's. */
 static const float kvalues_mxfp4[16] = {0.0f, 1.0f, 2.0f, 3.0f, 4.0f, 6.0f, 8.0f, 12.0f, -0.0f, -1.0f, -2.0f, -3.0f, -4.0f, -6.0f, -8.0f, -12.0f};
@@ -87,11 +118,13 @@ static void deq_mxfp4(const uint8_t* b, float* y) {           /* block_mxfp4: gg
 
 static int type_geom(int t, int* nel, int* nby) {
   switch (t) { case 2: *nel = 32; *nby = 18; return 0; case 8: *nel = 32; *nby = 34; return 0;
+               case 12: *nel = 256; *nby = 144; return 0; case 13: *nel = 256; *nby = 176; return 0;
                case 14: *nel = 256; *nby = 210; return 0; case 39: *nel = 32; *nby = 17; return 0; }
   return -1;
 }
 static void deq_block(int t, const uint8_t* b, float* y) {
-  switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break; }
+  switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break;
+               case 12: deq_q4_k(b, y); break; case 13: deq_q5_k(b, y); break; }
 }
 
 /* ggml_data_to_tensor (tinygrad/llm/gguf.py:23): n_blocks blocks -> float32 */

@@ -1,10 +1,11 @@
-"""numpy restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for the four block layouts on the path,
+"""numpy restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for the block layouts on the path (Q4_0, Q8_0, Q6_K,
+MXFP4 and the Q4_K / Q5_K superblocks most GGUF model files are made of),
 plus the ggml reference quantizers used only to build synthetic models.  Test infrastructure only."""
 import numpy as np
 
-Q4_0, Q8_0, Q6_K, MXFP4, F32, F16 = 2, 8, 14, 39, 0, 1
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, F32, F16 = 2, 8, 12, 13, 14, 39, 0, 1
 # {ggml_type: (elements per block, bytes per block)}  tinygrad/llm/gguf.py:20-21
-GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q6_K: (256, 210), MXFP4: (32, 17)}
+GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17)}
 # tinygrad/llm/gguf.py:108-110 (== 2 * E2M1 values; ggml_common.py:218 kvalues_mxfp4)
 FP4_LUT = np.array([0.0, 1.0, 2.0, 3.0, 4.0, 6.0, 8.0, 12.0, -0.0, -1.0, -2.0, -3.0, -4.0, -6.0, -8.0, -12.0], dtype=np.float32)
 
@@ -40,6 +41,23 @@ def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
   q = ((xl | xh).view(np.int8) - np.int8(32)).reshape(nb, 256).astype(np.float32)
   return (d * q) * scales
 
+def _dequant_q45_k(blocks: np.ndarray, five: bool) -> np.ndarray:
+  """gguf.py:57-67  Q4_K (144 B: d, dmin, scales[12], qs[128]) / Q5_K (176 B: d, dmin, scales[12], qh[32], qs[128]):
+  (d * sc) * q - dmin * mn per 32-element sub-block, 6-bit sc / mn unpacked from the 12 scale bytes."""
+  nb = blocks.shape[0]
+  d, dmin = _f16(blocks[:, 0:2])[:, :, None], _f16(blocks[:, 2:4])[:, :, None]
+  s = blocks[:, 4:16]
+  sc = np.concatenate([s[:, 0:4] & 63, (s[:, 8:12] & 0xF) | ((s[:, 0:4] >> 6) << 4)], axis=-1).astype(np.float32)[:, :, None]
+  mn = np.concatenate([s[:, 4:8] & 63, (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)], axis=-1).astype(np.float32)[:, :, None]
+  off = 48 if five else 16
+  qs = blocks[:, off:off + 128].reshape(nb, 4, 32)
+  q = np.stack([qs & 0xF, qs >> 4], axis=2).reshape(nb, 8, 32)          # sub-blocks 2p (low nibbles), 2p+1 (high nibbles)
+  if five: q = q + q_to_uint8(blocks[:, 16:48], 1).reshape(nb, 8, 32) * np.uint8(16)
+  return ((d * sc) * q.astype(np.float32) - dmin * mn).reshape(nb, 256)
+
+def dequant_q4_k(blocks: np.ndarray) -> np.ndarray: return _dequant_q45_k(blocks, False)
+def dequant_q5_k(blocks: np.ndarray) -> np.ndarray: return _dequant_q45_k(blocks, True)
+
 def dequant_mxfp4(blocks: np.ndarray) -> np.ndarray:
   """gguf.py:105-114  d = bitcast_f32((e-1)<<23) (e>=2), 2^-127 (e==1), 2^-128 (e==0); value = LUT[code] * d"""
   e = blocks[:, 0].astype(np.uint32)
@@ -47,7 +65,7 @@ def dequant_mxfp4(blocks: np.ndarray) -> np.ndarray:
   d = np.where(e < 2, small, (e - 1) * np.uint32(0x00800000)).astype(np.uint32).view(np.float32)[:, None]
   return FP4_LUT[q_to_uint8(blocks[:, 1:17], 4)] * d
 
-_DEQ = {Q4_0: dequant_q4_0, Q8_0: dequant_q8_0, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
+_DEQ = {Q4_0: dequant_q4_0, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
 
 def ggml_data_to_tensor(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
   """gguf.py:23-119 restricted to the types on the path; returns flat float32 of n elements."""

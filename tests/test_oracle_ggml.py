@@ -72,7 +72,7 @@ def test_q6_k_brute_force_layout():
     out = og.ggml_data_to_tensor(b, 256, 14)
     np.testing.assert_array_equal(out, exp, err_msg=f"element {e}")
 
-@pytest.mark.parametrize("t", [2, 8, 14, 39])
+@pytest.mark.parametrize("t", [2, 8, 12, 13, 14, 39])
 def test_numpy_restatement_equals_scalar_c_loops(t):
   """Vectorised restatement of tinygrad/llm/gguf.py (field-major q_to_uint8) == independent scalar loops of the published ggml
   routines, bit for bit, on fully random bytes (NaN/Inf/subnormal scales included)."""
@@ -84,6 +84,32 @@ def test_numpy_restatement_equals_scalar_c_loops(t):
   c = cref.dequant(t, data)
   same = (a.view(np.uint32) == c.view(np.uint32)) | (np.isnan(a) & np.isnan(c))
   assert same.all()
+
+@pytest.mark.parametrize("t", [12, 13])
+def test_q4_k_q5_k_brute_force_layout(t):
+  """One weight at a time against ggml's dequantize_row_q4_K / q5_K index map: element e of a superblock sits in sub-block e // 32
+  (6-bit scale / min from get_scale_min_k4), nibble (e // 32) & 1 of qs[32 * (e // 64) + e % 32], fifth bit = bit e // 32 of qh[e % 32]."""
+  nby = og.GGML_QUANT[t][1]; qs_off = 48 if t == 13 else 16
+  def put_scale(b, sb, sc, mn):                                 # inverse of get_scale_min_k4
+    s = b[4:16]
+    if sb < 4: s[sb] = (int(s[sb]) & 0xC0) | sc; s[sb + 4] = (int(s[sb + 4]) & 0xC0) | mn
+    else:
+      s[sb + 4] = (sc & 0xF) | ((mn & 0xF) << 4)
+      s[sb - 4] = (int(s[sb - 4]) & 0x3F) | ((sc >> 4) << 6); s[sb] = (int(s[sb]) & 0x3F) | ((mn >> 4) << 6)
+  for e in [0, 1, 31, 32, 33, 63, 64, 100, 127, 128, 160, 191, 192, 223, 224, 255]:
+    b = np.zeros(nby, dtype=np.uint8)
+    b[0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8); b[2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+    sb = e // 32
+    put_scale(b, sb, 37, 51)                                    # both above 15: exercises the split high bits
+    q = 29 if t == 13 else 13
+    byte = qs_off + 32 * (e // 64) + e % 32
+    b[byte] = (q & 0xF) << (4 if sb & 1 else 0)
+    if t == 13 and q >> 4: b[16 + e % 32] = 1 << sb
+    exp = np.zeros(256, dtype=np.float32)
+    exp[32 * sb:32 * sb + 32] = -0.25 * 51                      # the sub-block's min applies to all its 32 weights
+    exp[e] = (0.5 * 37) * q - 0.25 * 51
+    np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, t), exp, err_msg=f"element {e}")
+    np.testing.assert_array_equal(cref.dequant(t, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
 
 def test_q6_k_association_order_is_exact():
   """(d*q)*sc == d*(sc*q) == (d*sc)*q in float32: 11 + 6 + 8 significant bits fit in 24."""

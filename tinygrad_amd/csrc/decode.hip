@@ -383,9 +383,10 @@ static int decode_staged_fmt(int ggml_type, long long K, int* nu) {
   int fmt = -1, uw = 64;
   switch (ggml_type) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
+    case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
-  if (fmt < 0 || K <= 0 || K % (ggml_type == GGML_Q6_K ? 256 : 64) != 0) return -1;
+  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K) ? 256 : 64) != 0) return -1;
   *nu = (int)(K / uw);
   return fmt;
 }

@@ -1,5 +1,5 @@
 // Block dequant kernels: bit-exact restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for Q4_0 (:46), Q8_0 (:56),
-// Q6_K (:68-72) and MXFP4 (:105-114).  One thread produces 4 consecutive output elements (one 16-byte or 8-byte store), so
+// Q4_K / Q5_K (:57-67), Q6_K (:68-72) and MXFP4 (:105-114).  One thread produces 4 consecutive output elements (one 16-byte or 8-byte store), so
 // stores are fully coalesced; the packed bytes are re-read through L1/L2 (this kernel is a load-time / test utility, the
 // decode path never materialises weights).
 // Float contraction is off for this file: every product below must round exactly like the reference's separate multiplies.
@@ -44,6 +44,30 @@ template <> struct Deq<GGML_Q6_K> {
     }
   }
 };
+// Q4_K (144 B: d, dmin, scales[12], qs[128]) and Q5_K (176 B: ... qh[32], qs[128]), tinygrad/llm/gguf.py:57-67: sub-block sb = e / 32
+// has a 6-bit scale and min packed in the 12 scale bytes; value = (d * sc) * q - dmin * mn with q = nibble (sb & 1) of
+// qs[32 * (sb / 2) + e % 32] (+ 16 * bit sb of qh[e % 32] for Q5_K).
+template <bool FIVE> struct DeqK45 {
+  static constexpr int NEL = 256, NBY = FIVE ? 176 : 144;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+    const float d = h2f_bits(ld2(b)), dmin = h2f_bits(ld2(b + 2));
+    const int sb = e0 >> 5, l = e0 & 31;
+    const uint8_t* s = b + 4;
+    int sc, mn;
+    if (sb < 4) { sc = s[sb] & 63; mn = s[sb + 4] & 63; }
+    else { sc = (s[sb + 4] & 0xF) | ((s[sb - 4] >> 6) << 4); mn = (s[sb + 4] >> 4) | ((s[sb] >> 6) << 4); }
+    const float d1 = d * (float)sc, m1 = dmin * (float)mn;
+    const uint8_t* q = b + (FIVE ? 48 : 16) + 32 * (sb >> 1) + l;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int v = (sb & 1) ? (q[i] >> 4) : (q[i] & 0xF);
+      if (FIVE) v += ((b[16 + l + i] >> sb) & 1) << 4;
+      o[i] = d1 * (float)v - m1;
+    }
+  }
+};
+template <> struct Deq<GGML_Q4_K> : DeqK45<false> {};
+template <> struct Deq<GGML_Q5_K> : DeqK45<true> {};
 template <> struct Deq<GGML_MXFP4> {
   static constexpr int NEL = 32, NBY = 17;
   static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
@@ -97,6 +121,8 @@ extern "C" int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* o
   switch (ggml_type) {
     case GGML_Q4_0: return launch_dequant<GGML_Q4_0>(blocks, n, out, out_dtype, s);
     case GGML_Q8_0: return launch_dequant<GGML_Q8_0>(blocks, n, out, out_dtype, s);
+    case GGML_Q4_K: return launch_dequant<GGML_Q4_K>(blocks, n, out, out_dtype, s);
+    case GGML_Q5_K: return launch_dequant<GGML_Q5_K>(blocks, n, out, out_dtype, s);
     case GGML_Q6_K: return launch_dequant<GGML_Q6_K>(blocks, n, out, out_dtype, s);
     case GGML_MXFP4: return launch_dequant<GGML_MXFP4>(blocks, n, out, out_dtype, s);
   }

@@ -77,7 +77,7 @@ template <> struct Fmt<GGML_Q4_0> {
     for (int k = 0; k < 8; k++) { lo = dot2(nx[k], 0x64086408u, lo); hi = dot2(nx[k + 8], 0x54805480u, hi); }   // 1032, 72
     c[0] = -(lo + hi);
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) { return h2f_bits(r.d) * a[0]; }
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
 };
 
 // ------------------------------------------------------------------------------------------------ Q8_0 (gguf.py:56)
@@ -110,7 +110,7 @@ template <> struct Fmt<GGML_Q8_0> {
     for (int k = 0; k < 16; k++) s = dot2(nx[k], 0x64806480u, s);   // 1152
     c[0] = -s;
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) { return h2f_bits(r.d) * a[0]; }
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
 };
 
 
@@ -180,7 +180,7 @@ template <> struct Fmt<F_Q4_0P> {
       c[j] = -(lo + hi);
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
   }
   // halfword index of row element e inside the staged activation buffer ([XV][nu] vectors of 4 fp16 pairs)
@@ -245,7 +245,7 @@ template <> struct Fmt<F_Q8_0P> {
       c[j] = -t;
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
   }
   static __device__ __forceinline__ int spos(int e, int nu) {
@@ -303,7 +303,7 @@ template <> struct Fmt<GGML_F16> {
     for (int v = 0; v < 8; v++) { xv[v].x = nx[4 * v]; xv[v].y = nx[4 * v + 1]; xv[v].z = nx[4 * v + 2]; xv[v].w = nx[4 * v + 3]; }
     c[0] = 0.f;
   }
-  static __device__ __forceinline__ float finish(const Raw&, const float* a) { return a[0]; }
+  static __device__ __forceinline__ float finish(const Raw&, const float* a, const float*) { return a[0]; }
   static __device__ __forceinline__ int spos(int e, int nu) { return e; }
   static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
@@ -348,7 +348,7 @@ template <> struct Fmt<GGML_MXFP4> {
     c[0] = 0.f;
   }
   // reference value = (2 * e2m1) * 2^(e-128) = e2m1 * 2^(e-127); e = 0 is the fp32 subnormal 2^-127
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
     return __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u) * a[0];
   }
   static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 5, b = e & 31, q = b & 15; return (((q >> 2) * nu + u) * 4 + (q & 3)) * 2 + (b >> 4); }
@@ -409,7 +409,7 @@ template <> struct Fmt<GGML_Q6_K> {
       c[j] = -s;
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a) {
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
     const int g8 = (r.d & 1) * 8;   // scales 8h + 2j + g live in bytes g, g+2 of sc0 (j = 0, 1) and sc1 (j = 2, 3)
     const float s0 = (float)(int)(int8_t)(r.sc0 >> g8), s1 = (float)(int)(int8_t)(r.sc0 >> (16 + g8));
     const float s2 = (float)(int)(int8_t)(r.sc1 >> g8), s3 = (float)(int)(int8_t)(r.sc1 >> (16 + g8));
@@ -433,6 +433,92 @@ template <> struct Fmt<GGML_Q6_K> {
 
 __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + __expf(-v)); }
 
+// ------------------------------------------------------------------------------------------------ Q4_K / Q5_K (gguf.py:57-67)
+// Superblock of 256 weights: fp16 d, dmin, 12 bytes of packed 6-bit (scale, min) for 8 sub-blocks of 32, [Q5_K: qh[32]], qs[128].
+// qs[32p + i] holds weight i of sub-block 2p (low nibble) and of sub-block 2p + 1 (high nibble); Q5_K adds 16 * bit sb of qh[i].
+// A unit is one such pair of sub-blocks (64 consecutive weights, 32 bytes of qs); accumulator group 0 is the low-nibble sub-block
+// (decoded as 1024 + q), group 1 the high-nibble one (64 + q, nibble left in place).  w = (d sc) q - dmin mn, so the unit's
+// contribution is d (sc0 S0 + sc1 S1) - dmin (mn0 X0 + mn1 X1) with S = sum q x and X = sum x; X comes out of the bias
+// corrections the lane already holds (c0 = -1024 X0, c1 = -64 X1).  Blocks are multiples of 16 bytes: all loads are aligned.
+template <bool FIVE> struct RawK45;
+template <> struct RawK45<false> { u32x4 q0, q1, hdr; uint32_t p; };
+template <> struct RawK45<true> { u32x4 q0, q1, hdr, h0, h1; uint32_t p; };
+template <bool FIVE> struct FmtK45 {
+  static constexpr int UW = 64, UPB = 4, BW = 256, BB = FIVE ? 176 : 144, QS = FIVE ? 48 : 16;
+  static __device__ __forceinline__ int unit_of(int e) { return e >> 6; }
+  static __device__ __forceinline__ int pair_of(int e) { return (e & 63) >> 1; }
+  static constexpr int XV = 8, NG = 2, NWV = 32;
+  typedef RawK45<FIVE> Raw;
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* b = row + (size_t)BB * (u >> 2); const int p = u & 3;
+    Raw r; r.hdr = ld16_a4(b); r.q0 = ld16_a4(b + QS + 32 * p); r.q1 = ld16_a4(b + QS + 32 * p + 16);
+    if constexpr (FIVE) { r.h0 = ld16_a4(b + 16); r.h1 = ld16_a4(b + 32); }
+    r.p = (uint32_t)p;
+    return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 2;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
+  // wv[16g + 2t + o] = weights (4t + o, 4t + o + 2) of group g (t = dword of the 32 qs bytes, o = odd byte)
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const uint32_t w = t < 4 ? r.q0[t & 3] : r.q1[t & 3], w8 = w >> 8;
+      uint32_t le = and_or(w, 0x000F000Fu, kc[0]), lo = and_or(w8, 0x000F000Fu, kc[0]);
+      uint32_t he = and_or(w, 0x00F000F0u, kc[1]), ho = and_or(w8, 0x00F000F0u, kc[1]);
+      if constexpr (FIVE) {
+        const uint32_t H = (t < 4 ? r.h0[t & 3] : r.h1[t & 3]) >> (2 * r.p);   // bit 0 / 1 of every byte: fifth bit of sub-block 2p / 2p + 1
+        le = and_or(H << 4, 0x00100010u, le); lo = and_or(H >> 4, 0x00100010u, lo);
+        he = and_or(H << 7, 0x01000100u, he); ho = and_or(H >> 1, 0x01000100u, ho);
+      }
+      wv[2 * t] = le; wv[2 * t + 1] = lo; wv[16 + 2 * t] = he; wv[16 + 2 * t + 1] = ho;
+    }
+  }
+  // nx[k] = natural pair k of the unit's 64 activations; xv[4g + v] = {E, O, E', O'} of dwords 2v, 2v + 1 of group g
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      const uint32_t* n = nx + 16 * g;
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        xv[4 * g + v].x = pack_even(n[4 * v], n[4 * v + 1]); xv[4 * g + v].y = pack_odd(n[4 * v], n[4 * v + 1]);
+        xv[4 * g + v].z = pack_even(n[4 * v + 2], n[4 * v + 3]); xv[4 * g + v].w = pack_odd(n[4 * v + 2], n[4 * v + 3]);
+      }
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; k++) s = dot2(n[k], g ? 0x54005400u : 0x64006400u, s);
+      c[g] = -s;
+    }
+  }
+  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float* c) {
+    // get_scale_min_k4 for sub-blocks 2p, 2p + 1: byte index i = 2 (p & 1) (+1) of scales[0..3] / [4..7] / [8..11]
+    const uint32_t sh = 16 * (r.p & 1);
+    const uint32_t y0 = (r.hdr.y >> sh) & 0xFF, y1 = (r.hdr.y >> (sh + 8)) & 0xFF, z0 = (r.hdr.z >> sh) & 0xFF, z1 = (r.hdr.z >> (sh + 8)) & 0xFF;
+    const uint32_t w0 = (r.hdr.w >> sh) & 0xFF, w1 = (r.hdr.w >> (sh + 8)) & 0xFF;
+    const bool hi = r.p >= 2;
+    const float sc0 = (float)(hi ? ((w0 & 0xF) | ((y0 >> 6) << 4)) : (y0 & 63)), sc1 = (float)(hi ? ((w1 & 0xF) | ((y1 >> 6) << 4)) : (y1 & 63));
+    const float mn0 = (float)(hi ? ((w0 >> 4) | ((z0 >> 6) << 4)) : (z0 & 63)), mn1 = (float)(hi ? ((w1 >> 4) | ((z1 >> 6) << 4)) : (z1 & 63));
+    const float d = h2f_bits(r.hdr.x & 0xFFFF), dmin = h2f_bits(r.hdr.x >> 16);
+    return d * (sc0 * a[0] + sc1 * a[1]) + dmin * (mn0 * (c[0] * (1.0f / 1024.0f)) + mn1 * (c[1] * (1.0f / 64.0f)));
+  }
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = e >> 6, g = (e >> 5) & 1, r = e & 31, wi = 2 * (r >> 2) + (r & 1);
+    return (((4 * g + (wi >> 2)) * nu + u) * 4 + (wi & 3)) * 2 + ((r >> 1) & 1);
+  }
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      const uint32_t k = g ? 0x54005400u : 0x64006400u;
+      float t = 0.f;
+#pragma unroll
+      for (int i = 4 * g; i < 4 * g + 4; i++) { t = dot2(xv[i].x, k, t); t = dot2(xv[i].y, k, t); t = dot2(xv[i].z, k, t); t = dot2(xv[i].w, k, t); }
+      c[g] = -t;
+    }
+  }
+};
+template <> struct Fmt<GGML_Q4_K> : FmtK45<false> {};
+template <> struct Fmt<GGML_Q5_K> : FmtK45<true> {};
+
 // unit_dot with the unit's activations already in registers (M = 1)
 template <int T>
 __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, const u32x4* xv, const float* cv, float& acc, const uint32_t* kc) {
@@ -452,7 +538,7 @@ __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, co
     }
     g[j] = t;
   }
-  acc += F::finish(raw, g);
+  acc += F::finish(raw, g, cv);
 }
 
 // M = 1 stores.  EPI 0: plain, EPI 1: + residual, EPI 2: silu(gate) * up into output row `row` of segment 0.
@@ -474,6 +560,8 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
     case F_Q4_0P: return Fmt<F_Q4_0P>::spos(e, nu);
     case F_Q8_0P: return Fmt<F_Q8_0P>::spos(e, nu);
     case GGML_Q6_K: return Fmt<GGML_Q6_K>::spos(e, nu);
+    case GGML_Q4_K: return Fmt<GGML_Q4_K>::spos(e, nu);
+    case GGML_Q5_K: return Fmt<GGML_Q5_K>::spos(e, nu);
     case GGML_MXFP4: return Fmt<GGML_MXFP4>::spos(e, nu);
     case GGML_F16: return Fmt<GGML_F16>::spos(e, nu);
   }

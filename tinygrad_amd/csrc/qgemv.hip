@@ -63,10 +63,11 @@ __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const 
   constexpr int VPG = F::XV / F::NG;   // x vectors per accumulator group
 #pragma unroll
   for (int m = 0; m < M; m++) {
-    float g[F::NG];
+    float g[F::NG], cc[F::NG];
 #pragma unroll
     for (int j = 0; j < F::NG; j++) {
       float s = cs[(m * F::NG + j) * cu + ul];
+      cc[j] = s;
 #pragma unroll
       for (int v = 0; v < VPG; v++) {
         const u32x4 xv = xs[(m * F::XV + j * VPG + v) * cu + ul];
@@ -75,7 +76,7 @@ __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const 
       }
       g[j] = s;
     }
-    acc[m] += F::finish(raw, g);
+    acc[m] += F::finish(raw, g, cc);
   }
 }
 
@@ -91,10 +92,11 @@ __device__ __forceinline__ void unit_dot_rows(const typename Fmt<T>::Raw* raw, c
   constexpr int VPG = F::XV / F::NG;   // x vectors per accumulator group
 #pragma unroll
   for (int m = 0; m < M; m++) {
-    float g[R][F::NG];
+    float g[R][F::NG], cc[F::NG];
 #pragma unroll
     for (int j = 0; j < F::NG; j++) {
       const float c0 = cs[(m * F::NG + j) * cu + ul];
+      cc[j] = c0;
       float s[R];
 #pragma unroll
       for (int r = 0; r < R; r++) s[r] = c0;
@@ -111,7 +113,7 @@ __device__ __forceinline__ void unit_dot_rows(const typename Fmt<T>::Raw* raw, c
       for (int r = 0; r < R; r++) g[r][j] = s[r];
     }
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r][m] += F::finish(raw[r], g[r]);
+    for (int r = 0; r < R; r++) acc[r][m] += F::finish(raw[r], g[r], cc);
     // one activation row's vectors live at a time: without this the scheduler hoists the LDS reads of all M rows (M x 32 VGPRs)
     if constexpr (M * R > 4) __builtin_amdgcn_sched_barrier(0);
   }
@@ -300,7 +302,7 @@ static int launch_qgemv(QArgs a, hipStream_t s) {
     if (grid > need) grid = need;
   } else {
     int cu = QG_LDS_BUDGET / 2 / per_unit;                 // two workgroups per CU
-    cu -= cu % (64 * F::UPB); if (cu < 64 * F::UPB) cu = 64 * F::UPB;
+    cu -= cu % 64; if (cu < 64) cu = 64;                   // whole waves of units (64 is a multiple of every format's units per block)
     TGA_REQUIRE((long long)cu * per_unit <= QG_LDS_BUDGET, "tga_qlinear: activations of one K chunk do not fit LDS");
     a.chunk_u = cu; a.nchunks = (a.nu + cu - 1) / cu;
     lds = (size_t)per_unit * cu;
@@ -350,9 +352,10 @@ static int staged_fmt(int ggml_type, long long K, int* nu) {
   int fmt = -1, uw = 64;
   switch (ggml_type) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
+    case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
-  if (fmt < 0 || K <= 0 || K % (ggml_type == GGML_Q6_K ? 256 : 64) != 0) return -1;
+  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K) ? 256 : 64) != 0) return -1;
   *nu = (int)(K / uw);
   return fmt;
 }
@@ -387,7 +390,7 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
   TGA_REQUIRE(epilogue != 1 || (y_dtype == TGA_F32 && resid), "tga_qlinear: the residual epilogue needs float32 y and resid pointers");
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: bw = 256; break; case GGML_F16: bw = 64; break;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: bw = 256; break; case GGML_F16: bw = 64; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   TGA_REQUIRE(ggml_type != GGML_F16 || M == 1, "tga_qlinear: dense fp16 weights are served for M = 1 only");
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
@@ -398,6 +401,7 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
   for (int i = 0; i < nseg; i++) {
     TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)), "tga_qlinear: segment %d has a null pointer or no rows", i);
     TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((uintptr_t)w[i] & 1) == 0, "tga_qlinear: weight pointer of segment %d must be 2-byte aligned", i);
+    TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K) || ((uintptr_t)w[i] & 3) == 0, "tga_qlinear: Q4_K / Q5_K weights of segment %d must be 4-byte aligned", i);
     a.w[i] = (const uint8_t*)w[i]; a.y[i] = y[i]; a.n[i] = n[i]; a.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr;
     TGA_REQUIRE(epilogue != 1 || a.resid[i], "tga_qlinear: null resid for segment %d", i);
     ntot += n[i];
@@ -427,6 +431,8 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
     case GGML_Q4_0: return pair ? launch_qgemv_m<F_Q4_0P>(a, M, s) : launch_qgemv_m<GGML_Q4_0>(a, M, s);
     case GGML_Q8_0: return pair ? launch_qgemv_m<F_Q8_0P>(a, M, s) : launch_qgemv_m<GGML_Q8_0>(a, M, s);
     case GGML_Q6_K: return launch_qgemv_m<GGML_Q6_K>(a, M, s);
+    case GGML_Q4_K: return launch_qgemv_m<GGML_Q4_K>(a, M, s);
+    case GGML_Q5_K: return launch_qgemv_m<GGML_Q5_K>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
   }
   return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
@@ -465,9 +471,11 @@ extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_u
   TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear_experts: y_dtype must be TGA_F16 or TGA_F32");
   int bw, bb;
   switch (ggml_type) { case GGML_Q4_0: bw = 32; bb = 18; break; case GGML_Q8_0: bw = 32; bb = 34; break; case GGML_MXFP4: bw = 32; bb = 17; break;
-    case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_F16: bw = 64; bb = 128; break;
+    case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_Q4_K: bw = 256; bb = 144; break; case GGML_Q5_K: bw = 256; bb = 176; break;
+    case GGML_F16: bw = 64; bb = 128; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   TGA_REQUIRE(K > 0 && K % bw == 0 && N > 0, "tga_qlinear_experts: K=%lld must be a positive multiple of %d", (long long)K, bw);
+  TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K) || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0), "tga_qlinear_experts: Q4_K / Q5_K weights must be 4-byte aligned");
   QArgs a = {};
   a.nseg = w_up ? 2 : 1; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = w_up ? 2 : 0; a.K = (int)K;
   a.w[0] = (const uint8_t*)w; a.w[1] = (const uint8_t*)w_up; a.y[0] = y; a.n[0] = N; a.n[1] = N; a.ntot = N;

@@ -262,6 +262,8 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
     case F_Q4_0P: return launch_fast_w<F_Q4_0P>(a, s);
     case F_Q8_0P: return launch_fast_w<F_Q8_0P>(a, s);
     case GGML_Q6_K: return launch_fast_w<GGML_Q6_K>(a, s);
+    case GGML_Q4_K: return launch_fast_w<GGML_Q4_K>(a, s);
+    case GGML_Q5_K: return launch_fast_w<GGML_Q5_K>(a, s);
     case GGML_MXFP4: return launch_fast_w<GGML_MXFP4>(a, s);
     case GGML_F16: return launch_fast_w<GGML_F16>(a, s);
   }

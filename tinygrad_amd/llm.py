@@ -140,7 +140,7 @@ class TransformerBlock:
                                          for l in (self.attn_q, self.attn_output, self.ffn_gate, self.ffn_down)) \
                   and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
     # RMSNorm folded into the consuming M = 1 linear (needs its register-resident fast path: K % 64, 4-byte aligned weights)
-    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type != rt.Q6_K or l.in_features % 256 == 0)
+    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K) or l.in_features % 256 == 0)
     self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
 
   def __call__(self, x: Buffer, stream):
@@ -216,7 +216,7 @@ class Transformer:
     self.output_norm = state_dict["output_norm.weight"][0]
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
-    self.fuse_head_norm = c.dim % (256 if out[1] == rt.Q6_K else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
+    self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
     self.stream = rt.Stream()
     self._graphs = {}
     # one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type

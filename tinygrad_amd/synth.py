@@ -2,7 +2,7 @@
 Pure numpy; generators draw from numpy.random.default_rng(seed) so tests, bench and the CPU baseline see identical bytes."""
 from __future__ import annotations
 import numpy as np
-from tinygrad_amd.runtime import GGML_QUANT, Q4_0, Q8_0, Q6_K, MXFP4
+from tinygrad_amd.runtime import GGML_QUANT, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4
 
 SEEDS = {1: 1001, 2: 1002, 3: 1003, 4: 1004, 5: 1005}
 
@@ -12,7 +12,7 @@ def _scales(rng, nblocks: int, sigma: float = 0.003) -> np.ndarray:
 
 def random_blocks(rng, ggml_type: int, n: int, k: int, sigma: float = 0.003, mx_exp=(119, 124)) -> np.ndarray:
   """(n, k) weight as raw GGUF block bytes: payload bytes uniform in 0..255 (nibbles uniform 0..15), scales valid.
-  Q8_0 quants avoid -128 (uniform in [-127, 127]); Q6_K sub-scales are int8 uniform in [-128, 127];
+  Q8_0 quants avoid -128 (uniform in [-127, 127]); Q6_K sub-scales are int8 uniform in [-128, 127]; Q4_K / Q5_K get valid d and dmin, their packed 6-bit scales and mins are uniform;
   MXFP4 exponent bytes are uniform in [mx_exp[0], mx_exp[1])."""
   nel, nby = GGML_QUANT[ggml_type]
   assert k % nel == 0
@@ -23,6 +23,7 @@ def random_blocks(rng, ggml_type: int, n: int, k: int, sigma: float = 0.003, mx_
     b[:, :2] = _scales(rng, nb, sigma)
     b[:, 2:] = rng.integers(-127, 128, size=(nb, 32), dtype=np.int8).view(np.uint8)
   elif ggml_type == Q6_K: b[:, 208:210] = _scales(rng, nb, sigma)
+  elif ggml_type in (Q4_K, Q5_K): b[:, 0:2] = _scales(rng, nb, sigma / 8); b[:, 2:4] = _scales(rng, nb, sigma / 8)   # d and dmin; 6-bit scales / mins stay random
   elif ggml_type == MXFP4: b[:, 0] = rng.integers(mx_exp[0], mx_exp[1], size=nb, dtype=np.uint8)
   return b.reshape(-1)
 
