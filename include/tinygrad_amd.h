@@ -120,7 +120,8 @@ int tga_moe_combine(const float* y, const float* probs, const float* resid, int 
  * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, pad[12]} so that one captured launch sequence serves
  * every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484). */
 
-/* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q8_0 / F16 / F32 table. */
+/* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K /
+ * MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant). */
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream);
 
 /* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL).

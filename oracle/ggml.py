@@ -133,3 +133,31 @@ def quantize_q6_k(w: np.ndarray) -> np.ndarray:
   out[:, 192:208] = sc.view(np.uint8)
   out[:, 208:210] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
   return out.reshape(-1)
+
+def _quantize_q45_k(w: np.ndarray, five: bool) -> np.ndarray:
+  """Simple min/max rule (NOT ggml's iterative make_qkx2_quants search): per 32-weight sub-block min m = max(0, -min x),
+  scale s = (max x + m) / qmax; superblock d = max s / 63, dmin = max m / 63 (fp16); 6-bit sc = round(s / d), mn = round(m / dmin);
+  q = clamp(round((x + dmin mn) / (d sc)), 0, qmax).  The byte packing is exactly the layout dequant_q4_k / dequant_q5_k decode."""
+  qmax = 31 if five else 15
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 8, 32)
+  nb = x.shape[0]
+  m = np.maximum(0, -x.min(axis=2)); s = (x.max(axis=2) + m) / np.float32(qmax)
+  d = (s.max(axis=1) / np.float32(63)).astype(np.float16).astype(np.float32); dmin = (m.max(axis=1) / np.float32(63)).astype(np.float16).astype(np.float32)
+  with np.errstate(divide="ignore", invalid="ignore"):
+    sc = np.where(d[:, None] > 0, np.rint(s / d[:, None]), 0).clip(0, 63).astype(np.uint8)
+    mn = np.where(dmin[:, None] > 0, np.rint(m / dmin[:, None]), 0).clip(0, 63).astype(np.uint8)
+    eff = d[:, None] * sc.astype(np.float32)
+    q = np.where(eff[:, :, None] > 0, np.rint((x + (dmin[:, None] * mn.astype(np.float32))[:, :, None]) / eff[:, :, None]), 0).clip(0, qmax).astype(np.uint8)
+  out = np.zeros((nb, 176 if five else 144), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2); out[:, 2:4] = dmin.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  sb = out[:, 4:16]                                                              # inverse of get_scale_min_k4
+  sb[:, 0:4] = (sc[:, 0:4] & 63) | ((sc[:, 4:8] >> 4) << 6)
+  sb[:, 4:8] = (mn[:, 0:4] & 63) | ((mn[:, 4:8] >> 4) << 6)
+  sb[:, 8:12] = (sc[:, 4:8] & 0xF) | ((mn[:, 4:8] & 0xF) << 4)
+  off = 48 if five else 16
+  out[:, off:off + 128] = ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).reshape(nb, 128)
+  if five: out[:, 16:48] = np.bitwise_or.reduce(((q >> 4) & 1) << np.arange(8, dtype=np.uint8)[None, :, None], axis=1)
+  return out.reshape(-1)
+
+def quantize_q4_k(w: np.ndarray) -> np.ndarray: return _quantize_q45_k(w, False)
+def quantize_q5_k(w: np.ndarray) -> np.ndarray: return _quantize_q45_k(w, True)

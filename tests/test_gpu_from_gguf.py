@@ -6,10 +6,30 @@ from oracle import ggml as og, gguf as ogguf, llm as ollm, linear as ol
 
 pytestmark = pytest.mark.gpu
 
-def _make_file(tmp_path, tied: bool):
+def _make_file(tmp_path, tied: bool, kquant: bool = False):
+  """kquant: the tensor-type mix of a Q4_K_M file (Q4_K linears and embedding, Q6_K for attn_v / ffn_down / output, one Q5_K matrix)."""
   rng = np.random.default_rng(11)
   c = dict(dim=256, hidden=512, H=4, KV=2, hd=64, L=2, vocab=512)
   def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
+  if kquant:
+    K4, K5, K6 = (12, og.quantize_q4_k), (13, og.quantize_q5_k), (14, og.quantize_q6_k)
+    tensors = [("token_embd.weight", (c["vocab"], c["dim"]), 12, og.quantize_q4_k(lin(c["vocab"], c["dim"]) * 16))]
+    for i in range(c["L"]):
+      p = f"blk.{i}."
+      mk = lambda name, rows, cols, tq: (p + name, (rows, cols), tq[0], tq[1](lin(rows, cols)))
+      tensors += [(p + "attn_norm.weight", (c["dim"],), 0, (1 + 0.1 * rng.standard_normal(c["dim"])).astype(np.float32)),
+                  mk("attn_q.weight", c["H"] * c["hd"], c["dim"], K4), mk("attn_k.weight", c["KV"] * c["hd"], c["dim"], K4),
+                  mk("attn_v.weight", c["KV"] * c["hd"], c["dim"], K6), mk("attn_output.weight", c["dim"], c["H"] * c["hd"], K5 if i else K4),
+                  (p + "ffn_norm.weight", (c["dim"],), 0, (1 + 0.1 * rng.standard_normal(c["dim"])).astype(np.float32)),
+                  mk("ffn_gate.weight", c["hidden"], c["dim"], K4), mk("ffn_up.weight", c["hidden"], c["dim"], K4), mk("ffn_down.weight", c["dim"], c["hidden"], K6)]
+    tensors.append(("output_norm.weight", (c["dim"],), 0, np.ones(c["dim"], np.float32)))
+    tensors.append(("output.weight", (c["vocab"], c["dim"]), 14, og.quantize_q6_k(lin(c["vocab"], c["dim"]))))
+    kvs = [("general.architecture", "qwen2"), ("qwen2.context_length", 96), ("qwen2.attention.head_count", c["H"]), ("qwen2.attention.head_count_kv", c["KV"]),
+           ("qwen2.block_count", c["L"]), ("qwen2.embedding_length", c["dim"]), ("qwen2.feed_forward_length", c["hidden"]),
+           ("qwen2.attention.layer_norm_rms_epsilon", 1e-6), ("qwen2.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(c["vocab"])])]
+    from tinygrad_amd.gguf import gguf_write
+    path = tmp_path / "q4_k_m.gguf"
+    return path, gguf_write(path, kvs, tensors)
   tensors = [("token_embd.weight", (c["vocab"], c["dim"]), 8, og.quantize_q8_0(lin(c["vocab"], c["dim"]) * 16))]
   for i in range(c["L"]):
     p = f"blk.{i}."
@@ -49,3 +69,24 @@ def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
+
+def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path):
+  """A file with the tensor types of a Q4_K_M model (Q4_K / Q5_K / Q6_K matrices, Q4_K embedding; q/k/v of mixed types, so the
+  block runs one launch per projection): greedy tokens and logits against the numpy restatement."""
+  from tinygrad_amd.llm import Transformer
+  path, raw = _make_file(tmp_path, False, kquant=True)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  assert model.layer_table is None                                     # K-quants take the per-op launches
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  prompt = [3, 200, 17, 450, 8]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3
+

@@ -120,7 +120,7 @@ def test_q6_k_association_order_is_exact():
 def test_quantizers_round_trip():
   rng = np.random.default_rng(0)
   w = rng.standard_normal(256 * 64).astype(np.float32)
-  for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0)):
+  for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0), (12, og.quantize_q4_k, 1 / 6.0), (13, og.quantize_q5_k, 1 / 13.0)):
     dq = og.ggml_data_to_tensor(qf(w), w.size, t)
     nel = og.GGML_QUANT[t][0] if t != 14 else 16
     amax = np.abs(w.reshape(-1, nel)).max(1, keepdims=True)

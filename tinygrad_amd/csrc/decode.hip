@@ -6,31 +6,31 @@
 #include "qfmt.h"
 #include "decode.h"
 #include "coherent.h"
+#include "deq.h"
 
-// ---------------------------------------------------------------------------------------------- embedding (Q4_0 / F16 / F32 row)
-// token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized.
+// ---------------------------------------------------------------------------------------------- embedding (one row of any table type)
+// token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized
+// (bit-exact block decode shared with tga_dequant).
+template <int T>
+__device__ __forceinline__ void embed_row_blocks(const uint8_t* __restrict__ table, int dim, int tok, float* __restrict__ out) {
+  const uint8_t* row = table + (size_t)tok * (dim / Deq<T>::NEL) * Deq<T>::NBY;
+  for (int e = threadIdx.x * 4; e < dim; e += 1024) {
+    float o[4];
+    Deq<T>::get4(row + (size_t)(e / Deq<T>::NEL) * Deq<T>::NBY, e % Deq<T>::NEL, o);
+    out[e] = o[0]; out[e + 1] = o[1]; out[e + 2] = o[2]; out[e + 3] = o[3];
+  }
+}
 __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, const DecodeState* st, float* __restrict__ out) {
   const int tok = st->token;
-  if (ggml_type == GGML_Q4_0) {
-    const uint8_t* row = table + (size_t)tok * (dim / 32) * 18;
-    for (int e = threadIdx.x; e < dim; e += 256) {
-      const uint8_t* b = row + (e >> 5) * 18; const int j = e & 31;
-      const float d = h2f_bits(ld2(b));
-      const int q = (j < 16) ? (b[2 + j] & 0xF) : (b[2 + j - 16] >> 4);
-      out[e] = (float)(q - 8) * d;
-    }
-  } else if (ggml_type == GGML_Q8_0) {
-    const uint8_t* row = table + (size_t)tok * (dim / 32) * 34;
-    for (int e = threadIdx.x; e < dim; e += 256) {
-      const uint8_t* b = row + (e >> 5) * 34;
-      out[e] = h2f_bits(ld2(b)) * (float)(int8_t)b[2 + (e & 31)];
-    }
-  } else if (ggml_type == GGML_F16) {
-    const uint16_t* row = (const uint16_t*)table + (size_t)tok * dim;
-    for (int e = threadIdx.x; e < dim; e += 256) out[e] = h2f_bits(row[e]);
-  } else {
-    const float* row = (const float*)table + (size_t)tok * dim;
-    for (int e = threadIdx.x; e < dim; e += 256) out[e] = row[e];
+  switch (ggml_type) {
+    case GGML_Q4_0: embed_row_blocks<GGML_Q4_0>(table, dim, tok, out); break;
+    case GGML_Q8_0: embed_row_blocks<GGML_Q8_0>(table, dim, tok, out); break;
+    case GGML_Q4_K: embed_row_blocks<GGML_Q4_K>(table, dim, tok, out); break;
+    case GGML_Q5_K: embed_row_blocks<GGML_Q5_K>(table, dim, tok, out); break;
+    case GGML_Q6_K: embed_row_blocks<GGML_Q6_K>(table, dim, tok, out); break;
+    case GGML_MXFP4: embed_row_blocks<GGML_MXFP4>(table, dim, tok, out); break;
+    case GGML_F16: { const uint16_t* row = (const uint16_t*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = h2f_bits(row[e]); break; }
+    default: { const float* row = (const float*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = row[e]; }
   }
 }
 
@@ -371,8 +371,10 @@ extern "C" {
 
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream) {
   TGA_REQUIRE(table && state && out, "tga_embed_row: null pointer");
-  TGA_REQUIRE(ggml_type == GGML_Q4_0 || ggml_type == GGML_Q8_0 || ggml_type == GGML_F16 || ggml_type == GGML_F32, "tga_embed_row: unsupported table type %d", ggml_type);
-  TGA_REQUIRE(dim > 0 && dim % 32 == 0, "tga_embed_row: dim=%d must be a positive multiple of 32", dim);
+  int blk = 0;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: blk = 256; break;
+    case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_row: unsupported table type %d", ggml_type); }
+  TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_row: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
   embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (const DecodeState*)state, out);
   TGA_LAUNCH_CHECK();
   return 0;

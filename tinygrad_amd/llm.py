@@ -142,16 +142,26 @@ class TransformerBlock:
     # RMSNorm folded into the consuming M = 1 linear (needs its register-resident fast path: K % 64, 4-byte aligned weights)
     fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K) or l.in_features % 256 == 0)
     self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
+    if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
 
   def __call__(self, x: Buffer, stream):
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     st = self.staged                                                     # producers write the consumer's staged order directly
-    if self.fuse_norm:                                                   # the q/k/v launch normalises the row while staging it
-      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], x, [s.q, s.k, s.v], stream=stream, norm=(self.attn_norm, c.norm_eps))
+    qkv, qkv_out = [self.attn_q, self.attn_k, self.attn_v], [s.q, s.k, s.v]
+    same = self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type
+    if self.fuse_norm and same:                                          # the q/k/v launch normalises the row while staging it
+      qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps))
     else:
       rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
-      qlinear_multi([self.attn_q, self.attn_k, self.attn_v], s.xn, [s.q, s.k, s.v], stream=stream)
+      if same: qlinear_multi(qkv, s.xn, qkv_out, stream=stream)
+      else:                                                              # mixed types (e.g. Q4_K q / k with a Q6_K v): one launch per run of equal types
+        i = 0
+        while i < 3:
+          j = i + 1
+          while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
+          qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream)
+          i = j
     if c.qk_norm: assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
     # full-width q/k RMSNorm before the head split (model.py:169) inside the attention launch
     rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
