@@ -5,6 +5,8 @@
   config 5  MXFP8 grouped GEMM at T = 4096, E = 128, k = 8 with Zipf routing (MFMA utilisation and GB/s), plus the measured
             register-only peak of the scaled FP8 MFMA
 
+  config 6  Q4_K / Q5_K dequant-GEMV at the same linear shapes (not a BASELINE config)
+
     python -m tinygrad_amd.benchmarks [--config N ...]        prints one JSON object per measurement
 
 Timing: HIP events around >= 100 back-to-back launches; weights are rotated over enough distinct copies to exceed the 256 MB
@@ -37,7 +39,12 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   wbytes = n * (k // nel) * nby
   copies = max(2, -(-int(1.25 * MALL_BYTES) // wbytes))
   big = Buffer((copies * wbytes,), np.uint8)
-  for c in range(copies): rt.check(rt.lib().tga_synth_weights(ggml_type, big.ptr + c * wbytes, n * k, 1000 + c, k ** -0.5, None))
+  if ggml_type in (rt.Q4_K, rt.Q5_K):                                         # no device-side writer for these: seeded host blocks, one upload per copy
+    from tinygrad_amd import synth
+    host = synth.random_blocks(np.random.default_rng(1002), ggml_type, n, k)
+    for c in range(copies): big.view(c * wbytes, (wbytes,), np.uint8).copyin(host)
+  else:
+    for c in range(copies): rt.check(rt.lib().tga_synth_weights(ggml_type, big.ptr + c * wbytes, n * k, 1000 + c, k ** -0.5, None))
   rt.synchronize()
   lins = [QuantLinear(big.view(c * wbytes, (wbytes,), np.uint8), ggml_type, n, k) for c in range(copies)]
   rng = np.random.default_rng(1002)
@@ -45,7 +52,7 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   s = rt.Stream()
   us = _time_launches(lambda i: lins[i](x, out=y, stream=s.handle), copies, iters, s)
   alg = wbytes + m * k * 2 + m * n * 2
-  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
+  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
   return {"case": f"{name} {n}x{k} M={m}", "avg_us": round(us, 2), "alg_bytes": alg, "GBps": round(alg / us / 1e3, 1),
           "frac_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_rotated": copies, "launches": iters}
 
@@ -55,6 +62,14 @@ def config2():
   out = []
   for t, n, k in ((rt.Q8_0, 4096, 4096), (rt.Q8_0, 14336, 4096), (rt.Q8_0, 4096, 14336), (rt.Q6_K, 128256, 4096)):
     for m in (1, 2, 4, 8): out.append(dict(config=2, **gemv_case(t, n, k, m, iters=100 if n > 100000 else 200)))
+  return out
+
+def kquants():
+  """Q4_K / Q5_K (the block types of Q4_K_M / Q5_K_M model files) at the Llama-3-8B linear shapes, M in {1, 8}."""
+  out = []
+  for t in (rt.Q4_K, rt.Q5_K):
+    for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
+      for m in (1, 8): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   return out
 
 def config4(steps: int = 64, ctx: int = 512):
@@ -144,12 +159,12 @@ def config5():
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5])
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K GEMV shapes")
   args = ap.parse_args()
   rt.init(0)
   print(json.dumps({"device": rt.device_name()}), flush=True)
   for cfg in args.config:
-    for row in {1: config1, 2: config2, 4: config4, 5: config5}[cfg](): print(json.dumps(row), flush=True)
+    for row in {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants}[cfg](): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":
   main()

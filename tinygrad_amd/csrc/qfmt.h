@@ -77,7 +77,7 @@ template <> struct Fmt<GGML_Q4_0> {
     for (int k = 0; k < 8; k++) { lo = dot2(nx[k], 0x64086408u, lo); hi = dot2(nx[k + 8], 0x54805480u, hi); }   // 1032, 72
     c[0] = -(lo + hi);
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
 };
 
 // ------------------------------------------------------------------------------------------------ Q8_0 (gguf.py:56)
@@ -110,7 +110,7 @@ template <> struct Fmt<GGML_Q8_0> {
     for (int k = 0; k < 16; k++) s = dot2(nx[k], 0x64806480u, s);   // 1152
     c[0] = -s;
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) { return h2f_bits(r.d) * a[0]; }
 };
 
 
@@ -180,7 +180,7 @@ template <> struct Fmt<F_Q4_0P> {
       c[j] = -(lo + hi);
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
   }
   // halfword index of row element e inside the staged activation buffer ([XV][nu] vectors of 4 fp16 pairs)
@@ -245,7 +245,7 @@ template <> struct Fmt<F_Q8_0P> {
       c[j] = -t;
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
   }
   static __device__ __forceinline__ int spos(int e, int nu) {
@@ -303,7 +303,7 @@ template <> struct Fmt<GGML_F16> {
     for (int v = 0; v < 8; v++) { xv[v].x = nx[4 * v]; xv[v].y = nx[4 * v + 1]; xv[v].z = nx[4 * v + 2]; xv[v].w = nx[4 * v + 3]; }
     c[0] = 0.f;
   }
-  static __device__ __forceinline__ float finish(const Raw&, const float* a, const float*) { return a[0]; }
+  static __device__ __forceinline__ float finish(const Raw&, const uint32_t*, const float* a, const float*) { return a[0]; }
   static __device__ __forceinline__ int spos(int e, int nu) { return e; }
   static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
@@ -348,7 +348,7 @@ template <> struct Fmt<GGML_MXFP4> {
     c[0] = 0.f;
   }
   // reference value = (2 * e2m1) * 2^(e-128) = e2m1 * 2^(e-127); e = 0 is the fp32 subnormal 2^-127
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u) * a[0];
   }
   static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 5, b = e & 31, q = b & 15; return (((q >> 2) * nu + u) * 4 + (q & 3)) * 2 + (b >> 4); }
@@ -409,7 +409,7 @@ template <> struct Fmt<GGML_Q6_K> {
       c[j] = -s;
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float*) {
+  static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     const int g8 = (r.d & 1) * 8;   // scales 8h + 2j + g live in bytes g, g+2 of sc0 (j = 0, 1) and sc1 (j = 2, 3)
     const float s0 = (float)(int)(int8_t)(r.sc0 >> g8), s1 = (float)(int)(int8_t)(r.sc0 >> (16 + g8));
     const float s2 = (float)(int)(int8_t)(r.sc1 >> g8), s3 = (float)(int)(int8_t)(r.sc1 >> (16 + g8));
@@ -447,7 +447,7 @@ template <bool FIVE> struct FmtK45 {
   static constexpr int UW = 64, UPB = 4, BW = 256, BB = FIVE ? 176 : 144, QS = FIVE ? 48 : 16;
   static __device__ __forceinline__ int unit_of(int e) { return e >> 6; }
   static __device__ __forceinline__ int pair_of(int e) { return (e & 63) >> 1; }
-  static constexpr int XV = 8, NG = 2, NWV = 32;
+  static constexpr int XV = 8, NG = 2, NWV = 36;
   typedef RawK45<FIVE> Raw;
   static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
     const uint8_t* b = row + (size_t)BB * (u >> 2); const int p = u & 3;
@@ -473,6 +473,15 @@ template <bool FIVE> struct FmtK45 {
       }
       wv[2 * t] = le; wv[2 * t + 1] = lo; wv[16 + 2 * t] = he; wv[16 + 2 * t + 1] = ho;
     }
+    // get_scale_min_k4 for sub-blocks 2p, 2p + 1: byte index i = 2 (p & 1) (+1) of scales[0..3] / [4..7] / [8..11]; branch-free blend
+    const uint32_t sh = 16 * (r.p & 1), hm = 0u - (r.p >> 1);                 // hm = all ones for sub-blocks 4..7
+    const uint32_t y0 = (r.hdr.y >> sh) & 0xFF, y1 = (r.hdr.y >> (sh + 8)) & 0xFF, z0 = (r.hdr.z >> sh) & 0xFF, z1 = (r.hdr.z >> (sh + 8)) & 0xFF;
+    const uint32_t w0 = (r.hdr.w >> sh) & 0xFF, w1 = (r.hdr.w >> (sh + 8)) & 0xFF;
+    const uint32_t sc0 = ((y0 & 63) & ~hm) | (((w0 & 0xF) | ((y0 >> 6) << 4)) & hm), sc1 = ((y1 & 63) & ~hm) | (((w1 & 0xF) | ((y1 >> 6) << 4)) & hm);
+    const uint32_t mn0 = ((z0 & 63) & ~hm) | (((w0 >> 4) | ((z0 >> 6) << 4)) & hm), mn1 = ((z1 & 63) & ~hm) | (((w1 >> 4) | ((z1 >> 6) << 4)) & hm);
+    const float d = h2f_bits(r.hdr.x & 0xFFFF), dmin = h2f_bits(r.hdr.x >> 16);
+    wv[32] = __builtin_bit_cast(uint32_t, d * (float)sc0); wv[33] = __builtin_bit_cast(uint32_t, d * (float)sc1);
+    wv[34] = __builtin_bit_cast(uint32_t, dmin * (float)mn0 * (1.0f / 1024.0f)); wv[35] = __builtin_bit_cast(uint32_t, dmin * (float)mn1 * (1.0f / 64.0f));
   }
   // nx[k] = natural pair k of the unit's 64 activations; xv[4g + v] = {E, O, E', O'} of dwords 2v, 2v + 1 of group g
   static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
@@ -490,16 +499,11 @@ template <bool FIVE> struct FmtK45 {
       c[g] = -s;
     }
   }
-  static __device__ __forceinline__ float finish(const Raw& r, const float* a, const float* c) {
-    // get_scale_min_k4 for sub-blocks 2p, 2p + 1: byte index i = 2 (p & 1) (+1) of scales[0..3] / [4..7] / [8..11]
-    const uint32_t sh = 16 * (r.p & 1);
-    const uint32_t y0 = (r.hdr.y >> sh) & 0xFF, y1 = (r.hdr.y >> (sh + 8)) & 0xFF, z0 = (r.hdr.z >> sh) & 0xFF, z1 = (r.hdr.z >> (sh + 8)) & 0xFF;
-    const uint32_t w0 = (r.hdr.w >> sh) & 0xFF, w1 = (r.hdr.w >> (sh + 8)) & 0xFF;
-    const bool hi = r.p >= 2;
-    const float sc0 = (float)(hi ? ((w0 & 0xF) | ((y0 >> 6) << 4)) : (y0 & 63)), sc1 = (float)(hi ? ((w1 & 0xF) | ((y1 >> 6) << 4)) : (y1 & 63));
-    const float mn0 = (float)(hi ? ((w0 >> 4) | ((z0 >> 6) << 4)) : (z0 & 63)), mn1 = (float)(hi ? ((w1 >> 4) | ((z1 >> 6) << 4)) : (z1 & 63));
-    const float d = h2f_bits(r.hdr.x & 0xFFFF), dmin = h2f_bits(r.hdr.x >> 16);
-    return d * (sc0 * a[0] + sc1 * a[1]) + dmin * (mn0 * (c[0] * (1.0f / 1024.0f)) + mn1 * (c[1] * (1.0f / 64.0f)));
+  // decode() leaves the unit's four scale factors behind the weights: wv[32..35] = d sc0, d sc1, dmin mn0 / 1024, dmin mn1 / 64
+  // (extracted once per unit, not once per activation row)
+  static __device__ __forceinline__ float finish(const Raw&, const uint32_t* wv, const float* a, const float* c) {
+    return __builtin_bit_cast(float, wv[32]) * a[0] + __builtin_bit_cast(float, wv[33]) * a[1]
+         + __builtin_bit_cast(float, wv[34]) * c[0] + __builtin_bit_cast(float, wv[35]) * c[1];
   }
   static __device__ __forceinline__ int spos(int e, int nu) {
     const int u = e >> 6, g = (e >> 5) & 1, r = e & 31, wi = 2 * (r >> 2) + (r & 1);
@@ -538,7 +542,7 @@ __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, co
     }
     g[j] = t;
   }
-  acc += F::finish(raw, g, cv);
+  acc += F::finish(raw, wv, g, cv);
 }
 
 // M = 1 stores.  EPI 0: plain, EPI 1: + residual, EPI 2: silu(gate) * up into output row `row` of segment 0.

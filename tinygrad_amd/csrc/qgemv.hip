@@ -76,7 +76,7 @@ __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const 
       }
       g[j] = s;
     }
-    acc[m] += F::finish(raw, g, cc);
+    acc[m] += F::finish(raw, wv, g, cc);
   }
 }
 
@@ -113,7 +113,7 @@ __device__ __forceinline__ void unit_dot_rows(const typename Fmt<T>::Raw* raw, c
       for (int r = 0; r < R; r++) g[r][j] = s[r];
     }
 #pragma unroll
-    for (int r = 0; r < R; r++) acc[r][m] += F::finish(raw[r], g[r], cc);
+    for (int r = 0; r < R; r++) acc[r][m] += F::finish(raw[r], wv[r], g[r], cc);
     // one activation row's vectors live at a time: without this the scheduler hoists the LDS reads of all M rows (M x 32 VGPRs)
     if constexpr (M * R > 4) __builtin_amdgcn_sched_barrier(0);
   }
