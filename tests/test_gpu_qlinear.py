@@ -20,8 +20,13 @@ def _check(y, x, W):
   ref64 = ol.linear_f64(x.astype(np.float32), W)
   e = ol.rel_err(y, ref64)
   assert e <= TOL, f"rel-err {e:.3e} vs float64 anchor"
-  # elementwise: allclose in the sense of the reference's VALIDATE_WITH_CPU harness (engine/realize.py:192-201), atol scaled to the output rms
-  np.testing.assert_allclose(y, ref64, rtol=TOL, atol=TOL * float(np.sqrt(np.mean(ref64 ** 2))))
+  # elementwise: allclose in the sense of the reference's VALIDATE_WITH_CPU harness (engine/realize.py:192-201), atol scaled to the output rms.
+  # The anchor is the exact-weight result or the result with weights rounded to fp16 (the reference's model path casts every weight to
+  # fp16, model.py:376; the matrix-core kernel for M >= 3 rounds them the same way, the dot2 kernels use them exactly)
+  atol = TOL * float(np.sqrt(np.mean(ref64 ** 2)))
+  with np.errstate(over="ignore"): ref16 = ol.linear_f64(x.astype(np.float32), W.astype(np.float16).astype(np.float32))
+  close = np.isclose(y, ref64, rtol=TOL, atol=atol) | np.isclose(y, ref16, rtol=TOL, atol=atol)
+  assert close.all(), f"{np.count_nonzero(~close)} of {close.size} outputs outside rtol/atol {TOL}"
   return e
 
 @pytest.mark.parametrize("t", [2, 8, 12, 13, 14, 39])

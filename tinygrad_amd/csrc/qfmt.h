@@ -37,6 +37,25 @@ __device__ __forceinline__ uint32_t pack_odd(uint32_t a, uint32_t b) { return (a
 
 template <int T> struct Fmt;
 
+// Decoded weights still carry their exponent-bias and integer offsets (1024 + q etc.) and no block scale.  to_f16 turns a decoded
+// unit into the true weights as fp16 pairs, (pattern - bias) * scale: the subtraction is exact in fp16 (small integers), the
+// product rounds once to fp16 - the same rounding as the reference's fp16 weight cast (tinygrad/llm/model.py:376).  Used by the
+// MFMA small-batch kernel, where one decode serves all activation rows and the block scale cannot be applied after the MFMA.
+__device__ __forceinline__ uint32_t h2_unbias_scale(uint32_t pattern, float bias, half2_t scale) {
+  const half2_t b = {(_Float16)bias, (_Float16)bias};
+  return as_u32((as_h2(pattern) - b) * scale);
+}
+// the same with a float32 scale: pattern * s - bias * s evaluated in float32 and rounded to fp16 once (v_fma_mix), for scales that are
+// themselves products (Q6_K: d * sub-scale) and would otherwise be rounded twice
+__device__ __forceinline__ uint32_t h2_unbias_scale_f32(uint32_t pattern, float scale, float neg_bias_scale) {
+  const half2_t p = as_h2(pattern);
+  half2_t o = {(_Float16)((float)p.x * scale + neg_bias_scale), (_Float16)((float)p.y * scale + neg_bias_scale)};
+  return as_u32(o);
+}
+__device__ __forceinline__ half2_t h2_splat_bits(uint32_t h16) { const _Float16 v = __builtin_bit_cast(_Float16, (uint16_t)h16); half2_t r = {v, v}; return r; }
+__device__ __forceinline__ half2_t h2_splat_f(float f) { const _Float16 v = (_Float16)f; half2_t r = {v, v}; return r; }
+
+
 // A constant the compiler must keep in a VGPR: VOP3 forms such as v_and_or_b32 / v_perm_b32 accept a single scalar
 // operand and no literal on this ISA, so (x & MASK) | BIAS only becomes one instruction when BIAS already lives in a VGPR.
 __device__ __forceinline__ uint32_t vgpr_const(uint32_t c) { asm("" : "+v"(c)); return c; }
@@ -183,6 +202,15 @@ template <> struct Fmt<F_Q4_0P> {
   static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.b.x >> 16) * a[1];
   }
+  static __device__ __forceinline__ void to_f16(const Raw& r, uint32_t* wv) {
+    const half2_t d0 = h2_splat_bits(r.a.x & 0xFFFFu), d1 = h2_splat_bits(r.b.x >> 16);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const half2_t d = i < 4 ? d0 : d1;
+      wv[4 * i + 0] = h2_unbias_scale(wv[4 * i + 0], 1032.f, d); wv[4 * i + 1] = h2_unbias_scale(wv[4 * i + 1], 72.f, d);
+      wv[4 * i + 2] = h2_unbias_scale(wv[4 * i + 2], 1032.f, d); wv[4 * i + 3] = h2_unbias_scale(wv[4 * i + 3], 72.f, d);
+    }
+  }
   // halfword index of row element e inside the staged activation buffer ([XV][nu] vectors of 4 fp16 pairs)
   static __device__ __forceinline__ int spos(int e, int nu) {
     const int u = e >> 6, w = e & 63, blk = w >> 5, b = w & 31, hi = b >> 4, q = b & 15;
@@ -247,6 +275,11 @@ template <> struct Fmt<F_Q8_0P> {
   }
   static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return h2f_bits(r.a.x & 0xFFFFu) * a[0] + h2f_bits(r.c.x >> 16) * a[1];
+  }
+  static __device__ __forceinline__ void to_f16(const Raw& r, uint32_t* wv) {
+    const half2_t d0 = h2_splat_bits(r.a.x & 0xFFFFu), d1 = h2_splat_bits(r.c.x >> 16);
+#pragma unroll
+    for (int i = 0; i < 32; i++) wv[i] = h2_unbias_scale(wv[i], 1152.f, i < 16 ? d0 : d1);
   }
   static __device__ __forceinline__ int spos(int e, int nu) {
     const int u = e >> 6, w = e & 63, blk = w >> 5, b = w & 31, n = b >> 1;
@@ -415,6 +448,14 @@ template <> struct Fmt<GGML_Q6_K> {
     const float s2 = (float)(int)(int8_t)(r.sc1 >> g8), s3 = (float)(int)(int8_t)(r.sc1 >> (16 + g8));
     return h2f_bits(r.d >> 16) * (s0 * a[0] + s1 * a[1] + s2 * a[2] + s3 * a[3]);
   }
+  static __device__ __forceinline__ void to_f16(const Raw& r, uint32_t* wv) {
+    const int g8 = (r.d & 1) * 8;
+    const float d = h2f_bits(r.d >> 16);
+    const float s[4] = {d * (float)(int)(int8_t)(r.sc0 >> g8), d * (float)(int)(int8_t)(r.sc0 >> (16 + g8)),
+                        d * (float)(int)(int8_t)(r.sc1 >> g8), d * (float)(int)(int8_t)(r.sc1 >> (16 + g8))};
+#pragma unroll
+    for (int i = 0; i < 32; i++) wv[i] = h2_unbias_scale_f32(wv[i], s[i >> 3], -1056.f * s[i >> 3]);
+  }
   static __device__ __forceinline__ int spos(int e, int nu) {
     const int u = unit_of(e), j = (e >> 5) & 3, i = e & 15, td = i >> 2, p = i & 3;
     return (((2 * j + (td >> 1)) * nu + u) * 4 + (td & 1) * 2 + (p & 1)) * 2 + (p >> 1);
@@ -505,6 +546,13 @@ template <bool FIVE> struct FmtK45 {
     return __builtin_bit_cast(float, wv[32]) * a[0] + __builtin_bit_cast(float, wv[33]) * a[1]
          + __builtin_bit_cast(float, wv[34]) * c[0] + __builtin_bit_cast(float, wv[35]) * c[1];
   }
+  // true weights (d sc) q - dmin mn as fp16, one rounding: group 0 patterns are 1024 + q, group 1 patterns 64 + q
+  static __device__ __forceinline__ void to_f16(const Raw&, uint32_t* wv) {
+    const float s0 = __builtin_bit_cast(float, wv[32]), s1 = __builtin_bit_cast(float, wv[33]);
+    const float c0 = -1024.f * s0 - 1024.f * __builtin_bit_cast(float, wv[34]), c1 = -64.f * s1 - 64.f * __builtin_bit_cast(float, wv[35]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) { wv[i] = h2_unbias_scale_f32(wv[i], s0, c0); wv[16 + i] = h2_unbias_scale_f32(wv[16 + i], s1, c1); }
+  }
   static __device__ __forceinline__ int spos(int e, int nu) {
     const int u = e >> 6, g = (e >> 5) & 1, r = e & 31, wi = 2 * (r >> 2) + (r & 1);
     return (((4 * g + (wi >> 2)) * nu + u) * 4 + (wi & 3)) * 2 + ((r >> 1) & 1);
@@ -571,3 +619,36 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
   }
   return e;
 }
+
+// ------------------------------------------------------------------------------------------------ activation staging (M rows, LDS)
+// LDS layout for units [u0, u0+cu): xs[(m*XV + t) * cu + (u-u0)] (u32x4), then cs[(m*NG + j) * cu + (u-u0)] (float)
+template <int T, int M>
+__device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs, int u0, int cu) {
+  using F = Fmt<T>;
+  constexpr int NP = F::UW / 2;
+  for (int i = threadIdx.x; i < M * cu; i += QG_THREADS) {
+    const int m = i / cu, ul = i - m * cu, u = u0 + ul;
+    // four consecutive pairs (8 activations) of a unit are contiguous in every format: 16-byte (fp16) / 2 x 16-byte (fp32) loads
+    uint32_t nx[NP];
+    if (a.x_f32) {
+      const float* x = (const float*)a.x + (long long)m * a.K;
+#pragma unroll
+      for (int k = 0; k < NP; k += 4) {
+        const f32x4 lo = *(const f32x4*)(x + F::xoff(u, k)), hi = *(const f32x4*)(x + F::xoff(u, k) + 4);
+        nx[k] = f2h_bits(lo.x) | (f2h_bits(lo.y) << 16); nx[k + 1] = f2h_bits(lo.z) | (f2h_bits(lo.w) << 16);
+        nx[k + 2] = f2h_bits(hi.x) | (f2h_bits(hi.y) << 16); nx[k + 3] = f2h_bits(hi.z) | (f2h_bits(hi.w) << 16);
+      }
+    } else {
+      const uint16_t* x = (const uint16_t*)a.x + (long long)m * a.K;
+#pragma unroll
+      for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(x + F::xoff(u, k)); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+    }
+    u32x4 xv[F::XV]; float c[F::NG];
+    F::stage(nx, xv, c);
+#pragma unroll
+    for (int t = 0; t < F::XV; t++) xs[(m * F::XV + t) * cu + ul] = xv[t];
+#pragma unroll
+    for (int j = 0; j < F::NG; j++) cs[(m * F::NG + j) * cu + ul] = c[j];
+  }
+}
+

@@ -1,0 +1,152 @@
+// Small-batch GEMM over GGUF blocks on the matrix cores (3 <= M <= 8 activation rows), for the same call sites as qgemv.hip
+// (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392).
+//
+// The dot2 kernel decodes a weight once per TWO activation rows and multiplies on the VALU, so from M = 4 on it is bound by
+// VALU issue, not by HBM.  Here a unit is decoded ONCE into true fp16 weights ((pattern - bias) * block scale, one fp16 rounding -
+// the rounding of the reference's fp16 weight cast, tinygrad/llm/model.py:376) and v_mfma_f32_16x16x32_f16 multiplies it with all
+// activation rows at once (M padded to 16 columns): the VALU work per weight byte no longer depends on M.
+//
+// Mapping: a wave owns 16 weight rows at a time.  Lane l = 16 g + r loads unit 4 s + g of row r (step s): the four lane groups
+// cover four consecutive units of each row.  A unit's XV vectors of 8 fp16 are the A operands of XV MFMAs; the B operand of lane
+// 16 g + c is activation row c's vector of the SAME unit (zero for c >= M), read from the LDS staging that qgemv.hip uses
+// ([row][vector][unit]).  Both operands of a lane group name the same 8 k-values element by element, which is all the MFMA needs.
+// The four waves of a workgroup take the steps of a row group round-robin (a split of K) and their 16 x 16 partial results meet
+// in LDS.  K is walked in LDS-sized chunks when M * K does not fit.
+#include "qfmt.h"
+
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+#define QM_THREADS 256
+#define QM_LDS_BUDGET (72 * 1024)     // activations of one chunk when two workgroups share a CU
+
+template <int T, int M>
+__global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs a) {
+  using F = Fmt<T>;
+  typedef typename F::Raw Raw;
+  extern __shared__ u32x4 lds[];
+  __shared__ float part[4][16][17];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  const long long ngroups = (a.ntot + 15) / 16;
+  for (long long grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
+    const long long row0 = grp * 16;
+    const long long myrow = row0 + r < a.ntot ? row0 + r : a.ntot - 1;   // ragged last group: reload a valid row, results dropped
+    const uint8_t* rowp = a.w[0] + myrow * a.row_bytes;
+    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int ch = 0; ch < a.nchunks; ch++) {
+      const int u0 = ch * a.chunk_u, cu = min(a.chunk_u, a.nu - u0);
+      u32x4* xs = lds; float* cs = (float*)(lds + M * F::XV * cu);
+      const int nsteps = (cu + 3) >> 2;                                 // steps of 4 units in this chunk; wave w takes s = w, w + 4, ...
+      Raw b0, b1;
+      auto issue = [&](Raw& buf, int s) { const int ul = 4 * s + g; buf = F::load(rowp, u0 + (ul < cu ? ul : cu - 1)); };
+      if (wave < nsteps) issue(b0, wave);                               // first loads ahead of the staging
+      if (a.nchunks > 1 || grp == (long long)blockIdx.x) {              // a single chunk is staged once per workgroup
+        __syncthreads();
+        stage_chunk<T, M>(a, xs, cs, u0, cu);
+        __syncthreads();
+      }
+      auto compute = [&](const Raw& buf, int s) {
+        const int ul = 4 * s + g;
+        uint32_t wv[F::NWV];
+        F::decode(buf, wv, kc);
+        F::to_f16(buf, wv);
+        const bool uval = ul < cu;
+        const int ulc = uval ? ul : cu - 1;
+#pragma unroll
+        for (int v = 0; v < F::XV; v++) {
+          u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
+          if (!uval) av = u32x4{0u, 0u, 0u, 0u};
+          u32x4 bv = {0u, 0u, 0u, 0u};
+          if (r < M) bv = xs[(r * F::XV + v) * cu + ulc];
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv), acc, 0, 0, 0);
+        }
+      };
+      for (int s = wave; s < nsteps; s += 8) {
+        if (s + 4 < nsteps) issue(b1, s + 4);
+        compute(b0, s);
+        if (s + 4 < nsteps) {
+          if (s + 8 < nsteps) issue(b0, s + 8);
+          compute(b1, s + 4);
+        }
+      }
+    }
+    // D: lane (g, c) holds weight rows 4 g + i (i = 0..3) for activation row c
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) part[wave][4 * g + i][r] = acc[i];
+    __syncthreads();
+    {
+      const int t = threadIdx.x, wr = t >> 4, c = t & 15;              // 256 threads = 16 weight rows x 16 activation rows
+      if (c < M && row0 + wr < a.ntot) {
+        const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
+        const long long o = (long long)c * a.ntot + row0 + wr;
+        if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+      }
+    }
+  }
+}
+
+static int qm_cu_count() {
+  static int n = 0;
+  if (!n) { int dev = 0; hipDeviceProp_t p; n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) ? p.multiProcessorCount : 256; }
+  return n;
+}
+
+template <int T, int M>
+static int launch_qgemm(QArgs a, hipStream_t s) {
+  using F = Fmt<T>;
+  const int per_unit = M * (16 * F::XV + 4 * F::NG);
+  a.nu = a.K / F::UW;
+  a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+  const long long ngroups = (a.ntot + 15) / 16;
+  // LDS budget for one chunk of activations: two workgroups per CU, or the whole CU when there is at most one row group per CU anyway
+  const int budget = ngroups <= qm_cu_count() ? 2 * QM_LDS_BUDGET : QM_LDS_BUDGET;
+  int cu = budget / per_unit; cu -= cu % 16; if (cu < 16) cu = 16;
+  if (cu >= a.nu) { a.chunk_u = a.nu; a.nchunks = 1; } else { a.nchunks = (a.nu + cu - 1) / cu; a.chunk_u = ((a.nu + a.nchunks - 1) / a.nchunks + 15) / 16 * 16; }
+  const size_t lds = (size_t)per_unit * a.chunk_u;
+  // single chunk: the activations are staged once per workgroup, so no more workgroups than stay resident (by LDS, at most 8 per
+  // CU); chunked K: every row group restages each chunk, one group per workgroup
+  int resident = (int)((160 * 1024) / (lds + 5 * 1024)); resident = resident < 1 ? 1 : resident > 8 ? 8 : resident;
+  long long grid = ngroups;
+  const long long cap = (long long)qm_cu_count() * (a.nchunks == 1 ? resident : 8);
+  if (grid > cap) grid = cap;
+  auto kern = qgemm_mfma_kernel<T, M>;
+  if (lds > 48 * 1024) {
+    static bool configured = false;
+    if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * QM_LDS_BUDGET + 4096)); configured = true; }
+  }
+  kern<<<dim3((unsigned)grid), dim3(QM_THREADS), lds, s>>>(a);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int T>
+static int launch_qgemm_m(const QArgs& a, int M, hipStream_t s) {
+  switch (M) {
+    case 3: return launch_qgemm<T, 3>(a, s);
+    case 4: return launch_qgemm<T, 4>(a, s);
+    case 5: return launch_qgemm<T, 5>(a, s);
+    case 6: return launch_qgemm<T, 6>(a, s);
+    case 7: return launch_qgemm<T, 7>(a, s);
+    case 8: return launch_qgemm<T, 8>(a, s);
+  }
+  return -1;
+}
+
+// Returns -1 when the call is outside this kernel's range (the caller then takes the dot2 kernel): plain single-segment linears
+// of the block-pair / superblock formats with 3 <= M <= 8.
+int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
+  if (M < 3 || M > 8 || a.nseg != 1 || a.epilogue != 0 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (((uintptr_t)a.x & 15) != 0) return -1;
+  switch (fmt) {
+    case F_Q4_0P: return launch_qgemm_m<F_Q4_0P>(a, M, s);
+    case F_Q8_0P: return launch_qgemm_m<F_Q8_0P>(a, M, s);
+    case GGML_Q6_K: return launch_qgemm_m<GGML_Q6_K>(a, M, s);
+    case GGML_Q4_K: return launch_qgemm_m<GGML_Q4_K>(a, M, s);
+    case GGML_Q5_K: return launch_qgemm_m<GGML_Q5_K>(a, M, s);
+  }
+  return -1;
+}

@@ -24,37 +24,6 @@
 #include "qfmt.h"
 
 // ------------------------------------------------------------------------------------------------ kernel
-// LDS layout for units [u0, u0+cu): xs[(m*XV + t) * cu + (u-u0)] (u32x4), then cs[(m*NG + j) * cu + (u-u0)] (float)
-template <int T, int M>
-__device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs, int u0, int cu) {
-  using F = Fmt<T>;
-  constexpr int NP = F::UW / 2;
-  for (int i = threadIdx.x; i < M * cu; i += QG_THREADS) {
-    const int m = i / cu, ul = i - m * cu, u = u0 + ul;
-    // four consecutive pairs (8 activations) of a unit are contiguous in every format: 16-byte (fp16) / 2 x 16-byte (fp32) loads
-    uint32_t nx[NP];
-    if (a.x_f32) {
-      const float* x = (const float*)a.x + (long long)m * a.K;
-#pragma unroll
-      for (int k = 0; k < NP; k += 4) {
-        const f32x4 lo = *(const f32x4*)(x + F::xoff(u, k)), hi = *(const f32x4*)(x + F::xoff(u, k) + 4);
-        nx[k] = f2h_bits(lo.x) | (f2h_bits(lo.y) << 16); nx[k + 1] = f2h_bits(lo.z) | (f2h_bits(lo.w) << 16);
-        nx[k + 2] = f2h_bits(hi.x) | (f2h_bits(hi.y) << 16); nx[k + 3] = f2h_bits(hi.z) | (f2h_bits(hi.w) << 16);
-      }
-    } else {
-      const uint16_t* x = (const uint16_t*)a.x + (long long)m * a.K;
-#pragma unroll
-      for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(x + F::xoff(u, k)); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
-    }
-    u32x4 xv[F::XV]; float c[F::NG];
-    F::stage(nx, xv, c);
-#pragma unroll
-    for (int t = 0; t < F::XV; t++) xs[(m * F::XV + t) * cu + ul] = xv[t];
-#pragma unroll
-    for (int j = 0; j < F::NG; j++) cs[(m * F::NG + j) * cu + ul] = c[j];
-  }
-}
-
 template <int T, int M>
 __device__ __forceinline__ void unit_dot(const typename Fmt<T>::Raw& raw, const u32x4* xs, const float* cs, int cu, int ul, float* acc, const uint32_t* kc) {
   using F = Fmt<T>;
@@ -346,6 +315,7 @@ static int launch_qgemv_m(const QArgs& a, int M, hipStream_t s) {
 }
 
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
+int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -424,6 +394,10 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
   if (M == 1) {
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
+  }
+  if (M >= 3) {                                                   // matrix-core small-batch kernel (plain single-segment linears)
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+    if (fmt >= 0) { const int rc = tga_qgemm_mfma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
   }
   TGA_REQUIRE(!norm_w, "tga_rmsnorm_qlinear: the fused norm needs the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, 16-byte aligned x, K <= 65536)");
   TGA_REQUIRE(!a.x_staged && !a.y_stage_fmt, "tga_qlinear: staged activations need the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, K <= 65536)");
