@@ -48,6 +48,7 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs a) {
         stage_chunk<T, M>(a, xs, cs, u0, cu);
         __syncthreads();
       }
+      const bool ragged = (cu & 3) != 0;
       auto compute = [&](const Raw& buf, int s) {
         const int ul = 4 * s + g;
         uint32_t wv[F::NWV];
@@ -58,7 +59,7 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs a) {
 #pragma unroll
         for (int v = 0; v < F::XV; v++) {
           u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
-          if (!uval) av = u32x4{0u, 0u, 0u, 0u};
+          if (ragged && !uval) av = u32x4{0u, 0u, 0u, 0u};      // (whole steps only when the chunk is a multiple of 4 units)
           u32x4 bv = {0u, 0u, 0u, 0u};
           if (r < M) bv = xs[(r * F::XV + v) * cu + ulc];
           acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv), acc, 0, 0, 0);
