@@ -72,22 +72,22 @@ def kquants():
       for m in (1, 8): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   return out
 
-def config4(steps: int = 64, ctx: int = 512):
+def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
   import time
   c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **OLMOE)
   model = Transformer(c, synth_state_moe(c, seed=1004), max_new=steps + 16)
   rt.synchronize()
   rng = np.random.default_rng(1004)
-  model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)], True)
-  for _ in range(8): model.decode_step(True)
+  model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)], use_graph)
+  for _ in range(8): model.decode_step(use_graph)
   rt.synchronize()
   t0 = time.perf_counter()
-  for _ in range(steps): model.decode_step(True)
+  for _ in range(steps): model.decode_step(use_graph)
   rt.synchronize()
   dt = (time.perf_counter() - t0) / steps
   expert_bytes = c.num_blocks * c.num_experts_per_tok * sum(e.expert_nbytes for e in (model.blk[0].ffn_gate_exps, model.blk[0].ffn_up_exps, model.blk[0].ffn_down_exps))
-  res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, graph replay + sync per token)",
+  res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, {'graph replay' if use_graph else 'eager launches'} + sync per token)",
           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "expert_bytes_per_token": expert_bytes, "weight_bytes_per_token": model.weight_bytes_per_token(),
           "weight_GBps_over_step": round(model.weight_bytes_per_token() / dt / 1e9, 1)}]
   # the expert GEMVs alone: B tokens x 8 experts, gate/up fused then down, distinct experts per slot, layers rotated
@@ -160,11 +160,13 @@ def config5():
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K GEMV shapes")
+  ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
   args = ap.parse_args()
   rt.init(0)
   print(json.dumps({"device": rt.device_name()}), flush=True)
   for cfg in args.config:
-    for row in {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants}[cfg](): print(json.dumps(row), flush=True)
+    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants}[cfg]
+    for row in (fn(use_graph=not args.no_graph) if cfg == 4 else fn()): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":
   main()
