@@ -179,6 +179,10 @@ int tga_decode_layers_trace(void* buf);
  * q = E4M3(clamp(x * 2^(127 - e8), +-448)) (RNE, tinygrad/dtype.py:237-260).  x: (rows, K) bf16 (x_is_bf16) or float32.
  * q: (rows, K) bytes; e8: (rows, K/32) bytes; packed (may be NULL): mx_pack layout (K/128, rows) uint32 (cdna_asm_gemm.py:161-163). */
 int tga_quantize_mxfp8(const void* x, int x_is_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream);
+/* fused_silu_mul_quantize_mxfp8 (extra/llama_kernels/fused_silu_mul_quantize_mxfp8/__init__.py:11-49, 91-104): act = w1 * sigmoid(w1) * w3 in
+ * float32 from two (rows, K) bf16 tensors (sigmoid = 1 / (1 + exp2(-w1 * log2 e))), quantized as tga_quantize_mxfp8 without an intermediate
+ * tensor; outputs as there. */
+int tga_silu_mul_quantize_mxfp8(const void* x_w1_bf16, const void* x_w3_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream);
 
 /* route (moe_routing.py:109-122) for one device group: top-k (descending, lower index first among equals), weights =
  * softmax(top values), per-expert counts padded to 256 -> off (E+1), dest_row[j] = off[e_j] + stable rank of assignment j among

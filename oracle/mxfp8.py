@@ -47,6 +47,13 @@ def quantize_mxfp8(x: np.ndarray):
   xs = np.clip(xb * qscale, -448.0, 448.0)
   return float_to_e4m3(xs).reshape(*batch, K), e8
 
+def silu_mul_quantize_mxfp8(x_w1: np.ndarray, x_w3: np.ndarray):
+  """extra/llama_kernels/fused_silu_mul_quantize_mxfp8/__init__.py:33-44: act = w1 * (1 / (1 + exp2(-w1 * log2 e))) * w3 in float32, then
+  quantize_mxfp8 of act."""
+  w1, w3 = np.asarray(x_w1, dtype=np.float32), np.asarray(x_w3, dtype=np.float32)
+  with np.errstate(over="ignore"): sig = (np.float32(1.0) / (np.float32(1.0) + np.exp2(w1 * np.float32(-1.4426950408889634)))).astype(np.float32)
+  return quantize_mxfp8((w1 * sig * w3).astype(np.float32))
+
 def block_scale(e8: np.ndarray) -> np.ndarray:
   """cdna_asm_gemm.py:165-173: dequant scale 2^(e8-127) broadcast to element shape."""
   return np.repeat(np.exp2(e8.astype(np.float32) - 127.0).astype(np.float32), 32, axis=-1)

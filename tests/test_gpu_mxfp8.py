@@ -21,6 +21,30 @@ def test_quantize_mxfp8_bit_exact(gpu):
   rq2, re82 = omx.quantize_mxfp8(moe.from_bf16_bits(xb))
   np.testing.assert_array_equal(e82.numpy(), re82); np.testing.assert_array_equal(q2.numpy(), rq2)
 
+def test_fused_silu_mul_quantize_mxfp8(gpu):
+  """silu(x_w1) * x_w3 quantized without an intermediate tensor (extra/llama_kernels/fused_silu_mul_quantize_mxfp8).  The product is
+  formed in float32 from exp2; where the device's exp2 differs from numpy's in the last ulp an E4M3 code may land on the other side of
+  a rounding boundary, so the bar is: block exponents equal, codes equal except for a < 1e-4 fraction, and those within one code."""
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(4)
+  w1 = (rng.standard_normal((256, 768)) * 3).astype(np.float32); w3 = rng.standard_normal((256, 768)).astype(np.float32)
+  w1[0, :32] = 0; w1[1, :32] = -40.0; w1[2, :32] = 30.0
+  b1, b3 = moe.to_bf16_bits(w1), moe.to_bf16_bits(w3)
+  q, e8, packed = moe.fused_silu_mul_quantize_mxfp8(gpu.Buffer.from_numpy(b1), gpu.Buffer.from_numpy(b3))
+  rq, re8 = omx.silu_mul_quantize_mxfp8(moe.from_bf16_bits(b1), moe.from_bf16_bits(b3))
+  ge8, gq = e8.numpy(), q.numpy()
+  assert np.mean(ge8 != re8) < 1e-4 and np.abs(ge8.astype(int) - re8.astype(int)).max() <= 1
+  same_block = np.repeat(ge8 == re8, 32, axis=-1)
+  diff = (gq != rq) & same_block
+  assert diff.mean() < 1e-4
+  mag = lambda c: (c & 0x7F).astype(int)
+  assert (np.abs(mag(gq[diff]) - mag(rq[diff])) <= 1).all()
+  np.testing.assert_array_equal(packed.numpy(), omx.mx_pack(ge8))
+  # against the unfused chain on the GPU itself (float32 product quantized by tga_quantize_mxfp8): same bar
+  act = moe.from_bf16_bits(b1); act = (act * (1.0 / (1.0 + np.exp2(act * np.float32(-1.4426950408889634)))) * moe.from_bf16_bits(b3)).astype(np.float32)
+  q2, e82, _ = moe.quantize_mxfp8(gpu.Buffer.from_numpy(act))
+  assert np.mean(q2.numpy() != gq) < 1e-4
+
 @pytest.mark.parametrize("T,E,k", [(300, 16, 4), (4096, 128, 8), (7, 5, 5)])
 def test_route_dispatch_combine(gpu, T, E, k):
   from tinygrad_amd import moe

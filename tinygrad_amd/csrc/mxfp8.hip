@@ -36,19 +36,28 @@ __device__ __forceinline__ uint32_t f_to_e4m3(float x) {
 // ------------------------------------------------------------------------------------------------ quantize_mxfp8
 // One thread per 32-element block: amax, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254), q = e4m3(clamp(x * 2^(127-e8), +-448)).
 // Also writes the packed scales of mx_pack: packed[k/128][row] = 4 consecutive e8 bytes (little-endian).
-template <bool BF16>
-__global__ __launch_bounds__(256) void quantize_mxfp8_kernel(const void* __restrict__ x, long long rows, int K, uint8_t* __restrict__ q,
+// MODE 0: x float32; 1: x bf16; 2: fused SwiGLU producer, value = w1 * sigmoid(w1) * w3 in float32 from two bf16 tensors x (= x_w1)
+// and x2 (= x_w3), sigmoid as 1 / (1 + exp2(-w1 * log2(e)))  (extra/llama_kernels/fused_silu_mul_quantize_mxfp8/__init__.py:33-36)
+template <int MODE>
+__global__ __launch_bounds__(256) void quantize_mxfp8_kernel(const void* __restrict__ x, const void* __restrict__ x2, long long rows, int K, uint8_t* __restrict__ q,
                                                              uint8_t* __restrict__ e8, uint8_t* __restrict__ packed) {
   const long long nb = rows * (K / 32);
   for (long long b = (long long)blockIdx.x * 256 + threadIdx.x; b < nb; b += (long long)gridDim.x * 256) {
     const long long row = b / (K / 32); const int kb = (int)(b % (K / 32));
     float v[32]; float amax = 0.f;
-    if (BF16) {
-      const u32x4* p = (const u32x4*)((const uint16_t*)x + row * K + kb * 32);
+    auto load_bf16 = [&](const void* src, float* o) {
+      const u32x4* p = (const u32x4*)((const uint16_t*)src + row * K + kb * 32);
 #pragma unroll
       for (int i = 0; i < 4; i++) { const u32x4 w = p[i];
-        v[8*i] = bf16_to_f(w.x & 0xFFFF); v[8*i+1] = bf16_to_f(w.x >> 16); v[8*i+2] = bf16_to_f(w.y & 0xFFFF); v[8*i+3] = bf16_to_f(w.y >> 16);
-        v[8*i+4] = bf16_to_f(w.z & 0xFFFF); v[8*i+5] = bf16_to_f(w.z >> 16); v[8*i+6] = bf16_to_f(w.w & 0xFFFF); v[8*i+7] = bf16_to_f(w.w >> 16); }
+        o[8*i] = bf16_to_f(w.x & 0xFFFF); o[8*i+1] = bf16_to_f(w.x >> 16); o[8*i+2] = bf16_to_f(w.y & 0xFFFF); o[8*i+3] = bf16_to_f(w.y >> 16);
+        o[8*i+4] = bf16_to_f(w.z & 0xFFFF); o[8*i+5] = bf16_to_f(w.z >> 16); o[8*i+6] = bf16_to_f(w.w & 0xFFFF); o[8*i+7] = bf16_to_f(w.w >> 16); }
+    };
+    if constexpr (MODE == 1) load_bf16(x, v);
+    else if constexpr (MODE == 2) {
+      float u[32];
+      load_bf16(x, v); load_bf16(x2, u);
+#pragma unroll
+      for (int i = 0; i < 32; i++) { const float sig = 1.0f / (1.0f + exp2f(v[i] * -1.4426950408889634f)); v[i] = v[i] * sig * u[i]; }
     } else {
       const f32x4* p = (const f32x4*)((const float*)x + row * K + kb * 32);
 #pragma unroll
@@ -376,8 +385,20 @@ int tga_quantize_mxfp8(const void* x, int x_is_bf16, int64_t rows, int64_t K, vo
   if (rows == 0) return 0;
   const long long nb = rows * (K / 32);
   const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
-  if (x_is_bf16) quantize_mxfp8_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>(x, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
-  else quantize_mxfp8_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>(x, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
+  if (x_is_bf16) quantize_mxfp8_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(x, nullptr, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
+  else quantize_mxfp8_kernel<0><<<grid, 256, 0, (hipStream_t)stream>>>(x, nullptr, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_silu_mul_quantize_mxfp8(const void* x_w1_bf16, const void* x_w3_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream) {
+  TGA_REQUIRE(x_w1_bf16 && x_w3_bf16 && q && e8, "tga_silu_mul_quantize_mxfp8: null pointer");
+  TGA_REQUIRE(rows >= 0 && K > 0 && K % 32 == 0, "tga_silu_mul_quantize_mxfp8: K=%lld must be a positive multiple of 32", (long long)K);
+  TGA_REQUIRE(!packed || K % 128 == 0, "tga_silu_mul_quantize_mxfp8: packed scales need K %% 128 == 0");
+  if (rows == 0) return 0;
+  const long long nb = rows * (K / 32);
+  const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
+  quantize_mxfp8_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(x_w1_bf16, x_w3_bf16, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
   TGA_LAUNCH_CHECK();
   return 0;
 }

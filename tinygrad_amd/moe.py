@@ -63,6 +63,16 @@ def quantize_mxfp8(x: Buffer, stream=None):
   rt.check(rt.lib().tga_quantize_mxfp8(x.ptr, int(x.dtype == np.uint16), rows, K, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
   return q, e8, packed
 
+def fused_silu_mul_quantize_mxfp8(x_w1: Buffer, x_w3: Buffer, stream=None):
+  """extra/llama_kernels/fused_silu_mul_quantize_mxfp8/__init__.py:91-104: (rows, K) bf16 bits x 2 -> MXFP8 of silu(x_w1) * x_w3,
+  same outputs as quantize_mxfp8 (the SwiGLU product never goes through memory)."""
+  assert x_w1.shape == x_w3.shape and x_w1.dtype == np.uint16 and x_w3.dtype == np.uint16, f"{x_w1.shape} != {x_w3.shape}"
+  rows, K = x_w1.shape
+  q, e8 = Buffer((rows, K), np.uint8), Buffer((rows, K // 32), np.uint8)
+  packed = Buffer((K // 128, rows), np.uint32) if K % 128 == 0 else None
+  rt.check(rt.lib().tga_silu_mul_quantize_mxfp8(x_w1.ptr, x_w3.ptr, rows, K, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
+  return q, e8, packed
+
 def grouped_mx_gemm(x: Buffer, w: tuple[Buffer, Buffer], expert_off: Buffer, stream=None, out: Buffer | None = None) -> Buffer:
   """moe_gemm.py:112-134 with pre-quantized weights w = (w_q (E,N,K) e4m3 bits, w_e8 (E,N,K/32)): quantizes x (M,K) bf16 to MXFP8 and
   runs the grouped GEMM; returns (M, N) bf16 bits."""
