@@ -138,11 +138,12 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
                          int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
-/* tga_attention_decode with the full-width q / k RMSNorm of model.py:169 (attn_q_norm over all n_heads * head_dim values, attn_k_norm
- * over all n_kv_heads * head_dim) applied before RoPE: q_norm_weight [n_heads * head_dim], k_norm_weight [n_kv_heads * head_dim]
- * float32, both NULL for no norm; q and k must be 16-byte aligned when the norm is on. */
+/* tga_attention_decode with the q / k RMSNorm of the reference applied before RoPE (attn_q_norm / attn_k_norm, float32 weights, both
+ * NULL for no norm).  norm_per_head = 0: one norm over all n_heads * head_dim (n_kv_heads * head_dim) values, weights of that length
+ * (model.py:169, OLMoE); norm_per_head = 1: one norm per head over its head_dim values, weights of head_dim values shared by all heads
+ * (model.py:180, Qwen3).  q and k must be 16-byte aligned when the norm is on. */
 int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
-                                void* cache_k, void* cache_v, float* partials, const void* state,
+                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
 /* argmax(-1) with first-max tie rule (tinygrad/mixin/op.py:866-891) + the bookkeeping of Transformer.generate (model.py:475-484):

@@ -57,7 +57,10 @@ class Model:
       q, k = self._lin(p + "attn_q.weight", n), self._lin(p + "attn_k.weight", n)
       if c.get("qk_norm", 0) and c["qk_norm"] != hd:                        # model.py:169: full-width q/k norm before the head split
         q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
-      q, k = apply_rope(q.reshape(H, hd), self.fc[pos]), apply_rope(k.reshape(KV, hd), self.fc[pos])
+      q, k = q.reshape(H, hd), k.reshape(KV, hd)
+      if c.get("qk_norm", 0) == hd:                                         # model.py:180: per-head q/k norm after the head split
+        q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
+      q, k = apply_rope(q, self.fc[pos]), apply_rope(k, self.fc[pos])
       v = self._lin(p + "attn_v.weight", n).reshape(KV, hd)
       self.ck[i, :, pos], self.cv[i, :, pos] = k.astype(self.kv_dtype), v.astype(self.kv_dtype)
       K = np.repeat(self.ck[i, :, :pos + 1].astype(np.float32), H // KV, axis=0)      # (H, T, hd)  GQA repeat_interleave

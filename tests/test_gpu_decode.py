@@ -80,8 +80,8 @@ def test_one_launch_blocks_equal_per_op_path(gpu, cfg, ltype):
   assert ol.rel_err(ka[:, :78], kb[:, :78]) <= 2e-3
   assert not a.s.sync.numpy().any()                                # barrier counters back at zero, no error flag
 
-@pytest.mark.parametrize("H,KV,hd,normed", [(8, 2, 128, False), (4, 4, 64, True), (12, 2, 128, True), (4, 2, 256, False), (16, 16, 128, True)],
-                         ids=["gqa4-hd128", "mha-hd64-qknorm", "gqa6-hd128-qknorm", "gqa2-hd256", "mha16-hd128-qknorm"])
+@pytest.mark.parametrize("H,KV,hd,normed", [(8, 2, 128, 0), (4, 4, 64, 1), (12, 2, 128, 1), (4, 2, 256, 0), (16, 16, 128, 1), (16, 8, 128, 2), (6, 2, 64, 2)],
+                         ids=["gqa4-hd128", "mha-hd64-qknorm", "gqa6-hd128-qknorm", "gqa2-hd256", "mha16-hd128-qknorm", "gqa2-hd128-headnorm", "gqa3-hd64-headnorm"])
 def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
   """tga_attention_decode(_normed) alone: (full-width q/k RMSNorm,) RoPE + fp16 KV append + GQA softmax attention at several positions."""
   from tinygrad_amd.llm import precompute_freqs_cis
@@ -92,7 +92,8 @@ def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
   part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2) + KV,), np.float32).zero_()
   ropeb = gpu.Buffer.from_numpy(rope)
   out = gpu.Buffer((H * hd,), np.float32)
-  qw, kw = (rng.standard_normal(n).astype(np.float32) for n in (H * hd, KV * hd))
+  # normed: 0 none, 1 full-width q/k norm (weights over all heads), 2 per-head norm (weights of head_dim values)
+  qw, kw = (rng.standard_normal(n).astype(np.float32) for n in ((H * hd, KV * hd) if normed != 2 else (hd, hd)))
   qwb, kwb = gpu.Buffer.from_numpy(qw), gpu.Buffer.from_numpy(kw)
   rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)
   for pos in range(0, 140):
@@ -100,9 +101,10 @@ def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
     st = np.zeros(16, np.int32); st[0] = pos
     qb, kb, vb, stb = (gpu.Buffer.from_numpy(t) for t in (q, k, v, st))       # keep the device buffers alive across the launch
     if normed:
-      gpu.check(gpu.lib().tga_attention_decode_normed(qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, 1e-5, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx,
-                                                      ropeb.ptr, None, out.ptr, 0, None))
-      q, k = ollm.rmsnorm(q, qw, 1e-5), ollm.rmsnorm(k, kw, 1e-5)
+      gpu.check(gpu.lib().tga_attention_decode_normed(qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, 1e-5, int(normed == 2), ck.ptr, cv.ptr, part.ptr, stb.ptr,
+                                                      H, KV, hd, ctx, ropeb.ptr, None, out.ptr, 0, None))
+      if normed == 2: q, k = ollm.rmsnorm(q.reshape(H, hd), qw, 1e-5).reshape(-1), ollm.rmsnorm(k.reshape(KV, hd), kw, 1e-5).reshape(-1)
+      else: q, k = ollm.rmsnorm(q, qw, 1e-5), ollm.rmsnorm(k, kw, 1e-5)
     else:
       gpu.check(gpu.lib().tga_attention_decode(qb.ptr, kb.ptr, vb.ptr, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None, out.ptr, 0, None))
     gpu.synchronize()

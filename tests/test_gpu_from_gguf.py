@@ -90,3 +90,40 @@ def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path):
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
 
+def test_from_gguf_qwen3_shape_per_head_qk_norm(gpu, tmp_path):
+  """A Qwen3-shaped file: n_heads * head_dim != embedding_length (key_length given), per-head attn_q_norm / attn_k_norm of head_dim
+  weights (model.py:180), Q8_0 matrices, tied embeddings."""
+  from tinygrad_amd.llm import Transformer
+  from tinygrad_amd.gguf import gguf_write
+  rng = np.random.default_rng(21)
+  dim, hidden, H, KV, hd, L, vocab = 256, 512, 4, 2, 128, 2, 512
+  def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
+  q8 = lambda name, rows, cols, amp=1.0: (name, (rows, cols), 8, og.quantize_q8_0(lin(rows, cols) * amp))
+  f32 = lambda name, n: (name, (n,), 0, (1 + 0.2 * rng.standard_normal(n)).astype(np.float32))
+  tensors = [q8("token_embd.weight", vocab, dim, 16.0)]
+  for i in range(L):
+    p = f"blk.{i}."
+    tensors += [f32(p + "attn_norm.weight", dim), q8(p + "attn_q.weight", H * hd, dim), q8(p + "attn_k.weight", KV * hd, dim), q8(p + "attn_v.weight", KV * hd, dim),
+                f32(p + "attn_q_norm.weight", hd), f32(p + "attn_k_norm.weight", hd), q8(p + "attn_output.weight", dim, H * hd),
+                f32(p + "ffn_norm.weight", dim), q8(p + "ffn_gate.weight", hidden, dim), q8(p + "ffn_up.weight", hidden, dim), q8(p + "ffn_down.weight", dim, hidden)]
+  tensors.append(f32("output_norm.weight", dim))
+  kvs = [("general.architecture", "qwen3"), ("qwen3.context_length", 96), ("qwen3.attention.head_count", H), ("qwen3.attention.head_count_kv", KV),
+         ("qwen3.attention.key_length", hd), ("qwen3.block_count", L), ("qwen3.embedding_length", dim), ("qwen3.feed_forward_length", hidden),
+         ("qwen3.attention.layer_norm_rms_epsilon", 1e-6), ("qwen3.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(vocab)])]
+  path = tmp_path / "qwen3.gguf"
+  raw = gguf_write(path, kvs, tensors)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  assert model.config.qk_norm == hd == model.config.head_dim and model.layer_table is None
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  prompt = [9, 100, 321, 5]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3
+

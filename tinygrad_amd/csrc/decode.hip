@@ -91,7 +91,8 @@ struct AttnArgs {
   float scale;
   _Float16* out16; float* out32;                       // attention output [n_heads*hd]
   int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
-  const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights over the whole q / k vectors
+  const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights: over the whole q / k vectors, or
+  int norm_per_head;                                           // per head (weights of head_dim values shared by all heads)
 };
 
 __device__ __forceinline__ u32x4 pack8_f16(const float* c) {
@@ -165,14 +166,21 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
     }
   }
   float qscale = 1.f, kscale = 1.f;
-  if (a.q_norm) {
+  const bool per_head = a.q_norm && a.norm_per_head;
+  if (a.q_norm && !per_head) {
     float sq, sk;
     block_sumsq2(a.q, a.n_heads * HD, a.k, a.n_kv * HD, red, sq, sk);
     qscale = 1.0f / sqrtf(sq / (float)(a.n_heads * HD) + a.norm_eps);
     kscale = 1.0f / sqrtf(sk / (float)(a.n_kv * HD) + a.norm_eps);
   }
-  auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[i] : a.q[i]; };
-  auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[i] : a.k[i]; };
+  if (per_head) {                                       // every wave sums this kv head's key for itself
+    float sk = 0.f;
+    for (int i = lane; i < HD; i += 64) { const float v = a.k[kvh * HD + i]; sk += v * v; }
+    kscale = 1.0f / sqrtf(wave_sum(sk) / (float)HD + a.norm_eps);
+  }
+  // normalised values: weight index = position in the whole vector, or inside the head for the per-head norm
+  auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[per_head ? i % HD : i] : a.q[i]; };
+  auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[per_head ? i % HD : i] : a.k[i]; };
   for (int i = tid; i < half; i += 256) {
     const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
     const float x1 = kval(kvh * HD + i), x2 = kval(kvh * HD + half + i);
@@ -194,6 +202,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
   for (int h0 = 0; h0 < group; h0 += 4) {
     if (h0 + wave < group) {                            // wave w rotates the query of head h0 + w
       const int head = kvh * group + h0 + wave;
+      if (per_head) {
+        float sq = 0.f;
+        for (int i = lane; i < HD; i += 64) { const float v = a.q[head * HD + i]; sq += v * v; }
+        qscale = 1.0f / sqrtf(wave_sum(sq) / (float)HD + a.norm_eps);
+      }
       for (int i = lane; i < half; i += 64) {
         const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
         const float x1 = qval(head * HD + i), x2 = qval(head * HD + half + i);
@@ -404,7 +417,7 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
 }
 
 int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
-                                void* cache_k, void* cache_v, float* partials, const void* state,
+                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
@@ -418,7 +431,7 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
   a.stage_fmt = 0; a.stage_nu = 0;
-  a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps;
+  a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps; a.norm_per_head = norm_per_head;
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
   const dim3 grid(n_kv_heads, a.nsplit);
   hipStream_t s = (hipStream_t)stream;
@@ -431,7 +444,7 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
 
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
                          int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
-  return tga_attention_decode_normed(q, k, v, nullptr, nullptr, 0.f, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx, rope_table,
+  return tga_attention_decode_normed(q, k, v, nullptr, nullptr, 0.f, 0, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx, rope_table,
                                      out_f16, out_f32, stage_type, stream);
 }
 

@@ -28,7 +28,7 @@ class TransformerConfig:
   head_dim: int
   rope_theta: float
   max_context: int
-  qk_norm: int = 0                 # width of attn_q_norm / attn_k_norm (OLMoE: the full projection width, model.py:169)
+  qk_norm: int = 0                 # width of attn_q_norm / attn_k_norm (OLMoE: the full projection width, model.py:169; Qwen3: head_dim, :180)
   num_experts: int = 0
   num_experts_per_tok: int = 0
   norm_topk_prob: bool = False
@@ -162,10 +162,9 @@ class TransformerBlock:
           while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
           qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream)
           i = j
-    if c.qk_norm: assert c.qk_norm != c.head_dim, "per-head qk norm is not built"
-    # full-width q/k RMSNorm before the head split (model.py:169) inside the attention launch
+    # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
     rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
-                                           self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
+                                           int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
                                            s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if st else 0, stream))
     qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150

@@ -46,7 +46,7 @@ def _declare(lib):
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
-    "tga_attention_decode_normed": [vp, vp, vp, vp, vp, ctypes.c_float, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
+    "tga_attention_decode_normed": [vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
     "tga_decode_layers": [vp, i, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, ctypes.c_float, vp],
     "tga_decode_layers_trace": [vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
