@@ -204,8 +204,9 @@ static int launch_fast(QArgs a, hipStream_t s) {
   constexpr int RS = (EPI == 2) ? 1 : R;
   const long long ngroups = (a.ntot + RS - 1) / RS;
   const size_t lds = (size_t)a.nu * (F::UW / 2 + 4) * 4;
-  // resident row teams per CU: 16 waves (<= 128 VGPRs) unless the staged activations in LDS (160 KB per CU) allow fewer
-  int wg_per_cu = 16 / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;
+  // row teams per CU: 8 waves (two 4-wave workgroups), fewer when the staged activations in LDS (160 KB per CU) say so.  Measured on
+  // the 8B decode step: 2 workgroups per CU 509 tok/s, 4 (all 16 wave slots) 499, 1 466 - more workgroups only add staging prologues.
+  int wg_per_cu = (a.sel ? 16 : 8) / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;   // (expert jobs share the grid: all 16 wave slots there)
   const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
   constexpr int TPW = WR * (H ? 2 : 1);                           // row teams per workgroup
   long long max_teams = (long long)fast_cu_count() * wg_per_cu * TPW;
