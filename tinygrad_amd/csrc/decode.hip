@@ -3,6 +3,7 @@
 // They restate, for one token, what tinygrad/llm/model.py:167-204 (_attention), :144-151 (block), :358-364 (forward) compute.
 // The position and token live in device memory so that one captured launch sequence can be replayed for every token
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
+#include <type_traits>
 #include "qfmt.h"
 #include "decode.h"
 #include "coherent.h"
@@ -305,21 +306,29 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
     for (int sp = lane; sp < ns; sp += 64) sw[gh * a.nsplit + sp] = __expf(sw[gh * a.nsplit + sp] - m) / l;
   }
   __syncthreads();
-  constexpr int SC = 16;
-  for (int idx = tid; idx < group * HD; idx += 256) {
-    const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
-    const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
-    float o = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += SC) {
-      float v[SC];
+  // weighted sum over the splits, one output at a time with SC split loads in flight; SC follows the number of splits (a fixed large
+  // batch would request mostly clamped duplicates at short contexts; both outputs of a thread in one batch measured slower)
+  auto merge_out = [&](auto tag) {
+    constexpr int SC = decltype(tag)::value;
+    for (int idx = tid; idx < group * HD; idx += 256) {
+      const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
+      const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
+      float o = 0.f;
+      for (int s0 = 0; s0 < ns; s0 += SC) {
+        float v[SC];
 #pragma unroll
-      for (int j = 0; j < SC; j++) v[j] = cld(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
+        for (int j = 0; j < SC; j++) v[j] = cld(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
 #pragma unroll
-      for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
+        for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
+      }
+      if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, head * HD + d, a.stage_nu) : head * HD + d] = (_Float16)o;
+      if (a.out32) a.out32[head * HD + d] = o;
     }
-    if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, head * HD + d, a.stage_nu) : head * HD + d] = (_Float16)o;
-    if (a.out32) a.out32[head * HD + d] = o;
-  }
+  };
+  if (ns <= 4) merge_out(std::integral_constant<int, 4>{});
+  else if (ns <= 8) merge_out(std::integral_constant<int, 8>{});
+  else if (ns <= 16) merge_out(std::integral_constant<int, 16>{});
+  else merge_out(std::integral_constant<int, 24>{});
 }
 
 // ---------------------------------------------------------------------------------------------- argmax + token bookkeeping

@@ -1,6 +1,10 @@
 // M = 1 dequant-GEMV fast path (decode): see qgemv.hip for the overall design.
 #include "qfmt.h"
 
+#ifndef QG1_DEPTH
+#define QG1_DEPTH 2        // row groups in flight per lane (loads of the next DEPTH - 1 groups are outstanding while one is multiplied); 3 measured slower (8B decode 496 vs 519 tok/s)
+#endif
+
 // ------------------------------------------------------------------------------------------------ M = 1 fast path
 // One activation row: each lane keeps the activations of ITS unit in registers for the whole kernel (no LDS traffic in the
 // loop).  A workgroup is WR x WK waves: the WK waves of a row team split K (wave wk owns units 64wk .. 64wk+63) and their
@@ -105,7 +109,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
         }
       }
     };
-    Raw b0[R], b1[R];
+    Raw b[QG1_DEPTH][R];                                      // ring of row groups in flight
     if (!staged && a.x_staged) {
       // producer-staged activations: XV coalesced 16-byte loads per lane, issued ahead of the first weight loads (loads return in
       // issue order, so the small activation reads must not queue behind the weight stream)
@@ -114,10 +118,10 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
 #pragma unroll
         for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
       }
-      if (cnt) issue(b0, lo);
+      if (cnt) issue(b[0], lo);
       F::cfromx(xv, cv);
       staged = true;
-    } else if (cnt) issue(b0, lo);
+    } else if (cnt) issue(b[0], lo);
     if (!staged) {
       // activations: coalesced global -> LDS (natural order, padded unit stride) -> this lane's unit -> staged registers
       // Loads of up to four (two) loop iterations are issued as one batch: a load per iteration would cost a memory round trip each.
@@ -178,15 +182,21 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
       }
       staged = true;
     }
+    // groups lo + RS .. lo + (DEPTH - 2) RS follow the first one (clamped past the end: surplus results are never used)
+    if (cnt) {
+#pragma unroll
+      for (int d = 1; d < QG1_DEPTH - 1; d++) issue(b[d], lo + (long long)d * RS);
+    }
     long long row = lo;
-    for (long long g = 0; g < cnt; g += 2) {
-      issue(b1, row + RS);                                       // prefetch (clamped past the end)
-      finish_group(b0, row);
-      row += RS;
-      if (g + 1 >= cnt) break;
-      issue(b0, row + RS);
-      finish_group(b1, row);
-      row += RS;
+    for (long long g = 0; g < cnt; g += QG1_DEPTH) {
+#pragma unroll
+      for (int d = 0; d < QG1_DEPTH; d++) {
+        if (g + d < cnt) {
+          issue(b[(d + QG1_DEPTH - 1) % QG1_DEPTH], row + (long long)(QG1_DEPTH - 1) * RS);   // the slot freed by the previous group
+          finish_group(b[d], row);
+          row += RS;
+        }
+      }
     }
   }
 }
@@ -229,13 +239,14 @@ static int launch_fast(QArgs a, hipStream_t s) {
   return 0;
 }
 
+static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
 template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
   if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice.
   // Measured per format at 14336 x 4096 and 4096 x 14336: two rows win for Q4_0, MXFP4, Q4_K (14.3 -> 11.4 us), Q5_K (18.1 -> 15.1 us)
   // and slightly for Q6_K; Q8_0 pairs (68-byte units) are no faster with two.
-  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K) && a.ntot >= (long long)fast_cu_count() * 16 * 2 / WK;
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K) && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu() / WK;
   if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
   return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);
 }
