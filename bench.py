@@ -4,14 +4,15 @@
 A step is one decoded token.  Random-init weights are written on the GPU as GGUF blocks (Q4_0 linears and embedding, Q6_K
 lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the model itself, then --warmup + --steps tokens
 are decoded greedily, one captured launch sequence per token with a host sync per token (as the reference's generate loop does).
-Prints ONE JSON line: tok/s, the roofline of the dominant kernel (the one-launch kernel that runs all 32 blocks of a token:
-every Q4_0 dequant-GEMV, RMSNorm, RoPE + KV append + attention) from HIP-event timings taken live, the same figures for the
-per-op dequant-GEMV kernels on the same weights, and a CPU baseline (C restatement of the reference arithmetic on a bounded
-sample of the same weights)."""
+Prints ONE JSON line: tok/s, the roofline of the dominant kernel from HIP-event timings taken live, the same figures for the other
+kernels of a block, and a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the same weights).
+Default path: one launch per op (five per block); the dominant kernel is then the fused ffn_gate + ffn_up dequant-GEMV with the
+ffn_norm folded in.  --fused: all 32 blocks of a token in one persistent launch (tga_decode_layers), which is then the kernel reported."""
 import argparse, json, os, sys, time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+GATE_UP_TRAFFIC_BYTES = 66621000   # 66 493 440 B fetched + 127 898 B written per launch (counter runs summarised in profiles/qgemv1_gate_up_hbm_traffic.md)
 
 def cpu_baseline(model, cfg, seconds_budget=20.0):
   """Times oracle/c (scalar C restatement of dequant + fp32-accumulate matmul, model-path numerics) on the GPU box's host
@@ -58,7 +59,8 @@ def main():
   ap.add_argument("--layers", type=int, default=32, help="reduce only for smoke runs; the reported config then says so")
   ap.add_argument("--no-cpu", action="store_true")
   ap.add_argument("--no-graph", action="store_true", help="eager launches instead of graph replay (for kernel-trace profiling)")
-  ap.add_argument("--per-op", action="store_true", help="one launch per op instead of the one-launch block kernel")
+  ap.add_argument("--fused", action="store_true", help="all blocks of a token in one persistent launch instead of one launch per op")
+  ap.add_argument("--per-op", action="store_true", help="(the default; kept so that older command lines still run)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py: this build measures one GPU only (no collectives, no sharding in this run); use --gpus 1", file=sys.stderr)
@@ -72,7 +74,7 @@ def main():
   max_ctx = ((args.prefill + max_new + 63) // 64) * 64
   c = TransformerConfig(max_context=max_ctx, **cfg)
   sd = synth_state(c, seed=1003)
-  model = Transformer(c, sd, max_new=max_new, fused=not args.per_op)
+  model = Transformer(c, sd, max_new=max_new, fused=args.fused)
   rt.synchronize()
 
   rng = np.random.default_rng(1003)
@@ -115,38 +117,35 @@ def main():
       phase = {"qkv_after_staging_us": round(span(0, 1), 2),
                "attention_us": round(span(2, 3), 2), "attn_output_us": round(span(4, 5), 2), "gate_up_us": round(span(6, 7), 2), "down_us": round(span(8, 9), 2),
                "block_us": round(float(np.median(np.diff(T[0, :, 0])) * 0.01), 2)}
-  # ---- the per-op dequant-GEMV kernels on the same weights: HIP events around each launch of a few eager per-op steps ----
+  # ---- the per-op kernels on the same weights: HIP events around each launch of a few eager steps (the launch sequence of
+  #      TransformerBlock.__call__: q/k/v with attn_norm folded in, attention, attn_output + residual, gate/up with ffn_norm folded in +
+  #      SwiGLU, down + residual) ----
   from tinygrad_amd.nn import qlinear_multi
-  durs = {"gate_up": [], "down": [], "qkv": [], "attn_output": []}
+  durs = {"gate_up": [], "down": [], "qkv": [], "attn_output": [], "attention": []}
   for _ in range(3):
     rt.check(L.tga_embed_row(model.token_embd.ptr, model.embd_type, c.dim, model.s.state.ptr, model.s.x.ptr, st))
     per = {k: [] for k in durs}
+    def timed(key, fn):
+      e = (rt.Event(), rt.Event()); e[0].record(st); fn(); e[1].record(st); per[key].append(e)
     for b in model.blk:
       s = model.s
-      rt.check(L.tga_rmsnorm(s.x.ptr, b.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, b.attn_q.ggml_type if b.staged else 0, st))
-      e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.xn, [s.q, s.k, s.v], stream=st, x_staged=b.staged)
-      e[1].record(st); per["qkv"].append(e)
-      rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                      c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if b.staged else 0, st))
-      e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.staged)
-      e[1].record(st); per["attn_output"].append(e)
-      rt.check(L.tga_rmsnorm(s.x.ptr, b.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, b.ffn_gate.ggml_type if b.staged else 0, st))
-      e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.ffn_gate, b.ffn_up], s.xn, [s.act], epilogue=2, stream=st, x_staged=b.staged, stage_out_for=b.ffn_down if b.staged else None)
-      e[1].record(st); per["gate_up"].append(e)
-      e = (rt.Event(), rt.Event()); e[0].record(st)
-      qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.staged)
-      e[1].record(st); per["down"].append(e)
+      sg = b.staged
+      timed("qkv", lambda: qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.x, [s.q, s.k, s.v], stream=st, norm=(b.attn_norm, c.norm_eps)))
+      timed("attention", lambda: rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
+                                          c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if sg else 0, st)))
+      timed("attn_output", lambda: qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=sg))
+      timed("gate_up", lambda: qlinear_multi([b.ffn_gate, b.ffn_up], s.x, [s.act], epilogue=2, stream=st, norm=(b.ffn_norm, c.norm_eps), stage_out_for=b.ffn_down if sg else None))
+      timed("down", lambda: qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=sg))
     rt.check(L.tga_advance_prompt(model.s.state.ptr, model.s.prompt.ptr, st))
     model.stream.synchronize()
     for k in durs: durs[k] += [a.elapsed_ms(b_) * 1e3 for a, b_ in per[k]]
   b0 = model.blk[0]
-  alg = {"gate_up": b0.ffn_gate.nbytes + b0.ffn_up.nbytes + c.dim * 2 + c.hidden_dim * 2,
+  ctx_now = args.prefill + args.warmup + args.steps
+  alg = {"gate_up": b0.ffn_gate.nbytes + b0.ffn_up.nbytes + c.dim * 8 + c.hidden_dim * 2,            # weights + fp32 row + norm weight + fp16 out
          "down": b0.ffn_down.nbytes + c.hidden_dim * 2 + c.dim * 8,
-         "qkv": b0.attn_q.nbytes + b0.attn_k.nbytes + b0.attn_v.nbytes + c.dim * 2 + (c.n_heads + 2 * c.n_kv_heads) * c.head_dim * 4,
-         "attn_output": b0.attn_output.nbytes + c.dim * 2 + c.dim * 8}
+         "qkv": b0.attn_q.nbytes + b0.attn_k.nbytes + b0.attn_v.nbytes + c.dim * 8 + (c.n_heads + 2 * c.n_kv_heads) * c.head_dim * 4,
+         "attn_output": b0.attn_output.nbytes + c.dim * 2 + c.dim * 8,
+         "attention": 2 * c.n_kv_heads * c.head_dim * ctx_now * 2}                                     # fp16 K and V rows read at this context
   kern = {k: {"avg_us": round(float(np.mean(v)), 3), "alg_bytes": int(alg[k]), "GBps": round(alg[k] / np.mean(v) / 1e3, 1),
               "frac_hbm": round(alg[k] / np.mean(v) / 1e3 / HBM_PEAK_GBS, 4)} for k, v in durs.items()}
   wbytes = model.weight_bytes_per_token()
@@ -164,7 +163,6 @@ def main():
   if fused_us:
     # algorithmic bytes of one launch: the seven Q4_0 matrices of every block + the fp16 K/V rows read at this context length
     blk_w = sum(l.nbytes for b in model.blk for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down))
-    ctx_now = args.prefill + args.warmup + args.steps
     alg_f = blk_w + 2 * c.num_blocks * c.n_kv_heads * c.head_dim * ctx_now * 2
     avg = float(np.mean(fused_us[1:]))
     out["roofline"] = {"bound": "hbm", "kernel": f"decode_layers_kernel<Q4_0 pair> (all {c.num_blocks} blocks of one token in one persistent launch: 4 dequant-GEMV phases + attention per block)",
@@ -179,9 +177,16 @@ def main():
       out["roofline"]["down_phase_GBps"] = round(alg["down"] / phase["down_us"] / 1e3, 1)
   else:
     dom = kern["gate_up"]
-    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU> (fused ffn_gate+ffn_up, 2x14336x4096)",
-                       "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"], "traffic": None,
-                       "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"], "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
+    per_block = sum(v["avg_us"] for v in kern.values())
+    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
+                                                 "one of five launches per block)",
+                       "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
+                       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py (counters scaled by a
+                       # 1 GiB copy kernel: x2.0000 and x1.0000)
+                       "traffic": GATE_UP_TRAFFIC_BYTES if c.num_blocks == 32 else None,
+                       "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"],
+                       "share_of_block_time": round(dom["avg_us"] / per_block, 3),
+                       "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
   if not args.no_cpu:
     out["cpu_baseline"] = cpu_baseline(model, cfg)
   print(json.dumps(out))

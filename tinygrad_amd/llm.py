@@ -215,7 +215,9 @@ class _Shared:
     self.out_tokens = Buffer((max(1, max_new),), np.int32).zero_()
 
 class Transformer:
-  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096, fused: bool = True):
+  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096, fused: bool = False):
+    """fused: run all blocks of a token in one persistent launch (tga_decode_layers; dense Q4_0 / Q8_0 models only).  The default is
+    one launch per op (five per dense block, seven per MoE block), which measures about 5 % faster on the 8B configuration."""
     self.config = c = config
     self.s = _Shared(c, max_new)
     self.max_new = max_new
@@ -228,7 +230,7 @@ class Transformer:
     self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
     self.stream = rt.Stream()
     self._graphs = {}
-    # one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
+    # optional: one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
     self.layer_table = self._build_layer_table() if fused else None
 
   def _build_layer_table(self):
