@@ -150,9 +150,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
   __shared__ float qs[4][HD];                           // rotated queries of the 4 heads in flight
   __shared__ float ks[HD], vs[HD];                      // rotated key / value of this token
   __shared__ float comb[4 * NGRP * CSTR];               // [head in flight][run]: o[HD], m, l
-  __shared__ float sw[2048];                            // merge weights; host guarantees group * nsplit <= 1024
   __shared__ float red[8];
-  __shared__ int last_flag;
   const int vr = lane / HD8, vp = lane % HD8;
   const int p0 = split * 64 + wave * 16;                // first position of this wave
   u32x4 kt[NVI], vt[NVI];
@@ -182,6 +180,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
   // normalised values: weight index = position in the whole vector, or inside the head for the per-head norm
   auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[per_head ? i % HD : i] : a.q[i]; };
   auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[per_head ? i % HD : i] : a.k[i]; };
+  // the query of this wave's first head pass is requested together with k, v and the rotation row (one memory round trip, not two)
+  constexpr int QPL = (HD / 2 + 63) / 64;               // query pairs per lane
+  float qx1[QPL], qx2[QPL], qc[QPL], qsn[QPL];
+  {
+    const int head = kvh * group + (wave < group ? wave : 0);
+#pragma unroll
+    for (int j = 0; j < QPL; j++) {
+      const int i = lane + 64 * j < half ? lane + 64 * j : half - 1;
+      qx1[j] = a.q[head * HD + i]; qx2[j] = a.q[head * HD + half + i];
+      qc[j] = a.rope[(size_t)pos * HD + i]; qsn[j] = a.rope[(size_t)pos * HD + half + i];
+    }
+  }
   for (int i = tid; i < half; i += 256) {
     const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
     const float x1 = kval(kvh * HD + i), x2 = kval(kvh * HD + half + i);
@@ -201,7 +211,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
     for (int i = 0; i < NVI; i++) if (p0 + i * RPI + vr >= pos) { kt[i] = kcur; vt[i] = vcur; }
   }
   for (int h0 = 0; h0 < group; h0 += 4) {
-    if (h0 + wave < group) {                            // wave w rotates the query of head h0 + w
+    if (h0 == 0 && !a.q_norm) {                         // first pass without a norm: the values are already here
+      if (wave < group) {
+#pragma unroll
+        for (int j = 0; j < QPL; j++) {
+          const int i = lane + 64 * j;
+          if (i < half) { qs[wave][i] = qx1[j] * qc[j] - qx2[j] * qsn[j]; qs[wave][half + i] = qx2[j] * qc[j] + qx1[j] * qsn[j]; }
+        }
+      }
+    } else if (h0 + wave < group) {                     // wave w rotates the query of head h0 + w
       const int head = kvh * group + h0 + wave;
       if (per_head) {
         float sq = 0.f;
@@ -270,65 +288,68 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
       }
       float* po = a.part + ((size_t)head * a.nsplit + split) * (HD + 2);
 #pragma unroll
-      for (int j = 0; j < HD / 64; j++) cst(&po[lane + 64 * j], od[j]);
-      if (lane == 0) { cst(&po[HD], m); cst(&po[HD + 1], l); }
+      for (int j = 0; j < HD / 64; j++) po[lane + 64 * j] = od[j];
+      if (lane == 0) { po[HD] = m; po[HD + 1] = l; }
     }
     __syncthreads();
   }
-  // ---- merge: the last split of this kv head to arrive combines its heads' partials ----
-  int* counters = (int*)(a.part + (size_t)a.n_heads * a.nsplit * (HD + 2));
-  const int ns = (pos >> 6) + 1;
-  stores_done();
-  __syncthreads();
-  if (tid == 0) {
-    const int prev = __hip_atomic_fetch_add(&counters[kvh], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last_flag = (prev == ns - 1);
-    if (prev == ns - 1) __hip_atomic_store(&counters[kvh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
-  }
-  __syncthreads();
-  if (!last_flag) return;
-  // (m, l) of every (head, split), then one wave per head forms the normalised weights, then the weighted sum with 16 splits in
-  // flight per output
-  for (int idx = tid; idx < group * ns; idx += 256) {
-    const int gh = idx / ns, sp = idx - gh * ns;
-    const float* ph = a.part + ((size_t)(kvh * group + gh) * a.nsplit + sp) * (HD + 2);
-    sw[gh * a.nsplit + sp] = cld(&ph[HD]);
-    sw[1024 + gh * a.nsplit + sp] = cld(&ph[HD + 1]);
-  }
-  __syncthreads();
-  for (int gh = wave; gh < group; gh += 4) {
+}
+
+// Second launch: one workgroup of HD threads per query head combines that head's split partials (max, sum, weighted V).  A kernel
+// boundary orders the partials; it costs less than publishing them inside one launch (write-through stores, completion wait, arrival
+// counter, cache-bypassing reads: four dependent memory round trips on the critical path of the last workgroup to arrive).
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs a) {
+  const int head = blockIdx.x, d = threadIdx.x;
+  const int pos = a.st->pos, ns = (pos >> 6) + 1;
+  __shared__ float sw[1024];                            // exp(m_s - m) / l per split
+  __shared__ float red[2 * (HD / 64)];
+  const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2);
+  auto run = [&](auto tag) {
+    constexpr int SC = decltype(tag)::value;             // split loads in flight per thread, sized by the number of splits
+    float v[SC];
+#pragma unroll
+    for (int j = 0; j < SC; j++) v[j] = ph[(size_t)min(j, ns - 1) * (HD + 2) + d];      // first batch of partial outputs, ahead of the weights
+    // m and l of the splits: thread t takes splits t, t + HD, ...
     float m = -INFINITY;
-    for (int sp = lane; sp < ns; sp += 64) m = fmaxf(m, sw[gh * a.nsplit + sp]);
+    for (int sp = d; sp < ns; sp += HD) m = fmaxf(m, ph[(size_t)sp * (HD + 2) + HD]);
     m = wave_max(m);
-    float l = 0.f;
-    for (int sp = lane; sp < ns; sp += 64) l += sw[1024 + gh * a.nsplit + sp] * __expf(sw[gh * a.nsplit + sp] - m);
-    l = wave_sum(l);
-    for (int sp = lane; sp < ns; sp += 64) sw[gh * a.nsplit + sp] = __expf(sw[gh * a.nsplit + sp] - m) / l;
-  }
-  __syncthreads();
-  // weighted sum over the splits, one output at a time with SC split loads in flight; SC follows the number of splits (a fixed large
-  // batch would request mostly clamped duplicates at short contexts; both outputs of a thread in one batch measured slower)
-  auto merge_out = [&](auto tag) {
-    constexpr int SC = decltype(tag)::value;
-    for (int idx = tid; idx < group * HD; idx += 256) {
-      const int gh = idx / HD, d = idx - gh * HD, head = kvh * group + gh;
-      const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2) + d;
-      float o = 0.f;
-      for (int s0 = 0; s0 < ns; s0 += SC) {
-        float v[SC];
+    if constexpr (HD > 64) {
+      if ((d & 63) == 0) red[d >> 6] = m;
+      __syncthreads();
+      m = red[0];
 #pragma unroll
-        for (int j = 0; j < SC; j++) v[j] = cld(&ph[(size_t)min(s0 + j, ns - 1) * (HD + 2)]);
-#pragma unroll
-        for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[gh * a.nsplit + s0 + j];
-      }
-      if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, head * HD + d, a.stage_nu) : head * HD + d] = (_Float16)o;
-      if (a.out32) a.out32[head * HD + d] = o;
+      for (int i = 1; i < HD / 64; i++) m = fmaxf(m, red[i]);
     }
+    float l = 0.f;
+    for (int sp = d; sp < ns; sp += HD) { const float e = __expf(ph[(size_t)sp * (HD + 2) + HD] - m); sw[sp] = e; l += ph[(size_t)sp * (HD + 2) + HD + 1] * e; }
+    l = wave_sum(l);
+    if constexpr (HD > 64) {
+      if ((d & 63) == 0) red[HD / 64 + (d >> 6)] = l;
+      __syncthreads();
+      l = 0.f;
+#pragma unroll
+      for (int i = 0; i < HD / 64; i++) l += red[HD / 64 + i];
+    } else __syncthreads();
+    const float inv = 1.0f / l;
+    float o = 0.f;
+    for (int s0 = 0; s0 < ns; s0 += SC) {
+      if (s0) {
+#pragma unroll
+        for (int j = 0; j < SC; j++) v[j] = ph[(size_t)min(s0 + j, ns - 1) * (HD + 2) + d];
+      }
+#pragma unroll
+      for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[s0 + j];
+    }
+    o *= inv;
+    const int e = head * HD + d;
+    if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, e, a.stage_nu) : e] = (_Float16)o;
+    if (a.out32) a.out32[e] = o;
   };
-  if (ns <= 4) merge_out(std::integral_constant<int, 4>{});
-  else if (ns <= 8) merge_out(std::integral_constant<int, 8>{});
-  else if (ns <= 16) merge_out(std::integral_constant<int, 16>{});
-  else merge_out(std::integral_constant<int, 24>{});
+  if (ns <= 4) run(std::integral_constant<int, 4>{});
+  else if (ns <= 8) run(std::integral_constant<int, 8>{});
+  else if (ns <= 16) run(std::integral_constant<int, 16>{});
+  else run(std::integral_constant<int, 32>{});
 }
 
 // ---------------------------------------------------------------------------------------------- argmax + token bookkeeping
@@ -447,6 +468,10 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   if (head_dim == 64) attn_decode_kernel<8><<<grid, 256, 0, s>>>(a);
   else if (head_dim == 128) attn_decode_kernel<16><<<grid, 256, 0, s>>>(a);
   else attn_decode_kernel<32><<<grid, 256, 0, s>>>(a);
+  TGA_LAUNCH_CHECK();
+  if (head_dim == 64) attn_merge_kernel<64><<<n_heads, 64, 0, s>>>(a);
+  else if (head_dim == 128) attn_merge_kernel<128><<<n_heads, 128, 0, s>>>(a);
+  else attn_merge_kernel<256><<<n_heads, 256, 0, s>>>(a);
   TGA_LAUNCH_CHECK();
   return 0;
 }
