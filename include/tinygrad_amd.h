@@ -19,6 +19,9 @@ extern "C" {
 #define TGA_F32 0
 #define TGA_F16 1
 #define TGA_Q4_0 2
+#define TGA_Q4_1 3
+#define TGA_Q5_0 6
+#define TGA_Q5_1 7
 #define TGA_Q8_0 8
 #define TGA_Q4_K 12
 #define TGA_Q5_K 13
@@ -54,7 +57,7 @@ int tga_graph_end(void* stream, void** graph_exec);
 int tga_graph_launch(void* graph_exec, void* stream);
 int tga_graph_destroy(void* graph_exec);
 
-/* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 8, 14, 39) ----
+/* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 3, 6, 7, 8, 12, 13, 14, 39) ----
  * blocks: device pointer to the raw GGUF tensor bytes; n: number of elements (multiple of the block size).
  * out_dtype TGA_F32: bit-exact ggml_data_to_tensor result.  TGA_F16: that result cast to fp16 round-to-nearest-even,
  * i.e. the weight the model path holds after tinygrad/llm/model.py:376. */
@@ -64,8 +67,10 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  * tinygrad/nn/__init__.py:177 -> Tensor.dot tinygrad/mixin/op.py:367-392 (float32 accumulation, dtype.py:212-216).
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
- * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  K must be a multiple of the type's block size.
- * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K (GGUF aligns tensor data to 32 bytes, gguf.py:144-148). */
+ * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  K must be a multiple of the type's block size
+ * (Q4_1 / Q5_0 / Q5_1 are served as block pairs: K % 64 == 0).
+ * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K/Q4_1/Q5_0/Q5_1 (GGUF aligns tensor data to 32 bytes,
+ * gguf.py:144-148). */
 int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,
                 int M, int64_t N, int64_t K, void* stream);
 
@@ -120,8 +125,8 @@ int tga_moe_combine(const float* y, const float* probs, const float* resid, int 
  * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, pad[12]} so that one captured launch sequence serves
  * every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484). */
 
-/* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K /
- * MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant). */
+/* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 /
+ * Q4_K / Q5_K / Q6_K / MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant). */
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream);
 
 /* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL).

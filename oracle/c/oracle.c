@@ -72,6 +72,25 @@ static void deq_q6_k(const uint8_t* b, float* y) {            /* block_q6_K: ggm
     y += 128; ql += 64; qh += 32; sc += 8;
   }
 }
+/* block_q4_1: d, m, qs[16]  (dequantize_row_q4_1; tinygrad/llm/gguf.py:47-49) */
+static void deq_q4_1(const uint8_t* b, float* y) {
+  uint16_t dh, mh; memcpy(&dh, b, 2); memcpy(&mh, b + 2, 2);
+  const float d = h2f(dh), m = h2f(mh);
+  for (int j = 0; j < 16; j++) { y[j] = (float)(b[4 + j] & 0x0F) * d + m; y[j + 16] = (float)(b[4 + j] >> 4) * d + m; }
+}
+/* block_q5_0: d, qh[4], qs[16] and block_q5_1: d, m, qh[4], qs[16]  (dequantize_row_q5_0 / q5_1; tinygrad/llm/gguf.py:50-55).
+ * ggml evaluates Q5_0 as (q - 16) * d; the reference evaluates q * d + (-16 * d).  Both are exact for finite d (5 x 11 significant
+ * bits), they differ for an infinite d, and bit-exactness is owed to the reference, so its form is the one used here. */
+static void deq_q5(const uint8_t* b, float* y, int one) {
+  uint16_t dh, mh = 0; memcpy(&dh, b, 2); if (one) memcpy(&mh, b + 2, 2);
+  const float d = h2f(dh), off = one ? h2f(mh) : -16.0f * d;
+  const uint8_t* p = b + (one ? 4 : 2);
+  uint32_t qh; memcpy(&qh, p, 4);
+  for (int j = 0; j < 16; j++) {
+    const int x0 = (p[4 + j] & 0x0F) | (int)(((qh >> j) & 1u) << 4), x1 = (p[4 + j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+    y[j] = (float)x0 * d + off; y[j + 16] = (float)x1 * d + off;
+  }
+}
 /* get_scale_min_k4 of ggml-quants.c: 6-bit scale and min of sub-block j from the 12 packed bytes */
 static void scale_min_k4(int j, const uint8_t* q, uint8_t* d, uint8_t* m) {
   if (j < 4) { *d = q[j] & 63; *m = q[j + 4] & 63; }
@@ -118,13 +137,15 @@ static void deq_mxfp4(const uint8_t* b, float* y) {           /* block_mxfp4: gg
 
 static int type_geom(int t, int* nel, int* nby) {
   switch (t) { case 2: *nel = 32; *nby = 18; return 0; case 8: *nel = 32; *nby = 34; return 0;
+               case 3: *nel = 32; *nby = 20; return 0; case 6: *nel = 32; *nby = 22; return 0; case 7: *nel = 32; *nby = 24; return 0;
                case 12: *nel = 256; *nby = 144; return 0; case 13: *nel = 256; *nby = 176; return 0;
                case 14: *nel = 256; *nby = 210; return 0; case 39: *nel = 32; *nby = 17; return 0; }
   return -1;
 }
 static void deq_block(int t, const uint8_t* b, float* y) {
   switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break;
-               case 12: deq_q4_k(b, y); break; case 13: deq_q5_k(b, y); break; }
+               case 12: deq_q4_k(b, y); break; case 13: deq_q5_k(b, y); break;
+               case 3: deq_q4_1(b, y); break; case 6: deq_q5(b, y, 0); break; case 7: deq_q5(b, y, 1); break; }
 }
 
 /* ggml_data_to_tensor (tinygrad/llm/gguf.py:23): n_blocks blocks -> float32 */

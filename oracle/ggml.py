@@ -1,11 +1,12 @@
 """numpy restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for the block layouts on the path (Q4_0, Q8_0, Q6_K,
-MXFP4 and the Q4_K / Q5_K superblocks most GGUF model files are made of),
+MXFP4, the Q4_K / Q5_K superblocks most GGUF model files are made of, and the older Q4_1 / Q5_0 / Q5_1 blocks),
 plus the ggml reference quantizers used only to build synthetic models.  Test infrastructure only."""
 import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, F32, F16 = 2, 8, 12, 13, 14, 39, 0, 1
+Q4_1, Q5_0, Q5_1 = 3, 6, 7
 # {ggml_type: (elements per block, bytes per block)}  tinygrad/llm/gguf.py:20-21
-GGML_QUANT = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17)}
+GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17)}
 # tinygrad/llm/gguf.py:108-110 (== 2 * E2M1 values; ggml_common.py:218 kvalues_mxfp4)
 FP4_LUT = np.array([0.0, 1.0, 2.0, 3.0, 4.0, 6.0, 8.0, 12.0, -0.0, -1.0, -2.0, -3.0, -4.0, -6.0, -8.0, -12.0], dtype=np.float32)
 
@@ -26,6 +27,22 @@ def _f16(b: np.ndarray) -> np.ndarray: return np.ascontiguousarray(b).view(np.fl
 def dequant_q4_0(blocks: np.ndarray) -> np.ndarray:
   """gguf.py:46  (q_to_uint8(qs,4).bitcast(int8) - 8) * float32(fp16 d)"""
   return (q_to_uint8(blocks[:, 2:], 4).view(np.int8) - np.int8(8)).astype(np.float32) * _f16(blocks[:, :2])
+
+def dequant_q4_1(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:47-49  block = fp16 d, fp16 m, 16 nibble bytes: q * d + m"""
+  d, m = _f16(blocks[:, 0:2]), _f16(blocks[:, 2:4])
+  return q_to_uint8(blocks[:, 4:], 4).astype(np.float32) * d + m
+
+def _dequant_q5(blocks: np.ndarray, one: bool) -> np.ndarray:
+  """gguf.py:50-55  Q5_0 (22 B: d, qh[4], qs[16]) / Q5_1 (24 B: d, m, qh[4], qs[16]): q = nibble + 16 * (bit e of the 32-bit qh),
+  value = q * d + (m for Q5_1, -16 * d for Q5_0)."""
+  d = _f16(blocks[:, :2]); off = 4 if one else 2
+  qh = np.swapaxes(q_to_uint8(blocks[:, off:off + 4], 1).reshape(-1, 8, 4), -1, -2).reshape(-1, 32)
+  q = (q_to_uint8(blocks[:, off + 4:], 4) + qh * np.uint8(16)).astype(np.float32)
+  return q * d + (_f16(blocks[:, 2:4]) if one else np.float32(-16) * d)
+
+def dequant_q5_0(blocks: np.ndarray) -> np.ndarray: return _dequant_q5(blocks, False)
+def dequant_q5_1(blocks: np.ndarray) -> np.ndarray: return _dequant_q5(blocks, True)
 
 def dequant_q8_0(blocks: np.ndarray) -> np.ndarray:
   """gguf.py:56  float32(fp16 d) * int8 qs"""
@@ -65,7 +82,7 @@ def dequant_mxfp4(blocks: np.ndarray) -> np.ndarray:
   d = np.where(e < 2, small, (e - 1) * np.uint32(0x00800000)).astype(np.uint32).view(np.float32)[:, None]
   return FP4_LUT[q_to_uint8(blocks[:, 1:17], 4)] * d
 
-_DEQ = {Q4_0: dequant_q4_0, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
+_DEQ = {Q4_0: dequant_q4_0, Q4_1: dequant_q4_1, Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
 
 def ggml_data_to_tensor(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
   """gguf.py:23-119 restricted to the types on the path; returns flat float32 of n elements."""
@@ -96,6 +113,50 @@ def quantize_q4_0(w: np.ndarray) -> np.ndarray:
   out = np.empty((x.shape[0], 18), dtype=np.uint8)
   out[:, :2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
   out[:, 2:] = q[:, :16] | (q[:, 16:] << 4)
+  return out.reshape(-1)
+
+def _pack_q5_bits(q: np.ndarray) -> np.ndarray:
+  """fifth bits of the 32 quants of each block as the little-endian 32-bit qh (bit e = element e), 4 bytes per block"""
+  bits = ((q >> 4) & 1).astype(np.uint32) << np.arange(32, dtype=np.uint32)[None, :]
+  return np.bitwise_or.reduce(bits, axis=1).astype("<u4").view(np.uint8).reshape(-1, 4)
+
+def quantize_q4_1(w: np.ndarray) -> np.ndarray:
+  """ggml rule (quantize_row_q4_1_ref): d = (max - min) / 15, m = min, q = min(15, int((x - min) / d + 0.5)); d, m stored as fp16."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 32)
+  mn, mx = x.min(axis=1), x.max(axis=1)
+  d = (mx - mn) / np.float32(15)
+  with np.errstate(divide="ignore"): idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+  q = np.minimum(15, ((x - mn[:, None]) * idv[:, None] + np.float32(0.5)).astype(np.int32)).astype(np.uint8)
+  out = np.empty((x.shape[0], 20), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2); out[:, 2:4] = mn.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 4:] = q[:, :16] | (q[:, 16:] << 4)
+  return out.reshape(-1)
+
+def quantize_q5_0(w: np.ndarray) -> np.ndarray:
+  """ggml rule (quantize_row_q5_0_ref): max = signed value of largest magnitude, d = max / -16, q = min(31, int8(x / d + 16.5));
+  nibbles in qs (element j low, j + 16 high), fifth bits in qh."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 32)
+  mx = x[np.arange(x.shape[0]), np.argmax(np.abs(x), axis=1)]
+  d = mx / np.float32(-16.0)
+  with np.errstate(divide="ignore"): idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+  q = np.minimum(31, (x * idv[:, None] + np.float32(16.5)).astype(np.int8)).astype(np.uint8)
+  out = np.empty((x.shape[0], 22), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:6] = _pack_q5_bits(q)
+  out[:, 6:] = (q[:, :16] & 0xF) | ((q[:, 16:] & 0xF) << 4)
+  return out.reshape(-1)
+
+def quantize_q5_1(w: np.ndarray) -> np.ndarray:
+  """ggml rule (quantize_row_q5_1_ref): d = (max - min) / 31, m = min, q = uint8((x - min) / d + 0.5)."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 32)
+  mn, mx = x.min(axis=1), x.max(axis=1)
+  d = (mx - mn) / np.float32(31)
+  with np.errstate(divide="ignore"): idv = np.where(d != 0, np.float32(1.0) / d, np.float32(0)).astype(np.float32)
+  q = np.minimum(31, ((x - mn[:, None]) * idv[:, None] + np.float32(0.5)).astype(np.int32)).astype(np.uint8)
+  out = np.empty((x.shape[0], 24), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2); out[:, 2:4] = mn.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 4:8] = _pack_q5_bits(q)
+  out[:, 8:] = (q[:, :16] & 0xF) | ((q[:, 16:] & 0xF) << 4)
   return out.reshape(-1)
 
 def quantize_q8_0(w: np.ndarray) -> np.ndarray:

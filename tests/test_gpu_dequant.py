@@ -5,7 +5,7 @@ from tinygrad_amd import synth
 from tinygrad_amd.runtime import GGML_QUANT
 
 pytestmark = pytest.mark.gpu
-TYPES = [2, 8, 12, 13, 14, 39]
+TYPES = [2, 3, 6, 7, 8, 12, 13, 14, 39]
 
 def _gpu_dequant(gpu, data, n, t, dtype=np.float32):
   from tinygrad_amd.gguf import ggml_data_to_tensor

@@ -72,7 +72,7 @@ def test_q6_k_brute_force_layout():
     out = og.ggml_data_to_tensor(b, 256, 14)
     np.testing.assert_array_equal(out, exp, err_msg=f"element {e}")
 
-@pytest.mark.parametrize("t", [2, 8, 12, 13, 14, 39])
+@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 39])
 def test_numpy_restatement_equals_scalar_c_loops(t):
   """Vectorised restatement of tinygrad/llm/gguf.py (field-major q_to_uint8) == independent scalar loops of the published ggml
   routines, bit for bit, on fully random bytes (NaN/Inf/subnormal scales included)."""
@@ -111,6 +111,38 @@ def test_q4_k_q5_k_brute_force_layout(t):
     np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, t), exp, err_msg=f"element {e}")
     np.testing.assert_array_equal(cref.dequant(t, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
 
+@pytest.mark.parametrize("t", [3, 6, 7])
+def test_q4_1_q5_0_q5_1_brute_force_layout(t):
+  """One weight at a time against ggml's block_q4_1 / block_q5_0 / block_q5_1 (dequantize_row_q4_1 / q5_0 / q5_1): element j < 16 is
+  the low nibble of qs[j], element j + 16 the high nibble; the fifth bit of element e is bit e of the little-endian 32-bit qh; the
+  value is q * d + m (Q4_1, Q5_1) or (q - 16) * d (Q5_0)."""
+  nby = og.GGML_QUANT[t][1]
+  qh_off = {3: None, 6: 2, 7: 4}[t]; qs_off = {3: 4, 6: 6, 7: 8}[t]
+  d, m = 0.5, -3.25
+  for e in range(32):
+    for q in ((1, 15) if t == 3 else (1, 15, 16, 31)):
+      b = np.zeros(nby, dtype=np.uint8)
+      b[0:2] = np.frombuffer(np.float16(d).tobytes(), np.uint8)
+      if t != 6: b[2:4] = np.frombuffer(np.float16(m).tobytes(), np.uint8)
+      b[qs_off + e % 16] = (q & 0xF) << (4 if e >= 16 else 0)
+      if q >> 4: b[qh_off + e // 8] = 1 << (e % 8)
+      base = -16 * d if t == 6 else m                              # what a zero quant decodes to
+      exp = np.full(32, base, dtype=np.float32); exp[e] = q * d + base
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 32, t), exp, err_msg=f"element {e} q {q}")
+      np.testing.assert_array_equal(cref.dequant(t, b[None]).reshape(-1), exp, err_msg=f"element {e} q {q} (C)")
+
+def test_q5_0_equals_q4_0_when_fifth_bits_mirror_the_sign():
+  """Q5_0 with q5 = 2 * q4 (fifth bit = top bit of the nibble, low bit 0) and half the scale decodes to the Q4_0 values:
+  (2 q - 16) * (d / 2) = (q - 8) * d - ties the new decoder to the Q4_0 one the reference's own tests pin."""
+  rng = np.random.default_rng(5)
+  q4 = rng.integers(0, 16, size=(64, 32)).astype(np.uint8)
+  d = np.float16(rng.uniform(0.01, 2.0, 64))
+  b4 = np.zeros((64, 18), np.uint8); b4[:, :2] = d.view(np.uint8).reshape(-1, 2); b4[:, 2:] = q4[:, :16] | (q4[:, 16:] << 4)
+  q5 = q4 * 2
+  b5 = np.zeros((64, 22), np.uint8); b5[:, :2] = (d / np.float16(2)).astype(np.float16).view(np.uint8).reshape(-1, 2)
+  b5[:, 2:6] = og._pack_q5_bits(q5); b5[:, 6:] = (q5[:, :16] & 0xF) | ((q5[:, 16:] & 0xF) << 4)
+  np.testing.assert_array_equal(og.ggml_data_to_tensor(b5, 64 * 32, 6), og.ggml_data_to_tensor(b4, 64 * 32, 2))
+
 def test_q6_k_association_order_is_exact():
   """(d*q)*sc == d*(sc*q) == (d*sc)*q in float32: 11 + 6 + 8 significant bits fit in 24."""
   rng = np.random.default_rng(3)
@@ -120,7 +152,8 @@ def test_q6_k_association_order_is_exact():
 def test_quantizers_round_trip():
   rng = np.random.default_rng(0)
   w = rng.standard_normal(256 * 64).astype(np.float32)
-  for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0), (12, og.quantize_q4_k, 1 / 6.0), (13, og.quantize_q5_k, 1 / 13.0)):
+  for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0), (12, og.quantize_q4_k, 1 / 6.0), (13, og.quantize_q5_k, 1 / 13.0),
+                      (3, og.quantize_q4_1, 1 / 7.0), (6, og.quantize_q5_0, 1 / 15.0), (7, og.quantize_q5_1, 1 / 15.0)):
     dq = og.ggml_data_to_tensor(qf(w), w.size, t)
     nel = og.GGML_QUANT[t][0] if t != 14 else 16
     amax = np.abs(w.reshape(-1, nel)).max(1, keepdims=True)

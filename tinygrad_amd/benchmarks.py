@@ -5,7 +5,7 @@
   config 5  MXFP8 grouped GEMM at T = 4096, E = 128, k = 8 with Zipf routing (MFMA utilisation and GB/s), plus the measured
             register-only peak of the scaled FP8 MFMA
 
-  config 6  Q4_K / Q5_K dequant-GEMV at the same linear shapes (not a BASELINE config)
+  config 6  Q4_K / Q5_K and Q4_1 / Q5_0 / Q5_1 dequant-GEMV at the same linear shapes (not a BASELINE config)
 
     python -m tinygrad_amd.benchmarks [--config N ...]        prints one JSON object per measurement
 
@@ -39,7 +39,7 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   wbytes = n * (k // nel) * nby
   copies = max(2, -(-int(1.25 * MALL_BYTES) // wbytes))
   big = Buffer((copies * wbytes,), np.uint8)
-  if ggml_type in (rt.Q4_K, rt.Q5_K):                                         # no device-side writer for these: seeded host blocks, one upload per copy
+  if ggml_type in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1):                                         # no device-side writer for these: seeded host blocks, one upload per copy
     from tinygrad_amd import synth
     host = synth.random_blocks(np.random.default_rng(1002), ggml_type, n, k)
     for c in range(copies): big.view(c * wbytes, (wbytes,), np.uint8).copyin(host)
@@ -52,7 +52,7 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   s = rt.Stream()
   us = _time_launches(lambda i: lins[i](x, out=y, stream=s.handle), copies, iters, s)
   alg = wbytes + m * k * 2 + m * n * 2
-  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
+  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_1: "Q4_1", rt.Q5_0: "Q5_0", rt.Q5_1: "Q5_1", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
   return {"case": f"{name} {n}x{k} M={m}", "avg_us": round(us, 2), "alg_bytes": alg, "GBps": round(alg / us / 1e3, 1),
           "frac_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_rotated": copies, "launches": iters}
 
@@ -65,9 +65,10 @@ def config2():
   return out
 
 def kquants():
-  """Q4_K / Q5_K (the block types of Q4_K_M / Q5_K_M model files) at the Llama-3-8B linear shapes, M in {1, 8}."""
+  """Q4_K / Q5_K (the block types of Q4_K_M / Q5_K_M model files) and the older Q4_1 / Q5_0 / Q5_1 blocks at the Llama-3-8B linear
+  shapes, M in {1, 8}."""
   out = []
-  for t in (rt.Q4_K, rt.Q5_K):
+  for t in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1):
     for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
       for m in (1, 8): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   return out
@@ -159,7 +160,7 @@ def config5():
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K GEMV shapes")
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes")
   ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
   args = ap.parse_args()
   rt.init(0)

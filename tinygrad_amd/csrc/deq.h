@@ -16,6 +16,33 @@ template <> struct Deq<GGML_Q4_0> {
     for (int i = 0; i < 4; i++) o[i] = (float)((int)((q[i] >> sh) & 0xF) - 8) * d;
   }
 };
+// Q4_1 (20 B: d, m, qs[16]), tinygrad/llm/gguf.py:47-49: q * d + m
+template <> struct Deq<GGML_Q4_1> {
+  static constexpr int NEL = 32, NBY = 20;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b)), m = h2f_bits(ld2(b + 2));
+    const int sh = (e0 >= 16) ? 4 : 0; const uint8_t* q = b + 4 + (e0 & 15);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = (float)((q[i] >> sh) & 0xF) * d + m;
+  }
+};
+// Q5_0 (22 B: d, qh[4], qs[16]) and Q5_1 (24 B: d, m, qh[4], qs[16]), tinygrad/llm/gguf.py:50-55: q = nibble + 16 * bit e of the
+// 32-bit qh; q * d + (m for Q5_1, -16 * d for Q5_0)
+template <bool ONE> struct DeqQ5 {
+  static constexpr int NEL = 32, NBY = ONE ? 24 : 22;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b)), off = ONE ? h2f_bits(ld2(b + 2)) : -16.0f * d;
+    const uint8_t* p = b + (ONE ? 4 : 2);
+    const uint32_t qh = (uint32_t)ld2(p) | ((uint32_t)ld2(p + 2) << 16);
+    const int sh = (e0 >= 16) ? 4 : 0; const uint8_t* q = p + 4 + (e0 & 15);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = (float)(((q[i] >> sh) & 0xF) | (((qh >> (e0 + i)) & 1u) << 4)) * d + off;
+  }
+};
+template <> struct Deq<GGML_Q5_0> : DeqQ5<false> {};
+template <> struct Deq<GGML_Q5_1> : DeqQ5<true> {};
 template <> struct Deq<GGML_Q8_0> {
   static constexpr int NEL = 32, NBY = 34;
   static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {

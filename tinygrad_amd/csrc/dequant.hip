@@ -1,4 +1,4 @@
-// Block dequant kernels: bit-exact restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for Q4_0 (:46), Q8_0 (:56),
+// Block dequant kernels: bit-exact restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for Q4_0 (:46), Q4_1 (:47-49), Q5_0 / Q5_1 (:50-55), Q8_0 (:56),
 // Q4_K / Q5_K (:57-67), Q6_K (:68-72) and MXFP4 (:105-114).  One thread produces 4 consecutive output elements (one 16-byte or 8-byte store), so
 // stores are fully coalesced; the packed bytes are re-read through L1/L2 (this kernel is a load-time / test utility, the
 // decode path never materialises weights).
@@ -41,6 +41,9 @@ extern "C" int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* o
   hipStream_t s = (hipStream_t)stream;
   switch (ggml_type) {
     case GGML_Q4_0: return launch_dequant<GGML_Q4_0>(blocks, n, out, out_dtype, s);
+    case GGML_Q4_1: return launch_dequant<GGML_Q4_1>(blocks, n, out, out_dtype, s);
+    case GGML_Q5_0: return launch_dequant<GGML_Q5_0>(blocks, n, out, out_dtype, s);
+    case GGML_Q5_1: return launch_dequant<GGML_Q5_1>(blocks, n, out, out_dtype, s);
     case GGML_Q8_0: return launch_dequant<GGML_Q8_0>(blocks, n, out, out_dtype, s);
     case GGML_Q4_K: return launch_dequant<GGML_Q4_K>(blocks, n, out, out_dtype, s);
     case GGML_Q5_K: return launch_dequant<GGML_Q5_K>(blocks, n, out, out_dtype, s);

@@ -571,6 +571,132 @@ template <bool FIVE> struct FmtK45 {
 template <> struct Fmt<GGML_Q4_K> : FmtK45<false> {};
 template <> struct Fmt<GGML_Q5_K> : FmtK45<true> {};
 
+// ------------------------------------------------------------------------------------------------ Q4_1 / Q5_0 / Q5_1 (gguf.py:47-55)
+// Blocks of 32 weights: fp16 d, [fp16 m], [qh: the 32 fifth bits, little endian], qs[16]; weight j is the low nibble of qs[j],
+// weight j + 16 the high nibble (+ 16 * bit of qh).  w = q d + m (Q4_1, Q5_1) or (q - 16) d (Q5_0).
+// A unit is a PAIR of blocks (64 weights; 40 / 44 / 48 bytes, 4-byte aligned) with four accumulator groups: (block, nibble half).
+// Low nibbles decode as 1024 + q, high nibbles stay in place as 64 + q; the fifth bit lands on mantissa bit 4 / bit 8.  The unit's
+// contribution is d_j (S_lo + S_hi) + off_j X_j per block with S = sum q x, X = sum x and off = m or -16 d; X comes out of the bias
+// corrections the lane already holds (c_lo = -1024 X_lo, c_hi = -64 X_hi).
+// Q5_0 blocks are 22 bytes: block 0's qs starts at byte 6 of the unit, so its first quant dword is assembled from the halves around
+// it and holds bytes (0, 1, 14, 15) of qs; the activations are staged in the matching order (as for the Q4_0 block pair).
+typedef u32x2 u32x2_a4 __attribute__((aligned(4)));
+__device__ __forceinline__ u32x2 ld8_a4(const uint8_t* p) { return *(const TGA_GLOBAL u32x2_a4*)p; }
+template <int KIND> struct FmtL {     // KIND 0: Q4_1, 1: Q5_0, 2: Q5_1
+  static constexpr bool FIVE = KIND != 0;
+  static constexpr int UW = 64, UPB = 1, BW = 64, BB = KIND == 0 ? 40 : KIND == 1 ? 44 : 48, ND = BB / 4;
+  static __device__ __forceinline__ int unit_of(int e) { return e >> 6; }
+  static __device__ __forceinline__ int pair_of(int e) { return (e & 63) >> 1; }
+  static constexpr int XV = 8, NG = 4, NWV = 36;
+  struct Raw { u32x4 a, b; uint32_t t[ND - 8]; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* p = row + BB * u; Raw r; r.a = ld16_a4(p); r.b = ld16_a4(p + 16);
+    if constexpr (KIND == 2) { const u32x4 v = ld16_a4(p + 32); r.t[0] = v.x; r.t[1] = v.y; r.t[2] = v.z; r.t[3] = v.w; }
+    else { const u32x2 v = ld8_a4(p + 32); r.t[0] = v.x; r.t[1] = v.y; if constexpr (KIND == 1) r.t[2] = ld4_a4(p + 40); }
+    return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 2;
+  static __device__ __forceinline__ void consts(uint32_t* kc) { kc[0] = vgpr_const(0x64006400u); kc[1] = vgpr_const(0x54005400u); }
+  // block 0 of a Q5_0 pair: quant dword i holds bytes (b0, b0 + 1, b2, b2 + 1) with (b0, b2) / 2 = (0, 7), (1, 2), (3, 4), (5, 6)
+  static __device__ __forceinline__ constexpr bool odd_block(int j) { return KIND == 1 && j == 0; }
+  // wv[8 (2j + hi) + 2i + o]: block j, nibble half hi, quant dword i, o = odd bytes of the dword
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+    const uint32_t D[12] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.t[0], r.t[1], ND > 10 ? r.t[ND > 10 ? 2 : 0] : 0u, ND > 11 ? r.t[ND > 11 ? 3 : 0] : 0u};
+    uint32_t Q[2][4], qh[2] = {0u, 0u}, hdr[2];
+    if constexpr (KIND == 0) { hdr[0] = D[0]; hdr[1] = D[5]; for (int i = 0; i < 4; i++) { Q[0][i] = D[1 + i]; Q[1][i] = D[6 + i]; } }
+    else if constexpr (KIND == 2) { hdr[0] = D[0]; hdr[1] = D[6]; qh[0] = D[1]; qh[1] = D[7]; for (int i = 0; i < 4; i++) { Q[0][i] = D[2 + i]; Q[1][i] = D[8 + i]; } }
+    else {
+      hdr[0] = D[0] & 0xFFFFu; hdr[1] = D[5] >> 16; qh[0] = __builtin_amdgcn_alignbit(D[1], D[0], 16); qh[1] = D[6];
+      Q[0][0] = __builtin_amdgcn_alignbit(D[5], D[1], 16); Q[0][1] = D[2]; Q[0][2] = D[3]; Q[0][3] = D[4];
+      for (int i = 0; i < 4; i++) Q[1][i] = D[7 + i];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t w = Q[j][i], w8 = w >> 8;
+        uint32_t le = and_or(w, 0x000F000Fu, kc[0]), lo = and_or(w8, 0x000F000Fu, kc[0]);
+        uint32_t he = and_or(w, 0x00F000F0u, kc[1]), ho = and_or(w8, 0x00F000F0u, kc[1]);
+        if constexpr (FIVE) {
+          // fifth bits of the dword's four bytes: t for the low-nibble weights (elements b0..b3), u for the high-nibble ones (16 + b)
+          uint32_t t, u;
+          if (odd_block(j)) {
+            if (i == 0) { t = (qh[j] & 3u) | ((qh[j] >> 12) & 0xCu); u = ((qh[j] >> 16) & 3u) | ((qh[j] >> 28) & 0xCu); }
+            else { t = (qh[j] >> (4 * i - 2)) & 0xFu; u = (qh[j] >> (4 * i + 14)) & 0xFu; }
+          } else { t = (qh[j] >> (4 * i)) & 0xFu; u = (qh[j] >> (4 * i + 16)) & 0xFu; }
+          const uint32_t X = t | (t << 14), Y = u | (u << 14);   // bits 0, 1 and 16, 17: bytes 0, 1 and 2, 3
+          le = and_or(X << 4, 0x00100010u, le); lo = and_or(X << 3, 0x00100010u, lo);
+          he = and_or(Y << 8, 0x01000100u, he); ho = and_or(Y << 7, 0x01000100u, ho);
+        }
+        wv[16 * j + 2 * i] = le; wv[16 * j + 2 * i + 1] = lo; wv[16 * j + 8 + 2 * i] = he; wv[16 * j + 8 + 2 * i + 1] = ho;
+      }
+    }
+    // scale slots: d0, d1, and off_j * (-1 / 64) with off = m (Q4_1, Q5_1) or -16 d (Q5_0)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const float d = h2f_bits(hdr[j] & 0xFFFFu);
+      wv[32 + j] = __builtin_bit_cast(uint32_t, d);
+      wv[34 + j] = __builtin_bit_cast(uint32_t, KIND == 1 ? d * 0.25f : h2f_bits(hdr[j] >> 16) * (-1.0f / 64.0f));
+    }
+  }
+  // nx[k] = natural pair k of the unit's 64 activations
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+    constexpr int P0[4] = {0, 1, 3, 5}, P2[4] = {7, 2, 4, 6};
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const uint32_t* n = nx + 8 * g;
+      const int j = g >> 1;
+#pragma unroll
+      for (int v = 0; v < 2; v++) {
+        const int a0 = odd_block(j) ? P0[2 * v] : 4 * v, a2 = odd_block(j) ? P2[2 * v] : 4 * v + 1;
+        const int b0 = odd_block(j) ? P0[2 * v + 1] : 4 * v + 2, b2 = odd_block(j) ? P2[2 * v + 1] : 4 * v + 3;
+        xv[2 * g + v].x = pack_even(n[a0], n[a2]); xv[2 * g + v].y = pack_odd(n[a0], n[a2]);
+        xv[2 * g + v].z = pack_even(n[b0], n[b2]); xv[2 * g + v].w = pack_odd(n[b0], n[b2]);
+      }
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; k++) s = dot2(n[k], (g & 1) ? 0x54005400u : 0x64006400u, s);
+      c[g] = -s;
+    }
+  }
+  static __device__ __forceinline__ float finish(const Raw&, const uint32_t* wv, const float* a, const float* c) {
+    return __builtin_bit_cast(float, wv[32]) * (a[0] + a[1]) + __builtin_bit_cast(float, wv[33]) * (a[2] + a[3])
+         + __builtin_bit_cast(float, wv[34]) * (c[0] * 0.0625f + c[1]) + __builtin_bit_cast(float, wv[35]) * (c[2] * 0.0625f + c[3]);
+  }
+  // true weights q d + off as fp16, one rounding
+  static __device__ __forceinline__ void to_f16(const Raw&, uint32_t* wv) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const float s = __builtin_bit_cast(float, wv[32 + j]), off = __builtin_bit_cast(float, wv[34 + j]) * -64.0f;
+      const float c_lo = off - 1024.f * s, c_hi = off - 64.f * s;
+#pragma unroll
+      for (int i = 0; i < 8; i++) { wv[16 * j + i] = h2_unbias_scale_f32(wv[16 * j + i], s, c_lo); wv[16 * j + 8 + i] = h2_unbias_scale_f32(wv[16 * j + 8 + i], s, c_hi); }
+    }
+  }
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = e >> 6, w = e & 63, j = w >> 5, b = w & 31, hi = b >> 4, q = b & 15, g = 2 * j + hi;
+    int i, p;
+    if (odd_block(j)) {
+      if (q < 2) { i = 0; p = q; } else if (q >= 14) { i = 0; p = q - 12; } else { i = 1 + ((q - 2) >> 2); p = (q - 2) & 3; }
+    } else { i = q >> 2; p = q & 3; }
+    return (((2 * g + (i >> 1)) * nu + u) * 4 + (i & 1) * 2 + (p & 1)) * 2 + (p >> 1);
+  }
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const uint32_t k = (g & 1) ? 0x54005400u : 0x64006400u;
+      float t = 0.f;
+#pragma unroll
+      for (int i = 2 * g; i < 2 * g + 2; i++) { t = dot2(xv[i].x, k, t); t = dot2(xv[i].y, k, t); t = dot2(xv[i].z, k, t); t = dot2(xv[i].w, k, t); }
+      c[g] = -t;
+    }
+  }
+};
+template <> struct Fmt<GGML_Q4_1> : FmtL<0> {};
+template <> struct Fmt<GGML_Q5_0> : FmtL<1> {};
+template <> struct Fmt<GGML_Q5_1> : FmtL<2> {};
+
 // unit_dot with the unit's activations already in registers (M = 1)
 template <int T>
 __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, const u32x4* xv, const float* cv, float& acc, const uint32_t* kc) {
@@ -614,6 +740,9 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
     case GGML_Q6_K: return Fmt<GGML_Q6_K>::spos(e, nu);
     case GGML_Q4_K: return Fmt<GGML_Q4_K>::spos(e, nu);
     case GGML_Q5_K: return Fmt<GGML_Q5_K>::spos(e, nu);
+    case GGML_Q4_1: return Fmt<GGML_Q4_1>::spos(e, nu);
+    case GGML_Q5_0: return Fmt<GGML_Q5_0>::spos(e, nu);
+    case GGML_Q5_1: return Fmt<GGML_Q5_1>::spos(e, nu);
     case GGML_MXFP4: return Fmt<GGML_MXFP4>::spos(e, nu);
     case GGML_F16: return Fmt<GGML_F16>::spos(e, nu);
   }

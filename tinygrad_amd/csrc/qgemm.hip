@@ -148,6 +148,9 @@ int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
     case GGML_Q6_K: return launch_qgemm_m<GGML_Q6_K>(a, M, s);
     case GGML_Q4_K: return launch_qgemm_m<GGML_Q4_K>(a, M, s);
     case GGML_Q5_K: return launch_qgemm_m<GGML_Q5_K>(a, M, s);
+    case GGML_Q4_1: return launch_qgemm_m<GGML_Q4_1>(a, M, s);
+    case GGML_Q5_0: return launch_qgemm_m<GGML_Q5_0>(a, M, s);
+    case GGML_Q5_1: return launch_qgemm_m<GGML_Q5_1>(a, M, s);
   }
   return -1;
 }

@@ -323,6 +323,7 @@ static int staged_fmt(int ggml_type, long long K, int* nu) {
   switch (ggml_type) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
     case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
+    case GGML_Q4_1: fmt = GGML_Q4_1; break; case GGML_Q5_0: fmt = GGML_Q5_0; break; case GGML_Q5_1: fmt = GGML_Q5_1; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
   if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K) ? 256 : 64) != 0) return -1;
@@ -361,7 +362,9 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
   switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: bw = 256; break; case GGML_F16: bw = 64; break;
+    case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: bw = 64; break;      // served as block pairs
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
+  const bool align4 = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q4_1 || ggml_type == GGML_Q5_0 || ggml_type == GGML_Q5_1;
   TGA_REQUIRE(ggml_type != GGML_F16 || M == 1, "tga_qlinear: dense fp16 weights are served for M = 1 only");
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
   TGA_REQUIRE(x, "tga_qlinear: null x");
@@ -371,7 +374,7 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
   for (int i = 0; i < nseg; i++) {
     TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)), "tga_qlinear: segment %d has a null pointer or no rows", i);
     TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((uintptr_t)w[i] & 1) == 0, "tga_qlinear: weight pointer of segment %d must be 2-byte aligned", i);
-    TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K) || ((uintptr_t)w[i] & 3) == 0, "tga_qlinear: Q4_K / Q5_K weights of segment %d must be 4-byte aligned", i);
+    TGA_REQUIRE(!align4 || ((uintptr_t)w[i] & 3) == 0, "tga_qlinear: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 weights of segment %d must be 4-byte aligned", i);
     a.w[i] = (const uint8_t*)w[i]; a.y[i] = y[i]; a.n[i] = n[i]; a.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr;
     TGA_REQUIRE(epilogue != 1 || a.resid[i], "tga_qlinear: null resid for segment %d", i);
     ntot += n[i];
@@ -407,6 +410,9 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
     case GGML_Q6_K: return launch_qgemv_m<GGML_Q6_K>(a, M, s);
     case GGML_Q4_K: return launch_qgemv_m<GGML_Q4_K>(a, M, s);
     case GGML_Q5_K: return launch_qgemv_m<GGML_Q5_K>(a, M, s);
+    case GGML_Q4_1: return launch_qgemv_m<GGML_Q4_1>(a, M, s);
+    case GGML_Q5_0: return launch_qgemv_m<GGML_Q5_0>(a, M, s);
+    case GGML_Q5_1: return launch_qgemv_m<GGML_Q5_1>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
   }
   return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
@@ -447,9 +453,11 @@ extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_u
   switch (ggml_type) { case GGML_Q4_0: bw = 32; bb = 18; break; case GGML_Q8_0: bw = 32; bb = 34; break; case GGML_MXFP4: bw = 32; bb = 17; break;
     case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_Q4_K: bw = 256; bb = 144; break; case GGML_Q5_K: bw = 256; bb = 176; break;
     case GGML_F16: bw = 64; bb = 128; break;
+    case GGML_Q4_1: bw = 64; bb = 40; break; case GGML_Q5_0: bw = 64; bb = 44; break; case GGML_Q5_1: bw = 64; bb = 48; break;   // block pairs
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   TGA_REQUIRE(K > 0 && K % bw == 0 && N > 0, "tga_qlinear_experts: K=%lld must be a positive multiple of %d", (long long)K, bw);
-  TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K) || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0), "tga_qlinear_experts: Q4_K / Q5_K weights must be 4-byte aligned");
+  TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q4_1 && ggml_type != GGML_Q5_0 && ggml_type != GGML_Q5_1) || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0),
+              "tga_qlinear_experts: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 weights must be 4-byte aligned");
   QArgs a = {};
   a.nseg = w_up ? 2 : 1; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = w_up ? 2 : 0; a.K = (int)K;
   a.w[0] = (const uint8_t*)w; a.w[1] = (const uint8_t*)w_up; a.y[0] = y; a.n[0] = N; a.n[1] = N; a.ntot = N;

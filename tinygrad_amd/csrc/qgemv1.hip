@@ -246,7 +246,7 @@ static int launch_fast_e(const QArgs& a, hipStream_t s) {
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice.
   // Measured per format at 14336 x 4096 and 4096 x 14336: two rows win for Q4_0, MXFP4, Q4_K (14.3 -> 11.4 us), Q5_K (18.1 -> 15.1 us)
   // and slightly for Q6_K; Q8_0 pairs (68-byte units) are no faster with two.
-  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K) && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu() / WK;
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1) && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu() / WK;
   if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
   return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);
 }
@@ -277,6 +277,9 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
     case GGML_Q6_K: return launch_fast_w<GGML_Q6_K>(a, s);
     case GGML_Q4_K: return launch_fast_w<GGML_Q4_K>(a, s);
     case GGML_Q5_K: return launch_fast_w<GGML_Q5_K>(a, s);
+    case GGML_Q4_1: return launch_fast_w<GGML_Q4_1>(a, s);
+    case GGML_Q5_0: return launch_fast_w<GGML_Q5_0>(a, s);
+    case GGML_Q5_1: return launch_fast_w<GGML_Q5_1>(a, s);
     case GGML_MXFP4: return launch_fast_w<GGML_MXFP4>(a, s);
     case GGML_F16: return launch_fast_w<GGML_F16>(a, s);
   }
