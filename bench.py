@@ -129,13 +129,12 @@ def main():
       e = (rt.Event(), rt.Event()); e[0].record(st); fn(); e[1].record(st); per[key].append(e)
     for b in model.blk:
       s = model.s
-      sg = b.staged
       timed("qkv", lambda: qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.x, [s.q, s.k, s.v], stream=st, norm=(b.attn_norm, c.norm_eps)))
       timed("attention", lambda: rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                          c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if sg else 0, st)))
-      timed("attn_output", lambda: qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=sg))
-      timed("gate_up", lambda: qlinear_multi([b.ffn_gate, b.ffn_up], s.x, [s.act], epilogue=2, stream=st, norm=(b.ffn_norm, c.norm_eps), stage_out_for=b.ffn_down if sg else None))
-      timed("down", lambda: qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=sg))
+                                          c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if b.stage_attn else 0, st)))
+      timed("attn_output", lambda: qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.stage_attn))
+      timed("gate_up", lambda: qlinear_multi([b.ffn_gate, b.ffn_up], s.x, [s.act], epilogue=2, stream=st, norm=(b.ffn_norm, c.norm_eps), stage_out_for=b.ffn_down if b.stage_act else None))
+      timed("down", lambda: qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.stage_act))
     rt.check(L.tga_advance_prompt(model.s.state.ptr, model.s.prompt.ptr, st))
     model.stream.synchronize()
     for k in durs: durs[k] += [a.elapsed_ms(b_) * 1e3 for a, b_ in per[k]]

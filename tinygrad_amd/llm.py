@@ -135,19 +135,20 @@ class TransformerBlock:
     self.cache_k = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.config, self.s = c, shared
-    # staged activations need every consumer of one activation to share a type and a staged layout (K % 64, Q6_K: % 256)
-    self.staged = (not self.moe) and all(l.ggml_type in (rt.Q4_0, rt.Q8_0, rt.F16) and l.in_features % 64 == 0 and l.in_features <= 65536
-                                         for l in (self.attn_q, self.attn_output, self.ffn_gate, self.ffn_down)) \
-                  and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
-    # RMSNorm folded into the consuming M = 1 linear (needs its register-resident fast path: K % 64, 4-byte aligned weights)
+    # the M = 1 GEMV's register-resident fast path: K % 64 (superblock types: % 256), 4-byte aligned weights
     fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K) or l.in_features % 256 == 0)
+    # RMSNorm folded into the consuming linear
     self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
+    # a producer with a single consumer writes its fp16 output in the order that consumer's GEMV reads it (no LDS staging there):
+    # attention -> attn_output, SwiGLU -> ffn_down, and the unfused ffn_norm -> ffn_gate / ffn_up
+    self.stage_attn = fast(self.attn_output)
+    self.stage_act = (not self.moe) and fast(self.ffn_down)
+    self.stage_xn = (not self.moe) and fast(self.ffn_gate) and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
     if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
 
   def __call__(self, x: Buffer, stream):
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
-    st = self.staged                                                     # producers write the consumer's staged order directly
     qkv, qkv_out = [self.attn_q, self.attn_k, self.attn_v], [s.q, s.k, s.v]
     same = self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type
     if self.fuse_norm and same:                                          # the q/k/v launch normalises the row while staging it
@@ -165,16 +166,16 @@ class TransformerBlock:
     # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
     rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
                                            int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
-                                           s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if st else 0, stream))
-    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
+                                           s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if self.stage_attn else 0, stream))
+    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_attn)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     if not self.moe:
       if self.fuse_norm:
-        qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps), stage_out_for=self.ffn_down if st else None)
+        qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps), stage_out_for=self.ffn_down if self.stage_act else None)
       else:
-        rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if st else 0, stream))
-        qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=st, stage_out_for=self.ffn_down if st else None)
-      qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=st)
+        rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if self.stage_xn else 0, stream))
+        qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=self.stage_xn, stage_out_for=self.ffn_down if self.stage_act else None)
+      qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_act)
       return
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
