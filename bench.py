@@ -6,7 +6,7 @@ lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the 
 are decoded greedily, one captured launch sequence per token with a host sync per token (as the reference's generate loop does).
 Prints ONE JSON line: tok/s, the roofline of the dominant kernel from HIP-event timings taken live, the same figures for the other
 kernels of a block, and a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the same weights).
-Default path: one launch per op (five per block); the dominant kernel is then the fused ffn_gate + ffn_up dequant-GEMV with the
+Default path: one launch per op (six per block, attention being two); the dominant kernel is then the fused ffn_gate + ffn_up dequant-GEMV with the
 ffn_norm folded in.  --fused: all 32 blocks of a token in one persistent launch (tga_decode_layers), which is then the kernel reported."""
 import argparse, json, os, sys, time
 import numpy as np
@@ -178,7 +178,7 @@ def main():
     dom = kern["gate_up"]
     per_block = sum(v["avg_us"] for v in kern.values())
     out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
-                                                 "one of five launches per block)",
+                                                 "one of six launches per block)",
                        "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
                        # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py (counters scaled by a
                        # 1 GiB copy kernel: x2.0000 and x1.0000)
