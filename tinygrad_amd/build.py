@@ -30,7 +30,7 @@ def build(force: bool = False, verbose: bool = False) -> pathlib.Path:
     if force or _stale(obj, [src] + headers): jobs.append((src, obj))
   def compile_one(job):
     src, obj = job
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *os.environ.get("TGA_HIPCC_EXTRA", "").split(), "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0: raise RuntimeError(f"hipcc failed for {src.name}:\n{r.stderr}")
     if verbose: print(f"compiled {src.name}", file=sys.stderr)

@@ -1,0 +1,371 @@
+// M = 1 dequant-GEMV fast path (decode): see qgemv.hip for the overall design.  This header holds the kernel and its launch
+// templates; qgemv1_*.hip instantiate them per weight format (separate translation units compile in parallel).
+#pragma once
+#include "qfmt.h"
+#include "host.h"
+
+#ifndef QG1_DEPTH
+#define QG1_DEPTH 3        // row groups in flight per lane: the loads of the next DEPTH - 1 groups are outstanding while one is multiplied
+#endif
+
+// ------------------------------------------------------------------------------------------------ M = 1 fast path
+// One activation row: each lane keeps the activations of ITS unit in registers for the whole kernel (no LDS traffic in the
+// loop).  A workgroup is WR x WK waves: the WK waves of a row team split K (wave wk owns units 64wk .. 64wk+63) and their
+// partial sums meet in LDS once per row group (the only LDS use in the loop: split-K partials); the WR teams own disjoint
+// row ranges.  Each team walks a contiguous range of row groups with a register ring of QG1_DEPTH groups.
+// Activations reach the registers through one LDS transpose per workgroup: coalesced 16-byte global loads of the plain row,
+// then each lane reads back the 64 (or 32) values of its unit (unit stride padded to spread LDS banks).
+// H (rows of at most 32 units, WK = 1): a row occupies half a wave, so each half-wave is a row team of its own (lanes 0-31 and
+// 32-63 walk different row ranges; the DPP sum stops at 32 lanes) instead of leaving half of the lanes without loads.
+//
+// EVERY LOAD IS ISSUED UNCONDITIONALLY, in straight-line code (rows and units clamped to valid ones, surplus results dropped; the
+// residual of the epilogue travels with its row group): the compiler places s_waitcnt from a per-path count of outstanding loads and
+// takes the most conservative count where paths join, so a load (or a store: they share the counter) inside a branch turns the
+// waits behind the join into "wait for everything" and the ring into a one-deep pipeline.  For the same reason the prologue kind
+// is a template parameter: with the activation format known at compile time the prologue is one basic block in which the small
+// activation reads go out first, the first weight loads second (loads return in issue order), and the staging arithmetic runs
+// while the weights are in flight.
+//   PRO 0  generic: flags read at run time (any activation type, any K); weights first, then the staging loops
+//   PRO 1  one float32 row of at most two 8-element pieces per thread with the RMSNorm folded in (kept in registers between the sum of
+//          squares and the scaling)
+//   PRO 2  activations already in the staged order of this format (written by the producing kernel)
+//   PRO 3  one fp16 row of at most two pieces per thread
+template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
+__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
+  using F = Fmt<T>;
+  typedef typename F::Raw Raw;
+  static_assert(WK == 1 || WR == 1, "row teams and K split are not combined");
+  static_assert(!H || WK == 1, "half-wave rows need the whole row inside one wave");
+  constexpr int HM = H ? 2 : 1;
+  constexpr int NT = WK * WR * 64;
+  constexpr int NP = F::UW / 2;                                  // dwords (fp16 pairs) per unit
+  constexpr int USTRIDE = NP + 4;                                // padded unit stride in dwords
+  constexpr int D = QG1_DEPTH;
+  extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
+  __shared__ float part[2][WK][R];
+  __shared__ float nred[NT / 64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wk = (WK > 1) ? wave : 0, wr = (WK > 1) ? 0 : wave;
+  const int hl = H ? (lane & 31) : lane, hrow = H ? (lane >> 5) : 0;
+  const int u = wk * 64 + hl;
+  const bool uvalid = u < a.nu;
+  const int uc = uvalid ? u : a.nu - 1;
+  const int job = blockIdx.y;
+  const long long eoff = a.sel ? (long long)a.sel[job] * a.estride : 0, yofs = (long long)job * a.ystride;
+  const long long xrow = a.sel ? job / a.xdiv : 0;
+  constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
+  const long long ngroups = (a.ntot + RS - 1) / RS;
+  const long long nteams = (long long)gridDim.x * WR * HM, team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
+  const long long gbase = ngroups / nteams, grem = ngroups % nteams;
+  const long long g0 = team * gbase + (team < grem ? team : grem), g1 = g0 + gbase + (team < grem ? 1 : 0);
+  const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  u32x4 xv[F::XV]; float cv[F::NG];
+  const int nseg = (EPI == 2) ? 1 : a.nseg;
+  int parity = 0;
+
+  // ---- the segment (weight matrix) the team is in
+  int seg = 0;
+  long long seg_start = 0, lo = 0, hi = 0, cnt = 0, last = 0;
+  const uint8_t *base0 = nullptr, *base1 = nullptr;
+  const float* resid = nullptr;
+  auto enter = [&](int sg) {
+    seg = sg;
+    const long long seg_rows = a.n[sg];
+    lo = row_lo - seg_start; hi = row_hi - seg_start;
+    if (lo < 0) lo = 0;
+    if (hi > seg_rows) hi = seg_rows;
+    seg_start += seg_rows;
+    cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;                 // row groups of this team inside the segment
+    last = hi > 0 ? hi - 1 : 0;                                  // rows beyond the range reload this one (always a valid row)
+    base0 = a.w[sg] + eoff;
+    base1 = ((EPI == 2) ? a.w[1] : a.w[sg]) + eoff;
+    if constexpr (EPI == 1) resid = a.resid[sg] + yofs;
+  };
+  struct Grp { Raw w[R]; float res[R]; };
+  auto issue = [&](Grp& g, long long row) {
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      long long rr = (EPI == 2) ? row : row + r;
+      rr = rr < last ? rr : last;
+      const uint8_t* rp = ((EPI == 2 && r == 1) ? base1 : base0) + rr * a.row_bytes;
+      if constexpr (T == GGML_F16) g.w[r] = F::load_nu(rp, uc, a.nu); else g.w[r] = F::load(rp, uc);
+    }
+    if constexpr (EPI == 1) {
+      if constexpr (WK > 1) { long long rr = row + (lane < R ? lane : 0); rr = rr < last ? rr : last; g.res[0] = resid[rr]; }   // wave 0, lane r stores row + r
+      else {
+#pragma unroll
+        for (int r = 0; r < R; r++) { long long rr = row + r; rr = rr < last ? rr : last; g.res[r] = resid[rr]; }
+      }
+    }
+  };
+  // multiply, reduce and store one row group
+  auto finish_group = [&](const Grp& g, long long row) {
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      acc[r] = 0.f;
+      unit_dot_reg<T>(g.w[r], xv, cv, acc[r], kc);
+      acc[r] = H ? half_sum_lane31(uvalid ? acc[r] : 0.f) : wave_sum_lane63(uvalid ? acc[r] : 0.f);
+    }
+    if constexpr (WK > 1) {
+      if (lane == 63) {
+#pragma unroll
+        for (int r = 0; r < R; r++) part[parity][wave][r] = acc[r];
+      }
+      __syncthreads();
+      if (wave == 0) {
+        float t = 0.f;
+        if (lane < R) {
+#pragma unroll
+          for (int j = 0; j < WK; j++) t += part[parity][j][lane];
+        }
+        if constexpr (EPI == 2) {
+          const float up = __shfl(t, 1, 64);
+          if (lane == 0) store_swiglu(a, row, t, up, yofs);
+        } else {
+          if constexpr (EPI == 1) t += g.res[0];
+          if (lane < R && row + lane < hi) store_one<0>(a, seg, row + lane, t, yofs);
+        }
+      }
+      parity ^= 1;
+    } else {
+      if (hl == (H ? 31 : 63)) {
+        if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1], yofs);
+        else {
+#pragma unroll
+          for (int r = 0; r < R; r++) if (row + r < hi) store_one<0>(a, seg, row + r, EPI == 1 ? acc[r] + g.res[r] : acc[r], yofs);
+        }
+      }
+    }
+  };
+  Grp b[D];                                                      // ring of row groups in flight
+  // walks the team's row groups of the current segment; group lo is already in flight in b[0]
+  auto run_segment = [&]() {
+#pragma unroll
+    for (int d = 1; d < D - 1; d++) issue(b[d], lo + (long long)d * RS);
+    long long row = lo, g = 0;
+    for (; g + D <= cnt; g += D) {
+#pragma unroll
+      for (int d = 0; d < D; d++) {
+        issue(b[(d + D - 1) % D], row + (long long)(D - 1) * RS);        // the slot freed by the previous group
+        finish_group(b[d], row);
+        row += RS;
+      }
+    }
+    // fewer than D groups left: their loads are already in flight (slots 0 .. D - 2), nothing more to issue
+#pragma unroll
+    for (int d = 0; d < D - 1; d++) {
+      if (g + d < cnt) finish_group(b[d], row);                  // (split K: the waves of a workgroup share cnt, so the barrier inside is uniform)
+      row += RS;
+    }
+  };
+
+  enter(0);
+  const int nq = a.K / 8;                                        // 16-byte fp16 pieces in the row
+  const f32x4* xr = (const f32x4*)((const float*)a.x + xrow * a.K);
+  const u32x4* xh = (const u32x4*)((const uint16_t*)a.x + xrow * a.K);
+  auto lds_to_regs = [&]() {
+    __syncthreads();
+    uint32_t nx[NP];
+#pragma unroll
+    for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + uc * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+    F::stage(nx, xv, cv);
+  };
+  // piece i (elements 8i .. 8i+7 as 4 fp16 pairs) into LDS: unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
+  auto put_piece = [&](int i, const u32x4& v) {
+    if constexpr (T == GGML_F16) *(u32x4*)(xlds + F::unit_of_nu(8 * i, a.nu) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v;
+    else *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
+  };
+  auto pack8 = [](const f32x4& l, const f32x4& h) {
+    u32x4 v;
+    v.x = f2h_bits(l.x) | (f2h_bits(l.y) << 16); v.y = f2h_bits(l.z) | (f2h_bits(l.w) << 16);
+    v.z = f2h_bits(h.x) | (f2h_bits(h.y) << 16); v.w = f2h_bits(h.z) | (f2h_bits(h.w) << 16);
+    return v;
+  };
+  if constexpr (PRO == 2) {
+    const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
+#pragma unroll
+    for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
+    issue(b[0], lo);
+    F::cfromx(xv, cv);
+  } else if constexpr (PRO == 1) {
+    f32x4 l4[2], h4[2], w0[2], w1[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const int i = (int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1;
+      l4[t] = xr[2 * i]; h4[t] = xr[2 * i + 1];
+      w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1];
+    }
+    issue(b[0], lo);
+    float ss = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const f32x4 l = l4[t], h = h4[t];
+      const float s8 = l.x * l.x + l.y * l.y + l.z * l.z + l.w * l.w + h.x * h.x + h.y * h.y + h.z * h.z + h.w * h.w;
+      ss += ((int)threadIdx.x + NT * t < nq) ? s8 : 0.f;
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) nred[wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT / 64; j++) tot += nred[j];
+    const float nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      f32x4 l = l4[t], h = h4[t];
+      l.x = (l.x * nscale) * w0[t].x; l.y = (l.y * nscale) * w0[t].y; l.z = (l.z * nscale) * w0[t].z; l.w = (l.w * nscale) * w0[t].w;
+      h.x = (h.x * nscale) * w1[t].x; h.y = (h.y * nscale) * w1[t].y; h.z = (h.z * nscale) * w1[t].z; h.w = (h.w * nscale) * w1[t].w;
+      const int i = (int)threadIdx.x + NT * t;
+      if (i < nq) put_piece(i, pack8(l, h));
+    }
+    lds_to_regs();
+  } else if constexpr (PRO == 3) {
+    u32x4 v[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
+    issue(b[0], lo);
+#pragma unroll
+    for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
+    lds_to_regs();
+  } else {
+    if (a.x_staged) {
+      const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
+#pragma unroll
+      for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
+      issue(b[0], lo);
+      F::cfromx(xv, cv);
+    } else {
+      issue(b[0], lo);
+      // Loads of up to four (two) loop iterations are issued as one batch: a load per iteration would cost a memory round trip each.
+      float nscale = 1.f;
+      if (a.norm_w) {                                            // fused RMSNorm: sum of squares over the workgroup first
+        float ss = 0.f;
+        for (int p = threadIdx.x; p < 2 * nq; p += NT * 4) {
+          f32x4 v[4];
+#pragma unroll
+          for (int t = 0; t < 4; t++) { const int i = p + NT * t; v[t] = xr[i < 2 * nq ? i : 2 * nq - 1]; }
+#pragma unroll
+          for (int t = 0; t < 4; t++) if (p + NT * t < 2 * nq) ss += v[t].x * v[t].x + v[t].y * v[t].y + v[t].z * v[t].z + v[t].w * v[t].w;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) nred[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int j = 0; j < NT / 64; j++) tot += nred[j];
+        nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+      }
+      for (int p = threadIdx.x; p < nq; p += NT * 2) {
+        u32x4 v[2]; f32x4 lo4[2], hi4[2], w0[2], w1[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int i = p + NT * t < nq ? p + NT * t : nq - 1;
+          if (a.x_f32) {
+            lo4[t] = xr[2 * i]; hi4[t] = xr[2 * i + 1];
+            if (a.norm_w) { w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1]; }
+          } else v[t] = xh[i];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          const int i = p + NT * t;
+          if (i >= nq) break;
+          if (a.x_f32) {
+            f32x4 l = lo4[t], h = hi4[t];
+            if (a.norm_w) {
+              l.x = (l.x * nscale) * w0[t].x; l.y = (l.y * nscale) * w0[t].y; l.z = (l.z * nscale) * w0[t].z; l.w = (l.w * nscale) * w0[t].w;
+              h.x = (h.x * nscale) * w1[t].x; h.y = (h.y * nscale) * w1[t].y; h.z = (h.z * nscale) * w1[t].z; h.w = (h.w * nscale) * w1[t].w;
+            }
+            v[t] = pack8(l, h);
+          }
+          put_piece(i, v[t]);
+        }
+      }
+      lds_to_regs();
+    }
+  }
+  run_segment();
+  // (a branch around loads is harmless here: the ring is empty between segments)
+  for (int sg = 1; sg < nseg; sg++) { enter(sg); if (cnt) { issue(b[0], lo); run_segment(); } }
+}
+
+// ------------------------------------------------------------------------------------------------ host side
+static int fast_cu_count() {
+  static int n = 0;
+  if (!n) { int dev = 0; hipDeviceProp_t p; n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) ? p.multiProcessorCount : 256; }
+  return n;
+}
+
+template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
+static int launch_fast_p(const QArgs& a, long long grid, size_t lds, hipStream_t s) {
+  auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H, PRO>;
+  if (lds > 48 * 1024) {
+    static bool configured = false;
+    if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); configured = true; }
+  }
+  kern<<<dim3((unsigned)grid, (unsigned)(a.sel ? a.xdiv_jobs : 1)), dim3(WK * WR * 64), lds, s>>>(a);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int T, int R, int WK, int WR, int EPI, bool H = false>
+static int launch_fast(QArgs a, hipStream_t s) {
+  using F = Fmt<T>;
+  constexpr int RS = (EPI == 2) ? 1 : R;
+  constexpr int NT = WK * WR * 64;
+  const long long ngroups = (a.ntot + RS - 1) / RS;
+  const size_t lds = (size_t)a.nu * (F::UW / 2 + 4) * 4;
+  // row teams per CU: 8 waves (two 4-wave workgroups), fewer when the staged activations in LDS (160 KB per CU) say so.  Measured on
+  // the 8B decode step: 8 or 12 waves per CU 570 tok/s, 16 (all wave slots) 564, 4 553.
+  int wg_per_cu = (a.sel ? 16 : 8) / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;   // (expert jobs share the grid: all 16 wave slots there)
+  const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
+  constexpr int TPW = WR * (H ? 2 : 1);                           // row teams per workgroup
+  long long max_teams = (long long)fast_cu_count() * wg_per_cu * TPW;
+  if (a.sel && a.xdiv_jobs > 1) { max_teams = (max_teams + a.xdiv_jobs - 1) / a.xdiv_jobs; if (max_teams < 1) max_teams = 1; }
+  long long per = (ngroups + max_teams - 1) / max_teams;           // row groups per team
+  // short rows: a team should own a few row groups, so that the activation staging of its workgroup is paid once per several
+  // rows, as long as every CU still gets a workgroup
+  long long per_min = ngroups / ((long long)fast_cu_count() * TPW); per_min = per_min < 1 ? 1 : per_min > 4 ? 4 : per_min;
+  if (!a.sel && per < per_min) per = per_min;
+  const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
+  long long grid = (teams + TPW - 1) / TPW;
+  if (grid < 1) grid = 1;
+  // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
+  const bool one_batch = a.K / 8 <= NT * 2;
+  if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
+  if constexpr (WK == 1 && EPI != 1) {
+    if (!a.x_staged && one_batch && a.norm_w && a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 1>(a, grid, lds, s);
+    if (!a.x_staged && one_batch && !a.norm_w && !a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 3>(a, grid, lds, s);
+  }
+  return launch_fast_p<T, R, WK, WR, EPI, H, 0>(a, grid, lds, s);
+}
+
+static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
+template <int T, int WK, int WR, bool H = false>
+static int launch_fast_e(const QArgs& a, hipStream_t s) {
+  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
+  // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice.
+  // Measured per format at 14336 x 4096 and 4096 x 14336: two rows win for Q4_0, MXFP4, Q4_K (14.3 -> 11.4 us), Q5_K (18.1 -> 15.1 us)
+  // and slightly for Q6_K; Q8_0 pairs (68-byte units) are no faster with two.
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1) && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu() / WK;
+  if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
+  return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);
+}
+
+// entry point per weight format, instantiated in qgemv1_*.hip
+template <int T>
+int qgemv1_launch_format(QArgs a, hipStream_t s) {
+  using F = Fmt<T>;
+  a.nu = a.K / F::UW;
+  a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+  const int waves = (a.nu + 63) / 64;
+  if (a.nu <= 32) return launch_fast_e<T, 1, 4, true>(a, s);
+  if (waves <= 1) return launch_fast_e<T, 1, 4>(a, s);
+  if (waves <= 2) return launch_fast_e<T, 2, 1>(a, s);
+  if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);
+  if (waves <= 8) return launch_fast_e<T, 8, 1>(a, s);
+  return launch_fast_e<T, 16, 1>(a, s);
+}

@@ -1,0 +1,6 @@
+// M = 1 dequant-GEMV kernels of these weight formats (template in qgemv1.h)
+#include "qgemv1.h"
+
+template int qgemv1_launch_format<GGML_Q4_1>(QArgs, hipStream_t);
+template int qgemv1_launch_format<GGML_Q5_0>(QArgs, hipStream_t);
+template int qgemv1_launch_format<GGML_Q5_1>(QArgs, hipStream_t);
