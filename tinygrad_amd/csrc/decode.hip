@@ -138,16 +138,21 @@ __device__ __forceinline__ void block_sumsq2(const float* q, int nq, const float
 // query heads of the group.  A wave's K and V tiles are 16 rows in one shared register layout: load instruction i covers rows
 // i*RPI + lane / HD8 (RPI = 64 / HD8) and lane % HD8 picks the 16-byte piece, so a lane only needs the 8 query values of its
 // piece.  Scores: 8 FMAs per instruction, then a DPP sum over the HD8 lanes of a row.  Each run of HD8 lanes keeps its own
-// softmax partial (its rows only); the partials meet in LDS and leave as one partial per (head, split).  Both tiles are
-// requested before anything else; the row of the current token (not in the cache yet) is patched in from LDS.
-// Partials cross workgroups inside the launch, so they move through write-through stores and cache-bypassing loads, and the
-// arrival counter is a relaxed device-scope atomic after the stores have completed (no cache write-back / invalidate).
-template <int HD8>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
+// softmax partial (its rows only); the partials meet in LDS and leave as one partial per (head, split) with plain stores: the
+// merge over splits is a launch of its own (attn_merge_kernel).
+//
+// The kernel is a chain of latencies, not of bytes, so its loads are arranged as ONE round trip: everything that does not depend
+// on the position (this token's q / k / v rows and norm weights, then the cached K / V tiles with rows clamped to the cache, not to
+// the position) is requested first, in straight-line code and small loads first (loads return in issue order); the position is a
+// scalar load in flight meanwhile, and only the rotation row waits for it.  NORM selects the q/k RMSNorm at compile time so that no
+// load sits behind a branch (a join makes the compiler wait for every outstanding load):
+//   0 none, 1 over the whole q and k vectors of at most 4096 values each (read in one batch), 2 per head, 3 over whole vectors of any length
+template <int HD8, int NORM>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
+  const AttnArgs a = args;                              // field reads become kernel-argument loads in the entry block
   constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = 4 * RPI, CSTR = HD + 4;
+  constexpr int QPL = (HD / 2 + 63) / 64;               // query pairs per lane
   const int kvh = blockIdx.x, split = blockIdx.y;
-  const int pos = a.st->pos;
-  if (split * 64 > pos) return;                         // nothing cached in this split yet
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = HD >> 1, group = a.n_heads / a.n_kv;
   __shared__ float qs[4][HD];                           // rotated queries of the 4 heads in flight
@@ -156,51 +161,105 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
   __shared__ float red[8];
   const int vr = lane / HD8, vp = lane % HD8;
   const int p0 = split * 64 + wave * 16;                // first position of this wave
+  // ---- loads that do not depend on the position
+  const int ki = tid < half ? tid : half - 1;           // thread t rotates pair t of the key and copies element t of the value (head_dim <= 256)
+  const int vi = tid < HD ? tid : HD - 1;
+  const float kx1 = a.k[kvh * HD + ki], kx2 = a.k[kvh * HD + half + ki];
+  const float vx = a.v[kvh * HD + vi];
+  const int head0 = kvh * group + (wave < group ? wave : 0);   // the head whose query this wave rotates in the first pass
+  float qx1[QPL], qx2[QPL];
+#pragma unroll
+  for (int j = 0; j < QPL; j++) {
+    const int i = lane + 64 * j < half ? lane + 64 * j : half - 1;
+    qx1[j] = a.q[head0 * HD + i]; qx2[j] = a.q[head0 * HD + half + i];
+  }
+  float kw1 = 1.f, kw2 = 1.f, qw1[QPL], qw2[QPL];
+  if constexpr (NORM != 0) {                            // weight index = position in the whole vector, or inside the head for the per-head norm
+    const int kb = NORM == 2 ? 0 : kvh * HD, qb = NORM == 2 ? 0 : head0 * HD;
+    kw1 = a.k_norm[kb + ki]; kw2 = a.k_norm[kb + half + ki];
+#pragma unroll
+    for (int j = 0; j < QPL; j++) {
+      const int i = lane + 64 * j < half ? lane + 64 * j : half - 1;
+      qw1[j] = a.q_norm[qb + i]; qw2[j] = a.q_norm[qb + half + i];
+    }
+  }
+  f32x4 nq4[4], nk4[4];
+  if constexpr (NORM == 1) {                            // the whole q and k vectors for the sums of squares: four 16-byte pieces per thread each
+    const int n4q = (a.n_heads * HD) >> 2, n4k = (a.n_kv * HD) >> 2;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int i = tid + 256 * t;
+      nq4[t] = ((const f32x4*)a.q)[i < n4q ? i : n4q - 1]; nk4[t] = ((const f32x4*)a.k)[i < n4k ? i : n4k - 1];
+    }
+  }
   u32x4 kt[NVI], vt[NVI];
   {
     const _Float16* kbase = a.cache_k + (size_t)kvh * a.max_ctx * HD + vp * 8;
     const _Float16* vbase = a.cache_v + (size_t)kvh * a.max_ctx * HD + vp * 8;
 #pragma unroll
     for (int i = 0; i < NVI; i++) {
-      const int r = p0 + i * RPI + vr, rc = r < pos ? r : pos;   // rows >= pos are replaced below
+      const int r = p0 + i * RPI + vr, rc = r < a.max_ctx ? r : a.max_ctx - 1;   // rows from the position on are replaced or masked below
       kt[i] = *(const u32x4*)(kbase + (size_t)rc * HD);
       vt[i] = *(const u32x4*)(vbase + (size_t)rc * HD);
     }
   }
+  // ---- the position, and the one load that needs it
+  const int pos = a.st->pos;
+  if (split * 64 > pos) return;                         // nothing cached in this split yet
+  const float kc = a.rope[(size_t)pos * HD + ki], ksn = a.rope[(size_t)pos * HD + half + ki];
+  float qc[QPL], qsn[QPL];
+#pragma unroll
+  for (int j = 0; j < QPL; j++) {
+    const int i = lane + 64 * j < half ? lane + 64 * j : half - 1;
+    qc[j] = a.rope[(size_t)pos * HD + i]; qsn[j] = a.rope[(size_t)pos * HD + half + i];
+  }
+  // ---- norms
   float qscale = 1.f, kscale = 1.f;
-  const bool per_head = a.q_norm && a.norm_per_head;
-  if (a.q_norm && !per_head) {
+  if constexpr (NORM == 1) {
+    const int n4q = (a.n_heads * HD) >> 2, n4k = (a.n_kv * HD) >> 2;
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int i = tid + 256 * t;
+      const f32x4 x = nq4[t], y = nk4[t];
+      s0 += i < n4q ? x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w : 0.f;
+      s1 += i < n4k ? y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w : 0.f;
+    }
+    s0 = wave_sum(s0); s1 = wave_sum(s1);
+    if (lane == 0) { red[wave] = s0; red[4 + wave] = s1; }
+    __syncthreads();
+    qscale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)(a.n_heads * HD) + a.norm_eps);
+    kscale = 1.0f / sqrtf((red[4] + red[5] + red[6] + red[7]) / (float)(a.n_kv * HD) + a.norm_eps);
+  } else if constexpr (NORM == 3) {
     float sq, sk;
     block_sumsq2(a.q, a.n_heads * HD, a.k, a.n_kv * HD, red, sq, sk);
     qscale = 1.0f / sqrtf(sq / (float)(a.n_heads * HD) + a.norm_eps);
     kscale = 1.0f / sqrtf(sk / (float)(a.n_kv * HD) + a.norm_eps);
+  } else if constexpr (NORM == 2) {                     // the key of this kv head over the workgroup, the wave's query inside the wave
+    float sk = tid < half ? kx1 * kx1 + kx2 * kx2 : 0.f, sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < QPL; j++) sq += lane + 64 * j < half ? qx1[j] * qx1[j] + qx2[j] * qx2[j] : 0.f;
+    sk = wave_sum(sk); sq = wave_sum(sq);
+    if (lane == 0) red[wave] = sk;
+    __syncthreads();
+    kscale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)HD + a.norm_eps);
+    qscale = 1.0f / sqrtf(sq / (float)HD + a.norm_eps);
   }
-  if (per_head) {                                       // every wave sums this kv head's key for itself
-    float sk = 0.f;
-    for (int i = lane; i < HD; i += 64) { const float v = a.k[kvh * HD + i]; sk += v * v; }
-    kscale = 1.0f / sqrtf(wave_sum(sk) / (float)HD + a.norm_eps);
+  // normalised values for the later head passes (weights re-read there)
+  auto qval = [&](int i) { return NORM != 0 ? (a.q[i] * qscale) * a.q_norm[NORM == 2 ? i % HD : i] : a.q[i]; };
+  if (tid < half) {
+    const float x1 = NORM != 0 ? (kx1 * kscale) * kw1 : kx1, x2 = NORM != 0 ? (kx2 * kscale) * kw2 : kx2;
+    ks[tid] = x1 * kc - x2 * ksn; ks[half + tid] = x2 * kc + x1 * ksn;
   }
-  // normalised values: weight index = position in the whole vector, or inside the head for the per-head norm
-  auto qval = [&](int i) { return a.q_norm ? (a.q[i] * qscale) * a.q_norm[per_head ? i % HD : i] : a.q[i]; };
-  auto kval = [&](int i) { return a.k_norm ? (a.k[i] * kscale) * a.k_norm[per_head ? i % HD : i] : a.k[i]; };
-  // the query of this wave's first head pass is requested together with k, v and the rotation row (one memory round trip, not two)
-  constexpr int QPL = (HD / 2 + 63) / 64;               // query pairs per lane
-  float qx1[QPL], qx2[QPL], qc[QPL], qsn[QPL];
-  {
-    const int head = kvh * group + (wave < group ? wave : 0);
+  if (tid < HD) vs[tid] = vx;
+  if (wave < group) {                                   // first pass: wave w rotates the query of head w
 #pragma unroll
     for (int j = 0; j < QPL; j++) {
-      const int i = lane + 64 * j < half ? lane + 64 * j : half - 1;
-      qx1[j] = a.q[head * HD + i]; qx2[j] = a.q[head * HD + half + i];
-      qc[j] = a.rope[(size_t)pos * HD + i]; qsn[j] = a.rope[(size_t)pos * HD + half + i];
+      const int i = lane + 64 * j;
+      const float x1 = NORM != 0 ? (qx1[j] * qscale) * qw1[j] : qx1[j], x2 = NORM != 0 ? (qx2[j] * qscale) * qw2[j] : qx2[j];
+      if (i < half) { qs[wave][i] = x1 * qc[j] - x2 * qsn[j]; qs[wave][half + i] = x2 * qc[j] + x1 * qsn[j]; }
     }
   }
-  for (int i = tid; i < half; i += 256) {
-    const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
-    const float x1 = kval(kvh * HD + i), x2 = kval(kvh * HD + half + i);
-    ks[i] = x1 * c - x2 * s; ks[half + i] = x2 * c + x1 * s;
-  }
-  for (int i = tid; i < HD; i += 256) vs[i] = a.v[kvh * HD + i];
   __syncthreads();
   if ((pos >> 6) == split) {                            // owner split appends this token to the cache
     for (int i = tid; i < HD; i += 256) {
@@ -214,28 +273,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs a) {
     for (int i = 0; i < NVI; i++) if (p0 + i * RPI + vr >= pos) { kt[i] = kcur; vt[i] = vcur; }
   }
   for (int h0 = 0; h0 < group; h0 += 4) {
-    if (h0 == 0 && !a.q_norm) {                         // first pass without a norm: the values are already here
-      if (wave < group) {
-#pragma unroll
-        for (int j = 0; j < QPL; j++) {
-          const int i = lane + 64 * j;
-          if (i < half) { qs[wave][i] = qx1[j] * qc[j] - qx2[j] * qsn[j]; qs[wave][half + i] = qx2[j] * qc[j] + qx1[j] * qsn[j]; }
+    if (h0 > 0) {                                       // later passes (more than four query heads per kv head): rotate the next four
+      if (h0 + wave < group) {
+        const int head = kvh * group + h0 + wave;
+        if constexpr (NORM == 2) {
+          float sq = 0.f;
+          for (int i = lane; i < HD; i += 64) { const float v = a.q[head * HD + i]; sq += v * v; }
+          qscale = 1.0f / sqrtf(wave_sum(sq) / (float)HD + a.norm_eps);
+        }
+        for (int i = lane; i < half; i += 64) {
+          const float c = a.rope[(size_t)pos * HD + i], sn = a.rope[(size_t)pos * HD + half + i];
+          const float x1 = qval(head * HD + i), x2 = qval(head * HD + half + i);
+          qs[wave][i] = x1 * c - x2 * sn; qs[wave][half + i] = x2 * c + x1 * sn;
         }
       }
-    } else if (h0 + wave < group) {                     // wave w rotates the query of head h0 + w
-      const int head = kvh * group + h0 + wave;
-      if (per_head) {
-        float sq = 0.f;
-        for (int i = lane; i < HD; i += 64) { const float v = a.q[head * HD + i]; sq += v * v; }
-        qscale = 1.0f / sqrtf(wave_sum(sq) / (float)HD + a.norm_eps);
-      }
-      for (int i = lane; i < half; i += 64) {
-        const float c = a.rope[(size_t)pos * HD + i], s = a.rope[(size_t)pos * HD + half + i];
-        const float x1 = qval(head * HD + i), x2 = qval(head * HD + half + i);
-        qs[wave][i] = x1 * c - x2 * s; qs[wave][half + i] = x2 * c + x1 * s;
-      }
+      __syncthreads();
     }
-    __syncthreads();
 #pragma unroll
     for (int hh = 0; hh < 4; hh++) {
       if (h0 + hh < group) {
@@ -469,9 +522,14 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
   const dim3 grid(n_kv_heads, a.nsplit);
   hipStream_t s = (hipStream_t)stream;
-  if (head_dim == 64) attn_decode_kernel<8><<<grid, 256, 0, s>>>(a);
-  else if (head_dim == 128) attn_decode_kernel<16><<<grid, 256, 0, s>>>(a);
-  else attn_decode_kernel<32><<<grid, 256, 0, s>>>(a);
+  const int norm = !q_norm_weight ? 0 : norm_per_head ? 2 : ((long long)n_heads * head_dim <= 4096 && (long long)n_kv_heads * head_dim <= 4096) ? 1 : 3;
+#define TGA_ATTN_LAUNCH(HD8) do { \
+    if (norm == 0) attn_decode_kernel<HD8, 0><<<grid, 256, 0, s>>>(a); else if (norm == 1) attn_decode_kernel<HD8, 1><<<grid, 256, 0, s>>>(a); \
+    else if (norm == 2) attn_decode_kernel<HD8, 2><<<grid, 256, 0, s>>>(a); else attn_decode_kernel<HD8, 3><<<grid, 256, 0, s>>>(a); } while (0)
+  if (head_dim == 64) TGA_ATTN_LAUNCH(8);
+  else if (head_dim == 128) TGA_ATTN_LAUNCH(16);
+  else TGA_ATTN_LAUNCH(32);
+#undef TGA_ATTN_LAUNCH
   TGA_LAUNCH_CHECK();
   if (head_dim == 64) attn_merge_kernel<64><<<n_heads, 64, 0, s>>>(a);
   else if (head_dim == 128) attn_merge_kernel<128><<<n_heads, 128, 0, s>>>(a);

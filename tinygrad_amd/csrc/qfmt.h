@@ -27,6 +27,8 @@ struct QArgs {
   // norm_w != nullptr (M = 1 fast path, fp32 x): the activation row is RMS-normalised while it is staged,
   // x * rsqrt(mean(x^2) + norm_eps) * norm_w (nn.RMSNorm, tinygrad/nn/__init__.py:296-304), then rounded to fp16.
   const float* norm_w; float norm_eps;
+  // M = 1 fast path: row groups per team and the remainder (the first team_rem teams take one more), so that the kernel divides nothing
+  int team_base, team_rem;
 };
 
 // staged position of element e for a consumer of format `fmt` (row length K = UW * nu)

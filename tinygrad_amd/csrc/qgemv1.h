@@ -31,7 +31,10 @@
 //   PRO 2  activations already in the staged order of this format (written by the producing kernel)
 //   PRO 3  one fp16 row of at most two pieces per thread
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
-__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
+__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) {
+  // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
+  // issued together (read at their points of use they arrive in dependent stages, each a scalar-cache miss of its own).
+  const QArgs a = args;
   using F = Fmt<T>;
   typedef typename F::Raw Raw;
   static_assert(WK == 1 || WR == 1, "row teams and K split are not combined");
@@ -55,9 +58,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs a) {
   const long long eoff = a.sel ? (long long)a.sel[job] * a.estride : 0, yofs = (long long)job * a.ystride;
   const long long xrow = a.sel ? job / a.xdiv : 0;
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
-  const long long ngroups = (a.ntot + RS - 1) / RS;
-  const long long nteams = (long long)gridDim.x * WR * HM, team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
-  const long long gbase = ngroups / nteams, grem = ngroups % nteams;
+  const long long team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
+  const long long gbase = a.team_base, grem = a.team_rem;       // ngroups / teams and ngroups % teams, from the host
   const long long g0 = team * gbase + (team < grem ? team : grem), g1 = g0 + gbase + (team < grem ? 1 : 0);
   const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
   uint32_t kc[F::NKC];
@@ -333,6 +335,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
   const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
   long long grid = (teams + TPW - 1) / TPW;
   if (grid < 1) grid = 1;
+  { const long long nteams = grid * TPW; a.team_base = (int)(ngroups / nteams); a.team_rem = (int)(ngroups % nteams); }
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
   const bool one_batch = a.K / 8 <= NT * 2;
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
