@@ -20,8 +20,10 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 #define QM_THREADS 256
 #define QM_LDS_BUDGET (72 * 1024)     // activations of one chunk when two workgroups share a CU
 
-template <int T, int M>
-__global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs a) {
+template <int T_, int M>
+__global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args) {
+  const QArgs a = args;                                  // field reads become kernel-argument loads in the entry block
+  constexpr int T = T_;
   using F = Fmt<T>;
   typedef typename F::Raw Raw;
   extern __shared__ u32x4 lds[];
@@ -31,6 +33,78 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs a) {
   uint32_t kc[F::NKC];
   F::consts(kc);
   const long long ngroups = (a.ntot + 15) / 16;
+  if (a.nchunks == 1) {
+    // ---- the whole K in LDS: one software pipeline over ALL (row group, step) pairs of this wave.  Every load is unconditional and in
+    // straight-line code (steps past the end reload the last one; a step that does not exist for this wave - K / 4 units not a multiple
+    // of 4 steps - multiplies zeros), so the compiler's s_waitcnt placement keeps three steps in flight; a load behind a branch would
+    // make the waits behind the join wait for everything.
+    const int cu = a.nu, nsteps = (cu + 3) >> 2, spw = (nsteps + 3) >> 2;   // steps per wave and row group, the same for the four waves
+    const long long G = ((long long)blockIdx.x < ngroups) ? (ngroups - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const long long T = G * spw;
+    u32x4* xs = lds;
+    const bool ragged = (cu & 3) != 0 || (nsteps & 3) != 0;
+    Raw b[3];
+    long long lj = 0; int li = 0;                                       // load stream: row group index (of this workgroup), step index
+    auto issue = [&](Raw& buf) {
+      const long long grp = (long long)blockIdx.x + lj * gridDim.x;
+      const long long row = grp * 16 + r, rowc = row < a.ntot ? row : a.ntot - 1;
+      const int ul = 4 * (wave + 4 * li) + g;
+      buf = F::load(a.w[0] + rowc * a.row_bytes, ul < cu ? ul : cu - 1);
+      const bool more = lj * spw + li + 1 < T;                          // past the end: stay on the last step
+      li = more ? (li + 1 == spw ? 0 : li + 1) : li;
+      lj = more && li == 0 ? lj + 1 : lj;
+    };
+    if (T > 0) {
+      issue(b[0]);
+      stage_chunk<T_, M>(a, xs, (float*)(lds + M * F::XV * cu), 0, cu);
+      __syncthreads();
+      issue(b[1]);
+      v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+      long long cj = 0; int ci = 0;                                     // compute stream
+      auto compute = [&](const Raw& buf) {
+        const int ul = 4 * (wave + 4 * ci) + g;
+        uint32_t wv[F::NWV];
+        F::decode(buf, wv, kc);
+        F::to_f16(buf, wv);
+        const bool uval = ul < cu;
+        const int ulc = uval ? ul : cu - 1;
+#pragma unroll
+        for (int v = 0; v < F::XV; v++) {
+          u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
+          if (ragged && !uval) av = u32x4{0u, 0u, 0u, 0u};
+          u32x4 bv = {0u, 0u, 0u, 0u};
+          if (r < M) bv = xs[(r * F::XV + v) * cu + ulc];
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv), acc, 0, 0, 0);
+        }
+        if (++ci == spw) {                                              // row group complete: the four waves' partial tiles meet in LDS
+          const long long row0 = ((long long)blockIdx.x + cj * gridDim.x) * 16;
+#pragma unroll
+          for (int i = 0; i < 4; i++) part[wave][4 * g + i][r] = acc[i];
+          __syncthreads();
+          {
+            const int t = threadIdx.x, wr = t >> 4, c = t & 15;          // 256 threads = 16 weight rows x 16 activation rows
+            if (c < M && row0 + wr < a.ntot) {
+              const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
+              const long long o = (long long)c * a.ntot + row0 + wr;
+              if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+            }
+          }
+          __syncthreads();
+          acc = v4f32{0.f, 0.f, 0.f, 0.f};
+          ci = 0; cj++;
+        }
+      };
+      long long t = 0;
+      for (; t + 3 <= T; t += 3) {
+        issue(b[2]); compute(b[0]);
+        issue(b[0]); compute(b[1]);
+        issue(b[1]); compute(b[2]);
+      }
+      if (t < T) compute(b[0]);
+      if (t + 1 < T) compute(b[1]);
+    }
+    return;
+  }
   for (long long grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
     const long long row0 = grp * 16;
     const long long myrow = row0 + r < a.ntot ? row0 + r : a.ntot - 1;   // ragged last group: reload a valid row, results dropped
