@@ -207,6 +207,10 @@ int tga_moe_combine_rows(const void* z_bf16, const int32_t* dest_row, const floa
  * Requires M % 256 == 0, N % 256 == 0, K % 128 == 0 (moe_gemm.py:120).  Rows at or beyond expert_off[E] are left untouched. */
 int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
                            const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
+/* bias add after a grouped GEMM (examples/mlperf/models/gpt_oss.py:219-224, `+ (onehot @ bias.float()).cast(bf16)`): in place,
+ * h[r, :] = bf16(h[r, :] + bf16(bias[e(r), :])) with e(r) the expert of row r's 256-row tile (moe_routing.py:98-104); bias (E, N) float32;
+ * rows at or beyond expert_off[E] are left untouched.  M % 256 == 0. */
+int tga_add_expert_bias(void* h_bf16, const float* bias, const int32_t* expert_off, int64_t M, int64_t N, int n_experts, void* stream);
 /* clamped interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98), bf16 (rows, 2I) -> (rows, I). */
 int tga_swiglu_interleaved(const void* h_bf16, int64_t rows, int two_inter, float limit, float alpha, void* y_bf16, void* stream);
 

@@ -90,3 +90,12 @@ def grouped_mx_gemm_ref(x_q, x_e8, w_q, w_e8, expert_off):
       wd = to_bf16(dequant_mxfp8(w_q[e], w_e8[e])).astype(np.float64)
       out[lo:hi] = to_bf16((xd[lo:hi] @ wd.T).astype(np.float32))
   return out
+
+def add_expert_bias(h_bf16: np.ndarray, bias: np.ndarray, expert_off: np.ndarray) -> np.ndarray:
+  """examples/mlperf/models/gpt_oss.py:219-224: h + (onehot(rows_e) @ bias.float()).cast(bf16) as a bf16 tensor add; h holds bf16 values as
+  float32.  Rows beyond expert_off[E] get no bias here (the reference's rows_e maps them to the last expert; they are padding)."""
+  out = np.array(h_bf16, dtype=np.float32, copy=True)
+  for e in range(bias.shape[0]):
+    lo, hi = int(expert_off[e]), int(expert_off[e + 1])
+    if hi > lo: out[lo:hi] = to_bf16(out[lo:hi] + to_bf16(bias[e])[None, :])
+  return out

@@ -97,3 +97,28 @@ def test_grouped_mxfp8_gemm(gpu, E, N, K, rows):
   full = np.zeros_like(ref)
   for e in range(E): full[off[e]:off[e + 1]] = x[off[e]:off[e + 1]] @ w[e].T
   assert np.abs(got[:used] - full[:used]).mean() / np.abs(full[:used]).mean() < 6e-2
+
+def test_dense_mx_gemm_and_expert_bias(gpu):
+  """The dense MXFP8 GEMM (one expert owning every row) against the oracle's matmul_mx semantics, then the per-expert bias add of
+  gpt_oss.py:219-224 on a grouped result (bias cast to bf16, bf16 add), bit for bit."""
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(12)
+  M, N, K = 512, 256, 256
+  x = moe.to_bf16_bits((rng.standard_normal((M, K)) * 0.5).astype(np.float32))
+  w = (rng.standard_normal((N, K)) * 0.5).astype(np.float32)
+  wq, we8 = omx.quantize_mxfp8(w)
+  out = moe.mx_gemm(gpu.Buffer.from_numpy(x), (gpu.Buffer.from_numpy(wq), gpu.Buffer.from_numpy(we8)))
+  xq, xe8 = omx.quantize_mxfp8(moe.from_bf16_bits(x))
+  ref = omx.grouped_mx_gemm_ref(xq, xe8, wq[None], we8[None], np.array([0, M], np.int32))
+  got = moe.from_bf16_bits(out.numpy())
+  np.testing.assert_allclose(got, ref, rtol=2 ** -7, atol=1e-3 * np.abs(ref).max())
+  # bias by expert on three experts' tiles, the last tile unrouted
+  E = 3
+  off = np.array([0, 256, 256, 512], dtype=np.int32)                 # expert 1 owns no rows
+  h = moe.to_bf16_bits(rng.standard_normal((768, N)).astype(np.float32))
+  bias = rng.standard_normal((E, N)).astype(np.float32)
+  hb = gpu.Buffer.from_numpy(h)
+  moe.add_expert_bias(hb, gpu.Buffer.from_numpy(bias), gpu.Buffer.from_numpy(off))
+  exp = omx.add_expert_bias(moe.from_bf16_bits(h), bias, off)
+  np.testing.assert_array_equal(hb.numpy(), moe.to_bf16_bits(exp))
+  assert (hb.numpy()[512:] == h[512:]).all()                         # rows beyond the routed range untouched

@@ -376,6 +376,21 @@ __global__ __launch_bounds__(256) void swiglu_interleaved_kernel(const uint16_t*
   }
 }
 
+// h[r, :] += bias[e(r), :] for the rows of every expert (examples/mlperf/models/gpt_oss.py:219-224: `+ (onehot @ bias.float()).cast(bf16)`
+// after each grouped GEMM): the bias row is cast to bf16 first and the sum of the two bf16 values is rounded to bf16, as the reference's
+// bf16 tensor add does.  Rows are located by 256-row tile (Routing.rows_e, moe_routing.py:98-104); rows at or beyond off[E] are left alone.
+__global__ __launch_bounds__(256) void add_expert_bias_kernel(uint16_t* __restrict__ h, const float* __restrict__ bias, const int* __restrict__ off, int n_experts, int N) {
+  const int tile = blockIdx.y, row0 = tile * 256;
+  if (row0 >= off[n_experts]) return;
+  int lo = 0, hi = n_experts;
+  while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (off[mid] <= row0) lo = mid; else hi = mid; }
+  const float* b = bias + (size_t)lo * N;
+  for (int c = blockIdx.x * 256 + threadIdx.x; c < N; c += gridDim.x * 256) {
+    const float bv = bf16_to_f(f_to_bf16(b[c]));
+    for (int r = 0; r < 256; r++) { uint16_t* p = h + (size_t)(row0 + r) * N + c; *p = f_to_bf16(bf16_to_f(*p) + bv); }
+  }
+}
+
 extern "C" {
 
 int tga_quantize_mxfp8(const void* x, int x_is_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream) {
@@ -453,6 +468,16 @@ int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_
   if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)grouped_mxfp8_gemm_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GG_STAGE_BYTES)); configured = true; }
   const long long tiles = ((M / GG_TILE) * (N / GG_TILE) + 7) / 8 * 8;     // workgroup b serves XCD b % 8
   grouped_mxfp8_gemm_lds_kernel<<<(unsigned)tiles, GG_THREADS, 2 * GG_STAGE_BYTES, (hipStream_t)stream>>>(g);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_add_expert_bias(void* h_bf16, const float* bias, const int32_t* expert_off, int64_t M, int64_t N, int n_experts, void* stream) {
+  TGA_REQUIRE(h_bf16 && bias && expert_off, "tga_add_expert_bias: null pointer");
+  TGA_REQUIRE(M >= 0 && M % 256 == 0 && N > 0 && n_experts >= 1, "tga_add_expert_bias: M=%lld must be a multiple of 256", (long long)M);
+  if (M == 0) return 0;
+  const int gx = (int)((N + 255) / 256 < 64 ? (N + 255) / 256 : 64);
+  add_expert_bias_kernel<<<dim3(gx, (unsigned)(M / 256)), 256, 0, (hipStream_t)stream>>>((uint16_t*)h_bf16, bias, expert_off, n_experts, (int)N);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -87,6 +87,23 @@ def grouped_mx_gemm(x: Buffer, w: tuple[Buffer, Buffer], expert_off: Buffer, str
   o._keep = (x_q, x_e8, x_si)
   return o
 
+def mx_gemm(x: Buffer, w: tuple[Buffer, Buffer], stream=None, out: Buffer | None = None) -> Buffer:
+  """The dense MXFP8 GEMM (hk_mxfp8_gemm, extra/gemm/cdna_asm_gemm.py:91-110): x (M, K) bf16 bits is quantized to MXFP8 and multiplied with
+  w = (w_q (N, K) e4m3 bits, w_e8 (N, K/32)) -> (M, N) bf16 bits.  One expert that owns every row: the grouped kernel with E = 1."""
+  w_q, w_e8 = w
+  (N, K), M = w_q.shape, x.shape[0]
+  off = Buffer.from_numpy(np.array([0, M], dtype=np.int32))
+  o = grouped_mx_gemm(x, (w_q.view(0, (1, N, K), np.uint8), w_e8.view(0, (1, N, K // 32), np.uint8)), off, stream, out)
+  o._keep = (*o._keep, off)
+  return o
+
+def add_expert_bias(h: Buffer, bias: Buffer, expert_off: Buffer, stream=None) -> Buffer:
+  """`+ (onehot @ bias.float()).cast(bf16)` after a grouped GEMM (examples/mlperf/models/gpt_oss.py:219-224), in place on h (M, N) bf16 bits;
+  bias (E, N) float32."""
+  M, N = h.shape
+  rt.check(rt.lib().tga_add_expert_bias(h.ptr, bias.ptr, expert_off.ptr, M, N, bias.shape[0], stream))
+  return h
+
 def swiglu(h: Buffer, limit: float = 7.0, alpha: float = 1.702, stream=None) -> Buffer:
   rows, two_i = h.shape
   y = Buffer((rows, two_i // 2), np.uint16)

@@ -44,6 +44,7 @@ def _declare(lib):
     "tga_moe_combine_rows": [vp, vp, vp, i, i, i, vp, vp],
     "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
     "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
+    "tga_add_expert_bias": [vp, vp, vp, i64, i64, i, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
