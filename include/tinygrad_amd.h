@@ -136,9 +136,9 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
 /* One token of TransformerBlock._attention after the q/k/v projections (model.py:180-197): half-split RoPE of q and k with the
  * freqs_cis table rope_table[max_ctx][head_dim] = cos half | sin half (model.py:16-19, 29-33), fp16 KV append at state.pos
  * (cache layout [n_kv_heads][max_ctx][head_dim]), GQA scaled-dot-product attention over positions 0..pos with softmax in
- * float32 (tinygrad/mixin/rand.py:298-327).  head_dim is 64, 128 or 256.  partials: workspace of
- * n_heads * ceil(max_ctx/64) * (head_dim + 2) floats followed by n_kv_heads int32 arrival counters that must be ZERO before the
- * first call (each call leaves them zero again); calls sharing one workspace must not overlap.
+ * float32 (tinygrad/mixin/rand.py:298-327).  head_dim is 64, 128 or 256.  Two launches: softmax partials per 64-position split,
+ * then their merge per query head.  partials: workspace of at least n_heads * ceil(max_ctx/64) * (head_dim + 2) floats that carries
+ * the split partials from the first launch to the second; calls sharing one workspace must not overlap.
  * stage_type != 0: out_f16 is written in the staged order of a consumer weight of that type with K = n_heads * head_dim. */
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
                          int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);

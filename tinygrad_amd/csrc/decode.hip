@@ -84,11 +84,11 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__
 // (tinygrad/llm/model.py:29-33) using the caller's freqs_cis table [max_ctx][hd] = cos half | sin half (precompute_freqs_cis,
 // model.py:16-19); the split that contains `pos` writes the rotated k and v into the fp16 cache.  With q_norm / k_norm the
 // full-width RMSNorm of model.py:169 (attn_q_norm / attn_k_norm over all heads at once) is applied to q and k first.
-// Softmax partials per split (max, sum, weighted V) go to `part`; the last split of a kv head to finish merges them.
+// Softmax partials per split (max, sum, weighted V) go to `part`; attn_merge_kernel, the next launch, merges them per query head.
 struct AttnArgs {
   const float* q; const float* k; const float* v;     // this token's projections: [n_heads*hd], [n_kv*hd], [n_kv*hd]
   _Float16* cache_k; _Float16* cache_v;                // [n_kv][max_ctx][hd]
-  float* part;                                         // [n_heads][nsplit][hd + 2], then n_kv int32 arrival counters (zero between launches)
+  float* part;                                         // [n_heads][nsplit][hd + 2]
   const DecodeState* st;
   int n_heads, n_kv, hd, max_ctx, nsplit;
   const float* rope;                                   // [max_ctx][hd]: cos(pos * f_i) for i < hd/2, then sin(pos * f_i)

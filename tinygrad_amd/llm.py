@@ -203,7 +203,7 @@ class _Shared:
     self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
     self.sync = Buffer((320,), np.uint32).zero_()                        # device-wide barrier counters + error flag of the fused launch
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
-    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters
+    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters of the one-launch block kernel
     self.act = Buffer((1, c.hidden_dim), f16)
     if c.num_experts:
       k = c.num_experts_per_tok
