@@ -91,6 +91,13 @@ int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml
                               const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
                               int y_stage_type, int64_t y_stage_K, void* stream);
 
+/* tga_rmsnorm_qlinear_multi on the row x_in + sum_j probs[j] * y_experts[j]: the MoE weighted sum over the selected experts' outputs and
+ * the block residual (tinygrad/llm/model.py:130, 150) folded into the next block's attn_norm -> attn_q/k/v launch (or output_norm -> output).
+ * The completed row is written to x_out, which must not alias x_in.  y_experts (k, K) and probs (k) float32, k <= 8, K <= 2048, plain epilogue. */
+int tga_moe_combine_rmsnorm_qlinear_multi(const float* y_experts, const float* probs, int k, const float* x_in, float* x_out,
+                                          const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y,
+                                          const int64_t* n, int y_dtype, int64_t K, void* stream);
+
 /* Staged activations (no counterpart in the reference; an M = 1 fast path): the decode GEMV keeps each lane's activations in
  * registers in the order its in-register decode produces weights, which is a fixed permutation of the row that depends on the
  * weight's (ggml_type, K).  tga_stage_activation writes that permutation as fp16 (K values); a linear then takes it with

@@ -82,6 +82,32 @@ def test_router_in_one_launch(gpu, dim, E, k, gating, normw):
   np.testing.assert_array_equal(sel.numpy(), rs[0])
   np.testing.assert_allclose(pr.numpy(), rp[0], rtol=2e-5, atol=1e-7)
 
+@pytest.mark.parametrize("t,dim,k", [(1, 2048, 8), (2, 1024, 4), (14, 512, 1), (39, 2048, 6)])
+def test_weighted_expert_sum_folded_into_the_next_linear(gpu, t, dim, k):
+  """tga_moe_combine_rmsnorm_qlinear_multi against tga_moe_combine followed by tga_rmsnorm_qlinear_multi: same completed row (bit for
+  bit: the same products in the same order), same linear outputs up to the summation order of the mean square."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi, moe_combine
+  rng = np.random.default_rng(dim + k + t)
+  ns = [192, 64]
+  if t == 1: ws = [(rng.standard_normal((n, dim)) * dim ** -0.5).astype(np.float16).view(np.uint8).reshape(-1) for n in ns]
+  else: ws = [synth.random_blocks(rng, t, n, dim) for n in ns]
+  layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, dim) for w, n in zip(ws, ns)]
+  x = rng.standard_normal((1, dim)).astype(np.float32); y = rng.standard_normal((k, dim)).astype(np.float32); p = rng.random(k).astype(np.float32)
+  nw = rng.standard_normal(dim).astype(np.float32)
+  xb, yb, pb, nwb = (gpu.Buffer.from_numpy(a) for a in (x, y, p, nw))
+  x_out = gpu.Buffer((1, dim), np.float32).zero_()
+  fused = [gpu.Buffer((1, n), np.float32) for n in ns]
+  qlinear_multi(layers, xb, fused, norm=(nwb, 1e-5), combine=(yb, pb, k, x_out))
+  x_ref = gpu.Buffer((1, dim), np.float32)
+  moe_combine(yb, pb, xb, 1, k, dim, x_ref)
+  plain = [gpu.Buffer((1, n), np.float32) for n in ns]
+  qlinear_multi(layers, x_ref, plain, norm=(nwb, 1e-5))
+  np.testing.assert_allclose(x_out.numpy(), x_ref.numpy(), rtol=1e-6, atol=1e-6)
+  np.testing.assert_allclose(x_out.numpy(), x + (y * p[:, None]).sum(0, keepdims=True), rtol=1e-5, atol=1e-5)
+  assert xb.numpy().tobytes() == x.tobytes()                           # the input row is left alone
+  for f, q in zip(fused, plain): assert ol.rel_err(f.numpy(), q.numpy()) <= 2e-4
+  with pytest.raises(RuntimeError): qlinear_multi(layers, xb, fused, norm=(nwb, 1e-5), combine=(yb, pb, 9, x_out))
+
 def test_moe_combine(gpu):
   from tinygrad_amd.nn import moe_combine
   rng = np.random.default_rng(3)

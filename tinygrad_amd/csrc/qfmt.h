@@ -27,6 +27,10 @@ struct QArgs {
   // norm_w != nullptr (M = 1 fast path, fp32 x): the activation row is RMS-normalised while it is staged,
   // x * rsqrt(mean(x^2) + norm_eps) * norm_w (nn.RMSNorm, tinygrad/nn/__init__.py:296-304), then rounded to fp16.
   const float* norm_w; float norm_eps;
+  // comb_y != nullptr (with norm_w): the activation row is first completed as x + sum_j comb_p[j] * comb_y[j] over comb_k rows of K values
+  // (the weighted sum over the selected experts' outputs plus the block residual, tinygrad/llm/model.py:130, 150); the completed row is
+  // also written to comb_x_out (a different buffer: every workgroup reads x) by the first workgroup.
+  const float* comb_y; const float* comb_p; int comb_k; float* comb_x_out;
   // M = 1 fast path: row groups per team and the remainder (the first team_rem teams take one more), so that the kernel divides nothing
   int team_base, team_rem;
 };

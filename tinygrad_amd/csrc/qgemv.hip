@@ -349,7 +349,8 @@ extern "C" int tga_stage_activation(int ggml_type, const void* x, int x_dtype, i
   return 0;
 }
 
-static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+struct CombineIn { const float* y; const float* p; int k; float* x_out; };
+static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
@@ -390,6 +391,11 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
     TGA_REQUIRE(M == 1 && x_dtype == TGA_F32 && ((uintptr_t)norm_w & 15) == 0, "tga_rmsnorm_qlinear: needs M = 1, float32 x and a 16-byte aligned norm weight");
     a.norm_w = norm_w; a.norm_eps = norm_eps;
   }
+  if (comb) {
+    TGA_REQUIRE(norm_w && comb->y && comb->p && comb->x_out && comb->k >= 1 && comb->k <= 8 && epilogue == 0, "tga_moe_combine_rmsnorm_qlinear_multi: needs the norm, 1..8 summands and the plain epilogue");
+    TGA_REQUIRE(((((uintptr_t)comb->y | (uintptr_t)comb->x_out | (uintptr_t)x) & 15) == 0) && K % 8 == 0, "tga_moe_combine_rmsnorm_qlinear_multi: rows must be 16-byte aligned");
+    a.comb_y = comb->y; a.comb_p = comb->p; a.comb_k = comb->k; a.comb_x_out = comb->x_out;
+  }
   hipStream_t s = (hipStream_t)stream;
   // block-pair units need an even number of blocks per row and 4-byte aligned rows
   bool pair = (K / 32) % 2 == 0;
@@ -402,6 +408,7 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemm_mfma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
   }
+  TGA_REQUIRE(!comb, "tga_moe_combine_rmsnorm_qlinear_multi: needs the M = 1 fast path with K <= 2048");
   TGA_REQUIRE(!norm_w, "tga_rmsnorm_qlinear: the fused norm needs the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, 16-byte aligned x, K <= 65536)");
   TGA_REQUIRE(!a.x_staged && !a.y_stage_fmt, "tga_qlinear: staged activations need the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, K <= 65536)");
   switch (ggml_type) {
@@ -421,7 +428,7 @@ static int qlinear_multi_impl(const float* norm_w, float norm_eps, int ggml_type
 extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                  const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                                  int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
-  return qlinear_multi_impl(nullptr, 0.f, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+  return qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, y_stage_type, y_stage_K, stream);
 }
 
 // RMSNorm (nn.RMSNorm, tinygrad/nn/__init__.py:296-304) of the float32 activation row folded into the M = 1 linear that consumes it
@@ -431,7 +438,19 @@ extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_ep
                                          const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
                                          int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(norm_weight, "tga_rmsnorm_qlinear_multi: null norm weight");
-  return qlinear_multi_impl(norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+  return qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+}
+
+// The MoE weighted sum and block residual (x += sum_j probs[j] * y[j], tinygrad/llm/model.py:130, 150) folded into the launch that
+// consumes the completed row: tga_rmsnorm_qlinear_multi on x_in + sum_j probs[j] * y[j], with the completed row written to x_out (by
+// one workgroup) for the residual adds that follow.  x_out must not be x_in: every workgroup reads x_in while one writes x_out.
+// y: (k, K) float32 rows, probs: k float32, k <= 8, K <= 2048.
+extern "C" int tga_moe_combine_rmsnorm_qlinear_multi(const float* y_experts, const float* probs, int k, const float* x_in, float* x_out,
+                                                     const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y,
+                                                     const int64_t* n, int y_dtype, int64_t K, void* stream) {
+  TGA_REQUIRE(norm_weight && y_experts && probs && x_in && x_out && x_in != x_out, "tga_moe_combine_rmsnorm_qlinear_multi: null pointer, or x_out aliases x_in");
+  const CombineIn c = {y_experts, probs, k, x_out};
+  return qlinear_multi_impl(&c, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x_in, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
 }
 
 extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,

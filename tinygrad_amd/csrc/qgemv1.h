@@ -30,6 +30,8 @@
 //          squares and the scaling)
 //   PRO 2  activations already in the staged order of this format (written by the producing kernel)
 //   PRO 3  one fp16 row of at most two pieces per thread
+//   PRO 5  PRO 1 for a row of at most one piece per thread that is first completed as x + sum_j p_j y_j (the MoE weighted sum and block
+//          residual that precede the next block's attn_norm): the launch that would only add vectors disappears
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
 __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) {
   // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
@@ -193,6 +195,39 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
     issue(b[0], lo);
     F::cfromx(xv, cv);
+  } else if constexpr (PRO == 5) {
+    constexpr int CK = 8;                                        // rows of the weighted sum (fewer: the surplus ones reload row 0 with weight 0)
+    const int i = (int)threadIdx.x < nq ? (int)threadIdx.x : nq - 1;
+    f32x4 l = xr[2 * i], h = xr[2 * i + 1];
+    const f32x4 w0 = ((const f32x4*)a.norm_w)[2 * i], w1 = ((const f32x4*)a.norm_w)[2 * i + 1];
+    f32x4 yl[CK], yh[CK]; float pj[CK];
+#pragma unroll
+    for (int j = 0; j < CK; j++) {
+      const int jc = j < a.comb_k ? j : 0;
+      const f32x4* yr = (const f32x4*)(a.comb_y + (size_t)jc * a.K);
+      yl[j] = yr[2 * i]; yh[j] = yr[2 * i + 1];
+      pj[j] = a.comb_p[jc];
+    }
+    issue(b[0], lo);
+#pragma unroll
+    for (int j = 0; j < CK; j++) {
+      const float p = j < a.comb_k ? pj[j] : 0.f;
+      l.x += p * yl[j].x; l.y += p * yl[j].y; l.z += p * yl[j].z; l.w += p * yl[j].w;
+      h.x += p * yh[j].x; h.y += p * yh[j].y; h.z += p * yh[j].z; h.w += p * yh[j].w;
+    }
+    if (blockIdx.x == 0 && blockIdx.y == 0 && (int)threadIdx.x < nq) { ((f32x4*)a.comb_x_out)[2 * i] = l; ((f32x4*)a.comb_x_out)[2 * i + 1] = h; }
+    float ss = (int)threadIdx.x < nq ? l.x * l.x + l.y * l.y + l.z * l.z + l.w * l.w + h.x * h.x + h.y * h.y + h.z * h.z + h.w * h.w : 0.f;
+    ss = wave_sum(ss);
+    if (lane == 0) nred[wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT / 64; j++) tot += nred[j];
+    const float nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+    l.x = (l.x * nscale) * w0.x; l.y = (l.y * nscale) * w0.y; l.z = (l.z * nscale) * w0.z; l.w = (l.w * nscale) * w0.w;
+    h.x = (h.x * nscale) * w1.x; h.y = (h.y * nscale) * w1.y; h.z = (h.z * nscale) * w1.z; h.w = (h.w * nscale) * w1.w;
+    if ((int)threadIdx.x < nq) put_piece((int)threadIdx.x, pack8(l, h));
+    lds_to_regs();
   } else if constexpr (PRO == 1) {
     f32x4 l4[2], h4[2], w0[2], w1[2];
 #pragma unroll
@@ -339,6 +374,13 @@ static int launch_fast(QArgs a, hipStream_t s) {
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
   const bool one_batch = a.K / 8 <= NT * 2;
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
+  if constexpr (WK == 1 && EPI == 0) {
+    if (a.comb_y) {
+      if (a.x_staged || !a.norm_w || !a.x_f32 || a.K / 8 > NT || a.comb_k > 8) return tga_set_error("tga_moe_combine_rmsnorm_qlinear_multi: needs one float32 row of at most %d values and at most 8 summands", 8 * NT);
+      return launch_fast_p<T, R, WK, WR, EPI, H, 5>(a, grid, lds, s);
+    }
+  }
+  if (a.comb_y) return tga_set_error("tga_moe_combine_rmsnorm_qlinear_multi: shape outside the fused path (K = %d)", a.K);
   if constexpr (WK == 1 && EPI != 1) {
     if (!a.x_staged && one_batch && a.norm_w && a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 1>(a, grid, lds, s);
     if (!a.x_staged && one_batch && !a.norm_w && !a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 3>(a, grid, lds, s);

@@ -144,14 +144,26 @@ class TransformerBlock:
     self.stage_attn = fast(self.attn_output)
     self.stage_act = (not self.moe) and fast(self.ffn_down)
     self.stage_xn = (not self.moe) and fast(self.ffn_gate) and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
+    # the previous block's weighted expert sum can be completed inside this block's q/k/v launch (one 8-value piece per thread: dim <= 2048)
+    self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
+                            and 0 < c.num_experts_per_tok <= 8
     if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
 
-  def __call__(self, x: Buffer, stream):
+  def __call__(self, x: Buffer, stream, pending: bool = False, defer: bool = False) -> tuple[Buffer, bool]:
+    """One block on the residual row x.  pending: the previous (MoE) block left its weighted expert sum + residual to this block
+    (expert outputs in s.y_e, weights in s.probs).  defer: leave this block's own weighted sum to the next launch.  Returns the buffer
+    that holds the residual row afterwards and whether a weighted sum is still pending."""
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     qkv, qkv_out = [self.attn_q, self.attn_k, self.attn_v], [s.q, s.k, s.v]
     same = self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type
-    if self.fuse_norm and same:                                          # the q/k/v launch normalises the row while staging it
+    if pending and not self.can_fold_combine:
+      moe_combine(s.y_e, s.probs, x, 1, c.num_experts_per_tok, c.dim, x, stream=stream); pending = False
+    if pending:                                                          # x + sum_j probs_j y_j completed inside the q/k/v launch, written to the other row buffer
+      x_new = s.x2 if x.ptr == s.x.ptr else s.x
+      qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps), combine=(s.y_e, s.probs, c.num_experts_per_tok, x_new))
+      x = x_new
+    elif self.fuse_norm and same:                                        # the q/k/v launch normalises the row while staging it
       qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps))
     else:
       rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
@@ -176,7 +188,7 @@ class TransformerBlock:
         rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if self.stage_xn else 0, stream))
         qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=self.stage_xn, stage_out_for=self.ffn_down if self.stage_act else None)
       qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_act)
-      return
+      return x, False
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
     if self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024:
@@ -189,7 +201,9 @@ class TransformerBlock:
       moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
     self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
     self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
+    if defer: return x, True                                            # the consumer of the completed row adds sum_j probs_j y_j + x itself
     moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)
+    return x, False
 
 class _Shared:
   """Activation buffers shared by all blocks (batch 1)."""
@@ -197,6 +211,7 @@ class _Shared:
     f32, f16 = np.float32, np.float16
     self.state = Buffer((16,), np.int32).zero_()
     self.x = Buffer((1, c.dim), f32)
+    self.x2 = Buffer((1, c.dim), f32)                                    # second residual row: a launch that completes x + sum_j p_j y_j writes here
     self.xn = Buffer((1, c.dim), f16)
     nq, nkv = c.n_heads * c.head_dim, c.n_kv_heads * c.head_dim
     self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v, contiguous for the fused block launch
@@ -229,6 +244,7 @@ class Transformer:
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
     self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
+    self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.num_experts_per_tok <= 8
     self.stream = rt.Stream()
     self._graphs = {}
     # optional: one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
@@ -262,13 +278,21 @@ class Transformer:
     if self.layer_table is not None:
       rt.check(L.tga_decode_layers(self.layer_table.ptr, c.num_blocks, self.layer_type, s.x.ptr, s.qkv.ptr, s.attn.ptr, s.act.ptr, s.attn_part.ptr,
                                    s.state.ptr, s.rope.ptr, s.sync.ptr, c.dim, c.hidden_dim, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, c.norm_eps, st))
-    else:
-      for b in self.blk: b(s.x, st)
+    x, pending = s.x, False
+    if self.layer_table is None:
+      nb = len(self.blk)
+      for i, b in enumerate(self.blk):
+        nxt = self.blk[i + 1].can_fold_combine if i + 1 < nb else (with_head and self.can_fold_head)
+        x, pending = b(x, st, pending, defer=nxt)
     if with_head:
-      if self.fuse_head_norm:                                          # output_norm inside the lm-head launch (model.py:362)
-        qlinear_multi([self.output], s.x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps))
+      if pending:                                                      # the last block's weighted sum completed inside the lm-head launch
+        x_new = s.x2 if x.ptr == s.x.ptr else s.x
+        qlinear_multi([self.output], x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps), combine=(s.y_e, s.probs, c.num_experts_per_tok, x_new))
+        x = x_new
+      elif self.fuse_head_norm:                                        # output_norm inside the lm-head launch (model.py:362)
+        qlinear_multi([self.output], x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps))
       else:
-        rt.check(L.tga_rmsnorm(s.x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
+        rt.check(L.tga_rmsnorm(x.ptr, self.output_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, st))
         self.output(s.xn, out=s.logits, stream=st)
       rt.check(L.tga_argmax_step(s.logits.ptr, c.vocab_size, s.am_v.ptr, s.am_i.ptr, s.state.ptr, s.prompt.ptr, s.out_tokens.ptr, self.max_new, st))
     else:

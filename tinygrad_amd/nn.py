@@ -32,12 +32,15 @@ class QuantLinear:
     return out
 
 def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None,
-                  x_staged: bool = False, stage_out_for: QuantLinear | None = None, norm: tuple[Buffer, float] | None = None):
+                  x_staged: bool = False, stage_out_for: QuantLinear | None = None, norm: tuple[Buffer, float] | None = None,
+                  combine: tuple[Buffer, Buffer, int, Buffer] | None = None):
   """Several QuantLinear layers over the same activation in one launch (attn_q/k/v, ffn_gate/ffn_up).
   epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x).
   x_staged: x is already in the staged order of these weights (stage_activation or a staging producer).
   stage_out_for: write the single fp16 output in the staged order of that consumer layer.
-  norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it."""
+  norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it.
+  combine = (y, probs, k, x_out) with norm: the row is first completed as x + sum_j probs[j] * y[j] (the MoE weighted sum + residual) and
+  the completed row is written to x_out (a buffer other than x)."""
   nseg = len(layers)
   t, k = layers[0].ggml_type, layers[0].in_features
   assert all(l.ggml_type == t and l.in_features == k for l in layers)
@@ -49,6 +52,11 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   r = VP(*[b.ptr for b in resid]) if resid is not None else None
   ydt = rt.dtype_code(outs[0].dtype)
   so = stage_out_for
+  if combine is not None:
+    assert norm is not None and m == 1 and x.dtype == np.float32 and not x_staged and epilogue == 0 and so is None and combine[3].ptr != x.ptr
+    rt.check(rt.lib().tga_moe_combine_rmsnorm_qlinear_multi(combine[0].ptr, combine[1].ptr, combine[2], x.ptr, combine[3].ptr, norm[0].ptr, norm[1],
+                                                            t, nseg, w, y, n, ydt, k, stream))
+    return outs
   if norm is not None:
     assert m == 1 and x.dtype == np.float32 and not x_staged
     rt.check(rt.lib().tga_rmsnorm_qlinear_multi(norm[0].ptr, norm[1], t, nseg, w, y, n, x.ptr, ydt, k, epilogue, r,
