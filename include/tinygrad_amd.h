@@ -26,7 +26,9 @@ extern "C" {
 #define TGA_Q4_K 12
 #define TGA_Q5_K 13
 #define TGA_Q6_K 14
+#define TGA_IQ4_XS 23   /* tga_dequant only */
 #define TGA_MXFP4 39
+#define TGA_Q1_0 41     /* tga_dequant only */
 /* activation dtype code: fp16 values in the staged order of the consuming weight (see tga_stage_activation) */
 #define TGA_F16_STAGED 101
 
@@ -57,7 +59,7 @@ int tga_graph_end(void* stream, void** graph_exec);
 int tga_graph_launch(void* graph_exec, void* stream);
 int tga_graph_destroy(void* graph_exec);
 
-/* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 3, 6, 7, 8, 12, 13, 14, 39) ----
+/* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 41) ----
  * blocks: device pointer to the raw GGUF tensor bytes; n: number of elements (multiple of the block size).
  * out_dtype TGA_F32: bit-exact ggml_data_to_tensor result.  TGA_F16: that result cast to fp16 round-to-nearest-even,
  * i.e. the weight the model path holds after tinygrad/llm/model.py:376. */

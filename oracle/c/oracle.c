@@ -91,6 +91,25 @@ static void deq_q5(const uint8_t* b, float* y, int one) {
     y[j] = (float)x0 * d + off; y[j + 16] = (float)x1 * d + off;
   }
 }
+/* block_iq4_xs: d, scales_h, scales_l[4], qs[128]  (dequantize_row_iq4_xs; tinygrad/llm/gguf.py:96-104) */
+static const int8_t kvalues_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+static void deq_iq4_xs(const uint8_t* b, float* y) {
+  uint16_t dh, sh; memcpy(&dh, b, 2); memcpy(&sh, b + 2, 2);
+  const float d = h2f(dh);
+  const uint8_t* qs = b + 8;
+  for (int ib = 0; ib < 8; ib++) {
+    const int ls = ((b[4 + ib / 2] >> (4 * (ib % 2))) & 0xf) | (((sh >> (2 * ib)) & 3) << 4);
+    const float dl = d * (float)(ls - 32);
+    for (int j = 0; j < 16; j++) { y[j] = dl * kvalues_iq4nl[qs[j] & 0xf]; y[j + 16] = dl * kvalues_iq4nl[qs[j] >> 4]; }
+    y += 32; qs += 16;
+  }
+}
+/* block_q1_0: d, 128 sign bits  (tinygrad/llm/gguf.py:115-118): d * (2 bit - 1) */
+static void deq_q1_0(const uint8_t* b, float* y) {
+  uint16_t dh; memcpy(&dh, b, 2);
+  const float d = h2f(dh);
+  for (int e = 0; e < 128; e++) y[e] = d * (float)((int)((b[2 + e / 8] >> (e % 8)) & 1) * 2 - 1);
+}
 /* get_scale_min_k4 of ggml-quants.c: 6-bit scale and min of sub-block j from the 12 packed bytes */
 static void scale_min_k4(int j, const uint8_t* q, uint8_t* d, uint8_t* m) {
   if (j < 4) { *d = q[j] & 63; *m = q[j + 4] & 63; }
@@ -137,6 +156,7 @@ static void deq_mxfp4(const uint8_t* b, float* y) {           /* block_mxfp4: gg
 
 static int type_geom(int t, int* nel, int* nby) {
   switch (t) { case 2: *nel = 32; *nby = 18; return 0; case 8: *nel = 32; *nby = 34; return 0;
+               case 23: *nel = 256; *nby = 136; return 0; case 41: *nel = 128; *nby = 18; return 0;
                case 3: *nel = 32; *nby = 20; return 0; case 6: *nel = 32; *nby = 22; return 0; case 7: *nel = 32; *nby = 24; return 0;
                case 12: *nel = 256; *nby = 144; return 0; case 13: *nel = 256; *nby = 176; return 0;
                case 14: *nel = 256; *nby = 210; return 0; case 39: *nel = 32; *nby = 17; return 0; }
@@ -145,6 +165,7 @@ static int type_geom(int t, int* nel, int* nby) {
 static void deq_block(int t, const uint8_t* b, float* y) {
   switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break;
                case 12: deq_q4_k(b, y); break; case 13: deq_q5_k(b, y); break;
+               case 23: deq_iq4_xs(b, y); break; case 41: deq_q1_0(b, y); break;
                case 3: deq_q4_1(b, y); break; case 6: deq_q5(b, y, 0); break; case 7: deq_q5(b, y, 1); break; }
 }
 

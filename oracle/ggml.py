@@ -5,8 +5,9 @@ import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, F32, F16 = 2, 8, 12, 13, 14, 39, 0, 1
 Q4_1, Q5_0, Q5_1 = 3, 6, 7
+IQ4_XS, Q1_0 = 23, 41
 # {ggml_type: (elements per block, bytes per block)}  tinygrad/llm/gguf.py:20-21
-GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17)}
+GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17), IQ4_XS: (256, 136), Q1_0: (128, 18)}
 # tinygrad/llm/gguf.py:108-110 (== 2 * E2M1 values; ggml_common.py:218 kvalues_mxfp4)
 FP4_LUT = np.array([0.0, 1.0, 2.0, 3.0, 4.0, 6.0, 8.0, 12.0, -0.0, -1.0, -2.0, -3.0, -4.0, -6.0, -8.0, -12.0], dtype=np.float32)
 
@@ -82,7 +83,30 @@ def dequant_mxfp4(blocks: np.ndarray) -> np.ndarray:
   d = np.where(e < 2, small, (e - 1) * np.uint32(0x00800000)).astype(np.uint32).view(np.float32)[:, None]
   return FP4_LUT[q_to_uint8(blocks[:, 1:17], 4)] * d
 
-_DEQ = {Q4_0: dequant_q4_0, Q4_1: dequant_q4_1, Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
+# ggml's kvalues_iq4nl (ggml-common.h; the reference reads it from its generated ggml_common module, gguf.py:98)
+KVALUES_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
+
+def dequant_iq4_xs(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:96-104  136 B: d, scales_h (u16), scales_l[4], qs[128]; eight sub-blocks of 32: scale = int8(nibble ib of scales_l |
+  (2 bits ib of scales_h) << 4) - 32; value = d * scale * lut[nibble], low nibbles = elements 0..15, high = 16..31 of the sub-block."""
+  nb = blocks.shape[0]
+  d = _f16(blocks[:, :2]).reshape(nb, 1, 1)
+  sl = blocks[:, 4:8]
+  scales_l = np.stack([sl & 0xF, sl >> 4], axis=2).reshape(nb, 8)
+  sh = np.ascontiguousarray(blocks[:, 2:4]).view(np.uint16).reshape(nb, 1)
+  scales_h = ((sh >> (np.arange(8, dtype=np.uint16) * 2)[None, :]) & 3).astype(np.uint8)
+  scales = ((scales_l | (scales_h << 4)).view(np.int8).astype(np.int32) - 32).astype(np.float32).reshape(nb, 8, 1)
+  qs = blocks[:, 8:].reshape(nb, 8, 16)
+  q = np.concatenate([qs & 0xF, qs >> 4], axis=2)
+  return ((d * scales) * KVALUES_IQ4NL[q]).reshape(nb, 256)
+
+def dequant_q1_0(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:115-118  18 B: fp16 d, 128 sign bits (element e = bit e % 8 of byte e // 8): d * (2 bit - 1).  The reference's result is
+  float16 (+-d); it is returned here as the same values in float32."""
+  bits = np.swapaxes(q_to_uint8(blocks[:, 2:], 1).reshape(-1, 8, 16), -1, -2).reshape(-1, 128).view(np.int8)
+  return _f16(blocks[:, :2]) * (bits.astype(np.float32) * 2 - 1)
+
+_DEQ = {IQ4_XS: dequant_iq4_xs, Q1_0: dequant_q1_0, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1, Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
 
 def ggml_data_to_tensor(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
   """gguf.py:23-119 restricted to the types on the path; returns flat float32 of n elements."""
@@ -218,6 +242,35 @@ def _quantize_q45_k(w: np.ndarray, five: bool) -> np.ndarray:
   off = 48 if five else 16
   out[:, off:off + 128] = ((q[:, 0::2] & 0xF) | ((q[:, 1::2] & 0xF) << 4)).reshape(nb, 128)
   if five: out[:, 16:48] = np.bitwise_or.reduce(((q >> 4) & 1) << np.arange(8, dtype=np.uint8)[None, :, None], axis=1)
+  return out.reshape(-1)
+
+def quantize_iq4_xs(w: np.ndarray) -> np.ndarray:
+  """Simple rule (NOT ggml's search): per 32-weight sub-block s = amax / 127, superblock d = max s / 31 (fp16), 6-bit field ls = 32 + round(s / d)
+  (positive scales only), code = index of the kvalues_iq4nl entry nearest to x / (d (ls - 32)).  Packing as dequant_iq4_xs decodes."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 8, 32)
+  nb = x.shape[0]
+  sb = np.abs(x).max(axis=2) / np.float32(127)
+  d = (sb.max(axis=1) / np.float32(31)).astype(np.float16).astype(np.float32)
+  with np.errstate(divide="ignore", invalid="ignore"):
+    ls = np.where(d[:, None] > 0, np.rint(sb / d[:, None]), 0).clip(0, 31).astype(np.uint8) + np.uint8(32)
+    eff = d[:, None] * (ls.astype(np.float32) - 32)
+    t = np.where(eff[:, :, None] > 0, x / eff[:, :, None], 0)
+  code = np.abs(t[..., None] - KVALUES_IQ4NL[None, None, None, :]).argmin(-1).astype(np.uint8)
+  out = np.zeros((nb, 136), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  sh = np.zeros(nb, dtype=np.uint16)
+  for ib in range(8): sh |= ((ls[:, ib] >> 4).astype(np.uint16) << np.uint16(2 * ib))
+  out[:, 2:4] = sh.view(np.uint8).reshape(-1, 2)
+  out[:, 4:8] = (ls[:, 0::2] & 0xF) | ((ls[:, 1::2] & 0xF) << 4)
+  out[:, 8:] = (code[:, :, :16] | (code[:, :, 16:] << 4)).reshape(nb, 128)
+  return out.reshape(-1)
+
+def quantize_q1_0(w: np.ndarray) -> np.ndarray:
+  """d = mean |x| over the 128-weight block (fp16), bit = x >= 0.  Packing as dequant_q1_0 decodes."""
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 128)
+  out = np.zeros((x.shape[0], 18), dtype=np.uint8)
+  out[:, 0:2] = np.abs(x).mean(axis=1).astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:] = np.packbits((x >= 0).astype(np.uint8).reshape(-1, 16, 8), axis=2, bitorder="little").reshape(-1, 16)
   return out.reshape(-1)
 
 def quantize_q4_k(w: np.ndarray) -> np.ndarray: return _quantize_q45_k(w, False)

@@ -72,7 +72,7 @@ def test_q6_k_brute_force_layout():
     out = og.ggml_data_to_tensor(b, 256, 14)
     np.testing.assert_array_equal(out, exp, err_msg=f"element {e}")
 
-@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 39])
+@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 41])
 def test_numpy_restatement_equals_scalar_c_loops(t):
   """Vectorised restatement of tinygrad/llm/gguf.py (field-major q_to_uint8) == independent scalar loops of the published ggml
   routines, bit for bit, on fully random bytes (NaN/Inf/subnormal scales included)."""
@@ -143,6 +143,39 @@ def test_q5_0_equals_q4_0_when_fifth_bits_mirror_the_sign():
   b5[:, 2:6] = og._pack_q5_bits(q5); b5[:, 6:] = (q5[:, :16] & 0xF) | ((q5[:, 16:] & 0xF) << 4)
   np.testing.assert_array_equal(og.ggml_data_to_tensor(b5, 64 * 32, 6), og.ggml_data_to_tensor(b4, 64 * 32, 2))
 
+def test_iq4_xs_brute_force_layout():
+  """One weight at a time against ggml's block_iq4_xs (dequantize_row_iq4_xs): sub-block ib = e // 32 has the 6-bit scale
+  (nibble ib of scales_l) | (bits 2 ib, 2 ib + 1 of scales_h) << 4, minus 32; element j < 16 of it is the low nibble of qs[16 ib + j],
+  element j + 16 the high nibble; the nibble indexes kvalues_iq4nl."""
+  kv = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
+  for e in [0, 1, 15, 16, 31, 32, 47, 48, 100, 127, 128, 200, 255]:
+    for code, ls in ((0, 45), (15, 3), (9, 63)):
+      b = np.zeros(136, dtype=np.uint8)
+      b[0:2] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+      ib, l = e // 32, e % 32
+      b[8:] = 0x88                                              # every nibble 8 -> kvalues[8] = 1
+      sl = np.zeros(8, np.uint8) + (32 & 0xF); shh = 0
+      for k in range(8): shh |= (32 >> 4) << (2 * k)             # all scales 32 -> (32 - 32) = 0: other sub-blocks decode to 0
+      sl[ib] = ls & 0xF; shh = (shh & ~(3 << (2 * ib))) | ((ls >> 4) << (2 * ib))
+      b[4:8] = sl[0::2] | (sl[1::2] << 4)
+      b[2:4] = np.frombuffer(np.uint16(shh).tobytes(), np.uint8)
+      byte = 8 + 16 * ib + l % 16
+      b[byte] = (0x80 | code) if l < 16 else (0x08 | (code << 4))
+      exp = np.zeros(256, dtype=np.float32)
+      exp[32 * ib:32 * ib + 32] = 0.25 * (ls - 32) * 1.0          # nibble 8 everywhere else in the sub-block
+      exp[e] = 0.25 * (ls - 32) * kv[code]
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, 23), exp, err_msg=f"element {e}")
+      np.testing.assert_array_equal(cref.dequant(23, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
+
+def test_q1_0_brute_force_layout():
+  """Q1_0: element e is bit e % 8 of byte 2 + e // 8; set bit -> +d, clear bit -> -d."""
+  for e in [0, 1, 7, 8, 9, 63, 64, 100, 127]:
+    b = np.zeros(18, dtype=np.uint8); b[0:2] = np.frombuffer(np.float16(1.5).tobytes(), np.uint8)
+    b[2 + e // 8] = 1 << (e % 8)
+    exp = np.full(128, -1.5, dtype=np.float32); exp[e] = 1.5
+    np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 128, 41), exp)
+    np.testing.assert_array_equal(cref.dequant(41, b[None]).reshape(-1), exp)
+
 def test_q6_k_association_order_is_exact():
   """(d*q)*sc == d*(sc*q) == (d*sc)*q in float32: 11 + 6 + 8 significant bits fit in 24."""
   rng = np.random.default_rng(3)
@@ -153,9 +186,9 @@ def test_quantizers_round_trip():
   rng = np.random.default_rng(0)
   w = rng.standard_normal(256 * 64).astype(np.float32)
   for t, qf, tol in ((2, og.quantize_q4_0, 1 / 7.0), (8, og.quantize_q8_0, 1 / 127.0), (14, og.quantize_q6_k, 1 / 30.0), (12, og.quantize_q4_k, 1 / 6.0), (13, og.quantize_q5_k, 1 / 13.0),
-                      (3, og.quantize_q4_1, 1 / 7.0), (6, og.quantize_q5_0, 1 / 15.0), (7, og.quantize_q5_1, 1 / 15.0)):
+                      (3, og.quantize_q4_1, 1 / 7.0), (6, og.quantize_q5_0, 1 / 15.0), (7, og.quantize_q5_1, 1 / 15.0), (23, og.quantize_iq4_xs, 1 / 7.0)):
     dq = og.ggml_data_to_tensor(qf(w), w.size, t)
-    nel = og.GGML_QUANT[t][0] if t != 14 else 16
+    nel = {14: 16, 23: 32}.get(t, og.GGML_QUANT[t][0])
     amax = np.abs(w.reshape(-1, nel)).max(1, keepdims=True)
     assert (np.abs(dq.reshape(-1, nel) - w.reshape(-1, nel)) <= tol * amax + 1e-6).all(), t
 

@@ -94,6 +94,39 @@ template <bool FIVE> struct DeqK45 {
 };
 template <> struct Deq<GGML_Q4_K> : DeqK45<false> {};
 template <> struct Deq<GGML_Q5_K> : DeqK45<true> {};
+// IQ4_XS (136 B: d, scales_h u16, scales_l[4], qs[128]), tinygrad/llm/gguf.py:96-104: eight sub-blocks of 32; 6-bit scale ls =
+// nibble ib of scales_l | 2 bits of scales_h << 4; value = (d * (ls - 32)) * kvalues_iq4nl[nibble]; qs[16 ib + j] holds elements j (low
+// nibble) and j + 16 (high nibble) of sub-block ib.
+__device__ __forceinline__ float iq4nl_value(uint32_t code) {
+  // ggml's kvalues_iq4nl, packed four int8 per dword
+  const uint32_t t[4] = {0xBFAD9881u, 0xF6EADDCFu, 0x26190D01u, 0x71594535u};   // -127 -104 -83 -65 | -49 -35 -22 -10 | 1 13 25 38 | 53 69 89 113
+  return (float)(int)(int8_t)(t[code >> 2] >> (8 * (code & 3)));
+}
+template <> struct Deq<GGML_IQ4_XS> {
+  static constexpr int NEL = 256, NBY = 136;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b));
+    const uint32_t sh = ld2(b + 2);
+    const int ib = e0 >> 5, l = e0 & 31;
+    const int ls = (int)(((b[4 + (ib >> 1)] >> (4 * (ib & 1))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4));
+    const float dl = d * (float)(ls - 32);
+    const int hi = (l >= 16) ? 4 : 0; const uint8_t* q = b + 8 + 16 * ib + (l & 15);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = dl * iq4nl_value((q[i] >> hi) & 0xF);
+  }
+};
+// Q1_0 (18 B: d, 128 sign bits), tinygrad/llm/gguf.py:115-118: value = d * (2 bit - 1), element e = bit e % 8 of byte e / 8
+template <> struct Deq<GGML_Q1_0> {
+  static constexpr int NEL = 128, NBY = 18;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b));
+    const uint32_t bits = b[2 + (e0 >> 3)] >> (e0 & 7);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = d * (float)((int)((bits >> i) & 1u) * 2 - 1);
+  }
+};
 template <> struct Deq<GGML_MXFP4> {
   static constexpr int NEL = 32, NBY = 17;
   static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {

@@ -2,12 +2,12 @@
 
 ggml_data_to_tensor(t, n, ggml_type) mirrors tinygrad/llm/gguf.py:23: `t` is the raw byte buffer (device Buffer of uint8, or a
 numpy array that is uploaded), `n` the element count, and the result is a flat float32 device Buffer of n elements, bit-exact
-with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), MXFP4 (39); native float32/float16 (0, 1) are reinterpreted in place.
+with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ4_XS (23), MXFP4 (39), Q1_0 (41); native float32/float16 (0, 1) are reinterpreted in place.
 Unknown types raise ValueError with the reference's message (gguf.py:119)."""
 from __future__ import annotations
 import numpy as np
 from tinygrad_amd import runtime as rt
-from tinygrad_amd.runtime import Buffer, GGML_QUANT
+from tinygrad_amd.runtime import Buffer, GGML_QUANT, GGML_DEQUANT_ONLY
 
 def _as_device_bytes(t) -> Buffer:
   if isinstance(t, Buffer): return t
@@ -17,8 +17,8 @@ def ggml_data_to_tensor(t, n: int, ggml_type: int, out_dtype=np.float32, stream=
   t = _as_device_bytes(t)
   if ggml_type == rt.F32: return t.view(0, (n,), np.float32)
   if ggml_type == rt.F16: return t.view(0, (n,), np.float16)
-  if ggml_type not in GGML_QUANT: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
-  nel, nby = GGML_QUANT[ggml_type]
+  if ggml_type not in GGML_QUANT and ggml_type not in GGML_DEQUANT_ONLY: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
+  nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]
   nfull = (n // nel) * nel                                   # gguf.py:45 uses whole blocks only
   if t.nbytes < (nfull // nel) * nby: raise ValueError(f"buffer of {t.nbytes} bytes holds fewer than {nfull // nel} blocks")
   out = Buffer((nfull,), out_dtype)
@@ -55,7 +55,7 @@ class GGUFTensor:
 
 def tensor_nbytes(ggml_type: int, n: int) -> int:
   if ggml_type in _NATIVE_ITEMSIZE: return _NATIVE_ITEMSIZE[ggml_type] * n
-  if ggml_type in GGML_QUANT: nel, nby = GGML_QUANT[ggml_type]; return (n // nel) * nby
+  if ggml_type in GGML_QUANT or ggml_type in GGML_DEQUANT_ONLY: nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]; return (n // nel) * nby
   raise ValueError(f"GGML type '{ggml_type}' is not supported!")
 
 def gguf_parse(raw: np.ndarray) -> tuple[dict, dict[str, GGUFTensor]]:

@@ -311,7 +311,7 @@ class Transformer:
     qk-norm).  Weights stay in their GGUF blocks on the device; F32 / BF16 matrices are cast to fp16 on the host (the reference
     casts every weight to fp16, model.py:376); for arch == 'llama' the rows of attn_q / attn_k are permuted from the interleaved
     to the half-split RoPE layout (model.py:409-419) by moving whole block rows."""
-    from tinygrad_amd.gguf import gguf_load, GGUF_F32_LIKE
+    from tinygrad_amd.gguf import gguf_load, ggml_data_to_tensor, GGUF_F32_LIKE
     kv, ts = gguf_load(gguf)
     arch = kv["general.architecture"]
     ctx = kv[f"{arch}.context_length"]
@@ -332,6 +332,9 @@ class Transformer:
         if typ != rt.F32: data = _to_f32(data, typ); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F32
       elif typ in GGUF_F32_LIKE:                                       # F32 / BF16 matrices -> fp16 (model.py:376)
         data = _to_f32(data, typ).astype(np.float16); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F16
+      elif typ in rt.GGML_DEQUANT_ONLY:                                # block types without an in-place linear kernel: the fp16 weight of model.py:376, made once
+        buf = ggml_data_to_tensor(buf, rows * cols, typ, out_dtype=np.float16); typ = rt.F16
+        data = buf.numpy()
       if arch == "llama" and (name.endswith("attn_q.weight") or name.endswith("attn_k.weight")):
         h = n_heads if name.endswith("attn_q.weight") else n_kv
         raw = np.ascontiguousarray(data).view(np.uint8).reshape(rows, -1)
