@@ -115,6 +115,14 @@ int tga_stage_activation(int ggml_type, const void* x, int x_dtype, int64_t K, v
 int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* sel, int n_jobs,
                         int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
 
+/* The expert gate/up jobs of ONE token with the gating inside the launch: every workgroup computes scores, pairwise top-k and weights from
+ * the router logits (tinygrad/llm/model.py:112-128; gating as tga_moe_gate) for itself, job j multiplies the j-th selected expert:
+ * y[j] = silu(x Wgate[e_j]^T) * (x Wup[e_j]^T).  The selection and the weights are written to sel_out / probs_out (k entries each) for
+ * the launches that follow.  x: one fp16 row of at most 4096 values; logits: n_experts float32 (tga_moe_router with k = 0 writes them). */
+int tga_qlinear_experts_routed(int ggml_type, const void* w_gate, const void* w_up, int64_t n_experts, const float* logits, int k,
+                               int gating, int norm_topk_prob, float scale, int32_t* sel_out, float* probs_out,
+                               const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
+
 /* Expert gating of FFNBlock._feed_forward (model.py:112-128): scores by ExpertGating (1 SOFTMAX, 2 SIGMOID, 3 SOFTMAX_WEIGHT,
  * 4 SQRT_SOFTPLUS; model.py:9-13), pairwise_topk selection (model.py:35-41: ascending, lower index wins ties), probabilities
  * gathered / renormalised / scaled.  logits (n_tokens, n_experts) float32 -> sel (n_tokens, k) int32, probs (n_tokens, k). */
@@ -124,7 +132,8 @@ int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int ga
  * NULL: h = fp16(x)), logits = h @ Wr^T for a dense fp16 router weight (n_experts, dim), then gating + top-k as tga_moe_gate.
  * xn_out_f16 (dim fp16, the activation of the expert GEMVs) may be NULL.  logits_ws: n_experts floats (the logits, readable
  * afterwards) followed by one int32 arrival counter that must be ZERO before the first call (each call leaves it zero); calls
- * sharing one workspace must not overlap.  dim % 8 == 0, dim <= 16384, n_experts <= 1024, k <= 64. */
+ * sharing one workspace must not overlap.  dim % 8 == 0, dim <= 16384, n_experts <= 1024, k <= 64.
+ * k = 0: logits only (sel / probs may be NULL, the counter is not touched): for a consumer that gates for itself (tga_qlinear_experts_routed). */
 int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
                    int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_ws, int32_t* sel, float* probs, void* stream);
 /* out[t] = resid[t] + sum_s probs[t, s] * y[t, s, :]  (model.py:130 and the residual add :150); resid may be NULL or alias out. */

@@ -108,6 +108,27 @@ def test_weighted_expert_sum_folded_into_the_next_linear(gpu, t, dim, k):
   for f, q in zip(fused, plain): assert ol.rel_err(f.numpy(), q.numpy()) <= 2e-4
   with pytest.raises(RuntimeError): qlinear_multi(layers, xb, fused, norm=(nwb, 1e-5), combine=(yb, pb, 9, x_out))
 
+@pytest.mark.parametrize("t,dim,n,E,k,gating", [(39, 2048, 256, 64, 8, 1), (2, 512, 128, 8, 2, 3), (1, 1024, 96, 130, 6, 2), (12, 1024, 64, 16, 4, 4)])
+def test_expert_gate_up_that_gates_for_itself(gpu, t, dim, n, E, k, gating):
+  """tga_qlinear_experts_routed (scores, top-k and weights computed inside the expert gate/up launch from the router logits) against
+  tga_moe_gate followed by tga_qlinear_experts: identical selection and weights, identical outputs."""
+  from tinygrad_amd.nn import ExpertWeights, moe_gate
+  rng = np.random.default_rng(dim + E + k)
+  mk = (lambda: synth.random_blocks(rng, t, E * n, dim)) if t != 1 else (lambda: (rng.standard_normal((E * n, dim)) * dim ** -0.5).astype(np.float16).view(np.uint8).reshape(-1))
+  ew, eu = ExpertWeights(gpu.Buffer.from_numpy(mk()), t, E, n, dim), ExpertWeights(gpu.Buffer.from_numpy(mk()), t, E, n, dim)
+  x = gpu.Buffer.from_numpy(synth.activations(rng, 1, dim, np.float16))
+  lg = gpu.Buffer.from_numpy(rng.standard_normal((1, E)).astype(np.float32))
+  sel0, p0, y0 = gpu.Buffer((k,), np.int32), gpu.Buffer((k,), np.float32), gpu.Buffer((k, n), np.float32)
+  moe_gate(lg, 1, E, k, sel0, p0, gating, True, 1.25)
+  ew(sel0, x, y0, jobs_per_x_row=k, up=eu)
+  sel1, p1, y1 = gpu.Buffer((k,), np.int32).zero_(), gpu.Buffer((k,), np.float32).zero_(), gpu.Buffer((k, n), np.float32).zero_()
+  ew(sel1, x, y1, jobs_per_x_row=k, up=eu, route=(lg, gating, True, 1.25, p1))
+  np.testing.assert_array_equal(sel1.numpy(), sel0.numpy())
+  np.testing.assert_array_equal(p1.numpy(), p0.numpy())
+  np.testing.assert_array_equal(y1.numpy(), y0.numpy())
+  rs, rp = omoe.gate_probs(lg.numpy(), k, gating, True, 1.25)
+  np.testing.assert_array_equal(sel1.numpy(), rs[0])
+
 def test_moe_combine(gpu):
   from tinygrad_amd.nn import moe_combine
   rng = np.random.default_rng(3)

@@ -1,53 +1,7 @@
 // MoE routing pieces of the decode path (tinygrad/llm/model.py:110-135): expert gating + pairwise top-k, and the weighted
 // sum over the selected experts' outputs.
 #include "coherent.h"
-
-// scores per ExpertGating (model.py:9-13, 116-121): 1 SOFTMAX, 2 SIGMOID, 3 SOFTMAX_WEIGHT (softmax over the selected logits),
-// 4 SQRT_SOFTPLUS.  Top-k by pairwise rank exactly as pairwise_topk (model.py:35-41): rank_i = #{j: s_i > s_j or (s_i == s_j and
-// i < j)}; the k highest ranks are emitted in ASCENDING rank order (the largest last), so among equal scores the lower index
-// ranks higher.  Runs on ONE wave (lane = threadIdx.x & 63 of the calling wave); lg may live in LDS or global memory, sc is
-// n_experts floats of LDS, tmp 192 floats of LDS.  The caller separates the call from earlier LDS writes with a barrier.
-__device__ __forceinline__ void gate_topk_wave(const float* lg, int n_experts, int k, int gating, int norm_topk, float scale,
-                                               int* __restrict__ sel, float* __restrict__ probs, float* sc, float* tmp, int lane) {
-  int* s_sel = (int*)tmp; float* s_p = tmp + 64; float* s_q = tmp + 128;
-  if (gating == 1 && norm_topk) { gating = 3; norm_topk = 0; }   // model.py:116-117 fast path (no selection bias)
-  float mx = -INFINITY;
-  for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, lg[i]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  if (gating == 1) { for (int i = lane; i < n_experts; i += 64) sum += expf(lg[i] - mx); sum = wave_sum(sum); }
-  for (int i = lane; i < n_experts; i += 64) {
-    const float v = lg[i];
-    float s;
-    if (gating == 3) s = v;
-    else if (gating == 1) s = expf(v - mx) * (1.0f / sum);
-    else if (gating == 2) s = 1.0f / (1.0f + expf(-v));
-    else s = sqrtf(log1pf(expf(v)));
-    sc[i] = s;
-  }
-  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's LDS writes are visible to its own lanes
-  for (int i = lane; i < n_experts; i += 64) {
-    const float si = sc[i];
-    int rank = 0;
-    for (int j = 0; j < n_experts; j++) { const float sj = sc[j]; rank += (si > sj) || (si == sj && i < j); }
-    const int slot = rank - (n_experts - k);
-    if (slot >= 0) { s_sel[slot] = i; s_p[slot] = si; }
-  }
-  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);
-  float p = lane < k ? s_p[lane] : 0.f;
-  if (gating == 3 && lane < k) {                          // softmax over the selected logits
-    float m2 = -INFINITY; for (int j = 0; j < k; j++) m2 = fmaxf(m2, s_p[j]);
-    float z = 0.f; for (int j = 0; j < k; j++) z += expf(s_p[j] - m2);
-    p = expf(p - m2) * (1.0f / z);
-  }
-  s_q[lane] = p;
-  __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);
-  if (lane < k) {
-    if (norm_topk) { float z = 0.f; for (int j = 0; j < k; j++) z += s_q[j]; p = p / z; }
-    sel[lane] = s_sel[lane];
-    probs[lane] = p * scale;
-  }
-}
+#include "moe_gate.h"
 
 // One workgroup (64 threads) per token.
 __global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ logits, int n_experts, int k, int gating, int norm_topk,
@@ -136,6 +90,10 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_kernel(const float*
     acc = dot2(w4.w, xv.w, dot2(w4.z, xv.z, dot2(w4.y, xv.y, dot2(w4.x, xv.x, acc))));
   }
   acc = wave_sum(acc);
+  if (k == 0) {                                         // logits only: the consumer (a later launch) gates for itself
+    if (lane == 0 && row < n_experts) logits_ws[row] = acc;
+    return;
+  }
   if (lane == 0 && row < n_experts) cst(&logits_ws[row], acc);
   stores_done();
   __syncthreads();
@@ -177,10 +135,10 @@ int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int ga
 
 int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
                    int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_ws, int32_t* sel, float* probs, void* stream) {
-  TGA_REQUIRE(x && router_w_f16 && logits_ws && sel && probs, "tga_moe_router: null pointer");
+  TGA_REQUIRE(x && router_w_f16 && logits_ws && (k == 0 || (sel && probs)), "tga_moe_router: null pointer");
   TGA_REQUIRE(dim >= 8 && dim % 8 == 0 && dim <= 16384 && ((uintptr_t)router_w_f16 & 15) == 0, "tga_moe_router: dim=%d must be a multiple of 8, at most 16384, with a 16-byte aligned weight", dim);
   TGA_REQUIRE((((uintptr_t)x | (uintptr_t)norm_weight | (uintptr_t)xn_out_f16) & 15) == 0, "tga_moe_router: x, norm_weight and xn_out must be 16-byte aligned");
-  TGA_REQUIRE(n_experts >= 1 && n_experts <= 1024 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_router: bad geometry (k <= 64, n_experts <= 1024)");
+  TGA_REQUIRE(n_experts >= 1 && n_experts <= 1024 && k >= 0 && k <= 64 && k <= n_experts, "tga_moe_router: bad geometry (k <= 64, n_experts <= 1024)");
   TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_router: unknown ExpertGating %d", gating);
   moe_router_kernel<<<(n_experts + 3) / 4, ROUTER_THREADS, 2 * n_experts * sizeof(float) + (size_t)dim * 2, (hipStream_t)stream>>>(
       x, norm_weight, norm_eps, (const _Float16*)router_w_f16, dim, n_experts, k, gating, norm_topk_prob, scale, (_Float16*)xn_out_f16, logits_ws, sel, probs);

@@ -20,7 +20,7 @@ struct QArgs {
   int chunk_u, nchunks; // units per LDS chunk
   // job indirection (MoE expert GEMVs): blockIdx.y = job; expert = sel[job]; weights shifted by expert * estride bytes;
   // activation row = job / xdiv; outputs shifted by job * ystride elements.  sel == nullptr: a single job.
-  const int* sel; long long estride, ystride; int xdiv, xdiv_jobs;   // xdiv_jobs: number of jobs (grid.y)
+  int* sel; long long estride, ystride; int xdiv, xdiv_jobs;   // xdiv_jobs: number of jobs (grid.y)
   // x_staged: x already holds fp16 activations in the consumer format's staged order (Fmt::spos).
   // y_stage_fmt / y_stage_nu: when y_stage_fmt != 0 the fp16 outputs are written in the staged order of THAT consumer format.
   int x_staged, y_stage_fmt, y_stage_nu;
@@ -31,6 +31,10 @@ struct QArgs {
   // (the weighted sum over the selected experts' outputs plus the block residual, tinygrad/llm/model.py:130, 150); the completed row is
   // also written to comb_x_out (a different buffer: every workgroup reads x) by the first workgroup.
   const float* comb_y; const float* comb_p; int comb_k; float* comb_x_out;
+  // route_logits != nullptr (expert gate/up jobs of one token): the kernel gates for itself - scores, pairwise top-k and weights of
+  // the route_k experts from the router logits (tinygrad/llm/model.py:112-128) - instead of reading sel; job j takes the j-th selected
+  // expert, and the first workgroup writes the selection and the weights to sel / route_probs_out for the launches that follow.
+  const float* route_logits; int route_E, route_k, route_gating, route_norm_topk; float route_scale; float* route_probs_out;
   // M = 1 fast path: row groups per team and the remainder (the first team_rem teams take one more), so that the kernel divides nothing
   int team_base, team_rem;
 };

@@ -462,8 +462,9 @@ extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dt
 // ExpertWeights.__call__ (tinygrad/llm/model.py:21-27): per (token, slot) job j, y[j] = x[j / jobs_per_x_row] @ W[sel[j]]^T over a
 // stacked (n_experts, N, K) weight; with w_up the output is silu(x Wgate[e]^T) * (x Wup[e]^T) (model.py:129).  Only the
 // selected experts' bytes are read (the indexed load the reference's codegen produces from weight[sel]).
-extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* sel, int n_jobs,
-                                   int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
+struct RouteIn { const float* logits; int k, gating, norm_topk; float scale; float* probs_out; };
+static int qlinear_experts_impl(const RouteIn* route, int ggml_type, const void* w, const void* w_up, int64_t n_experts, int32_t* sel, int n_jobs,
+                                int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
   TGA_REQUIRE(w && sel && x && y, "tga_qlinear_experts: null pointer");
   TGA_REQUIRE(n_jobs >= 1 && n_jobs <= 65535 && jobs_per_x_row >= 1 && n_experts >= 1, "tga_qlinear_experts: bad job geometry");
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32, "tga_qlinear_experts: x_dtype must be TGA_F16 or TGA_F32");
@@ -481,10 +482,33 @@ extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_u
   a.nseg = w_up ? 2 : 1; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = w_up ? 2 : 0; a.K = (int)K;
   a.w[0] = (const uint8_t*)w; a.w[1] = (const uint8_t*)w_up; a.y[0] = y; a.n[0] = N; a.n[1] = N; a.ntot = N;
   a.sel = sel; a.estride = (long long)N * (K / bw) * bb; a.ystride = N; a.xdiv = jobs_per_x_row; a.xdiv_jobs = n_jobs;
+  if (route) {
+    a.route_logits = route->logits; a.route_E = (int)n_experts; a.route_k = route->k; a.route_gating = route->gating; a.route_norm_topk = route->norm_topk;
+    a.route_scale = route->scale; a.route_probs_out = route->probs_out;
+  }
   const bool pair = (K / 32) % 2 == 0 && ((uintptr_t)w & 3) == 0 && (!w_up || ((uintptr_t)w_up & 3) == 0) && a.estride % 4 == 0;
   const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
   TGA_REQUIRE(fmt >= 0, "tga_qlinear_experts: Q4_0/Q8_0 expert weights need K %% 64 == 0 and 4-byte aligned experts");
   const int rc = tga_qgemv1_dispatch(fmt, a, (hipStream_t)stream);
   TGA_REQUIRE(rc >= 0, "tga_qlinear_experts: shape K=%lld outside the expert GEMV path", (long long)K);
   return rc;
+}
+
+extern "C" int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* sel, int n_jobs,
+                                   int jobs_per_x_row, const void* x, int x_dtype, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
+  return qlinear_experts_impl(nullptr, ggml_type, w, w_up, n_experts, (int32_t*)sel, n_jobs, jobs_per_x_row, x, x_dtype, y, y_dtype, N, K, stream);
+}
+
+// The expert gate/up jobs of ONE token with the gating inside the launch: every workgroup computes the scores, the pairwise top-k and
+// the weights from the router logits (tinygrad/llm/model.py:112-128) for itself, job j multiplies the j-th selected expert, and the
+// selection / weights are written to sel_out / probs_out (k entries) for the launches that follow (expert down, weighted sum).
+// y[j] = silu(x Wgate[e_j]^T) * (x Wup[e_j]^T), x one fp16 row of at most 4096 values.
+extern "C" int tga_qlinear_experts_routed(int ggml_type, const void* w_gate, const void* w_up, int64_t n_experts, const float* logits, int k,
+                                          int gating, int norm_topk_prob, float scale, int32_t* sel_out, float* probs_out,
+                                          const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
+  TGA_REQUIRE(logits && sel_out && probs_out && w_up, "tga_qlinear_experts_routed: null pointer");
+  TGA_REQUIRE(n_experts >= 1 && n_experts <= 1024 && k >= 1 && k <= 64 && k <= n_experts, "tga_qlinear_experts_routed: bad geometry (k <= 64, n_experts <= 1024)");
+  TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_qlinear_experts_routed: unknown ExpertGating %d", gating);
+  const RouteIn r = {logits, k, gating, norm_topk_prob, scale, probs_out};
+  return qlinear_experts_impl(&r, ggml_type, w_gate, w_up, n_experts, sel_out, k, k, x_f16, TGA_F16, y, y_dtype, N, K, stream);
 }

@@ -3,6 +3,7 @@
 #pragma once
 #include "qfmt.h"
 #include "host.h"
+#include "moe_gate.h"
 
 #ifndef QG1_DEPTH
 #define QG1_DEPTH 3        // row groups in flight per lane: the loads of the next DEPTH - 1 groups are outstanding while one is multiplied
@@ -30,6 +31,8 @@
 //          squares and the scaling)
 //   PRO 2  activations already in the staged order of this format (written by the producing kernel)
 //   PRO 3  one fp16 row of at most two pieces per thread
+//   PRO 6  PRO 3 for the expert gate/up jobs of one token with the gating done here: every workgroup computes scores and top-k from the
+//          router logits itself (64..1024 floats), so no selection has to cross workgroups inside the router's launch
 //   PRO 5  PRO 1 for a row of at most one piece per thread that is first completed as x + sum_j p_j y_j (the MoE weighted sum and block
 //          residual that precede the next block's attn_norm): the launch that would only add vectors disappears
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
@@ -57,7 +60,8 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   const bool uvalid = u < a.nu;
   const int uc = uvalid ? u : a.nu - 1;
   const int job = blockIdx.y;
-  const long long eoff = a.sel ? (long long)a.sel[job] * a.estride : 0, yofs = (long long)job * a.ystride;
+  long long eoff = (a.sel && PRO != 6) ? (long long)a.sel[job] * a.estride : 0;
+  const long long yofs = (long long)job * a.ystride;
   const long long xrow = a.sel ? job / a.xdiv : 0;
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
   const long long team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
@@ -77,6 +81,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   const float* resid = nullptr;
   auto enter = [&](int sg) {
     seg = sg;
+    if (sg == 0) seg_start = 0;
     const long long seg_rows = a.n[sg];
     lo = row_lo - seg_start; hi = row_hi - seg_start;
     if (lo < 0) lo = 0;
@@ -268,6 +273,23 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
 #pragma unroll
     for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
     lds_to_regs();
+  } else if constexpr (PRO == 6) {
+    __shared__ float tk_lg[1024], tk_sc[1024], tk_tmp[192], tk_p[64];
+    __shared__ int tk_sel[64];
+    u32x4 v[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
+    for (int i = threadIdx.x; i < a.route_E; i += NT) tk_lg[i] = a.route_logits[i];
+    __syncthreads();
+    if (wave == 0) gate_topk_wave(tk_lg, a.route_E, a.route_k, a.route_gating, a.route_norm_topk, a.route_scale, tk_sel, tk_p, tk_sc, tk_tmp, lane);
+    __syncthreads();
+    eoff = (long long)tk_sel[job] * a.estride;
+    enter(0);                                                    // the weight bases of the selected expert
+    if (blockIdx.x == 0 && job == 0 && (int)threadIdx.x < a.route_k) { a.sel[threadIdx.x] = tk_sel[threadIdx.x]; a.route_probs_out[threadIdx.x] = tk_p[threadIdx.x]; }
+    issue(b[0], lo);
+#pragma unroll
+    for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
+    lds_to_regs();
   } else {
     if (a.x_staged) {
       const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
@@ -381,6 +403,13 @@ static int launch_fast(QArgs a, hipStream_t s) {
     }
   }
   if (a.comb_y) return tga_set_error("tga_moe_combine_rmsnorm_qlinear_multi: shape outside the fused path (K = %d)", a.K);
+  if constexpr (WK == 1 && EPI == 2) {
+    if (a.route_logits) {
+      if (a.x_staged || a.norm_w || a.x_f32 || !one_batch || a.xdiv != a.xdiv_jobs) return tga_set_error("tga_qlinear_experts_routed: needs one fp16 row of at most %d values", 16 * NT);
+      return launch_fast_p<T, R, WK, WR, EPI, H, 6>(a, grid, lds, s);
+    }
+  }
+  if (a.route_logits) return tga_set_error("tga_qlinear_experts_routed: shape outside the routed path (K = %d)", a.K);
   if constexpr (WK == 1 && EPI != 1) {
     if (!a.x_staged && one_batch && a.norm_w && a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 1>(a, grid, lds, s);
     if (!a.x_staged && one_batch && !a.norm_w && !a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 3>(a, grid, lds, s);

@@ -144,6 +144,9 @@ class TransformerBlock:
     self.stage_attn = fast(self.attn_output)
     self.stage_act = (not self.moe) and fast(self.ffn_down)
     self.stage_xn = (not self.moe) and fast(self.ffn_gate) and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
+    # the expert gate/up launch can gate for itself: one fp16 row of at most 4096 values on one wave per row team
+    self.route_in_experts = self.moe and c.dim <= 4096 and c.dim % 64 == 0 and c.num_experts <= 1024 and c.num_experts_per_tok <= 64 \
+                            and (c.dim // (32 if self.ffn_gate_exps.ggml_type == rt.MXFP4 else 64)) <= 64
     # the previous block's weighted expert sum can be completed inside this block's q/k/v launch (one 8-value piece per thread: dim <= 2048)
     self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
                             and 0 < c.num_experts_per_tok <= 8
@@ -191,15 +194,22 @@ class TransformerBlock:
       return x, False
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
-    if self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024:
-      moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, s.router, xn_out=s.xn, gating=c.expert_gating_func,
-                 norm_topk_prob=c.norm_topk_prob, scale=c.routed_scaling_factor, stream=stream)
+    one_launch_router = self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024
+    if one_launch_router and self.route_in_experts:
+      # router logits only; the expert gate/up launch gates for itself (scores, top-k, weights) and writes sel / probs for the launches after it
+      moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, 0, None, None, s.router, xn_out=s.xn, stream=stream)
+      self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream,
+                         route=(s.router, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, s.probs))
     else:
-      rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
-      lg = s.router.view(0, (1, c.num_experts), np.float32)
-      self.ffn_gate_inp(s.xn, out=lg, stream=stream)
-      moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
-    self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
+      if one_launch_router:
+        moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, s.router, xn_out=s.xn, gating=c.expert_gating_func,
+                   norm_topk_prob=c.norm_topk_prob, scale=c.routed_scaling_factor, stream=stream)
+      else:
+        rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
+        lg = s.router.view(0, (1, c.num_experts), np.float32)
+        self.ffn_gate_inp(s.xn, out=lg, stream=stream)
+        moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
+      self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
     self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
     if defer: return x, True                                            # the consumer of the completed row adds sum_j probs_j y_j + x itself
     moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)

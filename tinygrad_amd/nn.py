@@ -80,8 +80,16 @@ class ExpertWeights:
     nel, nby = GGML_QUANT[self.ggml_type]
     return self.out_features * (self.in_features // nel) * nby
 
-  def __call__(self, sel: Buffer, x: Buffer, out: Buffer, jobs_per_x_row: int = 1, up: "ExpertWeights | None" = None, stream=None) -> Buffer:
+  def __call__(self, sel: Buffer, x: Buffer, out: Buffer, jobs_per_x_row: int = 1, up: "ExpertWeights | None" = None, stream=None,
+               route: tuple[Buffer, int, bool, float, Buffer] | None = None) -> Buffer:
+    """route = (logits, gating, norm_topk_prob, scale, probs_out) with `up`: the jobs of one token, gated inside the launch from the router
+    logits; sel (k entries) and probs_out receive the selection."""
     n_jobs = int(np.prod(sel.shape))
+    if route is not None:
+      assert up is not None and x.dtype == np.float16 and jobs_per_x_row == n_jobs
+      rt.check(rt.lib().tga_qlinear_experts_routed(self.ggml_type, self.blocks.ptr, up.blocks.ptr, self.num_experts, route[0].ptr, n_jobs, route[1], int(route[2]),
+                                                   route[3], sel.ptr, route[4].ptr, x.ptr, out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
+      return out
     rt.check(rt.lib().tga_qlinear_experts(self.ggml_type, self.blocks.ptr, up.blocks.ptr if up is not None else None, self.num_experts, sel.ptr, n_jobs,
                                           jobs_per_x_row, x.ptr, rt.dtype_code(x.dtype), out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
     return out
@@ -91,11 +99,12 @@ def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer,
 
 def moe_router(x: Buffer, norm_weight: Buffer | None, eps: float, router: QuantLinear, k: int, sel: Buffer, probs: Buffer, logits_ws: Buffer,
                xn_out: Buffer | None = None, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
-  """ffn_norm + router logits + gating + top-k of one token in one launch (dense fp16 router weight).
+  """ffn_norm + router logits + gating + top-k of one token in one launch (dense fp16 router weight).  k = 0: logits only (sel / probs None).
   logits_ws: n_experts + 1 float32, zero before the first use (the last word is an arrival counter)."""
   assert router.ggml_type == rt.F16 and logits_ws.nbytes >= 4 * (router.out_features + 1)
   rt.check(rt.lib().tga_moe_router(x.ptr, norm_weight.ptr if norm_weight is not None else None, eps, router.blocks.ptr, router.in_features, router.out_features, k,
-                                   gating, int(norm_topk_prob), scale, xn_out.ptr if xn_out is not None else None, logits_ws.ptr, sel.ptr, probs.ptr, stream))
+                                   gating, int(norm_topk_prob), scale, xn_out.ptr if xn_out is not None else None, logits_ws.ptr,
+                                   sel.ptr if sel is not None else None, probs.ptr if probs is not None else None, stream))
 
 def moe_combine(y: Buffer, probs: Buffer, resid: Buffer | None, n_tokens: int, k: int, dim: int, out: Buffer, stream=None):
   rt.check(rt.lib().tga_moe_combine(y.ptr, probs.ptr, resid.ptr if resid is not None else None, n_tokens, k, dim, out.ptr, stream))

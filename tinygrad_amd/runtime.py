@@ -38,6 +38,7 @@ def _declare(lib):
     "tga_moe_combine_rmsnorm_qlinear_multi": [vp, vp, i, vp, vp, vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), i, i64, vp],
     "tga_stage_activation": [i, vp, i, i64, vp, vp],
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
+    "tga_qlinear_experts_routed": [i, vp, vp, i64, vp, i, i, i, ctypes.c_float, vp, vp, vp, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
     "tga_moe_router": [vp, vp, ctypes.c_float, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp, vp, vp],
