@@ -243,7 +243,7 @@ class _Shared:
 class Transformer:
   def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096, fused: bool = False):
     """fused: run all blocks of a token in one persistent launch (tga_decode_layers; dense Q4_0 / Q8_0 models only).  The default is
-    one launch per op (six per dense block, eight per MoE block; attention is two), which measures about 10 % faster on the 8B configuration."""
+    one launch per op (six per dense block, seven per MoE block; attention is two), which measures about 10 % faster on the 8B configuration."""
     self.config = c = config
     self.s = _Shared(c, max_new)
     self.max_new = max_new
