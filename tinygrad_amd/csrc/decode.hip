@@ -355,19 +355,36 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 // boundary orders the partials; it costs less than publishing them inside one launch (write-through stores, completion wait, arrival
 // counter, cache-bypassing reads: four dependent memory round trips on the critical path of the last workgroup to arrive).
 template <int HD>
-__global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
+  const AttnArgs a = args;                              // field reads become kernel-argument loads in the entry block
+  constexpr int FB = 24, NB = 16;                       // splits read ahead of the position (contexts up to 1536 in one round trip), later batches
   const int head = blockIdx.x, d = threadIdx.x;
-  const int pos = a.st->pos, ns = (pos >> 6) + 1;
-  __shared__ float sw[1024];                            // exp(m_s - m) / l per split
+  __shared__ float sw[1024];                            // exp(m_s - m) per split
   __shared__ float red[2 * (HD / 64)];
-  const float* ph = a.part + (size_t)head * a.nsplit * (HD + 2);
-  auto run = [&](auto tag) {
-    constexpr int SC = decltype(tag)::value;             // split loads in flight per thread, sized by the number of splits
-    float v[SC];
+  const int nsp = a.nsplit;
+  const float* ph = a.part + (size_t)head * nsp * (HD + 2);
+  // position-independent loads first (splits that were never written are masked below): thread d takes (m, l) of split d, and every
+  // thread the first FB partial outputs of its dimension
+  const int spc = d < nsp ? d : nsp - 1;
+  const float mv = ph[(size_t)spc * (HD + 2) + HD], lv = ph[(size_t)spc * (HD + 2) + HD + 1];
+  float v[FB];
 #pragma unroll
-    for (int j = 0; j < SC; j++) v[j] = ph[(size_t)min(j, ns - 1) * (HD + 2) + d];      // first batch of partial outputs, ahead of the weights
-    // m and l of the splits: thread t takes splits t, t + HD, ...
-    float m = -INFINITY;
+  for (int j = 0; j < FB; j++) v[j] = ph[(size_t)(j < nsp ? j : nsp - 1) * (HD + 2) + d];
+  const int pos = a.st->pos, ns = (pos >> 6) + 1;
+  float m = -INFINITY, l = 0.f;
+  if (nsp <= HD) {
+    m = wave_max(d < ns ? mv : -INFINITY);
+    if constexpr (HD > 64) {
+      if ((d & 63) == 0) red[d >> 6] = m;
+      __syncthreads();
+      m = red[0];
+#pragma unroll
+      for (int i = 1; i < HD / 64; i++) m = fmaxf(m, red[i]);
+    }
+    const float e = d < ns ? __expf(mv - m) : 0.f;
+    if (d < ns) sw[d] = e;
+    l = d < ns ? lv * e : 0.f;
+  } else {                                              // more splits than threads: thread t takes splits t, t + HD, ...
     for (int sp = d; sp < ns; sp += HD) m = fmaxf(m, ph[(size_t)sp * (HD + 2) + HD]);
     m = wave_max(m);
     if constexpr (HD > 64) {
@@ -377,35 +394,30 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs a) {
 #pragma unroll
       for (int i = 1; i < HD / 64; i++) m = fmaxf(m, red[i]);
     }
-    float l = 0.f;
     for (int sp = d; sp < ns; sp += HD) { const float e = __expf(ph[(size_t)sp * (HD + 2) + HD] - m); sw[sp] = e; l += ph[(size_t)sp * (HD + 2) + HD + 1] * e; }
-    l = wave_sum(l);
-    if constexpr (HD > 64) {
-      if ((d & 63) == 0) red[HD / 64 + (d >> 6)] = l;
-      __syncthreads();
-      l = 0.f;
+  }
+  l = wave_sum(l);
+  if constexpr (HD > 64) {
+    if ((d & 63) == 0) red[HD / 64 + (d >> 6)] = l;
+    __syncthreads();
+    l = 0.f;
 #pragma unroll
-      for (int i = 0; i < HD / 64; i++) l += red[HD / 64 + i];
-    } else __syncthreads();
-    const float inv = 1.0f / l;
-    float o = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += SC) {
-      if (s0) {
+    for (int i = 0; i < HD / 64; i++) l += red[HD / 64 + i];
+  } else __syncthreads();
+  float o = 0.f;
 #pragma unroll
-        for (int j = 0; j < SC; j++) v[j] = ph[(size_t)min(s0 + j, ns - 1) * (HD + 2) + d];
-      }
+  for (int j = 0; j < FB; j++) o += j < ns ? v[j] * sw[j] : 0.f;
+  for (int s0 = FB; s0 < ns; s0 += NB) {
+    float w[NB];
 #pragma unroll
-      for (int j = 0; j < SC; j++) if (s0 + j < ns) o += v[j] * sw[s0 + j];
-    }
-    o *= inv;
-    const int e = head * HD + d;
-    if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, e, a.stage_nu) : e] = (_Float16)o;
-    if (a.out32) a.out32[e] = o;
-  };
-  if (ns <= 4) run(std::integral_constant<int, 4>{});
-  else if (ns <= 8) run(std::integral_constant<int, 8>{});
-  else if (ns <= 16) run(std::integral_constant<int, 16>{});
-  else run(std::integral_constant<int, 32>{});
+    for (int j = 0; j < NB; j++) w[j] = ph[(size_t)min(s0 + j, ns - 1) * (HD + 2) + d];
+#pragma unroll
+    for (int j = 0; j < NB; j++) o += s0 + j < ns ? w[j] * sw[s0 + j] : 0.f;
+  }
+  o *= 1.0f / l;
+  const int e = head * HD + d;
+  if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, e, a.stage_nu) : e] = (_Float16)o;
+  if (a.out32) a.out32[e] = o;
 }
 
 // ---------------------------------------------------------------------------------------------- argmax + token bookkeeping
