@@ -238,7 +238,7 @@ int tga_mfma_peak(int n_workgroups, int loops, float* scratch, void* stream);
 
 /* ---- synthetic-model writer (no counterpart in the reference, whose weights always come from GGUF files): fills `out` with
  * n_elements random-init weights U(-amp, amp) (nn.Linear's init range, tinygrad/nn/__init__.py:173-174) already quantized to
- * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule; TGA_F16: plain fp16 cast); TGA_F32 fills the
+ * GGUF blocks of ggml_type (TGA_Q4_0: ggml's reference rule; TGA_Q6_K: absmax rule; TGA_Q4_K: min/max rule; TGA_F16: plain fp16 cast); TGA_F32 fills the
  * constant `amp`; TGA_MXFP4 ignores amp: uniform E2M1 codes with E8M0 bytes uniform in [119, 123] (block scales 2^-8 .. 2^-4). */
 int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, uint32_t seed, float amp, void* stream);
 

@@ -64,3 +64,13 @@ def test_lm_head_sized_q6_k(gpu):
   out = _gpu_dequant(gpu, data, rows * k, 14)
   ref = og.ggml_data_to_tensor(data, rows * k, 14)
   assert out.tobytes() == ref.tobytes()
+
+def test_synth_q4_k_writer_produces_valid_blocks(gpu):
+  """tga_synth_weights(Q4_K): the blocks decode (oracle) to within one quantization step of U(-amp, amp) values: max |w| <= amp * (1 + 1/15)
+  and the values are spread (not a constant), i.e. a valid block stream of the right magnitude."""
+  n, amp = 256 * 64, 0.02
+  buf = gpu.Buffer((n // 256 * 144,), np.uint8)
+  gpu.check(gpu.lib().tga_synth_weights(12, buf.ptr, n, 77, amp, None))
+  w = og.ggml_data_to_tensor(buf.numpy(), n, 12)
+  assert np.isfinite(w).all() and np.abs(w).max() <= amp * 1.1 and w.std() > amp * 0.4
+  assert _gpu_dequant(gpu, buf.numpy(), n, 12).tobytes() == w.tobytes()

@@ -7,6 +7,8 @@
 
   config 6  Q4_K / Q5_K and Q4_1 / Q5_0 / Q5_1 dequant-GEMV at the same linear shapes (not a BASELINE config)
 
+  config 7  Llama-3-8B-architecture decode with the tensor-type mix of a Q4_K_M file (Q4_K, Q6_K for part of attn_v / ffn_down, Q6_K lm-head)
+
     python -m tinygrad_amd.benchmarks [--config N ...]        prints one JSON object per measurement
 
 Timing: HIP events around >= 100 back-to-back launches; weights are rotated over enough distinct copies to exceed the 256 MB
@@ -72,6 +74,26 @@ def kquants():
     for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
       for m in (1, 8): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   return out
+
+def config7(steps: int = 64, ctx: int = 1024):
+  """The 8B architecture of BASELINE config 3 with the tensor types of a Q4_K_M file, same procedure as bench.py (prefill through the model,
+  graph replay + sync per token)."""
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
+  import time
+  c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **LLAMA3_8B)
+  model = Transformer(c, synth_state(c, seed=1007, q4_k_m=True), max_new=steps + 16)
+  rt.synchronize()
+  rng = np.random.default_rng(1007)
+  model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)])
+  for _ in range(8): model.decode_step()
+  rt.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps): model.decode_step()
+  rt.synchronize()
+  dt = (time.perf_counter() - t0) / steps
+  wb = model.weight_bytes_per_token()
+  return [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, Q4_K_M tensor-type mix (Q4_K + Q6_K), graph replay + sync per token",
+           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
 
 def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
@@ -160,13 +182,13 @@ def config5():
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes")
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix")
   ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
   args = ap.parse_args()
   rt.init(0)
   print(json.dumps({"device": rt.device_name()}), flush=True)
   for cfg in args.config:
-    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants}[cfg]
+    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7}[cfg]
     for row in (fn(use_graph=not args.no_graph) if cfg == 4 else fn()): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":

@@ -98,6 +98,42 @@ __global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ out, 
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) out[i] = value;
 }
 
+// Q4_K: a min/max rule per 32-weight sub-block (min m = max(0, -min x), scale s = (max x + m) / 15), superblock d = max s / 63 and
+// dmin = max m / 63 in fp16, 6-bit sc = round(s / d), mn = round(m / dmin), q = clamp(round((x + dmin mn) / (d sc)), 0, 15), packed as
+// ggml's block_q4_K (get_scale_min_k4 layout).  Not ggml's iterative search: just a valid block stream of the right magnitude.
+__global__ __launch_bounds__(256) void synth_q4_k_kernel(uint8_t* __restrict__ out, int64_t nblocks, uint32_t seed, float amp) {
+  for (int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x; b < nblocks; b += (int64_t)gridDim.x * 256) {
+    uint8_t* o = out + b * 144;
+    float s[8], m[8]; float smax = 0.f, mmax = 0.f;
+    for (int g = 0; g < 8; g++) {
+      float lo = 0.f, hi = 0.f;
+      for (int i = 0; i < 32; i++) { const float x = rnd_uniform(seed, (uint64_t)b * 256 + g * 32 + i, amp); lo = fminf(lo, x); hi = fmaxf(hi, x); }
+      m[g] = -lo; s[g] = (hi + m[g]) / 15.0f; smax = fmaxf(smax, s[g]); mmax = fmaxf(mmax, m[g]);
+    }
+    const uint32_t dh = f2h_bits(smax / 63.0f), mh = f2h_bits(mmax / 63.0f);
+    const float d = h2f_bits(dh), dmin = h2f_bits(mh);
+    o[0] = dh & 0xFF; o[1] = dh >> 8; o[2] = mh & 0xFF; o[3] = mh >> 8;
+    int sc[8], mn[8];
+    for (int g = 0; g < 8; g++) { sc[g] = d > 0.f ? min(63, (int)rintf(s[g] / d)) : 0; mn[g] = dmin > 0.f ? min(63, (int)rintf(m[g] / dmin)) : 0; }
+    for (int j = 0; j < 4; j++) {
+      o[4 + j] = (uint8_t)((sc[j] & 63) | ((sc[j + 4] >> 4) << 6));
+      o[8 + j] = (uint8_t)((mn[j] & 63) | ((mn[j + 4] >> 4) << 6));
+      o[12 + j] = (uint8_t)((sc[j + 4] & 0xF) | ((mn[j + 4] & 0xF) << 4));
+    }
+    for (int p = 0; p < 4; p++) {                              // qs[32 p + i]: low nibble = sub-block 2p, high nibble = sub-block 2p + 1
+      for (int i = 0; i < 32; i++) {
+        int q[2];
+        for (int h = 0; h < 2; h++) {
+          const int g = 2 * p + h;
+          const float eff = d * (float)sc[g], x = rnd_uniform(seed, (uint64_t)b * 256 + g * 32 + i, amp);
+          q[h] = eff > 0.f ? max(0, min(15, (int)rintf((x + dmin * (float)mn[g]) / eff))) : 0;
+        }
+        o[16 + 32 * p + i] = (uint8_t)(q[0] | (q[1] << 4));
+      }
+    }
+  }
+}
+
 extern "C" int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, uint32_t seed, float amp, void* stream) {
   TGA_REQUIRE(out && n_elements >= 0, "tga_synth_weights: bad argument");
   hipStream_t s = (hipStream_t)stream;
@@ -114,6 +150,10 @@ extern "C" int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, u
     TGA_REQUIRE(n_elements % 256 == 0, "tga_synth_weights: Q6_K needs a multiple of 256 elements");
     const int64_t nb = n_elements / 256; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
     synth_q6_k_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, amp);
+  } else if (ggml_type == GGML_Q4_K) {
+    TGA_REQUIRE(n_elements % 256 == 0, "tga_synth_weights: Q4_K needs a multiple of 256 elements");
+    const int64_t nb = n_elements / 256; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
+    synth_q4_k_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, amp);
   } else if (ggml_type == GGML_F16) {
     const int grid = (int)((n_elements + 255) / 256 < 65536 ? (n_elements + 255) / 256 : 65536);
     synth_f16_kernel<<<grid, 256, 0, s>>>((_Float16*)out, n_elements, seed, amp);

@@ -83,10 +83,15 @@ def synth_state_moe(config: TransformerConfig, seed: int = 1004, dense_type: int
   mk("output.weight", (c.vocab_size, D), dense_type, D ** -0.5)
   return sd
 
-def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = rt.Q4_0, head_type: int = rt.Q6_K, stream=None) -> dict:
+def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = rt.Q4_0, head_type: int = rt.Q6_K, stream=None,
+                q4_k_m: bool = False) -> dict:
   """Random-init model written straight into HBM as GGUF blocks: {gguf tensor name: (Buffer, ggml_type, (rows, cols))}.
-  Linear and embedding weights ~ U(-1/sqrt(in), 1/sqrt(in)) quantized to linear_type, lm-head to head_type, norm weights 1."""
+  Linear and embedding weights ~ U(-1/sqrt(in), 1/sqrt(in)) quantized to linear_type, lm-head to head_type, norm weights 1.
+  q4_k_m: the tensor-type mix of a Q4_K_M file - Q4_K everywhere except attn_v / ffn_down, which are Q6_K in the first and last eighth
+  of the blocks and in every third block between (llama.cpp's use_more_bits rule), else Q4_K."""
   c, sd, tid = config, {}, [0]
+  if q4_k_m: linear_type = rt.Q4_K
+  def more_bits(i): n = c.num_blocks; return i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2
   def mk(name, rows, cols, t, amp):
     buf = Buffer((quant_nbytes(t, rows * cols),), np.uint8)
     tid[0] += 1
@@ -98,12 +103,13 @@ def synth_state(config: TransformerConfig, seed: int = 1003, linear_type: int = 
     mk(p + "attn_norm.weight", 1, c.dim, rt.F32, 1.0)
     mk(p + "attn_q.weight", c.n_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
     mk(p + "attn_k.weight", c.n_kv_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
-    mk(p + "attn_v.weight", c.n_kv_heads * c.head_dim, c.dim, linear_type, c.dim ** -0.5)
+    vd_type = rt.Q6_K if (q4_k_m and more_bits(i)) else linear_type
+    mk(p + "attn_v.weight", c.n_kv_heads * c.head_dim, c.dim, vd_type, c.dim ** -0.5)
     mk(p + "attn_output.weight", c.dim, c.n_heads * c.head_dim, linear_type, (c.n_heads * c.head_dim) ** -0.5)
     mk(p + "ffn_norm.weight", 1, c.dim, rt.F32, 1.0)
     mk(p + "ffn_gate.weight", c.hidden_dim, c.dim, linear_type, c.dim ** -0.5)
     mk(p + "ffn_up.weight", c.hidden_dim, c.dim, linear_type, c.dim ** -0.5)
-    mk(p + "ffn_down.weight", c.dim, c.hidden_dim, linear_type, c.hidden_dim ** -0.5)
+    mk(p + "ffn_down.weight", c.dim, c.hidden_dim, vd_type, c.hidden_dim ** -0.5)
   mk("output_norm.weight", 1, c.dim, rt.F32, 1.0)
   mk("output.weight", c.vocab_size, c.dim, head_type, c.dim ** -0.5)
   return sd
@@ -159,25 +165,23 @@ class TransformerBlock:
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     qkv, qkv_out = [self.attn_q, self.attn_k, self.attn_v], [s.q, s.k, s.v]
-    same = self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type
     if pending and not self.can_fold_combine:
       moe_combine(s.y_e, s.probs, x, 1, c.num_experts_per_tok, c.dim, x, stream=stream); pending = False
     if pending:                                                          # x + sum_j probs_j y_j completed inside the q/k/v launch, written to the other row buffer
       x_new = s.x2 if x.ptr == s.x.ptr else s.x
       qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps), combine=(s.y_e, s.probs, c.num_experts_per_tok, x_new))
       x = x_new
-    elif self.fuse_norm and same:                                        # the q/k/v launch normalises the row while staging it
-      qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps))
     else:
-      rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
-      if same: qlinear_multi(qkv, s.xn, qkv_out, stream=stream)
-      else:                                                              # mixed types (e.g. Q4_K q / k with a Q6_K v): one launch per run of equal types
-        i = 0
-        while i < 3:
-          j = i + 1
-          while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
-          qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream)
-          i = j
+      # one launch per run of equal block types (e.g. Q4_K q / k with a Q6_K v: two launches); each normalises the row while staging it
+      # when the fast path allows, else one RMSNorm launch feeds them
+      if not self.fuse_norm: rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
+      i = 0
+      while i < 3:
+        j = i + 1
+        while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
+        if self.fuse_norm: qlinear_multi(qkv[i:j], x, qkv_out[i:j], stream=stream, norm=(self.attn_norm, c.norm_eps))
+        else: qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream)
+        i = j
     # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
     rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
                                            int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
