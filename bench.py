@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Headline benchmark: Q4_0 Llama-3-8B-architecture greedy decode at batch 1 on one MI355X (BASELINE.json config 3).
+"""Headline benchmark: Q4_0 Llama-3-8B-architecture greedy decode at batch 1 on one MI355X (benchmark configuration 3).
 
 A step is one decoded token.  Random-init weights are written on the GPU as GGUF blocks (Q4_0 linears and embedding, Q6_K
 lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the model itself, then --warmup + --steps tokens
@@ -155,7 +155,7 @@ def main():
     "metric": "Q4_0 8B-arch decode tok/s @bs1; dequant-GEMV GB/s as % of HBM peak", "value": round(tok_s, 2), "unit": "tok/s",
     "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
     "scaling": "weak", "vs_baseline": None, "dtype": "f16 x q4_0/q6_k -> f32 accumulate", "data": "synthetic",
-    "config": {"workload": f"BASELINE config 3: Llama-3-8B-arch ({c.num_blocks} layers) Q4_0 linears + Q6_K lm-head, random-init, batch 1, "
+    "config": {"workload": f"benchmark configuration 3: Llama-3-8B-arch ({c.num_blocks} layers) Q4_0 linears + Q6_K lm-head, random-init, batch 1, "
                            f"fp16 KV prefilled with {args.prefill} random ids, greedy decode", "device": rt.device_name(),
                "weight_bytes_per_token": int(wbytes), "stream_GBps_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
                "frac_hbm_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},

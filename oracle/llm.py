@@ -4,7 +4,7 @@ Follows: Transformer.forward model.py:358-364; FFNBlock.__call__ :144-151; Trans
 precompute_freqs_cis :16-19; nn.RMSNorm tinygrad/nn/__init__.py:296-304; SDPA tinygrad/mixin/rand.py:298-327; silu
 tinygrad/mixin/elementwise.py:682-690; argmax tinygrad/mixin/op.py:866-891 (first index of the maximum).
 Weights are the float32 dequantization of the same GGUF bytes, cast to fp16 like model.py:376 (w_round_f16) - the model path.
-kv_dtype: the reference's cache is float32 by default (model.py:202); BASELINE config 3 asks for fp16, which is what the build runs."""
+kv_dtype: the reference's cache is float32 by default (model.py:202); benchmark configuration 3 asks for fp16, which is what the build runs."""
 import numpy as np
 from oracle import ggml, moe as omoe
 

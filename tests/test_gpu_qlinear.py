@@ -67,7 +67,7 @@ def test_f32_activations_and_f16_output(gpu, t):
   assert y16.tobytes() == y32.astype(np.float16).tobytes()
 
 def test_config1_q4_0_4096(gpu):
-  """BASELINE config 1 at full size: W 4096x4096 Q4_0, x fp16 [1,4096], fp32 accumulate, fp16 out (seed 1001)."""
+  """benchmark configuration 1 at full size: W 4096x4096 Q4_0, x fp16 [1,4096], fp32 accumulate, fp16 out (seed 1001)."""
   w, x, (n, k) = synth.config1()
   W = ol.weight_f32(w, n, k, 2)
   y32 = _run(gpu, 2, w, x, n, k, np.float32)

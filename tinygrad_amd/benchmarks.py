@@ -5,7 +5,7 @@
   config 5  MXFP8 grouped GEMM at T = 4096, E = 128, k = 8 with Zipf routing (MFMA utilisation and GB/s), plus the measured
             register-only peak of the scaled FP8 MFMA
 
-  config 6  Q4_K / Q5_K and Q4_1 / Q5_0 / Q5_1 dequant-GEMV at the same linear shapes (not a BASELINE config)
+  config 6  Q4_K / Q5_K and Q4_1 / Q5_0 / Q5_1 dequant-GEMV at the same linear shapes (not one of the benchmark's configurations)
 
   config 7  Llama-3-8B-architecture decode with the tensor-type mix of a Q4_K_M file (Q4_K, Q6_K for part of attn_v / ffn_down, Q6_K lm-head)
 
@@ -76,7 +76,7 @@ def kquants():
   return out
 
 def config7(steps: int = 64, ctx: int = 1024):
-  """The 8B architecture of BASELINE config 3 with the tensor types of a Q4_K_M file, same procedure as bench.py (prefill through the model,
+  """The 8B architecture of benchmark configuration 3 with the tensor types of a Q4_K_M file, same procedure as bench.py (prefill through the model,
   graph replay + sync per token)."""
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
   import time
@@ -182,7 +182,7 @@ def config5():
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = BASELINE configs; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix")
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix")
   ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
   args = ap.parse_args()
   rt.init(0)

@@ -1,4 +1,4 @@
-// MXFP8 MoE prefill path (BASELINE config 5): E4M3 quantisation with E8M0 per-32 block scales, token-sorted expert grouping
+// MXFP8 MoE prefill path (benchmark configuration 5): E4M3 quantisation with E8M0 per-32 block scales, token-sorted expert grouping
 // (route / dispatch / combine) and the grouped GEMM on CDNA4 scaled MFMA.
 // Reference: extra/gemm/cdna_asm_gemm.py:149-173 (quantize_mxfp8, mx_pack), extra/gemm/moe_routing.py:89-131 (route, dispatch,
 // combine), extra/gemm/moe_gemm.py:112-134 (grouped_mx_gemm; its HIP kernel source is absent from the reference tree).

@@ -1,6 +1,6 @@
 // Synthetic-model weight writer: fills device buffers with random-init weights already quantized to GGUF blocks, so an
 // 8B-parameter model can be materialised in HBM in well under a second (the reference has no quantizer: its weights arrive
-// quantized inside GGUF files; BASELINE config 3 asks for random-init weights quantized to Q4_0 with a Q6_K lm-head).
+// quantized inside GGUF files; benchmark configuration 3 asks for random-init weights quantized to Q4_0 with a Q6_K lm-head).
 // Values: w = amp * (2u - 1), u = 24-bit uniform from a murmur3-finalizer hash of (seed, element index), i.e. U(-amp, amp)
 // like nn.Linear's init U(-1/sqrt(in), 1/sqrt(in)) (tinygrad/nn/__init__.py:173-174).
 // Q4_0 uses ggml's reference rule (d = signed max / -8, q = min(15, int(x / d + 8.5))); Q6_K uses a plain absmax rule per
@@ -160,7 +160,7 @@ extern "C" int tga_synth_weights(int ggml_type, void* out, int64_t n_elements, u
   } else if (ggml_type == GGML_MXFP4) {
     TGA_REQUIRE(n_elements % 32 == 0, "tga_synth_weights: MXFP4 needs a multiple of 32 elements");
     const int64_t nb = n_elements / 32; const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
-    synth_mxfp4_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, -8, -4);   // amp unused: exponents ~ U[-8, -4] (BASELINE config 4)
+    synth_mxfp4_kernel<<<grid, 256, 0, s>>>((uint8_t*)out, nb, seed, -8, -4);   // amp unused: exponents ~ U[-8, -4] (benchmark configuration 4)
   } else if (ggml_type == GGML_F32) {
     const int grid = (int)((n_elements + 255) / 256 < 65536 ? (n_elements + 255) / 256 : 65536);
     fill_f32_kernel<<<grid, 256, 0, s>>>((float*)out, n_elements, amp);   // constant fill (norm weights = 1)

@@ -38,7 +38,7 @@ class TransformerConfig:
 LLAMA3_8B = dict(num_blocks=32, dim=4096, hidden_dim=14336, n_heads=32, n_kv_heads=8, norm_eps=1e-5, vocab_size=128256,
                  head_dim=128, rope_theta=500000.0)
 
-# OLMoE architecture of BASELINE config 4 (hidden_dim is the expert FFN width, as expert_feed_forward_length maps in model.py:422)
+# OLMoE architecture of benchmark configuration 4 (hidden_dim is the expert FFN width, as expert_feed_forward_length maps in model.py:422)
 OLMOE = dict(num_blocks=16, dim=2048, hidden_dim=1024, n_heads=16, n_kv_heads=16, norm_eps=1e-5, vocab_size=50304, head_dim=128,
              rope_theta=10000.0, qk_norm=2048, num_experts=64, num_experts_per_tok=8, norm_topk_prob=False, expert_gating_func=1)
 
