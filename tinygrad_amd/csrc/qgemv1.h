@@ -421,11 +421,11 @@ static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from
 template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
   if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
-  // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice.
-  // Measured per format at 14336 x 4096 and 4096 x 14336: two rows win for Q4_0, MXFP4, Q4_K (14.3 -> 11.4 us), Q5_K (18.1 -> 15.1 us)
-  // and slightly for Q6_K; Q8_0 pairs (68-byte units) are no faster with two.
-  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1) && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu() / WK
-                  && !(T == GGML_Q6_K && WK > 1);     // Q6_K rows split over several waves: 4096 x 14336 19.3 us with two rows, 17.4 with one
+  // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice, for Q8_0 pairs
+  // (68-byte units: no faster with two) and when the waves of a workgroup split K - with the three-deep ring a single row per step is
+  // faster there (4096 x 14336: Q4_0 in the 8B decode step 12.5 -> 11.7 us, Q4_K 13.2 -> 12.2, Q6_K 19.3 -> 17.4, Q5_0 16.2 -> 15.2).
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1)
+                  && WK == 1 && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu();
   if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
   return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);
 }
