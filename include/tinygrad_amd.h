@@ -26,6 +26,9 @@ extern "C" {
 #define TGA_Q4_K 12
 #define TGA_Q5_K 13
 #define TGA_Q6_K 14
+#define TGA_IQ3_XXS 18  /* tga_dequant only */
+#define TGA_IQ3_S 21    /* tga_dequant only */
+#define TGA_IQ2_S 22    /* tga_dequant only */
 #define TGA_IQ4_XS 23   /* tga_dequant only */
 #define TGA_MXFP4 39
 #define TGA_Q1_0 41     /* tga_dequant only */

@@ -104,6 +104,64 @@ static void deq_iq4_xs(const uint8_t* b, float* y) {
     y += 32; qs += 16;
   }
 }
+/* The codebook types.  An entry of a codebook is kept as its digits over the codebook's alphabet (iq_grids.h). */
+#include "iq_grids.h"
+static int iq3xxs_value(int idx, int j) { const int dg = (IQ3XXS_CODE[idx] >> (3 * j)) & 7; return dg == 7 ? 62 : 4 + 8 * dg; }
+static int iq3s_value(int idx, int j) { return 1 + 2 * ((IQ3S_CODE[idx] >> (3 * j)) & 7); }
+static int iq2s_value(int idx, int j) { int c = IQ2S_CODE[idx]; for (int i = 0; i < j; i++) c /= 3; static const int a[3] = {8, 25, 43}; return a[c % 3]; }
+/* block_iq3_xxs: d, qs[64] indices, 8 x uint32 {4 x 7-bit sign index, 4-bit scale}  (dequantize_row_iq3_xxs; tinygrad/llm/gguf.py:73-81) */
+static void deq_iq3_xxs(const uint8_t* b, float* y) {
+  uint16_t dh; memcpy(&dh, b, 2);
+  const float d = h2f(dh);
+  const uint8_t* qs = b + 2;
+  for (int ib = 0; ib < 8; ib++) {
+    uint32_t aux; memcpy(&aux, b + 66 + 4 * ib, 4);
+    const float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
+    for (int l = 0; l < 4; l++) {
+      const uint32_t s7 = (aux >> (7 * l)) & 127;
+      const uint32_t signs = s7 | ((__builtin_popcount(s7) & 1) << 7);     /* ksigns_iq2xs: the eighth bit makes the parity even */
+      for (int j = 0; j < 4; j++) {
+        y[j]     = db * (float)iq3xxs_value(qs[2 * l], j)     * ((signs >> j) & 1 ? -1.0f : 1.0f);
+        y[j + 4] = db * (float)iq3xxs_value(qs[2 * l + 1], j) * ((signs >> (j + 4)) & 1 ? -1.0f : 1.0f);
+      }
+      y += 8;
+    }
+    qs += 8;
+  }
+}
+/* block_iq3_s: d, qs[64], qh[8], signs[32], scales[4]  (dequantize_row_iq3_s; tinygrad/llm/gguf.py:82-88) */
+static void deq_iq3_s(const uint8_t* b, float* y) {
+  uint16_t dh; memcpy(&dh, b, 2);
+  const float d = h2f(dh);
+  const uint8_t *qs = b + 2, *qh = b + 66, *sg = b + 74, *sc = b + 106;
+  for (int ib = 0; ib < 8; ib++) {
+    const float db = d * (float)(1 + 2 * ((sc[ib / 2] >> (4 * (ib % 2))) & 0xf));
+    for (int l = 0; l < 4; l++) {
+      const int i0 = qs[2 * l] | (((qh[ib] >> (2 * l)) & 1) << 8), i1 = qs[2 * l + 1] | (((qh[ib] >> (2 * l + 1)) & 1) << 8);
+      for (int j = 0; j < 4; j++) {
+        y[j]     = db * (float)iq3s_value(i0, j) * ((sg[l] >> j) & 1 ? -1.0f : 1.0f);
+        y[j + 4] = db * (float)iq3s_value(i1, j) * ((sg[l] >> (j + 4)) & 1 ? -1.0f : 1.0f);
+      }
+      y += 8;
+    }
+    qs += 8; sg += 4;
+  }
+}
+/* block_iq2_s: d, qs[32] indices + 32 sign bytes, qh[8], scales[8]  (dequantize_row_iq2_s; tinygrad/llm/gguf.py:89-95) */
+static void deq_iq2_s(const uint8_t* b, float* y) {
+  uint16_t dh; memcpy(&dh, b, 2);
+  const float d = h2f(dh);
+  const uint8_t *qs = b + 2, *sg = b + 34, *qh = b + 66, *sc = b + 74;
+  for (int ib = 0; ib < 8; ib++) {
+    const float db[2] = {d * (0.5f + (float)(sc[ib] & 0xf)) * 0.25f, d * (0.5f + (float)(sc[ib] >> 4)) * 0.25f};
+    for (int l = 0; l < 4; l++) {
+      const int idx = qs[l] | (((qh[ib] >> (2 * l)) & 3) << 8);
+      for (int j = 0; j < 8; j++) y[j] = db[l / 2] * (float)iq2s_value(idx, j) * ((sg[l] >> j) & 1 ? -1.0f : 1.0f);
+      y += 8;
+    }
+    qs += 4; sg += 4;
+  }
+}
 /* block_q1_0: d, 128 sign bits  (tinygrad/llm/gguf.py:115-118): d * (2 bit - 1) */
 static void deq_q1_0(const uint8_t* b, float* y) {
   uint16_t dh; memcpy(&dh, b, 2);
@@ -157,6 +215,7 @@ static void deq_mxfp4(const uint8_t* b, float* y) {           /* block_mxfp4: gg
 static int type_geom(int t, int* nel, int* nby) {
   switch (t) { case 2: *nel = 32; *nby = 18; return 0; case 8: *nel = 32; *nby = 34; return 0;
                case 23: *nel = 256; *nby = 136; return 0; case 41: *nel = 128; *nby = 18; return 0;
+               case 18: *nel = 256; *nby = 98; return 0; case 21: *nel = 256; *nby = 110; return 0; case 22: *nel = 256; *nby = 82; return 0;
                case 3: *nel = 32; *nby = 20; return 0; case 6: *nel = 32; *nby = 22; return 0; case 7: *nel = 32; *nby = 24; return 0;
                case 12: *nel = 256; *nby = 144; return 0; case 13: *nel = 256; *nby = 176; return 0;
                case 14: *nel = 256; *nby = 210; return 0; case 39: *nel = 32; *nby = 17; return 0; }
@@ -166,6 +225,7 @@ static void deq_block(int t, const uint8_t* b, float* y) {
   switch (t) { case 2: deq_q4_0(b, y); break; case 8: deq_q8_0(b, y); break; case 14: deq_q6_k(b, y); break; case 39: deq_mxfp4(b, y); break;
                case 12: deq_q4_k(b, y); break; case 13: deq_q5_k(b, y); break;
                case 23: deq_iq4_xs(b, y); break; case 41: deq_q1_0(b, y); break;
+               case 18: deq_iq3_xxs(b, y); break; case 21: deq_iq3_s(b, y); break; case 22: deq_iq2_s(b, y); break;
                case 3: deq_q4_1(b, y); break; case 6: deq_q5(b, y, 0); break; case 7: deq_q5(b, y, 1); break; }
 }
 

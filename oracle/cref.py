@@ -22,7 +22,7 @@ def lib():
     _lib.orc_f2h.restype, _lib.orc_f2h.argtypes = ctypes.c_uint16, [ctypes.c_float]
   return _lib
 
-_GEOM = {2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210), 23: (256, 136), 39: (32, 17), 41: (128, 18)}
+_GEOM = {2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210), 18: (256, 98), 21: (256, 110), 22: (256, 82), 23: (256, 136), 39: (32, 17), 41: (128, 18)}
 
 def dequant(ggml_type: int, blocks: np.ndarray, threads: int = 1) -> np.ndarray:
   nel, nby = _GEOM[ggml_type]

@@ -6,8 +6,10 @@ import numpy as np
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4, F32, F16 = 2, 8, 12, 13, 14, 39, 0, 1
 Q4_1, Q5_0, Q5_1 = 3, 6, 7
 IQ4_XS, Q1_0 = 23, 41
+IQ3_XXS, IQ3_S, IQ2_S = 18, 21, 22
 # {ggml_type: (elements per block, bytes per block)}  tinygrad/llm/gguf.py:20-21
-GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17), IQ4_XS: (256, 136), Q1_0: (128, 18)}
+GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17), IQ4_XS: (256, 136), Q1_0: (128, 18),
+              IQ3_XXS: (256, 98), IQ3_S: (256, 110), IQ2_S: (256, 82)}
 # tinygrad/llm/gguf.py:108-110 (== 2 * E2M1 values; ggml_common.py:218 kvalues_mxfp4)
 FP4_LUT = np.array([0.0, 1.0, 2.0, 3.0, 4.0, 6.0, 8.0, 12.0, -0.0, -1.0, -2.0, -3.0, -4.0, -6.0, -8.0, -12.0], dtype=np.float32)
 
@@ -106,7 +108,50 @@ def dequant_q1_0(blocks: np.ndarray) -> np.ndarray:
   bits = np.swapaxes(q_to_uint8(blocks[:, 2:], 1).reshape(-1, 8, 16), -1, -2).reshape(-1, 128).view(np.int8)
   return _f16(blocks[:, :2]) * (bits.astype(np.float32) * 2 - 1)
 
-_DEQ = {IQ4_XS: dequant_iq4_xs, Q1_0: dequant_q1_0, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1, Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
+def _sign_pm1(sign_bytes: np.ndarray) -> np.ndarray:
+  """bit k of byte b -> element 8 b + k: +1.0 where the bit is clear, -1.0 where it is set (gguf.py:79, 86, 92)."""
+  return np.where(q_to_uint8(sign_bytes.reshape(-1, sign_bytes.shape[-1], 1), 1).reshape(sign_bytes.shape[0], -1) == 0, np.float32(1), np.float32(-1))
+
+def dequant_iq3_xxs(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:73-81  98 B: d, 64 codebook indices (4 values each), 8 uint32 words; word ib of sub-block ib (32 values): bits 28..31 =
+  scale s, four 7-bit sign indices at bits 0, 7, 14, 21 (one per 8 values; the 8th sign bit makes the parity even).
+  value = d * (s + 0.5) * 0.5 * grid * sign."""
+  from oracle.iq_grids import grid
+  nb = blocks.shape[0]
+  d = _f16(blocks[:, :2]).reshape(nb, 1, 1, 1)
+  words = np.ascontiguousarray(blocks[:, 66:98]).view(np.uint32).reshape(nb, 8)
+  db = d * ((words >> 28).astype(np.float32) + np.float32(0.5)).reshape(nb, 8, 1, 1) * np.float32(0.5)
+  sign_idx = ((words[:, :, None] >> np.array([0, 7, 14, 21], dtype=np.uint32)) & 0x7F).reshape(nb, 32)
+  even_signs = np.array([i | (0x80 if bin(i).count("1") % 2 else 0) for i in range(128)], dtype=np.uint8)
+  signs = _sign_pm1(even_signs[sign_idx]).reshape(nb, 8, 4, 8)
+  g = grid("iq3xxs")[blocks[:, 2:66]].reshape(nb, 8, 4, 8)
+  return (db * g * signs).reshape(nb, 256)
+
+def dequant_iq3_s(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:82-88  110 B: d, qs[64] (low 8 index bits), qh[8] (bit i % 8 of qh[i // 8] = 9th bit of index i), signs[32], scales[4]
+  (nibble ib of sub-block ib).  value = d * (1 + 2 nibble) * grid[index] * sign."""
+  from oracle.iq_grids import grid
+  nb = blocks.shape[0]
+  d = _f16(blocks[:, :2]).reshape(nb, 1, 1, 1)
+  scales = (1 + 2 * q_to_uint8(blocks[:, 106:110].reshape(nb, 4, 1), 4).reshape(nb, 8)).astype(np.float32).reshape(nb, 8, 1, 1)
+  qh = q_to_uint8(blocks[:, 66:74].reshape(nb, 8, 1), 1).reshape(nb, 64).astype(np.uint16)
+  signs = _sign_pm1(blocks[:, 74:106]).reshape(nb, 8, 4, 8)
+  q = blocks[:, 2:66].astype(np.uint16) + (qh << 8)
+  return (d * scales * grid("iq3s")[q].reshape(nb, 8, 4, 8) * signs).reshape(nb, 256)
+
+def dequant_iq2_s(blocks: np.ndarray) -> np.ndarray:
+  """gguf.py:89-95  82 B: d, qs[32] (low 8 index bits), signs[32], qh[8] (2-bit field i % 4 of qh[i // 4] = index bits 8..9), scales[8]
+  (nibble g of the g-th run of 16 values).  value = d * (nibble + 0.5) * 0.25 * grid[index] * sign, 8 values per index."""
+  from oracle.iq_grids import grid
+  nb = blocks.shape[0]
+  d = _f16(blocks[:, :2]).reshape(nb, 1, 1, 1)
+  db = d * (q_to_uint8(blocks[:, 74:82].reshape(nb, 8, 1), 4).reshape(nb, 16).astype(np.float32) + np.float32(0.5)).reshape(nb, 16, 1, 1) * np.float32(0.25)
+  signs = _sign_pm1(blocks[:, 34:66]).reshape(nb, 16, 2, 8)
+  qh = q_to_uint8(blocks[:, 66:74].reshape(nb, 8, 1), 2).reshape(nb, 32).astype(np.uint16)
+  q = blocks[:, 2:34].astype(np.uint16) + (qh << 8)
+  return (db * grid("iq2s")[q].reshape(nb, 16, 2, 8) * signs).reshape(nb, 256)
+
+_DEQ = {IQ3_XXS: dequant_iq3_xxs, IQ3_S: dequant_iq3_s, IQ2_S: dequant_iq2_s, IQ4_XS: dequant_iq4_xs, Q1_0: dequant_q1_0, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1, Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q5_K: dequant_q5_k, Q6_K: dequant_q6_k, MXFP4: dequant_mxfp4}
 
 def ggml_data_to_tensor(data: np.ndarray, n: int, ggml_type: int) -> np.ndarray:
   """gguf.py:23-119 restricted to the types on the path; returns flat float32 of n elements."""
@@ -271,6 +316,70 @@ def quantize_q1_0(w: np.ndarray) -> np.ndarray:
   out = np.zeros((x.shape[0], 18), dtype=np.uint8)
   out[:, 0:2] = np.abs(x).mean(axis=1).astype(np.float16).view(np.uint8).reshape(-1, 2)
   out[:, 2:] = np.packbits((x >= 0).astype(np.uint8).reshape(-1, 16, 8), axis=2, bitorder="little").reshape(-1, 16)
+  return out.reshape(-1)
+
+def _nearest_entry(mag: np.ndarray, table: np.ndarray) -> np.ndarray:
+  """index of the codebook entry (rows of `table`) nearest in L2 to every row of `mag`."""
+  return (np.float32(-2) * (mag @ table.T) + (table * table).sum(1)[None, :]).argmin(1)
+
+def _d_and_steps(amax_run: np.ndarray, top: float, step_of_d, n_steps: int = 16):
+  """block scale d (fp16) and per-run integer step so that step_of_d(step) * d * top covers the run's largest magnitude."""
+  eff = amax_run / np.float32(top)
+  d = (eff.max(axis=1, keepdims=True) / np.float32(step_of_d(n_steps - 1))).astype(np.float16).astype(np.float32)
+  safe = np.where(d > 0, d, np.float32(1))
+  steps = np.arange(n_steps, dtype=np.float32)
+  step = np.abs(eff[..., None] / safe[..., None] - step_of_d(steps)[None, None, :]).argmin(-1)
+  return d, step.astype(np.uint8), safe * step_of_d(step.astype(np.float32))
+
+def quantize_iq3_xxs(w: np.ndarray) -> np.ndarray:
+  """Simple IQ3_XXS writer for synthetic models (not ggml's search): per 32 weights the 4-bit step nearest to max|x| / 62, per 4 weights the
+  nearest codebook entry; where a run of eight has an odd number of negative weights the smallest one loses its sign (the format stores
+  seven sign bits and fixes the eighth by parity).  Packing as dequant_iq3_xxs decodes."""
+  from oracle.iq_grids import grid
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 8, 32); nb = x.shape[0]
+  d, s, db = _d_and_steps(np.abs(x).max(-1), 62, lambda t: (t + np.float32(0.5)) * np.float32(0.5))
+  idx = _nearest_entry((np.abs(x) / db[..., None]).reshape(-1, 4), grid("iq3xxs")).reshape(nb, 64)
+  neg = (x < 0).reshape(nb, 32, 8)
+  odd = neg.sum(-1) % 2 == 1
+  flip = np.abs(x).reshape(nb, 32, 8).argmin(-1)
+  neg[odd, flip[odd]] ^= True
+  s7 = (neg[:, :, :7] * (1 << np.arange(7))).sum(-1).astype(np.uint32).reshape(nb, 8, 4)
+  words = (s.astype(np.uint32) << 28) | (s7 << (7 * np.arange(4, dtype=np.uint32))).sum(-1).astype(np.uint32)
+  out = np.zeros((nb, 98), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:66] = idx.astype(np.uint8)
+  out[:, 66:98] = np.ascontiguousarray(words.astype("<u4")).view(np.uint8).reshape(nb, 32)
+  return out.reshape(-1)
+
+def quantize_iq3_s(w: np.ndarray) -> np.ndarray:
+  """Simple IQ3_S writer (not ggml's search): per 32 weights the odd multiplier 1 + 2 nibble nearest to max|x| / 15 / d, per 4 weights the nearest of
+  the 512 codebook entries, one sign bit per weight.  Packing as dequant_iq3_s decodes."""
+  from oracle.iq_grids import grid
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 8, 32); nb = x.shape[0]
+  d, nib, dl = _d_and_steps(np.abs(x).max(-1), 15, lambda t: 1 + 2 * t)
+  idx = _nearest_entry((np.abs(x) / dl[..., None]).reshape(-1, 4), grid("iq3s")).reshape(nb, 64)
+  out = np.zeros((nb, 110), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:66] = (idx & 255).astype(np.uint8)
+  out[:, 66:74] = np.packbits((idx >> 8).astype(np.uint8).reshape(nb, 8, 8), axis=2, bitorder="little").reshape(nb, 8)
+  out[:, 74:106] = np.packbits((x < 0).astype(np.uint8).reshape(nb, 32, 8), axis=2, bitorder="little").reshape(nb, 32)
+  out[:, 106:110] = nib[:, 0::2] | (nib[:, 1::2] << 4)
+  return out.reshape(-1)
+
+def quantize_iq2_s(w: np.ndarray) -> np.ndarray:
+  """Simple IQ2_S writer (not ggml's search): per 16 weights the nibble whose (nibble + 0.5) / 4 is nearest to max|x| / 43 / d, per 8 weights the nearest
+  of the 1024 codebook entries, one sign bit per weight.  Packing as dequant_iq2_s decodes."""
+  from oracle.iq_grids import grid
+  x = np.ascontiguousarray(w, dtype=np.float32).reshape(-1, 16, 16); nb = x.shape[0]
+  d, nib, dl = _d_and_steps(np.abs(x).max(-1), 43, lambda t: (t + np.float32(0.5)) * np.float32(0.25))
+  idx = _nearest_entry((np.abs(x) / dl[..., None]).reshape(-1, 8), grid("iq2s")).reshape(nb, 32)
+  out = np.zeros((nb, 82), dtype=np.uint8)
+  out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+  out[:, 2:34] = (idx & 255).astype(np.uint8)
+  out[:, 34:66] = np.packbits((x < 0).astype(np.uint8).reshape(nb, 32, 8), axis=2, bitorder="little").reshape(nb, 32)
+  hi = (idx >> 8).astype(np.uint8).reshape(nb, 8, 4)
+  out[:, 66:74] = hi[:, :, 0] | (hi[:, :, 1] << 2) | (hi[:, :, 2] << 4) | (hi[:, :, 3] << 6)
+  out[:, 74:82] = nib[:, 0::2] | (nib[:, 1::2] << 4)
   return out.reshape(-1)
 
 def quantize_q4_k(w: np.ndarray) -> np.ndarray: return _quantize_q45_k(w, False)

@@ -6,7 +6,7 @@ from tinygrad_amd.runtime import GGML_QUANT, GGML_DEQUANT_ONLY
 GGML_QUANT = {**GGML_QUANT, **GGML_DEQUANT_ONLY}
 
 pytestmark = pytest.mark.gpu
-TYPES = [2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 41]
+TYPES = [2, 3, 6, 7, 8, 12, 13, 14, 18, 21, 22, 23, 39, 41]
 
 def _gpu_dequant(gpu, data, n, t, dtype=np.float32):
   from tinygrad_amd.gguf import ggml_data_to_tensor

@@ -6,16 +6,18 @@ from oracle import ggml as og, gguf as ogguf, llm as ollm, linear as ol
 
 pytestmark = pytest.mark.gpu
 
-def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False, expand: bool = False):
+def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False, expand: bool = False, codebook: bool = False):
   """kquant: the tensor-type mix of a Q4_K_M file (Q4_K linears and embedding, Q6_K for attn_v / ffn_down / output, one Q5_K matrix).
   legacy: the same mix with Q4_1 / Q5_0 / Q5_1 in place of Q4_K / Q5_K / Q6_K.
-  expand: IQ4_XS / Q1_0 / Q6_K: the first two have no in-place linear kernel and are expanded to fp16 when the model is loaded."""
+  expand: IQ4_XS / Q1_0 / Q6_K: the first two have no in-place linear kernel and are expanded to fp16 when the model is loaded.
+  codebook: IQ3_S / IQ2_S / IQ3_XXS, all three expanded to fp16 at load."""
   rng = np.random.default_rng(11)
   c = dict(dim=256, hidden=512, H=4, KV=2, hd=64, L=2, vocab=512)
   def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
-  if kquant or legacy or expand:
+  if kquant or legacy or expand or codebook:
     K4, K5, K6 = (12, og.quantize_q4_k), (13, og.quantize_q5_k), (14, og.quantize_q6_k)
     if expand: K4, K5 = (23, og.quantize_iq4_xs), (41, og.quantize_q1_0)
+    if codebook: K4, K5, K6 = (21, og.quantize_iq3_s), (22, og.quantize_iq2_s), (18, og.quantize_iq3_xxs)
     if legacy: K4, K5, K6 = (3, og.quantize_q4_1), (6, og.quantize_q5_0), (7, og.quantize_q5_1)
     tensors = [("token_embd.weight", (c["vocab"], c["dim"]), K4[0], K4[1](lin(c["vocab"], c["dim"]) * 16))]
     for i in range(c["L"]):
@@ -32,7 +34,7 @@ def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False,
            ("qwen2.block_count", c["L"]), ("qwen2.embedding_length", c["dim"]), ("qwen2.feed_forward_length", c["hidden"]),
            ("qwen2.attention.layer_norm_rms_epsilon", 1e-6), ("qwen2.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(c["vocab"])])]
     from tinygrad_amd.gguf import gguf_write
-    path = tmp_path / ("legacy.gguf" if legacy else "expand.gguf" if expand else "q4_k_m.gguf")
+    path = tmp_path / ("legacy.gguf" if legacy else "expand.gguf" if expand else "codebook.gguf" if codebook else "q4_k_m.gguf")
     return path, gguf_write(path, kvs, tensors)
   tensors = [("token_embd.weight", (c["vocab"], c["dim"]), 8, og.quantize_q8_0(lin(c["vocab"], c["dim"]) * 16))]
   for i in range(c["L"]):
@@ -74,13 +76,13 @@ def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
 
-@pytest.mark.parametrize("legacy", [0, 1, 2], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-q1_0-expanded"])
+@pytest.mark.parametrize("legacy", [0, 1, 2, 3], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-q1_0-expanded", "iq3_s-iq2_s-iq3_xxs-expanded"])
 def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path, legacy):
   """A file with the tensor types of a Q4_K_M model (Q4_K / Q5_K / Q6_K matrices, Q4_K embedding; q/k/v of mixed types, so the
   block runs one launch per projection), and the same mix with the older Q4_1 / Q5_0 / Q5_1 blocks: greedy tokens and logits against
-  the numpy restatement.  Third case: IQ4_XS / Q1_0 matrices, which are expanded to the reference's fp16 weight (model.py:376) at load."""
+  the numpy restatement.  Third and fourth case: IQ4_XS / Q1_0 and IQ3_S / IQ2_S / IQ3_XXS matrices, which are expanded to the reference's fp16 weight (model.py:376) at load."""
   from tinygrad_amd.llm import Transformer
-  path, raw = _make_file(tmp_path, False, kquant=legacy == 0, legacy=legacy == 1, expand=legacy == 2)
+  path, raw = _make_file(tmp_path, False, kquant=legacy == 0, legacy=legacy == 1, expand=legacy == 2, codebook=legacy == 3)
   model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
   assert model.layer_table is None                                     # K-quants take the per-op launches
   cfg, weights, _ = ogguf.from_gguf_weights(raw)

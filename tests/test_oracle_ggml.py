@@ -72,7 +72,7 @@ def test_q6_k_brute_force_layout():
     out = og.ggml_data_to_tensor(b, 256, 14)
     np.testing.assert_array_equal(out, exp, err_msg=f"element {e}")
 
-@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 41])
+@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 18, 21, 22, 23, 39, 41])
 def test_numpy_restatement_equals_scalar_c_loops(t):
   """Vectorised restatement of tinygrad/llm/gguf.py (field-major q_to_uint8) == independent scalar loops of the published ggml
   routines, bit for bit, on fully random bytes (NaN/Inf/subnormal scales included)."""
@@ -167,6 +167,87 @@ def test_iq4_xs_brute_force_layout():
       np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, 23), exp, err_msg=f"element {e}")
       np.testing.assert_array_equal(cref.dequant(23, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
 
+def test_codebooks_are_the_published_tables():
+  """The three codebooks, expanded as _ggml_iq_grid does (gguf.py:11-13: value i = byte i of the packed word), hash to the SHA-256 of the
+  tables the format publishes (ggml-common.h iq3xxs_grid / iq3s_grid / iq2s_grid = tinygrad/runtime/autogen/ggml_common.py:214-216), taken
+  from that text; a few entries are also spelled out (little-endian bytes of the published words 0x0c140c14, 0x3e341c04, 0x05090507,
+  0x0f0f0101, 0x0819081919191919, 0x192b080819191908)."""
+  import hashlib
+  from oracle.iq_grids import grid_u8
+  want = {"iq3xxs": ((256, 4), "46e35f5a997efdee6c99ce57854c8a0d4f0ff8ca57e5e8a60c0793ea580acf5d"),
+          "iq3s": ((512, 4), "bd1af4945a1717c65610b0284e4628b9a1ba3b306fae3a06f6e5f597356e349f"),
+          "iq2s": ((1024, 8), "e1aa1473412b0552c2174c30ef22ab4073f6a181b85a17056e8249bd2932fd88")}
+  for name, (shape, digest) in want.items():
+    g = grid_u8(name)
+    assert g.shape == shape and g.dtype == np.uint8
+    assert hashlib.sha256(g.tobytes()).hexdigest() == digest, name
+    words = sum(g[:, i].astype(np.uint64) << np.uint64(8 * i) for i in range(shape[1]))
+    assert (words[1:] > words[:-1]).all(), name                     # the published tables are sorted as integers
+  assert grid_u8("iq3xxs")[77].tolist() == [0x14, 0x0c, 0x14, 0x0c] and grid_u8("iq3xxs")[255].tolist() == [0x04, 0x1c, 0x34, 0x3e]
+  assert grid_u8("iq3s")[256].tolist() == [7, 5, 9, 5] and grid_u8("iq3s")[511].tolist() == [1, 1, 15, 15]
+  assert grid_u8("iq2s")[256].tolist() == [0x19, 0x19, 0x19, 0x19, 0x19, 0x08, 0x19, 0x08] and grid_u8("iq2s")[770].tolist() == [0x08, 0x19, 0x19, 0x19, 0x08, 0x08, 0x2b, 0x19]
+
+_D = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+
+def test_iq3_xxs_brute_force_layout():
+  """One weight at a time against ggml's block_iq3_xxs (dequantize_row_iq3_xxs): sub-block ib = e // 32 reads word ib at byte 66 + 4 ib: bits
+  28..31 scale s (db = d (s + 0.5) / 2), bits 7 l..7 l + 6 the sign index of its l-th run of eight (the eighth sign bit = odd parity of the
+  seven); index byte 2 + e // 4 selects four values."""
+  entry = {5: [62, 12, 4, 4], 77: [20, 12, 20, 12], 255: [4, 28, 52, 62]}
+  for e in [0, 3, 4, 7, 8, 31, 32, 45, 100, 127, 128, 199, 254, 255]:
+    for idx, s in ((5, 5), (77, 15), (255, 1)):
+      b = np.zeros(98, dtype=np.uint8); b[0:2] = _D
+      ib, l, k = e // 32, (e % 32) // 8, e % 8
+      s7 = (1 << k) if k < 7 else 1                              # odd parity: element 7 of the run flips as well
+      b[66 + 4 * ib:70 + 4 * ib] = np.frombuffer(np.uint32((s << 28) | (s7 << (7 * l))).tobytes(), np.uint8)
+      b[2 + e // 4] = idx
+      exp = np.full(256, 0.25 * 0.5 * 0.5 * 4, dtype=np.float32)
+      db = 0.25 * (s + 0.5) * 0.5
+      exp[32 * ib:32 * ib + 32] = db * 4
+      exp[4 * (e // 4):4 * (e // 4) + 4] = [db * v for v in entry[idx]]
+      run = 32 * ib + 8 * l
+      for kk in ({k, 7} if k < 7 else {0, 7}): exp[run + kk] = -exp[run + kk]
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, 18), exp, err_msg=f"element {e}")
+      np.testing.assert_array_equal(cref.dequant(18, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
+
+def test_iq3_s_brute_force_layout():
+  """block_iq3_s (dequantize_row_iq3_s): 9-bit index i = e // 4 = qs[i] | bit i % 8 of qh[i // 8] << 8 (qs at byte 2, qh at 66); sign of element e = bit
+  e % 8 of byte 74 + e // 8; scale of sub-block ib = 1 + 2 * nibble ib of the four bytes at 106."""
+  entry = {3: [11, 1, 1, 1], 256: [7, 5, 9, 5], 300: [3, 5, 3, 7], 511: [1, 1, 15, 15]}
+  for e in [0, 3, 4, 7, 8, 31, 32, 45, 100, 127, 128, 199, 254, 255]:
+    for idx, nib in ((3, 6), (256, 15), (300, 1), (511, 9)):
+      b = np.zeros(110, dtype=np.uint8); b[0:2] = _D
+      ib, i = e // 32, e // 4
+      b[106 + ib // 2] = nib << (4 * (ib % 2))
+      b[2 + i] = idx & 255; b[66 + i // 8] = (idx >> 8) << (i % 8)
+      b[74 + e // 8] = 1 << (e % 8)
+      exp = np.full(256, 0.25, dtype=np.float32)                 # entry 0 = (1, 1, 1, 1), scale 1
+      dl = 0.25 * (1 + 2 * nib)
+      exp[32 * ib:32 * ib + 32] = dl
+      exp[4 * i:4 * i + 4] = [dl * v for v in entry[idx]]
+      exp[e] = -exp[e]
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, 21), exp, err_msg=f"element {e}")
+      np.testing.assert_array_equal(cref.dequant(21, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
+
+def test_iq2_s_brute_force_layout():
+  """block_iq2_s (dequantize_row_iq2_s): 10-bit index i = e // 8 = qs[i] | 2-bit field i % 4 of qh[i // 4] << 8 (qs at byte 2, qh at 66), eight values per
+  index; sign of element e = bit e % 8 of byte 34 + i; the g-th run of 16 has db = d (nibble g + 0.5) / 4, nibbles in the eight bytes at 74."""
+  entry = {2: [25, 25, 8, 8, 8, 8, 8, 8], 255: [43, 8, 25, 25, 25, 8, 25, 8], 513: [25, 8, 8, 25, 25, 8, 8, 25], 770: [8, 25, 25, 25, 8, 8, 43, 25], 1023: [43] * 8}
+  for e in [0, 7, 8, 15, 16, 31, 32, 45, 100, 127, 128, 199, 248, 255]:
+    for idx, nib in ((2, 7), (255, 15), (513, 1), (770, 4), (1023, 10)):
+      b = np.zeros(82, dtype=np.uint8); b[0:2] = _D
+      g, i = e // 16, e // 8
+      b[74 + g // 2] = nib << (4 * (g % 2))
+      b[2 + i] = idx & 255; b[66 + i // 4] = (idx >> 8) << (2 * (i % 4))
+      b[34 + i] = 1 << (e % 8)
+      exp = np.full(256, 0.25 * 0.5 * 0.25 * 8, dtype=np.float32)   # entry 0 = eight 8s, nibble 0
+      dl = 0.25 * (nib + 0.5) * 0.25
+      exp[16 * g:16 * g + 16] = dl * 8
+      exp[8 * i:8 * i + 8] = [dl * v for v in entry[idx]]
+      exp[e] = -exp[e]
+      np.testing.assert_array_equal(og.ggml_data_to_tensor(b, 256, 22), exp, err_msg=f"element {e}")
+      np.testing.assert_array_equal(cref.dequant(22, b[None]).reshape(-1), exp, err_msg=f"element {e} (C)")
+
 def test_q1_0_brute_force_layout():
   """Q1_0: element e is bit e % 8 of byte 2 + e // 8; set bit -> +d, clear bit -> -d."""
   for e in [0, 1, 7, 8, 9, 63, 64, 100, 127]:
@@ -191,6 +272,10 @@ def test_quantizers_round_trip():
     nel = {14: 16, 23: 32}.get(t, og.GGML_QUANT[t][0])
     amax = np.abs(w.reshape(-1, nel)).max(1, keepdims=True)
     assert (np.abs(dq.reshape(-1, nel) - w.reshape(-1, nel)) <= tol * amax + 1e-6).all(), t
+  # the codebook types: a vector codebook bounds no single weight's error; the decoded weights must follow the originals closely
+  for t, qf, corr in ((18, og.quantize_iq3_xxs, 0.97), (21, og.quantize_iq3_s, 0.98), (22, og.quantize_iq2_s, 0.95)):
+    dq = og.ggml_data_to_tensor(qf(w), w.size, t)
+    assert np.corrcoef(dq, w)[0, 1] > corr and (np.sign(dq) == np.sign(w)).mean() > 0.93, t
 
 def test_unknown_type_raises():
   with pytest.raises(ValueError): og.ggml_data_to_tensor(np.zeros(512, np.uint8), 256, 1337)   # test/unit/test_gguf.py:114-116

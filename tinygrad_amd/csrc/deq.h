@@ -2,6 +2,7 @@
 // Float contraction is off inside every get4: each product must round exactly like the reference's separate multiplies.
 #pragma once
 #include "common.h"
+#include "iq_grids.h"
 
 // 4 consecutive dequantized values starting at element e0 (a multiple of 4) of block `b`.
 template <int T> struct Deq;
@@ -114,6 +115,63 @@ template <> struct Deq<GGML_IQ4_XS> {
     const int hi = (l >= 16) ? 4 : 0; const uint8_t* q = b + 8 + 16 * ib + (l & 15);
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = dl * iq4nl_value((q[i] >> hi) & 0xF);
+  }
+};
+// The codebook types (tinygrad/llm/gguf.py:73-95).  A codebook entry is kept as its digits over the codebook's alphabet (iq_grids.h); sign bit k
+// of a sign byte negates value k of its run of eight.
+__device__ __forceinline__ float pm1(uint32_t bits, int k) { return ((bits >> k) & 1u) ? -1.0f : 1.0f; }
+// IQ3_XXS (98 B: d, qs[64], 8 uint32 words), gguf.py:73-81: word ib of sub-block ib holds the scale s in bits 28..31 and four 7-bit sign indices
+// (an eighth bit makes each sign byte's parity even); value = ((d * (s + 0.5)) * 0.5) * grid * sign, 4 values per index byte.
+template <> struct Deq<GGML_IQ3_XXS> {
+  static constexpr int NEL = 256, NBY = 98;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b));
+    const int ib = e0 >> 5, l = (e0 >> 3) & 3;
+    const uint8_t* w = b + 66 + 4 * ib;
+    const uint32_t aux = (uint32_t)ld2(w) | ((uint32_t)ld2(w + 2) << 16);
+    const float db = d * ((float)(aux >> 28) + 0.5f) * 0.5f;
+    const uint32_t s7 = (aux >> (7 * l)) & 127u, signs = (s7 | ((__builtin_popcount(s7) & 1u) << 7)) >> (e0 & 4);
+    const uint32_t code = IQ3XXS_CODE[b[2 + (e0 >> 2)]];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t dg = (code >> (3 * i)) & 7u;
+      o[i] = db * (float)(dg == 7u ? 62u : 4u + 8u * dg) * pm1(signs, i);
+    }
+  }
+};
+// IQ3_S (110 B: d, qs[64], qh[8], signs[32], scales[4]), gguf.py:82-88: index i = qs[i] | bit i % 8 of qh[i / 8] << 8;
+// value = ((d * (1 + 2 nibble ib)) * grid) * sign
+template <> struct Deq<GGML_IQ3_S> {
+  static constexpr int NEL = 256, NBY = 110;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b));
+    const int ib = e0 >> 5, i = e0 >> 2;
+    const float dl = d * (float)(1 + 2 * (int)((b[106 + (ib >> 1)] >> (4 * (ib & 1))) & 0xF));
+    const uint32_t code = IQ3S_CODE[(uint32_t)b[2 + i] | ((((uint32_t)b[66 + (i >> 3)] >> (i & 7)) & 1u) << 8)];
+    const uint32_t signs = (uint32_t)b[74 + (e0 >> 3)] >> (e0 & 4);
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = dl * (float)(1u + 2u * ((code >> (3 * k)) & 7u)) * pm1(signs, k);
+  }
+};
+// IQ2_S (82 B: d, qs[32], signs[32], qh[8], scales[8]), gguf.py:89-95: index i = qs[i] | 2-bit field i % 4 of qh[i / 4] << 8, 8 values per index;
+// value = (((d * (nibble g + 0.5)) * 0.25) * grid) * sign, g = the run of 16 values
+template <> struct Deq<GGML_IQ2_S> {
+  static constexpr int NEL = 256, NBY = 82;
+  static __device__ __forceinline__ void get4(const uint8_t* b, int e0, float* o) {
+#pragma clang fp contract(off)
+    const float d = h2f_bits(ld2(b));
+    const int g = e0 >> 4, i = e0 >> 3;
+    const float dl = d * ((float)((b[74 + (g >> 1)] >> (4 * (g & 1))) & 0xF) + 0.5f) * 0.25f;
+    uint32_t code = IQ2S_CODE[(uint32_t)b[2 + i] | ((((uint32_t)b[66 + (i >> 2)] >> (2 * (i & 3))) & 3u) << 8)];
+    if (e0 & 4) code /= 81u;                                   // skip the first four base-3 digits
+    const uint32_t signs = (uint32_t)b[34 + i] >> (e0 & 4);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const uint32_t t = code % 3u; code /= 3u;
+      o[k] = dl * (float)(8u + 17u * t + (t >> 1)) * pm1(signs, k);   // {8, 25, 43}
+    }
   }
 };
 // Q1_0 (18 B: d, 128 sign bits), tinygrad/llm/gguf.py:115-118: value = d * (2 bit - 1), element e = bit e % 8 of byte e / 8

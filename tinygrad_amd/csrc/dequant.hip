@@ -1,5 +1,5 @@
 // Block dequant kernels: bit-exact restatement of ggml_data_to_tensor (tinygrad/llm/gguf.py:23-119) for Q4_0 (:46), Q4_1 (:47-49), Q5_0 / Q5_1 (:50-55), Q8_0 (:56),
-// Q4_K / Q5_K (:57-67), Q6_K (:68-72), IQ4_XS (:96-104), MXFP4 (:105-114) and Q1_0 (:115-118).  One thread produces 4 consecutive output elements (one 16-byte or 8-byte store), so
+// Q4_K / Q5_K (:57-67), Q6_K (:68-72), IQ3_XXS / IQ3_S / IQ2_S (:73-95), IQ4_XS (:96-104), MXFP4 (:105-114) and Q1_0 (:115-118).  One thread produces 4 consecutive output elements (one 16-byte or 8-byte store), so
 // stores are fully coalesced; the packed bytes are re-read through L1/L2 (this kernel is a load-time / test utility, the
 // decode path never materialises weights).
 #include "deq.h"
@@ -50,6 +50,9 @@ extern "C" int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* o
     case GGML_Q6_K: return launch_dequant<GGML_Q6_K>(blocks, n, out, out_dtype, s);
     case GGML_MXFP4: return launch_dequant<GGML_MXFP4>(blocks, n, out, out_dtype, s);
     case GGML_IQ4_XS: return launch_dequant<GGML_IQ4_XS>(blocks, n, out, out_dtype, s);
+    case GGML_IQ3_XXS: return launch_dequant<GGML_IQ3_XXS>(blocks, n, out, out_dtype, s);
+    case GGML_IQ3_S: return launch_dequant<GGML_IQ3_S>(blocks, n, out, out_dtype, s);
+    case GGML_IQ2_S: return launch_dequant<GGML_IQ2_S>(blocks, n, out, out_dtype, s);
     case GGML_Q1_0: return launch_dequant<GGML_Q1_0>(blocks, n, out, out_dtype, s);
   }
   return tga_set_error("GGML type '%d' is not supported!", ggml_type);   // message of tinygrad/llm/gguf.py:119

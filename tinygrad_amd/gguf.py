@@ -2,7 +2,7 @@
 
 ggml_data_to_tensor(t, n, ggml_type) mirrors tinygrad/llm/gguf.py:23: `t` is the raw byte buffer (device Buffer of uint8, or a
 numpy array that is uploaded), `n` the element count, and the result is a flat float32 device Buffer of n elements, bit-exact
-with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ4_XS (23), MXFP4 (39), Q1_0 (41); native float32/float16 (0, 1) are reinterpreted in place.
+with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ3_XXS (18), IQ3_S (21), IQ2_S (22), IQ4_XS (23), MXFP4 (39), Q1_0 (41); native float32/float16 (0, 1) are reinterpreted in place.
 Unknown types raise ValueError with the reference's message (gguf.py:119)."""
 from __future__ import annotations
 import numpy as np

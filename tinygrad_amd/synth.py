@@ -19,7 +19,7 @@ def random_blocks(rng, ggml_type: int, n: int, k: int, sigma: float = 0.003, mx_
   assert k % nel == 0
   nb = n * (k // nel)
   b = rng.integers(0, 256, size=(nb, nby), dtype=np.uint8)
-  if ggml_type in (Q4_0, Q5_0, 23, 41): b[:, :2] = _scales(rng, nb, sigma)   # (23 = IQ4_XS, 41 = Q1_0: dequant only)
+  if ggml_type in (Q4_0, Q5_0, 18, 21, 22, 23, 41): b[:, :2] = _scales(rng, nb, sigma)   # (18 / 21 / 22 = IQ3_XXS / IQ3_S / IQ2_S, 23 = IQ4_XS, 41 = Q1_0: dequant only)
   elif ggml_type in (Q4_1, Q5_1):                                       # d > 0 and a signed fp16 minimum of the same magnitude as the weights
     b[:, :2] = _scales(rng, nb, sigma)
     b[:, 2:4] = np.float16(rng.standard_normal(nb) * sigma * 4).view(np.uint8).reshape(nb, 2)
