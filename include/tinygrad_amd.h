@@ -210,6 +210,10 @@ int tga_quantize_mxfp8(const void* x, int x_is_bf16, int64_t rows, int64_t K, vo
  * float32 from two (rows, K) bf16 tensors (sigmoid = 1 / (1 + exp2(-w1 * log2 e))), quantized as tga_quantize_mxfp8 without an intermediate
  * tensor; outputs as there. */
 int tga_silu_mul_quantize_mxfp8(const void* x_w1_bf16, const void* x_w3_bf16, int64_t rows, int64_t K, void* q, void* e8, void* packed, void* stream);
+/* transpose_quantize_mxfp8 (extra/llama_kernels/transpose_quantize_mxfp8/__init__.py:24-37): the outputs of tga_quantize_mxfp8 for the
+ * transpose of g without forming it.  g: (M, N) bf16, M % 32 == 0, N % 64 == 0 (the reference asks N % 256); q: (N, M) bytes; e8: (N, M/32)
+ * bytes; packed (may be NULL; needs M % 128 == 0): (M/128, N) uint32. */
+int tga_transpose_quantize_mxfp8(const void* g_bf16, int64_t M, int64_t N, void* q, void* e8, void* packed, void* stream);
 
 /* route (moe_routing.py:109-122) for one device group: top-k (descending, lower index first among equals), weights =
  * softmax(top values), per-expert counts padded to 256 -> off (E+1), dest_row[j] = off[e_j] + stable rank of assignment j among

@@ -54,6 +54,12 @@ def silu_mul_quantize_mxfp8(x_w1: np.ndarray, x_w3: np.ndarray):
   with np.errstate(over="ignore"): sig = (np.float32(1.0) / (np.float32(1.0) + np.exp2(w1 * np.float32(-1.4426950408889634)))).astype(np.float32)
   return quantize_mxfp8((w1 * sig * w3).astype(np.float32))
 
+def transpose_quantize_mxfp8(g: np.ndarray):
+  """extra/llama_kernels/transpose_quantize_mxfp8/__init__.py:24-25: "(q, e8, si) == quantize_mxfp8(g.T)" for g (M, N): q (N, M), e8 (N, M/32),
+  si = mx_pack(e8) (M/128, N)."""
+  q, e8 = quantize_mxfp8(np.ascontiguousarray(np.asarray(g, dtype=np.float32).T))
+  return q, e8, (mx_pack(e8) if e8.shape[1] % 4 == 0 else None)
+
 def block_scale(e8: np.ndarray) -> np.ndarray:
   """cdna_asm_gemm.py:165-173: dequant scale 2^(e8-127) broadcast to element shape."""
   return np.repeat(np.exp2(e8.astype(np.float32) - 127.0).astype(np.float32), 32, axis=-1)

@@ -21,6 +21,25 @@ def test_quantize_mxfp8_bit_exact(gpu):
   rq2, re82 = omx.quantize_mxfp8(moe.from_bf16_bits(xb))
   np.testing.assert_array_equal(e82.numpy(), re82); np.testing.assert_array_equal(q2.numpy(), rq2)
 
+@pytest.mark.parametrize("M,N", [(256, 512), (96, 64), (384, 320)])
+def test_transpose_quantize_mxfp8_bit_exact(gpu, M, N):
+  """transpose_quantize_mxfp8(g) == quantize_mxfp8(g.T) (extra/llama_kernels/transpose_quantize_mxfp8/__init__.py:24-25): bit-exact against the
+  oracle and against this library's own row-wise quantizer fed the transposed matrix; M = 96 has a partial 128-row tile and no packed scales."""
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(M + N)
+  g = (rng.standard_normal((M, N)) * np.exp2(rng.integers(-20, 12, size=(1, N)))).astype(np.float32)
+  g[:32, 0] = 0; g[32:64, 1] = 2.0 ** -3; g[5, 2] = 448.0; g[:32, 3] = 1e-30
+  gb = moe.to_bf16_bits(g)
+  q, e8, si = moe.transpose_quantize_mxfp8(gpu.Buffer.from_numpy(gb))
+  rq, re8, rsi = omx.transpose_quantize_mxfp8(moe.from_bf16_bits(gb))
+  assert q.shape == (N, M) and e8.shape == (N, M // 32)
+  np.testing.assert_array_equal(e8.numpy(), re8); np.testing.assert_array_equal(q.numpy(), rq)
+  if M % 128 == 0: np.testing.assert_array_equal(si.numpy(), rsi)
+  else: assert si is None and rsi is None
+  q2, e82, si2 = moe.quantize_mxfp8(gpu.Buffer.from_numpy(np.ascontiguousarray(gb.T)))
+  np.testing.assert_array_equal(q2.numpy(), q.numpy()); np.testing.assert_array_equal(e82.numpy(), e8.numpy())
+  if M % 128 == 0: np.testing.assert_array_equal(si2.numpy(), si.numpy())
+
 def test_fused_silu_mul_quantize_mxfp8(gpu):
   """silu(x_w1) * x_w3 quantized without an intermediate tensor (extra/llama_kernels/fused_silu_mul_quantize_mxfp8).  The product is
   formed in float32 from exp2; where the device's exp2 differs from numpy's in the last ulp an E4M3 code may land on the other side of

@@ -36,6 +36,25 @@ __device__ __forceinline__ uint32_t f_to_e4m3(float x) {
 // ------------------------------------------------------------------------------------------------ quantize_mxfp8
 // One thread per 32-element block: amax, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254), q = e4m3(clamp(x * 2^(127-e8), +-448)).
 // Also writes the packed scales of mx_pack: packed[k/128][row] = 4 consecutive e8 bytes (little-endian).
+// One 32-element block: e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254); out = 32 E4M3 bytes of clamp(v * 2^(127 - e8), +-448).
+__device__ __forceinline__ int mx_quant32(const float* v, uint32_t* out) {
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+  int ex; (void)frexpf(amax, &ex);                         // floor(log2(a)) = ex - 1
+  // below the smallest normal float the reference's max(amax, 1e-38) floor gives floor(log2) = -127 -> e8 = 0
+  int e = amax < 1.17549435e-38f ? 0 : ex - 1 + 127; e = e < 0 ? 0 : (e > 254 ? 254 : e);
+  const float qs = __builtin_bit_cast(float, (uint32_t)(254 - e) << 23);   // 2^(127 - e), exact for e in 0..253; e = 254 -> 2^-127 below
+  const float scale = (e == 254) ? __builtin_bit_cast(float, 0x00400000u) : qs;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) { float s = v[4 * i + j] * scale; s = fminf(fmaxf(s, -448.0f), 448.0f); w |= f_to_e4m3(s) << (8 * j); }
+    out[i] = w;
+  }
+  return e;
+}
 // MODE 0: x float32; 1: x bf16; 2: fused SwiGLU producer, value = w1 * sigmoid(w1) * w3 in float32 from two bf16 tensors x (= x_w1)
 // and x2 (= x_w3), sigmoid as 1 / (1 + exp2(-w1 * log2(e)))  (extra/llama_kernels/fused_silu_mul_quantize_mxfp8/__init__.py:33-36)
 template <int MODE>
@@ -44,7 +63,7 @@ __global__ __launch_bounds__(256) void quantize_mxfp8_kernel(const void* __restr
   const long long nb = rows * (K / 32);
   for (long long b = (long long)blockIdx.x * 256 + threadIdx.x; b < nb; b += (long long)gridDim.x * 256) {
     const long long row = b / (K / 32); const int kb = (int)(b % (K / 32));
-    float v[32]; float amax = 0.f;
+    float v[32];
     auto load_bf16 = [&](const void* src, float* o) {
       const u32x4* p = (const u32x4*)((const uint16_t*)src + row * K + kb * 32);
 #pragma unroll
@@ -63,26 +82,43 @@ __global__ __launch_bounds__(256) void quantize_mxfp8_kernel(const void* __restr
 #pragma unroll
       for (int i = 0; i < 8; i++) { const f32x4 w = p[i]; v[4*i] = w.x; v[4*i+1] = w.y; v[4*i+2] = w.z; v[4*i+3] = w.w; }
     }
-#pragma unroll
-    for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
-    int ex; (void)frexpf(amax, &ex);                         // floor(log2(a)) = ex - 1
-    // below the smallest normal float the reference's max(amax, 1e-38) floor gives floor(log2) = -127 -> e8 = 0
-    int e = amax < 1.17549435e-38f ? 0 : ex - 1 + 127; e = e < 0 ? 0 : (e > 254 ? 254 : e);
-    const float qs = __builtin_bit_cast(float, (uint32_t)(254 - e) << 23);   // 2^(127 - e), exact for e in 0..253; e = 254 -> 2^-127 below
-    const float scale = (e == 254) ? __builtin_bit_cast(float, 0x00400000u) : qs;
     uint32_t out[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      uint32_t w = 0;
-#pragma unroll
-      for (int j = 0; j < 4; j++) { float s = v[4 * i + j] * scale; s = fminf(fmaxf(s, -448.0f), 448.0f); w |= f_to_e4m3(s) << (8 * j); }
-      out[i] = w;
-    }
+    const int e = mx_quant32(v, out);
     u32x4* qo = (u32x4*)(q + row * K + kb * 32);
     qo[0] = u32x4{out[0], out[1], out[2], out[3]}; qo[1] = u32x4{out[4], out[5], out[6], out[7]};
     e8[row * (K / 32) + kb] = (uint8_t)e;
     if (packed) packed[((long long)(kb >> 2) * rows + row) * 4 + (kb & 3)] = (uint8_t)e;
   }
+}
+
+// transpose_quantize_mxfp8 (extra/llama_kernels/transpose_quantize_mxfp8/__init__.py:24-37) == quantize_mxfp8(g.T) without the transposed
+// tensor: g (M, N) bf16 -> q (N, M), e8 (N, M / 32), packed (M / 128, N).  One workgroup takes 128 rows x 64 columns of g through LDS
+// (row-wise 16-byte loads, column-wise reads), thread (column c, 32-row run r) quantizes one block, and the four runs of a column fill one
+// 128-byte line of q.
+__global__ __launch_bounds__(256) void transpose_quantize_mxfp8_kernel(const uint16_t* __restrict__ g, int M, int N, uint8_t* __restrict__ q,
+                                                                       uint8_t* __restrict__ e8, uint8_t* __restrict__ packed) {
+  __shared__ uint16_t tile[128][64 + 8];                    // 144-byte rows: 16-byte aligned, column reads of a wave hit 32 different banks
+  const int n0 = blockIdx.x * 64, m0 = blockIdx.y * 128, t = threadIdx.x;
+#pragma unroll
+  for (int p = 0; p < 4; p++) {
+    const int r = p * 32 + (t >> 3), c8 = (t & 7) * 8;
+    u32x4 w = {0, 0, 0, 0};
+    if (m0 + r < M) w = *(const u32x4*)(g + (size_t)(m0 + r) * N + n0 + c8);
+    *(u32x4*)&tile[r][c8] = w;
+  }
+  __syncthreads();
+  const int c = t & 63, run = t >> 6;
+  if (m0 + run * 32 >= M) return;
+  float v[32];
+#pragma unroll
+  for (int i = 0; i < 32; i++) v[i] = bf16_to_f(tile[run * 32 + i][c]);
+  uint32_t out[8];
+  const int e = mx_quant32(v, out);
+  const int kb = (m0 >> 5) + run;
+  u32x4* qo = (u32x4*)(q + (size_t)(n0 + c) * M + m0 + run * 32);
+  qo[0] = u32x4{out[0], out[1], out[2], out[3]}; qo[1] = u32x4{out[4], out[5], out[6], out[7]};
+  e8[(size_t)(n0 + c) * (M / 32) + kb] = (uint8_t)e;
+  if (packed) packed[((size_t)(kb >> 2) * N + n0 + c) * 4 + (kb & 3)] = (uint8_t)e;
 }
 
 // ------------------------------------------------------------------------------------------------ route
@@ -414,6 +450,17 @@ int tga_silu_mul_quantize_mxfp8(const void* x_w1_bf16, const void* x_w3_bf16, in
   const long long nb = rows * (K / 32);
   const int grid = (int)((nb + 255) / 256 < 65536 ? (nb + 255) / 256 : 65536);
   quantize_mxfp8_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(x_w1_bf16, x_w3_bf16, rows, (int)K, (uint8_t*)q, (uint8_t*)e8, (uint8_t*)packed);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_transpose_quantize_mxfp8(const void* g_bf16, int64_t M, int64_t N, void* q, void* e8, void* packed, void* stream) {
+  TGA_REQUIRE(g_bf16 && q && e8, "tga_transpose_quantize_mxfp8: null pointer");
+  TGA_REQUIRE(M > 0 && N > 0 && M % 32 == 0 && N % 64 == 0, "tga_transpose_quantize_mxfp8: M=%lld must be a multiple of 32 and N=%lld of 64", (long long)M, (long long)N);
+  TGA_REQUIRE(!packed || M % 128 == 0, "tga_transpose_quantize_mxfp8: packed scales need M %% 128 == 0");
+  TGA_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && (M + 127) / 128 <= 65535, "tga_transpose_quantize_mxfp8: matrix too large");
+  transpose_quantize_mxfp8_kernel<<<dim3((unsigned)(N / 64), (unsigned)((M + 127) / 128)), 256, 0, (hipStream_t)stream>>>((const uint16_t*)g_bf16, (int)M, (int)N, (uint8_t*)q, (uint8_t*)e8,
+                                                                                                                        (uint8_t*)packed);
   TGA_LAUNCH_CHECK();
   return 0;
 }

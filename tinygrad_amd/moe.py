@@ -73,6 +73,17 @@ def fused_silu_mul_quantize_mxfp8(x_w1: Buffer, x_w3: Buffer, stream=None):
   rt.check(rt.lib().tga_silu_mul_quantize_mxfp8(x_w1.ptr, x_w3.ptr, rows, K, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
   return q, e8, packed
 
+def transpose_quantize_mxfp8(g: Buffer, stream=None):
+  """extra/llama_kernels/transpose_quantize_mxfp8/__init__.py:24-37: g (M, N) bf16 bits -> (q, e8, si) == quantize_mxfp8(g.T): q uint8 (N, M),
+  e8 uint8 (N, M/32), si uint32 (M/128, N) (None when M % 128 != 0); the transposed tensor is never formed."""
+  assert len(g.shape) == 2 and g.dtype == np.uint16, f"{g.shape} {g.dtype}"
+  M, N = g.shape
+  assert M % 32 == 0 and N % 64 == 0, f"M={M} must%32, N={N} must%64"
+  q, e8 = Buffer((N, M), np.uint8), Buffer((N, M // 32), np.uint8)
+  packed = Buffer((M // 128, N), np.uint32) if M % 128 == 0 else None
+  rt.check(rt.lib().tga_transpose_quantize_mxfp8(g.ptr, M, N, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
+  return q, e8, packed
+
 def grouped_mx_gemm(x: Buffer, w: tuple[Buffer, Buffer], expert_off: Buffer, stream=None, out: Buffer | None = None) -> Buffer:
   """moe_gemm.py:112-134 with pre-quantized weights w = (w_q (E,N,K) e4m3 bits, w_e8 (E,N,K/32)): quantizes x (M,K) bf16 to MXFP8 and
   runs the grouped GEMM; returns (M, N) bf16 bits."""
