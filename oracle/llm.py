@@ -55,13 +55,16 @@ class Model:
       p = f"blk.{i}."
       n = rmsnorm(x, self.w[p + "attn_norm.weight"].reshape(-1), eps)
       q, k = self._lin(p + "attn_q.weight", n), self._lin(p + "attn_k.weight", n)
+      if p + "attn_q.bias" in self.w: q, k = q + self.w[p + "attn_q.bias"].reshape(-1), k + self.w[p + "attn_k.bias"].reshape(-1)   # Linear(bias=qkv_bias), model.py:161-163
       if c.get("qk_norm", 0) and c["qk_norm"] != hd:                        # model.py:169: full-width q/k norm before the head split
         q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
       q, k = q.reshape(H, hd), k.reshape(KV, hd)
       if c.get("qk_norm", 0) == hd:                                         # model.py:180: per-head q/k norm after the head split
         q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
       q, k = apply_rope(q, self.fc[pos]), apply_rope(k, self.fc[pos])
-      v = self._lin(p + "attn_v.weight", n).reshape(KV, hd)
+      v = self._lin(p + "attn_v.weight", n)
+      if p + "attn_v.bias" in self.w: v = v + self.w[p + "attn_v.bias"].reshape(-1)
+      v = v.reshape(KV, hd)
       self.ck[i, :, pos], self.cv[i, :, pos] = k.astype(self.kv_dtype), v.astype(self.kv_dtype)
       K = np.repeat(self.ck[i, :, :pos + 1].astype(np.float32), H // KV, axis=0)      # (H, T, hd)  GQA repeat_interleave
       V = np.repeat(self.cv[i, :, :pos + 1].astype(np.float32), H // KV, axis=0)

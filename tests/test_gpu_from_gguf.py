@@ -135,3 +135,54 @@ def test_from_gguf_qwen3_shape_per_head_qk_norm(gpu, tmp_path):
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
 
+
+def _qwen2_file(tmp_path, extra=()):
+  """A Qwen2-shaped file: q / k / v projections with bias vectors (Linear(bias=qkv_bias), model.py:161-163, 443), Q8_0 matrices, F32 biases."""
+  from tinygrad_amd.gguf import gguf_write
+  rng = np.random.default_rng(33)
+  dim, hidden, H, KV, hd, L, vocab = 256, 512, 4, 2, 64, 2, 512
+  def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
+  q8 = lambda name, rows, cols, amp=1.0: (name, (rows, cols), 8, og.quantize_q8_0(lin(rows, cols) * amp))
+  f32 = lambda name, n, mean=1.0, sd=0.2: (name, (n,), 0, (mean + sd * rng.standard_normal(n)).astype(np.float32))
+  tensors = [q8("token_embd.weight", vocab, dim, 16.0)]
+  for i in range(L):
+    p = f"blk.{i}."
+    tensors += [f32(p + "attn_norm.weight", dim), q8(p + "attn_q.weight", H * hd, dim), f32(p + "attn_q.bias", H * hd, 0.0, 0.5),
+                q8(p + "attn_k.weight", KV * hd, dim), f32(p + "attn_k.bias", KV * hd, 0.0, 0.5), q8(p + "attn_v.weight", KV * hd, dim), f32(p + "attn_v.bias", KV * hd, 0.0, 0.5),
+                q8(p + "attn_output.weight", dim, H * hd), f32(p + "ffn_norm.weight", dim), q8(p + "ffn_gate.weight", hidden, dim), q8(p + "ffn_up.weight", hidden, dim),
+                q8(p + "ffn_down.weight", dim, hidden)]
+  tensors += [f32("output_norm.weight", dim), q8("output.weight", vocab, dim)]
+  tensors += list(extra)
+  kvs = [("general.architecture", "qwen2"), ("qwen2.context_length", 96), ("qwen2.attention.head_count", H), ("qwen2.attention.head_count_kv", KV),
+         ("qwen2.block_count", L), ("qwen2.embedding_length", dim), ("qwen2.feed_forward_length", hidden),
+         ("qwen2.attention.layer_norm_rms_epsilon", 1e-6), ("qwen2.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(vocab)])]
+  path = tmp_path / "qwen2.gguf"
+  return path, gguf_write(path, kvs, tensors)
+
+def test_from_gguf_qwen2_shape_qkv_bias(gpu, tmp_path):
+  from tinygrad_amd.llm import Transformer
+  path, raw = _qwen2_file(tmp_path)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  assert model.blk[0].qkv_bias is not None
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  prompt = [9, 100, 321, 5]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3
+  # the biases matter: without them the oracle's logits for the same token stream are far away
+  o3 = ollm.Model(cfg, {k: v for k, v in weights.items() if not k.endswith(".bias")}, 64, w_round_f16=False, act_round_f16=True)
+  for pos, t in enumerate(prompt + ref[:-1]): lg3 = o3.forward(t, pos)
+  assert ol.rel_err(lg3, lg) > 0.05
+
+def test_from_gguf_rejects_tensors_it_would_drop(gpu, tmp_path):
+  """A tensor the built path has no use for (here a shared expert's gate) is an error, not a silently different model."""
+  from tinygrad_amd.llm import Transformer
+  path, _ = _qwen2_file(tmp_path, extra=[("blk.0.ffn_gate_shexp.weight", (64, 256), 8, og.quantize_q8_0(np.zeros((64, 256), np.float32)))])
+  with pytest.raises(NotImplementedError, match="ffn_gate_shexp"): Transformer.from_gguf(path, max_context=64, max_new=8)

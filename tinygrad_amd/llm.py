@@ -121,6 +121,16 @@ def _to_f32(data: np.ndarray, typ: int) -> np.ndarray:
   if typ == 30: return (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32)      # bfloat16
   raise NotImplementedError(f"ggml type {typ} for a norm / dense tensor")
 
+class _Consumed(dict):
+  """A state dict that remembers which tensors the model took."""
+  def __init__(self, *a):
+    super().__init__(*a); self.used = set()
+  def __getitem__(self, k):
+    self.used.add(k); return super().__getitem__(k)
+  def get(self, k, default=None):
+    if k in self: self.used.add(k)
+    return super().get(k, default)
+
 class TransformerBlock:
   """One decode step of the reference's TransformerBlock/FFNBlock (tinygrad/llm/model.py:144-204) for batch 1."""
   def __init__(self, config: TransformerConfig, sd: dict, i: int, shared):
@@ -135,6 +145,8 @@ class TransformerBlock:
       self.ffn_gate_exps, self.ffn_up_exps, self.ffn_down_exps = ex("ffn_gate_exps.weight"), ex("ffn_up_exps.weight"), ex("ffn_down_exps.weight")
     else:
       self.ffn_gate, self.ffn_up, self.ffn_down = lin("ffn_gate.weight"), lin("ffn_up.weight"), lin("ffn_down.weight")
+    # Linear(bias=config.qkv_bias) of model.py:161-163: the float32 bias rows enter the q / k / v launch as its additive row
+    self.qkv_bias = [sd[p + f"attn_{n}.bias"][0] for n in "qkv"] if p + "attn_q.bias" in sd else None
     self.q_norm = sd[p + "attn_q_norm.weight"][0] if c.qk_norm else None
     self.k_norm = sd[p + "attn_k_norm.weight"][0] if c.qk_norm else None
     # KV cache: fp16 [n_kv_heads][max_context][head_dim] each (reference: one [2,B,KvH,ctx,Hd] tensor, model.py:202)
@@ -155,7 +167,7 @@ class TransformerBlock:
                             and (c.dim // (32 if self.ffn_gate_exps.ggml_type == rt.MXFP4 else 64)) <= 64
     # the previous block's weighted expert sum can be completed inside this block's q/k/v launch (one 8-value piece per thread: dim <= 2048)
     self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
-                            and 0 < c.num_experts_per_tok <= 8
+                            and 0 < c.num_experts_per_tok <= 8 and self.qkv_bias is None
     if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
 
   def __call__(self, x: Buffer, stream, pending: bool = False, defer: bool = False) -> tuple[Buffer, bool]:
@@ -179,8 +191,9 @@ class TransformerBlock:
       while i < 3:
         j = i + 1
         while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
-        if self.fuse_norm: qlinear_multi(qkv[i:j], x, qkv_out[i:j], stream=stream, norm=(self.attn_norm, c.norm_eps))
-        else: qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream)
+        bias = dict(epilogue=1, resid=self.qkv_bias[i:j]) if self.qkv_bias is not None else {}
+        if self.fuse_norm: qlinear_multi(qkv[i:j], x, qkv_out[i:j], stream=stream, norm=(self.attn_norm, c.norm_eps), **bias)
+        else: qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream, **bias)
         i = j
     # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
     rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
@@ -267,6 +280,7 @@ class Transformer:
   def _build_layer_table(self):
     c = self.config
     if c.num_experts or c.qk_norm or c.head_dim not in (64, 128) or c.n_heads * c.head_dim != c.dim: return None
+    if any(b.qkv_bias is not None for b in self.blk): return None
     if c.dim % 64 or c.hidden_dim % 64 or max(c.dim, c.hidden_dim) > 16384: return None
     if c.n_heads // c.n_kv_heads * ((c.max_context + 63) // 64) > 1024: return None
     t0 = self.blk[0].attn_q.ggml_type
@@ -341,9 +355,9 @@ class Transformer:
       if name == "rope_freqs.weight": continue                         # unused by the reference too (model.py:446)
       rows, cols = (int(np.prod(t.shape[:-1])), t.shape[-1]) if len(t.shape) > 1 else (1, t.shape[0])
       typ, buf, data = t.ggml_type, t.buffer, t.data
-      is_norm = name.endswith("_norm.weight")
-      if is_norm:
-        if typ != rt.F32: data = _to_f32(data, typ); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F32
+      is_norm = name.endswith("_norm.weight") or name.endswith(".bias")
+      if is_norm:                                                      # norm weights and biases: float32 rows holding the reference's fp16 values (model.py:376)
+        data = _to_f32(data, typ).astype(np.float16).astype(np.float32); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F32
       elif typ in GGUF_F32_LIKE:                                       # F32 / BF16 matrices -> fp16 (model.py:376)
         data = _to_f32(data, typ).astype(np.float16); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F16
       elif typ in rt.GGML_DEQUANT_ONLY:                                # block types without an in-place linear kernel: the fp16 weight of model.py:376, made once
@@ -367,7 +381,11 @@ class Transformer:
       num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
       norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe",)),
       expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0))
-    return Transformer(config, sd, max_new=max_new), kv
+    sd = _Consumed(sd)
+    model = Transformer(config, sd, max_new=max_new)
+    if (left := sorted(set(sd) - sd.used)):                            # e.g. shared experts, expert selection bias, leading dense blocks: not silently dropped
+      raise NotImplementedError(f"tensors the built path does not consume: {left[:8]}{' ...' if len(left) > 8 else ''}")
+    return model, kv
 
   def reset(self, tokens: list[int]):
     """Start a new sequence: position 0, first prompt token loaded, nothing cached (no KV-prefix reuse)."""
