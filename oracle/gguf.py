@@ -53,5 +53,6 @@ def from_gguf_weights(raw: bytes):
              head_dim=kv.get(f"{arch}.attention.key_length", dim // H), rope_theta=kv[f"{arch}.rope.freq_base"],
              qk_norm=int(sd["blk.0.attn_q_norm.weight"].shape[0]) if "blk.0.attn_q_norm.weight" in sd else 0,
              num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
-             norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", False), expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1))
+             norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe", "qwen35moe", "kimi-linear")),   # model.py:432
+             expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0))
   return cfg, sd, kv

@@ -186,3 +186,45 @@ def test_from_gguf_rejects_tensors_it_would_drop(gpu, tmp_path):
   from tinygrad_amd.llm import Transformer
   path, _ = _qwen2_file(tmp_path, extra=[("blk.0.ffn_gate_shexp.weight", (64, 256), 8, og.quantize_q8_0(np.zeros((64, 256), np.float32)))])
   with pytest.raises(NotImplementedError, match="ffn_gate_shexp"): Transformer.from_gguf(path, max_context=64, max_new=8)
+
+def test_from_gguf_qwen3moe_shape_expert_stacks(gpu, tmp_path):
+  """A Qwen3-MoE-shaped file with the tensor types of a Q4_K_M file: Q4_K expert gate / up stacks and Q6_K down stacks stored as three-dimensional
+  tensors (E, out, in), an F32 router, per-head q/k norms, top-k weights normalised by the architecture's default (model.py:432)."""
+  from tinygrad_amd.llm import Transformer
+  from tinygrad_amd.gguf import gguf_write
+  rng = np.random.default_rng(55)
+  dim, hidden, H, KV, hd, L, vocab, E, k = 256, 256, 4, 2, 64, 2, 512, 8, 2
+  def lin(*shape): return (rng.uniform(-1, 1, shape) * shape[-1] ** -0.5).astype(np.float32)
+  q4 = lambda name, *shape, amp=1.0: (name, shape, 12, og.quantize_q4_k(lin(*shape) * amp))
+  q6 = lambda name, *shape: (name, shape, 14, og.quantize_q6_k(lin(*shape)))
+  f32 = lambda name, n: (name, (n,), 0, (1 + 0.2 * rng.standard_normal(n)).astype(np.float32))
+  tensors = [q4("token_embd.weight", vocab, dim, amp=16.0)]
+  for i in range(L):
+    p = f"blk.{i}."
+    tensors += [f32(p + "attn_norm.weight", dim), q4(p + "attn_q.weight", H * hd, dim), q4(p + "attn_k.weight", KV * hd, dim), q6(p + "attn_v.weight", KV * hd, dim),
+                f32(p + "attn_q_norm.weight", hd), f32(p + "attn_k_norm.weight", hd), q4(p + "attn_output.weight", dim, H * hd), f32(p + "ffn_norm.weight", dim),
+                (p + "ffn_gate_inp.weight", (E, dim), 0, lin(E, dim) * 4), q4(p + "ffn_gate_exps.weight", E, hidden, dim), q4(p + "ffn_up_exps.weight", E, hidden, dim),
+                q6(p + "ffn_down_exps.weight", E, dim, hidden)]
+  tensors += [f32("output_norm.weight", dim), q6("output.weight", vocab, dim)]
+  kvs = [("general.architecture", "qwen3moe"), ("qwen3moe.context_length", 96), ("qwen3moe.attention.head_count", H), ("qwen3moe.attention.head_count_kv", KV),
+         ("qwen3moe.attention.key_length", hd), ("qwen3moe.block_count", L), ("qwen3moe.embedding_length", dim), ("qwen3moe.feed_forward_length", 4 * hidden),
+         ("qwen3moe.expert_feed_forward_length", hidden), ("qwen3moe.expert_count", E), ("qwen3moe.expert_used_count", k),
+         ("qwen3moe.attention.layer_norm_rms_epsilon", 1e-6), ("qwen3moe.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(vocab)])]
+  path = tmp_path / "qwen3moe.gguf"
+  raw = gguf_write(path, kvs, tensors)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  c = model.config
+  assert c.num_experts == E and c.num_experts_per_tok == k and c.hidden_dim == hidden and c.norm_topk_prob and c.qk_norm == hd
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  assert cfg["norm_topk_prob"] and weights["blk.0.ffn_gate_exps.weight"].shape == (E, hidden, dim)
+  prompt = [9, 100, 321, 5, 77]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3
