@@ -51,6 +51,7 @@ def from_gguf_weights(raw: bytes):
   cfg = dict(num_blocks=kv[f"{arch}.block_count"], dim=dim, hidden_dim=kv.get(f"{arch}.expert_feed_forward_length", kv.get(f"{arch}.feed_forward_length", 0)),
              n_heads=H, n_kv_heads=KV, norm_eps=kv[f"{arch}.attention.layer_norm_rms_epsilon"], vocab_size=len(kv["tokenizer.ggml.tokens"]),
              head_dim=kv.get(f"{arch}.attention.key_length", dim // H), rope_theta=kv[f"{arch}.rope.freq_base"],
+             rope_dim=kv.get(f"{arch}.rope.dimension_count", kv.get(f"{arch}.attention.key_length", dim // H)),   # model.py:406
              qk_norm=int(sd["blk.0.attn_q_norm.weight"].shape[0]) if "blk.0.attn_q_norm.weight" in sd else 0,
              num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
              norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe", "qwen35moe", "kimi-linear")),   # model.py:432

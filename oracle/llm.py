@@ -37,7 +37,8 @@ class Model:
       return w.astype(np.float16).astype(np.float32) if (w_round_f16 and t not in (0,)) else w.astype(np.float32)
     self.w = {name: (deq(name) if isinstance(tensors[name], tuple) else np.asarray(tensors[name], dtype=np.float32)) for name in tensors}
     if "output.weight" not in self.w: self.w["output.weight"] = self.w["token_embd.weight"]
-    self.fc = precompute_freqs_cis(cfg["head_dim"], max_context, cfg["rope_theta"])
+    self.rd = cfg.get("rope_dim") or cfg["head_dim"]                        # model.py:63, 204
+    self.fc = precompute_freqs_cis(self.rd, max_context, cfg["rope_theta"])
     L, kv, hd = cfg["num_blocks"], cfg["n_kv_heads"], cfg["head_dim"]
     self.ck = np.zeros((L, kv, max_context, hd), dtype=kv_dtype)
     self.cv = np.zeros((L, kv, max_context, hd), dtype=kv_dtype)
@@ -61,7 +62,9 @@ class Model:
       q, k = q.reshape(H, hd), k.reshape(KV, hd)
       if c.get("qk_norm", 0) == hd:                                         # model.py:180: per-head q/k norm after the head split
         q, k = rmsnorm(q, self.w[p + "attn_q_norm.weight"].reshape(-1), eps), rmsnorm(k, self.w[p + "attn_k_norm.weight"].reshape(-1), eps)
-      q, k = apply_rope(q, self.fc[pos]), apply_rope(k, self.fc[pos])
+      rd = self.rd                                                          # model.py:180-181: only the first rope_dim values of a head rotate
+      q = np.concatenate([apply_rope(q[:, :rd], self.fc[pos]), q[:, rd:]], axis=-1)
+      k = np.concatenate([apply_rope(k[:, :rd], self.fc[pos]), k[:, rd:]], axis=-1)
       v = self._lin(p + "attn_v.weight", n)
       if p + "attn_v.bias" in self.w: v = v + self.w[p + "attn_v.bias"].reshape(-1)
       v = v.reshape(KV, hd)

@@ -228,3 +228,47 @@ def test_from_gguf_qwen3moe_shape_expert_stacks(gpu, tmp_path):
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
+
+def test_from_gguf_partial_rotary(gpu, tmp_path):
+  """rope.dimension_count < head_dim (model.py:180-181, 406): only the first 24 of a head's 64 values rotate.  The file also carries q / k biases and
+  per-head q / k norm weights, which follow the same per-head reordering as the q / k rows at load."""
+  from tinygrad_amd.llm import Transformer
+  from tinygrad_amd.gguf import gguf_write
+  rng = np.random.default_rng(77)
+  dim, hidden, H, KV, hd, rd, L, vocab = 256, 512, 4, 2, 64, 24, 2, 512
+  def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
+  q8 = lambda name, rows, cols, amp=1.0: (name, (rows, cols), 8, og.quantize_q8_0(lin(rows, cols) * amp))
+  f32 = lambda name, n, mean=1.0, sd=0.2: (name, (n,), 0, (mean + sd * rng.standard_normal(n)).astype(np.float32))
+  tensors = [q8("token_embd.weight", vocab, dim, 16.0)]
+  for i in range(L):
+    p = f"blk.{i}."
+    tensors += [f32(p + "attn_norm.weight", dim), q8(p + "attn_q.weight", H * hd, dim, 3.0), f32(p + "attn_q.bias", H * hd, 0.0, 0.5),
+                q8(p + "attn_k.weight", KV * hd, dim, 3.0), f32(p + "attn_k.bias", KV * hd, 0.0, 0.5), q8(p + "attn_v.weight", KV * hd, dim), f32(p + "attn_v.bias", KV * hd, 0.0, 0.5),
+                f32(p + "attn_q_norm.weight", hd, 1.0, 0.5), f32(p + "attn_k_norm.weight", hd, 1.0, 0.5),
+                q8(p + "attn_output.weight", dim, H * hd), f32(p + "ffn_norm.weight", dim), q8(p + "ffn_gate.weight", hidden, dim), q8(p + "ffn_up.weight", hidden, dim),
+                q8(p + "ffn_down.weight", dim, hidden)]
+  tensors += [f32("output_norm.weight", dim), q8("output.weight", vocab, dim)]
+  kvs = [("general.architecture", "qwen3"), ("qwen3.context_length", 96), ("qwen3.attention.head_count", H), ("qwen3.attention.head_count_kv", KV),
+         ("qwen3.attention.key_length", hd), ("qwen3.rope.dimension_count", rd), ("qwen3.block_count", L), ("qwen3.embedding_length", dim), ("qwen3.feed_forward_length", hidden),
+         ("qwen3.attention.layer_norm_rms_epsilon", 1e-6), ("qwen3.rope.freq_base", 10000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(vocab)])]
+  path = tmp_path / "partial_rope.gguf"
+  raw = gguf_write(path, kvs, tensors)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  assert model.config.rope_dim == rd and model.config.qk_norm == hd
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  assert cfg["rope_dim"] == rd
+  prompt = [9, 100, 321, 5, 44, 12, 400]
+  got = list(model.generate(prompt, 12))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  ref, margins = o.generate(prompt, 12)
+  print(f"min top-2 margin {min(margins):.4f}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3
+  # the rotation width matters: the oracle with full-width rotation gives other logits for the same token stream
+  o3 = ollm.Model(dict(cfg, rope_dim=hd), weights, 64, w_round_f16=False, act_round_f16=True)
+  for pos, t in enumerate(prompt + ref[:-1]): lg3 = o3.forward(t, pos)
+  assert ol.rel_err(lg3, lg) > 0.01

@@ -34,6 +34,7 @@ class TransformerConfig:
   norm_topk_prob: bool = False
   expert_gating_func: int = 1      # ExpertGating.SOFTMAX (model.py:9-13)
   routed_scaling_factor: float = 1.0
+  rope_dim: int = 0                # rotated leading values of a head (model.py:63, 180-181); 0 = head_dim
 
 LLAMA3_8B = dict(num_blocks=32, dim=4096, hidden_dim=14336, n_heads=32, n_kv_heads=8, norm_eps=1e-5, vocab_size=128256,
                  head_dim=128, rope_theta=500000.0)
@@ -47,6 +48,22 @@ def precompute_freqs_cis(dim: int, end: int, theta: float) -> np.ndarray:
   freqs = (np.float32(1.0) / (np.float32(theta) ** (np.arange(0, dim, 2, dtype=np.float32)[:dim // 2] / np.float32(dim)))).astype(np.float32)
   ang = (np.arange(end, dtype=np.float32)[:, None] * freqs[None, :]).astype(np.float32)
   return np.concatenate([np.cos(ang), np.sin(ang)], axis=-1).astype(np.float32)
+
+def partial_rope_order(head_dim: int, rope_dim: int) -> np.ndarray:
+  """Order of a head's values that turns the reference's partial rotation (pairs (i, i + rope_dim/2) of the first rope_dim values, the rest untouched,
+  model.py:180-181) into a rotation over pairs (i, i + head_dim/2) whose trailing pairs are identities: rotated first halves, first half of the
+  untouched values, rotated second halves, second half of the untouched values.  q and k (rows, biases, norm weights) take the same order, so
+  every q . k is unchanged."""
+  rh, rest = rope_dim // 2, (head_dim - rope_dim) // 2
+  return np.concatenate([np.arange(rh), rope_dim + np.arange(rest), rh + np.arange(rh), rope_dim + rest + np.arange(rest)])
+
+def rope_table(head_dim: int, rope_dim: int, end: int, theta: float) -> np.ndarray:
+  """[end][head_dim] rotation rows (cos half | sin half); with rope_dim < head_dim the frequencies are those of rope_dim (model.py:204) and the
+  trailing pairs of partial_rope_order get cos 1, sin 0."""
+  fc = precompute_freqs_cis(rope_dim, end, theta)
+  if rope_dim == head_dim: return fc
+  rh, rest = rope_dim // 2, (head_dim - rope_dim) // 2
+  return np.concatenate([fc[:, :rh], np.ones((end, rest), np.float32), fc[:, rh:], np.zeros((end, rest), np.float32)], axis=-1)
 
 def quant_nbytes(ggml_type: int, n: int) -> int:
   if ggml_type == rt.F32: return 4 * n
@@ -253,7 +270,7 @@ class _Shared:
       self.act_e, self.y_e = Buffer((k, c.hidden_dim), f16), Buffer((k, c.dim), f32)
     self.logits = Buffer((1, c.vocab_size), f32)
     self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)
-    self.rope = Buffer.from_numpy(precompute_freqs_cis(c.head_dim, c.max_context, c.rope_theta))
+    self.rope = Buffer.from_numpy(rope_table(c.head_dim, c.rope_dim or c.head_dim, c.max_context, c.rope_theta))
     self.prompt = Buffer((c.max_context,), np.int32).zero_()
     self.out_tokens = Buffer((max(1, max_new),), np.int32).zero_()
 
@@ -348,7 +365,8 @@ class Transformer:
     dim = kv[f"{arch}.embedding_length"]
     head_dim = kv.get(f"{arch}.attention.key_length", dim // n_heads)
     rope_dim = kv.get(f"{arch}.rope.dimension_count", head_dim)
-    if rope_dim != head_dim: raise NotImplementedError("partial rotary embeddings are not built")
+    if rope_dim != head_dim and (arch == "llama" or rope_dim % 2 or (head_dim - rope_dim) % 2 or not 0 < rope_dim < head_dim):
+      raise NotImplementedError(f"rope dimension {rope_dim} of head_dim {head_dim} for architecture {arch} is not built")
     if kv.get(f"{arch}.attention.kv_lora_rank", 0) or arch in ("qwen35", "qwen35moe", "kimi-linear"): raise NotImplementedError(f"architecture {arch} is outside the built path")
     sd = {}
     for name, t in ts.items():
@@ -370,6 +388,11 @@ class Transformer:
         idx = np.arange(rows).reshape(h, per // 2, 2).transpose(0, 2, 1).reshape(-1)   # "n (h two) d -> n (two h) d"
         buf = Buffer.from_numpy(np.ascontiguousarray(raw[idx]).reshape(-1))
       shape = (rows, cols) if len(t.shape) <= 2 else tuple(t.shape)
+      if rope_dim != head_dim and name.split(".")[-2] in ("attn_q", "attn_k", "attn_q_norm", "attn_k_norm"):
+        # partial rotary: reorder every head's rows (or per-value weights) so that the kernel's pairs (i, i + head_dim/2) are the reference's
+        raw = np.ascontiguousarray(buf.numpy() if data is None else data).view(np.uint8).reshape(rows if len(t.shape) > 1 else cols, -1)
+        idx = (np.arange(raw.shape[0]).reshape(-1, head_dim)[:, partial_rope_order(head_dim, rope_dim)]).reshape(-1)
+        buf = Buffer.from_numpy(np.ascontiguousarray(raw[idx]).reshape(-1))
       sd[name] = (buf, typ, shape)
     if "output.weight" not in sd: sd["output.weight"] = sd["token_embd.weight"]        # tied embeddings, model.py:379
     config = TransformerConfig(
@@ -380,7 +403,8 @@ class Transformer:
       qk_norm=int(sd["blk.0.attn_q_norm.weight"][2][-1]) if "blk.0.attn_q_norm.weight" in sd else 0,
       num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
       norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe",)),
-      expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0))
+      expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0),
+      rope_dim=rope_dim if rope_dim != head_dim else 0)
     sd = _Consumed(sd)
     model = Transformer(config, sd, max_new=max_new)
     if (left := sorted(set(sd) - sd.used)):                            # e.g. shared experts, expert selection bias, leading dense blocks: not silently dropped
