@@ -4,6 +4,13 @@ import pytest
 ROOT = pathlib.Path(__file__).resolve().parent.parent
 if str(ROOT) not in sys.path: sys.path.insert(0, str(ROOT))
 
+def golden_kats():
+  """The reference tests' known-answer vectors for block dequant (tests/golden/ggml_dequant_kat.json): (name, type, n, block bytes, expected float32)."""
+  import json, numpy as np
+  g = json.loads((ROOT / "tests" / "golden" / "ggml_dequant_kat.json").read_text())
+  return [(k, v["ggml_type"], v["n"], np.array(v["block"], dtype=np.uint8), np.frombuffer(bytes.fromhex(v["expected_f32_hex"]), dtype=np.float32))
+          for k, v in g.items() if isinstance(v, dict)]
+
 def pytest_configure(config):
   config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 

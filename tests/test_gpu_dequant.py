@@ -12,6 +12,13 @@ def _gpu_dequant(gpu, data, n, t, dtype=np.float32):
   from tinygrad_amd.gguf import ggml_data_to_tensor
   return ggml_data_to_tensor(data, n, t, out_dtype=dtype).numpy()
 
+from conftest import golden_kats
+
+@pytest.mark.parametrize("name,t,n,block,exp", golden_kats(), ids=[k[0] for k in golden_kats()])
+def test_golden_fixture_vectors(gpu, name, t, n, block, exp):
+  """The committed fixture of the reference tests' vectors through the device kernel, bit for bit."""
+  assert _gpu_dequant(gpu, block, n, t).tobytes() == exp.tobytes()
+
 def test_q8_0_reference_kat(gpu):
   # test/unit/test_gguf.py:36-40
   block = np.frombuffer(np.float16(2.0).tobytes() + np.arange(1, 33, dtype=np.int8).tobytes(), dtype=np.uint8).copy()

@@ -3,6 +3,13 @@ the published ggml loops, brute force on the bit layout, and closed forms."""
 import numpy as np, pytest
 from oracle import ggml as og, cref
 
+from conftest import golden_kats
+
+@pytest.mark.parametrize("name,t,n,block,exp", golden_kats(), ids=[k[0] for k in golden_kats()])
+def test_golden_fixture_vectors(name, t, n, block, exp):
+  """The committed fixture of the reference tests' vectors, bit for bit (incl. the sign of -0.0)."""
+  assert og.ggml_data_to_tensor(block, n, t).tobytes() == exp.tobytes()
+
 def test_q8_0_reference_kat():
   # test/unit/test_gguf.py:36-40
   block = np.frombuffer(np.float16(2.0).tobytes() + np.arange(1, 33, dtype=np.int8).tobytes(), dtype=np.uint8).copy()
