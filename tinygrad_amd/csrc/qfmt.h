@@ -37,6 +37,8 @@ struct QArgs {
   const float* route_logits; int route_E, route_k, route_gating, route_norm_topk; float route_scale; float* route_probs_out;
   // M = 1 fast path: row groups per team and the remainder (the first team_rem teams take one more), so that the kernel divides nothing
   int team_base, team_rem;
+  int team_skew, team_first;   // the first team_first teams own team_skew row groups more than that, the others as many fewer (0: no skew)
+  int team_stride;             // > 0: team t owns row groups t, t + team_stride, ... of the one matrix instead of a contiguous range
 };
 
 // staged position of element e for a consumer of format `fmt` (row length K = UW * nu)

@@ -5,6 +5,9 @@
 #include "host.h"
 #include "moe_gate.h"
 
+#ifndef QG1_WR
+#define QG1_WR 8           // row teams (waves) per workgroup when one wave covers a row: one workgroup per CU
+#endif
 #ifndef QG1_DEPTH
 #define QG1_DEPTH 3        // row groups in flight per lane: the loads of the next DEPTH - 1 groups are outstanding while one is multiplied
 #endif
@@ -13,7 +16,14 @@
 // One activation row: each lane keeps the activations of ITS unit in registers for the whole kernel (no LDS traffic in the
 // loop).  A workgroup is WR x WK waves: the WK waves of a row team split K (wave wk owns units 64wk .. 64wk+63) and their
 // partial sums meet in LDS once per row group (the only LDS use in the loop: split-K partials); the WR teams own disjoint
-// row ranges.  Each team walks a contiguous range of row groups with a register ring of QG1_DEPTH groups.
+// row ranges.  Each team walks its row groups with a register ring of QG1_DEPTH groups.
+// Which row groups a team owns.  A CU's vector memory pipeline returns data in request order, so everything a wave asks for waits behind what
+// the waves that reached the CU before it have asked for.  Measured with per-wave clock stamps on the 2 x 14336 x 4096 gate/up launch with two
+// 4-wave workgroups per CU: the workgroup that arrives second starts 0.2 us later, but holds its activations 1.4 us later, its first weights 2.9 us
+// later and ends 2.4 us later than the first (1.3 us on the 4096 x 14336 down projection).  Hence: (a) rows that one wave covers run as ONE 8-wave
+// workgroup per CU (QG1_WR), whose waves all request their activations before any weight; (b) where two workgroups per CU remain (K split over
+// the waves), the first pass of workgroups owns team_skew row groups more and the second pass as many fewer; (c) a launch over one matrix
+// interleaves its teams (team t owns groups t, t + teams, ...), so that the whole chip walks one contiguous window of the matrix.
 // Activations reach the registers through one LDS transpose per workgroup: coalesced 16-byte global loads of the plain row,
 // then each lane reads back the 64 (or 32) values of its unit (unit stride padded to spread LDS banks).
 // H (rows of at most 32 units, WK = 1): a row occupies half a wave, so each half-wave is a row team of its own (lanes 0-31 and
@@ -66,8 +76,11 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
   const long long team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
   const long long gbase = a.team_base, grem = a.team_rem;       // ngroups / teams and ngroups % teams, from the host
-  const long long g0 = team * gbase + (team < grem ? team : grem), g1 = g0 + gbase + (team < grem ? 1 : 0);
+  const long long nfirst = a.team_first, sk = a.team_skew;
+  const long long g0 = team * gbase + (team < grem ? team : grem) + sk * (team < nfirst ? team : 2 * nfirst - team);
+  const long long g1 = g0 + gbase + (team < grem ? 1 : 0) + (team < nfirst ? sk : -sk);
   const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
+  const long long rstep = a.team_stride ? (long long)a.team_stride * RS : RS;     // rows from one row group of the team to its next
   uint32_t kc[F::NKC];
   F::consts(kc);
   u32x4 xv[F::XV]; float cv[F::NG];
@@ -88,6 +101,10 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     if (hi > seg_rows) hi = seg_rows;
     seg_start += seg_rows;
     cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;                 // row groups of this team inside the segment
+    if (a.team_stride) {                                         // interleaved teams (one matrix): groups team, team + stride, ...
+      lo = team * RS; hi = seg_rows;
+      cnt = lo < hi ? ((hi - lo + RS - 1) / RS + a.team_stride - 1) / a.team_stride : 0;
+    }
     last = hi > 0 ? hi - 1 : 0;                                  // rows beyond the range reload this one (always a valid row)
     base0 = a.w[sg] + eoff;
     base1 = ((EPI == 2) ? a.w[1] : a.w[sg]) + eoff;
@@ -154,21 +171,21 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   // walks the team's row groups of the current segment; group lo is already in flight in b[0]
   auto run_segment = [&]() {
 #pragma unroll
-    for (int d = 1; d < D - 1; d++) issue(b[d], lo + (long long)d * RS);
+    for (int d = 1; d < D - 1; d++) issue(b[d], lo + (long long)d * rstep);
     long long row = lo, g = 0;
     for (; g + D <= cnt; g += D) {
 #pragma unroll
       for (int d = 0; d < D; d++) {
-        issue(b[(d + D - 1) % D], row + (long long)(D - 1) * RS);        // the slot freed by the previous group
+        issue(b[(d + D - 1) % D], row + (long long)(D - 1) * rstep);        // the slot freed by the previous group
         finish_group(b[d], row);
-        row += RS;
+        row += rstep;
       }
     }
     // fewer than D groups left: their loads are already in flight (slots 0 .. D - 2), nothing more to issue
 #pragma unroll
     for (int d = 0; d < D - 1; d++) {
       if (g + d < cnt) finish_group(b[d], row);                  // (split K: the waves of a workgroup share cnt, so the barrier inside is uniform)
-      row += RS;
+      row += rstep;
     }
   };
 
@@ -377,8 +394,8 @@ static int launch_fast(QArgs a, hipStream_t s) {
   constexpr int NT = WK * WR * 64;
   const long long ngroups = (a.ntot + RS - 1) / RS;
   const size_t lds = (size_t)a.nu * (F::UW / 2 + 4) * 4;
-  // row teams per CU: 8 waves (two 4-wave workgroups), fewer when the staged activations in LDS (160 KB per CU) say so.  Measured on
-  // the 8B decode step: 8 or 12 waves per CU 570 tok/s, 16 (all wave slots) 564, 4 553.
+  // row teams per CU: 8 waves (one 8-wave workgroup or two 4-wave ones), fewer when the staged activations in LDS (160 KB per CU) say so.
+  // Measured on the 8B decode step: 8 or 12 waves per CU 570 tok/s, 16 (all wave slots) 564, 4 553.
   int wg_per_cu = (a.sel ? 16 : 8) / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;   // (expert jobs share the grid: all 16 wave slots there)
   const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
   constexpr int TPW = WR * (H ? 2 : 1);                           // row teams per workgroup
@@ -389,10 +406,15 @@ static int launch_fast(QArgs a, hipStream_t s) {
   // rows, as long as every CU still gets a workgroup
   long long per_min = ngroups / ((long long)fast_cu_count() * TPW); per_min = per_min < 1 ? 1 : per_min > 4 ? 4 : per_min;
   if (!a.sel && per < per_min) per = per_min;
-  const long long teams = (ngroups + per - 1) / per;               // every team gets `per` groups (the last maybe fewer)
+  long long teams = (ngroups + per - 1) / per;                     // every team gets `per` groups (the last maybe fewer)
+  if (!H && WR == 8 && !a.sel) teams = ngroups < max_teams ? ngroups : max_teams;   // one workgroup per CU: the row groups are spread over all CUs
   long long grid = (teams + TPW - 1) / TPW;
   if (grid < 1) grid = 1;
-  { const long long nteams = grid * TPW; a.team_base = (int)(ngroups / nteams); a.team_rem = (int)(ngroups % nteams); }
+  { const long long nteams = grid * TPW; a.team_base = (int)(ngroups / nteams); a.team_rem = (int)(ngroups % nteams);
+    // exactly two workgroups per CU: the pass that reaches the CUs first takes one row group more per team, the second pass one fewer
+    const bool two_per_cu = grid == 2LL * fast_cu_count() && !a.sel && a.team_base > 2;
+    a.team_skew = two_per_cu ? 1 : 0; a.team_first = two_per_cu ? (int)(nteams / 2) : 0;
+    a.team_stride = (!a.team_skew && !a.sel && (EPI == 2 || a.nseg == 1)) ? (int)nteams : 0; }
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
   const bool one_batch = a.K / 8 <= NT * 2;
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
@@ -420,7 +442,9 @@ static int launch_fast(QArgs a, hipStream_t s) {
 static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
 template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
-  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
+  // the SwiGLU pair (seven row groups per team on the 8B shapes) is the one case that measures faster as two 4-wave workgroups per CU with the
+  // skewed split (16.2 us against 16.8 us as one 8-wave workgroup); every other launch is faster as one 8-wave workgroup (q/k/v 9.4 -> 8.2 us)
+  if (a.epilogue == 2) return launch_fast<T, 2, WK, (WR == 8 ? 4 : WR), 2, H>(a, s);
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice, for Q8_0 pairs
   // (68-byte units: no faster with two) and when the waves of a workgroup split K - with the three-deep ring a single row per step is
   // faster there (4096 x 14336: Q4_0 in the 8B decode step 12.5 -> 11.7 us, Q4_K 13.2 -> 12.2, Q6_K 19.3 -> 17.4, Q5_0 16.2 -> 15.2).
@@ -438,7 +462,7 @@ int qgemv1_launch_format(QArgs a, hipStream_t s) {
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const int waves = (a.nu + 63) / 64;
   if (a.nu <= 32) return launch_fast_e<T, 1, 4, true>(a, s);
-  if (waves <= 1) return launch_fast_e<T, 1, 4>(a, s);
+  if (waves <= 1) return launch_fast_e<T, 1, QG1_WR>(a, s);
   if (waves <= 2) return launch_fast_e<T, 2, 1>(a, s);
   if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);
   if (waves <= 8) return launch_fast_e<T, 8, 1>(a, s);
