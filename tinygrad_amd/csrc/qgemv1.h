@@ -76,11 +76,13 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
   const long long team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
   const long long gbase = a.team_base, grem = a.team_rem;       // ngroups / teams and ngroups % teams, from the host
-  const long long nfirst = a.team_first, sk = a.team_skew;
+  // (half-wave teams keep equal contiguous ranges and a compile-time row step: their row numbers live in vector registers, where a run-time
+  // step turns every load address into 64-bit vector arithmetic - 0.6 us on the 2048-wide fp16 launches of the MoE decode step)
+  const long long nfirst = H ? 0 : a.team_first, sk = H ? 0 : a.team_skew;
   const long long g0 = team * gbase + (team < grem ? team : grem) + sk * (team < nfirst ? team : 2 * nfirst - team);
   const long long g1 = g0 + gbase + (team < grem ? 1 : 0) + (team < nfirst ? sk : -sk);
   const long long row_lo = g0 * RS, row_hi = g1 * RS < a.ntot ? g1 * RS : a.ntot;
-  const long long rstep = a.team_stride ? (long long)a.team_stride * RS : RS;     // rows from one row group of the team to its next
+  const long long rstep = (!H && a.team_stride) ? (long long)a.team_stride * RS : RS;     // rows from one row group of the team to its next
   uint32_t kc[F::NKC];
   F::consts(kc);
   u32x4 xv[F::XV]; float cv[F::NG];
@@ -101,7 +103,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     if (hi > seg_rows) hi = seg_rows;
     seg_start += seg_rows;
     cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;                 // row groups of this team inside the segment
-    if (a.team_stride) {                                         // interleaved teams (one matrix): groups team, team + stride, ...
+    if (!H && a.team_stride) {                                   // interleaved teams (one matrix): groups team, team + stride, ...
       lo = team * RS; hi = seg_rows;
       cnt = lo < hi ? ((hi - lo + RS - 1) / RS + a.team_stride - 1) / a.team_stride : 0;
     }
@@ -412,9 +414,9 @@ static int launch_fast(QArgs a, hipStream_t s) {
   if (grid < 1) grid = 1;
   { const long long nteams = grid * TPW; a.team_base = (int)(ngroups / nteams); a.team_rem = (int)(ngroups % nteams);
     // exactly two workgroups per CU: the pass that reaches the CUs first takes one row group more per team, the second pass one fewer
-    const bool two_per_cu = grid == 2LL * fast_cu_count() && !a.sel && a.team_base > 2;
+    const bool two_per_cu = !H && grid == 2LL * fast_cu_count() && !a.sel && a.team_base > 2;
     a.team_skew = two_per_cu ? 1 : 0; a.team_first = two_per_cu ? (int)(nteams / 2) : 0;
-    a.team_stride = (!a.team_skew && !a.sel && (EPI == 2 || a.nseg == 1)) ? (int)nteams : 0; }
+    a.team_stride = (!H && !a.team_skew && !a.sel && (EPI == 2 || a.nseg == 1)) ? (int)nteams : 0; }
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
   const bool one_batch = a.K / 8 <= NT * 2;
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
