@@ -12,7 +12,7 @@ import argparse, json, os, sys, time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
-GATE_UP_TRAFFIC_BYTES = 66694000   # 66 572 288 B fetched + 121 958 B written per launch (counter runs summarised in profiles/qgemv1_gate_up_hbm_traffic.md)
+GATE_UP_TRAFFIC_BYTES = 66702500   # 66 609 152 B fetched + 93 389 B written per launch (counter runs summarised in profiles/qgemv1_gate_up_hbm_traffic.md)
 
 def cpu_baseline(model, cfg, seconds_budget=20.0):
   """Times oracle/c (scalar C restatement of dequant + fp32-accumulate matmul, model-path numerics) on the GPU box's host
