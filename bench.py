@@ -190,7 +190,7 @@ def main():
   else:
     dom = kern["gate_up"]
     per_block = sum(v["avg_us"] for v in kern.values())
-    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=4, SwiGLU, norm prologue> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
+    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=8, SwiGLU, norm prologue> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
                                                  "one of six launches per block)",
                        "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
                        # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py (counters scaled by a

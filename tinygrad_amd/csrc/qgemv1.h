@@ -21,9 +21,9 @@
 // the waves that reached the CU before it have asked for.  Measured with per-wave clock stamps on the 2 x 14336 x 4096 gate/up launch with two
 // 4-wave workgroups per CU: the workgroup that arrives second starts 0.2 us later, but holds its activations 1.4 us later, its first weights 2.9 us
 // later and ends 2.4 us later than the first (1.3 us on the 4096 x 14336 down projection).  Hence: (a) rows that one wave covers run as ONE 8-wave
-// workgroup per CU (QG1_WR), whose waves all request their activations before any weight; (b) where two workgroups per CU remain (K split over
-// the waves), the first pass of workgroups owns team_skew row groups more and the second pass as many fewer; (c) a launch over one matrix
-// interleaves its teams (team t owns groups t, t + teams, ...), so that the whole chip walks one contiguous window of the matrix.
+// workgroup per CU (QG1_WR) whose waves all hold their activations before any of them asks for weights (prologue 1); (b) where two workgroups per
+// CU remain (K split over the waves), the first pass of workgroups owns team_skew row groups more and the second pass as many fewer; (c) a
+// launch over one matrix interleaves its teams (team t owns groups t, t + teams, ...), so that the whole chip walks one contiguous window.
 // Activations reach the registers through one LDS transpose per workgroup: coalesced 16-byte global loads of the plain row,
 // then each lane reads back the 64 (or 32) values of its unit (unit stride padded to spread LDS banks).
 // H (rows of at most 32 units, WK = 1): a row occupies half a wave, so each half-wave is a row team of its own (lanes 0-31 and
@@ -34,8 +34,9 @@
 // takes the most conservative count where paths join, so a load (or a store: they share the counter) inside a branch turns the
 // waits behind the join into "wait for everything" and the ring into a one-deep pipeline.  For the same reason the prologue kind
 // is a template parameter: with the activation format known at compile time the prologue is one basic block in which the small
-// activation reads go out first, the first weight loads second (loads return in issue order), and the staging arithmetic runs
-// while the weights are in flight.
+// activation reads go out first, the first weight loads second (loads return in issue order; prologue 1 holds them back until the
+// workgroup's sum of squares is complete, i.e. until every wave has its activations), and the staging arithmetic runs while the weights
+// are in flight.
 //   PRO 0  generic: flags read at run time (any activation type, any K); weights first, then the staging loops
 //   PRO 1  one float32 row of at most two 8-element pieces per thread with the RMSNorm folded in (kept in registers between the sum of
 //          squares and the scaling)
@@ -232,7 +233,6 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
       yl[j] = yr[2 * i]; yh[j] = yr[2 * i + 1];
       pj[j] = a.comb_p[jc];
     }
-    issue(b[0], lo);
 #pragma unroll
     for (int j = 0; j < CK; j++) {
       const float p = j < a.comb_k ? pj[j] : 0.f;
@@ -244,6 +244,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     ss = wave_sum(ss);
     if (lane == 0) nred[wave] = ss;
     __syncthreads();
+    issue(b[0], lo);                                             // (as in prologue 1: weights once every wave holds its row)
     float tot = 0.f;
 #pragma unroll
     for (int j = 0; j < NT / 64; j++) tot += nred[j];
@@ -260,7 +261,6 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
       l4[t] = xr[2 * i]; h4[t] = xr[2 * i + 1];
       w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1];
     }
-    issue(b[0], lo);
     float ss = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; t++) {
@@ -271,6 +271,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     ss = wave_sum(ss);
     if (lane == 0) nred[wave] = ss;
     __syncthreads();
+    // the first weights go out only now, when every wave of the workgroup holds its activations: requested together with them, the weight
+    // misses of the waves that started first sit in front of the activation reads of the waves that started last (8B decode 602 -> 609 tok/s)
+    issue(b[0], lo);
     float tot = 0.f;
 #pragma unroll
     for (int j = 0; j < NT / 64; j++) tot += nred[j];
@@ -288,9 +291,10 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     u32x4 v[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
-    issue(b[0], lo);
 #pragma unroll
     for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
+    __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 1)
+    issue(b[0], lo);
     lds_to_regs();
   } else if constexpr (PRO == 6) {
     __shared__ float tk_lg[1024], tk_sc[1024], tk_tmp[192], tk_p[64];
@@ -444,9 +448,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
 static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
 template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
-  // the SwiGLU pair (seven row groups per team on the 8B shapes) is the one case that measures faster as two 4-wave workgroups per CU with the
-  // skewed split (16.2 us against 16.8 us as one 8-wave workgroup); every other launch is faster as one 8-wave workgroup (q/k/v 9.4 -> 8.2 us)
-  if (a.epilogue == 2) return launch_fast<T, 2, WK, (WR == 8 ? 4 : WR), 2, H>(a, s);
+  if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice, for Q8_0 pairs
   // (68-byte units: no faster with two) and when the waves of a workgroup split K - with the three-deep ring a single row per step is
   // faster there (4096 x 14336: Q4_0 in the 8B decode step 12.5 -> 11.7 us, Q4_K 13.2 -> 12.2, Q6_K 19.3 -> 17.4, Q5_0 16.2 -> 15.2).
