@@ -59,7 +59,10 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   constexpr int NT = WK * WR * 64;
   constexpr int NP = F::UW / 2;                                  // dwords (fp16 pairs) per unit
   constexpr int USTRIDE = NP + 4;                                // padded unit stride in dwords
-  constexpr int D = QG1_DEPTH;
+  // Ring depth per launch kind, each measured in the 8B decode step: the SwiGLU pair and the residual epilogue over rows that one wave covers
+  // are faster with two row groups per lane (gate/up 15.8 -> 15.0 us, attn_output 5.45 -> 5.26 us), the plain epilogue and the split-K launches
+  // with three (q/k/v 8.2 against 8.6 us, down 9.6 against 10.5 us); four is slower everywhere (578 against 607 tok/s).
+  constexpr int D = (WK == 1 && !H && EPI != 0) ? 2 : QG1_DEPTH;
   extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
   __shared__ float part[2][WK][R];
   __shared__ float nred[NT / 64];
@@ -445,7 +448,10 @@ static int launch_fast(QArgs a, hipStream_t s) {
   return launch_fast_p<T, R, WK, WR, EPI, H, 0>(a, grid, lds, s);
 }
 
-static constexpr int r2_rows_per_cu() { return 16; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
+#ifndef QG1_R2_ROWS
+#define QG1_R2_ROWS 16
+#endif
+static constexpr int r2_rows_per_cu() { return QG1_R2_ROWS; }   // two rows per step from 16 rows per CU on (8B decode: q/k/v and attn_output with two rows 508 -> 519 tok/s)
 template <int T, int WK, int WR, bool H = false>
 static int launch_fast_e(const QArgs& a, hipStream_t s) {
   if (a.epilogue == 2) return launch_fast<T, 2, WK, WR, 2, H>(a, s);
