@@ -200,3 +200,42 @@ def test_rmsnorm_folded_into_the_linear(gpu, t, k):
   with pytest.raises(RuntimeError, match="fast path"):
     qlinear_multi([bad], gpu.Buffer.from_numpy(x[:, :96].copy()), [gpu.Buffer((1, 8), np.float32)], norm=(nwb, 1e-5))
 
+
+@pytest.mark.parametrize("case", ["interleaved_ragged", "interleaved_residual", "swiglu_pair", "split_k_skewed", "fewer_groups_than_teams"])
+def test_row_team_schedules_write_every_row(gpu, case):
+  """The M = 1 launches hand row groups to their wave teams in three ways on a 256-CU part: interleaved (team t owns groups t, t + teams, ...),
+  contiguous with the first pass of workgroups owning one group more than the second (two workgroups per CU), and contiguous and equal.
+  Row counts here leave remainders everywhere (teams with unequal counts, a last group of one row); outputs start as NaN so that a row
+  nobody wrote, or wrote twice with different values, shows."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(4242)
+  t = 2
+  n, k = {"interleaved_ragged": (13843, 4096), "interleaved_residual": (13843, 4096), "swiglu_pair": (7001, 4096),
+          "split_k_skewed": (4603, 14336), "fewer_groups_than_teams": (100, 4096)}[case]
+  x = synth.activations(rng, 1, k, np.float16)
+  xb = gpu.Buffer.from_numpy(x)
+  w = synth.random_blocks(rng, t, n, k)
+  lin = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  ref = ol.linear_f64(x.astype(np.float32), ol.weight_f32(w, n, k, t))
+  nan = np.full((1, n), np.nan, np.float32)
+  if case in ("interleaved_ragged", "fewer_groups_than_teams"):
+    out = gpu.Buffer.from_numpy(nan)
+    qlinear_multi([lin], xb, [out])
+    y = out.numpy()
+  elif case in ("interleaved_residual", "split_k_skewed"):
+    res = rng.standard_normal((1, n)).astype(np.float32)
+    out = gpu.Buffer.from_numpy(res)
+    qlinear_multi([lin], xb, [out], epilogue=1, resid=[out])
+    y = out.numpy(); ref = ref + res
+  else:
+    w2 = synth.random_blocks(rng, t, n, k)
+    lin2 = QuantLinear(gpu.Buffer.from_numpy(w2), t, n, k)
+    out = gpu.Buffer.from_numpy(nan)
+    qlinear_multi([lin, lin2], xb, [out], epilogue=2)
+    y = out.numpy()
+    up = ol.linear_f64(x.astype(np.float32), ol.weight_f32(w2, n, k, t))
+    ref = ref / (1 + np.exp(-ref)) * up
+  assert np.isfinite(y).all(), f"{np.count_nonzero(~np.isfinite(y))} rows not written"
+  assert ol.rel_err(y, ref) <= TOL
+  atol = TOL * float(np.sqrt(np.mean(ref ** 2)))
+  assert np.isclose(y, ref, rtol=TOL, atol=atol).all()
