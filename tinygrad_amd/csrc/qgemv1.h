@@ -63,6 +63,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   // are faster with two row groups per lane (gate/up 15.8 -> 15.0 us, attn_output 5.45 -> 5.26 us), the plain epilogue and the split-K launches
   // with three (q/k/v 8.2 against 8.6 us, down 9.6 against 10.5 us); four is slower everywhere (578 against 607 tok/s).
   constexpr int D = (WK == 1 && !H && EPI != 0) ? 2 : QG1_DEPTH;
+  constexpr int NPC = (NT >= 512) ? 1 : 2;                        // 8-element activation pieces per thread in prologues 1 and 3 (rows of at most 8 NT NPC values)
   extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
   __shared__ float part[2][WK][R];
   __shared__ float nred[NT / 64];
@@ -259,14 +260,14 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   } else if constexpr (PRO == 1) {
     f32x4 l4[2], h4[2], w0[2], w1[2];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
+    for (int t = 0; t < NPC; t++) {
       const int i = (int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1;
       l4[t] = xr[2 * i]; h4[t] = xr[2 * i + 1];
       w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1];
     }
     float ss = 0.f;
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
+    for (int t = 0; t < NPC; t++) {
       const f32x4 l = l4[t], h = h4[t];
       const float s8 = l.x * l.x + l.y * l.y + l.z * l.z + l.w * l.w + h.x * h.x + h.y * h.y + h.z * h.z + h.w * h.w;
       ss += ((int)threadIdx.x + NT * t < nq) ? s8 : 0.f;
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     for (int j = 0; j < NT / 64; j++) tot += nred[j];
     const float nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
+    for (int t = 0; t < NPC; t++) {
       f32x4 l = l4[t], h = h4[t];
       l.x = (l.x * nscale) * w0[t].x; l.y = (l.y * nscale) * w0[t].y; l.z = (l.z * nscale) * w0[t].z; l.w = (l.w * nscale) * w0[t].w;
       h.x = (h.x * nscale) * w1[t].x; h.y = (h.y * nscale) * w1[t].y; h.z = (h.z * nscale) * w1[t].z; h.w = (h.w * nscale) * w1[t].w;
@@ -293,9 +294,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   } else if constexpr (PRO == 3) {
     u32x4 v[2];
 #pragma unroll
-    for (int t = 0; t < 2; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
+    for (int t = 0; t < NPC; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
 #pragma unroll
-    for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
+    for (int t = 0; t < NPC; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
     __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 1)
     issue(b[0], lo);
     lds_to_regs();
@@ -425,7 +426,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
     a.team_skew = two_per_cu ? 1 : 0; a.team_first = two_per_cu ? (int)(nteams / 2) : 0;
     a.team_stride = (!H && !a.team_skew && !a.sel && (EPI == 2 || a.nseg == 1)) ? (int)nteams : 0; }
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
-  const bool one_batch = a.K / 8 <= NT * 2;
+  const bool one_batch = a.K / 8 <= NT * (NT >= 512 ? 1 : 2);
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
   if constexpr (WK == 1 && EPI == 0) {
     if (a.comb_y) {
