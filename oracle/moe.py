@@ -2,7 +2,7 @@
 
 pairwise_topk, ExpertGating, FFNBlock._feed_forward (MoE branch): tinygrad/llm/model.py:9-13, 35-41, 110-135.
 route / dispatch / combine / m_max_for / Routing.rows_e: extra/gemm/moe_routing.py:89-131 (single device group, G = 1).
-PARITY UNPINNED for route/dispatch/combine: the reference holds no test for them; they are pinned by invariants only."""
+The reference holds no test for route / dispatch / combine; they are pinned by a hand-worked case and invariants (tests/test_oracle_pins.py)."""
 import numpy as np
 
 BLOCK_ROW = 256

@@ -1,0 +1,187 @@
+"""Pins for the oracle functions that no reference test covers: route / rows_e on a hand-computed case, grouped_mx_gemm_ref against a
+brute-force loop in exact rational arithmetic, and the wiring of llm.Model.forward through closed forms (each one built so that a
+plausible mistake - a tile too many, weights permuted against their experts, a transposed operand, np.tile for np.repeat, a cache
+row written at the wrong position, the FFN fed from the wrong residual - changes the expected numbers)."""
+from fractions import Fraction
+import struct
+import numpy as np
+from oracle import moe as omoe, mxfp8 as omx, llm as ollm
+
+# ------------------------------------------------------------------------------------------------ route (extra/gemm/moe_routing.py:109-122)
+def test_route_hand_computed_tie_and_empty_expert():
+  """T = 3, E = 4, k = 2.  Worked by hand from moe_routing.py:109-122 and Tensor.topk's order (descending, lower index first among equals):
+    token 0 logits [1, 1, 0, -1]      -> experts (0, 1), a tie, weights softmax(1, 1) = (1/2, 1/2)
+    token 1 logits [0, 3, -5, 2]      -> experts (1, 3), weights softmax(3, 2) = (e/(1+e), 1/(1+e))
+    token 2 logits [.5, -1, -2, .5]   -> experts (0, 3), a tie across a gap, weights (1/2, 1/2)
+  flattened assignments j = 0..5 go to experts 0, 1, 1, 3, 0, 3; expert 2 gets nothing.  counts (2, 2, 0, 2) -> padded (256, 256, 0, 256)
+  -> off = (0, 256, 512, 512, 768); dest_row = off[e] + (rank of j among the assignments of e) = (0, 256, 257, 512, 1, 513);
+  m_l = (ceil(6 / 256) + 4) * 256 = 1280; tile -> expert = #(off[:4] <= 256 t) - 1 = (0, 1, 3, 3, 3): the empty expert owns no tile."""
+  lg = np.array([[1, 1, 0, -1], [0, 3, -5, 2], [0.5, -1, -2, 0.5]], dtype=np.float32)
+  r = omoe.route(lg, 2, 4)
+  np.testing.assert_array_equal(r["topi"], [[0, 1], [1, 3], [0, 3]])
+  e = np.e
+  np.testing.assert_allclose(r["weights"], [[0.5, 0.5], [e / (1 + e), 1 / (1 + e)], [0.5, 0.5]], rtol=1e-6)
+  np.testing.assert_array_equal(r["off"], [0, 256, 512, 512, 768])
+  np.testing.assert_array_equal(r["dest_row"], [0, 256, 257, 512, 1, 513])
+  assert r["m_l"] == 1280 and omoe.m_max_for(3, 2, 4) == 1280
+  np.testing.assert_array_equal(omoe.rows_e(r["off"], r["m_l"]), [0, 1, 3, 3, 3])
+  # dispatch / combine on rows that identify their token: xg holds token j // k at dest_row[j], zero elsewhere; combine weighs slot s by weights[t, s]
+  x = np.array([[1.0, 10.0], [2.0, 20.0], [3.0, 30.0]], dtype=np.float32)
+  xg = omoe.dispatch(x, r, 2)
+  assert xg.shape == (1280, 2)
+  for row, tok in {0: 0, 1: 2, 256: 0, 257: 1, 512: 1, 513: 2}.items(): np.testing.assert_array_equal(xg[row], x[tok])
+  assert np.count_nonzero(xg.any(axis=1)) == 6
+  y = np.zeros((1280, 1), dtype=np.float32); y[[0, 256, 257, 512, 1, 513], 0] = [100, 200, 300, 400, 500, 600]   # y[dest_row[j]] = 100 (j + 1)
+  out = omoe.combine(y, r, 3, 2)
+  np.testing.assert_allclose(out[:, 0], [150.0, (300 * e + 400) / (1 + e), 550.0], rtol=1e-6)
+
+def test_route_padding_is_minimal_at_tile_boundaries():
+  """256 assignments to one expert need exactly one tile, 257 need two (off by one in the ceil would show here)."""
+  for n, tiles in ((255, 1), (256, 1), (257, 2), (512, 2), (513, 3)):
+    lg = np.full((n, 3), -1.0, dtype=np.float32); lg[:, 1] = 1.0
+    r = omoe.route(lg, 1, 3)
+    np.testing.assert_array_equal(r["off"], [0, 0, 256 * tiles, 256 * tiles])
+    np.testing.assert_array_equal(r["dest_row"], np.arange(n))
+    np.testing.assert_allclose(r["weights"], 1.0)
+
+# ------------------------------------------------------------------------------------------------ grouped_mx_gemm_ref
+def _e4m3_value(b: int) -> Fraction:
+  """OCP E4M3 (fn) by its definition: sign, 4-bit exponent with bias 7, 3-bit mantissa; exponent 0 = subnormal m / 8 * 2^-6."""
+  s, ex, m = -1 if b & 0x80 else 1, (b >> 3) & 0xF, b & 7
+  v = Fraction(m, 8) * Fraction(1, 64) if ex == 0 else (1 + Fraction(m, 8)) * (Fraction(2) ** (ex - 7))
+  return s * v
+
+def _bf16_rne(v: float) -> float:
+  """float32 -> bfloat16, round to nearest even, through the bit pattern."""
+  (u,) = struct.unpack("<I", struct.pack("<f", v))
+  u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+  return struct.unpack("<f", struct.pack("<I", u))[0]
+
+def test_grouped_mx_gemm_ref_against_exact_brute_force():
+  """Two 256-row tiles, three experts of which the middle one is empty; every output element recomputed as an exact rational sum over k of
+  e4m3(x) 2^(ex-127) e4m3(w[e]) 2^(ew-127) with e chosen by the row's offset range, then rounded float32 -> bf16."""
+  rng = np.random.default_rng(7)
+  M, N, K, E = 512, 3, 64, 3
+  off = np.array([0, 256, 256, 512], dtype=np.int32)
+  codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)          # every finite E4M3 code
+  xq, wq = rng.choice(codes, (M, K)), rng.choice(codes, (E, N, K))
+  xe, we = rng.integers(120, 131, (M, K // 32), dtype=np.uint8), rng.integers(120, 131, (E, N, K // 32), dtype=np.uint8)
+  got = omx.grouped_mx_gemm_ref(xq, xe, wq, we, off)
+  val = [_e4m3_value(c) for c in range(256)]
+  rows = list(range(0, 8)) + [255, 256, 257, 300, 511]                                       # both sides of the expert boundary
+  exact, ulp_off = 0, 0
+  for r in rows:
+    e = 0 if r < 256 else 2
+    for n in range(N):
+      acc = Fraction(0)
+      for k in range(K):
+        acc += val[xq[r, k]] * Fraction(2) ** (int(xe[r, k // 32]) - 127) * val[wq[e, n, k]] * Fraction(2) ** (int(we[e, n, k // 32]) - 127)
+      want = _bf16_rne(float(np.float32(float(acc))))
+      if got[r, n] == want: exact += 1
+      else:
+        assert abs(got[r, n] - want) <= abs(want) * 2.0 ** -7, (r, n, got[r, n], want)      # one bf16 ulp (float64 vs exact accumulation before the rounding)
+        ulp_off += 1
+  assert exact >= 0.95 * len(rows) * N, (exact, ulp_off)
+  # a transposed or mis-scaled operand is far outside a bf16 ulp: the check above has teeth
+  bad = omx.grouped_mx_gemm_ref(xq, xe, wq[::-1], we[::-1], off)
+  assert np.abs(bad[:8] - got[:8]).max() > 2.0 ** -6 * np.abs(got[:8]).max()
+
+# ------------------------------------------------------------------------------------------------ llm.Model.forward wiring
+def _model(H=4, KV=2, hd=8, dim=32, hidden=32, vocab=16, blocks=1, seed=0, **over):
+  """A float32 (ggml type 0) model whose matrices are set by the caller: {name: array} overrides on top of zeros / identities."""
+  rng = np.random.default_rng(seed)
+  cfg = dict(num_blocks=blocks, dim=dim, hidden_dim=hidden, n_heads=H, n_kv_heads=KV, norm_eps=1e-5, vocab_size=vocab, head_dim=hd, rope_theta=10000.0)
+  t = {"token_embd.weight": rng.standard_normal((vocab, dim)).astype(np.float32), "output_norm.weight": np.ones((1, dim), np.float32),
+       "output.weight": np.eye(vocab, dim, dtype=np.float32)}
+  for i in range(blocks):
+    p = f"blk.{i}."
+    t.update({p + "attn_norm.weight": np.ones((1, dim), np.float32), p + "ffn_norm.weight": np.ones((1, dim), np.float32),
+              p + "attn_q.weight": rng.standard_normal((H * hd, dim)).astype(np.float32), p + "attn_k.weight": rng.standard_normal((KV * hd, dim)).astype(np.float32),
+              p + "attn_v.weight": rng.standard_normal((KV * hd, dim)).astype(np.float32), p + "attn_output.weight": np.zeros((dim, H * hd), np.float32),
+              p + "ffn_gate.weight": rng.standard_normal((hidden, dim)).astype(np.float32), p + "ffn_up.weight": rng.standard_normal((hidden, dim)).astype(np.float32),
+              p + "ffn_down.weight": np.zeros((dim, hidden), np.float32)})
+  t.update(over)
+  tensors = {k: (np.ascontiguousarray(v).view(np.uint8).reshape(-1), 0, v.shape) for k, v in t.items()}
+  return ollm.Model(cfg, tensors, 16, w_round_f16=False, kv_dtype=np.float32), t, cfg
+
+def _rms(x, eps=1e-5): return x / np.sqrt(np.mean(x * x) + eps)
+
+def test_forward_residual_passes_through_when_projections_are_zero():
+  """attn_output = 0 and ffn_down = 0 in both blocks: the row that reaches output_norm is the embedding row itself."""
+  m, t, cfg = _model(blocks=2)
+  for tok, pos in ((3, 0), (7, 1), (3, 2)):
+    lg = m.forward(tok, pos)
+    np.testing.assert_allclose(lg, _rms(t["token_embd.weight"][tok])[:cfg["vocab_size"]], rtol=1e-5, atol=1e-6)
+
+def test_forward_single_position_returns_v_with_gqa_mapping():
+  """Position 0 holds one key: softmax over one score is 1, so head h outputs the value row of kv head h // (H / KV).  The values are made
+  constant per kv head through attn_v.bias (weight 0), attn_output is the identity, so the logits show x + c[h // group] block by block."""
+  H, KV, hd, dim = 4, 2, 8, 32
+  c = np.array([5.0, -3.0], dtype=np.float32)
+  m, t, cfg = _model(H, KV, hd, dim, **{"blk.0.attn_v.weight": np.zeros((KV * hd, dim), np.float32), "blk.0.attn_q.bias": np.zeros((1, H * hd), np.float32),
+                                        "blk.0.attn_k.bias": np.zeros((1, KV * hd), np.float32), "blk.0.attn_v.bias": np.repeat(c, hd)[None, :].astype(np.float32),
+                                        "blk.0.attn_output.weight": np.eye(dim, H * hd, dtype=np.float32), "output.weight": np.eye(dim, dim, dtype=np.float32),
+                                        "token_embd.weight": np.random.default_rng(1).standard_normal((32, dim)).astype(np.float32)}, vocab=32)
+  x = t["token_embd.weight"][9]
+  want = x + np.repeat(c[[0, 0, 1, 1]], hd)                       # heads 0, 1 -> kv head 0; heads 2, 3 -> kv head 1 (repeat_interleave, not tile)
+  np.testing.assert_allclose(m.forward(9, 0), _rms(want), rtol=1e-5, atol=1e-6)
+
+def test_forward_uniform_attention_averages_the_cached_values():
+  """attn_k = 0: every score is 0, the softmax is uniform over positions 0..pos, so the attention output at position p is the mean of the values
+  written at 0..p - each token's value row must have been written at its own position and all of them read back."""
+  H, KV, hd, dim = 2, 2, 8, 16
+  rng = np.random.default_rng(2)
+  Wv = rng.standard_normal((KV * hd, dim)).astype(np.float32)
+  m, t, cfg = _model(H, KV, hd, dim, hidden=16, vocab=16, **{"blk.0.attn_k.weight": np.zeros((KV * hd, dim), np.float32), "blk.0.attn_v.weight": Wv,
+                                                              "blk.0.attn_output.weight": np.eye(dim, H * hd, dtype=np.float32), "output.weight": np.eye(dim, dim, dtype=np.float32)})
+  toks = [4, 11, 6, 11]
+  vals = []
+  for pos, tok in enumerate(toks):
+    x = t["token_embd.weight"][tok]
+    vals.append(Wv @ _rms(x))
+    want = x + np.mean(vals, axis=0)
+    np.testing.assert_allclose(m.forward(tok, pos), _rms(want), rtol=2e-5, atol=2e-6)
+
+def test_forward_attention_prefers_the_matching_key_across_positions():
+  """RoPE makes q . k depend on the distance only: with q = k projections (one head) and a sharp scale, the token attends to the cached position
+  that holds the SAME token at distance 0 (itself) rather than to a different token, and the rotation keeps |q . k| of the self score at |k|^2."""
+  H = KV = 1; hd = dim = 16
+  rng = np.random.default_rng(3)
+  P = (rng.standard_normal((hd, dim)) * 4).astype(np.float32)
+  m, t, cfg = _model(H, KV, hd, dim, hidden=16, vocab=16, **{"blk.0.attn_q.weight": P, "blk.0.attn_k.weight": P, "blk.0.attn_v.weight": np.eye(hd, dim, dtype=np.float32),
+                                                              "blk.0.attn_output.weight": np.eye(dim, hd, dtype=np.float32), "output.weight": np.eye(dim, dim, dtype=np.float32)})
+  a, b = t["token_embd.weight"][1], t["token_embd.weight"][2]
+  m.forward(1, 0)
+  lg = m.forward(2, 1)                                             # scores: (q_b . R(-1) k_a, |k_b|^2) / 4; the self score dominates by construction of the scale
+  qa, qb = P @ _rms(a), P @ _rms(b)
+  self_score = float(qb @ qb) / 4
+  assert self_score > 40                                           # the softmax is saturated unless the self score were computed wrongly
+  np.testing.assert_allclose(lg, _rms(b + _rms(b)), rtol=1e-4, atol=1e-5)   # value = eye @ rms(b): attention returns (almost exactly) the token's own value
+
+def test_forward_ffn_reads_the_post_attention_residual():
+  """h = x + attention, out = h + down(silu(gate n) * up n) with n = rmsnorm(h): gate = up = down = identity make the FFN term silu(n) * n, and
+  a non-zero attention term (constant value rows, single position) separates h from x."""
+  H = KV = 2; hd = 8; dim = 16
+  c = np.array([2.0, -1.0], dtype=np.float32)
+  I = np.eye(dim, dtype=np.float32)
+  m, t, cfg = _model(H, KV, hd, dim, hidden=dim, vocab=16, **{"blk.0.attn_v.weight": np.zeros((KV * hd, dim), np.float32), "blk.0.attn_q.bias": np.zeros((1, H * hd), np.float32),
+                                                               "blk.0.attn_k.bias": np.zeros((1, KV * hd), np.float32), "blk.0.attn_v.bias": np.repeat(c, hd)[None, :].astype(np.float32),
+                                                               "blk.0.attn_output.weight": I, "blk.0.ffn_gate.weight": I, "blk.0.ffn_up.weight": I, "blk.0.ffn_down.weight": I,
+                                                               "output.weight": I})
+  x = t["token_embd.weight"][5]
+  h = x + np.repeat(c, hd)
+  n = _rms(h)
+  want = h + (n / (1 + np.exp(-n))) * n
+  np.testing.assert_allclose(m.forward(5, 0), _rms(want), rtol=1e-5, atol=1e-6)
+  wrong = x + (_rms(x) / (1 + np.exp(-_rms(x)))) * _rms(x) + np.repeat(c, hd)          # FFN fed from x instead of h: measurably different
+  assert np.abs(_rms(wrong) - _rms(want)).max() > 1e-2
+
+def test_generate_is_greedy_first_maximum():
+  """generate() feeds prompt tokens at consecutive positions and picks the FIRST index of the maximum (a tie is made with a duplicated output row)."""
+  dim = 16
+  out_w = np.eye(16, dim, dtype=np.float32); out_w[9] = out_w[4]                          # rows 4 and 9 always tie
+  emb = np.zeros((16, dim), np.float32)
+  for tok in range(16): emb[tok, 4 if tok % 2 == 0 else (tok + 1) % 16] = 1.0             # even tokens point at the tied pair, odd token t at t + 1
+  m, t, cfg = _model(2, 2, 8, dim, hidden=16, vocab=16, **{"token_embd.weight": emb, "output.weight": out_w})
+  toks, margins = m.generate([1], 3)
+  assert toks == [2, 4, 4] and margins[1] == 0.0                                          # 1 -> 2; 2 -> tie(4, 9) -> 4; 4 -> tie -> 4
