@@ -4,24 +4,115 @@
 A step is one decoded token.  Random-init weights are written on the GPU as GGUF blocks (Q4_0 linears and embedding, Q6_K
 lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the model itself, then --warmup + --steps tokens
 are decoded greedily, one captured launch sequence per token with a host sync per token (as the reference's generate loop does).
-Prints ONE JSON line: tok/s, the roofline of the dominant kernel from HIP-event timings taken live, the same figures for the other
-kernels of a block, and a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the same weights).
-Default path: one launch per op (six per block, attention being two); the dominant kernel is then the fused ffn_gate + ffn_up dequant-GEMV with the
-ffn_norm folded in.  --fused: all 32 blocks of a token in one persistent launch (tga_decode_layers), which is then the kernel reported."""
+Prints ONE JSON line: tok/s, the roofline of the dominant kernel from HIP-event timings taken live (the fused ffn_norm + ffn_gate + ffn_up +
+SwiGLU dequant-GEMV, one of six launches per block), the same figures for the other kernels of a block, a parity gate (outside the timed
+region: one more decoded token of the SAME model recomputed on the CPU from the GPU's own KV cache, and every linear of layer 0 on a fresh
+row; the run exits non-zero when a bar is missed), a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the
+same weights) and the kernel-level figures of the other benchmark configurations measured in the same process."""
 import argparse, json, os, sys, time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
-GATE_UP_TRAFFIC_BYTES = 66702500   # 66 609 152 B fetched + 93 389 B written per launch (counter runs summarised in profiles/qgemv1_gate_up_hbm_traffic.md)
+# HBM bytes per launch of the dominant kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE) of
+# `python -m tinygrad_amd.benchmarks --traffic`, each scaled by what the same counter reads for a 1 GiB copy kernel (x2.0000 and x1.0000):
+# 66 609 152 B fetched + 93 389 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
+GATE_UP_TRAFFIC_BYTES = 66702500
+PARITY_TOL = 1e-3
 
-def cpu_baseline(model, cfg, seconds_budget=20.0):
+def _host_layer(model, i):
+  b = model.blk[i]
+  lins = dict(attn_q=b.attn_q, attn_k=b.attn_k, attn_v=b.attn_v, attn_output=b.attn_output, ffn_gate=b.ffn_gate, ffn_up=b.ffn_up, ffn_down=b.ffn_down)
+  return {k: (l.ggml_type, l.blocks.view(0, (l.nbytes,), np.uint8).numpy(), l.out_features, l.in_features) for k, l in lins.items()}
+
+def parity_gate(model, c, threads):
+  """Checks, against the C / numpy restatement of the reference's model-path numerics (fp32 activations, fp16-rounded weights, fp32 accumulate,
+  fp16 KV cache), (1) the seven linears of layer 0 and 4096 spread rows of the lm-head on a fresh random row, through the same fused entry
+  points the decode step uses, and (2) one more decoded token of the benchmark model itself: the CPU recomputes the whole step for the same
+  input token from the GPU's own KV cache of the earlier positions and must arrive at the same greedy token with logits within the bar."""
+  from oracle import cref, llm as ollm, linear as ol
+  from tinygrad_amd import runtime as rt
+  from tinygrad_amd.nn import qlinear_multi, stage_activation
+  lin = lambda t, w, x, n, k: cref.linear(t, w, np.ascontiguousarray(x, dtype=np.float32).reshape(1, -1), n, k, w_round_f16=True, threads=threads)[0]
+  rng = np.random.default_rng(7)
+  B = rt.Buffer.from_numpy
+  b0, host0 = model.blk[0], _host_layer(model, 0)
+  checked, worst = [], 0.0
+  def note(name, got, ref):
+    nonlocal worst
+    e = ol.rel_err(np.asarray(got).reshape(-1), np.asarray(ref).reshape(-1)); worst = max(worst, e); checked.append({"what": name, "rel_err": float(f"{e:.3e}")})
+  # ---- (1) layer 0's launches on a fresh row
+  x = (rng.standard_normal((1, c.dim)) * 2).astype(np.float32)
+  an, fn = b0.attn_norm.numpy().reshape(-1), b0.ffn_norm.numpy().reshape(-1)
+  xn = ollm.rmsnorm(x, an, c.norm_eps)
+  q, k, v = (rt.Buffer((1, n), np.float32) for n in (b0.attn_q.out_features, b0.attn_k.out_features, b0.attn_v.out_features))
+  qlinear_multi([b0.attn_q, b0.attn_k, b0.attn_v], B(x), [q, k, v], norm=(b0.attn_norm, c.norm_eps))
+  for nm, got in (("attn_q", q), ("attn_k", k), ("attn_v", v)): note("blk.0." + nm, got.numpy(), lin(*host0[nm][:2], xn, *host0[nm][2:]))
+  attn = rng.standard_normal((1, b0.attn_output.in_features)).astype(np.float16)
+  h = B(x.copy())
+  qlinear_multi([b0.attn_output], stage_activation(b0.attn_output, B(attn)) if b0.stage_attn else B(attn), [h], epilogue=1, resid=[h], x_staged=b0.stage_attn)
+  note("blk.0.attn_output + residual", h.numpy(), x[0] + lin(*host0["attn_output"][:2], attn, *host0["attn_output"][2:]))
+  act = rt.Buffer((1, c.hidden_dim), np.float16)
+  qlinear_multi([b0.ffn_gate, b0.ffn_up], h, [act], epilogue=2, norm=(b0.ffn_norm, c.norm_eps))
+  hn = ollm.rmsnorm(h.numpy(), fn, c.norm_eps)
+  aref = ollm.silu(lin(*host0["ffn_gate"][:2], hn, *host0["ffn_gate"][2:])) * lin(*host0["ffn_up"][:2], hn, *host0["ffn_up"][2:])
+  note("blk.0.silu(ffn_gate) * ffn_up", act.numpy(), aref)
+  a16 = aref.astype(np.float16).reshape(1, -1)
+  out = B(h.numpy())
+  qlinear_multi([b0.ffn_down], stage_activation(b0.ffn_down, B(a16)) if b0.stage_act else B(a16), [out], epilogue=1, resid=[out], x_staged=b0.stage_act)
+  note("blk.0.ffn_down + residual", out.numpy(), h.numpy()[0] + lin(*host0["ffn_down"][:2], a16, *host0["ffn_down"][2:]))
+  head = model.output
+  row_bytes = head.nbytes // head.out_features
+  lg = rt.Buffer((1, c.vocab_size), np.float32)
+  qlinear_multi([head], B(x), [lg], norm=(model.output_norm, c.norm_eps))
+  xo = ollm.rmsnorm(x, model.output_norm.numpy().reshape(-1), c.norm_eps)
+  lgh = lg.numpy()[0]
+  got_rows, ref_rows = [], []
+  for r0 in np.linspace(0, c.vocab_size - 512, 8).astype(int):
+    r0 = int(r0) & ~1
+    wslice = head.blocks.view(r0 * row_bytes, (512 * row_bytes,), np.uint8).numpy()
+    ref_rows.append(lin(head.ggml_type, wslice, xo, 512, c.dim)); got_rows.append(lgh[r0:r0 + 512])
+  note("output_norm + lm-head (8 x 512 spread rows)", np.concatenate(got_rows), np.concatenate(ref_rows))
+  # ---- (2) one more token of the benchmark model, recomputed on the CPU from the GPU's KV cache
+  st = model.s.state.numpy()
+  pos, tok = int(st[0]), int(st[1])
+  model.decode_step(True)
+  lg_gpu, tok_gpu = model.logits(), int(model.s.state.numpy()[1])
+  H, KV, hd = c.n_heads, c.n_kv_heads, c.head_dim
+  fc = ollm.precompute_freqs_cis(hd, pos + 1, c.rope_theta)[pos]
+  emb_row_bytes = model.token_embd.nbytes // c.vocab_size
+  from oracle import ggml as og
+  xr = og.ggml_data_to_tensor(model.token_embd.view(tok * emb_row_bytes, (emb_row_bytes,), np.uint8).numpy(), c.dim, model.embd_type).astype(np.float32)
+  for i, b in enumerate(model.blk):
+    hl = _host_layer(model, i)
+    n1 = ollm.rmsnorm(xr, b.attn_norm.numpy().reshape(-1), c.norm_eps)
+    qv, kv_, vv = (lin(*hl[nm][:2], n1, *hl[nm][2:]) for nm in ("attn_q", "attn_k", "attn_v"))
+    qr, kr = ollm.apply_rope(qv.reshape(H, hd), fc), ollm.apply_rope(kv_.reshape(KV, hd), fc)
+    ck, cv = b.cache_k.numpy()[:, :pos + 1].astype(np.float32), b.cache_v.numpy()[:, :pos + 1].astype(np.float32)
+    ck[:, pos], cv[:, pos] = kr.astype(np.float16).astype(np.float32), vv.reshape(KV, hd).astype(np.float16).astype(np.float32)   # this token's own rows, recomputed
+    Kh, Vh = np.repeat(ck, H // KV, axis=0), np.repeat(cv, H // KV, axis=0)
+    sc = np.einsum("hd,htd->ht", qr, Kh).astype(np.float32) / np.float32(np.sqrt(hd))
+    e = np.exp(sc - sc.max(-1, keepdims=True)); pr = e / e.sum(-1, keepdims=True)
+    at = np.einsum("ht,htd->hd", pr, Vh).astype(np.float32).reshape(-1)
+    hh = xr + lin(*hl["attn_output"][:2], at, *hl["attn_output"][2:])
+    n2 = ollm.rmsnorm(hh, b.ffn_norm.numpy().reshape(-1), c.norm_eps)
+    ff = ollm.silu(lin(*hl["ffn_gate"][:2], n2, *hl["ffn_gate"][2:])) * lin(*hl["ffn_up"][:2], n2, *hl["ffn_up"][2:])
+    xr = hh + lin(*hl["ffn_down"][:2], ff, *hl["ffn_down"][2:])
+  xo = ollm.rmsnorm(xr, model.output_norm.numpy().reshape(-1), c.norm_eps)
+  lg_cpu = lin(head.ggml_type, head.blocks.view(0, (head.nbytes,), np.uint8).numpy(), xo, c.vocab_size, c.dim)
+  note(f"full decode step at position {pos} ({c.num_blocks} blocks + lm-head): logits", lg_gpu, lg_cpu)
+  top2 = np.partition(lg_cpu, -2)[-2:]
+  tok_cpu = int(np.argmax(lg_cpu))
+  res = {"bar_rel_err": PARITY_TOL, "max_rel_err": float(f"{worst:.3e}"), "greedy_token_gpu": tok_gpu, "greedy_token_cpu": tok_cpu,
+         "cpu_top2_margin": float(f"{float(top2[1] - top2[0]):.4e}"), "checked": checked,
+         "ok": bool(worst <= PARITY_TOL and tok_gpu == tok_cpu)}
+  return res
+
+def cpu_baseline(model, cfg, threads_all):
   """Times oracle/c (scalar C restatement of dequant + fp32-accumulate matmul, model-path numerics) on the GPU box's host
-  cores: the 7 linears of layer 0 plus a 1/32 row slice of the lm-head, extrapolated to one token (32 layers + full head)."""
+  cores: the 7 linears of layer 0 plus a 1/32 row slice of the lm-head, extrapolated to one token (32 layers + full head).  Protocol: 2 warm-up
+  passes, then the median of 5 timed passes (7 on one thread when they fit 20 s), wall clock."""
   from oracle import cref
-  b = model.blk[0]
-  lins = [("attn_q", b.attn_q), ("attn_k", b.attn_k), ("attn_v", b.attn_v), ("attn_output", b.attn_output),
-          ("ffn_gate", b.ffn_gate), ("ffn_up", b.ffn_up), ("ffn_down", b.ffn_down)]
-  host = [(l.ggml_type, l.blocks.view(0, (l.nbytes,), np.uint8).numpy(), l.out_features, l.in_features) for _, l in lins]
+  host = list(_host_layer(model, 0).values())
   head = model.output
   hrows = head.out_features // 32
   hbytes = hrows * (head.nbytes // head.out_features)
@@ -34,21 +125,26 @@ def cpu_baseline(model, cfg, seconds_budget=20.0):
     cref.linear(head.ggml_type, hw, rng.standard_normal((1, head.in_features)).astype(np.float32), hrows, head.in_features, w_round_f16=True, threads=threads)
     t2 = time.perf_counter()
     return (t1 - t0), (t2 - t1) * 32
-  one_pass(1)                                             # warm-up (page in, build)
-  reps = []
-  t_start = time.perf_counter()
-  while len(reps) < 3 or (time.perf_counter() - t_start < seconds_budget / 2 and len(reps) < 9): reps.append(one_pass(1))
-  layer_s, head_s = np.median([r[0] for r in reps]), np.median([r[1] for r in reps])
-  tok_s_1 = 1.0 / (cfg["num_blocks"] * layer_s + head_s)
-  cores = len(os.sched_getaffinity(0))
-  nthr = min(cores, cref.max_threads())
-  one_pass(nthr)
-  repn = [one_pass(nthr) for _ in range(3)]
-  tok_s_n = 1.0 / (cfg["num_blocks"] * np.median([r[0] for r in repn]) + np.median([r[1] for r in repn]))
+  def measure(threads, budget_s):
+    one_pass(threads); one_pass(threads)                  # two warm-ups
+    reps, t_start = [], time.perf_counter()
+    while len(reps) < 5 or (len(reps) < 7 and time.perf_counter() - t_start < budget_s): reps.append(one_pass(threads))
+    return 1.0 / (cfg["num_blocks"] * np.median([r[0] for r in reps]) + np.median([r[1] for r in reps])), len(reps)
+  tok_s_1, n1 = measure(1, 12.0)
+  tok_s_n, nn = measure(threads_all, 4.0)
   return {"value": round(tok_s_1, 4), "unit": "tok/s", "cores": 1, "kind": "port",
-          "sample": "oracle/c scalar restatement (dequant -> fp16-rounded weight -> fp32 MAC), 1 thread: the 7 linears of layer 0 + 1/32 of the "
-                    "lm-head rows, median of >=3 passes, extrapolated to 32 layers + full lm-head (attention/norms excluded)",
-          "all_cores": {"value": round(tok_s_n, 4), "cores": int(nthr)}}
+          "sample": f"oracle/c scalar restatement (dequant -> fp16-rounded weight -> fp32 MAC), 1 thread: the 7 linears of layer 0 + 1/32 of the "
+                    f"lm-head rows, 2 warm-ups then the median of {n1} passes, extrapolated to {cfg['num_blocks']} layers + full lm-head (attention/norms excluded)",
+          "all_cores": {"value": round(tok_s_n, 4), "cores": int(threads_all), "passes": nn}}
+
+def other_configs():
+  """Kernel-level figures of benchmark configurations 1, 2, 4 and 5 (python -m tinygrad_amd.benchmarks) measured in this process."""
+  from tinygrad_amd import benchmarks as bm
+  out = {}
+  for name, fn in (("config1", bm.config1), ("config2", bm.config2), ("config4", bm.config4), ("config5", bm.config5)):
+    try: out[name] = [{k: v for k, v in row.items() if k != "config"} for row in fn()]
+    except Exception as e: out[name] = {"error": f"{type(e).__name__}: {e}"}
+  return out
 
 def main():
   ap = argparse.ArgumentParser()
@@ -57,10 +153,10 @@ def main():
   ap.add_argument("--warmup", type=int, default=8)
   ap.add_argument("--prefill", type=int, default=1024)
   ap.add_argument("--layers", type=int, default=32, help="reduce only for smoke runs; the reported config then says so")
-  ap.add_argument("--no-cpu", action="store_true")
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--no-parity", action="store_true", help="skip the parity gate (profiling runs)")
+  ap.add_argument("--no-other", action="store_true", help="skip the kernel-level figures of the other configurations")
   ap.add_argument("--no-graph", action="store_true", help="eager launches instead of graph replay (for kernel-trace profiling)")
-  ap.add_argument("--fused", action="store_true", help="all blocks of a token in one persistent launch instead of one launch per op")
-  ap.add_argument("--per-op", action="store_true", help="(the default; kept so that older command lines still run)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py: this build measures one GPU only (no collectives, no sharding in this run); use --gpus 1", file=sys.stderr)
@@ -70,11 +166,11 @@ def main():
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
   rt.init(0)
   cfg = dict(LLAMA3_8B); cfg["num_blocks"] = args.layers
-  max_new = args.steps + args.warmup + 16                    # + the eager steps of the per-kernel timing below
+  max_new = args.steps + args.warmup + 16                    # + the parity step and the eager steps of the per-kernel timing below
   max_ctx = ((args.prefill + max_new + 63) // 64) * 64
   c = TransformerConfig(max_context=max_ctx, **cfg)
   sd = synth_state(c, seed=1003)
-  model = Transformer(c, sd, max_new=max_new, fused=args.fused)
+  model = Transformer(c, sd, max_new=max_new)
   rt.synchronize()
 
   rng = np.random.default_rng(1003)
@@ -87,38 +183,19 @@ def main():
   for _ in range(args.steps): model.decode_step(ug)          # graph launch + stream sync per token
   rt.synchronize()
   dt = time.perf_counter() - t0
+  model.check_state()
   ms_per_step = dt / args.steps * 1e3
   tok_s = args.steps / dt
+  threads_all = min(len(os.sched_getaffinity(0)), 64)
+  parity = None
+  if not args.no_parity:
+    from oracle import cref
+    parity = parity_gate(model, c, min(threads_all, cref.max_threads()))
 
-  # ---- live timing of the dominant kernel: HIP events (on the model's stream) around the one-launch block kernel of eager steps ----
-  st = model.stream.handle
-  L = rt.lib()
-  fused_us, phase = [], None
-  if model.layer_table is not None:
-    s_ = model.s
-    tb = rt.Buffer((8 * 11 * c.num_blocks,), np.uint64).zero_()
-    for it in range(8):
-      rt.check(L.tga_embed_row(model.token_embd.ptr, model.embd_type, c.dim, s_.state.ptr, s_.x.ptr, st))
-      if it == 7: rt.check(L.tga_decode_layers_trace(tb.ptr))
-      e0, e1 = rt.Event(), rt.Event(); e0.record(st)
-      rt.check(L.tga_decode_layers(model.layer_table.ptr, c.num_blocks, model.layer_type, s_.x.ptr, s_.qkv.ptr, s_.attn.ptr, s_.act.ptr, s_.attn_part.ptr,
-                                   s_.state.ptr, s_.rope.ptr, s_.sync.ptr, c.dim, c.hidden_dim, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, c.norm_eps, st))
-      e1.record(st)
-      rt.check(L.tga_advance_prompt(s_.state.ptr, s_.prompt.ptr, st))
-      model.stream.synchronize()
-      fused_us.append(e0.elapsed_ms(e1) * 1e3)
-    rt.check(L.tga_decode_layers_trace(None))
-    model.check_fused()
-    if c.num_blocks > 2:
-      # wall-clock stamps (100 MHz) of workgroups 0, 73, ... at the phase boundaries of every block: time from the start of a
-      # phase (all workgroups past the barrier) to the last sampled workgroup finishing it, median over the inner blocks
-      T = tb.numpy().astype(np.int64).reshape(8, c.num_blocks, 11)[:, 1:-1]
-      span = lambda i0, i1: float(np.median(T[:, :, i1].max(0) - T[:, :, i0].min(0)) * 0.01)
-      phase = {"qkv_after_staging_us": round(span(0, 1), 2),
-               "attention_us": round(span(2, 3), 2), "attn_output_us": round(span(4, 5), 2), "gate_up_us": round(span(6, 7), 2), "down_us": round(span(8, 9), 2),
-               "block_us": round(float(np.median(np.diff(T[0, :, 0])) * 0.01), 2)}
   # ---- the per-op kernels on the same weights, timed with HIP events on the model's stream (the launches of TransformerBlock.__call__:
   #      q/k/v with attn_norm folded in, attention, attn_output + residual, gate/up with ffn_norm folded in + SwiGLU, down + residual) ----
+  st = model.stream.handle
+  L = rt.lib()
   from tinygrad_amd.nn import qlinear_multi
   durs = {"gate_up": [], "down": [], "qkv": [], "attn_output": [], "attention": []}
   s = model.s
@@ -152,7 +229,7 @@ def main():
     if it > 0:
       for k in durs: durs[k].append(ev[k][0].elapsed_ms(ev[k][1]) * 1e3 / len(model.blk))
   b0 = model.blk[0]
-  ctx_now = args.prefill + args.warmup + args.steps
+  ctx_now = int(model.s.state.numpy()[0])
   alg = {"gate_up": b0.ffn_gate.nbytes + b0.ffn_up.nbytes + c.dim * 8 + c.hidden_dim * 2,            # weights + fp32 row + norm weight + fp16 out
          "down": b0.ffn_down.nbytes + c.hidden_dim * 2 + c.dim * 8,
          "qkv": b0.attn_q.nbytes + b0.attn_k.nbytes + b0.attn_v.nbytes + c.dim * 8 + (c.n_heads + 2 * c.n_kv_heads) * c.head_dim * 4,
@@ -172,36 +249,28 @@ def main():
                "weight_bytes_per_token": int(wbytes), "stream_GBps_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9, 1),
                "frac_hbm_over_whole_step": round((wbytes + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
   }
-  if fused_us:
-    # algorithmic bytes of one launch: the seven Q4_0 matrices of every block + the fp16 K/V rows read at this context length
-    blk_w = sum(l.nbytes for b in model.blk for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down))
-    alg_f = blk_w + 2 * c.num_blocks * c.n_kv_heads * c.head_dim * ctx_now * 2
-    avg = float(np.mean(fused_us[1:]))
-    out["roofline"] = {"bound": "hbm", "kernel": f"decode_layers_kernel<Q4_0 pair> (all {c.num_blocks} blocks of one token in one persistent launch: 4 dequant-GEMV phases + attention per block)",
-                       "achieved": round(alg_f / avg / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_f / avg / 1e3 / HBM_PEAK_GBS, 4),
-                       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py at context 1024
-                       # (counters scaled by a 1 GiB copy kernel: x2.0000 and x1.0000): 4 100.5 MB fetched + 43.0 MB written
-                       "traffic": 4143500000 if c.num_blocks == 32 else None,
-                       "avg_launch_us": round(avg, 2), "alg_bytes_per_launch": int(alg_f), "phase_us_inside_launch": phase,
-                       "per_op_kernels": kern}
-    if phase:
-      out["roofline"]["gate_up_phase_GBps"] = round(alg["gate_up"] / phase["gate_up_us"] / 1e3, 1)
-      out["roofline"]["down_phase_GBps"] = round(alg["down"] / phase["down_us"] / 1e3, 1)
-  else:
-    dom = kern["gate_up"]
-    per_block = sum(v["avg_us"] for v in kern.values())
-    out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=8, SwiGLU, norm prologue> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
-                                                 "one of six launches per block)",
-                       "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
-                       # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of tinygrad_amd/traffic_probe.py (counters scaled by a
-                       # 1 GiB copy kernel: x2.0000 and x1.0000)
-                       "traffic": GATE_UP_TRAFFIC_BYTES if c.num_blocks == 32 else None,
-                       "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"],
-                       "share_of_block_time": round(dom["avg_us"] / per_block, 3),
-                       "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
+  dom = kern["gate_up"]
+  per_block = sum(v["avg_us"] for v in kern.values())
+  out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=8, SwiGLU, norm prologue> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
+                                               "one of six launches per block)",
+                     "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
+                     "traffic": GATE_UP_TRAFFIC_BYTES if c.num_blocks == 32 else None,
+                     "traffic_source": "recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run",
+                     "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"],
+                     "timing": "HIP events on the launch stream around the 32 gate/up launches of all blocks issued back to back, three repetitions; the rocprofv3 kernel-trace "
+                               "average of the same kernel inside the decode step is in profiles/decode_llama3_8b_q4_0_kernel_stats.md",
+                     "share_of_block_time": round(dom["avg_us"] / per_block, 3),
+                     "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
+  if parity is not None: out["parity"] = parity
   if not args.no_cpu:
-    out["cpu_baseline"] = cpu_baseline(model, cfg)
+    from oracle import cref
+    out["cpu_baseline"] = cpu_baseline(model, cfg, min(threads_all, cref.max_threads()))
+  if not args.no_other:
+    out["other_configs"] = other_configs()
   print(json.dumps(out))
+  if parity is not None and not parity["ok"]:
+    print(f"bench.py: PARITY GATE FAILED: max rel-err {parity['max_rel_err']} (bar {PARITY_TOL}), greedy token gpu {parity['greedy_token_gpu']} cpu {parity['greedy_token_cpu']}", file=sys.stderr)
+    sys.exit(1)
 
 if __name__ == "__main__":
   main()

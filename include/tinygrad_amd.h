@@ -143,8 +143,11 @@ int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, con
 int tga_moe_combine(const float* y, const float* probs, const float* resid, int n_tokens, int k, int dim, float* out, void* stream);
 
 /* ---- decode-step neighbours of the linears (batch 1), tinygrad/llm/model.py:144-204, 358-364 ----
- * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, pad[12]} so that one captured launch sequence serves
- * every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484). */
+ * `state` is a 64-byte device record {int32 pos, token, step, n_prompt, error, vocab, pad[10]} so that one captured launch sequence
+ * serves every position (the reference binds a symbolic start_pos into its replayed graph, model.py:464-484).  vocab = rows of the
+ * embedding table (0: token ids are not checked).  error is a bit mask the kernels set instead of reading or writing out of bounds:
+ * bit 0 = tga_embed_row met a token id outside [0, vocab) and read row 0; bit 1 = tga_attention_decode met pos outside [0, max_ctx)
+ * and did nothing.  The caller checks and clears it after synchronising. */
 
 /* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 /
  * Q4_K / Q5_K / Q6_K / MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant). */
@@ -179,27 +182,6 @@ int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i
 /* prompt step that skips the output projection: token = prompt[pos + 1], pos += 1. */
 int tga_advance_prompt(void* state, const int* prompt, void* stream);
 
-/* All transformer blocks of one batch-1 decode step in one persistent launch (dense llama-family blocks whose seven linears share
- * one type, Q4_0 or Q8_0): per block attn_norm -> q/k/v -> RoPE + KV append + attention -> attn_output + residual -> ffn_norm ->
- * silu(gate) * up -> down + residual (tinygrad/llm/model.py:144-204), the same arithmetic as the per-op entry points above.
- * layer_table: device array of n_layers records of 11 pointers {attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down
- * (GGUF block bytes, 4-byte aligned), attn_norm, ffn_norm (float32), cache_k, cache_v (fp16 [n_kv_heads][max_ctx][head_dim])}.
- * x: residual stream, float32 [dim], updated in place.  Workspaces: qkv float32 [(n_heads + 2 n_kv_heads) * head_dim],
- * attn_f16 fp16 [dim], act_f16 fp16 [hidden], partials as for tga_attention_decode, sync: 1280 bytes, zero at first use (uint32
- * arrival counters, error flag at [2]; a launch leaves the counters at zero).  The launch is sized to be resident as a
- * whole and synchronises its workgroups through `sync`; run one such launch at a time per device.  A barrier wait that does not
- * complete within a bounded number of polls sets the uint32 sync[2] to 1 and ends the launch with incomplete results and dirty
- * counters (zero all 1280 bytes before the next launch).
- * Constraints: n_heads * head_dim == dim, head_dim 64 or 128, dim and hidden multiples of 64 and <= 16384. */
-int tga_decode_layers(const void* layer_table, int n_layers, int weight_type, float* x, float* qkv, void* attn_f16, void* act_f16,
-                      float* partials, const void* state, const float* rope_table, void* sync, int dim, int hidden, int n_heads,
-                      int n_kv_heads, int head_dim, int max_ctx, float eps, void* stream);
-
-/* Profiling aid for tga_decode_layers (no counterpart in the reference): buf = device buffer of >= 8 * 11 * n_layers uint64 that
- * later launches fill with 100 MHz wall-clock stamps, [w][block][11], taken by workgroups 73 * w (w < 8) at the phase
- * boundaries of every block; NULL = off. */
-int tga_decode_layers_trace(void* buf);
-
 /* ---- MXFP8 MoE prefill path: extra/gemm/cdna_asm_gemm.py, extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py ---- */
 
 /* quantize_mxfp8 (cdna_asm_gemm.py:149-159): per 32 block along K, e8 = clamp(floor(log2(max(amax, 1e-38))) + 127, 0, 254),
@@ -229,12 +211,29 @@ int tga_moe_combine_rows(const void* z_bf16, const int32_t* dest_row, const floa
 /* grouped_mx_gemm's kernel (moe_gemm.py:31-48, 112-134), same operand list and order as the reference's custom kernel:
  * C (M,N) bf16 = A (M,K) e4m3 . B[e(tile)] (E,N,K) e4m3 ^T with E8M0 1x32 scales x_e8 (M,K/32), w_e8 (E,N,K/32); e(tile) from
  * expert_off (E+1) as Routing.rows_e (moe_routing.py:98-104).  x_si / w_si (the mx_pack copies) are accepted and unused.
- * Requires M % 256 == 0, N % 256 == 0, K % 128 == 0 (moe_gemm.py:120).  Rows at or beyond expert_off[E] are left untouched. */
+ * Requires M % 256 == 0, N % 256 == 0, K % 128 == 0 (moe_gemm.py:120).  Every 256-row tile of C is written: the tiles at or beyond
+ * expert_off[E] are multiplied with expert E - 1, which is what rows_e assigns them (dispatch leaves those rows of A zero, so they come out 0). */
 int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
                            const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
+/* The same product restricted to the routed tiles (rows below expert_off[E]); the rows of C beyond keep their contents.  For callers that
+ * only gather routed rows afterwards (combine, moe_routing.py:128-131): M is the worst-case m_l, of which a fifth is unrouted at benchmark
+ * configuration 5's size.  No packed-scale operands (they are unused). */
+int tga_grouped_mxfp8_gemm_routed(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
+                                  int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
+/* Device symbol for a pre-compiled PROGRAM bound through Tensor.custom_kernel (tinygrad/tensor.py:390-396, extra/gemm/moe_gemm.py:36-48):
+ *   extern "C" __global__ void tga_grouped_mxfp8_gemm_kernel(bf16* C, const fp8* A, const fp8* B, const uint32_t* x_si, const uint32_t* w_si,
+ *                                                            const uint8_t* x_e8, const uint8_t* w_e8, const int32_t* expert_off,
+ *                                                            int M, int N, int K, int E);
+ * one pointer per buffer in the order of the sink's sources, the scalar variables after them (tinygrad/uop/ops.py:1194-1198); launch
+ * 512 threads x (M / 256) * (N / 256) workgroups with no dynamic LDS.  Same arithmetic as tga_grouped_mxfp8_gemm, which launches it through
+ * the runtime API.  The code object is inside libtinygrad_amd.so; tga_kernel_symbol returns its host-side handle for hipLaunchKernel. */
+int tga_kernel_symbol(const char* name, const void** host_function);
+/* HIPProgram.__call__ (tinygrad/runtime/ops_hip.py:36-57): launches a kernel handle from tga_kernel_symbol; grid[3] counts workgroups,
+ * block[3] threads, args is an array of pointers to the argument values in declaration order; no dynamic LDS. */
+int tga_launch_kernel(const void* host_function, const uint32_t* grid, const uint32_t* block, void** args, void* stream);
 /* bias add after a grouped GEMM (examples/mlperf/models/gpt_oss.py:219-224, `+ (onehot @ bias.float()).cast(bf16)`): in place,
- * h[r, :] = bf16(h[r, :] + bf16(bias[e(r), :])) with e(r) the expert of row r's 256-row tile (moe_routing.py:98-104); bias (E, N) float32;
- * rows at or beyond expert_off[E] are left untouched.  M % 256 == 0. */
+ * h[r, :] = bf16(h[r, :] + bf16(bias[e(r), :])) with e(r) the expert of row r's 256-row tile (moe_routing.py:98-104: the tiles at or beyond
+ * expert_off[E] belong to expert E - 1); bias (E, N) float32.  M % 256 == 0. */
 int tga_add_expert_bias(void* h_bf16, const float* bias, const int32_t* expert_off, int64_t M, int64_t N, int n_experts, void* stream);
 /* clamped interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98), bf16 (rows, 2I) -> (rows, I). */
 int tga_swiglu_interleaved(const void* h_bf16, int64_t rows, int two_inter, float limit, float alpha, void* y_bf16, void* stream);

@@ -82,26 +82,64 @@ def to_bf16(x: np.ndarray) -> np.ndarray:
   u = ((u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
   return u.view(np.float32)
 
+def tile_experts(expert_off, M: int) -> np.ndarray:
+  """Routing.rows_e (extra/gemm/moe_routing.py:98-104) per 256-row tile: expert = #(off[:E] <= 256 t) - 1, i.e. the last expert whose offset
+  is <= the tile's first row; the tiles at or beyond off[E] therefore belong to expert E - 1."""
+  off = np.asarray(expert_off).reshape(-1)
+  E = off.shape[0] - 1
+  tr = np.arange(M // 256) * 256
+  return ((tr[:, None] >= off[None, :E]).sum(-1) - 1).astype(np.int32)
+
 def grouped_mx_gemm_ref(x_q, x_e8, w_q, w_e8, expert_off):
   """Semantic definition of grouped_mx_gemm (extra/gemm/moe_gemm.py:112-134) through the reference's non-grouped fallback
   matmul_mx (examples/mlperf/models/gpt_oss.py:64-83): bf16(dequant x) @ bf16(dequant w[e])^T accumulated in float, stored as
-  bf16, where rows [off[e], off[e+1]) belong to expert e.  Returned as float32 holding bf16 values; rows outside any expert's
-  range stay 0 here (the kernel's result there is unspecified padding)."""
+  bf16, where e is the expert of the row's 256-row tile (tile_experts above; the kernel indexes B by tile, moe_gemm.py:36-48).
+  Returned as float32 holding bf16 values."""
   xd = to_bf16(dequant_mxfp8(x_q, x_e8)).astype(np.float64)
   M, N = x_q.shape[0], w_q.shape[1]
   out = np.zeros((M, N), dtype=np.float32)
-  for e in range(w_q.shape[0]):
-    lo, hi = int(expert_off[e]), int(expert_off[e + 1])
-    if hi > lo:
-      wd = to_bf16(dequant_mxfp8(w_q[e], w_e8[e])).astype(np.float64)
-      out[lo:hi] = to_bf16((xd[lo:hi] @ wd.T).astype(np.float32))
+  te = tile_experts(expert_off, M)
+  for e in np.unique(te):
+    rows = np.repeat(te == e, 256)
+    wd = to_bf16(dequant_mxfp8(w_q[e], w_e8[e])).astype(np.float64)
+    out[rows] = to_bf16((xd[rows] @ wd.T).astype(np.float32))
   return out
 
 def add_expert_bias(h_bf16: np.ndarray, bias: np.ndarray, expert_off: np.ndarray) -> np.ndarray:
   """examples/mlperf/models/gpt_oss.py:219-224: h + (onehot(rows_e) @ bias.float()).cast(bf16) as a bf16 tensor add; h holds bf16 values as
-  float32.  Rows beyond expert_off[E] get no bias here (the reference's rows_e maps them to the last expert; they are padding)."""
+  float32.  rows_e gives the tiles at or beyond expert_off[E] to the last expert."""
   out = np.array(h_bf16, dtype=np.float32, copy=True)
-  for e in range(bias.shape[0]):
-    lo, hi = int(expert_off[e]), int(expert_off[e + 1])
-    if hi > lo: out[lo:hi] = to_bf16(out[lo:hi] + to_bf16(bias[e])[None, :])
+  rows_e = np.repeat(tile_experts(expert_off, out.shape[0]), 256)
+  return to_bf16(out + to_bf16(bias)[rows_e])
+
+def swiglu_interleaved(h_bf16: np.ndarray, limit: float = 7.0, alpha: float = 1.702) -> np.ndarray:
+  """swiglu of examples/mlperf/models/gpt_oss.py:94-98 on a bf16 tensor (values held as float32): glu = h[..., ::2].clamp(max=limit),
+  lin = h[..., 1::2].clamp(-limit, limit), (glu * sigmoid(alpha * glu)) * (lin + 1); every elementwise result is a bf16 tensor, so each
+  step rounds to bf16 (the sigmoid counted as one step)."""
+  h = np.asarray(h_bf16, dtype=np.float32)
+  glu, lin = np.minimum(h[..., ::2], np.float32(limit)), np.clip(h[..., 1::2], -np.float32(limit), np.float32(limit))
+  sg = to_bf16(np.float32(1.0) / (np.float32(1.0) + np.exp(-to_bf16(np.float32(alpha) * glu))))
+  return to_bf16(to_bf16(glu * sg) * to_bf16(lin + np.float32(1.0)))
+
+def matmul_mx(x_bf16: np.ndarray, w_q: np.ndarray, w_e8: np.ndarray) -> np.ndarray:
+  """examples/mlperf/models/gpt_oss.py:64-83, the non-ASM branch: quant_dequant_mx(x) @ dequant_weight(w).T -> bf16 (bf16 values as float32)."""
+  xq, xe = quantize_mxfp8(x_bf16)
+  xd = to_bf16(dequant_mxfp8(xq, xe)).astype(np.float64)
+  wd = to_bf16(dequant_mxfp8(w_q, w_e8)).astype(np.float64)
+  return to_bf16((xd @ wd.T).astype(np.float32))
+
+def moe_feed_forward_loop(inp_bf16, logits, k, w_gate_up, w_gate_up_e8, b_gate_up, w_down, w_down_e8, b_down, limit: float = 7.0):
+  """The reference's per-expert loop, examples/mlperf/models/gpt_oss.py:227-238 (the definition the grouped branch :213-226 must agree with):
+  weights = softmax over the logits at or above the k-th largest, out = sum_e bf16(weights[:, e]) * (matmul_mx(swiglu(matmul_mx(inp, gu_e) +
+  b_gu[e]), dn_e) + b_dn[e]), every tensor bf16.  inp (T, D) bf16 values; returns (T, D) bf16 values as float32."""
+  T, E = logits.shape
+  thresh = np.sort(logits, axis=-1)[:, E - k][:, None]
+  masked = np.where(logits >= thresh, logits, -np.inf).astype(np.float32)
+  ex = np.exp(masked - masked.max(-1, keepdims=True)); wts = (ex / ex.sum(-1, keepdims=True)).astype(np.float32)
+  out = None
+  for e in range(E):
+    gate_up = to_bf16(matmul_mx(inp_bf16, w_gate_up[e], w_gate_up_e8[e]) + to_bf16(b_gate_up[e])[None, :])
+    y = to_bf16(matmul_mx(swiglu_interleaved(gate_up, limit), w_down[e], w_down_e8[e]) + to_bf16(b_down[e])[None, :])
+    contrib = to_bf16(to_bf16(wts[:, e:e + 1]) * y)
+    out = contrib if out is None else to_bf16(out + contrib)
   return out

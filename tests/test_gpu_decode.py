@@ -1,51 +1,64 @@
 """Greedy decode of a small llama-architecture model on the GPU vs the numpy restatement of tinygrad/llm/model.py.
 
-The weights are written on the GPU as GGUF blocks; the SAME bytes are read back and given to the oracle.  Bars: final-step logits
-within rel-err 1e-3 of the oracle run with the build's stated activation rounding (fp16 into each linear, fp16 KV), within 5e-3 of
-the pure reference numerics, and the first 32 greedy tokens equal (the oracle's minimum top-2 margin is printed)."""
+The weights are written on the GPU as GGUF blocks; the SAME bytes are read back and given to the oracle, which runs the REFERENCE's
+numerics (float32 activations into fp16-rounded weights, model.py:359, 376; fp16 KV cache as benchmark configuration 3 states).  Bars:
+the first 32 greedy tokens equal the oracle's (its minimum top-2 margin is printed), and the logits of every one of those steps
+within rel-err 1e-3 of the oracle's logits for the same token history."""
 import numpy as np, pytest
 from oracle import llm as ollm, linear as ol
+from decode_helpers import greedy_vs_reference_numerics
 
 pytestmark = pytest.mark.gpu
 
 SMALL = dict(num_blocks=2, dim=256, hidden_dim=512, n_heads=4, n_kv_heads=2, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=500000.0)
 
-def _build(gpu, cfg, max_context, seed=1003, fused=True, linear_type=None):
+def _build(gpu, cfg, max_context, seed=1003, linear_type=None):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state
   from tinygrad_amd import runtime as rt
   c = TransformerConfig(max_context=max_context, **cfg)
   sd = synth_state(c, seed=seed, linear_type=rt.Q4_0 if linear_type is None else linear_type)
   gpu.synchronize()
   host = {k: (b.numpy(), t, shp) for k, (b, t, shp) in sd.items()}
-  m = Transformer(c, sd, max_new=64, fused=fused)
-  assert (m.layer_table is not None) == fused
-  return m, host
+  return Transformer(c, sd, max_new=64), host
 
-@pytest.mark.parametrize("fused", [True, False], ids=["one-launch", "per-op"])
-def test_small_model_logits_and_tokens(gpu, fused):
-  model, host = _build(gpu, SMALL, 128, fused=fused)
+def test_small_model_logits_and_tokens(gpu):
+  model, host = _build(gpu, SMALL, 128)
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=70)]      # spans two 64-position attention splits
-  got = list(model.generate(prompt, 32, use_graph=True))
-  lg_gpu = model.logits()
-  o16 = ollm.Model(SMALL, host, 128, act_round_f16=True)
-  ref_tokens, margins = o16.generate(prompt, 32)
-  print(f"oracle min top-2 logit margin over 32 steps: {min(margins):.4f} (logit rms {np.sqrt(np.mean(lg_gpu ** 2)):.4f})")
-  assert got == ref_tokens
-  # logits of the last step: replay the oracle's last forward
-  o16b = ollm.Model(SMALL, host, 128, act_round_f16=True)
-  pos = 0
-  for t in prompt[:-1]: o16b.forward(t, pos); pos += 1
-  cur = prompt[-1]
-  for _ in range(32): lg = o16b.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
-  assert ol.rel_err(lg_gpu, lg) <= 1e-3
-  # pure reference numerics (fp32 activations into fp16 weights): the fp16 activation rounding stays a small perturbation
-  oref = ollm.Model(SMALL, host, 128, act_round_f16=False)
-  pos = 0
-  for t in prompt[:-1]: oref.forward(t, pos); pos += 1
-  cur = prompt[-1]
-  for tk in got: lgr = oref.forward(cur, pos); pos += 1; cur = tk
-  assert ol.rel_err(lg_gpu, lgr) <= 5e-3
+  oref = ollm.Model(SMALL, host, 128, act_round_f16=False)                      # the reference's numerics: nothing of the build's rounding
+  got, ref, worst, margin, rms = greedy_vs_reference_numerics(model, oref, prompt, 32)
+  print(f"oracle (reference numerics) min top-2 logit margin over 32 steps: {margin:.4f} (logit rms {rms:.4f}); worst logits rel-err {worst:.2e}")
+  assert got == ref
+  assert worst <= 1e-3
+
+def test_context_and_token_guards(gpu):
+  """The sequence ends at max_context like the reference's generate loop (tinygrad/llm/model.py:475), ids outside the vocabulary are refused on
+  the host, and the kernels themselves refuse (flag, no access) a position or token outside their tables."""
+  model, _ = _build(gpu, SMALL, 64, seed=3)
+  out = list(model.generate([1, 2, 3], 1000))
+  assert len(out) == 61                                                          # 3 prompt tokens + 61 generated = max_context
+  model.decode_step()                                                            # the last cache position (63) can still be processed ...
+  with pytest.raises(RuntimeError, match="context full"): model.decode_step()    # ... position 64 does not exist
+  with pytest.raises(ValueError): model.reset([SMALL["vocab_size"]])
+  with pytest.raises(ValueError): model.reset([-1])
+  with pytest.raises(ValueError): model.reset(list(range(64)))
+  # device-side refusal: a state record whose position / token lie outside the tables
+  model.reset([1, 2])
+  st = model.s.state.numpy(); st[0] = 64; model.s.state.copyin(st)             # pos == max_context
+  before = model.blk[0].cache_k.numpy().copy()
+  model._step(True); model.stream.synchronize()
+  np.testing.assert_array_equal(model.blk[0].cache_k.numpy(), before)
+  with pytest.raises(RuntimeError, match="position beyond max_context"): model.check_state()
+  model.reset([1, 2])
+  st = model.s.state.numpy(); st[1] = 1 << 30; model.s.state.copyin(st)        # token id far outside the table
+  model._step(True); model.stream.synchronize()
+  with pytest.raises(RuntimeError, match="token id outside the vocabulary"): model.check_state()
+  # NaN logits: the argmax stays inside the row (index 0), never 2^31 - 1
+  lg = np.full(SMALL["vocab_size"], np.nan, np.float32)
+  stb = gpu.Buffer.from_numpy(np.zeros(16, np.int32)); outt = gpu.Buffer((4,), np.int32).zero_(); pr = gpu.Buffer((8,), np.int32).zero_()
+  lgb, sv, si = gpu.Buffer.from_numpy(lg), gpu.Buffer((256,), np.float32), gpu.Buffer((256,), np.int32)
+  gpu.check(gpu.lib().tga_argmax_step(lgb.ptr, lg.size, sv.ptr, si.ptr, stb.ptr, pr.ptr, outt.ptr, 4, None))
+  assert outt.numpy()[0] == 0
 
 def test_graph_replay_equals_eager(gpu):
   model, _ = _build(gpu, SMALL, 128, seed=77)
@@ -56,29 +69,19 @@ def test_graph_replay_equals_eager(gpu):
   assert a == b
   np.testing.assert_array_equal(la, model.logits())
 
-# shapes that take the other template paths of the one-launch kernel: head_dim 128, K split over four waves (K > 4096), Q8_0
+# wider shapes: head_dim 128, K split over four waves (K > 4096), Q8_0
 WIDE = dict(num_blocks=2, dim=1024, hidden_dim=4608, n_heads=8, n_kv_heads=1, norm_eps=1e-5, vocab_size=512, head_dim=128, rope_theta=10000.0)
 WIDE_D = dict(num_blocks=2, dim=4352, hidden_dim=256, n_heads=34, n_kv_heads=17, norm_eps=1e-5, vocab_size=256, head_dim=128, rope_theta=10000.0)
 
 @pytest.mark.parametrize("cfg,ltype", [(WIDE, "Q4_0"), (WIDE, "Q8_0"), (WIDE_D, "Q4_0"), (SMALL, "Q8_0")], ids=["wide-hidden-q4", "wide-hidden-q8", "wide-dim-q4", "small-q8"])
-def test_one_launch_blocks_equal_per_op_path(gpu, cfg, ltype):
-  """tga_decode_layers against the per-op launches on the same weights: same greedy tokens, logits within 1e-3 (both paths
-  round activations to fp16 at the same points; fp32 summation order differs and flips a few of those roundings), KV cache contents equal to fp16 rounding of nearly equal values."""
+def test_wider_models_vs_reference_numerics(gpu, cfg, ltype):
   from tinygrad_amd import runtime as rt
-  lt = getattr(rt, ltype)
-  a, _ = _build(gpu, cfg, 192, seed=11, fused=True, linear_type=lt)
-  b, _ = _build(gpu, cfg, 192, seed=11, fused=False, linear_type=lt)
+  model, host = _build(gpu, cfg, 192, seed=11, linear_type=getattr(rt, ltype))
   rng = np.random.default_rng(3)
   prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=67)]
-  ta = list(a.generate(prompt, 12, use_graph=True))
-  tb = list(b.generate(prompt, 12, use_graph=True))
-  la, lb = a.logits(), b.logits()
-  assert np.isfinite(la).all()
-  assert ta == tb
-  assert ol.rel_err(la, lb) <= 1e-3
-  ka, kb = a.blk[1].cache_k.numpy().astype(np.float32), b.blk[1].cache_k.numpy().astype(np.float32)
-  assert ol.rel_err(ka[:, :78], kb[:, :78]) <= 2e-3
-  assert not a.s.sync.numpy().any()                                # barrier counters back at zero, no error flag
+  got, ref, worst, margin, rms = greedy_vs_reference_numerics(model, ollm.Model(cfg, host, 192, act_round_f16=False), prompt, 12)
+  print(f"min top-2 margin {margin:.4f}, logit rms {rms:.4f}, worst logits rel-err {worst:.2e}")
+  assert got == ref and worst <= 1e-3
 
 @pytest.mark.parametrize("H,KV,hd,normed", [(8, 2, 128, 0), (4, 4, 64, 1), (12, 2, 128, 1), (4, 2, 256, 0), (16, 16, 128, 1), (16, 8, 128, 2), (6, 2, 64, 2)],
                          ids=["gqa4-hd128", "mha-hd64-qknorm", "gqa6-hd128-qknorm", "gqa2-hd256", "mha16-hd128-qknorm", "gqa2-hd128-headnorm", "gqa3-hd64-headnorm"])
@@ -89,7 +92,7 @@ def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
   rng = np.random.default_rng(5 + H)
   rope = precompute_freqs_cis(hd, ctx, 10000.0)
   ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
-  part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2) + KV,), np.float32).zero_()
+  part = gpu.Buffer((H * ((ctx + 63) // 64) * (hd + 2),), np.float32).zero_()
   ropeb = gpu.Buffer.from_numpy(rope)
   out = gpu.Buffer((H * hd,), np.float32)
   # normed: 0 none, 1 full-width q/k norm (weights over all heads), 2 per-head norm (weights of head_dim values)
@@ -117,7 +120,6 @@ def test_attention_decode_kernel_vs_numpy(gpu, H, KV, hd, normed):
       ref = np.einsum("ht,htd->hd", p, V).reshape(-1)
       assert ol.rel_err(out.numpy(), ref) <= 1e-4, pos
   assert ck.numpy().tobytes() == rk.tobytes() or ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
-  assert not part.numpy()[-KV:].view(np.int32).any()                 # arrival counters back at zero
 
 def test_rmsnorm_argmax_embed(gpu):
   rng = np.random.default_rng(9)
@@ -135,27 +137,6 @@ def test_rmsnorm_argmax_embed(gpu):
   lgb, sv, si = gpu.Buffer.from_numpy(lg), gpu.Buffer((256,), np.float32), gpu.Buffer((256,), np.int32)
   gpu.check(gpu.lib().tga_argmax_step(lgb.ptr, lg.size, sv.ptr, si.ptr, stb.ptr, pr.ptr, outt.ptr, 4, None))
   assert outt.numpy()[0] == 777 and list(stb.numpy()[:3]) == [1, 777, 1]
-
-def test_decode_layers_argument_checks_and_trace(gpu):
-  """tga_decode_layers rejects shapes outside its contract with a message (no launch), and the phase trace fills its buffer."""
-  from tinygrad_amd import runtime as rt
-  L = rt.lib()
-  m, _ = _build(gpu, SMALL, 128, seed=5)
-  s, c = m.s, m.config
-  call = lambda **kw: L.tga_decode_layers(m.layer_table.ptr, kw.get("n_layers", c.num_blocks), kw.get("wtype", m.layer_type), s.x.ptr, s.qkv.ptr, s.attn.ptr, s.act.ptr,
-                                          s.attn_part.ptr, s.state.ptr, s.rope.ptr, s.sync.ptr, kw.get("dim", c.dim), kw.get("hidden", c.hidden_dim), c.n_heads, c.n_kv_heads,
-                                          kw.get("hd", c.head_dim), c.max_context, c.norm_eps, m.stream.handle)
-  for bad in (dict(wtype=rt.Q6_K), dict(hd=32), dict(dim=c.dim + 64), dict(hidden=c.hidden_dim + 32), dict(n_layers=0)):
-    assert call(**bad) != 0
-    assert b"tga_decode_layers" in L.tga_last_error()
-  tb = rt.Buffer((8 * 11 * c.num_blocks,), np.uint64).zero_()
-  rt.check(L.tga_decode_layers_trace(tb.ptr))
-  try:
-    out = list(m.generate([1, 2, 3], 2, use_graph=False))
-  finally:
-    rt.check(L.tga_decode_layers_trace(None))
-  t = tb.numpy().reshape(8, c.num_blocks, 11)[0].astype(np.int64)
-  assert len(out) == 2 and (t > 0).all() and (np.diff(t.reshape(-1)) >= 0).all()      # workgroup 0's stamps are in program order
 
 def test_copy_kernel_and_mfma_peak_run(gpu):
   from tinygrad_amd import runtime as rt

@@ -66,11 +66,11 @@ def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
   cfg, weights, _ = ogguf.from_gguf_weights(raw)
   prompt = [1, 77, 300, 9, 410, 3]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)         # weights already prepared (fp16-rounded, permuted)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)         # weights already prepared (fp16-rounded, permuted)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
@@ -84,15 +84,14 @@ def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path, legacy):
   from tinygrad_amd.llm import Transformer
   path, raw = _make_file(tmp_path, False, kquant=legacy == 0, legacy=legacy == 1, expand=legacy == 2, codebook=legacy == 3)
   model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
-  assert model.layer_table is None                                     # K-quants take the per-op launches
   cfg, weights, _ = ogguf.from_gguf_weights(raw)
   prompt = [3, 200, 17, 450, 8]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
@@ -121,15 +120,15 @@ def test_from_gguf_qwen3_shape_per_head_qk_norm(gpu, tmp_path):
   path = tmp_path / "qwen3.gguf"
   raw = gguf_write(path, kvs, tensors)
   model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
-  assert model.config.qk_norm == hd == model.config.head_dim and model.layer_table is None
+  assert model.config.qk_norm == hd == model.config.head_dim
   cfg, weights, _ = ogguf.from_gguf_weights(raw)
   prompt = [9, 100, 321, 5]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
@@ -167,17 +166,17 @@ def test_from_gguf_qwen2_shape_qkv_bias(gpu, tmp_path):
   cfg, weights, _ = ogguf.from_gguf_weights(raw)
   prompt = [9, 100, 321, 5]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
   # the biases matter: without them the oracle's logits for the same token stream are far away
-  o3 = ollm.Model(cfg, {k: v for k, v in weights.items() if not k.endswith(".bias")}, 64, w_round_f16=False, act_round_f16=True)
+  o3 = ollm.Model(cfg, {k: v for k, v in weights.items() if not k.endswith(".bias")}, 64, w_round_f16=False, act_round_f16=False)
   for pos, t in enumerate(prompt + ref[:-1]): lg3 = o3.forward(t, pos)
   assert ol.rel_err(lg3, lg) > 0.05
 
@@ -219,11 +218,11 @@ def test_from_gguf_qwen3moe_shape_expert_stacks(gpu, tmp_path):
   assert cfg["norm_topk_prob"] and weights["blk.0.ffn_gate_exps.weight"].shape == (E, hidden, dim)
   prompt = [9, 100, 321, 5, 77]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
@@ -259,16 +258,16 @@ def test_from_gguf_partial_rotary(gpu, tmp_path):
   assert cfg["rope_dim"] == rd
   prompt = [9, 100, 321, 5, 44, 12, 400]
   got = list(model.generate(prompt, 12))
-  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True)
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
   ref, margins = o.generate(prompt, 12)
   print(f"min top-2 margin {min(margins):.4f}")
   assert got == ref
-  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=True); pos = 0
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
   for t in prompt[:-1]: o2.forward(t, pos); pos += 1
   cur = prompt[-1]
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
   # the rotation width matters: the oracle with full-width rotation gives other logits for the same token stream
-  o3 = ollm.Model(dict(cfg, rope_dim=hd), weights, 64, w_round_f16=False, act_round_f16=True)
+  o3 = ollm.Model(dict(cfg, rope_dim=hd), weights, 64, w_round_f16=False, act_round_f16=False)
   for pos, t in enumerate(prompt + ref[:-1]): lg3 = o3.forward(t, pos)
   assert ol.rel_err(lg3, lg) > 0.01

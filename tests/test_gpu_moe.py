@@ -151,14 +151,8 @@ def test_small_olmoe_decode(gpu):
   model = Transformer(c, sd, max_new=64)
   rng = np.random.default_rng(1004)
   prompt = [int(t) for t in rng.integers(0, 512, size=20)]
-  got = list(model.generate(prompt, 16))
-  lg_gpu = model.logits()
-  o = ollm.Model(SMALL_MOE, host, 128, act_round_f16=True)
-  ref, margins = o.generate(prompt, 16)
-  print(f"oracle min top-2 margin {min(margins):.4f}")
+  from decode_helpers import greedy_vs_reference_numerics
+  got, ref, worst, margin, rms = greedy_vs_reference_numerics(model, ollm.Model(SMALL_MOE, host, 128, act_round_f16=False), prompt, 32)
+  print(f"oracle (reference numerics) min top-2 margin over 32 steps {margin:.4f} (logit rms {rms:.4f}); worst logits rel-err {worst:.2e}")
   assert got == ref
-  o2 = ollm.Model(SMALL_MOE, host, 128, act_round_f16=True); pos = 0
-  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
-  cur = prompt[-1]
-  for _ in range(16): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
-  assert ol.rel_err(lg_gpu, lg) <= 1e-3
+  assert worst <= 1e-3

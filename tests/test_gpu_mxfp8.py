@@ -97,7 +97,7 @@ def test_grouped_mxfp8_gemm(gpu, E, N, K, rows):
   from tinygrad_amd import moe
   rng = np.random.default_rng(N + K)
   off = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
-  M = int(off[-1]) + 256                                                          # one unrouted tile at the end
+  M = int(off[-1]) + 256                                                          # one tile beyond expert_off[E]: expert E - 1's by rows_e (moe_routing.py:98-104)
   x = (rng.standard_normal((M, K)) * 0.5).astype(np.float32)
   w = (rng.standard_normal((E, N, K)) * 0.5).astype(np.float32)
   xq, xe8 = omx.quantize_mxfp8(x); wq, we8 = omx.quantize_mxfp8(w)
@@ -106,15 +106,32 @@ def test_grouped_mxfp8_gemm(gpu, E, N, K, rows):
   gpu.check(gpu.lib().tga_grouped_mxfp8_gemm(C.ptr, bufs[0].ptr, bufs[1].ptr, None, None, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr, M, N, K, E, None))
   got = moe.from_bf16_bits(C.numpy())
   ref = omx.grouped_mx_gemm_ref(xq, xe8, wq, we8, off)
-  used = int(off[-1])
+  used = M
   err_mx = np.abs(got[:used] - ref[:used]).mean() / np.abs(ref[:used]).mean()
   assert err_mx < 1e-2, err_mx                                                    # the reference's bar
   # tighter: bf16 output of a float32 accumulation of exactly representable products: within one bf16 ulp of the oracle
   np.testing.assert_allclose(got[:used], ref[:used], rtol=2 ** -7, atol=1e-3 * np.abs(ref).max())
-  assert (got[used:] == 0).all()                                                  # unrouted tile untouched
+  # the routed-only variant writes the same values below expert_off[E] and nothing beyond
+  C2 = gpu.Buffer((M, N), np.uint16).zero_()
+  gpu.check(gpu.lib().tga_grouped_mxfp8_gemm_routed(C2.ptr, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, bufs[4].ptr, M, N, K, E, None))
+  np.testing.assert_array_equal(C2.numpy()[:off[-1]], C.numpy()[:off[-1]]); assert (C2.numpy()[off[-1]:] == 0).all()
+  # the pointer-argument kernel a Tensor.custom_kernel PROGRAM would bind (arguments in sink order, then the scalars), launched like
+  # HIPProgram.__call__ does: 512 threads x (M / 256) (N / 256) workgroups
+  import ctypes
+  fn = ctypes.c_void_p()
+  gpu.check(gpu.lib().tga_kernel_symbol(b"tga_grouped_mxfp8_gemm_kernel", ctypes.byref(fn)))
+  C3 = gpu.Buffer((M, N), np.uint16).zero_()
+  vals = [ctypes.c_void_p(C3.ptr), ctypes.c_void_p(bufs[0].ptr), ctypes.c_void_p(bufs[1].ptr), ctypes.c_void_p(None), ctypes.c_void_p(None), ctypes.c_void_p(bufs[2].ptr),
+          ctypes.c_void_p(bufs[3].ptr), ctypes.c_void_p(bufs[4].ptr), ctypes.c_int(M), ctypes.c_int(N), ctypes.c_int(K), ctypes.c_int(E)]
+  args = (ctypes.c_void_p * len(vals))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in vals])
+  grid, block = (ctypes.c_uint32 * 3)((M // 256) * (N // 256), 1, 1), (ctypes.c_uint32 * 3)(512, 1, 1)
+  gpu.check(gpu.lib().tga_launch_kernel(fn, grid, block, args, None)); gpu.synchronize()
+  np.testing.assert_array_equal(C3.numpy(), C.numpy())
+  assert gpu.lib().tga_kernel_symbol(b"no_such_kernel", ctypes.byref(fn)) != 0
   # against the unquantized product: the reference's second bar (< 6e-2)
   full = np.zeros_like(ref)
   for e in range(E): full[off[e]:off[e + 1]] = x[off[e]:off[e + 1]] @ w[e].T
+  full[off[-1]:] = x[off[-1]:] @ w[E - 1].T
   assert np.abs(got[:used] - full[:used]).mean() / np.abs(full[:used]).mean() < 6e-2
 
 def test_dense_mx_gemm_and_expert_bias(gpu):
@@ -131,7 +148,7 @@ def test_dense_mx_gemm_and_expert_bias(gpu):
   ref = omx.grouped_mx_gemm_ref(xq, xe8, wq[None], we8[None], np.array([0, M], np.int32))
   got = moe.from_bf16_bits(out.numpy())
   np.testing.assert_allclose(got, ref, rtol=2 ** -7, atol=1e-3 * np.abs(ref).max())
-  # bias by expert on three experts' tiles, the last tile unrouted
+  # bias by expert on three experts' tiles; the last tile lies beyond expert_off[E] and takes the last expert's bias (rows_e)
   E = 3
   off = np.array([0, 256, 256, 512], dtype=np.int32)                 # expert 1 owns no rows
   h = moe.to_bf16_bits(rng.standard_normal((768, N)).astype(np.float32))
@@ -140,4 +157,42 @@ def test_dense_mx_gemm_and_expert_bias(gpu):
   moe.add_expert_bias(hb, gpu.Buffer.from_numpy(bias), gpu.Buffer.from_numpy(off))
   exp = omx.add_expert_bias(moe.from_bf16_bits(h), bias, off)
   np.testing.assert_array_equal(hb.numpy(), moe.to_bf16_bits(exp))
-  assert (hb.numpy()[512:] == h[512:]).all()                         # rows beyond the routed range untouched
+  assert (hb.numpy()[512:] != h[512:]).any()                         # rows beyond expert_off[E] got expert E - 1's bias
+
+def test_swiglu_interleaved(gpu):
+  """The clamped interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98) on bf16 rows, bit for bit against the
+  oracle's bf16 chain except where the device's exp differs by an ulp before the bf16 rounding (at most one bf16 ulp, a handful of elements)."""
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(21)
+  h = moe.to_bf16_bits((rng.standard_normal((300, 512)) * 4).astype(np.float32))
+  h[0, :8] = moe.to_bf16_bits(np.array([100, 100, -100, -100, 7, -7, 0, 0], np.float32))
+  y = moe.swiglu(gpu.Buffer.from_numpy(h)).numpy()
+  ref = omx.swiglu_interleaved(moe.from_bf16_bits(h))
+  got = moe.from_bf16_bits(y)
+  assert y.shape == (300, 256)
+  np.testing.assert_allclose(got, ref, rtol=2 ** -7, atol=1e-30)
+  assert (moe.to_bf16_bits(ref) == y).mean() > 0.99
+
+def test_moe_feed_forward_composition(gpu):
+  """moe.moe_feed_forward (route -> dispatch -> grouped GEMM + bias -> SwiGLU -> grouped GEMM + bias -> combine, gpt_oss.py:213-226) against the
+  reference's per-expert loop (gpt_oss.py:227-238) restated in the oracle; the reference has no test of its own for either branch, the
+  loop is the definition (oracle pinned in tests/test_oracle_pins.py).  Bar: the reference's MXFP8 GEMM bar (mean rel-err < 1e-2), since the two
+  branches round to bf16 at different points (the loop weighs and sums bf16 contributions expert by expert, the grouped branch weighs rows)."""
+  from tinygrad_amd import moe
+  rng = np.random.default_rng(33)
+  T, D, I, E, k = 96, 256, 256, 6, 2
+  inp = moe.to_bf16_bits(rng.standard_normal((T, D)).astype(np.float32))
+  logits = rng.standard_normal((T, E)).astype(np.float32); logits[:, 4] = -30.0       # expert 4 is never selected: an empty range
+  wgu, wdn = (rng.standard_normal((E, 2 * I, D)) * D ** -0.5).astype(np.float32), (rng.standard_normal((E, D, I)) * I ** -0.5).astype(np.float32)
+  bgu, bdn = (rng.standard_normal((E, 2 * I)) * 0.1).astype(np.float32), (rng.standard_normal((E, D)) * 0.1).astype(np.float32)
+  (gq, ge), (dq, de) = omx.quantize_mxfp8(wgu), omx.quantize_mxfp8(wdn)
+  B = gpu.Buffer.from_numpy
+  ref = omx.moe_feed_forward_loop(moe.from_bf16_bits(inp), logits, k, gq, ge, bgu, dq, de, bdn)
+  for routed_only in (True, False):
+    out = moe.moe_feed_forward(B(inp), B(logits), k, (B(gq), B(ge)), B(bgu), (B(dq), B(de)), B(bdn), routed_only=routed_only)
+    got = moe.from_bf16_bits(out.numpy())
+    assert got.shape == (T, D) and np.isfinite(got).all()
+    err = np.abs(got - ref).mean() / np.abs(ref).mean()
+    print(f"moe_feed_forward vs per-expert loop (routed_only={routed_only}): mean rel-err {err:.2e}")
+    assert err < 1e-2
+    np.testing.assert_allclose(got, ref, rtol=0.05, atol=0.02 * np.abs(ref).max())

@@ -58,20 +58,21 @@ def _bf16_rne(v: float) -> float:
   return struct.unpack("<f", struct.pack("<I", u))[0]
 
 def test_grouped_mx_gemm_ref_against_exact_brute_force():
-  """Two 256-row tiles, three experts of which the middle one is empty; every output element recomputed as an exact rational sum over k of
+  """Three 256-row tiles, three experts of which the middle one is empty and the last tile lies beyond expert_off[E] (rows_e gives it to the
+  last expert, moe_routing.py:98-104); every output element recomputed as an exact rational sum over k of
   e4m3(x) 2^(ex-127) e4m3(w[e]) 2^(ew-127) with e chosen by the row's offset range, then rounded float32 -> bf16."""
   rng = np.random.default_rng(7)
-  M, N, K, E = 512, 3, 64, 3
+  M, N, K, E = 768, 3, 64, 3
   off = np.array([0, 256, 256, 512], dtype=np.int32)
   codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)          # every finite E4M3 code
   xq, wq = rng.choice(codes, (M, K)), rng.choice(codes, (E, N, K))
   xe, we = rng.integers(120, 131, (M, K // 32), dtype=np.uint8), rng.integers(120, 131, (E, N, K // 32), dtype=np.uint8)
   got = omx.grouped_mx_gemm_ref(xq, xe, wq, we, off)
   val = [_e4m3_value(c) for c in range(256)]
-  rows = list(range(0, 8)) + [255, 256, 257, 300, 511]                                       # both sides of the expert boundary
+  rows = list(range(0, 8)) + [255, 256, 257, 300, 511, 512, 700, 767]                        # both sides of the expert boundary, and the tile beyond off[E]
   exact, ulp_off = 0, 0
   for r in rows:
-    e = 0 if r < 256 else 2
+    e = 0 if r < 256 else 2                                                                  # (row 512 and beyond: off[E] = 512, so the last expert)
     for n in range(N):
       acc = Fraction(0)
       for k in range(K):
@@ -85,6 +86,49 @@ def test_grouped_mx_gemm_ref_against_exact_brute_force():
   # a transposed or mis-scaled operand is far outside a bf16 ulp: the check above has teeth
   bad = omx.grouped_mx_gemm_ref(xq, xe, wq[::-1], we[::-1], off)
   assert np.abs(bad[:8] - got[:8]).max() > 2.0 ** -6 * np.abs(got[:8]).max()
+
+def test_tile_experts_bias_and_swiglu_closed_forms():
+  off = np.array([0, 256, 256, 512], dtype=np.int32)
+  np.testing.assert_array_equal(omx.tile_experts(off, 1024), [0, 2, 2, 2])                   # empty expert 1 owns nothing; tiles beyond off[E] -> E - 1
+  h = np.zeros((1024, 2), np.float32); bias = np.array([[1.0, 2.0], [10.0, 20.0], [100.0, 200.0]], np.float32)
+  hb = omx.add_expert_bias(h, bias, off)
+  np.testing.assert_array_equal(hb[[0, 255, 256, 511, 512, 1023]], [[1, 2], [1, 2], [100, 200], [100, 200], [100, 200], [100, 200]])
+  # swiglu: interleaved (glu, linear) pairs, glu clamped above only, linear on both sides; float64 closed form within bf16 rounding of the chain
+  rng = np.random.default_rng(5)
+  hh = omx.to_bf16((rng.standard_normal((7, 16)) * 5).astype(np.float32))
+  glu, lin = np.minimum(hh[:, ::2].astype(np.float64), 7.0), np.clip(hh[:, 1::2].astype(np.float64), -7.0, 7.0)
+  want = glu / (1 + np.exp(-1.702 * glu)) * (lin + 1)
+  # (rounding alpha * glu to bf16 moves the sigmoid's argument by up to |alpha glu| 2^-9 <= 2.3 %, the three products add 2^-9 each)
+  np.testing.assert_allclose(omx.swiglu_interleaved(hh), want, rtol=0.035, atol=1e-6)
+  big = np.array([[100.0, 100.0, -100.0, -100.0]], np.float32)
+  np.testing.assert_allclose(omx.swiglu_interleaved(big), [[7.0 * 8.0, -0.0]], atol=1e-30)   # glu 100 -> 7, lin 100 -> 7 (+1); glu -100 * sigmoid(-170) = -0
+
+def test_moe_feed_forward_loop_against_float64_closed_form():
+  """The per-expert loop (gpt_oss.py:227-238) on operands that MXFP8 holds exactly: the result must be the float64 value of
+  sum over the top-k experts of softmax_topk(logits)_e * (swiglu(x Wgu_e^T + bgu_e) Wdn_e^T + bdn_e), up to the bf16 roundings of the chain."""
+  rng = np.random.default_rng(9)
+  T, D, I, E, k = 5, 32, 32, 4, 2
+  vals = np.array([0, 0.5, 1, 1.5, 2, -0.5, -1, -1.5, -2], np.float32)
+  x = rng.choice(vals, (T, D)); wgu = rng.choice(vals, (E, 2 * I, D)) * 0.25; wdn = rng.choice(vals, (E, D, I)) * 0.25
+  bgu = rng.choice(vals, (E, 2 * I)); bdn = rng.choice(vals, (E, D))
+  logits = rng.standard_normal((T, E)).astype(np.float32)
+  (gq, ge), (dq, de) = omx.quantize_mxfp8(wgu), omx.quantize_mxfp8(wdn)
+  np.testing.assert_array_equal(omx.dequant_mxfp8(gq, ge), wgu)                               # exactly representable: no quantization error in the operands
+  got = omx.moe_feed_forward_loop(x, logits, k, gq, ge, bgu, dq, de, bdn)
+  want = np.zeros((T, D))
+  for t in range(T):
+    top = np.argsort(-logits[t])[:k]
+    w = np.exp(logits[t, top] - logits[t, top].max()); w /= w.sum()
+    for wi, e in zip(w, top):
+      gu = wgu[e].astype(np.float64) @ x[t] + bgu[e]
+      glu, lin = np.minimum(gu[::2], 7.0), np.clip(gu[1::2], -7.0, 7.0)
+      y = glu / (1 + np.exp(-1.702 * glu)) * (lin + 1)
+      yq = omx.dequant_mxfp8(*omx.quantize_mxfp8(omx.to_bf16(y.astype(np.float32))[None, :]))[0]      # the activation of the second GEMM is MXFP8 too
+      want[t] += wi * (wdn[e].astype(np.float64) @ yq + bdn[e])
+  assert np.abs(got - want).max() <= 0.03 * np.abs(want).max()
+  # teeth: using the wrong expert's down projection is far outside that bound
+  wrong = omx.moe_feed_forward_loop(x, logits, k, gq, ge, bgu, dq[::-1], de[::-1], bdn)
+  assert np.abs(wrong - want).max() > 0.2 * np.abs(want).max()
 
 # ------------------------------------------------------------------------------------------------ llm.Model.forward wiring
 def _model(H=4, KV=2, hd=8, dim=32, hidden=32, vocab=16, blocks=1, seed=0, **over):

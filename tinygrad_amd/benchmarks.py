@@ -180,13 +180,36 @@ def config5():
                 "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
   return res
 
+def traffic(steps: int = 4):
+  """Workload for the HBM-traffic counter runs (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE, one run each):
+
+      rocprofv3 --pmc FETCH_SIZE --output-format csv -d out -o t -- python3 -m tinygrad_amd.benchmarks --traffic
+
+  one 1 GiB plain copy kernel (the yardstick: it must read 1 GiB and write 1 GiB), then a few eager decode steps of the benchmark model
+  after a two-token prompt.  The dequant-GEMV launches do not depend on the context length, so the KV cache is not prefilled: a counter run
+  intercepts every dispatch, and a 1024-token prefill would be 200 000 of them."""
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
+  n = 1 << 30
+  a, b = Buffer((n,), np.uint8).zero_(), Buffer((n,), np.uint8)
+  rt.check(rt.lib().tga_copy_kernel(b.ptr, a.ptr, n, None)); rt.synchronize()
+  c = TransformerConfig(max_context=64, **LLAMA3_8B)
+  model = Transformer(c, synth_state(c, seed=1003), max_new=16)
+  model.prefill([17, 4242], use_graph=False)
+  for _ in range(steps): model.decode_step(use_graph=False)
+  model.check_state()
+  return [{"traffic_probe": "done", "copy_bytes": n, "decode_steps": steps}]
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix")
   ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
+  ap.add_argument("--traffic", action="store_true", help="only the workload of the HBM-traffic counter runs (see traffic())")
   args = ap.parse_args()
   rt.init(0)
   print(json.dumps({"device": rt.device_name()}), flush=True)
+  if args.traffic:
+    for row in traffic(): print(json.dumps(row), flush=True)
+    return
   for cfg in args.config:
     fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7}[cfg]
     for row in (fn(use_graph=not args.no_graph) if cfg == 4 else fn()): print(json.dumps(row), flush=True)

@@ -21,8 +21,12 @@ __device__ __forceinline__ void embed_row_blocks(const uint8_t* __restrict__ tab
     out[e] = o[0]; out[e + 1] = o[1]; out[e + 2] = o[2]; out[e + 3] = o[3];
   }
 }
-__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, const DecodeState* st, float* __restrict__ out) {
-  const int tok = st->token;
+__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, DecodeState* st, float* __restrict__ out) {
+  int tok = st->token;
+  if (tok < 0 || (st->vocab > 0 && tok >= st->vocab)) {         // a token id outside the table (e.g. argmax over NaN logits): row 0 is read instead, the host sees the flag
+    if (threadIdx.x == 0) atomicOr(&st->error, 1);
+    tok = 0;
+  }
   switch (ggml_type) {
     case GGML_Q4_0: embed_row_blocks<GGML_Q4_0>(table, dim, tok, out); break;
     case GGML_Q8_0: embed_row_blocks<GGML_Q8_0>(table, dim, tok, out); break;
@@ -89,7 +93,7 @@ struct AttnArgs {
   const float* q; const float* k; const float* v;     // this token's projections: [n_heads*hd], [n_kv*hd], [n_kv*hd]
   _Float16* cache_k; _Float16* cache_v;                // [n_kv][max_ctx][hd]
   float* part;                                         // [n_heads][nsplit][hd + 2]
-  const DecodeState* st;
+  DecodeState* st;
   int n_heads, n_kv, hd, max_ctx, nsplit;
   const float* rope;                                   // [max_ctx][hd]: cos(pos * f_i) for i < hd/2, then sin(pos * f_i)
   float scale;
@@ -205,6 +209,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
   }
   // ---- the position, and the one load that needs it
   const int pos = a.st->pos;
+  if (pos >= a.max_ctx || pos < 0) {                    // no cache row and no rotation row for this position: nothing is read or written, the host sees the flag
+    if (kvh == 0 && split == 0 && tid == 0) atomicOr(&a.st->error, 2);
+    return;
+  }
   if (split * 64 > pos) return;                         // nothing cached in this split yet
   const float kc = a.rope[(size_t)pos * HD + ki], ksn = a.rope[(size_t)pos * HD + half + ki];
   float qc[QPL], qsn[QPL];
@@ -371,6 +379,7 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
 #pragma unroll
   for (int j = 0; j < FB; j++) v[j] = ph[(size_t)(j < nsp ? j : nsp - 1) * (HD + 2) + d];
   const int pos = a.st->pos, ns = (pos >> 6) + 1;
+  if (pos >= a.max_ctx || pos < 0) return;              // refused by the split launch (state.error): the output row keeps its contents
   float m = -INFINITY, l = 0.f;
   if (nsp <= HD) {
     m = wave_max(d < ns ? mv : -INFINITY);
@@ -423,7 +432,7 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
 // ---------------------------------------------------------------------------------------------- argmax + token bookkeeping
 // argmax(-1) with the reference's tie rule: the first index of the maximum (tinygrad/mixin/op.py:866-891).
 __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int n, float* __restrict__ pv, int* __restrict__ pi) {
-  float best = -INFINITY; int bi = 0x7fffffff;
+  float best = -INFINITY; int bi = 0;                   // (no finite or -inf maximum at all, i.e. NaN logits: index 0, never an index outside the row)
   for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
     const float v = logits[i];
     if (v > best || (v == best && i < bi)) { best = v; bi = i; }
@@ -445,7 +454,7 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
 __global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi, int np, DecodeState* st,
                                                            const int* __restrict__ prompt, int* __restrict__ out_tokens, int max_tokens) {
   __shared__ float sv[256]; __shared__ int si[256];
-  float best = -INFINITY; int bi = 0x7fffffff;
+  float best = -INFINITY; int bi = 0;
   for (int i = threadIdx.x; i < np; i += 256) {
     const float v = pv[i]; const int ix = pi[i];
     if (v > best || (v == best && ix < bi)) { best = v; bi = ix; }
@@ -486,7 +495,7 @@ int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, 
   switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: blk = 256; break;
     case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_row: unsupported table type %d", ggml_type); }
   TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_row: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
-  embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (const DecodeState*)state, out);
+  embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out);
   TGA_LAUNCH_CHECK();
   return 0;
 }
@@ -525,7 +534,7 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   TGA_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr), "tga_attention_decode: q and k norm weights come together");
   TGA_REQUIRE(!q_norm_weight || ((((uintptr_t)q | (uintptr_t)k) & 15) == 0), "tga_attention_decode: q and k must be 16-byte aligned for the fused norm");
   AttnArgs a;
-  a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (const DecodeState*)state;
+  a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (DecodeState*)state;
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;

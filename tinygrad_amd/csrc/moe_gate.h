@@ -26,6 +26,7 @@ __device__ __forceinline__ void gate_topk_wave(const float* lg, int n_experts, i
     else s = sqrtf(log1pf(expf(v)));
     sc[i] = s;
   }
+  s_sel[lane] = 0; s_p[lane] = 0.f;                       // a slot no rank lands in (NaN scores compare false with everything) selects expert 0, like the reference's zero-filled scatter
   __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's LDS writes are visible to its own lanes
   for (int i = lane; i < n_experts; i += 64) {
     const float si = sc[i];

@@ -4,6 +4,7 @@
 // combine), extra/gemm/moe_gemm.py:112-134 (grouped_mx_gemm; its HIP kernel source is absent from the reference tree).
 #include "common.h"
 #include "host.h"
+#include <string.h>
 
 typedef int v8i32 __attribute__((ext_vector_type(8)));
 typedef float v4f32 __attribute__((ext_vector_type(4)));
@@ -217,69 +218,17 @@ __global__ __launch_bounds__(256) void combine_kernel(const uint16_t* __restrict
 
 // ------------------------------------------------------------------------------------------------ grouped MXFP8 GEMM
 // C[r, :] = deq(A[r, :]) . deq(B[e(r)])^T, float32 accumulate, bf16 store; e(r) = expert owning the 256-row tile of r
-// (Routing.rows_e, moe_routing.py:98-104).  A (M, K) e4m3 row-major; B (E, N, K) e4m3; scales E8M0 per 32 along K.
-// Workgroup = 4 waves (2 x 2), tile 128 x 128, each wave 64 x 64 = 4 x 4 MFMA tiles of v_mfma_scale_f32_16x16x128_f8f6f4.
-// Operand layout of that instruction as measured on MI355X: lane l = 16 g + r supplies row (A) / column (B) r; its 32 operand
-// bytes are K = 16 g + 0..15 followed by K = 64 + 16 g + 0..15 of the 128-wide K step; byte 0 of its scale register (op_sel 0)
+// (Routing.rows_e, moe_routing.py:98-104: the last expert whose offset is <= the tile's first row, so the tiles at or beyond
+// expert_off[E] belong to expert E - 1).  A (M, K) e4m3 row-major; B (E, N, K) e4m3; scales E8M0 per 32 along K.
+// Operand layout of v_mfma_scale_f32_16x16x128_f8f6f4 as measured on MI355X: lane l = 16 g + r supplies row (A) / column (B) r; its 32
+// operand bytes are K = 16 g + 0..15 followed by K = 64 + 16 g + 0..15 of the 128-wide K step; byte 0 of its scale register (op_sel 0)
 // is the E8M0 scale of the 32-block K = 32 g .. 32 g + 31 of row / column r (so a lane's scale does NOT belong to the lane's
 // own bytes); the 16 x 16 result has column l % 16 and rows 4 * (l / 16) + 0..3 in the lane's 4 accumulator registers.
 struct GemmArgs {
   uint16_t* C; const uint8_t* A; const uint8_t* B; const uint8_t* a_e8; const uint8_t* b_e8; const int* off;
   int M, N, K, E;
+  int routed_only;          // != 0: tiles at or beyond expert_off[E] are skipped (their rows of C keep their contents)
 };
-
-__global__ __launch_bounds__(256) void grouped_mxfp8_gemm_kernel(const GemmArgs g) {
-  const int tiles_n = g.N / 128;
-  const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;
-  const int row0 = tm * 128;
-  if (row0 >= g.off[g.E]) return;                           // beyond the last expert's padded range: nothing routed there
-  int lo = 0, hi = g.E;
-  while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (g.off[mid] <= row0) lo = mid; else hi = mid; }
-  // skip experts with an empty range that share the offset (off[mid] == off[mid+1]): take the last expert whose offset <= row0
-  const int e = lo;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int l16 = lane & 15, kb = lane >> 4;
-  const int KB = g.K / 32;
-  const uint8_t* Ap = g.A + (size_t)(row0 + wm * 64 + l16) * g.K + kb * 16;
-  const uint8_t* Bp = g.B + ((size_t)e * g.N + tn * 128 + wn * 64 + l16) * g.K + kb * 16;
-  const uint8_t* As = g.a_e8 + (size_t)(row0 + wm * 64 + l16) * KB + kb;
-  const uint8_t* Bs = g.b_e8 + ((size_t)e * g.N + tn * 128 + wn * 64 + l16) * KB + kb;
-  v4f32 acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < g.K; k0 += 128) {
-    v8i32 a[4], b[4]; int sa[4], sb[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const u32x4* pa = (const u32x4*)(Ap + (size_t)i * 16 * g.K + k0);
-      const u32x4 a0 = pa[0], a1 = pa[4];                     // K = 16 kb + 0..15 and 64 + 16 kb + 0..15
-      a[i] = v8i32{(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w, (int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
-      sa[i] = As[(size_t)i * 16 * KB + (k0 >> 5)];
-      const u32x4* pb = (const u32x4*)(Bp + (size_t)i * 16 * g.K + k0);
-      const u32x4 b0 = pb[0], b1 = pb[4];
-      b[i] = v8i32{(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
-      sb[i] = Bs[(size_t)i * 16 * KB + (k0 >> 5)];
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[i], b[j], acc[i][j], 0, 0, 0, sa[i], 0, sb[j]);
-  }
-  // store: lane holds column l16 and rows 4*kb + r of each 16 x 16 tile
-#pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const size_t row = (size_t)row0 + wm * 64 + i * 16 + kb * 4 + r, col = (size_t)tn * 128 + wn * 64 + j * 16 + l16;
-        g.C[row * g.N + col] = f_to_bf16(acc[i][j][r]);
-      }
-}
 
 // ---- LDS-tiled variant: 256 x 256 output tile per workgroup, 8 waves as 2 (M) x 4 (N), each 128 x 64 = 8 x 4 MFMAs per K step of
 // 128, two LDS stages of 64 KB (two waves per SIMD: one multiplies while the other waits on LDS).  A 16-row x 128-byte operand
@@ -298,17 +247,26 @@ __device__ __forceinline__ int gg_slot_off(int R, int c) {       // byte offset 
   return sub * 2048 + p * 1024 + ((16 * g + (r ^ (g + 4 * p))) << 4);
 }
 
-__global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(const GemmArgs g) {
-  extern __shared__ uint8_t smem[];                          // [stage][A 32 KB | B 32 KB | 512 scale dwords]
-  const int tiles_n = g.N / GG_TILE, ntiles = gridDim.x;
-  // consecutive workgroups go to different XCDs: give each XCD a contiguous run of tiles so that the N tiles of one row block
-  // (which share the activation tile) and the row blocks of one expert (which share the weight tile) meet in one L2
-  // (only the tiles below the last expert's padded range exist: the XCDs share those evenly)
-  const int nact = (g.off[g.E] / GG_TILE) * tiles_n;          // routed row blocks x column blocks
-  const int per_xcd = (nact + 7) / 8;
-  const int tile = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
-  if ((int)(blockIdx.x / 8) >= per_xcd || tile >= nact) return;
-  (void)ntiles;
+// Which tile workgroup b computes.  Consecutive workgroups go to different XCDs (the dispatcher deals them round-robin), so XCD x = b % 8
+// gets a contiguous run of the routed tiles: the N tiles of one row block (which share the activation tile) and the row blocks of one
+// expert (which share the weight tile) meet in one L2.  The routed tiles (rows below expert_off[E]) are shared evenly; the workgroups an
+// XCD has left take the tiles beyond, in order.  A bijection from [0, gridDim.x) onto the (M / 256) (N / 256) tiles for any grid size.
+__device__ __forceinline__ int gg_tile_of_workgroup(int b, int nwg, int nact, bool& routed) {
+  const int x = b & 7, j = b >> 3;
+  const int cnt_a = nact / 8 + (x < nact % 8), start_a = x * (nact / 8) + min(x, nact % 8);
+  routed = j < cnt_a;
+  if (routed) return start_a + j;
+  const int start_g = x * (nwg / 8) + min(x, nwg % 8);
+  return nact + (start_g - start_a) + (j - cnt_a);
+}
+
+__device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8_t* smem) {
+  const int tiles_n = g.N / GG_TILE;
+  const int off_end = min(max(g.off[g.E], 0), g.M);             // an offset table that overruns the matrix is clamped to it
+  const int nact = (off_end / GG_TILE) * tiles_n;              // routed row blocks x column blocks
+  bool routed;
+  const int tile = gg_tile_of_workgroup((int)blockIdx.x, (int)gridDim.x, nact, routed);
+  if (tile >= (g.M / GG_TILE) * tiles_n || (!routed && g.routed_only)) return;
   const int tm = tile / tiles_n, tn = tile % tiles_n;
   const int row0 = tm * GG_TILE;
   int lo = 0, hi = g.E;
@@ -398,6 +356,26 @@ __global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(cons
   }
 }
 
+
+// C-ABI launch: arguments in one by-value record.
+__global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(const GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) uint8_t smem[2 * GG_STAGE_BYTES];   // [stage][A 32 KB | B 32 KB | 512 scale dwords]
+  grouped_mxfp8_gemm_tile(g, smem);
+}
+
+// The same kernel with the argument list a pre-compiled PROGRAM bound through Tensor.custom_kernel hands over: one pointer per buffer in
+// the order of the sink's sources (extra/gemm/moe_gemm.py:36-48: C, A, B, x_si, w_si, x_e8, w_e8, expert_off), then the scalar
+// variables (tinygrad/uop/ops.py:1194-1198).  Launch: 512 threads x (M / 256) (N / 256) workgroups, no dynamic LDS (the reference's HIP
+// runtime passes 0 shared bytes, tinygrad/runtime/ops_hip.py:44-47), so the two 66 KB stages are static.  x_si / w_si are not read.
+extern "C" __global__ __launch_bounds__(GG_THREADS) void tga_grouped_mxfp8_gemm_kernel(uint16_t* C, const uint8_t* A, const uint8_t* B, const uint32_t* x_si,
+                                                                                        const uint32_t* w_si, const uint8_t* x_e8, const uint8_t* w_e8,
+                                                                                        const int* expert_off, int M, int N, int K, int E) {
+  __shared__ __attribute__((aligned(16))) uint8_t smem[2 * GG_STAGE_BYTES];
+  (void)x_si; (void)w_si;
+  GemmArgs g; g.C = C; g.A = A; g.B = B; g.a_e8 = x_e8; g.b_e8 = w_e8; g.off = expert_off; g.M = M; g.N = N; g.K = K; g.E = E; g.routed_only = 0;
+  grouped_mxfp8_gemm_tile(g, smem);
+}
+
 // clamped, interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98): bf16 in/out
 __global__ __launch_bounds__(256) void swiglu_interleaved_kernel(const uint16_t* __restrict__ h, long long rows, int two_inter, float limit, float alpha, uint16_t* __restrict__ y) {
   const int inter = two_inter / 2;
@@ -414,10 +392,10 @@ __global__ __launch_bounds__(256) void swiglu_interleaved_kernel(const uint16_t*
 
 // h[r, :] += bias[e(r), :] for the rows of every expert (examples/mlperf/models/gpt_oss.py:219-224: `+ (onehot @ bias.float()).cast(bf16)`
 // after each grouped GEMM): the bias row is cast to bf16 first and the sum of the two bf16 values is rounded to bf16, as the reference's
-// bf16 tensor add does.  Rows are located by 256-row tile (Routing.rows_e, moe_routing.py:98-104); rows at or beyond off[E] are left alone.
+// bf16 tensor add does.  Rows are located by 256-row tile (Routing.rows_e, moe_routing.py:98-104: the last expert whose offset is <= the tile's
+// first row, so the tiles at or beyond off[E] get the last expert's bias).
 __global__ __launch_bounds__(256) void add_expert_bias_kernel(uint16_t* __restrict__ h, const float* __restrict__ bias, const int* __restrict__ off, int n_experts, int N) {
   const int tile = blockIdx.y, row0 = tile * 256;
-  if (row0 >= off[n_experts]) return;
   int lo = 0, hi = n_experts;
   while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (off[mid] <= row0) lo = mid; else hi = mid; }
   const float* b = bias + (size_t)lo * N;
@@ -502,21 +480,36 @@ int tga_moe_combine_rows(const void* z_bf16, const int32_t* dest_row, const floa
   return 0;
 }
 
-int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
-                           const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
-  (void)x_si; (void)w_si;   // the packed (K/128, rows) scale copies the reference's kernel reads are accepted but not needed here
+static int grouped_mxfp8_gemm_launch(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
+                                     int64_t M, int64_t N, int64_t K, int n_experts, int routed_only, void* stream) {
   TGA_REQUIRE(C && A && B && x_e8 && w_e8 && expert_off, "tga_grouped_mxfp8_gemm: null pointer");
   // the reference's precondition (extra/gemm/moe_gemm.py:120)
   TGA_REQUIRE(M % 256 == 0 && N % 256 == 0 && K % 128 == 0, "grouped mxfp8 needs M%%256,N%%256,K%%128, got (%lld, %lld) (%d, %lld, %lld)",
               (long long)M, (long long)K, n_experts, (long long)N, (long long)K);
+  TGA_REQUIRE(M > 0 && N > 0 && K > 0 && n_experts >= 1 && (M / GG_TILE) * (N / GG_TILE) < (1ll << 31) && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
+              "tga_grouped_mxfp8_gemm: empty or oversized problem (%lld, %lld, %lld), %d experts", (long long)M, (long long)N, (long long)K, n_experts);
   GemmArgs g; g.C = (uint16_t*)C; g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.a_e8 = (const uint8_t*)x_e8; g.b_e8 = (const uint8_t*)w_e8;
-  g.off = expert_off; g.M = (int)M; g.N = (int)N; g.K = (int)K; g.E = n_experts;
-  static bool configured = false;
-  if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)grouped_mxfp8_gemm_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GG_STAGE_BYTES)); configured = true; }
-  const long long tiles = ((M / GG_TILE) * (N / GG_TILE) + 7) / 8 * 8;     // workgroup b serves XCD b % 8
-  grouped_mxfp8_gemm_lds_kernel<<<(unsigned)tiles, GG_THREADS, 2 * GG_STAGE_BYTES, (hipStream_t)stream>>>(g);
+  g.off = expert_off; g.M = (int)M; g.N = (int)N; g.K = (int)K; g.E = n_experts; g.routed_only = routed_only;
+  grouped_mxfp8_gemm_lds_kernel<<<(unsigned)((M / GG_TILE) * (N / GG_TILE)), GG_THREADS, 0, (hipStream_t)stream>>>(g);
   TGA_LAUNCH_CHECK();
   return 0;
+}
+
+int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
+                           const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
+  (void)x_si; (void)w_si;   // the packed (K/128, rows) scale copies the reference's kernel reads are accepted but not needed here
+  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 0, stream);
+}
+
+int tga_grouped_mxfp8_gemm_routed(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
+                                  int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
+  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 1, stream);
+}
+
+int tga_kernel_symbol(const char* name, const void** host_function) {
+  TGA_REQUIRE(name && host_function, "tga_kernel_symbol: null pointer");
+  if (strcmp(name, "tga_grouped_mxfp8_gemm_kernel") == 0) { *host_function = (const void*)tga_grouped_mxfp8_gemm_kernel; return 0; }
+  return tga_set_error("tga_kernel_symbol: no kernel named '%s'", name);
 }
 
 int tga_add_expert_bias(void* h_bf16, const float* bias, const int32_t* expert_off, int64_t M, int64_t N, int n_experts, void* stream) {

@@ -190,8 +190,8 @@ static int launch_qgemm(QArgs a, hipStream_t s) {
   if (grid > cap) grid = cap;
   auto kern = qgemm_mfma_kernel<T, M>;
   if (lds > 48 * 1024) {
-    static bool configured = false;
-    if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * QM_LDS_BUDGET + 4096)); configured = true; }
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * QM_LDS_BUDGET + 4096);   // once per instantiation, thread-safe
+    TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)grid), dim3(QM_THREADS), lds, s>>>(a);
   TGA_LAUNCH_CHECK();

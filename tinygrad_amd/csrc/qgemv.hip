@@ -280,8 +280,8 @@ static int launch_qgemv(QArgs a, hipStream_t s) {
   if (grid < 1) grid = 1;
   auto kern = qgemv_kernel<T, M, R>;
   if (lds > 48 * 1024) {
-    static size_t configured = 0;   // per instantiation
-    if (lds > configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, QG_LDS_BUDGET)); configured = QG_LDS_BUDGET; }
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, QG_LDS_BUDGET);   // once per instantiation, thread-safe
+    TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)grid), dim3(QG_THREADS), lds, s>>>(a);
   TGA_LAUNCH_CHECK();

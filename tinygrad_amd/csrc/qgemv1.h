@@ -389,8 +389,9 @@ template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
 static int launch_fast_p(const QArgs& a, long long grid, size_t lds, hipStream_t s) {
   auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H, PRO>;
   if (lds > 48 * 1024) {
-    static bool configured = false;
-    if (!configured) { TGA_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024)); configured = true; }
+    // once per instantiation; the initialisation of a function-local static is serialised by the language, so concurrent first calls are safe
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)grid, (unsigned)(a.sel ? a.xdiv_jobs : 1)), dim3(WK * WR * 64), lds, s>>>(a);
   TGA_LAUNCH_CHECK();

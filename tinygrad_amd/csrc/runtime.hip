@@ -66,6 +66,15 @@ int tga_event_record(void* ev, void* stream) { TGA_HIP(hipEventRecord((hipEvent_
 int tga_event_sync(void* ev) { TGA_HIP(hipEventSynchronize((hipEvent_t)ev)); return 0; }
 int tga_event_elapsed_ms(void* start, void* stop, float* ms) { TGA_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop)); return 0; }
 
+// HIPProgram.__call__ (tinygrad/runtime/ops_hip.py:36-57): launch a kernel of this library by its host-side handle with an array of
+// pointers to the argument values (hipLaunchKernel's convention), grid counted in workgroups, no dynamic LDS.
+int tga_launch_kernel(const void* host_function, const uint32_t* grid, const uint32_t* block, void** args, void* stream) {
+  TGA_REQUIRE(host_function && grid && block && args, "tga_launch_kernel: null pointer");
+  TGA_REQUIRE(grid[0] && grid[1] && grid[2] && block[0] && block[1] && block[2] && (uint64_t)block[0] * block[1] * block[2] <= 1024, "tga_launch_kernel: empty grid or block, or more than 1024 threads");
+  TGA_HIP(hipLaunchKernel(host_function, dim3(grid[0], grid[1], grid[2]), dim3(block[0], block[1], block[2]), args, 0, (hipStream_t)stream));
+  return 0;
+}
+
 int tga_graph_begin(void* stream) {
   TGA_REQUIRE(stream, "tga_graph_begin: capture needs a non-null stream");
   TGA_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));

@@ -258,11 +258,10 @@ class _Shared:
     self.x2 = Buffer((1, c.dim), f32)                                    # second residual row: a launch that completes x + sum_j p_j y_j writes here
     self.xn = Buffer((1, c.dim), f16)
     nq, nkv = c.n_heads * c.head_dim, c.n_kv_heads * c.head_dim
-    self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v, contiguous for the fused block launch
+    self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v
     self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
-    self.sync = Buffer((320,), np.uint32).zero_()                        # device-wide barrier counters + error flag of the fused launch
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
-    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2) + c.n_kv_heads,), f32).zero_()   # + arrival counters of the one-launch block kernel
+    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
     self.act = Buffer((1, c.hidden_dim), f16)
     if c.num_experts:
       k = c.num_experts_per_tok
@@ -275,9 +274,8 @@ class _Shared:
     self.out_tokens = Buffer((max(1, max_new),), np.int32).zero_()
 
 class Transformer:
-  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096, fused: bool = False):
-    """fused: run all blocks of a token in one persistent launch (tga_decode_layers; dense Q4_0 / Q8_0 models only).  The default is
-    one launch per op (six per dense block, seven per MoE block; attention is two), which measures about 10 % faster on the 8B configuration."""
+  def __init__(self, config: TransformerConfig, state_dict: dict, max_new: int = 4096):
+    """One launch per op (six per dense block, seven per MoE block; attention is two), captured once per token kind and replayed."""
     self.config = c = config
     self.s = _Shared(c, max_new)
     self.max_new = max_new
@@ -291,44 +289,25 @@ class Transformer:
     self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.num_experts_per_tok <= 8
     self.stream = rt.Stream()
     self._graphs = {}
-    # optional: one persistent launch for all blocks (tga_decode_layers) when every block is dense with seven linears of one Q4_0 / Q8_0 type
-    self.layer_table = self._build_layer_table() if fused else None
+    self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
 
-  def _build_layer_table(self):
-    c = self.config
-    if c.num_experts or c.qk_norm or c.head_dim not in (64, 128) or c.n_heads * c.head_dim != c.dim: return None
-    if any(b.qkv_bias is not None for b in self.blk): return None
-    if c.dim % 64 or c.hidden_dim % 64 or max(c.dim, c.hidden_dim) > 16384: return None
-    if c.n_heads // c.n_kv_heads * ((c.max_context + 63) // 64) > 1024: return None
-    t0 = self.blk[0].attn_q.ggml_type
-    if t0 not in (rt.Q4_0, rt.Q8_0): return None
-    rows = []
-    for b in self.blk:
-      lins = (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down)
-      if any(l.ggml_type != t0 or l.blocks.ptr % 4 for l in lins): return None
-      rows.append([l.blocks.ptr for l in lins] + [b.attn_norm.ptr, b.ffn_norm.ptr, b.cache_k.ptr, b.cache_v.ptr])
-    self.layer_type = t0
-    return Buffer.from_numpy(np.array(rows, dtype=np.uint64))
-
-  def check_fused(self):
-    """Raises when a fused block launch gave up on its device-wide barrier (results of that step are incomplete)."""
-    if self.layer_table is not None and int(self.s.sync.numpy()[2]) != 0:
-      self.s.sync.zero_()
-      raise RuntimeError("tga_decode_layers: a barrier wait timed out (launch not resident as a whole?)")
+  def check_state(self):
+    """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
+    lookup, bit 1 = a position at or beyond max_context reached the attention launch).  The kernels clamp / skip instead of faulting."""
+    err = int(self.s.state.numpy()[4])
+    if err:
+      st = self.s.state.numpy(); st[4] = 0; self.s.state.copyin(st)
+      raise RuntimeError(f"decode state error {err}: " + ", ".join(m for b, m in ((1, "token id outside the vocabulary"), (2, "position beyond max_context")) if err & b))
 
   # one token through all blocks; with_head adds output_norm + output + argmax (model.py:358-364)
   def _step(self, with_head: bool):
     c, s, L, st = self.config, self.s, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
-    if self.layer_table is not None:
-      rt.check(L.tga_decode_layers(self.layer_table.ptr, c.num_blocks, self.layer_type, s.x.ptr, s.qkv.ptr, s.attn.ptr, s.act.ptr, s.attn_part.ptr,
-                                   s.state.ptr, s.rope.ptr, s.sync.ptr, c.dim, c.hidden_dim, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, c.norm_eps, st))
     x, pending = s.x, False
-    if self.layer_table is None:
-      nb = len(self.blk)
-      for i, b in enumerate(self.blk):
-        nxt = self.blk[i + 1].can_fold_combine if i + 1 < nb else (with_head and self.can_fold_head)
-        x, pending = b(x, st, pending, defer=nxt)
+    nb = len(self.blk)
+    for i, b in enumerate(self.blk):
+      nxt = self.blk[i + 1].can_fold_combine if i + 1 < nb else (with_head and self.can_fold_head)
+      x, pending = b(x, st, pending, defer=nxt)
     if with_head:
       if pending:                                                      # the last block's weighted sum completed inside the lm-head launch
         x_new = s.x2 if x.ptr == s.x.ptr else s.x
@@ -414,11 +393,13 @@ class Transformer:
   def reset(self, tokens: list[int]):
     """Start a new sequence: position 0, first prompt token loaded, nothing cached (no KV-prefix reuse)."""
     c, s = self.config, self.s
-    assert 1 <= len(tokens) < c.max_context
+    if not 1 <= len(tokens) < c.max_context: raise ValueError(f"prompt of {len(tokens)} tokens does not fit max_context {c.max_context}")
+    if min(tokens) < 0 or max(tokens) >= c.vocab_size: raise ValueError(f"token id outside the vocabulary of {c.vocab_size}")
     prompt = np.zeros(c.max_context, dtype=np.int32); prompt[:len(tokens)] = tokens
     s.prompt.copyin(prompt)
-    st = np.zeros(16, dtype=np.int32); st[1], st[3] = tokens[0], len(tokens)
+    st = np.zeros(16, dtype=np.int32); st[1], st[3], st[5] = tokens[0], len(tokens), c.vocab_size
     s.state.copyin(st)
+    self._n_prompt, self._steps_done = len(tokens), 0
 
   def prefill(self, tokens: list[int], use_graph: bool = True):
     """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step."""
@@ -426,21 +407,26 @@ class Transformer:
     for _ in range(len(tokens) - 1):
       if use_graph: self._graph(False).launch()
       else: self._step(False)
+    self._steps_done = len(tokens) - 1
     self.stream.synchronize()
-    self.check_fused()
 
   def decode_step(self, use_graph: bool = True, sync: bool = True):
+    """One token.  The position it occupies must exist in the KV cache and the rotation table: like the reference's generate loop
+    (`while len(tokens) < self.max_context`, tinygrad/llm/model.py:475) the sequence ends at max_context."""
+    if self._steps_done >= self.config.max_context: raise RuntimeError(f"context full: position {self._steps_done} is beyond max_context {self.config.max_context}")
     if use_graph: self._graph(True).launch()
     else: self._step(True)
+    self._steps_done += 1
     if sync: self.stream.synchronize()
 
   def generate(self, tokens: list[int], max_new_tokens: int, use_graph: bool = True):
-    """Greedy decoding (temperature 0): yields one token id per step, like Transformer.generate (model.py:464-484)."""
+    """Greedy decoding (temperature 0): yields one token id per step, like Transformer.generate (model.py:464-484), and like it stops when
+    the context is full (model.py:475)."""
     self.prefill(tokens, use_graph)
-    for i in range(max_new_tokens):
+    for i in range(min(max_new_tokens, self.config.max_context - len(tokens), self.max_new)):
       self.decode_step(use_graph, sync=True)                          # the reference syncs once per token too (out.item(), model.py:482)
-      self.check_fused()
       yield int(self.s.out_tokens.view(4 * i, (1,), np.int32).numpy()[0])
+    self.check_state()
 
   def logits(self) -> np.ndarray: return self.s.logits.numpy().reshape(-1)
 

@@ -50,14 +50,14 @@ def _declare(lib):
     "tga_moe_dispatch": [vp, vp, vp, vp, i, i, i, i64, i, vp, vp],
     "tga_moe_combine_rows": [vp, vp, vp, i, i, i, vp, vp],
     "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
+    "tga_grouped_mxfp8_gemm_routed": [vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
+    "tga_kernel_symbol": [ctypes.c_char_p, c_void_pp], "tga_launch_kernel": [vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32), c_void_pp, vp],
     "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
     "tga_add_expert_bias": [vp, vp, vp, i64, i64, i, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
     "tga_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
     "tga_attention_decode_normed": [vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, i, vp],
-    "tga_decode_layers": [vp, i, i, vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, i, i, ctypes.c_float, vp],
-    "tga_decode_layers_trace": [vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
     "tga_advance_prompt": [vp, vp, vp],
     "tga_copy_kernel": [vp, vp, ctypes.c_size_t, vp],
