@@ -35,6 +35,7 @@ def parity_gate(model, c, threads):
   lin = lambda t, w, x, n, k: cref.linear(t, w, np.ascontiguousarray(x, dtype=np.float32).reshape(1, -1), n, k, w_round_f16=True, threads=threads)[0]
   rng = np.random.default_rng(7)
   B = rt.Buffer.from_numpy
+  f32 = lambda buf: np.ascontiguousarray(buf.numpy()).view(np.uint8).view(np.float32).reshape(-1)      # norm weights are float32 rows kept in byte buffers
   b0, host0 = model.blk[0], _host_layer(model, 0)
   checked, worst = [], 0.0
   def note(name, got, ref):
@@ -42,7 +43,7 @@ def parity_gate(model, c, threads):
     e = ol.rel_err(np.asarray(got).reshape(-1), np.asarray(ref).reshape(-1)); worst = max(worst, e); checked.append({"what": name, "rel_err": float(f"{e:.3e}")})
   # ---- (1) layer 0's launches on a fresh row
   x = (rng.standard_normal((1, c.dim)) * 2).astype(np.float32)
-  an, fn = b0.attn_norm.numpy().reshape(-1), b0.ffn_norm.numpy().reshape(-1)
+  an, fn = f32(b0.attn_norm), f32(b0.ffn_norm)
   xn = ollm.rmsnorm(x, an, c.norm_eps)
   q, k, v = (rt.Buffer((1, n), np.float32) for n in (b0.attn_q.out_features, b0.attn_k.out_features, b0.attn_v.out_features))
   qlinear_multi([b0.attn_q, b0.attn_k, b0.attn_v], B(x), [q, k, v], norm=(b0.attn_norm, c.norm_eps))
@@ -64,7 +65,7 @@ def parity_gate(model, c, threads):
   row_bytes = head.nbytes // head.out_features
   lg = rt.Buffer((1, c.vocab_size), np.float32)
   qlinear_multi([head], B(x), [lg], norm=(model.output_norm, c.norm_eps))
-  xo = ollm.rmsnorm(x, model.output_norm.numpy().reshape(-1), c.norm_eps)
+  xo = ollm.rmsnorm(x, f32(model.output_norm), c.norm_eps)
   lgh = lg.numpy()[0]
   got_rows, ref_rows = [], []
   for r0 in np.linspace(0, c.vocab_size - 512, 8).astype(int):
@@ -84,7 +85,7 @@ def parity_gate(model, c, threads):
   xr = og.ggml_data_to_tensor(model.token_embd.view(tok * emb_row_bytes, (emb_row_bytes,), np.uint8).numpy(), c.dim, model.embd_type).astype(np.float32)
   for i, b in enumerate(model.blk):
     hl = _host_layer(model, i)
-    n1 = ollm.rmsnorm(xr, b.attn_norm.numpy().reshape(-1), c.norm_eps)
+    n1 = ollm.rmsnorm(xr, f32(b.attn_norm), c.norm_eps)
     qv, kv_, vv = (lin(*hl[nm][:2], n1, *hl[nm][2:]) for nm in ("attn_q", "attn_k", "attn_v"))
     qr, kr = ollm.apply_rope(qv.reshape(H, hd), fc), ollm.apply_rope(kv_.reshape(KV, hd), fc)
     ck, cv = b.cache_k.numpy()[:, :pos + 1].astype(np.float32), b.cache_v.numpy()[:, :pos + 1].astype(np.float32)
@@ -94,10 +95,10 @@ def parity_gate(model, c, threads):
     e = np.exp(sc - sc.max(-1, keepdims=True)); pr = e / e.sum(-1, keepdims=True)
     at = np.einsum("ht,htd->hd", pr, Vh).astype(np.float32).reshape(-1)
     hh = xr + lin(*hl["attn_output"][:2], at, *hl["attn_output"][2:])
-    n2 = ollm.rmsnorm(hh, b.ffn_norm.numpy().reshape(-1), c.norm_eps)
+    n2 = ollm.rmsnorm(hh, f32(b.ffn_norm), c.norm_eps)
     ff = ollm.silu(lin(*hl["ffn_gate"][:2], n2, *hl["ffn_gate"][2:])) * lin(*hl["ffn_up"][:2], n2, *hl["ffn_up"][2:])
     xr = hh + lin(*hl["ffn_down"][:2], ff, *hl["ffn_down"][2:])
-  xo = ollm.rmsnorm(xr, model.output_norm.numpy().reshape(-1), c.norm_eps)
+  xo = ollm.rmsnorm(xr, f32(model.output_norm), c.norm_eps)
   lg_cpu = lin(head.ggml_type, head.blocks.view(0, (head.nbytes,), np.uint8).numpy(), xo, c.vocab_size, c.dim)
   note(f"full decode step at position {pos} ({c.num_blocks} blocks + lm-head): logits", lg_gpu, lg_cpu)
   top2 = np.partition(lg_cpu, -2)[-2:]
