@@ -202,6 +202,14 @@ int tga_transpose_quantize_mxfp8(const void* g_bf16, int64_t M, int64_t N, void*
  * those of expert e_j in flattened (token, slot) order.  scratch: int32[n_tokens*k + ceil(n_tokens*k/1024)*n_experts]. */
 int tga_moe_route(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
                   int32_t* counts, int32_t* scratch, void* stream);
+/* tga_moe_route without a workspace argument and without any allocation (no counterpart in the reference; for callers that cannot
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The ranks and per-chunk counts live in a
+ * 512 KiB device array inside the library, one copy per GPU, held until the process ends; tga_init(device) must have run on the current
+ * device.  Limits: n_tokens * k <= 65536 and n_tokens * k + ceil(n_tokens * k / 1024) * n_experts <= 131072, else an error and no launch.
+ * Nothing in the workspace has to start at zero (every word read was written by the same call), but all calls on one GPU share it: calls
+ * that overlap on one GPU (two streams, two threads) race.  Same results as tga_moe_route. */
+int tga_moe_route_static(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
+                         int32_t* counts, void* stream);
 /* dispatch (moe_routing.py:124-126): xg[dest_row[j], :] = x[j / k, :] (bf16 rows); rows no assignment maps to are zero-filled. */
 int tga_moe_dispatch(const void* x_bf16, const int32_t* dest_row, const int32_t* off, const int32_t* counts, int n_tokens, int k, int n_experts,
                      int64_t m_l, int D, void* xg_bf16, void* stream);

@@ -6,6 +6,7 @@
 #include "../../include/tinygrad_amd.h"
 
 int tga_set_error(const char* fmt, ...);   // stores the per-thread message, returns 1
+extern "C" int tga_route_scratch_setup(int device);   // mxfp8.hip: looks up the static routing workspace of the current device (tga_init calls it)
 
 #define TGA_HIP(expr) do { hipError_t _e = (expr); if (_e != hipSuccess) \
   return tga_set_error("HIP Error %d, %s  [%s at %s:%d]", (int)_e, hipGetErrorString(_e), #expr, __FILE__, __LINE__); } while (0)

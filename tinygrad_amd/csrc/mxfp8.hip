@@ -443,13 +443,12 @@ int tga_transpose_quantize_mxfp8(const void* g_bf16, int64_t M, int64_t N, void*
   return 0;
 }
 
-int tga_moe_route(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
-                  int32_t* counts, int32_t* scratch, void* stream) {
-  TGA_REQUIRE(logits && weights && topi && dest_row && off && counts && scratch, "tga_moe_route: null pointer");
-  TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 8192 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_route: bad geometry");
-  hipStream_t s = (hipStream_t)stream;
+static int moe_route_launch(const char* who, const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
+                            int32_t* counts, int32_t* scratch, hipStream_t s) {
+  TGA_REQUIRE(logits && weights && topi && dest_row && off && counts && scratch, "%s: null pointer", who);
+  TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 8192 && k >= 1 && k <= 64 && k <= n_experts, "%s: bad geometry", who);
   const int n_assign = n_tokens * k, nchunks = (n_assign + 1023) / 1024;
-  int* local_rank = scratch; int* chunk_cnt = scratch + n_assign;
+  int* local_rank = scratch; int* chunk_cnt = scratch + n_assign;          // both are written in full before they are read: nothing has to start at zero
   route_topk_kernel<<<n_tokens, 64, n_experts * sizeof(float), s>>>(logits, n_experts, k, topi, weights);
   TGA_LAUNCH_CHECK();
   route_rank_kernel<<<nchunks, 256, 0, s>>>(topi, n_assign, n_experts, local_rank, chunk_cnt);
@@ -459,6 +458,40 @@ int tga_moe_route(const float* logits, int n_tokens, int n_experts, int k, float
   route_dest_kernel<<<(n_assign + 255) / 256, 256, 0, s>>>(topi, local_rank, chunk_cnt, off, n_assign, n_experts, dest_row);
   TGA_LAUNCH_CHECK();
   return 0;
+}
+
+int tga_moe_route(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
+                  int32_t* counts, int32_t* scratch, void* stream) {
+  return moe_route_launch("tga_moe_route", logits, n_tokens, n_experts, k, weights, topi, dest_row, off, counts, scratch, (hipStream_t)stream);
+}
+
+// ---- tga_moe_route for callers that cannot allocate: its workspace (the per-assignment ranks and the per-chunk expert counts) is this
+// file-scope device array instead of a caller buffer.  Every GPU the library runs on holds its own copy of the array at its own address
+// until the process ends; `scratch` itself is only the host-side stand-in of the symbol, so the device address is looked up once per
+// device (tga_init, with that device current) and everything below uses that pointer.
+#define ROUTE_STATIC_WORDS (2 * 65536)                       // int32: n_tokens * k + ceil(n_tokens * k / 1024) * n_experts must fit (512 KiB)
+#define ROUTE_MAX_DEVICES 64
+static __device__ __align__(256) int32_t scratch[ROUTE_STATIC_WORDS];
+static int32_t* g_route_scratch[ROUTE_MAX_DEVICES];          // device address of `scratch` on device d, filled by tga_route_scratch_setup(d)
+
+int tga_route_scratch_setup(int device) {                    // called by tga_init after hipSetDevice(device)
+  TGA_REQUIRE(device >= 0 && device < ROUTE_MAX_DEVICES, "tga_init: device %d is beyond the %d devices the static workspace table covers", device, ROUTE_MAX_DEVICES);
+  if (g_route_scratch[device]) return 0;
+  int32_t* p = nullptr;
+  TGA_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+  g_route_scratch[device] = p;
+  return 0;
+}
+
+int tga_moe_route_static(const float* logits, int n_tokens, int n_experts, int k, float* weights, int32_t* topi, int32_t* dest_row, int32_t* off,
+                         int32_t* counts, void* stream) {
+  int dev = -1;
+  TGA_HIP(hipGetDevice(&dev));
+  TGA_REQUIRE(dev >= 0 && dev < ROUTE_MAX_DEVICES && g_route_scratch[dev], "tga_moe_route_static: tga_init has not run on device %d", dev);
+  TGA_REQUIRE(n_tokens >= 1 && k >= 1 && n_experts >= 1 && (long long)n_tokens * k <= 65536, "tga_moe_route_static: n_tokens * k = %lld exceeds the static workspace (65536 assignments)", (long long)n_tokens * k);
+  const long long words = (long long)n_tokens * k + (((long long)n_tokens * k + 1023) / 1024) * n_experts;
+  TGA_REQUIRE(words <= ROUTE_STATIC_WORDS, "tga_moe_route_static: %lld workspace words needed, the static workspace holds %d (n_tokens * k + ceil(n_tokens * k / 1024) * n_experts)", words, ROUTE_STATIC_WORDS);
+  return moe_route_launch("tga_moe_route_static", logits, n_tokens, n_experts, k, weights, topi, dest_row, off, counts, g_route_scratch[dev], (hipStream_t)stream);
 }
 
 int tga_moe_dispatch(const void* x_bf16, const int32_t* dest_row, const int32_t* off, const int32_t* counts, int n_tokens, int k, int n_experts,

@@ -23,7 +23,7 @@ int tga_init(int device) {
   hipDeviceProp_t p;
   TGA_HIP(hipGetDeviceProperties(&p, device));
   TGA_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, "tga_init: kernels are built for gfx950 only, device is %s", p.gcnArchName);
-  return 0;
+  return tga_route_scratch_setup(device);                   // device address of the static workspace of tga_moe_route_static on this GPU
 }
 
 int tga_device_name(char* buf, size_t len) {

@@ -30,10 +30,16 @@ class Routing:
   topi: Buffer         # (T, k) int32
   counts: Buffer       # (E,) int32
 
-def route(logits: Buffer, experts_per_tok: int, n_experts: int, stream=None) -> Routing:
+def route(logits: Buffer, experts_per_tok: int, n_experts: int, stream=None, out: Routing | None = None) -> Routing:
+  """moe_routing.py:109-122.  out: a Routing whose buffers are reused; the call then allocates nothing at all (tga_moe_route_static keeps its
+  workspace inside the library), e.g. while a HIP graph is being captured."""
   T, E = logits.shape
   assert E == n_experts
   k = experts_per_tok
+  if out is not None:
+    assert out.weights.shape == (T, k) and out.off.shape == (E + 1,)
+    rt.check(rt.lib().tga_moe_route_static(logits.ptr, T, E, k, out.weights.ptr, out.topi.ptr, out.dest_row.ptr, out.off.ptr, out.counts.ptr, stream))
+    return out
   w, topi, dest, off, cnt = Buffer((T, k), np.float32), Buffer((T, k), np.int32), Buffer((T * k,), np.int32), Buffer((E + 1,), np.int32), Buffer((E,), np.int32)
   scratch = Buffer((T * k + ((T * k + 1023) // 1024) * E,), np.int32)
   rt.check(rt.lib().tga_moe_route(logits.ptr, T, E, k, w.ptr, topi.ptr, dest.ptr, off.ptr, cnt.ptr, scratch.ptr, stream))

@@ -47,6 +47,7 @@ def _declare(lib):
     "tga_silu_mul_quantize_mxfp8": [vp, vp, i64, i64, vp, vp, vp, vp],
     "tga_transpose_quantize_mxfp8": [vp, i64, i64, vp, vp, vp, vp],
     "tga_moe_route": [vp, i, i, i, vp, vp, vp, vp, vp, vp, vp],
+    "tga_moe_route_static": [vp, i, i, i, vp, vp, vp, vp, vp, vp],
     "tga_moe_dispatch": [vp, vp, vp, vp, i, i, i, i64, i, vp, vp],
     "tga_moe_combine_rows": [vp, vp, vp, i, i, i, vp, vp],
     "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
