@@ -2,7 +2,7 @@
 
 ggml_data_to_tensor(t, n, ggml_type) mirrors tinygrad/llm/gguf.py:23: `t` is the raw byte buffer (device Buffer of uint8, or a
 numpy array that is uploaded), `n` the element count, and the result is a flat float32 device Buffer of n elements, bit-exact
-with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ3_XXS (18), IQ3_S (21), IQ2_S (22), IQ4_XS (23), MXFP4 (39), Q1_0 (41); native float32/float16 (0, 1) are reinterpreted in place.
+with the reference for Q4_0 (2), Q4_1 (3), Q5_0 (6), Q5_1 (7), Q8_0 (8), Q4_K (12), Q5_K (13), Q6_K (14), IQ3_XXS (18), IQ3_S (21), IQ2_S (22), IQ4_XS (23), MXFP4 (39), Q1_0 (41); native float32/float16 (0, 1) and the other native types (int8 24, int16 25, int32 26, int64 27, float64 28; bfloat16 30 as its uint16 bit patterns) are reinterpreted in place.
 Unknown types raise ValueError with the reference's message (gguf.py:119)."""
 from __future__ import annotations
 import numpy as np
@@ -17,6 +17,9 @@ def ggml_data_to_tensor(t, n: int, ggml_type: int, out_dtype=np.float32, stream=
   t = _as_device_bytes(t)
   if ggml_type == rt.F32: return t.view(0, (n,), np.float32)
   if ggml_type == rt.F16: return t.view(0, (n,), np.float16)
+  if ggml_type in _NATIVE_NUMPY:                              # int8 / int16 / int32 / int64 / float64 / bfloat16: the same bytes under their own type (gguf.py:35-36)
+    dt = _NATIVE_NUMPY[ggml_type]
+    return t.view(0, (n,), dt)                                # bfloat16 (30) has no numpy type: its bit patterns come back as uint16
   if ggml_type not in GGML_QUANT and ggml_type not in GGML_DEQUANT_ONLY: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
   nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]
   nfull = (n // nel) * nel                                   # gguf.py:45 uses whole blocks only
@@ -33,6 +36,7 @@ import io, pathlib, re, struct
 from dataclasses import dataclass
 
 _NATIVE_ITEMSIZE = {0: 4, 1: 2, 24: 1, 25: 2, 26: 4, 27: 8, 28: 8, 30: 2}         # gguf.py:16-17
+_NATIVE_NUMPY = {24: np.int8, 25: np.int16, 26: np.int32, 27: np.int64, 28: np.float64, 30: np.uint16}
 GGUF_F32_LIKE = (0, 30)                                                             # float32, bfloat16
 
 def _rd(fmt, n, r): return struct.unpack("<" + fmt, r.read(n))[0]
@@ -78,12 +82,20 @@ def gguf_parse(raw: np.ndarray) -> tuple[dict, dict[str, GGUFTensor]]:
     tensors[name] = GGUFTensor(name, typ, tuple(reversed(dims)), raw[data_start + off: data_start + off + nb])
   return kv, tensors
 
+_FIRST_SPLIT = re.compile(r"-00001-of-\d{5}\.gguf$")
+
 def _split_paths(path: pathlib.Path, kv: dict) -> list[pathlib.Path]:
-  """gguf.py:151-155."""
-  if (total := kv.get("split.count", 1)) <= 1: return [path]
-  if kv.get("split.no", 0) != 0: raise ValueError(f"multi-part GGUF must be loaded from the first split, got split.no={kv['split.no']}")
-  if not (m := re.match(r"^(.*)-00001-of-\d{5}\.gguf$", str(path))): raise ValueError(f"first split path must end with -00001-of-NNNNN.gguf: {path}")
-  return [pathlib.Path(f"{m.group(1)}-{i:05d}-of-{total:05d}.gguf") for i in range(1, total + 1)]
+  """Every part of a model that llama.cpp's gguf-split wrote as <stem>-00001-of-000NN.gguf ... (the rule of gguf.py:151-155): the part count
+  comes from the first part's `split.count`; loading has to start at part 1 because only that one carries the metadata."""
+  n_parts = int(kv.get("split.count", 1))
+  if n_parts <= 1: return [path]
+  this_part = int(kv.get("split.no", 0))
+  if this_part != 0: raise ValueError(f"multi-part GGUF must be loaded from the first split, got split.no={this_part}")
+  name = str(path)
+  hit = _FIRST_SPLIT.search(name)
+  if hit is None: raise ValueError(f"first split path must end with -00001-of-NNNNN.gguf: {path}")
+  stem = name[:hit.start()]
+  return [pathlib.Path(f"{stem}-{part:05d}-of-{n_parts:05d}.gguf") for part in range(1, n_parts + 1)]
 
 def gguf_load(fn, upload: bool = True) -> tuple[dict, dict[str, GGUFTensor]]:
   """gguf_load (gguf.py:157-176): returns (kv_data, {name: GGUFTensor}).  fn: path or uint8 numpy array.  Multi-part splits are

@@ -342,7 +342,8 @@ class Transformer:
     max_context = min(max_context, ctx) if max_context is not None else ctx
     n_heads, n_kv = kv[f"{arch}.attention.head_count"], kv[f"{arch}.attention.head_count_kv"]
     dim = kv[f"{arch}.embedding_length"]
-    head_dim = kv.get(f"{arch}.attention.key_length", dim // n_heads)
+    head_dim = kv.get(f"{arch}.attention.key_length_mla", kv.get(f"{arch}.attention.key_length", dim // n_heads))
+    num_blocks = kv[f"{arch}.block_count"] - kv.get(f"{arch}.nextn_predict_layers", 0)     # trailing next-token-prediction layers are not part of the decoder (model.py:424)
     rope_dim = kv.get(f"{arch}.rope.dimension_count", head_dim)
     if rope_dim != head_dim and (arch == "llama" or rope_dim % 2 or (head_dim - rope_dim) % 2 or not 0 < rope_dim < head_dim):
       raise NotImplementedError(f"rope dimension {rope_dim} of head_dim {head_dim} for architecture {arch} is not built")
@@ -350,6 +351,8 @@ class Transformer:
     sd = {}
     for name, t in ts.items():
       if name == "rope_freqs.weight": continue                         # unused by the reference too (model.py:446)
+      if name.startswith("blk.") and int(name.split(".")[1]) >= num_blocks: continue     # next-token-prediction layers
+      if arch == "glm4moe": name = name.replace("post_attention_norm", "ffn_norm")       # model.py:403-404
       rows, cols = (int(np.prod(t.shape[:-1])), t.shape[-1]) if len(t.shape) > 1 else (1, t.shape[0])
       typ, buf, data = t.ggml_type, t.buffer, t.data
       is_norm = name.endswith("_norm.weight") or name.endswith(".bias")
@@ -375,7 +378,7 @@ class Transformer:
       sd[name] = (buf, typ, shape)
     if "output.weight" not in sd: sd["output.weight"] = sd["token_embd.weight"]        # tied embeddings, model.py:379
     config = TransformerConfig(
-      num_blocks=kv[f"{arch}.block_count"], dim=dim,
+      num_blocks=num_blocks, dim=dim,
       hidden_dim=kv.get(f"{arch}.expert_feed_forward_length", kv.get(f"{arch}.feed_forward_length", 0)),
       n_heads=n_heads, n_kv_heads=n_kv, norm_eps=kv[f"{arch}.attention.layer_norm_rms_epsilon"], vocab_size=len(kv["tokenizer.ggml.tokens"]),
       head_dim=head_dim, rope_theta=kv[f"{arch}.rope.freq_base"], max_context=max_context,
