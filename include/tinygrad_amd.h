@@ -72,7 +72,7 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  * tinygrad/nn/__init__.py:177 -> Tensor.dot tinygrad/mixin/op.py:367-392 (float32 accumulation, dtype.py:212-216).
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
- * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  K must be a multiple of the type's block size
+ * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
  * (Q4_1 / Q5_0 / Q5_1 are served as block pairs: K % 64 == 0).
  * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K/Q4_1/Q5_0/Q5_1 (GGUF aligns tensor data to 32 bytes,
  * gguf.py:144-148). */
@@ -181,6 +181,35 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
 int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i, void* state, const int* prompt, int* out_tokens, int max_tokens, void* stream);
 /* prompt step that skips the output projection: token = prompt[pos + 1], pos += 1. */
 int tga_advance_prompt(void* state, const int* prompt, void* stream);
+
+/* ---- batched decode: 2..8 sequences in lockstep at one position (the reference's (B, T) token batch, tinygrad/llm/model.py:358-364 with
+ * B > 1; ExpertWeights.__call__ over a (B, T, k) selection, :21-27).  The dense linears take tga_qlinear_multi with M = B. ---- */
+
+/* token_embd(tokens) for n_rows tokens listed in device memory (model.py:359): out (n_rows, dim) float32.  state: the decode record, only
+ * for its vocab / error fields (ids outside [0, vocab) read row 0 and set error bit 0). */
+int tga_embed_rows(const void* table, int ggml_type, int dim, const int32_t* tokens, int n_rows, void* state, float* out, void* stream);
+/* tga_rmsnorm over `rows` rows of dim values (one workgroup per row); outputs (rows, dim). */
+int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream);
+/* tga_attention_decode_normed for `batch` sequences at the shared position state.pos: q (batch, n_heads * head_dim), k / v (batch, n_kv_heads *
+ * head_dim), caches (batch, n_kv_heads, max_ctx, head_dim) fp16, partials batch times the single-sequence workspace, outputs (batch, n_heads * head_dim). */
+int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+/* tga_argmax_step / tga_advance_prompt for a batch: while state.pos + 1 < state.n_prompt the next token of sequence b is prompts[b * prompt_stride +
+ * pos + 1]; otherwise (logits != NULL) the first index of the maximum of logits row b (model.py:364 at temperature 0) goes to tokens[b] and
+ * out_tokens[state.step * batch + b].  Then pos += 1 (and step += 1 when tokens were sampled).  logits NULL: a prompt step without lm-head. */
+int tga_argmax_rows_step(const float* logits, int batch, int n, void* state, const int32_t* prompts, int prompt_stride, int32_t* tokens, int32_t* out_tokens,
+                         int max_steps, void* stream);
+/* Groups the (token, slot) jobs of a batch by expert: table = n_experts records of 16 int32 {number of jobs that selected the expert (at most 8:
+ * the experts of one token are distinct, model.py:35-41, and a batch has at most 8 tokens), their job indices}.  flags: one int32 the caller
+ * zeroes; bit 0 is set when an expert was selected by more than 8 jobs, bit 1 for an expert id outside [0, n_experts) (such jobs are dropped). */
+int tga_expert_jobs(const int32_t* sel, int n_jobs, int n_experts, int32_t* table, int32_t* flags, void* stream);
+/* ExpertWeights.__call__ (model.py:21-27) for the jobs of a batch with every selected expert streamed ONCE: for each expert with jobs, one
+ * small-batch GEMM on the matrix cores over its (N, K) weight and the fp16 activation rows of its jobs (job j reads row j / jobs_per_x_row of
+ * x_f16, writes row j of y (n_jobs, N)); w_up != NULL: y = silu(x Wgate[e]^T) * (x Wup[e]^T) (model.py:129).  Weights are rounded to fp16 once
+ * (the reference's fp16 weight cast, model.py:376), products accumulate in float32.  table from tga_expert_jobs. */
+int tga_qlinear_experts_grouped(int ggml_type, const void* w, const void* w_up, int64_t n_experts, const int32_t* table, int n_jobs, int jobs_per_x_row,
+                                const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
 
 /* ---- MXFP8 MoE prefill path: extra/gemm/cdna_asm_gemm.py, extra/gemm/moe_routing.py, extra/gemm/moe_gemm.py ---- */
 

@@ -80,6 +80,10 @@ class Model:
         kx = c["num_experts_per_tok"]
         logits = self._lin(p + "ffn_gate_inp.weight", n2)
         sel, probs = omoe.gate_probs(logits[None, :], kx, c.get("expert_gating_func", 1), c.get("norm_topk_prob", False), c.get("routed_scaling_factor", 1.0))
+        # how far the selection is from a tie: gap between the k-th and the (k+1)-th router logit (a test that compares token streams reports
+        # it: top-k is discontinuous, an input within rounding noise of a tie may legitimately select another expert)
+        srt = np.sort(logits)
+        self.min_route_gap = min(getattr(self, "min_route_gap", np.inf), float(srt[-kx] - srt[-kx - 1]) if logits.size > kx else np.inf)
         n2l = n2.astype(np.float16).astype(np.float32) if self.act16 else n2
         acc = np.zeros_like(x, dtype=np.float64)
         for sl in range(kx):

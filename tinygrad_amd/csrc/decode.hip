@@ -21,8 +21,10 @@ __device__ __forceinline__ void embed_row_blocks(const uint8_t* __restrict__ tab
     out[e] = o[0]; out[e + 1] = o[1]; out[e + 2] = o[2]; out[e + 3] = o[3];
   }
 }
-__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, DecodeState* st, float* __restrict__ out) {
-  int tok = st->token;
+__global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, DecodeState* st, float* __restrict__ out,
+                                                        const int* __restrict__ tokens) {
+  int tok = tokens ? tokens[blockIdx.x] : st->token;     // batched decode: one workgroup per sequence, its token from the list
+  out += (size_t)blockIdx.x * dim;
   if (tok < 0 || (st->vocab > 0 && tok >= st->vocab)) {         // a token id outside the table (e.g. argmax over NaN logits): row 0 is read instead, the host sees the flag
     if (threadIdx.x == 0) atomicOr(&st->error, 1);
     tok = 0;
@@ -48,6 +50,9 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, int dim, float eps,
                                                        _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu) {
   __shared__ float red[16];
+  x += (size_t)blockIdx.x * dim;                        // one workgroup per row
+  if (out16) out16 += (size_t)blockIdx.x * dim;
+  if (out32) out32 += (size_t)blockIdx.x * dim;
   // two elements per thread and loop pass are requested together and kept for the second pass (rows up to 2048 values never reload)
   float s = 0.f, v0 = 0.f, v1 = 0.f, w0 = 0.f, w1 = 0.f;
   const int e0 = threadIdx.x, e1 = threadIdx.x + 1024;
@@ -101,7 +106,16 @@ struct AttnArgs {
   int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
   const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights: over the whole q / k vectors, or
   int norm_per_head;                                           // per head (weights of head_dim values shared by all heads)
+  // batched decode (sequences in lockstep at one position): sequence z = blockIdx.z (split launch) / blockIdx.y (merge launch) uses the
+  // operands shifted by z times these element strides; all zero for a single sequence
+  long long q_bs, kv_bs, cache_bs, part_bs, out_bs;
 };
+__device__ __forceinline__ AttnArgs attn_args_of_sequence(AttnArgs a, int z) {
+  a.q += z * a.q_bs; a.k += z * a.kv_bs; a.v += z * a.kv_bs; a.cache_k += z * a.cache_bs; a.cache_v += z * a.cache_bs; a.part += z * a.part_bs;
+  if (a.out16) a.out16 += z * a.out_bs;
+  if (a.out32) a.out32 += z * a.out_bs;
+  return a;
+}
 
 __device__ __forceinline__ u32x4 pack8_f16(const float* c) {
   u32x4 r = {f2h_bits(c[0]) | (f2h_bits(c[1]) << 16), f2h_bits(c[2]) | (f2h_bits(c[3]) << 16),
@@ -153,7 +167,7 @@ __device__ __forceinline__ void block_sumsq2(const float* q, int nq, const float
 //   0 none, 1 over the whole q and k vectors of at most 4096 values each (read in one batch), 2 per head, 3 over whole vectors of any length
 template <int HD8, int NORM>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
-  const AttnArgs a = args;                              // field reads become kernel-argument loads in the entry block
+  const AttnArgs a = attn_args_of_sequence(args, blockIdx.z);   // field reads become kernel-argument loads in the entry block
   constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = 4 * RPI, CSTR = HD + 4;
   constexpr int QPL = (HD / 2 + 63) / 64;               // query pairs per lane
   const int kvh = blockIdx.x, split = blockIdx.y;
@@ -364,7 +378,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 // counter, cache-bypassing reads: four dependent memory round trips on the critical path of the last workgroup to arrive).
 template <int HD>
 __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
-  const AttnArgs a = args;                              // field reads become kernel-argument loads in the entry block
+  const AttnArgs a = attn_args_of_sequence(args, blockIdx.y);   // field reads become kernel-argument loads in the entry block
   constexpr int FB = 24, NB = 16;                       // splits read ahead of the position (contexts up to 1536 in one round trip), later batches
   const int head = blockIdx.x, d = threadIdx.x;
   __shared__ float sw[1024];                            // exp(m_s - m) per split
@@ -486,6 +500,37 @@ __global__ void advance_prompt_kernel(DecodeState* st, const int* __restrict__ p
   st->pos = next;
 }
 
+// Batched decode (sequences in lockstep): workgroup b takes sequence b.  While prompt tokens remain the next input of sequence b is
+// prompts[b][pos + 1]; afterwards the first index of the row maximum (logits == nullptr: a prompt step that ran no lm-head) is stored at
+// out_tokens[step][b] and fed back.  The shared position advances in a launch of its own (advance_batch_kernel), after every row has read it.
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restrict__ logits, int n, const DecodeState* st, const int* __restrict__ prompts, int prompt_stride,
+                                                           int* __restrict__ tokens, int* __restrict__ out_tokens, int max_steps, int batch) {
+  const int b = blockIdx.x, next = st->pos + 1;
+  if (next < st->n_prompt || !logits) { if (threadIdx.x == 0 && next < st->n_prompt) tokens[b] = prompts[(size_t)b * prompt_stride + next]; return; }
+  const float* row = logits + (size_t)b * n;
+  float best = -INFINITY; int bi = 0;
+  for (int i = threadIdx.x; i < n; i += 1024) { const float v = row[i]; if (v > best || (v == best && i < bi)) { best = v; bi = i; } }
+  __shared__ float sv[1024]; __shared__ int si[1024];
+  sv[threadIdx.x] = best; si[threadIdx.x] = bi;
+  __syncthreads();
+  for (int o = 512; o > 0; o >>= 1) {
+    if (threadIdx.x < o) {
+      const float v = sv[threadIdx.x + o]; const int i = si[threadIdx.x + o];
+      if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && i < si[threadIdx.x])) { sv[threadIdx.x] = v; si[threadIdx.x] = i; }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    tokens[b] = si[0];
+    if (out_tokens && st->step < max_steps) out_tokens[(size_t)st->step * batch + b] = si[0];
+  }
+}
+__global__ void advance_batch_kernel(DecodeState* st, int had_logits) {
+  const int next = st->pos + 1;
+  if (next >= st->n_prompt && had_logits) st->step += 1;
+  st->pos = next;
+}
+
 // ---------------------------------------------------------------------------------------------- C-ABI
 extern "C" {
 
@@ -495,7 +540,18 @@ int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, 
   switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: blk = 256; break;
     case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_row: unsupported table type %d", ggml_type); }
   TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_row: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
-  embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out);
+  embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out, nullptr);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_embed_rows(const void* table, int ggml_type, int dim, const int32_t* tokens, int n_rows, void* state, float* out, void* stream) {
+  TGA_REQUIRE(table && state && out && tokens && n_rows >= 1, "tga_embed_rows: null pointer or no rows");
+  int blk = 0;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: blk = 256; break;
+    case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_rows: unsupported table type %d", ggml_type); }
+  TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_rows: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
+  embed_row_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out, tokens);
   TGA_LAUNCH_CHECK();
   return 0;
 }
@@ -514,19 +570,23 @@ static int decode_staged_fmt(int ggml_type, long long K, int* nu) {
   return fmt;
 }
 
-int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream) {
+int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(x && weight && (out_f16 || out_f32), "tga_rmsnorm: null pointer");
-  TGA_REQUIRE(dim > 0, "tga_rmsnorm: dim=%d", dim);
+  TGA_REQUIRE(dim > 0 && rows >= 1, "tga_rmsnorm: rows=%d dim=%d", rows, dim);
   int sfmt = 0, snu = 0;
   if (stage_type) { sfmt = decode_staged_fmt(stage_type, dim, &snu); TGA_REQUIRE(sfmt >= 0, "tga_rmsnorm: no staged layout for type %d with K=%d", stage_type, dim); }
-  rmsnorm_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu);
+  rmsnorm_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu);
   TGA_LAUNCH_CHECK();
   return 0;
 }
+int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream) {
+  return tga_rmsnorm_rows(x, weight, 1, dim, eps, out_f16, out_f32, stage_type, stream);
+}
 
-int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
-                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
-                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
+static int attention_launch(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                            int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                            int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
+  TGA_REQUIRE(batch >= 1 && batch <= 65535, "tga_attention_decode: batch=%d", batch);
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table && (out_f16 || out_f32), "tga_attention_decode: null pointer");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
   TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode: head_dim=%d must be 64, 128 or 256", head_dim);
@@ -540,8 +600,10 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
   a.stage_fmt = 0; a.stage_nu = 0;
   a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps; a.norm_per_head = norm_per_head;
+  a.q_bs = (long long)n_heads * head_dim; a.kv_bs = (long long)n_kv_heads * head_dim; a.cache_bs = (long long)n_kv_heads * max_ctx * head_dim;
+  a.part_bs = (long long)n_heads * a.nsplit * (head_dim + 2); a.out_bs = (long long)n_heads * head_dim;
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
-  const dim3 grid(n_kv_heads, a.nsplit);
+  const dim3 grid(n_kv_heads, a.nsplit, batch);
   hipStream_t s = (hipStream_t)stream;
   const int norm = !q_norm_weight ? 0 : norm_per_head ? 2 : ((long long)n_heads * head_dim <= 4096 && (long long)n_kv_heads * head_dim <= 4096) ? 1 : 3;
 #define TGA_ATTN_LAUNCH(HD8) do { \
@@ -552,11 +614,26 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
   else TGA_ATTN_LAUNCH(32);
 #undef TGA_ATTN_LAUNCH
   TGA_LAUNCH_CHECK();
-  if (head_dim == 64) attn_merge_kernel<64><<<n_heads, 64, 0, s>>>(a);
-  else if (head_dim == 128) attn_merge_kernel<128><<<n_heads, 128, 0, s>>>(a);
-  else attn_merge_kernel<256><<<n_heads, 256, 0, s>>>(a);
+  const dim3 mgrid(n_heads, batch);
+  if (head_dim == 64) attn_merge_kernel<64><<<mgrid, 64, 0, s>>>(a);
+  else if (head_dim == 128) attn_merge_kernel<128><<<mgrid, 128, 0, s>>>(a);
+  else attn_merge_kernel<256><<<mgrid, 256, 0, s>>>(a);
   TGA_LAUNCH_CHECK();
   return 0;
+}
+
+int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
+  return attention_launch(1, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+                          rope_table, out_f16, out_f32, stage_type, stream);
+}
+
+int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
+  return attention_launch(batch, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+                          rope_table, out_f16, out_f32, 0, stream);
 }
 
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
@@ -572,6 +649,16 @@ int tga_argmax_step(const float* logits, int n, float* scratch_v, int* scratch_i
   argmax_partial_kernel<<<np, 256, 0, (hipStream_t)stream>>>(logits, n, scratch_v, scratch_i);
   TGA_LAUNCH_CHECK();
   argmax_final_kernel<<<1, 256, 0, (hipStream_t)stream>>>(scratch_v, scratch_i, np, (DecodeState*)state, prompt, out_tokens, max_tokens);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_argmax_rows_step(const float* logits, int batch, int n, void* state, const int32_t* prompts, int prompt_stride, int32_t* tokens, int32_t* out_tokens,
+                         int max_steps, void* stream) {
+  TGA_REQUIRE(state && prompts && tokens && batch >= 1 && (!logits || n > 0), "tga_argmax_rows_step: null pointer or empty rows");
+  argmax_rows_kernel<<<batch, 1024, 0, (hipStream_t)stream>>>(logits, n, (const DecodeState*)state, prompts, prompt_stride, tokens, out_tokens, max_steps, batch);
+  TGA_LAUNCH_CHECK();
+  advance_batch_kernel<<<1, 1, 0, (hipStream_t)stream>>>((DecodeState*)state, logits != nullptr);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -349,6 +349,7 @@ template <> struct Fmt<GGML_F16> {
     c[0] = 0.f;
   }
   static __device__ __forceinline__ float finish(const Raw&, const uint32_t*, const float* a, const float*) { return a[0]; }
+  static __device__ __forceinline__ void to_f16(const Raw&, uint32_t*) {}      // already the fp16 weights
   static __device__ __forceinline__ int spos(int e, int nu) { return e; }
   static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }
 };
@@ -395,6 +396,17 @@ template <> struct Fmt<GGML_MXFP4> {
   // reference value = (2 * e2m1) * 2^(e-128) = e2m1 * 2^(e-127); e = 0 is the fp32 subnormal 2^-127
   static __device__ __forceinline__ float finish(const Raw& r, const uint32_t*, const float* a, const float*) {
     return __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u) * a[0];
+  }
+  // true weights e2m1 * 2^(e-127) as fp16 (exact unless the scale leaves the fp16 range, where the reference's fp16 weight cast saturates too)
+  static __device__ __forceinline__ void to_f16(const Raw& r, uint32_t* wv) {
+    const float sc = __builtin_bit_cast(float, r.e ? (r.e << 23) : 0x00400000u);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      wv[4 * t + 0] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], sc, 0));
+      wv[4 * t + 1] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], sc, 1));
+      wv[4 * t + 2] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], sc, 2));
+      wv[4 * t + 3] = as_u32(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(r.q[t], sc, 3));
+    }
   }
   static __device__ __forceinline__ int spos(int e, int nu) { const int u = e >> 5, b = e & 31, q = b & 15; return (((q >> 2) * nu + u) * 4 + (q & 3)) * 2 + (b >> 4); }
   static __device__ __forceinline__ void cfromx(const u32x4*, float* c) { c[0] = 0.f; }

@@ -366,7 +366,6 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: bw = 64; break;      // served as block pairs
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   const bool align4 = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q4_1 || ggml_type == GGML_Q5_0 || ggml_type == GGML_Q5_1;
-  TGA_REQUIRE(ggml_type != GGML_F16 || M == 1, "tga_qlinear: dense fp16 weights are served for M = 1 only");
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
   TGA_REQUIRE(x, "tga_qlinear: null x");
   QArgs a = {};
@@ -421,6 +420,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     case GGML_Q5_0: return launch_qgemv_m<GGML_Q5_0>(a, M, s);
     case GGML_Q5_1: return launch_qgemv_m<GGML_Q5_1>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
+    case GGML_F16: return launch_qgemv_m<GGML_F16>(a, M, s);
   }
   return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
 }

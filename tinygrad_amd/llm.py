@@ -13,7 +13,7 @@ from dataclasses import dataclass
 import numpy as np
 from tinygrad_amd import runtime as rt
 from tinygrad_amd.runtime import Buffer, GGML_QUANT
-from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine, moe_router
+from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine, moe_router, expert_jobs, experts_grouped
 
 @dataclass(frozen=True)
 class TransformerConfig:
@@ -441,3 +441,143 @@ class Transformer:
       if b.moe: n += b.ffn_gate_inp.nbytes + self.config.num_experts_per_tok * sum(e.expert_nbytes for e in (b.ffn_gate_exps, b.ffn_up_exps, b.ffn_down_exps))
       else: n += sum(l.nbytes for l in (b.ffn_gate, b.ffn_up, b.ffn_down))
     return n
+
+
+class BatchedTransformer:
+  """2..8 sequences decoded in lockstep at one shared position: the reference's forward over a (B, 1) token batch (tinygrad/llm/model.py:358-364).
+  Dense linears run as small-batch GEMMs over the GGUF blocks (M = B); in a MoE block the B * k (token, slot) jobs are grouped by expert, so an
+  expert selected by several tokens is streamed once (ExpertWeights over a (B, T, k) selection, model.py:21-27, 110-135).  Same state dict and
+  config as Transformer; every sequence has its own KV cache; prompts of one batch have equal length."""
+  def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024):
+    if not 1 <= batch <= 8: raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
+    self.config, self.batch, self.max_new = config, batch, max_new
+    c, B = config, batch
+    f32, f16 = np.float32, np.float16
+    lin = lambda name: QuantLinear(state_dict[name][0], state_dict[name][1], *state_dict[name][2])
+    emb = state_dict["token_embd.weight"]
+    self.token_embd, self.embd_type = emb[0], emb[1]
+    self.output_norm = state_dict["output_norm.weight"][0]
+    out = state_dict.get("output.weight", emb)
+    self.output = QuantLinear(out[0], out[1], *out[2])
+    self.blk = []
+    nq, nkv = c.n_heads * c.head_dim, c.n_kv_heads * c.head_dim
+    for i in range(c.num_blocks):
+      p, b = f"blk.{i}.", {}
+      for nm in ("attn_q", "attn_k", "attn_v", "attn_output"): b[nm] = lin(p + nm + ".weight")
+      b["attn_norm"], b["ffn_norm"] = state_dict[p + "attn_norm.weight"][0], state_dict[p + "ffn_norm.weight"][0]
+      b["q_norm"] = state_dict[p + "attn_q_norm.weight"][0] if c.qk_norm else None
+      b["k_norm"] = state_dict[p + "attn_k_norm.weight"][0] if c.qk_norm else None
+      if p + "attn_q.bias" in state_dict:                                # Linear(bias=qkv_bias), model.py:161-163: one bias row per sequence for the additive epilogue
+        b["bias"] = [Buffer.from_numpy(np.tile(state_dict[p + f"attn_{n}.bias"][0].numpy().view(np.uint8).view(f32).reshape(1, -1), (B, 1))) for n in "qkv"]
+      if c.num_experts:
+        ex = lambda name: ExpertWeights(state_dict[p + name][0], state_dict[p + name][1], *state_dict[p + name][2])
+        b["router"] = lin(p + "ffn_gate_inp.weight")
+        b["gate_exps"], b["up_exps"], b["down_exps"] = ex("ffn_gate_exps.weight"), ex("ffn_up_exps.weight"), ex("ffn_down_exps.weight")
+      else:
+        for nm in ("ffn_gate", "ffn_up", "ffn_down"): b[nm] = lin(p + nm + ".weight")
+        if b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
+      b["cache_k"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
+      b["cache_v"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
+      self.blk.append(b)
+    k = max(1, c.num_experts_per_tok)
+    self.state = Buffer((16,), np.int32).zero_()
+    self.tokens = Buffer((B,), np.int32).zero_()
+    self.x, self.xn = Buffer((B, c.dim), f32), Buffer((B, c.dim), f16)
+    self.q, self.k, self.v = Buffer((B, nq), f32), Buffer((B, nkv), f32), Buffer((B, nkv), f32)
+    self.attn = Buffer((B, nq), f16)
+    self.attn_part = Buffer((B * c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
+    self.act = Buffer((B, max(1, c.hidden_dim)), f16)
+    if c.num_experts:
+      self.router_logits, self.sel, self.probs = Buffer((B, c.num_experts), f32), Buffer((B * k,), np.int32), Buffer((B * k,), f32)
+      self.job_table, self.job_flags = Buffer((c.num_experts, 16), np.int32).zero_(), Buffer((1,), np.int32).zero_()
+      self.act_e, self.y_e = Buffer((B * k, c.hidden_dim), f16), Buffer((B * k, c.dim), f32)
+    self.logits_buf = Buffer((B, c.vocab_size), f32)
+    self.rope = Buffer.from_numpy(rope_table(c.head_dim, c.rope_dim or c.head_dim, c.max_context, c.rope_theta))
+    self.prompts = Buffer((B, c.max_context), np.int32).zero_()
+    self.out_tokens = Buffer((max(1, max_new), B), np.int32).zero_()
+    self.stream = rt.Stream()
+    self._graphs, self._steps_done = {}, 0
+
+  def _linear(self, layers, x, outs, **kw): qlinear_multi(layers, x, outs, stream=self.stream.handle, **kw)
+
+  def _step(self, with_head: bool):
+    c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
+    rt.check(L.tga_embed_rows(self.token_embd.ptr, self.embd_type, c.dim, self.tokens.ptr, B, self.state.ptr, self.x.ptr, st))
+    for b in self.blk:
+      # h = x + attention(attn_norm(x))                                                   model.py:149
+      rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["attn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
+      while i < 3:                                                     # one launch per run of equal block types
+        j = i + 1
+        while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
+        bias = dict(epilogue=1, resid=b["bias"][i:j]) if "bias" in b else {}
+        self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
+        i = j
+      rt.check(L.tga_attention_decode_batched(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
+                                              c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
+                                              c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn.ptr, None, st))
+      self._linear([b["attn_output"]], self.attn, [self.x], epilogue=1, resid=[self.x])
+      # x = h + feed_forward(ffn_norm(h))                                                   model.py:150
+      rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      if not c.num_experts:
+        self._linear([b["ffn_gate"], b["ffn_up"]], self.xn, [self.act], epilogue=2)
+        self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
+        continue
+      k = c.num_experts_per_tok                                         # model.py:110-135
+      b["router"](self.xn, out=self.router_logits, stream=st)
+      moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st)
+      expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
+      experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
+      experts_grouped(b["down_exps"], self.job_table, B * k, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
+      moe_combine(self.y_e, self.probs, self.x, B, k, c.dim, self.x, stream=st)
+    if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
+      rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      self.output(self.xn, out=self.logits_buf, stream=st)
+    rt.check(L.tga_argmax_rows_step(self.logits_buf.ptr if with_head else None, B, c.vocab_size, self.state.ptr, self.prompts.ptr, c.max_context, self.tokens.ptr,
+                                    self.out_tokens.ptr, self.max_new, st))
+
+  def _graph(self, with_head: bool) -> rt.Graph:
+    if with_head not in self._graphs:
+      g = rt.Graph(self.stream)
+      with g: self._step(with_head)
+      self._graphs[with_head] = g
+    return self._graphs[with_head]
+
+  def prefill(self, prompts: list[list[int]], use_graph: bool = True):
+    c, B = self.config, self.batch
+    n = len(prompts[0])
+    if len(prompts) != B or any(len(p) != n for p in prompts): raise ValueError(f"need {B} prompts of equal length")
+    if not 1 <= n < c.max_context: raise ValueError(f"prompt of {n} tokens does not fit max_context {c.max_context}")
+    if min(map(min, prompts)) < 0 or max(map(max, prompts)) >= c.vocab_size: raise ValueError(f"token id outside the vocabulary of {c.vocab_size}")
+    pr = np.zeros((B, c.max_context), np.int32); pr[:, :n] = np.array(prompts, np.int32)
+    self.prompts.copyin(pr)
+    self.tokens.copyin(np.ascontiguousarray(pr[:, 0]))
+    st = np.zeros(16, np.int32); st[3], st[5] = n, c.vocab_size
+    self.state.copyin(st)
+    for _ in range(n - 1):
+      if use_graph: self._graph(False).launch()
+      else: self._step(False)
+    self._steps_done = n - 1
+    self.stream.synchronize()
+
+  def decode_step(self, use_graph: bool = True, sync: bool = True):
+    if self._steps_done >= self.config.max_context: raise RuntimeError(f"context full: position {self._steps_done} is beyond max_context {self.config.max_context}")
+    if use_graph: self._graph(True).launch()
+    else: self._step(True)
+    self._steps_done += 1
+    if sync: self.stream.synchronize()
+
+  def generate(self, prompts: list[list[int]], max_new_tokens: int, use_graph: bool = True):
+    """Greedy decoding of every sequence: yields the list of B token ids of each step."""
+    self.prefill(prompts, use_graph)
+    for i in range(min(max_new_tokens, self.config.max_context - len(prompts[0]), self.max_new)):
+      self.decode_step(use_graph)
+      yield [int(t) for t in self.out_tokens.view(4 * i * self.batch, (self.batch,), np.int32).numpy()]
+    self.check_state()
+
+  def check_state(self):
+    err = int(self.state.numpy()[4])
+    flags = int(self.job_flags.numpy()[0]) if self.config.num_experts else 0
+    if err or flags: raise RuntimeError(f"batched decode refused an input: state error {err}, expert grouping flags {flags}")
+
+  def logits(self) -> np.ndarray: return self.logits_buf.numpy()

@@ -114,3 +114,15 @@ def stage_activation(layer: QuantLinear, x: Buffer, out: Buffer | None = None, s
   out = out if out is not None else Buffer((1, layer.in_features), np.float16)
   rt.check(rt.lib().tga_stage_activation(layer.ggml_type, x.ptr, rt.dtype_code(x.dtype), layer.in_features, out.ptr, stream))
   return out
+
+def expert_jobs(sel: Buffer, n_experts: int, table: Buffer, flags: Buffer, stream=None):
+  """Groups the (token, slot) jobs of a batch by expert (table: n_experts x 16 int32; flags: one int32 the caller zeroed)."""
+  rt.check(rt.lib().tga_expert_jobs(sel.ptr, int(np.prod(sel.shape)), n_experts, table.ptr, flags.ptr, stream))
+
+def experts_grouped(w: ExpertWeights, table: Buffer, n_jobs: int, x: Buffer, out: Buffer, jobs_per_x_row: int = 1, up: ExpertWeights | None = None, stream=None) -> Buffer:
+  """ExpertWeights.__call__ for a batch with every selected expert streamed once (tga_qlinear_experts_grouped): x fp16 rows, job j reads row
+  j // jobs_per_x_row and writes row j of out (n_jobs, out_features); with `up`, out = silu(gate) * up."""
+  assert x.dtype == np.float16 and x.shape[-1] == w.in_features
+  rt.check(rt.lib().tga_qlinear_experts_grouped(w.ggml_type, w.blocks.ptr, up.blocks.ptr if up is not None else None, w.num_experts, table.ptr, n_jobs, jobs_per_x_row,
+                                                x.ptr, out.ptr, rt.dtype_code(out.dtype), w.out_features, w.in_features, stream))
+  return out
