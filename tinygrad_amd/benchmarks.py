@@ -99,7 +99,8 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
   import time
   c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **OLMOE)
-  model = Transformer(c, synth_state_moe(c, seed=1004), max_new=steps + 16)
+  model_sd = synth_state_moe(c, seed=1004)
+  model = Transformer(c, model_sd, max_new=steps + 16)
   rt.synchronize()
   rng = np.random.default_rng(1004)
   model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)], use_graph)
@@ -113,6 +114,23 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, {'graph replay' if use_graph else 'eager launches'} + sync per token)",
           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "expert_bytes_per_token": expert_bytes, "weight_bytes_per_token": model.weight_bytes_per_token(),
           "weight_GBps_over_step": round(model.weight_bytes_per_token() / dt / 1e9, 1)}]
+  # batched decode: B sequences in lockstep (dense linears as small-batch GEMMs, the B * 8 expert jobs grouped by expert)
+  from tinygrad_amd.llm import BatchedTransformer
+  sd = {k: v for k, v in model_sd.items()}
+  for B in (2, 4, 8):
+    bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
+    bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)], use_graph)
+    for _ in range(4): bm.decode_step(use_graph)
+    rt.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps): bm.decode_step(use_graph)
+    rt.synchronize()
+    dtb = (time.perf_counter() - t0) / steps
+    bm.check_state()
+    distinct = float(np.mean([len(np.unique(bm.sel.numpy()))]))
+    res.append({"config": 4, "case": f"OLMoE-arch decode B={B} ctx {ctx} (sequences in lockstep, expert jobs grouped by expert; last layer of the last step: {int(distinct)} distinct experts for {B * c.num_experts_per_tok} jobs)",
+                "tok_s": round(B / dtb, 1), "ms_per_step": round(dtb * 1e3, 4)})
+    del bm
   # the expert GEMVs alone: B tokens x 8 experts, gate/up fused then down, distinct experts per slot, layers rotated
   k, s = c.num_experts_per_tok, rt.Stream()
   for B in (1, 2, 4, 8):
