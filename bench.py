@@ -157,6 +157,7 @@ def main():
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
   ap.add_argument("--no-parity", action="store_true", help="skip the parity gate (profiling runs)")
   ap.add_argument("--no-other", action="store_true", help="skip the kernel-level figures of the other configurations")
+  ap.add_argument("--replay", choices=("cmdlist", "graph"), default="cmdlist", help="how the captured step is replayed: plain launches in capture order, or hipGraphLaunch")
   ap.add_argument("--no-graph", action="store_true", help="eager launches instead of graph replay (for kernel-trace profiling)")
   args = ap.parse_args()
   if args.gpus != 1:
@@ -172,6 +173,7 @@ def main():
   c = TransformerConfig(max_context=max_ctx, **cfg)
   sd = synth_state(c, seed=1003)
   model = Transformer(c, sd, max_new=max_new)
+  model.replay = args.replay
   rt.synchronize()
 
   rng = np.random.default_rng(1003)

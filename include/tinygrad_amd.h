@@ -61,6 +61,13 @@ int tga_graph_begin(void* stream);
 int tga_graph_end(void* stream, void** graph_exec);
 int tga_graph_launch(void* graph_exec, void* stream);
 int tga_graph_destroy(void* graph_exec);
+/* The same replay without hipGraphLaunch: tga_graph_begin, the launches, then tga_cmdlist_end keeps the captured kernel launches (function, grid,
+ * block, dynamic LDS, argument values) and tga_cmdlist_launch enqueues them one after the other on the stream, in capture order.  Only kernel
+ * launches captured on one stream are accepted.  Per kernel this costs less on the GPU than a graph node does (0.3-0.5 us measured). */
+int tga_cmdlist_end(void* stream, void** cmdlist);
+int tga_cmdlist_launch(void* cmdlist, void* stream);
+int tga_cmdlist_size(void* cmdlist);
+int tga_cmdlist_destroy(void* cmdlist);
 
 /* ---- block dequant: ggml_data_to_tensor, tinygrad/llm/gguf.py:23-119 (types 2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 41) ----
  * blocks: device pointer to the raw GGUF tensor bytes; n: number of elements (multiple of the block size).
@@ -107,7 +114,7 @@ int tga_moe_combine_rmsnorm_qlinear_multi(const float* y_experts, const float* p
  * registers in the order its in-register decode produces weights, which is a fixed permutation of the row that depends on the
  * weight's (ggml_type, K).  tga_stage_activation writes that permutation as fp16 (K values); a linear then takes it with
  * x_dtype = TGA_F16_STAGED and skips its own staging.  Producers can emit the order directly: tga_rmsnorm / tga_attention_decode
- * (stage_type, stage_K) and tga_qlinear_multi (y_stage_type != 0: the single fp16 output, of length y_stage_K, is written in the
+ * (stage_type, stage_K) and tga_qlinear_multi with the SwiGLU epilogue (y_stage_type != 0: the fp16 output, of length y_stage_K, is written in the
  * staged order of a consumer weight of that type whose K = y_stage_K).  Requires K % 64 == 0 (Q4_K / Q5_K / Q6_K: % 256). */
 int tga_stage_activation(int ggml_type, const void* x, int x_dtype, int64_t K, void* out_f16, void* stream);
 

@@ -748,7 +748,7 @@ template <int EPI>
 __device__ __forceinline__ void store_one(const QArgs& a, int seg, long long row, float v, long long yofs = 0) {
   if constexpr (EPI == 1) v += a.resid[seg][yofs + row];
   if (a.y_f32) ((float*)a.y[seg])[yofs + row] = v;
-  else ((_Float16*)a.y[seg])[yofs + (a.y_stage_fmt ? staged_pos(a.y_stage_fmt, (int)row, a.y_stage_nu) : row)] = (_Float16)v;
+  else ((_Float16*)a.y[seg])[yofs + row] = (_Float16)v;        // (the staged output order exists for the SwiGLU epilogue only: store_swiglu)
 }
 __device__ __forceinline__ void store_swiglu(const QArgs& a, long long row, float gate, float up, long long yofs = 0) {
   const float o = silu_f(gate) * up;

@@ -381,7 +381,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
   }
   a.ntot = (epilogue == 2) ? n[0] : ntot;
   if (y_stage_type) {
-    TGA_REQUIRE(M == 1 && y_dtype == TGA_F16 && (nseg == 1 || epilogue == 2), "tga_qlinear: staged output needs M = 1, fp16 y and a single output");
+    TGA_REQUIRE(M == 1 && y_dtype == TGA_F16 && epilogue == 2, "tga_qlinear: staged output needs M = 1, fp16 y and the SwiGLU epilogue");
     TGA_REQUIRE(y_stage_K == a.ntot, "tga_qlinear: staged output length %lld must equal the output rows %lld", (long long)y_stage_K, (long long)a.ntot);
     a.y_stage_fmt = staged_fmt(y_stage_type, y_stage_K, &a.y_stage_nu);
     TGA_REQUIRE(a.y_stage_fmt >= 0, "tga_qlinear: no staged layout for consumer type %d with K=%lld", y_stage_type, (long long)y_stage_K);

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     cnt = hi > lo ? (hi - lo + RS - 1) / RS : 0;                 // row groups of this team inside the segment
     if (!H && a.team_stride) {                                   // interleaved teams (one matrix): groups team, team + stride, ...
       lo = team * RS; hi = seg_rows;
-      cnt = lo < hi ? ((hi - lo + RS - 1) / RS + a.team_stride - 1) / a.team_stride : 0;
+      cnt = gbase + (team < grem ? 1 : 0);                       // the stride is the number of teams: team_base groups each, one more for the first team_rem (no division here)
     }
     last = hi > 0 ? hi - 1 : 0;                                  // rows beyond the range reload this one (always a valid row)
     base0 = a.w[sg] + eoff;

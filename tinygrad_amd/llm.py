@@ -290,6 +290,7 @@ class Transformer:
     self.stream = rt.Stream()
     self._graphs = {}
     self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
+    self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
 
   def check_state(self):
     """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
@@ -322,9 +323,9 @@ class Transformer:
     else:
       rt.check(L.tga_advance_prompt(s.state.ptr, s.prompt.ptr, st))
 
-  def _graph(self, with_head: bool) -> rt.Graph:
+  def _graph(self, with_head: bool):
     if with_head not in self._graphs:
-      g = rt.Graph(self.stream)
+      g = (rt.CommandList if self.replay == "cmdlist" else rt.Graph)(self.stream)
       with g: self._step(with_head)
       self._graphs[with_head] = g
     return self._graphs[with_head]

@@ -32,6 +32,7 @@ def _declare(lib):
     "tga_event_create": [c_void_pp], "tga_event_destroy": [vp], "tga_event_record": [vp, vp], "tga_event_sync": [vp],
     "tga_event_elapsed_ms": [vp, vp, ctypes.POINTER(ctypes.c_float)],
     "tga_graph_begin": [vp], "tga_graph_end": [vp, c_void_pp], "tga_graph_launch": [vp, vp], "tga_graph_destroy": [vp],
+    "tga_cmdlist_end": [vp, c_void_pp], "tga_cmdlist_launch": [vp, vp], "tga_cmdlist_size": [vp], "tga_cmdlist_destroy": [vp],
     "tga_dequant": [i, vp, i64, vp, i, vp],
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
     "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, i, i64, vp],
@@ -176,6 +177,19 @@ class Graph:
   def launch(self): check(lib().tga_graph_launch(self.handle, self.stream.handle))
   def __del__(self):
     if getattr(self, "handle", None) and _lib is not None: _lib.tga_graph_destroy(ctypes.c_void_p(self.handle)); self.handle = None
+
+class CommandList:
+  """Graph's interface over tga_cmdlist_*: the captured kernel launches are enqueued one after the other instead of going through hipGraphLaunch."""
+  def __init__(self, stream: Stream): self.stream, self.handle = stream, None
+  def __enter__(self): check(lib().tga_graph_begin(self.stream.handle)); return self
+  def __exit__(self, et, ev, tb):
+    p = ctypes.c_void_p(); st = lib().tga_cmdlist_end(self.stream.handle, ctypes.byref(p))
+    if et is None: check(st); self.handle = p.value
+    return False
+  def launch(self): check(lib().tga_cmdlist_launch(self.handle, self.stream.handle))
+  def __len__(self): return lib().tga_cmdlist_size(self.handle)
+  def __del__(self):
+    if getattr(self, "handle", None) and _lib is not None: _lib.tga_cmdlist_destroy(ctypes.c_void_p(self.handle)); self.handle = None
 
 def dtype_code(dt) -> int:
   dt = np.dtype(dt)
