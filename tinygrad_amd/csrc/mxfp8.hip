@@ -260,51 +260,82 @@ __device__ __forceinline__ int gg_tile_of_workgroup(int b, int nwg, int nact, bo
   return nact + (start_g - start_a) + (j - cnt_a);
 }
 
-__device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8_t* smem) {
-  const int tiles_n = g.N / GG_TILE;
-  const int off_end = min(max(g.off[g.E], 0), g.M);             // an offset table that overruns the matrix is clamped to it
-  const int nact = (off_end / GG_TILE) * tiles_n;              // routed row blocks x column blocks
-  bool routed;
-  const int tile = gg_tile_of_workgroup((int)blockIdx.x, (int)gridDim.x, nact, routed);
-  if (tile >= (g.M / GG_TILE) * tiles_n || (!routed && g.routed_only)) return;
-  const int tm = tile / tiles_n, tn = tile % tiles_n;
-  const int row0 = tm * GG_TILE;
-  int lo = 0, hi = g.E;
-  while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (g.off[mid] <= row0) lo = mid; else hi = mid; }
-  const int e = lo;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// A workgroup walks the tiles b, b + gridDim.x, ... of the map above (the C-ABI launch starts one workgroup per CU; a launch with one
+// workgroup per tile, as a PROGRAM bound through Tensor.custom_kernel makes, runs the same code with one trip).  Measured per tile with
+// wall-clock stamps before this loop existed (config 5 gate/up, 16 K steps): 3.6 us until the first stage is in LDS, 36.5 us in the K loop,
+// 6.2 us in the epilogue (manual bf16 rounding, 8-byte stores in 32-byte runs) and 1.1-1.8 us until the CU has its next workgroup.  Here
+//   * the landing registers, which the last K step used to fill with a reload that was dropped, receive the FIRST step of the workgroup's next
+//     tile, so the next tile starts with its operands already in LDS;
+//   * the expert offsets sit in LDS (one read of the table per workgroup, binary search without memory round trips);
+//   * the epilogue rounds with v_cvt_pk_bf16_f32 and turns the accumulators through the idle LDS stage (wave-private 32-row slabs), so that a
+//     store instruction writes eight whole 128-byte row segments.
+#define GG_OFF_MAX 4096                                           // expert offsets 0 .. E kept in LDS when E < GG_OFF_MAX
+#define GG_EPI_PITCH 144                                          // bytes per 64-column bf16 row in the epilogue slab (128 + 16: conflict-free 8-byte writes)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {          // round to nearest even (tinygrad/dtype.py:224-226); one v_cvt_pk_bf16_f32
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+struct GGCur { const uint8_t* A; const uint8_t* B; const uint8_t* sc; int row0, tn; };   // scalar (wave-uniform) state of one tile
+
+__device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8_t* smem, int* s_off) {
+  const int tiles_n = g.N / GG_TILE, tiles_total = (g.M / GG_TILE) * tiles_n;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2, wn = wave & 3;
   const int r16 = lane & 15, kg = lane >> 4;
   const int KB = g.K / 32, nsteps = g.K / 128;
-  const uint8_t* Ag = g.A + (size_t)row0 * g.K;
-  const uint8_t* Bg = g.B + ((size_t)e * g.N + (size_t)tn * GG_TILE) * g.K;
-  // this thread's 4 + 4 chunks per step: rows cpy_r + 64 j, 16-byte piece cpy_c
+  const bool off_in_lds = g.E < GG_OFF_MAX;
+  if (off_in_lds) for (int i = tid; i <= g.E; i += GG_THREADS) s_off[i] = g.off[i];
+  const int off_end = min(max(g.off[g.E], 0), g.M);             // an offset table that overruns the matrix is clamped to it
+  const int nact = (off_end / GG_TILE) * tiles_n;              // routed row blocks x column blocks
+  __syncthreads();
+  // first virtual workgroup index >= b (in steps of the grid size) that has a tile to compute, or -1
+  auto find_tile = [&](int b, int& tile) {
+    for (; b < tiles_total; b += (int)gridDim.x) {
+      bool routed;
+      const int t = gg_tile_of_workgroup(b, tiles_total, nact, routed);
+      if (t < tiles_total && (routed || !g.routed_only)) { tile = t; return b; }
+    }
+    return -1;
+  };
+  auto setup = [&](int tile, GGCur& c) {
+    const int tm = tile / tiles_n;
+    c.tn = tile % tiles_n; c.row0 = tm * GG_TILE;
+    int lo = 0, hi = g.E;                                       // the last expert whose offset is <= the tile's first row
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      const int v = off_in_lds ? __builtin_amdgcn_readfirstlane(s_off[mid]) : g.off[mid];
+      if (v <= c.row0) lo = mid; else hi = mid;
+    }
+    const size_t wrow = (size_t)lo * g.N + (size_t)c.tn * GG_TILE;
+    c.A = g.A + (size_t)c.row0 * g.K;
+    c.B = g.B + wrow * g.K;
+    // scale dwords (the four E8M0 bytes of K blocks 4s .. 4s+3 of one row) travel through LDS too: thread t < 256 copies activation
+    // row t's, thread t >= 256 weight row t - 256's; lane (g, r) of sub-tile i then takes byte g of row 16 i + r
+    c.sc = wave < 4 ? g.a_e8 + (size_t)c.row0 * KB : g.b_e8 + wrow * KB;
+  };
+  // this thread's 4 + 4 chunks per step: rows cpy_r + 64 j, 16-byte piece cpy_c (a 32-bit offset from the tile's scalar base)
   const int cpy_c = tid & 7, cpy_r = tid >> 3;
   int cpy_off[4];
 #pragma unroll
   for (int j = 0; j < 4; j++) cpy_off[j] = gg_slot_off(cpy_r + 64 * j, cpy_c);
-  const uint8_t* a_src = Ag + (size_t)cpy_r * g.K + cpy_c * 16;
-  const uint8_t* b_src = Bg + (size_t)cpy_r * g.K + cpy_c * 16;
-  // scale dwords (the four E8M0 bytes of K blocks 4s .. 4s+3 of one row) travel through LDS too: thread t < 256 copies activation
-  // row t's, thread t >= 256 weight row t - 256's; lane (g, r) of sub-tile i then takes byte g of row 16 i + r
-  const uint8_t* sc_src = tid < GG_TILE ? g.a_e8 + (size_t)(row0 + tid) * KB : g.b_e8 + ((size_t)e * g.N + (size_t)tn * GG_TILE + (tid - GG_TILE)) * KB;
+  const uint32_t cpy_voff = (uint32_t)cpy_r * (uint32_t)g.K + (uint32_t)cpy_c * 16u;
+  const uint32_t sc_voff = (uint32_t)(tid & (GG_TILE - 1)) * (uint32_t)KB;
+  const size_t rows64 = (size_t)64 * g.K;
   // fragment read offsets of this lane inside a sub-tile (plane 0 / plane 1)
   const int f0 = ((16 * kg + (r16 ^ kg)) << 4), f1 = 1024 + ((16 * kg + (r16 ^ (kg + 4))) << 4);
 
-  v4f32 acc[8][4];                                            // [m sub-tile][n sub-tile]
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
-
   u32x4 stg_a[4], stg_b[4]; uint32_t stg_sc;
-  auto load_step = [&](int s) {
+  // one of the nine loads of a step: 2 j = activation rows cpy_r + 64 j, 2 j + 1 = weight rows, 8 = the scale dword
+  auto load_piece = [&](const GGCur& c, int s, int which) {
+    const size_t ks = (size_t)s * 128;
+    if (which == 8) stg_sc = *(const uint32_t*)(c.sc + 4 * s + sc_voff);
+    else if (which & 1) stg_b[which >> 1] = *(const u32x4*)(c.B + ks + (which >> 1) * rows64 + cpy_voff);
+    else stg_a[which >> 1] = *(const u32x4*)(c.A + ks + (which >> 1) * rows64 + cpy_voff);
+  };
+  auto load_step = [&](const GGCur& c, int s) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      stg_a[j] = *(const u32x4*)(a_src + (size_t)(64 * j) * g.K + (size_t)s * 128);
-      stg_b[j] = *(const u32x4*)(b_src + (size_t)(64 * j) * g.K + (size_t)s * 128);
-    }
-    stg_sc = *(const uint32_t*)(sc_src + 4 * s);
+    for (int w = 0; w < 9; w++) load_piece(c, s, w);
   };
   auto store_step = [&](int stage) {
     uint8_t* base = smem + stage * GG_STAGE_BYTES;
@@ -312,55 +343,108 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
     for (int j = 0; j < 4; j++) { *(u32x4*)(base + cpy_off[j]) = stg_a[j]; *(u32x4*)(base + GG_TILE * 128 + cpy_off[j]) = stg_b[j]; }
     ((uint32_t*)(base + 2 * GG_TILE * 128))[tid] = stg_sc;
   };
-  load_step(0);
+
+  int tile;
+  int b = find_tile((int)blockIdx.x, tile);
+  if (b < 0) return;
+  GGCur cur;
+  setup(tile, cur);
+  load_step(cur, 0);
   store_step(0);
   __syncthreads();
-  for (int s = 0; s < nsteps; s++) {
-    load_step(s + 1 < nsteps ? s + 1 : s);                    // the last step reloads itself (dropped)
-    __builtin_amdgcn_sched_barrier(0);                        // the loads of the next step stay ahead of this step's MFMAs
-    const uint8_t* base = smem + (s & 1) * GG_STAGE_BYTES;
-    const uint8_t* As = base + wm * 8 * 2048;
-    const uint8_t* Bs = base + GG_TILE * 128 + wn * 4 * 2048;
-    const uint32_t* sA = (const uint32_t*)(base + 2 * GG_TILE * 128) + wm * 128 + r16;
-    const uint32_t* sB = (const uint32_t*)(base + 2 * GG_TILE * 128) + GG_TILE + wn * 64 + r16;
-    v8i32 bf[4]; int sb[4];
+  int par = 0;                                                   // LDS stage of the current tile's step 0
+  while (true) {
+    int tile_n;
+    const int bn = find_tile(b + (int)gridDim.x, tile_n);
+    GGCur nxt = cur;
+    if (bn >= 0) setup(tile_n, nxt);
+    const int nxt_step = bn >= 0 ? 0 : nsteps - 1;             // no further tile: the last step reloads itself (dropped)
+
+    v4f32 acc[8][4];                                            // [m sub-tile][n sub-tile]
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const u32x4 y0 = *(const u32x4*)(Bs + j * 2048 + f0), y1 = *(const u32x4*)(Bs + j * 2048 + f1);
-      bf[j] = v8i32{(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
-      sb[j] = (int)(sB[16 * j] >> (8 * kg));
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
+
+    for (int s = 0; s < nsteps; s++) {
+      const bool lastk = s + 1 == nsteps;
+      GGCur src = cur;
+      if (lastk) src = nxt;
+      // The loads of the next step (of this tile, or the first step of the next tile) are issued one per sub-tile, between the MFMA groups: a
+      // CU takes 24-38 cycles to accept a 64 x 16-byte load, so the 72 loads of a step issued together held the last wave back by 1.1 us
+      // before it could start multiplying (measured with wall-clock stamps per phase), and the barrier passed that on to every wave.
+      const int ls = lastk ? nxt_step : s + 1;
+      load_piece(src, ls, 8);
+      const uint8_t* base = smem + ((par + s) & 1) * GG_STAGE_BYTES;
+      const uint8_t* As = base + wm * 8 * 2048;
+      const uint8_t* Bs = base + GG_TILE * 128 + wn * 4 * 2048;
+      const uint32_t* sA = (const uint32_t*)(base + 2 * GG_TILE * 128) + wm * 128 + r16;
+      const uint32_t* sB = (const uint32_t*)(base + 2 * GG_TILE * 128) + GG_TILE + wn * 64 + r16;
+      v8i32 bf[4]; int sb[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const u32x4 y0 = *(const u32x4*)(Bs + j * 2048 + f0), y1 = *(const u32x4*)(Bs + j * 2048 + f1);
+        bf[j] = v8i32{(int)y0.x, (int)y0.y, (int)y0.z, (int)y0.w, (int)y1.x, (int)y1.y, (int)y1.z, (int)y1.w};
+        sb[j] = (int)(sB[16 * j] >> (8 * kg));
+      }
+      // the activation fragment of sub-tile i + 1 is requested before the MFMAs of sub-tile i are issued: they run while it arrives
+      auto frag = [&](int i, v8i32& af, int& sa) {
+        const u32x4 x0 = *(const u32x4*)(As + i * 2048 + f0), x1 = *(const u32x4*)(As + i * 2048 + f1);
+        af = v8i32{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
+        sa = (int)sA[16 * i];
+      };
+      v8i32 af[2]; int sa[2];
+      frag(0, af[0], sa[0]);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        if (i + 1 < 8) frag(i + 1, af[(i + 1) & 1], sa[(i + 1) & 1]);
+        load_piece(src, ls, i);
+        __builtin_amdgcn_sched_barrier(0);
+        const int sai = sa[i & 1] >> (8 * kg);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, 0, sb[j], 0, sai);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      store_step((par + s + 1) & 1);
+      __syncthreads();
     }
+    // ---- epilogue.  The stage the last step was read from is idle now (the other one already holds the next tile's first step).  A lane holds
+    // output row (activation row) r16 of m sub-tile i, columns 4 kg .. 4 kg + 3 of n sub-tile j; 32 rows at a time go through the wave's slab.
+    {
+      uint8_t* slab = smem + ((par + nsteps - 1) & 1) * GG_STAGE_BYTES + wave * (32 * GG_EPI_PITCH);
+      uint16_t* cw = g.C + (size_t)(cur.row0 + wm * 128) * g.N + (size_t)cur.tn * GG_TILE + wn * 64;
+      const int rrow = lane >> 3, rc = lane & 7;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const u32x4 x0 = *(const u32x4*)(As + i * 2048 + f0), x1 = *(const u32x4*)(As + i * 2048 + f1);
-      const v8i32 af = v8i32{(int)x0.x, (int)x0.y, (int)x0.z, (int)x0.w, (int)x1.x, (int)x1.y, (int)x1.z, (int)x1.w};
-      const int sa = (int)(sA[16 * i] >> (8 * kg));
+      for (int q = 0; q < 4; q++) {
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af, acc[i][j], 0, 0, 0, sb[j], 0, sa);
+        for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const v4f32 v = acc[2 * q + ii][j];
+            *(u32x2*)(slab + (16 * ii + r16) * GG_EPI_PITCH + 32 * j + 8 * kg) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // LDS operations of a wave execute in order: ordering for the compiler only
+        u32x4 o[4];
+#pragma unroll
+        for (int p2 = 0; p2 < 4; p2++) o[p2] = *(const u32x4*)(slab + (rrow + 8 * p2) * GG_EPI_PITCH + 16 * rc);
+#pragma unroll
+        for (int p2 = 0; p2 < 4; p2++) *(u32x4*)(cw + (size_t)(32 * q + rrow + 8 * p2) * g.N + 8 * rc) = o[p2];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);
-    store_step((s + 1) & 1);
-    __syncthreads();
-  }
-  // lane: output row (activation row) r16 of m sub-tile i, columns 4 kg .. 4 kg + 3 of n sub-tile j
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    uint16_t* crow = g.C + (size_t)(row0 + wm * 128 + 16 * i + r16) * g.N + (size_t)tn * GG_TILE + wn * 64 + 4 * kg;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const v4f32 v = acc[i][j];
-      u32x2 o = {(uint32_t)f_to_bf16(v[0]) | ((uint32_t)f_to_bf16(v[1]) << 16), (uint32_t)f_to_bf16(v[2]) | ((uint32_t)f_to_bf16(v[3]) << 16)};
-      *(u32x2*)(crow + 16 * j) = o;
-    }
+    if (bn < 0) break;
+    __syncthreads();                                             // the slabs are free before any wave's next step writes that stage
+    par = (par + nsteps) & 1; cur = nxt; b = bn;
   }
 }
-
 
 // C-ABI launch: arguments in one by-value record.
 __global__ __launch_bounds__(GG_THREADS) void grouped_mxfp8_gemm_lds_kernel(const GemmArgs g) {
   __shared__ __attribute__((aligned(16))) uint8_t smem[2 * GG_STAGE_BYTES];   // [stage][A 32 KB | B 32 KB | 512 scale dwords]
-  grouped_mxfp8_gemm_tile(g, smem);
+  __shared__ int s_off[GG_OFF_MAX];
+  grouped_mxfp8_gemm_tile(g, smem, s_off);
 }
 
 // The same kernel with the argument list a pre-compiled PROGRAM bound through Tensor.custom_kernel hands over: one pointer per buffer in
@@ -371,9 +455,10 @@ extern "C" __global__ __launch_bounds__(GG_THREADS) void tga_grouped_mxfp8_gemm_
                                                                                         const uint32_t* w_si, const uint8_t* x_e8, const uint8_t* w_e8,
                                                                                         const int* expert_off, int M, int N, int K, int E) {
   __shared__ __attribute__((aligned(16))) uint8_t smem[2 * GG_STAGE_BYTES];
+  __shared__ int s_off[GG_OFF_MAX];
   (void)x_si; (void)w_si;
   GemmArgs g; g.C = C; g.A = A; g.B = B; g.a_e8 = x_e8; g.b_e8 = w_e8; g.off = expert_off; g.M = M; g.N = N; g.K = K; g.E = E; g.routed_only = 0;
-  grouped_mxfp8_gemm_tile(g, smem);
+  grouped_mxfp8_gemm_tile(g, smem, s_off);
 }
 
 // clamped, interleaved SwiGLU between the two grouped GEMMs (examples/mlperf/models/gpt_oss.py:94-98): bf16 in/out
@@ -523,7 +608,10 @@ static int grouped_mxfp8_gemm_launch(void* C, const void* A, const void* B, cons
               "tga_grouped_mxfp8_gemm: empty or oversized problem (%lld, %lld, %lld), %d experts", (long long)M, (long long)N, (long long)K, n_experts);
   GemmArgs g; g.C = (uint16_t*)C; g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.a_e8 = (const uint8_t*)x_e8; g.b_e8 = (const uint8_t*)w_e8;
   g.off = expert_off; g.M = (int)M; g.N = (int)N; g.K = (int)K; g.E = n_experts; g.routed_only = routed_only;
-  grouped_mxfp8_gemm_lds_kernel<<<(unsigned)((M / GG_TILE) * (N / GG_TILE)), GG_THREADS, 0, (hipStream_t)stream>>>(g);
+  // one workgroup per CU (its 148 KB of LDS fill the CU anyway); each walks its share of the tiles
+  static const int n_cu = [] { int dev = 0, n = 0; return (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256; }();
+  const long long tiles = (M / GG_TILE) * (N / GG_TILE);
+  grouped_mxfp8_gemm_lds_kernel<<<(unsigned)(tiles < n_cu ? tiles : n_cu), GG_THREADS, 0, (hipStream_t)stream>>>(g);
   TGA_LAUNCH_CHECK();
   return 0;
 }
