@@ -337,11 +337,15 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
 #pragma unroll
     for (int w = 0; w < 9; w++) load_piece(c, s, w);
   };
-  auto store_step = [&](int stage) {
+  auto store_piece = [&](int stage, int which) {
     uint8_t* base = smem + stage * GG_STAGE_BYTES;
+    if (which == 8) ((uint32_t*)(base + 2 * GG_TILE * 128))[tid] = stg_sc;
+    else if (which & 1) *(u32x4*)(base + GG_TILE * 128 + cpy_off[which >> 1]) = stg_b[which >> 1];
+    else *(u32x4*)(base + cpy_off[which >> 1]) = stg_a[which >> 1];
+  };
+  auto store_step = [&](int stage) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) { *(u32x4*)(base + cpy_off[j]) = stg_a[j]; *(u32x4*)(base + GG_TILE * 128 + cpy_off[j]) = stg_b[j]; }
-    ((uint32_t*)(base + 2 * GG_TILE * 128))[tid] = stg_sc;
+    for (int w = 0; w < 9; w++) store_piece(stage, w);
   };
 
   int tile;
@@ -398,16 +402,18 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         if (i + 1 < 8) frag(i + 1, af[(i + 1) & 1], sa[(i + 1) & 1]);
-        load_piece(src, ls, i);
+        if (i < 4) { load_piece(src, ls, 2 * i); load_piece(src, ls, 2 * i + 1); }
         __builtin_amdgcn_sched_barrier(0);
         const int sai = sa[i & 1] >> (8 * kg);
 #pragma unroll
         for (int j = 0; j < 4; j++)
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, 0, sb[j], 0, sai);
         __builtin_amdgcn_sched_barrier(0);
+        // the other stage was last read one step ago: the landed pieces go there while the second half of the MFMAs runs
+        if (i >= 4) { store_piece((par + s + 1) & 1, 2 * (i - 4)); store_piece((par + s + 1) & 1, 2 * (i - 4) + 1); __builtin_amdgcn_sched_barrier(0); }
       }
       __builtin_amdgcn_sched_barrier(0);
-      store_step((par + s + 1) & 1);
+      store_piece((par + s + 1) & 1, 8);
       __syncthreads();
     }
     // ---- epilogue.  The stage the last step was read from is idle now (the other one already holds the next tile's first step).  A lane holds
