@@ -15,8 +15,9 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE) of
 # `python -m tinygrad_amd.benchmarks --traffic`, each scaled by what the same counter reads for a 1 GiB copy kernel (x2.0000 and x1.0000):
-# 66 609 152 B fetched + 93 389 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
-GATE_UP_TRAFFIC_BYTES = 66702500
+# 66 514 125 B fetched + 71 680 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
+GATE_UP_TRAFFIC_BYTES = 66585805
+GATE_UP_ROCPROF_AVG_US = 14.88    # rocprofv3 --kernel-trace --stats average of the same kernel (profiles/decode_llama3_8b_q4_0_kernel_stats.md)
 PARITY_TOL = 1e-3
 
 def _host_layer(model, i):
@@ -260,8 +261,11 @@ def main():
                      "traffic": GATE_UP_TRAFFIC_BYTES if c.num_blocks == 32 else None,
                      "traffic_source": "recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run",
                      "avg_launch_us": dom["avg_us"], "alg_bytes_per_launch": dom["alg_bytes"],
-                     "timing": "HIP events on the launch stream around the 32 gate/up launches of all blocks issued back to back, three repetitions; the rocprofv3 kernel-trace "
-                               "average of the same kernel inside the decode step is in profiles/decode_llama3_8b_q4_0_kernel_stats.md",
+                     "rocprof_avg_us": GATE_UP_ROCPROF_AVG_US if c.num_blocks == 32 else None,
+                     "frac_by_rocprof_avg": round(dom["alg_bytes"] / GATE_UP_ROCPROF_AVG_US / 1e3 / HBM_PEAK_GBS, 4) if c.num_blocks == 32 else None,
+                     "timing": "achieved / frac: HIP events on the launch stream around the 32 gate/up launches of all blocks issued back to back, three repetitions (live, this run); "
+                               "rocprof_avg_us / frac_by_rocprof_avg: the recorded rocprofv3 kernel-trace average of the same kernel in an eagerly launched decode "
+                               "(profiles/decode_llama3_8b_q4_0_kernel_stats.md), not re-measured by this run",
                      "share_of_block_time": round(dom["avg_us"] / per_block, 3),
                      "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
   if parity is not None: out["parity"] = parity
