@@ -138,6 +138,11 @@ int tga_qlinear_experts_routed(int ggml_type, const void* w_gate, const void* w_
  * gathered / renormalised / scaled.  logits (n_tokens, n_experts) float32 -> sel (n_tokens, k) int32, probs (n_tokens, k). */
 int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int gating, int norm_topk_prob, float scale,
                  int32_t* sel, float* probs, void* stream);
+/* The same with the expert selection bias of model.py:113, 123 (`exp_probs_b`): experts are ranked by score + selection_bias[e] (n_experts
+ * float32), the probabilities are gathered from the unbiased scores; with a bias the SOFTMAX + norm_topk_prob shortcut of model.py:116-117
+ * does not apply, as in the reference. */
+int tga_moe_gate_biased(const float* logits, const float* selection_bias, int n_tokens, int n_experts, int k, int gating, int norm_topk_prob, float scale,
+                        int32_t* sel, float* probs, void* stream);
 /* Router of ONE token in one launch (model.py:112-128 with the block's ffn_norm, :150): h = fp16(RMSNorm(x) * norm_weight) (norm_weight
  * NULL: h = fp16(x)), logits = h @ Wr^T for a dense fp16 router weight (n_experts, dim), then gating + top-k as tga_moe_gate.
  * xn_out_f16 (dim fp16, the activation of the expert GEMVs) may be NULL.  logits_ws: n_experts floats (the logits, readable

@@ -39,6 +39,7 @@ def from_gguf_weights(raw: bytes):
   sd = {k: v.astype(np.float16).astype(np.float32) for k, v in sd.items()}                      # model.py:376
   if "output.weight" not in sd: sd["output.weight"] = sd["token_embd.weight"]                    # model.py:379
   arch = kv["general.architecture"]
+  if arch in ("qwen35", "qwen35moe", "glm4moe"): sd = {k.replace("post_attention_norm", "ffn_norm"): v for k, v in sd.items()}   # model.py:403-404
   H, KV = kv[f"{arch}.attention.head_count"], kv[f"{arch}.attention.head_count_kv"]
   for name in list(sd):
     if arch == "llama" and "attn_q.weight" in name:
@@ -48,7 +49,8 @@ def from_gguf_weights(raw: bytes):
       w = sd[name].reshape(KV, sd[name].shape[0] // KV, -1)
       sd[name] = w.reshape(KV, -1, 2, w.shape[-1]).transpose(0, 2, 1, 3).reshape(-1, w.shape[-1])
   dim = kv[f"{arch}.embedding_length"]
-  cfg = dict(num_blocks=kv[f"{arch}.block_count"], dim=dim, hidden_dim=kv.get(f"{arch}.expert_feed_forward_length", kv.get(f"{arch}.feed_forward_length", 0)),
+  cfg = dict(num_blocks=kv[f"{arch}.block_count"] - kv.get(f"{arch}.nextn_predict_layers", 0), dim=dim,
+             leading_dense_blocks=kv.get(f"{arch}.leading_dense_block_count", 0),                  # model.py:438; the other MoE extras are read off the tensors hidden_dim=kv.get(f"{arch}.expert_feed_forward_length", kv.get(f"{arch}.feed_forward_length", 0)),
              n_heads=H, n_kv_heads=KV, norm_eps=kv[f"{arch}.attention.layer_norm_rms_epsilon"], vocab_size=len(kv["tokenizer.ggml.tokens"]),
              head_dim=kv.get(f"{arch}.attention.key_length", dim // H), rope_theta=kv[f"{arch}.rope.freq_base"],
              rope_dim=kv.get(f"{arch}.rope.dimension_count", kv.get(f"{arch}.attention.key_length", dim // H)),   # model.py:406

@@ -76,13 +76,14 @@ class Model:
       attn = np.einsum("ht,htd->hd", pr, V).astype(np.float32).reshape(-1)
       h = x + self._lin(p + "attn_output.weight", attn)
       n2 = rmsnorm(h, self.w[p + "ffn_norm.weight"].reshape(-1), eps)
-      if c.get("num_experts", 0):                                           # model.py:110-135
+      if c.get("num_experts", 0) and i >= c.get("leading_dense_blocks", 0):   # model.py:84 (leading blocks stay dense), 110-135
         kx = c["num_experts_per_tok"]
         logits = self._lin(p + "ffn_gate_inp.weight", n2)
-        sel, probs = omoe.gate_probs(logits[None, :], kx, c.get("expert_gating_func", 1), c.get("norm_topk_prob", False), c.get("routed_scaling_factor", 1.0))
+        bias = self.w[p + "exp_probs_b.bias"].reshape(-1) if p + "exp_probs_b.bias" in self.w else None     # model.py:113, 123: ranks by score + bias
+        sel, probs = omoe.gate_probs(logits[None, :], kx, c.get("expert_gating_func", 1), c.get("norm_topk_prob", False), c.get("routed_scaling_factor", 1.0), bias=bias)
         # how far the selection is from a tie: gap between the k-th and the (k+1)-th router logit (a test that compares token streams reports
         # it: top-k is discontinuous, an input within rounding noise of a tie may legitimately select another expert)
-        srt = np.sort(logits)
+        srt = np.sort(logits if bias is None else omoe.gate_scores(logits, c.get("expert_gating_func", 1)) + bias)
         self.min_route_gap = min(getattr(self, "min_route_gap", np.inf), float(srt[-kx] - srt[-kx - 1]) if logits.size > kx else np.inf)
         n2l = n2.astype(np.float16).astype(np.float32) if self.act16 else n2
         acc = np.zeros_like(x, dtype=np.float64)
@@ -93,7 +94,14 @@ class Model:
           a = silu(g) * u
           if self.act16: a = a.astype(np.float16).astype(np.float32)
           acc += np.float64(probs[0, sl]) * (a.astype(np.float64) @ self.w[p + "ffn_down_exps.weight"][e].astype(np.float64).T).astype(np.float32)
-        x = h + acc.astype(np.float32)
+        out = acc.astype(np.float32)
+        if p + "ffn_gate_shexp.weight" in self.w:                             # model.py:131-134: the shared expert, optionally scaled by a sigmoid gate
+          sh = self._lin(p + "ffn_down_shexp.weight", silu(self._lin(p + "ffn_gate_shexp.weight", n2)) * self._lin(p + "ffn_up_shexp.weight", n2))
+          if p + "ffn_gate_inp_shexp.weight" in self.w:
+            gl = self._lin(p + "ffn_gate_inp_shexp.weight", n2).reshape(-1)[0]          # (x * w).sum(-1)
+            sh = sh * (np.float32(1.0) / (np.float32(1.0) + np.exp(-gl)))
+          out = out + sh
+        x = h + out
         self.last_sel = sel[0]
       else:
         x = h + self._lin(p + "ffn_down.weight", silu(self._lin(p + "ffn_gate.weight", n2)) * self._lin(p + "ffn_up.weight", n2))

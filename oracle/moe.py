@@ -24,6 +24,14 @@ def softmax(x, axis=-1):
   e = np.exp(x - x.max(axis=axis, keepdims=True))
   return e * (1.0 / e.sum(axis=axis, keepdims=True))
 
+def gate_scores(logits: np.ndarray, gating=SOFTMAX) -> np.ndarray:
+  """The scores the selection bias is added to (model.py:118-121)."""
+  logits = logits.astype(np.float32)
+  if gating == SOFTMAX_WEIGHT: return logits
+  if gating == SOFTMAX: return softmax(logits)
+  if gating == SIGMOID: return 1.0 / (1.0 + np.exp(-logits))
+  return np.sqrt(np.log1p(np.exp(logits)))
+
 def gate_probs(logits: np.ndarray, k: int, gating=SOFTMAX, norm_topk_prob=False, scale=1.0, bias=None):
   """model.py:112-128 -> (sel (.., k) int32, probs (.., k) float32)."""
   logits = logits.astype(np.float32)

@@ -271,3 +271,56 @@ def test_from_gguf_partial_rotary(gpu, tmp_path):
   o3 = ollm.Model(dict(cfg, rope_dim=hd), weights, 64, w_round_f16=False, act_round_f16=False)
   for pos, t in enumerate(prompt + ref[:-1]): lg3 = o3.forward(t, pos)
   assert ol.rel_err(lg3, lg) > 0.01
+
+def test_from_gguf_glm4moe_shape(gpu, tmp_path):
+  """A GLM-4.5-shaped file (model.py:403-404, 424, 434-443): `post_attention_norm` tensor names, one leading dense block with its own FFN width, sigmoid
+  gating with `exp_probs_b` selection biases, normalised and scaled top-k weights, one shared expert (`expert_shared_count` x the expert width), q / k / v
+  biases, partial rotary, and a trailing next-token-prediction layer that the decoder must not load."""
+  from tinygrad_amd.llm import Transformer
+  from tinygrad_amd.gguf import gguf_write
+  rng = np.random.default_rng(91)
+  dim, hidden, dense_hidden, H, KV, hd, rd, L, vocab, E, k = 256, 128, 512, 4, 2, 64, 32, 3, 512, 8, 2
+  def lin(*shape): return (rng.uniform(-1, 1, shape) * shape[-1] ** -0.5).astype(np.float32)
+  q8 = lambda name, *shape, amp=1.0: (name, shape, 8, og.quantize_q8_0(lin(*shape) * amp))
+  f32 = lambda name, n, mean=1.0, sd=0.2: (name, (n,), 0, (mean + sd * rng.standard_normal(n)).astype(np.float32))
+  tensors = [q8("token_embd.weight", vocab, dim, amp=16.0)]
+  for i in range(L + 1):                                                # block L is the next-token-prediction layer
+    p = f"blk.{i}."
+    tensors += [f32(p + "attn_norm.weight", dim), q8(p + "attn_q.weight", H * hd, dim), f32(p + "attn_q.bias", H * hd, 0.0, 0.3), q8(p + "attn_k.weight", KV * hd, dim),
+                f32(p + "attn_k.bias", KV * hd, 0.0, 0.3), q8(p + "attn_v.weight", KV * hd, dim), f32(p + "attn_v.bias", KV * hd, 0.0, 0.3),
+                q8(p + "attn_output.weight", dim, H * hd), f32(p + "post_attention_norm.weight", dim)]
+    if i == 0:
+      tensors += [q8(p + "ffn_gate.weight", dense_hidden, dim), q8(p + "ffn_up.weight", dense_hidden, dim), q8(p + "ffn_down.weight", dim, dense_hidden)]
+    else:
+      tensors += [(p + "ffn_gate_inp.weight", (E, dim), 0, lin(E, dim) * 4), f32(p + "exp_probs_b.bias", E, 0.0, 0.3),
+                  q8(p + "ffn_gate_exps.weight", E, hidden, dim), q8(p + "ffn_up_exps.weight", E, hidden, dim), q8(p + "ffn_down_exps.weight", E, dim, hidden),
+                  q8(p + "ffn_gate_shexp.weight", hidden, dim), q8(p + "ffn_up_shexp.weight", hidden, dim), q8(p + "ffn_down_shexp.weight", dim, hidden)]
+    if i == L: tensors += [f32(p + "nextn.enorm.weight", dim), q8(p + "nextn.eh_proj.weight", dim, 2 * dim)]
+  tensors += [f32("output_norm.weight", dim), q8("output.weight", vocab, dim)]
+  a = "glm4moe"
+  kvs = [("general.architecture", a), (f"{a}.context_length", 96), (f"{a}.attention.head_count", H), (f"{a}.attention.head_count_kv", KV),
+         (f"{a}.attention.key_length", hd), (f"{a}.rope.dimension_count", rd), (f"{a}.block_count", L + 1), (f"{a}.nextn_predict_layers", 1),
+         (f"{a}.embedding_length", dim), (f"{a}.feed_forward_length", dense_hidden), (f"{a}.expert_feed_forward_length", hidden),
+         (f"{a}.expert_count", E), (f"{a}.expert_used_count", k), (f"{a}.expert_shared_count", 1), (f"{a}.leading_dense_block_count", 1),
+         (f"{a}.expert_gating_func", 2), (f"{a}.expert_weights_norm", True), (f"{a}.expert_weights_scale", 1.5),
+         (f"{a}.attention.layer_norm_rms_epsilon", 1e-5), (f"{a}.rope.freq_base", 10000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(vocab)])]
+  path = tmp_path / "glm4moe.gguf"
+  raw = gguf_write(path, kvs, tensors)
+  model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
+  c = model.config
+  assert (c.num_blocks, c.leading_dense_blocks, c.dense_hidden_dim, c.shared_expert_dim, c.shared_expert_gate, c.expert_bias) == (L, 1, dense_hidden, hidden, False, True)
+  assert c.expert_gating_func == 2 and c.norm_topk_prob and c.routed_scaling_factor == 1.5 and c.rope_dim == rd
+  assert [b.moe for b in model.blk] == [False, True, True]
+  cfg, weights, _ = ogguf.from_gguf_weights(raw)
+  assert cfg["num_blocks"] == L and cfg["leading_dense_blocks"] == 1 and "blk.1.ffn_norm.weight" in weights
+  prompt = [9, 100, 321, 5, 77, 410]
+  got = list(model.generate(prompt, 16))
+  o = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False)
+  ref, margins = o.generate(prompt, 16)
+  print(f"min top-2 margin {min(margins):.4f}, min biased-score gap {o.min_route_gap:.2e}")
+  assert got == ref
+  o2 = ollm.Model(cfg, weights, 64, w_round_f16=False, act_round_f16=False); pos = 0
+  for t in prompt[:-1]: o2.forward(t, pos); pos += 1
+  cur = prompt[-1]
+  for _ in range(16): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
+  assert ol.rel_err(model.logits(), lg) <= 1e-3

@@ -156,3 +156,61 @@ def test_small_olmoe_decode(gpu):
   print(f"oracle (reference numerics) min top-2 margin over 32 steps {margin:.4f} (logit rms {rms:.4f}); worst logits rel-err {worst:.2e}")
   assert got == ref
   assert worst <= 1e-3
+
+@pytest.mark.parametrize("gating", [1, 2, 3, 4])
+@pytest.mark.parametrize("norm", [False, True])
+def test_gating_with_selection_bias_vs_oracle(gpu, gating, norm):
+  """exp_probs_b (model.py:113, 123): ranks by score + bias, weights from the unbiased scores; the hand case of tests/test_oracle_pins.py first."""
+  from tinygrad_amd.nn import moe_gate
+  def gate(lg, bias, k, g, nrm, scale):
+    T, E = lg.shape
+    sel, pr = gpu.Buffer((T, k), np.int32), gpu.Buffer((T, k), np.float32)
+    moe_gate(gpu.Buffer.from_numpy(lg), T, E, k, sel, pr, g, nrm, scale, bias=gpu.Buffer.from_numpy(bias))
+    return sel.numpy(), pr.numpy()
+  sel, p = gate(np.array([[0.0, np.log(3.0), -np.log(3.0), 0.0]], np.float32), np.array([0.0, 0.0, 1.0, 0.0], np.float32), 2, 2, False, 1.0)
+  assert sel.tolist() == [[1, 2]]
+  np.testing.assert_allclose(p, [[0.75, 0.25]], rtol=1e-6)
+  rng = np.random.default_rng(100 + 10 * gating + norm)
+  lg = rng.standard_normal((9, 96)).astype(np.float32) * 2
+  bias = rng.uniform(-0.5, 0.5, 96).astype(np.float32)
+  sel, p = gate(lg, bias, 8, gating, norm, 1.75)
+  rs, rp = omoe.gate_probs(lg, 8, gating, norm, 1.75, bias=bias)
+  np.testing.assert_array_equal(sel, rs)
+  np.testing.assert_allclose(p, rp, rtol=2e-5, atol=1e-7)
+  assert (sel != omoe.gate_probs(lg, 8, gating, norm, 1.75)[0]).any()             # the bias changes at least one selection in this sample
+
+GLM_LIKE = dict(num_blocks=3, dim=512, hidden_dim=256, n_heads=8, n_kv_heads=2, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,
+                num_experts=8, num_experts_per_tok=2, norm_topk_prob=True, expert_gating_func=2, routed_scaling_factor=1.5,
+                leading_dense_blocks=1, dense_hidden_dim=768, shared_expert_dim=256, shared_expert_gate=True, expert_bias=True)
+
+@pytest.mark.parametrize("gate", [True, False], ids=["gated_shared_expert", "plain_shared_expert"])
+def test_small_glm4moe_like_decode(gpu, gate):
+  """The model-zoo extras of FFNBlock (model.py:84, 99-103, 113, 131-134) together: a leading dense block, sigmoid gating with an expert selection
+  bias, normalised and scaled top-k weights, and a shared expert (with and without its sigmoid gate) on every MoE block; 32 greedy tokens against
+  the oracle on reference numerics."""
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe
+  from decode_helpers import greedy_vs_reference_numerics
+  cfg = dict(GLM_LIKE, shared_expert_gate=gate)
+  c = TransformerConfig(max_context=128, **cfg)
+  sd = synth_state_moe(c, seed=1009)
+  gpu.synchronize()
+  host = {k: (b.numpy(), t, shp) for k, (b, t, shp) in sd.items()}
+  model = Transformer(c, sd, max_new=64)
+  assert [b.moe for b in model.blk] == [False, True, True] and model.blk[1].shared and (model.blk[1].sh_gate_inp is not None) == gate
+  rng = np.random.default_rng(1009)
+  prompt = [int(t) for t in rng.integers(0, 512, size=20)]
+  oracle = ollm.Model(cfg, host, 128, act_round_f16=False)
+  got, ref, worst, margin, rms = greedy_vs_reference_numerics(model, oracle, prompt, 32)
+  print(f"oracle (reference numerics) min top-2 margin over 32 steps {margin:.4f} (logit rms {rms:.4f}); worst logits rel-err {worst:.2e}; min biased-score gap {oracle.min_route_gap:.2e}")
+  assert got == ref
+  assert worst <= 1e-3
+  # every extra matters: dropping any one of them moves the oracle's logits far away from the GPU's
+  lg_gpu = model.logits()
+  hist = prompt + got[:-1]
+  for drop in ("exp_probs_b.bias", "ffn_gate_shexp.weight"):
+    host2 = {k: v for k, v in host.items() if not k.endswith(drop)}
+    if drop == "ffn_gate_shexp.weight": host2 = {k: v for k, v in host2.items() if "shexp" not in k}
+    o2 = ollm.Model(cfg, host2, 128, act_round_f16=False)
+    for pos, t in enumerate(hist): lg2 = o2.forward(t, pos)
+    print(f"without {drop}: logits rel-err {ol.rel_err(lg2, lg_gpu):.3f}")
+    assert ol.rel_err(lg2, lg_gpu) > 5e-3, drop                                    # five times the parity bar

@@ -229,3 +229,67 @@ def test_generate_is_greedy_first_maximum():
   m, t, cfg = _model(2, 2, 8, dim, hidden=16, vocab=16, **{"token_embd.weight": emb, "output.weight": out_w})
   toks, margins = m.generate([1], 3)
   assert toks == [2, 4, 4] and margins[1] == 0.0                                          # 1 -> 2; 2 -> tie(4, 9) -> 4; 4 -> tie -> 4
+
+# ---- expert selection bias, shared expert and leading dense blocks of FFNBlock._feed_forward (model.py:84, 113, 123, 131-134) ----
+
+def test_selection_bias_ranks_but_does_not_weigh():
+  """Hand case, SIGMOID gating (no softmax coupling): logits 0, ln 3, -ln 3, ln 1 -> scores 1/2, 3/4, 1/4, 1/2.  Without a bias the top-2 is
+  {1, then the lower index of the tie 0 / 3}; a bias of +1 on expert 2 must SELECT expert 2 yet weigh it with its unbiased score 1/4."""
+  lg = np.array([[0.0, np.log(3.0), -np.log(3.0), 0.0]], np.float32)
+  sel, p = omoe.gate_probs(lg, 2, gating=omoe.SIGMOID)
+  assert sel.tolist() == [[0, 1]]                        # ascending rank: expert 0 (tie with 3, lower index ranks higher), then expert 1
+  np.testing.assert_allclose(p, [[0.5, 0.75]], rtol=1e-6)
+  bias = np.array([0.0, 0.0, 1.0, 0.0], np.float32)
+  sel, p = omoe.gate_probs(lg, 2, gating=omoe.SIGMOID, bias=bias)
+  assert sel.tolist() == [[1, 2]]                        # biased scores 0.5, 0.75, 1.25, 0.5: expert 2 on top, then expert 1
+  np.testing.assert_allclose(p, [[0.75, 0.25]], rtol=1e-6)
+  sel, p = omoe.gate_probs(lg, 2, gating=omoe.SIGMOID, norm_topk_prob=True, scale=2.0, bias=bias)
+  np.testing.assert_allclose(p, [[1.5, 0.5]], rtol=1e-6)  # normalised over the unbiased scores of the selection, then scaled
+  # with a bias the SOFTMAX + normalise shortcut of model.py:116-117 must NOT be taken: weights are softmax scores renormalised, not a softmax of logits
+  lg2 = np.array([[2.0, 1.0, 0.0]], np.float32)
+  sc = np.exp(lg2[0]) / np.exp(lg2[0]).sum()
+  sel, p = omoe.gate_probs(lg2, 2, gating=omoe.SOFTMAX, norm_topk_prob=True, bias=np.array([0.0, 0.0, 5.0], np.float32))
+  assert sel.tolist() == [[0, 2]]
+  np.testing.assert_allclose(p[0], np.array([sc[0], sc[2]]) / (sc[0] + sc[2]), rtol=1e-6)
+
+def _tiny_moe_weights(rng, L=2, D=8, H=4, E=3, lead=0, shared=0, gate=False, bias=False, vocab=16, hd=4):
+  w = {"token_embd.weight": rng.standard_normal((vocab, D)).astype(np.float32), "output_norm.weight": np.ones(D, np.float32), "output.weight": rng.standard_normal((vocab, D)).astype(np.float32)}
+  for i in range(L):
+    p = f"blk.{i}."
+    w.update({p + "attn_norm.weight": np.ones(D, np.float32), p + "ffn_norm.weight": np.ones(D, np.float32),
+              p + "attn_q.weight": rng.standard_normal((2 * hd, D)).astype(np.float32), p + "attn_k.weight": rng.standard_normal((hd, D)).astype(np.float32),
+              p + "attn_v.weight": rng.standard_normal((hd, D)).astype(np.float32), p + "attn_output.weight": np.zeros((D, 2 * hd), np.float32)})
+    if i < lead:
+      w.update({p + "ffn_gate.weight": rng.standard_normal((6, D)).astype(np.float32), p + "ffn_up.weight": rng.standard_normal((6, D)).astype(np.float32),
+                p + "ffn_down.weight": rng.standard_normal((D, 6)).astype(np.float32)})
+      continue
+    w.update({p + "ffn_gate_inp.weight": rng.standard_normal((E, D)).astype(np.float32), p + "ffn_gate_exps.weight": rng.standard_normal((E, H, D)).astype(np.float32),
+              p + "ffn_up_exps.weight": rng.standard_normal((E, H, D)).astype(np.float32), p + "ffn_down_exps.weight": np.zeros((E, D, H), np.float32)})
+    if shared:
+      w.update({p + "ffn_gate_shexp.weight": rng.standard_normal((shared, D)).astype(np.float32), p + "ffn_up_shexp.weight": rng.standard_normal((shared, D)).astype(np.float32),
+                p + "ffn_down_shexp.weight": rng.standard_normal((D, shared)).astype(np.float32)})
+      if gate: w[p + "ffn_gate_inp_shexp.weight"] = np.zeros((1, D), np.float32)
+    if bias: w[p + "exp_probs_b.bias"] = rng.standard_normal(E).astype(np.float32)
+  return w
+
+def test_shared_expert_and_leading_dense_block_wiring():
+  """attn_output = 0 and routed ffn_down_exps = 0, so a block adds exactly its always-on feed-forward to the residual row:
+  block 0 (leading dense block) x += ffn_down(silu(ffn_gate n) * ffn_up n), block 1 (MoE) x += shared expert, halved by its zero-weight gate
+  (sigmoid(0) = 1/2).  Computed here in float64 from the definitions; a block that took the wrong branch, dropped the shared expert or ignored the
+  gate misses by O(1)."""
+  rng = np.random.default_rng(12)
+  cfg = dict(num_blocks=2, dim=8, hidden_dim=4, n_heads=2, n_kv_heads=1, norm_eps=1e-5, vocab_size=16, head_dim=4, rope_theta=10000.0,
+             num_experts=3, num_experts_per_tok=2, leading_dense_blocks=1)
+  for gate in (False, True):
+    w = _tiny_moe_weights(rng, lead=1, shared=5, gate=gate)
+    m = ollm.Model(cfg, w, 8, w_round_f16=False, kv_dtype=np.float32)
+    lg = m.forward(3, 0)
+    f64 = lambda a: a.astype(np.float64)
+    rms = lambda v: v / np.sqrt((v * v).mean() + 1e-5)
+    silu = lambda v: v / (1 + np.exp(-v))
+    x = f64(w["token_embd.weight"][3])
+    n = rms(x); x = x + f64(w["blk.0.ffn_down.weight"]) @ (silu(f64(w["blk.0.ffn_gate.weight"]) @ n) * (f64(w["blk.0.ffn_up.weight"]) @ n))
+    n = rms(x); sh = f64(w["blk.1.ffn_down_shexp.weight"]) @ (silu(f64(w["blk.1.ffn_gate_shexp.weight"]) @ n) * (f64(w["blk.1.ffn_up_shexp.weight"]) @ n))
+    x = x + (0.5 * sh if gate else sh)
+    ref = f64(w["output.weight"]) @ rms(x)
+    np.testing.assert_allclose(lg, ref, rtol=2e-4, atol=2e-4)

@@ -4,12 +4,13 @@
 #include "moe_gate.h"
 
 // One workgroup (64 threads) per token.
-__global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ logits, int n_experts, int k, int gating, int norm_topk,
+__global__ __launch_bounds__(64) void moe_gate_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int n_experts, int k, int gating, int norm_topk,
                                                       float scale, int* __restrict__ sel, float* __restrict__ probs) {
-  extern __shared__ float sc[];                         // n_experts scores
+  extern __shared__ float sc[];                         // n_experts scores (+ n_experts biased scores when there is a selection bias)
   __shared__ float tmp[192];
   const int t = blockIdx.x;
-  gate_topk_wave(logits + (size_t)t * n_experts, n_experts, k, gating, norm_topk, scale, sel + (size_t)t * k, probs + (size_t)t * k, sc, tmp, threadIdx.x);
+  gate_topk_wave(logits + (size_t)t * n_experts, n_experts, k, gating, norm_topk, scale, sel + (size_t)t * k, probs + (size_t)t * k, sc, tmp, threadIdx.x,
+                 bias, sc + n_experts);
 }
 
 // Router of one token in one launch (tinygrad/llm/model.py:112-121 with the block's ffn_norm, :150): h = RMSNorm(x) * weight rounded
@@ -128,7 +129,17 @@ int tga_moe_gate(const float* logits, int n_tokens, int n_experts, int k, int ga
   TGA_REQUIRE(logits && sel && probs, "tga_moe_gate: null pointer");
   TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 4096 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_gate: bad geometry (k <= 64, n_experts <= 4096)");
   TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_gate: unknown ExpertGating %d", gating);
-  moe_gate_kernel<<<n_tokens, 64, n_experts * sizeof(float), (hipStream_t)stream>>>(logits, n_experts, k, gating, norm_topk_prob, scale, sel, probs);
+  moe_gate_kernel<<<n_tokens, 64, n_experts * sizeof(float), (hipStream_t)stream>>>(logits, nullptr, n_experts, k, gating, norm_topk_prob, scale, sel, probs);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_moe_gate_biased(const float* logits, const float* selection_bias, int n_tokens, int n_experts, int k, int gating, int norm_topk_prob, float scale,
+                        int32_t* sel, float* probs, void* stream) {
+  TGA_REQUIRE(logits && selection_bias && sel && probs, "tga_moe_gate_biased: null pointer");
+  TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 4096 && k >= 1 && k <= 64 && k <= n_experts, "tga_moe_gate_biased: bad geometry (k <= 64, n_experts <= 4096)");
+  TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_gate_biased: unknown ExpertGating %d", gating);
+  moe_gate_kernel<<<n_tokens, 64, 2 * n_experts * sizeof(float), (hipStream_t)stream>>>(logits, selection_bias, n_experts, k, gating, norm_topk_prob, scale, sel, probs);
   TGA_LAUNCH_CHECK();
   return 0;
 }

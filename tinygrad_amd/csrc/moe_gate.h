@@ -8,10 +8,14 @@
 // i < j)}; the k highest ranks are emitted in ASCENDING rank order (the largest last), so among equal scores the lower index
 // ranks higher.  Runs on ONE wave (lane = threadIdx.x & 63 of the calling wave); lg may live in LDS or global memory, sc is
 // n_experts floats of LDS, tmp 192 floats of LDS.  The caller separates the call from earlier LDS writes with a barrier.
+// bias (optional, n_experts floats): the expert selection bias of model.py:113, 123 - experts are ranked by score + bias, the weights are
+// gathered from the unbiased scores; scb is then n_experts more floats of LDS for the biased scores (without a bias pass scb = sc).
 __device__ __forceinline__ void gate_topk_wave(const float* lg, int n_experts, int k, int gating, int norm_topk, float scale,
-                                               int* __restrict__ sel, float* __restrict__ probs, float* sc, float* tmp, int lane) {
+                                               int* __restrict__ sel, float* __restrict__ probs, float* sc, float* tmp, int lane,
+                                               const float* bias = nullptr, float* scb = nullptr) {
   int* s_sel = (int*)tmp; float* s_p = tmp + 64; float* s_q = tmp + 128;
-  if (gating == 1 && norm_topk) { gating = 3; norm_topk = 0; }   // model.py:116-117 fast path (no selection bias)
+  if (!bias) scb = sc;
+  if (gating == 1 && norm_topk && !bias) { gating = 3; norm_topk = 0; }   // model.py:116-117 fast path (only without a selection bias)
   float mx = -INFINITY;
   for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, lg[i]);
   mx = wave_max(mx);
@@ -25,15 +29,16 @@ __device__ __forceinline__ void gate_topk_wave(const float* lg, int n_experts, i
     else if (gating == 2) s = 1.0f / (1.0f + expf(-v));
     else s = sqrtf(log1pf(expf(v)));
     sc[i] = s;
+    if (bias) scb[i] = s + bias[i];
   }
   s_sel[lane] = 0; s_p[lane] = 0.f;                       // a slot no rank lands in (NaN scores compare false with everything) selects expert 0, like the reference's zero-filled scatter
   __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);   // this wave's LDS writes are visible to its own lanes
   for (int i = lane; i < n_experts; i += 64) {
-    const float si = sc[i];
+    const float si = scb[i];
     int rank = 0;
-    for (int j = 0; j < n_experts; j++) { const float sj = sc[j]; rank += (si > sj) || (si == sj && i < j); }
+    for (int j = 0; j < n_experts; j++) { const float sj = scb[j]; rank += (si > sj) || (si == sj && i < j); }
     const int slot = rank - (n_experts - k);
-    if (slot >= 0) { s_sel[slot] = i; s_p[slot] = si; }
+    if (slot >= 0) { s_sel[slot] = i; s_p[slot] = sc[i]; }
   }
   __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_s_waitcnt(0xc07f);
   float p = lane < k ? s_p[lane] : 0.f;

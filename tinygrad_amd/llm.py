@@ -35,6 +35,15 @@ class TransformerConfig:
   expert_gating_func: int = 1      # ExpertGating.SOFTMAX (model.py:9-13)
   routed_scaling_factor: float = 1.0
   rope_dim: int = 0                # rotated leading values of a head (model.py:63, 180-181); 0 = head_dim
+  leading_dense_blocks: int = 0    # the first blocks of an MoE model that keep a dense FFN of width dense_hidden_dim (model.py:84, 441)
+  dense_hidden_dim: int = 0
+  shared_expert_dim: int = 0       # width of the always-on shared expert FFN added to the routed sum (model.py:99-103, 131-134); 0 = none
+  shared_expert_gate: bool = False # the shared expert's output is scaled by sigmoid(x . ffn_gate_inp_shexp) (model.py:133)
+  expert_bias: bool = False        # exp_probs_b: experts are ranked by score + bias, weighted by the score (model.py:113, 123)
+
+  @property
+  def n_summands(self) -> int:     # rows of the weighted sum a MoE block leaves: the routed experts and the shared expert
+    return self.num_experts_per_tok + (1 if self.shared_expert_dim else 0)
 
 LLAMA3_8B = dict(num_blocks=32, dim=4096, hidden_dim=14336, n_heads=32, n_kv_heads=8, norm_eps=1e-5, vocab_size=128256,
                  head_dim=128, rope_theta=500000.0)
@@ -72,7 +81,8 @@ def quant_nbytes(ggml_type: int, n: int) -> int:
   return n // nel * nby
 
 def synth_state_moe(config: TransformerConfig, seed: int = 1004, dense_type: int = rt.F16, expert_type: int = rt.MXFP4, stream=None) -> dict:
-  """OLMoE-architecture random model: fp16 attention / router / embedding / lm-head, MXFP4 expert stacks (E, out, in), norms 1."""
+  """OLMoE-architecture random model: fp16 attention / router / embedding / lm-head, MXFP4 expert stacks (E, out, in), norms 1.  The config's
+  leading dense blocks, shared expert (with or without its sigmoid gate) and expert selection bias are written when it asks for them."""
   c, sd, tid = config, {}, [0]
   def mk(name, shape, t, amp):
     n = int(np.prod(shape))
@@ -92,10 +102,21 @@ def synth_state_moe(config: TransformerConfig, seed: int = 1004, dense_type: int
       mk(p + "attn_q_norm.weight", (1, c.n_heads * c.head_dim), rt.F32, 1.0)
       mk(p + "attn_k_norm.weight", (1, c.n_kv_heads * c.head_dim), rt.F32, 1.0)
     mk(p + "ffn_norm.weight", (1, D), rt.F32, 1.0)
+    if i < c.leading_dense_blocks:
+      Hd = c.dense_hidden_dim
+      mk(p + "ffn_gate.weight", (Hd, D), dense_type, D ** -0.5); mk(p + "ffn_up.weight", (Hd, D), dense_type, D ** -0.5); mk(p + "ffn_down.weight", (D, Hd), dense_type, Hd ** -0.5)
+      continue
     mk(p + "ffn_gate_inp.weight", (E, D), dense_type, D ** -0.5)
     mk(p + "ffn_gate_exps.weight", (E, H, D), expert_type, D ** -0.5)
     mk(p + "ffn_up_exps.weight", (E, H, D), expert_type, D ** -0.5)
     mk(p + "ffn_down_exps.weight", (E, D, H), expert_type, H ** -0.5)
+    if c.shared_expert_dim:
+      Hs = c.shared_expert_dim
+      mk(p + "ffn_gate_shexp.weight", (Hs, D), dense_type, D ** -0.5); mk(p + "ffn_up_shexp.weight", (Hs, D), dense_type, D ** -0.5); mk(p + "ffn_down_shexp.weight", (D, Hs), dense_type, Hs ** -0.5)
+      if c.shared_expert_gate: mk(p + "ffn_gate_inp_shexp.weight", (1, D), dense_type, D ** -0.5)
+    if c.expert_bias:                                                    # float32 holding fp16 values, like every tensor the reference loads (model.py:376)
+      bias = np.random.default_rng(seed * 31 + i).uniform(-0.3, 0.3, E).astype(np.float16).astype(np.float32)
+      sd[p + "exp_probs_b.bias"] = (Buffer.from_numpy(bias), rt.F32, (1, E))
   mk("output_norm.weight", (1, D), rt.F32, 1.0)
   mk("output.weight", (c.vocab_size, D), dense_type, D ** -0.5)
   return sd
@@ -155,11 +176,17 @@ class TransformerBlock:
     lin = lambda name: QuantLinear(sd[p + name][0], sd[p + name][1], *sd[p + name][2])
     self.attn_norm, self.ffn_norm = sd[p + "attn_norm.weight"][0], sd[p + "ffn_norm.weight"][0]
     self.attn_q, self.attn_k, self.attn_v, self.attn_output = lin("attn_q.weight"), lin("attn_k.weight"), lin("attn_v.weight"), lin("attn_output.weight")
-    self.moe = c.num_experts > 0
+    self.moe = c.num_experts > 0 and i >= c.leading_dense_blocks       # leading blocks of an MoE model are dense (model.py:84)
     if self.moe:
       ex = lambda name: ExpertWeights(sd[p + name][0], sd[p + name][1], *sd[p + name][2])
       self.ffn_gate_inp = lin("ffn_gate_inp.weight")                      # router
       self.ffn_gate_exps, self.ffn_up_exps, self.ffn_down_exps = ex("ffn_gate_exps.weight"), ex("ffn_up_exps.weight"), ex("ffn_down_exps.weight")
+      self.sel_bias = sd[p + "exp_probs_b.bias"][0] if c.expert_bias else None       # float32 (n_experts,)
+      self.shared = c.shared_expert_dim > 0
+      if self.shared:
+        self.sh_gate, self.sh_up, self.sh_down = lin("ffn_gate_shexp.weight"), lin("ffn_up_shexp.weight"), lin("ffn_down_shexp.weight")
+        self.sh_gate_inp = lin("ffn_gate_inp_shexp.weight") if c.shared_expert_gate else None     # (1, dim)
+        if self.sh_gate.ggml_type != self.sh_up.ggml_type: raise NotImplementedError("ffn_gate_shexp and ffn_up_shexp of different ggml types are not built")
     else:
       self.ffn_gate, self.ffn_up, self.ffn_down = lin("ffn_gate.weight"), lin("ffn_up.weight"), lin("ffn_down.weight")
     # Linear(bias=config.qkv_bias) of model.py:161-163: the float32 bias rows enter the q / k / v launch as its additive row
@@ -179,26 +206,27 @@ class TransformerBlock:
     self.stage_attn = fast(self.attn_output)
     self.stage_act = (not self.moe) and fast(self.ffn_down)
     self.stage_xn = (not self.moe) and fast(self.ffn_gate) and self.ffn_gate.ggml_type == self.ffn_up.ggml_type
+    self.stage_sh = self.moe and self.shared and fast(self.sh_down)
     # the expert gate/up launch can gate for itself: one fp16 row of at most 4096 values on one wave per row team
-    self.route_in_experts = self.moe and c.dim <= 4096 and c.dim % 64 == 0 and c.num_experts <= 1024 and c.num_experts_per_tok <= 64 \
+    self.route_in_experts = self.moe and self.sel_bias is None and c.dim <= 4096 and c.dim % 64 == 0 and c.num_experts <= 1024 and c.num_experts_per_tok <= 64 \
                             and (c.dim // (32 if self.ffn_gate_exps.ggml_type == rt.MXFP4 else 64)) <= 64
     # the previous block's weighted expert sum can be completed inside this block's q/k/v launch (one 8-value piece per thread: dim <= 2048)
     self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
-                            and 0 < c.num_experts_per_tok <= 8 and self.qkv_bias is None
+                            and 0 < c.n_summands <= 8 and self.qkv_bias is None
     if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
 
-  def __call__(self, x: Buffer, stream, pending: bool = False, defer: bool = False) -> tuple[Buffer, bool]:
-    """One block on the residual row x.  pending: the previous (MoE) block left its weighted expert sum + residual to this block
+  def __call__(self, x: Buffer, stream, pending: int = 0, defer: bool = False) -> tuple[Buffer, int]:
+    """One block on the residual row x.  pending > 0: the previous (MoE) block left its weighted sum over that many rows + residual to this block
     (expert outputs in s.y_e, weights in s.probs).  defer: leave this block's own weighted sum to the next launch.  Returns the buffer
     that holds the residual row afterwards and whether a weighted sum is still pending."""
     c, s, L = self.config, self.s, rt.lib()
     # h = x + attention(attn_norm(x))                                                     model.py:149
     qkv, qkv_out = [self.attn_q, self.attn_k, self.attn_v], [s.q, s.k, s.v]
     if pending and not self.can_fold_combine:
-      moe_combine(s.y_e, s.probs, x, 1, c.num_experts_per_tok, c.dim, x, stream=stream); pending = False
+      moe_combine(s.y_e, s.probs, x, 1, pending, c.dim, x, stream=stream); pending = 0
     if pending:                                                          # x + sum_j probs_j y_j completed inside the q/k/v launch, written to the other row buffer
       x_new = s.x2 if x.ptr == s.x.ptr else s.x
-      qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps), combine=(s.y_e, s.probs, c.num_experts_per_tok, x_new))
+      qlinear_multi(qkv, x, qkv_out, stream=stream, norm=(self.attn_norm, c.norm_eps), combine=(s.y_e, s.probs, pending, x_new))
       x = x_new
     else:
       # one launch per run of equal block types (e.g. Q4_K q / k with a Q6_K v: two launches); each normalises the row while staging it
@@ -225,7 +253,7 @@ class TransformerBlock:
         rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if self.stage_xn else 0, stream))
         qlinear_multi([self.ffn_gate, self.ffn_up], s.xn, [s.act], epilogue=2, stream=stream, x_staged=self.stage_xn, stage_out_for=self.ffn_down if self.stage_act else None)
       qlinear_multi([self.ffn_down], s.act, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_act)
-      return x, False
+      return x, 0
     # MoE feed-forward (model.py:110-135): router -> gating + pairwise top-k -> selected experts' SwiGLU -> weighted sum (+ residual)
     k = c.num_experts_per_tok
     one_launch_router = self.ffn_gate_inp.ggml_type == rt.F16 and c.dim % 8 == 0 and c.dim <= 16384 and c.num_experts <= 1024
@@ -235,19 +263,33 @@ class TransformerBlock:
       self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream,
                          route=(s.router, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, s.probs))
     else:
-      if one_launch_router:
+      if one_launch_router and self.sel_bias is not None:                # logits in one launch, then the gating with the selection bias
+        moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, 0, None, None, s.router, xn_out=s.xn, stream=stream)
+        moe_gate(s.router.view(0, (1, c.num_experts), np.float32), 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob,
+                 c.routed_scaling_factor, stream=stream, bias=self.sel_bias)
+      elif one_launch_router:
         moe_router(x, self.ffn_norm, c.norm_eps, self.ffn_gate_inp, k, s.sel, s.probs, s.router, xn_out=s.xn, gating=c.expert_gating_func,
                    norm_topk_prob=c.norm_topk_prob, scale=c.routed_scaling_factor, stream=stream)
       else:
         rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
         lg = s.router.view(0, (1, c.num_experts), np.float32)
         self.ffn_gate_inp(s.xn, out=lg, stream=stream)
-        moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream)
+        moe_gate(lg, 1, c.num_experts, k, s.sel, s.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=stream, bias=self.sel_bias)
       self.ffn_gate_exps(s.sel, s.xn, s.act_e, jobs_per_x_row=k, up=self.ffn_up_exps, stream=stream)      # silu(gate_e x) * (up_e x) per slot
     self.ffn_down_exps(s.sel, s.act_e, s.y_e, jobs_per_x_row=1, stream=stream)
-    if defer: return x, True                                            # the consumer of the completed row adds sum_j probs_j y_j + x itself
-    moe_combine(s.y_e, s.probs, x, 1, k, c.dim, x, stream=stream)
-    return x, False
+    n_sum = k
+    if self.shared:
+      # the shared expert (model.py:131-134) is one more row of the weighted sum: its output goes to row k of y_e, its weight (1, or the
+      # sigmoid gate) to probs[k]
+      qlinear_multi([self.sh_gate, self.sh_up], s.xn, [s.act_sh], epilogue=2, stream=stream, stage_out_for=self.sh_down if self.stage_sh else None)
+      qlinear_multi([self.sh_down], s.act_sh, [s.y_sh], stream=stream, x_staged=self.stage_sh)
+      if self.sh_gate_inp is not None:
+        self.sh_gate_inp(s.xn, out=s.sh_logit, stream=stream)
+        moe_gate(s.sh_logit, 1, 1, 1, s.sh_sel, s.p_sh, 2, False, 1.0, stream=stream)     # sigmoid of the one logit
+      n_sum = k + 1
+    if defer: return x, n_sum                                           # the consumer of the completed row adds sum_j probs_j y_j + x itself
+    moe_combine(s.y_e, s.probs, x, 1, n_sum, c.dim, x, stream=stream)
+    return x, 0
 
 class _Shared:
   """Activation buffers shared by all blocks (batch 1)."""
@@ -262,11 +304,15 @@ class _Shared:
     self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
     self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
-    self.act = Buffer((1, c.hidden_dim), f16)
+    self.act = Buffer((1, max(c.hidden_dim, c.dense_hidden_dim)), f16)
     if c.num_experts:
       k = c.num_experts_per_tok
-      self.router, self.sel, self.probs = Buffer((1, c.num_experts + 1), f32).zero_(), Buffer((k,), np.int32), Buffer((k,), f32)   # logits + arrival counter
-      self.act_e, self.y_e = Buffer((k, c.hidden_dim), f16), Buffer((k, c.dim), f32)
+      self.router, self.sel = Buffer((1, c.num_experts + 1), f32).zero_(), Buffer((k,), np.int32)     # logits + arrival counter
+      self.probs = Buffer.from_numpy(np.ones(k + 1, dtype=f32))           # k routed weights + the shared expert's (1 unless it is gated)
+      self.act_e, self.y_e = Buffer((k, c.hidden_dim), f16), Buffer((k + 1, c.dim), f32)
+      self.y_sh, self.p_sh = self.y_e.view(4 * k * c.dim, (1, c.dim), f32), self.probs.view(4 * k, (1,), f32)
+      self.act_sh = Buffer((1, max(1, c.shared_expert_dim)), f16)
+      self.sh_logit, self.sh_sel = Buffer((1, 1), f32), Buffer((1,), np.int32)
     self.logits = Buffer((1, c.vocab_size), f32)
     self.am_v, self.am_i = Buffer((256,), f32), Buffer((256,), np.int32)
     self.rope = Buffer.from_numpy(rope_table(c.head_dim, c.rope_dim or c.head_dim, c.max_context, c.rope_theta))
@@ -286,7 +332,7 @@ class Transformer:
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
     self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
-    self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.num_experts_per_tok <= 8
+    self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.n_summands <= 8
     self.stream = rt.Stream()
     self._graphs = {}
     self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
@@ -304,7 +350,7 @@ class Transformer:
   def _step(self, with_head: bool):
     c, s, L, st = self.config, self.s, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
-    x, pending = s.x, False
+    x, pending = s.x, 0
     nb = len(self.blk)
     for i, b in enumerate(self.blk):
       nxt = self.blk[i + 1].can_fold_combine if i + 1 < nb else (with_head and self.can_fold_head)
@@ -312,7 +358,7 @@ class Transformer:
     if with_head:
       if pending:                                                      # the last block's weighted sum completed inside the lm-head launch
         x_new = s.x2 if x.ptr == s.x.ptr else s.x
-        qlinear_multi([self.output], x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps), combine=(s.y_e, s.probs, c.num_experts_per_tok, x_new))
+        qlinear_multi([self.output], x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps), combine=(s.y_e, s.probs, pending, x_new))
         x = x_new
       elif self.fuse_head_norm:                                        # output_norm inside the lm-head launch (model.py:362)
         qlinear_multi([self.output], x, [s.logits], stream=st, norm=(self.output_norm, c.norm_eps))
@@ -387,10 +433,14 @@ class Transformer:
       num_experts=kv.get(f"{arch}.expert_count", 0), num_experts_per_tok=kv.get(f"{arch}.expert_used_count", 0),
       norm_topk_prob=kv.get(f"{arch}.expert_weights_norm", arch in ("qwen3moe",)),
       expert_gating_func=kv.get(f"{arch}.expert_gating_func", 1), routed_scaling_factor=kv.get(f"{arch}.expert_weights_scale", 1.0),
-      rope_dim=rope_dim if rope_dim != head_dim else 0)
+      rope_dim=rope_dim if rope_dim != head_dim else 0,
+      leading_dense_blocks=(lead := kv.get(f"{arch}.leading_dense_block_count", 0)),
+      dense_hidden_dim=kv.get(f"{arch}.feed_forward_length", 0) if lead else 0,
+      shared_expert_dim=kv.get(f"{arch}.expert_shared_feed_forward_length", kv.get(f"{arch}.expert_shared_count", 0) * kv.get(f"{arch}.expert_feed_forward_length", 0)),
+      shared_expert_gate=f"blk.{lead}.ffn_gate_inp_shexp.weight" in sd, expert_bias=f"blk.{lead}.exp_probs_b.bias" in sd)
     sd = _Consumed(sd)
     model = Transformer(config, sd, max_new=max_new)
-    if (left := sorted(set(sd) - sd.used)):                            # e.g. shared experts, expert selection bias, leading dense blocks: not silently dropped
+    if (left := sorted(set(sd) - sd.used)):                            # nothing a file carries is silently dropped
       raise NotImplementedError(f"tensors the built path does not consume: {left[:8]}{' ...' if len(left) > 8 else ''}")
     return model, kv
 
@@ -439,7 +489,9 @@ class Transformer:
     n = self.output.nbytes
     for b in self.blk:
       n += sum(l.nbytes for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output))
-      if b.moe: n += b.ffn_gate_inp.nbytes + self.config.num_experts_per_tok * sum(e.expert_nbytes for e in (b.ffn_gate_exps, b.ffn_up_exps, b.ffn_down_exps))
+      if b.moe:
+        n += b.ffn_gate_inp.nbytes + self.config.num_experts_per_tok * sum(e.expert_nbytes for e in (b.ffn_gate_exps, b.ffn_up_exps, b.ffn_down_exps))
+        if b.shared: n += sum(l.nbytes for l in (b.sh_gate, b.sh_up, b.sh_down))
       else: n += sum(l.nbytes for l in (b.ffn_gate, b.ffn_up, b.ffn_down))
     return n
 
@@ -451,6 +503,8 @@ class BatchedTransformer:
   config as Transformer; every sequence has its own KV cache; prompts of one batch have equal length."""
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024):
     if not 1 <= batch <= 8: raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
+    if config.leading_dense_blocks or config.shared_expert_dim or config.expert_bias:
+      raise NotImplementedError("leading dense blocks, shared experts and the expert selection bias are built for batch 1 (Transformer) only")
     self.config, self.batch, self.max_new = config, batch, max_new
     c, B = config, batch
     f32, f16 = np.float32, np.float16

@@ -94,8 +94,12 @@ class ExpertWeights:
                                           jobs_per_x_row, x.ptr, rt.dtype_code(x.dtype), out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
     return out
 
-def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer, probs: Buffer, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):
-  rt.check(rt.lib().tga_moe_gate(logits.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
+def moe_gate(logits: Buffer, n_tokens: int, n_experts: int, k: int, sel: Buffer, probs: Buffer, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None,
+             bias: Buffer | None = None):
+  """bias: the float32 expert selection bias (`exp_probs_b`, model.py:113): ranks by score + bias, weights from the scores."""
+  if bias is not None:
+    rt.check(rt.lib().tga_moe_gate_biased(logits.ptr, bias.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
+  else: rt.check(rt.lib().tga_moe_gate(logits.ptr, n_tokens, n_experts, k, gating, int(norm_topk_prob), scale, sel.ptr, probs.ptr, stream))
 
 def moe_router(x: Buffer, norm_weight: Buffer | None, eps: float, router: QuantLinear, k: int, sel: Buffer, probs: Buffer, logits_ws: Buffer,
                xn_out: Buffer | None = None, gating: int = 1, norm_topk_prob: bool = False, scale: float = 1.0, stream=None):

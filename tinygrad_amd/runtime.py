@@ -42,6 +42,7 @@ def _declare(lib):
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
     "tga_qlinear_experts_routed": [i, vp, vp, i64, vp, i, i, i, ctypes.c_float, vp, vp, vp, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
+    "tga_moe_gate_biased": [vp, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
     "tga_moe_router": [vp, vp, ctypes.c_float, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp, vp, vp],
     "tga_quantize_mxfp8": [vp, i, i64, i64, vp, vp, vp, vp],
