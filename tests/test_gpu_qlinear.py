@@ -118,6 +118,26 @@ def test_multi_segment_and_epilogues(gpu):
   ref = a / (1 + np.exp(-a)) * b
   assert ol.rel_err(out.numpy(), ref) <= TOL
 
+@pytest.mark.parametrize("t", [2, 8, 14, 1, 39], ids=["q4_0", "q8_0", "q6_k", "f16", "mxfp4"])
+@pytest.mark.parametrize("m", [2, 3, 5, 8])
+def test_multi_segment_small_batch(gpu, t, m):
+  """q / k / v in one launch at 2..8 activation rows: from three rows on the matrix-core kernel walks all three matrices (every one a multiple of
+  16 rows); a segment that is not (130 rows) sends the call to the dot2 kernel.  Both against the float64 anchor."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(770 + t + m)
+  k = 1024
+  for ns in ([512, 128, 144], [512, 128, 130]):
+    mk = lambda n: (rng.standard_normal((n, k)) * k ** -0.5).astype(np.float16).view(np.uint8).reshape(-1) if t == 1 else synth.random_blocks(rng, t, n, k)
+    ws = [mk(n) for n in ns]
+    x = synth.activations(rng, m, k, np.float16)
+    layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+    outs = [gpu.Buffer((m, n), np.float32) for n in ns]
+    for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    qlinear_multi(layers, gpu.Buffer.from_numpy(x), outs)
+    for o, w, n in zip(outs, ws, ns):
+      wf = w.view(np.float16).astype(np.float32).reshape(n, k) if t == 1 else ol.weight_f32(w, n, k, t)
+      assert ol.rel_err(o.numpy(), ol.linear_f64(x.astype(np.float32), wf)) <= TOL, (ns, n)
+
 def test_argument_errors(gpu):
   from tinygrad_amd.nn import QuantLinear
   w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))

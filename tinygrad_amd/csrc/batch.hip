@@ -153,14 +153,22 @@ static int exp_cu_count() {
 }
 
 template <int T, bool TWO>
-static int launch_qexperts(ExpArgs a, int n_experts, int n_jobs, hipStream_t s) {
+static int launch_qexperts(ExpArgs a, int n_experts, int n_jobs, int xdiv_hint, hipStream_t s) {
   using F = Fmt<T>;
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const size_t lds = (size_t)EXP_MAX_ROWS * F::XV * a.nu * 16;
   TGA_REQUIRE(lds <= 144 * 1024, "tga_qlinear_experts_grouped: K=%d does not fit the activation staging (%zu bytes of LDS)", a.K, lds);
   const long long ngroups = (a.N + 15) / 16;
-  long long gx = (2LL * exp_cu_count() + n_jobs - 1) / n_jobs;      // about two workgroups per CU when every job has its own expert
+  // About two workgroups per CU over the experts that have jobs.  How many do is only known on the device; the launch is sized for the number
+  // expected when the tokens pick independently (n_jobs = B k jobs over E experts, each token k distinct ones): E (1 - (1 - k / E)^B) with
+  // k = jobs_per_x_row for the gate/up launch; the down launch (one job per row) is told the same k through xdiv_hint.
+  const int kk = xdiv_hint > 0 ? xdiv_hint : 1, nb = (n_jobs + kk - 1) / kk;
+  double miss = 1.0; for (int t = 0; t < nb; t++) miss *= 1.0 - (double)(kk < n_experts ? kk : n_experts) / (double)n_experts;
+  double distinct = (double)n_experts * (1.0 - miss); if (distinct < 1.0) distinct = 1.0; if (distinct > n_jobs) distinct = n_jobs;
+  // (measured on the OLMoE-arch batched step, B = 8: 1 / 2 / 3 / 4 workgroups per CU = 3196 / 3699 / 3755 / 3812 tok/s; 32 KB of staged rows per workgroup)
+  const int wg_per_cu = 4;
+  long long gx = (long long)((double)wg_per_cu * exp_cu_count() / distinct + 0.5);
   if (gx > ngroups) gx = ngroups;
   if (gx < 1) gx = 1;
   auto kern = qexperts_mfma_kernel<T, TWO>;
@@ -174,8 +182,8 @@ static int launch_qexperts(ExpArgs a, int n_experts, int n_jobs, hipStream_t s) 
 }
 
 template <int T>
-static int launch_qexperts_t(const ExpArgs& a, int n_experts, int n_jobs, hipStream_t s) {
-  return a.w_up ? launch_qexperts<T, true>(a, n_experts, n_jobs, s) : launch_qexperts<T, false>(a, n_experts, n_jobs, s);
+static int launch_qexperts_t(const ExpArgs& a, int n_experts, int n_jobs, int xdiv_hint, hipStream_t s) {
+  return a.w_up ? launch_qexperts<T, true>(a, n_experts, n_jobs, xdiv_hint, s) : launch_qexperts<T, false>(a, n_experts, n_jobs, xdiv_hint, s);
 }
 
 extern "C" {
@@ -207,17 +215,18 @@ int tga_qlinear_experts_grouped(int ggml_type, const void* w, const void* w_up, 
   TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0 && a.estride % 4 == 0), "tga_qlinear_experts_grouped: expert weights must be 4-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   const int E = (int)n_experts;
+  const int k_hint = jobs_per_x_row > 1 ? jobs_per_x_row : 8;       // the down launch has one job per activation row: assume eight experts per token
   switch (ggml_type) {
-    case GGML_Q4_0: return launch_qexperts_t<F_Q4_0P>(a, E, n_jobs, s);
-    case GGML_Q8_0: return launch_qexperts_t<F_Q8_0P>(a, E, n_jobs, s);
-    case GGML_MXFP4: return launch_qexperts_t<GGML_MXFP4>(a, E, n_jobs, s);
-    case GGML_Q6_K: return launch_qexperts_t<GGML_Q6_K>(a, E, n_jobs, s);
-    case GGML_Q4_K: return launch_qexperts_t<GGML_Q4_K>(a, E, n_jobs, s);
-    case GGML_Q5_K: return launch_qexperts_t<GGML_Q5_K>(a, E, n_jobs, s);
-    case GGML_Q4_1: return launch_qexperts_t<GGML_Q4_1>(a, E, n_jobs, s);
-    case GGML_Q5_0: return launch_qexperts_t<GGML_Q5_0>(a, E, n_jobs, s);
-    case GGML_Q5_1: return launch_qexperts_t<GGML_Q5_1>(a, E, n_jobs, s);
-    case GGML_F16: return launch_qexperts_t<GGML_F16>(a, E, n_jobs, s);
+    case GGML_Q4_0: return launch_qexperts_t<F_Q4_0P>(a, E, n_jobs, k_hint, s);
+    case GGML_Q8_0: return launch_qexperts_t<F_Q8_0P>(a, E, n_jobs, k_hint, s);
+    case GGML_MXFP4: return launch_qexperts_t<GGML_MXFP4>(a, E, n_jobs, k_hint, s);
+    case GGML_Q6_K: return launch_qexperts_t<GGML_Q6_K>(a, E, n_jobs, k_hint, s);
+    case GGML_Q4_K: return launch_qexperts_t<GGML_Q4_K>(a, E, n_jobs, k_hint, s);
+    case GGML_Q5_K: return launch_qexperts_t<GGML_Q5_K>(a, E, n_jobs, k_hint, s);
+    case GGML_Q4_1: return launch_qexperts_t<GGML_Q4_1>(a, E, n_jobs, k_hint, s);
+    case GGML_Q5_0: return launch_qexperts_t<GGML_Q5_0>(a, E, n_jobs, k_hint, s);
+    case GGML_Q5_1: return launch_qexperts_t<GGML_Q5_1>(a, E, n_jobs, k_hint, s);
+    case GGML_F16: return launch_qexperts_t<GGML_F16>(a, E, n_jobs, k_hint, s);
   }
   return tga_set_error("tga_qlinear_experts_grouped: no kernel for type %d", ggml_type);
 }

@@ -33,6 +33,23 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
   uint32_t kc[F::NKC];
   F::consts(kc);
   const long long ngroups = (a.ntot + 15) / 16;
+  // Several weight matrices in one launch (q / k / v): rows run over the segments in order, every segment a multiple of 16 rows (checked by the
+  // dispatch), so a 16-row group lies inside one segment.  first row of a group -> segment, first row inside the segment
+  auto seg_of = [&](long long row0, int& sg, long long& local0) {
+    sg = 0; local0 = row0;
+    if (a.nseg > 1 && local0 >= a.n[0]) { local0 -= a.n[0]; sg = 1; if (a.nseg > 2 && local0 >= a.n[1]) { local0 -= a.n[1]; sg = 2; } }
+  };
+  auto store_tile = [&](long long row0) {                           // 256 threads = 16 weight rows x 16 activation rows
+    int sg; long long l0; seg_of(row0, sg, l0);
+    const int t = threadIdx.x, wr = t >> 4, c = t & 15;
+    const long long nrows = a.n[sg];
+    if (c < M && l0 + wr < nrows) {
+      const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
+      const long long o = (long long)c * nrows + l0 + wr;
+      void* yb = sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
+      if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
+    }
+  };
   if (a.nchunks == 1) {
     // ---- the whole K in LDS: one software pipeline over ALL (row group, step) pairs of this wave.  Every load is unconditional and in
     // straight-line code (steps past the end reload the last one; a step that does not exist for this wave - K / 4 units not a multiple
@@ -47,9 +64,11 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
     long long lj = 0; int li = 0;                                       // load stream: row group index (of this workgroup), step index
     auto issue = [&](Raw& buf) {
       const long long grp = (long long)blockIdx.x + lj * gridDim.x;
-      const long long row = grp * 16 + r, rowc = row < a.ntot ? row : a.ntot - 1;
+      int sg; long long l0; seg_of(grp * 16, sg, l0);
+      const long long row = l0 + r, rowc = row < a.n[sg] ? row : a.n[sg] - 1;
+      const uint8_t* wb = sg == 0 ? a.w[0] : sg == 1 ? a.w[1] : a.w[2];
       const int ul = 4 * (wave + 4 * li) + g;
-      buf = F::load(a.w[0] + rowc * a.row_bytes, ul < cu ? ul : cu - 1);
+      buf = F::load(wb + rowc * a.row_bytes, ul < cu ? ul : cu - 1);
       const bool more = lj * spw + li + 1 < T;                          // past the end: stay on the last step
       li = more ? (li + 1 == spw ? 0 : li + 1) : li;
       lj = more && li == 0 ? lj + 1 : lj;
@@ -81,14 +100,7 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
 #pragma unroll
           for (int i = 0; i < 4; i++) part[wave][4 * g + i][r] = acc[i];
           __syncthreads();
-          {
-            const int t = threadIdx.x, wr = t >> 4, c = t & 15;          // 256 threads = 16 weight rows x 16 activation rows
-            if (c < M && row0 + wr < a.ntot) {
-              const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
-              const long long o = (long long)c * a.ntot + row0 + wr;
-              if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
-            }
-          }
+          store_tile(row0);
           __syncthreads();
           acc = v4f32{0.f, 0.f, 0.f, 0.f};
           ci = 0; cj++;
@@ -107,8 +119,9 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
   }
   for (long long grp = blockIdx.x; grp < ngroups; grp += gridDim.x) {
     const long long row0 = grp * 16;
-    const long long myrow = row0 + r < a.ntot ? row0 + r : a.ntot - 1;   // ragged last group: reload a valid row, results dropped
-    const uint8_t* rowp = a.w[0] + myrow * a.row_bytes;
+    int sg0; long long l00; seg_of(row0, sg0, l00);
+    const long long myrow = l00 + r < a.n[sg0] ? l00 + r : a.n[sg0] - 1;   // ragged last group: reload a valid row, results dropped
+    const uint8_t* rowp = (sg0 == 0 ? a.w[0] : sg0 == 1 ? a.w[1] : a.w[2]) + myrow * a.row_bytes;
     v4f32 acc = {0.f, 0.f, 0.f, 0.f};
     for (int ch = 0; ch < a.nchunks; ch++) {
       const int u0 = ch * a.chunk_u, cu = min(a.chunk_u, a.nu - u0);
@@ -153,14 +166,7 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
 #pragma unroll
     for (int i = 0; i < 4; i++) part[wave][4 * g + i][r] = acc[i];
     __syncthreads();
-    {
-      const int t = threadIdx.x, wr = t >> 4, c = t & 15;              // 256 threads = 16 weight rows x 16 activation rows
-      if (c < M && row0 + wr < a.ntot) {
-        const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
-        const long long o = (long long)c * a.ntot + row0 + wr;
-        if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
-      }
-    }
+    store_tile(row0);
   }
 }
 
@@ -211,10 +217,11 @@ static int launch_qgemm_m(const QArgs& a, int M, hipStream_t s) {
   return -1;
 }
 
-// Returns -1 when the call is outside this kernel's range (the caller then takes the dot2 kernel): plain single-segment linears
-// of the block-pair / superblock formats with 3 <= M <= 8.
+// Returns -1 when the call is outside this kernel's range (the caller then takes the dot2 kernel): plain linears over one to three
+// matrices (q / k / v in one launch; with several, each a multiple of 16 rows) of the block-pair / superblock formats with 3 <= M <= 8.
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (M < 3 || M > 8 || a.nseg != 1 || a.epilogue != 0 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue != 0 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (a.nseg > 1) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return -1;      // several matrices: every 16-row group inside one of them
   if (((uintptr_t)a.x & 15) != 0) return -1;
   switch (fmt) {
     case F_Q4_0P: return launch_qgemm_m<F_Q4_0P>(a, M, s);
