@@ -106,9 +106,11 @@ def test_batched_dense_decode(gpu, B):
   prompts = [[int(t) for t in rng.integers(0, 512, size=66)] for _ in range(B)]          # past the first 64-position attention split
   _per_sequence_check(gpu, BatchedTransformer(c, sd, B, max_new=32), SMALL, host, prompts, 12, 128)
 
+@pytest.mark.parametrize("path", ["jobs", "grouped"])
 @pytest.mark.parametrize("B", [1, 2, 5, 8])
-def test_batched_olmoe_arch_decode(gpu, B):
-  """Benchmark configuration 4's architecture (fp16 attention / router, MXFP4 experts, full-width q/k norm) at batch 1..8."""
+def test_batched_olmoe_arch_decode(gpu, B, path):
+  """Benchmark configuration 4's architecture (fp16 attention / router, MXFP4 experts, full-width q/k norm) at batch 1..8, with the experts as one
+  GEMV per (sequence, slot) job and as one small-batch GEMM per selected expert."""
   from tinygrad_amd.llm import BatchedTransformer, TransformerConfig, synth_state_moe
   c = TransformerConfig(max_context=128, **SMALL_MOE)
   sd = synth_state_moe(c, seed=1004)
@@ -126,7 +128,9 @@ def test_batched_olmoe_arch_decode(gpu, B):
     if min(gaps) > 1.5e-3: break                                    # (router logits are O(1); fp16 rounding of the activations moves them by a few 1e-4)
   print(f"prompt set {attempt}: smallest router logit gap between the last selected and the first rejected expert {min(gaps):.4f}")
   assert min(gaps) > 1.5e-3
-  _per_sequence_check(gpu, BatchedTransformer(c, sd, B, max_new=32), SMALL_MOE, host, prompts, 16, 128)
+  model = BatchedTransformer(c, sd, B, max_new=32)
+  model.expert_path = path
+  _per_sequence_check(gpu, model, SMALL_MOE, host, prompts, 16, 128)
 
 def test_batched_equals_single_sequence_path(gpu):
   """Sequence b of a batch produces the tokens the batch-1 Transformer produces for the same prompt."""

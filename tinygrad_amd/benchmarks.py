@@ -114,7 +114,7 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, {'graph replay' if use_graph else 'eager launches'} + sync per token)",
           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "expert_bytes_per_token": expert_bytes, "weight_bytes_per_token": model.weight_bytes_per_token(),
           "weight_GBps_over_step": round(model.weight_bytes_per_token() / dt / 1e9, 1)}]
-  # batched decode: B sequences in lockstep (dense linears as small-batch GEMMs, the B * 8 expert jobs grouped by expert)
+  # batched decode: B sequences in lockstep (dense linears as small-batch GEMMs, one expert GEMV per (sequence, slot) job)
   from tinygrad_amd.llm import BatchedTransformer
   sd = {k: v for k, v in model_sd.items()}
   for B in (2, 4, 8):
@@ -128,7 +128,7 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
     dtb = (time.perf_counter() - t0) / steps
     bm.check_state()
     distinct = float(np.mean([len(np.unique(bm.sel.numpy()))]))
-    res.append({"config": 4, "case": f"OLMoE-arch decode B={B} ctx {ctx} (sequences in lockstep, expert jobs grouped by expert; last layer of the last step: {int(distinct)} distinct experts for {B * c.num_experts_per_tok} jobs)",
+    res.append({"config": 4, "case": f"OLMoE-arch decode B={B} ctx {ctx} (sequences in lockstep, one expert GEMV per (sequence, slot) job; last layer of the last step: {int(distinct)} distinct experts for {B * c.num_experts_per_tok} jobs)",
                 "tok_s": round(B / dtb, 1), "ms_per_step": round(dtb * 1e3, 4)})
     del bm
   # the expert GEMVs alone: B tokens x 8 experts, gate/up fused then down, distinct experts per slot, layers rotated

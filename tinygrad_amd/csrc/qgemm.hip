@@ -44,8 +44,9 @@ __global__ __launch_bounds__(QM_THREADS) void qgemm_mfma_kernel(const QArgs args
     const int t = threadIdx.x, wr = t >> 4, c = t & 15;
     const long long nrows = a.n[sg];
     if (c < M && l0 + wr < nrows) {
-      const float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
+      float v = part[0][wr][c] + part[1][wr][c] + part[2][wr][c] + part[3][wr][c];
       const long long o = (long long)c * nrows + l0 + wr;
+      if (a.epilogue == 1) v += (sg == 0 ? a.resid[0] : sg == 1 ? a.resid[1] : a.resid[2])[o];      // y = resid + x W^T (may be in place: each element is read and written by one thread)
       void* yb = sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
       if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
     }
@@ -217,10 +218,11 @@ static int launch_qgemm_m(const QArgs& a, int M, hipStream_t s) {
   return -1;
 }
 
-// Returns -1 when the call is outside this kernel's range (the caller then takes the dot2 kernel): plain linears over one to three
+// Returns -1 when the call is outside this kernel's range (the caller then takes the dot2 kernel): linears (plain or with the residual / bias
+// row added) over one to three
 // matrices (q / k / v in one launch; with several, each a multiple of 16 rows) of the block-pair / superblock formats with 3 <= M <= 8.
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue != 0 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 1 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
   if (a.nseg > 1) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return -1;      // several matrices: every 16-row group inside one of them
   if (((uintptr_t)a.x & 15) != 0) return -1;
   switch (fmt) {

@@ -8,6 +8,7 @@ and one token step is captured once and replayed (the reference's TinyJit replay
 Numerics that differ from the reference's defaults, stated once: activations entering a linear are rounded to fp16
 (reference: fp32 activations x fp16 weights), the KV cache is fp16 (config 3; reference default is fp32)."""
 from __future__ import annotations
+import os
 import ctypes
 from dataclasses import dataclass
 import numpy as np
@@ -552,6 +553,8 @@ class BatchedTransformer:
     self.out_tokens = Buffer((max(1, max_new), B), np.int32).zero_()
     self.stream = rt.Stream()
     self._graphs, self._steps_done = {}, 0
+    self.replay = "cmdlist"                                          # as Transformer.replay
+    self.expert_path = os.environ.get("TGA_EXPERT_PATH", "jobs")      # "jobs": one GEMV per (sequence, slot); "grouped": one small-batch GEMM per selected expert
 
   def _linear(self, layers, x, outs, **kw): qlinear_multi(layers, x, outs, stream=self.stream.handle, **kw)
 
@@ -581,9 +584,13 @@ class BatchedTransformer:
       k = c.num_experts_per_tok                                         # model.py:110-135
       b["router"](self.xn, out=self.router_logits, stream=st)
       moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st)
-      expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
-      experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
-      experts_grouped(b["down_exps"], self.job_table, B * k, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
+      if self.expert_path == "grouped":                                # one small-batch GEMM per selected expert (its weights read once by the kernel)
+        expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
+        experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
+        experts_grouped(b["down_exps"], self.job_table, B * k, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
+      else:                                                              # one GEMV per (sequence, slot) job; an expert picked twice is read twice, the second time from cache
+        b["gate_exps"](self.sel, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
+        b["down_exps"](self.sel, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
       moe_combine(self.y_e, self.probs, self.x, B, k, c.dim, self.x, stream=st)
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
@@ -591,9 +598,9 @@ class BatchedTransformer:
     rt.check(L.tga_argmax_rows_step(self.logits_buf.ptr if with_head else None, B, c.vocab_size, self.state.ptr, self.prompts.ptr, c.max_context, self.tokens.ptr,
                                     self.out_tokens.ptr, self.max_new, st))
 
-  def _graph(self, with_head: bool) -> rt.Graph:
+  def _graph(self, with_head: bool):
     if with_head not in self._graphs:
-      g = rt.Graph(self.stream)
+      g = (rt.CommandList if self.replay == "cmdlist" else rt.Graph)(self.stream)
       with g: self._step(with_head)
       self._graphs[with_head] = g
     return self._graphs[with_head]
