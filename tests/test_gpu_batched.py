@@ -142,3 +142,32 @@ def test_batched_equals_single_sequence_path(gpu):
   got = list(BatchedTransformer(c, sd, 4, max_new=32).generate(prompts, 10))
   single = Transformer(c, sd, max_new=32)
   for b in range(4): assert [g[b] for g in got] == list(single.generate(prompts[b], 10)), b
+
+GLM_LIKE = dict(num_blocks=3, dim=512, hidden_dim=256, n_heads=8, n_kv_heads=2, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,
+                num_experts=8, num_experts_per_tok=2, norm_topk_prob=True, expert_gating_func=2, routed_scaling_factor=1.5,
+                leading_dense_blocks=1, dense_hidden_dim=768, shared_expert_dim=256, shared_expert_gate=True, expert_bias=True)
+
+@pytest.mark.parametrize("B,gate", [(2, True), (5, True), (4, False)])
+def test_batched_glm4moe_like_decode(gpu, B, gate):
+  """A leading dense block, sigmoid gating with a selection bias, scaled normalised weights and a (gated or plain) shared expert, at batch 2..5."""
+  from tinygrad_amd.llm import BatchedTransformer, TransformerConfig, synth_state_moe
+  cfg = dict(GLM_LIKE, shared_expert_gate=gate)
+  c = TransformerConfig(max_context=128, **cfg)
+  sd = synth_state_moe(c, seed=1010)
+  gpu.synchronize()
+  host = {k: (b.numpy(), t, shp) for k, (b, t, shp) in sd.items()}
+  # prompts clear of selection near-ties, as above.  The ranked quantity is sigmoid(logit) + bias here: a sigmoid passes on at most a quarter of
+  # a logit's rounding noise, so the bar is a quarter of the one on router logits.
+  bar = 4e-4
+  for attempt in range(40):
+    rng = np.random.default_rng(20 + B + 100 * attempt)
+    prompts = [[int(t) for t in rng.integers(0, 512, size=12)] for _ in range(B)]
+    gaps = []
+    for p in prompts:
+      o = ollm.Model(cfg, host, 128, act_round_f16=False); o.generate(p, 16); gaps.append(o.min_route_gap)
+    if min(gaps) > bar: break
+  print(f"prompt set {attempt}: smallest biased-score gap {min(gaps):.4f}")
+  assert min(gaps) > bar
+  model = BatchedTransformer(c, sd, B, max_new=32)
+  assert [b["moe"] for b in model.blk] == [False, True, True]
+  _per_sequence_check(gpu, model, cfg, host, prompts, 16, 128)

@@ -31,7 +31,8 @@ int tga_device_name(char* buf, size_t len) {
   int dev = 0; hipDeviceProp_t p;
   TGA_HIP(hipGetDevice(&dev));
   TGA_HIP(hipGetDeviceProperties(&p, dev));
-  snprintf(buf, len, "%s (%s, %d CUs, %.0f MHz)", p.name, p.gcnArchName, p.multiProcessorCount, p.clockRate / 1000.0);
+  // (the marketing name is empty on some driver / container combinations: the architecture string then stands for it)
+  snprintf(buf, len, "%s (%s, %d CUs, %.0f MHz)", p.name[0] ? p.name : "AMD GPU", p.gcnArchName, p.multiProcessorCount, p.clockRate / 1000.0);
   return 0;
 }
 

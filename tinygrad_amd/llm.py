@@ -504,8 +504,6 @@ class BatchedTransformer:
   config as Transformer; every sequence has its own KV cache; prompts of one batch have equal length."""
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024):
     if not 1 <= batch <= 8: raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
-    if config.leading_dense_blocks or config.shared_expert_dim or config.expert_bias:
-      raise NotImplementedError("leading dense blocks, shared experts and the expert selection bias are built for batch 1 (Transformer) only")
     self.config, self.batch, self.max_new = config, batch, max_new
     c, B = config, batch
     f32, f16 = np.float32, np.float16
@@ -525,10 +523,16 @@ class BatchedTransformer:
       b["k_norm"] = state_dict[p + "attn_k_norm.weight"][0] if c.qk_norm else None
       if p + "attn_q.bias" in state_dict:                                # Linear(bias=qkv_bias), model.py:161-163: one bias row per sequence for the additive epilogue
         b["bias"] = [Buffer.from_numpy(np.tile(state_dict[p + f"attn_{n}.bias"][0].numpy().view(np.uint8).view(f32).reshape(1, -1), (B, 1))) for n in "qkv"]
-      if c.num_experts:
+      b["moe"] = c.num_experts > 0 and i >= c.leading_dense_blocks       # leading blocks of an MoE model are dense (model.py:84)
+      if b["moe"]:
         ex = lambda name: ExpertWeights(state_dict[p + name][0], state_dict[p + name][1], *state_dict[p + name][2])
         b["router"] = lin(p + "ffn_gate_inp.weight")
         b["gate_exps"], b["up_exps"], b["down_exps"] = ex("ffn_gate_exps.weight"), ex("ffn_up_exps.weight"), ex("ffn_down_exps.weight")
+        b["sel_bias"] = state_dict[p + "exp_probs_b.bias"][0] if c.expert_bias else None
+        if c.shared_expert_dim:                                          # model.py:99-103, 131-134
+          for nm in ("ffn_gate_shexp", "ffn_up_shexp", "ffn_down_shexp"): b[nm] = lin(p + nm + ".weight")
+          b["gate_inp_shexp"] = lin(p + "ffn_gate_inp_shexp.weight") if c.shared_expert_gate else None
+          if b["ffn_gate_shexp"].ggml_type != b["ffn_up_shexp"].ggml_type: raise NotImplementedError("ffn_gate_shexp and ffn_up_shexp of different ggml types are not built")
       else:
         for nm in ("ffn_gate", "ffn_up", "ffn_down"): b[nm] = lin(p + nm + ".weight")
         if b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
@@ -542,7 +546,10 @@ class BatchedTransformer:
     self.q, self.k, self.v = Buffer((B, nq), f32), Buffer((B, nkv), f32), Buffer((B, nkv), f32)
     self.attn = Buffer((B, nq), f16)
     self.attn_part = Buffer((B * c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
-    self.act = Buffer((B, max(1, c.hidden_dim)), f16)
+    self.act = Buffer((B, max(1, c.hidden_dim, c.dense_hidden_dim)), f16)
+    if c.shared_expert_dim:
+      self.act_sh, self.y_sh = Buffer((B, c.shared_expert_dim), f16), Buffer((B, c.dim), f32)
+      self.p_sh, self.sh_logit, self.sh_sel = Buffer.from_numpy(np.ones(B, dtype=f32)), Buffer((B, 1), f32), Buffer((B,), np.int32)   # weight 1 unless the shared expert is gated
     if c.num_experts:
       self.router_logits, self.sel, self.probs = Buffer((B, c.num_experts), f32), Buffer((B * k,), np.int32), Buffer((B * k,), f32)
       self.job_table, self.job_flags = Buffer((c.num_experts, 16), np.int32).zero_(), Buffer((1,), np.int32).zero_()
@@ -577,13 +584,13 @@ class BatchedTransformer:
       self._linear([b["attn_output"]], self.attn, [self.x], epilogue=1, resid=[self.x])
       # x = h + feed_forward(ffn_norm(h))                                                   model.py:150
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
-      if not c.num_experts:
+      if not b["moe"]:
         self._linear([b["ffn_gate"], b["ffn_up"]], self.xn, [self.act], epilogue=2)
         self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
         continue
       k = c.num_experts_per_tok                                         # model.py:110-135
       b["router"](self.xn, out=self.router_logits, stream=st)
-      moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st)
+      moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st, bias=b["sel_bias"])
       if self.expert_path == "grouped":                                # one small-batch GEMM per selected expert (its weights read once by the kernel)
         expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
         experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
@@ -592,6 +599,13 @@ class BatchedTransformer:
         b["gate_exps"](self.sel, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
         b["down_exps"](self.sel, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
       moe_combine(self.y_e, self.probs, self.x, B, k, c.dim, self.x, stream=st)
+      if c.shared_expert_dim:                                            # + shared expert, each row scaled by 1 or by sigmoid(xn . ffn_gate_inp_shexp)
+        self._linear([b["ffn_gate_shexp"], b["ffn_up_shexp"]], self.xn, [self.act_sh], epilogue=2)
+        self._linear([b["ffn_down_shexp"]], self.act_sh, [self.y_sh])
+        if b["gate_inp_shexp"] is not None:
+          b["gate_inp_shexp"](self.xn, out=self.sh_logit, stream=st)
+          moe_gate(self.sh_logit, B, 1, 1, self.sh_sel, self.p_sh, 2, False, 1.0, stream=st)
+        moe_combine(self.y_sh, self.p_sh, self.x, B, 1, c.dim, self.x, stream=st)
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       self.output(self.xn, out=self.logits_buf, stream=st)
