@@ -269,6 +269,12 @@ int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_
  * configuration 5's size.  No packed-scale operands (they are unused). */
 int tga_grouped_mxfp8_gemm_routed(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
                                   int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
+/* The routed-tiles product for callers that also know how many rows of every expert are routed (Routing.counts, moe_routing.py:109-127): inside an
+ * expert's range the rows at or beyond its count are padding (dispatch zeroes them); their 16-row groups are not multiplied and their rows of C are
+ * written as zeros.  With zero padding rows of A and finite weights that is the reference's result; when the padding rows of A are not zero
+ * (e.g. the second GEMM of a feed-forward whose first GEMM added an expert bias to them) these rows differ from it - combine never reads them. */
+int tga_grouped_mxfp8_gemm_counts(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off, const int32_t* counts,
+                                  int64_t M, int64_t N, int64_t K, int n_experts, void* stream);
 /* Device symbol for a pre-compiled PROGRAM bound through Tensor.custom_kernel (tinygrad/tensor.py:390-396, extra/gemm/moe_gemm.py:36-48):
  *   extern "C" __global__ void tga_grouped_mxfp8_gemm_kernel(bf16* C, const fp8* A, const fp8* B, const uint32_t* x_si, const uint32_t* w_si,
  *                                                            const uint8_t* x_e8, const uint8_t* w_e8, const int32_t* expert_off,

@@ -196,3 +196,30 @@ def test_moe_feed_forward_composition(gpu):
     print(f"moe_feed_forward vs per-expert loop (routed_only={routed_only}): mean rel-err {err:.2e}")
     assert err < 1e-2
     np.testing.assert_allclose(got, ref, rtol=0.05, atol=0.02 * np.abs(ref).max())
+
+def test_grouped_gemm_with_counts_skips_padding(gpu):
+  """tga_grouped_mxfp8_gemm_counts: routed rows equal the routed-tiles product bit for bit; padding rows inside an expert's range come out as zeros even
+  when A holds garbage there; rows beyond expert_off[E] keep their contents.  Experts of 1, 16, 17, 128, 129, 255, 256 and 300 rows and an empty one."""
+  rng = np.random.default_rng(41)
+  counts = np.array([1, 16, 17, 0, 128, 129, 255, 256, 300], np.int32)
+  E, N, K = len(counts), 512, 384
+  off = np.concatenate([[0], np.cumsum((counts + 255) // 256 * 256)]).astype(np.int32)
+  M = int(off[-1]) + 512                                              # two tiles beyond the routed range
+  def rand_mx(rows):
+    q = rng.integers(0, 256, size=(rows, K), dtype=np.uint8); q[(q & 0x7F) == 0x7F] = 0x38
+    return q, rng.integers(121, 126, size=(rows, K // 32), dtype=np.uint8)
+  xq, xe = rand_mx(M); wq, we = rand_mx(E * N)                         # padding rows of A are random too: they must not reach the output
+  bufs = [gpu.Buffer.from_numpy(a) for a in (xq, wq, xe, we)]
+  offb, cntb = gpu.Buffer.from_numpy(off), gpu.Buffer.from_numpy(counts)
+  C1, C2 = gpu.Buffer((M, N), np.uint16), gpu.Buffer((M, N), np.uint16)
+  for C in (C1, C2): gpu.check(gpu.lib().tga_memset(C.ptr, 0xAB, C.nbytes, None))
+  gpu.check(gpu.lib().tga_grouped_mxfp8_gemm_routed(C1.ptr, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, offb.ptr, M, N, K, E, None))
+  gpu.check(gpu.lib().tga_grouped_mxfp8_gemm_counts(C2.ptr, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, offb.ptr, cntb.ptr, M, N, K, E, None))
+  c1, c2 = C1.numpy(), C2.numpy()
+  for e in range(E):
+    lo, n, hi = int(off[e]), int(counts[e]), int(off[e + 1])
+    np.testing.assert_array_equal(c2[lo:lo + n], c1[lo:lo + n], err_msg=f"routed rows of expert {e}")
+    pad16 = lo + (n + 15) // 16 * 16                                  # rows of a 16-row group that also holds routed rows are multiplied like them
+    np.testing.assert_array_equal(c2[lo + n:pad16], c1[lo + n:pad16])
+    assert (c2[pad16:hi] == 0).all(), f"padding rows of expert {e}"
+  assert (c2[off[-1]:] == 0xABAB).all()

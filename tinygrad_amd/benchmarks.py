@@ -192,6 +192,8 @@ def config5():
     us = _time_launches(fn, 1, 50, s)
     fn_all = lambda i: rt.check(L.tga_grouped_mxfp8_gemm(out.ptr, xq.ptr, wq.ptr, None, None, xe.ptr, we.ptr, r.off.ptr, r.m_l, N, K, E, s.handle))
     us_all = _time_launches(fn_all, 1, 50, s)
+    fn_cnt = lambda i: rt.check(L.tga_grouped_mxfp8_gemm_counts(out.ptr, xq.ptr, wq.ptr, xe.ptr, we.ptr, r.off.ptr, r.counts.ptr, r.m_l, N, K, E, s.handle))
+    us_cnt = _time_launches(fn_cnt, 1, 50, s)
     flops_unpadded = 2 * T * k * N * K
     flops_padded = 2 * m_used * N * K
     nbytes = E * N * K + E * N * K // 32 + T * k * K + T * k * K // 32 + T * k * N * 2
@@ -200,7 +202,8 @@ def config5():
                 "TFLOPs_unpadded": round(flops_unpadded / us / 1e6, 1), "mfma_utilisation_vs_5_PFLOPs": round(flops_unpadded / us / 1e6 / MFMA_FP8_PEAK_TFLOPS, 4),
                 "TFLOPs_with_padding_rows": round(flops_padded / us / 1e6, 1), "alg_bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                 "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                "avg_us_all_tiles_of_m_l": round(us_all, 1), "rows_m_l": int(r.m_l)})
+                "avg_us_all_tiles_of_m_l": round(us_all, 1), "rows_m_l": int(r.m_l),
+                "avg_us_routed_rows_only": round(us_cnt, 1), "mfma_utilisation_routed_rows_only": round(flops_unpadded / us_cnt / 1e6 / MFMA_FP8_PEAK_TFLOPS, 4)})
   return res
 
 def traffic(steps: int = 4):

@@ -228,6 +228,7 @@ struct GemmArgs {
   uint16_t* C; const uint8_t* A; const uint8_t* B; const uint8_t* a_e8; const uint8_t* b_e8; const int* off;
   int M, N, K, E;
   int routed_only;          // != 0: tiles at or beyond expert_off[E] are skipped (their rows of C keep their contents)
+  const int* counts;        // optional: routed rows per expert; rows of an expert's range at or beyond its count are padding - not multiplied, written as zeros
 };
 
 // ---- LDS-tiled variant: 256 x 256 output tile per workgroup, 8 waves as 2 (M) x 4 (N), each 128 x 64 = 8 x 4 MFMAs per K step of
@@ -276,7 +277,7 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {          // round to nearest even (tinygrad/dtype.py:224-226); one v_cvt_pk_bf16_f32
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
-struct GGCur { const uint8_t* A; const uint8_t* B; const uint8_t* sc; int row0, tn; };   // scalar (wave-uniform) state of one tile
+struct GGCur { const uint8_t* A; const uint8_t* B; const uint8_t* sc; int row0, tn, valid; };   // valid: rows of the tile that are not padding   // scalar (wave-uniform) state of one tile
 
 __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8_t* smem, int* s_off) {
   const int tiles_n = g.N / GG_TILE, tiles_total = (g.M / GG_TILE) * tiles_n;
@@ -306,6 +307,11 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
       const int mid = (lo + hi) >> 1;
       const int v = off_in_lds ? __builtin_amdgcn_readfirstlane(s_off[mid]) : g.off[mid];
       if (v <= c.row0) lo = mid; else hi = mid;
+    }
+    c.valid = GG_TILE;
+    if (g.counts && c.row0 < off_end) {                         // (tiles beyond the routed range have no count: all of their rows are multiplied)
+      const int first = off_in_lds ? __builtin_amdgcn_readfirstlane(s_off[lo]) : g.off[lo];
+      c.valid = min(max(first + g.counts[lo] - c.row0, 0), GG_TILE);
     }
     const size_t wrow = (size_t)lo * g.N + (size_t)c.tn * GG_TILE;
     c.A = g.A + (size_t)c.row0 * g.K;
@@ -370,6 +376,8 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
 #pragma unroll
       for (int j = 0; j < 4; j++) acc[i][j] = v4f32{0.f, 0.f, 0.f, 0.f};
 
+    // 16-row sub-tiles of this wave that hold routed rows (8 without counts); the others keep their zero accumulators
+    const int nsub = min(max((cur.valid - wm * 128 + 15) >> 4, 0), 8);
     for (int s = 0; s < nsteps; s++) {
       const bool lastk = s + 1 == nsteps;
       GGCur src = cur;
@@ -385,6 +393,7 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
       const uint32_t* sA = (const uint32_t*)(base + 2 * GG_TILE * 128) + wm * 128 + r16;
       const uint32_t* sB = (const uint32_t*)(base + 2 * GG_TILE * 128) + GG_TILE + wn * 64 + r16;
       v8i32 bf[4]; int sb[4];
+      if (nsub > 0)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const u32x4 y0 = *(const u32x4*)(Bs + j * 2048 + f0), y1 = *(const u32x4*)(Bs + j * 2048 + f1);
@@ -398,16 +407,18 @@ __device__ __forceinline__ void grouped_mxfp8_gemm_tile(const GemmArgs& g, uint8
         sa = (int)sA[16 * i];
       };
       v8i32 af[2]; int sa[2];
-      frag(0, af[0], sa[0]);
+      if (nsub > 0) frag(0, af[0], sa[0]);
 #pragma unroll
       for (int i = 0; i < 8; i++) {
-        if (i + 1 < 8) frag(i + 1, af[(i + 1) & 1], sa[(i + 1) & 1]);
+        if (i + 1 < nsub) frag(i + 1, af[(i + 1) & 1], sa[(i + 1) & 1]);
         if (i < 4) { load_piece(src, ls, 2 * i); load_piece(src, ls, 2 * i + 1); }
         __builtin_amdgcn_sched_barrier(0);
-        const int sai = sa[i & 1] >> (8 * kg);
+        if (i < nsub) {                                         // (a branch around LDS reads and MFMAs only: the global loads stay unconditional)
+          const int sai = sa[i & 1] >> (8 * kg);
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, 0, sb[j], 0, sai);
+          for (int j = 0; j < 4; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[j], af[i & 1], acc[i][j], 0, 0, 0, sb[j], 0, sai);
+        }
         __builtin_amdgcn_sched_barrier(0);
         // the other stage was last read one step ago: the landed pieces go there while the second half of the MFMAs runs
         if (i >= 4) { store_piece((par + s + 1) & 1, 2 * (i - 4)); store_piece((par + s + 1) & 1, 2 * (i - 4) + 1); __builtin_amdgcn_sched_barrier(0); }
@@ -463,7 +474,7 @@ extern "C" __global__ __launch_bounds__(GG_THREADS) void tga_grouped_mxfp8_gemm_
   __shared__ __attribute__((aligned(16))) uint8_t smem[2 * GG_STAGE_BYTES];
   __shared__ int s_off[GG_OFF_MAX];
   (void)x_si; (void)w_si;
-  GemmArgs g; g.C = C; g.A = A; g.B = B; g.a_e8 = x_e8; g.b_e8 = w_e8; g.off = expert_off; g.M = M; g.N = N; g.K = K; g.E = E; g.routed_only = 0;
+  GemmArgs g; g.C = C; g.A = A; g.B = B; g.a_e8 = x_e8; g.b_e8 = w_e8; g.off = expert_off; g.M = M; g.N = N; g.K = K; g.E = E; g.routed_only = 0; g.counts = nullptr;
   grouped_mxfp8_gemm_tile(g, smem, s_off);
 }
 
@@ -605,7 +616,7 @@ int tga_moe_combine_rows(const void* z_bf16, const int32_t* dest_row, const floa
 }
 
 static int grouped_mxfp8_gemm_launch(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
-                                     int64_t M, int64_t N, int64_t K, int n_experts, int routed_only, void* stream) {
+                                     int64_t M, int64_t N, int64_t K, int n_experts, int routed_only, const int32_t* counts, void* stream) {
   TGA_REQUIRE(C && A && B && x_e8 && w_e8 && expert_off, "tga_grouped_mxfp8_gemm: null pointer");
   // the reference's precondition (extra/gemm/moe_gemm.py:120)
   TGA_REQUIRE(M % 256 == 0 && N % 256 == 0 && K % 128 == 0, "grouped mxfp8 needs M%%256,N%%256,K%%128, got (%lld, %lld) (%d, %lld, %lld)",
@@ -613,7 +624,7 @@ static int grouped_mxfp8_gemm_launch(void* C, const void* A, const void* B, cons
   TGA_REQUIRE(M > 0 && N > 0 && K > 0 && n_experts >= 1 && (M / GG_TILE) * (N / GG_TILE) < (1ll << 31) && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
               "tga_grouped_mxfp8_gemm: empty or oversized problem (%lld, %lld, %lld), %d experts", (long long)M, (long long)N, (long long)K, n_experts);
   GemmArgs g; g.C = (uint16_t*)C; g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.a_e8 = (const uint8_t*)x_e8; g.b_e8 = (const uint8_t*)w_e8;
-  g.off = expert_off; g.M = (int)M; g.N = (int)N; g.K = (int)K; g.E = n_experts; g.routed_only = routed_only;
+  g.off = expert_off; g.M = (int)M; g.N = (int)N; g.K = (int)K; g.E = n_experts; g.routed_only = routed_only; g.counts = counts;
   // one workgroup per CU (its 148 KB of LDS fill the CU anyway); each walks its share of the tiles
   static const int n_cu = [] { int dev = 0, n = 0; return (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256; }();
   const long long tiles = (M / GG_TILE) * (N / GG_TILE);
@@ -625,12 +636,18 @@ static int grouped_mxfp8_gemm_launch(void* C, const void* A, const void* B, cons
 int tga_grouped_mxfp8_gemm(void* C, const void* A, const void* B, const void* x_si, const void* w_si, const void* x_e8, const void* w_e8,
                            const int32_t* expert_off, int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
   (void)x_si; (void)w_si;   // the packed (K/128, rows) scale copies the reference's kernel reads are accepted but not needed here
-  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 0, stream);
+  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 0, nullptr, stream);
 }
 
 int tga_grouped_mxfp8_gemm_routed(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off,
                                   int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
-  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 1, stream);
+  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 1, nullptr, stream);
+}
+
+int tga_grouped_mxfp8_gemm_counts(void* C, const void* A, const void* B, const void* x_e8, const void* w_e8, const int32_t* expert_off, const int32_t* counts,
+                                  int64_t M, int64_t N, int64_t K, int n_experts, void* stream) {
+  TGA_REQUIRE(counts, "tga_grouped_mxfp8_gemm_counts: null counts");
+  return grouped_mxfp8_gemm_launch(C, A, B, x_e8, w_e8, expert_off, M, N, K, n_experts, 1, counts, stream);
 }
 
 int tga_kernel_symbol(const char* name, const void** host_function) {

@@ -90,11 +90,13 @@ def transpose_quantize_mxfp8(g: Buffer, stream=None):
   rt.check(rt.lib().tga_transpose_quantize_mxfp8(g.ptr, M, N, q.ptr, e8.ptr, packed.ptr if packed is not None else None, stream))
   return q, e8, packed
 
-def grouped_mx_gemm(x: Buffer | tuple, w: tuple[Buffer, Buffer], expert_off: Buffer, stream=None, out: Buffer | None = None, routed_only: bool = False) -> Buffer:
+def grouped_mx_gemm(x: Buffer | tuple, w: tuple[Buffer, Buffer], expert_off: Buffer, stream=None, out: Buffer | None = None, routed_only: bool = False,
+                    counts: Buffer | None = None) -> Buffer:
   """moe_gemm.py:112-134 with pre-quantized weights w = (w_q (E,N,K) e4m3 bits, w_e8 (E,N,K/32)): quantizes x (M,K) bf16 to MXFP8 and
   runs the grouped GEMM; returns (M, N) bf16 bits.  x may also be an already quantized (x_q, x_e8) pair (a producer that quantizes for itself,
   e.g. fused_silu_mul_quantize_mxfp8).  routed_only: skip the tiles at or beyond expert_off[E] (their rows of the result are not written);
-  the default writes every tile as the reference does."""
+  the default writes every tile as the reference does.  counts (with routed_only): the routed rows per expert - padding rows inside an expert's
+  range are not multiplied and come out as zeros."""
   w_q, w_e8 = w
   E, N, K2 = w_q.shape
   M, K = x[0].shape if isinstance(x, tuple) else x.shape
@@ -102,7 +104,9 @@ def grouped_mx_gemm(x: Buffer | tuple, w: tuple[Buffer, Buffer], expert_off: Buf
   assert M % 256 == 0 and N % 256 == 0 and K % 128 == 0, f"grouped mxfp8 needs M%256,N%256,K%128, got {(M, K)} {w_q.shape}"   # moe_gemm.py:120
   x_q, x_e8, x_si = (x[0], x[1], None) if isinstance(x, tuple) else quantize_mxfp8(x, stream)
   o = out if out is not None else Buffer((M, N), np.uint16)
-  if routed_only: rt.check(rt.lib().tga_grouped_mxfp8_gemm_routed(o.ptr, x_q.ptr, w_q.ptr, x_e8.ptr, w_e8.ptr, expert_off.ptr, M, N, K, E, stream))
+  if routed_only and counts is not None:
+    rt.check(rt.lib().tga_grouped_mxfp8_gemm_counts(o.ptr, x_q.ptr, w_q.ptr, x_e8.ptr, w_e8.ptr, expert_off.ptr, counts.ptr, M, N, K, E, stream))
+  elif routed_only: rt.check(rt.lib().tga_grouped_mxfp8_gemm_routed(o.ptr, x_q.ptr, w_q.ptr, x_e8.ptr, w_e8.ptr, expert_off.ptr, M, N, K, E, stream))
   else: rt.check(rt.lib().tga_grouped_mxfp8_gemm(o.ptr, x_q.ptr, w_q.ptr, x_si.ptr if x_si is not None else None, None, x_e8.ptr, w_e8.ptr, expert_off.ptr, M, N, K, E, stream))
   o._keep = (x_q, x_e8, x_si)
   return o
@@ -143,9 +147,10 @@ def moe_feed_forward(inp: Buffer, logits: Buffer, experts_per_tok: int, w_gate_u
   assert D % 256 == 0 and N2 % 256 == 0 and (N2 // 2) % 256 == 0, f"dim {D}, 2*inter {N2} and inter {N2 // 2} must be multiples of 256"
   r = route(logits, experts_per_tok, E, stream)
   xg = dispatch(inp, r, stream)
-  h = add_expert_bias(grouped_mx_gemm(xg, w_gate_up, r.off, stream, routed_only=routed_only), b_gate_up, r.off, stream)
+  cnt = r.counts if routed_only else None                     # padding rows are never gathered by combine: their 16-row groups are not multiplied
+  h = add_expert_bias(grouped_mx_gemm(xg, w_gate_up, r.off, stream, routed_only=routed_only, counts=cnt), b_gate_up, r.off, stream)
   y = swiglu(h, swiglu_limit, stream=stream)
-  z = add_expert_bias(grouped_mx_gemm(y, w_down, r.off, stream, routed_only=routed_only), b_down, r.off, stream)
+  z = add_expert_bias(grouped_mx_gemm(y, w_down, r.off, stream, routed_only=routed_only, counts=cnt), b_down, r.off, stream)
   out = combine(z, r, T, experts_per_tok, stream)
   out._keep = (r, xg, h, y, z)                                                  # alive until the stream has run
   return out

@@ -54,6 +54,7 @@ def _declare(lib):
     "tga_moe_combine_rows": [vp, vp, vp, i, i, i, vp, vp],
     "tga_grouped_mxfp8_gemm": [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
     "tga_grouped_mxfp8_gemm_routed": [vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
+    "tga_grouped_mxfp8_gemm_counts": [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i, vp],
     "tga_kernel_symbol": [ctypes.c_char_p, c_void_pp], "tga_launch_kernel": [vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32), c_void_pp, vp],
     "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
     "tga_add_expert_bias": [vp, vp, vp, i64, i64, i, vp],
