@@ -60,14 +60,34 @@ def test_context_and_token_guards(gpu):
   gpu.check(gpu.lib().tga_argmax_step(lgb.ptr, lg.size, sv.ptr, si.ptr, stb.ptr, pr.ptr, outt.ptr, 4, None))
   assert outt.numpy()[0] == 0
 
-def test_graph_replay_equals_eager(gpu):
+@pytest.mark.parametrize("replay", ["cmdlist", "graph"])
+def test_graph_replay_equals_eager(gpu, replay):
+  """The captured step replayed as plain launches in capture order (tga_cmdlist_*) and through hipGraphLaunch: same tokens and logits as eager
+  launches, over several replays with host synchronisation between them."""
   model, _ = _build(gpu, SMALL, 128, seed=77)
+  model.replay = replay
   prompt = [5, 17, 300, 42, 8]
   a = list(model.generate(prompt, 16, use_graph=False))
   la = model.logits().copy()
   b = list(model.generate(prompt, 16, use_graph=True))
   assert a == b
   np.testing.assert_array_equal(la, model.logits())
+  if replay == "cmdlist": assert len(model._graph(True)) > 10                          # one entry per kernel of the step
+
+def test_command_list_takes_kernel_launches_only(gpu):
+  """A capture that holds anything but kernel launches (here a memset) is refused when the list is built; the stream stays usable."""
+  from tinygrad_amd import runtime as rt
+  s = rt.Stream()
+  buf = gpu.Buffer((256,), np.float32)
+  cl = rt.CommandList(s)
+  with pytest.raises(RuntimeError, match="not a kernel launch"):
+    with cl: gpu.check(gpu.lib().tga_memset(buf.ptr, 0, buf.nbytes, s.handle))
+  ok = rt.CommandList(s)
+  with ok: gpu.check(gpu.lib().tga_synth_weights(0, buf.ptr, 256, 1, 3.0, s.handle))    # a fill kernel: float32 "weights" are a constant fill
+  assert len(ok) == 1
+  for _ in range(3): ok.launch()
+  s.synchronize()
+  assert (buf.numpy() == 3.0).all()
 
 # wider shapes: head_dim 128, K split over four waves (K > 4096), Q8_0
 WIDE = dict(num_blocks=2, dim=1024, hidden_dim=4608, n_heads=8, n_kv_heads=1, norm_eps=1e-5, vocab_size=512, head_dim=128, rope_theta=10000.0)
