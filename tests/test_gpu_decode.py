@@ -74,6 +74,36 @@ def test_graph_replay_equals_eager(gpu, replay):
   np.testing.assert_array_equal(la, model.logits())
   if replay == "cmdlist": assert len(model._graph(True)) > 10                          # one entry per kernel of the step
 
+def test_kv_prefix_reuse_equals_fresh_model(gpu):
+  """A prompt that shares a prefix with what the KV cache holds is prefilled from the first differing position only (Transformer.get_start_pos,
+  tinygrad/llm/model.py:455-462, used at 472-473), with the tokens and logits of a model that starts from nothing; a follow-up turn (prompt +
+  reply + new tokens) runs only the new tokens."""
+  model, _ = _build(gpu, SMALL, 128, seed=11)
+  fresh, _ = _build(gpu, SMALL, 128, seed=11)
+  rng = np.random.default_rng(11)
+  p1 = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=70)]
+  p2 = p1[:40] + [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=12)]
+  if p2[40] == p1[40]: p2[40] = (p2[40] + 1) % SMALL["vocab_size"]
+  list(model.generate(p1, 8))
+  assert model.prefill_steps == 69
+  assert model.get_start_pos(p2) == 40
+  got = list(model.generate(p2, 8)); lg = model.logits().copy()
+  assert model.prefill_steps == len(p2) - 1 - 40
+  want = list(fresh.generate(p2, 8))
+  assert fresh.prefill_steps == len(p2) - 1
+  assert got == want
+  np.testing.assert_array_equal(lg, fresh.logits())
+  p3 = p2 + got + [7, 9, 11]                                                            # the next turn of a conversation
+  got3 = list(model.generate(p3, 8)); lg3 = model.logits().copy()
+  assert model.prefill_steps == 3
+  fresh2, _ = _build(gpu, SMALL, 128, seed=11)
+  assert got3 == list(fresh2.generate(p3, 8))
+  np.testing.assert_array_equal(lg3, fresh2.logits())
+  assert model.get_start_pos(p3) == len(p3) - 1                                          # the same prompt again: nothing to prefill
+  assert list(model.generate(p3, 8)) == got3 and model.prefill_steps == 0
+  model.prefill(p3, reuse_cache=False)
+  assert model.prefill_steps == len(p3) - 1
+
 def test_command_list_takes_kernel_launches_only(gpu):
   """A capture that holds anything but kernel launches (here a memset) is refused when the list is built; the stream stays usable."""
   from tinygrad_amd import runtime as rt

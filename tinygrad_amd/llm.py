@@ -337,6 +337,7 @@ class Transformer:
     self.stream = rt.Stream()
     self._graphs = {}
     self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
+    self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
 
   def check_state(self):
@@ -445,24 +446,40 @@ class Transformer:
       raise NotImplementedError(f"tensors the built path does not consume: {left[:8]}{' ...' if len(left) > 8 else ''}")
     return model, kv
 
-  def reset(self, tokens: list[int]):
-    """Start a new sequence: position 0, first prompt token loaded, nothing cached (no KV-prefix reuse)."""
+  def get_start_pos(self, tokens: list[int]) -> int:
+    """How many leading positions of the KV cache can be kept for this prompt (Transformer.get_start_pos, model.py:455-462): the longest common
+    prefix of tokens[:-1] and the tokens whose keys and values the cache holds."""
+    n = 0
+    for a, b in zip(tokens[:-1], self._cached_tokens):
+      if a != b: break
+      n += 1
+    return n
+
+  def reset(self, tokens: list[int], start_pos: int = 0):
+    """Start a sequence at position start_pos (the cache rows below it are kept): the prompt table, the position and the first input token."""
     c, s = self.config, self.s
     if not 1 <= len(tokens) < c.max_context: raise ValueError(f"prompt of {len(tokens)} tokens does not fit max_context {c.max_context}")
     if min(tokens) < 0 or max(tokens) >= c.vocab_size: raise ValueError(f"token id outside the vocabulary of {c.vocab_size}")
+    if not 0 <= start_pos < len(tokens): raise ValueError(f"start position {start_pos} outside the prompt of {len(tokens)} tokens")
     prompt = np.zeros(c.max_context, dtype=np.int32); prompt[:len(tokens)] = tokens
     s.prompt.copyin(prompt)
-    st = np.zeros(16, dtype=np.int32); st[1], st[3], st[5] = tokens[0], len(tokens), c.vocab_size
+    st = np.zeros(16, dtype=np.int32); st[0], st[1], st[3], st[5] = start_pos, tokens[start_pos], len(tokens), c.vocab_size
     s.state.copyin(st)
-    self._n_prompt, self._steps_done = len(tokens), 0
+    self._n_prompt, self._steps_done = len(tokens), start_pos
+    self._cached_tokens = list(tokens[:start_pos])
 
-  def prefill(self, tokens: list[int], use_graph: bool = True):
-    """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step."""
-    self.reset(tokens)
-    for _ in range(len(tokens) - 1):
+  def prefill(self, tokens: list[int], use_graph: bool = True, reuse_cache: bool = True):
+    """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step.  Like the reference's generate
+    (model.py:472-473) the positions whose tokens equal what the cache already holds are not recomputed."""
+    start = self.get_start_pos(tokens) if reuse_cache else 0
+    self.reset(tokens, start)
+    self.prefill_steps = len(tokens) - 1 - start                        # (what the last call actually ran)
+    for _ in range(self.prefill_steps):
       if use_graph: self._graph(False).launch()
       else: self._step(False)
     self._steps_done = len(tokens) - 1
+    self._cached_tokens = list(tokens[:-1])
+    self._last_input = tokens[-1]
     self.stream.synchronize()
 
   def decode_step(self, use_graph: bool = True, sync: bool = True):
@@ -472,6 +489,7 @@ class Transformer:
     if use_graph: self._graph(True).launch()
     else: self._step(True)
     self._steps_done += 1
+    self._cached_tokens.append(self._last_input); self._last_input = None    # this step wrote its input token's keys and values; the next input is on the device
     if sync: self.stream.synchronize()
 
   def generate(self, tokens: list[int], max_new_tokens: int, use_graph: bool = True):
@@ -480,7 +498,9 @@ class Transformer:
     self.prefill(tokens, use_graph)
     for i in range(min(max_new_tokens, self.config.max_context - len(tokens), self.max_new)):
       self.decode_step(use_graph, sync=True)                          # the reference syncs once per token too (out.item(), model.py:482)
-      yield int(self.s.out_tokens.view(4 * i, (1,), np.int32).numpy()[0])
+      tok = int(self.s.out_tokens.view(4 * i, (1,), np.int32).numpy()[0])
+      self._last_input = tok                                          # (model.py:483: the cache then holds tokens[:-1])
+      yield tok
     self.check_state()
 
   def logits(self) -> np.ndarray: return self.s.logits.numpy().reshape(-1)
