@@ -138,6 +138,49 @@ def test_multi_segment_small_batch(gpu, t, m):
       wf = w.view(np.float16).astype(np.float32).reshape(n, k) if t == 1 else ol.weight_f32(w, n, k, t)
       assert ol.rel_err(o.numpy(), ol.linear_f64(x.astype(np.float32), wf)) <= TOL, (ns, n)
 
+@pytest.mark.parametrize("t", [2, 8], ids=["q4_0", "q8_0"])
+@pytest.mark.parametrize("n,k,m", [(16, 1024, 3), (4096 + 48, 1024, 8), (14336, 4096, 4), (4112, 4096, 8), (512, 2048, 5), (1040, 8192, 4), (272, 8192, 8), (4096, 3072, 7)])
+def test_small_batch_weights_through_lds(gpu, t, n, k, m):
+  """The matrix-core kernel that streams the weights into LDS with contiguous 16-byte pieces (Q4_0 / Q8_0 pairs, K a multiple of 1024, rows a
+  multiple of 16): one stage per row group (K = 1024) up to eight, one row group per workgroup up to several with a ragged share, the largest
+  activation blocks that still leave room for a ring of three stages, and (8192, M = 8) which does not and takes the register-fed kernel.
+  Against the C restatement (exact weights, float32 accumulate) and, for the first rows, the float64 anchor; float32 and fp16 activations."""
+  rng = np.random.default_rng(n + k + m + t)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  y = _run(gpu, t, w, x, n, k)
+  ref = cref.linear(t, w, x, n, k, threads=8)
+  assert ol.rel_err(y, ref) <= TOL
+  rows = min(n, 64)
+  nel, nby = GGML_QUANT[t]
+  W = ol.weight_f32(w[:rows * (k // nel) * nby], rows, k, t)
+  assert ol.rel_err(y[:, :rows], ol.linear_f64(x.astype(np.float32), W)) <= TOL
+  y32 = _run(gpu, t, w, x.astype(np.float32), n, k)                      # float32 activations are rounded to fp16 while they are staged
+  np.testing.assert_array_equal(y32, y)
+  y16 = _run(gpu, t, w, x, n, k, ydt=np.float16)
+  assert y16.tobytes() == y.astype(np.float16).tobytes()
+
+def test_small_batch_through_lds_segments_and_residual(gpu):
+  """q / k / v of a llama block shape in one launch at M = 4 and the residual epilogue in place, on the LDS-fed kernel's range."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(4242)
+  k, m = 2048, 4
+  ns = [2048, 512, 512]
+  for t in (2, 8):
+    ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+    x = synth.activations(rng, m, k, np.float16)
+    layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+    outs = [gpu.Buffer((m, n), np.float32) for n in ns]
+    for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    xb = gpu.Buffer.from_numpy(x)
+    qlinear_multi(layers, xb, outs)
+    refs = [ol.linear_f64(x.astype(np.float32), ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]
+    for o, r in zip(outs, refs): assert ol.rel_err(o.numpy(), r) <= TOL
+    res = [rng.standard_normal((m, n)).astype(np.float32) for n in ns]
+    rb = [gpu.Buffer.from_numpy(r) for r in res]
+    qlinear_multi(layers, xb, rb, epilogue=1, resid=rb)
+    for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL
+
 def test_argument_errors(gpu):
   from tinygrad_amd.nn import QuantLinear
   w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))

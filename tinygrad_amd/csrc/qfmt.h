@@ -775,33 +775,44 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
 
 // ------------------------------------------------------------------------------------------------ activation staging (M rows, LDS)
 // LDS layout for units [u0, u0+cu): xs[(m*XV + t) * cu + (u-u0)] (u32x4), then cs[(m*NG + j) * cu + (u-u0)] (float)
-template <int T, int M>
-__device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs, int u0, int cu) {
+// one staging item = one unit of one activation row: stage_fetch reads its K values (as fp16 pairs), stage_put writes its vectors to LDS
+template <int T>
+__device__ __forceinline__ void stage_fetch(const QArgs& a, int m, int u, uint32_t* nx) {
   using F = Fmt<T>;
   constexpr int NP = F::UW / 2;
-  for (int i = threadIdx.x; i < M * cu; i += QG_THREADS) {
-    const int m = i / cu, ul = i - m * cu, u = u0 + ul;
-    // four consecutive pairs (8 activations) of a unit are contiguous in every format: 16-byte (fp16) / 2 x 16-byte (fp32) loads
-    uint32_t nx[NP];
-    if (a.x_f32) {
-      const float* x = (const float*)a.x + (long long)m * a.K;
+  // four consecutive pairs (8 activations) of a unit are contiguous in every format: 16-byte (fp16) / 2 x 16-byte (fp32) loads
+  if (a.x_f32) {
+    const float* x = (const float*)a.x + (long long)m * a.K;
 #pragma unroll
-      for (int k = 0; k < NP; k += 4) {
-        const f32x4 lo = *(const f32x4*)(x + F::xoff(u, k)), hi = *(const f32x4*)(x + F::xoff(u, k) + 4);
-        nx[k] = f2h_bits(lo.x) | (f2h_bits(lo.y) << 16); nx[k + 1] = f2h_bits(lo.z) | (f2h_bits(lo.w) << 16);
-        nx[k + 2] = f2h_bits(hi.x) | (f2h_bits(hi.y) << 16); nx[k + 3] = f2h_bits(hi.z) | (f2h_bits(hi.w) << 16);
-      }
-    } else {
-      const uint16_t* x = (const uint16_t*)a.x + (long long)m * a.K;
-#pragma unroll
-      for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(x + F::xoff(u, k)); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+    for (int k = 0; k < NP; k += 4) {
+      const f32x4 lo = *(const f32x4*)(x + F::xoff(u, k)), hi = *(const f32x4*)(x + F::xoff(u, k) + 4);
+      nx[k] = f2h_bits(lo.x) | (f2h_bits(lo.y) << 16); nx[k + 1] = f2h_bits(lo.z) | (f2h_bits(lo.w) << 16);
+      nx[k + 2] = f2h_bits(hi.x) | (f2h_bits(hi.y) << 16); nx[k + 3] = f2h_bits(hi.z) | (f2h_bits(hi.w) << 16);
     }
-    u32x4 xv[F::XV]; float c[F::NG];
-    F::stage(nx, xv, c);
+  } else {
+    const uint16_t* x = (const uint16_t*)a.x + (long long)m * a.K;
 #pragma unroll
-    for (int t = 0; t < F::XV; t++) xs[(m * F::XV + t) * cu + ul] = xv[t];
+    for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(x + F::xoff(u, k)); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+  }
+}
+template <int T>
+__device__ __forceinline__ void stage_put(const uint32_t* nx, u32x4* xs, float* cs, int m, int ul, int cu) {
+  using F = Fmt<T>;
+  u32x4 xv[F::XV]; float c[F::NG];
+  F::stage(nx, xv, c);
 #pragma unroll
-    for (int j = 0; j < F::NG; j++) cs[(m * F::NG + j) * cu + ul] = c[j];
+  for (int t = 0; t < F::XV; t++) xs[(m * F::XV + t) * cu + ul] = xv[t];
+#pragma unroll
+  for (int j = 0; j < F::NG; j++) cs[(m * F::NG + j) * cu + ul] = c[j];
+}
+template <int T, int M, int NT = QG_THREADS>
+__device__ __forceinline__ void stage_chunk(const QArgs& a, u32x4* xs, float* cs, int u0, int cu, int first = -1) {
+  using F = Fmt<T>;
+  for (int i = first < 0 ? (int)threadIdx.x : first; i < M * cu; i += NT) {
+    const int m = i / cu, ul = i - m * cu;
+    uint32_t nx[F::UW / 2];
+    stage_fetch<T>(a, m, u0 + ul, nx);
+    stage_put<T>(nx, xs, cs, m, ul, cu);
   }
 }
 

@@ -1,0 +1,252 @@
+// Small-batch GEMM over Q4_0 / Q8_0 block pairs (3 <= M <= 8, K <= 4096) with the weights streamed into LDS by direct-to-LDS loads: the same
+// call sites and arithmetic as qgemm.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392;
+// a unit is decoded once into fp16 weights and v_mfma_f32_16x16x32_f16 multiplies it with all activation rows).
+//
+// Why a second kernel.  The MFMA operand layout wants lane (g, r) to hold a unit of weight ROW r, so a register load touches sixteen rows
+// with 144- or 272-byte runs: measured on a 14336 x 4096 Q8_0 matrix, that lane -> address map streams at 3.4 TB/s where fully contiguous
+// 16-byte pieces stream at 5.3 TB/s, and the Q4_0 kernel (half the bytes, the same number of scattered pieces) is no faster than the Q8_0
+// one.  Here global memory is read in contiguous 16-byte pieces, 1 KB per wave instruction (global_load_lds_dwordx4: lane l's piece lands at
+// LDS base + 16 l), and the operand layout is produced by the LDS reads: each lane picks its unit out of the staged rows.
+//
+// A slot is 16 weight rows x 16 units (1024 values of K); its rows lie in LDS with a pitch of one piece more than their length, which
+// spreads the sixteen rows over the banks.  A stage is two slots (2048 values of K): waves 0-3 multiply the four steps (4 units x 16 rows
+// each) of the first, waves 4-7 those of the second.  The eight waves of the workgroup (one per CU) issue a stage's pieces together and
+// keep nb - 1 stages in flight in a ring of nb.  One barrier per stage orders "all pieces of stage s have landed" before its reads and
+// "everyone is done with stage s - 1" before its slots are requested again; the partial tiles of the waves meet in LDS once per row
+// group and are reduced after the next stage's barrier.
+// A wave meets the same units of K in every row group (K <= 4096: at most two), so its activation operands - lane (g, c): the eight
+// vectors of row c's unit, zeros for c >= M - stay in registers for the whole launch; LDS holds nothing but the ring.
+#include "qfmt.h"
+
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+#define QD_NW 8                       // waves per workgroup
+#define QD_SU 16                      // units per stage
+#define QD_LDS_CU (160 * 1024)
+#define QD_MAX_NB 4
+
+template <int T> struct DmaFmt;
+template <> struct DmaFmt<F_Q4_0P> {
+  static constexpr int UB = 36;
+  static __device__ __forceinline__ Fmt<F_Q4_0P>::Raw from_lds(const uint32_t* p) {
+    Fmt<F_Q4_0P>::Raw r;
+    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = p[8];
+    return r;
+  }
+};
+template <> struct DmaFmt<F_Q8_0P> {
+  static constexpr int UB = 68;
+  static __device__ __forceinline__ Fmt<F_Q8_0P>::Raw from_lds(const uint32_t* p) {
+    Fmt<F_Q8_0P>::Raw r;
+    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = u32x4{p[8], p[9], p[10], p[11]}; r.d = u32x4{p[12], p[13], p[14], p[15]}; r.e = p[16];
+    return r;
+  }
+};
+
+// at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave)
+__device__ __forceinline__ void qd_wait_vm(int n) {
+  switch (n) {
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+  }
+}
+
+template <int T_, bool MS, int NSS>
+__global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args, const int M, const int nb) {
+  const QArgs a = args;
+  using F = Fmt<T_>;
+  using DF = DmaFmt<T_>;
+  typedef typename F::Raw Raw;
+  constexpr int UB = DF::UB;
+  constexpr int PR = QD_SU * UB / 16;                    // 16-byte pieces of one row in a slot
+  constexpr int PITCH = (PR + 1) * 16;                   // LDS bytes from one row of the slot to the next
+  constexpr int SLOTS = 16 * (PR + 1);
+  constexpr int NI = (SLOTS + 63) / 64;                  // wave instructions (1 KB each) per slot
+  constexpr int SLOT_BYTES = NI * 1024;
+  constexpr int NI2 = 2 * NI;                            // ... per stage
+  constexpr int IMAX = (NI2 + QD_NW - 1) / QD_NW;        // instructions of one wave per stage, at most
+  constexpr int BASE = NI2 / QD_NW;                      // ... and at least
+  extern __shared__ u32x4 lds[];
+  __shared__ float part[2][QD_NW][16][9];
+  char* ring = (char*)lds;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int half = wave >> 2, step = wave & 3;           // this wave's slot of a stage and its step inside the slot
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  const int cu = a.nu, nslots = cu / QD_SU, spg = (nslots + 1) >> 1;   // stages per row group (NSS >= spg)
+  const long long ngroups = a.ntot / 16;
+  auto seg_of = [&](long long row0, int& sg, long long& local0) {
+    sg = 0; local0 = row0;
+    if constexpr (MS) { if (local0 >= a.n[0]) { local0 -= a.n[0]; sg = 1; if (a.nseg > 2 && local0 >= a.n[1]) { local0 -= a.n[1]; sg = 2; } } }
+  };
+  auto rows_of = [&](int sg) -> long long { return !MS ? a.n[0] : sg == 0 ? a.n[0] : sg == 1 ? a.n[1] : a.n[2]; };
+  auto w_of = [&](int sg) -> const uint8_t* { return !MS ? a.w[0] : sg == 0 ? a.w[0] : sg == 1 ? a.w[1] : a.w[2]; };
+  auto store_tile = [&](long long row0, int p) {                    // 256 threads = 16 weight rows x 16 activation rows
+    int sg; long long l0; seg_of(row0, sg, l0);
+    const int t = threadIdx.x, wr = (t >> 4) & 15, c = t & 15;
+    const long long nrows = rows_of(sg);
+    if (t < 256 && c < M && l0 + wr < nrows) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < QD_NW; w++) v += part[p][w][wr][c];
+      const long long o = (long long)c * nrows + l0 + wr;
+      if (a.epilogue == 1) v += (!MS ? a.resid[0] : sg == 0 ? a.resid[0] : sg == 1 ? a.resid[1] : a.resid[2])[o];
+      void* yb = !MS ? a.y[0] : sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
+      if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
+    }
+  };
+  const long long G = ((long long)blockIdx.x < ngroups) ? (ngroups - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+  const long long S = G * spg;                           // stages of this workgroup
+  if (S == 0) return;
+
+  // where this lane's pieces of a stage come from: position 64 j + lane of the two padded slots = (slot, row, piece); the pad piece of a row
+  // and the positions past the last row repeat a valid piece (they land in the slot's slack).  When K ends inside a stage (an odd number of
+  // slots), the second slot repeats the first: nothing reads it.
+  long long doff[IMAX], doff_odd[IMAX];
+#pragma unroll
+  for (int i = 0; i < IMAX; i++) {
+    const int j = wave + QD_NW * i, sl = j >= NI ? 1 : 0;
+    const int sigma = 64 * (j - sl * NI) + lane;
+    int rr = sigma / (PR + 1), q = sigma - rr * (PR + 1);
+    rr = rr < 16 ? rr : 15; q = q < PR ? q : PR - 1;
+    doff_odd[i] = (long long)rr * a.row_bytes + q * 16;
+    doff[i] = doff_odd[i] + sl * (QD_SU * UB);
+  }
+  long long ij = 0; int ist = 0, islot = 0;              // issue stream: row group index (of this workgroup), stage in the group, ring position
+  auto issue_stage = [&]() {
+    const long long grp = (long long)blockIdx.x + ij * gridDim.x;
+    int sg; long long l0; seg_of(grp * 16, sg, l0);
+    const uint8_t* base = w_of(sg) + l0 * a.row_bytes + (long long)ist * (2 * QD_SU * UB);
+    char* dst = ring + (size_t)islot * (2 * SLOT_BYTES);
+    const bool two = 2 * ist + 1 < nslots;
+#pragma unroll
+    for (int i = 0; i < IMAX; i++) {
+      const int j = wave + QD_NW * i;
+      if (j < NI2)                                                     // (the same for the whole wave)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + (two ? doff[i] : doff_odd[i])), (__attribute__((address_space(3))) void*)(dst + j * 1024), 16, 0, 0);
+    }
+    if (++ist == spg) { ist = 0; ij++; }
+    islot = islot + 1 == nb ? 0 : islot + 1;
+  };
+
+  // this lane's activation operands: requested first (loads return in issue order), the weights second
+  u32x4 bfrag[NSS][F::XV];
+  {
+    uint32_t nx[NSS][F::UW / 2];
+    bool have[NSS];
+#pragma unroll
+    for (int ss = 0; ss < NSS; ss++) {
+      const int u = (2 * ss + half) * QD_SU + 4 * step + g;
+      have[ss] = r < M && u < cu;
+      stage_fetch<T_>(a, r < M ? r : 0, u < cu ? u : cu - 1, nx[ss]);   // (unconditional: a valid row and unit; dropped below)
+    }
+    for (int k = 0; k < nb - 1; k++) if (k < S) issue_stage();
+#pragma unroll
+    for (int ss = 0; ss < NSS; ss++) {
+      float c[F::NG];
+      F::stage(nx[ss], bfrag[ss], c);
+#pragma unroll
+      for (int v = 0; v < F::XV; v++) if (!have[ss]) bfrag[ss][v] = u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+
+  v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  long long cj = 0; int cst = 0, cslot = 0, par = 0;     // compute stream
+  long long pend_row0 = -1; int pend_par = 0;            // row group whose partial tiles wait for the next barrier
+  auto multiply = [&](const u32x4* bv) {
+    const Raw buf = DF::from_lds((const uint32_t*)(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH + (4 * step + g) * UB));
+    uint32_t wv[F::NWV];
+    F::decode(buf, wv, kc);
+    F::to_f16(buf, wv);
+#pragma unroll
+    for (int v = 0; v < F::XV; v++) {
+      const u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
+      if (v & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[v]), acc1, 0, 0, 0);
+      else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[v]), acc0, 0, 0, 0);
+    }
+  };
+  for (long long s = 0; s < S; s++) {
+    const long long after = S - 1 - s;
+    qd_wait_vm((int)(after < nb - 2 ? after : nb - 2) * BASE);         // this wave's pieces of stage s have landed (later stages may be in flight)
+    __syncthreads();                                                   // ... and everyone else's; everyone is done with stage s - 1
+    if (pend_row0 >= 0) { store_tile(pend_row0, pend_par); pend_row0 = -1; }
+    if (s + nb - 1 < S) issue_stage();                                 // into the ring position stage s - 1 was read from
+    if (2 * cst + half < nslots) {                                     // (the slot exists: K may end inside the stage)
+      if (NSS == 1 || cst == 0) multiply(bfrag[0]); else multiply(bfrag[NSS - 1]);
+    }
+    cslot = cslot + 1 == nb ? 0 : cslot + 1;
+    if (++cst == spg) {                                                // row group complete: the waves' partial tiles go to LDS
+      if (r < 9) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
+      }
+      pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * 16; pend_par = par;
+      par ^= 1;
+      acc0 = v4f32{0.f, 0.f, 0.f, 0.f}; acc1 = v4f32{0.f, 0.f, 0.f, 0.f};
+      cst = 0; cj++;
+    }
+  }
+  __syncthreads();
+  if (pend_row0 >= 0) store_tile(pend_row0, pend_par);
+}
+
+static int qd_cu_count() {
+  static int n = 0;
+  if (!n) { int dev = 0; hipDeviceProp_t p; n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess) ? p.multiProcessorCount : 256; }
+  return n;
+}
+
+template <int T, bool MS, int NSS>
+static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hipStream_t s) {
+  auto kern = qgemm_dma_kernel<T, MS, NSS>;
+  static const hipError_t configured = [&]() {
+    hipFuncAttributes fa;
+    hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
+    if (e != hipSuccess) return e;
+    return hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(QD_LDS_CU - fa.sharedSizeBytes));
+  }();
+  TGA_HIP(configured);
+  const long long ngroups = a.ntot / 16;
+  const long long cap = (long long)qd_cu_count() * per_cu;
+  const long long grid = ngroups < cap ? ngroups : cap;
+  kern<<<dim3((unsigned)grid), dim3(QD_NW * 64), lds, s>>>(a, M, nb);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int T>
+static int launch_qd(QArgs a, int M, hipStream_t s) {
+  using F = Fmt<T>;
+  constexpr int UB = DmaFmt<T>::UB;
+  constexpr int STAGE_BYTES = 2 * ((16 * (QD_SU * UB / 16 + 1) + 63) / 64) * 1024;
+  a.nu = a.K / F::UW;
+  a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+  if (a.K % (F::UW * QD_SU) != 0 || a.K > 4 * F::UW * QD_SU) return -1;   // whole slots only, at most four (two stages per row group)
+  constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
+  int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 9 - 1024) / STAGE_BYTES);
+  if (nb > QD_MAX_NB) nb = QD_MAX_NB;
+  if (nb < 2) return -1;
+  const size_t lds = (size_t)nb * STAGE_BYTES;
+  const bool two = a.K > 2 * F::UW * QD_SU;
+  if (a.nseg > 1) return two ? launch_qd_k<T, true, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, true, 1>(a, M, nb, per_cu, lds, s);
+  return two ? launch_qd_k<T, false, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1>(a, M, nb, per_cu, lds, s);
+}
+
+// Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
+// 3 <= M <= 8, K = 1024, 2048, 3072 or 4096, every matrix a multiple of 16 rows at a 16-byte aligned address.
+int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
+  if (fmt != F_Q4_0P && fmt != F_Q8_0P) return -1;
+  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 1 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
+  if (((uintptr_t)a.x & 15) != 0) return -1;
+  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);
+}
