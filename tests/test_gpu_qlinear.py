@@ -160,6 +160,46 @@ def test_small_batch_weights_through_lds(gpu, t, n, k, m):
   y16 = _run(gpu, t, w, x, n, k, ydt=np.float16)
   assert y16.tobytes() == y.astype(np.float16).tobytes()
 
+@pytest.mark.parametrize("t", [2, 8], ids=["q4_0", "q8_0"])
+@pytest.mark.parametrize("n,k", [(300, 4096), (4096 + 3, 4096), (14336, 4096), (200, 14336), (64, 6144), (129, 2112)])
+def test_two_rows_on_the_single_row_kernel(gpu, t, n, k):
+  """M = 2 for Q4_0 / Q8_0 rows of more than 32 block pairs runs on the single-row kernel's walk with two sets of activations in registers:
+  rows that one wave covers (K <= 4096) and K split over four waves, ragged row counts, more row groups than teams.  Exact weights, so the bar is
+  the float64 anchor of the exact dequantized weights (first rows) and the C restatement (all rows); fp32 activations and fp16 outputs as well."""
+  rng = np.random.default_rng(2 * n + k + t)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, 2, k, np.float16)
+  y = _run(gpu, t, w, x, n, k)
+  assert ol.rel_err(y, cref.linear(t, w, x, n, k, threads=8)) <= TOL
+  rows = min(n, 64)
+  nel, nby = GGML_QUANT[t]
+  W = ol.weight_f32(w[:rows * (k // nel) * nby], rows, k, t)
+  assert ol.rel_err(y[:, :rows], ol.linear_f64(x.astype(np.float32), W)) <= TOL
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
+  assert _run(gpu, t, w, x, n, k, ydt=np.float16).tobytes() == y.astype(np.float16).tobytes()
+
+def test_two_rows_segments_and_residual(gpu):
+  """q / k / v in one launch at M = 2 (K = 4096: the two-row walk over three matrices, teams crossing from one matrix into the next) and the
+  residual epilogue in place."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(2424)
+  k, m = 4096, 2
+  ns = [1000, 136, 130]
+  for t in (2, 8):
+    ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+    x = synth.activations(rng, m, k, np.float16)
+    layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+    outs = [gpu.Buffer((m, n), np.float32) for n in ns]
+    for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    xb = gpu.Buffer.from_numpy(x)
+    qlinear_multi(layers, xb, outs)
+    refs = [ol.linear_f64(x.astype(np.float32), ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]
+    for o, r in zip(outs, refs): assert ol.rel_err(o.numpy(), r) <= TOL
+    res = [rng.standard_normal((m, n)).astype(np.float32) for n in ns]
+    rb = [gpu.Buffer.from_numpy(r) for r in res]
+    qlinear_multi(layers, xb, rb, epilogue=1, resid=rb)
+    for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL
+
 def test_small_batch_through_lds_segments_and_residual(gpu):
   """q / k / v of a llama block shape in one launch at M = 4 and the residual epilogue in place, on the LDS-fed kernel's range."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

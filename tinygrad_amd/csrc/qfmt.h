@@ -743,6 +743,31 @@ __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, co
   acc += F::finish(raw, wv, g, cv);
 }
 
+// the same for MR activation rows: one decode, MR sets of dot products
+template <int T, int MR>
+__device__ __forceinline__ void unit_dot_reg_m(const typename Fmt<T>::Raw& raw, const u32x4 (*xv)[Fmt<T>::XV], const float (*cv)[Fmt<T>::NG], float* acc, const uint32_t* kc) {
+  using F = Fmt<T>;
+  uint32_t wv[F::NWV];
+  F::decode(raw, wv, kc);
+  constexpr int VPG = F::XV / F::NG;
+#pragma unroll
+  for (int m = 0; m < MR; m++) {
+    float g[F::NG];
+#pragma unroll
+    for (int j = 0; j < F::NG; j++) {
+      float t = cv[m][j];
+#pragma unroll
+      for (int v = 0; v < VPG; v++) {
+        const u32x4 x = xv[m][j * VPG + v];
+        const int wi = 4 * (j * VPG + v);
+        t = dot2(wv[wi + 0], x.x, t); t = dot2(wv[wi + 1], x.y, t); t = dot2(wv[wi + 2], x.z, t); t = dot2(wv[wi + 3], x.w, t);
+      }
+      g[j] = t;
+    }
+    acc[m] += F::finish(raw, wv, g, cv[m]);
+  }
+}
+
 // M = 1 stores.  EPI 0: plain, EPI 1: + residual, EPI 2: silu(gate) * up into output row `row` of segment 0.
 template <int EPI>
 __device__ __forceinline__ void store_one(const QArgs& a, int seg, long long row, float v, long long yofs = 0) {

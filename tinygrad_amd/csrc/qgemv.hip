@@ -317,6 +317,7 @@ static int launch_qgemv_m(const QArgs& a, int M, hipStream_t s) {
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    // qgemm_dma.hip
+int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -403,6 +404,10 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
   if (M == 1) {
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
+  }
+  if (M == 2 && pair && !comb && !norm_w) {                       // two rows on the single-row kernel's walk (Q4_0 / Q8_0 pairs)
+    const int fmt = ggml_type == GGML_Q4_0 ? F_Q4_0P : ggml_type == GGML_Q8_0 ? F_Q8_0P : -1;
+    if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
   }
   if (M >= 3) {                                                   // matrix-core small-batch kernels: weights through LDS where that kernel applies, else through registers
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;

@@ -46,8 +46,12 @@
 //          router logits itself (64..1024 floats), so no selection has to cross workgroups inside the router's launch
 //   PRO 5  PRO 1 for a row of at most one piece per thread that is first completed as x + sum_j p_j y_j (the MoE weighted sum and block
 //          residual that precede the next block's attn_norm): the launch that would only add vectors disappears
-template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
+//
+// MR > 1 (several activation rows; instantiated for two; generic prologue, no fused SwiGLU): the same walk over the weights with MR sets of activations in registers;
+// a unit is decoded once and multiplied with every row.  Outputs and residuals are (MR, rows) per matrix.
+template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
 __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) {
+  static_assert(MR == 1 || (PRO == 0 && EPI != 2), "several activation rows: generic prologue, plain or residual epilogue");
   // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
   // issued together (read at their points of use they arrive in dependent stages, each a scalar-cache miss of its own).
   const QArgs a = args;
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   constexpr int D = (WK == 1 && !H && EPI != 0) ? 2 : QG1_DEPTH;
   constexpr int NPC = (NT >= 512) ? 1 : 2;                        // 8-element activation pieces per thread in prologues 1 and 3 (rows of at most 8 NT NPC values)
   extern __shared__ uint32_t xlds[];                             // nu * USTRIDE dwords
-  __shared__ float part[2][WK][R];
+  __shared__ float part[2][WK][R * MR];
   __shared__ float nred[NT / 64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -90,19 +94,20 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   const long long rstep = (!H && a.team_stride) ? (long long)a.team_stride * RS : RS;     // rows from one row group of the team to its next
   uint32_t kc[F::NKC];
   F::consts(kc);
-  u32x4 xv[F::XV]; float cv[F::NG];
+  u32x4 xv[MR][F::XV]; float cv[MR][F::NG];
   const int nseg = (EPI == 2) ? 1 : a.nseg;
   int parity = 0;
 
   // ---- the segment (weight matrix) the team is in
   int seg = 0;
-  long long seg_start = 0, lo = 0, hi = 0, cnt = 0, last = 0;
+  long long seg_start = 0, lo = 0, hi = 0, cnt = 0, last = 0, seg_n = 0;
   const uint8_t *base0 = nullptr, *base1 = nullptr;
   const float* resid = nullptr;
   auto enter = [&](int sg) {
     seg = sg;
     if (sg == 0) seg_start = 0;
     const long long seg_rows = a.n[sg];
+    seg_n = seg_rows;
     lo = row_lo - seg_start; hi = row_hi - seg_start;
     if (lo < 0) lo = 0;
     if (hi > seg_rows) hi = seg_rows;
@@ -117,7 +122,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     base1 = ((EPI == 2) ? a.w[1] : a.w[sg]) + eoff;
     if constexpr (EPI == 1) resid = a.resid[sg] + yofs;
   };
-  struct Grp { Raw w[R]; float res[R]; };
+  struct Grp { Raw w[R]; float res[R * MR]; };
   auto issue = [&](Grp& g, long long row) {
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -127,31 +132,43 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
       if constexpr (T == GGML_F16) g.w[r] = F::load_nu(rp, uc, a.nu); else g.w[r] = F::load(rp, uc);
     }
     if constexpr (EPI == 1) {
-      if constexpr (WK > 1) { long long rr = row + (lane < R ? lane : 0); rr = rr < last ? rr : last; g.res[0] = resid[rr]; }   // wave 0, lane r stores row + r
-      else {
+      if constexpr (WK > 1) {                                      // wave 0, lane m R + r stores row + r of activation row m
+        const int lm = lane < R * MR ? lane / R : 0, lr = lane < R * MR ? lane % R : 0;
+        long long rr = row + lr; rr = rr < last ? rr : last; g.res[0] = resid[lm * seg_n + rr];
+      } else {
 #pragma unroll
-        for (int r = 0; r < R; r++) { long long rr = row + r; rr = rr < last ? rr : last; g.res[r] = resid[rr]; }
+        for (int m = 0; m < MR; m++) {
+#pragma unroll
+          for (int r = 0; r < R; r++) { long long rr = row + r; rr = rr < last ? rr : last; g.res[m * R + r] = resid[m * seg_n + rr]; }
+        }
       }
     }
   };
   // multiply, reduce and store one row group
   auto finish_group = [&](const Grp& g, long long row) {
-    float acc[R];
+    float acc[MR][R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-      acc[r] = 0.f;
-      unit_dot_reg<T>(g.w[r], xv, cv, acc[r], kc);
-      acc[r] = H ? half_sum_lane31(uvalid ? acc[r] : 0.f) : wave_sum_lane63(uvalid ? acc[r] : 0.f);
+      float am[MR];
+#pragma unroll
+      for (int m = 0; m < MR; m++) am[m] = 0.f;
+      if constexpr (MR == 1) unit_dot_reg<T>(g.w[r], xv[0], cv[0], am[0], kc);
+      else unit_dot_reg_m<T, MR>(g.w[r], xv, cv, am, kc);
+#pragma unroll
+      for (int m = 0; m < MR; m++) acc[m][r] = H ? half_sum_lane31(uvalid ? am[m] : 0.f) : wave_sum_lane63(uvalid ? am[m] : 0.f);
     }
     if constexpr (WK > 1) {
       if (lane == 63) {
 #pragma unroll
-        for (int r = 0; r < R; r++) part[parity][wave][r] = acc[r];
+        for (int m = 0; m < MR; m++) {
+#pragma unroll
+          for (int r = 0; r < R; r++) part[parity][wave][m * R + r] = acc[m][r];
+        }
       }
       __syncthreads();
       if (wave == 0) {
         float t = 0.f;
-        if (lane < R) {
+        if (lane < R * MR) {
 #pragma unroll
           for (int j = 0; j < WK; j++) t += part[parity][j][lane];
         }
@@ -160,16 +177,20 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
           if (lane == 0) store_swiglu(a, row, t, up, yofs);
         } else {
           if constexpr (EPI == 1) t += g.res[0];
-          if (lane < R && row + lane < hi) store_one<0>(a, seg, row + lane, t, yofs);
+          const int lm = lane / R, lr = lane % R;
+          if (lane < R * MR && row + lr < hi) store_one<0>(a, seg, row + lr, t, yofs + lm * seg_n);
         }
       }
       parity ^= 1;
     } else {
       if (hl == (H ? 31 : 63)) {
-        if constexpr (EPI == 2) store_swiglu(a, row, acc[0], acc[R - 1], yofs);
+        if constexpr (EPI == 2) store_swiglu(a, row, acc[0][0], acc[0][R - 1], yofs);
         else {
 #pragma unroll
-          for (int r = 0; r < R; r++) if (row + r < hi) store_one<0>(a, seg, row + r, EPI == 1 ? acc[r] + g.res[r] : acc[r], yofs);
+          for (int m = 0; m < MR; m++) {
+#pragma unroll
+            for (int r = 0; r < R; r++) if (row + r < hi) store_one<0>(a, seg, row + r, EPI == 1 ? acc[m][r] + g.res[m * R + r] : acc[m][r], yofs + m * seg_n);
+          }
         }
       }
     }
@@ -202,15 +223,18 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   const u32x4* xh = (const u32x4*)((const uint16_t*)a.x + xrow * a.K);
   auto lds_to_regs = [&]() {
     __syncthreads();
-    uint32_t nx[NP];
 #pragma unroll
-    for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + uc * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
-    F::stage(nx, xv, cv);
+    for (int m = 0; m < MR; m++) {
+      uint32_t nx[NP];
+#pragma unroll
+      for (int k = 0; k < NP; k += 4) { const u32x4 v = *(const u32x4*)(xlds + (m * a.nu + uc) * USTRIDE + k); nx[k] = v.x; nx[k + 1] = v.y; nx[k + 2] = v.z; nx[k + 3] = v.w; }
+      F::stage(nx, xv[m], cv[m]);
+    }
   };
   // piece i (elements 8i .. 8i+7 as 4 fp16 pairs) into LDS: unit F::unit_of(8i) at pair F::pair_of(8i) (4 consecutive pairs stay inside one unit run)
-  auto put_piece = [&](int i, const u32x4& v) {
-    if constexpr (T == GGML_F16) *(u32x4*)(xlds + F::unit_of_nu(8 * i, a.nu) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v;
-    else *(u32x4*)(xlds + F::unit_of(8 * i) * USTRIDE + F::pair_of(8 * i)) = v;
+  auto put_piece = [&](int i, const u32x4& v, int m = 0) {
+    if constexpr (T == GGML_F16) *(u32x4*)(xlds + (m * a.nu + F::unit_of_nu(8 * i, a.nu)) * USTRIDE + F::pair_of_nu(8 * i, a.nu)) = v;
+    else *(u32x4*)(xlds + (m * a.nu + F::unit_of(8 * i)) * USTRIDE + F::pair_of(8 * i)) = v;
   };
   auto pack8 = [](const f32x4& l, const f32x4& h) {
     u32x4 v;
@@ -221,9 +245,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   if constexpr (PRO == 2) {
     const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
 #pragma unroll
-    for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
+    for (int t = 0; t < F::XV; t++) xv[0][t] = xs[t * a.nu + uc];
     issue(b[0], lo);
-    F::cfromx(xv, cv);
+    F::cfromx(xv[0], cv[0]);
   } else if constexpr (PRO == 5) {
     constexpr int CK = 8;                                        // rows of the weighted sum (fewer: the surplus ones reload row 0 with weight 0)
     const int i = (int)threadIdx.x < nq ? (int)threadIdx.x : nq - 1;
@@ -321,9 +345,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     if (a.x_staged) {
       const u32x4* xs = (const u32x4*)a.x + xrow * (long long)F::XV * a.nu;
 #pragma unroll
-      for (int t = 0; t < F::XV; t++) xv[t] = xs[t * a.nu + uc];
+      for (int t = 0; t < F::XV; t++) xv[0][t] = xs[t * a.nu + uc];
       issue(b[0], lo);
-      F::cfromx(xv, cv);
+      F::cfromx(xv[0], cv[0]);
     } else {
       issue(b[0], lo);
       // Loads of up to four (two) loop iterations are issued as one batch: a load per iteration would cost a memory round trip each.
@@ -345,15 +369,18 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
         for (int j = 0; j < NT / 64; j++) tot += nred[j];
         nscale = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
       }
+      for (int m = 0; m < MR; m++) {
+      const f32x4* xr_m = xr + (size_t)m * (a.K / 4);
+      const u32x4* xh_m = xh + (size_t)m * (a.K / 8);
       for (int p = threadIdx.x; p < nq; p += NT * 2) {
         u32x4 v[2]; f32x4 lo4[2], hi4[2], w0[2], w1[2];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
           const int i = p + NT * t < nq ? p + NT * t : nq - 1;
           if (a.x_f32) {
-            lo4[t] = xr[2 * i]; hi4[t] = xr[2 * i + 1];
+            lo4[t] = xr_m[2 * i]; hi4[t] = xr_m[2 * i + 1];
             if (a.norm_w) { w0[t] = ((const f32x4*)a.norm_w)[2 * i]; w1[t] = ((const f32x4*)a.norm_w)[2 * i + 1]; }
-          } else v[t] = xh[i];
+          } else v[t] = xh_m[i];
         }
 #pragma unroll
         for (int t = 0; t < 2; t++) {
@@ -367,8 +394,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
             }
             v[t] = pack8(l, h);
           }
-          put_piece(i, v[t]);
+          put_piece(i, v[t], m);
         }
+      }
       }
       lds_to_regs();
     }
@@ -385,9 +413,9 @@ static int fast_cu_count() {
   return n;
 }
 
-template <int T, int R, int WK, int WR, int EPI, bool H, int PRO>
+template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
 static int launch_fast_p(const QArgs& a, long long grid, size_t lds, hipStream_t s) {
-  auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H, PRO>;
+  auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H, PRO, MR>;
   if (lds > 48 * 1024) {
     // once per instantiation; the initialisation of a function-local static is serialised by the language, so concurrent first calls are safe
     static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
@@ -398,13 +426,13 @@ static int launch_fast_p(const QArgs& a, long long grid, size_t lds, hipStream_t
   return 0;
 }
 
-template <int T, int R, int WK, int WR, int EPI, bool H = false>
+template <int T, int R, int WK, int WR, int EPI, bool H = false, int MR = 1>
 static int launch_fast(QArgs a, hipStream_t s) {
   using F = Fmt<T>;
   constexpr int RS = (EPI == 2) ? 1 : R;
   constexpr int NT = WK * WR * 64;
   const long long ngroups = (a.ntot + RS - 1) / RS;
-  const size_t lds = (size_t)a.nu * (F::UW / 2 + 4) * 4;
+  const size_t lds = (size_t)MR * a.nu * (F::UW / 2 + 4) * 4;
   // row teams per CU: 8 waves (one 8-wave workgroup or two 4-wave ones), fewer when the staged activations in LDS (160 KB per CU) say so.
   // Measured on the 8B decode step: 8 or 12 waves per CU 570 tok/s, 16 (all wave slots) 564, 4 553.
   int wg_per_cu = (a.sel ? 16 : 8) / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;   // (expert jobs share the grid: all 16 wave slots there)
@@ -428,6 +456,8 @@ static int launch_fast(QArgs a, hipStream_t s) {
     a.team_stride = (!H && !a.team_skew && !a.sel && (EPI == 2 || a.nseg == 1)) ? (int)nteams : 0; }
   // prologue kind (the specialised ones exist for the shapes the decode step uses; everything else takes the generic prologue)
   const bool one_batch = a.K / 8 <= NT * (NT >= 512 ? 1 : 2);
+  if constexpr (MR > 1) return launch_fast_p<T, R, WK, WR, EPI, H, 0, MR>(a, grid, lds, s);
+  else {
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
   if constexpr (WK == 1 && EPI == 0) {
     if (a.comb_y) {
@@ -448,6 +478,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
     if (!a.x_staged && one_batch && !a.norm_w && !a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 3>(a, grid, lds, s);
   }
   return launch_fast_p<T, R, WK, WR, EPI, H, 0>(a, grid, lds, s);
+  }
 }
 
 #ifndef QG1_R2_ROWS
@@ -479,4 +510,24 @@ int qgemv1_launch_format(QArgs a, hipStream_t s) {
   if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);
   if (waves <= 8) return launch_fast_e<T, 8, 1>(a, s);
   return launch_fast_e<T, 16, 1>(a, s);
+}
+
+// Two activation rows on the same kernel (one weight row per step, generic prologue): plain or residual epilogue, rows that one wave covers
+// or K split over four waves.  Returns -1 outside that range.
+template <int T, int MR>
+static int qgemv1_launch_multi_m(const QArgs& a, int waves, hipStream_t s) {
+  if (waves <= 1) return a.epilogue == 1 ? launch_fast<T, 1, 1, QG1_WR, 1, false, MR>(a, s) : launch_fast<T, 1, 1, QG1_WR, 0, false, MR>(a, s);
+  return a.epilogue == 1 ? launch_fast<T, 1, 4, 1, 1, false, MR>(a, s) : launch_fast<T, 1, 4, 1, 0, false, MR>(a, s);
+}
+template <int T>
+int qgemv1_launch_multi(QArgs a, int M, hipStream_t s) {
+  using F = Fmt<T>;
+  a.nu = a.K / F::UW;
+  a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+  const int waves = (a.nu + 63) / 64;
+  if (a.nu <= 32 || waves > 4 || a.epilogue > 1 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y || a.route_logits) return -1;
+  // two rows only: every further row adds 3 us on a 14336 x 4096 matrix (the dot2 chains and lane reductions of a wave do not overlap
+  // enough with two waves per SIMD; Q4_0: 9.8 / 13.0 / 15.7 / 18.7 us at M = 1..4), so from three rows on the matrix-core kernels win
+  if (M == 2) return qgemv1_launch_multi_m<T, 2>(a, waves, s);
+  return -1;
 }
