@@ -405,8 +405,8 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
   }
-  if (M == 2 && pair && !comb && !norm_w) {                       // two rows on the single-row kernel's walk (Q4_0 / Q8_0 pairs)
-    const int fmt = ggml_type == GGML_Q4_0 ? F_Q4_0P : ggml_type == GGML_Q8_0 ? F_Q8_0P : -1;
+  if (M == 2 && !comb && !norm_w) {                               // two rows on the single-row kernel's walk (Q4_0 / Q8_0 pairs, Q6_K)
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
     if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
   }
   if (M >= 3) {                                                   // matrix-core small-batch kernels: weights through LDS where that kernel applies, else through registers

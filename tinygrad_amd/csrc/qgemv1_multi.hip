@@ -1,4 +1,4 @@
-// The M = 1 dequant-GEMV kernel with two activation rows (qgemv1.h, MR = 2) for the Q4_0 / Q8_0 block pairs: the load pattern of the
+// The M = 1 dequant-GEMV kernel with two activation rows (qgemv1.h, MR = 2) for the Q4_0 / Q8_0 block pairs and Q6_K: the load pattern of the
 // single-row kernel (one weight row per wave instruction group, lane = unit) streams better than the matrix-core kernels' sixteen-row
 // pattern, and a second row of dot2 work per decoded unit still fits under the stream (Q8_0 14336 x 4096: 17.2 us against 19.1 us on the
 // LDS-staged dot2 kernel; Q4_0: 13.0 us).
@@ -6,6 +6,7 @@
 
 template int qgemv1_launch_multi<F_Q4_0P>(QArgs, int, hipStream_t);
 template int qgemv1_launch_multi<F_Q8_0P>(QArgs, int, hipStream_t);
+template int qgemv1_launch_multi<GGML_Q6_K>(QArgs, int, hipStream_t);
 
 // Returns -1 when the call is outside this path's range (the caller falls back to the matrix-core or the LDS-staged kernel).
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
@@ -13,6 +14,7 @@ int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   switch (fmt) {
     case F_Q4_0P: return qgemv1_launch_multi<F_Q4_0P>(a, M, s);
     case F_Q8_0P: return qgemv1_launch_multi<F_Q8_0P>(a, M, s);
+    case GGML_Q6_K: return qgemv1_launch_multi<GGML_Q6_K>(a, M, s);
   }
   return -1;
 }
