@@ -207,6 +207,16 @@ int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, flo
 int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                  int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                  int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+/* Attention for `rows` consecutive positions state.pos .. state.pos + rows - 1 of ONE sequence (the chunked prefill of Transformer.generate,
+ * tinygrad/llm/model.py:464, 476-481; causal mask `_attention`, model.py:227-229): q (rows, n_heads * head_dim), k / v (rows, n_kv_heads * head_dim),
+ * one cache (n_kv_heads, max_ctx, head_dim) fp16.  A first launch rotates and appends every row's key / value, a second attends from the cache (row r sees the
+ * positions up to its own), a third merges the splits.  partials: rows times the single-sequence workspace.  Outputs (rows, n_heads * head_dim). */
+int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+/* After a chunk of `rows` prompt positions: state.pos += rows and tokens[r] = prompt[state.pos + r] (entries past max_ctx - 1 read the last one): the
+ * input ids of the next chunk (model.py:477-480 slices the prompt on the host; here the captured step advances itself). */
+int tga_chunk_advance(void* state, const int32_t* prompt, int rows, int32_t* tokens, int max_ctx, void* stream);
 /* tga_argmax_step / tga_advance_prompt for a batch: while state.pos + 1 < state.n_prompt the next token of sequence b is prompts[b * prompt_stride +
  * pos + 1]; otherwise (logits != NULL) the first index of the maximum of logits row b (model.py:364 at temperature 0) goes to tokens[b] and
  * out_tokens[state.step * batch + b].  Then pos += 1 (and step += 1 when tokens were sampled).  logits NULL: a prompt step without lm-head. */

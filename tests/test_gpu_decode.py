@@ -80,6 +80,7 @@ def test_kv_prefix_reuse_equals_fresh_model(gpu):
   reply + new tokens) runs only the new tokens."""
   model, _ = _build(gpu, SMALL, 128, seed=11)
   fresh, _ = _build(gpu, SMALL, 128, seed=11)
+  model.prefill_chunk = fresh.prefill_chunk = 1                                          # token by token on both sides: the comparison below is bit for bit
   rng = np.random.default_rng(11)
   p1 = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=70)]
   p2 = p1[:40] + [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=12)]
@@ -97,12 +98,77 @@ def test_kv_prefix_reuse_equals_fresh_model(gpu):
   got3 = list(model.generate(p3, 8)); lg3 = model.logits().copy()
   assert model.prefill_steps == 3
   fresh2, _ = _build(gpu, SMALL, 128, seed=11)
+  fresh2.prefill_chunk = 1
   assert got3 == list(fresh2.generate(p3, 8))
   np.testing.assert_array_equal(lg3, fresh2.logits())
   assert model.get_start_pos(p3) == len(p3) - 1                                          # the same prompt again: nothing to prefill
   assert list(model.generate(p3, 8)) == got3 and model.prefill_steps == 0
   model.prefill(p3, reuse_cache=False)
   assert model.prefill_steps == len(p3) - 1
+
+@pytest.mark.parametrize("n_prompt", [9, 16, 61, 70, 131])
+def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt):
+  """Prompt positions computed eight at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
+  tinygrad/llm/model.py:464, 476-481) against the same model prefilled token by token and against the oracle: the KV caches agree to fp16 rounding of
+  slightly different float32 results, the logits of the following decode steps stay within 1e-3 of the oracle's for the same token history, and the
+  greedy tokens are the oracle's.  Prompt lengths that leave 0..7 positions for the token-by-token tail and cross the 64-position splits."""
+  model, host = _build(gpu, SMALL, 192, seed=21)
+  single, _ = _build(gpu, SMALL, 192, seed=21)
+  single.prefill_chunk = 1
+  rng = np.random.default_rng(21 + n_prompt)
+  prompt = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=n_prompt)]
+  model.prefill(prompt); single.prefill(prompt)
+  assert model.prefill_steps == single.prefill_steps == n_prompt - 1
+  assert model._chunker is not None and single._chunker is None
+  for bm, bs in zip(model.blk, single.blk):
+    for cm, cs in ((bm.cache_k, bs.cache_k), (bm.cache_v, bs.cache_v)):
+      a, b = cm.numpy().astype(np.float32)[:, :n_prompt - 1], cs.numpy().astype(np.float32)[:, :n_prompt - 1]
+      assert ol.rel_err(a, b) <= 2e-3
+      assert not cm.numpy()[:, n_prompt - 1:].any()                                    # nothing beyond the prompt was written
+  oref = ollm.Model(SMALL, host, 192, act_round_f16=False)
+  got, ref, worst, margin, rms = greedy_vs_reference_numerics(model, oref, prompt, 12)
+  print(f"prompt {n_prompt}: min top-2 margin {margin:.4f}, worst logits rel-err {worst:.2e}")
+  assert got == ref and worst <= 1e-3
+
+def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
+  """tga_attention_prefill_chunk alone: eight consecutive positions per call over one cache (per-head q/k norm, GQA), each row against numpy attention over
+  the positions up to its own; tga_chunk_advance moves the position and loads the next ids."""
+  from tinygrad_amd.llm import precompute_freqs_cis
+  H, KV, hd, ctx, B = 8, 2, 128, 256, 8
+  rng = np.random.default_rng(88)
+  rope = precompute_freqs_cis(hd, ctx, 10000.0)
+  ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
+  part = gpu.Buffer((B * H * ((ctx + 63) // 64) * (hd + 2),), np.float32).zero_()
+  ropeb = gpu.Buffer.from_numpy(rope)
+  out = gpu.Buffer((B, H * hd), np.float32)
+  qw, kw = rng.standard_normal(hd).astype(np.float32), rng.standard_normal(hd).astype(np.float32)
+  qwb, kwb = gpu.Buffer.from_numpy(qw), gpu.Buffer.from_numpy(kw)
+  prompt = np.arange(ctx, dtype=np.int32) * 3 % 101
+  pb, tokb = gpu.Buffer.from_numpy(prompt), gpu.Buffer((B,), np.int32).zero_()
+  st = np.zeros(16, np.int32); st[0] = 0
+  stb = gpu.Buffer.from_numpy(st)
+  rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)
+  for chunk in range(18):                                                              # positions 0 .. 143: across two split boundaries
+    pos0 = chunk * B
+    q, k, v = (rng.standard_normal((B, n)).astype(np.float32) * 1.5 for n in (H * hd, KV * hd, KV * hd))
+    qb, kb, vb = (gpu.Buffer.from_numpy(t) for t in (q, k, v))
+    gpu.check(gpu.lib().tga_attention_prefill_chunk(B, qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, 1e-5, 1, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr,
+                                                    None, out.ptr, None))
+    gpu.check(gpu.lib().tga_chunk_advance(stb.ptr, pb.ptr, B, tokb.ptr, ctx, None))
+    gpu.synchronize()
+    o = out.numpy()
+    for r in range(B):
+      pos = pos0 + r
+      qn, kn = ollm.rmsnorm(q[r].reshape(H, hd), qw, 1e-5), ollm.rmsnorm(k[r].reshape(KV, hd), kw, 1e-5)
+      qr, kr = ollm.apply_rope(qn, rope[pos]), ollm.apply_rope(kn, rope[pos])
+      rk[:, pos], rv[:, pos] = kr.astype(np.float16), v[r].reshape(KV, hd).astype(np.float16)
+      K = np.repeat(rk[:, :pos + 1].astype(np.float32), H // KV, axis=0); V = np.repeat(rv[:, :pos + 1].astype(np.float32), H // KV, axis=0)
+      sc = np.einsum("hd,htd->ht", qr, K) / np.sqrt(hd)
+      e = np.exp(sc - sc.max(-1, keepdims=True)); p = e / e.sum(-1, keepdims=True)
+      assert ol.rel_err(o[r], np.einsum("ht,htd->hd", p, V).reshape(-1)) <= 1e-4, pos
+    assert int(stb.numpy()[0]) == pos0 + B
+    np.testing.assert_array_equal(tokb.numpy(), prompt[np.minimum(pos0 + B + np.arange(B), ctx - 1)])
+  assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
 
 def test_command_list_takes_kernel_launches_only(gpu):
   """A capture that holds anything but kernel launches (here a memset) is refused when the list is built; the stream stays usable."""

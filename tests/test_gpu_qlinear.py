@@ -201,6 +201,26 @@ def test_two_rows_segments_and_residual(gpu):
     qlinear_multi(layers, xb, rb, epilogue=1, resid=rb)
     for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL
 
+@pytest.mark.parametrize("t", [2, 8], ids=["q4_0", "q8_0"])
+@pytest.mark.parametrize("n,k,m", [(8, 1024, 3), (264, 2048, 8), (2056, 3072, 5), (14336, 4096, 8), (4096, 4096, 4)])
+def test_small_batch_swiglu_through_lds(gpu, t, n, k, m):
+  """silu(gate) * up (tinygrad/llm/model.py:137) at 3..8 activation rows on the LDS-fed matrix-core kernel: a row group is eight gate rows and the same
+  eight up rows.  Against the float64 product of the exact dequantized weights; fp16 and float32 outputs."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(n + k + m + 7 * t)
+  wg, wu = synth.random_blocks(rng, t, n, k), synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  layers = [QuantLinear(gpu.Buffer.from_numpy(wg), t, n, k), QuantLinear(gpu.Buffer.from_numpy(wu), t, n, k)]
+  xb = gpu.Buffer.from_numpy(x)
+  a = ol.linear_f64(x.astype(np.float32), ol.weight_f32(wg, n, k, t)); b = ol.linear_f64(x.astype(np.float32), ol.weight_f32(wu, n, k, t))
+  ref = a / (1 + np.exp(-a)) * b
+  for ydt in (np.float32, np.float16):
+    out = gpu.Buffer((m, n), ydt)
+    gpu.check(gpu.lib().tga_memset(out.ptr, 0xFF, out.nbytes, None))
+    qlinear_multi(layers, xb, [out], epilogue=2)
+    y = out.numpy().astype(np.float32)
+    assert ol.rel_err(y, ref) <= (TOL if ydt == np.float32 else 2 * TOL), ydt
+
 def test_small_batch_through_lds_segments_and_residual(gpu):
   """q / k / v of a llama block shape in one launch at M = 4 and the residual epilogue in place, on the LDS-fed kernel's range."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

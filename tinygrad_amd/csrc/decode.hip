@@ -109,6 +109,10 @@ struct AttnArgs {
   // batched decode (sequences in lockstep at one position): sequence z = blockIdx.z (split launch) / blockIdx.y (merge launch) uses the
   // operands shifted by z times these element strides; all zero for a single sequence
   long long q_bs, kv_bs, cache_bs, part_bs, out_bs;
+  // chunked prefill (rows z = 0, 1, ... are consecutive positions of ONE sequence: cache_bs = 0, row z sits at position st->pos + z pos_step):
+  // chunk 1 = the launch that only rotates and appends every row's key / value, chunk 2 = the launch that attends from the cache alone
+  // (the rows of the chunk were appended by the launch before; a row sees the positions up to its own).  0: decode.
+  int chunk, pos_step;
 };
 __device__ __forceinline__ AttnArgs attn_args_of_sequence(AttnArgs a, int z) {
   a.q += z * a.q_bs; a.k += z * a.kv_bs; a.v += z * a.kv_bs; a.cache_k += z * a.cache_bs; a.cache_v += z * a.cache_bs; a.part += z * a.part_bs;
@@ -168,6 +172,7 @@ __device__ __forceinline__ void block_sumsq2(const float* q, int nq, const float
 template <int HD8, int NORM>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
   const AttnArgs a = attn_args_of_sequence(args, blockIdx.z);   // field reads become kernel-argument loads in the entry block
+  const int zrow = blockIdx.z * a.pos_step;
   constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = 4 * RPI, CSTR = HD + 4;
   constexpr int QPL = (HD / 2 + 63) / 64;               // query pairs per lane
   const int kvh = blockIdx.x, split = blockIdx.y;
@@ -222,7 +227,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
     }
   }
   // ---- the position, and the one load that needs it
-  const int pos = a.st->pos;
+  const int pos = a.st->pos + zrow;
   if (pos >= a.max_ctx || pos < 0) {                    // no cache row and no rotation row for this position: nothing is read or written, the host sees the flag
     if (kvh == 0 && split == 0 && tid == 0) atomicOr(&a.st->error, 2);
     return;
@@ -283,13 +288,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
     }
   }
   __syncthreads();
-  if ((pos >> 6) == split) {                            // owner split appends this token to the cache
+  if (a.chunk == 1 || (a.chunk == 0 && (pos >> 6) == split)) {   // owner split appends this token to the cache (chunked prefill: the append launch, one workgroup per row and kv head)
     for (int i = tid; i < HD; i += 256) {
       a.cache_k[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)ks[i];
       a.cache_v[((size_t)kvh * a.max_ctx + pos) * HD + i] = (_Float16)vs[i];
     }
   }
-  {
+  if (a.chunk == 1) return;
+  if (a.chunk == 0) {                                   // (chunked prefill reads this row's key / value, like those of the rows before it, from the cache)
     const u32x4 kcur = pack8_f16(ks + vp * 8), vcur = pack8_f16(vs + vp * 8);   // rounded to fp16 exactly like the cached copy
 #pragma unroll
     for (int i = 0; i < NVI; i++) if (p0 + i * RPI + vr >= pos) { kt[i] = kcur; vt[i] = vcur; }
@@ -392,7 +398,7 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
   float v[FB];
 #pragma unroll
   for (int j = 0; j < FB; j++) v[j] = ph[(size_t)(j < nsp ? j : nsp - 1) * (HD + 2) + d];
-  const int pos = a.st->pos, ns = (pos >> 6) + 1;
+  const int pos = a.st->pos + blockIdx.y * a.pos_step, ns = (pos >> 6) + 1;
   if (pos >= a.max_ctx || pos < 0) return;              // refused by the split launch (state.error): the output row keeps its contents
   float m = -INFINITY, l = 0.f;
   if (nsp <= HD) {
@@ -531,6 +537,14 @@ __global__ void advance_batch_kernel(DecodeState* st, int had_logits) {
   st->pos = next;
 }
 
+// chunked prefill: the next `rows` prompt tokens become the input rows, the position moves on by `rows` (positions past the prompt table read its last entry)
+__global__ void chunk_advance_kernel(DecodeState* st, const int* __restrict__ prompt, int rows, int* __restrict__ tokens, int max_ctx) {
+  const int np = st->pos + rows;
+  __syncthreads();
+  if ((int)threadIdx.x < rows) { const int i = np + (int)threadIdx.x; tokens[threadIdx.x] = prompt[i < max_ctx ? (i < 0 ? 0 : i) : max_ctx - 1]; }
+  if (threadIdx.x == 0) st->pos = np;
+}
+
 // ---------------------------------------------------------------------------------------------- C-ABI
 extern "C" {
 
@@ -583,7 +597,7 @@ int tga_rmsnorm(const float* x, const float* weight, int dim, float eps, void* o
   return tga_rmsnorm_rows(x, weight, 1, dim, eps, out_f16, out_f32, stage_type, stream);
 }
 
-static int attention_launch(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+static int attention_launch(int chunk, int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                             int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                             int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
   TGA_REQUIRE(batch >= 1 && batch <= 65535, "tga_attention_decode: batch=%d", batch);
@@ -602,18 +616,24 @@ static int attention_launch(int batch, const float* q, const float* k, const flo
   a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps; a.norm_per_head = norm_per_head;
   a.q_bs = (long long)n_heads * head_dim; a.kv_bs = (long long)n_kv_heads * head_dim; a.cache_bs = (long long)n_kv_heads * max_ctx * head_dim;
   a.part_bs = (long long)n_heads * a.nsplit * (head_dim + 2); a.out_bs = (long long)n_heads * head_dim;
+  a.chunk = 0; a.pos_step = 0;
+  if (chunk) { a.cache_bs = 0; a.pos_step = 1; }
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
-  const dim3 grid(n_kv_heads, a.nsplit, batch);
+  dim3 grid(n_kv_heads, a.nsplit, batch);
   hipStream_t s = (hipStream_t)stream;
   const int norm = !q_norm_weight ? 0 : norm_per_head ? 2 : ((long long)n_heads * head_dim <= 4096 && (long long)n_kv_heads * head_dim <= 4096) ? 1 : 3;
 #define TGA_ATTN_LAUNCH(HD8) do { \
     if (norm == 0) attn_decode_kernel<HD8, 0><<<grid, 256, 0, s>>>(a); else if (norm == 1) attn_decode_kernel<HD8, 1><<<grid, 256, 0, s>>>(a); \
     else if (norm == 2) attn_decode_kernel<HD8, 2><<<grid, 256, 0, s>>>(a); else attn_decode_kernel<HD8, 3><<<grid, 256, 0, s>>>(a); } while (0)
-  if (head_dim == 64) TGA_ATTN_LAUNCH(8);
-  else if (head_dim == 128) TGA_ATTN_LAUNCH(16);
-  else TGA_ATTN_LAUNCH(32);
+  for (int pass = chunk ? 1 : 0; pass <= (chunk ? 2 : 0); pass++) {   // chunked prefill: append every row, then attend from the cache
+    a.chunk = pass;
+    grid = dim3(n_kv_heads, pass == 1 ? 1 : a.nsplit, batch);
+    if (head_dim == 64) TGA_ATTN_LAUNCH(8);
+    else if (head_dim == 128) TGA_ATTN_LAUNCH(16);
+    else TGA_ATTN_LAUNCH(32);
+    TGA_LAUNCH_CHECK();
+  }
 #undef TGA_ATTN_LAUNCH
-  TGA_LAUNCH_CHECK();
   const dim3 mgrid(n_heads, batch);
   if (head_dim == 64) attn_merge_kernel<64><<<mgrid, 64, 0, s>>>(a);
   else if (head_dim == 128) attn_merge_kernel<128><<<mgrid, 128, 0, s>>>(a);
@@ -625,15 +645,30 @@ static int attention_launch(int batch, const float* q, const float* k, const flo
 int tga_attention_decode_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
-  return attention_launch(1, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+  return attention_launch(0, 1, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_f16, out_f32, stage_type, stream);
 }
 
 int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                  int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                  int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
-  return attention_launch(batch, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+  return attention_launch(0, batch, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_f16, out_f32, 0, stream);
+}
+
+int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
+  TGA_REQUIRE(rows >= 1 && rows <= 64, "tga_attention_prefill_chunk: rows=%d", rows);
+  return attention_launch(1, rows, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+                          rope_table, out_f16, out_f32, 0, stream);
+}
+
+int tga_chunk_advance(void* state, const int32_t* prompt, int rows, int32_t* tokens, int max_ctx, void* stream) {
+  TGA_REQUIRE(state && prompt && tokens && rows >= 1 && rows <= 64 && max_ctx >= 1, "tga_chunk_advance: null pointer or rows=%d outside 1..64", rows);
+  chunk_advance_kernel<<<1, 64, 0, (hipStream_t)stream>>>((DecodeState*)state, prompt, rows, tokens, max_ctx);
+  TGA_LAUNCH_CHECK();
+  return 0;
 }
 
 int tga_attention_decode(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,

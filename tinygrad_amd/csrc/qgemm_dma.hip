@@ -59,8 +59,11 @@ __device__ __forceinline__ void qd_wait_vm(int n) {
   }
 }
 
-template <int T_, bool MS, int NSS>
+// SW: silu(gate) * up (dense SwiGLU, tinygrad/llm/model.py:137) over the two matrices w[0] / w[1]: a row group is eight rows of the gate matrix followed
+// by the same eight rows of the up matrix, so the partial tiles of both meet in one reduction and the product is formed before the store.
+template <int T_, bool MS, int NSS, bool SW = false>
 __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args, const int M, const int nb) {
+  static_assert(!(MS && SW), "the SwiGLU pair is not combined with the q / k / v walk");
   const QArgs a = args;
   using F = Fmt<T_>;
   using DF = DmaFmt<T_>;
@@ -83,7 +86,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   uint32_t kc[F::NKC];
   F::consts(kc);
   const int cu = a.nu, nslots = cu / QD_SU, spg = (nslots + 1) >> 1;   // stages per row group (NSS >= spg)
-  const long long ngroups = a.ntot / 16;
+  constexpr int GR = SW ? 8 : 16;                        // output rows per row group
+  const long long ngroups = (SW ? a.n[0] : a.ntot) / GR;
   auto seg_of = [&](long long row0, int& sg, long long& local0) {
     sg = 0; local0 = row0;
     if constexpr (MS) { if (local0 >= a.n[0]) { local0 -= a.n[0]; sg = 1; if (a.nseg > 2 && local0 >= a.n[1]) { local0 -= a.n[1]; sg = 2; } } }
@@ -94,6 +98,17 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     int sg; long long l0; seg_of(row0, sg, l0);
     const int t = threadIdx.x, wr = (t >> 4) & 15, c = t & 15;
     const long long nrows = rows_of(sg);
+    if constexpr (SW) {
+      if (t < 256 && wr < 8 && c < M && l0 + wr < nrows) {
+        float gate = 0.f, up = 0.f;
+#pragma unroll
+        for (int w = 0; w < QD_NW; w++) { gate += part[p][w][wr][c]; up += part[p][w][wr + 8][c]; }
+        const float v = silu_f(gate) * up;
+        const long long o = (long long)c * nrows + l0 + wr;
+        if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+      }
+      return;
+    }
     if (t < 256 && c < M && l0 + wr < nrows) {
       float v = 0.f;
 #pragma unroll
@@ -112,27 +127,31 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   // and the positions past the last row repeat a valid piece (they land in the slot's slack).  When K ends inside a stage (an odd number of
   // slots), the second slot repeats the first: nothing reads it.
   long long doff[IMAX], doff_odd[IMAX];
+  bool from_up[IMAX];                                    // (SW) rows 8 .. 15 of the slot come from the up matrix
 #pragma unroll
   for (int i = 0; i < IMAX; i++) {
     const int j = wave + QD_NW * i, sl = j >= NI ? 1 : 0;
     const int sigma = 64 * (j - sl * NI) + lane;
     int rr = sigma / (PR + 1), q = sigma - rr * (PR + 1);
     rr = rr < 16 ? rr : 15; q = q < PR ? q : PR - 1;
-    doff_odd[i] = (long long)rr * a.row_bytes + q * 16;
+    from_up[i] = SW && rr >= 8;
+    doff_odd[i] = (long long)(SW ? (rr & 7) : rr) * a.row_bytes + q * 16;
     doff[i] = doff_odd[i] + sl * (QD_SU * UB);
   }
   long long ij = 0; int ist = 0, islot = 0;              // issue stream: row group index (of this workgroup), stage in the group, ring position
   auto issue_stage = [&]() {
     const long long grp = (long long)blockIdx.x + ij * gridDim.x;
-    int sg; long long l0; seg_of(grp * 16, sg, l0);
-    const uint8_t* base = w_of(sg) + l0 * a.row_bytes + (long long)ist * (2 * QD_SU * UB);
+    int sg; long long l0; seg_of(grp * GR, sg, l0);
+    const long long goff = l0 * a.row_bytes + (long long)ist * (2 * QD_SU * UB);
+    const uint8_t* base = w_of(sg) + goff;
+    const uint8_t* base_up = SW ? a.w[1] + goff : base;
     char* dst = ring + (size_t)islot * (2 * SLOT_BYTES);
     const bool two = 2 * ist + 1 < nslots;
 #pragma unroll
     for (int i = 0; i < IMAX; i++) {
       const int j = wave + QD_NW * i;
       if (j < NI2)                                                     // (the same for the whole wave)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + (two ? doff[i] : doff_odd[i])), (__attribute__((address_space(3))) void*)(dst + j * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)((from_up[i] ? base_up : base) + (two ? doff[i] : doff_odd[i])), (__attribute__((address_space(3))) void*)(dst + j * 1024), 16, 0, 0);
     }
     if (++ist == spg) { ist = 0; ij++; }
     islot = islot + 1 == nb ? 0 : islot + 1;
@@ -189,7 +208,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
 #pragma unroll
         for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
       }
-      pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * 16; pend_par = par;
+      pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * GR; pend_par = par;
       par ^= 1;
       acc0 = v4f32{0.f, 0.f, 0.f, 0.f}; acc1 = v4f32{0.f, 0.f, 0.f, 0.f};
       cst = 0; cj++;
@@ -205,9 +224,9 @@ static int qd_cu_count() {
   return n;
 }
 
-template <int T, bool MS, int NSS>
+template <int T, bool MS, int NSS, bool SW = false>
 static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hipStream_t s) {
-  auto kern = qgemm_dma_kernel<T, MS, NSS>;
+  auto kern = qgemm_dma_kernel<T, MS, NSS, SW>;
   static const hipError_t configured = [&]() {
     hipFuncAttributes fa;
     hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
@@ -215,7 +234,7 @@ static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hi
     return hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(QD_LDS_CU - fa.sharedSizeBytes));
   }();
   TGA_HIP(configured);
-  const long long ngroups = a.ntot / 16;
+  const long long ngroups = SW ? a.n[0] / 8 : a.ntot / 16;
   const long long cap = (long long)qd_cu_count() * per_cu;
   const long long grid = ngroups < cap ? ngroups : cap;
   kern<<<dim3((unsigned)grid), dim3(QD_NW * 64), lds, s>>>(a, M, nb);
@@ -237,6 +256,7 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   if (nb < 2) return -1;
   const size_t lds = (size_t)nb * STAGE_BYTES;
   const bool two = a.K > 2 * F::UW * QD_SU;
+  if (a.epilogue == 2) return two ? launch_qd_k<T, false, 2, true>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1, true>(a, M, nb, per_cu, lds, s);
   if (a.nseg > 1) return two ? launch_qd_k<T, true, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, true, 1>(a, M, nb, per_cu, lds, s);
   return two ? launch_qd_k<T, false, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1>(a, M, nb, per_cu, lds, s);
 }
@@ -245,7 +265,11 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 // 3 <= M <= 8, K = 1024, 2048, 3072 or 4096, every matrix a multiple of 16 rows at a 16-byte aligned address.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P) return -1;
-  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 1 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
+    if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
+    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);
+  }
   for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;
   return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);

@@ -339,6 +339,8 @@ class Transformer:
     self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
     self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
+    self._state_dict, self._chunker = state_dict, None               # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
+    self.prefill_chunk = 8                                           # prompt positions per prefill step (the reference's chunks hold 32, model.py:464); 1: token by token
 
   def check_state(self):
     """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
@@ -472,9 +474,13 @@ class Transformer:
     """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step.  Like the reference's generate
     (model.py:472-473) the positions whose tokens equal what the cache already holds are not recomputed."""
     start = self.get_start_pos(tokens) if reuse_cache else 0
+    self.prefill_steps = len(tokens) - 1 - start                        # (positions the last call actually computed)
+    B = self.prefill_chunk
+    if 2 <= B <= 8 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
+      if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
+      start += self._chunker.prefill_chunks(tokens, start, (len(tokens) - 1 - start) // B, use_graph)
     self.reset(tokens, start)
-    self.prefill_steps = len(tokens) - 1 - start                        # (what the last call actually ran)
-    for _ in range(self.prefill_steps):
+    for _ in range(len(tokens) - 1 - start):
       if use_graph: self._graph(False).launch()
       else: self._step(False)
     self._steps_done = len(tokens) - 1
@@ -522,9 +528,11 @@ class BatchedTransformer:
   Dense linears run as small-batch GEMMs over the GGUF blocks (M = B); in a MoE block the B * k (token, slot) jobs are grouped by expert, so an
   expert selected by several tokens is streamed once (ExpertWeights over a (B, T, k) selection, model.py:21-27, 110-135).  Same state dict and
   config as Transformer; every sequence has its own KV cache; prompts of one batch have equal length."""
-  def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024):
+  def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024, chunk_of: "Transformer | None" = None):
+    """chunk_of: the rows are `batch` consecutive prompt positions of that Transformer's sequence instead of `batch` sequences (chunked prefill,
+    model.py:464, 476-481): its KV caches and rotation table are used, the attention is causal inside the chunk, no token is sampled."""
     if not 1 <= batch <= 8: raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
-    self.config, self.batch, self.max_new = config, batch, max_new
+    self.config, self.batch, self.max_new, self.chunk_of = config, batch, max_new, chunk_of
     c, B = config, batch
     f32, f16 = np.float32, np.float16
     lin = lambda name: QuantLinear(state_dict[name][0], state_dict[name][1], *state_dict[name][2])
@@ -556,8 +564,10 @@ class BatchedTransformer:
       else:
         for nm in ("ffn_gate", "ffn_up", "ffn_down"): b[nm] = lin(p + nm + ".weight")
         if b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
-      b["cache_k"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
-      b["cache_v"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
+      if chunk_of is not None: b["cache_k"], b["cache_v"] = chunk_of.blk[i].cache_k, chunk_of.blk[i].cache_v
+      else:
+        b["cache_k"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
+        b["cache_v"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
       self.blk.append(b)
     k = max(1, c.num_experts_per_tok)
     self.state = Buffer((16,), np.int32).zero_()
@@ -574,9 +584,9 @@ class BatchedTransformer:
       self.router_logits, self.sel, self.probs = Buffer((B, c.num_experts), f32), Buffer((B * k,), np.int32), Buffer((B * k,), f32)
       self.job_table, self.job_flags = Buffer((c.num_experts, 16), np.int32).zero_(), Buffer((1,), np.int32).zero_()
       self.act_e, self.y_e = Buffer((B * k, c.hidden_dim), f16), Buffer((B * k, c.dim), f32)
-    self.logits_buf = Buffer((B, c.vocab_size), f32)
-    self.rope = Buffer.from_numpy(rope_table(c.head_dim, c.rope_dim or c.head_dim, c.max_context, c.rope_theta))
-    self.prompts = Buffer((B, c.max_context), np.int32).zero_()
+    self.logits_buf = Buffer((B, c.vocab_size), f32) if chunk_of is None else None
+    self.rope = Buffer.from_numpy(rope_table(c.head_dim, c.rope_dim or c.head_dim, c.max_context, c.rope_theta)) if chunk_of is None else chunk_of.s.rope
+    self.prompts = Buffer((B if chunk_of is None else 1, c.max_context), np.int32).zero_()
     self.out_tokens = Buffer((max(1, max_new), B), np.int32).zero_()
     self.stream = rt.Stream()
     self._graphs, self._steps_done = {}, 0
@@ -598,9 +608,10 @@ class BatchedTransformer:
         bias = dict(epilogue=1, resid=b["bias"][i:j]) if "bias" in b else {}
         self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
         i = j
-      rt.check(L.tga_attention_decode_batched(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
-                                              c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
-                                              c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn.ptr, None, st))
+      attention = L.tga_attention_prefill_chunk if self.chunk_of is not None else L.tga_attention_decode_batched
+      rt.check(attention(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
+                         c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
+                         c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn.ptr, None, st))
       self._linear([b["attn_output"]], self.attn, [self.x], epilogue=1, resid=[self.x])
       # x = h + feed_forward(ffn_norm(h))                                                   model.py:150
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
@@ -629,6 +640,9 @@ class BatchedTransformer:
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       self.output(self.xn, out=self.logits_buf, stream=st)
+    if self.chunk_of is not None:                                        # the next B prompt tokens, B positions on
+      rt.check(L.tga_chunk_advance(self.state.ptr, self.prompts.ptr, B, self.tokens.ptr, c.max_context, st))
+      return
     rt.check(L.tga_argmax_rows_step(self.logits_buf.ptr if with_head else None, B, c.vocab_size, self.state.ptr, self.prompts.ptr, c.max_context, self.tokens.ptr,
                                     self.out_tokens.ptr, self.max_new, st))
 
@@ -638,6 +652,27 @@ class BatchedTransformer:
       with g: self._step(with_head)
       self._graphs[with_head] = g
     return self._graphs[with_head]
+
+  def prefill_chunks(self, tokens: list[int], start: int, n_chunks: int, use_graph: bool = True) -> int:
+    """Chunked prefill for `chunk_of`: computes the positions start .. start + n_chunks * batch - 1 of the prompt, `batch` at a time, into its KV caches.
+    Returns the number of positions done."""
+    c, B = self.config, self.batch
+    if self.chunk_of is None: raise RuntimeError("prefill_chunks needs a model built with chunk_of")
+    if n_chunks <= 0: return 0
+    if not (0 <= start and start + n_chunks * B <= len(tokens) < c.max_context): raise ValueError(f"chunks {start}+{n_chunks}x{B} outside the prompt of {len(tokens)} tokens")
+    if min(tokens) < 0 or max(tokens) >= c.vocab_size: raise ValueError(f"token id outside the vocabulary of {c.vocab_size}")
+    pr = np.zeros((1, c.max_context), np.int32); pr[0, :len(tokens)] = tokens
+    self.prompts.copyin(pr)
+    self.tokens.copyin(np.ascontiguousarray(pr[0, start:start + B]))
+    st = np.zeros(16, np.int32); st[0], st[3], st[5] = start, len(tokens), c.vocab_size
+    self.state.copyin(st)
+    self.chunk_of.stream.synchronize()
+    for _ in range(n_chunks):
+      if use_graph: self._graph(False).launch()
+      else: self._step(False)
+    self.stream.synchronize()
+    self.check_state()
+    return n_chunks * B
 
   def prefill(self, prompts: list[list[int]], use_graph: bool = True):
     c, B = self.config, self.batch

@@ -61,6 +61,8 @@ def _declare(lib):
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_embed_rows": [vp, i, i, vp, i, vp, vp, vp], "tga_rmsnorm_rows": [vp, vp, i, i, ctypes.c_float, vp, vp, i, vp],
     "tga_attention_decode_batched": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
+    "tga_attention_prefill_chunk": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
+    "tga_chunk_advance": [vp, vp, i, vp, i, vp],
     "tga_argmax_rows_step": [vp, i, i, vp, vp, i, vp, vp, i, vp],
     "tga_expert_jobs": [vp, i, i, vp, vp, vp], "tga_qlinear_experts_grouped": [i, vp, vp, i64, vp, i, i, vp, vp, i, i64, i64, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
