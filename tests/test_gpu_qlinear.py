@@ -161,11 +161,12 @@ def test_small_batch_weights_through_lds(gpu, t, n, k, m):
   assert y16.tobytes() == y.astype(np.float16).tobytes()
 
 @pytest.mark.parametrize("t", [2, 8, 14], ids=["q4_0", "q8_0", "q6_k"])
-@pytest.mark.parametrize("n,k", [(300, 4096), (4096 + 3, 4096), (14336, 4096), (200, 14336), (64, 6144), (129, 2112)])
+@pytest.mark.parametrize("n,k", [(8192 + 3, 4096), (14336, 4096), (2400, 14336), (5500, 6144), (15889, 2112), (300, 4096)])
 def test_two_rows_on_the_single_row_kernel(gpu, t, n, k):
   if t == 14 and k % 256: k = k // 256 * 256 + 256                       # Q6_K rows are whole 256-value superblocks
   """M = 2 for Q4_0 / Q8_0 rows of more than 32 block pairs runs on the single-row kernel's walk with two sets of activations in registers:
-  rows that one wave covers (K <= 4096) and K split over four waves, ragged row counts, more row groups than teams.  Exact weights, so the bar is
+  rows that one wave covers (K <= 4096) and K split over four waves, ragged row counts, more row groups than teams (from 2^25 weights on; the last,
+  smaller shape stays on the LDS-staged kernel).  Exact weights, so the bar is
   the float64 anchor of the exact dequantized weights (first rows) and the C restatement (all rows); fp32 activations and fp16 outputs as well."""
   rng = np.random.default_rng(2 * n + k + t)
   w = synth.random_blocks(rng, t, n, k)
@@ -185,7 +186,7 @@ def test_two_rows_segments_and_residual(gpu):
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(2424)
   k, m = 4096, 2
-  ns = [1000, 136, 130]
+  ns = [8192, 136, 130]
   for t in (2, 8):
     ws = [synth.random_blocks(rng, t, n, k) for n in ns]
     x = synth.activations(rng, m, k, np.float16)
