@@ -203,10 +203,11 @@ def test_two_rows_segments_and_residual(gpu):
     for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL
 
 @pytest.mark.parametrize("t", [2, 8], ids=["q4_0", "q8_0"])
-@pytest.mark.parametrize("n,k,m", [(8, 1024, 3), (264, 2048, 8), (2056, 3072, 5), (14336, 4096, 8), (4096, 4096, 4)])
+@pytest.mark.parametrize("n,k,m", [(8, 1024, 3), (264, 2048, 8), (2056, 3072, 5), (14336, 4096, 8), (4096, 4096, 4), (14336, 4096, 2), (8200 + 1, 4096, 2), (2400, 14336, 2), (300, 4096, 2)])
 def test_small_batch_swiglu_through_lds(gpu, t, n, k, m):
   """silu(gate) * up (tinygrad/llm/model.py:137) at 3..8 activation rows on the LDS-fed matrix-core kernel: a row group is eight gate rows and the same
-  eight up rows.  Against the float64 product of the exact dequantized weights; fp16 and float32 outputs."""
+  eight up rows.  At two rows (from 2^25 weights per matrix on) the single-row kernel's walk with two sets of activations forms the product, rows that one
+  wave covers and K split over four waves.  Against the float64 product of the exact dequantized weights; fp16 and float32 outputs."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(n + k + m + 7 * t)
   wg, wu = synth.random_blocks(rng, t, n, k), synth.random_blocks(rng, t, n, k)

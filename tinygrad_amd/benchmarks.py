@@ -95,6 +95,40 @@ def config7(steps: int = 64, ctx: int = 1024):
   return [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, Q4_K_M tensor-type mix (Q4_K + Q6_K), graph replay + sync per token",
            "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
 
+def config8(steps: int = 32, ctx: int = 1024):
+  """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 8 / 4 / 2 / 1 positions, and decoded
+  with 2, 4 and 8 sequences in lockstep (dense linears as small-batch GEMMs)."""
+  from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
+  import time
+  c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **LLAMA3_8B)
+  sd = synth_state(c, seed=1003)
+  model = Transformer(c, sd, max_new=16)
+  rt.synchronize()
+  rng = np.random.default_rng(1003)
+  prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
+  res = []
+  for chunk in (8, 4, 2, 1):
+    model.prefill_chunk = chunk
+    model.prefill(prompt[:4 * 8 + 3], reuse_cache=False)               # captures the step kinds this chunk size uses
+    t0 = time.perf_counter()
+    model.prefill(prompt, reuse_cache=False)
+    dt = time.perf_counter() - t0
+    res.append({"config": 8, "case": f"Llama-3-8B-arch Q4_0 prefill of {ctx - 1} positions, {chunk} per step", "ms": round(dt * 1e3, 1), "positions_per_s": round((ctx - 1) / dt, 1)})
+  del model
+  for B in (2, 4, 8):
+    bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
+    bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)])
+    for _ in range(4): bm.decode_step()
+    rt.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps): bm.decode_step()
+    rt.synchronize()
+    dtb = (time.perf_counter() - t0) / steps
+    bm.check_state()
+    res.append({"config": 8, "case": f"Llama-3-8B-arch Q4_0 decode B={B} ctx {ctx} (sequences in lockstep)", "tok_s": round(B / dtb, 1), "ms_per_step": round(dtb * 1e3, 4)})
+    del bm
+  return res
+
 def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
   import time
@@ -227,7 +261,7 @@ def traffic(steps: int = 4):
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix")
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix; 8 = 8B chunked prefill and batched dense decode")
   ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
   ap.add_argument("--traffic", action="store_true", help="only the workload of the HBM-traffic counter runs (see traffic())")
   args = ap.parse_args()
@@ -237,7 +271,7 @@ def main():
     for row in traffic(): print(json.dumps(row), flush=True)
     return
   for cfg in args.config:
-    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7}[cfg]
+    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7, 8: config8}[cfg]
     for row in (fn(use_graph=not args.no_graph) if cfg == 4 else fn()): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":

@@ -51,7 +51,7 @@
 // a unit is decoded once and multiplied with every row.  Outputs and residuals are (MR, rows) per matrix.
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
 __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) {
-  static_assert(MR == 1 || (PRO == 0 && EPI != 2), "several activation rows: generic prologue, plain or residual epilogue");
+  static_assert(MR == 1 || PRO == 0, "several activation rows: generic prologue");
   // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
   // issued together (read at their points of use they arrive in dependent stages, each a scalar-cache miss of its own).
   const QArgs a = args;
@@ -172,9 +172,9 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
 #pragma unroll
           for (int j = 0; j < WK; j++) t += part[parity][j][lane];
         }
-        if constexpr (EPI == 2) {
-          const float up = __shfl(t, 1, 64);
-          if (lane == 0) store_swiglu(a, row, t, up, yofs);
+        if constexpr (EPI == 2) {                               // lane 2 m holds the gate sum of activation row m, lane 2 m + 1 its up sum
+          const float up = __shfl(t, lane + 1, 64);
+          if (lane < R * MR && (lane & 1) == 0) store_swiglu(a, row, t, up, yofs + (lane >> 1) * seg_n);
         } else {
           if constexpr (EPI == 1) t += g.res[0];
           const int lm = lane / R, lr = lane % R;
@@ -184,8 +184,10 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
       parity ^= 1;
     } else {
       if (hl == (H ? 31 : 63)) {
-        if constexpr (EPI == 2) store_swiglu(a, row, acc[0][0], acc[0][R - 1], yofs);
-        else {
+        if constexpr (EPI == 2) {
+#pragma unroll
+          for (int m = 0; m < MR; m++) store_swiglu(a, row, acc[m][0], acc[m][R - 1], yofs + m * seg_n);
+        } else {
 #pragma unroll
           for (int m = 0; m < MR; m++) {
 #pragma unroll
@@ -512,10 +514,11 @@ int qgemv1_launch_format(QArgs a, hipStream_t s) {
   return launch_fast_e<T, 16, 1>(a, s);
 }
 
-// Two activation rows on the same kernel (one weight row per step, generic prologue): plain or residual epilogue, rows that one wave covers
-// or K split over four waves.  Returns -1 outside that range.
+// Two activation rows on the same kernel (one weight row per step, generic prologue): plain, residual or SwiGLU epilogue, rows that one wave
+// covers or K split over four waves.  Returns -1 outside that range.
 template <int T, int MR>
 static int qgemv1_launch_multi_m(const QArgs& a, int waves, hipStream_t s) {
+  if (a.epilogue == 2) return waves <= 1 ? launch_fast<T, 2, 1, QG1_WR, 2, false, MR>(a, s) : launch_fast<T, 2, 4, 1, 2, false, MR>(a, s);   // a row group = the gate row and the up row
   if (waves <= 1) return a.epilogue == 1 ? launch_fast<T, 1, 1, QG1_WR, 1, false, MR>(a, s) : launch_fast<T, 1, 1, QG1_WR, 0, false, MR>(a, s);
   return a.epilogue == 1 ? launch_fast<T, 1, 4, 1, 1, false, MR>(a, s) : launch_fast<T, 1, 4, 1, 0, false, MR>(a, s);
 }
@@ -525,7 +528,7 @@ int qgemv1_launch_multi(QArgs a, int M, hipStream_t s) {
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const int waves = (a.nu + 63) / 64;
-  if (a.nu <= 32 || waves > 4 || a.epilogue > 1 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y || a.route_logits) return -1;
+  if (a.nu <= 32 || waves > 4 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y || a.route_logits) return -1;
   // two rows only: every further row adds 3 us on a 14336 x 4096 matrix (the dot2 chains and lane reductions of a wave do not overlap
   // enough with two waves per SIMD; Q4_0: 9.8 / 13.0 / 15.7 / 18.7 us at M = 1..4), so from three rows on the matrix-core kernels win
   if (M == 2) return qgemv1_launch_multi_m<T, 2>(a, waves, s);
