@@ -8,9 +8,9 @@
 // one.  Here global memory is read in contiguous 16-byte pieces, 1 KB per wave instruction (global_load_lds_dwordx4: lane l's piece lands at
 // LDS base + 16 l), and the operand layout is produced by the LDS reads: each lane picks its unit out of the staged rows.
 //
-// A slot is 16 weight rows x 16 units (1024 values of K); its rows lie in LDS with a pitch of one piece more than their length, which
-// spreads the sixteen rows over the banks.  A stage is two slots (2048 values of K): waves 0-3 multiply the four steps (4 units x 16 rows
-// each) of the first, waves 4-7 those of the second.  The eight waves of the workgroup (one per CU) issue a stage's pieces together and
+// A slot is 16 weight rows x 16 or 32 units (1024 / 2048 values of K); its rows lie in LDS with a pitch of one piece more than their length, which
+// spreads the sixteen rows over the banks.  A stage is two slots: waves 0-3 multiply the steps (4 units x 16 rows each; one or two per
+// wave) of the first, waves 4-7 those of the second.  The eight waves of the workgroup (one per CU) issue a stage's pieces together and
 // keep nb - 1 stages in flight in a ring of nb.  One barrier per stage orders "all pieces of stage s have landed" before its reads and
 // "everyone is done with stage s - 1" before its slots are requested again; the partial tiles of the waves meet in LDS once per row
 // group and are reduced after the next stage's barrier.
@@ -22,9 +22,8 @@ typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef float v4f32 __attribute__((ext_vector_type(4)));
 
 #define QD_NW 8                       // waves per workgroup
-#define QD_SU 16                      // units per stage
 #define QD_LDS_CU (160 * 1024)
-#define QD_MAX_NB 4
+#define QD_MAX_NB 3
 
 template <int T> struct DmaFmt;
 template <> struct DmaFmt<F_Q4_0P> {
@@ -47,22 +46,21 @@ template <> struct DmaFmt<F_Q8_0P> {
 // at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave)
 __device__ __forceinline__ void qd_wait_vm(int n) {
   switch (n) {
-    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
-    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+#define QD_W(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
+    QD_W(1) QD_W(2) QD_W(3) QD_W(4) QD_W(5) QD_W(6) QD_W(7) QD_W(8) QD_W(9) QD_W(10) QD_W(11) QD_W(12) QD_W(13) QD_W(14) QD_W(15) QD_W(16)
+    QD_W(17) QD_W(18) QD_W(19) QD_W(20) QD_W(21) QD_W(22) QD_W(23) QD_W(24)
+#undef QD_W
     default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
   }
 }
 
 // SW: silu(gate) * up (dense SwiGLU, tinygrad/llm/model.py:137) over the two matrices w[0] / w[1]: a row group is eight rows of the gate matrix followed
 // by the same eight rows of the up matrix, so the partial tiles of both meet in one reduction and the product is formed before the store.
-template <int T_, bool MS, int NSS, bool SW = false>
+// SU: units per slot (16 or 32): a longer run of every row per slot streams better (Q4_0: 576-byte runs at 16 units, 1152 at 32) and halves the
+// number of stages, a wave then multiplies SU / 16 steps of its slot per stage.
+template <int T_, bool MS, int NSS, bool SW, int SU>
 __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args, const int M, const int nb) {
+  constexpr int QD_SU = SU, SPW = SU / 16;               // steps of one wave per slot
   static_assert(!(MS && SW), "the SwiGLU pair is not combined with the q / k / v walk");
   const QArgs a = args;
   using F = Fmt<T_>;
@@ -158,19 +156,19 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   };
 
   // this lane's activation operands: requested first (loads return in issue order), the weights second
-  u32x4 bfrag[NSS][F::XV];
+  u32x4 bfrag[NSS * SPW][F::XV];
   {
-    uint32_t nx[NSS][F::UW / 2];
-    bool have[NSS];
+    uint32_t nx[NSS * SPW][F::UW / 2];
+    bool have[NSS * SPW];
 #pragma unroll
-    for (int ss = 0; ss < NSS; ss++) {
-      const int u = (2 * ss + half) * QD_SU + 4 * step + g;
+    for (int ss = 0; ss < NSS * SPW; ss++) {
+      const int u = (2 * (ss / SPW) + half) * QD_SU + 4 * (step + 4 * (ss % SPW)) + g;
       have[ss] = r < M && u < cu;
       stage_fetch<T_>(a, r < M ? r : 0, u < cu ? u : cu - 1, nx[ss]);   // (unconditional: a valid row and unit; dropped below)
     }
     for (int k = 0; k < nb - 1; k++) if (k < S) issue_stage();
 #pragma unroll
-    for (int ss = 0; ss < NSS; ss++) {
+    for (int ss = 0; ss < NSS * SPW; ss++) {
       float c[F::NG];
       F::stage(nx[ss], bfrag[ss], c);
 #pragma unroll
@@ -181,8 +179,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
   long long cj = 0; int cst = 0, cslot = 0, par = 0;     // compute stream
   long long pend_row0 = -1; int pend_par = 0;            // row group whose partial tiles wait for the next barrier
-  auto multiply = [&](const u32x4* bv) {
-    const Raw buf = DF::from_lds((const uint32_t*)(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH + (4 * step + g) * UB));
+  auto multiply = [&](const u32x4* bv, int k) {
+    const Raw buf = DF::from_lds((const uint32_t*)(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH + (4 * (step + 4 * k) + g) * UB));
     uint32_t wv[F::NWV];
     F::decode(buf, wv, kc);
     F::to_f16(buf, wv);
@@ -200,7 +198,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     if (pend_row0 >= 0) { store_tile(pend_row0, pend_par); pend_row0 = -1; }
     if (s + nb - 1 < S) issue_stage();                                 // into the ring position stage s - 1 was read from
     if (2 * cst + half < nslots) {                                     // (the slot exists: K may end inside the stage)
-      if (NSS == 1 || cst == 0) multiply(bfrag[0]); else multiply(bfrag[NSS - 1]);
+#pragma unroll
+      for (int k = 0; k < SPW; k++) { if (NSS == 1 || cst == 0) multiply(bfrag[k], k); else multiply(bfrag[(NSS - 1) * SPW + k], k); }
     }
     cslot = cslot + 1 == nb ? 0 : cslot + 1;
     if (++cst == spg) {                                                // row group complete: the waves' partial tiles go to LDS
@@ -224,9 +223,9 @@ static int qd_cu_count() {
   return n;
 }
 
-template <int T, bool MS, int NSS, bool SW = false>
+template <int T, bool MS, int NSS, bool SW, int SU>
 static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hipStream_t s) {
-  auto kern = qgemm_dma_kernel<T, MS, NSS, SW>;
+  auto kern = qgemm_dma_kernel<T, MS, NSS, SW, SU>;
   static const hipError_t configured = [&]() {
     hipFuncAttributes fa;
     hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
@@ -242,23 +241,38 @@ static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hi
   return 0;
 }
 
+template <int T, int SU>
+static int launch_qd_su(QArgs a, int M, hipStream_t s) {
+  using F = Fmt<T>;
+  constexpr int UB = DmaFmt<T>::UB;
+  constexpr int STAGE_BYTES = 2 * ((16 * (SU * UB / 16 + 1) + 63) / 64) * 1024;
+  constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
+  int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 9 - 1024) / STAGE_BYTES);
+  if (nb > QD_MAX_NB) nb = QD_MAX_NB;                                 // (deeper rings were measured: no faster at four stages, slower at seven)
+  if (nb < 2) return -1;
+  const size_t lds = (size_t)nb * STAGE_BYTES;
+  if constexpr (SU == 32) {                                           // K <= 4096: at most two slots, one stage per row group
+    if (a.epilogue == 2) return launch_qd_k<T, false, 1, true, SU>(a, M, nb, per_cu, lds, s);
+    if (a.nseg > 1) return launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
+    return launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
+  } else {
+    const bool two = a.K > 2 * F::UW * SU;
+    if (a.epilogue == 2) return two ? launch_qd_k<T, false, 2, true, SU>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1, true, SU>(a, M, nb, per_cu, lds, s);
+    if (a.nseg > 1) return two ? launch_qd_k<T, true, 2, false, SU>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
+    return two ? launch_qd_k<T, false, 2, false, SU>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
+  }
+}
+
 template <int T>
 static int launch_qd(QArgs a, int M, hipStream_t s) {
   using F = Fmt<T>;
-  constexpr int UB = DmaFmt<T>::UB;
-  constexpr int STAGE_BYTES = 2 * ((16 * (QD_SU * UB / 16 + 1) + 63) / 64) * 1024;
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
-  if (a.K % (F::UW * QD_SU) != 0 || a.K > 4 * F::UW * QD_SU) return -1;   // whole slots only, at most four (two stages per row group)
-  constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
-  int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 9 - 1024) / STAGE_BYTES);
-  if (nb > QD_MAX_NB) nb = QD_MAX_NB;
-  if (nb < 2) return -1;
-  const size_t lds = (size_t)nb * STAGE_BYTES;
-  const bool two = a.K > 2 * F::UW * QD_SU;
-  if (a.epilogue == 2) return two ? launch_qd_k<T, false, 2, true>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1, true>(a, M, nb, per_cu, lds, s);
-  if (a.nseg > 1) return two ? launch_qd_k<T, true, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, true, 1>(a, M, nb, per_cu, lds, s);
-  return two ? launch_qd_k<T, false, 2>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1>(a, M, nb, per_cu, lds, s);
+  if (a.K % (F::UW * 16) != 0 || a.K > 4 * F::UW * 16) return -1;       // whole slots of 16 units, at most 4096 values of K
+  // Q4_0: slots of 32 units where K is whole in them (1152-byte runs, one stage per row group: 14336 x 4096 at M = 4 / 8 14.7 / 15.6 -> 13.5 / 14.4 us);
+  // Q8_0 keeps 16 (1088-byte runs already; with 32 the ring holds two stages only: 17.6 / 18.3 against 17.0 / 18.0 us)
+  if constexpr (T == F_Q4_0P) { if (a.K % (F::UW * 32) == 0) return launch_qd_su<T, 32>(a, M, s); }
+  return launch_qd_su<T, 16>(a, M, s);
 }
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
