@@ -106,20 +106,21 @@ def test_kv_prefix_reuse_equals_fresh_model(gpu):
   model.prefill(p3, reuse_cache=False)
   assert model.prefill_steps == len(p3) - 1
 
-@pytest.mark.parametrize("n_prompt", [9, 16, 61, 70, 131])
-def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt):
-  """Prompt positions computed eight at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
+@pytest.mark.parametrize("chunk", [8, 16, 5])
+@pytest.mark.parametrize("n_prompt", [9, 17, 61, 70, 131])
+def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
+  """Prompt positions computed eight or sixteen (or five) at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
   tinygrad/llm/model.py:464, 476-481) against the same model prefilled token by token and against the oracle: the KV caches agree to fp16 rounding of
   slightly different float32 results, the logits of the following decode steps stay within 1e-3 of the oracle's for the same token history, and the
   greedy tokens are the oracle's.  Prompt lengths that leave 0..7 positions for the token-by-token tail and cross the 64-position splits."""
   model, host = _build(gpu, SMALL, 192, seed=21)
   single, _ = _build(gpu, SMALL, 192, seed=21)
-  single.prefill_chunk = 1
+  model.prefill_chunk, single.prefill_chunk = chunk, 1
   rng = np.random.default_rng(21 + n_prompt)
   prompt = [int(t) for t in rng.integers(0, SMALL["vocab_size"], size=n_prompt)]
   model.prefill(prompt); single.prefill(prompt)
   assert model.prefill_steps == single.prefill_steps == n_prompt - 1
-  assert model._chunker is not None and single._chunker is None
+  assert (model._chunker is not None) == (n_prompt - 1 >= chunk) and single._chunker is None
   for bm, bs in zip(model.blk, single.blk):
     for cm, cs in ((bm.cache_k, bs.cache_k), (bm.cache_v, bs.cache_v)):
       a, b = cm.numpy().astype(np.float32)[:, :n_prompt - 1], cs.numpy().astype(np.float32)[:, :n_prompt - 1]

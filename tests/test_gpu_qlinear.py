@@ -223,6 +223,45 @@ def test_small_batch_swiglu_through_lds(gpu, t, n, k, m):
     y = out.numpy().astype(np.float32)
     assert ol.rel_err(y, ref) <= (TOL if ydt == np.float32 else 2 * TOL), ydt
 
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 16), (2, 528, 2048, 9), (8, 14336, 4096, 13), (8, 64, 1024, 16), (2, 200, 14336, 16), (14, 300, 4096, 11), (2, 257, 1024, 12), (1, 96, 2048, 16)])
+def test_nine_to_sixteen_rows(gpu, t, n, k, m):
+  """Prefill chunks of up to sixteen rows: one launch of the LDS-fed kernel where it applies (all sixteen columns of the MFMA tile), otherwise two
+  calls of at most eight rows (K beyond 4096, other formats, ragged row counts).  Against the C restatement run in blocks of eight rows."""
+  rng = np.random.default_rng(3 * n + k + m + t)
+  if t == 1: w = (rng.standard_normal((n, k)) * k ** -0.5).astype(np.float16).view(np.uint8).reshape(-1)
+  else: w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  y = _run(gpu, t, w, x, n, k)
+  if t == 1: ref = ol.linear_f64(x.astype(np.float32), w.view(np.float16).astype(np.float32).reshape(n, k))
+  else: ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
+
+def test_sixteen_rows_segments_residual_and_swiglu(gpu):
+  """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(1616)
+  m = 16
+  for t, k, ns in ((2, 2048, [2048, 512, 512]), (8, 1024, [512, 128, 130]), (14, 1024, [64, 32, 32])):
+    ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+    x = synth.activations(rng, m, k, np.float16)
+    layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+    outs = [gpu.Buffer((m, n), np.float32) for n in ns]
+    for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    xb = gpu.Buffer.from_numpy(x)
+    qlinear_multi(layers, xb, outs)
+    refs = [ol.linear_f64(x.astype(np.float32), ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]
+    for o, r in zip(outs, refs): assert ol.rel_err(o.numpy(), r) <= TOL, (t, k)
+    res = [rng.standard_normal((m, n)).astype(np.float32) for n in ns]
+    rb = [gpu.Buffer.from_numpy(r) for r in res]
+    qlinear_multi(layers, xb, rb, epilogue=1, resid=rb)
+    for o, r0, r in zip(rb, res, refs): assert ol.rel_err(o.numpy(), r0 + r) <= TOL, (t, k)
+    g = [layers[1], QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, t, ns[1], k)), t, ns[1], k)]
+    out = gpu.Buffer((m, ns[1]), np.float32)                              # (float32: products of random Q6_K rows leave the fp16 range)
+    qlinear_multi(g, xb, [out], epilogue=2)
+    a, b = refs[1], ol.linear_f64(x.astype(np.float32), ol.weight_f32(g[1].blocks.numpy(), ns[1], k, t))
+    assert ol.rel_err(out.numpy(), a / (1 + np.exp(-a)) * b) <= TOL, (t, k)
+
 def test_small_batch_through_lds_segments_and_residual(gpu):
   """q / k / v of a llama block shape in one launch at M = 4 and the residual epilogue in place, on the LDS-fed kernel's range."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
@@ -249,7 +288,8 @@ def test_argument_errors(gpu):
   w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))
   with pytest.raises(ValueError): QuantLinear(w, 1337, 4, 32)
   lin = QuantLinear(w, 2, 4, 32)
-  with pytest.raises(AssertionError): lin(gpu.Buffer((9, 32), np.float16))
+  with pytest.raises(AssertionError): lin(gpu.Buffer((17, 32), np.float16))
+  with pytest.raises(RuntimeError, match="out of range 1..16"): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 17, 4, 32, None))
   with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))
   # Q4_1 / Q5_0 / Q5_1 rows are read as block pairs: an odd number of blocks per row is refused
   with pytest.raises(RuntimeError, match="multiple of 64"): gpu.check(gpu.lib().tga_qlinear(3, w.ptr, w.ptr, 1, w.ptr, 0, 1, 1, 96, None))

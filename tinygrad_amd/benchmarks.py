@@ -96,7 +96,7 @@ def config7(steps: int = 64, ctx: int = 1024):
            "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
 
 def config8(steps: int = 32, ctx: int = 1024):
-  """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 8 / 4 / 2 / 1 positions, and decoded
+  """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 16 / 8 / 4 / 2 / 1 positions, and decoded
   with 2, 4 and 8 sequences in lockstep (dense linears as small-batch GEMMs)."""
   from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
   import time
@@ -107,9 +107,9 @@ def config8(steps: int = 32, ctx: int = 1024):
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
   res = []
-  for chunk in (8, 4, 2, 1):
+  for chunk in (16, 8, 4, 2, 1):
     model.prefill_chunk = chunk
-    model.prefill(prompt[:4 * 8 + 3], reuse_cache=False)               # captures the step kinds this chunk size uses
+    model.prefill(prompt[:4 * 16 + 3], reuse_cache=False)              # captures the step kinds this chunk size uses
     t0 = time.perf_counter()
     model.prefill(prompt, reuse_cache=False)
     dt = time.perf_counter() - t0

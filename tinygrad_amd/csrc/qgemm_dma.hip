@@ -1,4 +1,4 @@
-// Small-batch GEMM over Q4_0 / Q8_0 block pairs (3 <= M <= 8, K <= 4096) with the weights streamed into LDS by direct-to-LDS loads: the same
+// Small-batch GEMM over Q4_0 / Q8_0 block pairs (3 <= M <= 16: the sixteen columns of the MFMA tile; K <= 4096) with the weights streamed into LDS by direct-to-LDS loads: the same
 // call sites and arithmetic as qgemm.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392;
 // a unit is decoded once into fp16 weights and v_mfma_f32_16x16x32_f16 multiplies it with all activation rows).
 //
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   constexpr int IMAX = (NI2 + QD_NW - 1) / QD_NW;        // instructions of one wave per stage, at most
   constexpr int BASE = NI2 / QD_NW;                      // ... and at least
   extern __shared__ u32x4 lds[];
-  __shared__ float part[2][QD_NW][16][9];
+  __shared__ float part[2][QD_NW][16][17];
   char* ring = (char*)lds;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
@@ -203,10 +203,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     }
     cslot = cslot + 1 == nb ? 0 : cslot + 1;
     if (++cst == spg) {                                                // row group complete: the waves' partial tiles go to LDS
-      if (r < 9) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
-      }
+      for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
       pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * GR; pend_par = par;
       par ^= 1;
       acc0 = v4f32{0.f, 0.f, 0.f, 0.f}; acc1 = v4f32{0.f, 0.f, 0.f, 0.f};
@@ -247,7 +245,7 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   constexpr int UB = DmaFmt<T>::UB;
   constexpr int STAGE_BYTES = 2 * ((16 * (SU * UB / 16 + 1) + 63) / 64) * 1024;
   constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
-  int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 9 - 1024) / STAGE_BYTES);
+  int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;                                 // (deeper rings were measured: no faster at four stages, slower at seven)
   if (nb < 2) return -1;
   const size_t lds = (size_t)nb * STAGE_BYTES;
@@ -276,10 +274,10 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 }
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
-// 3 <= M <= 8, K = 1024, 2048, 3072 or 4096, every matrix a multiple of 16 rows at a 16-byte aligned address.
+// 3 <= M <= 16, K = 1024, 2048, 3072 or 4096, every matrix a multiple of 16 rows at a 16-byte aligned address.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P) return -1;
-  if (M < 3 || M > 8 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
     return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);

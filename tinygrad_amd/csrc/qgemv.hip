@@ -1,4 +1,4 @@
-// Fused GGUF block dequant + GEMV / small-batch GEMM (1 <= M <= 8) for gfx950.
+// Fused GGUF block dequant + GEMV / small-batch GEMM (1 <= M <= 8; 9 .. 16 rows for the chunked prefill, see qlinear_multi_impl) for gfx950.
 //
 // Replaces the kernel(s) tinygrad schedules for  x.linear(W.T)  (tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392)
 // when W is the lazy ggml_data_to_tensor expression over raw GGUF bytes (tinygrad/llm/gguf.py:46,56,68-72,105-114).
@@ -356,7 +356,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
-  TGA_REQUIRE(M >= 1 && M <= 8, "tga_qlinear: M=%d out of range 1..8", M);
+  TGA_REQUIRE(M >= 1 && M <= 16, "tga_qlinear: M=%d out of range 1..16", M);
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
   TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
   TGA_REQUIRE(epilogue >= 0 && epilogue <= 2, "tga_qlinear: epilogue=%d unknown", epilogue);
@@ -413,6 +413,22 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     if (fmt >= 0) { const int rc = tga_qgemm_mfma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
+  }
+  if (M > 8) {                                                    // 9..16 rows outside the LDS-fed kernel's range: two calls of at most eight rows ((M, n) outputs: row blocks are contiguous)
+    TGA_REQUIRE(!comb && !norm_w && !a.x_staged && !a.y_stage_fmt, "tga_qlinear: more than 8 rows only for plain activations");
+    const size_t xs = x_dtype == TGA_F32 ? 4 : 2, ys = y_dtype == TGA_F32 ? 4 : 2;
+    for (int m0 = 0; m0 < M; m0 += 8) {
+      const void* wv[QG_MAX_SEG]; void* yv[QG_MAX_SEG]; const void* rv[QG_MAX_SEG];
+      for (int i = 0; i < nseg; i++) {
+        wv[i] = w[i];
+        yv[i] = y[i] ? (char*)y[i] + (size_t)m0 * n[i] * ys : nullptr;
+        rv[i] = (epilogue == 1) ? (const char*)resid[i] + (size_t)m0 * n[i] * 4 : nullptr;
+      }
+      const int rc = qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, wv, yv, n, (const char*)x + (size_t)m0 * K * xs, x_dtype, y_dtype, M - m0 < 8 ? M - m0 : 8, K,
+                                        epilogue, epilogue == 1 ? rv : nullptr, 0, 0, stream);
+      if (rc) return rc;
+    }
+    return 0;
   }
   TGA_REQUIRE(!comb, "tga_moe_combine_rmsnorm_qlinear_multi: needs the M = 1 fast path with K <= 2048");
   TGA_REQUIRE(!norm_w, "tga_rmsnorm_qlinear: the fused norm needs the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, 16-byte aligned x, K <= 65536)");

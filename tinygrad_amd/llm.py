@@ -340,7 +340,7 @@ class Transformer:
     self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
     self._state_dict, self._chunker = state_dict, None               # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
-    self.prefill_chunk = 8                                           # prompt positions per prefill step (the reference's chunks hold 32, model.py:464); 1: token by token
+    self.prefill_chunk = 16                                          # prompt positions per prefill step, 2..16 (the reference's chunks hold 32, model.py:464); 1: token by token
 
   def check_state(self):
     """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
@@ -476,7 +476,7 @@ class Transformer:
     start = self.get_start_pos(tokens) if reuse_cache else 0
     self.prefill_steps = len(tokens) - 1 - start                        # (positions the last call actually computed)
     B = self.prefill_chunk
-    if 2 <= B <= 8 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
+    if 2 <= B <= 16 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
       if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
       start += self._chunker.prefill_chunks(tokens, start, (len(tokens) - 1 - start) // B, use_graph)
     self.reset(tokens, start)
@@ -531,8 +531,10 @@ class BatchedTransformer:
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024, chunk_of: "Transformer | None" = None):
     """chunk_of: the rows are `batch` consecutive prompt positions of that Transformer's sequence instead of `batch` sequences (chunked prefill,
     model.py:464, 476-481): its KV caches and rotation table are used, the attention is causal inside the chunk, no token is sampled."""
-    if not 1 <= batch <= 8: raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
-    self.config, self.batch, self.max_new, self.chunk_of = config, batch, max_new, chunk_of
+    if not 1 <= batch <= (8 if chunk_of is None else 16): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
+    self.config, self.batch, self.max_new = config, batch, max_new
+    # (no reference back to the Transformer: a cycle would leave its buffers to the cycle collector, which may free them in the middle of a stream capture)
+    self.chunked, self._owner_stream = chunk_of is not None, (chunk_of.stream if chunk_of is not None else None)
     c, B = config, batch
     f32, f16 = np.float32, np.float16
     lin = lambda name: QuantLinear(state_dict[name][0], state_dict[name][1], *state_dict[name][2])
@@ -608,7 +610,7 @@ class BatchedTransformer:
         bias = dict(epilogue=1, resid=b["bias"][i:j]) if "bias" in b else {}
         self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
         i = j
-      attention = L.tga_attention_prefill_chunk if self.chunk_of is not None else L.tga_attention_decode_batched
+      attention = L.tga_attention_prefill_chunk if self.chunked else L.tga_attention_decode_batched
       rt.check(attention(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
                          c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
                          c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn.ptr, None, st))
@@ -640,7 +642,7 @@ class BatchedTransformer:
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
       rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       self.output(self.xn, out=self.logits_buf, stream=st)
-    if self.chunk_of is not None:                                        # the next B prompt tokens, B positions on
+    if self.chunked:                                                     # the next B prompt tokens, B positions on
       rt.check(L.tga_chunk_advance(self.state.ptr, self.prompts.ptr, B, self.tokens.ptr, c.max_context, st))
       return
     rt.check(L.tga_argmax_rows_step(self.logits_buf.ptr if with_head else None, B, c.vocab_size, self.state.ptr, self.prompts.ptr, c.max_context, self.tokens.ptr,
@@ -657,7 +659,7 @@ class BatchedTransformer:
     """Chunked prefill for `chunk_of`: computes the positions start .. start + n_chunks * batch - 1 of the prompt, `batch` at a time, into its KV caches.
     Returns the number of positions done."""
     c, B = self.config, self.batch
-    if self.chunk_of is None: raise RuntimeError("prefill_chunks needs a model built with chunk_of")
+    if not self.chunked: raise RuntimeError("prefill_chunks needs a model built with chunk_of")
     if n_chunks <= 0: return 0
     if not (0 <= start and start + n_chunks * B <= len(tokens) < c.max_context): raise ValueError(f"chunks {start}+{n_chunks}x{B} outside the prompt of {len(tokens)} tokens")
     if min(tokens) < 0 or max(tokens) >= c.vocab_size: raise ValueError(f"token id outside the vocabulary of {c.vocab_size}")
@@ -666,7 +668,7 @@ class BatchedTransformer:
     self.tokens.copyin(np.ascontiguousarray(pr[0, start:start + B]))
     st = np.zeros(16, np.int32); st[0], st[3], st[5] = start, len(tokens), c.vocab_size
     self.state.copyin(st)
-    self.chunk_of.stream.synchronize()
+    self._owner_stream.synchronize()
     for _ in range(n_chunks):
       if use_graph: self._graph(False).launch()
       else: self._step(False)

@@ -170,12 +170,29 @@ class Event:
   def __del__(self):
     if getattr(self, "handle", None) and _lib is not None: _lib.tga_event_destroy(ctypes.c_void_p(self.handle)); self.handle = None
 
+def _capture_begin(stream: Stream) -> bool:
+  """Starts a stream capture with Python's cycle collector held off: a collection in the middle of a capture could free device buffers of dead
+  objects (hipFree is not allowed while a capture is open: it invalidates the capture).  Returns whether the collector has to be switched on again."""
+  import gc
+  was = gc.isenabled()
+  gc.collect(); gc.disable()
+  try: check(lib().tga_graph_begin(stream.handle))
+  except Exception:
+    if was: gc.enable()
+    raise
+  return was
+
+def _capture_done(was_enabled: bool):
+  import gc
+  if was_enabled: gc.enable()
+
 class Graph:
   """Captured launch sequence replayed per decode step (the reference's TinyJit replay, tinygrad/engine/jit.py:163-198)."""
   def __init__(self, stream: Stream): self.stream, self.handle = stream, None
-  def __enter__(self): check(lib().tga_graph_begin(self.stream.handle)); return self
+  def __enter__(self): self._gc = _capture_begin(self.stream); return self
   def __exit__(self, et, ev, tb):
     p = ctypes.c_void_p(); st = lib().tga_graph_end(self.stream.handle, ctypes.byref(p))
+    _capture_done(self._gc)
     if et is None: check(st); self.handle = p.value
     return False
   def launch(self): check(lib().tga_graph_launch(self.handle, self.stream.handle))
@@ -185,9 +202,10 @@ class Graph:
 class CommandList:
   """Graph's interface over tga_cmdlist_*: the captured kernel launches are enqueued one after the other instead of going through hipGraphLaunch."""
   def __init__(self, stream: Stream): self.stream, self.handle = stream, None
-  def __enter__(self): check(lib().tga_graph_begin(self.stream.handle)); return self
+  def __enter__(self): self._gc = _capture_begin(self.stream); return self
   def __exit__(self, et, ev, tb):
     p = ctypes.c_void_p(); st = lib().tga_cmdlist_end(self.stream.handle, ctypes.byref(p))
+    _capture_done(self._gc)
     if et is None: check(st); self.handle = p.value
     return False
   def launch(self): check(lib().tga_cmdlist_launch(self.handle, self.stream.handle))
