@@ -237,6 +237,25 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 14336, 16), (8, 4096, 14336, 8), (2, 256, 5120, 3), (8, 48, 14336, 9), (2, 4112, 8192, 13), (8, 1024, 6144, 16)])
+def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
+  """K beyond 4096 on the LDS-fed kernel (one matrix): the activations stream beside the weights, whole lines per load, and reach
+  the operand layout through a wave-private piece of LDS; float32 activations are rounded on the way into it.  Plain and with the residual added in place, 0xFF-filled outputs, against the C
+  restatement run in blocks of eight rows."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(7 * n + k + m + t)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  y = _run(gpu, t, w, x, n, k)
+  assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
+  layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  res = rng.standard_normal((m, n)).astype(np.float32)
+  rb = gpu.Buffer.from_numpy(res)
+  qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
+  assert ol.rel_err(rb.numpy(), res + ref) <= TOL
+
 def test_sixteen_rows_segments_residual_and_swiglu(gpu):
   """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

@@ -16,6 +16,10 @@
 // group and are reduced after the next stage's barrier.
 // A wave meets the same units of K in every row group (K <= 4096: at most two), so its activation operands - lane (g, c): the eight
 // vectors of row c's unit, zeros for c >= M - stay in registers for the whole launch; LDS holds nothing but the ring.
+// K > 4096 (XS): the activations are streamed too.  A wave reads the 512 bytes of every activation row that its step of the next stage multiplies in
+// whole 128-byte lines (eight loads of 1 KB, two rows each: a lane-per-unit read would touch 64 lines per instruction and use 16 bytes of each),
+// issued in front of the weight pieces of the stage after (loads return in issue order: the wait that lets the weights of later stages stay in
+// flight then covers them), and turns them into the operand layout through a wave-private piece of LDS.
 #include "qfmt.h"
 
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
@@ -58,10 +62,12 @@ __device__ __forceinline__ void qd_wait_vm(int n) {
 // by the same eight rows of the up matrix, so the partial tiles of both meet in one reduction and the product is formed before the store.
 // SU: units per slot (16 or 32): a longer run of every row per slot streams better (Q4_0: 576-byte runs at 16 units, 1152 at 32) and halves the
 // number of stages, a wave then multiplies SU / 16 steps of its slot per stage.
-template <int T_, bool MS, int NSS, bool SW, int SU>
+#define QD_XT_PITCH 528                // bytes between activation rows in a wave's transposition buffer (512 + one piece: sixteen rows spread over the banks)
+template <int T_, bool MS, int NSS, bool SW, int SU, bool XS = false, bool XF = false>      // XF: (XS) float32 activations
 __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args, const int M, const int nb) {
   constexpr int QD_SU = SU, SPW = SU / 16;               // steps of one wave per slot
   static_assert(!(MS && SW), "the SwiGLU pair is not combined with the q / k / v walk");
+  static_assert(!XS || (SPW == 1 && !MS && !SW), "streamed activations: one step per wave and stage, a single matrix");
   const QArgs a = args;
   using F = Fmt<T_>;
   using DF = DmaFmt<T_>;
@@ -156,8 +162,33 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   };
 
   // this lane's activation operands: requested first (loads return in issue order), the weights second
-  u32x4 bfrag[NSS * SPW][F::XV];
-  {
+  u32x4 bfrag[XS ? 1 : NSS * SPW][F::XV];
+  constexpr int NXI = XF ? 16 : 8;                       // (XS) load instructions per stage: one row of 256 float32 or two rows of 256 fp16 each
+  u32x4 xin[NXI];                                        // (XS) the wave's activation pieces of the next stage on their way in (requesting them two stages ahead
+                                                         // gained nothing: a stage waits 0.1 us for its loads, the rest is issue, LDS round trips and the barrier)
+  const int xrows = M > 8 ? 16 : 8;                      // (XS) activation rows in the transposition buffer
+  char* xt = ring + (size_t)nb * (2 * SLOT_BYTES) + (size_t)wave * xrows * QD_XT_PITCH;
+  auto fetch_x = [&](int st, u32x4 (&xs)[NXI]) __attribute__((always_inline)) {     // stage st of a row group: 256 consecutive values of every activation row
+    const int u0 = (2 * st + half) * QD_SU + 4 * step;   // (u0 + 3 < cu wherever the slot exists: K is whole slots)
+    const int uc = u0 + 3 < cu ? u0 : cu - 4;
+#pragma unroll
+    for (int v = 0; v < NXI; v++) {
+      if ((XF ? v : 2 * v) < xrows) {                    // (the same for the whole workgroup)
+        int row = XF ? v : 2 * v + (lane >> 5); row = row < M ? row : 0;
+        const char* p = XF ? (const char*)((const float*)a.x + (long long)row * a.K + 64 * uc + 4 * lane)
+                           : (const char*)((const uint16_t*)a.x + (long long)row * a.K + 64 * uc + 8 * (lane & 31));
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xs[v]) : "v"(p) : "memory");
+      }
+    }
+  };
+  auto pin_x = [&](u32x4 (&xs)[NXI]) __attribute__((always_inline)) {       // no use of the pieces moves in front of the wait that precedes this
+    asm volatile("" : "+v"(xs[0]), "+v"(xs[1]), "+v"(xs[2]), "+v"(xs[3]), "+v"(xs[4]), "+v"(xs[5]), "+v"(xs[6]), "+v"(xs[7]) :: "memory");
+    if constexpr (XF) asm volatile("" : "+v"(xs[8]), "+v"(xs[9]), "+v"(xs[10]), "+v"(xs[11]), "+v"(xs[12]), "+v"(xs[13]), "+v"(xs[14]), "+v"(xs[15]) :: "memory");
+  };
+  if constexpr (XS) {
+    fetch_x(0, xin);
+    for (int k = 0; k < nb - 1; k++) if (k < S) issue_stage();
+  } else {
     uint32_t nx[NSS * SPW][F::UW / 2];
     bool have[NSS * SPW];
 #pragma unroll
@@ -191,6 +222,58 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
       else acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[v]), acc0, 0, 0, 0);
     }
   };
+  auto finish_stage = [&]() __attribute__((always_inline)) {
+    cslot = cslot + 1 == nb ? 0 : cslot + 1;
+    if (++cst == spg) {                                                // row group complete: the waves' partial tiles go to LDS
+#pragma unroll
+      for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
+      pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * GR; pend_par = par;
+      par ^= 1;
+      acc0 = v4f32{0.f, 0.f, 0.f, 0.f}; acc1 = v4f32{0.f, 0.f, 0.f, 0.f};
+      cst = 0; cj++;
+    }
+  };
+  // (XS) one stage; the activations of stage s sit in register set `set`
+  auto xs_stage = [&](long long s, u32x4 (&xs)[NXI]) __attribute__((always_inline)) {
+    const long long after = S - 1 - s;
+    // queue of this wave: ... x(s), weights(s + 1) | x(s + 1), weights(s + 2) ...: with the weights of stage s + 1 (and nothing else) allowed to be
+    // outstanding, the weights of stage s and the activations of stage s have arrived
+    qd_wait_vm((int)(after < nb - 2 ? after : nb - 2) * BASE);
+    pin_x(xs);
+#pragma unroll
+    for (int v = 0; v < NXI; v++) {
+      if constexpr (XF) {
+        if (v < xrows) {
+          const f32x4 f = __builtin_bit_cast(f32x4, xs[v]);
+          *(uint2*)(xt + v * QD_XT_PITCH + 8 * lane) = uint2{f2h_bits(f.x) | (f2h_bits(f.y) << 16), f2h_bits(f.z) | (f2h_bits(f.w) << 16)};
+        }
+      } else {
+        if (2 * v < xrows) *(u32x4*)(xt + (2 * v + (lane >> 5)) * QD_XT_PITCH + 16 * (lane & 31)) = xs[v];
+      }
+    }
+    // (a __syncthreads() here makes the compiler wait for every outstanding vector-memory operation in front of the barrier)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (pend_row0 >= 0) { store_tile(pend_row0, pend_par); pend_row0 = -1; }
+    // one request site in the loop: the compiler must have no reason to copy the pieces from one set of registers to another while they are on
+    // their way (it takes them for present as soon as the request is issued)
+    fetch_x(cst + 1 == spg ? 0 : cst + 1, xs);                           // (past the last stage: a valid address, never used)
+    if (s + nb - 1 < S) issue_stage();
+    if (2 * cst + half < nslots) {
+      uint32_t nx[F::UW / 2];
+      const char* src = xt + (r < xrows ? r : 0) * QD_XT_PITCH + 128 * g;
+#pragma unroll
+      for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * j); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
+      float c[F::NG];
+      F::stage(nx, bfrag[0], c);
+#pragma unroll
+      for (int v = 0; v < F::XV; v++) if (r >= M) bfrag[0][v] = u32x4{0u, 0u, 0u, 0u};
+      multiply(bfrag[0], 0);
+    }
+    finish_stage();
+  };
+  if constexpr (XS) {
+    for (long long s = 0; s < S; s++) xs_stage(s, xin);
+  } else {
   for (long long s = 0; s < S; s++) {
     const long long after = S - 1 - s;
     qd_wait_vm((int)(after < nb - 2 ? after : nb - 2) * BASE);         // this wave's pieces of stage s have landed (later stages may be in flight)
@@ -201,16 +284,10 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
 #pragma unroll
       for (int k = 0; k < SPW; k++) { if (NSS == 1 || cst == 0) multiply(bfrag[k], k); else multiply(bfrag[(NSS - 1) * SPW + k], k); }
     }
-    cslot = cslot + 1 == nb ? 0 : cslot + 1;
-    if (++cst == spg) {                                                // row group complete: the waves' partial tiles go to LDS
-#pragma unroll
-      for (int i = 0; i < 4; i++) part[par][wave][4 * g + i][r] = acc0[i] + acc1[i];
-      pend_row0 = ((long long)blockIdx.x + cj * gridDim.x) * GR; pend_par = par;
-      par ^= 1;
-      acc0 = v4f32{0.f, 0.f, 0.f, 0.f}; acc1 = v4f32{0.f, 0.f, 0.f, 0.f};
-      cst = 0; cj++;
-    }
+    finish_stage();
   }
+  }
+  if constexpr (XS) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); pin_x(xin); }   // the last request is never used: it has arrived before the wave ends
   __syncthreads();
   if (pend_row0 >= 0) store_tile(pend_row0, pend_par);
 }
@@ -221,9 +298,9 @@ static int qd_cu_count() {
   return n;
 }
 
-template <int T, bool MS, int NSS, bool SW, int SU>
+template <int T, bool MS, int NSS, bool SW, int SU, bool XS = false, bool XF = false>
 static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hipStream_t s) {
-  auto kern = qgemm_dma_kernel<T, MS, NSS, SW, SU>;
+  auto kern = qgemm_dma_kernel<T, MS, NSS, SW, SU, XS, XF>;
   static const hipError_t configured = [&]() {
     hipFuncAttributes fa;
     hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
@@ -261,12 +338,29 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   }
 }
 
+// K > 4096: activations streamed beside the weights (one matrix, plain or residual epilogue)
+template <int T>
+static int launch_qd_xs(const QArgs& a, int M, hipStream_t s) {
+  constexpr int UB = DmaFmt<T>::UB, SU = 16;
+  constexpr int STAGE_BYTES = 2 * ((16 * (SU * UB / 16 + 1) + 63) / 64) * 1024;
+  const long long xt_bytes = (long long)QD_NW * (M > 8 ? 16 : 8) * QD_XT_PITCH;
+  int nb = (int)((QD_LDS_CU - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024 - xt_bytes) / STAGE_BYTES);
+  if (nb > QD_MAX_NB) nb = QD_MAX_NB;
+  if (nb < 2) return -1;
+  const size_t lds = (size_t)nb * STAGE_BYTES + (size_t)xt_bytes;
+  return a.x_f32 ? launch_qd_k<T, false, 1, false, SU, true, true>(a, M, nb, 1, lds, s) : launch_qd_k<T, false, 1, false, SU, true, false>(a, M, nb, 1, lds, s);
+}
+
 template <int T>
 static int launch_qd(QArgs a, int M, hipStream_t s) {
   using F = Fmt<T>;
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
-  if (a.K % (F::UW * 16) != 0 || a.K > 4 * F::UW * 16) return -1;       // whole slots of 16 units, at most 4096 values of K
+  if (a.K % (F::UW * 16) != 0) return -1;                                // whole slots of 16 units
+  if (a.K > 4 * F::UW * 16) {
+    if (a.nseg != 1 || a.epilogue > 1) return -1;
+    return launch_qd_xs<T>(a, M, s);
+  }
   // Q4_0: slots of 32 units where K is whole in them (1152-byte runs, one stage per row group: 14336 x 4096 at M = 4 / 8 14.7 / 15.6 -> 13.5 / 14.4 us);
   // Q8_0 keeps 16 (1088-byte runs already; with 32 the ring holds two stages only: 17.6 / 18.3 against 17.0 / 18.0 us)
   if constexpr (T == F_Q4_0P) { if (a.K % (F::UW * 32) == 0) return launch_qd_su<T, 32>(a, M, s); }
@@ -274,7 +368,8 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 }
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
-// 3 <= M <= 16, K = 1024, 2048, 3072 or 4096, every matrix a multiple of 16 rows at a 16-byte aligned address.
+// 3 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
+// 16 rows at a 16-byte aligned address.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P) return -1;
   if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
