@@ -21,6 +21,7 @@
 // issued in front of the weight pieces of the stage after (loads return in issue order: the wait that lets the weights of later stages stay in
 // flight then covers them), and turns them into the operand layout through a wave-private piece of LDS.
 #include "qfmt.h"
+#include <type_traits>
 
 typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef float v4f32 __attribute__((ext_vector_type(4)));
@@ -189,22 +190,69 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     fetch_x(0, xin);
     for (int k = 0; k < nb - 1; k++) if (k < S) issue_stage();
   } else {
-    uint32_t nx[NSS * SPW][F::UW / 2];
-    bool have[NSS * SPW];
+    // Every activation row's 256 values of a step are read in whole lines (a lane-per-unit read touches 64 lines per instruction and uses 16 bytes
+    // of each) and reach the operand layout through LDS: the ring position that the first stages do not use yet, 8 KB per wave, the 16-byte pieces
+    // of row c rotated by c so that writes and reads are free of bank conflicts.
+    constexpr int NST = NSS * SPW;
+    char* xb = ring + (size_t)(nb - 1) * (2 * SLOT_BYTES) + (size_t)wave * 8192;
+    bool have[NST]; int uc[NST];
 #pragma unroll
-    for (int ss = 0; ss < NSS * SPW; ss++) {
-      const int u = (2 * (ss / SPW) + half) * QD_SU + 4 * (step + 4 * (ss % SPW)) + g;
-      have[ss] = r < M && u < cu;
-      stage_fetch<T_>(a, r < M ? r : 0, u < cu ? u : cu - 1, nx[ss]);   // (unconditional: a valid row and unit; dropped below)
+    for (int ss = 0; ss < NST; ss++) {
+      const int u0 = (2 * (ss / SPW) + half) * QD_SU + 4 * (step + 4 * (ss % SPW));
+      have[ss] = r < M && u0 + g < cu;
+      uc[ss] = u0 + 3 < cu ? u0 : cu - 4;                // (K is whole slots of at least 16 units)
     }
-    for (int k = 0; k < nb - 1; k++) if (k < S) issue_stage();
+    // The requests are inline assembly and the wait is counted by hand: a compiler-placed wait would also cover the weight pieces issued behind
+    // them (it cannot count those), i.e. the operands would be formed only after the first stages have landed.  Requests, wait and the writes to
+    // LDS are straight-line code per row count (4, 8 or 16 rows: what a workgroup reads of the activations is as much as it reads of a Q4_0
+    // matrix at sixteen rows): a request behind a condition would give the compiler a reason to move the pieces between registers while they
+    // are on their way (it takes them for present as soon as the request is issued).
+    const int mine = (NI2 - wave + QD_NW - 1) / QD_NW;   // this wave's pieces per stage
+    auto prologue = [&](auto rows_tag, auto f32_tag) __attribute__((always_inline)) {
+      constexpr int XR = decltype(rows_tag)::value;      // rows requested (rows at and beyond M repeat row 0 and are dropped)
+      constexpr bool F32 = decltype(f32_tag)::value;
+      constexpr int NV = F32 ? XR : XR / 2;              // float32: instruction v = row v, lane l = values 4 l .. 4 l + 3; fp16: rows 2 v and 2 v + 1, lane l = piece l & 31 of row 2 v + (l >> 5)
+      u32x4 xq[NST][NV];
 #pragma unroll
-    for (int ss = 0; ss < NSS * SPW; ss++) {
-      float c[F::NG];
-      F::stage(nx[ss], bfrag[ss], c);
+      for (int ss = 0; ss < NST; ss++)
 #pragma unroll
-      for (int v = 0; v < F::XV; v++) if (!have[ss]) bfrag[ss][v] = u32x4{0u, 0u, 0u, 0u};
-    }
+        for (int v = 0; v < NV; v++) {
+          const int row = F32 ? v : 2 * v + (lane >> 5);
+          const char* ptr = F32 ? (const char*)((const float*)a.x + (long long)(row < M ? row : 0) * a.K + 64 * uc[ss] + 4 * lane)
+                                : (const char*)((const uint16_t*)a.x + (long long)(row < M ? row : 0) * a.K + 64 * uc[ss] + 8 * (lane & 31));
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xq[ss][v]) : "v"(ptr) : "memory");
+        }
+      int issued = 0;
+      for (int k = 0; k < nb - 1; k++) if (k < S) { issue_stage(); issued++; }
+      qd_wait_vm(issued * mine);
+#pragma unroll
+      for (int ss = 0; ss < NST; ss++) {
+#pragma unroll
+        for (int v = 0; v < NV; v++) asm volatile("" : "+v"(xq[ss][v]) :: "memory");      // no use of the pieces moves in front of the wait
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+          if constexpr (F32) {
+            const f32x4 f = __builtin_bit_cast(f32x4, xq[ss][v]);
+            *(uint2*)(xb + v * 512 + 16 * (((lane >> 1) + v) & 31) + 8 * (lane & 1)) = uint2{f2h_bits(f.x) | (f2h_bits(f.y) << 16), f2h_bits(f.z) | (f2h_bits(f.w) << 16)};
+          } else {
+            const int row = 2 * v + (lane >> 5);
+            *(u32x4*)(xb + row * 512 + 16 * (((lane & 31) + row) & 31)) = xq[ss][v];
+          }
+        }
+        uint32_t nx[F::UW / 2];
+        const int c = r < XR ? r : 0;
+        const char* src = xb + c * 512;
+#pragma unroll
+        for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * ((8 * g + j + c) & 31)); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
+        float cs[F::NG];
+        F::stage(nx, bfrag[ss], cs);
+#pragma unroll
+        for (int v = 0; v < F::XV; v++) if (!have[ss]) bfrag[ss][v] = u32x4{0u, 0u, 0u, 0u};
+      }
+    };
+    typedef std::integral_constant<int, 4> R4; typedef std::integral_constant<int, 8> R8; typedef std::integral_constant<int, 16> R16;
+    if (a.x_f32) { if (M > 8) prologue(R16{}, std::true_type{}); else if (M > 4) prologue(R8{}, std::true_type{}); else prologue(R4{}, std::true_type{}); }
+    else { if (M > 8) prologue(R16{}, std::false_type{}); else if (M > 4) prologue(R8{}, std::false_type{}); else prologue(R4{}, std::false_type{}); }
   }
 
   v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
@@ -325,7 +373,10 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;                                 // (deeper rings were measured: no faster at four stages, slower at seven)
   if (nb < 2) return -1;
-  const size_t lds = (size_t)nb * STAGE_BYTES;
+  size_t lds = (size_t)nb * STAGE_BYTES;
+  const size_t with_x = (size_t)(nb - 1) * STAGE_BYTES + (size_t)QD_NW * 8192;   // the activations pass through the last ring position and what follows it
+  if (with_x > lds) lds = with_x;
+  if (lds > (size_t)QD_LDS_CU - sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) return -1;
   if constexpr (SU == 32) {                                           // K <= 4096: at most two slots, one stage per row group
     if (a.epilogue == 2) return launch_qd_k<T, false, 1, true, SU>(a, M, nb, per_cu, lds, s);
     if (a.nseg > 1) return launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
