@@ -256,6 +256,30 @@ def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
   qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
   assert ol.rel_err(rb.numpy(), res + ref) <= TOL
 
+@pytest.mark.parametrize("n,k,m", [(16, 2048, 3), (4096 + 48, 4096, 8), (1024, 4096, 16), (4112, 2048, 5), (272, 4096, 11)])
+def test_small_batch_q6_k_through_lds(gpu, n, k, m):
+  """Q6_K on the kernel that streams the weights into LDS (one matrix, K = 2048 or 4096, rows a multiple of 16): a slot is eight superblocks of 210
+  bytes per row, a wave's step one superblock read at 2-byte alignment.  Plain and with the residual, fp16 and float32 activations, against the C
+  restatement run in blocks of eight rows and, for the first rows, the float64 anchor."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  t = 14
+  rng = np.random.default_rng(6 * n + k + m)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  y = _run(gpu, t, w, x, n, k)
+  assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
+  rows = min(n, 64)
+  nel, nby = GGML_QUANT[t]
+  W = ol.weight_f32(w[:rows * (k // nel) * nby], rows, k, t)
+  assert ol.rel_err(y[:, :rows], ol.linear_f64(x.astype(np.float32), W)) <= TOL
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
+  layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  res = rng.standard_normal((m, n)).astype(np.float32)
+  rb = gpu.Buffer.from_numpy(res)
+  qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
+  assert ol.rel_err(rb.numpy(), res + ref) <= TOL
+
 def test_sixteen_rows_segments_residual_and_swiglu(gpu):
   """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

@@ -1,4 +1,4 @@
-// Small-batch GEMM over Q4_0 / Q8_0 block pairs (3 <= M <= 16: the sixteen columns of the MFMA tile; K <= 4096) with the weights streamed into LDS by direct-to-LDS loads: the same
+// Small-batch GEMM over Q4_0 / Q8_0 block pairs and Q6_K (3 <= M <= 16: the sixteen columns of the MFMA tile) with the weights streamed into LDS by direct-to-LDS loads: the same
 // call sites and arithmetic as qgemm.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392;
 // a unit is decoded once into fp16 weights and v_mfma_f32_16x16x32_f16 multiplies it with all activation rows).
 //
@@ -30,20 +30,51 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 #define QD_LDS_CU (160 * 1024)
 #define QD_MAX_NB 3
 
+// slot_bytes(su): bytes of su units of one row; PAD: 16-byte pieces between the rows of a slot in LDS (the pitch spreads sixteen rows over the banks);
+// from_lds(row, u): unit u of a slot's row.
 template <int T> struct DmaFmt;
 template <> struct DmaFmt<F_Q4_0P> {
-  static constexpr int UB = 36;
-  static __device__ __forceinline__ Fmt<F_Q4_0P>::Raw from_lds(const uint32_t* p) {
+  static constexpr int PAD = 1;
+  static constexpr int slot_bytes(int su) { return su * 36; }
+  static __device__ __forceinline__ Fmt<F_Q4_0P>::Raw from_lds(const char* row, int u) {
+    const uint32_t* p = (const uint32_t*)(row + 36 * u);
     Fmt<F_Q4_0P>::Raw r;
     r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = p[8];
     return r;
   }
 };
 template <> struct DmaFmt<F_Q8_0P> {
-  static constexpr int UB = 68;
-  static __device__ __forceinline__ Fmt<F_Q8_0P>::Raw from_lds(const uint32_t* p) {
+  static constexpr int PAD = 1;
+  static constexpr int slot_bytes(int su) { return su * 68; }
+  static __device__ __forceinline__ Fmt<F_Q8_0P>::Raw from_lds(const char* row, int u) {
+    const uint32_t* p = (const uint32_t*)(row + 68 * u);
     Fmt<F_Q8_0P>::Raw r;
     r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = u32x4{p[8], p[9], p[10], p[11]}; r.d = u32x4{p[12], p[13], p[14], p[15]}; r.e = p[16];
+    return r;
+  }
+};
+
+// Q6_K (gguf.py:68-72): four units = one superblock of 210 bytes, so a slot is 32 units = 8 superblocks = 105 pieces and a wave's step of four units is one
+// superblock; superblocks are 2-byte aligned in the slot's row: every 16-byte piece is read as its enclosing aligned dwords and funnel-shifted (by 0 or 16 bits,
+// the same for the whole wave), as Fmt<GGML_Q6_K>::load does from global memory.
+__device__ __forceinline__ u32x4 lds16_a2(const char* p, uint32_t& tail_dword, uint32_t& sh) {
+  const uint32_t a = (uint32_t)(uintptr_t)p; sh = (a & 2u) * 8u;
+  const uint32_t* q = (const uint32_t*)(p - (a & 3u));
+  const uint32_t v0 = q[0], v1 = q[1], v2 = q[2], v3 = q[3], e = q[4];
+  tail_dword = e;
+  return u32x4{__builtin_amdgcn_alignbit(v1, v0, sh), __builtin_amdgcn_alignbit(v2, v1, sh), __builtin_amdgcn_alignbit(v3, v2, sh), __builtin_amdgcn_alignbit(e, v3, sh)};
+}
+template <> struct DmaFmt<GGML_Q6_K> {
+  static constexpr int PAD = 2;                          // pitch 107 pieces = 428 dwords = 44 mod 64: sixteen rows on sixteen different bank quads
+  static constexpr int slot_bytes(int su) { return su / 4 * 210; }
+  static __device__ __forceinline__ Fmt<GGML_Q6_K>::Raw from_lds(const char* row, int u) {
+    const char* p = row + 210 * (u >> 2); const int h = (u >> 1) & 1, g = u & 1;
+    uint32_t tail, sh;
+    Fmt<GGML_Q6_K>::Raw r;
+    r.a = lds16_a2(p + 64 * h + 16 * g, tail, sh); r.b = lds16_a2(p + 64 * h + 32 + 16 * g, tail, sh); r.h = lds16_a2(p + 128 + 32 * h + 16 * g, tail, sh);
+    const u32x4 sc = lds16_a2(p + 192, tail, sh);          // sc[0..15]; the tail dword holds d (bytes 208, 209)
+    r.sc0 = h ? sc.z : sc.x; r.sc1 = h ? sc.w : sc.y;
+    r.d = (uint32_t)g | (__builtin_amdgcn_alignbit(0u, tail, sh) << 16);
     return r;
   }
 };
@@ -73,10 +104,11 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   using F = Fmt<T_>;
   using DF = DmaFmt<T_>;
   typedef typename F::Raw Raw;
-  constexpr int UB = DF::UB;
-  constexpr int PR = QD_SU * UB / 16;                    // 16-byte pieces of one row in a slot
-  constexpr int PITCH = (PR + 1) * 16;                   // LDS bytes from one row of the slot to the next
-  constexpr int SLOTS = 16 * (PR + 1);
+  constexpr int SB = DF::slot_bytes(QD_SU);              // bytes of one row in a slot
+  static_assert(SB % 16 == 0, "a slot's row is whole 16-byte pieces");
+  constexpr int PR = SB / 16;                            // ... in 16-byte pieces
+  constexpr int PITCH = (PR + DF::PAD) * 16;             // LDS bytes from one row of the slot to the next
+  constexpr int SLOTS = 16 * (PR + DF::PAD);
   constexpr int NI = (SLOTS + 63) / 64;                  // wave instructions (1 KB each) per slot
   constexpr int SLOT_BYTES = NI * 1024;
   constexpr int NI2 = 2 * NI;                            // ... per stage
@@ -137,17 +169,17 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   for (int i = 0; i < IMAX; i++) {
     const int j = wave + QD_NW * i, sl = j >= NI ? 1 : 0;
     const int sigma = 64 * (j - sl * NI) + lane;
-    int rr = sigma / (PR + 1), q = sigma - rr * (PR + 1);
+    int rr = sigma / (PR + DF::PAD), q = sigma - rr * (PR + DF::PAD);
     rr = rr < 16 ? rr : 15; q = q < PR ? q : PR - 1;
     from_up[i] = SW && rr >= 8;
     doff_odd[i] = (long long)(SW ? (rr & 7) : rr) * a.row_bytes + q * 16;
-    doff[i] = doff_odd[i] + sl * (QD_SU * UB);
+    doff[i] = doff_odd[i] + sl * SB;
   }
   long long ij = 0; int ist = 0, islot = 0;              // issue stream: row group index (of this workgroup), stage in the group, ring position
   auto issue_stage = [&]() {
     const long long grp = (long long)blockIdx.x + ij * gridDim.x;
     int sg; long long l0; seg_of(grp * GR, sg, l0);
-    const long long goff = l0 * a.row_bytes + (long long)ist * (2 * QD_SU * UB);
+    const long long goff = l0 * a.row_bytes + (long long)ist * (2 * SB);
     const uint8_t* base = w_of(sg) + goff;
     const uint8_t* base_up = SW ? a.w[1] + goff : base;
     char* dst = ring + (size_t)islot * (2 * SLOT_BYTES);
@@ -243,7 +275,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
         const int c = r < XR ? r : 0;
         const char* src = xb + c * 512;
 #pragma unroll
-        for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * ((8 * g + j + c) & 31)); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
+        for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * ((F::xoff(g, 4 * j) / 8 + c) & 31)); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
         float cs[F::NG];
         F::stage(nx, bfrag[ss], cs);
 #pragma unroll
@@ -259,7 +291,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   long long cj = 0; int cst = 0, cslot = 0, par = 0;     // compute stream
   long long pend_row0 = -1; int pend_par = 0;            // row group whose partial tiles wait for the next barrier
   auto multiply = [&](const u32x4* bv, int k) {
-    const Raw buf = DF::from_lds((const uint32_t*)(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH + (4 * (step + 4 * k) + g) * UB));
+    const Raw buf = DF::from_lds(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH, 4 * (step + 4 * k) + g);
     uint32_t wv[F::NWV];
     F::decode(buf, wv, kc);
     F::to_f16(buf, wv);
@@ -367,8 +399,7 @@ static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hi
 template <int T, int SU>
 static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   using F = Fmt<T>;
-  constexpr int UB = DmaFmt<T>::UB;
-  constexpr int STAGE_BYTES = 2 * ((16 * (SU * UB / 16 + 1) + 63) / 64) * 1024;
+  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::slot_bytes(SU) / 16 + DmaFmt<T>::PAD) + 63) / 64) * 1024;
   constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
   int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;                                 // (deeper rings were measured: no faster at four stages, slower at seven)
@@ -377,7 +408,10 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   const size_t with_x = (size_t)(nb - 1) * STAGE_BYTES + (size_t)QD_NW * 8192;   // the activations pass through the last ring position and what follows it
   if (with_x > lds) lds = with_x;
   if (lds > (size_t)QD_LDS_CU - sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) return -1;
-  if constexpr (SU == 32) {                                           // K <= 4096: at most two slots, one stage per row group
+  if constexpr (T == GGML_Q6_K) {                                     // (one matrix, plain or residual epilogue: the lm-head and single linears)
+    if (a.epilogue == 2 || a.nseg > 1) return -1;
+    return launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
+  } else if constexpr (SU == 32) {                                    // K <= 4096: at most two slots, one stage per row group
     if (a.epilogue == 2) return launch_qd_k<T, false, 1, true, SU>(a, M, nb, per_cu, lds, s);
     if (a.nseg > 1) return launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
     return launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
@@ -392,8 +426,8 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
 // K > 4096: activations streamed beside the weights (one matrix, plain or residual epilogue)
 template <int T>
 static int launch_qd_xs(const QArgs& a, int M, hipStream_t s) {
-  constexpr int UB = DmaFmt<T>::UB, SU = 16;
-  constexpr int STAGE_BYTES = 2 * ((16 * (SU * UB / 16 + 1) + 63) / 64) * 1024;
+  constexpr int SU = 16;
+  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::slot_bytes(SU) / 16 + DmaFmt<T>::PAD) + 63) / 64) * 1024;
   const long long xt_bytes = (long long)QD_NW * (M > 8 ? 16 : 8) * QD_XT_PITCH;
   int nb = (int)((QD_LDS_CU - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024 - xt_bytes) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;
@@ -407,28 +441,33 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   using F = Fmt<T>;
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
-  if (a.K % (F::UW * 16) != 0) return -1;                                // whole slots of 16 units
-  if (a.K > 4 * F::UW * 16) {
-    if (a.nseg != 1 || a.epilogue > 1) return -1;
-    return launch_qd_xs<T>(a, M, s);
+  if constexpr (T == GGML_Q6_K) {                                        // slots of 32 units (8 superblocks = 1680 bytes: whole 16-byte pieces), K = 2048 or 4096
+    if (a.K % (F::UW * 32) != 0 || a.K > 2 * F::UW * 32) return -1;
+    return launch_qd_su<T, 32>(a, M, s);
+  } else {
+    if (a.K % (F::UW * 16) != 0) return -1;                              // whole slots of 16 units
+    if (a.K > 4 * F::UW * 16) {
+      if (a.nseg != 1 || a.epilogue > 1) return -1;
+      return launch_qd_xs<T>(a, M, s);
+    }
+    // Q4_0: slots of 32 units where K is whole in them (1152-byte runs, one stage per row group: 14336 x 4096 at M = 4 / 8 14.7 / 15.6 -> 13.5 / 14.4 us);
+    // Q8_0 keeps 16 (1088-byte runs already; with 32 the ring holds two stages only: 17.6 / 18.3 against 17.0 / 18.0 us)
+    if constexpr (T == F_Q4_0P) { if (a.K % (F::UW * 32) == 0) return launch_qd_su<T, 32>(a, M, s); }
+    return launch_qd_su<T, 16>(a, M, s);
   }
-  // Q4_0: slots of 32 units where K is whole in them (1152-byte runs, one stage per row group: 14336 x 4096 at M = 4 / 8 14.7 / 15.6 -> 13.5 / 14.4 us);
-  // Q8_0 keeps 16 (1088-byte runs already; with 32 the ring holds two stages only: 17.6 / 18.3 against 17.0 / 18.0 us)
-  if constexpr (T == F_Q4_0P) { if (a.K % (F::UW * 32) == 0) return launch_qd_su<T, 32>(a, M, s); }
-  return launch_qd_su<T, 16>(a, M, s);
 }
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
 // 3 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
-// 16 rows at a 16-byte aligned address.
+// 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (fmt != F_Q4_0P && fmt != F_Q8_0P) return -1;
+  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K) return -1;
   if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
-    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);
+    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : -1;
   }
   for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;
-  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : launch_qd<F_Q8_0P>(a, M, s);
+  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : launch_qd<GGML_Q6_K>(a, M, s);
 }
