@@ -133,6 +133,12 @@ int tga_qlinear_experts(int ggml_type, const void* w, const void* w_up, int64_t 
 int tga_qlinear_experts_routed(int ggml_type, const void* w_gate, const void* w_up, int64_t n_experts, const float* logits, int k,
                                int gating, int norm_topk_prob, float scale, int32_t* sel_out, float* probs_out,
                                const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
+/* The same for n_tokens tokens in one launch (the (B, T, k) selection of ExpertWeights.__call__, model.py:21-27, gated per token as model.py:112-128):
+ * jobs t k .. t k + k - 1 are token t's, gated from row t of logits (n_tokens, n_experts); x (n_tokens, K) fp16, y (n_tokens k, N),
+ * sel_out / probs_out (n_tokens, k). */
+int tga_qlinear_experts_routed_rows(int ggml_type, const void* w_gate, const void* w_up, int64_t n_experts, const float* logits, int n_tokens, int k,
+                                    int gating, int norm_topk_prob, float scale, int32_t* sel_out, float* probs_out,
+                                    const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream);
 
 /* Expert gating of FFNBlock._feed_forward (model.py:112-128): scores by ExpertGating (1 SOFTMAX, 2 SIGMOID, 3 SOFTMAX_WEIGHT,
  * 4 SQRT_SOFTPLUS; model.py:9-13), pairwise_topk selection (model.py:35-41: ascending, lower index wins ties), probabilities
@@ -203,6 +209,11 @@ int tga_advance_prompt(void* state, const int* prompt, void* stream);
 int tga_embed_rows(const void* table, int ggml_type, int dim, const int32_t* tokens, int n_rows, void* state, float* out, void* stream);
 /* tga_rmsnorm over `rows` rows of dim values (one workgroup per row); outputs (rows, dim). */
 int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream);
+/* tga_moe_combine followed by tga_rmsnorm_rows in one launch: every row of x is completed IN PLACE as x[t] + sum_s probs[t, s] * y[t, s, :] (the weighted
+ * sum over the selected experts' outputs and the block residual, tinygrad/llm/model.py:130, 150; the same sums in the same order as tga_moe_combine) and the
+ * next block's attn_norm - or output_norm - is taken of the completed row (nn.RMSNorm, tinygrad/nn/__init__.py:296-304).  y (rows, k, dim), probs (rows, k). */
+int tga_moe_combine_rmsnorm_rows(const float* y, const float* probs, float* x, const float* weight, int rows, int k, int dim, float eps, void* out_f16,
+                                 float* out_f32, void* stream);
 /* tga_attention_decode_normed for `batch` sequences at the shared position state.pos: q (batch, n_heads * head_dim), k / v (batch, n_kv_heads *
  * head_dim), caches (batch, n_kv_heads, max_ctx, head_dim) fp16, partials batch times the single-sequence workspace, outputs (batch, n_heads * head_dim). */
 int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,

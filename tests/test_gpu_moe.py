@@ -108,26 +108,28 @@ def test_weighted_expert_sum_folded_into_the_next_linear(gpu, t, dim, k):
   for f, q in zip(fused, plain): assert ol.rel_err(f.numpy(), q.numpy()) <= 2e-4
   with pytest.raises(RuntimeError): qlinear_multi(layers, xb, fused, norm=(nwb, 1e-5), combine=(yb, pb, 9, x_out))
 
+@pytest.mark.parametrize("T", [1, 3, 8])
 @pytest.mark.parametrize("t,dim,n,E,k,gating", [(39, 2048, 256, 64, 8, 1), (2, 512, 128, 8, 2, 3), (1, 1024, 96, 130, 6, 2), (12, 1024, 64, 16, 4, 4)])
-def test_expert_gate_up_that_gates_for_itself(gpu, t, dim, n, E, k, gating):
-  """tga_qlinear_experts_routed (scores, top-k and weights computed inside the expert gate/up launch from the router logits) against
-  tga_moe_gate followed by tga_qlinear_experts: identical selection and weights, identical outputs."""
+def test_expert_gate_up_that_gates_for_itself(gpu, t, dim, n, E, k, gating, T):
+  """tga_qlinear_experts_routed / _routed_rows (scores, top-k and weights computed inside the expert gate/up launch from the router logits, every
+  workgroup for its own token) against tga_moe_gate followed by tga_qlinear_experts: identical selection and weights, identical outputs, for
+  one token and for several tokens in one launch."""
   from tinygrad_amd.nn import ExpertWeights, moe_gate
-  rng = np.random.default_rng(dim + E + k)
+  rng = np.random.default_rng(dim + E + k + T)
   mk = (lambda: synth.random_blocks(rng, t, E * n, dim)) if t != 1 else (lambda: (rng.standard_normal((E * n, dim)) * dim ** -0.5).astype(np.float16).view(np.uint8).reshape(-1))
   ew, eu = ExpertWeights(gpu.Buffer.from_numpy(mk()), t, E, n, dim), ExpertWeights(gpu.Buffer.from_numpy(mk()), t, E, n, dim)
-  x = gpu.Buffer.from_numpy(synth.activations(rng, 1, dim, np.float16))
-  lg = gpu.Buffer.from_numpy(rng.standard_normal((1, E)).astype(np.float32))
-  sel0, p0, y0 = gpu.Buffer((k,), np.int32), gpu.Buffer((k,), np.float32), gpu.Buffer((k, n), np.float32)
-  moe_gate(lg, 1, E, k, sel0, p0, gating, True, 1.25)
+  x = gpu.Buffer.from_numpy(synth.activations(rng, T, dim, np.float16))
+  lg = gpu.Buffer.from_numpy(rng.standard_normal((T, E)).astype(np.float32))
+  sel0, p0, y0 = gpu.Buffer((T * k,), np.int32), gpu.Buffer((T * k,), np.float32), gpu.Buffer((T * k, n), np.float32)
+  moe_gate(lg, T, E, k, sel0, p0, gating, True, 1.25)
   ew(sel0, x, y0, jobs_per_x_row=k, up=eu)
-  sel1, p1, y1 = gpu.Buffer((k,), np.int32).zero_(), gpu.Buffer((k,), np.float32).zero_(), gpu.Buffer((k, n), np.float32).zero_()
+  sel1, p1, y1 = gpu.Buffer((T * k,), np.int32).zero_(), gpu.Buffer((T * k,), np.float32).zero_(), gpu.Buffer((T * k, n), np.float32).zero_()
   ew(sel1, x, y1, jobs_per_x_row=k, up=eu, route=(lg, gating, True, 1.25, p1))
   np.testing.assert_array_equal(sel1.numpy(), sel0.numpy())
   np.testing.assert_array_equal(p1.numpy(), p0.numpy())
   np.testing.assert_array_equal(y1.numpy(), y0.numpy())
   rs, rp = omoe.gate_probs(lg.numpy(), k, gating, True, 1.25)
-  np.testing.assert_array_equal(sel1.numpy(), rs[0])
+  np.testing.assert_array_equal(sel1.numpy().reshape(T, k), rs)
 
 def test_moe_combine(gpu):
   from tinygrad_amd.nn import moe_combine
@@ -137,6 +139,30 @@ def test_moe_combine(gpu):
   out = gpu.Buffer((T, D), np.float32)
   moe_combine(gpu.Buffer.from_numpy(y), gpu.Buffer.from_numpy(p), gpu.Buffer.from_numpy(r), T, k, D, out)
   np.testing.assert_allclose(out.numpy(), r + (y * p[:, :, None]).sum(1), rtol=1e-5, atol=1e-5)
+
+@pytest.mark.parametrize("T,k,D", [(3, 8, 2048), (8, 2, 256), (16, 8, 4096), (2, 3, 6152)])
+def test_moe_combine_folded_into_the_next_norm(gpu, T, k, D):
+  """tga_moe_combine_rmsnorm_rows against tga_moe_combine followed by tga_rmsnorm_rows: the completed rows and both norm outputs bit for bit (rows of up to
+  2048 values stay in registers, longer ones are read back by the thread that completed them), and the rows against numpy."""
+  from tinygrad_amd.nn import moe_combine
+  L = gpu.lib()
+  rng = np.random.default_rng(T + k + D)
+  y, p = rng.standard_normal((T, k, D)).astype(np.float32), rng.random((T, k)).astype(np.float32)
+  r, w = rng.standard_normal((T, D)).astype(np.float32), (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+  yb, pb, wb = gpu.Buffer.from_numpy(y), gpu.Buffer.from_numpy(p), gpu.Buffer.from_numpy(w)
+  x0, h0, f0 = gpu.Buffer.from_numpy(r), gpu.Buffer((T, D), np.float16), gpu.Buffer((T, D), np.float32)
+  moe_combine(yb, pb, x0, T, k, D, x0)
+  gpu.check(L.tga_rmsnorm_rows(x0.ptr, wb.ptr, T, D, 1e-5, h0.ptr, f0.ptr, 0, None))
+  x1, h1, f1 = gpu.Buffer.from_numpy(r), gpu.Buffer((T, D), np.float16), gpu.Buffer((T, D), np.float32)
+  for b in (h1, f1): gpu.check(L.tga_memset(b.ptr, 0xFF, b.nbytes, None))
+  gpu.check(L.tga_moe_combine_rmsnorm_rows(yb.ptr, pb.ptr, x1.ptr, wb.ptr, T, k, D, 1e-5, h1.ptr, f1.ptr, None))
+  np.testing.assert_array_equal(x1.numpy(), x0.numpy())
+  np.testing.assert_array_equal(f1.numpy(), f0.numpy())
+  assert h1.numpy().tobytes() == h0.numpy().tobytes()
+  full = r + (y * p[:, :, None]).sum(1)
+  np.testing.assert_allclose(x1.numpy(), full, rtol=1e-5, atol=1e-5)
+  ref = full / np.sqrt((full.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-5) * w
+  np.testing.assert_allclose(f1.numpy(), ref, rtol=2e-5, atol=2e-5)
 
 SMALL_MOE = dict(num_blocks=2, dim=256, hidden_dim=128, n_heads=4, n_kv_heads=4, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,
                  qk_norm=256, num_experts=8, num_experts_per_tok=2, norm_topk_prob=False, expert_gating_func=1)

@@ -47,22 +47,44 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 // ---------------------------------------------------------------------------------------------- RMSNorm
 // nn.RMSNorm (tinygrad/nn/__init__.py:296-304): x * rsqrt(mean(x^2) + eps), then * weight.  Output fp16 (the activation the
 // dequant-GEMV multiplies) and optionally fp32.
-__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, int dim, float eps,
-                                                       _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu) {
+// COMB: the row is first completed in place as x + sum_j probs[row, j] * y[row, j, :] (the weighted sum over the selected experts' outputs plus the block
+// residual, tinygrad/llm/model.py:130, 150) - the same expression, in the same order, as moe_combine_kernel - and the norm is taken of the completed row.
+template <bool COMB>
+__global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* x, const float* __restrict__ w, int dim, float eps,
+                                                       _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu,
+                                                       float* x_rw, const float* __restrict__ y, const float* __restrict__ probs, int k) {
   __shared__ float red[16];
-  x += (size_t)blockIdx.x * dim;                        // one workgroup per row
-  if (out16) out16 += (size_t)blockIdx.x * dim;
-  if (out32) out32 += (size_t)blockIdx.x * dim;
+  const int row = blockIdx.x;                           // one workgroup per row
+  x += (size_t)row * dim;
+  if (out16) out16 += (size_t)row * dim;
+  if (out32) out32 += (size_t)row * dim;
+  auto value = [&](int e) {                             // element e of the (completed) row; COMB: also written back (read again below only by the thread that wrote it)
+    float a = x[e];
+    if constexpr (COMB) {
+      for (int j0 = 0; j0 < k; j0 += 8) {               // eight experts' values requested together, added in order
+        float yy[8], pp[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) { const int j = j0 + i < k ? j0 + i : k - 1; pp[i] = probs[(size_t)row * k + j]; yy[i] = y[((size_t)row * k + j) * dim + e]; }
+#pragma unroll
+        for (int i = 0; i < 8; i++) if (j0 + i < k) a += pp[i] * yy[i];
+      }
+      x_rw[(size_t)row * dim + e] = a;
+    }
+    return a;
+  };
   // two elements per thread and loop pass are requested together and kept for the second pass (rows up to 2048 values never reload)
   float s = 0.f, v0 = 0.f, v1 = 0.f, w0 = 0.f, w1 = 0.f;
   const int e0 = threadIdx.x, e1 = threadIdx.x + 1024;
-  if (e0 < dim) { v0 = x[e0]; w0 = w[e0]; }
-  if (e1 < dim) { v1 = x[e1]; w1 = w[e1]; }
+  if (e0 < dim) { v0 = value(e0); w0 = w[e0]; }
+  if (e1 < dim) { v1 = value(e1); w1 = w[e1]; }
   s = v0 * v0 + v1 * v1;
   for (int b = threadIdx.x + 2048; b < dim; b += 4096) {
     float t[4];
 #pragma unroll
-    for (int j = 0; j < 4; j++) t[j] = x[b + 1024 * j < dim ? b + 1024 * j : dim - 1];
+    for (int j = 0; j < 4; j++) {
+      if constexpr (COMB) t[j] = b + 1024 * j < dim ? value(b + 1024 * j) : 0.f;      // (an element is completed exactly once)
+      else t[j] = value(b + 1024 * j < dim ? b + 1024 * j : dim - 1);
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) if (b + 1024 * j < dim) s += t[j] * t[j];
   }
@@ -589,7 +611,15 @@ int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, flo
   TGA_REQUIRE(dim > 0 && rows >= 1, "tga_rmsnorm: rows=%d dim=%d", rows, dim);
   int sfmt = 0, snu = 0;
   if (stage_type) { sfmt = decode_staged_fmt(stage_type, dim, &snu); TGA_REQUIRE(sfmt >= 0, "tga_rmsnorm: no staged layout for type %d with K=%d", stage_type, dim); }
-  rmsnorm_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu);
+  rmsnorm_kernel<false><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu, nullptr, nullptr, nullptr, 0);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+int tga_moe_combine_rmsnorm_rows(const float* y, const float* probs, float* x, const float* weight, int rows, int k, int dim, float eps, void* out_f16, float* out_f32,
+                                 void* stream) {
+  TGA_REQUIRE(y && probs && x && weight && (out_f16 || out_f32), "tga_moe_combine_rmsnorm_rows: null pointer");
+  TGA_REQUIRE(dim > 0 && rows >= 1 && k >= 1, "tga_moe_combine_rmsnorm_rows: rows=%d k=%d dim=%d", rows, k, dim);
+  rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k);
   TGA_LAUNCH_CHECK();
   return 0;
 }

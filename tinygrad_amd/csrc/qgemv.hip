@@ -535,3 +535,16 @@ extern "C" int tga_qlinear_experts_routed(int ggml_type, const void* w_gate, con
   const RouteIn r = {logits, k, gating, norm_topk_prob, scale, probs_out};
   return qlinear_experts_impl(&r, ggml_type, w_gate, w_up, n_experts, sel_out, k, k, x_f16, TGA_F16, y, y_dtype, N, K, stream);
 }
+
+// The same for n_tokens tokens in one launch (ExpertWeights.__call__ over a (B, T, k) selection, model.py:21-27): jobs t k .. t k + k - 1 are token t's,
+// gated from row t of the logits; x (n_tokens, K) fp16, y (n_tokens k, N), sel_out / probs_out (n_tokens, k).
+extern "C" int tga_qlinear_experts_routed_rows(int ggml_type, const void* w_gate, const void* w_up, int64_t n_experts, const float* logits, int n_tokens, int k,
+                                               int gating, int norm_topk_prob, float scale, int32_t* sel_out, float* probs_out,
+                                               const void* x_f16, void* y, int y_dtype, int64_t N, int64_t K, void* stream) {
+  TGA_REQUIRE(logits && sel_out && probs_out && w_up, "tga_qlinear_experts_routed_rows: null pointer");
+  TGA_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= 1024 && k >= 1 && k <= 64 && k <= n_experts, "tga_qlinear_experts_routed_rows: bad geometry (k <= 64, n_experts <= 1024)");
+  TGA_REQUIRE((long long)n_tokens * k <= 65535, "tga_qlinear_experts_routed_rows: %d x %d jobs exceed one launch", n_tokens, k);
+  TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_qlinear_experts_routed_rows: unknown ExpertGating %d", gating);
+  const RouteIn r = {logits, k, gating, norm_topk_prob, scale, probs_out};
+  return qlinear_experts_impl(&r, ggml_type, w_gate, w_up, n_experts, sel_out, n_tokens * k, k, x_f16, TGA_F16, y, y_dtype, N, K, stream);
+}

@@ -332,13 +332,17 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     u32x4 v[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) v[t] = xh[(int)threadIdx.x + NT * t < nq ? (int)threadIdx.x + NT * t : nq - 1];
-    for (int i = threadIdx.x; i < a.route_E; i += NT) tk_lg[i] = a.route_logits[i];
+    // jobs xrow * k .. xrow * k + k - 1 belong to token xrow: every workgroup gates its own token
+    const int slot = job - (int)xrow * a.route_k;
+    for (int i = threadIdx.x; i < a.route_E; i += NT) tk_lg[i] = a.route_logits[xrow * a.route_E + i];
     __syncthreads();
     if (wave == 0) gate_topk_wave(tk_lg, a.route_E, a.route_k, a.route_gating, a.route_norm_topk, a.route_scale, tk_sel, tk_p, tk_sc, tk_tmp, lane);
     __syncthreads();
-    eoff = (long long)tk_sel[job] * a.estride;
+    eoff = (long long)tk_sel[slot] * a.estride;
     enter(0);                                                    // the weight bases of the selected expert
-    if (blockIdx.x == 0 && job == 0 && (int)threadIdx.x < a.route_k) { a.sel[threadIdx.x] = tk_sel[threadIdx.x]; a.route_probs_out[threadIdx.x] = tk_p[threadIdx.x]; }
+    if (blockIdx.x == 0 && slot == 0 && (int)threadIdx.x < a.route_k) {
+      a.sel[xrow * a.route_k + threadIdx.x] = tk_sel[threadIdx.x]; a.route_probs_out[xrow * a.route_k + threadIdx.x] = tk_p[threadIdx.x];
+    }
     issue(b[0], lo);
 #pragma unroll
     for (int t = 0; t < 2; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
@@ -470,7 +474,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
   if (a.comb_y) return tga_set_error("tga_moe_combine_rmsnorm_qlinear_multi: shape outside the fused path (K = %d)", a.K);
   if constexpr (WK == 1 && EPI == 2) {
     if (a.route_logits) {
-      if (a.x_staged || a.norm_w || a.x_f32 || !one_batch || a.xdiv != a.xdiv_jobs) return tga_set_error("tga_qlinear_experts_routed: needs one fp16 row of at most %d values", 16 * NT);
+      if (a.x_staged || a.norm_w || a.x_f32 || !one_batch || a.xdiv != a.route_k || a.xdiv_jobs % a.route_k != 0) return tga_set_error("tga_qlinear_experts_routed: needs fp16 rows of at most %d values and k jobs per row", 16 * NT);
       return launch_fast_p<T, R, WK, WR, EPI, H, 6>(a, grid, lds, s);
     }
   }

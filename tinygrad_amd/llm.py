@@ -600,9 +600,17 @@ class BatchedTransformer:
   def _step(self, with_head: bool):
     c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_rows(self.token_embd.ptr, self.embd_type, c.dim, self.tokens.ptr, B, self.state.ptr, self.x.ptr, st))
+    # The weighted sum over a block's selected experts plus its residual (model.py:130, 150) is completed by the NEXT norm's launch (the next block's attn_norm
+    # or output_norm): `pending` says that x still lacks it.
+    pending = False
+    def norm(weight):
+      nonlocal pending
+      if pending: rt.check(L.tga_moe_combine_rmsnorm_rows(self.y_e.ptr, self.probs.ptr, self.x.ptr, weight.ptr, B, c.num_experts_per_tok, c.dim, c.norm_eps, self.xn.ptr, None, st))
+      else: rt.check(L.tga_rmsnorm_rows(self.x.ptr, weight.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      pending = False
     for b in self.blk:
       # h = x + attention(attn_norm(x))                                                   model.py:149
-      rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["attn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      norm(b["attn_norm"])
       qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
       while i < 3:                                                     # one launch per run of equal block types
         j = i + 1
@@ -623,14 +631,18 @@ class BatchedTransformer:
         continue
       k = c.num_experts_per_tok                                         # model.py:110-135
       b["router"](self.xn, out=self.router_logits, stream=st)
-      moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st, bias=b["sel_bias"])
+      self_gated = self.expert_path != "grouped" and b["sel_bias"] is None and self.xn.dtype == np.float16 and c.dim <= 4096   # the gate/up launch gates for itself (as the batch-1 step does)
+      if not self_gated:
+        moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st, bias=b["sel_bias"])
       if self.expert_path == "grouped":                                # one small-batch GEMM per selected expert (its weights read once by the kernel)
         expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
         experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
         experts_grouped(b["down_exps"], self.job_table, B * k, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
       else:                                                              # one GEMV per (sequence, slot) job; an expert picked twice is read twice, the second time from cache
-        b["gate_exps"](self.sel, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
+        route = (self.router_logits, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, self.probs) if self_gated else None
+        b["gate_exps"](self.sel, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st, route=route)
         b["down_exps"](self.sel, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
+      if not c.shared_expert_dim: pending = True; continue            # x + sum_j p_j y_j: left to the next norm's launch
       moe_combine(self.y_e, self.probs, self.x, B, k, c.dim, self.x, stream=st)
       if c.shared_expert_dim:                                            # + shared expert, each row scaled by 1 or by sigmoid(xn . ffn_gate_inp_shexp)
         self._linear([b["ffn_gate_shexp"], b["ffn_up_shexp"]], self.xn, [self.act_sh], epilogue=2)
@@ -640,8 +652,10 @@ class BatchedTransformer:
           moe_gate(self.sh_logit, B, 1, 1, self.sh_sel, self.p_sh, 2, False, 1.0, stream=st)
         moe_combine(self.y_sh, self.p_sh, self.x, B, 1, c.dim, self.x, stream=st)
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
-      rt.check(L.tga_rmsnorm_rows(self.x.ptr, self.output_norm.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      norm(self.output_norm)
       self.output(self.xn, out=self.logits_buf, stream=st)
+    elif pending:                                                        # (a prompt step ends with the last block: nothing reads x afterwards, but keep it whole)
+      moe_combine(self.y_e, self.probs, self.x, B, c.num_experts_per_tok, c.dim, self.x, stream=st)
     if self.chunked:                                                     # the next B prompt tokens, B positions on
       rt.check(L.tga_chunk_advance(self.state.ptr, self.prompts.ptr, B, self.tokens.ptr, c.max_context, st))
       return

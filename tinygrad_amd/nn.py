@@ -82,13 +82,18 @@ class ExpertWeights:
 
   def __call__(self, sel: Buffer, x: Buffer, out: Buffer, jobs_per_x_row: int = 1, up: "ExpertWeights | None" = None, stream=None,
                route: tuple[Buffer, int, bool, float, Buffer] | None = None) -> Buffer:
-    """route = (logits, gating, norm_topk_prob, scale, probs_out) with `up`: the jobs of one token, gated inside the launch from the router
-    logits; sel (k entries) and probs_out receive the selection."""
+    """route = (logits, gating, norm_topk_prob, scale, probs_out) with `up`: the jobs are gated inside the launch from the router logits (one row per
+    token, jobs_per_x_row = k jobs each); sel and probs_out receive the selection."""
     n_jobs = int(np.prod(sel.shape))
     if route is not None:
-      assert up is not None and x.dtype == np.float16 and jobs_per_x_row == n_jobs
-      rt.check(rt.lib().tga_qlinear_experts_routed(self.ggml_type, self.blocks.ptr, up.blocks.ptr, self.num_experts, route[0].ptr, n_jobs, route[1], int(route[2]),
-                                                   route[3], sel.ptr, route[4].ptr, x.ptr, out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
+      assert up is not None and x.dtype == np.float16 and n_jobs % jobs_per_x_row == 0
+      if jobs_per_x_row == n_jobs:
+        rt.check(rt.lib().tga_qlinear_experts_routed(self.ggml_type, self.blocks.ptr, up.blocks.ptr, self.num_experts, route[0].ptr, n_jobs, route[1], int(route[2]),
+                                                     route[3], sel.ptr, route[4].ptr, x.ptr, out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))
+      else:                                                              # several tokens: jobs_per_x_row = k jobs each, gated from their own row of the logits
+        rt.check(rt.lib().tga_qlinear_experts_routed_rows(self.ggml_type, self.blocks.ptr, up.blocks.ptr, self.num_experts, route[0].ptr, n_jobs // jobs_per_x_row,
+                                                          jobs_per_x_row, route[1], int(route[2]), route[3], sel.ptr, route[4].ptr, x.ptr, out.ptr, rt.dtype_code(out.dtype),
+                                                          self.out_features, self.in_features, stream))
       return out
     rt.check(rt.lib().tga_qlinear_experts(self.ggml_type, self.blocks.ptr, up.blocks.ptr if up is not None else None, self.num_experts, sel.ptr, n_jobs,
                                           jobs_per_x_row, x.ptr, rt.dtype_code(x.dtype), out.ptr, rt.dtype_code(out.dtype), self.out_features, self.in_features, stream))

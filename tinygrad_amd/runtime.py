@@ -41,6 +41,7 @@ def _declare(lib):
     "tga_stage_activation": [i, vp, i, i64, vp, vp],
     "tga_qlinear_experts": [i, vp, vp, i64, vp, i, i, vp, i, vp, i, i64, i64, vp],
     "tga_qlinear_experts_routed": [i, vp, vp, i64, vp, i, i, i, ctypes.c_float, vp, vp, vp, vp, i, i64, i64, vp],
+    "tga_qlinear_experts_routed_rows": [i, vp, vp, i64, vp, i, i, i, i, ctypes.c_float, vp, vp, vp, vp, i, i64, i64, vp],
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_gate_biased": [vp, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
@@ -60,6 +61,7 @@ def _declare(lib):
     "tga_add_expert_bias": [vp, vp, vp, i64, i64, i, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
     "tga_embed_rows": [vp, i, i, vp, i, vp, vp, vp], "tga_rmsnorm_rows": [vp, vp, i, i, ctypes.c_float, vp, vp, i, vp],
+    "tga_moe_combine_rmsnorm_rows": [vp, vp, vp, vp, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_attention_decode_batched": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
     "tga_attention_prefill_chunk": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
     "tga_chunk_advance": [vp, vp, i, vp, i, vp],
