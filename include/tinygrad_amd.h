@@ -158,6 +158,10 @@ int tga_moe_gate_biased(const float* logits, const float* selection_bias, int n_
  * k = 0: logits only (sel / probs may be NULL, the counter is not touched): for a consumer that gates for itself (tga_qlinear_experts_routed). */
 int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int dim, int n_experts, int k,
                    int gating, int norm_topk_prob, float scale, void* xn_out_f16, float* logits_ws, int32_t* sel, float* probs, void* stream);
+/* tga_moe_router with k = 0 over `rows` tokens in one launch: xn (rows, dim) fp16 = ffn_norm(x) (model.py:150) and logits (rows, n_experts) = xn . router^T
+ * (ffn_gate_inp, model.py:112); the gating is left to the consumer (tga_qlinear_experts_routed_rows or tga_moe_gate). */
+int tga_moe_router_rows(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int rows, int dim, int n_experts,
+                        void* xn_out_f16, float* logits, void* stream);
 /* out[t] = resid[t] + sum_s probs[t, s] * y[t, s, :]  (model.py:130 and the residual add :150); resid may be NULL or alias out. */
 int tga_moe_combine(const float* y, const float* probs, const float* resid, int n_tokens, int k, int dim, float* out, void* stream);
 

@@ -82,6 +82,27 @@ def test_router_in_one_launch(gpu, dim, E, k, gating, normw):
   np.testing.assert_array_equal(sel.numpy(), rs[0])
   np.testing.assert_allclose(pr.numpy(), rp[0], rtol=2e-5, atol=1e-7)
 
+@pytest.mark.parametrize("T,dim,E", [(1, 2048, 64), (5, 2048, 64), (8, 256, 8), (3, 1024, 130)])
+def test_router_logits_for_several_tokens(gpu, T, dim, E):
+  """tga_moe_router_rows (ffn_norm + router logits of T tokens in one launch) against the single-token launch row by row: same fp16 rows, same logits, bit
+  for bit; and the logits against float64."""
+  from tinygrad_amd import runtime as rt
+  L = gpu.lib()
+  rng = np.random.default_rng(T + dim + E)
+  x = (rng.standard_normal((T, dim)) * 2).astype(np.float32); nw = rng.standard_normal(dim).astype(np.float32)
+  wr = (rng.standard_normal((E, dim)) * dim ** -0.5).astype(np.float16)
+  xb, nb, wb = gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw), gpu.Buffer.from_numpy(wr)
+  xn, lg = gpu.Buffer((T, dim), np.float16), gpu.Buffer((T, E), np.float32)
+  for b in (xn, lg): gpu.check(L.tga_memset(b.ptr, 0xFF, b.nbytes, None))
+  gpu.check(L.tga_moe_router_rows(xb.ptr, nb.ptr, 1e-5, wb.ptr, T, dim, E, xn.ptr, lg.ptr, None))
+  for t in range(T):
+    xn1, lg1 = gpu.Buffer((dim,), np.float16), gpu.Buffer((E + 1,), np.float32).zero_()
+    gpu.check(L.tga_moe_router(xb.ptr + 4 * t * dim, nb.ptr, 1e-5, wb.ptr, dim, E, 0, 1, 0, 1.0, xn1.ptr, lg1.ptr, None, None, None))
+    assert xn.numpy()[t].tobytes() == xn1.numpy().tobytes()
+    np.testing.assert_array_equal(lg.numpy()[t], lg1.numpy()[:E])
+  ref = xn.numpy().astype(np.float64) @ wr.astype(np.float64).T
+  assert ol.rel_err(lg.numpy(), ref.astype(np.float32)) <= 1e-3
+
 @pytest.mark.parametrize("t,dim,k", [(1, 2048, 8), (2, 1024, 4), (14, 512, 1), (39, 2048, 6)])
 def test_weighted_expert_sum_folded_into_the_next_linear(gpu, t, dim, k):
   """tga_moe_combine_rmsnorm_qlinear_multi against tga_moe_combine followed by tga_rmsnorm_qlinear_multi: same completed row (bit for

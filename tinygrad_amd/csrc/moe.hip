@@ -30,6 +30,9 @@ __global__ __launch_bounds__(ROUTER_THREADS) void moe_router_kernel(const float*
   __shared__ float tmp[192];
   __shared__ int last_flag;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // blockIdx.y: the token (logits-only launches over several rows: tga_moe_router_rows)
+  x += (size_t)blockIdx.y * dim; logits_ws += (size_t)blockIdx.y * n_experts;
+  if (xn_out) xn_out += (size_t)blockIdx.y * dim;
   const int row = blockIdx.x * 4 + wave, rowc = row < n_experts ? row : n_experts - 1;
   const int np = dim / 8;                               // 16-byte pieces per row
   const _Float16* wrow = wr + (size_t)rowc * dim;
@@ -153,6 +156,19 @@ int tga_moe_router(const float* x, const float* norm_weight, float norm_eps, con
   TGA_REQUIRE(gating >= 1 && gating <= 4, "tga_moe_router: unknown ExpertGating %d", gating);
   moe_router_kernel<<<(n_experts + 3) / 4, ROUTER_THREADS, 2 * n_experts * sizeof(float) + (size_t)dim * 2, (hipStream_t)stream>>>(
       x, norm_weight, norm_eps, (const _Float16*)router_w_f16, dim, n_experts, k, gating, norm_topk_prob, scale, (_Float16*)xn_out_f16, logits_ws, sel, probs);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+
+int tga_moe_router_rows(const float* x, const float* norm_weight, float norm_eps, const void* router_w_f16, int rows, int dim, int n_experts,
+                        void* xn_out_f16, float* logits, void* stream) {
+  TGA_REQUIRE(x && router_w_f16 && logits, "tga_moe_router_rows: null pointer");
+  TGA_REQUIRE(rows >= 1 && rows <= 65535 && dim >= 8 && dim % 8 == 0 && dim <= 16384 && ((uintptr_t)router_w_f16 & 15) == 0,
+              "tga_moe_router_rows: rows=%d, dim=%d must be a multiple of 8, at most 16384, with a 16-byte aligned weight", rows, dim);
+  TGA_REQUIRE((((uintptr_t)x | (uintptr_t)norm_weight | (uintptr_t)xn_out_f16) & 15) == 0, "tga_moe_router_rows: x, norm_weight and xn_out must be 16-byte aligned");
+  TGA_REQUIRE(n_experts >= 1 && n_experts <= 1024, "tga_moe_router_rows: n_experts <= 1024");
+  moe_router_kernel<<<dim3((n_experts + 3) / 4, rows), ROUTER_THREADS, 2 * n_experts * sizeof(float) + (size_t)dim * 2, (hipStream_t)stream>>>(
+      x, norm_weight, norm_eps, (const _Float16*)router_w_f16, dim, n_experts, 0, 1, 0, 1.f, (_Float16*)xn_out_f16, logits, nullptr, nullptr);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -624,13 +624,17 @@ class BatchedTransformer:
                          c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn.ptr, None, st))
       self._linear([b["attn_output"]], self.attn, [self.x], epilogue=1, resid=[self.x])
       # x = h + feed_forward(ffn_norm(h))                                                   model.py:150
-      rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+      fused_router = b["moe"] and b["router"].ggml_type == rt.F16 and c.dim % 8 == 0 and c.num_experts <= 1024   # ffn_norm and the router logits in one launch (as the batch-1 step)
+      if fused_router:
+        rt.check(L.tga_moe_router_rows(self.x.ptr, b["ffn_norm"].ptr, c.norm_eps, b["router"].blocks.ptr, B, c.dim, c.num_experts, self.xn.ptr, self.router_logits.ptr, st))
+      else:
+        rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       if not b["moe"]:
         self._linear([b["ffn_gate"], b["ffn_up"]], self.xn, [self.act], epilogue=2)
         self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
         continue
       k = c.num_experts_per_tok                                         # model.py:110-135
-      b["router"](self.xn, out=self.router_logits, stream=st)
+      if not fused_router: b["router"](self.xn, out=self.router_logits, stream=st)
       self_gated = self.expert_path != "grouped" and b["sel_bias"] is None and self.xn.dtype == np.float16 and c.dim <= 4096   # the gate/up launch gates for itself (as the batch-1 step does)
       if not self_gated:
         moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st, bias=b["sel_bias"])

@@ -45,6 +45,7 @@ def _declare(lib):
     "tga_moe_gate": [vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_gate_biased": [vp, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_moe_combine": [vp, vp, vp, i, i, i, vp, vp],
+    "tga_moe_router_rows": [vp, vp, ctypes.c_float, vp, i, i, i, vp, vp, vp],
     "tga_moe_router": [vp, vp, ctypes.c_float, vp, i, i, i, i, i, ctypes.c_float, vp, vp, vp, vp, vp],
     "tga_quantize_mxfp8": [vp, i, i64, i64, vp, vp, vp, vp],
     "tga_silu_mul_quantize_mxfp8": [vp, vp, i64, i64, vp, vp, vp, vp],
