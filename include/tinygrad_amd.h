@@ -104,6 +104,12 @@ int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml
                               const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
                               int y_stage_type, int64_t y_stage_K, void* stream);
 
+/* The same for M rows (batched decode steps and prefill chunks): x (M, K) float32 BEFORE the norm.  One launch where the LDS-fed small-batch kernel applies
+ * (Q4_0 / Q8_0 / Q6_K, 3 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
+ * tga_qlinear_multi on it.  xn_scratch_f16 is clobbered or left untouched accordingly. */
+int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                             const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream);
+
 /* tga_rmsnorm_qlinear_multi on the row x_in + sum_j probs[j] * y_experts[j]: the MoE weighted sum over the selected experts' outputs and
  * the block residual (tinygrad/llm/model.py:130, 150) folded into the next block's attn_norm -> attn_q/k/v launch (or output_norm -> output).
  * The completed row is written to x_out, which must not alias x_in.  y_experts (k, K) and probs (k) float32, k <= 8, K <= 2048, plain epilogue. */

@@ -280,6 +280,39 @@ def test_small_batch_q6_k_through_lds(gpu, n, k, m):
   qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
   assert ol.rel_err(rb.numpy(), res + ref) <= TOL
 
+@pytest.mark.parametrize("t,k,ns,m,epi", [(2, 4096, [512, 128, 128], 16, 0), (2, 2048, [256, 64, 64], 5, 0), (8, 4096, [1024, 1024], 8, 2), (2, 4096, [448, 448], 3, 2),
+                                            (14, 4096, [272], 4, 0), (8, 1024, [64], 16, 0), (12, 4096, [256, 64, 64], 6, 0), (2, 8192, [128], 8, 0), (2, 4096, [200], 2, 0)])
+def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
+  """tga_rmsnorm_qlinear_rows (the RMSNorm in front of q/k/v or gate/up folded into the LDS-fed small-batch kernel's prologue) against tga_rmsnorm_rows
+  followed by tga_qlinear_multi, and against the float64 anchor of the normalised fp16 rows.  The last cases are outside the kernel that folds the norm
+  (Q4_K, K beyond 4096, two rows, more than eight rows): there the call IS the two launches, bit for bit."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  L = gpu.lib()
+  rng = np.random.default_rng(sum(ns) + k + m + t)
+  ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+  layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
+  x = (rng.standard_normal((m, k)) * np.exp(rng.standard_normal((m, 1)))).astype(np.float32)       # rows of different magnitudes
+  nw = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+  xb, nb = gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw)
+  nout = 1 if epi == 2 else len(ns)
+  xn0 = gpu.Buffer((m, k), np.float16)
+  gpu.check(L.tga_rmsnorm_rows(xb.ptr, nb.ptr, m, k, 1e-5, xn0.ptr, None, 0, None))
+  o0 = [gpu.Buffer((m, ns[i]), np.float32) for i in range(nout)]
+  qlinear_multi(layers, xn0, o0, epilogue=epi)
+  o1 = [gpu.Buffer((m, ns[i]), np.float32) for i in range(nout)]
+  for o in o1: gpu.check(L.tga_memset(o.ptr, 0xFF, o.nbytes, None))
+  scratch = gpu.Buffer((m, k), np.float16)
+  gpu.check(L.tga_memset(scratch.ptr, 0xFF, scratch.nbytes, None))
+  qlinear_multi(layers, xb, o1, epilogue=epi, norm=(nb, 1e-5, scratch))
+  folded = t in (2, 8, 14) and k <= 4096 and 3 <= m <= 8 and all(n % (8 if epi == 2 else 16) == 0 for n in ns)
+  assert (scratch.numpy().view(np.uint16) == 0xFFFF).all() == folded       # one launch: the scratch rows were not needed
+  h = xn0.numpy().astype(np.float32)
+  refs = [ol.linear_f64(h, ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]
+  if epi == 2: refs = [refs[0] / (1 + np.exp(-refs[0])) * refs[1]]
+  for a, b, ref in zip(o1, o0, refs):
+    if folded: assert ol.rel_err(a.numpy(), b.numpy()) <= 2e-4 and ol.rel_err(a.numpy(), ref) <= TOL      # the sum of squares is associated differently: an fp16 value may round the other way
+    else: np.testing.assert_array_equal(a.numpy(), b.numpy())
+
 def test_sixteen_rows_segments_residual_and_swiglu(gpu):
   """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

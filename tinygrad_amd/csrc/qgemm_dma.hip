@@ -227,12 +227,13 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     // of row c rotated by c so that writes and reads are free of bank conflicts.
     constexpr int NST = NSS * SPW;
     char* xb = ring + (size_t)(nb - 1) * (2 * SLOT_BYTES) + (size_t)wave * 8192;
-    bool have[NST]; int uc[NST];
+    bool have[NST], stepok[NST]; int uc[NST];
 #pragma unroll
     for (int ss = 0; ss < NST; ss++) {
       const int u0 = (2 * (ss / SPW) + half) * QD_SU + 4 * (step + 4 * (ss % SPW));
       have[ss] = r < M && u0 + g < cu;
-      uc[ss] = u0 + 3 < cu ? u0 : cu - 4;                // (K is whole slots of at least 16 units)
+      stepok[ss] = u0 + 3 < cu;                          // the step's four units exist (over all waves and steps every unit of a row exactly once)
+      uc[ss] = stepok[ss] ? u0 : cu - 4;                 // (K is whole slots of at least 16 units)
     }
     // The requests are inline assembly and the wait is counted by hand: a compiler-placed wait would also cover the weight pieces issued behind
     // them (it cannot count those), i.e. the operands would be formed only after the first stages have landed.  Requests, wait and the writes to
@@ -240,9 +241,14 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     // matrix at sixteen rows): a request behind a condition would give the compiler a reason to move the pieces between registers while they
     // are on their way (it takes them for present as soon as the request is issued).
     const int mine = (NI2 - wave + QD_NW - 1) / QD_NW;   // this wave's pieces per stage
-    auto prologue = [&](auto rows_tag, auto f32_tag) __attribute__((always_inline)) {
+    // NORM (float32 rows): the rows are RMS-normalised on the way (nn.RMSNorm, tinygrad/nn/__init__.py:296-304: x * rsqrt(mean(x^2) + eps) * weight, the
+    // attn_norm / ffn_norm in front of q/k/v and gate/up, tinygrad/llm/model.py:149-150): every wave sums the squares of the 256 values per row that its
+    // steps hold, the eight waves' sums meet in LDS (one more barrier), and the values are scaled before they are rounded to fp16.
+    auto prologue = [&](auto rows_tag, auto f32_tag, auto norm_tag) __attribute__((always_inline)) {
       constexpr int XR = decltype(rows_tag)::value;      // rows requested (rows at and beyond M repeat row 0 and are dropped)
       constexpr bool F32 = decltype(f32_tag)::value;
+      constexpr bool NORM = decltype(norm_tag)::value;
+      static_assert(!NORM || F32, "the folded norm reads float32 rows");
       constexpr int NV = F32 ? XR : XR / 2;              // float32: instruction v = row v, lane l = values 4 l .. 4 l + 3; fp16: rows 2 v and 2 v + 1, lane l = piece l & 31 of row 2 v + (l >> 5)
       u32x4 xq[NST][NV];
 #pragma unroll
@@ -254,9 +260,43 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
                                 : (const char*)((const uint16_t*)a.x + (long long)(row < M ? row : 0) * a.K + 64 * uc[ss] + 8 * (lane & 31));
           asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xq[ss][v]) : "v"(ptr) : "memory");
         }
+      u32x4 nwq[NORM ? NST : 1];                         // the norm weight of the step's columns (this lane: 4 values)
+      if constexpr (NORM) {
+#pragma unroll
+        for (int ss = 0; ss < NST; ss++) { const float* ptr = a.norm_w + 64 * uc[ss] + 4 * lane; asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(nwq[ss]) : "v"(ptr) : "memory"); }
+      }
       int issued = 0;
       for (int k = 0; k < nb - 1; k++) if (k < S) { issue_stage(); issued++; }
       qd_wait_vm(issued * mine);
+      float sc[NORM ? NV : 1];
+      if constexpr (NORM) {
+#pragma unroll
+        for (int ss = 0; ss < NST; ss++) {
+          asm volatile("" : "+v"(nwq[ss]) :: "memory");
+#pragma unroll
+          for (int v = 0; v < NV; v++) asm volatile("" : "+v"(xq[ss][v]) :: "memory");
+        }
+        float ps[NV];
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+          ps[v] = 0.f;
+#pragma unroll
+          for (int ss = 0; ss < NST; ss++) { const f32x4 f = __builtin_bit_cast(f32x4, xq[ss][v]); ps[v] += stepok[ss] ? f.x * f.x + f.y * f.y + f.z * f.z + f.w * f.w : 0.f; }
+          ps[v] = wave_sum(ps[v]);
+        }
+        if (lane == 0) {
+#pragma unroll
+          for (int v = 0; v < NV; v++) part[0][wave][v][0] = ps[v];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < QD_NW; w++) t += part[0][w][v][0];
+          sc[v] = 1.0f / sqrtf(t / (float)a.K + a.norm_eps);
+        }
+      }
 #pragma unroll
       for (int ss = 0; ss < NST; ss++) {
 #pragma unroll
@@ -264,7 +304,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
 #pragma unroll
         for (int v = 0; v < NV; v++) {
           if constexpr (F32) {
-            const f32x4 f = __builtin_bit_cast(f32x4, xq[ss][v]);
+            f32x4 f = __builtin_bit_cast(f32x4, xq[ss][v]);
+            if constexpr (NORM) { const f32x4 nw = __builtin_bit_cast(f32x4, nwq[ss]); f.x = (f.x * sc[v]) * nw.x; f.y = (f.y * sc[v]) * nw.y; f.z = (f.z * sc[v]) * nw.z; f.w = (f.w * sc[v]) * nw.w; }
             *(uint2*)(xb + v * 512 + 16 * (((lane >> 1) + v) & 31) + 8 * (lane & 1)) = uint2{f2h_bits(f.x) | (f2h_bits(f.y) << 16), f2h_bits(f.z) | (f2h_bits(f.w) << 16)};
           } else {
             const int row = 2 * v + (lane >> 5);
@@ -283,8 +324,10 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
       }
     };
     typedef std::integral_constant<int, 4> R4; typedef std::integral_constant<int, 8> R8; typedef std::integral_constant<int, 16> R16;
-    if (a.x_f32) { if (M > 8) prologue(R16{}, std::true_type{}); else if (M > 4) prologue(R8{}, std::true_type{}); else prologue(R4{}, std::true_type{}); }
-    else { if (M > 8) prologue(R16{}, std::false_type{}); else if (M > 4) prologue(R8{}, std::false_type{}); else prologue(R4{}, std::false_type{}); }
+    typedef std::true_type Yes; typedef std::false_type No;
+    if (a.norm_w) { if (M > 8) prologue(R16{}, Yes{}, Yes{}); else if (M > 4) prologue(R8{}, Yes{}, Yes{}); else prologue(R4{}, Yes{}, Yes{}); }     // (the launch has checked: float32 rows)
+    else if (a.x_f32) { if (M > 8) prologue(R16{}, Yes{}, No{}); else if (M > 4) prologue(R8{}, Yes{}, No{}); else prologue(R4{}, Yes{}, No{}); }
+    else { if (M > 8) prologue(R16{}, No{}, No{}); else if (M > 4) prologue(R8{}, No{}, No{}); else prologue(R4{}, No{}, No{}); }
   }
 
   v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
@@ -462,7 +505,8 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 // 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K) return -1;
-  if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w) return -1;
+  if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
+  if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
     return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : -1;

@@ -389,7 +389,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     TGA_REQUIRE(a.y_stage_fmt >= 0, "tga_qlinear: no staged layout for consumer type %d with K=%lld", y_stage_type, (long long)y_stage_K);
   }
   if (norm_w) {
-    TGA_REQUIRE(M == 1 && x_dtype == TGA_F32 && ((uintptr_t)norm_w & 15) == 0, "tga_rmsnorm_qlinear: needs M = 1, float32 x and a 16-byte aligned norm weight");
+    TGA_REQUIRE((M == 1 || !comb) && x_dtype == TGA_F32 && ((uintptr_t)norm_w & 15) == 0, "tga_rmsnorm_qlinear: needs float32 x and a 16-byte aligned norm weight (M = 1 with the expert sum)");
     a.norm_w = norm_w; a.norm_eps = norm_eps;
   }
   if (comb) {
@@ -408,6 +408,11 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
   if (M == 2 && !comb && !norm_w) {                               // two rows on the single-row kernel's walk (Q4_0 / Q8_0 pairs, Q6_K)
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
     if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
+  }
+  if (M >= 2 && norm_w) {                                         // several rows with the norm folded in: the LDS-fed kernel or nothing (-2: the caller norms first)
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+    if (M >= 3 && fmt >= 0) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
+    return -2;
   }
   if (M >= 3) {                                                   // matrix-core small-batch kernels: weights through LDS where that kernel applies, else through registers
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
@@ -462,6 +467,23 @@ extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_ep
                                          int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(norm_weight, "tga_rmsnorm_qlinear_multi: null norm weight");
   return qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+}
+
+// tga_rmsnorm_rows followed by tga_qlinear_multi for M rows: one launch where the LDS-fed small-batch kernel folds the norm into its prologue (Q4_0 / Q8_0 / Q6_K,
+// 3 <= M <= 8, K <= 4096), otherwise the norm into xn_scratch (M, K) fp16 and the linears on that.
+extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                                        const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream) {
+  TGA_REQUIRE(norm_weight && x && xn_scratch_f16, "tga_rmsnorm_qlinear_rows: null pointer");
+  TGA_REQUIRE(M >= 1 && M <= 16 && K > 0 && K <= (1 << 24), "tga_rmsnorm_qlinear_rows: M=%d (1..16), K=%lld", M, (long long)K);
+  // up to eight rows: beyond, what every workgroup reads and normalises again (M float32 rows) costs more than the norm's own launch (8B-arch prefill in
+  // chunks of sixteen: 208 ms folded against 195 ms; chunks of eight 320 against 328, of four 562 against 610)
+  if (M >= 2 && M <= 8 && ((uintptr_t)norm_weight & 15) == 0) {
+    const int rc = qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, M, K, epilogue, resid, 0, 0, stream);
+    if (rc != -2) return rc;
+  }
+  const int rc = tga_rmsnorm_rows(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, nullptr, 0, stream);
+  if (rc) return rc;
+  return qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, M, K, epilogue, resid, 0, 0, stream);
 }
 
 // The MoE weighted sum and block residual (x += sum_j probs[j] * y[j], tinygrad/llm/model.py:130, 150) folded into the launch that

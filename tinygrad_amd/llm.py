@@ -610,13 +610,15 @@ class BatchedTransformer:
       pending = False
     for b in self.blk:
       # h = x + attention(attn_norm(x))                                                   model.py:149
-      norm(b["attn_norm"])
       qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
+      one_qkv = all(l.ggml_type == qkv[0].ggml_type for l in qkv) and not pending
+      if not one_qkv: norm(b["attn_norm"])
       while i < 3:                                                     # one launch per run of equal block types
         j = i + 1
         while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
         bias = dict(epilogue=1, resid=b["bias"][i:j]) if "bias" in b else {}
-        self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
+        if one_qkv: self._linear(qkv, self.x, outs, norm=(b["attn_norm"], c.norm_eps, self.xn), **bias)      # the norm inside the launch where the kernel can
+        else: self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
         i = j
       attention = L.tga_attention_prefill_chunk if self.chunked else L.tga_attention_decode_batched
       rt.check(attention(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
@@ -627,10 +629,10 @@ class BatchedTransformer:
       fused_router = b["moe"] and b["router"].ggml_type == rt.F16 and c.dim % 8 == 0 and c.num_experts <= 1024   # ffn_norm and the router logits in one launch (as the batch-1 step)
       if fused_router:
         rt.check(L.tga_moe_router_rows(self.x.ptr, b["ffn_norm"].ptr, c.norm_eps, b["router"].blocks.ptr, B, c.dim, c.num_experts, self.xn.ptr, self.router_logits.ptr, st))
-      else:
+      elif b["moe"]:
         rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       if not b["moe"]:
-        self._linear([b["ffn_gate"], b["ffn_up"]], self.xn, [self.act], epilogue=2)
+        self._linear([b["ffn_gate"], b["ffn_up"]], self.x, [self.act], epilogue=2, norm=(b["ffn_norm"], c.norm_eps, self.xn))
         self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
         continue
       k = c.num_experts_per_tok                                         # model.py:110-135

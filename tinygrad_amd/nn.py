@@ -38,7 +38,8 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x).
   x_staged: x is already in the staged order of these weights (stage_activation or a staging producer).
   stage_out_for: write the single fp16 output in the staged order of that consumer layer.
-  norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it.
+  norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it; norm = (weight, eps, scratch) for several
+  float32 rows (scratch: an fp16 buffer of x's shape that receives the normalised rows when the kernel at hand cannot fold the norm).
   combine = (y, probs, k, x_out) with norm: the row is first completed as x + sum_j probs[j] * y[j] (the MoE weighted sum + residual) and
   the completed row is written to x_out (a buffer other than x)."""
   nseg = len(layers)
@@ -56,6 +57,10 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
     assert norm is not None and m == 1 and x.dtype == np.float32 and not x_staged and epilogue == 0 and so is None and combine[3].ptr != x.ptr
     rt.check(rt.lib().tga_moe_combine_rmsnorm_qlinear_multi(combine[0].ptr, combine[1].ptr, combine[2], x.ptr, combine[3].ptr, norm[0].ptr, norm[1],
                                                             t, nseg, w, y, n, ydt, k, stream))
+    return outs
+  if norm is not None and len(norm) == 3:                                # rows with a scratch: one launch where the LDS-fed kernel folds the norm in, else norm + linears
+    assert x.dtype == np.float32 and not x_staged and so is None and len(norm) == 3, "norm = (weight, eps, fp16 scratch of x's shape) for several rows"
+    rt.check(rt.lib().tga_rmsnorm_qlinear_rows(norm[0].ptr, norm[1], t, nseg, w, y, n, x.ptr, norm[2].ptr, ydt, m, k, epilogue, r, stream))
     return outs
   if norm is not None:
     assert m == 1 and x.dtype == np.float32 and not x_staged
