@@ -39,47 +39,61 @@ def test_no_scratch(kernels):
     m = re.search(r"\.set " + re.escape(name) + r"\.private_seg_size, (\d+)", text)
     assert m and int(m.group(1)) == 0, (name, m and m.group(1))
 
-def test_prologue_requests_untouched_until_the_wait(kernels):
-  """K <= 4096 kernels: every run of activation requests is followed by the hand-written wait before anything else names their registers."""
-  _, ks = kernels
-  checked = 0
-  for name, L in ks.items():
-    if not name.endswith("ELb0ELb0EEv5QArgsii"): continue                   # (streamed-activation kernels: next test)
-    i = 0
-    while i < len(L):
-      if "global_load_dwordx4" not in L[i]: i += 1; continue
-      S, j, last = set(), i, i
-      while j < len(L) and not re.search(r"ds_write_b(128|64)", L[j]):
-        m = re.search(r"global_load_dwordx4 v\[(\d+):(\d+)\]", L[j])
-        if m: S.update(range(int(m.group(1)), int(m.group(2)) + 1)); last = j
-        j += 1
-      w = next((k for k in range(last + 1, len(L)) if "s_waitcnt vmcnt" in L[k] and "ASMSTART" in L[k - 1]), None)
-      assert w is not None, (name, last)
-      for q in range(last + 1, w):
-        assert not (_regs(L[q]) & S) or "global_load_dwordx4" in L[q], (name, q + 1, L[q].strip())
-      checked += 1; i = j
-  assert checked >= 30
+def _touches_in_flight(L):
+  """Forward data flow over the kernel's basic blocks: a request (`global_load_dwordx4 v[a:b]`, only written as inline assembly in this file) puts its destination
+  registers in flight; the source passes them through an asm statement marked "; landed" right behind the hand-counted wait, which lands them all (the wait itself is a
+  switch over immediates that the compiler lowers to a tree of branches with paths no run takes, so it cannot serve as the landing point of a path-insensitive
+  analysis); an instruction that names a register in flight - other than a request that overwrites it - is a finding.  Returns the findings as (line number, text)."""
+  ins = []                                                                     # (line index, text) of instructions; labels -> index of the next instruction
+  labels = {}
+  for i, l in enumerate(L):
+    m = re.match(r"(\.LBB\d+_\d+):", l)
+    if m: labels[m.group(1)] = len(ins); continue
+    if l.strip() == "; landed": ins.append((i, "; landed")); continue
+    t = l.split(";")[0].strip()
+    if not l.startswith("\t") or not t or t.startswith("."): continue
+    ins.append((i, t))
+  n = len(ins)
+  succ = [[] for _ in range(n)]
+  for k, (_, t) in enumerate(ins):
+    op = t.split()[0]
+    if op == "s_endpgm": continue
+    if op == "s_branch": succ[k].append(labels[t.split()[1]]); continue
+    if op.startswith("s_cbranch"): succ[k].append(labels[t.split()[1]])
+    if k + 1 < n: succ[k].append(k + 1)
+  state = [None] * n                                                           # registers in flight BEFORE instruction k
+  state[0] = frozenset()
+  work, found = [0], {}
+  while work:
+    k = work.pop()
+    cur, (li, t) = state[k], ins[k]
+    m = re.match(r"global_load_dwordx4 v\[(\d+):(\d+)\]", t)
+    if m: out = cur | frozenset(range(int(m.group(1)), int(m.group(2)) + 1))   # (its address registers are read at issue: not a use of data in flight)
+    elif t == "; landed": out = frozenset()
+    else:
+      if _regs(t) & cur: found[li + 1] = t
+      out = cur
+    for j in succ[k]:
+      new = out if state[j] is None else state[j] | out
+      if new != state[j]: state[j] = new; work.append(j)
+  return sorted(found.items())
 
-def test_streamed_requests_untouched_around_the_loop(kernels):
-  """K > 4096 kernels: inside the stage loop the request registers are named only by the LDS writes / conversions that consume them, by code between
-  those and the next requests (where they are dead), and by the requests themselves - nothing between the requests and the loop's end."""
+def test_requests_in_flight_are_not_touched(kernels):
+  """Every kernel of the file, K <= 4096 (requests in the prologue) and K > 4096 (one request site in the stage loop, waited for in the next pass)."""
   _, ks = kernels
-  checked = 0
   for name, L in ks.items():
-    if "ELb1ELb0EEv5QArgsii" not in name and "ELb1ELb1EEv5QArgsii" not in name: continue
-    S = set()
-    for l in L:
-      m = re.search(r"global_load_dwordx4 v\[(\d+):(\d+)\]", l)
-      if m: S.update(range(int(m.group(1)), int(m.group(2)) + 1))
-    hdr = max(i for i, l in enumerate(L) if "Loop Header" in l)
-    bars = [i for i, l in enumerate(L) if "s_barrier" in l and i > hdr]
-    assert len(bars) >= 2, name                                              # the stage barrier and the one behind the loop
-    loop_bar, end_bar = bars[0], bars[-1]
-    reqs = [i for i in range(loop_bar, end_bar) if "global_load_dwordx4" in L[i]]
-    assert reqs, name
-    for q in range(reqs[-1] + 1, end_bar):                                   # requests ... end of the loop body (in layout order)
-      assert not (_regs(L[q]) & S), (name, q + 1, L[q].strip())
-    first_use = next(i for i in range(hdr, loop_bar) if _regs(L[i]) & S)
-    assert any("ASMSTART" in L[k] for k in range(max(hdr, first_use - 12), first_use)), (name, first_use + 1, L[first_use].strip())   # first use sits behind the wait / pin
-    checked += 1
-  assert checked == 4
+    assert any("global_load_dwordx4" in l for l in L), name
+    bad = _touches_in_flight(L)
+    assert not bad, (name, bad[:5])
+
+def test_the_check_itself():
+  """The data-flow check on hand-made listings: a copy of a register in flight is found on a straight path, around a loop's back edge and behind a branch; uses behind
+  the landing mark and reuse of the request's address registers are not."""
+  ok = ["\tglobal_load_dwordx4 v[4:7], v[4:5], off", "\ts_cbranch_scc1 .LBB0_2", "\tv_mov_b32_e32 v9, v1", ".LBB0_2:", "\ts_waitcnt vmcnt(0)", "\t; landed", "\tv_mov_b32_e32 v8, v5", "\ts_endpgm"]
+  assert _touches_in_flight(ok) == []
+  straight = ["\tglobal_load_dwordx4 v[4:7], v[2:3], off", "\tv_mov_b32_e32 v8, v5", "\t; landed", "\ts_endpgm"]
+  assert [t for _, t in _touches_in_flight(straight)] == ["v_mov_b32_e32 v8, v5"]
+  branch = ["\tglobal_load_dwordx4 v[4:7], v[2:3], off", "\ts_cbranch_scc1 .LBB0_2", "\t; landed", "\ts_branch .LBB0_3", ".LBB0_2:", "\tv_add_u32_e32 v6, v1, v2", "\t; landed", ".LBB0_3:", "\ts_endpgm"]
+  assert [t for _, t in _touches_in_flight(branch)] == ["v_add_u32_e32 v6, v1, v2"]
+  loop = [".LBB0_1:", "\tv_mov_b32_e32 v9, v4", "\t; landed", "\tds_write_b128 v1, v[4:7]", "\tglobal_load_dwordx4 v[4:7], v[2:3], off", "\ts_cbranch_scc1 .LBB0_1", "\t; landed", "\ts_endpgm"]
+  assert [t for _, t in _touches_in_flight(loop)] == ["v_mov_b32_e32 v9, v4"]

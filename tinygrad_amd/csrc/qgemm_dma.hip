@@ -79,7 +79,9 @@ template <> struct DmaFmt<GGML_Q6_K> {
   }
 };
 
-// at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave)
+// at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave).  Behind it, the registers of inline-assembly
+// requests are passed through an empty asm statement with the comment "; landed": no use of them can move in front of the wait, and the comment marks
+// the place in the generated assembly for tests/test_isa_invariants.py
 __device__ __forceinline__ void qd_wait_vm(int n) {
   switch (n) {
 #define QD_W(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
@@ -215,8 +217,8 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     }
   };
   auto pin_x = [&](u32x4 (&xs)[NXI]) __attribute__((always_inline)) {       // no use of the pieces moves in front of the wait that precedes this
-    asm volatile("" : "+v"(xs[0]), "+v"(xs[1]), "+v"(xs[2]), "+v"(xs[3]), "+v"(xs[4]), "+v"(xs[5]), "+v"(xs[6]), "+v"(xs[7]) :: "memory");
-    if constexpr (XF) asm volatile("" : "+v"(xs[8]), "+v"(xs[9]), "+v"(xs[10]), "+v"(xs[11]), "+v"(xs[12]), "+v"(xs[13]), "+v"(xs[14]), "+v"(xs[15]) :: "memory");
+    asm volatile("; landed" : "+v"(xs[0]), "+v"(xs[1]), "+v"(xs[2]), "+v"(xs[3]), "+v"(xs[4]), "+v"(xs[5]), "+v"(xs[6]), "+v"(xs[7]) :: "memory");
+    if constexpr (XF) asm volatile("; landed" : "+v"(xs[8]), "+v"(xs[9]), "+v"(xs[10]), "+v"(xs[11]), "+v"(xs[12]), "+v"(xs[13]), "+v"(xs[14]), "+v"(xs[15]) :: "memory");
   };
   if constexpr (XS) {
     fetch_x(0, xin);
@@ -272,9 +274,9 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
       if constexpr (NORM) {
 #pragma unroll
         for (int ss = 0; ss < NST; ss++) {
-          asm volatile("" : "+v"(nwq[ss]) :: "memory");
+          asm volatile("; landed" : "+v"(nwq[ss]) :: "memory");
 #pragma unroll
-          for (int v = 0; v < NV; v++) asm volatile("" : "+v"(xq[ss][v]) :: "memory");
+          for (int v = 0; v < NV; v++) asm volatile("; landed" : "+v"(xq[ss][v]) :: "memory");
         }
         float ps[NV];
 #pragma unroll
@@ -300,7 +302,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
 #pragma unroll
       for (int ss = 0; ss < NST; ss++) {
 #pragma unroll
-        for (int v = 0; v < NV; v++) asm volatile("" : "+v"(xq[ss][v]) :: "memory");      // no use of the pieces moves in front of the wait
+        for (int v = 0; v < NV; v++) asm volatile("; landed" : "+v"(xq[ss][v]) :: "memory");      // no use of the pieces moves in front of the wait
 #pragma unroll
         for (int v = 0; v < NV; v++) {
           if constexpr (F32) {
