@@ -54,6 +54,18 @@ template <> struct DmaFmt<F_Q8_0P> {
   }
 };
 
+// fp16 weights (model.py:376 keeps dense tensors as fp16): a unit is 64 consecutive weights = eight aligned pieces, nothing to decode
+template <> struct DmaFmt<GGML_F16> {
+  static constexpr int PAD = 1;
+  static constexpr int slot_bytes(int su) { return su * 128; }
+  static __device__ __forceinline__ Fmt<GGML_F16>::Raw from_lds(const char* row, int u) {
+    const u32x4* p = (const u32x4*)(row + 128 * u);
+    Fmt<GGML_F16>::Raw r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.q[i] = p[i];
+    return r;
+  }
+};
 // Q6_K (gguf.py:68-72): four units = one superblock of 210 bytes, so a slot is 32 units = 8 superblocks = 105 pieces and a wave's step of four units is one
 // superblock; superblocks are 2-byte aligned in the slot's row: every 16-byte piece is read as its enclosing aligned dwords and funnel-shifted (by 0 or 16 bits,
 // the same for the whole wave), as Fmt<GGML_Q6_K>::load does from global memory.
@@ -456,6 +468,11 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   if constexpr (T == GGML_Q6_K) {                                     // (one matrix, plain or residual epilogue: the lm-head and single linears)
     if (a.epilogue == 2 || a.nseg > 1) return -1;
     return launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
+  } else if constexpr (T == GGML_F16) {                               // (plain or residual epilogue, one to three matrices)
+    if (a.epilogue == 2) return -1;
+    const bool two = a.K > 2 * F::UW * SU;
+    if (a.nseg > 1) return two ? launch_qd_k<T, true, 2, false, SU>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
+    return two ? launch_qd_k<T, false, 2, false, SU>(a, M, nb, per_cu, lds, s) : launch_qd_k<T, false, 1, false, SU>(a, M, nb, per_cu, lds, s);
   } else if constexpr (SU == 32) {                                    // K <= 4096: at most two slots, one stage per row group
     if (a.epilogue == 2) return launch_qd_k<T, false, 1, true, SU>(a, M, nb, per_cu, lds, s);
     if (a.nseg > 1) return launch_qd_k<T, true, 1, false, SU>(a, M, nb, per_cu, lds, s);
@@ -489,6 +506,9 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   if constexpr (T == GGML_Q6_K) {                                        // slots of 32 units (8 superblocks = 1680 bytes: whole 16-byte pieces), K = 2048 or 4096
     if (a.K % (F::UW * 32) != 0 || a.K > 2 * F::UW * 32) return -1;
     return launch_qd_su<T, 32>(a, M, s);
+  } else if constexpr (T == GGML_F16) {
+    if (a.K % (F::UW * 16) != 0 || a.K > 4 * F::UW * 16) return -1;      // whole slots of 16 units (2 KB per row), K <= 4096
+    return launch_qd_su<T, 16>(a, M, s);
   } else {
     if (a.K % (F::UW * 16) != 0) return -1;                              // whole slots of 16 units
     if (a.K > 4 * F::UW * 16) {
@@ -504,9 +524,9 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
 // 3 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
-// 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096.
+// 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096; fp16 weights: K <= 4096, no SwiGLU pair.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K) return -1;
+  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16) return -1;
   if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
   if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
@@ -515,5 +535,5 @@ int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   }
   for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;
-  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : launch_qd<GGML_Q6_K>(a, M, s);
+  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : fmt == GGML_Q6_K ? launch_qd<GGML_Q6_K>(a, M, s) : launch_qd<GGML_F16>(a, M, s);
 }
