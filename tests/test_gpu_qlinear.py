@@ -369,6 +369,14 @@ def test_argument_errors(gpu):
   with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))
   # Q4_1 / Q5_0 / Q5_1 rows are read as block pairs: an odd number of blocks per row is refused
   with pytest.raises(RuntimeError, match="multiple of 64"): gpu.check(gpu.lib().tga_qlinear(3, w.ptr, w.ptr, 1, w.ptr, 0, 1, 1, 96, None))
+  # the entry points of the batched steps refuse what they cannot launch
+  L, f = gpu.lib(), gpu.Buffer((64,), np.float32).zero_()
+  with pytest.raises(RuntimeError, match="null pointer"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, None, 1, 4, 32, 0, None, None))
+  with pytest.raises(RuntimeError, match="1..16"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, f.ptr, 1, 17, 32, 0, None, None))
+  with pytest.raises(RuntimeError, match="multiple of 8"): gpu.check(L.tga_moe_router_rows(f.ptr, f.ptr, 1e-5, f.ptr, 2, 20, 4, f.ptr, f.ptr, None))
+  with pytest.raises(RuntimeError, match="rows=0"): gpu.check(L.tga_moe_combine_rmsnorm_rows(f.ptr, f.ptr, f.ptr, f.ptr, 0, 2, 16, 1e-5, f.ptr, None, None))
+  with pytest.raises(RuntimeError, match="exceed one launch"):
+    gpu.check(L.tga_qlinear_experts_routed_rows(2, w.ptr, w.ptr, 8, f.ptr, 40000, 2, 1, 0, 1.0, f.ptr, f.ptr, f.ptr, f.ptr, 1, 4, 64, None))
 
 @pytest.mark.parametrize("t,k", [(2, 4096), (2, 14336), (8, 4096), (14, 4096), (39, 2048), (1, 2048), (12, 4096), (13, 2048), (3, 2048), (6, 4096), (7, 1024)])
 def test_staged_activations_equal_plain_path(gpu, t, k):
