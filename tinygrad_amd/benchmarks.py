@@ -109,7 +109,7 @@ def config8(steps: int = 32, ctx: int = 1024):
   res = []
   for chunk in (16, 8, 4, 2, 1):
     model.prefill_chunk = chunk
-    model.prefill(prompt[:4 * 16 + 3], reuse_cache=False)              # captures the step kinds this chunk size uses
+    model.prefill(prompt[:4 * 16 + 16], reuse_cache=False)             # captures the step kinds this chunk size uses (whole chunks, the tail steps of eight and four, single positions)
     t0 = time.perf_counter()
     model.prefill(prompt, reuse_cache=False)
     dt = time.perf_counter() - t0

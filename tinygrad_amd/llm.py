@@ -339,7 +339,7 @@ class Transformer:
     self._n_prompt, self._steps_done = 0, 0                          # host mirror of the device-side position bookkeeping (for the context guard)
     self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
-    self._state_dict, self._chunker = state_dict, None               # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
+    self._state_dict, self._chunker, self._tail_chunkers = state_dict, None, {}   # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
     self.prefill_chunk = 16                                          # prompt positions per prefill step, 2..16 (the reference's chunks hold 32, model.py:464); 1: token by token
 
   def check_state(self):
@@ -479,6 +479,10 @@ class Transformer:
     if 2 <= B <= 16 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
       if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
       start += self._chunker.prefill_chunks(tokens, start, (len(tokens) - 1 - start) // B, use_graph)
+      for b in (8, 4):                                                  # what is left: one step of eight and / or four positions before the single ones
+        if b < B and len(tokens) - 1 - start >= b:                      # (fifteen single steps are a tenth of a 1023-position prefill)
+          if b not in self._tail_chunkers: self._tail_chunkers[b] = BatchedTransformer(self.config, self._state_dict, b, max_new=1, chunk_of=self)
+          start += self._tail_chunkers[b].prefill_chunks(tokens, start, 1, use_graph)
     self.reset(tokens, start)
     for _ in range(len(tokens) - 1 - start):
       if use_graph: self._graph(False).launch()
