@@ -105,7 +105,7 @@ int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml
                               int y_stage_type, int64_t y_stage_K, void* stream);
 
 /* The same for M rows (batched decode steps and prefill chunks): x (M, K) float32 BEFORE the norm.  One launch where the LDS-fed small-batch kernel applies
- * (Q4_0 / Q8_0 / Q6_K, 3 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
+ * (Q4_0 / Q8_0 / Q6_K / fp16, 2 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
  * tga_qlinear_multi on it.  xn_scratch_f16 is clobbered or left untouched accordingly. */
 int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                              const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream);

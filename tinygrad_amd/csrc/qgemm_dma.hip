@@ -523,11 +523,11 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 }
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
-// 3 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
+// 2 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
 // 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096; fp16 weights: K <= 4096, no SwiGLU pair.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16) return -1;
-  if (M < 3 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
+  if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
   if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;

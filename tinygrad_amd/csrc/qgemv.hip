@@ -405,14 +405,18 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
   }
-  if (M == 2 && !comb && !norm_w) {                               // two rows on the single-row kernel's walk (Q4_0 / Q8_0 pairs, Q6_K)
-    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
-    if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
-  }
   if (M >= 2 && norm_w) {                                         // several rows with the norm folded in: the LDS-fed kernel or nothing (-2: the caller norms first)
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
-    if (M >= 3 && fmt >= 0) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
+    if (fmt >= 0) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     return -2;
+  }
+  if (M == 2 && !comb) {
+    // two rows: the single-row kernel's walk (Q4_0 / Q8_0 pairs, Q6_K) from 2^25 weights on, below that the LDS-fed matrix-core kernel where it applies
+    // (Q4_0 4096 x 4096: 7.4 us against 9.1 us on the LDS-staged dot2 kernel, which takes the rest)
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
+    if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
+    const int fmt2 = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+    if (fmt2 >= 0 && a.ntot * (long long)a.K < (1ll << 25)) { const int rc = tga_qgemm_dma_dispatch(fmt2, a, M, s); if (rc >= 0) return rc; }
   }
   if (M >= 3) {                                                   // matrix-core small-batch kernels: weights through LDS where that kernel applies, else through registers
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
@@ -470,7 +474,7 @@ extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_ep
 }
 
 // tga_rmsnorm_rows followed by tga_qlinear_multi for M rows: one launch where the LDS-fed small-batch kernel folds the norm into its prologue (Q4_0 / Q8_0 / Q6_K,
-// 3 <= M <= 8, K <= 4096), otherwise the norm into xn_scratch (M, K) fp16 and the linears on that.
+// 2 <= M <= 8, K <= 4096), otherwise the norm into xn_scratch (M, K) fp16 and the linears on that.
 extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                         const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream) {
   TGA_REQUIRE(norm_weight && x && xn_scratch_f16, "tga_rmsnorm_qlinear_rows: null pointer");
