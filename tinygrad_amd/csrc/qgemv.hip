@@ -414,6 +414,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     // two rows: the single-row kernel's walk (Q4_0 / Q8_0 pairs, Q6_K) from 2^25 weights on, below that the LDS-fed matrix-core kernel where it applies
     // (Q4_0 4096 x 4096: 7.4 us against 9.1 us on the LDS-staged dot2 kernel, which takes the rest)
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
+    if (fmt == F_Q8_0P && a.K > 4096) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }   // (Q8_0 4096 x 14336: streamed activations 17.3 us, the walk 18.7)
     if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     const int fmt2 = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt2 >= 0 && a.ntot * (long long)a.K < (1ll << 25)) { const int rc = tga_qgemm_dma_dispatch(fmt2, a, M, s); if (rc >= 0) return rc; }
