@@ -255,6 +255,28 @@ def test_rmsnorm_argmax_embed(gpu):
   gpu.check(gpu.lib().tga_argmax_step(lgb.ptr, lg.size, sv.ptr, si.ptr, stb.ptr, pr.ptr, outt.ptr, 4, None))
   assert outt.numpy()[0] == 777 and list(stb.numpy()[:3]) == [1, 777, 1]
 
+@pytest.mark.parametrize("n", [128256, 50257, 1023, 7])
+def test_argmax_of_several_rows(gpu, n):
+  """tga_argmax_rows_step: the first index of every row's maximum (ties, a maximum in the last elements, rows that start off a 16-byte boundary when n is
+  odd, NaN entries that never win) is fed back and stored at out_tokens[step][b]; the shared state moves on once."""
+  rng = np.random.default_rng(n)
+  B = 5
+  lg = rng.standard_normal((B, n)).astype(np.float32)
+  lg[0, [n // 3, n - 1]] = 9.0                                       # a tie: the first wins
+  lg[1, n - 1] = 11.0                                                # the last element
+  lg[2, 0] = 12.0
+  lg[3, n // 2] = np.nan; lg[3, n - 2] = 10.0
+  lg[4, :] = -np.inf                                                 # nothing compares greater: index 0
+  ref = [n // 3, n - 1, 0, n - 2, 0]
+  st = np.zeros(16, np.int32)                                        # pos 0, no prompt left (n_prompt 0): every row samples
+  stb = gpu.Buffer.from_numpy(st); pr = gpu.Buffer((B, 8), np.int32).zero_()
+  toks = gpu.Buffer((B,), np.int32).zero_(); outt = gpu.Buffer((4, B), np.int32).zero_()
+  lgb = gpu.Buffer.from_numpy(lg)
+  gpu.check(gpu.lib().tga_argmax_rows_step(lgb.ptr, B, n, stb.ptr, pr.ptr, 8, toks.ptr, outt.ptr, 4, None))
+  assert list(toks.numpy()) == ref and list(outt.numpy()[0]) == ref
+  after = stb.numpy()
+  assert after[0] == 1 and after[2] == 1                             # pos and step moved on by one
+
 def test_copy_kernel_and_mfma_peak_run(gpu):
   from tinygrad_amd import runtime as rt
   L = rt.lib()

@@ -256,6 +256,45 @@ def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
   qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
   assert ol.rel_err(rb.numpy(), res + ref) <= TOL
 
+@pytest.mark.parametrize("t", [12, 13], ids=["q4_k", "q5_k"])
+@pytest.mark.parametrize("n,k,m", [(16, 2048, 3), (4096 + 48, 4096, 8), (1024, 4096, 16), (4112, 2048, 5), (272, 4096, 11), (1040, 14336, 8), (64, 5120, 13), (2048, 8192, 2), (512, 4096, 2)])
+def test_small_batch_q4_k_q5_k_through_lds(gpu, t, n, k, m):
+  """Q4_K / Q5_K on the kernel that streams the weights into LDS: a slot is eight superblocks of 144 / 176 bytes per row (K = 2048 or 4096), four with
+  the activations streamed beside the weights (K beyond 4096, one matrix); a wave's step is one superblock per row.  Plain, with the residual, as the
+  SwiGLU pair and as three matrices of one launch; fp16 and float32 activations; against the C restatement run in blocks of eight rows and the float64 anchor."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(5 * n + k + m + t)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  y = _run(gpu, t, w, x, n, k)
+  assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
+  rows = min(n, 64)
+  nel, nby = GGML_QUANT[t]
+  W = ol.weight_f32(w[:rows * (k // nel) * nby], rows, k, t)
+  assert ol.rel_err(y[:, :rows], ol.linear_f64(x.astype(np.float32), W)) <= TOL
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
+  layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  xb = gpu.Buffer.from_numpy(x)
+  res = rng.standard_normal((m, n)).astype(np.float32)
+  rb = gpu.Buffer.from_numpy(res)
+  qlinear_multi([layer], xb, [rb], epilogue=1, resid=[rb])
+  assert ol.rel_err(rb.numpy(), res + ref) <= TOL
+  if k <= 4096:
+    n2 = max(16, n // 4 // 16 * 16)
+    w2 = synth.random_blocks(rng, t, n2, k)
+    ref2 = np.concatenate([cref.linear(t, w2, x[i:i + 8], n2, k, threads=8) for i in range(0, m, 8)])
+    l2 = QuantLinear(gpu.Buffer.from_numpy(w2), t, n2, k)
+    outs = [gpu.Buffer((m, n), np.float32), gpu.Buffer((m, n2), np.float32), gpu.Buffer((m, n2), np.float16)]
+    for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    qlinear_multi([layer, l2], xb, outs[:2])
+    np.testing.assert_array_equal(outs[0].numpy(), y)
+    assert ol.rel_err(outs[1].numpy(), ref2) <= TOL
+    r1 = ref2[:, :n2]; g = ref[:, :n2].astype(np.float64)
+    lg = QuantLinear(gpu.Buffer.from_numpy(w[:n2 * (k // nel) * nby].copy()), t, n2, k)
+    qlinear_multi([lg, l2], xb, [outs[2]], epilogue=2)
+    assert ol.rel_err(outs[2].numpy().astype(np.float32), g / (1 + np.exp(-g)) * r1) <= 2 * TOL
+
 @pytest.mark.parametrize("n,k,m", [(16, 2048, 3), (4096 + 48, 4096, 8), (1024, 4096, 16), (4112, 2048, 5), (272, 4096, 11)])
 def test_small_batch_q6_k_through_lds(gpu, n, k, m):
   """Q6_K on the kernel that streams the weights into LDS (one matrix, K = 2048 or 4096, rows a multiple of 16): a slot is eight superblocks of 210
@@ -281,11 +320,12 @@ def test_small_batch_q6_k_through_lds(gpu, n, k, m):
   assert ol.rel_err(rb.numpy(), res + ref) <= TOL
 
 @pytest.mark.parametrize("t,k,ns,m,epi", [(2, 4096, [512, 128, 128], 16, 0), (2, 2048, [256, 64, 64], 5, 0), (8, 4096, [1024, 1024], 8, 2), (2, 4096, [448, 448], 3, 2),
-                                            (14, 4096, [272], 4, 0), (2, 4096, [512, 128, 128], 2, 0), (8, 4096, [256, 256], 2, 2), (8, 1024, [64], 16, 0), (12, 4096, [256, 64, 64], 6, 0), (2, 8192, [128], 8, 0), (2, 4096, [200], 2, 0)])
+                                            (14, 4096, [272], 4, 0), (2, 4096, [512, 128, 128], 2, 0), (8, 4096, [256, 256], 2, 2), (12, 4096, [256, 64, 64], 6, 0), (13, 2048, [264, 264], 7, 2),
+                                            (8, 1024, [64], 16, 0), (3, 4096, [256, 64, 64], 6, 0), (2, 8192, [128], 8, 0), (2, 4096, [200], 2, 0)])
 def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
   """tga_rmsnorm_qlinear_rows (the RMSNorm in front of q/k/v or gate/up folded into the LDS-fed small-batch kernel's prologue) against tga_rmsnorm_rows
   followed by tga_qlinear_multi, and against the float64 anchor of the normalised fp16 rows.  The last cases are outside the kernel that folds the norm
-  (Q4_K, K beyond 4096, two rows, more than eight rows): there the call IS the two launches, bit for bit."""
+  (more than eight rows, Q4_1, K beyond 4096, ragged row counts): there the call IS the two launches, bit for bit."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   L = gpu.lib()
   rng = np.random.default_rng(sum(ns) + k + m + t)
@@ -304,7 +344,7 @@ def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
   scratch = gpu.Buffer((m, k), np.float16)
   gpu.check(L.tga_memset(scratch.ptr, 0xFF, scratch.nbytes, None))
   qlinear_multi(layers, xb, o1, epilogue=epi, norm=(nb, 1e-5, scratch))
-  folded = t in (2, 8, 14) and k <= 4096 and 2 <= m <= 8 and all(n % (8 if epi == 2 else 16) == 0 for n in ns)
+  folded = t in (2, 8, 12, 13, 14) and k <= 4096 and 2 <= m <= 8 and all(n % (8 if epi == 2 else 16) == 0 for n in ns)
   assert (scratch.numpy().view(np.uint16) == 0xFFFF).all() == folded       # one launch: the scratch rows were not needed
   h = xn0.numpy().astype(np.float32)
   refs = [ol.linear_f64(h, ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]

@@ -77,14 +77,16 @@ def kquants():
 
 def config7(steps: int = 64, ctx: int = 1024):
   """The 8B architecture of benchmark configuration 3 with the tensor types of a Q4_K_M file, same procedure as bench.py (prefill through the model,
-  graph replay + sync per token)."""
-  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
+  graph replay + sync per token); then the prefill alone (16 positions per step) and 2 / 4 / 8 sequences decoded in lockstep."""
+  from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
   import time
   c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **LLAMA3_8B)
-  model = Transformer(c, synth_state(c, seed=1007, q4_k_m=True), max_new=steps + 16)
+  sd = synth_state(c, seed=1007, q4_k_m=True)
+  model = Transformer(c, sd, max_new=steps + 16)
   rt.synchronize()
   rng = np.random.default_rng(1007)
-  model.prefill([int(t) for t in rng.integers(0, c.vocab_size, size=ctx)])
+  prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
+  model.prefill(prompt)
   for _ in range(8): model.decode_step()
   rt.synchronize()
   t0 = time.perf_counter()
@@ -92,8 +94,27 @@ def config7(steps: int = 64, ctx: int = 1024):
   rt.synchronize()
   dt = (time.perf_counter() - t0) / steps
   wb = model.weight_bytes_per_token()
-  return [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, Q4_K_M tensor-type mix (Q4_K + Q6_K), graph replay + sync per token",
-           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
+  mix = "Q4_K_M tensor-type mix (Q4_K + Q6_K)"
+  res = [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, {mix}, graph replay + sync per token",
+          "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
+  t0 = time.perf_counter()
+  model.prefill(prompt, reuse_cache=False)                               # (every step kind was captured by the first prefill)
+  dtp = time.perf_counter() - t0
+  res.append({"config": 7, "case": f"Llama-3-8B-arch prefill of {ctx - 1} positions, {model.prefill_chunk} per step, {mix}", "ms": round(dtp * 1e3, 1), "positions_per_s": round((ctx - 1) / dtp, 1)})
+  del model
+  for B in (2, 4, 8):
+    bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
+    bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)])
+    for _ in range(4): bm.decode_step()
+    rt.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps): bm.decode_step()
+    rt.synchronize()
+    dtb = (time.perf_counter() - t0) / steps
+    bm.check_state()
+    res.append({"config": 7, "case": f"Llama-3-8B-arch decode B={B} ctx {ctx} (sequences in lockstep), {mix}", "tok_s": round(B / dtb, 1), "ms_per_step": round(dtb * 1e3, 4)})
+    del bm
+  return res
 
 def config8(steps: int = 32, ctx: int = 1024):
   """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 16 / 8 / 4 / 2 / 1 positions, and decoded

@@ -91,6 +91,24 @@ template <> struct DmaFmt<GGML_Q6_K> {
   }
 };
 
+// Q4_K / Q5_K (gguf.py:57-67): four units = one superblock of 144 / 176 bytes = 9 / 11 aligned pieces; a wave's step of four units is one superblock per row
+// (lane group g: sub-block pair g), every read is an aligned 16-byte piece.
+template <bool FIVE> struct DmaFmtK45 {
+  using F = FmtK45<FIVE>;
+  static constexpr int PAD = 1;                          // pitches of 37 / 73 (Q4_K) and 45 / 89 (Q5_K) pieces: sixteen rows on sixteen different bank quads
+  static constexpr int slot_bytes(int su) { return su / 4 * F::BB; }
+  static __device__ __forceinline__ typename F::Raw from_lds(const char* row, int u) {
+    const char* b = row + F::BB * (u >> 2); const int p = u & 3;
+    typename F::Raw r;
+    r.hdr = *(const u32x4*)b; r.q0 = *(const u32x4*)(b + F::QS + 32 * p); r.q1 = *(const u32x4*)(b + F::QS + 32 * p + 16);
+    if constexpr (FIVE) { r.h0 = *(const u32x4*)(b + 16); r.h1 = *(const u32x4*)(b + 32); }
+    r.p = (uint32_t)p;
+    return r;
+  }
+};
+template <> struct DmaFmt<GGML_Q4_K> : DmaFmtK45<false> {};
+template <> struct DmaFmt<GGML_Q5_K> : DmaFmtK45<true> {};
+
 // at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave).  Behind it, the registers of inline-assembly
 // requests are passed through an empty asm statement with the comment "; landed": no use of them can move in front of the wait, and the comment marks
 // the place in the generated assembly for tests/test_isa_invariants.py
@@ -509,6 +527,15 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   } else if constexpr (T == GGML_F16) {
     if (a.K % (F::UW * 16) != 0 || a.K > 4 * F::UW * 16) return -1;      // whole slots of 16 units (2 KB per row), K <= 4096
     return launch_qd_su<T, 16>(a, M, s);
+  } else if constexpr (T == GGML_Q4_K || T == GGML_Q5_K) {
+    if (a.K % (F::UW * 16) != 0) return -1;                              // whole slots of 16 units (4 superblocks)
+    if (a.K > 4 * F::UW * 16) {
+      if (a.nseg != 1 || a.epilogue > 1) return -1;
+      return launch_qd_xs<T>(a, M, s);
+    }
+    // Q4_K: slots of 32 units (K = 2048 or 4096); Q5_K: of 16 (three stages of 32 units and the activations' way through LDS do not fit beside each other)
+    if constexpr (T == GGML_Q4_K) { if (a.K % (F::UW * 32) != 0) return -1; return launch_qd_su<T, 32>(a, M, s); }
+    else return launch_qd_su<T, 16>(a, M, s);
   } else {
     if (a.K % (F::UW * 16) != 0) return -1;                              // whole slots of 16 units
     if (a.K > 4 * F::UW * 16) {
@@ -526,14 +553,22 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 // 2 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
 // 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096; fp16 weights: K <= 4096, no SwiGLU pair.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16) return -1;
+  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16 && fmt != GGML_Q4_K && fmt != GGML_Q5_K) return -1;
   if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
   if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
-    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : -1;
+    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : fmt == GGML_Q4_K ? launch_qd<GGML_Q4_K>(a, M, s)
+         : fmt == GGML_Q5_K ? launch_qd<GGML_Q5_K>(a, M, s) : -1;
   }
   for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;
-  return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : fmt == GGML_Q6_K ? launch_qd<GGML_Q6_K>(a, M, s) : launch_qd<GGML_F16>(a, M, s);
+  switch (fmt) {
+    case F_Q4_0P: return launch_qd<F_Q4_0P>(a, M, s);
+    case F_Q8_0P: return launch_qd<F_Q8_0P>(a, M, s);
+    case GGML_Q6_K: return launch_qd<GGML_Q6_K>(a, M, s);
+    case GGML_Q4_K: return launch_qd<GGML_Q4_K>(a, M, s);
+    case GGML_Q5_K: return launch_qd<GGML_Q5_K>(a, M, s);
+  }
+  return launch_qd<GGML_F16>(a, M, s);
 }

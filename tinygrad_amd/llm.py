@@ -615,13 +615,16 @@ class BatchedTransformer:
     for b in self.blk:
       # h = x + attention(attn_norm(x))                                                   model.py:149
       qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
-      one_qkv = all(l.ggml_type == qkv[0].ggml_type for l in qkv) and not pending
-      if not one_qkv: norm(b["attn_norm"])
+      # the norm inside the launch where the kernel can: always for one run of equal block types (the call norms first where it cannot), for several runs
+      # (a Q4_K_M file keeps attn_v as Q6_K in half of the blocks) only in the range where every run's kernel folds it
+      same = all(l.ggml_type == qkv[0].ggml_type for l in qkv)
+      fold = not pending and (same or (2 <= B <= 8 and c.dim <= 4096 and c.dim % 2048 == 0 and all(l.out_features % 16 == 0 for l in qkv)))
+      if not fold: norm(b["attn_norm"])
       while i < 3:                                                     # one launch per run of equal block types
         j = i + 1
         while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
         bias = dict(epilogue=1, resid=b["bias"][i:j]) if "bias" in b else {}
-        if one_qkv: self._linear(qkv, self.x, outs, norm=(b["attn_norm"], c.norm_eps, self.xn), **bias)      # the norm inside the launch where the kernel can
+        if fold: self._linear(qkv[i:j], self.x, outs[i:j], norm=(b["attn_norm"], c.norm_eps, self.xn), **bias)
         else: self._linear(qkv[i:j], self.xn, outs[i:j], **bias)
         i = j
       attention = L.tga_attention_prefill_chunk if self.chunked else L.tga_attention_decode_batched
@@ -662,8 +665,8 @@ class BatchedTransformer:
           moe_gate(self.sh_logit, B, 1, 1, self.sh_sel, self.p_sh, 2, False, 1.0, stream=st)
         moe_combine(self.y_sh, self.p_sh, self.x, B, 1, c.dim, self.x, stream=st)
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
-      norm(self.output_norm)
-      self.output(self.xn, out=self.logits_buf, stream=st)
+      if pending or not 2 <= B <= 8: norm(self.output_norm); self.output(self.xn, out=self.logits_buf, stream=st)
+      else: self._linear([self.output], self.x, [self.logits_buf], norm=(self.output_norm, c.norm_eps, self.xn))
     elif pending:                                                        # (a prompt step ends with the last block: nothing reads x afterwards, but keep it whole)
       moe_combine(self.y_e, self.probs, self.x, B, c.num_experts_per_tok, c.dim, self.x, stream=st)
     if self.chunked:                                                     # the next B prompt tokens, B positions on
