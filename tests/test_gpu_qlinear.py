@@ -237,11 +237,13 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
-@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 14336, 16), (8, 4096, 14336, 8), (2, 256, 5120, 3), (8, 48, 14336, 9), (2, 4112, 8192, 13), (8, 1024, 6144, 16)])
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 14336, 16), (8, 4096, 14336, 8), (2, 256, 5120, 3), (8, 48, 14336, 9), (2, 4112, 8192, 13), (8, 1024, 6144, 16),
+                                       (14, 4096, 14336, 8), (14, 48, 8192, 3), (14, 1040, 6144, 16), (14, 64, 5120, 5), (14, 272, 14336, 7)])
 def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
   """K beyond 4096 on the LDS-fed kernel (one matrix): the activations stream beside the weights, whole lines per load, and reach
-  the operand layout through a wave-private piece of LDS; float32 activations are rounded on the way into it.  Plain and with the residual added in place, 0xFF-filled outputs, against the C
-  restatement run in blocks of eight rows."""
+  the operand layout through a wave-private piece of LDS; float32 activations are rounded on the way into it.  Q6_K: slots of four superblocks (840 bytes) fetched
+  as windows of 53 aligned pieces, the second slot of a stage 8 bytes into its window (K a multiple of 2048; beyond eight rows the ring holds two stages instead of three;
+  K = 5120 takes the register-fed kernel).  Plain and with the residual added in place, against the C restatement run in blocks of eight rows."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(7 * n + k + m + t)
   w = synth.random_blocks(rng, t, n, k)

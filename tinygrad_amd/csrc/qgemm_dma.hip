@@ -1,4 +1,4 @@
-// Small-batch GEMM over Q4_0 / Q8_0 block pairs and Q6_K (3 <= M <= 16: the sixteen columns of the MFMA tile) with the weights streamed into LDS by direct-to-LDS loads: the same
+// Small-batch GEMM over Q4_0 / Q8_0 block pairs, Q4_K / Q5_K / Q6_K superblocks and fp16 weights (2 <= M <= 16: the sixteen columns of the MFMA tile) with the weights streamed into LDS by direct-to-LDS loads: the same
 // call sites and arithmetic as qgemm.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392;
 // a unit is decoded once into fp16 weights and v_mfma_f32_16x16x32_f16 multiplies it with all activation rows).
 //
@@ -32,8 +32,16 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 
 // slot_bytes(su): bytes of su units of one row; PAD: 16-byte pieces between the rows of a slot in LDS (the pitch spreads sixteen rows over the banks);
 // from_lds(row, u): unit u of a slot's row.
+// Geometry of a slot whose rows are whole 16-byte pieces at 16-byte aligned offsets: pieces(su) per row, the second slot of a stage second_off(su) bytes
+// behind the first, stage_stride(su) bytes of a row per stage, the slot's first unit skew(su, half) bytes into the staged row.
+template <class D> struct DmaPlain {
+  static constexpr int pieces(int su) { return D::slot_bytes(su) / 16; }
+  static constexpr int second_off(int su) { return D::slot_bytes(su); }
+  static constexpr int stage_stride(int su) { return 2 * D::slot_bytes(su); }
+  static constexpr int skew(int, int) { return 0; }
+};
 template <int T> struct DmaFmt;
-template <> struct DmaFmt<F_Q4_0P> {
+template <> struct DmaFmt<F_Q4_0P> : DmaPlain<DmaFmt<F_Q4_0P>> {
   static constexpr int PAD = 1;
   static constexpr int slot_bytes(int su) { return su * 36; }
   static __device__ __forceinline__ Fmt<F_Q4_0P>::Raw from_lds(const char* row, int u) {
@@ -43,7 +51,7 @@ template <> struct DmaFmt<F_Q4_0P> {
     return r;
   }
 };
-template <> struct DmaFmt<F_Q8_0P> {
+template <> struct DmaFmt<F_Q8_0P> : DmaPlain<DmaFmt<F_Q8_0P>> {
   static constexpr int PAD = 1;
   static constexpr int slot_bytes(int su) { return su * 68; }
   static __device__ __forceinline__ Fmt<F_Q8_0P>::Raw from_lds(const char* row, int u) {
@@ -55,7 +63,7 @@ template <> struct DmaFmt<F_Q8_0P> {
 };
 
 // fp16 weights (model.py:376 keeps dense tensors as fp16): a unit is 64 consecutive weights = eight aligned pieces, nothing to decode
-template <> struct DmaFmt<GGML_F16> {
+template <> struct DmaFmt<GGML_F16> : DmaPlain<DmaFmt<GGML_F16>> {
   static constexpr int PAD = 1;
   static constexpr int slot_bytes(int su) { return su * 128; }
   static __device__ __forceinline__ Fmt<GGML_F16>::Raw from_lds(const char* row, int u) {
@@ -77,8 +85,13 @@ __device__ __forceinline__ u32x4 lds16_a2(const char* p, uint32_t& tail_dword, u
   return u32x4{__builtin_amdgcn_alignbit(v1, v0, sh), __builtin_amdgcn_alignbit(v2, v1, sh), __builtin_amdgcn_alignbit(v3, v2, sh), __builtin_amdgcn_alignbit(e, v3, sh)};
 }
 template <> struct DmaFmt<GGML_Q6_K> {
-  static constexpr int PAD = 2;                          // pitch 107 pieces = 428 dwords = 44 mod 64: sixteen rows on sixteen different bank quads
-  static constexpr int slot_bytes(int su) { return su / 4 * 210; }
+  static constexpr int PAD = 2;                          // pitches of 107 and 55 pieces = 428 and 220 dwords = 44 and 28 mod 64: sixteen rows on sixteen different bank quads
+  // Slots of 16 units (K beyond 4096, an even number of slots): 4 superblocks = 840 bytes start 8 bytes off a 16-byte boundary in every second slot.  A stage
+  // (1680 bytes of a row) is fetched as two windows of 53 aligned pieces, [0, 848) and [832, 1680): the second slot's units start 8 bytes into its window.
+  static constexpr int pieces(int su) { return su == 32 ? 105 : 53; }
+  static constexpr int second_off(int su) { return su == 32 ? 1680 : 832; }
+  static constexpr int stage_stride(int su) { return su / 4 * 210 * 2; }
+  static constexpr int skew(int su, int half) { return su == 32 ? 0 : 8 * half; }
   static __device__ __forceinline__ Fmt<GGML_Q6_K>::Raw from_lds(const char* row, int u) {
     const char* p = row + 210 * (u >> 2); const int h = (u >> 1) & 1, g = u & 1;
     uint32_t tail, sh;
@@ -93,7 +106,7 @@ template <> struct DmaFmt<GGML_Q6_K> {
 
 // Q4_K / Q5_K (gguf.py:57-67): four units = one superblock of 144 / 176 bytes = 9 / 11 aligned pieces; a wave's step of four units is one superblock per row
 // (lane group g: sub-block pair g), every read is an aligned 16-byte piece.
-template <bool FIVE> struct DmaFmtK45 {
+template <bool FIVE> struct DmaFmtK45 : DmaPlain<DmaFmtK45<FIVE>> {
   using F = FmtK45<FIVE>;
   static constexpr int PAD = 1;                          // pitches of 37 / 73 (Q4_K) and 45 / 89 (Q5_K) pieces: sixteen rows on sixteen different bank quads
   static constexpr int slot_bytes(int su) { return su / 4 * F::BB; }
@@ -136,9 +149,9 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   using F = Fmt<T_>;
   using DF = DmaFmt<T_>;
   typedef typename F::Raw Raw;
-  constexpr int SB = DF::slot_bytes(QD_SU);              // bytes of one row in a slot
-  static_assert(SB % 16 == 0, "a slot's row is whole 16-byte pieces");
-  constexpr int PR = SB / 16;                            // ... in 16-byte pieces
+  constexpr int PR = DF::pieces(QD_SU);                  // 16-byte pieces of one row in a slot
+  constexpr int SECOND = DF::second_off(QD_SU), STRIDE = DF::stage_stride(QD_SU);
+  static_assert(SECOND % 16 == 0 && STRIDE % 16 == 0, "slots are fetched in aligned 16-byte pieces");
   constexpr int PITCH = (PR + DF::PAD) * 16;             // LDS bytes from one row of the slot to the next
   constexpr int SLOTS = 16 * (PR + DF::PAD);
   constexpr int NI = (SLOTS + 63) / 64;                  // wave instructions (1 KB each) per slot
@@ -205,13 +218,13 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     rr = rr < 16 ? rr : 15; q = q < PR ? q : PR - 1;
     from_up[i] = SW && rr >= 8;
     doff_odd[i] = (long long)(SW ? (rr & 7) : rr) * a.row_bytes + q * 16;
-    doff[i] = doff_odd[i] + sl * SB;
+    doff[i] = doff_odd[i] + sl * SECOND;
   }
   long long ij = 0; int ist = 0, islot = 0;              // issue stream: row group index (of this workgroup), stage in the group, ring position
   auto issue_stage = [&]() {
     const long long grp = (long long)blockIdx.x + ij * gridDim.x;
     int sg; long long l0; seg_of(grp * GR, sg, l0);
-    const long long goff = l0 * a.row_bytes + (long long)ist * (2 * SB);
+    const long long goff = l0 * a.row_bytes + (long long)ist * STRIDE;
     const uint8_t* base = w_of(sg) + goff;
     const uint8_t* base_up = SW ? a.w[1] + goff : base;
     char* dst = ring + (size_t)islot * (2 * SLOT_BYTES);
@@ -366,7 +379,7 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
   long long cj = 0; int cst = 0, cslot = 0, par = 0;     // compute stream
   long long pend_row0 = -1; int pend_par = 0;            // row group whose partial tiles wait for the next barrier
   auto multiply = [&](const u32x4* bv, int k) {
-    const Raw buf = DF::from_lds(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH, 4 * (step + 4 * k) + g);
+    const Raw buf = DF::from_lds(ring + (size_t)cslot * (2 * SLOT_BYTES) + half * SLOT_BYTES + r * PITCH + DF::skew(QD_SU, half), 4 * (step + 4 * k) + g);
     uint32_t wv[F::NWV];
     F::decode(buf, wv, kc);
     F::to_f16(buf, wv);
@@ -415,9 +428,9 @@ __global__ __launch_bounds__(QD_NW * 64) void qgemm_dma_kernel(const QArgs args,
     if (s + nb - 1 < S) issue_stage();
     if (2 * cst + half < nslots) {
       uint32_t nx[F::UW / 2];
-      const char* src = xt + (r < xrows ? r : 0) * QD_XT_PITCH + 128 * g;
+      const char* src = xt + (r < xrows ? r : 0) * QD_XT_PITCH;           // (the pieces of unit g in the format's own order: 64 consecutive values except for Q6_K)
 #pragma unroll
-      for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * j); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
+      for (int j = 0; j < 8; j++) { const u32x4 t4 = *(const u32x4*)(src + 16 * (F::xoff(g, 4 * j) / 8)); nx[4 * j] = t4.x; nx[4 * j + 1] = t4.y; nx[4 * j + 2] = t4.z; nx[4 * j + 3] = t4.w; }
       float c[F::NG];
       F::stage(nx, bfrag[0], c);
 #pragma unroll
@@ -474,7 +487,7 @@ static int launch_qd_k(const QArgs& a, int M, int nb, int per_cu, size_t lds, hi
 template <int T, int SU>
 static int launch_qd_su(QArgs a, int M, hipStream_t s) {
   using F = Fmt<T>;
-  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::slot_bytes(SU) / 16 + DmaFmt<T>::PAD) + 63) / 64) * 1024;
+  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::pieces(SU) + DmaFmt<T>::PAD) + 63) / 64) * 1024;
   constexpr int per_cu = 1;                                           // one workgroup per CU (two, each with half the ring, were no faster: 17.4 against 14.9 us on Q4_0 14336 x 4096)
   int nb = (int)((QD_LDS_CU / per_cu - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;                                 // (deeper rings were measured: no faster at four stages, slower at seven)
@@ -507,7 +520,7 @@ static int launch_qd_su(QArgs a, int M, hipStream_t s) {
 template <int T>
 static int launch_qd_xs(const QArgs& a, int M, hipStream_t s) {
   constexpr int SU = 16;
-  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::slot_bytes(SU) / 16 + DmaFmt<T>::PAD) + 63) / 64) * 1024;
+  constexpr int STAGE_BYTES = 2 * ((16 * (DmaFmt<T>::pieces(SU) + DmaFmt<T>::PAD) + 63) / 64) * 1024;
   const long long xt_bytes = (long long)QD_NW * (M > 8 ? 16 : 8) * QD_XT_PITCH;
   int nb = (int)((QD_LDS_CU - (long long)sizeof(float) * 2 * QD_NW * 16 * 17 - 1024 - xt_bytes) / STAGE_BYTES);
   if (nb > QD_MAX_NB) nb = QD_MAX_NB;
@@ -522,7 +535,11 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   if constexpr (T == GGML_Q6_K) {                                        // slots of 32 units (8 superblocks = 1680 bytes: whole 16-byte pieces), K = 2048 or 4096
-    if (a.K % (F::UW * 32) != 0 || a.K > 2 * F::UW * 32) return -1;
+    if (a.K % (F::UW * 32) != 0) return -1;
+    if (a.K > 2 * F::UW * 32) {                                          // beyond 4096: slots of 16 units with the activations streamed beside them (beyond eight rows the ring holds two stages: 4096 x 14336 at 16 rows 27 us, as two launches of eight 47)
+      if (a.nseg != 1 || a.epilogue > 1) return -1;
+      return launch_qd_xs<T>(a, M, s);
+    }
     return launch_qd_su<T, 32>(a, M, s);
   } else if constexpr (T == GGML_F16) {
     if (a.K % (F::UW * 16) != 0 || a.K > 4 * F::UW * 16) return -1;      // whole slots of 16 units (2 KB per row), K <= 4096
@@ -549,9 +566,10 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
   }
 }
 
-// Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): Q4_0 / Q8_0 block pairs,
-// 2 <= M <= 16, K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix), every matrix a multiple of
-// 16 rows at a 16-byte aligned address; Q6_K: one matrix, K = 2048 or 4096; fp16 weights: K <= 4096, no SwiGLU pair.
+// Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): 2 <= M <= 16, every matrix a multiple of
+// 16 rows at a 16-byte aligned address (8 rows for the SwiGLU pair);
+// Q4_0 / Q8_0 block pairs: K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix); Q4_K / Q5_K: K = 2048 or 4096 (Q5_K: and 1024, 3072), larger
+// multiples of 1024 for one matrix; Q6_K: one matrix, K a multiple of 2048; fp16 weights: K <= 4096, no SwiGLU pair.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16 && fmt != GGML_Q4_K && fmt != GGML_Q5_K) return -1;
   if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
