@@ -68,11 +68,12 @@ def config2():
 
 def kquants():
   """Q4_K / Q5_K (the block types of Q4_K_M / Q5_K_M model files) and the older Q4_1 / Q5_0 / Q5_1 blocks at the Llama-3-8B linear
-  shapes, M in {1, 8}."""
+  shapes, M in {1, 8} (Q4_K / Q5_K: and 4, 16), and the Q6_K ffn_down of a Q4_K_M file."""
   out = []
   for t in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1):
     for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
-      for m in (1, 8): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
+      for m in ((1, 4, 8, 16) if t in (rt.Q4_K, rt.Q5_K) else (1, 8)): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
+  for m in (1, 4, 8, 16): out.append(dict(config="k-quants", **gemv_case(rt.Q6_K, 4096, 14336, m, iters=200)))
   return out
 
 def config7(steps: int = 64, ctx: int = 1024):
