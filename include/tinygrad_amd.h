@@ -104,6 +104,14 @@ int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_eps, int ggml
                               const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
                               int y_stage_type, int64_t y_stage_K, void* stream);
 
+/* tga_rmsnorm_qlinear_multi with the plain epilogue for matrices of DIFFERENT block types over the same row: segment i has type ggml_types[i].  A Q4_K_M / Q5_K_M
+ * file keeps attn_v as Q6_K beside Q4_K / Q5_K attn_q / attn_k in half of its blocks, and tinygrad/llm/model.py:161-163 applies the three linears to one
+ * normalised row.  Runs of equal consecutive types are one launch each; a (Q4_K | Q5_K) run followed by a Q6_K run shares ONE launch when K is 2304..4096
+ * and x, norm_weight are 16-byte aligned.  Results are those of tga_rmsnorm_qlinear_multi per run; the shared launch is another build of the same walk and may round
+ * a float32 sum differently (within 2e-6 of the largest output). */
+int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_eps, int nseg, const int32_t* ggml_types, const void* const* w, void* const* y, const int64_t* n,
+                              const float* x, int y_dtype, int64_t K, void* stream);
+
 /* The same for M rows (batched decode steps and prefill chunks): x (M, K) float32 BEFORE the norm.  One launch where the LDS-fed small-batch kernel applies
  * (Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K / fp16, 2 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
  * tga_qlinear_multi on it.  xn_scratch_f16 is clobbered or left untouched accordingly. */

@@ -355,6 +355,44 @@ def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
     if folded: assert ol.rel_err(a.numpy(), b.numpy()) <= 2e-4 and ol.rel_err(a.numpy(), ref) <= TOL      # the sum of squares is associated differently: an fp16 value may round the other way
     else: np.testing.assert_array_equal(a.numpy(), b.numpy())
 
+@pytest.mark.parametrize("types,k,ns", [((12, 12, 14), 4096, [4096, 1024, 1024]), ((13, 13, 14), 2560, [512, 128, 128]), ((12, 12, 14), 2304, [48, 9, 7]), ((12, 14), 4096, [6000, 200]),
+                                        ((2, 2, 8), 4096, [256, 64, 64]), ((12, 14, 12), 4096, [256, 64, 64]), ((12, 12, 14), 8192, [128, 64, 64]), ((14, 14, 14), 4096, [256, 64, 64]),
+                                        ((12, 12, 14), 2048, [128, 64, 64])])
+def test_norm_and_linears_of_mixed_block_types(gpu, types, k, ns):
+  """tga_rmsnorm_qlinear_mixed (Q4_K / Q5_K attn_q, attn_k and a Q6_K attn_v of one block in ONE launch of the single-row kernel: the first workgroups walk the first
+  set, the others the second) against tga_rmsnorm_qlinear_multi per run of equal types (to float32 rounding of the sums: 2e-6 of the largest output), and against the float64 anchor of the normalised fp16 row.
+  The later cases are outside the shared launch (other type pairs, three runs, K beyond 4096 or rows of at most 32 units, a single run): there the call IS one launch per run."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi, qlinear_mixed
+  rng = np.random.default_rng(sum(ns) + k + sum(types))
+  ws = [synth.random_blocks(rng, t, n, k) for t, n in zip(types, ns)]
+  layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, t, n in zip(ws, types, ns)]
+  x = (rng.standard_normal((1, k)) * 3).astype(np.float32)
+  nw = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+  xb, nb = gpu.Buffer.from_numpy(x), gpu.Buffer.from_numpy(nw)
+  o0 = [gpu.Buffer((1, n), np.float32) for n in ns]
+  i = 0
+  while i < len(ns):
+    j = i + 1
+    while j < len(ns) and types[j] == types[i]: j += 1
+    qlinear_multi(layers[i:j], xb, o0[i:j], norm=(nb, 1e-5))
+    i = j
+  for ydt in (np.float32, np.float16):
+    o1 = [gpu.Buffer((1, n), ydt) for n in ns]
+    for o in o1: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
+    qlinear_mixed(layers, xb, o1, norm=(nb, 1e-5))
+    shared = len(set(types)) == 2 and types[-1] == 14 and types[0] in (12, 13) and list(types) == sorted(types) and 2048 < k <= 4096
+    for a, b in zip(o1, o0):
+      if not shared: assert a.numpy().tobytes() == b.numpy().astype(ydt).tobytes()
+      else:                                                          # another build of the same walk: the compiler contracts the float32 sums differently
+        e = ol.rel_err(a.numpy().astype(np.float32), b.numpy())
+        assert e <= (2e-6 if ydt == np.float32 else 1e-3), (e, ydt)
+  xn = gpu.Buffer((1, k), np.float16)
+  gpu.check(gpu.lib().tga_rmsnorm(xb.ptr, nb.ptr, k, 1e-5, xn.ptr, None, 0, None))
+  h = xn.numpy().astype(np.float32)
+  for o, o16, w, t, n in zip(o0, o1, ws, types, ns):
+    ref = ol.linear_f64(h, ol.weight_f32(w, n, k, t))
+    assert ol.rel_err(o.numpy(), ref) <= TOL and ol.rel_err(o16.numpy().astype(np.float32), ref) <= 2 * TOL
+
 def test_sixteen_rows_segments_residual_and_swiglu(gpu):
   """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi

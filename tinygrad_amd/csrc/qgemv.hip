@@ -474,6 +474,42 @@ extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_ep
   return qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
 }
 
+// tga_rmsnorm_qlinear_multi (plain epilogue) for matrices of different block types over the same row: runs of equal types are one launch each, and the two
+// runs of a Q4_K_M / Q5_K_M block (Q4_K or Q5_K attn_q / attn_k, Q6_K attn_v) share a launch where the single-row kernel's two-set variant applies.
+int tga_qgemv1_two_dispatch(int fmt_a, int fmt_b, const QArgs& a, const QArgs& b, hipStream_t s);   // qgemv1_two.hip
+extern "C" int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_eps, int nseg, const int32_t* ggml_types, const void* const* w, void* const* y, const int64_t* n,
+                                         const float* x, int y_dtype, int64_t K, void* stream) {
+  TGA_REQUIRE(norm_weight && ggml_types && w && y && n && x, "tga_rmsnorm_qlinear_mixed: null pointer");
+  TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_rmsnorm_qlinear_mixed: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
+  TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_rmsnorm_qlinear_mixed: y_dtype must be TGA_F16 or TGA_F32");
+  int cut = 1;                                                    // end of the first run
+  while (cut < nseg && ggml_types[cut] == ggml_types[0]) cut++;
+  bool two_runs = cut < nseg;
+  for (int i = cut + 1; i < nseg; i++) two_runs = two_runs && ggml_types[i] == ggml_types[cut];
+  if (two_runs && K > 0 && K <= 4096 && (((uintptr_t)norm_weight | (uintptr_t)x) & 15) == 0) {
+    QArgs q[2] = {};
+    bool ok = true;
+    for (int r = 0; r < 2; r++) {
+      QArgs& a = q[r];
+      const int i0 = r ? cut : 0, i1 = r ? nseg : cut;
+      a.nseg = i1 - i0; a.x = x; a.x_f32 = 1; a.y_f32 = y_dtype == TGA_F32; a.K = (int)K; a.norm_w = norm_weight; a.norm_eps = norm_eps;
+      for (int i = i0; i < i1; i++) {
+        ok = ok && n[i] > 0 && w[i] && y[i] && ((uintptr_t)w[i] & 3) == 0;
+        a.w[i - i0] = (const uint8_t*)w[i]; a.y[i - i0] = y[i]; a.n[i - i0] = n[i]; a.ntot += n[i];
+      }
+    }
+    if (ok) { const int rc = tga_qgemv1_two_dispatch(ggml_types[0], ggml_types[cut], q[0], q[1], (hipStream_t)stream); if (rc >= 0) return rc; }
+  }
+  for (int i0 = 0; i0 < nseg;) {                                  // one launch per run (the checks of tga_rmsnorm_qlinear_multi apply to each)
+    int i1 = i0 + 1;
+    while (i1 < nseg && ggml_types[i1] == ggml_types[i0]) i1++;
+    const int rc = qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_types[i0], i1 - i0, w + i0, y + i0, n + i0, x, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
+    if (rc) return rc;
+    i0 = i1;
+  }
+  return 0;
+}
+
 // tga_rmsnorm_rows followed by tga_qlinear_multi for M rows: one launch where the LDS-fed small-batch kernel folds the norm into its prologue (Q4_0 / Q8_0 / Q6_K,
 // 2 <= M <= 8, K <= 4096), otherwise the norm into xn_scratch (M, K) fp16 and the linears on that.
 extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,

@@ -49,8 +49,9 @@
 //
 // MR > 1 (several activation rows; instantiated for two; generic prologue, no fused SwiGLU): the same walk over the weights with MR sets of activations in registers;
 // a unit is decoded once and multiplied with every row.  Outputs and residuals are (MR, rows) per matrix.
+// bx: the workgroup's index among those of this matrix set (blockIdx.x where a launch serves one set, see qgemv1_two_kernel)
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
-__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) {
+__device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx) {
   static_assert(MR == 1 || PRO == 0, "several activation rows: generic prologue");
   // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
   // issued together (read at their points of use they arrive in dependent stages, each a scalar-cache miss of its own).
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   const long long yofs = (long long)job * a.ystride;
   const long long xrow = a.sel ? job / a.xdiv : 0;
   constexpr int RS = (EPI == 2) ? 1 : R;                         // output rows per row group
-  const long long team = ((long long)blockIdx.x * WR + wr) * HM + hrow;
+  const long long team = ((long long)bx * WR + wr) * HM + hrow;
   const long long gbase = a.team_base, grem = a.team_rem;       // ngroups / teams and ngroups % teams, from the host
   // (half-wave teams keep equal contiguous ranges and a compile-time row step: their row numbers live in vector registers, where a run-time
   // step turns every load address into 64-bit vector arithmetic - 0.6 us on the 2048-wide fp16 launches of the MoE decode step)
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
       l.x += p * yl[j].x; l.y += p * yl[j].y; l.z += p * yl[j].z; l.w += p * yl[j].w;
       h.x += p * yh[j].x; h.y += p * yh[j].y; h.z += p * yh[j].z; h.w += p * yh[j].w;
     }
-    if (blockIdx.x == 0 && blockIdx.y == 0 && (int)threadIdx.x < nq) { ((f32x4*)a.comb_x_out)[2 * i] = l; ((f32x4*)a.comb_x_out)[2 * i + 1] = h; }
+    if (bx == 0 && blockIdx.y == 0 && (int)threadIdx.x < nq) { ((f32x4*)a.comb_x_out)[2 * i] = l; ((f32x4*)a.comb_x_out)[2 * i + 1] = h; }
     float ss = (int)threadIdx.x < nq ? l.x * l.x + l.y * l.y + l.z * l.z + l.w * l.w + h.x * h.x + h.y * h.y + h.z * h.z + h.w * h.w : 0.f;
     ss = wave_sum(ss);
     if (lane == 0) nred[wave] = ss;
@@ -340,7 +341,7 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
     __syncthreads();
     eoff = (long long)tk_sel[slot] * a.estride;
     enter(0);                                                    // the weight bases of the selected expert
-    if (blockIdx.x == 0 && slot == 0 && (int)threadIdx.x < a.route_k) {
+    if (bx == 0 && slot == 0 && (int)threadIdx.x < a.route_k) {
       a.sel[xrow * a.route_k + threadIdx.x] = tk_sel[threadIdx.x]; a.route_probs_out[xrow * a.route_k + threadIdx.x] = tk_p[threadIdx.x];
     }
     issue(b[0], lo);
@@ -410,6 +411,31 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
   run_segment();
   // (a branch around loads is harmless here: the ring is empty between segments)
   for (int sg = 1; sg < nseg; sg++) { enter(sg); if (cnt) { issue(b[0], lo); run_segment(); } }
+}
+
+template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
+__global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) { qgemv1_body<T, R, WK, WR, EPI, H, PRO, MR>(args, blockIdx.x); }
+
+// Two sets of matrices of different block types over the same activation row in one launch (a Q4_K_M file keeps attn_v as Q6_K beside Q4_K attn_q / attn_k;
+// tinygrad/llm/model.py:161-163 applies the three linears to one normalised row): the first `split` workgroups walk set a, the others set b.  Rows that one
+// wave covers, plain epilogue.
+// Behind the branch the compiler reads a set's fields from the kernel-argument segment where they are used: a dozen scalar loads, one after the other, each a
+// scalar-cache miss of its own (9.5 us for the 8B shape).  The entry block therefore reads one dword of every 64-byte line of the segment - ten independent loads,
+// one miss time together - so that the later ones hit.  The loads are inline assembly with their wait inside the statement: written in the source (one field per
+// line summed into an operand of an empty statement), they made the compiler allocate 256 registers and spill.
+template <int TA, int TB, int R, int WR, int PRO>
+__global__ __launch_bounds__(WR * 64) void qgemv1_two_kernel(const QArgs a, const QArgs b, const unsigned split) {
+  static_assert(2 * sizeof(QArgs) + sizeof(unsigned) > 0x240 && 2 * sizeof(QArgs) + sizeof(unsigned) <= 0x280, "ten lines of kernel arguments");
+  {
+    const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+    int t0, t1, t2, t3, t4, t5, t6, t7, t8, t9;
+    asm volatile("s_load_dword %0, %10, 0x0\n\ts_load_dword %1, %10, 0x40\n\ts_load_dword %2, %10, 0x80\n\ts_load_dword %3, %10, 0xc0\n\ts_load_dword %4, %10, 0x100\n\t"
+                 "s_load_dword %5, %10, 0x140\n\ts_load_dword %6, %10, 0x180\n\ts_load_dword %7, %10, 0x1c0\n\ts_load_dword %8, %10, 0x200\n\ts_load_dword %9, %10, 0x240\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9) : "s"(ka) : "memory");
+  }
+  if (blockIdx.x < split) qgemv1_body<TA, R, 1, WR, 0, false, PRO>(a, blockIdx.x);
+  else qgemv1_body<TB, R, 1, WR, 0, false, PRO>(b, blockIdx.x - split);
 }
 
 // ------------------------------------------------------------------------------------------------ host side
@@ -516,6 +542,47 @@ int qgemv1_launch_format(QArgs a, hipStream_t s) {
   if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);
   if (waves <= 8) return launch_fast_e<T, 8, 1>(a, s);
   return launch_fast_e<T, 16, 1>(a, s);
+}
+
+// One launch for two sets of matrices of different block types (qgemv1_two_kernel): float32 row with the norm folded in, rows of 33..64 units (one wave per row),
+// plain epilogue.  One workgroup per CU, dealt to the sets by their bytes; inside a set the row groups are spread as a launch of its own would.  Returns -1 outside that range.
+template <int TA, int TB>
+int qgemv1_launch_two(QArgs a, QArgs b, hipStream_t s) {
+  using FA = Fmt<TA>; using FB = Fmt<TB>;
+  static_assert(FA::UW == FB::UW, "both sets stage the row in units of the same width");
+  constexpr int WR = QG1_WR, NT = WR * 64;
+  if (a.K != b.K || a.K % FA::BW != 0 || a.K % FB::BW != 0) return -1;
+  a.nu = a.K / FA::UW; b.nu = b.K / FB::UW;
+  a.row_bytes = (long long)(a.K / FA::BW) * FA::BB; b.row_bytes = (long long)(b.K / FB::BW) * FB::BB;
+  if (a.nu <= 32 || a.nu > 64 || a.K / 8 > NT) return -1;
+  for (const QArgs* q : {&a, &b})
+    if (q->epilogue || q->sel || q->x_staged || q->y_stage_fmt || !q->norm_w || !q->x_f32 || q->comb_y || q->route_logits || q->ntot <= 0) return -1;
+  const size_t lds = (size_t)a.nu * (FA::UW / 2 + 4) * 4;
+  const long long cus = fast_cu_count();
+  const int R = (a.ntot + b.ntot >= cus * r2_rows_per_cu()) ? 2 : 1;
+  // the split that makes the longest team shortest (row groups come whole: dealing the workgroups by bytes alone left the 58 workgroups of a 1024-row Q6_K attn_v
+  // with two row groups per team where 64 have one: 11.4 us for the 8B shape); among equals the one that leaves set a the most workgroups
+  const long long nga = (a.ntot + R - 1) / R, ngb = (b.ntot + R - 1) / R;
+  long long gb = 1, best = -1;
+  for (long long g = 1; g < cus; g++) {
+    const long long ta = (nga + (cus - g) * WR - 1) / ((cus - g) * WR) * a.row_bytes, tb = (ngb + g * WR - 1) / (g * WR) * b.row_bytes;
+    const long long t = ta > tb ? ta : tb;
+    if (best < 0 || t < best) { best = t; gb = g; }
+  }
+  long long ga = cus - gb;
+  auto fit = [&](QArgs& q, long long& g) {                       // no more workgroups than the set has row groups for; row groups per team and the remainder
+    const long long ngroups = (q.ntot + R - 1) / R, most = (ngroups + WR - 1) / WR;
+    if (g > most) g = most;
+    const long long nteams = g * WR;
+    q.team_base = (int)(ngroups / nteams); q.team_rem = (int)(ngroups % nteams);
+    q.team_skew = 0; q.team_first = 0;
+    q.team_stride = q.nseg == 1 ? (int)nteams : 0;
+  };
+  fit(a, ga); fit(b, gb);
+  if (R == 2) qgemv1_two_kernel<TA, TB, 2, WR, 1><<<dim3((unsigned)(ga + gb)), dim3(NT), lds, s>>>(a, b, (unsigned)ga);
+  else qgemv1_two_kernel<TA, TB, 1, WR, 1><<<dim3((unsigned)(ga + gb)), dim3(NT), lds, s>>>(a, b, (unsigned)ga);
+  TGA_LAUNCH_CHECK();
+  return 0;
 }
 
 // Two activation rows on the same kernel (one weight row per step, generic prologue): plain, residual or SwiGLU epilogue, rows that one wave

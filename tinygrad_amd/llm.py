@@ -14,7 +14,7 @@ from dataclasses import dataclass
 import numpy as np
 from tinygrad_amd import runtime as rt
 from tinygrad_amd.runtime import Buffer, GGML_QUANT
-from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, moe_gate, moe_combine, moe_router, expert_jobs, experts_grouped
+from tinygrad_amd.nn import QuantLinear, ExpertWeights, qlinear_multi, qlinear_mixed, moe_gate, moe_combine, moe_router, expert_jobs, experts_grouped
 
 @dataclass(frozen=True)
 class TransformerConfig:
@@ -234,6 +234,8 @@ class TransformerBlock:
       # when the fast path allows, else one RMSNorm launch feeds them
       if not self.fuse_norm: rt.check(L.tga_rmsnorm(x.ptr, self.attn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
       i = 0
+      if self.fuse_norm and self.qkv_bias is None and len({l.ggml_type for l in qkv}) > 1:      # (the call shares one launch between two runs where it can)
+        qlinear_mixed(qkv, x, qkv_out, norm=(self.attn_norm, c.norm_eps), stream=stream); i = 3
       while i < 3:
         j = i + 1
         while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1

@@ -31,6 +31,16 @@ class QuantLinear:
                                   m, self.out_features, self.in_features, stream))
     return out
 
+def qlinear_mixed(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], norm: tuple[Buffer, float], stream=None):
+  """Layers of different block types over the same float32 row x with RMSNorm(x) * weight folded in (Q4_K attn_q / attn_k beside a Q6_K attn_v): one launch
+  per run of equal types, a single launch for the pairs the two-set kernel serves."""
+  nseg, k = len(layers), layers[0].in_features
+  assert all(l.in_features == k for l in layers) and x.dtype == np.float32 and len(outs) == nseg
+  VP = ctypes.c_void_p * nseg
+  rt.check(rt.lib().tga_rmsnorm_qlinear_mixed(norm[0].ptr, norm[1], nseg, (ctypes.c_int32 * nseg)(*[l.ggml_type for l in layers]), VP(*[l.blocks.ptr for l in layers]),
+                                              VP(*[o.ptr for o in outs]), (ctypes.c_int64 * nseg)(*[l.out_features for l in layers]), x.ptr, rt.dtype_code(outs[0].dtype), k, stream))
+  return outs
+
 def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None,
                   x_staged: bool = False, stage_out_for: QuantLinear | None = None, norm: tuple[Buffer, float] | None = None,
                   combine: tuple[Buffer, Buffer, int, Buffer] | None = None):

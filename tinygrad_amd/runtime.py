@@ -37,6 +37,7 @@ def _declare(lib):
     "tga_qlinear": [i, vp, vp, i, vp, i, i, i64, i64, vp],
     "tga_qlinear_multi": [i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i, i, i64, i, c_void_pp, i, i64, vp],
     "tga_rmsnorm_qlinear_multi": [vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i64, i, c_void_pp, i, i64, vp],
+    "tga_rmsnorm_qlinear_mixed": [vp, ctypes.c_float, i, ctypes.POINTER(ctypes.c_int32), c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, i, i64, vp],
     "tga_rmsnorm_qlinear_rows": [vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), vp, vp, i, i, i64, i, c_void_pp, vp],
     "tga_moe_combine_rmsnorm_qlinear_multi": [vp, vp, i, vp, vp, vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, ctypes.POINTER(i64), i, i64, vp],
     "tga_stage_activation": [i, vp, i, i64, vp, vp],
