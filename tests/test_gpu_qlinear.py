@@ -258,11 +258,12 @@ def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
   qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
   assert ol.rel_err(rb.numpy(), res + ref) <= TOL
 
-@pytest.mark.parametrize("t", [12, 13], ids=["q4_k", "q5_k"])
+@pytest.mark.parametrize("t", [12, 13, 3, 6, 7], ids=["q4_k", "q5_k", "q4_1", "q5_0", "q5_1"])
 @pytest.mark.parametrize("n,k,m", [(16, 2048, 3), (4096 + 48, 4096, 8), (1024, 4096, 16), (4112, 2048, 5), (272, 4096, 11), (1040, 14336, 8), (64, 5120, 13), (2048, 8192, 2), (512, 4096, 2)])
 def test_small_batch_q4_k_q5_k_through_lds(gpu, t, n, k, m):
   """Q4_K / Q5_K on the kernel that streams the weights into LDS: a slot is eight superblocks of 144 / 176 bytes per row (K = 2048 or 4096), four with
-  the activations streamed beside the weights (K beyond 4096, one matrix); a wave's step is one superblock per row.  Plain, with the residual, as the
+  the activations streamed beside the weights (K beyond 4096, one matrix); a wave's step is one superblock per row.  Q4_1 / Q5_0 / Q5_1: slots of sixteen
+  block pairs of 40 / 44 / 48 bytes.  Plain, with the residual, as the
   SwiGLU pair and as three matrices of one launch; fp16 and float32 activations; against the C restatement run in blocks of eight rows and the float64 anchor."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(5 * n + k + m + t)
@@ -323,11 +324,11 @@ def test_small_batch_q6_k_through_lds(gpu, n, k, m):
 
 @pytest.mark.parametrize("t,k,ns,m,epi", [(2, 4096, [512, 128, 128], 16, 0), (2, 2048, [256, 64, 64], 5, 0), (8, 4096, [1024, 1024], 8, 2), (2, 4096, [448, 448], 3, 2),
                                             (14, 4096, [272], 4, 0), (2, 4096, [512, 128, 128], 2, 0), (8, 4096, [256, 256], 2, 2), (12, 4096, [256, 64, 64], 6, 0), (13, 2048, [264, 264], 7, 2),
-                                            (8, 1024, [64], 16, 0), (3, 4096, [256, 64, 64], 6, 0), (2, 8192, [128], 8, 0), (2, 4096, [200], 2, 0)])
+                                            (3, 4096, [256, 64, 64], 6, 0), (8, 1024, [64], 16, 0), (39, 4096, [256, 64, 64], 6, 0), (2, 8192, [128], 8, 0), (2, 4096, [200], 2, 0)])
 def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
   """tga_rmsnorm_qlinear_rows (the RMSNorm in front of q/k/v or gate/up folded into the LDS-fed small-batch kernel's prologue) against tga_rmsnorm_rows
   followed by tga_qlinear_multi, and against the float64 anchor of the normalised fp16 rows.  The last cases are outside the kernel that folds the norm
-  (more than eight rows, Q4_1, K beyond 4096, ragged row counts): there the call IS the two launches, bit for bit."""
+  (more than eight rows, MXFP4, K beyond 4096, ragged row counts): there the call IS the two launches, bit for bit."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   L = gpu.lib()
   rng = np.random.default_rng(sum(ns) + k + m + t)
@@ -346,7 +347,7 @@ def test_norm_folded_into_the_small_batch_kernel(gpu, t, k, ns, m, epi):
   scratch = gpu.Buffer((m, k), np.float16)
   gpu.check(L.tga_memset(scratch.ptr, 0xFF, scratch.nbytes, None))
   qlinear_multi(layers, xb, o1, epilogue=epi, norm=(nb, 1e-5, scratch))
-  folded = t in (2, 8, 12, 13, 14) and k <= 4096 and 2 <= m <= 8 and all(n % (8 if epi == 2 else 16) == 0 for n in ns)
+  folded = t in (2, 8, 12, 13, 14, 3, 6, 7) and k <= 4096 and 2 <= m <= 8 and all(n % (8 if epi == 2 else 16) == 0 for n in ns)
   assert (scratch.numpy().view(np.uint16) == 0xFFFF).all() == folded       # one launch: the scratch rows were not needed
   h = xn0.numpy().astype(np.float32)
   refs = [ol.linear_f64(h, ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]

@@ -1,4 +1,4 @@
-// Small-batch GEMM over Q4_0 / Q8_0 block pairs, Q4_K / Q5_K / Q6_K superblocks and fp16 weights (2 <= M <= 16: the sixteen columns of the MFMA tile) with the weights streamed into LDS by direct-to-LDS loads: the same
+// Small-batch GEMM over Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 block pairs, Q4_K / Q5_K / Q6_K superblocks and fp16 weights (2 <= M <= 16: the sixteen columns of the MFMA tile) with the weights streamed into LDS by direct-to-LDS loads: the same
 // call sites and arithmetic as qgemm.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392;
 // a unit is decoded once into fp16 weights and v_mfma_f32_16x16x32_f16 multiplies it with all activation rows).
 //
@@ -121,6 +121,25 @@ template <bool FIVE> struct DmaFmtK45 : DmaPlain<DmaFmtK45<FIVE>> {
 };
 template <> struct DmaFmt<GGML_Q4_K> : DmaFmtK45<false> {};
 template <> struct DmaFmt<GGML_Q5_K> : DmaFmtK45<true> {};
+
+// Q4_1 / Q5_0 / Q5_1 block pairs (gguf.py:47-55): units of 40 / 44 / 48 bytes at 4-byte aligned offsets of the slot's row; 16 units are 40 / 44 / 48 pieces
+// (pitches of 41 / 45 / 49 pieces = 36 / 52 / 4 mod 64 dwords: sixteen rows on sixteen different bank quads)
+template <int KIND> struct DmaFmtL : DmaPlain<DmaFmtL<KIND>> {
+  using F = FmtL<KIND>;
+  static constexpr int PAD = 1;
+  static constexpr int slot_bytes(int su) { return su * F::BB; }
+  static __device__ __forceinline__ typename F::Raw from_lds(const char* row, int u) {
+    const uint32_t* p = (const uint32_t*)(row + F::BB * u);
+    typename F::Raw r;
+    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]};
+#pragma unroll
+    for (int i = 0; i < F::ND - 8; i++) r.t[i] = p[8 + i];
+    return r;
+  }
+};
+template <> struct DmaFmt<GGML_Q4_1> : DmaFmtL<0> {};
+template <> struct DmaFmt<GGML_Q5_0> : DmaFmtL<1> {};
+template <> struct DmaFmt<GGML_Q5_1> : DmaFmtL<2> {};
 
 // at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave).  Behind it, the registers of inline-assembly
 // requests are passed through an empty asm statement with the comment "; landed": no use of them can move in front of the wait, and the comment marks
@@ -568,16 +587,24 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 
 // Returns -1 when the call is outside this kernel's range (the caller then takes the register-fed MFMA kernel): 2 <= M <= 16, every matrix a multiple of
 // 16 rows at a 16-byte aligned address (8 rows for the SwiGLU pair);
-// Q4_0 / Q8_0 block pairs: K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix); Q4_K / Q5_K: K = 2048 or 4096 (Q5_K: and 1024, 3072), larger
+// Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 block pairs: K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix); Q4_K / Q5_K: K = 2048 or 4096 (Q5_K: and 1024, 3072), larger
 // multiples of 1024 for one matrix; Q6_K: one matrix, K a multiple of 2048; fp16 weights: K <= 4096, no SwiGLU pair.
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16 && fmt != GGML_Q4_K && fmt != GGML_Q5_K) return -1;
+  if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16 && fmt != GGML_Q4_K && fmt != GGML_Q5_K && fmt != GGML_Q4_1 && fmt != GGML_Q5_0 && fmt != GGML_Q5_1) return -1;
   if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
   if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
   if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
     if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
-    return fmt == F_Q4_0P ? launch_qd<F_Q4_0P>(a, M, s) : fmt == F_Q8_0P ? launch_qd<F_Q8_0P>(a, M, s) : fmt == GGML_Q4_K ? launch_qd<GGML_Q4_K>(a, M, s)
-         : fmt == GGML_Q5_K ? launch_qd<GGML_Q5_K>(a, M, s) : -1;
+    switch (fmt) {
+      case F_Q4_0P: return launch_qd<F_Q4_0P>(a, M, s);
+      case F_Q8_0P: return launch_qd<F_Q8_0P>(a, M, s);
+      case GGML_Q4_K: return launch_qd<GGML_Q4_K>(a, M, s);
+      case GGML_Q5_K: return launch_qd<GGML_Q5_K>(a, M, s);
+      case GGML_Q4_1: return launch_qd<GGML_Q4_1>(a, M, s);
+      case GGML_Q5_0: return launch_qd<GGML_Q5_0>(a, M, s);
+      case GGML_Q5_1: return launch_qd<GGML_Q5_1>(a, M, s);
+    }
+    return -1;
   }
   for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
   if (((uintptr_t)a.x & 15) != 0) return -1;
@@ -587,6 +614,9 @@ int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
     case GGML_Q6_K: return launch_qd<GGML_Q6_K>(a, M, s);
     case GGML_Q4_K: return launch_qd<GGML_Q4_K>(a, M, s);
     case GGML_Q5_K: return launch_qd<GGML_Q5_K>(a, M, s);
+    case GGML_Q4_1: return launch_qd<GGML_Q4_1>(a, M, s);
+    case GGML_Q5_0: return launch_qd<GGML_Q5_0>(a, M, s);
+    case GGML_Q5_1: return launch_qd<GGML_Q5_1>(a, M, s);
   }
   return launch_qd<GGML_F16>(a, M, s);
 }
