@@ -80,7 +80,7 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
  * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8 (the decode range); 9 <= M <= 16 is taken too, for prefill chunks: one launch where the
- * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
+ * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows; 17 <= M <= 64 (plain fp16 / float32 activations) runs as blocks of sixteen rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
  * (Q4_1 / Q5_0 / Q5_1 are served as block pairs: K % 64 == 0).
  * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K/Q4_1/Q5_0/Q5_1 (GGUF aligns tensor data to 32 bytes,
  * gguf.py:144-148). */
@@ -114,7 +114,7 @@ int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_eps, int nseg
 
 /* The same for M rows (batched decode steps and prefill chunks): x (M, K) float32 BEFORE the norm.  One launch where the LDS-fed small-batch kernel applies
  * (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K / Q6_K / fp16, 2 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
- * tga_qlinear_multi on it.  xn_scratch_f16 is clobbered or left untouched accordingly. */
+ * tga_qlinear_multi on it (M up to 64).  xn_scratch_f16 is clobbered or left untouched accordingly. */
 int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                              const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream);
 

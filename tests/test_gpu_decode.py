@@ -106,10 +106,10 @@ def test_kv_prefix_reuse_equals_fresh_model(gpu):
   model.prefill(p3, reuse_cache=False)
   assert model.prefill_steps == len(p3) - 1
 
-@pytest.mark.parametrize("chunk", [8, 16, 5])
+@pytest.mark.parametrize("chunk", [8, 16, 5, 32, 24, 64])
 @pytest.mark.parametrize("n_prompt", [9, 17, 61, 70, 131])
 def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
-  """Prompt positions computed eight or sixteen (or five) at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
+  """Prompt positions computed eight, sixteen or thirty-two (or five, or twenty-four) at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
   tinygrad/llm/model.py:464, 476-481) against the same model prefilled token by token and against the oracle: the KV caches agree to fp16 rounding of
   slightly different float32 results, the logits of the following decode steps stay within 1e-3 of the oracle's for the same token history, and the
   greedy tokens are the oracle's.  Prompt lengths that leave 0..7 positions for the token-by-token tail and cross the 64-position splits."""

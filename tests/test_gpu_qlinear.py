@@ -237,6 +237,32 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 32), (12, 528, 2048, 24), (8, 200, 14336, 40), (14, 1024, 4096, 64), (2, 512, 14336, 17)])
+def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
+  """Prefill chunks of more than sixteen rows are blocks of sixteen (and a rest) through the same kernels: plain, with the residual in place and with the norm in front
+  (tga_rmsnorm_qlinear_rows), against the C restatement run in blocks of eight rows."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  rng = np.random.default_rng(3 * n + k + m + t)
+  w = synth.random_blocks(rng, t, n, k)
+  x = synth.activations(rng, m, k, np.float16)
+  ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  y = _run(gpu, t, w, x, n, k)
+  assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
+  np.testing.assert_array_equal(y[:16], _run(gpu, t, w, x[:16], n, k))
+  layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  res = rng.standard_normal((m, n)).astype(np.float32)
+  rb = gpu.Buffer.from_numpy(res)
+  qlinear_multi([layer], gpu.Buffer.from_numpy(x), [rb], epilogue=1, resid=[rb])
+  assert ol.rel_err(rb.numpy(), res + ref) <= TOL
+  x32 = (rng.standard_normal((m, k)) * 2).astype(np.float32); nw = (1 + 0.2 * rng.standard_normal(k)).astype(np.float32)
+  xn = gpu.Buffer((m, k), np.float16); nb = gpu.Buffer.from_numpy(nw); out = gpu.Buffer((m, n), np.float32)
+  qlinear_multi([layer], gpu.Buffer.from_numpy(x32), [out], norm=(nb, 1e-5, xn))
+  h = xn.numpy()
+  hn = x32 / np.sqrt((x32.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-5) * nw
+  assert ol.rel_err(h.astype(np.float32), hn.astype(np.float32)) <= 1e-3
+  refn = np.concatenate([cref.linear(t, w, h[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+  assert ol.rel_err(out.numpy(), refn) <= TOL
+
 @pytest.mark.parametrize("t,n,k,m", [(2, 4096, 14336, 16), (8, 4096, 14336, 8), (2, 256, 5120, 3), (8, 48, 14336, 9), (2, 4112, 8192, 13), (8, 1024, 6144, 16),
                                        (14, 4096, 14336, 8), (14, 48, 8192, 3), (14, 1040, 6144, 16), (14, 64, 5120, 5), (14, 272, 14336, 7)])
 def test_small_batch_long_rows_through_lds(gpu, t, n, k, m):
@@ -445,15 +471,15 @@ def test_argument_errors(gpu):
   w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))
   with pytest.raises(ValueError): QuantLinear(w, 1337, 4, 32)
   lin = QuantLinear(w, 2, 4, 32)
-  with pytest.raises(AssertionError): lin(gpu.Buffer((17, 32), np.float16))
-  with pytest.raises(RuntimeError, match="out of range 1..16"): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 17, 4, 32, None))
+  with pytest.raises(AssertionError): lin(gpu.Buffer((65, 32), np.float16))
+  with pytest.raises(RuntimeError, match="out of range 1..64"): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 65, 4, 32, None))
   with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))
   # Q4_1 / Q5_0 / Q5_1 rows are read as block pairs: an odd number of blocks per row is refused
   with pytest.raises(RuntimeError, match="multiple of 64"): gpu.check(gpu.lib().tga_qlinear(3, w.ptr, w.ptr, 1, w.ptr, 0, 1, 1, 96, None))
   # the entry points of the batched steps refuse what they cannot launch
   L, f = gpu.lib(), gpu.Buffer((64,), np.float32).zero_()
   with pytest.raises(RuntimeError, match="null pointer"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, None, 1, 4, 32, 0, None, None))
-  with pytest.raises(RuntimeError, match="1..16"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, f.ptr, 1, 17, 32, 0, None, None))
+  with pytest.raises(RuntimeError, match="1..64"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, f.ptr, 1, 65, 32, 0, None, None))
   with pytest.raises(RuntimeError, match="multiple of 8"): gpu.check(L.tga_moe_router_rows(f.ptr, f.ptr, 1e-5, f.ptr, 2, 20, 4, f.ptr, f.ptr, None))
   with pytest.raises(RuntimeError, match="rows=0"): gpu.check(L.tga_moe_combine_rmsnorm_rows(f.ptr, f.ptr, f.ptr, f.ptr, 0, 2, 16, 1e-5, f.ptr, None, None))
   with pytest.raises(RuntimeError, match="exceed one launch"):

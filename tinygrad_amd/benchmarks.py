@@ -118,7 +118,7 @@ def config7(steps: int = 64, ctx: int = 1024):
   return res
 
 def config8(steps: int = 32, ctx: int = 1024):
-  """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 16 / 8 / 4 / 2 / 1 positions, and decoded
+  """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 64 / 32 / 16 / 8 / 4 / 2 / 1 positions, and decoded
   with 2, 4 and 8 sequences in lockstep (dense linears as small-batch GEMMs)."""
   from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
   import time
@@ -129,9 +129,9 @@ def config8(steps: int = 32, ctx: int = 1024):
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
   res = []
-  for chunk in (16, 8, 4, 2, 1):
+  for chunk in (64, 32, 16, 8, 4, 2, 1):
     model.prefill_chunk = chunk
-    model.prefill(prompt[:4 * 16 + 16], reuse_cache=False)             # captures the step kinds this chunk size uses (whole chunks, the tail steps of eight and four, single positions)
+    model.prefill(prompt[:2 * 64 + 64], reuse_cache=False)             # captures the step kinds this chunk size uses (whole chunks, the tail steps of sixteen, eight and four, single positions)
     t0 = time.perf_counter()
     model.prefill(prompt, reuse_cache=False)
     dt = time.perf_counter() - t0

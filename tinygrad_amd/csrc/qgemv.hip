@@ -354,9 +354,35 @@ extern "C" int tga_stage_activation(int ggml_type, const void* x, int x_dtype, i
 struct CombineIn { const float* y; const float* p; int k; float* x_out; };
 static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
+                              int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
+// M rows as calls of at most `block` rows ((M, n) outputs and (M, K) activations: row blocks are contiguous)
+static int qlinear_row_blocks(int block, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n, const void* x, int x_dtype, int y_dtype, int M, int64_t K,
+                              int epilogue, const void* const* resid, void* stream) {
+  const size_t xs = x_dtype == TGA_F32 ? 4 : 2, ys = y_dtype == TGA_F32 ? 4 : 2;
+  for (int m0 = 0; m0 < M; m0 += block) {
+    const void* wv[QG_MAX_SEG]; void* yv[QG_MAX_SEG]; const void* rv[QG_MAX_SEG];
+    for (int i = 0; i < nseg; i++) {
+      wv[i] = w[i];
+      yv[i] = y[i] ? (char*)y[i] + (size_t)m0 * n[i] * ys : nullptr;
+      rv[i] = (epilogue == 1) ? (const char*)resid[i] + (size_t)m0 * n[i] * 4 : nullptr;
+    }
+    const int rc = qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, wv, yv, n, (const char*)x + (size_t)m0 * K * xs, x_dtype, y_dtype, M - m0 < block ? M - m0 : block, K,
+                                      epilogue, epilogue == 1 ? rv : nullptr, 0, 0, stream);
+    if (rc) return rc;
+  }
+  return 0;
+}
+static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                              const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
-  TGA_REQUIRE(M >= 1 && M <= 16, "tga_qlinear: M=%d out of range 1..16", M);
+  TGA_REQUIRE(M >= 1 && M <= 64, "tga_qlinear: M=%d out of range 1..64", M);
+  if (M > 16) {                                                   // prefill chunks of up to 64 positions: blocks of sixteen rows (every block after the first finds the weights in the Infinity Cache)
+    TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG && !comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32) && !y_stage_type && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
+                "tga_qlinear: more than 16 rows only for plain fp16 / float32 activations");
+    for (int i = 0; i < nseg; i++) TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]), "tga_qlinear: segment %d has a null pointer or no rows", i);
+    return qlinear_row_blocks(16, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
+  }
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
   TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
   TGA_REQUIRE(epilogue >= 0 && epilogue <= 2, "tga_qlinear: epilogue=%d unknown", epilogue);
@@ -424,21 +450,9 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
     if (fmt >= 0) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     if (fmt >= 0) { const int rc = tga_qgemm_mfma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
   }
-  if (M > 8) {                                                    // 9..16 rows outside the LDS-fed kernel's range: two calls of at most eight rows ((M, n) outputs: row blocks are contiguous)
+  if (M > 8) {                                                    // 9..16 rows outside the LDS-fed kernel's range: two calls of at most eight rows
     TGA_REQUIRE(!comb && !norm_w && !a.x_staged && !a.y_stage_fmt, "tga_qlinear: more than 8 rows only for plain activations");
-    const size_t xs = x_dtype == TGA_F32 ? 4 : 2, ys = y_dtype == TGA_F32 ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 8) {
-      const void* wv[QG_MAX_SEG]; void* yv[QG_MAX_SEG]; const void* rv[QG_MAX_SEG];
-      for (int i = 0; i < nseg; i++) {
-        wv[i] = w[i];
-        yv[i] = y[i] ? (char*)y[i] + (size_t)m0 * n[i] * ys : nullptr;
-        rv[i] = (epilogue == 1) ? (const char*)resid[i] + (size_t)m0 * n[i] * 4 : nullptr;
-      }
-      const int rc = qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, wv, yv, n, (const char*)x + (size_t)m0 * K * xs, x_dtype, y_dtype, M - m0 < 8 ? M - m0 : 8, K,
-                                        epilogue, epilogue == 1 ? rv : nullptr, 0, 0, stream);
-      if (rc) return rc;
-    }
-    return 0;
+    return qlinear_row_blocks(8, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
   }
   TGA_REQUIRE(!comb, "tga_moe_combine_rmsnorm_qlinear_multi: needs the M = 1 fast path with K <= 2048");
   TGA_REQUIRE(!norm_w, "tga_rmsnorm_qlinear: the fused norm needs the M = 1 fast path (K %% 64 == 0, 4-byte aligned weights, 16-byte aligned x, K <= 65536)");
@@ -515,7 +529,7 @@ extern "C" int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_ep
 extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                         const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream) {
   TGA_REQUIRE(norm_weight && x && xn_scratch_f16, "tga_rmsnorm_qlinear_rows: null pointer");
-  TGA_REQUIRE(M >= 1 && M <= 16 && K > 0 && K <= (1 << 24), "tga_rmsnorm_qlinear_rows: M=%d (1..16), K=%lld", M, (long long)K);
+  TGA_REQUIRE(M >= 1 && M <= 64 && K > 0 && K <= (1 << 24), "tga_rmsnorm_qlinear_rows: M=%d (1..64), K=%lld", M, (long long)K);
   // up to eight rows: beyond, what every workgroup reads and normalises again (M float32 rows) costs more than the norm's own launch (8B-arch prefill in
   // chunks of sixteen: 208 ms folded against 195 ms; chunks of eight 320 against 328, of four 562 against 610)
   if (M >= 2 && M <= 8 && ((uintptr_t)norm_weight & 15) == 0) {

@@ -342,7 +342,7 @@ class Transformer:
     self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
     self._state_dict, self._chunker, self._tail_chunkers = state_dict, None, {}   # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
-    self.prefill_chunk = 16                                          # prompt positions per prefill step, 2..16 (the reference's chunks hold 32, model.py:464); 1: token by token
+    self.prefill_chunk = 64                                          # prompt positions per prefill step, 2..64 (the reference's chunks hold 32, model.py:464; MoE models: at most 16); 1: token by token
 
   def check_state(self):
     """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
@@ -478,10 +478,11 @@ class Transformer:
     start = self.get_start_pos(tokens) if reuse_cache else 0
     self.prefill_steps = len(tokens) - 1 - start                        # (positions the last call actually computed)
     B = self.prefill_chunk
-    if 2 <= B <= 16 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
+    if B > 16 and self.config.num_experts: B = 16                       # (MoE blocks keep steps of sixteen positions: longer ones are not measured there)
+    if 2 <= B <= 64 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
       if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
       start += self._chunker.prefill_chunks(tokens, start, (len(tokens) - 1 - start) // B, use_graph)
-      for b in (8, 4):                                                  # what is left: one step of eight and / or four positions before the single ones
+      for b in (32, 16, 8, 4):                                          # what is left: one step each of 32, 16, 8 and / or 4 positions before the single ones
         if b < B and len(tokens) - 1 - start >= b:                      # (fifteen single steps are a tenth of a 1023-position prefill)
           if b not in self._tail_chunkers: self._tail_chunkers[b] = BatchedTransformer(self.config, self._state_dict, b, max_new=1, chunk_of=self)
           start += self._tail_chunkers[b].prefill_chunks(tokens, start, 1, use_graph)
@@ -537,7 +538,7 @@ class BatchedTransformer:
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024, chunk_of: "Transformer | None" = None):
     """chunk_of: the rows are `batch` consecutive prompt positions of that Transformer's sequence instead of `batch` sequences (chunked prefill,
     model.py:464, 476-481): its KV caches and rotation table are used, the attention is causal inside the chunk, no token is sampled."""
-    if not 1 <= batch <= (8 if chunk_of is None else 16): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
+    if not 1 <= batch <= (8 if chunk_of is None else 64): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
     self.config, self.batch, self.max_new = config, batch, max_new
     # (no reference back to the Transformer: a cycle would leave its buffers to the cycle collector, which may free them in the middle of a stream capture)
     self.chunked, self._owner_stream = chunk_of is not None, (chunk_of.stream if chunk_of is not None else None)
