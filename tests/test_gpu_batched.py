@@ -95,7 +95,7 @@ SMALL = dict(num_blocks=2, dim=256, hidden_dim=512, n_heads=4, n_kv_heads=2, nor
 SMALL_MOE = dict(num_blocks=2, dim=256, hidden_dim=128, n_heads=4, n_kv_heads=4, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,
                  qk_norm=256, num_experts=8, num_experts_per_tok=2, norm_topk_prob=False, expert_gating_func=1)
 
-@pytest.mark.parametrize("B", [2, 3, 8])
+@pytest.mark.parametrize("B", [2, 3, 8, 16, 11])
 def test_batched_dense_decode(gpu, B):
   from tinygrad_amd.llm import BatchedTransformer, TransformerConfig, synth_state
   c = TransformerConfig(max_context=128, **SMALL)
@@ -107,9 +107,9 @@ def test_batched_dense_decode(gpu, B):
   _per_sequence_check(gpu, BatchedTransformer(c, sd, B, max_new=32), SMALL, host, prompts, 12, 128)
 
 @pytest.mark.parametrize("path", ["jobs", "grouped"])
-@pytest.mark.parametrize("B", [1, 2, 5, 8])
+@pytest.mark.parametrize("B", [1, 2, 5, 8, 16])
 def test_batched_olmoe_arch_decode(gpu, B, path):
-  """Benchmark configuration 4's architecture (fp16 attention / router, MXFP4 experts, full-width q/k norm) at batch 1..8, with the experts as one
+  """Benchmark configuration 4's architecture (fp16 attention / router, MXFP4 experts, full-width q/k norm) at batch 1..16, with the experts as one
   GEMV per (sequence, slot) job and as one small-batch GEMM per selected expert."""
   from tinygrad_amd.llm import BatchedTransformer, TransformerConfig, synth_state_moe
   c = TransformerConfig(max_context=128, **SMALL_MOE)
@@ -119,17 +119,19 @@ def test_batched_olmoe_arch_decode(gpu, B, path):
   # top-k routing is discontinuous: a router logit gap below the rounding noise of the fp16 activations (about 1e-3 of the logit scale) may select
   # another expert on either side.  The prompts are drawn until the oracle's own run stays clear of such ties (gap reported), so that a
   # mismatch below is a defect and not a coin flip.
-  for attempt in range(40):
-    rng = np.random.default_rng(10 + B + 100 * attempt)
-    prompts = [[int(t) for t in rng.integers(0, 512, size=12)] for _ in range(B)]
-    gaps = []
-    for p in prompts:
-      o = ollm.Model(SMALL_MOE, host, 128, act_round_f16=False); o.generate(p, 16); gaps.append(o.min_route_gap)
-    if min(gaps) > 1.5e-3: break                                    # (router logits are O(1); fp16 rounding of the activations moves them by a few 1e-4)
-  print(f"prompt set {attempt}: smallest router logit gap between the last selected and the first rejected expert {min(gaps):.4f}")
-  assert min(gaps) > 1.5e-3
+  rng = np.random.default_rng(10 + B)
+  prompts, gaps, drawn = [], [], 0
+  while len(prompts) < B and drawn < 40 * B:                        # (every sequence's prompt is drawn on its own: sixteen clear ones in one draw are rare)
+    p = [int(t) for t in rng.integers(0, 512, size=12)]; drawn += 1
+    o = ollm.Model(SMALL_MOE, host, 128, act_round_f16=False); o.generate(p, 16)
+    if o.min_route_gap > 1.5e-3: prompts.append(p); gaps.append(o.min_route_gap)   # (router logits are O(1); fp16 rounding of the activations moves them by a few 1e-4)
+  print(f"{drawn} prompts drawn for {B}: smallest router logit gap between the last selected and the first rejected expert {min(gaps):.4f}")
+  assert len(prompts) == B
   model = BatchedTransformer(c, sd, B, max_new=32)
   model.expert_path = path
+  if path == "grouped" and B > 8:                                   # (the job table of the grouped path holds eight rows per expert)
+    with pytest.raises(ValueError, match="batch <= 8"): model.prefill(prompts, False)
+    return
   _per_sequence_check(gpu, model, SMALL_MOE, host, prompts, 16, 128)
 
 def test_batched_equals_single_sequence_path(gpu):

@@ -103,7 +103,7 @@ def config7(steps: int = 64, ctx: int = 1024):
   dtp = time.perf_counter() - t0
   res.append({"config": 7, "case": f"Llama-3-8B-arch prefill of {ctx - 1} positions, {model.prefill_chunk} per step, {mix}", "ms": round(dtp * 1e3, 1), "positions_per_s": round((ctx - 1) / dtp, 1)})
   del model
-  for B in (2, 4, 8):
+  for B in (2, 4, 8, 16):
     bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
     bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)])
     for _ in range(4): bm.decode_step()
@@ -119,7 +119,7 @@ def config7(steps: int = 64, ctx: int = 1024):
 
 def config8(steps: int = 32, ctx: int = 1024):
   """Not a BASELINE configuration: the 8B architecture of configuration 3 (Q4_0, Q6_K lm-head) prefilled in chunks of 64 / 32 / 16 / 8 / 4 / 2 / 1 positions, and decoded
-  with 2, 4 and 8 sequences in lockstep (dense linears as small-batch GEMMs)."""
+  with 2, 4, 8 and 16 sequences in lockstep (dense linears as small-batch GEMMs)."""
   from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
   import time
   c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **LLAMA3_8B)
@@ -137,7 +137,7 @@ def config8(steps: int = 32, ctx: int = 1024):
     dt = time.perf_counter() - t0
     res.append({"config": 8, "case": f"Llama-3-8B-arch Q4_0 prefill of {ctx - 1} positions, {chunk} per step", "ms": round(dt * 1e3, 1), "positions_per_s": round((ctx - 1) / dt, 1)})
   del model
-  for B in (2, 4, 8):
+  for B in (2, 4, 8, 16):
     bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
     bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)])
     for _ in range(4): bm.decode_step()
@@ -173,7 +173,7 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   # batched decode: B sequences in lockstep (dense linears as small-batch GEMMs, one expert GEMV per (sequence, slot) job)
   from tinygrad_amd.llm import BatchedTransformer
   sd = {k: v for k, v in model_sd.items()}
-  for B in (2, 4, 8):
+  for B in (2, 4, 8, 16):
     bm = BatchedTransformer(c, sd, B, max_new=steps + 16)
     bm.prefill([[int(t) for t in rng.integers(0, c.vocab_size, size=ctx)] for _ in range(B)], use_graph)
     for _ in range(4): bm.decode_step(use_graph)

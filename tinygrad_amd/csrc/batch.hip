@@ -1,4 +1,4 @@
-// Pieces of the batched decode step (2..8 sequences in lockstep) that have no batch-1 twin: the expert GEMMs of a MoE block with the
+// Pieces of the batched decode step (2..8 sequences in lockstep on this path) that have no batch-1 twin: the expert GEMMs of a MoE block with the
 // (token, slot) jobs grouped by expert, so that an expert selected by several tokens is streamed once (ExpertWeights.__call__ over a
 // (B, T, k) selection, tinygrad/llm/model.py:21-27, 110-135; the reference's indexed load reads every selected expert once per job).
 //

@@ -538,7 +538,7 @@ class BatchedTransformer:
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024, chunk_of: "Transformer | None" = None):
     """chunk_of: the rows are `batch` consecutive prompt positions of that Transformer's sequence instead of `batch` sequences (chunked prefill,
     model.py:464, 476-481): its KV caches and rotation table are used, the attention is causal inside the chunk, no token is sampled."""
-    if not 1 <= batch <= (8 if chunk_of is None else 64): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..8")
+    if not 1 <= batch <= (16 if chunk_of is None else 64): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..16")
     self.config, self.batch, self.max_new = config, batch, max_new
     # (no reference back to the Transformer: a cycle would leave its buffers to the cycle collector, which may free them in the middle of a stream capture)
     self.chunked, self._owner_stream = chunk_of is not None, (chunk_of.stream if chunk_of is not None else None)
@@ -650,6 +650,7 @@ class BatchedTransformer:
       self_gated = self.expert_path != "grouped" and b["sel_bias"] is None and self.xn.dtype == np.float16 and c.dim <= 4096   # the gate/up launch gates for itself (as the batch-1 step does)
       if not self_gated:
         moe_gate(self.router_logits, B, c.num_experts, k, self.sel, self.probs, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, stream=st, bias=b["sel_bias"])
+      if self.expert_path == "grouped" and B > 8: raise ValueError("the grouped expert path keeps at most eight rows per expert (one per sequence): batch <= 8")
       if self.expert_path == "grouped":                                # one small-batch GEMM per selected expert (its weights read once by the kernel)
         expert_jobs(self.sel, c.num_experts, self.job_table, self.job_flags, stream=st)
         experts_grouped(b["gate_exps"], self.job_table, B * k, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st)
