@@ -76,7 +76,7 @@ def kquants():
   for m in (1, 4, 8, 16): out.append(dict(config="k-quants", **gemv_case(rt.Q6_K, 4096, 14336, m, iters=200)))
   return out
 
-def config7(steps: int = 64, ctx: int = 1024):
+def config7(steps: int = 64, ctx: int = 1024, use_graph: bool = True):
   """The 8B architecture of benchmark configuration 3 with the tensor types of a Q4_K_M file, same procedure as bench.py (prefill through the model,
   graph replay + sync per token); then the prefill alone (16 positions per step) and 2 / 4 / 8 sequences decoded in lockstep."""
   from tinygrad_amd.llm import Transformer, BatchedTransformer, TransformerConfig, synth_state, LLAMA3_8B
@@ -87,17 +87,18 @@ def config7(steps: int = 64, ctx: int = 1024):
   rt.synchronize()
   rng = np.random.default_rng(1007)
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
-  model.prefill(prompt)
-  for _ in range(8): model.decode_step()
+  model.prefill(prompt, use_graph)
+  for _ in range(8): model.decode_step(use_graph)
   rt.synchronize()
   t0 = time.perf_counter()
-  for _ in range(steps): model.decode_step()
+  for _ in range(steps): model.decode_step(use_graph)
   rt.synchronize()
   dt = (time.perf_counter() - t0) / steps
   wb = model.weight_bytes_per_token()
   mix = "Q4_K_M tensor-type mix (Q4_K + Q6_K)"
-  res = [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, {mix}, graph replay + sync per token",
+  res = [{"config": 7, "case": f"Llama-3-8B-arch decode B=1 ctx {ctx}, {mix}, {'graph replay' if use_graph else 'eager launches'} + sync per token",
           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "weight_bytes_per_token": wb, "weight_GBps_over_step": round(wb / dt / 1e9, 1)}]
+  if not use_graph: return res                                          # (a profiler's run: the single-sequence step is what it is after)
   t0 = time.perf_counter()
   model.prefill(prompt, reuse_cache=False)                               # (every step kind was captured by the first prefill)
   dtp = time.perf_counter() - t0
@@ -284,7 +285,7 @@ def traffic(steps: int = 4):
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix; 8 = 8B chunked prefill and batched dense decode")
-  ap.add_argument("--no-graph", action="store_true", help="config 4: launch eagerly instead of replaying a captured graph (for profilers)")
+  ap.add_argument("--no-graph", action="store_true", help="configs 4 and 7: launch eagerly instead of replaying a captured graph (for profilers)")
   ap.add_argument("--traffic", action="store_true", help="only the workload of the HBM-traffic counter runs (see traffic())")
   args = ap.parse_args()
   rt.init(0)
@@ -294,7 +295,7 @@ def main():
     return
   for cfg in args.config:
     fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7, 8: config8}[cfg]
-    for row in (fn(use_graph=not args.no_graph) if cfg == 4 else fn()): print(json.dumps(row), flush=True)
+    for row in (fn(use_graph=not args.no_graph) if cfg in (4, 7) else fn()): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":
   main()
