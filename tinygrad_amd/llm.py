@@ -479,13 +479,24 @@ class Transformer:
     self.prefill_steps = len(tokens) - 1 - start                        # (positions the last call actually computed)
     B = self.prefill_chunk
     if B > 16 and self.config.num_experts: B = 16                       # (MoE blocks keep steps of sixteen positions: longer ones are not measured there)
-    if 2 <= B <= 64 and self.prefill_steps >= B:                        # whole chunks of B positions as small-batch steps (model.py:476-481), the rest token by token
-      if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
-      start += self._chunker.prefill_chunks(tokens, start, (len(tokens) - 1 - start) // B, use_graph)
-      for b in (32, 16, 8, 4):                                          # what is left: one step each of 32, 16, 8 and / or 4 positions before the single ones
-        if b < B and len(tokens) - 1 - start >= b:                      # (fifteen single steps are a tenth of a 1023-position prefill)
-          if b not in self._tail_chunkers: self._tail_chunkers[b] = BatchedTransformer(self.config, self._state_dict, b, max_new=1, chunk_of=self)
-          start += self._tail_chunkers[b].prefill_chunks(tokens, start, 1, use_graph)
+    # Whole chunks as small-batch steps (model.py:476-481) of the largest size that the prompt holds (the chosen one, else 32, 16, 8 or 4 positions).  Dense models: what
+    # they leave is ONE more chunk that ends at the last position and computes some positions again - every row of a step depends on the cache and on its own token
+    # only, so the same values are written again - instead of a ladder of smaller steps and up to three single ones (seven steps, a tenth of a 1023-position prefill).
+    # MoE models keep the ladder (one step each of 8 and / or 4 positions, then single ones).
+    overlap = not self.config.num_experts
+    for b in [B] + [t for t in (32, 16, 8, 4) if t < B]:
+      total = len(tokens) - 1 - start
+      if not 2 <= b <= 64 or total < b: continue
+      if b == B:
+        if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
+        chunker = self._chunker
+      else:
+        if b not in self._tail_chunkers: self._tail_chunkers[b] = BatchedTransformer(self.config, self._state_dict, b, max_new=1, chunk_of=self)
+        chunker = self._tail_chunkers[b]
+      start += chunker.prefill_chunks(tokens, start, total // b, use_graph)
+      if overlap:
+        if start < len(tokens) - 1: chunker.prefill_chunks(tokens, len(tokens) - 1 - b, 1, use_graph); start = len(tokens) - 1
+        break
     self.reset(tokens, start)
     for _ in range(len(tokens) - 1 - start):
       if use_graph: self._graph(False).launch()
