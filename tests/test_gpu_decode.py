@@ -112,7 +112,7 @@ def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
   """Prompt positions computed eight, sixteen or thirty-two (or five, or twenty-four) at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
   tinygrad/llm/model.py:464, 476-481) against the same model prefilled token by token and against the oracle: the KV caches agree to fp16 rounding of
   slightly different float32 results, the logits of the following decode steps stay within 1e-3 of the oracle's for the same token history, and the
-  greedy tokens are the oracle's.  Prompt lengths that leave 0..7 positions for the token-by-token tail and cross the 64-position splits."""
+  greedy tokens are the oracle's.  Prompt lengths that leave 0..7 positions behind the whole chunks (computed by one more chunk that ends at the last position) and cross the 64-position splits."""
   model, host = _build(gpu, SMALL, 192, seed=21)
   single, _ = _build(gpu, SMALL, 192, seed=21)
   model.prefill_chunk, single.prefill_chunk = chunk, 1
