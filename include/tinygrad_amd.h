@@ -212,6 +212,14 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
+/* tga_rmsnorm_qlinear_multi (single row) for the q / k / v launch of a decode step, with a hint for the attention launch behind it (no counterpart in the
+ * reference): every lane also reads one dword of one 128-byte line of the cached K / V rows below state.pos and of the rotation row of that position, each on
+ * the XCD whose attention workgroups will read it, so that the attention finds them in L2.  Same results as tga_rmsnorm_qlinear_multi; caches
+ * [n_kv_heads][max_ctx][head_dim] fp16, rope_table [max_ctx][head_dim] float32.  The hint is dropped unless n_kv_heads is a multiple of 8. */
+int tga_rmsnorm_qlinear_multi_touch(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                                    const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
+                                    const void* state, const void* cache_k, const void* cache_v, const void* rope_table, int n_kv_heads, int head_dim, int max_ctx,
+                                    void* stream);
 /* argmax(-1) with first-max tie rule (tinygrad/mixin/op.py:866-891) + the bookkeeping of Transformer.generate (model.py:475-484):
  * while state.pos + 1 < state.n_prompt the next input token is prompt[pos + 1]; otherwise the argmax token is stored at
  * out_tokens[state.step] and fed back.  scratch_v / scratch_i: 256 floats / 256 int32. */

@@ -4,6 +4,7 @@
 // The position and token live in device memory so that one captured launch sequence can be replayed for every token
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
 #include <type_traits>
+#include <stdlib.h>
 #include "qfmt.h"
 #include "decode.h"
 #include "coherent.h"
@@ -142,6 +143,11 @@ __device__ __forceinline__ AttnArgs attn_args_of_sequence(AttnArgs a, int z) {
   if (a.out32) a.out32 += z * a.out_bs;
   return a;
 }
+
+// One rotated pair of apply_rope (tinygrad/llm/model.py:29-33): (x1 c - x2 s, x2 c + x1 s).  Written as one rounded product and one fused multiply-add, so
+// that every kernel that rotates (the two attention kernels, decode and prefill) produces the same bits whatever the compiler would contract on its own.
+__device__ __forceinline__ float rope_lo(float x1, float x2, float c, float s) { return __builtin_fmaf(x1, c, -(x2 * s)); }
+__device__ __forceinline__ float rope_hi(float x1, float x2, float c, float s) { return __builtin_fmaf(x2, c, x1 * s); }
 
 __device__ __forceinline__ u32x4 pack8_f16(const float* c) {
   u32x4 r = {f2h_bits(c[0]) | (f2h_bits(c[1]) << 16), f2h_bits(c[2]) | (f2h_bits(c[3]) << 16),
@@ -298,7 +304,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
   auto qval = [&](int i) { return NORM != 0 ? (a.q[i] * qscale) * a.q_norm[NORM == 2 ? i % HD : i] : a.q[i]; };
   if (tid < half) {
     const float x1 = NORM != 0 ? (kx1 * kscale) * kw1 : kx1, x2 = NORM != 0 ? (kx2 * kscale) * kw2 : kx2;
-    ks[tid] = x1 * kc - x2 * ksn; ks[half + tid] = x2 * kc + x1 * ksn;
+    ks[tid] = rope_lo(x1, x2, kc, ksn); ks[half + tid] = rope_hi(x1, x2, kc, ksn);
   }
   if (tid < HD) vs[tid] = vx;
   if (wave < group) {                                   // first pass: wave w rotates the query of head w
@@ -306,7 +312,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
     for (int j = 0; j < QPL; j++) {
       const int i = lane + 64 * j;
       const float x1 = NORM != 0 ? (qx1[j] * qscale) * qw1[j] : qx1[j], x2 = NORM != 0 ? (qx2[j] * qscale) * qw2[j] : qx2[j];
-      if (i < half) { qs[wave][i] = x1 * qc[j] - x2 * qsn[j]; qs[wave][half + i] = x2 * qc[j] + x1 * qsn[j]; }
+      if (i < half) { qs[wave][i] = rope_lo(x1, x2, qc[j], qsn[j]); qs[wave][half + i] = rope_hi(x1, x2, qc[j], qsn[j]); }
     }
   }
   __syncthreads();
@@ -334,7 +340,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
         for (int i = lane; i < half; i += 64) {
           const float c = a.rope[(size_t)pos * HD + i], sn = a.rope[(size_t)pos * HD + half + i];
           const float x1 = qval(head * HD + i), x2 = qval(head * HD + half + i);
-          qs[wave][i] = x1 * c - x2 * sn; qs[wave][half + i] = x2 * c + x1 * sn;
+          qs[wave][i] = rope_lo(x1, x2, c, sn); qs[wave][half + i] = rope_hi(x1, x2, c, sn);
         }
       }
       __syncthreads();
@@ -398,6 +404,132 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
       if (lane == 0) { po[HD] = m; po[HD + 1] = l; }
     }
     __syncthreads();
+  }
+}
+
+// The attention of one token as ONE launch whose consumer merges (tga_attn_merge_qlinear): workgroup = (query head, split of SP = 128 IT positions), eight waves
+// of 16 rows per tile, IT tiles per wave, every cached row of the split requested up front (rows clamped to the cache, not to the position), at most four splits.
+// The flattened workgroup index is kv head + n_kv (head in group + group * split): with n_kv a multiple of 8 all readers of a kv head's rows run on one XCD.
+// A split that starts beyond the position writes an empty partial (max -inf, sum 0).  Partials: [n_heads][n_splits][head_dim + 4] = weighted V, max, sum, 2 pad.
+template <int HD8, int IT, int NW>
+__global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) {
+  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = NW * RPI, CSTR = HD + 4, PS = HD + 4, SP = 16 * NW * IT;
+  const int group = a.n_heads / a.n_kv;
+  const int kvh = blockIdx.x % a.n_kv, rest = blockIdx.x / a.n_kv, hh = rest % group, split = rest / group, head = kvh * group + hh;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = HD >> 1;
+  __shared__ float qs[HD], ks[HD], vs[HD];
+  __shared__ float comb[NGRP * CSTR];                   // [run]: o[HD], m, l
+  const int vr = lane / HD8, vp = lane % HD8;
+  const int p0 = split * SP + wave * 16;                // first position of this wave's first tile; tile t starts 16 NW t further
+  // ---- loads that do not depend on the position
+  const int ki = tid < half ? tid : half - 1, vi = tid < HD ? tid : HD - 1;
+  const float kx1 = a.k[kvh * HD + ki], kx2 = a.k[kvh * HD + half + ki], vx = a.v[kvh * HD + vi];
+  const float qx1 = a.q[head * HD + ki], qx2 = a.q[head * HD + half + ki];
+  u32x4 kt[IT][NVI], vt[IT][NVI];
+  {
+    const _Float16* kbase = a.cache_k + (size_t)kvh * a.max_ctx * HD + vp * 8;
+    const _Float16* vbase = a.cache_v + (size_t)kvh * a.max_ctx * HD + vp * 8;
+#pragma unroll
+    for (int t = 0; t < IT; t++) {
+#pragma unroll
+      for (int i = 0; i < NVI; i++) {
+        const int r = p0 + t * 16 * NW + i * RPI + vr, rc = r < a.max_ctx ? r : a.max_ctx - 1;
+        kt[t][i] = *(const u32x4*)(kbase + (size_t)rc * HD);
+        vt[t][i] = *(const u32x4*)(vbase + (size_t)rc * HD);
+      }
+    }
+  }
+  const int pos = a.st->pos;
+  if (pos >= a.max_ctx || pos < 0) {                    // no cache row and no rotation row for this position: nothing is written, the host sees the flag
+    if (blockIdx.x == 0 && tid == 0) atomicOr(&a.st->error, 2);
+    return;
+  }
+  float* po = a.part + ((size_t)head * a.nsplit + split) * PS;
+  if (split * SP > pos) {                               // nothing cached in this split yet
+    if (tid < HD) po[tid] = 0.f;
+    if (tid == 0) { po[HD] = -INFINITY; po[HD + 1] = 0.f; }
+    return;
+  }
+  const float rc_ = a.rope[(size_t)pos * HD + ki], rs_ = a.rope[(size_t)pos * HD + half + ki];
+  if (tid < half) {
+    ks[tid] = rope_lo(kx1, kx2, rc_, rs_); ks[half + tid] = rope_hi(kx1, kx2, rc_, rs_);
+    qs[tid] = rope_lo(qx1, qx2, rc_, rs_); qs[half + tid] = rope_hi(qx1, qx2, rc_, rs_);
+  }
+  if (tid < HD) vs[tid] = vx;
+  __syncthreads();
+  if (hh == 0 && pos / SP == split && tid < HD) {       // one workgroup per kv head appends this token to the cache
+    a.cache_k[((size_t)kvh * a.max_ctx + pos) * HD + tid] = (_Float16)ks[tid];
+    a.cache_v[((size_t)kvh * a.max_ctx + pos) * HD + tid] = (_Float16)vs[tid];
+  }
+  const u32x4 kcur = pack8_f16(ks + vp * 8), vcur = pack8_f16(vs + vp * 8);   // rounded to fp16 exactly like the cached copy
+  float qq[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) qq[j] = qs[vp * 8 + j];
+  float sc[IT][NVI];
+  float m = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < IT; t++) {
+#pragma unroll
+    for (int i = 0; i < NVI; i++) {
+      const int r = p0 + t * 16 * NW + i * RPI + vr;
+      const u32x4 kk = r >= pos ? kcur : kt[t][i];
+      const half2_t k0 = as_h2(kk.x), k1 = as_h2(kk.y), k2 = as_h2(kk.z), k3 = as_h2(kk.w);
+      float s = qq[0] * (float)k0.x; s += qq[1] * (float)k0.y; s += qq[2] * (float)k1.x; s += qq[3] * (float)k1.y;
+      s += qq[4] * (float)k2.x; s += qq[5] * (float)k2.y; s += qq[6] * (float)k3.x; s += qq[7] * (float)k3.y;
+      s = run_sum<HD8>(s);
+      sc[t][i] = r <= pos ? s * a.scale : -INFINITY;
+      m = fmaxf(m, sc[t][i]);
+    }
+  }
+  // softmax partial of this lane run (its rows of every tile): no cross-lane traffic, the fold below sums the runs
+  float l = 0.f;
+  f32x4 o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < IT; t++) {
+#pragma unroll
+    for (int i = 0; i < NVI; i++) {
+      const int r = p0 + t * 16 * NW + i * RPI + vr;
+      const float pj = r <= pos ? __expf(sc[t][i] - m) : 0.f;
+      l += pj;
+      const u32x4 vv = r >= pos ? vcur : vt[t][i];
+      const half2_t v0 = as_h2(vv.x), v1 = as_h2(vv.y), v2 = as_h2(vv.z), v3 = as_h2(vv.w);
+      o0.x += pj * (float)v0.x; o0.y += pj * (float)v0.y; o0.z += pj * (float)v1.x; o0.w += pj * (float)v1.y;
+      o1.x += pj * (float)v2.x; o1.y += pj * (float)v2.y; o1.z += pj * (float)v3.x; o1.w += pj * (float)v3.y;
+    }
+  }
+  float* cw = comb + (size_t)(wave * RPI + vr) * CSTR;
+  *(f32x4*)(cw + vp * 8) = o0; *(f32x4*)(cw + vp * 8 + 4) = o1;
+  if (vp == 0) { cw[HD] = m; cw[HD + 1] = l; }
+  __syncthreads();
+  // fold of the row-run partials into the split partial: the run maximum by every thread, then thread (part, d) sums every NP-th run of dimension d
+  // and the NP parts meet in LDS (the q / k / v rows, no longer needed)
+  constexpr int NP = NW * 64 / HD, GP = NGRP / NP;
+  static_assert(NGRP % NP == 0 && NP >= 1 && NP <= 16, "fold layout");
+  __shared__ float fold_o[NP][HD], fold_l[NP];
+  float mm = -INFINITY;                                 // the first run of wave 0 always holds a valid position: mm is finite
+#pragma unroll
+  for (int g = 0; g < NGRP; g++) mm = fmaxf(mm, comb[g * CSTR + HD]);
+  {
+    const int part = tid / HD, d = tid % HD;
+    float ll = 0.f, od = 0.f;
+#pragma unroll
+    for (int j = 0; j < GP; j++) {
+      const int g = part + NP * j;
+      const float mg = comb[g * CSTR + HD];
+      const float wg = mg == -INFINITY ? 0.f : __expf(mg - mm);   // a run without valid rows contributes nothing
+      ll += wg * comb[g * CSTR + HD + 1];
+      od += wg * comb[g * CSTR + d];
+    }
+    fold_o[part][d] = od;
+    if (d == 0) fold_l[part] = ll;
+  }
+  __syncthreads();
+  if (tid < HD) {
+    float od = 0.f, ll = 0.f;
+#pragma unroll
+    for (int q = 0; q < NP; q++) { od += fold_o[q][tid]; ll += fold_l[q]; }
+    po[tid] = od;
+    if (tid == 0) { po[HD] = mm; po[HD + 1] = ll; }
   }
 }
 
@@ -706,6 +838,43 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream) {
   return attention_launch(0, 1, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_f16, out_f32, stage_type, stream);
+}
+
+// Tiles per wave (1..4) and number of splits (at most six) of the one-launch attention for a cache of max_ctx positions, nw waves per workgroup; 0: too long
+static int attn_split1_waves() { static const int nw = getenv("TGA_ATTN_WAVES") ? atoi(getenv("TGA_ATTN_WAVES")) : 8; return nw == 4 || nw == 16 ? nw : 8; }
+static int attn_split1_tiles(int max_ctx, int* n_splits) {
+  static const int forced = getenv("TGA_ATTN_TILES") ? atoi(getenv("TGA_ATTN_TILES")) : 0;
+  const int rows = 16 * attn_split1_waves();
+  for (int it = 1; it <= 4; it++) { const int s = (max_ctx + rows * it - 1) / (rows * it); if (s <= 6 && (!forced || it == forced || it == 4)) { *n_splits = s; return it; } }
+  *n_splits = 0; return 0;
+}
+int tga_attention_split_plan(int max_ctx, int* n_splits) {
+  TGA_REQUIRE(n_splits && max_ctx > 0, "tga_attention_split_plan: null pointer or max_ctx=%d", max_ctx);
+  attn_split1_tiles(max_ctx, n_splits);
+  return 0;
+}
+int tga_attention_decode_split(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                               int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream) {
+  TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table, "tga_attention_decode_split: null pointer");
+  TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode_split: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
+  TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode_split: head_dim=%d must be 64, 128 or 256", head_dim);
+  TGA_REQUIRE(((uintptr_t)partials & 15) == 0, "tga_attention_decode_split: partials must be 16-byte aligned");
+  int ns = 0; const int it = max_ctx > 0 ? attn_split1_tiles(max_ctx, &ns) : 0;
+  TGA_REQUIRE(it > 0, "tga_attention_decode_split: max_ctx=%d outside 1..2048 (tga_attention_split_plan reports 0 splits)", max_ctx);
+  AttnArgs a = {};
+  a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (DecodeState*)state;
+  a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = ns;
+  a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
+  const unsigned grid = (unsigned)(n_heads * ns);
+  hipStream_t s = (hipStream_t)stream;
+#define TGA_SPLIT1_W(HD8, NW) do { if (it == 1) attn_split1_kernel<HD8, 1, NW><<<grid, NW * 64, 0, s>>>(a); else if (it == 2) attn_split1_kernel<HD8, 2, NW><<<grid, NW * 64, 0, s>>>(a); \
+    else if (it == 3) attn_split1_kernel<HD8, 3, NW><<<grid, NW * 64, 0, s>>>(a); else attn_split1_kernel<HD8, 4, NW><<<grid, NW * 64, 0, s>>>(a); } while (0)
+#define TGA_SPLIT1(HD8) do { const int nw = attn_split1_waves(); if (nw == 4) TGA_SPLIT1_W(HD8, 4); else if (nw == 16) TGA_SPLIT1_W(HD8, 16); else TGA_SPLIT1_W(HD8, 8); } while (0)
+  if (head_dim == 64) TGA_SPLIT1(8); else if (head_dim == 128) TGA_SPLIT1(16); else TGA_SPLIT1(32);
+#undef TGA_SPLIT1_W
+#undef TGA_SPLIT1
+  TGA_LAUNCH_CHECK();
+  return 0;
 }
 
 int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,

@@ -24,9 +24,13 @@ struct QArgs {
   // x_staged: x already holds fp16 activations in the consumer format's staged order (Fmt::spos).
   // y_stage_fmt / y_stage_nu: when y_stage_fmt != 0 the fp16 outputs are written in the staged order of THAT consumer format.
   int x_staged, y_stage_fmt, y_stage_nu;
+  // attn_S > 0 (M = 1 fast path, residual epilogue): x holds float32 split partials of the attention, [K >> attn_hd_log2 heads][attn_S][head_dim + 4] =
+  // weighted V (head_dim), max, sum, 2 pad; the row is their merge, sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m), rounded to fp16
+  // (the two fields sit where the struct had padding: qgemv1_two_kernel counts on the size of two of these)
+  int attn_S;
   // norm_w != nullptr (M = 1 fast path, fp32 x): the activation row is RMS-normalised while it is staged,
   // x * rsqrt(mean(x^2) + norm_eps) * norm_w (nn.RMSNorm, tinygrad/nn/__init__.py:296-304), then rounded to fp16.
-  const float* norm_w; float norm_eps;
+  const float* norm_w; float norm_eps; int attn_hd_log2;
   // comb_y != nullptr (with norm_w): the activation row is first completed as x + sum_j comb_p[j] * comb_y[j] over comb_k rows of K values
   // (the weighted sum over the selected experts' outputs plus the block residual, tinygrad/llm/model.py:130, 150); the completed row is
   // also written to comb_x_out (a different buffer: every workgroup reads x) by the first workgroup.
@@ -39,6 +43,11 @@ struct QArgs {
   int team_base, team_rem;
   int team_skew, team_first;   // the first team_first teams own team_skew row groups more than that, the others as many fewer (0: no skew)
   int team_stride;             // > 0: team t owns row groups t, t + team_stride, ... of the one matrix instead of a contiguous range
+  // touch_pos != nullptr (prologue 1, the q / k / v launch): every lane reads one dword of one 128-byte line of what the attention launch behind this one
+  // will ask for - the cached K / V rows below *touch_pos of the kv heads whose attention workgroups run on this workgroup's XCD, and the rotation row of
+  // that position - so that those lines wait in that XCD's L2 (caches [touch_n_kv][touch_max_ctx] rows of touch_row_bytes; nothing depends on it)
+  const int* touch_pos; const uint8_t* touch_k; const uint8_t* touch_v; const uint8_t* touch_rope;
+  int touch_n_kv, touch_max_ctx, touch_row_bytes, touch_rope_row_bytes;
 };
 
 // staged position of element e for a consumer of format `fmt` (row length K = UW * nu)

@@ -352,7 +352,10 @@ extern "C" int tga_stage_activation(int ggml_type, const void* x, int x_dtype, i
 }
 
 struct CombineIn { const float* y; const float* p; int k; float* x_out; };
-static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+// n_splits > 0: x holds the split partials of the attention (tga_attention_decode_split), merged while the row is staged.  touch_pos: the launch also touches
+// the cache rows and the rotation row that the attention launch behind it will read (QArgs::touch_*)
+struct AttnIn { int n_splits, head_dim; const int* touch_pos; const void* k; const void* v; const void* rope; int n_kv, max_ctx; };
+static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
 // M rows as calls of at most `block` rows ((M, n) outputs and (M, K) activations: row blocks are contiguous)
@@ -366,13 +369,13 @@ static int qlinear_row_blocks(int block, int ggml_type, int nseg, const void* co
       yv[i] = y[i] ? (char*)y[i] + (size_t)m0 * n[i] * ys : nullptr;
       rv[i] = (epilogue == 1) ? (const char*)resid[i] + (size_t)m0 * n[i] * 4 : nullptr;
     }
-    const int rc = qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, wv, yv, n, (const char*)x + (size_t)m0 * K * xs, x_dtype, y_dtype, M - m0 < block ? M - m0 : block, K,
+    const int rc = qlinear_multi_impl(nullptr, nullptr, nullptr, 0.f, ggml_type, nseg, wv, yv, n, (const char*)x + (size_t)m0 * K * xs, x_dtype, y_dtype, M - m0 < block ? M - m0 : block, K,
                                       epilogue, epilogue == 1 ? rv : nullptr, 0, 0, stream);
     if (rc) return rc;
   }
   return 0;
 }
-static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
@@ -427,6 +430,25 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
   // block-pair units need an even number of blocks per row and 4-byte aligned rows
   bool pair = (K / 32) % 2 == 0;
   for (int i = 0; i < nseg; i++) pair = pair && ((uintptr_t)w[i] & 3) == 0;
+  if (attn && attn->touch_pos) {
+    TGA_REQUIRE(M == 1 && norm_w && attn->k && attn->v && attn->rope && attn->n_kv > 0 && attn->max_ctx > 0 && (attn->head_dim == 64 || attn->head_dim == 128 || attn->head_dim == 256),
+                "tga_rmsnorm_qlinear_multi_touch: null pointer or bad cache shape");
+    if (attn->n_kv % 8 == 0) {                                    // (else the attention workgroups of a kv head do not share an XCD: nothing to aim at)
+      a.touch_pos = attn->touch_pos; a.touch_k = (const uint8_t*)attn->k; a.touch_v = (const uint8_t*)attn->v; a.touch_rope = (const uint8_t*)attn->rope;
+      a.touch_n_kv = attn->n_kv; a.touch_max_ctx = attn->max_ctx; a.touch_row_bytes = attn->head_dim * 2; a.touch_rope_row_bytes = attn->head_dim * 4;
+    }
+  }
+  if (attn && attn->n_splits > 0) {
+    const int hd = attn->head_dim;
+    TGA_REQUIRE(M == 1 && nseg == 1 && epilogue == 1 && x_dtype == TGA_F32 && !norm_w && !comb && !y_stage_type, "tga_attn_merge_qlinear: one matrix, one row, residual epilogue");
+    TGA_REQUIRE((hd == 64 || hd == 128 || hd == 256) && K % hd == 0 && attn->n_splits >= 1 && attn->n_splits <= 6 && ((uintptr_t)x & 15) == 0,
+                "tga_attn_merge_qlinear: head_dim=%d n_splits=%d (1..6 splits, 16-byte aligned partials)", hd, attn->n_splits);
+    a.attn_S = attn->n_splits; a.attn_hd_log2 = hd == 64 ? 6 : hd == 128 ? 7 : 8;
+    const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
+    const int rc = fmt >= 0 ? tga_qgemv1_dispatch(fmt, a, s) : -1;
+    if (rc < 0) return tga_set_error("tga_attn_merge_qlinear: needs the M = 1 fast path with rows of 33..64 units (2048 < K <= 4096) and 4-byte aligned weights");
+    return rc;
+  }
   if (M == 1) {
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt >= 0) { const int rc = tga_qgemv1_dispatch(fmt, a, s); if (rc >= 0) return rc; }
@@ -472,10 +494,19 @@ static int qlinear_multi_impl(const CombineIn* comb, const float* norm_w, float 
   return tga_set_error("tga_qlinear: no kernel for type %d with this shape (K=%lld)", ggml_type, (long long)K);
 }
 
+// attn_output + residual of one token whose activation row is still in split partials (model.py:198 after :194-197): the merge over the splits
+// (max, sum, weighted V, division) happens while the row is staged, so the attention needs no merge launch
+extern "C" int tga_attn_merge_qlinear(int ggml_type, const void* w, float* y, int64_t N, int64_t K, const float* resid, const float* partials, int n_splits, int head_dim, void* stream) {
+  TGA_REQUIRE(w && y && resid && partials, "tga_attn_merge_qlinear: null pointer");
+  const AttnIn in = {n_splits, head_dim, nullptr, nullptr, nullptr, nullptr, 0, 0};
+  const void* wv[1] = {w}; void* yv[1] = {y}; const void* rv[1] = {resid}; const int64_t nv[1] = {N};
+  return qlinear_multi_impl(nullptr, &in, nullptr, 0.f, ggml_type, 1, wv, yv, nv, partials, TGA_F32, TGA_F32, 1, K, 1, rv, 0, 0, stream);
+}
+
 extern "C" int tga_qlinear_multi(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                  const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                                  int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
-  return qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+  return qlinear_multi_impl(nullptr, nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, y_stage_type, y_stage_K, stream);
 }
 
 // RMSNorm (nn.RMSNorm, tinygrad/nn/__init__.py:296-304) of the float32 activation row folded into the M = 1 linear that consumes it
@@ -485,7 +516,18 @@ extern "C" int tga_rmsnorm_qlinear_multi(const float* norm_weight, float norm_ep
                                          const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
                                          int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(norm_weight, "tga_rmsnorm_qlinear_multi: null norm weight");
-  return qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+  return qlinear_multi_impl(nullptr, nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, y_stage_type, y_stage_K, stream);
+}
+
+// tga_rmsnorm_qlinear_multi for the q / k / v launch of a decode step: its lanes also read one dword each of the lines that the attention launch behind it
+// will ask for first (cached K / V rows below state.pos, the rotation row of that position), on the XCD that will ask
+extern "C" int tga_rmsnorm_qlinear_multi_touch(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
+                                               const void* x, int y_dtype, int64_t K, int epilogue, const void* const* resid,
+                                               const void* state, const void* cache_k, const void* cache_v, const void* rope_table, int n_kv_heads, int head_dim, int max_ctx,
+                                               void* stream) {
+  TGA_REQUIRE(norm_weight && state, "tga_rmsnorm_qlinear_multi_touch: null norm weight or state");
+  const AttnIn in = {0, head_dim, (const int*)state, cache_k, cache_v, rope_table, n_kv_heads, max_ctx};
+  return qlinear_multi_impl(nullptr, &in, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, 1, K, epilogue, resid, 0, 0, stream);
 }
 
 // tga_rmsnorm_qlinear_multi (plain epilogue) for matrices of different block types over the same row: runs of equal types are one launch each, and the two
@@ -517,7 +559,7 @@ extern "C" int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_ep
   for (int i0 = 0; i0 < nseg;) {                                  // one launch per run (the checks of tga_rmsnorm_qlinear_multi apply to each)
     int i1 = i0 + 1;
     while (i1 < nseg && ggml_types[i1] == ggml_types[i0]) i1++;
-    const int rc = qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_types[i0], i1 - i0, w + i0, y + i0, n + i0, x, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
+    const int rc = qlinear_multi_impl(nullptr, nullptr, norm_weight, norm_eps, ggml_types[i0], i1 - i0, w + i0, y + i0, n + i0, x, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
     if (rc) return rc;
     i0 = i1;
   }
@@ -533,12 +575,12 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
   // up to eight rows: beyond, what every workgroup reads and normalises again (M float32 rows) costs more than the norm's own launch (8B-arch prefill in
   // chunks of sixteen: 208 ms folded against 195 ms; chunks of eight 320 against 328, of four 562 against 610)
   if (M >= 2 && M <= 8 && ((uintptr_t)norm_weight & 15) == 0) {
-    const int rc = qlinear_multi_impl(nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, M, K, epilogue, resid, 0, 0, stream);
+    const int rc = qlinear_multi_impl(nullptr, nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, M, K, epilogue, resid, 0, 0, stream);
     if (rc != -2) return rc;
   }
   const int rc = tga_rmsnorm_rows(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, nullptr, 0, stream);
   if (rc) return rc;
-  return qlinear_multi_impl(nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, M, K, epilogue, resid, 0, 0, stream);
+  return qlinear_multi_impl(nullptr, nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, M, K, epilogue, resid, 0, 0, stream);
 }
 
 // The MoE weighted sum and block residual (x += sum_j probs[j] * y[j], tinygrad/llm/model.py:130, 150) folded into the launch that
@@ -550,7 +592,7 @@ extern "C" int tga_moe_combine_rmsnorm_qlinear_multi(const float* y_experts, con
                                                      const int64_t* n, int y_dtype, int64_t K, void* stream) {
   TGA_REQUIRE(norm_weight && y_experts && probs && x_in && x_out && x_in != x_out, "tga_moe_combine_rmsnorm_qlinear_multi: null pointer, or x_out aliases x_in");
   const CombineIn c = {y_experts, probs, k, x_out};
-  return qlinear_multi_impl(&c, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x_in, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
+  return qlinear_multi_impl(&c, nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x_in, TGA_F32, y_dtype, 1, K, 0, nullptr, 0, 0, stream);
 }
 
 extern "C" int tga_qlinear(int ggml_type, const void* w, const void* x, int x_dtype, void* y, int y_dtype,

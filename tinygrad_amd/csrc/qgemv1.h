@@ -44,18 +44,46 @@
 //   PRO 3  one fp16 row of at most two pieces per thread
 //   PRO 6  PRO 3 for the expert gate/up jobs of one token with the gating done here: every workgroup computes scores and top-k from the
 //          router logits itself (64..1024 floats), so no selection has to cross workgroups inside the router's launch
+//   PRO 8  PRO 1 of the q / k / v launch of a decode step with a hint for the attention launch behind it: every lane also reads one dword of a cache
+//          line that the attention will ask for (kv_touch)
+//   PRO 7  the row is merged from the attention's split partials (one 8-element piece per thread), so the attention has no merge launch
 //   PRO 5  PRO 1 for a row of at most one piece per thread that is first completed as x + sum_j p_j y_j (the MoE weighted sum and block
 //          residual that precede the next block's attn_norm): the launch that would only add vectors disappears
 //
 // MR > 1 (several activation rows; instantiated for two; generic prologue, no fused SwiGLU): the same walk over the weights with MR sets of activations in registers;
 // a unit is decoded once and multiplied with every row.  Outputs and residuals are (MR, rows) per matrix.
 // bx: the workgroup's index among those of this matrix set (blockIdx.x where a launch serves one set, see qgemv1_two_kernel)
+// One dword of one line per lane for the attention launch that follows a q / k / v launch (QArgs::touch_*, prologue 8), branch-free: beyond the lines
+// there are a lane reads the last one again.  Workgroup bx runs on XCD bx % 8; the attention workgroups of kv head h run on
+// XCD h % 8 when the number of kv heads is a multiple of 8 (the host only asks then).  Lines of an XCD: K rows [0, pos) and V rows [0, pos) of each of its
+// heads, then the rotation row of pos; thread t of the XCD's workgroups takes line t.
+template <int NT>
+__device__ __forceinline__ uint32_t kv_touch(const QArgs& a, const unsigned bx, int pos) {
+  pos = pos < 0 ? 0 : pos > a.touch_max_ctx - 1 ? a.touch_max_ctx - 1 : pos;
+  const int x = bx & 7, t = (int)(bx >> 3) * NT + (int)threadIdx.x;
+  const int npl = (pos * a.touch_row_bytes + 127) >> 7;            // lines of the K (or V) rows below pos of one head
+  const int heads = (a.touch_n_kv - x + 7) >> 3, nrope = (a.touch_rope_row_bytes + 127) >> 7;
+  const int nkv = heads * 2 * npl, total = nkv + nrope;
+  const int idx = t < total ? t : total - 1;
+  const int hk = idx / (npl > 0 ? npl : 1), line = idx - hk * npl;
+  // (addresses by arithmetic, not by selects of pointers: a select between computed pointers can come out as a branch around the load, and a load
+  // behind a branch makes the compiler wait for every load in flight where the paths join)
+  const uintptr_t kb = (uintptr_t)a.touch_k, vb = (uintptr_t)a.touch_v;
+  const uintptr_t kvb = kb ^ ((kb ^ vb) & (uintptr_t)0 - (uintptr_t)(hk & 1));
+  const uintptr_t kvp = kvb + ((size_t)(x + 8 * (hk >> 1)) * a.touch_max_ctx * a.touch_row_bytes) + ((size_t)line << 7);
+  const uintptr_t rp = (uintptr_t)a.touch_rope + (size_t)pos * a.touch_rope_row_bytes + ((size_t)(idx >= nkv ? idx - nkv : 0) << 7);
+  const uintptr_t p = kvp ^ ((kvp ^ rp) & (uintptr_t)0 - (uintptr_t)(idx >= nkv));
+  return *(const __attribute__((address_space(1))) uint32_t*)p;   // (a global load: a flat one from an integer address would also count as an LDS operation)
+}
+
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
 __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx) {
   static_assert(MR == 1 || PRO == 0, "several activation rows: generic prologue");
   // A local copy: its field reads become kernel-argument loads in the entry block, where they merge into a few wide scalar loads
   // issued together (read at their points of use they arrive in dependent stages, each a scalar-cache miss of its own).
   const QArgs a = args;
+  int tpos = 0;
+  if constexpr (PRO == 8) tpos = *a.touch_pos;                    // (read at the kernel's entry: a scalar load whose miss the prologue hides)
   using F = Fmt<T>;
   typedef typename F::Raw Raw;
   static_assert(WK == 1 || WR == 1, "row teams and K split are not combined");
@@ -98,6 +126,7 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
   u32x4 xv[MR][F::XV]; float cv[MR][F::NG];
   const int nseg = (EPI == 2) ? 1 : a.nseg;
   int parity = 0;
+  uint32_t touched = 0;                                          // (prologue 8: the dword of the cache line this lane touches for the attention launch, see kv_touch)
 
   // ---- the segment (weight matrix) the team is in
   int seg = 0;
@@ -284,7 +313,7 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
     h.x = (h.x * nscale) * w1.x; h.y = (h.y * nscale) * w1.y; h.z = (h.z * nscale) * w1.z; h.w = (h.w * nscale) * w1.w;
     if ((int)threadIdx.x < nq) put_piece((int)threadIdx.x, pack8(l, h));
     lds_to_regs();
-  } else if constexpr (PRO == 1) {
+  } else if constexpr (PRO == 1 || PRO == 8) {
     f32x4 l4[2], h4[2], w0[2], w1[2];
 #pragma unroll
     for (int t = 0; t < NPC; t++) {
@@ -305,6 +334,7 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
     // the first weights go out only now, when every wave of the workgroup holds its activations: requested together with them, the weight
     // misses of the waves that started first sit in front of the activation reads of the waves that started last (8B decode 602 -> 609 tok/s)
     issue(b[0], lo);
+    if constexpr (PRO == 8) touched = kv_touch<NT>(a, bx, tpos);
     float tot = 0.f;
 #pragma unroll
     for (int j = 0; j < NT / 64; j++) tot += nred[j];
@@ -325,6 +355,37 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
 #pragma unroll
     for (int t = 0; t < NPC; t++) { const int i = (int)threadIdx.x + NT * t; if (i < nq) put_piece(i, v[t]); }
     __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 1)
+    issue(b[0], lo);
+    lds_to_regs();
+  } else if constexpr (PRO == 7) {
+    // the row is the merge of the attention's split partials (attn_split1_kernel): thread t merges elements 8t .. 8t + 7 of its head.  All loads are
+    // one batch (surplus splits reload split 0 with weight 0); a split without cached positions carries max = -inf, sum = 0.
+    const int i = (int)threadIdx.x < nq ? (int)threadIdx.x : nq - 1;
+    const int hd = 1 << a.attn_hd_log2, head = (8 * i) >> a.attn_hd_log2, d0 = 8 * i - (head << a.attn_hd_log2), ps = hd + 4;
+    const float* ph = (const float*)a.x + (size_t)head * a.attn_S * ps;
+    constexpr int MS = 6;                                        // most splits (surplus slots reload split 0 with weight 0)
+    f32x4 pl[MS], phh[MS]; float pm[MS], pls[MS];
+#pragma unroll
+    for (int sp = 0; sp < MS; sp++) {
+      const int sc = sp < a.attn_S ? sp : 0;
+      pl[sp] = *(const f32x4*)(ph + sc * ps + d0); phh[sp] = *(const f32x4*)(ph + sc * ps + d0 + 4);
+      pm[sp] = ph[sc * ps + hd]; pls[sp] = ph[sc * ps + hd + 1];
+    }
+    float mx = pm[0];
+#pragma unroll
+    for (int sp = 1; sp < MS; sp++) mx = fmaxf(mx, sp < a.attn_S ? pm[sp] : pm[0]);
+    f32x4 l = {0.f, 0.f, 0.f, 0.f}, h = {0.f, 0.f, 0.f, 0.f}; float lsum = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < MS; sp++) {
+      const float e = (sp < a.attn_S && pm[sp] != -INFINITY) ? __expf(pm[sp] - mx) : 0.f;
+      lsum += e * pls[sp];
+      l.x += e * pl[sp].x; l.y += e * pl[sp].y; l.z += e * pl[sp].z; l.w += e * pl[sp].w;
+      h.x += e * phh[sp].x; h.y += e * phh[sp].y; h.z += e * phh[sp].z; h.w += e * phh[sp].w;
+    }
+    const float inv = 1.0f / lsum;
+    l.x *= inv; l.y *= inv; l.z *= inv; l.w *= inv; h.x *= inv; h.y *= inv; h.z *= inv; h.w *= inv;
+    if ((int)threadIdx.x < nq) put_piece((int)threadIdx.x, pack8(l, h));
+    __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 3)
     issue(b[0], lo);
     lds_to_regs();
   } else if constexpr (PRO == 6) {
@@ -411,6 +472,7 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
   run_segment();
   // (a branch around loads is harmless here: the ring is empty between segments)
   for (int sg = 1; sg < nseg; sg++) { enter(sg); if (cnt) { issue(b[0], lo); run_segment(); } }
+  if constexpr (PRO == 8) asm volatile("" :: "v"(touched));      // the touch has to be a load that is used: an empty statement takes its register
 }
 
 template <int T, int R, int WK, int WR, int EPI, bool H, int PRO, int MR = 1>
@@ -420,19 +482,20 @@ __global__ __launch_bounds__(WK * WR * 64) void qgemv1_kernel(const QArgs args) 
 // tinygrad/llm/model.py:161-163 applies the three linears to one normalised row): the first `split` workgroups walk set a, the others set b.  Rows that one
 // wave covers, plain epilogue.
 // Behind the branch the compiler reads a set's fields from the kernel-argument segment where they are used: a dozen scalar loads, one after the other, each a
-// scalar-cache miss of its own (9.5 us for the 8B shape).  The entry block therefore reads one dword of every 64-byte line of the segment - ten independent loads,
+// scalar-cache miss of its own (9.5 us for the 8B shape).  The entry block therefore reads one dword of every 64-byte line of the segment - twelve independent loads,
 // one miss time together - so that the later ones hit.  The loads are inline assembly with their wait inside the statement: written in the source (one field per
 // line summed into an operand of an empty statement), they made the compiler allocate 256 registers and spill.
 template <int TA, int TB, int R, int WR, int PRO>
 __global__ __launch_bounds__(WR * 64) void qgemv1_two_kernel(const QArgs a, const QArgs b, const unsigned split) {
-  static_assert(2 * sizeof(QArgs) + sizeof(unsigned) > 0x240 && 2 * sizeof(QArgs) + sizeof(unsigned) <= 0x280, "ten lines of kernel arguments");
+  static_assert(2 * sizeof(QArgs) + sizeof(unsigned) > 0x2c0 && 2 * sizeof(QArgs) + sizeof(unsigned) <= 0x300, "twelve lines of kernel arguments");
   {
     const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
-    int t0, t1, t2, t3, t4, t5, t6, t7, t8, t9;
-    asm volatile("s_load_dword %0, %10, 0x0\n\ts_load_dword %1, %10, 0x40\n\ts_load_dword %2, %10, 0x80\n\ts_load_dword %3, %10, 0xc0\n\ts_load_dword %4, %10, 0x100\n\t"
-                 "s_load_dword %5, %10, 0x140\n\ts_load_dword %6, %10, 0x180\n\ts_load_dword %7, %10, 0x1c0\n\ts_load_dword %8, %10, 0x200\n\ts_load_dword %9, %10, 0x240\n\t"
+    int t0, t1, t2, t3, t4, t5, t6, t7, t8, t9, t10, t11;
+    asm volatile("s_load_dword %0, %12, 0x0\n\ts_load_dword %1, %12, 0x40\n\ts_load_dword %2, %12, 0x80\n\ts_load_dword %3, %12, 0xc0\n\ts_load_dword %4, %12, 0x100\n\t"
+                 "s_load_dword %5, %12, 0x140\n\ts_load_dword %6, %12, 0x180\n\ts_load_dword %7, %12, 0x1c0\n\ts_load_dword %8, %12, 0x200\n\ts_load_dword %9, %12, 0x240\n\t"
+                 "s_load_dword %10, %12, 0x280\n\ts_load_dword %11, %12, 0x2c0\n\t"
                  "s_waitcnt lgkmcnt(0)"
-                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9) : "s"(ka) : "memory");
+                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9), "=&s"(t10), "=&s"(t11) : "s"(ka) : "memory");
   }
   if (blockIdx.x < split) qgemv1_body<TA, R, 1, WR, 0, false, PRO>(a, blockIdx.x);
   else qgemv1_body<TB, R, 1, WR, 0, false, PRO>(b, blockIdx.x - split);
@@ -490,6 +553,13 @@ static int launch_fast(QArgs a, hipStream_t s) {
   const bool one_batch = a.K / 8 <= NT * (NT >= 512 ? 1 : 2);
   if constexpr (MR > 1) return launch_fast_p<T, R, WK, WR, EPI, H, 0, MR>(a, grid, lds, s);
   else {
+  if constexpr (EPI == 1 && WK == 1 && !H) {
+    if (a.attn_S > 0) {
+      if (a.K / 8 > NT || a.x_staged || !a.x_f32 || a.sel) return tga_set_error("tga_attn_merge_qlinear: needs one float32 partial row set of at most %d values", 8 * NT);
+      return launch_fast_p<T, R, WK, WR, EPI, H, 7>(a, grid, lds, s);
+    }
+  }
+  if (a.attn_S > 0) return tga_set_error("tga_attn_merge_qlinear: shape outside the fused path (K = %d)", a.K);
   if constexpr (EPI == 1) { if (a.x_staged) return launch_fast_p<T, R, WK, WR, EPI, H, 2>(a, grid, lds, s); }
   if constexpr (WK == 1 && EPI == 0) {
     if (a.comb_y) {
@@ -506,6 +576,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
   }
   if (a.route_logits) return tga_set_error("tga_qlinear_experts_routed: shape outside the routed path (K = %d)", a.K);
   if constexpr (WK == 1 && EPI != 1) {
+    if constexpr (EPI == 0 && !H) { if (!a.x_staged && one_batch && a.norm_w && a.x_f32 && a.touch_pos) return launch_fast_p<T, R, WK, WR, EPI, H, 8>(a, grid, lds, s); }
     if (!a.x_staged && one_batch && a.norm_w && a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 1>(a, grid, lds, s);
     if (!a.x_staged && one_batch && !a.norm_w && !a.x_f32) return launch_fast_p<T, R, WK, WR, EPI, H, 3>(a, grid, lds, s);
   }

@@ -215,6 +215,13 @@ class TransformerBlock:
     self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
                             and 0 < c.n_summands <= 8 and self.qkv_bias is None
     if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
+    # The attention as one launch whose split partials attn_output merges (no q / k norm, cache of at most 2048 positions, attn_output rows of 33..64 units)
+    ns = ctypes.c_int(0)
+    rt.check(rt.lib().tga_attention_split_plan(c.max_context, ctypes.byref(ns)))
+    ao = self.attn_output
+    self.fused_attn = ns.value if (os.environ.get("TGA_ATTN", "fused") == "fused" and not c.qk_norm and fast(ao) and ao.ggml_type != rt.MXFP4
+                                   and 2048 < ao.in_features <= 4096 and ao.in_features == c.n_heads * c.head_dim) else 0
+    self.kv_touch = os.environ.get("TGA_KV_TOUCH", "1") == "1" and c.n_kv_heads % 8 == 0      # the q / k / v launch touches the cache rows for the attention launch
 
   def __call__(self, x: Buffer, stream, pending: int = 0, defer: bool = False) -> tuple[Buffer, int]:
     """One block on the residual row x.  pending > 0: the previous (MoE) block left its weighted sum over that many rows + residual to this block
@@ -240,14 +247,22 @@ class TransformerBlock:
         j = i + 1
         while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
         bias = dict(epilogue=1, resid=self.qkv_bias[i:j]) if self.qkv_bias is not None else {}
-        if self.fuse_norm: qlinear_multi(qkv[i:j], x, qkv_out[i:j], stream=stream, norm=(self.attn_norm, c.norm_eps), **bias)
+        touch = (s.state, self.cache_k, self.cache_v, s.rope, c.n_kv_heads, c.head_dim, c.max_context) if (self.kv_touch and j == 3) else None
+        if self.fuse_norm: qlinear_multi(qkv[i:j], x, qkv_out[i:j], stream=stream, norm=(self.attn_norm, c.norm_eps), touch=touch, **bias)
         else: qlinear_multi(qkv[i:j], s.xn, qkv_out[i:j], stream=stream, **bias)
         i = j
     # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
-    rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
-                                           int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
-                                           s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if self.stage_attn else 0, stream))
-    qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_attn)
+    if self.fused_attn:
+      # one launch leaves split partials, attn_output merges them while it stages its row (no merge launch)
+      rt.check(L.tga_attention_decode_split(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim,
+                                            c.max_context, s.rope.ptr, stream))
+      ao = self.attn_output
+      rt.check(L.tga_attn_merge_qlinear(ao.ggml_type, ao.blocks.ptr, x.ptr, ao.out_features, ao.in_features, x.ptr, s.attn_part.ptr, self.fused_attn, c.head_dim, stream))
+    else:
+      rt.check(L.tga_attention_decode_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
+                                             int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim, c.max_context,
+                                             s.rope.ptr, s.attn.ptr, None, self.attn_output.ggml_type if self.stage_attn else 0, stream))
+      qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_attn)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     if not self.moe:
       if self.fuse_norm:
@@ -306,7 +321,7 @@ class _Shared:
     self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v
     self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
-    self.attn_part = Buffer((c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
+    self.attn_part = Buffer((c.n_heads * max(((c.max_context + 63) // 64) * (c.head_dim + 2), 6 * (c.head_dim + 4)),), f32).zero_()   # (two-launch layout or up to six split partials)
     self.act = Buffer((1, max(c.hidden_dim, c.dense_hidden_dim)), f16)
     if c.num_experts:
       k = c.num_experts_per_tok

@@ -43,7 +43,7 @@ def qlinear_mixed(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], norm
 
 def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epilogue: int = 0, resid: list[Buffer] | None = None, stream=None,
                   x_staged: bool = False, stage_out_for: QuantLinear | None = None, norm: tuple[Buffer, float] | None = None,
-                  combine: tuple[Buffer, Buffer, int, Buffer] | None = None):
+                  combine: tuple[Buffer, Buffer, int, Buffer] | None = None, touch: tuple | None = None):
   """Several QuantLinear layers over the same activation in one launch (attn_q/k/v, ffn_gate/ffn_up).
   epilogue 0: plain; 1: outs[i] = resid[i] + linear; 2: outs[0] = silu(layers[0](x)) * layers[1](x).
   x_staged: x is already in the staged order of these weights (stage_activation or a staging producer).
@@ -51,7 +51,8 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   norm = (weight, eps): x is one float32 row and RMSNorm(x) * weight is applied while the kernel stages it; norm = (weight, eps, scratch) for several
   float32 rows (scratch: an fp16 buffer of x's shape that receives the normalised rows when the kernel at hand cannot fold the norm).
   combine = (y, probs, k, x_out) with norm: the row is first completed as x + sum_j probs[j] * y[j] (the MoE weighted sum + residual) and
-  the completed row is written to x_out (a buffer other than x)."""
+  the completed row is written to x_out (a buffer other than x).
+  touch = (state, cache_k, cache_v, rope table, n_kv_heads, head_dim, max_context) with norm: the launch also touches what the attention launch behind it reads first."""
   nseg = len(layers)
   t, k = layers[0].ggml_type, layers[0].in_features
   assert all(l.ggml_type == t and l.in_features == k for l in layers)
@@ -71,6 +72,11 @@ def qlinear_multi(layers: list[QuantLinear], x: Buffer, outs: list[Buffer], epil
   if norm is not None and len(norm) == 3:                                # rows with a scratch: one launch where the LDS-fed kernel folds the norm in, else norm + linears
     assert x.dtype == np.float32 and not x_staged and so is None and len(norm) == 3, "norm = (weight, eps, fp16 scratch of x's shape) for several rows"
     rt.check(rt.lib().tga_rmsnorm_qlinear_rows(norm[0].ptr, norm[1], t, nseg, w, y, n, x.ptr, norm[2].ptr, ydt, m, k, epilogue, r, stream))
+    return outs
+  if norm is not None and touch is not None and so is None:              # touch = (state, cache_k, cache_v, rope table, n_kv_heads, head_dim, max_context)
+    assert m == 1 and x.dtype == np.float32 and not x_staged
+    rt.check(rt.lib().tga_rmsnorm_qlinear_multi_touch(norm[0].ptr, norm[1], t, nseg, w, y, n, x.ptr, ydt, k, epilogue, r, touch[0].ptr, touch[1].ptr, touch[2].ptr, touch[3].ptr,
+                                                      touch[4], touch[5], touch[6], stream))
     return outs
   if norm is not None:
     assert m == 1 and x.dtype == np.float32 and not x_staged
