@@ -84,7 +84,7 @@ def parity_gate(model, c, threads):
   fc = ollm.precompute_freqs_cis(hd, pos + 1, c.rope_theta)[pos]
   emb_row_bytes = model.token_embd.nbytes // c.vocab_size
   from oracle import ggml as og
-  xr = og.ggml_data_to_tensor(model.token_embd.view(tok * emb_row_bytes, (emb_row_bytes,), np.uint8).numpy(), c.dim, model.embd_type).astype(np.float32)
+  xr = og.ggml_data_to_tensor(model.token_embd.view(tok * emb_row_bytes, (emb_row_bytes,), np.uint8).numpy(), c.dim, model.embd_type).astype(np.float16).astype(np.float32)   # the table is an fp16 weight (model.py:376)
   cpu_s = 0.0                                                    # CPU time of the recomputed step itself (weights and KV rows already copied to the host)
   for i, b in enumerate(model.blk):
     hl = _host_layer(model, i)

@@ -46,7 +46,7 @@ int tga_memcpy_d2h(void* dst, const void* src, size_t n);  /* ops_hip.py:67-69, 
 int tga_memcpy_d2d(void* dst, const void* src, size_t n, void* stream);
 /* device-to-device copy done by a plain kernel (n bytes, 16-byte aligned): a known-size yardstick for hardware traffic counters. */
 int tga_copy_kernel(void* dst, const void* src, size_t n, void* stream);
-int tga_memset(void* dst, int value, size_t n, void* stream);
+int tga_memset(void* dst, int value, size_t n, void* stream);   /* hipMemsetAsync; refused (error) on a stream that is capturing */
 int tga_sync(void);                                        /* ops_hip.py:22-24 hipDeviceSynchronize */
 int tga_stream_create(void** stream);
 int tga_stream_destroy(void* stream);
@@ -187,7 +187,7 @@ int tga_moe_combine(const float* y, const float* probs, const float* resid, int 
  * and did nothing.  The caller checks and clears it after synchronising. */
 
 /* token_embd(tokens).float() for the token in state (model.py:359): dequantizes one row of a Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q8_0 /
- * Q4_K / Q5_K / Q6_K / MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant). */
+ * Q4_K / Q5_K / Q6_K / MXFP4 / F16 / F32 table (bit-exact block decode, as tga_dequant, rounded to fp16: the reference's table is an fp16 weight, model.py:376). */
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream);
 
 /* nn.RMSNorm (tinygrad/nn/__init__.py:296-304): (x * rsqrt(mean(x^2) + eps)) * weight; writes fp16 and/or fp32 (either may be NULL).

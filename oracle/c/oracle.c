@@ -11,6 +11,7 @@
 #include <string.h>
 #include <math.h>
 #include <stdlib.h>
+#include <immintrin.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -39,6 +40,12 @@ static inline uint16_t f2h(float f) {
   if (e < -14) return (uint16_t)(s | r);                           /* subnormal (r may carry into exponent 1: fine) */
   return (uint16_t)(s | (((uint32_t)(e + 15) << 10) + (r - 0x400u)));
 }
+/* x[i] = float32(float16(x[i])), round-to-nearest-even, n a multiple of 8: the F16C conversions (part of the x86-64-v3 baseline this file is built for), which
+ * tests/test_oracle_ggml.py holds against the bit-level f2h / h2f above.  The per-weight software round trip was most of orc_linear's time. */
+static inline void round_f16_block(float* x, int n) {
+  for (int j = 0; j < n; j += 8) _mm256_storeu_ps(x + j, _mm256_cvtph_ps(_mm256_cvtps_ph(_mm256_loadu_ps(x + j), _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC)));
+}
+void orc_round_f16(float* x, int64_t n) { for (int64_t j = 0; j + 8 <= n; j += 8) round_f16_block(x + j, 8); for (int64_t j = n & ~(int64_t)7; j < n; j++) x[j] = h2f(f2h(x[j])); }
 float orc_h2f(uint16_t h) { return h2f(h); }
 uint16_t orc_f2h(float f) { return f2h(f); }
 
@@ -256,7 +263,7 @@ int orc_linear(int ggml_type, const uint8_t* w, const void* x, float* y, int M, 
     const uint8_t* row = w + n * bpr * nby;
     for (int64_t b = 0; b < bpr; b++) {
       deq_block(ggml_type, row + b * nby, wb);
-      if (w_round_f16) for (int j = 0; j < nel; j++) wb[j] = h2f(f2h(wb[j]));
+      if (w_round_f16) round_f16_block(wb, nel);
       for (int m = 0; m < M; m++) {
         const float* xr = xf + (int64_t)m * K + b * nel; float a = acc[m];
         if (prod_round_f16) for (int j = 0; j < nel; j++) a += h2f(f2h(xr[j] * wb[j]));

@@ -18,6 +18,7 @@ def lib():
     _lib.orc_dequant.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int]
     _lib.orc_linear.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
                                 ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    _lib.orc_round_f16.argtypes, _lib.orc_round_f16.restype = [ctypes.c_void_p, ctypes.c_int64], None
     _lib.orc_h2f.restype, _lib.orc_h2f.argtypes = ctypes.c_float, [ctypes.c_uint16]
     _lib.orc_f2h.restype, _lib.orc_f2h.argtypes = ctypes.c_uint16, [ctypes.c_float]
   return _lib
@@ -42,6 +43,12 @@ def linear(ggml_type: int, w: np.ndarray, x: np.ndarray, n: int, k: int, w_round
   rc = lib().orc_linear(ggml_type, w.ctypes.data, x.ctypes.data, y.ctypes.data, x.shape[0], n, k,
                         int(x.dtype == np.float16), int(w_round_f16), int(prod_round_f16), threads)
   assert rc == 0, rc
+  return y
+
+def round_f16(x: np.ndarray) -> np.ndarray:
+  """float32 -> nearest fp16 -> float32 through the conversion orc_linear uses for its weights."""
+  y = np.ascontiguousarray(x, dtype=np.float32).copy()
+  lib().orc_round_f16(y.ctypes.data, y.size)
   return y
 
 def max_threads() -> int: return lib().orc_max_threads()

@@ -41,10 +41,32 @@ def gate_probs(logits: np.ndarray, k: int, gating=SOFTMAX, norm_topk_prob=False,
   elif gating == SIGMOID: scores = 1.0 / (1.0 + np.exp(-logits))
   else: scores = np.sqrt(np.log1p(np.exp(logits)))
   _, sel = pairwise_topk(scores if bias is None else scores + bias, k)
+  return sel, selection_probs(scores, sel, gating, norm_topk_prob, scale)
+
+def selection_probs(scores: np.ndarray, sel: np.ndarray, gating, norm_topk_prob, scale) -> np.ndarray:
+  """The weights of a given selection (model.py:124-128): the selected scores, softmaxed over the selection for SOFTMAX_WEIGHT, optionally normalised
+  to sum 1, times the routed scaling factor.  gating / norm_topk_prob as gate_probs has resolved them."""
   probs = np.take_along_axis(scores, sel, axis=-1)
   if gating == SOFTMAX_WEIGHT: probs = softmax(probs)
   if norm_topk_prob: probs = probs / probs.sum(axis=-1, keepdims=True)
-  return sel, (probs * scale).astype(np.float32)
+  return (probs * scale).astype(np.float32)
+
+def follow_selection(logits: np.ndarray, forced, k: int, gating=SOFTMAX, norm_topk_prob=False, scale=1.0, tie=0.0):
+  """gate_probs of one token's router logits (E,), except that a given selection is adopted where it differs from the own top-k only in experts whose
+  router logits lie within `tie` of each other (a near-tie may fall either way between two correct implementations).  Returns (sel (k,), probs (k,),
+  followed: the own selection was replaced).  Raises when the given selection differs beyond that."""
+  logits = logits.astype(np.float32)
+  sel, probs = gate_probs(logits[None, :], k, gating, norm_topk_prob, scale)
+  forced = np.asarray(forced).astype(np.int64).reshape(-1)
+  if set(forced.tolist()) == set(sel[0].tolist()): return sel[0], probs[0], False
+  diff = sorted(set(forced.tolist()) ^ set(sel[0].tolist()))
+  spread = float(logits[diff].max() - logits[diff].min())
+  if len(forced) != k or len(set(forced.tolist())) != k or spread > tie:
+    raise AssertionError(f"expert selection {sorted(forced.tolist())} differs from the own {sorted(sel[0].tolist())} beyond a near-tie: router logits of {diff} spread {spread:.3e} > {tie:.1e}")
+  if gating == SOFTMAX and norm_topk_prob: gating, norm_topk_prob = SOFTMAX_WEIGHT, False
+  scores = gate_scores(logits, gating)
+  order = np.array(sorted(forced.tolist(), key=lambda e: (scores[e], -e)), dtype=np.int32)      # ascending, the lower index ranks higher among equals
+  return order, selection_probs(scores[None, :], order[None, :], gating, norm_topk_prob, scale)[0], True
 
 def silu(x): return x * (1.0 / (1.0 + np.exp(-x)))
 

@@ -172,13 +172,14 @@ def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
   assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
 
 def test_command_list_takes_kernel_launches_only(gpu):
-  """A capture that holds anything but kernel launches (here a memset) is refused when the list is built; the stream stays usable."""
+  """A capture that holds anything but kernel launches (here a device-to-device copy, which the capture records as a copy node; the graph is never
+  instantiated) is refused when the list is built; the stream stays usable."""
   from tinygrad_amd import runtime as rt
   s = rt.Stream()
-  buf = gpu.Buffer((256,), np.float32)
+  buf, src = gpu.Buffer((256,), np.float32), gpu.Buffer((256,), np.float32).zero_()
   cl = rt.CommandList(s)
   with pytest.raises(RuntimeError, match="not a kernel launch"):
-    with cl: gpu.check(gpu.lib().tga_memset(buf.ptr, 0, buf.nbytes, s.handle))
+    with cl: gpu.check(gpu.lib().tga_memcpy_d2d(buf.ptr, src.ptr, buf.nbytes, s.handle))
   ok = rt.CommandList(s)
   with ok: gpu.check(gpu.lib().tga_synth_weights(0, buf.ptr, 256, 1, 3.0, s.handle))    # a fill kernel: float32 "weights" are a constant fill
   assert len(ok) == 1

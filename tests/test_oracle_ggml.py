@@ -297,3 +297,16 @@ def test_fp16_conversions_exhaustive():
   xs = (rng.standard_normal(5000) * np.float32(10.0) ** rng.integers(-9, 6, 5000)).astype(np.float32)
   with np.errstate(over="ignore"): exp = xs.astype(np.float16).view(np.uint16)
   assert all(L.orc_f2h(float(v)) == int(e) for v, e in zip(xs, exp))
+
+def test_c_vector_f16_rounding_equals_the_bit_level_conversion():
+  """orc_linear rounds its dequantized weights to fp16 with the CPU's conversion instructions; the bit-level f2h / h2f of the same file (checked against numpy
+  above) must give the same float for normals, subnormals, ties, overflow and signed zeros."""
+  rng = np.random.default_rng(11)
+  xs = np.concatenate([rng.standard_normal(4096).astype(np.float32) * s for s in (1e-8, 1e-5, 1e-3, 1.0, 300.0, 7e4)] +
+                      [np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, -65520.0, 2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25, 2.0 ** -14, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 5.9604645e-08], np.float32)])
+  got = cref.round_f16(xs)
+  with np.errstate(over="ignore"): want = xs.astype(np.float16).astype(np.float32)
+  assert got.tobytes() == want.tobytes()
+  L = cref.lib()
+  sw = np.array([L.orc_h2f(L.orc_f2h(float(v))) for v in xs[-64:]], np.float32)
+  assert sw.tobytes() == got[-64:].tobytes()

@@ -12,14 +12,14 @@
 
 // ---------------------------------------------------------------------------------------------- embedding (one row of any table type)
 // token_embd(tokens).float() for one token: tinygrad/llm/model.py:359.  The table stays in GGUF blocks; only the row is dequantized
-// (bit-exact block decode shared with tga_dequant).
+// (bit-exact block decode shared with tga_dequant, then rounded to fp16: the reference casts the table to fp16 like every weight, model.py:376).
 template <int T>
 __device__ __forceinline__ void embed_row_blocks(const uint8_t* __restrict__ table, int dim, int tok, float* __restrict__ out) {
   const uint8_t* row = table + (size_t)tok * (dim / Deq<T>::NEL) * Deq<T>::NBY;
   for (int e = threadIdx.x * 4; e < dim; e += 1024) {
     float o[4];
     Deq<T>::get4(row + (size_t)(e / Deq<T>::NEL) * Deq<T>::NBY, e % Deq<T>::NEL, o);
-    out[e] = o[0]; out[e + 1] = o[1]; out[e + 2] = o[2]; out[e + 3] = o[3];
+    out[e] = (float)(_Float16)o[0]; out[e + 1] = (float)(_Float16)o[1]; out[e + 2] = (float)(_Float16)o[2]; out[e + 3] = (float)(_Float16)o[3];
   }
 }
 __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restrict__ table, int ggml_type, int dim, DecodeState* st, float* __restrict__ out,
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
     case GGML_Q6_K: embed_row_blocks<GGML_Q6_K>(table, dim, tok, out); break;
     case GGML_MXFP4: embed_row_blocks<GGML_MXFP4>(table, dim, tok, out); break;
     case GGML_F16: { const uint16_t* row = (const uint16_t*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = h2f_bits(row[e]); break; }
-    default: { const float* row = (const float*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = row[e]; }
+    default: { const float* row = (const float*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = (float)(_Float16)row[e]; }
   }
 }
 

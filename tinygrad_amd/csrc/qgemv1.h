@@ -385,8 +385,8 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
     const float inv = 1.0f / lsum;
     l.x *= inv; l.y *= inv; l.z *= inv; l.w *= inv; h.x *= inv; h.y *= inv; h.z *= inv; h.w *= inv;
     if ((int)threadIdx.x < nq) put_piece((int)threadIdx.x, pack8(l, h));
-    __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 3)
-    issue(b[0], lo);
+    __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 3; requested
+    issue(b[0], lo);                                             // in front of the partials they cost 2 % of the decode step)
     lds_to_regs();
   } else if constexpr (PRO == 6) {
     __shared__ float tk_lg[1024], tk_sc[1024], tk_tmp[192], tk_p[64];

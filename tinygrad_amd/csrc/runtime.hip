@@ -55,7 +55,15 @@ int tga_copy_kernel(void* dst, const void* src, size_t n, void* stream) {
   TGA_LAUNCH_CHECK();
   return 0;
 }
-int tga_memset(void* dst, int value, size_t n, void* stream) { TGA_HIP(hipMemsetAsync(dst, value, n, (hipStream_t)stream)); return 0; }
+// (refused while the stream is capturing: a memset node in a replayed graph has given wrong results on this platform; captured code clears with a fill kernel)
+int tga_memset(void* dst, int value, size_t n, void* stream) {
+  if (stream) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    TGA_HIP(hipStreamIsCapturing((hipStream_t)stream, &cs));
+    TGA_REQUIRE(cs == hipStreamCaptureStatusNone, "tga_memset: the stream is capturing; use a fill kernel inside a capture");
+  }
+  TGA_HIP(hipMemsetAsync(dst, value, n, (hipStream_t)stream)); return 0;
+}
 int tga_sync(void) { TGA_HIP(hipDeviceSynchronize()); return 0; }
 
 int tga_stream_create(void** stream) { TGA_HIP(hipStreamCreate((hipStream_t*)stream)); return 0; }   // default priority only

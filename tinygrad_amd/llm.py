@@ -368,7 +368,9 @@ class Transformer:
       raise RuntimeError(f"decode state error {err}: " + ", ".join(m for b, m in ((1, "token id outside the vocabulary"), (2, "position beyond max_context")) if err & b))
 
   # one token through all blocks; with_head adds output_norm + output + argmax (model.py:358-364)
-  def _step(self, with_head: bool):
+  def _step(self, with_head: bool, on_block=None):
+    """The launches of one token.  on_block(i): called when block i's launches have been issued (eager stepping only; e.g. to read back s.sel, the
+    experts block i selected, after a synchronisation)."""
     c, s, L, st = self.config, self.s, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_row(self.token_embd.ptr, self.embd_type, c.dim, s.state.ptr, s.x.ptr, st))
     x, pending = s.x, 0
@@ -376,6 +378,7 @@ class Transformer:
     for i, b in enumerate(self.blk):
       nxt = self.blk[i + 1].can_fold_combine if i + 1 < nb else (with_head and self.can_fold_head)
       x, pending = b(x, st, pending, defer=nxt)
+      if on_block is not None: on_block(i)
     if with_head:
       if pending:                                                      # the last block's weighted sum completed inside the lm-head launch
         x_new = s.x2 if x.ptr == s.x.ptr else s.x
@@ -413,6 +416,8 @@ class Transformer:
     head_dim = kv.get(f"{arch}.attention.key_length_mla", kv.get(f"{arch}.attention.key_length", dim // n_heads))
     num_blocks = kv[f"{arch}.block_count"] - kv.get(f"{arch}.nextn_predict_layers", 0)     # trailing next-token-prediction layers are not part of the decoder (model.py:424)
     rope_dim = kv.get(f"{arch}.rope.dimension_count", head_dim)
+    v_head_dim = kv.get(f"{arch}.attention.value_length_mla", kv.get(f"{arch}.attention.value_length", head_dim))     # model.py from_gguf: v_head_dim
+    if v_head_dim != head_dim: raise NotImplementedError(f"value heads of {v_head_dim} values beside key heads of {head_dim} are not built")
     if rope_dim != head_dim and (arch == "llama" or rope_dim % 2 or (head_dim - rope_dim) % 2 or not 0 < rope_dim < head_dim):
       raise NotImplementedError(f"rope dimension {rope_dim} of head_dim {head_dim} for architecture {arch} is not built")
     if kv.get(f"{arch}.attention.kv_lora_rank", 0) or arch in ("qwen35", "qwen35moe", "kimi-linear"): raise NotImplementedError(f"architecture {arch} is outside the built path")
@@ -487,12 +492,14 @@ class Transformer:
     self._n_prompt, self._steps_done = len(tokens), start_pos
     self._cached_tokens = list(tokens[:start_pos])
 
-  def prefill(self, tokens: list[int], use_graph: bool = True, reuse_cache: bool = True):
+  def prefill(self, tokens: list[int], use_graph: bool = True, reuse_cache: bool = True, on_block=None):
     """Feeds all but the last prompt token (KV cache fill); the last one is consumed by the first decode step.  Like the reference's generate
-    (model.py:472-473) the positions whose tokens equal what the cache already holds are not recomputed."""
+    (model.py:472-473) the positions whose tokens equal what the cache already holds are not recomputed.  on_block: token by token with eager launches,
+    on_block(i) after the launches of block i of every position (see _step)."""
     start = self.get_start_pos(tokens) if reuse_cache else 0
     self.prefill_steps = len(tokens) - 1 - start                        # (positions the last call actually computed)
-    B = self.prefill_chunk
+    self._cached_tokens = self._cached_tokens[:start]                   # the rows from here on are about to be overwritten: if a step below raises, they are not claimed
+    B = self.prefill_chunk if on_block is None else 1
     if B > 16 and self.config.num_experts: B = 16                       # (MoE blocks keep steps of sixteen positions: longer ones are not measured there)
     # Whole chunks as small-batch steps (model.py:476-481) of the largest size that the prompt holds (the chosen one, else 32, 16, 8 or 4 positions).  Dense models: what
     # they leave is ONE more chunk that ends at the last position and computes some positions again - every row of a step depends on the cache and on its own token
@@ -514,19 +521,19 @@ class Transformer:
         break
     self.reset(tokens, start)
     for _ in range(len(tokens) - 1 - start):
-      if use_graph: self._graph(False).launch()
-      else: self._step(False)
+      if use_graph and on_block is None: self._graph(False).launch()
+      else: self._step(False, on_block)
     self._steps_done = len(tokens) - 1
     self._cached_tokens = list(tokens[:-1])
     self._last_input = tokens[-1]
     self.stream.synchronize()
 
-  def decode_step(self, use_graph: bool = True, sync: bool = True):
+  def decode_step(self, use_graph: bool = True, sync: bool = True, on_block=None):
     """One token.  The position it occupies must exist in the KV cache and the rotation table: like the reference's generate loop
-    (`while len(tokens) < self.max_context`, tinygrad/llm/model.py:475) the sequence ends at max_context."""
+    (`while len(tokens) < self.max_context`, tinygrad/llm/model.py:475) the sequence ends at max_context.  on_block: eager launches with that hook (see _step)."""
     if self._steps_done >= self.config.max_context: raise RuntimeError(f"context full: position {self._steps_done} is beyond max_context {self.config.max_context}")
-    if use_graph: self._graph(True).launch()
-    else: self._step(True)
+    if use_graph and on_block is None: self._graph(True).launch()
+    else: self._step(True, on_block)
     self._steps_done += 1
     self._cached_tokens.append(self._last_input); self._last_input = None    # this step wrote its input token's keys and values; the next input is on the device
     if sync: self.stream.synchronize()
@@ -630,7 +637,7 @@ class BatchedTransformer:
 
   def _linear(self, layers, x, outs, **kw): qlinear_multi(layers, x, outs, stream=self.stream.handle, **kw)
 
-  def _step(self, with_head: bool):
+  def _step(self, with_head: bool, on_block=None):
     c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
     rt.check(L.tga_embed_rows(self.token_embd.ptr, self.embd_type, c.dim, self.tokens.ptr, B, self.state.ptr, self.x.ptr, st))
     # The weighted sum over a block's selected experts plus its residual (model.py:130, 150) is completed by the NEXT norm's launch (the next block's attn_norm
@@ -641,7 +648,8 @@ class BatchedTransformer:
       if pending: rt.check(L.tga_moe_combine_rmsnorm_rows(self.y_e.ptr, self.probs.ptr, self.x.ptr, weight.ptr, B, c.num_experts_per_tok, c.dim, c.norm_eps, self.xn.ptr, None, st))
       else: rt.check(L.tga_rmsnorm_rows(self.x.ptr, weight.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       pending = False
-    for b in self.blk:
+    done = (lambda i: on_block(i)) if on_block is not None else (lambda i: None)     # on_block(i): block i's launches have been issued (eager stepping only; e.g. to read back self.sel)
+    for bi, b in enumerate(self.blk):
       # h = x + attention(attn_norm(x))                                                   model.py:149
       qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
       # the norm inside the launch where the kernel can: always for one run of equal block types (the call norms first where it cannot), for several runs
@@ -670,7 +678,7 @@ class BatchedTransformer:
       if not b["moe"]:
         self._linear([b["ffn_gate"], b["ffn_up"]], self.x, [self.act], epilogue=2, norm=(b["ffn_norm"], c.norm_eps, self.xn))
         self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
-        continue
+        done(bi); continue
       k = c.num_experts_per_tok                                         # model.py:110-135
       if not fused_router: b["router"](self.xn, out=self.router_logits, stream=st)
       self_gated = self.expert_path != "grouped" and b["sel_bias"] is None and self.xn.dtype == np.float16 and c.dim <= 4096   # the gate/up launch gates for itself (as the batch-1 step does)
@@ -685,7 +693,7 @@ class BatchedTransformer:
         route = (self.router_logits, c.expert_gating_func, c.norm_topk_prob, c.routed_scaling_factor, self.probs) if self_gated else None
         b["gate_exps"](self.sel, self.xn, self.act_e, jobs_per_x_row=k, up=b["up_exps"], stream=st, route=route)
         b["down_exps"](self.sel, self.act_e, self.y_e, jobs_per_x_row=1, stream=st)
-      if not c.shared_expert_dim: pending = True; continue            # x + sum_j p_j y_j: left to the next norm's launch
+      if not c.shared_expert_dim: pending = True; done(bi); continue  # x + sum_j p_j y_j: left to the next norm's launch
       moe_combine(self.y_e, self.probs, self.x, B, k, c.dim, self.x, stream=st)
       if c.shared_expert_dim:                                            # + shared expert, each row scaled by 1 or by sigmoid(xn . ffn_gate_inp_shexp)
         self._linear([b["ffn_gate_shexp"], b["ffn_up_shexp"]], self.xn, [self.act_sh], epilogue=2)
@@ -694,6 +702,7 @@ class BatchedTransformer:
           b["gate_inp_shexp"](self.xn, out=self.sh_logit, stream=st)
           moe_gate(self.sh_logit, B, 1, 1, self.sh_sel, self.p_sh, 2, False, 1.0, stream=st)
         moe_combine(self.y_sh, self.p_sh, self.x, B, 1, c.dim, self.x, stream=st)
+      done(bi)
     if with_head:                                                        # output(output_norm(x)) and the greedy token of every sequence, model.py:362-364
       if pending or not 2 <= B <= 8: norm(self.output_norm); self.output(self.xn, out=self.logits_buf, stream=st)
       else: self._linear([self.output], self.x, [self.logits_buf], norm=(self.output_norm, c.norm_eps, self.xn))
@@ -733,7 +742,7 @@ class BatchedTransformer:
     self.check_state()
     return n_chunks * B
 
-  def prefill(self, prompts: list[list[int]], use_graph: bool = True):
+  def prefill(self, prompts: list[list[int]], use_graph: bool = True, on_block=None):
     c, B = self.config, self.batch
     n = len(prompts[0])
     if len(prompts) != B or any(len(p) != n for p in prompts): raise ValueError(f"need {B} prompts of equal length")
@@ -745,15 +754,15 @@ class BatchedTransformer:
     st = np.zeros(16, np.int32); st[3], st[5] = n, c.vocab_size
     self.state.copyin(st)
     for _ in range(n - 1):
-      if use_graph: self._graph(False).launch()
-      else: self._step(False)
+      if use_graph and on_block is None: self._graph(False).launch()
+      else: self._step(False, on_block)
     self._steps_done = n - 1
     self.stream.synchronize()
 
-  def decode_step(self, use_graph: bool = True, sync: bool = True):
+  def decode_step(self, use_graph: bool = True, sync: bool = True, on_block=None):
     if self._steps_done >= self.config.max_context: raise RuntimeError(f"context full: position {self._steps_done} is beyond max_context {self.config.max_context}")
-    if use_graph: self._graph(True).launch()
-    else: self._step(True)
+    if use_graph and on_block is None: self._graph(True).launch()
+    else: self._step(True, on_block)
     self._steps_done += 1
     if sync: self.stream.synchronize()
 
@@ -768,6 +777,9 @@ class BatchedTransformer:
   def check_state(self):
     err = int(self.state.numpy()[4])
     flags = int(self.job_flags.numpy()[0]) if self.config.num_experts else 0
-    if err or flags: raise RuntimeError(f"batched decode refused an input: state error {err}, expert grouping flags {flags}")
+    if err or flags:                                                    # cleared before raising, so that the next check reports the next steps only
+      st = self.state.numpy(); st[4] = 0; self.state.copyin(st)
+      if flags: self.job_flags.zero_()
+      raise RuntimeError(f"batched decode refused an input: state error {err}, expert grouping flags {flags}")
 
   def logits(self) -> np.ndarray: return self.logits_buf.numpy()

@@ -3,7 +3,7 @@
 Mirrors the reference's HIP device glue (tinygrad/runtime/ops_hip.py:9-70): a non-zero status becomes RuntimeError with the
 library's message, buffers are explicit device allocations owned by the Python side."""
 from __future__ import annotations
-import ctypes, pathlib
+import ctypes, os, pathlib
 import numpy as np
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, MXFP4 = 0, 1, 2, 8, 12, 13, 14, 39
@@ -17,7 +17,7 @@ GGML_DEQUANT_ONLY = {IQ3_XXS: (256, 98), IQ3_S: (256, 110), IQ2_S: (256, 82), IQ
 GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), MXFP4: (32, 17)}
 _NP_DTYPE = {F32: np.float32, F16: np.float16}
 
-_LIB_PATH = pathlib.Path(__file__).resolve().parent / "libtinygrad_amd.so"
+_LIB_PATH = pathlib.Path(os.environ.get("TGA_LIB") or pathlib.Path(__file__).resolve().parent / "libtinygrad_amd.so")   # (TGA_LIB: another build of the same library)
 _lib = None
 _initialised = False
 
