@@ -152,7 +152,9 @@ def config8(steps: int = 32, ctx: int = 1024):
     del bm
   return res
 
-def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
+def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True, gate=None):
+  """gate(model, state dict, config) -> dict: called with the timed batch-1 model and the timed eight-sequence model after their runs; its result is reported
+  with the figures (bench.py passes a one-step check against the CPU restatement; this package itself holds no checker)."""
   from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state_moe, OLMOE
   import time
   c = TransformerConfig(max_context=((ctx + steps + 16 + 63) // 64) * 64, **OLMOE)
@@ -171,6 +173,7 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
   res = [{"config": 4, "case": f"OLMoE-arch decode B=1 ctx {ctx} (MXFP4 experts exponents 119..123, fp16 dense weights, {'graph replay' if use_graph else 'eager launches'} + sync per token)",
           "tok_s": round(1.0 / dt, 1), "ms_per_token": round(dt * 1e3, 4), "expert_bytes_per_token": expert_bytes, "weight_bytes_per_token": model.weight_bytes_per_token(),
           "weight_GBps_over_step": round(model.weight_bytes_per_token() / dt / 1e9, 1)}]
+  if gate is not None: res[0]["parity"] = gate(model, model_sd, c)
   # batched decode: B sequences in lockstep (dense linears as small-batch GEMMs, one expert GEMV per (sequence, slot) job)
   from tinygrad_amd.llm import BatchedTransformer
   sd = {k: v for k, v in model_sd.items()}
@@ -187,6 +190,7 @@ def config4(steps: int = 64, ctx: int = 512, use_graph: bool = True):
     distinct = float(np.mean([len(np.unique(bm.sel.numpy()))]))
     res.append({"config": 4, "case": f"OLMoE-arch decode B={B} ctx {ctx} (sequences in lockstep, one expert GEMV per (sequence, slot) job; last layer of the last step: {int(distinct)} distinct experts for {B * c.num_experts_per_tok} jobs)",
                 "tok_s": round(B / dtb, 1), "ms_per_step": round(dtb * 1e3, 4)})
+    if gate is not None and B == 8: res[-1]["parity"] = gate(bm, sd, c)
     del bm
   # the expert GEMVs alone: B tokens x 8 experts, gate/up fused then down, distinct experts per slot, layers rotated
   k, s = c.num_experts_per_tok, rt.Stream()
