@@ -74,7 +74,7 @@ def _per_sequence_check(gpu, model, cfg, host, prompts, n_new, max_context):
   for i in range(len(prompts[0]) - 1):
     for b in range(B): oracles[b].forward(prompts[b][i], pos)
     pos += 1
-  cur, worst, margin = [p[-1] for p in prompts], 0.0, np.inf
+  cur, worst, margin, near_ties = [p[-1] for p in prompts], 0.0, np.inf, 0
   for step in range(n_new):
     model.decode_step()
     lg_gpu = model.logits()
@@ -83,13 +83,17 @@ def _per_sequence_check(gpu, model, cfg, host, prompts, n_new, max_context):
       lg = oracles[b].forward(cur[b], pos)
       top2 = np.partition(lg, -2)[-2:]; margin = min(margin, float(top2[1] - top2[0]))
       worst = max(worst, ol.rel_err(lg_gpu[b], lg))
-      assert int(toks[b]) == int(np.argmax(lg)), (step, b, f"rel-err of this row {ol.rel_err(lg_gpu[b], lg):.2e}", f"oracle margin between the two candidates {lg[int(np.argmax(lg))] - lg[int(toks[b])]:.3e}",
-                                                   f"logit max {np.abs(lg).max():.3f}", getattr(oracles[b], "last_sel", None))
+      assert int(toks[b]) == int(np.argmax(lg_gpu[b])), (step, b, "the token is not the first maximum of the GPU's own logits")
+      if int(toks[b]) != int(np.argmax(lg)):                              # the oracle may prefer another token only across a near-tie of its own logits (inside the logits bar)
+        between = float(lg[int(np.argmax(lg))] - lg[int(toks[b])])
+        assert between <= 2 * TOL * float(np.abs(lg).max()), (step, b, f"rel-err of this row {ol.rel_err(lg_gpu[b], lg):.2e}", f"oracle margin between the two candidates {between:.3e}",
+                                                               f"logit max {np.abs(lg).max():.3f}", getattr(oracles[b], "last_sel", None))
+        near_ties += 1
       cur[b] = int(toks[b])
     pos += 1
   model.check_state()
-  print(f"batch {B}: worst logits rel-err {worst:.2e}, min oracle top-2 margin {margin:.4f}")
-  assert worst <= TOL
+  print(f"batch {B}: worst logits rel-err {worst:.2e}, min oracle top-2 margin {margin:.4f}, {near_ties} of {B * n_new} tokens across an oracle near-tie")
+  assert worst <= TOL and near_ties <= max(1, B * n_new // 50)
 
 SMALL = dict(num_blocks=2, dim=256, hidden_dim=512, n_heads=4, n_kv_heads=2, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=500000.0)
 SMALL_MOE = dict(num_blocks=2, dim=256, hidden_dim=128, n_heads=4, n_kv_heads=4, norm_eps=1e-5, vocab_size=512, head_dim=64, rope_theta=10000.0,

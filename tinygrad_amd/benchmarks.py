@@ -41,7 +41,7 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   wbytes = n * (k // nel) * nby
   copies = max(2, -(-int(1.25 * MALL_BYTES) // wbytes))
   big = Buffer((copies * wbytes,), np.uint8)
-  if ggml_type in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1):                                         # no device-side writer for these: seeded host blocks, one upload per copy
+  if ggml_type in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1, rt.IQ4_XS):                                       # no device-side writer for these: seeded host blocks, one upload per copy
     from tinygrad_amd import synth
     host = synth.random_blocks(np.random.default_rng(1002), ggml_type, n, k)
     for c in range(copies): big.view(c * wbytes, (wbytes,), np.uint8).copyin(host)
@@ -54,7 +54,7 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   s = rt.Stream()
   us = _time_launches(lambda i: lins[i](x, out=y, stream=s.handle), copies, iters, s)
   alg = wbytes + m * k * 2 + m * n * 2
-  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_1: "Q4_1", rt.Q5_0: "Q5_0", rt.Q5_1: "Q5_1", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
+  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_1: "Q4_1", rt.Q5_0: "Q5_0", rt.Q5_1: "Q5_1", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.IQ4_XS: "IQ4_XS", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
   return {"case": f"{name} {n}x{k} M={m}", "avg_us": round(us, 2), "alg_bytes": alg, "GBps": round(alg / us / 1e3, 1),
           "frac_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_rotated": copies, "launches": iters}
 
@@ -70,7 +70,7 @@ def kquants():
   """Q4_K / Q5_K (the block types of Q4_K_M / Q5_K_M model files) and the older Q4_1 / Q5_0 / Q5_1 blocks at the Llama-3-8B linear
   shapes, M in {1, 8} (Q4_K / Q5_K: and 4, 16), and the Q6_K ffn_down of a Q4_K_M file."""
   out = []
-  for t in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1):
+  for t in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1, rt.IQ4_XS):
     for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
       for m in ((1, 4, 8, 16) if t in (rt.Q4_K, rt.Q5_K) else (1, 8)): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   for m in (1, 4, 8, 16): out.append(dict(config="k-quants", **gemv_case(rt.Q6_K, 4096, 14336, m, iters=200)))

@@ -604,6 +604,86 @@ template <bool FIVE> struct FmtK45 {
 template <> struct Fmt<GGML_Q4_K> : FmtK45<false> {};
 template <> struct Fmt<GGML_Q5_K> : FmtK45<true> {};
 
+// ------------------------------------------------------------------------------------------------ IQ4_XS (gguf.py:96-104)
+// Superblock of 256 weights, 136 bytes: fp16 d, uint16 scales_h, scales_l[4], qs[128].  Sub-block s (32 weights) = qs[16 s .. 16 s + 15], weight j the low
+// nibble of byte j, weight j + 16 the high nibble (the Q4_0 order); its 6-bit scale is ls = (nibble s of scales_l | bits 2 s, 2 s + 1 of scales_h << 4) - 32;
+// w = d ls kvalues_iq4nl[code], a 16-entry table of int8 values.  A unit is a pair of sub-blocks (64 consecutive weights, 32 bytes of qs at an 8-byte
+// aligned offset), accumulator group g = sub-block 2 p + g.  The table lives in four registers as bytes value + 128: two v_perm_b32 look four codes up in
+// either half of it, a third picks per byte by the code's top bit, a fourth pairs the bytes with an 0x64 exponent byte, so that a weight decodes to the
+// fp16 pattern 1024 + 128 + value (bias 1152, removed through the accumulator's start value like every other format's).
+template <> struct Fmt<GGML_IQ4_XS> {
+  static constexpr int UW = 64, UPB = 4, BW = 256, BB = 136;
+  static __device__ __forceinline__ int unit_of(int e) { return e >> 6; }
+  static __device__ __forceinline__ int pair_of(int e) { return (e & 63) >> 1; }
+  static constexpr int XV = 8, NG = 2, NWV = 34;
+  struct Raw { u32x4 q0, q1; uint32_t h0, h1, p; };
+  static __device__ __forceinline__ Raw load(const uint8_t* row, int u) {
+    const uint8_t* b = row + (size_t)BB * (u >> 2); const int p = u & 3;
+    Raw r; r.h0 = ld4_a4(b); r.h1 = ld4_a4(b + 4); r.q0 = ld16_a4(b + 8 + 32 * p); r.q1 = ld16_a4(b + 24 + 32 * p); r.p = (uint32_t)p;
+    return r;
+  }
+  static __device__ __forceinline__ int xoff(int u, int k) { return 64 * u + 2 * k; }
+  static constexpr int NKC = 5;
+  // kvalues_iq4nl + 128 = 1, 24, 45, 63 | 79, 93, 106, 118 | 129, 141, 153, 166 | 181, 197, 217, 241
+  static __device__ __forceinline__ void consts(uint32_t* kc) {
+    kc[0] = vgpr_const(0x3F2D1801u); kc[1] = vgpr_const(0x766A5D4Fu); kc[2] = vgpr_const(0xA6998D81u); kc[3] = vgpr_const(0xF1D9C5B5u); kc[4] = vgpr_const(0x64646464u);
+  }
+  // the table bytes of four codes (bits 0..3 of every byte of `codes`; the upper nibbles are ignored)
+  static __device__ __forceinline__ uint32_t lut4(uint32_t codes, const uint32_t* kc) {
+    const uint32_t sel = codes & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(kc[1], kc[0], sel), hi = __builtin_amdgcn_perm(kc[3], kc[2], sel);
+    return __builtin_amdgcn_perm(hi, lo, and_or(codes >> 1, 0x04040404u, 0x03020100u));      // byte i from lo (selector i) or from hi (4 + i) by the code's bit 3
+  }
+  // wv[4 (4 g + t) + {0, 1, 2, 3}] = weights (4t, 4t+1), (4t+2, 4t+3), (16+4t, 16+4t+1), (16+4t+2, 16+4t+3) of sub-block 2 p + g (t = dword of its 16 bytes)
+  static __device__ __forceinline__ void decode(const Raw& r, uint32_t* wv, const uint32_t* kc) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t w = i < 4 ? r.q0[i & 3] : r.q1[i & 3];
+      const uint32_t l = lut4(w, kc), h = lut4(w >> 4, kc);
+      wv[4 * i + 0] = __builtin_amdgcn_perm(kc[4], l, 0x04010400u); wv[4 * i + 1] = __builtin_amdgcn_perm(kc[4], l, 0x04030402u);
+      wv[4 * i + 2] = __builtin_amdgcn_perm(kc[4], h, 0x04010400u); wv[4 * i + 3] = __builtin_amdgcn_perm(kc[4], h, 0x04030402u);
+    }
+    const uint32_t lb = (r.h1 >> (8 * r.p)) & 0xFF, hs = (r.h0 >> (16 + 4 * r.p)) & 0xF;
+    const int ls0 = (int)((lb & 0xF) | ((hs & 3) << 4)) - 32, ls1 = (int)((lb >> 4) | ((hs >> 2) << 4)) - 32;
+    const float d = h2f_bits(r.h0 & 0xFFFF);
+    wv[32] = __builtin_bit_cast(uint32_t, d * (float)ls0); wv[33] = __builtin_bit_cast(uint32_t, d * (float)ls1);
+  }
+  // nx[k] = natural pair k of the unit's 64 activations; xv[4 g + t] = pairs 2t, 2t + 1, 8 + 2t, 8 + 2t + 1 of sub-block g
+  static __device__ __forceinline__ void stage(const uint32_t* nx, u32x4* xv, float* c) {
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      const uint32_t* n = nx + 16 * g;
+#pragma unroll
+      for (int t = 0; t < 4; t++) { xv[4 * g + t].x = n[2 * t]; xv[4 * g + t].y = n[2 * t + 1]; xv[4 * g + t].z = n[8 + 2 * t]; xv[4 * g + t].w = n[8 + 2 * t + 1]; }
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; k++) s = dot2(n[k], 0x64806480u, s);        // 1152
+      c[g] = -s;
+    }
+  }
+  static __device__ __forceinline__ float finish(const Raw&, const uint32_t* wv, const float* a, const float*) {
+    return __builtin_bit_cast(float, wv[32]) * a[0] + __builtin_bit_cast(float, wv[33]) * a[1];
+  }
+  static __device__ __forceinline__ void to_f16(const Raw&, uint32_t* wv) {
+    const float s0 = __builtin_bit_cast(float, wv[32]), s1 = __builtin_bit_cast(float, wv[33]);
+#pragma unroll
+    for (int i = 0; i < 16; i++) { wv[i] = h2_unbias_scale_f32(wv[i], s0, -1152.f * s0); wv[16 + i] = h2_unbias_scale_f32(wv[16 + i], s1, -1152.f * s1); }
+  }
+  static __device__ __forceinline__ int spos(int e, int nu) {
+    const int u = e >> 6, g = (e >> 5) & 1, r = e & 31, hi = r >> 4, q = r & 15, t = q >> 2, k = q & 3;
+    return (((4 * g + t) * nu + u) * 4 + hi * 2 + (k >> 1)) * 2 + (k & 1);
+  }
+  static __device__ __forceinline__ void cfromx(const u32x4* xv, float* c) {
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+      float t = 0.f;
+#pragma unroll
+      for (int i = 4 * g; i < 4 * g + 4; i++) { t = dot2(xv[i].x, 0x64806480u, t); t = dot2(xv[i].y, 0x64806480u, t); t = dot2(xv[i].z, 0x64806480u, t); t = dot2(xv[i].w, 0x64806480u, t); }
+      c[g] = -t;
+    }
+  }
+};
+
 // ------------------------------------------------------------------------------------------------ Q4_1 / Q5_0 / Q5_1 (gguf.py:47-55)
 // Blocks of 32 weights: fp16 d, [fp16 m], [qh: the 32 fifth bits, little endian], qs[16]; weight j is the low nibble of qs[j],
 // weight j + 16 the high nibble (+ 16 * bit of qh).  w = q d + m (Q4_1, Q5_1) or (q - 16) d (Q5_0).
@@ -801,6 +881,7 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
     case GGML_Q4_1: return Fmt<GGML_Q4_1>::spos(e, nu);
     case GGML_Q5_0: return Fmt<GGML_Q5_0>::spos(e, nu);
     case GGML_Q5_1: return Fmt<GGML_Q5_1>::spos(e, nu);
+    case GGML_IQ4_XS: return Fmt<GGML_IQ4_XS>::spos(e, nu);
     case GGML_MXFP4: return Fmt<GGML_MXFP4>::spos(e, nu);
     case GGML_F16: return Fmt<GGML_F16>::spos(e, nu);
   }

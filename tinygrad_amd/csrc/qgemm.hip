@@ -270,6 +270,7 @@ int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
     case GGML_Q4_1: return launch_qgemm_m<GGML_Q4_1>(a, M, s);
     case GGML_Q5_0: return launch_qgemm_m<GGML_Q5_0>(a, M, s);
     case GGML_Q5_1: return launch_qgemm_m<GGML_Q5_1>(a, M, s);
+    case GGML_IQ4_XS: return launch_qgemm_m<GGML_IQ4_XS>(a, M, s);
     case GGML_F16: return launch_qgemm_m<GGML_F16>(a, M, s);
     case GGML_MXFP4: return launch_qgemm_m<GGML_MXFP4>(a, M, s);
   }

@@ -325,10 +325,10 @@ static int staged_fmt(int ggml_type, long long K, int* nu) {
   switch (ggml_type) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
     case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
-    case GGML_Q4_1: fmt = GGML_Q4_1; break; case GGML_Q5_0: fmt = GGML_Q5_0; break; case GGML_Q5_1: fmt = GGML_Q5_1; break;
+    case GGML_Q4_1: fmt = GGML_Q4_1; break; case GGML_Q5_0: fmt = GGML_Q5_0; break; case GGML_Q5_1: fmt = GGML_Q5_1; break; case GGML_IQ4_XS: fmt = GGML_IQ4_XS; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
-  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K) ? 256 : 64) != 0) return -1;
+  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_IQ4_XS) ? 256 : 64) != 0) return -1;
   *nu = (int)(K / uw);
   return fmt;
 }
@@ -393,10 +393,10 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
   TGA_REQUIRE(epilogue != 1 || (y_dtype == TGA_F32 && resid), "tga_qlinear: the residual epilogue needs float32 y and resid pointers");
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: bw = 256; break; case GGML_F16: bw = 64; break;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: bw = 256; break; case GGML_F16: bw = 64; break;
     case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: bw = 64; break;      // served as block pairs
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
-  const bool align4 = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q4_1 || ggml_type == GGML_Q5_0 || ggml_type == GGML_Q5_1;
+  const bool align4 = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q4_1 || ggml_type == GGML_Q5_0 || ggml_type == GGML_Q5_1 || ggml_type == GGML_IQ4_XS;
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
   TGA_REQUIRE(x, "tga_qlinear: null x");
   QArgs a = {};
@@ -405,7 +405,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
   for (int i = 0; i < nseg; i++) {
     TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)), "tga_qlinear: segment %d has a null pointer or no rows", i);
     TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((uintptr_t)w[i] & 1) == 0, "tga_qlinear: weight pointer of segment %d must be 2-byte aligned", i);
-    TGA_REQUIRE(!align4 || ((uintptr_t)w[i] & 3) == 0, "tga_qlinear: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 weights of segment %d must be 4-byte aligned", i);
+    TGA_REQUIRE(!align4 || ((uintptr_t)w[i] & 3) == 0, "tga_qlinear: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 / IQ4_XS weights of segment %d must be 4-byte aligned", i);
     a.w[i] = (const uint8_t*)w[i]; a.y[i] = y[i]; a.n[i] = n[i]; a.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr;
     TGA_REQUIRE(epilogue != 1 || a.resid[i], "tga_qlinear: null resid for segment %d", i);
     ntot += n[i];
@@ -488,6 +488,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     case GGML_Q4_1: return launch_qgemv_m<GGML_Q4_1>(a, M, s);
     case GGML_Q5_0: return launch_qgemv_m<GGML_Q5_0>(a, M, s);
     case GGML_Q5_1: return launch_qgemv_m<GGML_Q5_1>(a, M, s);
+    case GGML_IQ4_XS: return launch_qgemv_m<GGML_IQ4_XS>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
     case GGML_F16: return launch_qgemv_m<GGML_F16>(a, M, s);
   }

@@ -594,7 +594,7 @@ static int launch_fast_e(const QArgs& a, hipStream_t s) {
   // two rows per step keep more bytes in flight per lane; a single row when there are too few rows to fill the chip twice, for Q8_0 pairs
   // (68-byte units: no faster with two) and when the waves of a workgroup split K - with the three-deep ring a single row per step is
   // faster there (4096 x 14336: Q4_0 in the 8B decode step 12.5 -> 11.7 us, Q4_K 13.2 -> 12.2, Q6_K 19.3 -> 17.4, Q5_0 16.2 -> 15.2).
-  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1)
+  const bool r2 = (T == F_Q4_0P || T == GGML_MXFP4 || T == GGML_Q6_K || T == GGML_Q4_K || T == GGML_Q5_K || T == GGML_Q4_1 || T == GGML_Q5_0 || T == GGML_Q5_1 || T == GGML_IQ4_XS)
                   && WK == 1 && a.ntot >= (long long)fast_cu_count() * r2_rows_per_cu();
   if (a.epilogue == 1) return r2 ? launch_fast<T, 2, WK, WR, 1, H>(a, s) : launch_fast<T, 1, WK, WR, 1, H>(a, s);
   return r2 ? launch_fast<T, 2, WK, WR, 0, H>(a, s) : launch_fast<T, 1, WK, WR, 0, H>(a, s);

@@ -12,6 +12,7 @@ extern template int qgemv1_launch_format<GGML_Q5_K>(QArgs, hipStream_t);
 extern template int qgemv1_launch_format<GGML_Q4_1>(QArgs, hipStream_t);
 extern template int qgemv1_launch_format<GGML_Q5_0>(QArgs, hipStream_t);
 extern template int qgemv1_launch_format<GGML_Q5_1>(QArgs, hipStream_t);
+extern template int qgemv1_launch_format<GGML_IQ4_XS>(QArgs, hipStream_t);
 
 // Returns -1 when the shape is outside the fast path (caller falls back to the LDS-staged kernel).
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
@@ -28,6 +29,7 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s) {
     case GGML_Q4_1: return qgemv1_launch_format<GGML_Q4_1>(a, s);
     case GGML_Q5_0: return qgemv1_launch_format<GGML_Q5_0>(a, s);
     case GGML_Q5_1: return qgemv1_launch_format<GGML_Q5_1>(a, s);
+    case GGML_IQ4_XS: return qgemv1_launch_format<GGML_IQ4_XS>(a, s);
     case GGML_MXFP4: return qgemv1_launch_format<GGML_MXFP4>(a, s);
     case GGML_F16: return qgemv1_launch_format<GGML_F16>(a, s);
   }

@@ -199,7 +199,7 @@ class TransformerBlock:
     self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.config, self.s = c, shared
     # the M = 1 GEMV's register-resident fast path: K % 64 (superblock types: % 256), 4-byte aligned weights
-    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K) or l.in_features % 256 == 0)
+    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K, rt.IQ4_XS) or l.in_features % 256 == 0)
     # RMSNorm folded into the consuming linear
     self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
     # a producer with a single consumer writes its fp16 output in the order that consumer's GEMV reads it (no LDS staging there):
@@ -349,7 +349,7 @@ class Transformer:
     self.output_norm = state_dict["output_norm.weight"][0]
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
-    self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
+    self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K, rt.IQ4_XS) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
     self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.n_summands <= 8
     self.stream = rt.Stream()
     self._graphs = {}
