@@ -58,7 +58,7 @@ def test_one_launch_attention_and_merging_linear(gpu, H, KV, hd, ctx, positions)
   ck0 = (rng.standard_normal((KV, ctx, hd)) * 0.7).astype(np.float16)
   cv0 = rng.standard_normal((KV, ctx, hd)).astype(np.float16)
   part_old = rt.Buffer((H * ((ctx + 63) // 64) * (hd + 2),), np.float32).zero_()
-  part_new = rt.Buffer((H * ns.value * (hd + 4),), np.float32).zero_()
+  part_new = rt.Buffer((H * (ns.value * hd + 16),), np.float32).zero_()
   ropeb = rt.Buffer.from_numpy(rope)
   for pos in positions:
     q = rng.standard_normal((H, hd)).astype(np.float32); k = rng.standard_normal((KV, hd)).astype(np.float32); v = rng.standard_normal((KV, hd)).astype(np.float32)
@@ -106,7 +106,7 @@ def test_one_launch_attention_refuses_what_it_cannot_serve(gpu):
   # a position outside the cache: flag, nothing written
   st2 = np.zeros(16, np.int32); st2[0] = 64
   stb = rt.Buffer.from_numpy(st2)
-  ck = rt.Buffer.from_numpy(np.ones((8, 64, 128), np.float16)); part = rt.Buffer((8 * 1 * 132,), np.float32).zero_()
+  ck = rt.Buffer.from_numpy(np.ones((8, 64, 128), np.float16)); part = rt.Buffer((8 * (1 * 128 + 16),), np.float32).zero_()
   rt.check(L.tga_attention_decode_split(b.ptr, b.ptr, b.ptr, ck.ptr, ck.ptr, part.ptr, stb.ptr, 8, 8, 128, 64, b.ptr, None))
   rt.synchronize()
   assert int(stb.numpy()[4]) == 2 and np.all(ck.numpy() == 1) and not part.numpy().any()

@@ -411,10 +411,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 // The attention of one token as ONE launch whose consumer merges (tga_attn_merge_qlinear): workgroup = (query head, split of SP = 128 IT positions), eight waves
 // of 16 rows per tile, IT tiles per wave, every cached row of the split requested up front (rows clamped to the cache, not to the position), at most four splits.
 // The flattened workgroup index is kv head + n_kv (head in group + group * split): with n_kv a multiple of 8 all readers of a kv head's rows run on one XCD.
-// A split that starts beyond the position writes an empty partial (max -inf, sum 0).  Partials: [n_heads][n_splits][head_dim + 4] = weighted V, max, sum, 2 pad.
+// A split that starts beyond the position writes an empty partial (max -inf, sum 0).  Partials per head: [n_splits][head_dim] weighted V sums, then the
+// (max, sum) pairs of the splits in 16 floats.
 template <int HD8, int IT, int NW>
 __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) {
-  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = NW * RPI, CSTR = HD + 4, PS = HD + 4, SP = 16 * NW * IT;
+  constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = NW * RPI, CSTR = HD + 4, SP = 16 * NW * IT;
   const int group = a.n_heads / a.n_kv;
   const int kvh = blockIdx.x % a.n_kv, rest = blockIdx.x / a.n_kv, hh = rest % group, split = rest / group, head = kvh * group + hh;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = HD >> 1;
@@ -445,10 +446,12 @@ __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) 
     if (blockIdx.x == 0 && tid == 0) atomicOr(&a.st->error, 2);
     return;
   }
-  float* po = a.part + ((size_t)head * a.nsplit + split) * PS;
+  float* ph_ = a.part + (size_t)head * (a.nsplit * HD + 16);
+  float* po = ph_ + (size_t)split * HD;                    // this split's weighted V sums
+  float* pml = ph_ + (size_t)a.nsplit * HD + 2 * split;    // and its (max, sum)
   if (split * SP > pos) {                               // nothing cached in this split yet
     if (tid < HD) po[tid] = 0.f;
-    if (tid == 0) { po[HD] = -INFINITY; po[HD + 1] = 0.f; }
+    if (tid == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
     return;
   }
   const float rc_ = a.rope[(size_t)pos * HD + ki], rs_ = a.rope[(size_t)pos * HD + half + ki];
@@ -530,7 +533,7 @@ __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) 
 #pragma unroll
     for (int q = 0; q < NP; q++) { od += fold_o[q][tid]; ll += fold_l[q]; }
     po[tid] = od;
-    if (tid == 0) { po[HD] = mm; po[HD + 1] = ll; }
+    if (tid == 0) { pml[0] = mm; pml[1] = ll; }
   }
 }
 

@@ -24,8 +24,8 @@ struct QArgs {
   // x_staged: x already holds fp16 activations in the consumer format's staged order (Fmt::spos).
   // y_stage_fmt / y_stage_nu: when y_stage_fmt != 0 the fp16 outputs are written in the staged order of THAT consumer format.
   int x_staged, y_stage_fmt, y_stage_nu;
-  // attn_S > 0 (M = 1 fast path, residual epilogue): x holds float32 split partials of the attention, [K >> attn_hd_log2 heads][attn_S][head_dim + 4] =
-  // weighted V (head_dim), max, sum, 2 pad; the row is their merge, sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m), rounded to fp16
+  // attn_S > 0 (M = 1 fast path, residual epilogue): x holds float32 split partials of the attention, per head (K >> attn_hd_log2 heads) [attn_S][head_dim]
+  // weighted V sums followed by 16 floats holding the splits' (max, sum) pairs; the row is their merge, sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m), rounded to fp16
   // (the two fields sit where the struct had padding: qgemv1_two_kernel counts on the size of two of these)
   int attn_S;
   // norm_w != nullptr (M = 1 fast path, fp32 x): the activation row is RMS-normalised while it is staged,

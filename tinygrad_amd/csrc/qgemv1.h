@@ -53,6 +53,34 @@
 // MR > 1 (several activation rows; instantiated for two; generic prologue, no fused SwiGLU): the same walk over the weights with MR sets of activations in registers;
 // a unit is decoded once and multiplied with every row.  Outputs and residuals are (MR, rows) per matrix.
 // bx: the workgroup's index among those of this matrix set (blockIdx.x where a launch serves one set, see qgemv1_two_kernel)
+// Eight values of one head's attention row from its S split partials: ph = [S][hd] weighted V sums, then (max, sum) pairs of the S splits (six pairs, then
+// four floats of padding); merged = sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m).
+template <int S>
+__device__ __forceinline__ void attn_merge_piece(const float* ph, int hd, int d0, f32x4& l, f32x4& h) {
+  f32x4 pl[S], phh[S], ml[3];
+#pragma unroll
+  for (int sp = 0; sp < S; sp++) { pl[sp] = gld16f(ph + sp * hd + d0); phh[sp] = gld16f(ph + sp * hd + d0 + 4); }
+#pragma unroll
+  for (int j = 0; j < (S + 1) / 2; j++) ml[j] = gld16f(ph + S * hd + 4 * j);
+  float pm[S], pls[S];
+#pragma unroll
+  for (int sp = 0; sp < S; sp++) { pm[sp] = (sp & 1) ? ml[sp >> 1].z : ml[sp >> 1].x; pls[sp] = (sp & 1) ? ml[sp >> 1].w : ml[sp >> 1].y; }
+  float mx = pm[0];
+#pragma unroll
+  for (int sp = 1; sp < S; sp++) mx = fmaxf(mx, pm[sp]);
+  l = f32x4{0.f, 0.f, 0.f, 0.f}; h = f32x4{0.f, 0.f, 0.f, 0.f};
+  float lsum = 0.f;
+#pragma unroll
+  for (int sp = 0; sp < S; sp++) {
+    const float e = pm[sp] != -INFINITY ? __expf(pm[sp] - mx) : 0.f;
+    lsum += e * pls[sp];
+    l.x += e * pl[sp].x; l.y += e * pl[sp].y; l.z += e * pl[sp].z; l.w += e * pl[sp].w;
+    h.x += e * phh[sp].x; h.y += e * phh[sp].y; h.z += e * phh[sp].z; h.w += e * phh[sp].w;
+  }
+  const float inv = 1.0f / lsum;
+  l.x *= inv; l.y *= inv; l.z *= inv; l.w *= inv; h.x *= inv; h.y *= inv; h.z *= inv; h.w *= inv;
+}
+
 // One dword of one line per lane for the attention launch that follows a q / k / v launch (QArgs::touch_*, prologue 8), branch-free: beyond the lines
 // there are a lane reads the last one again.  Workgroup bx runs on XCD bx % 8; the attention workgroups of kv head h run on
 // XCD h % 8 when the number of kv heads is a multiple of 8 (the host only asks then).  Lines of an XCD: K rows [0, pos) and V rows [0, pos) of each of its
@@ -358,32 +386,16 @@ __device__ __forceinline__ void qgemv1_body(const QArgs& args, const unsigned bx
     issue(b[0], lo);
     lds_to_regs();
   } else if constexpr (PRO == 7) {
-    // the row is the merge of the attention's split partials (attn_split1_kernel): thread t merges elements 8t .. 8t + 7 of its head.  All loads are
-    // one batch (surplus splits reload split 0 with weight 0); a split without cached positions carries max = -inf, sum = 0.
+    // the row is the merge of the attention's split partials (attn_split1_kernel): thread t merges elements 8t .. 8t + 7 of its head; a split
+    // without cached positions carries max = -inf, sum = 0.  One instantiation per number of splits, so that exactly its loads go out, as one batch.
     const int i = (int)threadIdx.x < nq ? (int)threadIdx.x : nq - 1;
-    const int hd = 1 << a.attn_hd_log2, head = (8 * i) >> a.attn_hd_log2, d0 = 8 * i - (head << a.attn_hd_log2), ps = hd + 4;
-    const float* ph = (const float*)a.x + (size_t)head * a.attn_S * ps;
-    constexpr int MS = 6;                                        // most splits (surplus slots reload split 0 with weight 0)
-    f32x4 pl[MS], phh[MS]; float pm[MS], pls[MS];
-#pragma unroll
-    for (int sp = 0; sp < MS; sp++) {
-      const int sc = sp < a.attn_S ? sp : 0;
-      pl[sp] = *(const f32x4*)(ph + sc * ps + d0); phh[sp] = *(const f32x4*)(ph + sc * ps + d0 + 4);
-      pm[sp] = ph[sc * ps + hd]; pls[sp] = ph[sc * ps + hd + 1];
+    const int hd = 1 << a.attn_hd_log2, head = (8 * i) >> a.attn_hd_log2, d0 = 8 * i - (head << a.attn_hd_log2);
+    const float* ph = (const float*)a.x + (size_t)head * (a.attn_S * hd + 16);
+    f32x4 l, h;
+    switch (a.attn_S) {
+      case 1: attn_merge_piece<1>(ph, hd, d0, l, h); break; case 2: attn_merge_piece<2>(ph, hd, d0, l, h); break; case 3: attn_merge_piece<3>(ph, hd, d0, l, h); break;
+      case 4: attn_merge_piece<4>(ph, hd, d0, l, h); break; case 5: attn_merge_piece<5>(ph, hd, d0, l, h); break; default: attn_merge_piece<6>(ph, hd, d0, l, h); break;
     }
-    float mx = pm[0];
-#pragma unroll
-    for (int sp = 1; sp < MS; sp++) mx = fmaxf(mx, sp < a.attn_S ? pm[sp] : pm[0]);
-    f32x4 l = {0.f, 0.f, 0.f, 0.f}, h = {0.f, 0.f, 0.f, 0.f}; float lsum = 0.f;
-#pragma unroll
-    for (int sp = 0; sp < MS; sp++) {
-      const float e = (sp < a.attn_S && pm[sp] != -INFINITY) ? __expf(pm[sp] - mx) : 0.f;
-      lsum += e * pls[sp];
-      l.x += e * pl[sp].x; l.y += e * pl[sp].y; l.z += e * pl[sp].z; l.w += e * pl[sp].w;
-      h.x += e * phh[sp].x; h.y += e * phh[sp].y; h.z += e * phh[sp].z; h.w += e * phh[sp].w;
-    }
-    const float inv = 1.0f / lsum;
-    l.x *= inv; l.y *= inv; l.z *= inv; l.w *= inv; h.x *= inv; h.y *= inv; h.z *= inv; h.w *= inv;
     if ((int)threadIdx.x < nq) put_piece((int)threadIdx.x, pack8(l, h));
     __syncthreads();                                             // every wave holds its pieces: only now the first weights (as in prologue 3; requested
     issue(b[0], lo);                                             // in front of the partials they cost 2 % of the decode step)

@@ -321,7 +321,7 @@ class _Shared:
     self.qkv = Buffer((1, nq + 2 * nkv), f32)                          # q | k | v
     self.q, self.k, self.v = self.qkv.view(0, (1, nq), f32), self.qkv.view(4 * nq, (1, nkv), f32), self.qkv.view(4 * (nq + nkv), (1, nkv), f32)
     self.attn = Buffer((1, c.n_heads * c.head_dim), f16)
-    self.attn_part = Buffer((c.n_heads * max(((c.max_context + 63) // 64) * (c.head_dim + 2), 6 * (c.head_dim + 4)),), f32).zero_()   # (two-launch layout or up to six split partials)
+    self.attn_part = Buffer((c.n_heads * max(((c.max_context + 63) // 64) * (c.head_dim + 2), 6 * c.head_dim + 16),), f32).zero_()   # (two-launch layout or up to six split partials + their (max, sum) pairs)
     self.act = Buffer((1, max(c.hidden_dim, c.dense_hidden_dim)), f16)
     if c.num_experts:
       k = c.num_experts_per_tok
