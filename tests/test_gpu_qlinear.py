@@ -237,10 +237,12 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
-@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 32), (12, 528, 2048, 24), (8, 200, 14336, 40), (14, 1024, 4096, 64), (2, 512, 14336, 17)])
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 32), (12, 528, 2048, 24), (8, 200, 14336, 40), (14, 1024, 4096, 64), (2, 512, 14336, 17), (13, 300, 4096, 48), (23, 528, 4096, 64), (12, 4096, 4096, 17),
+                                     (8, 1000, 1024, 33), (14, 72, 256, 50), (2, 200, 2048 + 32, 40), (3, 200, 2048, 40), (39, 256, 2048, 24)])
 def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
-  """Prefill chunks of more than sixteen rows are blocks of sixteen (and a rest) through the same kernels: plain, with the residual in place and with the norm in front
-  (tga_rmsnorm_qlinear_rows), against the C restatement run in blocks of eight rows."""
+  """Prefill chunks of 17 .. 64 rows: one pass of the 64-column kernel where it applies (K a multiple of 256, its formats), otherwise blocks of sixteen (and a rest)
+  through the small-batch kernels: plain, with the residual in place and with the norm in front (tga_rmsnorm_qlinear_rows), against the C restatement run in
+  blocks of eight rows."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(3 * n + k + m + t)
   w = synth.random_blocks(rng, t, n, k)
@@ -248,7 +250,8 @@ def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
   ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
   y = _run(gpu, t, w, x, n, k)
   assert y.shape == (m, n) and ol.rel_err(y, ref) <= TOL
-  np.testing.assert_array_equal(y[:16], _run(gpu, t, w, x[:16], n, k))
+  assert ol.rel_err(y[:16], _run(gpu, t, w, x[:16], n, k)) <= 1e-4        # (the sixteen-row kernels sum K in another order)
+  np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
   layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
   res = rng.standard_normal((m, n)).astype(np.float32)
   rb = gpu.Buffer.from_numpy(res)
@@ -262,6 +265,27 @@ def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
   assert ol.rel_err(h.astype(np.float32), hn.astype(np.float32)) <= 1e-3
   refn = np.concatenate([cref.linear(t, w, h[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
   assert ol.rel_err(out.numpy(), refn) <= TOL
+
+def test_seventeen_rows_on_more_streams_than_workspace_slots(gpu):
+  """The 64-column kernel keeps its staged activations and split-K partial tiles in a per-device workspace of a few slots, one per stream; a call on a
+  further stream runs blocks of sixteen rows instead.  Six streams, two calls each (the second finds its stream's slot again): every result within the bar,
+  and equal between the two calls of a stream."""
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  from tinygrad_amd import runtime as rt
+  rng = np.random.default_rng(64)
+  t, n, k, m = 2, 1024, 4096, 40
+  w = synth.random_blocks(rng, t, n, k)
+  layer = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
+  streams = [rt.Stream() for _ in range(6)]
+  for st in streams:
+    x = synth.activations(rng, m, k, np.float16)
+    ref = np.concatenate([cref.linear(t, w, x[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
+    xb = gpu.Buffer.from_numpy(x)
+    outs = [gpu.Buffer((m, n), np.float32) for _ in range(2)]
+    for o in outs: qlinear_multi([layer], xb, [o], stream=st.handle)
+    st.synchronize()
+    assert ol.rel_err(outs[0].numpy(), ref) <= TOL
+    np.testing.assert_array_equal(outs[0].numpy(), outs[1].numpy())
 
 @pytest.mark.parametrize("t,n,k,m", [(2, 4096, 14336, 16), (8, 4096, 14336, 8), (2, 256, 5120, 3), (8, 48, 14336, 9), (2, 4112, 8192, 13), (8, 1024, 6144, 16),
                                        (14, 4096, 14336, 8), (14, 48, 8192, 3), (14, 1040, 6144, 16), (14, 64, 5120, 5), (14, 272, 14336, 7)])
@@ -420,12 +444,14 @@ def test_norm_and_linears_of_mixed_block_types(gpu, types, k, ns):
     ref = ol.linear_f64(h, ol.weight_f32(w, n, k, t))
     assert ol.rel_err(o.numpy(), ref) <= TOL and ol.rel_err(o16.numpy().astype(np.float32), ref) <= 2 * TOL
 
-def test_sixteen_rows_segments_residual_and_swiglu(gpu):
-  """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows, on the LDS-fed kernel's range and outside it."""
+@pytest.mark.parametrize("m", [16, 17, 37, 64])
+def test_sixteen_and_more_rows_segments_residual_and_swiglu(gpu, m):
+  """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows (on the LDS-fed kernel's range and outside it) and at
+  17 .. 64 rows (the 64-column kernel; segments that are no multiple of sixteen rows go through blocks of sixteen)."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
-  rng = np.random.default_rng(1616)
-  m = 16
-  for t, k, ns in ((2, 2048, [2048, 512, 512]), (8, 1024, [512, 128, 130]), (14, 1024, [64, 32, 32])):
+  rng = np.random.default_rng(1616 + m)
+  for t, k, ns in ((2, 2048, [2048, 512, 512]), (8, 1024, [512, 128, 130]), (14, 1024, [64, 32, 32]), (12, 2048, [272, 48, 48]), (13, 1024, [100, 100]), (23, 1024, [80, 16, 16])):
+    if len(ns) == 2: ns = [ns[0], ns[1], ns[1]]
     ws = [synth.random_blocks(rng, t, n, k) for n in ns]
     x = synth.activations(rng, m, k, np.float16)
     layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]

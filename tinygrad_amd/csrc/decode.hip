@@ -5,6 +5,7 @@
 // (the reference binds symbolic start_pos into a replayed JIT graph: tinygrad/llm/model.py:464-484).
 #include <type_traits>
 #include <stdlib.h>
+#include <string.h>
 #include "qfmt.h"
 #include "decode.h"
 #include "coherent.h"
@@ -405,6 +406,133 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
       if (lane == 0) { po[HD] = m; po[HD + 1] = l; }
     }
     __syncthreads();
+  }
+}
+
+// Chunked prefill, the attending launch on the matrix cores (chunk rows z = 0, 1, ... are consecutive positions of one sequence; the launch before has rotated
+// and appended every row's key / value).  Workgroup = (kv head, split of 64 cached positions, tile of 16 chunk rows): the per-row workgroups of
+// attn_decode_kernel read every 32 KB K / V tile once per row and query-head group - 64 rows x 8 kv heads x 16 splits = 268 MB of L2 reads per layer at a
+// context of 1024 - here a tile is read once per sixteen rows.  Wave w serves query head w of the group (w + 4, ... for larger groups):
+//   S^T = K Q^T   v_mfma_f32_16x16x32_f16, A = lane (g, r): 8 values 32 j + 8 g .. of cached key 16 t + r (16-byte loads straight from the cache), B = lane (g, c):
+//                 the same 8 values of chunk row c's rotated query, rounded to fp16, in registers for the whole launch; D = lane (g, c): keys 16 t + 4 g + i of row c
+//   softmax partial of the split per chunk row: the 16 scores of a lane, then the four lanes of a row (m, l: float32; a row sees the positions up to its own)
+//   O^T = V^T P^T A = lane (g, r): V of 8 keys for dimension 16 h + r, B = lane (g, c): exp(s - m) of the SAME 8 keys for row c, rounded to fp16 - the eight
+//                 keys a lane holds after the first product (tiles 2 u and 2 u + 1, rows 4 g + i) are taken as they are, and the V tile is written to LDS
+//                 transposed with its keys in that order, so that the A operand is one 16-byte LDS read
+// The partial (float32 weighted V sums, max, sum) goes where attn_decode_kernel writes it; attn_merge_kernel finishes.  Deviation from the float32 products of
+// the per-row kernel: the rotated query and the probabilities are rounded to fp16 (2^-11 relative each, fp32 accumulation).
+template <int HD8>
+__global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, const int rows) {
+  typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+  typedef float v4f32 __attribute__((ext_vector_type(4)));
+  constexpr int HD = HD8 * 8, NJ = HD / 32, NH = HD / 16, half = HD / 2;
+  constexpr int VP = 64 + 8;                            // halfwords per transposed V row (64 keys + 16 bytes: rows 16 bytes apart in the banks)
+  __shared__ __attribute__((aligned(16))) uint16_t vts[HD * VP];
+  const int kvh = blockIdx.x, split = blockIdx.y, rz = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
+  const int group = a.n_heads / a.n_kv;
+  const int row = 16 * rz + c < rows ? 16 * rz + c : rows - 1;             // this lane's chunk row (a tile that the chunk ends in repeats the last row, stored by nobody)
+  const bool row_ok = 16 * rz + c < rows;
+  // ---- loads that do not depend on the position: the V tile (lane = key, pieces 4 wave .. 4 wave + 3 of HD8), the K operands, the first head's query
+  const int key0 = split * 64;
+  u32x4 vv[HD8 / 4];
+  {
+    const int kr = key0 + lane < a.max_ctx ? key0 + lane : a.max_ctx - 1;
+    const _Float16* vb = a.cache_v + ((size_t)kvh * a.max_ctx + kr) * HD;
+#pragma unroll
+    for (int i = 0; i < HD8 / 4; i++) vv[i] = *(const u32x4*)(vb + 8 * ((HD8 / 4) * wave + i));
+  }
+  u32x4 kt[4][NJ];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int kr = key0 + 16 * t + c < a.max_ctx ? key0 + 16 * t + c : a.max_ctx - 1;   // (rows beyond the cache are masked below: they lie beyond every position)
+    const _Float16* kb = a.cache_k + ((size_t)kvh * a.max_ctx + kr) * HD + 8 * g;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) kt[t][j] = *(const u32x4*)(kb + 32 * j);
+  }
+  const int pos0 = a.st->pos;
+  const int last = pos0 + (16 * rz + 15 < rows ? 16 * rz + 15 : rows - 1);   // the last position of this row tile
+  if (pos0 < 0 || last >= a.max_ctx) return;             // (refused by the appending launch: state.error)
+  if (key0 > last) return;                               // nothing of this split is visible to the tile
+  const int pos = pos0 + row;
+  // ---- the V tile transposed: key j of the split goes to slot 32 (j / 32) + 8 ((j % 16) / 4) + 4 ((j % 32) / 16) + j % 4 of every dimension's row
+  {
+    const int j = lane, slot = (j & 32) + 8 * ((j & 15) >> 2) + 4 * ((j >> 4) & 1) + (j & 3);
+#pragma unroll
+    for (int i = 0; i < HD8 / 4; i++) {
+      const int d0 = 8 * ((HD8 / 4) * wave + i);
+      const uint32_t w[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
+#pragma unroll
+      for (int e = 0; e < 8; e++) vts[(d0 + e) * VP + slot] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
+  }
+  __syncthreads();
+  for (int hh = wave; hh < group; hh += 4) {
+    const int head = kvh * group + hh;
+    // the rotated query of (row, head): the lane's values 32 j + 8 g + e; the partner of a low value is the value half further, in the same lane (j + NJ / 2)
+    u32x4 qb[NJ];
+    {
+      const float* qrow = a.q + (size_t)row * a.q_bs + (size_t)head * HD;
+      const float* rr = a.rope + (size_t)pos * HD;
+#pragma unroll
+      for (int j = 0; j < NJ / 2; j++) {
+        float lo[8], hi[8];
+#pragma unroll
+        for (int e4 = 0; e4 < 8; e4 += 4) {
+          const int i = 32 * j + 8 * g + e4;
+          const f32x4 x1 = *(const f32x4*)(qrow + i), x2 = *(const f32x4*)(qrow + half + i), cs = *(const f32x4*)(rr + i), sn = *(const f32x4*)(rr + half + i);
+          lo[e4] = rope_lo(x1.x, x2.x, cs.x, sn.x); lo[e4 + 1] = rope_lo(x1.y, x2.y, cs.y, sn.y); lo[e4 + 2] = rope_lo(x1.z, x2.z, cs.z, sn.z); lo[e4 + 3] = rope_lo(x1.w, x2.w, cs.w, sn.w);
+          hi[e4] = rope_hi(x1.x, x2.x, cs.x, sn.x); hi[e4 + 1] = rope_hi(x1.y, x2.y, cs.y, sn.y); hi[e4 + 2] = rope_hi(x1.z, x2.z, cs.z, sn.z); hi[e4 + 3] = rope_hi(x1.w, x2.w, cs.w, sn.w);
+        }
+        qb[j] = pack8_f16(lo); qb[j + NJ / 2] = pack8_f16(hi);
+      }
+    }
+    // scores of the 64 keys x 16 rows
+    v4f32 sc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      sc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < NJ; j++) sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qb[j]), sc[t], 0, 0, 0);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float sv = key0 + 16 * t + 4 * g + i <= pos ? sc[t][i] * a.scale : -INFINITY;
+        sc[t][i] = sv; m = fmaxf(m, sv);
+      }
+    }
+    m = fmaxf(m, __shfl_xor(m, 16, 64)); m = fmaxf(m, __shfl_xor(m, 32, 64));
+    const bool seen = m != -INFINITY;                    // (false: the row lies before this split)
+    float l = 0.f;
+    float pr[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) { const float pj = seen ? __expf(sc[t][i] - m) : 0.f; pr[t][i] = pj; l += pj; }
+    }
+    l += __shfl_xor(l, 16, 64); l += __shfl_xor(l, 32, 64);
+    u32x4 pb[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const float e8[8] = {pr[2 * u][0], pr[2 * u][1], pr[2 * u][2], pr[2 * u][3], pr[2 * u + 1][0], pr[2 * u + 1][1], pr[2 * u + 1][2], pr[2 * u + 1][3]};
+      pb[u] = pack8_f16(e8);
+    }
+    // weighted V sums: dimension tile h, lane (g, c) ends with dimensions 16 h + 4 g + i of row c
+    float* po = a.part + (size_t)row * a.part_bs + ((size_t)head * a.nsplit + split) * (HD + 2);
+#pragma unroll
+    for (int h = 0; h < NH; h++) {
+      v4f32 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        const u32x4 va = *(const u32x4*)(vts + (16 * h + c) * VP + 32 * u + 8 * g);
+        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, va), __builtin_bit_cast(v8f16, pb[u]), o, 0, 0, 0);
+      }
+      if (row_ok && seen) { float* pd = po + 16 * h + 4 * g; pd[0] = o[0]; pd[1] = o[1]; pd[2] = o[2]; pd[3] = o[3]; }
+    }
+    if (row_ok && seen && g == 0) { po[HD] = m; po[HD + 1] = l; }
   }
 }
 
@@ -820,8 +948,16 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
 #define TGA_ATTN_LAUNCH(HD8) do { \
     if (norm == 0) attn_decode_kernel<HD8, 0><<<grid, 256, 0, s>>>(a); else if (norm == 1) attn_decode_kernel<HD8, 1><<<grid, 256, 0, s>>>(a); \
     else if (norm == 2) attn_decode_kernel<HD8, 2><<<grid, 256, 0, s>>>(a); else attn_decode_kernel<HD8, 3><<<grid, 256, 0, s>>>(a); } while (0)
+  static const bool chunk_mfma_off = getenv("TGA_ATTN_CHUNK") && !strcmp(getenv("TGA_ATTN_CHUNK"), "rows");
+  const bool chunk_mfma = chunk && batch > 8 && norm == 0 && (head_dim == 64 || head_dim == 128) && !chunk_mfma_off && !stage_type;   // chunks of more than eight rows attend on the matrix cores
   for (int pass = chunk ? 1 : 0; pass <= (chunk ? 2 : 0); pass++) {   // chunked prefill: append every row, then attend from the cache
     a.chunk = pass;
+    if (pass == 2 && chunk_mfma) {
+      const dim3 cgrid(n_kv_heads, a.nsplit, (batch + 15) / 16);
+      if (head_dim == 64) attn_chunk_mfma_kernel<8><<<cgrid, 256, 0, s>>>(a, batch); else attn_chunk_mfma_kernel<16><<<cgrid, 256, 0, s>>>(a, batch);
+      TGA_LAUNCH_CHECK();
+      break;
+    }
     grid = dim3(n_kv_heads, pass == 1 ? 1 : a.nsplit, batch);
     if (head_dim == 64) TGA_ATTN_LAUNCH(8);
     else if (head_dim == 128) TGA_ATTN_LAUNCH(16);

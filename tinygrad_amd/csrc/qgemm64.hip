@@ -1,0 +1,313 @@
+// Prefill GEMM over GGUF blocks: 17 .. 64 activation rows (the positions of one prefill step, tinygrad/llm/model.py:464, 476-481: a T > 1 call of the same
+// linears, x.linear(W.T) over the lazily dequantized weight, tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392) in ONE pass over the weights.
+// The small-batch kernels multiply sixteen rows per pass (the sixteen columns of one MFMA tile), so a step of 64 positions decoded every weight four times;
+// here a unit is decoded once into fp16 weights (the reference's own fp16 weight cast, model.py:376) and multiplied with two or four column groups.
+//
+// Up to three launches per call, all on the caller's stream:
+//  1. q64_stage_kernel: the activations - up to 64 rows x K, fp16 or float32 - are permuted ONCE into the formats' staged order (Fmt::stage), laid out per step
+//     of 256 values of K as [vector][column group][unit][column] 16-byte pieces: exactly the bytes the multiplying workgroups want in LDS, rows at and beyond M
+//     as zeros.  (When every workgroup staged for itself, each of its 256 threads fetched one 128-byte line in eight instructions that touch 64 lines each:
+//     the texture path, not the matrix cores, set the pace - gate/up of the 8B shapes 54 us, of which 20 us were that fetch.)
+//  2. qgemm64_kernel: a workgroup is four waves and owns 64 weight rows (SwiGLU pair: 32 gate rows and the same 32 up rows), wave w rows 16 w .. 16 w + 15, over
+//     a contiguous range of steps.  As in qgemm.hip lane 16 g + r loads unit 4 s + g of weight row r straight from global memory (a ring of three steps in
+//     flight), decodes it and supplies the A operands of eight v_mfma_f32_16x16x32_f16 per column group; the B operand of lane 16 g + c is the matching vector
+//     of activation row c of that column group, read from LDS.  The staged activations of a step are a straight copy, 1 KB per wave instruction: requested
+//     while the step before is multiplied, written to the other of two LDS stages behind it, one barrier per step.  (Direct-to-LDS loads for this copy,
+//     three stages deep, made the compiler drain every outstanding load - the weight ring included - at each use of a weight register: ordinary loads
+//     keep its counting exact.)
+//     Matrices of few rows (4096: 64 row tiles for 256 CUs) split K over gridDim.y workgroups per row tile, which write float32 partial tiles.
+//  3. q64_reduce_kernel (only when K was split): y = [residual +] the partials summed in the order of K - the same sum whichever workgroup finished first.
+// Without a split the multiplying kernel stores for itself: plain, + residual (in place allowed: every element is read and written by one lane), or
+// silu(gate) * up, for which a lane's gate rows and the matching up rows sit 32 lanes apart.
+//
+// The staged activations (at most 4 MB) and the partial tiles (at most 8 MB) live in a workspace that tga_init allocates once per device: Q64_SLOTS slots, a
+// stream keeps the slot it was given first (launches of one stream are ordered, so they may share one), a call on a further stream gets none and is told to
+// run blocks of sixteen rows instead.
+#include "qfmt.h"
+#include <mutex>
+
+typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+#define Q64_MAX_K 32768
+#define Q64_XS_BYTES ((size_t)64 * Q64_MAX_K * 2)
+#define Q64_PART_BYTES ((size_t)8 << 20)
+#define Q64_SLOTS 4
+#define Q64_MAX_DEVICES 64
+
+struct Q64X {
+  u32x4* xs;            // staged activations: [step][8 vectors][NCG column groups][4 units][16 columns] pieces
+  float* part;          // (K split) partial tiles [split][64 columns][np rows]
+  int ks, np;
+};
+
+template <int T_, int NCG>
+__global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const int M, u32x4* __restrict__ xs) {
+  using F = Fmt<T_>;
+  const int tid = threadIdx.x, scol = tid & 63, sug = tid >> 6, s = blockIdx.x;      // this thread's item: activation row scol, unit 4 s + sug
+  if (scol >= 16 * NCG) return;
+  uint32_t nx[F::UW / 2];
+  stage_fetch<T_>(args, scol < M ? scol : 0, 4 * s + sug, nx);
+  u32x4 xv[F::XV]; float cs[F::NG];
+  F::stage(nx, xv, cs);
+  u32x4* dst = xs + (size_t)s * (F::XV * NCG * 64) + (scol >> 4) * 64 + sug * 16 + (scol & 15);
+#pragma unroll
+  for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = scol < M ? xv[v] : u32x4{0u, 0u, 0u, 0u};
+}
+
+template <int T_, bool MS, bool SW, int NCG>
+__global__ __launch_bounds__(256) void qgemm64_kernel(const QArgs args, const int M, const Q64X ex) {
+  const QArgs a = args;
+  using F = Fmt<T_>;
+  typedef typename F::Raw Raw;
+  static_assert(F::UW == 64 && F::XV == 8, "units of 64 weights in eight vectors");
+  static_assert(!(MS && SW), "the SwiGLU pair is not combined with the q / k / v walk");
+  constexpr int SP = F::XV * NCG * 64;                    // 16-byte pieces of one stage
+  constexpr int NI = SP / 256;                            // pieces per thread and stage (8 or 4)
+  extern __shared__ u32x4 lds[];                          // two stages of SP pieces
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  uint32_t kc[F::NKC];
+  F::consts(kc);
+  const int nsteps = a.nu >> 2;                           // (the launch has checked: whole steps)
+  const int ky = blockIdx.y, s0 = (int)((long long)ky * nsteps / ex.ks), n = (int)((long long)(ky + 1) * nsteps / ex.ks) - s0;   // this workgroup's steps
+  constexpr int WR = SW ? 8 : 16;                         // output rows of one wave
+  // the 16 weight rows of this wave: one segment (q / k / v: every segment a multiple of 16 rows), rows at and beyond its end repeat the last one
+  const long long grow0 = ((long long)blockIdx.x * 4 + wave) * WR;     // first output row of the wave (over all segments)
+  long long row0 = grow0;
+  const uint8_t* wb = a.w[0]; long long nrows = a.n[0]; int sg = 0;
+  if constexpr (MS) {
+    if (row0 >= a.n[0]) { row0 -= a.n[0]; sg = 1; wb = a.w[1]; nrows = a.n[1]; if (a.nseg > 2 && row0 >= a.n[1]) { row0 -= a.n[1]; sg = 2; wb = a.w[2]; nrows = a.n[2]; } }
+  }
+  const bool wave_has_rows = row0 < nrows;
+  long long wrow = row0 + (SW ? (r & 7) : r); wrow = wrow < nrows ? wrow : nrows - 1; wrow = wrow < 0 ? 0 : wrow;
+  const uint8_t* rowp = ((SW && r >= 8) ? a.w[1] : wb) + wrow * a.row_bytes;
+
+  // this thread's pieces of a stage: 64 (NI wave + j) + lane, j < NI - a straight copy, 1 KB per wave instruction
+  u32x4 xr[NI];
+  auto fetch = [&](int i) __attribute__((always_inline)) {
+    const u32x4* src = ex.xs + (size_t)(s0 + i) * SP + wave * NI * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < NI; j++) xr[j] = src[j * 64];
+  };
+  auto put = [&](int st) __attribute__((always_inline)) {
+    u32x4* dst = lds + st * SP + wave * NI * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < NI; j++) dst[j * 64] = xr[j];
+  };
+  Raw wq[3];
+  fetch(0);                                               // activations first, weights second: loads return in issue order
+  wq[0] = F::load(rowp, 4 * s0 + g);
+  wq[1] = F::load(rowp, 4 * (s0 + (n > 1 ? 1 : 0)) + g);
+  put(0);
+  __syncthreads();
+  v4f32 acc[NCG];
+#pragma unroll
+  for (int cg = 0; cg < NCG; cg++) acc[cg] = v4f32{0.f, 0.f, 0.f, 0.f};
+  auto compute = [&](const Raw& buf, int slot) __attribute__((always_inline)) {
+    uint32_t wv[F::NWV];
+    F::decode(buf, wv, kc);
+    F::to_f16(buf, wv);
+    const u32x4* src = lds + slot * SP + lane;
+#pragma unroll
+    for (int v = 0; v < F::XV; v++) {
+      const u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
+#pragma unroll
+      for (int cg = 0; cg < NCG; cg++)
+        acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, src[(v * NCG + cg) * 64]), acc[cg], 0, 0, 0);
+    }
+  };
+  auto step = [&](const Raw& cur, Raw& nxt2, int i) __attribute__((always_inline)) {
+    const int i1 = i + 1 < n ? i + 1 : n - 1, i2 = i + 2 < n ? i + 2 : n - 1;
+    fetch(i1);                                            // (past the end: the last step again, staged into a buffer nobody reads)
+    nxt2 = F::load(rowp, 4 * (s0 + i2) + g);
+    compute(cur, i & 1);
+    put((i + 1) & 1);
+    __syncthreads();
+  };
+  int i = 0;
+  for (; i + 3 <= n; i += 3) { step(wq[0], wq[2], i); step(wq[1], wq[0], i + 1); step(wq[2], wq[1], i + 2); }
+  if (i < n) { step(wq[0], wq[2], i); i++; }
+  if (i < n) { step(wq[1], wq[0], i); i++; }
+
+  // ---- epilogue: lane (g, c) holds, per column group, activation row 16 cg + c x weight rows 4 g .. 4 g + 3 of the wave
+  const int c = r;
+  if (ex.ks > 1) {                                        // partial tile: [split][column][padded row], every lane stores its four rows
+#pragma unroll
+    for (int cg = 0; cg < NCG; cg++)
+      *(v4f32*)(ex.part + ((size_t)ky * 64 + 16 * cg + c) * ex.np + grow0 + 4 * g) = acc[cg];
+    return;
+  }
+  if (!wave_has_rows) return;
+  if constexpr (SW) {
+#pragma unroll
+    for (int cg = 0; cg < NCG; cg++) {
+      float up[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) up[k] = __shfl_down(acc[cg][k], 32, 64);
+      const int col = 16 * cg + c;
+      if (g < 2 && col < M) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const long long row = row0 + 4 * g + k;
+          if (row < nrows) {
+            const float v = silu_f(acc[cg][k]) * up[k];
+            const long long o = (long long)col * nrows + row;
+            if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+          }
+        }
+      }
+    }
+  } else {
+    void* yb = !MS ? a.y[0] : sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
+    const float* rb = a.epilogue == 1 ? (!MS ? a.resid[0] : sg == 0 ? a.resid[0] : sg == 1 ? a.resid[1] : a.resid[2]) : nullptr;
+#pragma unroll
+    for (int cg = 0; cg < NCG; cg++) {
+      const int col = 16 * cg + c;
+      if (col < M) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+          const long long row = row0 + 4 * g + k;
+          if (row < nrows) {
+            const long long o = (long long)col * nrows + row;
+            float v = acc[cg][k];
+            if (rb) v += rb[o];
+            if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
+          }
+        }
+      }
+    }
+  }
+}
+
+// y = [residual +] sum over the splits, in the order of K.  One thread per (activation row, four consecutive padded weight rows).
+__global__ __launch_bounds__(256) void q64_reduce_kernel(const QArgs a, const int M, const float* __restrict__ part, const int ks, const int np) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int q = np >> 2;
+  const int m = (int)(idx / q); long long row = 4 * (idx - (long long)m * q);
+  if (m >= M) return;
+  v4f32 v = *(const v4f32*)(part + (size_t)m * np + row);
+  for (int k = 1; k < ks; k++) { const v4f32 t = *(const v4f32*)(part + ((size_t)k * 64 + m) * np + row); v += t; }
+  int sg = 0; long long nrows = a.n[0];
+  if (a.nseg > 1 && row >= a.n[0]) { row -= a.n[0]; sg = 1; nrows = a.n[1]; if (a.nseg > 2 && row >= a.n[1]) { row -= a.n[1]; sg = 2; nrows = a.n[2]; } }
+  void* yb = sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
+  const float* rb = a.epilogue == 1 ? (sg == 0 ? a.resid[0] : sg == 1 ? a.resid[1] : a.resid[2]) : nullptr;
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    if (row + k < nrows) {
+      const long long o = (long long)m * nrows + row + k;
+      float t = v[k];
+      if (rb) t += rb[o];
+      if (a.y_f32) ((float*)yb)[o] = t; else ((_Float16*)yb)[o] = (_Float16)t;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------- workspace
+static uint8_t* g_q64_ws[Q64_MAX_DEVICES];                 // device d: Q64_SLOTS x (staged activations, partial tiles), allocated by tga_qgemm64_setup(d)
+static hipStream_t g_q64_owner[Q64_MAX_DEVICES][Q64_SLOTS];
+static bool g_q64_taken[Q64_MAX_DEVICES][Q64_SLOTS];
+static std::mutex g_q64_mu;
+
+int tga_qgemm64_setup(int device) {                         // called by tga_init after hipSetDevice(device)
+  TGA_REQUIRE(device >= 0 && device < Q64_MAX_DEVICES, "tga_init: device %d is beyond the %d devices the prefill workspace table covers", device, Q64_MAX_DEVICES);
+  std::lock_guard<std::mutex> lk(g_q64_mu);
+  if (g_q64_ws[device]) return 0;
+  void* p = nullptr;
+  TGA_HIP(hipMalloc(&p, Q64_SLOTS * (Q64_XS_BYTES + Q64_PART_BYTES)));
+  g_q64_ws[device] = (uint8_t*)p;
+  return 0;
+}
+
+static uint8_t* q64_slot(hipStream_t s) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= Q64_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lk(g_q64_mu);
+  if (!g_q64_ws[dev]) return nullptr;
+  int free_slot = -1;
+  for (int i = 0; i < Q64_SLOTS; i++) {
+    if (g_q64_taken[dev][i] && g_q64_owner[dev][i] == s) return g_q64_ws[dev] + (size_t)i * (Q64_XS_BYTES + Q64_PART_BYTES);
+    if (!g_q64_taken[dev][i] && free_slot < 0) free_slot = i;
+  }
+  if (free_slot < 0) return nullptr;
+  g_q64_taken[dev][free_slot] = true; g_q64_owner[dev][free_slot] = s;
+  return g_q64_ws[dev] + (size_t)free_slot * (Q64_XS_BYTES + Q64_PART_BYTES);
+}
+
+// The stream is about to be destroyed (tga_stream_destroy, which has waited for its work): the slot it holds, on whichever device, is free again.
+void tga_qgemm64_release(hipStream_t s) {
+  std::lock_guard<std::mutex> lk(g_q64_mu);
+  for (int d = 0; d < Q64_MAX_DEVICES; d++)
+    for (int i = 0; i < Q64_SLOTS; i++)
+      if (g_q64_taken[d][i] && g_q64_owner[d][i] == s) g_q64_taken[d][i] = false;
+}
+
+template <int T, bool MS, bool SW, int NCG>
+static int launch_q64_v(const QArgs& a, int M, long long tiles, uint8_t* ws, hipStream_t s) {
+  using F = Fmt<T>;
+  auto kern = qgemm64_kernel<T, MS, SW, NCG>;
+  static const int env_ks = getenv("TGA_Q64_KS") ? atoi(getenv("TGA_Q64_KS")) : 0;
+  constexpr size_t stage_bytes = (size_t)F::XV * NCG * 64 * 16;
+  static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * stage_bytes));
+  TGA_HIP(configured);
+  const int nsteps = a.nu >> 2;
+  Q64X ex;
+  ex.xs = (u32x4*)ws; ex.part = (float*)(ws + Q64_XS_BYTES); ex.np = (int)(tiles * 64);
+  // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows; about 512 workgroups of at least four steps, partial tiles within the workspace
+  int ks = 1;
+  if (!SW && tiles < 192) {
+    ks = (int)((512 + tiles / 2) / tiles);
+    if (ks > nsteps / 4) ks = nsteps / 4;
+  }
+  if (env_ks >= 1 && !SW) ks = env_ks < nsteps ? env_ks : nsteps;
+  while (ks > 1 && (size_t)ks * 64 * ex.np * 4 > Q64_PART_BYTES) ks--;
+  if (ks < 1) ks = 1;
+  ex.ks = ks;
+  q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
+  TGA_LAUNCH_CHECK();
+  kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(256), 2 * stage_bytes, s>>>(a, M, ex);
+  TGA_LAUNCH_CHECK();
+  if (ks > 1) {
+    const long long items = (long long)M * (ex.np / 4);
+    q64_reduce_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s>>>(a, M, ex.part, ks, ex.np);
+    TGA_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+template <int T>
+static int launch_q64(QArgs a, int M, uint8_t* ws, hipStream_t s) {
+  using F = Fmt<T>;
+  if constexpr (F::UW != 64 || F::XV != 8) return -1;
+  else {
+    a.nu = a.K / F::UW;
+    a.row_bytes = (long long)(a.K / F::BW) * F::BB;
+    const bool two = M <= 32;                             // two column groups instead of four: half the MFMAs and half the staged bytes
+    if (a.epilogue == 2) { const long long t = (a.n[0] + 31) / 32; return two ? launch_q64_v<T, false, true, 2>(a, M, t, ws, s) : launch_q64_v<T, false, true, 4>(a, M, t, ws, s); }
+    const long long tiles = (a.ntot + 63) / 64;
+    if (a.nseg > 1) return two ? launch_q64_v<T, true, false, 2>(a, M, tiles, ws, s) : launch_q64_v<T, true, false, 4>(a, M, tiles, ws, s);
+    return two ? launch_q64_v<T, false, false, 2>(a, M, tiles, ws, s) : launch_q64_v<T, false, false, 4>(a, M, tiles, ws, s);
+  }
+}
+
+// Returns -1 when the call is outside this kernel's range (the caller then runs blocks of sixteen rows): 17 .. 64 rows of fp16 or float32 activations, K a
+// multiple of 256 up to Q64_MAX_K, one to three matrices (several: each a multiple of 16 rows) with the plain or residual epilogue, or the SwiGLU pair; and
+// when no workspace slot is left for the stream.
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
+  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y) return -1;
+  if (a.nseg > 1 && a.epilogue != 2) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return -1;
+  if (((uintptr_t)a.x & 15) != 0) return -1;
+  switch (fmt) { case F_Q4_0P: case F_Q8_0P: case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_F16: break; default: return -1; }
+  uint8_t* ws = q64_slot(s);
+  if (!ws) return -1;
+  switch (fmt) {
+    case F_Q4_0P: return launch_q64<F_Q4_0P>(a, M, ws, s);
+    case F_Q8_0P: return launch_q64<F_Q8_0P>(a, M, ws, s);
+    case GGML_Q6_K: return launch_q64<GGML_Q6_K>(a, M, ws, s);
+    case GGML_Q4_K: return launch_q64<GGML_Q4_K>(a, M, ws, s);
+    case GGML_Q5_K: return launch_q64<GGML_Q5_K>(a, M, ws, s);
+    case GGML_IQ4_XS: return launch_q64<GGML_IQ4_XS>(a, M, ws, s);
+    case GGML_F16: return launch_q64<GGML_F16>(a, M, ws, s);
+  }
+  return -1;
+}

@@ -318,6 +318,7 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    // qgemm_dma.hip
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);       // qgemm64.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -384,6 +385,23 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG && !comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32) && !y_stage_type && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
                 "tga_qlinear: more than 16 rows only for plain fp16 / float32 activations");
     for (int i = 0; i < nseg; i++) TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]), "tga_qlinear: segment %d has a null pointer or no rows", i);
+    TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
+    TGA_REQUIRE(epilogue != 1 || y_dtype == TGA_F32, "tga_qlinear: the residual epilogue needs float32 y");
+    TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
+    {                                                             // one pass over the weights for all rows where the 64-column kernel applies (qgemm64.hip)
+      bool pair64 = K > 0 && (K / 32) % 2 == 0;
+      for (int i = 0; i < nseg; i++) pair64 = pair64 && ((uintptr_t)w[i] & 3) == 0;
+      const int fmt64 = ggml_type == GGML_Q4_0 ? (pair64 ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair64 ? F_Q8_0P : -1) : ggml_type;
+      if (fmt64 >= 0 && pair64) {
+        QArgs q = {};
+        q.nseg = nseg; q.x = x; q.x_f32 = x_dtype == TGA_F32; q.y_f32 = y_dtype == TGA_F32; q.epilogue = epilogue; q.K = (int)K;
+        long long nt = 0;
+        for (int i = 0; i < nseg; i++) { q.w[i] = (const uint8_t*)w[i]; q.y[i] = y[i]; q.n[i] = n[i]; q.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr; nt += n[i]; }
+        q.ntot = epilogue == 2 ? n[0] : nt;
+        const int rc = tga_qgemm64_dispatch(fmt64, q, M, (hipStream_t)stream);
+        if (rc >= 0) return rc;
+      }
+    }
     return qlinear_row_blocks(16, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
   }
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
