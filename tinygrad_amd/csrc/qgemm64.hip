@@ -55,8 +55,8 @@ __global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const 
   for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = scol < M ? xv[v] : u32x4{0u, 0u, 0u, 0u};
 }
 
-template <int T_, bool MS, bool SW, int NCG>
-__global__ __launch_bounds__(256) void qgemm64_kernel(const QArgs args, const int M, const Q64X ex) {
+template <int T_, bool MS, bool SW, int NCG, int NT>
+__global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const int M, const Q64X ex) {
   const QArgs a = args;
   using F = Fmt<T_>;
   typedef typename F::Raw Raw;
@@ -71,58 +71,89 @@ __global__ __launch_bounds__(256) void qgemm64_kernel(const QArgs args, const in
   F::consts(kc);
   const int nsteps = a.nu >> 2;                           // (the launch has checked: whole steps)
   const int ky = blockIdx.y, s0 = (int)((long long)ky * nsteps / ex.ks), n = (int)((long long)(ky + 1) * nsteps / ex.ks) - s0;   // this workgroup's steps
-  constexpr int WR = SW ? 8 : 16;                         // output rows of one wave
-  // the 16 weight rows of this wave: one segment (q / k / v: every segment a multiple of 16 rows), rows at and beyond its end repeat the last one
-  const long long grow0 = ((long long)blockIdx.x * 4 + wave) * WR;     // first output row of the wave (over all segments)
-  long long row0 = grow0;
-  const uint8_t* wb = a.w[0]; long long nrows = a.n[0]; int sg = 0;
-  if constexpr (MS) {
-    if (row0 >= a.n[0]) { row0 -= a.n[0]; sg = 1; wb = a.w[1]; nrows = a.n[1]; if (a.nseg > 2 && row0 >= a.n[1]) { row0 -= a.n[1]; sg = 2; wb = a.w[2]; nrows = a.n[2]; } }
+  constexpr int WR = SW ? 8 : 16;                         // output rows of one weight tile
+  // The NT weight tiles of this wave, 16 weight rows each (SwiGLU: 8 gate rows and the same 8 up rows).  A tile lies in one segment (q / k / v: every segment a
+  // multiple of 16 rows); rows at and beyond the segment's end repeat its last one.
+  long long grow0[NT], row0[NT], nrows[NT]; int sg[NT]; bool has_rows[NT]; const uint8_t* rowp[NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) {
+    grow0[t] = (((long long)blockIdx.x * 4 + wave) * NT + t) * WR;     // first output row of the tile (over all segments)
+    row0[t] = grow0[t];
+    const uint8_t* wb = a.w[0]; nrows[t] = a.n[0]; sg[t] = 0;
+    if constexpr (MS) {
+      if (row0[t] >= a.n[0]) {
+        row0[t] -= a.n[0]; sg[t] = 1; wb = a.w[1]; nrows[t] = a.n[1];
+        if (a.nseg > 2 && row0[t] >= a.n[1]) { row0[t] -= a.n[1]; sg[t] = 2; wb = a.w[2]; nrows[t] = a.n[2]; }
+      }
+    }
+    has_rows[t] = row0[t] < nrows[t];
+    long long wrow = row0[t] + (SW ? (r & 7) : r); wrow = wrow < nrows[t] ? wrow : nrows[t] - 1; wrow = wrow < 0 ? 0 : wrow;
+    rowp[t] = ((SW && r >= 8) ? a.w[1] : wb) + wrow * a.row_bytes;
   }
-  const bool wave_has_rows = row0 < nrows;
-  long long wrow = row0 + (SW ? (r & 7) : r); wrow = wrow < nrows ? wrow : nrows - 1; wrow = wrow < 0 ? 0 : wrow;
-  const uint8_t* rowp = ((SW && r >= 8) ? a.w[1] : wb) + wrow * a.row_bytes;
 
-  // this thread's pieces of a stage: 64 (NI wave + j) + lane, j < NI - a straight copy, 1 KB per wave instruction
-  u32x4 xr[NI];
-  auto fetch = [&](int i) __attribute__((always_inline)) {
-    const u32x4* src = ex.xs + (size_t)(s0 + i) * SP + wave * NI * 64 + lane;
+  // Waves 4 .. 7 stage: wave 4 + w copies pieces 64 (NI w + j) + lane, j < NI, of every stage - 1 KB per instruction - two steps ahead of its use, through two
+  // register sets in turn.  They issue nothing else, so these loads (L2 hits) never queue behind a weight load from HBM: loads return in the order of issue,
+  // and a copy requested by the multiplying waves themselves arrived no earlier than the weights requested a step before it.
+  if (wave >= 4) {
+    const int sw = wave - 4;
+    u32x4 xa[NI], xb[NI];
+    auto fetch = [&](int i, u32x4 (&xr)[NI]) __attribute__((always_inline)) {
+      const u32x4* src = ex.xs + (size_t)(s0 + (i < n ? i : n - 1)) * SP + sw * NI * 64 + lane;   // (past the end: the last stage again, never written to LDS)
 #pragma unroll
-    for (int j = 0; j < NI; j++) xr[j] = src[j * 64];
-  };
-  auto put = [&](int st) __attribute__((always_inline)) {
-    u32x4* dst = lds + st * SP + wave * NI * 64 + lane;
+      for (int j = 0; j < NI; j++) xr[j] = src[j * 64];
+    };
+    auto put = [&](int st, const u32x4 (&xr)[NI]) __attribute__((always_inline)) {
+      u32x4* dst = lds + st * SP + sw * NI * 64 + lane;
 #pragma unroll
-    for (int j = 0; j < NI; j++) dst[j * 64] = xr[j];
-  };
-  Raw wq[3];
-  fetch(0);                                               // activations first, weights second: loads return in issue order
-  wq[0] = F::load(rowp, 4 * s0 + g);
-  wq[1] = F::load(rowp, 4 * (s0 + (n > 1 ? 1 : 0)) + g);
-  put(0);
+      for (int j = 0; j < NI; j++) dst[j * 64] = xr[j];
+    };
+    fetch(0, xa); fetch(1, xb);
+    put(0, xa);
+    fetch(2, xa);
+    __syncthreads();
+    int i = 0;                                            // step i: stage i + 1 goes to LDS (requested two steps ago), stage i + 3 is requested
+    for (; i + 2 <= n; i += 2) {
+      put((i + 1) & 1, xb); fetch(i + 3, xb); __syncthreads();
+      put(i & 1, xa); fetch(i + 4, xa); __syncthreads();
+    }
+    if (i < n) { put((i + 1) & 1, xb); __syncthreads(); }
+    return;
+  }
+  Raw wq[3][NT];
+#pragma unroll
+  for (int t = 0; t < NT; t++) wq[0][t] = F::load(rowp[t], 4 * s0 + g);
+#pragma unroll
+  for (int t = 0; t < NT; t++) wq[1][t] = F::load(rowp[t], 4 * (s0 + (n > 1 ? 1 : 0)) + g);
   __syncthreads();
-  v4f32 acc[NCG];
+  v4f32 acc[NT][NCG];
 #pragma unroll
-  for (int cg = 0; cg < NCG; cg++) acc[cg] = v4f32{0.f, 0.f, 0.f, 0.f};
-  auto compute = [&](const Raw& buf, int slot) __attribute__((always_inline)) {
-    uint32_t wv[F::NWV];
-    F::decode(buf, wv, kc);
-    F::to_f16(buf, wv);
+  for (int t = 0; t < NT; t++)
+#pragma unroll
+    for (int cg = 0; cg < NCG; cg++) acc[t][cg] = v4f32{0.f, 0.f, 0.f, 0.f};
+  auto compute = [&](const Raw (&buf)[NT], int slot) __attribute__((always_inline)) {
+    uint32_t wv[NT][F::NWV];
+#pragma unroll
+    for (int t = 0; t < NT; t++) { F::decode(buf[t], wv[t], kc); F::to_f16(buf[t], wv[t]); }
     const u32x4* src = lds + slot * SP + lane;
 #pragma unroll
     for (int v = 0; v < F::XV; v++) {
-      const u32x4 av = {wv[4 * v], wv[4 * v + 1], wv[4 * v + 2], wv[4 * v + 3]};
+      u32x4 bv[NCG];                                      // a B operand is read once and meets the NT weight tiles
 #pragma unroll
-      for (int cg = 0; cg < NCG; cg++)
-        acc[cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, src[(v * NCG + cg) * 64]), acc[cg], 0, 0, 0);
+      for (int cg = 0; cg < NCG; cg++) bv[cg] = src[(v * NCG + cg) * 64];
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        const u32x4 av = {wv[t][4 * v], wv[t][4 * v + 1], wv[t][4 * v + 2], wv[t][4 * v + 3]};
+#pragma unroll
+        for (int cg = 0; cg < NCG; cg++)
+          acc[t][cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[cg]), acc[t][cg], 0, 0, 0);
+      }
     }
   };
-  auto step = [&](const Raw& cur, Raw& nxt2, int i) __attribute__((always_inline)) {
-    const int i1 = i + 1 < n ? i + 1 : n - 1, i2 = i + 2 < n ? i + 2 : n - 1;
-    fetch(i1);                                            // (past the end: the last step again, staged into a buffer nobody reads)
-    nxt2 = F::load(rowp, 4 * (s0 + i2) + g);
+  auto step = [&](const Raw (&cur)[NT], Raw (&nxt2)[NT], int i) __attribute__((always_inline)) {
+    const int i2 = i + 2 < n ? i + 2 : n - 1;
+#pragma unroll
+    for (int t = 0; t < NT; t++) nxt2[t] = F::load(rowp[t], 4 * (s0 + i2) + g);
     compute(cur, i & 1);
-    put((i + 1) & 1);
     __syncthreads();
   };
   int i = 0;
@@ -130,49 +161,52 @@ __global__ __launch_bounds__(256) void qgemm64_kernel(const QArgs args, const in
   if (i < n) { step(wq[0], wq[2], i); i++; }
   if (i < n) { step(wq[1], wq[0], i); i++; }
 
-  // ---- epilogue: lane (g, c) holds, per column group, activation row 16 cg + c x weight rows 4 g .. 4 g + 3 of the wave
+  // ---- epilogue: lane (g, c) holds, per tile and column group, activation row 16 cg + c x weight rows 4 g .. 4 g + 3 of the tile
   const int c = r;
-  if (ex.ks > 1) {                                        // partial tile: [split][column][padded row], every lane stores its four rows
 #pragma unroll
-    for (int cg = 0; cg < NCG; cg++)
-      *(v4f32*)(ex.part + ((size_t)ky * 64 + 16 * cg + c) * ex.np + grow0 + 4 * g) = acc[cg];
-    return;
-  }
-  if (!wave_has_rows) return;
-  if constexpr (SW) {
+  for (int t = 0; t < NT; t++) {
+    if (ex.ks > 1) {                                      // partial tile: [split][column][padded row], every lane stores its four rows
 #pragma unroll
-    for (int cg = 0; cg < NCG; cg++) {
-      float up[4];
+      for (int cg = 0; cg < NCG; cg++)
+        *(v4f32*)(ex.part + ((size_t)ky * 64 + 16 * cg + c) * ex.np + grow0[t] + 4 * g) = acc[t][cg];
+      continue;
+    }
+    if (!has_rows[t]) continue;
+    if constexpr (SW) {
 #pragma unroll
-      for (int k = 0; k < 4; k++) up[k] = __shfl_down(acc[cg][k], 32, 64);
-      const int col = 16 * cg + c;
-      if (g < 2 && col < M) {
+      for (int cg = 0; cg < NCG; cg++) {
+        float up[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-          const long long row = row0 + 4 * g + k;
-          if (row < nrows) {
-            const float v = silu_f(acc[cg][k]) * up[k];
-            const long long o = (long long)col * nrows + row;
-            if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+        for (int k = 0; k < 4; k++) up[k] = __shfl_down(acc[t][cg][k], 32, 64);
+        const int col = 16 * cg + c;
+        if (g < 2 && col < M) {
+#pragma unroll
+          for (int k = 0; k < 4; k++) {
+            const long long row = row0[t] + 4 * g + k;
+            if (row < nrows[t]) {
+              const float v = silu_f(acc[t][cg][k]) * up[k];
+              const long long o = (long long)col * nrows[t] + row;
+              if (a.y_f32) ((float*)a.y[0])[o] = v; else ((_Float16*)a.y[0])[o] = (_Float16)v;
+            }
           }
         }
       }
-    }
-  } else {
-    void* yb = !MS ? a.y[0] : sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
-    const float* rb = a.epilogue == 1 ? (!MS ? a.resid[0] : sg == 0 ? a.resid[0] : sg == 1 ? a.resid[1] : a.resid[2]) : nullptr;
+    } else {
+      void* yb = !MS ? a.y[0] : sg[t] == 0 ? a.y[0] : sg[t] == 1 ? a.y[1] : a.y[2];
+      const float* rb = a.epilogue == 1 ? (!MS ? a.resid[0] : sg[t] == 0 ? a.resid[0] : sg[t] == 1 ? a.resid[1] : a.resid[2]) : nullptr;
 #pragma unroll
-    for (int cg = 0; cg < NCG; cg++) {
-      const int col = 16 * cg + c;
-      if (col < M) {
+      for (int cg = 0; cg < NCG; cg++) {
+        const int col = 16 * cg + c;
+        if (col < M) {
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-          const long long row = row0 + 4 * g + k;
-          if (row < nrows) {
-            const long long o = (long long)col * nrows + row;
-            float v = acc[cg][k];
-            if (rb) v += rb[o];
-            if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
+          for (int k = 0; k < 4; k++) {
+            const long long row = row0[t] + 4 * g + k;
+            if (row < nrows[t]) {
+              const long long o = (long long)col * nrows[t] + row;
+              float v = acc[t][cg][k];
+              if (rb) v += rb[o];
+              if (a.y_f32) ((float*)yb)[o] = v; else ((_Float16*)yb)[o] = (_Float16)v;
+            }
           }
         }
       }
@@ -242,30 +276,36 @@ void tga_qgemm64_release(hipStream_t s) {
       if (g_q64_taken[d][i] && g_q64_owner[d][i] == s) g_q64_taken[d][i] = false;
 }
 
-template <int T, bool MS, bool SW, int NCG>
-static int launch_q64_v(const QArgs& a, int M, long long tiles, uint8_t* ws, hipStream_t s) {
-  using F = Fmt<T>;
-  auto kern = qgemm64_kernel<T, MS, SW, NCG>;
+static int q64_split(bool sw, long long tiles, int nsteps) {   // workgroups per row tile: about 512 workgroups of at least four steps, partial tiles within the workspace
   static const int env_ks = getenv("TGA_Q64_KS") ? atoi(getenv("TGA_Q64_KS")) : 0;
+  int ks = 1;
+  if (!sw && tiles < 192) {
+    ks = (int)((512 + tiles / 2) / tiles);
+    if (ks > nsteps / 4) ks = nsteps / 4;
+  }
+  if (env_ks >= 1 && !sw) ks = env_ks < nsteps ? env_ks : nsteps;
+  if (ks < 1) ks = 1;
+  return ks;
+}
+
+template <int T, bool MS, bool SW, int NCG, int NT>
+static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
+  using F = Fmt<T>;
+  auto kern = qgemm64_kernel<T, MS, SW, NCG, NT>;
   constexpr size_t stage_bytes = (size_t)F::XV * NCG * 64 * 16;
   static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * stage_bytes));
   TGA_HIP(configured);
   const int nsteps = a.nu >> 2;
+  const long long tiles = (a.ntot + 64 * NT / (SW ? 2 : 1) - 1) / (64 * NT / (SW ? 2 : 1));   // workgroups over the rows: 64 NT weight rows each (SwiGLU: half of them gate rows)
   Q64X ex;
-  ex.xs = (u32x4*)ws; ex.part = (float*)(ws + Q64_XS_BYTES); ex.np = (int)(tiles * 64);
-  // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows; about 512 workgroups of at least four steps, partial tiles within the workspace
-  int ks = 1;
-  if (!SW && tiles < 192) {
-    ks = (int)((512 + tiles / 2) / tiles);
-    if (ks > nsteps / 4) ks = nsteps / 4;
-  }
-  if (env_ks >= 1 && !SW) ks = env_ks < nsteps ? env_ks : nsteps;
+  ex.xs = (u32x4*)ws; ex.part = (float*)(ws + Q64_XS_BYTES); ex.np = (int)(tiles * 64 * NT);
+  // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows
+  int ks = q64_split(SW, tiles, nsteps);
   while (ks > 1 && (size_t)ks * 64 * ex.np * 4 > Q64_PART_BYTES) ks--;
-  if (ks < 1) ks = 1;
   ex.ks = ks;
   q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
   TGA_LAUNCH_CHECK();
-  kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(256), 2 * stage_bytes, s>>>(a, M, ex);
+  kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(512), 2 * stage_bytes, s>>>(a, M, ex);
   TGA_LAUNCH_CHECK();
   if (ks > 1) {
     const long long items = (long long)M * (ex.np / 4);
@@ -273,6 +313,20 @@ static int launch_q64_v(const QArgs& a, int M, long long tiles, uint8_t* ws, hip
     TGA_LAUNCH_CHECK();
   }
   return 0;
+}
+
+template <int T, bool MS, bool SW, int NCG>
+static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
+  using F = Fmt<T>;
+  // Two weight tiles per wave halve the activation bytes that reach a CU (global -> LDS -> operand) per weight; taken when the row tiles of 128, split over K,
+  // still fill the chip.  (fp16 weights: a unit is 128 bytes per lane, a ring of three steps for two tiles does not fit the registers.)
+  static const int env_nt = getenv("TGA_Q64_NT") ? atoi(getenv("TGA_Q64_NT")) : 0;
+  const int nsteps = a.nu >> 2;
+  const long long rows_wg2 = SW ? 64 : 128, tiles2 = (a.ntot + rows_wg2 - 1) / rows_wg2;
+  bool two = sizeof(typename F::Raw) <= 64 && tiles2 * q64_split(SW, tiles2, nsteps) >= 224;
+  if (env_nt == 1) two = false; else if (env_nt == 2) two = sizeof(typename F::Raw) <= 64;
+  if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, s); }
+  return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, s);
 }
 
 template <int T>
@@ -283,10 +337,9 @@ static int launch_q64(QArgs a, int M, uint8_t* ws, hipStream_t s) {
     a.nu = a.K / F::UW;
     a.row_bytes = (long long)(a.K / F::BW) * F::BB;
     const bool two = M <= 32;                             // two column groups instead of four: half the MFMAs and half the staged bytes
-    if (a.epilogue == 2) { const long long t = (a.n[0] + 31) / 32; return two ? launch_q64_v<T, false, true, 2>(a, M, t, ws, s) : launch_q64_v<T, false, true, 4>(a, M, t, ws, s); }
-    const long long tiles = (a.ntot + 63) / 64;
-    if (a.nseg > 1) return two ? launch_q64_v<T, true, false, 2>(a, M, tiles, ws, s) : launch_q64_v<T, true, false, 4>(a, M, tiles, ws, s);
-    return two ? launch_q64_v<T, false, false, 2>(a, M, tiles, ws, s) : launch_q64_v<T, false, false, 4>(a, M, tiles, ws, s);
+    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, s) : launch_q64_t<T, false, true, 4>(a, M, ws, s);
+    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, s) : launch_q64_t<T, true, false, 4>(a, M, ws, s);
+    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, s) : launch_q64_t<T, false, false, 4>(a, M, ws, s);
   }
 }
 
