@@ -55,9 +55,16 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 template <bool COMB>
 __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* x, const float* __restrict__ w, int dim, float eps,
                                                        _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu,
-                                                       float* x_rw, const float* __restrict__ y, const float* __restrict__ probs, int k) {
+                                                       float* x_rw, const float* __restrict__ y, const float* __restrict__ probs, int k,
+                                                       _Float16* __restrict__ rows_staged, int rs_ncg, int rows_real) {
   __shared__ float red[16];
   const int row = blockIdx.x;                           // one workgroup per row
+  // rows_staged != nullptr: the normalised rows also go, in the order of rows_staged_pos(stage_fmt, ., stage_nu, row, rs_ncg), to the buffer that the
+  // 17 .. 64 row GEMM multiplies from (out16 then keeps the plain order); workgroups at and beyond rows_real only fill their rows of it with zeros
+  if (rows_staged && row >= rows_real) {
+    for (int e = threadIdx.x; e < dim; e += blockDim.x) rows_staged[rows_staged_pos(stage_fmt, e, stage_nu, row, rs_ncg)] = (_Float16)0.f;
+    return;
+  }
   x += (size_t)row * dim;
   if (out16) out16 += (size_t)row * dim;
   if (out32) out32 += (size_t)row * dim;
@@ -99,7 +106,8 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* x, const flo
   for (int i = 0; i < nw; i++) tot += red[i];
   const float scale = 1.0f / sqrtf(tot / (float)dim + eps);
   auto emit = [&](int e, float v) {
-    if (out16) out16[stage_fmt ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
+    if (out16) out16[stage_fmt && !rows_staged ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
+    if (rows_staged) rows_staged[rows_staged_pos(stage_fmt, e, stage_nu, row, rs_ncg)] = (_Float16)v;
     if (out32) out32[e] = v;
   };
   if (e0 < dim) emit(e0, (v0 * scale) * w0);
@@ -904,15 +912,24 @@ int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, flo
   TGA_REQUIRE(dim > 0 && rows >= 1, "tga_rmsnorm: rows=%d dim=%d", rows, dim);
   int sfmt = 0, snu = 0;
   if (stage_type) { sfmt = decode_staged_fmt(stage_type, dim, &snu); TGA_REQUIRE(sfmt >= 0, "tga_rmsnorm: no staged layout for type %d with K=%d", stage_type, dim); }
-  rmsnorm_kernel<false><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu, nullptr, nullptr, nullptr, 0);
+  rmsnorm_kernel<false><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu, nullptr, nullptr, nullptr, 0, nullptr, 0, 0);
   TGA_LAUNCH_CHECK();
   return 0;
 }
+}  // extern "C"
+// tga_rmsnorm_rows whose fp16 rows also go to `staged`, in the layout the 17 .. 64 row GEMM multiplies from (format fmt of nu units per row, ncg column groups of
+// sixteen rows; the rows from `rows` up to 16 ncg are zeros there)
+int tga_rmsnorm_rows_staged64(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, int fmt, int nu, void* staged, int ncg, void* stream) {
+  rmsnorm_kernel<false><<<16 * ncg, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, nullptr, fmt, nu, nullptr, nullptr, nullptr, 0, (_Float16*)staged, ncg, rows);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+extern "C" {
 int tga_moe_combine_rmsnorm_rows(const float* y, const float* probs, float* x, const float* weight, int rows, int k, int dim, float eps, void* out_f16, float* out_f32,
                                  void* stream) {
   TGA_REQUIRE(y && probs && x && weight && (out_f16 || out_f32), "tga_moe_combine_rmsnorm_rows: null pointer");
   TGA_REQUIRE(dim > 0 && rows >= 1 && k >= 1, "tga_moe_combine_rmsnorm_rows: rows=%d k=%d dim=%d", rows, k, dim);
-  rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k);
+  rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k, nullptr, 0, 0);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -888,6 +888,15 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
   return e;
 }
 
+// Halfword index of element e of activation row m in the layout the 17 .. 64 row GEMM (qgemm64.hip) multiplies from, for a consumer of format fmt with nu
+// units per row and ncg column groups: per step of four units [vector][column group][unit][column] 16-byte pieces (the formats' staged vectors, Fmt::stage).
+__device__ __forceinline__ size_t rows_staged_pos(int fmt, int e, int nu, int m, int ncg) {
+  int u, i, h;
+  if (fmt == GGML_F16) { u = e >> 6; i = (e >> 3) & 7; h = e & 7; }                      // (fp16 weights: the vectors are the unit's values in order)
+  else { const int full = staged_pos(fmt, e, nu); h = full & 7; const int t = full >> 3; i = t / nu; u = t - i * nu; }
+  return ((size_t)(u >> 2) * (8 * ncg * 64) + (i * ncg + (m >> 4)) * 64 + (u & 3) * 16 + (m & 15)) * 8 + h;
+}
+
 // ------------------------------------------------------------------------------------------------ activation staging (M rows, LDS)
 // LDS layout for units [u0, u0+cu): xs[(m*XV + t) * cu + (u-u0)] (u32x4), then cs[(m*NG + j) * cu + (u-u0)] (float)
 // one staging item = one unit of one activation row: stage_fetch reads its K values (as fp16 pairs), stage_put writes its vectors to LDS

@@ -34,6 +34,9 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 #define Q64_PART_BYTES ((size_t)8 << 20)
 #define Q64_SLOTS 4
 #define Q64_MAX_DEVICES 64
+#ifndef Q64_RING
+#define Q64_RING 3
+#endif
 
 struct Q64X {
   u32x4* xs;            // staged activations: [step][8 vectors][NCG column groups][4 units][16 columns] pieces
@@ -119,11 +122,12 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
     if (i < n) { put((i + 1) & 1, xb); __syncthreads(); }
     return;
   }
-  Raw wq[3][NT];
+  constexpr int RD = Q64_RING;                            // weight steps in flight, the one being multiplied included
+  Raw wq[RD][NT];
 #pragma unroll
-  for (int t = 0; t < NT; t++) wq[0][t] = F::load(rowp[t], 4 * s0 + g);
+  for (int k = 0; k < RD - 1; k++)
 #pragma unroll
-  for (int t = 0; t < NT; t++) wq[1][t] = F::load(rowp[t], 4 * (s0 + (n > 1 ? 1 : 0)) + g);
+    for (int t = 0; t < NT; t++) wq[k][t] = F::load(rowp[t], 4 * (s0 + (k < n ? k : n - 1)) + g);
   __syncthreads();
   v4f32 acc[NT][NCG];
 #pragma unroll
@@ -150,16 +154,19 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
     }
   };
   auto step = [&](const Raw (&cur)[NT], Raw (&nxt2)[NT], int i) __attribute__((always_inline)) {
-    const int i2 = i + 2 < n ? i + 2 : n - 1;
+    const int i2 = i + RD - 1 < n ? i + RD - 1 : n - 1;
 #pragma unroll
     for (int t = 0; t < NT; t++) nxt2[t] = F::load(rowp[t], 4 * (s0 + i2) + g);
     compute(cur, i & 1);
     __syncthreads();
   };
   int i = 0;
-  for (; i + 3 <= n; i += 3) { step(wq[0], wq[2], i); step(wq[1], wq[0], i + 1); step(wq[2], wq[1], i + 2); }
-  if (i < n) { step(wq[0], wq[2], i); i++; }
-  if (i < n) { step(wq[1], wq[0], i); i++; }
+  for (; i + RD <= n; i += RD) {
+#pragma unroll
+    for (int k = 0; k < RD; k++) step(wq[k], wq[(k + RD - 1) % RD], i + k);
+  }
+#pragma unroll
+  for (int k = 0; k < RD - 1; k++) if (i < n) { step(wq[k], wq[(k + RD - 1) % RD], i); i++; }
 
   // ---- epilogue: lane (g, c) holds, per tile and column group, activation row 16 cg + c x weight rows 4 g .. 4 g + 3 of the tile
   const int c = r;
@@ -289,7 +296,7 @@ static int q64_split(bool sw, long long tiles, int nsteps) {   // workgroups per
 }
 
 template <int T, bool MS, bool SW, int NCG, int NT>
-static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
+static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
   using F = Fmt<T>;
   auto kern = qgemm64_kernel<T, MS, SW, NCG, NT>;
   constexpr size_t stage_bytes = (size_t)F::XV * NCG * 64 * 16;
@@ -303,8 +310,10 @@ static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
   int ks = q64_split(SW, tiles, nsteps);
   while (ks > 1 && (size_t)ks * 64 * ex.np * 4 > Q64_PART_BYTES) ks--;
   ex.ks = ks;
-  q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
-  TGA_LAUNCH_CHECK();
+  if (!prestaged) {
+    q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
+    TGA_LAUNCH_CHECK();
+  }
   kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(512), 2 * stage_bytes, s>>>(a, M, ex);
   TGA_LAUNCH_CHECK();
   if (ks > 1) {
@@ -316,7 +325,7 @@ static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
 }
 
 template <int T, bool MS, bool SW, int NCG>
-static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
+static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
   using F = Fmt<T>;
   // Two weight tiles per wave halve the activation bytes that reach a CU (global -> LDS -> operand) per weight; taken when the row tiles of 128, split over K,
   // still fill the chip.  (fp16 weights: a unit is 128 bytes per lane, a ring of three steps for two tiles does not fit the registers.)
@@ -325,42 +334,55 @@ static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, hipStream_t s) {
   const long long rows_wg2 = SW ? 64 : 128, tiles2 = (a.ntot + rows_wg2 - 1) / rows_wg2;
   bool two = sizeof(typename F::Raw) <= 64 && tiles2 * q64_split(SW, tiles2, nsteps) >= 224;
   if (env_nt == 1) two = false; else if (env_nt == 2) two = sizeof(typename F::Raw) <= 64;
-  if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, s); }
-  return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, s);
+  if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, prestaged, s); }
+  return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, prestaged, s);
 }
 
 template <int T>
-static int launch_q64(QArgs a, int M, uint8_t* ws, hipStream_t s) {
+static int launch_q64(QArgs a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
   using F = Fmt<T>;
   if constexpr (F::UW != 64 || F::XV != 8) return -1;
   else {
     a.nu = a.K / F::UW;
     a.row_bytes = (long long)(a.K / F::BW) * F::BB;
     const bool two = M <= 32;                             // two column groups instead of four: half the MFMAs and half the staged bytes
-    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, s) : launch_q64_t<T, false, true, 4>(a, M, ws, s);
-    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, s) : launch_q64_t<T, true, false, 4>(a, M, ws, s);
-    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, s) : launch_q64_t<T, false, false, 4>(a, M, ws, s);
+    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, true, 4>(a, M, ws, prestaged, s);
+    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, true, false, 4>(a, M, ws, prestaged, s);
+    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, false, 4>(a, M, ws, prestaged, s);
   }
 }
 
-// Returns -1 when the call is outside this kernel's range (the caller then runs blocks of sixteen rows): 17 .. 64 rows of fp16 or float32 activations, K a
-// multiple of 256 up to Q64_MAX_K, one to three matrices (several: each a multiple of 16 rows) with the plain or residual epilogue, or the SwiGLU pair; and
-// when no workspace slot is left for the stream.
-int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
-  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y) return -1;
-  if (a.nseg > 1 && a.epilogue != 2) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return -1;
-  if (((uintptr_t)a.x & 15) != 0) return -1;
-  switch (fmt) { case F_Q4_0P: case F_Q8_0P: case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_F16: break; default: return -1; }
+// Whether the call is inside this kernel's range: 17 .. 64 rows of fp16 or float32 activations, K a multiple of 256 up to Q64_MAX_K, one to three matrices
+// (several: each a multiple of 16 rows) with the plain or residual epilogue, or the SwiGLU pair, in one of the formats with units of 64 weights.
+static bool q64_in_range(int fmt, const QArgs& a, int M) {
+  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y) return false;
+  if (a.nseg > 1 && a.epilogue != 2) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return false;
+  if (((uintptr_t)a.x & 15) != 0) return false;
+  switch (fmt) { case F_Q4_0P: case F_Q8_0P: case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_F16: return true; }
+  return false;
+}
+
+// For a producer that writes the activations in the multiplying layout itself (rows_staged_pos in qfmt.h, ncg column groups): where to, or nullptr when the call
+// is outside the kernel's range or the stream holds no workspace slot.  The call that follows passes prestaged = true.
+void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* ncg) {
+  if (!q64_in_range(fmt, a, M)) return nullptr;
+  *ncg = M <= 32 ? 2 : 4;
+  return q64_slot(s);
+}
+
+// Returns -1 when the call is outside this kernel's range or no workspace slot is left for the stream (the caller then runs blocks of sixteen rows).
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, bool prestaged, hipStream_t s) {
+  if (!q64_in_range(fmt, a, M)) return -1;
   uint8_t* ws = q64_slot(s);
   if (!ws) return -1;
   switch (fmt) {
-    case F_Q4_0P: return launch_q64<F_Q4_0P>(a, M, ws, s);
-    case F_Q8_0P: return launch_q64<F_Q8_0P>(a, M, ws, s);
-    case GGML_Q6_K: return launch_q64<GGML_Q6_K>(a, M, ws, s);
-    case GGML_Q4_K: return launch_q64<GGML_Q4_K>(a, M, ws, s);
-    case GGML_Q5_K: return launch_q64<GGML_Q5_K>(a, M, ws, s);
-    case GGML_IQ4_XS: return launch_q64<GGML_IQ4_XS>(a, M, ws, s);
-    case GGML_F16: return launch_q64<GGML_F16>(a, M, ws, s);
+    case F_Q4_0P: return launch_q64<F_Q4_0P>(a, M, ws, prestaged, s);
+    case F_Q8_0P: return launch_q64<F_Q8_0P>(a, M, ws, prestaged, s);
+    case GGML_Q6_K: return launch_q64<GGML_Q6_K>(a, M, ws, prestaged, s);
+    case GGML_Q4_K: return launch_q64<GGML_Q4_K>(a, M, ws, prestaged, s);
+    case GGML_Q5_K: return launch_q64<GGML_Q5_K>(a, M, ws, prestaged, s);
+    case GGML_IQ4_XS: return launch_q64<GGML_IQ4_XS>(a, M, ws, prestaged, s);
+    case GGML_F16: return launch_q64<GGML_F16>(a, M, ws, prestaged, s);
   }
   return -1;
 }

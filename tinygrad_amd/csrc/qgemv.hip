@@ -318,7 +318,9 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    // qgemm_dma.hip
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
-int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);       // qgemm64.hip
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, bool prestaged, hipStream_t s);       // qgemm64.hip
+void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* ncg);              // qgemm64.hip
+int tga_rmsnorm_rows_staged64(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, int fmt, int nu, void* staged, int ncg, void* stream);   // decode.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -359,6 +361,20 @@ struct AttnIn { int n_splits, head_dim; const int* touch_pos; const void* k; con
 static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
+// the arguments of the 17 .. 64 row GEMM (qgemm64.hip) for a call whose pointers and epilogue have been checked; false: a format or alignment it does not take
+static bool q64_args(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n, const void* x, int x_dtype, int y_dtype, int64_t K,
+                     int epilogue, const void* const* resid, QArgs& q, int& fmt64) {
+  bool pair64 = K > 0 && (K / 32) % 2 == 0;
+  for (int i = 0; i < nseg; i++) pair64 = pair64 && ((uintptr_t)w[i] & 3) == 0;
+  fmt64 = ggml_type == GGML_Q4_0 ? (pair64 ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair64 ? F_Q8_0P : -1) : ggml_type;
+  if (fmt64 < 0 || !pair64) return false;
+  q = QArgs{};
+  q.nseg = nseg; q.x = x; q.x_f32 = x_dtype == TGA_F32; q.y_f32 = y_dtype == TGA_F32; q.epilogue = epilogue; q.K = (int)K;
+  long long nt = 0;
+  for (int i = 0; i < nseg; i++) { q.w[i] = (const uint8_t*)w[i]; q.y[i] = y[i]; q.n[i] = n[i]; q.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr; nt += n[i]; }
+  q.ntot = epilogue == 2 ? n[0] : nt;
+  return true;
+}
 // M rows as calls of at most `block` rows ((M, n) outputs and (M, K) activations: row blocks are contiguous)
 static int qlinear_row_blocks(int block, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n, const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, void* stream) {
@@ -389,16 +405,9 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     TGA_REQUIRE(epilogue != 1 || y_dtype == TGA_F32, "tga_qlinear: the residual epilogue needs float32 y");
     TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
     {                                                             // one pass over the weights for all rows where the 64-column kernel applies (qgemm64.hip)
-      bool pair64 = K > 0 && (K / 32) % 2 == 0;
-      for (int i = 0; i < nseg; i++) pair64 = pair64 && ((uintptr_t)w[i] & 3) == 0;
-      const int fmt64 = ggml_type == GGML_Q4_0 ? (pair64 ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair64 ? F_Q8_0P : -1) : ggml_type;
-      if (fmt64 >= 0 && pair64) {
-        QArgs q = {};
-        q.nseg = nseg; q.x = x; q.x_f32 = x_dtype == TGA_F32; q.y_f32 = y_dtype == TGA_F32; q.epilogue = epilogue; q.K = (int)K;
-        long long nt = 0;
-        for (int i = 0; i < nseg; i++) { q.w[i] = (const uint8_t*)w[i]; q.y[i] = y[i]; q.n[i] = n[i]; q.resid[i] = epilogue == 1 ? (const float*)resid[i] : nullptr; nt += n[i]; }
-        q.ntot = epilogue == 2 ? n[0] : nt;
-        const int rc = tga_qgemm64_dispatch(fmt64, q, M, (hipStream_t)stream);
+      QArgs q; int fmt64;
+      if (q64_args(ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, K, epilogue, resid, q, fmt64)) {
+        const int rc = tga_qgemm64_dispatch(fmt64, q, M, false, (hipStream_t)stream);
         if (rc >= 0) return rc;
       }
     }
@@ -596,6 +605,21 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
   if (M >= 2 && M <= 8 && ((uintptr_t)norm_weight & 15) == 0) {
     const int rc = qlinear_multi_impl(nullptr, nullptr, norm_weight, norm_eps, ggml_type, nseg, w, y, n, x, TGA_F32, y_dtype, M, K, epilogue, resid, 0, 0, stream);
     if (rc != -2) return rc;
+  }
+  if (M > 16 && nseg >= 1 && nseg <= QG_MAX_SEG && w && y && n && (y_dtype == TGA_F16 || y_dtype == TGA_F32) && epilogue >= 0 && epilogue <= 2 && (epilogue != 1 || (resid && y_dtype == TGA_F32)) &&
+      (epilogue != 2 || (nseg == 2 && n[0] == n[1]))) {
+    // 17 .. 64 rows on the 64-column kernel: the norm's launch writes the rows in the layout that kernel multiplies from as well (no staging launch)
+    bool ok = true;
+    for (int i = 0; i < nseg; i++) ok = ok && n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]);
+    QArgs q; int fmt64, ncg = 0;
+    if (ok && q64_args(ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, K, epilogue, resid, q, fmt64)) {
+      void* staged = tga_qgemm64_staging(fmt64, q, M, (hipStream_t)stream, &ncg);
+      if (staged) {
+        if (const int rc = tga_rmsnorm_rows_staged64(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, fmt64, (int)(K / 64), staged, ncg, stream)) return rc;
+        const int rc = tga_qgemm64_dispatch(fmt64, q, M, true, (hipStream_t)stream);
+        if (rc >= 0) return rc;                                   // (cannot be refused here: the same checks have passed above)
+      }
+    }
   }
   const int rc = tga_rmsnorm_rows(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, nullptr, 0, stream);
   if (rc) return rc;
