@@ -5,7 +5,7 @@ A step is one decoded token.  Random-init weights are written on the GPU as GGUF
 lm-head), the fp16 KV cache is prefilled with 1024 random token ids through the model itself, then --warmup + --steps tokens
 are decoded greedily, one captured launch sequence per token with a host sync per token (as the reference's generate loop does).
 Prints ONE JSON line: tok/s, the roofline of the dominant kernel from HIP-event timings taken live (the fused ffn_norm + ffn_gate + ffn_up +
-SwiGLU dequant-GEMV, one of six launches per block), the same figures for the other kernels of a block, a parity gate (outside the timed
+SwiGLU dequant-GEMV, one of five launches per block), the same figures for the other kernels of a block, a parity gate (outside the timed
 region: one more decoded token of the SAME model recomputed on the CPU from the GPU's own KV cache, and every linear of layer 0 on a fresh
 row; the run exits non-zero when a bar is missed), a CPU baseline (C restatement of the reference arithmetic on a bounded sample of the
 same weights) and the kernel-level figures of the other benchmark configurations measured in the same process."""
@@ -15,10 +15,10 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE) of
 # `python -m tinygrad_amd.benchmarks --traffic`, each scaled by what the same counter reads for a 1 GiB copy kernel (x2.0000 and x1.0000):
-# 66 514 125 B fetched + 71 680 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
-GATE_UP_TRAFFIC_BYTES = 66585805
-GATE_UP_ROCPROF_AVG_US = 15.45    # rocprofv3 --kernel-trace --stats average of the same kernel over every call of an eagerly launched run (profiles/decode_llama3_8b_q4_0_kernel_stats.md)
-GATE_UP_ROCPROF_B2B_US = 14.46    # the same trace, only the passes that issue the 32 launches back to back (the region the HIP events below bracket)
+# 66 509 824 B fetched + 71 680 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
+GATE_UP_TRAFFIC_BYTES = 66581504
+GATE_UP_ROCPROF_AVG_US = 14.86    # rocprofv3 --kernel-trace --stats average of the same kernel over every call of an eagerly launched run (profiles/decode_llama3_8b_q4_0_kernel_stats.md)
+GATE_UP_ROCPROF_B2B_US = 14.48    # the same trace, only the passes that issue the 32 launches back to back (the region the HIP events below bracket)
 PARITY_TOL = 1e-3
 
 def _host_layer(model, i):
@@ -244,18 +244,26 @@ def main():
     from oracle import cref
     parity = parity_gate(model, c, min(threads_all, cref.max_threads()))
 
-  # ---- the per-op kernels on the same weights, timed with HIP events on the model's stream (the launches of TransformerBlock.__call__:
-  #      q/k/v with attn_norm folded in, attention, attn_output + residual, gate/up with ffn_norm folded in + SwiGLU, down + residual) ----
+  # ---- the per-op kernels on the same weights, timed with HIP events on the model's stream (the five launches of TransformerBlock.__call__:
+  #      q/k/v with attn_norm folded in (it also touches the cache rows the attention will read), the attention as one launch that leaves split
+  #      partials, attn_output + residual merging those partials while it stages its row, gate/up with ffn_norm folded in + SwiGLU, down + residual) ----
   st = model.stream.handle
   L = rt.lib()
   from tinygrad_amd.nn import qlinear_multi
   durs = {"gate_up": [], "down": [], "qkv": [], "attn_output": [], "attention": []}
   s = model.s
+  b_first = model.blk[0]
+  fused = bool(b_first.fused_attn)                             # the attention as one launch whose partials attn_output merges (TransformerBlock.__call__)
+  touch = lambda b: (s.state, b.cache_k, b.cache_v, s.rope, c.n_kv_heads, c.head_dim, c.max_context) if b.kv_touch else None
   ops = {
-    "qkv": lambda b: qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.x, [s.q, s.k, s.v], stream=st, norm=(b.attn_norm, c.norm_eps)),
-    "attention": lambda b: rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
-                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if b.stage_attn else 0, st)),
-    "attn_output": lambda b: qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.stage_attn),
+    "qkv": lambda b: qlinear_multi([b.attn_q, b.attn_k, b.attn_v], s.x, [s.q, s.k, s.v], stream=st, norm=(b.attn_norm, c.norm_eps), touch=touch(b)),
+    "attention": (lambda b: rt.check(L.tga_attention_decode_split(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads,
+                                     c.head_dim, c.max_context, s.rope.ptr, st))) if fused else
+                 (lambda b: rt.check(L.tga_attention_decode(s.q.ptr, s.k.ptr, s.v.ptr, b.cache_k.ptr, b.cache_v.ptr, s.attn_part.ptr, s.state.ptr,
+                                     c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, s.rope.ptr, s.attn.ptr, None, b.attn_output.ggml_type if b.stage_attn else 0, st))),
+    "attn_output": (lambda b: rt.check(L.tga_attn_merge_qlinear(b.attn_output.ggml_type, b.attn_output.blocks.ptr, s.x.ptr, b.attn_output.out_features, b.attn_output.in_features,
+                                       s.x.ptr, s.attn_part.ptr, b.fused_attn, c.head_dim, st))) if fused else
+                   (lambda b: qlinear_multi([b.attn_output], s.attn, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.stage_attn)),
     "gate_up": lambda b: qlinear_multi([b.ffn_gate, b.ffn_up], s.x, [s.act], epilogue=2, stream=st, norm=(b.ffn_norm, c.norm_eps), stage_out_for=b.ffn_down if b.stage_act else None),
     "down": lambda b: qlinear_multi([b.ffn_down], s.act, [s.x], epilogue=1, resid=[s.x], stream=st, x_staged=b.stage_act),
   }
@@ -304,7 +312,7 @@ def main():
   dom = kern["gate_up"]
   per_block = sum(v["avg_us"] for v in kern.values())
   out["roofline"] = {"bound": "hbm", "kernel": "qgemv1_kernel<Q4_0 pair, R=2, WK=1, WR=8, SwiGLU, norm prologue> (ffn_norm + ffn_gate + ffn_up + silu*mul in one launch, 2 x 14336 x 4096; "
-                                               "one of six launches per block)",
+                                               "one of five launches per block)",
                      "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
                      "traffic": GATE_UP_TRAFFIC_BYTES if c.num_blocks == 32 else None,
                      "traffic_source": "recorded rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run",

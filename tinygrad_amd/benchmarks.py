@@ -286,16 +286,38 @@ def traffic(steps: int = 4):
   model.check_state()
   return [{"traffic_probe": "done", "copy_bytes": n, "decode_steps": steps}]
 
+def prefill_trace(chunk: int = 64):
+  """Workload for the kernel trace of a chunked prefill (rocprofv3 --kernel-trace --stats -- python3 -m tinygrad_amd.benchmarks --prefill 64): the 8B architecture
+  of configuration 3 (Q4_0, Q6_K lm-head), 1023 positions in steps of `chunk`, launched eagerly twice (the first pass also sizes the step models); the
+  wall time of the second pass is reported (eager launches: the replayed steps of configuration 8 are faster)."""
+  from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state, LLAMA3_8B
+  import time
+  c = TransformerConfig(max_context=1152, **LLAMA3_8B)
+  model = Transformer(c, synth_state(c, seed=1003), max_new=4)
+  model.prefill_chunk = chunk
+  rng = np.random.default_rng(1003)
+  prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=1024)]
+  model.prefill(prompt, False, reuse_cache=False)
+  rt.synchronize()
+  t0 = time.perf_counter()
+  model.prefill(prompt, False, reuse_cache=False)
+  rt.synchronize()
+  return [{"prefill_trace": "done", "positions": 1023, "per_step": chunk, "eager_ms": round((time.perf_counter() - t0) * 1e3, 1)}]
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix; 8 = 8B chunked prefill and batched dense decode")
   ap.add_argument("--no-graph", action="store_true", help="configs 4 and 7: launch eagerly instead of replaying a captured graph (for profilers)")
   ap.add_argument("--traffic", action="store_true", help="only the workload of the HBM-traffic counter runs (see traffic())")
+  ap.add_argument("--prefill", type=int, default=0, metavar="CHUNK", help="only the workload of the prefill kernel trace, CHUNK positions per step (see prefill_trace())")
   args = ap.parse_args()
   rt.init(0)
   print(json.dumps({"device": rt.device_name()}), flush=True)
   if args.traffic:
     for row in traffic(): print(json.dumps(row), flush=True)
+    return
+  if args.prefill:
+    for row in prefill_trace(args.prefill): print(json.dumps(row), flush=True)
     return
   for cfg in args.config:
     fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7, 8: config8}[cfg]

@@ -345,7 +345,9 @@ static int launch_q64(QArgs a, int M, uint8_t* ws, bool prestaged, hipStream_t s
   else {
     a.nu = a.K / F::UW;
     a.row_bytes = (long long)(a.K / F::BW) * F::BB;
-    const bool two = M <= 32;                             // two column groups instead of four: half the MFMAs and half the staged bytes
+    // two column groups instead of four: half the MFMAs and half the staged bytes.  (One group, for up to sixteen rows, was measured and dropped: the kernel
+    // streams weights at about 2.5 TB/s - Q8_0 14336 x 4096 at M = 8 24.6 us, the Q6_K lm-head 211 us - where the LDS-fed small-batch kernels take 18.4 / 134.)
+    const bool two = M <= 32;
     if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, true, 4>(a, M, ws, prestaged, s);
     if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, true, false, 4>(a, M, ws, prestaged, s);
     return two ? launch_q64_t<T, false, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, false, 4>(a, M, ws, prestaged, s);

@@ -397,19 +397,19 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
   TGA_REQUIRE(M >= 1 && M <= 64, "tga_qlinear: M=%d out of range 1..64", M);
-  if (M > 16) {                                                   // prefill chunks of up to 64 positions: blocks of sixteen rows (every block after the first finds the weights in the Infinity Cache)
-    TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG && !comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32) && !y_stage_type && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
+  // 17 .. 64 rows (prefill steps): one pass over the weights on the 64-column kernel where it applies (qgemm64.hip), else blocks of sixteen rows (every block
+  // after the first finds the weights in the Infinity Cache)
+  if (M > 16) {
+    TGA_REQUIRE(!comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32) && !y_stage_type && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
                 "tga_qlinear: more than 16 rows only for plain fp16 / float32 activations");
-    for (int i = 0; i < nseg; i++) TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]), "tga_qlinear: segment %d has a null pointer or no rows", i);
     TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
     TGA_REQUIRE(epilogue != 1 || y_dtype == TGA_F32, "tga_qlinear: the residual epilogue needs float32 y");
     TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
-    {                                                             // one pass over the weights for all rows where the 64-column kernel applies (qgemm64.hip)
-      QArgs q; int fmt64;
-      if (q64_args(ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, K, epilogue, resid, q, fmt64)) {
-        const int rc = tga_qgemm64_dispatch(fmt64, q, M, false, (hipStream_t)stream);
-        if (rc >= 0) return rc;
-      }
+    for (int i = 0; i < nseg; i++) TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]), "tga_qlinear: segment %d has a null pointer or no rows", i);
+    QArgs q; int fmt64;
+    if (q64_args(ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, K, epilogue, resid, q, fmt64)) {
+      const int rc = tga_qgemm64_dispatch(fmt64, q, M, false, (hipStream_t)stream);
+      if (rc >= 0) return rc;
     }
     return qlinear_row_blocks(16, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
   }
