@@ -37,7 +37,7 @@ extern "C" {
 
 /* ---- runtime: replaces HIPDevice / HIPAllocator / HIPProgram timing in tinygrad/runtime/ops_hip.py:12-70 ---- */
 const char* tga_last_error(void);
-int tga_init(int device);                                  /* hipSetDevice + kernel attribute set-up; ops_hip.py:14-20 */
+int tga_init(int device);                                  /* hipSetDevice + kernel attribute set-up; ops_hip.py:14-20.  Also allocates, once per device, the 48 MB workspace of the 17 .. 64 row linears */
 int tga_device_name(char* buf, size_t len);
 int tga_malloc(void** ptr, size_t nbytes);                 /* ops_hip.py:60-62 */
 int tga_free(void* ptr);                                   /* ops_hip.py:63 */
@@ -49,7 +49,7 @@ int tga_copy_kernel(void* dst, const void* src, size_t n, void* stream);
 int tga_memset(void* dst, int value, size_t n, void* stream);   /* hipMemsetAsync; refused (error) on a stream that is capturing */
 int tga_sync(void);                                        /* ops_hip.py:22-24 hipDeviceSynchronize */
 int tga_stream_create(void** stream);
-int tga_stream_destroy(void* stream);
+int tga_stream_destroy(void* stream);                      /* waits for the stream's work, gives its slot of that workspace back, destroys it */
 int tga_stream_sync(void* stream);
 int tga_event_create(void** ev);                           /* ops_hip.py:49-57 wait=True timing */
 int tga_event_destroy(void* ev);
@@ -80,7 +80,7 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
  * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8 (the decode range); 9 <= M <= 16 is taken too, for prefill chunks: one launch where the
- * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows; 17 <= M <= 64 (plain fp16 / float32 activations) runs as blocks of sixteen rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
+ * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows; 17 <= M <= 64 (plain fp16 / float32 activations; a prefill step) is one pass over the weights on a 64-column matrix-core tile where it applies (Q4_0 / Q8_0 pairs, Q4_K, Q5_K, Q6_K, IQ4_XS, fp16; K a multiple of 256 up to 32768; several matrices: each a multiple of 16 rows; staged rows and split-K partial sums in the per-device workspace of tga_init, one slot per stream), otherwise blocks of sixteen rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
  * (Q4_1 / Q5_0 / Q5_1 are served as block pairs: K % 64 == 0).
  * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K/Q4_1/Q5_0/Q5_1 (GGUF aligns tensor data to 32 bytes,
  * gguf.py:144-148). */
@@ -212,6 +212,18 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
+/* tga_attention_decode as ONE launch whose consumer merges (model.py:167-198 up to the softmax-weighted V sums; no q / k norm).  A workgroup serves one query
+ * head and one split of the cache; tga_attention_split_plan reports the number of splits for max_ctx: at most six, 0 when the cache is too long for this path
+ * (max_ctx beyond 3072).  partials: n_heads * (n_splits * head_dim + 16) floats, per head [n_splits][head_dim] weighted V sums followed by the splits'
+ * (max, sum) pairs; 16-byte aligned.  A split that starts beyond state.pos leaves an empty partial (max -inf, sum 0).  The merge is tga_attn_merge_qlinear's. */
+int tga_attention_split_plan(int max_ctx, int* n_splits);
+int tga_attention_decode_split(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                               int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream);
+/* attn_output + residual (model.py:198, 149) over the attention row that tga_attention_decode_split left as partials: y = resid + merge(partials) W^T, float32,
+ * y may be resid.  The merge per head - sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m), rounded to fp16 - happens while the launch stages its
+ * activation row.  K = n_heads * head_dim, 2048 < K <= 4096 (rows of 33..64 units); block types with a single-row kernel except MXFP4; n_splits 1..6. */
+int tga_attn_merge_qlinear(int ggml_type, const void* w, float* y, int64_t N, int64_t K, const float* resid, const float* partials, int n_splits, int head_dim, void* stream);
+
 /* tga_rmsnorm_qlinear_multi (single row) for the q / k / v launch of a decode step, with a hint for the attention launch behind it (no counterpart in the
  * reference): every lane also reads one dword of one 128-byte line of the cached K / V rows below state.pos and of the rotation row of that position, each on
  * the XCD whose attention workgroups will read it, so that the attention finds them in L2.  Same results as tga_rmsnorm_qlinear_multi; caches
@@ -248,7 +260,7 @@ int tga_attention_decode_batched(int batch, const float* q, const float* k, cons
 /* Attention for `rows` consecutive positions state.pos .. state.pos + rows - 1 of ONE sequence (the chunked prefill of Transformer.generate,
  * tinygrad/llm/model.py:464, 476-481; causal mask `_attention`, model.py:227-229): q (rows, n_heads * head_dim), k / v (rows, n_kv_heads * head_dim),
  * one cache (n_kv_heads, max_ctx, head_dim) fp16.  A first launch rotates and appends every row's key / value, a second attends from the cache (row r sees the
- * positions up to its own), a third merges the splits.  partials: rows times the single-sequence workspace.  Outputs (rows, n_heads * head_dim). */
+ * positions up to its own; more than eight rows of head_dim 64 / 128 without q / k norm: on the matrix cores, queries and probabilities rounded to fp16), a third merges the splits.  partials: rows times the single-sequence workspace.  Outputs (rows, n_heads * head_dim). */
 int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);

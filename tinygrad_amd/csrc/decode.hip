@@ -544,8 +544,8 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
   }
 }
 
-// The attention of one token as ONE launch whose consumer merges (tga_attn_merge_qlinear): workgroup = (query head, split of SP = 128 IT positions), eight waves
-// of 16 rows per tile, IT tiles per wave, every cached row of the split requested up front (rows clamped to the cache, not to the position), at most four splits.
+// The attention of one token as ONE launch whose consumer merges (tga_attn_merge_qlinear): workgroup = (query head, split of SP = 16 NW IT positions), NW waves
+// of 16 rows per tile, IT tiles per wave, every cached row of the split requested up front (rows clamped to the cache, not to the position), at most six splits.
 // The flattened workgroup index is kv head + n_kv (head in group + group * split): with n_kv a multiple of 8 all readers of a kv head's rows run on one XCD.
 // A split that starts beyond the position writes an empty partial (max -inf, sum 0).  Partials per head: [n_splits][head_dim] weighted V sums, then the
 // (max, sum) pairs of the splits in 16 floats.
