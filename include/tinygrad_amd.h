@@ -260,7 +260,7 @@ int tga_attention_decode_batched(int batch, const float* q, const float* k, cons
 /* Attention for `rows` consecutive positions state.pos .. state.pos + rows - 1 of ONE sequence (the chunked prefill of Transformer.generate,
  * tinygrad/llm/model.py:464, 476-481; causal mask `_attention`, model.py:227-229): q (rows, n_heads * head_dim), k / v (rows, n_kv_heads * head_dim),
  * one cache (n_kv_heads, max_ctx, head_dim) fp16.  A first launch rotates and appends every row's key / value, a second attends from the cache (row r sees the
- * positions up to its own; more than eight rows of head_dim 64 / 128 without q / k norm: on the matrix cores, queries and probabilities rounded to fp16), a third merges the splits.  partials: rows times the single-sequence workspace.  Outputs (rows, n_heads * head_dim). */
+ * positions up to its own; more than eight rows of head_dim 64 / 128 without q / k norm: on the matrix cores, probabilities rounded to fp16), a third merges the splits.  partials: rows times the single-sequence workspace.  Outputs (rows, n_heads * head_dim). */
 int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);

@@ -171,6 +171,50 @@ def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
     np.testing.assert_array_equal(tokb.numpy(), prompt[np.minimum(pos0 + B + np.arange(B), ctx - 1)])
   assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
 
+@pytest.mark.parametrize("H,KV,hd,B", [(8, 2, 128, 16), (8, 2, 128, 37), (4, 4, 64, 64), (16, 2, 64, 24), (8, 8, 128, 17), (8, 1, 128, 9)])
+def test_attention_prefill_chunk_on_the_matrix_cores_vs_numpy(gpu, H, KV, hd, B):
+  """tga_attention_prefill_chunk for more than eight rows without q / k norm (the launch that attends multiplies on the matrix cores: workgroup per kv head, 64-position
+  split and tile of sixteen rows, wave per query head of the group): steps of B consecutive positions over one cache up to position 150 and beyond two split
+  boundaries, groups of 1, 4 and 8 query heads per kv head (8: two passes of the four waves), row counts that end inside a tile; every row against numpy attention over the
+  positions up to its own.  The rotated queries and the probabilities are rounded to fp16 there: the bar is the linears' 1e-3."""
+  from tinygrad_amd.llm import precompute_freqs_cis
+  ctx = 256
+  rng = np.random.default_rng(1000 * H + 10 * KV + B)
+  rope = precompute_freqs_cis(hd, ctx, 10000.0)
+  ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
+  part = gpu.Buffer((B * H * ((ctx + 63) // 64) * (hd + 2),), np.float32).zero_()
+  ropeb = gpu.Buffer.from_numpy(rope)
+  out = gpu.Buffer((B, H * hd), np.float32)
+  out16 = gpu.Buffer((B, H * hd), np.float16)
+  prompt = np.arange(ctx, dtype=np.int32)
+  pb, tokb = gpu.Buffer.from_numpy(prompt), gpu.Buffer((B,), np.int32).zero_()
+  stb = gpu.Buffer.from_numpy(np.zeros(16, np.int32))
+  rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)
+  worst, pos0 = 0.0, 0
+  while pos0 + B <= 150 + B and pos0 + B < ctx:
+    q, k, v = (rng.standard_normal((B, n)).astype(np.float32) * 1.5 for n in (H * hd, KV * hd, KV * hd))
+    qb, kb, vb = (gpu.Buffer.from_numpy(t) for t in (q, k, v))
+    gpu.check(gpu.lib().tga_attention_prefill_chunk(B, qb.ptr, kb.ptr, vb.ptr, None, None, 0.0, 0, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr,
+                                                    out16.ptr, out.ptr, None))
+    gpu.check(gpu.lib().tga_chunk_advance(stb.ptr, pb.ptr, B, tokb.ptr, ctx, None))
+    gpu.synchronize()
+    o = out.numpy()
+    np.testing.assert_array_equal(out16.numpy(), o.astype(np.float16))
+    for r in range(B):
+      pos = pos0 + r
+      qr, kr = ollm.apply_rope(q[r].reshape(H, hd), rope[pos]), ollm.apply_rope(k[r].reshape(KV, hd), rope[pos])
+      rk[:, pos], rv[:, pos] = kr.astype(np.float16), v[r].reshape(KV, hd).astype(np.float16)
+      K = np.repeat(rk[:, :pos + 1].astype(np.float32), H // KV, axis=0); V = np.repeat(rv[:, :pos + 1].astype(np.float32), H // KV, axis=0)
+      sc = np.einsum("hd,htd->ht", qr, K) / np.sqrt(hd)
+      e = np.exp(sc - sc.max(-1, keepdims=True)); p = e / e.sum(-1, keepdims=True)
+      worst = max(worst, ol.rel_err(o[r], np.einsum("ht,htd->hd", p, V).reshape(-1)))
+    pos0 += B
+    assert int(stb.numpy()[0]) == pos0
+  print(f"H {H} KV {KV} hd {hd} B {B}: worst rel-err {worst:.2e}")
+  assert worst <= 1e-3, worst
+  assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
+  assert not ck.numpy()[:, pos0:].any() and not cv.numpy()[:, pos0:].any()
+
 def test_command_list_takes_kernel_launches_only(gpu):
   """A capture that holds anything but kernel launches (here a device-to-device copy, which the capture records as a copy node; the graph is never
   instantiated) is refused when the list is built; the stream stays usable."""

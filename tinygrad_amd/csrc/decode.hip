@@ -55,16 +55,9 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
 template <bool COMB>
 __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* x, const float* __restrict__ w, int dim, float eps,
                                                        _Float16* __restrict__ out16, float* __restrict__ out32, int stage_fmt, int stage_nu,
-                                                       float* x_rw, const float* __restrict__ y, const float* __restrict__ probs, int k,
-                                                       _Float16* __restrict__ rows_staged, int rs_ncg, int rows_real) {
+                                                       float* x_rw, const float* __restrict__ y, const float* __restrict__ probs, int k) {
   __shared__ float red[16];
   const int row = blockIdx.x;                           // one workgroup per row
-  // rows_staged != nullptr: the normalised rows also go, in the order of rows_staged_pos(stage_fmt, ., stage_nu, row, rs_ncg), to the buffer that the
-  // 17 .. 64 row GEMM multiplies from (out16 then keeps the plain order); workgroups at and beyond rows_real only fill their rows of it with zeros
-  if (rows_staged && row >= rows_real) {
-    for (int e = threadIdx.x; e < dim; e += blockDim.x) rows_staged[rows_staged_pos(stage_fmt, e, stage_nu, row, rs_ncg)] = (_Float16)0.f;
-    return;
-  }
   x += (size_t)row * dim;
   if (out16) out16 += (size_t)row * dim;
   if (out32) out32 += (size_t)row * dim;
@@ -106,8 +99,7 @@ __global__ __launch_bounds__(1024) void rmsnorm_kernel(const float* x, const flo
   for (int i = 0; i < nw; i++) tot += red[i];
   const float scale = 1.0f / sqrtf(tot / (float)dim + eps);
   auto emit = [&](int e, float v) {
-    if (out16) out16[stage_fmt && !rows_staged ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
-    if (rows_staged) rows_staged[rows_staged_pos(stage_fmt, e, stage_nu, row, rs_ncg)] = (_Float16)v;
+    if (out16) out16[stage_fmt ? staged_pos(stage_fmt, e, stage_nu) : e] = (_Float16)v;
     if (out32) out32[e] = v;
   };
   if (e0 < dim) emit(e0, (v0 * scale) * w0);
@@ -422,13 +414,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 // attn_decode_kernel read every 32 KB K / V tile once per row and query-head group - 64 rows x 8 kv heads x 16 splits = 268 MB of L2 reads per layer at a
 // context of 1024 - here a tile is read once per sixteen rows.  Wave w serves query head w of the group (w + 4, ... for larger groups):
 //   S^T = K Q^T   v_mfma_f32_16x16x32_f16, A = lane (g, r): 8 values 32 j + 8 g .. of cached key 16 t + r (16-byte loads straight from the cache), B = lane (g, c):
-//                 the same 8 values of chunk row c's rotated query, rounded to fp16, in registers for the whole launch; D = lane (g, c): keys 16 t + 4 g + i of row c
+//                 the same 8 values of chunk row c's rotated query as TWO fp16 operands (the rounded value and what the rounding left over, so the scores see the
+//                 float32 query: rounding it alone put the result at 1.0e-3 of the float32 attention on random rows); D = lane (g, c): keys 16 t + 4 g + i of row c
 //   softmax partial of the split per chunk row: the 16 scores of a lane, then the four lanes of a row (m, l: float32; a row sees the positions up to its own)
 //   O^T = V^T P^T A = lane (g, r): V of 8 keys for dimension 16 h + r, B = lane (g, c): exp(s - m) of the SAME 8 keys for row c, rounded to fp16 - the eight
 //                 keys a lane holds after the first product (tiles 2 u and 2 u + 1, rows 4 g + i) are taken as they are, and the V tile is written to LDS
 //                 transposed with its keys in that order, so that the A operand is one 16-byte LDS read
 // The partial (float32 weighted V sums, max, sum) goes where attn_decode_kernel writes it; attn_merge_kernel finishes.  Deviation from the float32 products of
-// the per-row kernel: the rotated query and the probabilities are rounded to fp16 (2^-11 relative each, fp32 accumulation).
+// the per-row kernel: the probabilities are rounded to fp16 (2^-11 relative, fp32 accumulation).
 template <int HD8>
 __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, const int rows) {
   typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
@@ -478,7 +471,7 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
   for (int hh = wave; hh < group; hh += 4) {
     const int head = kvh * group + hh;
     // the rotated query of (row, head): the lane's values 32 j + 8 g + e; the partner of a low value is the value half further, in the same lane (j + NJ / 2)
-    u32x4 qb[NJ];
+    u32x4 qb[NJ], qr[NJ];
     {
       const float* qrow = a.q + (size_t)row * a.q_bs + (size_t)head * HD;
       const float* rr = a.rope + (size_t)pos * HD;
@@ -493,6 +486,10 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
           hi[e4] = rope_hi(x1.x, x2.x, cs.x, sn.x); hi[e4 + 1] = rope_hi(x1.y, x2.y, cs.y, sn.y); hi[e4 + 2] = rope_hi(x1.z, x2.z, cs.z, sn.z); hi[e4 + 3] = rope_hi(x1.w, x2.w, cs.w, sn.w);
         }
         qb[j] = pack8_f16(lo); qb[j + NJ / 2] = pack8_f16(hi);
+        float lr[8], hr[8];                               // what the fp16 rounding left over: a second operand, so that the scores see the float32 queries
+#pragma unroll
+        for (int e = 0; e < 8; e++) { lr[e] = lo[e] - (float)(_Float16)lo[e]; hr[e] = hi[e] - (float)(_Float16)hi[e]; }
+        qr[j] = pack8_f16(lr); qr[j + NJ / 2] = pack8_f16(hr);
       }
     }
     // scores of the 64 keys x 16 rows
@@ -501,7 +498,10 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
     for (int t = 0; t < 4; t++) {
       sc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < NJ; j++) sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qb[j]), sc[t], 0, 0, 0);
+      for (int j = 0; j < NJ; j++) {
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qr[j]), sc[t], 0, 0, 0);
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qb[j]), sc[t], 0, 0, 0);
+      }
     }
     float m = -INFINITY;
 #pragma unroll
@@ -912,24 +912,15 @@ int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, flo
   TGA_REQUIRE(dim > 0 && rows >= 1, "tga_rmsnorm: rows=%d dim=%d", rows, dim);
   int sfmt = 0, snu = 0;
   if (stage_type) { sfmt = decode_staged_fmt(stage_type, dim, &snu); TGA_REQUIRE(sfmt >= 0, "tga_rmsnorm: no staged layout for type %d with K=%d", stage_type, dim); }
-  rmsnorm_kernel<false><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu, nullptr, nullptr, nullptr, 0, nullptr, 0, 0);
+  rmsnorm_kernel<false><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, sfmt, snu, nullptr, nullptr, nullptr, 0);
   TGA_LAUNCH_CHECK();
   return 0;
 }
-}  // extern "C"
-// tga_rmsnorm_rows whose fp16 rows also go to `staged`, in the layout the 17 .. 64 row GEMM multiplies from (format fmt of nu units per row, ncg column groups of
-// sixteen rows; the rows from `rows` up to 16 ncg are zeros there)
-int tga_rmsnorm_rows_staged64(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, int fmt, int nu, void* staged, int ncg, void* stream) {
-  rmsnorm_kernel<false><<<16 * ncg, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, nullptr, fmt, nu, nullptr, nullptr, nullptr, 0, (_Float16*)staged, ncg, rows);
-  TGA_LAUNCH_CHECK();
-  return 0;
-}
-extern "C" {
 int tga_moe_combine_rmsnorm_rows(const float* y, const float* probs, float* x, const float* weight, int rows, int k, int dim, float eps, void* out_f16, float* out_f32,
                                  void* stream) {
   TGA_REQUIRE(y && probs && x && weight && (out_f16 || out_f32), "tga_moe_combine_rmsnorm_rows: null pointer");
   TGA_REQUIRE(dim > 0 && rows >= 1 && k >= 1, "tga_moe_combine_rmsnorm_rows: rows=%d k=%d dim=%d", rows, k, dim);
-  rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k, nullptr, 0, 0);
+  rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -58,6 +58,56 @@ __global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const 
   for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = scol < M ? xv[v] : u32x4{0u, 0u, 0u, 0u};
 }
 
+// The RMSNorm in front of a linear (attn_norm -> q / k / v, ffn_norm -> gate / up; nn.RMSNorm, tinygrad/nn/__init__.py:296-304) and q64_stage_kernel in one launch: one
+// workgroup per row sums the squares of the float32 row, writes (x rsqrt(mean x^2 + eps)) w rounded to fp16 - rmsnorm_kernel's expression - to xn_out and to LDS, and
+// its threads then stage the row's units from LDS.  Workgroups at and beyond M fill their rows of the staged buffer with zeros.
+template <int T_, int NCG>
+__global__ __launch_bounds__(256) void q64_norm_stage_kernel(const float* __restrict__ x, const float* __restrict__ w, const int K, const float eps,
+                                                             _Float16* __restrict__ xn_out, u32x4* __restrict__ xs, const int M) {
+  using F = Fmt<T_>;
+  extern __shared__ u32x4 lds[];                          // the normalised fp16 row
+  __shared__ float red[4];
+  const int m = blockIdx.x, tid = threadIdx.x, nu = K >> 6;
+  auto dst_of = [&](int u) { return xs + (size_t)(u >> 2) * (F::XV * NCG * 64) + (m >> 4) * 64 + (u & 3) * 16 + (m & 15); };
+  if (m >= M) {
+    for (int u = tid; u < nu; u += 256) {
+      u32x4* dst = dst_of(u);
+#pragma unroll
+      for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = u32x4{0u, 0u, 0u, 0u};
+    }
+    return;
+  }
+  const f32x4* xr = (const f32x4*)(x + (size_t)m * K);
+  const f32x4* wr = (const f32x4*)w;
+  const int n4 = K >> 2;
+  float s = 0.f;
+  for (int i = tid; i < n4; i += 256) { const f32x4 v = xr[i]; s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+  s = wave_sum(s);
+  if ((tid & 63) == 0) red[tid >> 6] = s;
+  __syncthreads();
+  const float scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)K + eps);
+  uint32_t* row32 = (uint32_t*)lds;
+  uint32_t* out32 = (uint32_t*)(xn_out + (size_t)m * K);
+  for (int i = tid; i < n4; i += 256) {
+    const f32x4 v = xr[i], g = wr[i];
+    const uint32_t lo = f2h_bits((v.x * scale) * g.x) | (f2h_bits((v.y * scale) * g.y) << 16), hi = f2h_bits((v.z * scale) * g.z) | (f2h_bits((v.w * scale) * g.w) << 16);
+    row32[2 * i] = lo; row32[2 * i + 1] = hi;
+    out32[2 * i] = lo; out32[2 * i + 1] = hi;
+  }
+  __syncthreads();
+  QArgs q = {};
+  q.x = (const void*)lds; q.x_f32 = 0; q.K = K;
+  for (int u = tid; u < nu; u += 256) {
+    uint32_t nx[F::UW / 2];
+    stage_fetch<T_>(q, 0, u, nx);
+    u32x4 xv[F::XV]; float cs[F::NG];
+    F::stage(nx, xv, cs);
+    u32x4* dst = dst_of(u);
+#pragma unroll
+    for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = xv[v];
+  }
+}
+
 template <int T_, bool MS, bool SW, int NCG, int NT>
 __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const int M, const Q64X ex) {
   const QArgs a = args;
@@ -370,6 +420,36 @@ void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* nc
   if (!q64_in_range(fmt, a, M)) return nullptr;
   *ncg = M <= 32 ? 2 : 4;
   return q64_slot(s);
+}
+
+template <int T>
+static int launch_norm_stage(const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s) {
+  using F = Fmt<T>;
+  if constexpr (F::UW != 64 || F::XV != 8) return -1;
+  else {
+    static const hipError_t c2 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    static const hipError_t c4 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    TGA_HIP(c2); TGA_HIP(c4);
+    if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M);
+    else q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M);
+    TGA_LAUNCH_CHECK();
+    return 0;
+  }
+}
+// RMSNorm of M float32 rows of K values (K a multiple of 256 up to Q64_MAX_K, x and w 16-byte aligned) into xn_out (fp16 rows) and into `staged`, the buffer
+// tga_qgemm64_staging handed out for a consumer of format fmt
+int tga_qgemm64_norm_stage(int fmt, const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s) {
+  if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)xn_out) & 15) != 0 || K % 256 != 0 || K > Q64_MAX_K) return -1;
+  switch (fmt) {
+    case F_Q4_0P: return launch_norm_stage<F_Q4_0P>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case F_Q8_0P: return launch_norm_stage<F_Q8_0P>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case GGML_Q6_K: return launch_norm_stage<GGML_Q6_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case GGML_Q4_K: return launch_norm_stage<GGML_Q4_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case GGML_Q5_K: return launch_norm_stage<GGML_Q5_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case GGML_IQ4_XS: return launch_norm_stage<GGML_IQ4_XS>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case GGML_F16: return launch_norm_stage<GGML_F16>(x, w, K, eps, xn_out, staged, M, ncg, s);
+  }
+  return -1;
 }
 
 // Returns -1 when the call is outside this kernel's range or no workspace slot is left for the stream (the caller then runs blocks of sixteen rows).

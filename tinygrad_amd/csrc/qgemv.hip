@@ -320,7 +320,7 @@ int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    //
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
 int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, bool prestaged, hipStream_t s);       // qgemm64.hip
 void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* ncg);              // qgemm64.hip
-int tga_rmsnorm_rows_staged64(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, int fmt, int nu, void* staged, int ncg, void* stream);   // decode.hip
+int tga_qgemm64_norm_stage(int fmt, const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s);   // qgemm64.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -615,9 +615,12 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
     if (ok && q64_args(ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, K, epilogue, resid, q, fmt64)) {
       void* staged = tga_qgemm64_staging(fmt64, q, M, (hipStream_t)stream, &ncg);
       if (staged) {
-        if (const int rc = tga_rmsnorm_rows_staged64(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, fmt64, (int)(K / 64), staged, ncg, stream)) return rc;
-        const int rc = tga_qgemm64_dispatch(fmt64, q, M, true, (hipStream_t)stream);
-        if (rc >= 0) return rc;                                   // (cannot be refused here: the same checks have passed above)
+        const int rn = tga_qgemm64_norm_stage(fmt64, x, norm_weight, (int)K, norm_eps, xn_scratch_f16, staged, M, ncg, (hipStream_t)stream);
+        if (rn > 0) return rn;
+        if (rn == 0) {
+          const int rc = tga_qgemm64_dispatch(fmt64, q, M, true, (hipStream_t)stream);
+          if (rc >= 0) return rc;                                 // (cannot be refused here: the same checks have passed above)
+        }
       }
     }
   }
