@@ -264,6 +264,27 @@ int tga_attention_decode_batched(int batch, const float* q, const float* k, cons
 int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
+/* tga_attention_prefill_chunk for 17 .. 64 rows whose fp16 output is ONE buffer for all rows in the layout the 64-column GEMM multiplies from, for a consumer
+ * (attn_output) of block type consumer_type with K = n_heads * head_dim (a multiple of 256): 16 * (rows <= 32 ? 2 : 4) rows x K fp16 values; the rows at and beyond
+ * `rows` are not written (zero them once). */
+int tga_attention_prefill_chunk_staged(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                       int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                       int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_rows_staged, int consumer_type, void* stream);
+/* ---- a prefill step of 17 .. 64 rows (model.py:464, 476-481) with the rows handed from launch to launch in the layout the 64-column GEMM multiplies from: no
+ * counterpart in the reference (its scheduler fuses what it fuses); the results equal those of tga_rmsnorm_qlinear_rows / tga_qlinear_multi on plain rows up to the
+ * order of a float32 sum.  tga_qlinear_multi takes such rows with x_dtype TGA_F16_STAGED and M > 16, and writes them from the SwiGLU epilogue with y_stage_type. ---- */
+/* *ncg = column groups of sixteen rows (2 or 4: the buffer of the rows holds 16 * ncg x K fp16 values) when a linear of this type with rows of K values takes M rows
+ * in that layout, 0 when it does not. */
+int tga_rows_staged_plan(int ggml_type, int64_t K, int M, int* ncg);
+/* y = y + x W^T (attn_output, ffn_down: model.py:149-150) for one matrix over rows in that layout.  When the kernel splits K, the sum over the splits is left to the
+ * caller's next launch: *partials / *ks / *np describe the partial tiles (in the stream's workspace: valid until the next call with 17 .. 64 rows on this stream) and y
+ * is untouched; *ks = 0: y is complete. */
+int tga_qlinear_rows_deferred(int ggml_type, const void* w, int64_t N, int64_t K, const void* x_staged, int M, float* y, const float** partials, int* ks, int* np, void* stream);
+/* nn.RMSNorm (tinygrad/nn/__init__.py:296-304) of `rows` float32 rows, written as fp16 in that layout for a consumer of consumer_type (and to xn_out_f16 as plain
+ * rows when given).  partials != NULL: every row is first completed in place with what tga_qlinear_rows_deferred left. */
+int tga_rmsnorm_rows_stage(float* x, const float* partials, int ks, int np, const float* weight, float eps, int rows, int dim, int consumer_type, void* xn_out_f16, void* staged_out, void* stream);
+/* x += the sum of those partial tiles in the order of K (what the deferred call's own reduce launch would have done). */
+int tga_rows_add_partials(float* x, const float* partials, int ks, int np, int rows, int dim, void* stream);
 /* After a chunk of `rows` prompt positions: state.pos += rows and tokens[r] = prompt[state.pos + r] (entries past max_ctx - 1 read the last one): the
  * input ids of the next chunk (model.py:477-480 slices the prompt on the host; here the captured step advances itself). */
 int tga_chunk_advance(void* state, const int32_t* prompt, int rows, int32_t* tokens, int max_ctx, void* stream);

@@ -131,6 +131,28 @@ def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
   print(f"prompt {n_prompt}: min top-2 margin {margin:.4f}, worst logits rel-err {worst:.2e}")
   assert got == ref and worst <= 1e-3
 
+@pytest.mark.parametrize("ltype,chunk", [("Q4_0", 64), ("Q8_0", 24), ("Q4_K", 40), ("Q6_K", 32)])
+def test_prefill_steps_with_rows_in_the_multiplying_layout_equal_the_plain_steps(gpu, monkeypatch, ltype, chunk):
+  """A prefill in steps of 17 .. 64 positions hands its rows from launch to launch in the layout the 64-column kernel multiplies from and lets the norm launches complete
+  the split-K sums (BatchedTransformer.rows64); with TGA_ROWS64=0 the same steps run on plain rows.  Same kernels on the same fp16 values: the KV caches agree to the order
+  of a float32 sum, the decode steps that follow give the same tokens."""
+  from tinygrad_amd import runtime as rt
+  cfg = dict(SMALL, dim=512, hidden_dim=1024, n_heads=8, n_kv_heads=2) if ltype in ("Q4_K", "Q6_K") else SMALL
+  rng = np.random.default_rng(64 + chunk)
+  prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=150)]
+  caches, toks = [], []
+  for flag in ("1", "0"):
+    monkeypatch.setenv("TGA_ROWS64", flag)
+    model, _ = _build(gpu, cfg, 192, seed=33, linear_type=getattr(rt, ltype))
+    model.prefill_chunk = chunk
+    model.prefill(prompt)
+    assert bool(model._chunker.rows64) == (flag == "1")
+    caches.append([(b.cache_k.numpy().astype(np.float32), b.cache_v.numpy().astype(np.float32)) for b in model.blk])
+    toks.append(list(model.generate(prompt, 8)))
+  for (k1, v1), (k0, v0) in zip(*caches):
+    assert ol.rel_err(k1, k0) <= 1e-3 and ol.rel_err(v1, v0) <= 1e-3
+  assert toks[0] == toks[1]
+
 def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
   """tga_attention_prefill_chunk alone: eight consecutive positions per call over one cache (per-head q/k norm, GQA), each row against numpy attention over
   the positions up to its own; tga_chunk_advance moves the position and loads the next ids."""

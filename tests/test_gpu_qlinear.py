@@ -266,6 +266,64 @@ def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
   refn = np.concatenate([cref.linear(t, w, h[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
   assert ol.rel_err(out.numpy(), refn) <= TOL
 
+@pytest.mark.parametrize("t,dim,hidden,m", [(2, 1024, 2048, 40), (8, 512, 1024, 17), (12, 1024, 2304, 64), (14, 512, 1024, 33), (23, 1024, 1024, 24), (13, 256, 512, 50)])
+def test_rows_in_the_multiplying_layout_equal_plain_rows(gpu, t, dim, hidden, m):
+  """The entry points of a prefill step that hands its rows from launch to launch in the layout the 64-column kernel multiplies from (tga_rmsnorm_rows_stage ->
+  tga_qlinear_multi with staged x -> SwiGLU written for its consumer -> tga_qlinear_rows_deferred -> partial sums completed by the next norm or by
+  tga_rows_add_partials) against the same linears on plain rows (tga_rmsnorm_qlinear_rows, tga_qlinear_multi): the same kernels multiply the same fp16 values, so the
+  results agree to 1e-5 with the plain rows and bit for bit among the staged variants, except where a sum is taken in another order (residual first instead of last: 1e-6)."""
+  import ctypes
+  from tinygrad_amd.nn import QuantLinear, qlinear_multi
+  from tinygrad_amd import runtime as rt
+  L = gpu.lib()
+  rng = np.random.default_rng(7 * t + m)
+  ncg = ctypes.c_int(0)
+  gpu.check(L.tga_rows_staged_plan(t, dim, m, ctypes.byref(ncg)))
+  assert ncg.value == (2 if m <= 32 else 4)
+  gpu.check(L.tga_rows_staged_plan(39, 2048, m, ctypes.byref(ncg))); assert ncg.value == 0          # (MXFP4: no 64-column kernel)
+  gpu.check(L.tga_rows_staged_plan(t, dim, 16, ctypes.byref(ncg))); assert ncg.value == 0
+  R = 16 * (2 if m <= 32 else 4)
+  gate, up = (QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, t, hidden, dim)), t, hidden, dim) for _ in range(2))
+  down = QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, t, dim, hidden)), t, dim, hidden)
+  x = (rng.standard_normal((m, dim)) * 2).astype(np.float32)
+  nw = gpu.Buffer.from_numpy(((1 + 0.2 * rng.standard_normal(dim)) * (0.01 if t in (12, 13, 14, 23) else 1.0)).astype(np.float32))   # (random superblock scales are large: keep silu(g) * u inside fp16)
+  # plain rows: norm + gate/up + SwiGLU, then down + residual in place
+  xb, xn, act = gpu.Buffer.from_numpy(x), gpu.Buffer((m, dim), np.float16), gpu.Buffer((m, hidden), np.float16)
+  qlinear_multi([gate, up], xb, [act], epilogue=2, norm=(nw, 1e-5, xn))
+  qlinear_multi([down], act, [xb], epilogue=1, resid=[xb])
+  ref = xb.numpy()
+  # rows in the multiplying layout
+  xs = gpu.Buffer.from_numpy(x)
+  xn_st, act_st, xn2 = gpu.Buffer((R, dim), np.float16), gpu.Buffer((R, hidden), np.float16), gpu.Buffer((m, dim), np.float16)
+  for b in (xn_st, act_st): gpu.check(L.tga_memset(b.ptr, 0xFF, b.nbytes, None))
+  gpu.check(L.tga_rmsnorm_rows_stage(xs.ptr, None, 0, 0, nw.ptr, 1e-5, m, dim, t, xn2.ptr, xn_st.ptr, None))
+  np.testing.assert_array_equal(xn2.numpy(), xn.numpy())
+  VP2, I2 = ctypes.c_void_p * 2, ctypes.c_int64 * 2
+  gpu.check(L.tga_qlinear_multi(t, 2, VP2(gate.blocks.ptr, up.blocks.ptr), VP2(act_st.ptr, None), I2(hidden, hidden), xn_st.ptr, rt.F16_STAGED, rt.F16, m, dim, 2, None, t, hidden, None))
+  VP1, I1 = ctypes.c_void_p * 1, ctypes.c_int64 * 1
+  yb = gpu.Buffer.from_numpy(x)                                                           # down + residual over the staged rows, sum taken by the call itself
+  gpu.check(L.tga_qlinear_multi(t, 1, VP1(down.blocks.ptr), VP1(yb.ptr), I1(dim), act_st.ptr, rt.F16_STAGED, rt.F32, m, hidden, 1, VP1(yb.ptr), 0, 0, None))
+  staged = yb.numpy()
+  assert ol.rel_err(staged, ref) <= 1e-4                                                  # (the two SwiGLU epilogues are separate builds of silu(g) * u: a product may round the other way)
+  part, ks, npitch = ctypes.c_void_p(), ctypes.c_int(-1), ctypes.c_int(-1)
+  gpu.check(L.tga_qlinear_rows_deferred(t, down.blocks.ptr, dim, hidden, act_st.ptr, m, xs.ptr, ctypes.byref(part), ctypes.byref(ks), ctypes.byref(npitch), None))
+  if ks.value:
+    gpu.synchronize()
+    np.testing.assert_array_equal(xs.numpy(), x)                                          # the sum is pending: y untouched
+    xs2 = gpu.Buffer.from_numpy(x)
+    gpu.check(L.tga_rows_add_partials(xs2.ptr, part.value, ks.value, npitch.value, m, dim, None))
+    np.testing.assert_array_equal(xs2.numpy(), staged)
+    # ... or completed by the next norm's launch, which also normalises the completed rows
+    st2, xn3 = gpu.Buffer((R, dim), np.float16), gpu.Buffer((m, dim), np.float16)
+    gpu.check(L.tga_rmsnorm_rows_stage(xs.ptr, part.value, ks.value, npitch.value, nw.ptr, 1e-5, m, dim, t, xn3.ptr, st2.ptr, None))
+    assert ol.rel_err(xs.numpy(), staged) <= 1e-6
+    h = xs.numpy(); hn = h / np.sqrt((h.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-5) * nw.numpy()
+    assert ol.rel_err(xn3.numpy().astype(np.float32), hn.astype(np.float32)) <= 1e-3
+  else:
+    np.testing.assert_array_equal(xs.numpy(), staged)
+  # a staged call outside the kernel's range is refused, not run on other rows
+  assert L.tga_qlinear_multi(39, 2, VP2(gate.blocks.ptr, up.blocks.ptr), VP2(act_st.ptr, None), I2(hidden, hidden), xn_st.ptr, rt.F16_STAGED, rt.F16, m, dim, 2, None, 0, 0, None) != 0
+
 def test_seventeen_rows_on_more_streams_than_workspace_slots(gpu):
   """The 64-column kernel keeps its staged activations and split-K partial tiles in a per-device workspace of a few slots, one per stream; a call on a
   further stream runs blocks of sixteen rows instead.  Six streams, two calls each (the second finds its stream's slot again): every result within the bar,

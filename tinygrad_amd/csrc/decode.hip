@@ -129,6 +129,7 @@ struct AttnArgs {
   float scale;
   _Float16* out16; float* out32;                       // attention output [n_heads*hd]
   int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
+  int stage_rows_ncg;                                  // != 0 (rows of a prefill step): out16 is ONE buffer for all rows, in the layout the 17 .. 64 row GEMM multiplies from (rows_staged_pos)
   const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights: over the whole q / k vectors, or
   int norm_per_head;                                           // per head (weights of head_dim values shared by all heads)
   // batched decode (sequences in lockstep at one position): sequence z = blockIdx.z (split launch) / blockIdx.y (merge launch) uses the
@@ -739,7 +740,8 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
   }
   o *= 1.0f / l;
   const int e = head * HD + d;
-  if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, e, a.stage_nu) : e] = (_Float16)o;
+  if (a.stage_rows_ncg) args.out16[rows_staged_pos(a.stage_fmt, e, blockIdx.y, a.stage_rows_ncg)] = (_Float16)o;
+  else if (a.out16) a.out16[a.stage_fmt ? staged_pos(a.stage_fmt, e, a.stage_nu) : e] = (_Float16)o;
   if (a.out32) a.out32[e] = o;
 }
 
@@ -943,13 +945,18 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = (max_ctx + 63) / 64;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.out16 = (_Float16*)out_f16; a.out32 = out_f32;
-  a.stage_fmt = 0; a.stage_nu = 0;
+  a.stage_fmt = 0; a.stage_nu = 0; a.stage_rows_ncg = 0;
   a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps; a.norm_per_head = norm_per_head;
   a.q_bs = (long long)n_heads * head_dim; a.kv_bs = (long long)n_kv_heads * head_dim; a.cache_bs = (long long)n_kv_heads * max_ctx * head_dim;
   a.part_bs = (long long)n_heads * a.nsplit * (head_dim + 2); a.out_bs = (long long)n_heads * head_dim;
   a.chunk = 0; a.pos_step = 0;
   if (chunk) { a.cache_bs = 0; a.pos_step = 1; }
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
+  if (stage_type && chunk) {                            // the rows of a prefill step for the 17 .. 64 row GEMM
+    TGA_REQUIRE(out_f16 && batch >= 17 && batch <= 64 && ((long long)n_heads * head_dim) % 256 == 0 && stage_type != GGML_MXFP4 && stage_type != GGML_Q4_1 && stage_type != GGML_Q5_0 && stage_type != GGML_Q5_1,
+                "tga_attention_prefill_chunk: rows in the multiplying layout need 17..64 rows, n_heads * head_dim a multiple of 256 and a block type the 64-column kernel takes");
+    a.stage_rows_ncg = batch <= 32 ? 2 : 4;
+  }
   dim3 grid(n_kv_heads, a.nsplit, batch);
   hipStream_t s = (hipStream_t)stream;
   const int norm = !q_norm_weight ? 0 : norm_per_head ? 2 : ((long long)n_heads * head_dim <= 4096 && (long long)n_kv_heads * head_dim <= 4096) ? 1 : 3;
@@ -957,7 +964,7 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
     if (norm == 0) attn_decode_kernel<HD8, 0><<<grid, 256, 0, s>>>(a); else if (norm == 1) attn_decode_kernel<HD8, 1><<<grid, 256, 0, s>>>(a); \
     else if (norm == 2) attn_decode_kernel<HD8, 2><<<grid, 256, 0, s>>>(a); else attn_decode_kernel<HD8, 3><<<grid, 256, 0, s>>>(a); } while (0)
   static const bool chunk_mfma_off = getenv("TGA_ATTN_CHUNK") && !strcmp(getenv("TGA_ATTN_CHUNK"), "rows");
-  const bool chunk_mfma = chunk && batch > 8 && norm == 0 && (head_dim == 64 || head_dim == 128) && !chunk_mfma_off && !stage_type;   // chunks of more than eight rows attend on the matrix cores
+  const bool chunk_mfma = chunk && batch > 8 && norm == 0 && (head_dim == 64 || head_dim == 128) && !chunk_mfma_off;   // chunks of more than eight rows attend on the matrix cores
   for (int pass = chunk ? 1 : 0; pass <= (chunk ? 2 : 0); pass++) {   // chunked prefill: append every row, then attend from the cache
     a.chunk = pass;
     if (pass == 2 && chunk_mfma) {
@@ -1038,6 +1045,14 @@ int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const 
   TGA_REQUIRE(rows >= 1 && rows <= 64, "tga_attention_prefill_chunk: rows=%d", rows);
   return attention_launch(1, rows, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_f16, out_f32, 0, stream);
+}
+
+int tga_attention_prefill_chunk_staged(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
+                                       int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
+                                       int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_rows_staged, int consumer_type, void* stream) {
+  TGA_REQUIRE(rows >= 17 && rows <= 64 && consumer_type != 0, "tga_attention_prefill_chunk_staged: rows=%d (17..64), consumer type %d", rows, consumer_type);
+  return attention_launch(1, rows, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
+                          rope_table, out_rows_staged, nullptr, consumer_type, stream);
 }
 
 int tga_chunk_advance(void* state, const int32_t* prompt, int rows, int32_t* tokens, int max_ctx, void* stream) {

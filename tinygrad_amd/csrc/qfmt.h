@@ -888,12 +888,13 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
   return e;
 }
 
-// Halfword index of element e of activation row m in the layout the 17 .. 64 row GEMM (qgemm64.hip) multiplies from, for a consumer of format fmt with nu
-// units per row and ncg column groups: per step of four units [vector][column group][unit][column] 16-byte pieces (the formats' staged vectors, Fmt::stage).
-__device__ __forceinline__ size_t rows_staged_pos(int fmt, int e, int nu, int m, int ncg) {
+// Halfword index of element e of activation row m in the layout the 17 .. 64 row GEMM (qgemm64.hip) multiplies from, for a consumer of format fmt (units of 64
+// values) and ncg column groups: per step of four units [vector][column group][unit][column] 16-byte pieces (the formats' staged vectors, Fmt::stage).  The staged
+// position inside a superblock's four units does not depend on the row length, so it is taken for a row of four units (no division by the unit count).
+__device__ __forceinline__ size_t rows_staged_pos(int fmt, int e, int m, int ncg) {
   int u, i, h;
   if (fmt == GGML_F16) { u = e >> 6; i = (e >> 3) & 7; h = e & 7; }                      // (fp16 weights: the vectors are the unit's values in order)
-  else { const int full = staged_pos(fmt, e, nu); h = full & 7; const int t = full >> 3; i = t / nu; u = t - i * nu; }
+  else { const int full = staged_pos(fmt, e & 255, 4); h = full & 7; const int t = full >> 3; i = t >> 2; u = ((e >> 8) << 2) | (t & 3); }
   return ((size_t)(u >> 2) * (8 * ncg * 64) + (i * ncg + (m >> 4)) * 64 + (u & 3) * 16 + (m & 15)) * 8 + h;
 }
 

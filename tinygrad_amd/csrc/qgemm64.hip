@@ -38,6 +38,11 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 #define Q64_RING 3
 #endif
 
+// Options of a call (qgemv.hip fills them): prestaged - the activations already lie in the multiplying layout, in the workspace (xs_ext == nullptr) or in the caller's
+// buffer xs_ext; defer (residual epilogue, one matrix) - when K is split, the partial tiles are left for the caller's next launch to sum (q64_norm_stage_kernel,
+// tga_rows_add_partials) and part / ks / np say where they are; ks = 0 on return: nothing is pending, y is complete.
+struct Q64Opt { bool prestaged; const void* xs_ext; bool defer; float* part; int ks, np; };
+
 struct Q64X {
   u32x4* xs;            // staged activations: [step][8 vectors][NCG column groups][4 units][16 columns] pieces
   float* part;          // (K split) partial tiles [split][64 columns][np rows]
@@ -61,9 +66,12 @@ __global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const 
 // The RMSNorm in front of a linear (attn_norm -> q / k / v, ffn_norm -> gate / up; nn.RMSNorm, tinygrad/nn/__init__.py:296-304) and q64_stage_kernel in one launch: one
 // workgroup per row sums the squares of the float32 row, writes (x rsqrt(mean x^2 + eps)) w rounded to fp16 - rmsnorm_kernel's expression - to xn_out and to LDS, and
 // its threads then stage the row's units from LDS.  Workgroups at and beyond M fill their rows of the staged buffer with zeros.
+// part != nullptr: the row is first completed in place as x + the sum of the partial tiles a deferred linear left (ks splits of [64][np] float32, in the order of K:
+// what q64_reduce_kernel would have written).
 template <int T_, int NCG>
-__global__ __launch_bounds__(256) void q64_norm_stage_kernel(const float* __restrict__ x, const float* __restrict__ w, const int K, const float eps,
-                                                             _Float16* __restrict__ xn_out, u32x4* __restrict__ xs, const int M) {
+__global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__ x, const float* __restrict__ w, const int K, const float eps,
+                                                             _Float16* __restrict__ xn_out, u32x4* __restrict__ xs, const int M,
+                                                             const float* __restrict__ part, const int ks, const int np) {
   using F = Fmt<T_>;
   extern __shared__ u32x4 lds[];                          // the normalised fp16 row
   __shared__ float red[4];
@@ -77,11 +85,24 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(const float* __rest
     }
     return;
   }
-  const f32x4* xr = (const f32x4*)(x + (size_t)m * K);
+  f32x4* xr = (f32x4*)(x + (size_t)m * K);
   const f32x4* wr = (const f32x4*)w;
   const int n4 = K >> 2;
   float s = 0.f;
-  for (int i = tid; i < n4; i += 256) { const f32x4 v = xr[i]; s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w; }
+  for (int i = tid; i < n4; i += 256) {
+    f32x4 v = xr[i];
+    if (part) {                                           // (the same thread reads this piece again below: its own store, in program order)
+      for (int k0 = 0; k0 < ks; k0 += 8) {                // eight splits requested together, added in the order of K
+        f32x4 t[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) t[k] = *(const f32x4*)(part + ((size_t)(k0 + k < ks ? k0 + k : ks - 1) * 64 + m) * np + 4 * i);
+#pragma unroll
+        for (int k = 0; k < 8; k++) if (k0 + k < ks) { v.x += t[k].x; v.y += t[k].y; v.z += t[k].z; v.w += t[k].w; }
+      }
+      xr[i] = v;
+    }
+    s += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
   s = wave_sum(s);
   if ((tid & 63) == 0) red[tid >> 6] = s;
   __syncthreads();
@@ -92,7 +113,7 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(const float* __rest
     const f32x4 v = xr[i], g = wr[i];
     const uint32_t lo = f2h_bits((v.x * scale) * g.x) | (f2h_bits((v.y * scale) * g.y) << 16), hi = f2h_bits((v.z * scale) * g.z) | (f2h_bits((v.w * scale) * g.w) << 16);
     row32[2 * i] = lo; row32[2 * i + 1] = hi;
-    out32[2 * i] = lo; out32[2 * i + 1] = hi;
+    if (xn_out) { out32[2 * i] = lo; out32[2 * i + 1] = hi; }
   }
   __syncthreads();
   QArgs q = {};
@@ -220,6 +241,38 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
 
   // ---- epilogue: lane (g, c) holds, per tile and column group, activation row 16 cg + c x weight rows 4 g .. 4 g + 3 of the tile
   const int c = r;
+  if constexpr (SW && NT == 2) {
+    // silu(gate) * up in the layout the consuming linear multiplies from: the workgroup's 64 output rows are one unit of that linear's K, so the unit's eight
+    // vectors for every column are assembled in LDS (the stages are free now; the staging waves have left) and leave as 16-byte pieces, 256-byte runs per (vector,
+    // column group).  (As 2-byte stores straight from the accumulators the launch took 40.5 instead of 32 us.)  Not for a Q6_K consumer, whose units are not 64
+    // consecutive values: its rows take the general path below.
+    if (a.y_stage_fmt && a.y_stage_fmt != GGML_Q6_K) {
+      uint16_t* tile = (uint16_t*)lds;                    // [vector][column group][column] pieces of eight halves
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+#pragma unroll
+        for (int cg = 0; cg < NCG; cg++) {
+          float up[4];
+#pragma unroll
+          for (int k = 0; k < 4; k++) up[k] = __shfl_down(acc[t][cg][k], 32, 64);
+          if (g < 2) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+              const int lrow = (wave * NT + t) * 8 + 4 * g + k;                  // row inside the unit
+              const int hw = a.y_stage_fmt == GGML_F16 ? lrow : staged_pos(a.y_stage_fmt, lrow, 1);     // vector hw / 8, half hw % 8
+              const _Float16 hv = 16 * cg + c < M ? (_Float16)(silu_f(acc[t][cg][k]) * up[k]) : (_Float16)0.f;
+              tile[(((hw >> 3) * NCG + cg) * 16 + c) * 8 + (hw & 7)] = __builtin_bit_cast(uint16_t, hv);
+            }
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");            // (the four multiplying waves: the others have ended)
+      const long long u = blockIdx.x;                     // the consumer's unit
+      u32x4* dst = (u32x4*)a.y[0] + (size_t)(u >> 2) * (F::XV * NCG * 64) + (u & 3) * 16;
+      for (int p = tid; p < F::XV * NCG * 16; p += 256) dst[(p >> 4) * 64 + (p & 15)] = lds[p];
+      return;
+    }
+  }
 #pragma unroll
   for (int t = 0; t < NT; t++) {
     if (ex.ks > 1) {                                      // partial tile: [split][column][padded row], every lane stores its four rows
@@ -236,7 +289,15 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
 #pragma unroll
         for (int k = 0; k < 4; k++) up[k] = __shfl_down(acc[t][cg][k], 32, 64);
         const int col = 16 * cg + c;
-        if (g < 2 && col < M) {
+        if (a.y_stage_fmt) {                              // fp16 rows in the layout the consuming linear multiplies from (its K = these rows); rows at and beyond M as zeros
+          if (g < 2) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+              const long long row = row0[t] + 4 * g + k;
+              if (row < nrows[t]) ((_Float16*)a.y[0])[rows_staged_pos(a.y_stage_fmt, (int)row, col, NCG)] = col < M ? (_Float16)(silu_f(acc[t][cg][k]) * up[k]) : (_Float16)0.f;
+            }
+          }
+        } else if (g < 2 && col < M) {
 #pragma unroll
           for (int k = 0; k < 4; k++) {
             const long long row = row0[t] + 4 * g + k;
@@ -346,7 +407,7 @@ static int q64_split(bool sw, long long tiles, int nsteps) {   // workgroups per
 }
 
 template <int T, bool MS, bool SW, int NCG, int NT>
-static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
+static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, Q64Opt& o, hipStream_t s) {
   using F = Fmt<T>;
   auto kern = qgemm64_kernel<T, MS, SW, NCG, NT>;
   constexpr size_t stage_bytes = (size_t)F::XV * NCG * 64 * 16;
@@ -355,18 +416,20 @@ static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipS
   const int nsteps = a.nu >> 2;
   const long long tiles = (a.ntot + 64 * NT / (SW ? 2 : 1) - 1) / (64 * NT / (SW ? 2 : 1));   // workgroups over the rows: 64 NT weight rows each (SwiGLU: half of them gate rows)
   Q64X ex;
-  ex.xs = (u32x4*)ws; ex.part = (float*)(ws + Q64_XS_BYTES); ex.np = (int)(tiles * 64 * NT);
-  // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows
-  int ks = q64_split(SW, tiles, nsteps);
+  ex.xs = o.xs_ext ? (u32x4*)o.xs_ext : (u32x4*)ws; ex.part = ws ? (float*)(ws + Q64_XS_BYTES) : nullptr; ex.np = (int)(tiles * 64 * NT);
+  // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows (not without a workspace slot for the partial tiles)
+  int ks = ws ? q64_split(SW, tiles, nsteps) : 1;
   while (ks > 1 && (size_t)ks * 64 * ex.np * 4 > Q64_PART_BYTES) ks--;
   ex.ks = ks;
-  if (!prestaged) {
+  if (!o.prestaged) {
     q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
     TGA_LAUNCH_CHECK();
   }
   kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(512), 2 * stage_bytes, s>>>(a, M, ex);
   TGA_LAUNCH_CHECK();
-  if (ks > 1) {
+  o.ks = 0;
+  if (ks > 1 && o.defer) { o.part = ex.part; o.ks = ks; o.np = ex.np; }
+  else if (ks > 1) {
     const long long items = (long long)M * (ex.np / 4);
     q64_reduce_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s>>>(a, M, ex.part, ks, ex.np);
     TGA_LAUNCH_CHECK();
@@ -375,7 +438,7 @@ static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipS
 }
 
 template <int T, bool MS, bool SW, int NCG>
-static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
+static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, Q64Opt& o, hipStream_t s) {
   using F = Fmt<T>;
   // Two weight tiles per wave halve the activation bytes that reach a CU (global -> LDS -> operand) per weight; taken when the row tiles of 128, split over K,
   // still fill the chip.  (fp16 weights: a unit is 128 bytes per lane, a ring of three steps for two tiles does not fit the registers.)
@@ -384,12 +447,12 @@ static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, bool prestaged, hipS
   const long long rows_wg2 = SW ? 64 : 128, tiles2 = (a.ntot + rows_wg2 - 1) / rows_wg2;
   bool two = sizeof(typename F::Raw) <= 64 && tiles2 * q64_split(SW, tiles2, nsteps) >= 224;
   if (env_nt == 1) two = false; else if (env_nt == 2) two = sizeof(typename F::Raw) <= 64;
-  if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, prestaged, s); }
-  return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, prestaged, s);
+  if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, o, s); }
+  return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, o, s);
 }
 
 template <int T>
-static int launch_q64(QArgs a, int M, uint8_t* ws, bool prestaged, hipStream_t s) {
+static int launch_q64(QArgs a, int M, uint8_t* ws, Q64Opt& o, hipStream_t s) {
   using F = Fmt<T>;
   if constexpr (F::UW != 64 || F::XV != 8) return -1;
   else {
@@ -398,18 +461,19 @@ static int launch_q64(QArgs a, int M, uint8_t* ws, bool prestaged, hipStream_t s
     // two column groups instead of four: half the MFMAs and half the staged bytes.  (One group, for up to sixteen rows, was measured and dropped: the kernel
     // streams weights at about 2.5 TB/s - Q8_0 14336 x 4096 at M = 8 24.6 us, the Q6_K lm-head 211 us - where the LDS-fed small-batch kernels take 18.4 / 134.)
     const bool two = M <= 32;
-    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, true, 4>(a, M, ws, prestaged, s);
-    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, true, false, 4>(a, M, ws, prestaged, s);
-    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, prestaged, s) : launch_q64_t<T, false, false, 4>(a, M, ws, prestaged, s);
+    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, o, s) : launch_q64_t<T, false, true, 4>(a, M, ws, o, s);
+    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, o, s) : launch_q64_t<T, true, false, 4>(a, M, ws, o, s);
+    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, o, s) : launch_q64_t<T, false, false, 4>(a, M, ws, o, s);
   }
 }
 
 // Whether the call is inside this kernel's range: 17 .. 64 rows of fp16 or float32 activations, K a multiple of 256 up to Q64_MAX_K, one to three matrices
 // (several: each a multiple of 16 rows) with the plain or residual epilogue, or the SwiGLU pair, in one of the formats with units of 64 weights.
 static bool q64_in_range(int fmt, const QArgs& a, int M) {
-  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt || a.norm_w || a.comb_y) return false;
+  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || (a.y_stage_fmt && a.epilogue != 2) || a.norm_w || a.comb_y) return false;
   if (a.nseg > 1 && a.epilogue != 2) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return false;
   if (((uintptr_t)a.x & 15) != 0) return false;
+  if (a.y_stage_fmt && (a.y_f32 || a.y_stage_nu != (int)(a.n[0] / 64) || a.n[0] % 256 != 0)) return false;   // (staged SwiGLU rows: the consumer's K is this N)
   switch (fmt) { case F_Q4_0P: case F_Q8_0P: case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_F16: return true; }
   return false;
 }
@@ -423,48 +487,62 @@ void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* nc
 }
 
 template <int T>
-static int launch_norm_stage(const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s) {
+static int launch_norm_stage(float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, const float* part, int ks, int np, hipStream_t s) {
   using F = Fmt<T>;
   if constexpr (F::UW != 64 || F::XV != 8) return -1;
   else {
     static const hipError_t c2 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     static const hipError_t c4 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     TGA_HIP(c2); TGA_HIP(c4);
-    if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M);
-    else q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M);
+    if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    else q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
     TGA_LAUNCH_CHECK();
     return 0;
   }
 }
-// RMSNorm of M float32 rows of K values (K a multiple of 256 up to Q64_MAX_K, x and w 16-byte aligned) into xn_out (fp16 rows) and into `staged`, the buffer
-// tga_qgemm64_staging handed out for a consumer of format fmt
-int tga_qgemm64_norm_stage(int fmt, const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s) {
-  if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)xn_out) & 15) != 0 || K % 256 != 0 || K > Q64_MAX_K) return -1;
+// RMSNorm of M float32 rows of K values (K a multiple of 256 up to Q64_MAX_K, x and w 16-byte aligned) into xn_out (fp16 rows; may be null) and into `staged`, the
+// buffer of a consumer of format fmt in the multiplying layout (tga_qgemm64_staging's, or the caller's).  part != nullptr: the rows are first completed in place with
+// the partial tiles of a deferred linear (ks splits, row pitch np).  -1: outside the range.
+int tga_qgemm64_norm_stage(int fmt, float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, const float* part, int ks, int np, hipStream_t s) {
+  if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)xn_out | (uintptr_t)staged | (uintptr_t)part) & 15) != 0 || K % 256 != 0 || K > Q64_MAX_K || M < 1 || M > 16 * ncg || (ncg != 2 && ncg != 4)) return -1;
+  if (part && (ks < 1 || np < K || np % 4 != 0)) return -1;
   switch (fmt) {
-    case F_Q4_0P: return launch_norm_stage<F_Q4_0P>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case F_Q8_0P: return launch_norm_stage<F_Q8_0P>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case GGML_Q6_K: return launch_norm_stage<GGML_Q6_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case GGML_Q4_K: return launch_norm_stage<GGML_Q4_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case GGML_Q5_K: return launch_norm_stage<GGML_Q5_K>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case GGML_IQ4_XS: return launch_norm_stage<GGML_IQ4_XS>(x, w, K, eps, xn_out, staged, M, ncg, s);
-    case GGML_F16: return launch_norm_stage<GGML_F16>(x, w, K, eps, xn_out, staged, M, ncg, s);
+    case F_Q4_0P: return launch_norm_stage<F_Q4_0P>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case F_Q8_0P: return launch_norm_stage<F_Q8_0P>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case GGML_Q6_K: return launch_norm_stage<GGML_Q6_K>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case GGML_Q4_K: return launch_norm_stage<GGML_Q4_K>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case GGML_Q5_K: return launch_norm_stage<GGML_Q5_K>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case GGML_IQ4_XS: return launch_norm_stage<GGML_IQ4_XS>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
+    case GGML_F16: return launch_norm_stage<GGML_F16>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);
   }
   return -1;
 }
 
-// Returns -1 when the call is outside this kernel's range or no workspace slot is left for the stream (the caller then runs blocks of sixteen rows).
-int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, bool prestaged, hipStream_t s) {
+// Returns -1 when the call is outside this kernel's range or no workspace slot is left for the stream where one is needed (the caller then runs blocks of
+// sixteen rows): activations staged here need the slot; activations staged by the caller (o.xs_ext) run without one, with K unsplit.
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, Q64Opt& o, hipStream_t s) {
   if (!q64_in_range(fmt, a, M)) return -1;
   uint8_t* ws = q64_slot(s);
-  if (!ws) return -1;
+  if (!ws && !(o.prestaged && o.xs_ext)) return -1;
+  if (o.defer && (a.epilogue != 1 || a.nseg != 1)) return -1;
   switch (fmt) {
-    case F_Q4_0P: return launch_q64<F_Q4_0P>(a, M, ws, prestaged, s);
-    case F_Q8_0P: return launch_q64<F_Q8_0P>(a, M, ws, prestaged, s);
-    case GGML_Q6_K: return launch_q64<GGML_Q6_K>(a, M, ws, prestaged, s);
-    case GGML_Q4_K: return launch_q64<GGML_Q4_K>(a, M, ws, prestaged, s);
-    case GGML_Q5_K: return launch_q64<GGML_Q5_K>(a, M, ws, prestaged, s);
-    case GGML_IQ4_XS: return launch_q64<GGML_IQ4_XS>(a, M, ws, prestaged, s);
-    case GGML_F16: return launch_q64<GGML_F16>(a, M, ws, prestaged, s);
+    case F_Q4_0P: return launch_q64<F_Q4_0P>(a, M, ws, o, s);
+    case F_Q8_0P: return launch_q64<F_Q8_0P>(a, M, ws, o, s);
+    case GGML_Q6_K: return launch_q64<GGML_Q6_K>(a, M, ws, o, s);
+    case GGML_Q4_K: return launch_q64<GGML_Q4_K>(a, M, ws, o, s);
+    case GGML_Q5_K: return launch_q64<GGML_Q5_K>(a, M, ws, o, s);
+    case GGML_IQ4_XS: return launch_q64<GGML_IQ4_XS>(a, M, ws, o, s);
+    case GGML_F16: return launch_q64<GGML_F16>(a, M, ws, o, s);
   }
   return -1;
+}
+
+// x[m, :] += sum over the splits of the partial tiles a deferred call left (tga_qgemm64_dispatch with o.defer), in the order of K: rows x dim float32, in place
+int tga_qgemm64_add_partials(float* x, const float* part, int ks, int np, int rows, int dim, hipStream_t s) {
+  QArgs a = {};
+  a.nseg = 1; a.n[0] = dim; a.ntot = dim; a.y[0] = x; a.resid[0] = x; a.y_f32 = 1; a.epilogue = 1;
+  const long long items = (long long)rows * (np / 4);
+  q64_reduce_kernel<<<dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s>>>(a, rows, part, ks, np);
+  TGA_LAUNCH_CHECK();
+  return 0;
 }

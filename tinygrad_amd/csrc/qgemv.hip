@@ -318,9 +318,11 @@ int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    // qgemm_dma.hip
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
-int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, bool prestaged, hipStream_t s);       // qgemm64.hip
+struct Q64Opt { bool prestaged; const void* xs_ext; bool defer; float* part; int ks, np; };   // qgemm64.hip
+int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, Q64Opt& o, hipStream_t s);            // qgemm64.hip
+int tga_qgemm64_add_partials(float* x, const float* part, int ks, int np, int rows, int dim, hipStream_t s);   // qgemm64.hip
 void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* ncg);              // qgemm64.hip
-int tga_qgemm64_norm_stage(int fmt, const float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, hipStream_t s);   // qgemm64.hip
+int tga_qgemm64_norm_stage(int fmt, float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, const float* part, int ks, int np, hipStream_t s);   // qgemm64.hip
 
 // internal format id and unit count of the staged activation layout a weight of (ggml_type, K) consumes; fmt < 0: none
 static int staged_fmt(int ggml_type, long long K, int* nu) {
@@ -361,6 +363,15 @@ struct AttnIn { int n_splits, head_dim; const int* touch_pos; const void* k; con
 static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
+// the 64-column kernel's format for a weight of this type with rows of K values, -1: none (block pairs need an even number of blocks; K in steps of 256)
+static int q64_fmt_of(int ggml_type, int64_t K) {
+  if (K <= 0 || K % 256 != 0) return -1;
+  switch (ggml_type) {
+    case GGML_Q4_0: return F_Q4_0P; case GGML_Q8_0: return F_Q8_0P;
+    case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_F16: return ggml_type;
+  }
+  return -1;
+}
 // the arguments of the 17 .. 64 row GEMM (qgemm64.hip) for a call whose pointers and epilogue have been checked; false: a format or alignment it does not take
 static bool q64_args(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n, const void* x, int x_dtype, int y_dtype, int64_t K,
                      int epilogue, const void* const* resid, QArgs& q, int& fmt64) {
@@ -400,17 +411,27 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
   // 17 .. 64 rows (prefill steps): one pass over the weights on the 64-column kernel where it applies (qgemm64.hip), else blocks of sixteen rows (every block
   // after the first finds the weights in the Infinity Cache)
   if (M > 16) {
-    TGA_REQUIRE(!comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32) && !y_stage_type && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
-                "tga_qlinear: more than 16 rows only for plain fp16 / float32 activations");
+    // x_dtype TGA_F16_STAGED: x holds the rows in the layout the 64-column kernel multiplies from (written by tga_rmsnorm_rows_stage, by a SwiGLU launch with
+    // y_stage_type, or by tga_attention_prefill_chunk_staged); y_stage_type (SwiGLU): the fp16 rows are written in that layout for a consumer of that type
+    const bool xst = x_dtype == TGA_F16_STAGED;
+    TGA_REQUIRE(!comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32 || xst) && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
+                "tga_qlinear: more than 16 rows only for fp16 / float32 activations (plain, or in the multiplying layout)");
+    TGA_REQUIRE(!y_stage_type || (epilogue == 2 && y_dtype == TGA_F16 && y_stage_K == n[0]), "tga_qlinear: rows in a consumer's layout only from the SwiGLU epilogue, fp16, with y_stage_K = its rows");
     TGA_REQUIRE(y_dtype == TGA_F16 || y_dtype == TGA_F32, "tga_qlinear: y_dtype must be TGA_F16 or TGA_F32");
     TGA_REQUIRE(epilogue != 1 || y_dtype == TGA_F32, "tga_qlinear: the residual epilogue needs float32 y");
     TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
     for (int i = 0; i < nseg; i++) TGA_REQUIRE(n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]), "tga_qlinear: segment %d has a null pointer or no rows", i);
     QArgs q; int fmt64;
-    if (q64_args(ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, K, epilogue, resid, q, fmt64)) {
-      const int rc = tga_qgemm64_dispatch(fmt64, q, M, false, (hipStream_t)stream);
-      if (rc >= 0) return rc;
+    if (q64_args(ggml_type, nseg, w, y, n, x, xst ? TGA_F16 : x_dtype, y_dtype, K, epilogue, resid, q, fmt64)) {
+      bool ok = true;
+      if (y_stage_type) { q.y_stage_fmt = q64_fmt_of(y_stage_type, y_stage_K); q.y_stage_nu = (int)(y_stage_K / 64); ok = q.y_stage_fmt >= 0; }
+      if (ok) {
+        Q64Opt o = {xst, xst ? x : nullptr, false, nullptr, 0, 0};
+        const int rc = tga_qgemm64_dispatch(fmt64, q, M, o, (hipStream_t)stream);
+        if (rc >= 0) return rc;
+      }
     }
+    TGA_REQUIRE(!xst && !y_stage_type, "tga_qlinear: rows in the multiplying layout are outside the 64-column kernel's range here (tga_rows_staged_plan says which linears take them)");
     return qlinear_row_blocks(16, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
   }
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
@@ -615,10 +636,11 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
     if (ok && q64_args(ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, K, epilogue, resid, q, fmt64)) {
       void* staged = tga_qgemm64_staging(fmt64, q, M, (hipStream_t)stream, &ncg);
       if (staged) {
-        const int rn = tga_qgemm64_norm_stage(fmt64, x, norm_weight, (int)K, norm_eps, xn_scratch_f16, staged, M, ncg, (hipStream_t)stream);
+        const int rn = tga_qgemm64_norm_stage(fmt64, const_cast<float*>(x), norm_weight, (int)K, norm_eps, xn_scratch_f16, staged, M, ncg, nullptr, 0, 0, (hipStream_t)stream);
         if (rn > 0) return rn;
         if (rn == 0) {
-          const int rc = tga_qgemm64_dispatch(fmt64, q, M, true, (hipStream_t)stream);
+          Q64Opt o = {true, nullptr, false, nullptr, 0, 0};
+          const int rc = tga_qgemm64_dispatch(fmt64, q, M, o, (hipStream_t)stream);
           if (rc >= 0) return rc;                                 // (cannot be refused here: the same checks have passed above)
         }
       }
@@ -627,6 +649,49 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
   const int rc = tga_rmsnorm_rows(x, norm_weight, M, (int)K, norm_eps, xn_scratch_f16, nullptr, 0, stream);
   if (rc) return rc;
   return qlinear_multi_impl(nullptr, nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, M, K, epilogue, resid, 0, 0, stream);
+}
+
+// ---- a prefill step of 17 .. 64 rows with the rows handed from launch to launch in the layout the 64-column kernel multiplies from, and the split-K sums of the
+// residual linears completed by the norm launch behind them (llm.BatchedTransformer's step for chunks of more than sixteen positions)
+
+// Whether a linear of this type with rows of K values takes M activation rows in the multiplying layout: *ncg = column groups of sixteen rows (2 or 4; the buffer holds
+// 16 ncg x K fp16 values), 0 = no.
+extern "C" int tga_rows_staged_plan(int ggml_type, int64_t K, int M, int* ncg) {
+  TGA_REQUIRE(ncg, "tga_rows_staged_plan: null pointer");
+  *ncg = (M >= 17 && M <= 64 && K <= 32768 && q64_fmt_of(ggml_type, K) >= 0) ? (M <= 32 ? 2 : 4) : 0;
+  return 0;
+}
+
+// y = y + x W^T for one matrix (attn_output, ffn_down: the residual adds of model.py:149-150) over rows in the multiplying layout.  When the kernel splits K, the sum over
+// the splits is NOT taken: *partials / *ks / *np describe the partial tiles (in the stream's workspace, valid until the next call of 17 .. 64 rows on this stream) and y is
+// untouched - tga_rmsnorm_rows_stage (or tga_rows_add_partials) completes it.  *ks = 0: nothing is pending, y is complete.
+extern "C" int tga_qlinear_rows_deferred(int ggml_type, const void* w, int64_t N, int64_t K, const void* x_staged, int M, float* y, const float** partials, int* ks, int* np, void* stream) {
+  TGA_REQUIRE(w && x_staged && y && partials && ks && np && N > 0, "tga_qlinear_rows_deferred: null pointer or no rows");
+  const void* wv[1] = {w}; void* yv[1] = {y}; const void* rv[1] = {y}; const int64_t nv[1] = {N};
+  QArgs q; int fmt64;
+  TGA_REQUIRE(q64_args(ggml_type, 1, wv, yv, nv, x_staged, TGA_F16, TGA_F32, K, 1, rv, q, fmt64), "tga_qlinear_rows_deferred: type %d with K=%lld is outside the 64-column kernel's range", ggml_type, (long long)K);
+  Q64Opt o = {true, x_staged, true, nullptr, 0, 0};
+  const int rc = tga_qgemm64_dispatch(fmt64, q, M, o, (hipStream_t)stream);
+  TGA_REQUIRE(rc >= 0, "tga_qlinear_rows_deferred: M=%d, N=%lld, K=%lld outside the 64-column kernel's range", M, (long long)N, (long long)K);
+  *partials = o.part; *ks = o.ks; *np = o.np;
+  return rc;
+}
+
+// RMSNorm of `rows` float32 rows (nn.RMSNorm, tinygrad/nn/__init__.py:296-304) written as fp16 in the multiplying layout of a consumer of consumer_type (and, when
+// xn_out is given, as plain fp16 rows).  partials != NULL: every row is first completed in place with the partial tiles a tga_qlinear_rows_deferred call left.
+extern "C" int tga_rmsnorm_rows_stage(float* x, const float* partials, int ks, int np, const float* weight, float eps, int rows, int dim, int consumer_type, void* xn_out_f16, void* staged_out, void* stream) {
+  TGA_REQUIRE(x && weight && staged_out && rows >= 17 && rows <= 64, "tga_rmsnorm_rows_stage: null pointer or rows=%d outside 17..64", rows);
+  const int fmt = q64_fmt_of(consumer_type, dim);
+  TGA_REQUIRE(fmt >= 0, "tga_rmsnorm_rows_stage: no multiplying layout for type %d with K=%d", consumer_type, dim);
+  const int rc = tga_qgemm64_norm_stage(fmt, x, weight, dim, eps, xn_out_f16, staged_out, rows, rows <= 32 ? 2 : 4, partials, ks, np, (hipStream_t)stream);
+  TGA_REQUIRE(rc >= 0, "tga_rmsnorm_rows_stage: pointers must be 16-byte aligned, dim a multiple of 256 up to 32768");
+  return rc;
+}
+
+// x += the sum of the partial tiles a tga_qlinear_rows_deferred call left (what its own reduce launch would have done): rows x dim float32
+extern "C" int tga_rows_add_partials(float* x, const float* partials, int ks, int np, int rows, int dim, void* stream) {
+  TGA_REQUIRE(x && partials && ks >= 1 && np >= dim && np % 4 == 0 && rows >= 1 && rows <= 64 && dim > 0, "tga_rows_add_partials: null pointer or ks=%d np=%d rows=%d dim=%d", ks, np, rows, dim);
+  return tga_qgemm64_add_partials(x, partials, ks, np, rows, dim, (hipStream_t)stream);
 }
 
 // The MoE weighted sum and block residual (x += sum_j probs[j] * y[j], tinygrad/llm/model.py:130, 150) folded into the launch that

@@ -634,6 +634,19 @@ class BatchedTransformer:
     self._graphs, self._steps_done = {}, 0
     self.replay = "cmdlist"                                          # as Transformer.replay
     self.expert_path = os.environ.get("TGA_EXPERT_PATH", "jobs")      # "jobs": one GEMV per (sequence, slot); "grouped": one small-batch GEMM per selected expert
+    # Prefill steps of 17 .. 64 positions of a dense model: the rows pass from launch to launch in the layout the 64-column GEMM multiplies from (norm -> q/k/v and gate/up,
+    # attention -> attn_output, SwiGLU -> ffn_down: no staging launches) and the split-K sums of attn_output / ffn_down are completed by the norm launch behind them
+    self.rows64 = 0
+    if self.chunked and 17 <= B <= 64 and not c.num_experts and os.environ.get("TGA_ROWS64", "1") == "1":
+      def ncg_of(l):
+        n = ctypes.c_int(0); rt.check(rt.lib().tga_rows_staged_plan(l.ggml_type, l.in_features, B, ctypes.byref(n))); return n.value
+      ok = all("bias" not in b and not b["moe"] and b["attn_q"].ggml_type == b["attn_k"].ggml_type == b["attn_v"].ggml_type and b["ffn_gate"].ggml_type == b["ffn_up"].ggml_type
+               and all(ncg_of(b[nm]) for nm in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"))
+               and all(b[nm].out_features % 16 == 0 for nm in ("attn_q", "attn_k", "attn_v")) for b in self.blk)
+      if ok and c.dim % 256 == 0 and c.hidden_dim % 256 == 0 and nq % 256 == 0:
+        self.rows64 = 2 if B <= 32 else 4                              # column groups of sixteen rows in the layout
+        R = 16 * self.rows64
+        self.xn_st, self.attn_st, self.act_st = Buffer((R, c.dim), f16).zero_(), Buffer((R, nq), f16).zero_(), Buffer((R, c.hidden_dim), f16).zero_()
 
   def _linear(self, layers, x, outs, **kw): qlinear_multi(layers, x, outs, stream=self.stream.handle, **kw)
 
@@ -649,6 +662,10 @@ class BatchedTransformer:
       else: rt.check(L.tga_rmsnorm_rows(self.x.ptr, weight.ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       pending = False
     done = (lambda i: on_block(i)) if on_block is not None else (lambda i: None)     # on_block(i): block i's launches have been issued (eager stepping only; e.g. to read back self.sel)
+    if self.rows64:
+      self._blocks_rows64(done)
+      rt.check(L.tga_chunk_advance(self.state.ptr, self.prompts.ptr, B, self.tokens.ptr, c.max_context, st))
+      return
     for bi, b in enumerate(self.blk):
       # h = x + attention(attn_norm(x))                                                   model.py:149
       qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
@@ -713,6 +730,40 @@ class BatchedTransformer:
       return
     rt.check(L.tga_argmax_rows_step(self.logits_buf.ptr if with_head else None, B, c.vocab_size, self.state.ptr, self.prompts.ptr, c.max_context, self.tokens.ptr,
                                     self.out_tokens.ptr, self.max_new, st))
+
+  def _blocks_rows64(self, done):
+    """The blocks of a prefill step of 17 .. 64 rows (see rows64 in __init__): per block norm (+ the pending split-K sums of the linear before it) -> q/k/v -> attention ->
+    attn_output (sums deferred) -> norm -> gate/up + SwiGLU -> ffn_down (sums deferred); what the last block leaves pending is added at the end."""
+    c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
+    VP3, VP2, I3, I2 = ctypes.c_void_p * 3, ctypes.c_void_p * 2, ctypes.c_int64 * 3, ctypes.c_int64 * 2
+    pend = (None, 0, 0)                                                # partial tiles still to be added to self.x: (pointer, splits, row pitch)
+    def norm_stage(weight, consumer):
+      nonlocal pend
+      rt.check(L.tga_rmsnorm_rows_stage(self.x.ptr, pend[0], pend[1], pend[2], weight.ptr, c.norm_eps, B, c.dim, consumer.ggml_type, None, self.xn_st.ptr, st))
+      pend = (None, 0, 0)
+    def deferred(layer, x_st):
+      nonlocal pend
+      part, ks, np_ = ctypes.c_void_p(), ctypes.c_int(0), ctypes.c_int(0)
+      rt.check(L.tga_qlinear_rows_deferred(layer.ggml_type, layer.blocks.ptr, layer.out_features, layer.in_features, x_st.ptr, B, self.x.ptr,
+                                           ctypes.byref(part), ctypes.byref(ks), ctypes.byref(np_), st))
+      pend = (part.value, ks.value, np_.value) if ks.value else (None, 0, 0)
+    for bi, b in enumerate(self.blk):
+      q, k, v = b["attn_q"], b["attn_k"], b["attn_v"]
+      norm_stage(b["attn_norm"], q)
+      rt.check(L.tga_qlinear_multi(q.ggml_type, 3, VP3(q.blocks.ptr, k.blocks.ptr, v.blocks.ptr), VP3(self.q.ptr, self.k.ptr, self.v.ptr), I3(q.out_features, k.out_features, v.out_features),
+                                   self.xn_st.ptr, rt.F16_STAGED, rt.F32, B, q.in_features, 0, None, 0, 0, st))
+      ao = b["attn_output"]
+      rt.check(L.tga_attention_prefill_chunk_staged(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
+                                                    c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
+                                                    c.n_heads, c.n_kv_heads, c.head_dim, c.max_context, self.rope.ptr, self.attn_st.ptr, ao.ggml_type, st))
+      deferred(ao, self.attn_st)
+      g, u, d = b["ffn_gate"], b["ffn_up"], b["ffn_down"]
+      norm_stage(b["ffn_norm"], g)
+      rt.check(L.tga_qlinear_multi(g.ggml_type, 2, VP2(g.blocks.ptr, u.blocks.ptr), VP2(self.act_st.ptr, None), I2(g.out_features, u.out_features),
+                                   self.xn_st.ptr, rt.F16_STAGED, rt.F16, B, g.in_features, 2, None, d.ggml_type, d.in_features, st))
+      deferred(d, self.act_st)
+      done(bi)
+    if pend[1]: rt.check(L.tga_rows_add_partials(self.x.ptr, pend[0], pend[1], pend[2], B, c.dim, st))
 
   def _graph(self, with_head: bool):
     if with_head not in self._graphs:

@@ -68,6 +68,11 @@ def _declare(lib):
     "tga_attention_decode_batched": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
     "tga_attention_prefill_chunk": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
     "tga_chunk_advance": [vp, vp, i, vp, i, vp],
+    "tga_attention_prefill_chunk_staged": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, i, vp],
+    "tga_rows_staged_plan": [i, i64, i, ctypes.POINTER(i)],
+    "tga_qlinear_rows_deferred": [i, vp, i64, i64, vp, i, vp, ctypes.POINTER(vp), ctypes.POINTER(i), ctypes.POINTER(i), vp],
+    "tga_rmsnorm_rows_stage": [vp, vp, i, i, vp, ctypes.c_float, i, i, i, vp, vp, vp],
+    "tga_rows_add_partials": [vp, vp, i, i, i, i, vp],
     "tga_argmax_rows_step": [vp, i, i, vp, vp, i, vp, vp, i, vp],
     "tga_expert_jobs": [vp, i, i, vp, vp, vp], "tga_qlinear_experts_grouped": [i, vp, vp, i64, vp, i, i, vp, vp, i, i64, i64, vp],
     "tga_rmsnorm": [vp, vp, i, ctypes.c_float, vp, vp, i, vp],
