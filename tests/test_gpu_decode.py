@@ -131,19 +131,23 @@ def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
   print(f"prompt {n_prompt}: min top-2 margin {margin:.4f}, worst logits rel-err {worst:.2e}")
   assert got == ref and worst <= 1e-3
 
-@pytest.mark.parametrize("ltype,chunk", [("Q4_0", 64), ("Q8_0", 24), ("Q4_K", 40), ("Q6_K", 32)])
+@pytest.mark.parametrize("ltype,chunk", [("Q4_0", 64), ("Q8_0", 24), ("Q4_K", 40), ("Q6_K", 32), ("Q4_K_M", 48)])
 def test_prefill_steps_with_rows_in_the_multiplying_layout_equal_the_plain_steps(gpu, monkeypatch, ltype, chunk):
   """A prefill in steps of 17 .. 64 positions hands its rows from launch to launch in the layout the 64-column kernel multiplies from and lets the norm launches complete
   the split-K sums (BatchedTransformer.rows64); with TGA_ROWS64=0 the same steps run on plain rows.  Same kernels on the same fp16 values: the KV caches agree to the order
   of a float32 sum, the decode steps that follow give the same tokens."""
   from tinygrad_amd import runtime as rt
-  cfg = dict(SMALL, dim=512, hidden_dim=1024, n_heads=8, n_kv_heads=2) if ltype in ("Q4_K", "Q6_K") else SMALL
+  cfg = dict(SMALL, dim=512, hidden_dim=1024, n_heads=8, n_kv_heads=2) if ltype in ("Q4_K", "Q6_K", "Q4_K_M") else SMALL
   rng = np.random.default_rng(64 + chunk)
   prompt = [int(t) for t in rng.integers(0, cfg["vocab_size"], size=150)]
   caches, toks = [], []
   for flag in ("1", "0"):
     monkeypatch.setenv("TGA_ROWS64", flag)
-    model, _ = _build(gpu, cfg, 192, seed=33, linear_type=getattr(rt, ltype))
+    if ltype == "Q4_K_M":                                                                # Q4_K with attn_v / ffn_down as Q6_K in half of the blocks: q / k and v are two launches
+      from tinygrad_amd.llm import Transformer, TransformerConfig, synth_state
+      c = TransformerConfig(max_context=192, **cfg)
+      model = Transformer(c, synth_state(c, seed=33, q4_k_m=True), max_new=64)
+    else: model, _ = _build(gpu, cfg, 192, seed=33, linear_type=getattr(rt, ltype))
     model.prefill_chunk = chunk
     model.prefill(prompt)
     assert bool(model._chunker.rows64) == (flag == "1")

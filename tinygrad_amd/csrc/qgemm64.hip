@@ -210,17 +210,21 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
 #pragma unroll
     for (int t = 0; t < NT; t++) { F::decode(buf[t], wv[t], kc); F::to_f16(buf[t], wv[t]); }
     const u32x4* src = lds + slot * SP + lane;
+    u32x4 bv[2][NCG];                                     // a B operand is read once and meets the NT weight tiles; the operands of vector v + 1 are requested before
+#pragma unroll                                            // vector v is multiplied (left to itself the compiler waits for every pair of reads right behind them)
+    for (int cg = 0; cg < NCG; cg++) bv[0][cg] = src[cg * 64];
 #pragma unroll
     for (int v = 0; v < F::XV; v++) {
-      u32x4 bv[NCG];                                      // a B operand is read once and meets the NT weight tiles
+      if (v + 1 < F::XV) {
 #pragma unroll
-      for (int cg = 0; cg < NCG; cg++) bv[cg] = src[(v * NCG + cg) * 64];
+        for (int cg = 0; cg < NCG; cg++) bv[(v + 1) & 1][cg] = src[((v + 1) * NCG + cg) * 64];
+      }
 #pragma unroll
       for (int t = 0; t < NT; t++) {
         const u32x4 av = {wv[t][4 * v], wv[t][4 * v + 1], wv[t][4 * v + 2], wv[t][4 * v + 3]};
 #pragma unroll
         for (int cg = 0; cg < NCG; cg++)
-          acc[t][cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[cg]), acc[t][cg], 0, 0, 0);
+          acc[t][cg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, av), __builtin_bit_cast(v8f16, bv[v & 1][cg]), acc[t][cg], 0, 0, 0);
       }
     }
   };

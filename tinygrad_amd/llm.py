@@ -640,7 +640,7 @@ class BatchedTransformer:
     if self.chunked and 17 <= B <= 64 and not c.num_experts and os.environ.get("TGA_ROWS64", "1") == "1":
       def ncg_of(l):
         n = ctypes.c_int(0); rt.check(rt.lib().tga_rows_staged_plan(l.ggml_type, l.in_features, B, ctypes.byref(n))); return n.value
-      ok = all("bias" not in b and not b["moe"] and b["attn_q"].ggml_type == b["attn_k"].ggml_type == b["attn_v"].ggml_type and b["ffn_gate"].ggml_type == b["ffn_up"].ggml_type
+      ok = all("bias" not in b and not b["moe"] and b["ffn_gate"].ggml_type == b["ffn_up"].ggml_type
                and all(ncg_of(b[nm]) for nm in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"))
                and all(b[nm].out_features % 16 == 0 for nm in ("attn_q", "attn_k", "attn_v")) for b in self.blk)
       if ok and c.dim % 256 == 0 and c.hidden_dim % 256 == 0 and nq % 256 == 0:
@@ -735,7 +735,7 @@ class BatchedTransformer:
     """The blocks of a prefill step of 17 .. 64 rows (see rows64 in __init__): per block norm (+ the pending split-K sums of the linear before it) -> q/k/v -> attention ->
     attn_output (sums deferred) -> norm -> gate/up + SwiGLU -> ffn_down (sums deferred); what the last block leaves pending is added at the end."""
     c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
-    VP3, VP2, I3, I2 = ctypes.c_void_p * 3, ctypes.c_void_p * 2, ctypes.c_int64 * 3, ctypes.c_int64 * 2
+    VP2, I2 = ctypes.c_void_p * 2, ctypes.c_int64 * 2
     pend = (None, 0, 0)                                                # partial tiles still to be added to self.x: (pointer, splits, row pitch)
     def norm_stage(weight, consumer):
       nonlocal pend
@@ -748,10 +748,15 @@ class BatchedTransformer:
                                            ctypes.byref(part), ctypes.byref(ks), ctypes.byref(np_), st))
       pend = (part.value, ks.value, np_.value) if ks.value else (None, 0, 0)
     for bi, b in enumerate(self.blk):
-      q, k, v = b["attn_q"], b["attn_k"], b["attn_v"]
-      norm_stage(b["attn_norm"], q)
-      rt.check(L.tga_qlinear_multi(q.ggml_type, 3, VP3(q.blocks.ptr, k.blocks.ptr, v.blocks.ptr), VP3(self.q.ptr, self.k.ptr, self.v.ptr), I3(q.out_features, k.out_features, v.out_features),
-                                   self.xn_st.ptr, rt.F16_STAGED, rt.F32, B, q.in_features, 0, None, 0, 0, st))
+      qkv, outs, i = [b["attn_q"], b["attn_k"], b["attn_v"]], [self.q, self.k, self.v], 0
+      while i < 3:                                                     # one launch per run of equal block types (a Q4_K_M file keeps attn_v as Q6_K in half of the blocks), each over
+        j = i + 1                                                      # the rows in ITS type's layout: the norm launch runs once per run (the first completes the pending sums)
+        while j < 3 and qkv[j].ggml_type == qkv[i].ggml_type: j += 1
+        norm_stage(b["attn_norm"], qkv[i])
+        n = j - i
+        rt.check(L.tga_qlinear_multi(qkv[i].ggml_type, n, (ctypes.c_void_p * n)(*[l.blocks.ptr for l in qkv[i:j]]), (ctypes.c_void_p * n)(*[o.ptr for o in outs[i:j]]),
+                                     (ctypes.c_int64 * n)(*[l.out_features for l in qkv[i:j]]), self.xn_st.ptr, rt.F16_STAGED, rt.F32, B, qkv[i].in_features, 0, None, 0, 0, st))
+        i = j
       ao = b["attn_output"]
       rt.check(L.tga_attention_prefill_chunk_staged(B, self.q.ptr, self.k.ptr, self.v.ptr, b["q_norm"].ptr if c.qk_norm else None, b["k_norm"].ptr if c.qk_norm else None,
                                                     c.norm_eps, int(c.qk_norm == c.head_dim), b["cache_k"].ptr, b["cache_v"].ptr, self.attn_part.ptr, self.state.ptr,
