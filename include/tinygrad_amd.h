@@ -26,12 +26,12 @@ extern "C" {
 #define TGA_Q4_K 12
 #define TGA_Q5_K 13
 #define TGA_Q6_K 14
-#define TGA_IQ3_XXS 18  /* tga_dequant only */
-#define TGA_IQ3_S 21    /* tga_dequant only */
-#define TGA_IQ2_S 22    /* tga_dequant only */
-#define TGA_IQ4_XS 23   /* tga_dequant only */
+#define TGA_IQ3_XXS 18
+#define TGA_IQ3_S 21
+#define TGA_IQ2_S 22
+#define TGA_IQ4_XS 23
 #define TGA_MXFP4 39
-#define TGA_Q1_0 41     /* tga_dequant only */
+#define TGA_Q1_0 41     /* (every block type above is read in place by the linear entry points and expanded by tga_dequant) */
 /* activation dtype code: fp16 values in the staged order of the consuming weight (see tga_stage_activation) */
 #define TGA_F16_STAGED 101
 

@@ -20,7 +20,7 @@ def test_dense_f16_linear_small_batches(gpu, m):
   y = QuantLinear(gpu.Buffer.from_numpy(w.view(np.uint8).reshape(-1)), gpu.F16, n, k)(gpu.Buffer.from_numpy(x), out_dtype=np.float32).numpy()
   assert ol.rel_err(y, ol.linear_f64(x.astype(np.float32), w.astype(np.float32))) <= TOL
 
-@pytest.mark.parametrize("t,dim,n,E,k,B", [(39, 2048, 1024, 64, 8, 8), (39, 1024, 2048, 64, 8, 5), (2, 512, 130, 8, 2, 3), (1, 1024, 96, 16, 4, 8), (12, 1024, 64, 16, 4, 2), (14, 512, 48, 6, 3, 1)])
+@pytest.mark.parametrize("t,dim,n,E,k,B", [(39, 2048, 1024, 64, 8, 8), (39, 1024, 2048, 64, 8, 5), (2, 512, 130, 8, 2, 3), (1, 1024, 96, 16, 4, 8), (12, 1024, 64, 16, 4, 2), (14, 512, 48, 6, 3, 1), (23, 1024, 64, 8, 2, 4), (21, 512, 96, 8, 2, 5), (22, 1024, 48, 6, 3, 3), (18, 512, 64, 8, 4, 2), (41, 512, 64, 8, 2, 3)])
 def test_experts_grouped_against_per_job_gemv_and_oracle(gpu, t, dim, n, E, k, B):
   """Every (token, slot) job's row against the C restatement on that job's expert (model-path numerics: fp16-rounded weights), for the plain
   product with one activation row per job (the down projection's shape of call) and for silu(gate) * up with one row per token."""
@@ -28,7 +28,7 @@ def test_experts_grouped_against_per_job_gemv_and_oracle(gpu, t, dim, n, E, k, B
   from tinygrad_amd.runtime import GGML_QUANT
   rng = np.random.default_rng(dim + E + k + B)
   if t == 1: mk = lambda: _f16_weight(rng, E * n, dim).view(np.uint8).reshape(-1); row_bytes = 2 * dim
-  else: mk = lambda: synth.random_blocks(rng, t, E * n, dim); row_bytes = dim // GGML_QUANT[t][0] * GGML_QUANT[t][1]
+  else: mk = lambda: synth.random_blocks(rng, t, E * n, dim, sigma=0.0002 if t in (23, 18, 21, 22) else 0.003); row_bytes = dim // GGML_QUANT[t][0] * GGML_QUANT[t][1]   # (small scales where a block's range is wide: silu(gate) * up is stored as fp16)
   wg, wu = mk(), mk()
   ew, eu = ExpertWeights(gpu.Buffer.from_numpy(wg), t, E, n, dim), ExpertWeights(gpu.Buffer.from_numpy(wu), t, E, n, dim)
   sel_host = np.stack([rng.permutation(E)[:k] for _ in range(B)]).astype(np.int32).reshape(-1)     # distinct experts inside a token, repeats across tokens

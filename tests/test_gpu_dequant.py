@@ -2,8 +2,7 @@
 import numpy as np, pytest
 from oracle import ggml as og
 from tinygrad_amd import synth
-from tinygrad_amd.runtime import GGML_QUANT, GGML_DEQUANT_ONLY
-GGML_QUANT = {**GGML_QUANT, **GGML_DEQUANT_ONLY}
+from tinygrad_amd.runtime import GGML_QUANT
 
 pytestmark = pytest.mark.gpu
 TYPES = [2, 3, 6, 7, 8, 12, 13, 14, 18, 21, 22, 23, 39, 41]

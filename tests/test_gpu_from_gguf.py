@@ -9,8 +9,8 @@ pytestmark = pytest.mark.gpu
 def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False, expand: bool = False, codebook: bool = False):
   """kquant: the tensor-type mix of a Q4_K_M file (Q4_K linears and embedding, Q6_K for attn_v / ffn_down / output, one Q5_K matrix).
   legacy: the same mix with Q4_1 / Q5_0 / Q5_1 in place of Q4_K / Q5_K / Q6_K.
-  expand: IQ4_XS / Q1_0 / Q6_K: IQ4_XS matrices are read in place like the K-quants; Q1_0 has no in-place linear kernel and is expanded to fp16 when the model is loaded.
-  codebook: IQ3_S / IQ2_S / IQ3_XXS, all three expanded to fp16 at load."""
+  expand: IQ4_XS / Q1_0 / Q6_K.
+  codebook: IQ3_S / IQ2_S / IQ3_XXS.  Every one of these types stays in its blocks and is read in place."""
   rng = np.random.default_rng(11)
   c = dict(dim=256, hidden=512, H=4, KV=2, hd=64, L=2, vocab=512)
   def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
@@ -76,15 +76,25 @@ def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
 
-@pytest.mark.parametrize("legacy", [0, 1, 2, 3], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-in-place-q1_0-expanded", "iq3_s-iq2_s-iq3_xxs-expanded"])
+@pytest.mark.parametrize("legacy", [0, 1, 2, 3], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-q1_0", "iq3_s-iq2_s-iq3_xxs"])
 def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path, legacy):
   """A file with the tensor types of a Q4_K_M model (Q4_K / Q5_K / Q6_K matrices, Q4_K embedding; q/k/v of mixed types, so the
   block runs one launch per projection), and the same mix with the older Q4_1 / Q5_0 / Q5_1 blocks: greedy tokens and logits against
-  the numpy restatement.  Third case: IQ4_XS matrices read in place (embedding, attention, gate / up) beside a Q1_0 matrix, which is expanded to the reference's fp16 weight (model.py:376) at load; fourth: IQ3_S / IQ2_S / IQ3_XXS, all expanded at load."""
+  the numpy restatement.  Third case: IQ4_XS matrices (embedding, attention, gate / up) beside a Q1_0 matrix; fourth: IQ3_S / IQ2_S / IQ3_XXS (codebooks and sign patterns in LDS).  All read in place: the
+  model streams the file's 1.1 .. 4.25 bits per weight per token, not an fp16 expansion."""
   from tinygrad_amd.llm import Transformer
   path, raw = _make_file(tmp_path, False, kquant=legacy == 0, legacy=legacy == 1, expand=legacy == 2, codebook=legacy == 3)
   model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
-  if legacy == 2: assert model.blk[0].attn_q.ggml_type == 23 and model.embd_type == 23      # IQ4_XS stays in its blocks (4.25 bits per weight streamed per token, not 16)
+  if legacy == 2: assert model.blk[0].attn_q.ggml_type == 23 and model.embd_type == 23 and model.blk[1].attn_output.ggml_type == 41
+  if legacy == 3: assert model.blk[0].attn_q.ggml_type == 21 and model.blk[1].attn_output.ggml_type == 22 and model.blk[0].attn_v.ggml_type == 18 and model.embd_type == 21
+  if legacy in (2, 3):
+    # what a decode step streams is the file's packed bytes: per block type, weights * bytes per block / weights per block (an fp16 expansion would stream 2 bytes per weight)
+    from tinygrad_amd.runtime import GGML_QUANT
+    lins = [l for b in model.blk for l in (b.attn_q, b.attn_k, b.attn_v, b.attn_output, b.ffn_gate, b.ffn_up, b.ffn_down)] + [model.output]
+    packed = sum(l.out_features * l.in_features // GGML_QUANT[l.ggml_type][0] * GGML_QUANT[l.ggml_type][1] for l in lins)
+    nweights = sum(l.out_features * l.in_features for l in lins)
+    assert model.weight_bytes_per_token() == packed
+    print(f"weight bytes per token {packed} = {8 * packed / nweights:.2f} bits per weight (fp16 expansion: {2 * nweights})")
   cfg, weights, _ = ogguf.from_gguf_weights(raw)
   prompt = [3, 200, 17, 450, 8]
   got = list(model.generate(prompt, 12))

@@ -32,7 +32,7 @@ def test_gating_modes_vs_oracle(gpu, gating, norm):
   np.testing.assert_array_equal(sel, rs)
   np.testing.assert_allclose(p, rp, rtol=2e-5, atol=1e-7)
 
-@pytest.mark.parametrize("t,kdim,n", [(39, 2048, 1024), (39, 1024, 2048), (2, 512, 256), (8, 256, 192), (14, 512, 96), (12, 1024, 96), (13, 512, 128), (3, 512, 96), (6, 256, 128), (7, 1024, 64)])
+@pytest.mark.parametrize("t,kdim,n", [(39, 2048, 1024), (39, 1024, 2048), (2, 512, 256), (8, 256, 192), (14, 512, 96), (12, 1024, 96), (13, 512, 128), (3, 512, 96), (6, 256, 128), (7, 1024, 64), (23, 1024, 96), (18, 512, 96), (21, 1024, 64), (22, 512, 128), (41, 256, 96)])
 def test_expert_gemv_with_indirection(gpu, t, kdim, n):
   from tinygrad_amd.nn import ExpertWeights
   rng = np.random.default_rng(n + t)

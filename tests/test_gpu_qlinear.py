@@ -29,7 +29,7 @@ def _check(y, x, W):
   assert close.all(), f"{np.count_nonzero(~close)} of {close.size} outputs outside rtol/atol {TOL}"
   return e
 
-@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39])
+@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 18, 21, 22, 41])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_small_shapes_all_batches(gpu, t, m):
   rng = np.random.default_rng(1000 * t + m)
@@ -44,7 +44,8 @@ def test_small_shapes_all_batches(gpu, t, m):
   assert ol.rel_err(y, ym) <= TOL
 
 @pytest.mark.parametrize("t,k", [(2, 32), (2, 96), (2, 4096 + 32), (8, 32), (8, 160), (39, 32), (39, 2048 + 64), (14, 256), (14, 768), (14, 4096 + 256), (12, 256), (12, 4096 + 256), (23, 256), (23, 768), (23, 4096 + 256), (23, 16384), (13, 768), (13, 8192 + 512),
-                                 (3, 64), (3, 4096 + 64), (6, 192), (6, 2048 + 128), (7, 64), (7, 8192 + 64)])
+                                 (3, 64), (3, 4096 + 64), (6, 192), (6, 2048 + 128), (7, 64), (7, 8192 + 64),
+                                 (18, 256), (18, 4096 + 256), (21, 768), (21, 16384), (22, 256), (22, 8192 + 512), (41, 128), (41, 4096 + 128), (41, 32768 + 128)])
 def test_ragged_k(gpu, t, k):
   """K that is not a multiple of 64 units per row: partially filled waves."""
   rng = np.random.default_rng(k + t)
@@ -53,7 +54,7 @@ def test_ragged_k(gpu, t, k):
   x = synth.activations(rng, 2, k, np.float16)
   _check(_run(gpu, t, w, x, n, k), x, ol.weight_f32(w, n, k, t))
 
-@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39])
+@pytest.mark.parametrize("t", [2, 3, 6, 7, 8, 12, 13, 14, 23, 39, 18, 21, 22, 41])
 def test_f32_activations_and_f16_output(gpu, t):
   rng = np.random.default_rng(31 + t)
   n, k = 512, 2048
@@ -81,7 +82,7 @@ def test_config1_q4_0_4096(gpu):
   print(f"config1 rel-err vs f64 anchor {e:.2e}")
 
 @pytest.mark.parametrize("t,n,k,m", [(8, 4096, 14336, 8), (8, 512, 14336, 5), (2, 300, 14336, 8), (14, 200, 8192, 8), (12, 200, 14336, 8), (13, 136, 8192, 6), (23, 200, 14336, 8), (23, 4096, 4096, 5),
-                                     (3, 200, 14336, 8), (6, 136, 14336, 7), (7, 200, 8192, 8)])
+                                     (3, 200, 14336, 8), (6, 136, 14336, 7), (7, 200, 8192, 8), (22, 200, 14336, 8), (18, 136, 14336, 2), (21, 264, 16384, 7), (41, 200, 14336, 8)])
 def test_chunked_k_large_batch(gpu, t, n, k, m):
   """M*K activations beyond the LDS budget: the kernel walks K in chunks."""
   rng = np.random.default_rng(n + k + m)
@@ -118,7 +119,7 @@ def test_multi_segment_and_epilogues(gpu):
   ref = a / (1 + np.exp(-a)) * b
   assert ol.rel_err(out.numpy(), ref) <= TOL
 
-@pytest.mark.parametrize("t", [2, 8, 14, 1, 39], ids=["q4_0", "q8_0", "q6_k", "f16", "mxfp4"])
+@pytest.mark.parametrize("t", [2, 8, 14, 1, 39, 21, 22], ids=["q4_0", "q8_0", "q6_k", "f16", "mxfp4", "iq3_s", "iq2_s"])
 @pytest.mark.parametrize("m", [2, 3, 5, 8])
 def test_multi_segment_small_batch(gpu, t, m):
   """q / k / v in one launch at 2..8 activation rows: from three rows on the matrix-core kernel walks all three matrices (every one a multiple of
@@ -223,7 +224,7 @@ def test_small_batch_swiglu_through_lds(gpu, t, n, k, m):
     y = out.numpy().astype(np.float32)
     assert ol.rel_err(y, ref) <= (TOL if ydt == np.float32 else 2 * TOL), ydt
 
-@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 16), (2, 528, 2048, 9), (8, 14336, 4096, 13), (8, 64, 1024, 16), (2, 200, 14336, 16), (14, 300, 4096, 11), (2, 257, 1024, 12), (1, 96, 2048, 16), (23, 528, 4096, 16), (23, 300, 14336, 9)])
+@pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 16), (2, 528, 2048, 9), (8, 14336, 4096, 13), (8, 64, 1024, 16), (2, 200, 14336, 16), (14, 300, 4096, 11), (2, 257, 1024, 12), (1, 96, 2048, 16), (23, 528, 4096, 16), (23, 300, 14336, 9), (21, 300, 4096, 11), (41, 528, 2048, 16)])
 def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   """Prefill chunks of up to sixteen rows: one launch of the LDS-fed kernel where it applies (all sixteen columns of the MFMA tile), otherwise two
   calls of at most eight rows (K beyond 4096, other formats, ragged row counts).  Against the C restatement run in blocks of eight rows."""
@@ -238,7 +239,7 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
 @pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 32), (12, 528, 2048, 24), (8, 200, 14336, 40), (14, 1024, 4096, 64), (2, 512, 14336, 17), (13, 300, 4096, 48), (23, 528, 4096, 64), (12, 4096, 4096, 17),
-                                     (8, 1000, 1024, 33), (14, 72, 256, 50), (2, 200, 2048 + 32, 40), (3, 200, 2048, 40), (39, 256, 2048, 24)])
+                                     (8, 1000, 1024, 33), (14, 72, 256, 50), (2, 200, 2048 + 32, 40), (3, 200, 2048, 40), (39, 256, 2048, 24), (18, 528, 2048, 24), (22, 300, 4096, 40)])
 def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
   """Prefill chunks of 17 .. 64 rows: one pass of the 64-column kernel where it applies (K a multiple of 256, its formats), otherwise blocks of sixteen (and a rest)
   through the small-batch kernels: plain, with the residual in place and with the norm in front (tga_rmsnorm_qlinear_rows), against the C restatement run in
@@ -569,7 +570,7 @@ def test_argument_errors(gpu):
   with pytest.raises(RuntimeError, match="exceed one launch"):
     gpu.check(L.tga_qlinear_experts_routed_rows(2, w.ptr, w.ptr, 8, f.ptr, 40000, 2, 1, 0, 1.0, f.ptr, f.ptr, f.ptr, f.ptr, 1, 4, 64, None))
 
-@pytest.mark.parametrize("t,k", [(2, 4096), (2, 14336), (8, 4096), (14, 4096), (39, 2048), (1, 2048), (12, 4096), (13, 2048), (3, 2048), (6, 4096), (7, 1024), (23, 4096), (23, 14336)])
+@pytest.mark.parametrize("t,k", [(2, 4096), (2, 14336), (8, 4096), (14, 4096), (39, 2048), (1, 2048), (12, 4096), (13, 2048), (3, 2048), (6, 4096), (7, 1024), (23, 4096), (23, 14336), (18, 4096), (21, 2048), (22, 14336), (41, 2048)])
 def test_staged_activations_equal_plain_path(gpu, t, k):
   """tga_stage_activation + TGA_F16_STAGED gives the plain path's result (same products; only the order the per-block offset
   correction is summed in differs), and a SwiGLU output staged for a consumer feeds that consumer correctly."""
@@ -604,8 +605,8 @@ def test_swiglu_output_staged_for_the_down_projection(gpu):
   qlinear_multi([dn], act_s, [y_s], x_staged=True)
   assert ol.rel_err(y_s.numpy(), y_n.numpy()) <= 1e-5
 
-@pytest.mark.parametrize("t,k", [(2, 2048), (8, 512), (14, 1024), (39, 2048), (1, 2048), (2, 8192), (12, 4096), (13, 1024), (3, 1024), (6, 2048), (7, 4096), (23, 4096)],
-                         ids=["q4_0", "q8_0", "q6_k", "mxfp4", "f16", "q4_0-k8192", "q4_k", "q5_k", "q4_1", "q5_0", "q5_1", "iq4_xs"])
+@pytest.mark.parametrize("t,k", [(2, 2048), (8, 512), (14, 1024), (39, 2048), (1, 2048), (2, 8192), (12, 4096), (13, 1024), (3, 1024), (6, 2048), (7, 4096), (23, 4096), (18, 4096), (21, 1024), (22, 2048), (41, 4096)],
+                         ids=["q4_0", "q8_0", "q6_k", "mxfp4", "f16", "q4_0-k8192", "q4_k", "q5_k", "q4_1", "q5_0", "q5_1", "iq4_xs", "iq3_xxs", "iq3_s", "iq2_s", "q1_0"])
 def test_rmsnorm_folded_into_the_linear(gpu, t, k):
   """tga_rmsnorm_qlinear_multi against tga_rmsnorm followed by tga_qlinear_multi (same fp16 activation up to the summation order of
   the mean square) and against the float64 anchor on the fp16-rounded normalised row."""

@@ -37,11 +37,11 @@ def _time_launches(fn, n_variants: int, iters: int, stream: rt.Stream) -> float:
   return e0.elapsed_ms(e1) * 1e3 / iters
 
 def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
-  nel, nby = rt.GGML_QUANT[ggml_type]
+  nel, nby = rt.GGML_QUANT.get(ggml_type, (1, 2))                      # (fp16 rows otherwise)
   wbytes = n * (k // nel) * nby
   copies = max(2, -(-int(1.25 * MALL_BYTES) // wbytes))
   big = Buffer((copies * wbytes,), np.uint8)
-  if ggml_type in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1, rt.IQ4_XS):                                       # no device-side writer for these: seeded host blocks, one upload per copy
+  if ggml_type in (rt.Q4_K, rt.Q5_K, rt.Q4_1, rt.Q5_0, rt.Q5_1, rt.IQ4_XS, rt.IQ3_XXS, rt.IQ3_S, rt.IQ2_S, rt.Q1_0):       # no device-side writer for these: seeded host blocks, one upload per copy
     from tinygrad_amd import synth
     host = synth.random_blocks(np.random.default_rng(1002), ggml_type, n, k)
     for c in range(copies): big.view(c * wbytes, (wbytes,), np.uint8).copyin(host)
@@ -54,7 +54,8 @@ def gemv_case(ggml_type: int, n: int, k: int, m: int, iters: int = 200) -> dict:
   s = rt.Stream()
   us = _time_launches(lambda i: lins[i](x, out=y, stream=s.handle), copies, iters, s)
   alg = wbytes + m * k * 2 + m * n * 2
-  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_1: "Q4_1", rt.Q5_0: "Q5_0", rt.Q5_1: "Q5_1", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.IQ4_XS: "IQ4_XS", rt.MXFP4: "MXFP4", rt.F16: "F16"}[ggml_type]
+  name = {rt.Q4_0: "Q4_0", rt.Q8_0: "Q8_0", rt.Q4_1: "Q4_1", rt.Q5_0: "Q5_0", rt.Q5_1: "Q5_1", rt.Q4_K: "Q4_K", rt.Q5_K: "Q5_K", rt.Q6_K: "Q6_K", rt.IQ4_XS: "IQ4_XS", rt.MXFP4: "MXFP4", rt.F16: "F16",
+          rt.IQ3_XXS: "IQ3_XXS", rt.IQ3_S: "IQ3_S", rt.IQ2_S: "IQ2_S", rt.Q1_0: "Q1_0"}[ggml_type]
   return {"case": f"{name} {n}x{k} M={m}", "avg_us": round(us, 2), "alg_bytes": alg, "GBps": round(alg / us / 1e3, 1),
           "frac_hbm_peak": round(alg / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_rotated": copies, "launches": iters}
 
@@ -74,6 +75,15 @@ def kquants():
     for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
       for m in ((1, 4, 8, 16) if t in (rt.Q4_K, rt.Q5_K) else (1, 8)): out.append(dict(config="k-quants", **gemv_case(t, n, k, m, iters=200)))
   for m in (1, 4, 8, 16): out.append(dict(config="k-quants", **gemv_case(rt.Q6_K, 4096, 14336, m, iters=200)))
+  return out
+
+def codebooks():
+  """IQ3_XXS / IQ3_S / IQ2_S / Q1_0 read in place at the Llama-3-8B linear shapes, M in {1, 8}, beside the fp16 matrix of the same shape (what a load-time expansion would stream)."""
+  out = []
+  for n, k in ((4096, 4096), (14336, 4096), (4096, 14336)):
+    out.append(dict(config="codebooks", **gemv_case(rt.F16, n, k, 1, iters=200)))
+    for t in (rt.IQ3_XXS, rt.IQ3_S, rt.IQ2_S, rt.Q1_0):
+      for m in (1, 8): out.append(dict(config="codebooks", **gemv_case(t, n, k, m, iters=200)))
   return out
 
 def config7(steps: int = 64, ctx: int = 1024, use_graph: bool = True):
@@ -306,7 +316,7 @@ def prefill_trace(chunk: int = 64):
 
 def main():
   ap = argparse.ArgumentParser()
-  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix; 8 = 8B chunked prefill and batched dense decode")
+  ap.add_argument("--config", type=int, nargs="*", default=[1, 2, 4, 5], help="1, 2, 4, 5 = the benchmark's configurations; 6 = Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 / IQ4_XS GEMV shapes; 9 = IQ3_XXS / IQ3_S / IQ2_S / Q1_0 GEMV shapes; 7 = 8B decode with the Q4_K_M type mix; 8 = 8B chunked prefill and batched dense decode")
   ap.add_argument("--no-graph", action="store_true", help="configs 4 and 7: launch eagerly instead of replaying a captured graph (for profilers)")
   ap.add_argument("--traffic", action="store_true", help="only the workload of the HBM-traffic counter runs (see traffic())")
   ap.add_argument("--prefill", type=int, default=0, metavar="CHUNK", help="only the workload of the prefill kernel trace, CHUNK positions per step (see prefill_trace())")
@@ -320,7 +330,7 @@ def main():
     for row in prefill_trace(args.prefill): print(json.dumps(row), flush=True)
     return
   for cfg in args.config:
-    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7, 8: config8}[cfg]
+    fn = {1: config1, 2: config2, 4: config4, 5: config5, 6: kquants, 7: config7, 8: config8, 9: codebooks}[cfg]
     for row in (fn(use_graph=not args.no_graph) if cfg in (4, 7) else fn()): print(json.dumps(row), flush=True)
 
 if __name__ == "__main__":

@@ -158,7 +158,7 @@ static int launch_qexperts(ExpArgs a, int n_experts, int n_jobs, int xdiv_hint, 
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const size_t lds = (size_t)EXP_MAX_ROWS * F::XV * a.nu * 16;
-  TGA_REQUIRE(lds <= 144 * 1024, "tga_qlinear_experts_grouped: K=%d does not fit the activation staging (%zu bytes of LDS)", a.K, lds);
+  TGA_REQUIRE(lds <= 144 * 1024 - fmt_tab<F>(), "tga_qlinear_experts_grouped: K=%d does not fit the activation staging (%zu bytes of LDS)", a.K, lds);
   const long long ngroups = (a.N + 15) / 16;
   // About two workgroups per CU over the experts that have jobs.  How many do is only known on the device; the launch is sized for the number
   // expected when the tokens pick independently (n_jobs = B k jobs over E experts, each token k distinct ones): E (1 - (1 - k / E)^B) with
@@ -173,7 +173,7 @@ static int launch_qexperts(ExpArgs a, int n_experts, int n_jobs, int xdiv_hint, 
   if (gx < 1) gx = 1;
   auto kern = qexperts_mfma_kernel<T, TWO>;
   if (lds > 48 * 1024) {
-    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);   // once per instantiation, thread-safe
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024 - fmt_tab<F>());   // once per instantiation, thread-safe
     TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)gx, (unsigned)n_experts), dim3(EXP_THREADS), lds, s>>>(a);
@@ -207,12 +207,15 @@ int tga_qlinear_experts_grouped(int ggml_type, const void* w, const void* w_up, 
     case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_Q4_K: bw = 256; bb = 144; break; case GGML_Q5_K: bw = 256; bb = 176; break;
     case GGML_F16: bw = 64; bb = 128; break;
     case GGML_Q4_1: bw = 64; bb = 40; break; case GGML_Q5_0: bw = 64; bb = 44; break; case GGML_Q5_1: bw = 64; bb = 48; break;
+    case GGML_IQ4_XS: bw = 256; bb = 136; break; case GGML_IQ3_XXS: bw = 256; bb = 98; break; case GGML_IQ3_S: bw = 256; bb = 110; break; case GGML_IQ2_S: bw = 256; bb = 82; break;
+    case GGML_Q1_0: bw = 128; bb = 18; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   TGA_REQUIRE(K > 0 && K % bw == 0 && N > 0, "tga_qlinear_experts_grouped: K=%lld must be a positive multiple of %d", (long long)K, bw);
   ExpArgs a = {};
   a.w = (const uint8_t*)w; a.w_up = (const uint8_t*)w_up; a.estride = (long long)N * (K / bw) * bb; a.table = table;
   a.x = (const uint16_t*)x_f16; a.xdiv = jobs_per_x_row; a.y = y; a.y_f32 = y_dtype == TGA_F32; a.N = N; a.K = (int)K;
-  TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0 && a.estride % 4 == 0), "tga_qlinear_experts_grouped: expert weights must be 4-byte aligned");
+  const bool align2 = ggml_type == GGML_IQ3_XXS || ggml_type == GGML_IQ3_S || ggml_type == GGML_IQ2_S || ggml_type == GGML_Q1_0;      // (blocks of 98 / 110 / 82 / 18 bytes, read with 2-byte aligned loads)
+  TGA_REQUIRE(ggml_type == GGML_MXFP4 || ((((uintptr_t)w | (uintptr_t)w_up) & (align2 ? 1 : 3)) == 0 && a.estride % (align2 ? 2 : 4) == 0), "tga_qlinear_experts_grouped: expert weights must be 4-byte aligned (2-byte for IQ3 / IQ2 / Q1_0)");
   hipStream_t s = (hipStream_t)stream;
   const int E = (int)n_experts;
   const int k_hint = jobs_per_x_row > 1 ? jobs_per_x_row : 8;       // the down launch has one job per activation row: assume eight experts per token
@@ -227,6 +230,11 @@ int tga_qlinear_experts_grouped(int ggml_type, const void* w, const void* w_up, 
     case GGML_Q5_0: return launch_qexperts_t<GGML_Q5_0>(a, E, n_jobs, k_hint, s);
     case GGML_Q5_1: return launch_qexperts_t<GGML_Q5_1>(a, E, n_jobs, k_hint, s);
     case GGML_F16: return launch_qexperts_t<GGML_F16>(a, E, n_jobs, k_hint, s);
+    case GGML_IQ4_XS: return launch_qexperts_t<GGML_IQ4_XS>(a, E, n_jobs, k_hint, s);
+    case GGML_IQ3_XXS: return launch_qexperts_t<GGML_IQ3_XXS>(a, E, n_jobs, k_hint, s);
+    case GGML_IQ3_S: return launch_qexperts_t<GGML_IQ3_S>(a, E, n_jobs, k_hint, s);
+    case GGML_IQ2_S: return launch_qexperts_t<GGML_IQ2_S>(a, E, n_jobs, k_hint, s);
+    case GGML_Q1_0: return launch_qexperts_t<GGML_Q1_0>(a, E, n_jobs, k_hint, s);
   }
   return tga_set_error("tga_qlinear_experts_grouped: no kernel for type %d", ggml_type);
 }

@@ -13,6 +13,17 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // ggml type ids (tinygrad/llm/gguf.py:20-21 keys)
 enum { GGML_F32 = 0, GGML_F16 = 1, GGML_Q4_0 = 2, GGML_Q4_1 = 3, GGML_Q5_0 = 6, GGML_Q5_1 = 7, GGML_Q8_0 = 8, GGML_Q4_K = 12, GGML_Q5_K = 13, GGML_Q6_K = 14, GGML_IQ3_XXS = 18, GGML_IQ3_S = 21, GGML_IQ2_S = 22, GGML_IQ4_XS = 23, GGML_MXFP4 = 39, GGML_Q1_0 = 41 };
 
+// weights per block of a ggml block type (the (elements, bytes) table of tinygrad/llm/gguf.py:20-21); 0: not a block type
+static inline int tga_block_weights(int t) {
+  switch (t) {
+    case GGML_Q4_0: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: case GGML_Q8_0: case GGML_MXFP4: return 32;
+    case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: case GGML_IQ4_XS: return 256;
+    case GGML_Q1_0: return 128;
+    case GGML_F16: case GGML_F32: return 1;
+  }
+  return 0;
+}
+
 __device__ __forceinline__ half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
 __device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
 __device__ __forceinline__ float h2f_bits(uint32_t h16) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h16); }

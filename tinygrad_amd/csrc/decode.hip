@@ -41,6 +41,10 @@ __global__ __launch_bounds__(256) void embed_row_kernel(const uint8_t* __restric
     case GGML_Q5_1: embed_row_blocks<GGML_Q5_1>(table, dim, tok, out); break;
     case GGML_Q6_K: embed_row_blocks<GGML_Q6_K>(table, dim, tok, out); break;
     case GGML_IQ4_XS: embed_row_blocks<GGML_IQ4_XS>(table, dim, tok, out); break;
+    case GGML_IQ3_XXS: embed_row_blocks<GGML_IQ3_XXS>(table, dim, tok, out); break;
+    case GGML_IQ3_S: embed_row_blocks<GGML_IQ3_S>(table, dim, tok, out); break;
+    case GGML_IQ2_S: embed_row_blocks<GGML_IQ2_S>(table, dim, tok, out); break;
+    case GGML_Q1_0: embed_row_blocks<GGML_Q1_0>(table, dim, tok, out); break;
     case GGML_MXFP4: embed_row_blocks<GGML_MXFP4>(table, dim, tok, out); break;
     case GGML_F16: { const uint16_t* row = (const uint16_t*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = h2f_bits(row[e]); break; }
     default: { const float* row = (const float*)table + (size_t)tok * dim; for (int e = threadIdx.x; e < dim; e += 256) out[e] = (float)(_Float16)row[e]; }
@@ -876,8 +880,8 @@ extern "C" {
 int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, float* out, void* stream) {
   TGA_REQUIRE(table && state && out, "tga_embed_row: null pointer");
   int blk = 0;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: case GGML_IQ4_XS: blk = 256; break;
-    case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_row: unsupported table type %d", ggml_type); }
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: case GGML_IQ4_XS: case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: blk = 256; break;
+    case GGML_Q1_0: blk = 128; break; case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_row: unsupported table type %d", ggml_type); }
   TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_row: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
   embed_row_kernel<<<1, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out, nullptr);
   TGA_LAUNCH_CHECK();
@@ -887,8 +891,8 @@ int tga_embed_row(const void* table, int ggml_type, int dim, const void* state, 
 int tga_embed_rows(const void* table, int ggml_type, int dim, const int32_t* tokens, int n_rows, void* state, float* out, void* stream) {
   TGA_REQUIRE(table && state && out && tokens && n_rows >= 1, "tga_embed_rows: null pointer or no rows");
   int blk = 0;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: case GGML_IQ4_XS: blk = 256; break;
-    case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_rows: unsupported table type %d", ggml_type); }
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: blk = 32; break; case GGML_Q4_K: case GGML_Q5_K: case GGML_Q6_K: case GGML_IQ4_XS: case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: blk = 256; break;
+    case GGML_Q1_0: blk = 128; break; case GGML_F16: case GGML_F32: blk = 1; break; default: return tga_set_error("tga_embed_rows: unsupported table type %d", ggml_type); }
   TGA_REQUIRE(dim > 0 && dim % blk == 0 && dim % 4 == 0, "tga_embed_rows: dim=%d must be a positive multiple of 4 and of the table's block size %d", dim, blk);
   embed_row_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>((const uint8_t*)table, ggml_type, dim, (DecodeState*)state, out, tokens);
   TGA_LAUNCH_CHECK();
@@ -902,9 +906,10 @@ static int decode_staged_fmt(int ggml_type, long long K, int* nu) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
     case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
     case GGML_Q4_1: fmt = GGML_Q4_1; break; case GGML_Q5_0: fmt = GGML_Q5_0; break; case GGML_Q5_1: fmt = GGML_Q5_1; break; case GGML_IQ4_XS: fmt = GGML_IQ4_XS; break;
+    case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: case GGML_Q1_0: fmt = ggml_type; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
-  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_IQ4_XS) ? 256 : 64) != 0) return -1;
+  if (fmt < 0 || K <= 0 || K % tga_block_weights(ggml_type) != 0 || K % 64 != 0) return -1;
   *nu = (int)(K / uw);
   return fmt;
 }

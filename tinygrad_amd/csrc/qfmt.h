@@ -57,6 +57,10 @@ __device__ __forceinline__ uint32_t pack_even(uint32_t a, uint32_t b) { return (
 __device__ __forceinline__ uint32_t pack_odd(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xFFFF0000u); }     // (a.hi, b.hi)
 
 template <int T> struct Fmt;
+// bytes of LDS that a format's lookup tables take in every workgroup (the codebook types, qfmt_cb.h); 0 for the others
+template <class F, class = void> struct FmtTab { static constexpr int value = 0; };
+template <class F> struct FmtTab<F, decltype((void)F::TAB)> { static constexpr int value = F::TAB; };
+template <class F> constexpr int fmt_tab() { return FmtTab<F>::value; }
 
 // Decoded weights still carry their exponent-bias and integer offsets (1024 + q etc.) and no block scale.  to_f16 turns a decoded
 // unit into the true weights as fp16 pairs, (pattern - bias) * scale: the subtraction is exact in fp16 (small integers), the
@@ -810,6 +814,8 @@ template <> struct Fmt<GGML_Q4_1> : FmtL<0> {};
 template <> struct Fmt<GGML_Q5_0> : FmtL<1> {};
 template <> struct Fmt<GGML_Q5_1> : FmtL<2> {};
 
+#include "qfmt_cb.h"     // IQ3_XXS, IQ3_S, IQ2_S, Q1_0: codebooks and sign patterns in LDS
+
 // unit_dot with the unit's activations already in registers (M = 1)
 template <int T>
 __device__ __forceinline__ void unit_dot_reg(const typename Fmt<T>::Raw& raw, const u32x4* xv, const float* cv, float& acc, const uint32_t* kc) {
@@ -882,6 +888,7 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
     case GGML_Q5_0: return Fmt<GGML_Q5_0>::spos(e, nu);
     case GGML_Q5_1: return Fmt<GGML_Q5_1>::spos(e, nu);
     case GGML_IQ4_XS: return Fmt<GGML_IQ4_XS>::spos(e, nu);
+    case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: case GGML_Q1_0: return FmtCbBase::spos(e, nu);
     case GGML_MXFP4: return Fmt<GGML_MXFP4>::spos(e, nu);
     case GGML_F16: return Fmt<GGML_F16>::spos(e, nu);
   }

@@ -228,13 +228,13 @@ static int launch_qgemm(QArgs a, hipStream_t s) {
   const long long ngroups = (a.ntot + 15) / 16;
   const int cus = qm_cu_count();
   // LDS budget for one chunk of activations: two workgroups per CU, or the whole CU when there is at most one row group per CU anyway
-  const int budget = ngroups <= cus ? 2 * QM_LDS_BUDGET : QM_LDS_BUDGET;
+  const int budget = (ngroups <= cus ? 2 * QM_LDS_BUDGET : QM_LDS_BUDGET) - fmt_tab<F>();
   int cu = budget / per_unit; cu -= cu % 16; if (cu < 16) cu = 16;
   if (cu >= a.nu) { a.chunk_u = a.nu; a.nchunks = 1; } else { a.nchunks = (a.nu + cu - 1) / cu; a.chunk_u = ((a.nu + a.nchunks - 1) / a.nchunks + 15) / 16 * 16; }
   const size_t lds = (size_t)per_unit * a.chunk_u;
   // single chunk: the activations are staged once per workgroup, so no more workgroups than stay resident (by LDS, at most 8 per
   // CU); chunked K: every row group restages each chunk, one group per workgroup
-  int resident = (int)(QM_LDS_CU / (lds + 6 * 1024)); resident = resident < 1 ? 1 : resident > 8 ? 8 : resident;
+  int resident = (int)(QM_LDS_CU / (lds + 6 * 1024 + fmt_tab<F>())); resident = resident < 1 ? 1 : resident > 8 ? 8 : resident;
   long long grid = ngroups;
   const long long cap = (long long)cus * (a.nchunks == 1 ? resident : 8);
   if (grid > cap) grid = cap;
@@ -271,6 +271,10 @@ int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
     case GGML_Q5_0: return launch_qgemm_m<GGML_Q5_0>(a, M, s);
     case GGML_Q5_1: return launch_qgemm_m<GGML_Q5_1>(a, M, s);
     case GGML_IQ4_XS: return launch_qgemm_m<GGML_IQ4_XS>(a, M, s);
+    case GGML_IQ3_XXS: return launch_qgemm_m<GGML_IQ3_XXS>(a, M, s);
+    case GGML_IQ3_S: return launch_qgemm_m<GGML_IQ3_S>(a, M, s);
+    case GGML_IQ2_S: return launch_qgemm_m<GGML_IQ2_S>(a, M, s);
+    case GGML_Q1_0: return launch_qgemm_m<GGML_Q1_0>(a, M, s);
     case GGML_F16: return launch_qgemm_m<GGML_F16>(a, M, s);
     case GGML_MXFP4: return launch_qgemm_m<GGML_MXFP4>(a, M, s);
   }

@@ -261,7 +261,8 @@ static int launch_qgemv(QArgs a, hipStream_t s) {
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const long long ngroups = (a.epilogue == 2) ? a.ntot : (a.ntot + R - 1) / R;
   long long grid; size_t lds;
-  if ((long long)per_unit * a.nu <= QG_LDS_BUDGET) {
+  constexpr int BUDGET = QG_LDS_BUDGET - fmt_tab<F>();      // (a format's tables share the CU's LDS with the staged activations)
+  if ((long long)per_unit * a.nu <= BUDGET) {
     a.nchunks = 1; a.chunk_u = a.nu;
     lds = (size_t)per_unit * a.nu;
     // resident workgroups per CU by LDS (160 KB), capped at 4 (16 waves); never more workgroups than row groups need
@@ -270,9 +271,9 @@ static int launch_qgemv(QArgs a, hipStream_t s) {
     const long long need = (ngroups + QG_WAVES - 1) / QG_WAVES;
     if (grid > need) grid = need;
   } else {
-    int cu = QG_LDS_BUDGET / 2 / per_unit;                 // two workgroups per CU
+    int cu = (QG_LDS_BUDGET / 2 - fmt_tab<F>()) / per_unit;   // two workgroups per CU
     cu -= cu % 64; if (cu < 64) cu = 64;                   // whole waves of units (64 is a multiple of every format's units per block)
-    TGA_REQUIRE((long long)cu * per_unit <= QG_LDS_BUDGET, "tga_qlinear: activations of one K chunk do not fit LDS");
+    TGA_REQUIRE((long long)cu * per_unit <= BUDGET, "tga_qlinear: activations of one K chunk do not fit LDS");
     a.chunk_u = cu; a.nchunks = (a.nu + cu - 1) / cu;
     lds = (size_t)per_unit * cu;
     grid = (ngroups + QG_WAVES - 1) / QG_WAVES;
@@ -280,7 +281,7 @@ static int launch_qgemv(QArgs a, hipStream_t s) {
   if (grid < 1) grid = 1;
   auto kern = qgemv_kernel<T, M, R>;
   if (lds > 48 * 1024) {
-    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, QG_LDS_BUDGET);   // once per instantiation, thread-safe
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, BUDGET);   // once per instantiation, thread-safe
     TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)grid), dim3(QG_THREADS), lds, s>>>(a);
@@ -293,7 +294,7 @@ static int launch_qgemv_r(const QArgs& a, hipStream_t s) {
   // SwiGLU pairs gate/up rows: exactly two rows per group.  Otherwise two rows per wave step as well (more loads in flight
   // per lane); a single row per group when there are too few rows to fill the chip.
   if (a.epilogue == 2) return launch_qgemv<T, M, 2>(a, s);
-  const bool chunked = (long long)M * (16 * Fmt<T>::XV + 4 * Fmt<T>::NG) * (a.K / Fmt<T>::UW) > QG_LDS_BUDGET;
+  const bool chunked = (long long)M * (16 * Fmt<T>::XV + 4 * Fmt<T>::NG) * (a.K / Fmt<T>::UW) > QG_LDS_BUDGET - fmt_tab<Fmt<T>>();
   // (chunked K with several segments needs one row per group: a group must not straddle a segment)
   if ((chunked && a.nseg > 1) || a.ntot < (long long)cu_count() * QG_WAVES * 2) return launch_qgemv<T, M, 1>(a, s);
   return launch_qgemv<T, M, 2>(a, s);
@@ -331,9 +332,10 @@ static int staged_fmt(int ggml_type, long long K, int* nu) {
     case GGML_Q4_0: fmt = F_Q4_0P; break; case GGML_Q8_0: fmt = F_Q8_0P; break; case GGML_Q6_K: fmt = GGML_Q6_K; break;
     case GGML_Q4_K: fmt = GGML_Q4_K; break; case GGML_Q5_K: fmt = GGML_Q5_K; break;
     case GGML_Q4_1: fmt = GGML_Q4_1; break; case GGML_Q5_0: fmt = GGML_Q5_0; break; case GGML_Q5_1: fmt = GGML_Q5_1; break; case GGML_IQ4_XS: fmt = GGML_IQ4_XS; break;
+    case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: case GGML_Q1_0: fmt = ggml_type; break;
     case GGML_F16: fmt = GGML_F16; break; case GGML_MXFP4: fmt = GGML_MXFP4; uw = 32; break;
   }
-  if (fmt < 0 || K <= 0 || K % ((ggml_type == GGML_Q6_K || ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_IQ4_XS) ? 256 : 64) != 0) return -1;
+  if (fmt < 0 || K <= 0 || K % tga_block_weights(ggml_type) != 0 || K % 64 != 0) return -1;
   *nu = (int)(K / uw);
   return fmt;
 }
@@ -441,8 +443,9 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
   TGA_REQUIRE(epilogue != 1 || (y_dtype == TGA_F32 && resid), "tga_qlinear: the residual epilogue needs float32 y and resid pointers");
   TGA_REQUIRE(epilogue != 2 || (nseg == 2 && n[0] == n[1]), "tga_qlinear: the SwiGLU epilogue needs two segments of equal rows");
   int bw;
-  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: bw = 256; break; case GGML_F16: bw = 64; break;
+  switch (ggml_type) { case GGML_Q4_0: case GGML_Q8_0: case GGML_MXFP4: bw = 32; break; case GGML_Q6_K: case GGML_Q4_K: case GGML_Q5_K: case GGML_IQ4_XS: case GGML_IQ3_XXS: case GGML_IQ3_S: case GGML_IQ2_S: bw = 256; break; case GGML_F16: bw = 64; break;
     case GGML_Q4_1: case GGML_Q5_0: case GGML_Q5_1: bw = 64; break;      // served as block pairs
+    case GGML_Q1_0: bw = 128; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   const bool align4 = ggml_type == GGML_Q4_K || ggml_type == GGML_Q5_K || ggml_type == GGML_Q4_1 || ggml_type == GGML_Q5_0 || ggml_type == GGML_Q5_1 || ggml_type == GGML_IQ4_XS;
   TGA_REQUIRE(K > 0 && K % bw == 0 && K <= (1 << 24), "tga_qlinear: K=%lld must be a positive multiple of %d", (long long)K, bw);
@@ -537,6 +540,10 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     case GGML_Q5_0: return launch_qgemv_m<GGML_Q5_0>(a, M, s);
     case GGML_Q5_1: return launch_qgemv_m<GGML_Q5_1>(a, M, s);
     case GGML_IQ4_XS: return launch_qgemv_m<GGML_IQ4_XS>(a, M, s);
+    case GGML_IQ3_XXS: return launch_qgemv_m<GGML_IQ3_XXS>(a, M, s);
+    case GGML_IQ3_S: return launch_qgemv_m<GGML_IQ3_S>(a, M, s);
+    case GGML_IQ2_S: return launch_qgemv_m<GGML_IQ2_S>(a, M, s);
+    case GGML_Q1_0: return launch_qgemv_m<GGML_Q1_0>(a, M, s);
     case GGML_MXFP4: return launch_qgemv_m<GGML_MXFP4>(a, M, s);
     case GGML_F16: return launch_qgemv_m<GGML_F16>(a, M, s);
   }
@@ -727,10 +734,12 @@ static int qlinear_experts_impl(const RouteIn* route, int ggml_type, const void*
     case GGML_Q6_K: bw = 256; bb = 210; break; case GGML_Q4_K: bw = 256; bb = 144; break; case GGML_Q5_K: bw = 256; bb = 176; break;
     case GGML_F16: bw = 64; bb = 128; break;
     case GGML_Q4_1: bw = 64; bb = 40; break; case GGML_Q5_0: bw = 64; bb = 44; break; case GGML_Q5_1: bw = 64; bb = 48; break;   // block pairs
+    case GGML_IQ4_XS: bw = 256; bb = 136; break; case GGML_IQ3_XXS: bw = 256; bb = 98; break; case GGML_IQ3_S: bw = 256; bb = 110; break; case GGML_IQ2_S: bw = 256; bb = 82; break;
+    case GGML_Q1_0: bw = 128; bb = 18; break;
     default: return tga_set_error("GGML type '%d' is not supported!", ggml_type); }
   TGA_REQUIRE(K > 0 && K % bw == 0 && N > 0, "tga_qlinear_experts: K=%lld must be a positive multiple of %d", (long long)K, bw);
-  TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q4_1 && ggml_type != GGML_Q5_0 && ggml_type != GGML_Q5_1) || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0),
-              "tga_qlinear_experts: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 weights must be 4-byte aligned");
+  TGA_REQUIRE((ggml_type != GGML_Q4_K && ggml_type != GGML_Q5_K && ggml_type != GGML_Q4_1 && ggml_type != GGML_Q5_0 && ggml_type != GGML_Q5_1 && ggml_type != GGML_IQ4_XS) || ((((uintptr_t)w | (uintptr_t)w_up) & 3) == 0),
+              "tga_qlinear_experts: Q4_K / Q5_K / Q4_1 / Q5_0 / Q5_1 / IQ4_XS weights must be 4-byte aligned");
   QArgs a = {};
   a.nseg = w_up ? 2 : 1; a.x = x; a.x_f32 = x_dtype == TGA_F32; a.y_f32 = y_dtype == TGA_F32; a.epilogue = w_up ? 2 : 0; a.K = (int)K;
   a.w[0] = (const uint8_t*)w; a.w[1] = (const uint8_t*)w_up; a.y[0] = y; a.n[0] = N; a.n[1] = N; a.ntot = N;

@@ -525,7 +525,7 @@ static int launch_fast_p(const QArgs& a, long long grid, size_t lds, hipStream_t
   auto kern = qgemv1_kernel<T, R, WK, WR, EPI, H, PRO, MR>;
   if (lds > 48 * 1024) {
     // once per instantiation; the initialisation of a function-local static is serialised by the language, so concurrent first calls are safe
-    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    static const hipError_t configured = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024 - fmt_tab<Fmt<T>>());
     TGA_HIP(configured);
   }
   kern<<<dim3((unsigned)grid, (unsigned)(a.sel ? a.xdiv_jobs : 1)), dim3(WK * WR * 64), lds, s>>>(a);
@@ -543,7 +543,7 @@ static int launch_fast(QArgs a, hipStream_t s) {
   // row teams per CU: 8 waves (one 8-wave workgroup or two 4-wave ones), fewer when the staged activations in LDS (160 KB per CU) say so.
   // Measured on the 8B decode step: 8 or 12 waves per CU 570 tok/s, 16 (all wave slots) 564, 4 553.
   int wg_per_cu = (a.sel ? 16 : 8) / (WK * WR); if (wg_per_cu < 1) wg_per_cu = 1;   // (expert jobs share the grid: all 16 wave slots there)
-  const int by_lds = (int)((160 * 1024) / (lds + 1024)); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
+  const int by_lds = (int)((160 * 1024) / (lds + 1024 + fmt_tab<F>())); if (wg_per_cu > by_lds) wg_per_cu = by_lds < 1 ? 1 : by_lds;
   constexpr int TPW = WR * (H ? 2 : 1);                           // row teams per workgroup
   long long max_teams = (long long)fast_cu_count() * wg_per_cu * TPW;
   if (a.sel && a.xdiv_jobs > 1) { max_teams = (max_teams + a.xdiv_jobs - 1) / a.xdiv_jobs; if (max_teams < 1) max_teams = 1; }

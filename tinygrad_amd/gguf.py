@@ -7,7 +7,7 @@ Unknown types raise ValueError with the reference's message (gguf.py:119)."""
 from __future__ import annotations
 import numpy as np
 from tinygrad_amd import runtime as rt
-from tinygrad_amd.runtime import Buffer, GGML_QUANT, GGML_DEQUANT_ONLY
+from tinygrad_amd.runtime import Buffer, GGML_QUANT
 
 def _as_device_bytes(t) -> Buffer:
   if isinstance(t, Buffer): return t
@@ -20,8 +20,8 @@ def ggml_data_to_tensor(t, n: int, ggml_type: int, out_dtype=np.float32, stream=
   if ggml_type in _NATIVE_NUMPY:                              # int8 / int16 / int32 / int64 / float64 / bfloat16: the same bytes under their own type (gguf.py:35-36)
     dt = _NATIVE_NUMPY[ggml_type]
     return t.view(0, (n,), dt)                                # bfloat16 (30) has no numpy type: its bit patterns come back as uint16
-  if ggml_type not in GGML_QUANT and ggml_type not in GGML_DEQUANT_ONLY: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
-  nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]
+  if ggml_type not in GGML_QUANT: raise ValueError(f"GGML type '{ggml_type}' is not supported!")
+  nel, nby = GGML_QUANT[ggml_type]
   nfull = (n // nel) * nel                                   # gguf.py:45 uses whole blocks only
   if t.nbytes < (nfull // nel) * nby: raise ValueError(f"buffer of {t.nbytes} bytes holds fewer than {nfull // nel} blocks")
   out = Buffer((nfull,), out_dtype)
@@ -59,7 +59,7 @@ class GGUFTensor:
 
 def tensor_nbytes(ggml_type: int, n: int) -> int:
   if ggml_type in _NATIVE_ITEMSIZE: return _NATIVE_ITEMSIZE[ggml_type] * n
-  if ggml_type in GGML_QUANT or ggml_type in GGML_DEQUANT_ONLY: nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]; return (n // nel) * nby
+  if ggml_type in GGML_QUANT: nel, nby = GGML_QUANT[ggml_type]; return (n // nel) * nby
   raise ValueError(f"GGML type '{ggml_type}' is not supported!")
 
 def gguf_parse(raw: np.ndarray) -> tuple[dict, dict[str, GGUFTensor]]:

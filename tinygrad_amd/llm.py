@@ -75,6 +75,12 @@ def rope_table(head_dim: int, rope_dim: int, end: int, theta: float) -> np.ndarr
   rh, rest = rope_dim // 2, (head_dim - rope_dim) // 2
   return np.concatenate([fc[:, :rh], np.ones((end, rest), np.float32), fc[:, rh:], np.zeros((end, rest), np.float32)], axis=-1)
 
+def fast_k(ggml_type: int, k: int) -> bool:
+  """Rows of k values of this type are inside the range of the single-row kernel that keeps the activations in registers: whole blocks, whole units of 64,
+  at most 65536 values (32768 for the types whose lookup tables share the LDS with the row)."""
+  nel = GGML_QUANT.get(ggml_type, (64, 128))[0]
+  return k % 64 == 0 and k % nel == 0 and k <= (32768 if ggml_type in (rt.IQ3_XXS, rt.IQ3_S, rt.IQ2_S, rt.Q1_0) else 65536)
+
 def quant_nbytes(ggml_type: int, n: int) -> int:
   if ggml_type == rt.F32: return 4 * n
   if ggml_type == rt.F16: return 2 * n
@@ -199,7 +205,7 @@ class TransformerBlock:
     self.cache_v = Buffer((c.n_kv_heads, c.max_context, c.head_dim), np.float16).zero_()
     self.config, self.s = c, shared
     # the M = 1 GEMV's register-resident fast path: K % 64 (superblock types: % 256), 4-byte aligned weights
-    fast = lambda l: l.in_features % 64 == 0 and l.in_features <= 65536 and l.blocks.ptr % 4 == 0 and (l.ggml_type not in (rt.Q4_K, rt.Q5_K, rt.Q6_K, rt.IQ4_XS) or l.in_features % 256 == 0)
+    fast = lambda l: fast_k(l.ggml_type, l.in_features) and l.blocks.ptr % 4 == 0
     # RMSNorm folded into the consuming linear
     self.fuse_norm = all(fast(l) for l in (self.attn_q, self.attn_k, self.attn_v)) and (self.moe or all(fast(l) for l in (self.ffn_gate, self.ffn_up)))
     # a producer with a single consumer writes its fp16 output in the order that consumer's GEMV reads it (no LDS staging there):
@@ -349,7 +355,7 @@ class Transformer:
     self.output_norm = state_dict["output_norm.weight"][0]
     out = state_dict.get("output.weight", emb)                       # tied embeddings: model.py:379
     self.output = QuantLinear(out[0], out[1], *out[2])
-    self.fuse_head_norm = c.dim % (256 if out[1] in (rt.Q4_K, rt.Q5_K, rt.Q6_K, rt.IQ4_XS) else 64) == 0 and c.dim <= 65536 and out[0].ptr % 4 == 0
+    self.fuse_head_norm = fast_k(out[1], c.dim) and out[0].ptr % 4 == 0
     self.can_fold_head = self.fuse_head_norm and c.dim <= 2048 and 0 < c.n_summands <= 8
     self.stream = rt.Stream()
     self._graphs = {}
@@ -433,9 +439,6 @@ class Transformer:
         data = _to_f32(data, typ).astype(np.float16).astype(np.float32); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F32
       elif typ in GGUF_F32_LIKE:                                       # F32 / BF16 matrices -> fp16 (model.py:376)
         data = _to_f32(data, typ).astype(np.float16); buf = Buffer.from_numpy(data.view(np.uint8)); typ = rt.F16
-      elif typ in rt.GGML_DEQUANT_ONLY:                                # block types without an in-place linear kernel: the fp16 weight of model.py:376, made once
-        buf = ggml_data_to_tensor(buf, rows * cols, typ, out_dtype=np.float16); typ = rt.F16
-        data = buf.numpy()
       if arch == "llama" and (name.endswith("attn_q.weight") or name.endswith("attn_k.weight")):
         h = n_heads if name.endswith("attn_q.weight") else n_kv
         raw = np.ascontiguousarray(data).view(np.uint8).reshape(rows, -1)

@@ -12,9 +12,9 @@ IQ4_XS, Q1_0 = 23, 41
 IQ3_XXS, IQ3_S, IQ2_S = 18, 21, 22
 F16_STAGED = 101          # activation dtype code: fp16 in the staged order of the consuming weight (tga_stage_activation)
 # {ggml_type: (elements per block, bytes per block)}: tinygrad/llm/gguf.py:20-21
-# block types tga_dequant decodes but the linear kernels do not read in place: such weights are expanded to fp16 when a model is loaded
-GGML_DEQUANT_ONLY = {IQ3_XXS: (256, 98), IQ3_S: (256, 110), IQ2_S: (256, 82), Q1_0: (128, 18)}
-GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ4_XS: (256, 136), MXFP4: (32, 17)}
+# (every one of them is read in place by the linear kernels; tga_dequant expands any of them)
+GGML_QUANT = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210), IQ4_XS: (256, 136), MXFP4: (32, 17),
+              IQ3_XXS: (256, 98), IQ3_S: (256, 110), IQ2_S: (256, 82), Q1_0: (128, 18)}
 _NP_DTYPE = {F32: np.float32, F16: np.float16}
 
 _LIB_PATH = pathlib.Path(os.environ.get("TGA_LIB") or pathlib.Path(__file__).resolve().parent / "libtinygrad_amd.so")   # (TGA_LIB: another build of the same library)

@@ -14,12 +14,11 @@ def random_blocks(rng, ggml_type: int, n: int, k: int, sigma: float = 0.003, mx_
   """(n, k) weight as raw GGUF block bytes: payload bytes uniform in 0..255 (nibbles uniform 0..15), scales valid.
   Q8_0 quants avoid -128 (uniform in [-127, 127]); Q6_K sub-scales are int8 uniform in [-128, 127]; Q4_1 / Q5_1 get a valid d and m, Q5_0 a valid d; Q4_K / Q5_K get valid d and dmin, their packed 6-bit scales and mins are uniform;
   MXFP4 exponent bytes are uniform in [mx_exp[0], mx_exp[1])."""
-  from tinygrad_amd.runtime import GGML_DEQUANT_ONLY
-  nel, nby = GGML_QUANT.get(ggml_type) or GGML_DEQUANT_ONLY[ggml_type]
+  nel, nby = GGML_QUANT[ggml_type]
   assert k % nel == 0
   nb = n * (k // nel)
   b = rng.integers(0, 256, size=(nb, nby), dtype=np.uint8)
-  if ggml_type in (Q4_0, Q5_0, 18, 21, 22, 23, 41): b[:, :2] = _scales(rng, nb, sigma)   # (18 / 21 / 22 = IQ3_XXS / IQ3_S / IQ2_S, 23 = IQ4_XS, 41 = Q1_0: dequant only)
+  if ggml_type in (Q4_0, Q5_0, 18, 21, 22, 23, 41): b[:, :2] = _scales(rng, nb, sigma)   # (18 / 21 / 22 = IQ3_XXS / IQ3_S / IQ2_S, 23 = IQ4_XS, 41 = Q1_0)
   elif ggml_type in (Q4_1, Q5_1):                                       # d > 0 and a signed fp16 minimum of the same magnitude as the weights
     b[:, :2] = _scales(rng, nb, sigma)
     b[:, 2:4] = np.float16(rng.standard_normal(nb) * sigma * 4).view(np.uint8).reshape(nb, 2)
