@@ -245,6 +245,9 @@ int tga_advance_prompt(void* state, const int* prompt, void* stream);
 /* token_embd(tokens) for n_rows tokens listed in device memory (model.py:359): out (n_rows, dim) float32.  state: the decode record, only
  * for its vocab / error fields (ids outside [0, vocab) read row 0 and set error bit 0). */
 int tga_embed_rows(const void* table, int ggml_type, int dim, const int32_t* tokens, int n_rows, void* state, float* out, void* stream);
+/* out[i] = fp16(silu(gate[i]) * up[i]) over n float32 values: the feed-forward activation of tinygrad/llm/model.py:137 for a block whose ffn_gate and ffn_up are of
+ * different block types (two linear launches, then this; equal types take the SwiGLU epilogue of tga_qlinear_multi instead). */
+int tga_silu_mul(const float* gate, const float* up, int64_t n, void* out_f16, void* stream);
 /* tga_rmsnorm over `rows` rows of dim values (one workgroup per row); outputs (rows, dim). */
 int tga_rmsnorm_rows(const float* x, const float* weight, int rows, int dim, float eps, void* out_f16, float* out_f32, int stage_type, void* stream);
 /* tga_moe_combine followed by tga_rmsnorm_rows in one launch: every row of x is completed IN PLACE as x[t] + sum_s probs[t, s] * y[t, s, :] (the weighted

@@ -6,11 +6,12 @@ from oracle import ggml as og, gguf as ogguf, llm as ollm, linear as ol
 
 pytestmark = pytest.mark.gpu
 
-def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False, expand: bool = False, codebook: bool = False):
+def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False, expand: bool = False, codebook: bool = False, split_ffn: bool = False):
   """kquant: the tensor-type mix of a Q4_K_M file (Q4_K linears and embedding, Q6_K for attn_v / ffn_down / output, one Q5_K matrix).
   legacy: the same mix with Q4_1 / Q5_0 / Q5_1 in place of Q4_K / Q5_K / Q6_K.
   expand: IQ4_XS / Q1_0 / Q6_K.
-  codebook: IQ3_S / IQ2_S / IQ3_XXS.  Every one of these types stays in its blocks and is read in place."""
+  codebook: IQ3_S / IQ2_S / IQ3_XXS.  Every one of these types stays in its blocks and is read in place.
+  split_ffn: ffn_up of another block type than ffn_gate (Q6_K beside Q4_K)."""
   rng = np.random.default_rng(11)
   c = dict(dim=256, hidden=512, H=4, KV=2, hd=64, L=2, vocab=512)
   def lin(rows, cols): return (rng.uniform(-1, 1, (rows, cols)) * cols ** -0.5).astype(np.float32)
@@ -27,14 +28,14 @@ def _make_file(tmp_path, tied: bool, kquant: bool = False, legacy: bool = False,
                   mk("attn_q.weight", c["H"] * c["hd"], c["dim"], K4), mk("attn_k.weight", c["KV"] * c["hd"], c["dim"], K4),
                   mk("attn_v.weight", c["KV"] * c["hd"], c["dim"], K6), mk("attn_output.weight", c["dim"], c["H"] * c["hd"], K5 if i else K4),
                   (p + "ffn_norm.weight", (c["dim"],), 0, (1 + 0.1 * rng.standard_normal(c["dim"])).astype(np.float32)),
-                  mk("ffn_gate.weight", c["hidden"], c["dim"], K4), mk("ffn_up.weight", c["hidden"], c["dim"], K4), mk("ffn_down.weight", c["dim"], c["hidden"], K6)]
+                  mk("ffn_gate.weight", c["hidden"], c["dim"], K4), mk("ffn_up.weight", c["hidden"], c["dim"], K6 if split_ffn else K4), mk("ffn_down.weight", c["dim"], c["hidden"], K6)]
     tensors.append(("output_norm.weight", (c["dim"],), 0, np.ones(c["dim"], np.float32)))
     tensors.append(("output.weight", (c["vocab"], c["dim"]), K6[0], K6[1](lin(c["vocab"], c["dim"]))))
     kvs = [("general.architecture", "qwen2"), ("qwen2.context_length", 96), ("qwen2.attention.head_count", c["H"]), ("qwen2.attention.head_count_kv", c["KV"]),
            ("qwen2.block_count", c["L"]), ("qwen2.embedding_length", c["dim"]), ("qwen2.feed_forward_length", c["hidden"]),
            ("qwen2.attention.layer_norm_rms_epsilon", 1e-6), ("qwen2.rope.freq_base", 1000000.0), ("tokenizer.ggml.tokens", [f"t{i}" for i in range(c["vocab"])])]
     from tinygrad_amd.gguf import gguf_write
-    path = tmp_path / ("legacy.gguf" if legacy else "expand.gguf" if expand else "codebook.gguf" if codebook else "q4_k_m.gguf")
+    path = tmp_path / ("legacy.gguf" if legacy else "expand.gguf" if expand else "codebook.gguf" if codebook else "split_ffn.gguf" if split_ffn else "q4_k_m.gguf")
     return path, gguf_write(path, kvs, tensors)
   tensors = [("token_embd.weight", (c["vocab"], c["dim"]), 8, og.quantize_q8_0(lin(c["vocab"], c["dim"]) * 16))]
   for i in range(c["L"]):
@@ -76,14 +77,15 @@ def test_from_gguf_greedy_decode(gpu, tmp_path, tied):
   for _ in range(12): lg = o2.forward(cur, pos); pos += 1; cur = int(np.argmax(lg))
   assert ol.rel_err(model.logits(), lg) <= 1e-3
 
-@pytest.mark.parametrize("legacy", [0, 1, 2, 3], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-q1_0", "iq3_s-iq2_s-iq3_xxs"])
+@pytest.mark.parametrize("legacy", [0, 1, 2, 3, 4], ids=["q4_k_m", "q4_1-q5_0-q5_1", "iq4_xs-q1_0", "iq3_s-iq2_s-iq3_xxs", "ffn_gate-q4_k-ffn_up-q6_k"])
 def test_from_gguf_q4_k_m_type_mix(gpu, tmp_path, legacy):
   """A file with the tensor types of a Q4_K_M model (Q4_K / Q5_K / Q6_K matrices, Q4_K embedding; q/k/v of mixed types, so the
   block runs one launch per projection), and the same mix with the older Q4_1 / Q5_0 / Q5_1 blocks: greedy tokens and logits against
   the numpy restatement.  Third case: IQ4_XS matrices (embedding, attention, gate / up) beside a Q1_0 matrix; fourth: IQ3_S / IQ2_S / IQ3_XXS (codebooks and sign patterns in LDS).  All read in place: the
-  model streams the file's 1.1 .. 4.25 bits per weight per token, not an fp16 expansion."""
+  model streams the file's 1.1 .. 4.25 bits per weight per token, not an fp16 expansion.  Fifth: ffn_gate and ffn_up of different block types (two launches and an elementwise
+  silu(gate) * up, model.py:137)."""
   from tinygrad_amd.llm import Transformer
-  path, raw = _make_file(tmp_path, False, kquant=legacy == 0, legacy=legacy == 1, expand=legacy == 2, codebook=legacy == 3)
+  path, raw = _make_file(tmp_path, False, kquant=legacy in (0, 4), legacy=legacy == 1, expand=legacy == 2, codebook=legacy == 3, split_ffn=legacy == 4)
   model, kv = Transformer.from_gguf(path, max_context=64, max_new=32)
   if legacy == 2: assert model.blk[0].attn_q.ggml_type == 23 and model.embd_type == 23 and model.blk[1].attn_output.ggml_type == 41
   if legacy == 3: assert model.blk[0].attn_q.ggml_type == 21 and model.blk[1].attn_output.ggml_type == 22 and model.blk[0].attn_v.ggml_type == 18 and model.embd_type == 21

@@ -874,6 +874,13 @@ __global__ void chunk_advance_kernel(DecodeState* st, const int* __restrict__ pr
   if (threadIdx.x == 0) st->pos = np;
 }
 
+// silu(gate) * up over n float32 values, rounded to fp16 (the feed-forward's activation, tinygrad/llm/model.py:137, where ffn_gate and ffn_up are of different
+// block types and run as two launches instead of one with the SwiGLU epilogue)
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up, int n, _Float16* __restrict__ out) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (_Float16)(silu_f(gate[i]) * up[i]);
+}
+
 // ---------------------------------------------------------------------------------------------- C-ABI
 extern "C" {
 
@@ -928,6 +935,12 @@ int tga_moe_combine_rmsnorm_rows(const float* y, const float* probs, float* x, c
   TGA_REQUIRE(y && probs && x && weight && (out_f16 || out_f32), "tga_moe_combine_rmsnorm_rows: null pointer");
   TGA_REQUIRE(dim > 0 && rows >= 1 && k >= 1, "tga_moe_combine_rmsnorm_rows: rows=%d k=%d dim=%d", rows, k, dim);
   rmsnorm_kernel<true><<<rows, 1024, 0, (hipStream_t)stream>>>(x, weight, dim, eps, (_Float16*)out_f16, out_f32, 0, 0, x, y, probs, k);
+  TGA_LAUNCH_CHECK();
+  return 0;
+}
+int tga_silu_mul(const float* gate, const float* up, int64_t n, void* out_f16, void* stream) {
+  TGA_REQUIRE(gate && up && out_f16 && n > 0 && n < (1ll << 31), "tga_silu_mul: null pointer or bad length");
+  silu_mul_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(gate, up, (int)n, (_Float16*)out_f16);
   TGA_LAUNCH_CHECK();
   return 0;
 }

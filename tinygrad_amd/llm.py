@@ -220,7 +220,11 @@ class TransformerBlock:
     # the previous block's weighted expert sum can be completed inside this block's q/k/v launch (one 8-value piece per thread: dim <= 2048)
     self.can_fold_combine = self.fuse_norm and self.attn_q.ggml_type == self.attn_k.ggml_type == self.attn_v.ggml_type and c.dim <= 2048 \
                             and 0 < c.n_summands <= 8 and self.qkv_bias is None
-    if not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
+    # ffn_gate and ffn_up of different block types: two launches and an elementwise silu(gate) * up instead of one launch with the SwiGLU epilogue
+    self.split_gate_up = not self.moe and self.ffn_gate.ggml_type != self.ffn_up.ggml_type
+    if self.split_gate_up:
+      self.stage_act = False
+      if not hasattr(shared, "gate32"): shared.gate32, shared.up32 = (Buffer((1, max(c.hidden_dim, c.dense_hidden_dim)), np.float32) for _ in range(2))
     # The attention as one launch whose split partials attn_output merges (no q / k norm, cache of at most 2048 positions, attn_output rows of 33..64 units)
     ns = ctypes.c_int(0)
     rt.check(rt.lib().tga_attention_split_plan(c.max_context, ctypes.byref(ns)))
@@ -271,7 +275,13 @@ class TransformerBlock:
       qlinear_multi([self.attn_output], s.attn, [x], epilogue=1, resid=[x], stream=stream, x_staged=self.stage_attn)
     # x = h + ffn_down(silu(ffn_gate(n)) * ffn_up(n)), n = ffn_norm(h)                     model.py:137,150
     if not self.moe:
-      if self.fuse_norm:
+      if self.split_gate_up:
+        rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, 0, stream))
+        h = self.ffn_gate.out_features
+        g32, u32 = s.gate32.view(0, (1, h), np.float32), s.up32.view(0, (1, h), np.float32)
+        self.ffn_gate(s.xn, out=g32, stream=stream); self.ffn_up(s.xn, out=u32, stream=stream)
+        rt.check(L.tga_silu_mul(g32.ptr, u32.ptr, h, s.act.ptr, stream))
+      elif self.fuse_norm:
         qlinear_multi([self.ffn_gate, self.ffn_up], x, [s.act], epilogue=2, stream=stream, norm=(self.ffn_norm, c.norm_eps), stage_out_for=self.ffn_down if self.stage_act else None)
       else:
         rt.check(L.tga_rmsnorm(x.ptr, self.ffn_norm.ptr, c.dim, c.norm_eps, s.xn.ptr, None, self.ffn_gate.ggml_type if self.stage_xn else 0, stream))
@@ -608,7 +618,6 @@ class BatchedTransformer:
           if b["ffn_gate_shexp"].ggml_type != b["ffn_up_shexp"].ggml_type: raise NotImplementedError("ffn_gate_shexp and ffn_up_shexp of different ggml types are not built")
       else:
         for nm in ("ffn_gate", "ffn_up", "ffn_down"): b[nm] = lin(p + nm + ".weight")
-        if b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type: raise NotImplementedError("ffn_gate and ffn_up of different ggml types are not built")
       if chunk_of is not None: b["cache_k"], b["cache_v"] = chunk_of.blk[i].cache_k, chunk_of.blk[i].cache_v
       else:
         b["cache_k"] = Buffer((B, c.n_kv_heads, c.max_context, c.head_dim), f16).zero_()
@@ -622,6 +631,8 @@ class BatchedTransformer:
     self.attn = Buffer((B, nq), f16)
     self.attn_part = Buffer((B * c.n_heads * ((c.max_context + 63) // 64) * (c.head_dim + 2),), f32).zero_()
     self.act = Buffer((B, max(1, c.hidden_dim, c.dense_hidden_dim)), f16)
+    if any(not b["moe"] and b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type for b in self.blk):      # (gate and up rows of such a block, before silu(gate) * up)
+      self.gate32, self.up32 = Buffer((B, max(c.hidden_dim, c.dense_hidden_dim)), f32), Buffer((B, max(c.hidden_dim, c.dense_hidden_dim)), f32)
     if c.shared_expert_dim:
       self.act_sh, self.y_sh = Buffer((B, c.shared_expert_dim), f16), Buffer((B, c.dim), f32)
       self.p_sh, self.sh_logit, self.sh_sel = Buffer.from_numpy(np.ones(B, dtype=f32)), Buffer((B, 1), f32), Buffer((B,), np.int32)   # weight 1 unless the shared expert is gated
@@ -696,7 +707,13 @@ class BatchedTransformer:
       elif b["moe"]:
         rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
       if not b["moe"]:
-        self._linear([b["ffn_gate"], b["ffn_up"]], self.x, [self.act], epilogue=2, norm=(b["ffn_norm"], c.norm_eps, self.xn))
+        if b["ffn_gate"].ggml_type != b["ffn_up"].ggml_type:             # two launches and an elementwise silu(gate) * up (the SwiGLU epilogue pairs rows of one block type)
+          rt.check(L.tga_rmsnorm_rows(self.x.ptr, b["ffn_norm"].ptr, B, c.dim, c.norm_eps, self.xn.ptr, None, 0, st))
+          h = b["ffn_gate"].out_features
+          g32, u32 = self.gate32.view(0, (B, h), np.float32), self.up32.view(0, (B, h), np.float32)
+          self._linear([b["ffn_gate"]], self.xn, [g32]); self._linear([b["ffn_up"]], self.xn, [u32])
+          rt.check(L.tga_silu_mul(g32.ptr, u32.ptr, B * h, self.act.ptr, st))
+        else: self._linear([b["ffn_gate"], b["ffn_up"]], self.x, [self.act], epilogue=2, norm=(b["ffn_norm"], c.norm_eps, self.xn))
         self._linear([b["ffn_down"]], self.act, [self.x], epilogue=1, resid=[self.x])
         done(bi); continue
       k = c.num_experts_per_tok                                         # model.py:110-135

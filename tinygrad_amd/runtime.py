@@ -63,7 +63,7 @@ def _declare(lib):
     "tga_swiglu_interleaved": [vp, i64, i, ctypes.c_float, ctypes.c_float, vp, vp],
     "tga_add_expert_bias": [vp, vp, vp, i64, i64, i, vp],
     "tga_embed_row": [vp, i, i, vp, vp, vp],
-    "tga_embed_rows": [vp, i, i, vp, i, vp, vp, vp], "tga_rmsnorm_rows": [vp, vp, i, i, ctypes.c_float, vp, vp, i, vp],
+    "tga_embed_rows": [vp, i, i, vp, i, vp, vp, vp], "tga_rmsnorm_rows": [vp, vp, i, i, ctypes.c_float, vp, vp, i, vp], "tga_silu_mul": [vp, vp, ctypes.c_int64, vp, vp],
     "tga_moe_combine_rmsnorm_rows": [vp, vp, vp, vp, i, i, i, ctypes.c_float, vp, vp, vp],
     "tga_attention_decode_batched": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
     "tga_attention_prefill_chunk": [i, vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp, vp, vp],
