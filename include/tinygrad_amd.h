@@ -212,16 +212,20 @@ int tga_attention_decode_normed(const float* q, const float* k, const float* v, 
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, int stage_type, void* stream);
 
-/* tga_attention_decode as ONE launch whose consumer merges (model.py:167-198 up to the softmax-weighted V sums; no q / k norm).  A workgroup serves one query
+/* tga_attention_decode as ONE launch whose consumer merges (model.py:167-198 up to the softmax-weighted V sums; _normed: with the q / k RMSNorm of
+ * tga_attention_decode_normed, over the whole rows or per head, q and k 16-byte aligned).  A workgroup serves one query
  * head and one split of the cache; tga_attention_split_plan reports the number of splits for max_ctx: at most six, 0 when the cache is too long for this path
  * (max_ctx beyond 3072).  partials: n_heads * (n_splits * head_dim + 16) floats, per head [n_splits][head_dim] weighted V sums followed by the splits'
  * (max, sum) pairs; 16-byte aligned.  A split that starts beyond state.pos leaves an empty partial (max -inf, sum 0).  The merge is tga_attn_merge_qlinear's. */
 int tga_attention_split_plan(int max_ctx, int* n_splits);
 int tga_attention_decode_split(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
                                int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream);
+int tga_attention_decode_split_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps, int norm_per_head,
+                                      void* cache_k, void* cache_v, float* partials, const void* state,
+                                      int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream);
 /* attn_output + residual (model.py:198, 149) over the attention row that tga_attention_decode_split left as partials: y = resid + merge(partials) W^T, float32,
  * y may be resid.  The merge per head - sum_s e_s o_s / sum_s e_s l_s with e_s = exp(m_s - max m), rounded to fp16 - happens while the launch stages its
- * activation row.  K = n_heads * head_dim, 2048 < K <= 4096 (rows of 33..64 units); block types with a single-row kernel except MXFP4; n_splits 1..6. */
+ * activation row.  K = n_heads * head_dim <= 4096 (rows of at most 64 units, one wave per row); block types with a single-row kernel except MXFP4; n_splits 1..6. */
 int tga_attn_merge_qlinear(int ggml_type, const void* w, float* y, int64_t N, int64_t K, const float* resid, const float* partials, int n_splits, int head_dim, void* stream);
 
 /* tga_rmsnorm_qlinear_multi (single row) for the q / k / v launch of a decode step, with a hint for the attention launch behind it (no counterpart in the

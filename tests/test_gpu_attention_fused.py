@@ -92,6 +92,62 @@ def test_one_launch_attention_and_merging_linear(gpu, H, KV, hd, ctx, positions)
     # the two paths group their sums differently, so an fp16 activation may round the other way: close, not bit-equal
     assert ol.rel_err(res["one launch"][0], res["two launches"][0]) <= 2e-4
 
+@pytest.mark.parametrize("H,KV,hd,ctx,per_head", [(16, 16, 128, 576, 0), (8, 2, 128, 300, 1), (32, 8, 128, 1152, 1), (16, 4, 64, 200, 0), (4, 2, 256, 128, 1)],
+                         ids=["olmoe-whole-row", "qwen3-per-head-k1024", "per-head-k4096", "whole-row-hd64", "per-head-hd256"])
+def test_one_launch_attention_with_qk_norm(gpu, H, KV, hd, ctx, per_head):
+  """tga_attention_decode_split_normed + tga_attn_merge_qlinear against tga_attention_decode_normed followed by the plain linear: the q / k RMSNorm over the whole
+  rows (model.py:169) or per head (model.py:180), attn_output rows of 1024 .. 4096 values (rows of at most 32 units take the whole-wave kernel with idle lanes),
+  and both against the float64 attention of the normalised rows."""
+  rt, L = gpu, gpu.lib()
+  from tinygrad_amd import synth
+  rng = np.random.default_rng(H * 100 + hd + ctx + per_head)
+  K, N = H * hd, 384
+  ns = ctypes.c_int(0)
+  rt.check(L.tga_attention_split_plan(ctx, ctypes.byref(ns)))
+  w = synth.random_blocks(rng, rt.Q8_0, N, K)
+  wf = og.ggml_data_to_tensor(w, N * K, rt.Q8_0).reshape(N, K).astype(np.float64)
+  wb = rt.Buffer.from_numpy(w)
+  rope = _rope_table(hd, ctx); ropeb = rt.Buffer.from_numpy(rope)
+  ck0 = (rng.standard_normal((KV, ctx, hd)) * 0.7).astype(np.float16); cv0 = rng.standard_normal((KV, ctx, hd)).astype(np.float16)
+  qw = (1 + 0.3 * rng.standard_normal(hd if per_head else H * hd)).astype(np.float32); kw = (1 + 0.3 * rng.standard_normal(hd if per_head else KV * hd)).astype(np.float32)
+  qwb, kwb = rt.Buffer.from_numpy(qw), rt.Buffer.from_numpy(kw)
+  eps = 1e-6
+  def normed(x, wgt):                                                        # float32 RMSNorm as the kernels take it: (x * rsqrt(mean(x^2) + eps)) * weight
+    if per_head: return ((x / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + eps)) * wgt).astype(np.float32)
+    flat = x.reshape(-1)
+    return ((flat / np.sqrt((flat.astype(np.float64) ** 2).mean() + eps)) * wgt).astype(np.float32).reshape(x.shape)
+  part_old = rt.Buffer((H * ((ctx + 63) // 64) * (hd + 2),), np.float32).zero_()
+  part_new = rt.Buffer((H * (ns.value * hd + 16),), np.float32).zero_()
+  for pos in (0, 1, min(127, ctx - 1), min(130, ctx - 1), ctx - 1):
+    q = (rng.standard_normal((H, hd)) * 2).astype(np.float32); k = (rng.standard_normal((KV, hd)) * 3).astype(np.float32); v = rng.standard_normal((KV, hd)).astype(np.float32)
+    x = rng.standard_normal((1, N)).astype(np.float32)
+    st = np.zeros(16, np.int32); st[0] = pos
+    ref_row, k16, v16 = _attention_f64(normed(q, qw), normed(k, kw), v, ck0, cv0, pos, rope)
+    y_ref = x[0] + wf @ ref_row
+    res = {}
+    for name in ("two launches", "one launch"):
+      cK, cV, stb = rt.Buffer.from_numpy(ck0), rt.Buffer.from_numpy(cv0), rt.Buffer.from_numpy(st)
+      qb, kb, vb, y = rt.Buffer.from_numpy(q), rt.Buffer.from_numpy(k), rt.Buffer.from_numpy(v), rt.Buffer.from_numpy(x.copy())
+      if name == "two launches":
+        attn = rt.Buffer((1, K), np.float16)
+        rt.check(L.tga_attention_decode_normed(qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, eps, per_head, cK.ptr, cV.ptr, part_old.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, attn.ptr, None, 0, None))
+        wv, yv, rv, nv = (ctypes.c_void_p * 1)(wb.ptr), (ctypes.c_void_p * 1)(y.ptr), (ctypes.c_void_p * 1)(y.ptr), (ctypes.c_int64 * 1)(N)
+        rt.check(L.tga_qlinear_multi(rt.Q8_0, 1, wv, yv, nv, attn.ptr, rt.dtype_code(np.float16), rt.dtype_code(np.float32), 1, K, 1, rv, 0, 0, None))
+      else:
+        rt.check(L.tga_attention_decode_split_normed(qb.ptr, kb.ptr, vb.ptr, qwb.ptr, kwb.ptr, eps, per_head, cK.ptr, cV.ptr, part_new.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr, None))
+        rt.check(L.tga_attn_merge_qlinear(rt.Q8_0, wb.ptr, y.ptr, N, K, y.ptr, part_new.ptr, ns.value, hd, None))
+      rt.synchronize()
+      assert int(stb.numpy()[4]) == 0
+      res[name] = (y.numpy()[0].copy(), cK.numpy(), cV.numpy())
+      e = ol.rel_err(res[name][0], y_ref)
+      assert e <= 1e-3, f"{name} at position {pos}: rel-err {e:.2e} against the float64 attention + linear"
+      np.testing.assert_allclose(res[name][1][:, pos].astype(np.float32), k16.astype(np.float32), rtol=2e-3, atol=2e-3); np.testing.assert_array_equal(res[name][2][:, pos], v16)
+      keep = np.ones(ctx, bool); keep[pos] = False
+      np.testing.assert_array_equal(res[name][1][:, keep], ck0[:, keep]); np.testing.assert_array_equal(res[name][2][:, keep], cv0[:, keep])
+    assert ol.rel_err(res["one launch"][0], res["two launches"][0]) <= 2e-4
+    # (the two kernels sum the squares in different orders: an appended key may differ by one fp16 ulp)
+    np.testing.assert_allclose(res["one launch"][1][:, pos].astype(np.float32), res["two launches"][1][:, pos].astype(np.float32), rtol=2e-3, atol=2e-3)
+
 def test_one_launch_attention_refuses_what_it_cannot_serve(gpu):
   rt, L = gpu, gpu.lib()
   ns = ctypes.c_int(7)
@@ -101,7 +157,7 @@ def test_one_launch_attention_refuses_what_it_cannot_serve(gpu):
   st = rt.Buffer.from_numpy(np.zeros(16, np.int32))
   assert L.tga_attention_decode_split(b.ptr, b.ptr, b.ptr, b.ptr, b.ptr, b.ptr, st.ptr, 8, 8, 128, 4096, b.ptr, None) != 0
   assert L.tga_attention_decode_split(b.ptr, b.ptr, b.ptr, b.ptr, b.ptr, b.ptr, st.ptr, 8, 3, 128, 64, b.ptr, None) != 0      # heads not a multiple of kv heads
-  assert L.tga_attn_merge_qlinear(rt.Q4_0, b.ptr, b.ptr, 64, 1024, b.ptr, b.ptr, 2, 128, None) != 0                              # K outside 2048 < K <= 4096
+  assert L.tga_attn_merge_qlinear(rt.Q4_0, b.ptr, b.ptr, 64, 8192, b.ptr, b.ptr, 2, 128, None) != 0                              # rows of more than 64 units
   assert L.tga_attn_merge_qlinear(rt.Q4_0, b.ptr, b.ptr, 64, 4096, b.ptr, b.ptr, 7, 128, None) != 0                              # more than six splits
   # a position outside the cache: flag, nothing written
   st2 = np.zeros(16, np.int32); st2[0] = 64

@@ -554,7 +554,9 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
 // The flattened workgroup index is kv head + n_kv (head in group + group * split): with n_kv a multiple of 8 all readers of a kv head's rows run on one XCD.
 // A split that starts beyond the position writes an empty partial (max -inf, sum 0).  Partials per head: [n_splits][head_dim] weighted V sums, then the
 // (max, sum) pairs of the splits in 16 floats.
-template <int HD8, int IT, int NW>
+// NORM: q and k pass through an RMSNorm before the rotation (nn.RMSNorm, tinygrad/nn/__init__.py:296-304): 1 = over the whole q / k rows with weights of that
+// length (model.py:169), 2 = per head with head_dim weights (model.py:180); the workgroup sums the squares for itself.
+template <int HD8, int IT, int NW, int NORM>
 __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) {
   constexpr int HD = HD8 * 8, RPI = 64 / HD8, NVI = 16 / RPI, NGRP = NW * RPI, CSTR = HD + 4, SP = 16 * NW * IT;
   const int group = a.n_heads / a.n_kv;
@@ -568,6 +570,20 @@ __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) 
   const int ki = tid < half ? tid : half - 1, vi = tid < HD ? tid : HD - 1;
   const float kx1 = a.k[kvh * HD + ki], kx2 = a.k[kvh * HD + half + ki], vx = a.v[kvh * HD + vi];
   const float qx1 = a.q[head * HD + ki], qx2 = a.q[head * HD + half + ki];
+  float kw1 = 1.f, kw2 = 1.f, qw1 = 1.f, qw2 = 1.f, ssq = 0.f, ssk = 0.f;   // norm weights of this thread's pairs; its share of the sums of squares
+  if constexpr (NORM != 0) {
+    const int kb = NORM == 2 ? 0 : kvh * HD, qb = NORM == 2 ? 0 : head * HD;
+    kw1 = a.k_norm[kb + ki]; kw2 = a.k_norm[kb + half + ki]; qw1 = a.q_norm[qb + ki]; qw2 = a.q_norm[qb + half + ki];
+    if constexpr (NORM == 2) { if (tid < half) { ssq = qx1 * qx1 + qx2 * qx2; ssk = kx1 * kx1 + kx2 * kx2; } }
+    else {
+      const int n4q = (a.n_heads * HD) >> 2, n4k = (a.n_kv * HD) >> 2, nmax = n4q > n4k ? n4q : n4k;
+      for (int i = tid; i < nmax; i += NW * 64) {
+        const f32x4 x = ((const f32x4*)a.q)[i < n4q ? i : n4q - 1], y = ((const f32x4*)a.k)[i < n4k ? i : n4k - 1];
+        if (i < n4q) ssq += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        if (i < n4k) ssk += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+      }
+    }
+  }
   u32x4 kt[IT][NVI], vt[IT][NVI];
   {
     const _Float16* kbase = a.cache_k + (size_t)kvh * a.max_ctx * HD + vp * 8;
@@ -596,9 +612,23 @@ __global__ __launch_bounds__(NW * 64) void attn_split1_kernel(const AttnArgs a) 
     return;
   }
   const float rc_ = a.rope[(size_t)pos * HD + ki], rs_ = a.rope[(size_t)pos * HD + half + ki];
+  float qscale = 1.f, kscale = 1.f;
+  if constexpr (NORM != 0) {
+    __shared__ float red[2][NW];
+    ssq = wave_sum(ssq); ssk = wave_sum(ssk);
+    if (lane == 0) { red[0][wave] = ssq; red[1][wave] = ssk; }
+    __syncthreads();
+    float sq = 0.f, sk = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) { sq += red[0][w]; sk += red[1][w]; }
+    qscale = 1.0f / sqrtf(sq / (float)(NORM == 2 ? HD : a.n_heads * HD) + a.norm_eps);
+    kscale = 1.0f / sqrtf(sk / (float)(NORM == 2 ? HD : a.n_kv * HD) + a.norm_eps);
+  }
   if (tid < half) {
-    ks[tid] = rope_lo(kx1, kx2, rc_, rs_); ks[half + tid] = rope_hi(kx1, kx2, rc_, rs_);
-    qs[tid] = rope_lo(qx1, qx2, rc_, rs_); qs[half + tid] = rope_hi(qx1, qx2, rc_, rs_);
+    const float k1 = NORM != 0 ? (kx1 * kscale) * kw1 : kx1, k2 = NORM != 0 ? (kx2 * kscale) * kw2 : kx2;
+    const float q1 = NORM != 0 ? (qx1 * qscale) * qw1 : qx1, q2 = NORM != 0 ? (qx2 * qscale) * qw2 : qx2;
+    ks[tid] = rope_lo(k1, k2, rc_, rs_); ks[half + tid] = rope_hi(k1, k2, rc_, rs_);
+    qs[tid] = rope_lo(q1, q2, rc_, rs_); qs[half + tid] = rope_hi(q1, q2, rc_, rs_);
   }
   if (tid < HD) vs[tid] = vx;
   __syncthreads();
@@ -1026,9 +1056,12 @@ int tga_attention_split_plan(int max_ctx, int* n_splits) {
   attn_split1_tiles(max_ctx, n_splits);
   return 0;
 }
-int tga_attention_decode_split(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
-                               int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream) {
+static int attention_decode_split(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps, int norm_per_head,
+                                  void* cache_k, void* cache_v, float* partials, const void* state,
+                                  int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream) {
   TGA_REQUIRE(q && k && v && cache_k && cache_v && partials && state && rope_table, "tga_attention_decode_split: null pointer");
+  TGA_REQUIRE(!q_norm_weight == !k_norm_weight, "tga_attention_decode_split: q and k norm weights come together");
+  TGA_REQUIRE(!q_norm_weight || ((((uintptr_t)q | (uintptr_t)k) & 15) == 0), "tga_attention_decode_split: normed q and k rows must be 16-byte aligned");
   TGA_REQUIRE(n_kv_heads > 0 && n_heads % n_kv_heads == 0, "tga_attention_decode_split: n_heads=%d must be a multiple of n_kv_heads=%d", n_heads, n_kv_heads);
   TGA_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "tga_attention_decode_split: head_dim=%d must be 64, 128 or 256", head_dim);
   TGA_REQUIRE(((uintptr_t)partials & 15) == 0, "tga_attention_decode_split: partials must be 16-byte aligned");
@@ -1038,16 +1071,29 @@ int tga_attention_decode_split(const float* q, const float* k, const float* v, v
   a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (DecodeState*)state;
   a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = ns;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
+  a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps;
+  const int norm = q_norm_weight ? (norm_per_head ? 2 : 1) : 0;
   const unsigned grid = (unsigned)(n_heads * ns);
   hipStream_t s = (hipStream_t)stream;
-#define TGA_SPLIT1_W(HD8, NW) do { if (it == 1) attn_split1_kernel<HD8, 1, NW><<<grid, NW * 64, 0, s>>>(a); else if (it == 2) attn_split1_kernel<HD8, 2, NW><<<grid, NW * 64, 0, s>>>(a); \
-    else if (it == 3) attn_split1_kernel<HD8, 3, NW><<<grid, NW * 64, 0, s>>>(a); else attn_split1_kernel<HD8, 4, NW><<<grid, NW * 64, 0, s>>>(a); } while (0)
+#define TGA_SPLIT1_N(HD8, IT, NW) do { if (norm == 0) attn_split1_kernel<HD8, IT, NW, 0><<<grid, NW * 64, 0, s>>>(a); else if (norm == 1) attn_split1_kernel<HD8, IT, NW, 1><<<grid, NW * 64, 0, s>>>(a); \
+    else attn_split1_kernel<HD8, IT, NW, 2><<<grid, NW * 64, 0, s>>>(a); } while (0)
+#define TGA_SPLIT1_W(HD8, NW) do { if (it == 1) TGA_SPLIT1_N(HD8, 1, NW); else if (it == 2) TGA_SPLIT1_N(HD8, 2, NW); else if (it == 3) TGA_SPLIT1_N(HD8, 3, NW); else TGA_SPLIT1_N(HD8, 4, NW); } while (0)
 #define TGA_SPLIT1(HD8) do { const int nw = attn_split1_waves(); if (nw == 4) TGA_SPLIT1_W(HD8, 4); else if (nw == 16) TGA_SPLIT1_W(HD8, 16); else TGA_SPLIT1_W(HD8, 8); } while (0)
   if (head_dim == 64) TGA_SPLIT1(8); else if (head_dim == 128) TGA_SPLIT1(16); else TGA_SPLIT1(32);
+#undef TGA_SPLIT1_N
 #undef TGA_SPLIT1_W
 #undef TGA_SPLIT1
   TGA_LAUNCH_CHECK();
   return 0;
+}
+int tga_attention_decode_split(const float* q, const float* k, const float* v, void* cache_k, void* cache_v, float* partials, const void* state,
+                               int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream) {
+  return attention_decode_split(q, k, v, nullptr, nullptr, 0.f, 0, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx, rope_table, stream);
+}
+int tga_attention_decode_split_normed(const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps, int norm_per_head,
+                                      void* cache_k, void* cache_v, float* partials, const void* state,
+                                      int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* stream) {
+  return attention_decode_split(q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx, rope_table, stream);
 }
 
 int tga_attention_decode_batched(int batch, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,

@@ -497,7 +497,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     a.attn_S = attn->n_splits; a.attn_hd_log2 = hd == 64 ? 6 : hd == 128 ? 7 : 8;
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     const int rc = fmt >= 0 ? tga_qgemv1_dispatch(fmt, a, s) : -1;
-    if (rc < 0) return tga_set_error("tga_attn_merge_qlinear: needs the M = 1 fast path with rows of 33..64 units (2048 < K <= 4096) and 4-byte aligned weights");
+    if (rc < 0) return tga_set_error("tga_attn_merge_qlinear: needs the M = 1 fast path with rows of at most 64 units (K <= 4096) and 4-byte aligned weights");
     return rc;
   }
   if (M == 1) {

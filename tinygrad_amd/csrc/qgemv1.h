@@ -619,7 +619,7 @@ int qgemv1_launch_format(QArgs a, hipStream_t s) {
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   const int waves = (a.nu + 63) / 64;
-  if (a.nu <= 32) return launch_fast_e<T, 1, 4, true>(a, s);
+  if (a.nu <= 32 && !a.attn_S) return launch_fast_e<T, 1, 4, true>(a, s);      // (the merge prologue exists for whole-wave row teams: shorter rows leave lanes without a unit)
   if (waves <= 1) return launch_fast_e<T, 1, QG1_WR>(a, s);
   if (waves <= 2) return launch_fast_e<T, 2, 1>(a, s);
   if (waves <= 4) return launch_fast_e<T, 4, 1>(a, s);

@@ -225,12 +225,12 @@ class TransformerBlock:
     if self.split_gate_up:
       self.stage_act = False
       if not hasattr(shared, "gate32"): shared.gate32, shared.up32 = (Buffer((1, max(c.hidden_dim, c.dense_hidden_dim)), np.float32) for _ in range(2))
-    # The attention as one launch whose split partials attn_output merges (no q / k norm, cache of at most 2048 positions, attn_output rows of 33..64 units)
+    # The attention as one launch whose split partials attn_output merges (cache of at most six splits, attn_output rows of at most 64 units; the q / k norm inside the launch)
     ns = ctypes.c_int(0)
     rt.check(rt.lib().tga_attention_split_plan(c.max_context, ctypes.byref(ns)))
     ao = self.attn_output
-    self.fused_attn = ns.value if (os.environ.get("TGA_ATTN", "fused") == "fused" and not c.qk_norm and fast(ao) and ao.ggml_type != rt.MXFP4
-                                   and 2048 < ao.in_features <= 4096 and ao.in_features == c.n_heads * c.head_dim) else 0
+    self.fused_attn = ns.value if (os.environ.get("TGA_ATTN", "fused") == "fused" and fast(ao) and ao.ggml_type != rt.MXFP4
+                                   and 512 <= ao.in_features <= 4096 and ao.in_features == c.n_heads * c.head_dim) else 0
     self.kv_touch = os.environ.get("TGA_KV_TOUCH", "1") == "1" and c.n_kv_heads % 8 == 0      # the q / k / v launch touches the cache rows for the attention launch
 
   def __call__(self, x: Buffer, stream, pending: int = 0, defer: bool = False) -> tuple[Buffer, int]:
@@ -264,8 +264,9 @@ class TransformerBlock:
     # q/k RMSNorm inside the attention launch: full-width before the head split (model.py:169) or per head after it (model.py:180)
     if self.fused_attn:
       # one launch leaves split partials, attn_output merges them while it stages its row (no merge launch)
-      rt.check(L.tga_attention_decode_split(s.q.ptr, s.k.ptr, s.v.ptr, self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim,
-                                            c.max_context, s.rope.ptr, stream))
+      rt.check(L.tga_attention_decode_split_normed(s.q.ptr, s.k.ptr, s.v.ptr, self.q_norm.ptr if c.qk_norm else None, self.k_norm.ptr if c.qk_norm else None, c.norm_eps,
+                                                   int(c.qk_norm == c.head_dim), self.cache_k.ptr, self.cache_v.ptr, s.attn_part.ptr, s.state.ptr, c.n_heads, c.n_kv_heads, c.head_dim,
+                                                   c.max_context, s.rope.ptr, stream))
       ao = self.attn_output
       rt.check(L.tga_attn_merge_qlinear(ao.ggml_type, ao.blocks.ptr, x.ptr, ao.out_features, ao.in_features, x.ptr, s.attn_part.ptr, self.fused_attn, c.head_dim, stream))
     else:

@@ -81,6 +81,7 @@ def _declare(lib):
     "tga_attention_split_plan": [i, vp],
     "tga_rmsnorm_qlinear_multi_touch": [vp, ctypes.c_float, i, i, c_void_pp, c_void_pp, vp, vp, i, i64, i, c_void_pp, vp, vp, vp, vp, i, i, i, vp],
     "tga_attention_decode_split": [vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp, vp],
+    "tga_attention_decode_split_normed": [vp, vp, vp, vp, vp, ctypes.c_float, i, vp, vp, vp, vp, i, i, i, i, vp, vp],
     "tga_attn_merge_qlinear": [i, vp, vp, i64, i64, vp, vp, i, i, vp],
     "tga_argmax_step": [vp, i, vp, vp, vp, vp, vp, i, vp],
     "tga_advance_prompt": [vp, vp, vp],
