@@ -37,7 +37,7 @@ extern "C" {
 
 /* ---- runtime: replaces HIPDevice / HIPAllocator / HIPProgram timing in tinygrad/runtime/ops_hip.py:12-70 ---- */
 const char* tga_last_error(void);
-int tga_init(int device);                                  /* hipSetDevice + kernel attribute set-up; ops_hip.py:14-20.  Also allocates, once per device, the 48 MB workspace of the 17 .. 64 row linears */
+int tga_init(int device);                                  /* hipSetDevice + kernel attribute set-up; ops_hip.py:14-20.  Also allocates, once per device, the 160 MB workspace of the 17 .. 128 row linears */
 int tga_device_name(char* buf, size_t len);
 int tga_malloc(void** ptr, size_t nbytes);                 /* ops_hip.py:60-62 */
 int tga_free(void* ptr);                                   /* ops_hip.py:63 */
@@ -80,7 +80,7 @@ int tga_dequant(int ggml_type, const void* blocks, int64_t n, void* out, int out
  *   y[m, n] = sum_k x[m, k] * W[n, k],   W = dequant(w) as (N, K) row-major with quant blocks along K (gguf.py:148).
  * x: (M, K) row-major, x_dtype TGA_F16 or TGA_F32 (F32 activations are rounded to fp16 before the multiply).
  * y: (M, N) row-major, y_dtype TGA_F16 or TGA_F32.  1 <= M <= 8 (the decode range); 9 <= M <= 16 is taken too, for prefill chunks: one launch where the
- * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows; 17 <= M <= 64 (plain fp16 / float32 activations; a prefill step) is one pass over the weights on a 64-column matrix-core tile where it applies (Q4_0 / Q8_0 pairs, Q4_K, Q5_K, Q6_K, IQ4_XS, fp16; K a multiple of 256 up to 32768; several matrices: each a multiple of 16 rows; staged rows and split-K partial sums in the per-device workspace of tga_init, one slot per stream), otherwise blocks of sixteen rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
+ * LDS-fed matrix-core kernel applies (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K, K a multiple of 1024 (Q4_K: of 2048 up to 4096), rows a multiple of 16; K beyond 4096: one matrix, plain or residual epilogue; Q6_K: one matrix, K a multiple of 2048), otherwise two calls of at most eight rows; 17 <= M <= 128 (plain fp16 / float32 activations; a prefill step) is one pass over the weights on a matrix-core tile of two, four or eight column groups where it applies (Q4_0 / Q8_0 pairs, Q4_K, Q5_K, Q6_K, IQ4_XS, fp16; K a multiple of 256 up to 32768; several matrices: each a multiple of 16 rows; staged rows and split-K partial sums in the per-device workspace of tga_init, one slot per stream), otherwise blocks of sixteen rows.  Dense fp16 weights (TGA_F16, K % 64 == 0) are served too.  K must be a multiple of the type's block size
  * (Q4_1 / Q5_0 / Q5_1 are served as block pairs: K % 64 == 0).
  * w must be 2-byte aligned for Q4_0/Q8_0/Q6_K and 4-byte aligned for Q4_K/Q5_K/Q4_1/Q5_0/Q5_1 (GGUF aligns tensor data to 32 bytes,
  * gguf.py:144-148). */
@@ -114,7 +114,7 @@ int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_eps, int nseg
 
 /* The same for M rows (batched decode steps and prefill chunks): x (M, K) float32 BEFORE the norm.  One launch where the LDS-fed small-batch kernel applies
  * (Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 / Q4_K / Q5_K / Q6_K / fp16, 2 <= M <= 8, K <= 4096: the norm is folded into its prologue); otherwise tga_rmsnorm_rows into xn_scratch_f16 (M, K) followed by
- * tga_qlinear_multi on it (M up to 64).  xn_scratch_f16 is clobbered or left untouched accordingly. */
+ * tga_qlinear_multi on it (M up to 128).  xn_scratch_f16 is clobbered or left untouched accordingly. */
 int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                              const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream);
 
@@ -271,20 +271,20 @@ int tga_attention_decode_batched(int batch, const float* q, const float* k, cons
 int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream);
-/* tga_attention_prefill_chunk for 17 .. 64 rows whose fp16 output is ONE buffer for all rows in the layout the 64-column GEMM multiplies from, for a consumer
+/* tga_attention_prefill_chunk for 17 .. 128 rows whose fp16 output is ONE buffer for all rows in the layout the prefill GEMM multiplies from, for a consumer
  * (attn_output) of block type consumer_type with K = n_heads * head_dim (a multiple of 256): 16 * (rows <= 32 ? 2 : 4) rows x K fp16 values; the rows at and beyond
  * `rows` are not written (zero them once). */
 int tga_attention_prefill_chunk_staged(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                        int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                        int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_rows_staged, int consumer_type, void* stream);
-/* ---- a prefill step of 17 .. 64 rows (model.py:464, 476-481) with the rows handed from launch to launch in the layout the 64-column GEMM multiplies from: no
+/* ---- a prefill step of 17 .. 128 rows (model.py:464, 476-481) with the rows handed from launch to launch in the layout the prefill GEMM multiplies from: no
  * counterpart in the reference (its scheduler fuses what it fuses); the results equal those of tga_rmsnorm_qlinear_rows / tga_qlinear_multi on plain rows up to the
  * order of a float32 sum.  tga_qlinear_multi takes such rows with x_dtype TGA_F16_STAGED and M > 16, and writes them from the SwiGLU epilogue with y_stage_type. ---- */
 /* *ncg = column groups of sixteen rows (2 or 4: the buffer of the rows holds 16 * ncg x K fp16 values) when a linear of this type with rows of K values takes M rows
  * in that layout, 0 when it does not. */
 int tga_rows_staged_plan(int ggml_type, int64_t K, int M, int* ncg);
 /* y = y + x W^T (attn_output, ffn_down: model.py:149-150) for one matrix over rows in that layout.  When the kernel splits K, the sum over the splits is left to the
- * caller's next launch: *partials / *ks / *np describe the partial tiles (in the stream's workspace: valid until the next call with 17 .. 64 rows on this stream) and y
+ * caller's next launch: *partials / *ks / *np describe the partial tiles (in the stream's workspace: valid until the next call with 17 .. 128 rows on this stream) and y
  * is untouched; *ks = 0: y is complete. */
 int tga_qlinear_rows_deferred(int ggml_type, const void* w, int64_t N, int64_t K, const void* x_staged, int M, float* y, const float** partials, int* ks, int* np, void* stream);
 /* nn.RMSNorm (tinygrad/nn/__init__.py:296-304) of `rows` float32 rows, written as fp16 in that layout for a consumer of consumer_type (and to xn_out_f16 as plain

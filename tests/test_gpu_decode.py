@@ -106,8 +106,8 @@ def test_kv_prefix_reuse_equals_fresh_model(gpu):
   model.prefill(p3, reuse_cache=False)
   assert model.prefill_steps == len(p3) - 1
 
-@pytest.mark.parametrize("chunk", [8, 16, 5, 32, 24, 64])
-@pytest.mark.parametrize("n_prompt", [9, 17, 61, 70, 131])
+@pytest.mark.parametrize("chunk", [8, 16, 5, 32, 24, 64, 128, 100])
+@pytest.mark.parametrize("n_prompt", [9, 17, 61, 70, 131, 180])
 def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
   """Prompt positions computed eight, sixteen or thirty-two (or five, or twenty-four) at a time (small-batch linears, causal attention inside the chunk: Transformer.generate's chunked prefill,
   tinygrad/llm/model.py:464, 476-481) against the same model prefilled token by token and against the oracle: the KV caches agree to fp16 rounding of
@@ -131,9 +131,9 @@ def test_chunked_prefill_vs_token_by_token_and_oracle(gpu, n_prompt, chunk):
   print(f"prompt {n_prompt}: min top-2 margin {margin:.4f}, worst logits rel-err {worst:.2e}")
   assert got == ref and worst <= 1e-3
 
-@pytest.mark.parametrize("ltype,chunk", [("Q4_0", 64), ("Q8_0", 24), ("Q4_K", 40), ("Q6_K", 32), ("Q4_K_M", 48)])
+@pytest.mark.parametrize("ltype,chunk", [("Q4_0", 64), ("Q8_0", 24), ("Q4_K", 40), ("Q6_K", 32), ("Q4_K_M", 48), ("Q4_0", 128), ("Q4_K_M", 100), ("Q8_0", 72)])
 def test_prefill_steps_with_rows_in_the_multiplying_layout_equal_the_plain_steps(gpu, monkeypatch, ltype, chunk):
-  """A prefill in steps of 17 .. 64 positions hands its rows from launch to launch in the layout the 64-column kernel multiplies from and lets the norm launches complete
+  """A prefill in steps of 17 .. 128 positions hands its rows from launch to launch in the layout the prefill kernel multiplies from and lets the norm launches complete
   the split-K sums (BatchedTransformer.rows64); with TGA_ROWS64=0 the same steps run on plain rows.  Same kernels on the same fp16 values: the KV caches agree to the order
   of a float32 sum, the decode steps that follow give the same tokens."""
   from tinygrad_amd import runtime as rt
@@ -197,7 +197,7 @@ def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
     np.testing.assert_array_equal(tokb.numpy(), prompt[np.minimum(pos0 + B + np.arange(B), ctx - 1)])
   assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
 
-@pytest.mark.parametrize("H,KV,hd,B", [(8, 2, 128, 16), (8, 2, 128, 37), (4, 4, 64, 64), (16, 2, 64, 24), (8, 8, 128, 17), (8, 1, 128, 9)])
+@pytest.mark.parametrize("H,KV,hd,B", [(8, 2, 128, 16), (8, 2, 128, 37), (4, 4, 64, 64), (16, 2, 64, 24), (8, 8, 128, 17), (8, 1, 128, 9), (8, 2, 128, 128), (4, 4, 64, 100)])
 def test_attention_prefill_chunk_on_the_matrix_cores_vs_numpy(gpu, H, KV, hd, B):
   """tga_attention_prefill_chunk for more than eight rows without q / k norm (the launch that attends multiplies on the matrix cores: workgroup per kv head, 64-position
   split and tile of sixteen rows, wave per query head of the group): steps of B consecutive positions over one cache up to position 150 and beyond two split

@@ -239,9 +239,10 @@ def test_nine_to_sixteen_rows(gpu, t, n, k, m):
   np.testing.assert_array_equal(_run(gpu, t, w, x.astype(np.float32), n, k), y)
 
 @pytest.mark.parametrize("t,n,k,m", [(2, 4096, 4096, 32), (12, 528, 2048, 24), (8, 200, 14336, 40), (14, 1024, 4096, 64), (2, 512, 14336, 17), (13, 300, 4096, 48), (23, 528, 4096, 64), (12, 4096, 4096, 17),
-                                     (8, 1000, 1024, 33), (14, 72, 256, 50), (2, 200, 2048 + 32, 40), (3, 200, 2048, 40), (39, 256, 2048, 24), (18, 528, 2048, 24), (22, 300, 4096, 40)])
+                                     (8, 1000, 1024, 33), (14, 72, 256, 50), (2, 200, 2048 + 32, 40), (3, 200, 2048, 40), (39, 256, 2048, 24), (18, 528, 2048, 24), (22, 300, 4096, 40),
+                                     (2, 4096, 4096, 128), (12, 528, 2048, 100), (8, 200, 14336, 65), (14, 1024, 4096, 128), (23, 528, 4096, 96), (13, 300, 4096, 80), (39, 256, 2048, 70)])
 def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
-  """Prefill chunks of 17 .. 64 rows: one pass of the 64-column kernel where it applies (K a multiple of 256, its formats), otherwise blocks of sixteen (and a rest)
+  """Prefill chunks of 17 .. 128 rows: one pass of the prefill kernel where it applies (K a multiple of 256, its formats), otherwise blocks of sixteen (and a rest)
   through the small-batch kernels: plain, with the residual in place and with the norm in front (tga_rmsnorm_qlinear_rows), against the C restatement run in
   blocks of eight rows."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
@@ -267,9 +268,9 @@ def test_seventeen_to_sixty_four_rows(gpu, t, n, k, m):
   refn = np.concatenate([cref.linear(t, w, h[i:i + 8], n, k, threads=8) for i in range(0, m, 8)])
   assert ol.rel_err(out.numpy(), refn) <= TOL
 
-@pytest.mark.parametrize("t,dim,hidden,m", [(2, 1024, 2048, 40), (8, 512, 1024, 17), (12, 1024, 2304, 64), (14, 512, 1024, 33), (23, 1024, 1024, 24), (13, 256, 512, 50)])
+@pytest.mark.parametrize("t,dim,hidden,m", [(2, 1024, 2048, 40), (8, 512, 1024, 17), (12, 1024, 2304, 64), (14, 512, 1024, 33), (23, 1024, 1024, 24), (13, 256, 512, 50), (2, 1024, 2048, 128), (12, 1024, 2304, 80), (14, 512, 1024, 100)])
 def test_rows_in_the_multiplying_layout_equal_plain_rows(gpu, t, dim, hidden, m):
-  """The entry points of a prefill step that hands its rows from launch to launch in the layout the 64-column kernel multiplies from (tga_rmsnorm_rows_stage ->
+  """The entry points of a prefill step that hands its rows from launch to launch in the layout the prefill kernel multiplies from (tga_rmsnorm_rows_stage ->
   tga_qlinear_multi with staged x -> SwiGLU written for its consumer -> tga_qlinear_rows_deferred -> partial sums completed by the next norm or by
   tga_rows_add_partials) against the same linears on plain rows (tga_rmsnorm_qlinear_rows, tga_qlinear_multi): the same kernels multiply the same fp16 values, so the
   results agree to 1e-5 with the plain rows and bit for bit among the staged variants, except where a sum is taken in another order (residual first instead of last: 1e-6)."""
@@ -280,10 +281,10 @@ def test_rows_in_the_multiplying_layout_equal_plain_rows(gpu, t, dim, hidden, m)
   rng = np.random.default_rng(7 * t + m)
   ncg = ctypes.c_int(0)
   gpu.check(L.tga_rows_staged_plan(t, dim, m, ctypes.byref(ncg)))
-  assert ncg.value == (2 if m <= 32 else 4)
-  gpu.check(L.tga_rows_staged_plan(39, 2048, m, ctypes.byref(ncg))); assert ncg.value == 0          # (MXFP4: no 64-column kernel)
+  assert ncg.value == (2 if m <= 32 else 4 if m <= 64 else 8)
+  gpu.check(L.tga_rows_staged_plan(39, 2048, m, ctypes.byref(ncg))); assert ncg.value == 0          # (MXFP4: no prefill kernel)
   gpu.check(L.tga_rows_staged_plan(t, dim, 16, ctypes.byref(ncg))); assert ncg.value == 0
-  R = 16 * (2 if m <= 32 else 4)
+  R = 16 * (2 if m <= 32 else 4 if m <= 64 else 8)
   gate, up = (QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, t, hidden, dim)), t, hidden, dim) for _ in range(2))
   down = QuantLinear(gpu.Buffer.from_numpy(synth.random_blocks(rng, t, dim, hidden)), t, dim, hidden)
   x = (rng.standard_normal((m, dim)) * 2).astype(np.float32)
@@ -326,7 +327,7 @@ def test_rows_in_the_multiplying_layout_equal_plain_rows(gpu, t, dim, hidden, m)
   assert L.tga_qlinear_multi(39, 2, VP2(gate.blocks.ptr, up.blocks.ptr), VP2(act_st.ptr, None), I2(hidden, hidden), xn_st.ptr, rt.F16_STAGED, rt.F16, m, dim, 2, None, 0, 0, None) != 0
 
 def test_seventeen_rows_on_more_streams_than_workspace_slots(gpu):
-  """The 64-column kernel keeps its staged activations and split-K partial tiles in a per-device workspace of a few slots, one per stream; a call on a
+  """The prefill kernel keeps its staged activations and split-K partial tiles in a per-device workspace of a few slots, one per stream; a call on a
   further stream runs blocks of sixteen rows instead.  Six streams, two calls each (the second finds its stream's slot again): every result within the bar,
   and equal between the two calls of a stream."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
@@ -503,10 +504,10 @@ def test_norm_and_linears_of_mixed_block_types(gpu, types, k, ns):
     ref = ol.linear_f64(h, ol.weight_f32(w, n, k, t))
     assert ol.rel_err(o.numpy(), ref) <= TOL and ol.rel_err(o16.numpy().astype(np.float32), ref) <= 2 * TOL
 
-@pytest.mark.parametrize("m", [16, 17, 37, 64])
+@pytest.mark.parametrize("m", [16, 17, 37, 64, 65, 100, 128])
 def test_sixteen_and_more_rows_segments_residual_and_swiglu(gpu, m):
   """q / k / v in one launch, the residual epilogue in place and silu(gate) * up at sixteen rows (on the LDS-fed kernel's range and outside it) and at
-  17 .. 64 rows (the 64-column kernel; segments that are no multiple of sixteen rows go through blocks of sixteen)."""
+  17 .. 128 rows (the prefill kernel; segments that are no multiple of sixteen rows go through blocks of sixteen)."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
   rng = np.random.default_rng(1616 + m)
   for t, k, ns in ((2, 2048, [2048, 512, 512]), (8, 1024, [512, 128, 130]), (14, 1024, [64, 32, 32]), (12, 2048, [272, 48, 48]), (13, 1024, [100, 100]), (23, 1024, [80, 16, 16])):
@@ -556,15 +557,15 @@ def test_argument_errors(gpu):
   w = gpu.Buffer.from_numpy(np.zeros(18 * 4, dtype=np.uint8))
   with pytest.raises(ValueError): QuantLinear(w, 1337, 4, 32)
   lin = QuantLinear(w, 2, 4, 32)
-  with pytest.raises(AssertionError): lin(gpu.Buffer((65, 32), np.float16))
-  with pytest.raises(RuntimeError, match="out of range 1..64"): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 65, 4, 32, None))
+  with pytest.raises(AssertionError): lin(gpu.Buffer((129, 32), np.float16))
+  with pytest.raises(RuntimeError, match="out of range 1..128"): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 129, 4, 32, None))
   with pytest.raises(RuntimeError): gpu.check(gpu.lib().tga_qlinear(2, w.ptr, w.ptr, 0, w.ptr, 0, 1, 4, 33, None))
   # Q4_1 / Q5_0 / Q5_1 rows are read as block pairs: an odd number of blocks per row is refused
   with pytest.raises(RuntimeError, match="multiple of 64"): gpu.check(gpu.lib().tga_qlinear(3, w.ptr, w.ptr, 1, w.ptr, 0, 1, 1, 96, None))
   # the entry points of the batched steps refuse what they cannot launch
   L, f = gpu.lib(), gpu.Buffer((64,), np.float32).zero_()
   with pytest.raises(RuntimeError, match="null pointer"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, None, 1, 4, 32, 0, None, None))
-  with pytest.raises(RuntimeError, match="1..64"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, f.ptr, 1, 65, 32, 0, None, None))
+  with pytest.raises(RuntimeError, match="1..128"): gpu.check(L.tga_rmsnorm_qlinear_rows(f.ptr, 1e-5, 2, 1, None, None, None, f.ptr, f.ptr, 1, 129, 32, 0, None, None))
   with pytest.raises(RuntimeError, match="multiple of 8"): gpu.check(L.tga_moe_router_rows(f.ptr, f.ptr, 1e-5, f.ptr, 2, 20, 4, f.ptr, f.ptr, None))
   with pytest.raises(RuntimeError, match="rows=0"): gpu.check(L.tga_moe_combine_rmsnorm_rows(f.ptr, f.ptr, f.ptr, f.ptr, 0, 2, 16, 1e-5, f.ptr, None, None))
   with pytest.raises(RuntimeError, match="exceed one launch"):

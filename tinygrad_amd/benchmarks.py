@@ -140,7 +140,7 @@ def config8(steps: int = 32, ctx: int = 1024):
   rng = np.random.default_rng(1003)
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=ctx)]
   res = []
-  for chunk in (64, 32, 16, 8, 4, 2, 1):
+  for chunk in (128, 96, 64, 32, 16, 8, 4, 2, 1):
     model.prefill_chunk = chunk
     model.prefill(prompt[:2 * 64 + 64], reuse_cache=False)             # captures the step kinds this chunk size uses (whole chunks, the tail steps of sixteen, eight and four, single positions)
     t0 = time.perf_counter()

@@ -133,7 +133,7 @@ struct AttnArgs {
   float scale;
   _Float16* out16; float* out32;                       // attention output [n_heads*hd]
   int stage_fmt, stage_nu;                             // != 0: out16 in the staged order of the consuming linear
-  int stage_rows_ncg;                                  // != 0 (rows of a prefill step): out16 is ONE buffer for all rows, in the layout the 17 .. 64 row GEMM multiplies from (rows_staged_pos)
+  int stage_rows_ncg;                                  // != 0 (rows of a prefill step): out16 is ONE buffer for all rows, in the layout the 17 .. 128 row GEMM multiplies from (rows_staged_pos)
   const float* q_norm; const float* k_norm; float norm_eps;   // optional RMSNorm weights: over the whole q / k vectors, or
   int norm_per_head;                                           // per head (weights of head_dim values shared by all heads)
   // batched decode (sequences in lockstep at one position): sequence z = blockIdx.z (split launch) / blockIdx.y (merge launch) uses the
@@ -1000,10 +1000,10 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
   a.chunk = 0; a.pos_step = 0;
   if (chunk) { a.cache_bs = 0; a.pos_step = 1; }
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
-  if (stage_type && chunk) {                            // the rows of a prefill step for the 17 .. 64 row GEMM
-    TGA_REQUIRE(out_f16 && batch >= 17 && batch <= 64 && ((long long)n_heads * head_dim) % 256 == 0 && stage_type != GGML_MXFP4 && stage_type != GGML_Q4_1 && stage_type != GGML_Q5_0 && stage_type != GGML_Q5_1,
-                "tga_attention_prefill_chunk: rows in the multiplying layout need 17..64 rows, n_heads * head_dim a multiple of 256 and a block type the 64-column kernel takes");
-    a.stage_rows_ncg = batch <= 32 ? 2 : 4;
+  if (stage_type && chunk) {                            // the rows of a prefill step for the 17 .. 128 row GEMM
+    TGA_REQUIRE(out_f16 && batch >= 17 && batch <= 128 && ((long long)n_heads * head_dim) % 256 == 0 && stage_type != GGML_MXFP4 && stage_type != GGML_Q4_1 && stage_type != GGML_Q5_0 && stage_type != GGML_Q5_1,
+                "tga_attention_prefill_chunk: rows in the multiplying layout need 17..128 rows, n_heads * head_dim a multiple of 256 and a block type the prefill kernel takes");
+    a.stage_rows_ncg = batch <= 32 ? 2 : batch <= 64 ? 4 : 8;
   }
   dim3 grid(n_kv_heads, a.nsplit, batch);
   hipStream_t s = (hipStream_t)stream;
@@ -1106,7 +1106,7 @@ int tga_attention_decode_batched(int batch, const float* q, const float* k, cons
 int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                 int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                 int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_f16, float* out_f32, void* stream) {
-  TGA_REQUIRE(rows >= 1 && rows <= 64, "tga_attention_prefill_chunk: rows=%d", rows);
+  TGA_REQUIRE(rows >= 1 && rows <= 128, "tga_attention_prefill_chunk: rows=%d", rows);
   return attention_launch(1, rows, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_f16, out_f32, 0, stream);
 }
@@ -1114,14 +1114,14 @@ int tga_attention_prefill_chunk(int rows, const float* q, const float* k, const 
 int tga_attention_prefill_chunk_staged(int rows, const float* q, const float* k, const float* v, const float* q_norm_weight, const float* k_norm_weight, float norm_eps,
                                        int norm_per_head, void* cache_k, void* cache_v, float* partials, const void* state,
                                        int n_heads, int n_kv_heads, int head_dim, int max_ctx, const float* rope_table, void* out_rows_staged, int consumer_type, void* stream) {
-  TGA_REQUIRE(rows >= 17 && rows <= 64 && consumer_type != 0, "tga_attention_prefill_chunk_staged: rows=%d (17..64), consumer type %d", rows, consumer_type);
+  TGA_REQUIRE(rows >= 17 && rows <= 128 && consumer_type != 0, "tga_attention_prefill_chunk_staged: rows=%d (17..128), consumer type %d", rows, consumer_type);
   return attention_launch(1, rows, q, k, v, q_norm_weight, k_norm_weight, norm_eps, norm_per_head, cache_k, cache_v, partials, state, n_heads, n_kv_heads, head_dim, max_ctx,
                           rope_table, out_rows_staged, nullptr, consumer_type, stream);
 }
 
 int tga_chunk_advance(void* state, const int32_t* prompt, int rows, int32_t* tokens, int max_ctx, void* stream) {
-  TGA_REQUIRE(state && prompt && tokens && rows >= 1 && rows <= 64 && max_ctx >= 1, "tga_chunk_advance: null pointer or rows=%d outside 1..64", rows);
-  chunk_advance_kernel<<<1, 64, 0, (hipStream_t)stream>>>((DecodeState*)state, prompt, rows, tokens, max_ctx);
+  TGA_REQUIRE(state && prompt && tokens && rows >= 1 && rows <= 128 && max_ctx >= 1, "tga_chunk_advance: null pointer or rows=%d outside 1..128", rows);
+  chunk_advance_kernel<<<1, 128, 0, (hipStream_t)stream>>>((DecodeState*)state, prompt, rows, tokens, max_ctx);
   TGA_LAUNCH_CHECK();
   return 0;
 }

@@ -895,7 +895,7 @@ __device__ __forceinline__ int staged_pos(int fmt, int e, int nu) {
   return e;
 }
 
-// Halfword index of element e of activation row m in the layout the 17 .. 64 row GEMM (qgemm64.hip) multiplies from, for a consumer of format fmt (units of 64
+// Halfword index of element e of activation row m in the layout the 17 .. 128 row GEMM (qgemm64.hip) multiplies from, for a consumer of format fmt (units of 64
 // values) and ncg column groups: per step of four units [vector][column group][unit][column] 16-byte pieces (the formats' staged vectors, Fmt::stage).  The staged
 // position inside a superblock's four units does not depend on the row length, so it is taken for a row of four units (no division by the unit count).
 __device__ __forceinline__ size_t rows_staged_pos(int fmt, int e, int m, int ncg) {

@@ -1,10 +1,11 @@
-// Prefill GEMM over GGUF blocks: 17 .. 64 activation rows (the positions of one prefill step, tinygrad/llm/model.py:464, 476-481: a T > 1 call of the same
+// Prefill GEMM over GGUF blocks: 17 .. 128 activation rows (the positions of one prefill step, tinygrad/llm/model.py:464, 476-481: a T > 1 call of the same
 // linears, x.linear(W.T) over the lazily dequantized weight, tinygrad/nn/__init__.py:177, tinygrad/mixin/op.py:367-392) in ONE pass over the weights.
 // The small-batch kernels multiply sixteen rows per pass (the sixteen columns of one MFMA tile), so a step of 64 positions decoded every weight four times;
-// here a unit is decoded once into fp16 weights (the reference's own fp16 weight cast, model.py:376) and multiplied with two or four column groups.
+// here a unit is decoded once into fp16 weights (the reference's own fp16 weight cast, model.py:376) and multiplied with two, four or eight column groups of
+// sixteen rows (up to 128 positions per pass: at 64 the pass is bound by how the weights stream, at 128 by the LDS reads of the B operands).
 //
 // Up to three launches per call, all on the caller's stream:
-//  1. q64_stage_kernel: the activations - up to 64 rows x K, fp16 or float32 - are permuted ONCE into the formats' staged order (Fmt::stage), laid out per step
+//  1. q64_stage_kernel: the activations - up to 128 rows x K, fp16 or float32 - are permuted ONCE into the formats' staged order (Fmt::stage), laid out per step
 //     of 256 values of K as [vector][column group][unit][column] 16-byte pieces: exactly the bytes the multiplying workgroups want in LDS, rows at and beyond M
 //     as zeros.  (When every workgroup staged for itself, each of its 256 threads fetched one 128-byte line in eight instructions that touch 64 lines each:
 //     the texture path, not the matrix cores, set the pace - gate/up of the 8B shapes 54 us, of which 20 us were that fetch.)
@@ -20,7 +21,7 @@
 // Without a split the multiplying kernel stores for itself: plain, + residual (in place allowed: every element is read and written by one lane), or
 // silu(gate) * up, for which a lane's gate rows and the matching up rows sit 32 lanes apart.
 //
-// The staged activations (at most 4 MB) and the partial tiles (at most 8 MB) live in a workspace that tga_init allocates once per device: Q64_SLOTS slots, a
+// The staged activations (at most 8 MB) and the partial tiles (at most 32 MB) live in a workspace that tga_init allocates once per device: Q64_SLOTS slots, a
 // stream keeps the slot it was given first (launches of one stream are ordered, so they may share one), a call on a further stream gets none and is told to
 // run blocks of sixteen rows instead.
 #include "qfmt.h"
@@ -30,8 +31,9 @@ typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
 typedef float v4f32 __attribute__((ext_vector_type(4)));
 
 #define Q64_MAX_K 32768
-#define Q64_XS_BYTES ((size_t)64 * Q64_MAX_K * 2)
-#define Q64_PART_BYTES ((size_t)8 << 20)
+#define Q64_COLS 128                  // activation rows of a call at most = columns of a partial tile's split
+#define Q64_XS_BYTES ((size_t)Q64_COLS * Q64_MAX_K * 2)
+#define Q64_PART_BYTES ((size_t)32 << 20)
 #define Q64_SLOTS 4
 #define Q64_MAX_DEVICES 64
 #ifndef Q64_RING
@@ -45,14 +47,14 @@ struct Q64Opt { bool prestaged; const void* xs_ext; bool defer; float* part; int
 
 struct Q64X {
   u32x4* xs;            // staged activations: [step][8 vectors][NCG column groups][4 units][16 columns] pieces
-  float* part;          // (K split) partial tiles [split][64 columns][np rows]
+  float* part;          // (K split) partial tiles [split][Q64_COLS columns][np rows]
   int ks, np;
 };
 
 template <int T_, int NCG>
 __global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const int M, u32x4* __restrict__ xs) {
   using F = Fmt<T_>;
-  const int tid = threadIdx.x, scol = tid & 63, sug = tid >> 6, s = blockIdx.x;      // this thread's item: activation row scol, unit 4 s + sug
+  const int tid = threadIdx.x, scol = (tid & 63) + 64 * blockIdx.y, sug = tid >> 6, s = blockIdx.x;      // this thread's item: activation row scol, unit 4 s + sug
   if (scol >= 16 * NCG) return;
   uint32_t nx[F::UW / 2];
   stage_fetch<T_>(args, scol < M ? scol : 0, 4 * s + sug, nx);
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__
       for (int k0 = 0; k0 < ks; k0 += 8) {                // eight splits requested together, added in the order of K
         f32x4 t[8];
 #pragma unroll
-        for (int k = 0; k < 8; k++) t[k] = *(const f32x4*)(part + ((size_t)(k0 + k < ks ? k0 + k : ks - 1) * 64 + m) * np + 4 * i);
+        for (int k = 0; k < 8; k++) t[k] = *(const f32x4*)(part + ((size_t)(k0 + k < ks ? k0 + k : ks - 1) * Q64_COLS + m) * np + 4 * i);
 #pragma unroll
         for (int k = 0; k < 8; k++) if (k0 + k < ks) { v.x += t[k].x; v.y += t[k].y; v.z += t[k].z; v.w += t[k].w; }
       }
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
   static_assert(F::UW == 64 && F::XV == 8, "units of 64 weights in eight vectors");
   static_assert(!(MS && SW), "the SwiGLU pair is not combined with the q / k / v walk");
   constexpr int SP = F::XV * NCG * 64;                    // 16-byte pieces of one stage
-  constexpr int NI = SP / 256;                            // pieces per thread and stage (8 or 4)
+  constexpr int NI = SP / 256;                            // pieces per thread and stage (4, 8 or 16)
   extern __shared__ u32x4 lds[];                          // two stages of SP pieces
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g = lane >> 4;
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(512) void qgemm64_kernel(const QArgs args, const in
     if (ex.ks > 1) {                                      // partial tile: [split][column][padded row], every lane stores its four rows
 #pragma unroll
       for (int cg = 0; cg < NCG; cg++)
-        *(v4f32*)(ex.part + ((size_t)ky * 64 + 16 * cg + c) * ex.np + grow0[t] + 4 * g) = acc[t][cg];
+        *(v4f32*)(ex.part + ((size_t)ky * Q64_COLS + 16 * cg + c) * ex.np + grow0[t] + 4 * g) = acc[t][cg];
       continue;
     }
     if (!has_rows[t]) continue;
@@ -343,7 +345,7 @@ __global__ __launch_bounds__(256) void q64_reduce_kernel(const QArgs a, const in
   const int m = (int)(idx / q); long long row = 4 * (idx - (long long)m * q);
   if (m >= M) return;
   v4f32 v = *(const v4f32*)(part + (size_t)m * np + row);
-  for (int k = 1; k < ks; k++) { const v4f32 t = *(const v4f32*)(part + ((size_t)k * 64 + m) * np + row); v += t; }
+  for (int k = 1; k < ks; k++) { const v4f32 t = *(const v4f32*)(part + ((size_t)k * Q64_COLS + m) * np + row); v += t; }
   int sg = 0; long long nrows = a.n[0];
   if (a.nseg > 1 && row >= a.n[0]) { row -= a.n[0]; sg = 1; nrows = a.n[1]; if (a.nseg > 2 && row >= a.n[1]) { row -= a.n[1]; sg = 2; nrows = a.n[2]; } }
   void* yb = sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
@@ -398,11 +400,11 @@ void tga_qgemm64_release(hipStream_t s) {
       if (g_q64_taken[d][i] && g_q64_owner[d][i] == s) g_q64_taken[d][i] = false;
 }
 
-static int q64_split(bool sw, long long tiles, int nsteps) {   // workgroups per row tile: about 512 workgroups of at least four steps, partial tiles within the workspace
+static int q64_split(bool sw, long long tiles, int nsteps, int ncg) {   // workgroups per row tile: about 512 workgroups (256 with eight column groups: one per CU) of at least four steps, partial tiles within the workspace
   static const int env_ks = getenv("TGA_Q64_KS") ? atoi(getenv("TGA_Q64_KS")) : 0;
   int ks = 1;
   if (!sw && tiles < 192) {
-    ks = (int)((512 + tiles / 2) / tiles);
+    ks = (int)(((ncg == 8 ? 256 : 512) + tiles / 2) / tiles);
     if (ks > nsteps / 4) ks = nsteps / 4;
   }
   if (env_ks >= 1 && !sw) ks = env_ks < nsteps ? env_ks : nsteps;
@@ -422,11 +424,11 @@ static int launch_q64_v(const QArgs& a, int M, uint8_t* ws, Q64Opt& o, hipStream
   Q64X ex;
   ex.xs = o.xs_ext ? (u32x4*)o.xs_ext : (u32x4*)ws; ex.part = ws ? (float*)(ws + Q64_XS_BYTES) : nullptr; ex.np = (int)(tiles * 64 * NT);
   // K split: row tiles alone leave most of the 256 CUs idle when the matrix has few rows (not without a workspace slot for the partial tiles)
-  int ks = ws ? q64_split(SW, tiles, nsteps) : 1;
-  while (ks > 1 && (size_t)ks * 64 * ex.np * 4 > Q64_PART_BYTES) ks--;
+  int ks = ws ? q64_split(SW, tiles, nsteps, NCG) : 1;
+  while (ks > 1 && (size_t)ks * Q64_COLS * ex.np * 4 > Q64_PART_BYTES) ks--;
   ex.ks = ks;
   if (!o.prestaged) {
-    q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps), dim3(256), 0, s>>>(a, M, ex.xs);
+    q64_stage_kernel<T, NCG><<<dim3((unsigned)nsteps, NCG > 4 ? 2 : 1), dim3(256), 0, s>>>(a, M, ex.xs);
     TGA_LAUNCH_CHECK();
   }
   kern<<<dim3((unsigned)tiles, (unsigned)ks), dim3(512), 2 * stage_bytes, s>>>(a, M, ex);
@@ -449,7 +451,7 @@ static int launch_q64_t(const QArgs& a, int M, uint8_t* ws, Q64Opt& o, hipStream
   static const int env_nt = getenv("TGA_Q64_NT") ? atoi(getenv("TGA_Q64_NT")) : 0;
   const int nsteps = a.nu >> 2;
   const long long rows_wg2 = SW ? 64 : 128, tiles2 = (a.ntot + rows_wg2 - 1) / rows_wg2;
-  bool two = sizeof(typename F::Raw) <= 64 && tiles2 * q64_split(SW, tiles2, nsteps) >= 224;
+  bool two = sizeof(typename F::Raw) <= 64 && (NCG == 8 || tiles2 * q64_split(SW, tiles2, nsteps, NCG) >= 224);      // (eight column groups: the LDS reads of the B operands set the pace, and a B operand meets both tiles)
   if (env_nt == 1) two = false; else if (env_nt == 2) two = sizeof(typename F::Raw) <= 64;
   if constexpr (sizeof(typename F::Raw) <= 64) { if (two) return launch_q64_v<T, MS, SW, NCG, 2>(a, M, ws, o, s); }
   return launch_q64_v<T, MS, SW, NCG, 1>(a, M, ws, o, s);
@@ -464,17 +466,18 @@ static int launch_q64(QArgs a, int M, uint8_t* ws, Q64Opt& o, hipStream_t s) {
     a.row_bytes = (long long)(a.K / F::BW) * F::BB;
     // two column groups instead of four: half the MFMAs and half the staged bytes.  (One group, for up to sixteen rows, was measured and dropped: the kernel
     // streams weights at about 2.5 TB/s - Q8_0 14336 x 4096 at M = 8 24.6 us, the Q6_K lm-head 211 us - where the LDS-fed small-batch kernels take 18.4 / 134.)
-    const bool two = M <= 32;
-    if (a.epilogue == 2) return two ? launch_q64_t<T, false, true, 2>(a, M, ws, o, s) : launch_q64_t<T, false, true, 4>(a, M, ws, o, s);
-    if (a.nseg > 1) return two ? launch_q64_t<T, true, false, 2>(a, M, ws, o, s) : launch_q64_t<T, true, false, 4>(a, M, ws, o, s);
-    return two ? launch_q64_t<T, false, false, 2>(a, M, ws, o, s) : launch_q64_t<T, false, false, 4>(a, M, ws, o, s);
+    // Eight groups (65 .. 128 rows): a pass over the weights costs what it costs at 64 rows - the weight stream, not the matrix cores, sets its pace.
+    const int ncg = M <= 32 ? 2 : M <= 64 ? 4 : 8;
+    if (a.epilogue == 2) return ncg == 2 ? launch_q64_t<T, false, true, 2>(a, M, ws, o, s) : ncg == 4 ? launch_q64_t<T, false, true, 4>(a, M, ws, o, s) : launch_q64_t<T, false, true, 8>(a, M, ws, o, s);
+    if (a.nseg > 1) return ncg == 2 ? launch_q64_t<T, true, false, 2>(a, M, ws, o, s) : ncg == 4 ? launch_q64_t<T, true, false, 4>(a, M, ws, o, s) : launch_q64_t<T, true, false, 8>(a, M, ws, o, s);
+    return ncg == 2 ? launch_q64_t<T, false, false, 2>(a, M, ws, o, s) : ncg == 4 ? launch_q64_t<T, false, false, 4>(a, M, ws, o, s) : launch_q64_t<T, false, false, 8>(a, M, ws, o, s);
   }
 }
 
-// Whether the call is inside this kernel's range: 17 .. 64 rows of fp16 or float32 activations, K a multiple of 256 up to Q64_MAX_K, one to three matrices
+// Whether the call is inside this kernel's range: 17 .. 128 rows of fp16 or float32 activations, K a multiple of 256 up to Q64_MAX_K, one to three matrices
 // (several: each a multiple of 16 rows) with the plain or residual epilogue, or the SwiGLU pair, in one of the formats with units of 64 weights.
 static bool q64_in_range(int fmt, const QArgs& a, int M) {
-  if (M < 17 || M > 64 || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || (a.y_stage_fmt && a.epilogue != 2) || a.norm_w || a.comb_y) return false;
+  if (M < 17 || M > Q64_COLS || a.K % 256 != 0 || a.K > Q64_MAX_K || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || (a.y_stage_fmt && a.epilogue != 2) || a.norm_w || a.comb_y) return false;
   if (a.nseg > 1 && a.epilogue != 2) for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0) return false;
   if (((uintptr_t)a.x & 15) != 0) return false;
   if (a.y_stage_fmt && (a.y_f32 || a.y_stage_nu != (int)(a.n[0] / 64) || a.n[0] % 256 != 0)) return false;   // (staged SwiGLU rows: the consumer's K is this N)
@@ -486,7 +489,7 @@ static bool q64_in_range(int fmt, const QArgs& a, int M) {
 // is outside the kernel's range or the stream holds no workspace slot.  The call that follows passes prestaged = true.
 void* tga_qgemm64_staging(int fmt, const QArgs& a, int M, hipStream_t s, int* ncg) {
   if (!q64_in_range(fmt, a, M)) return nullptr;
-  *ncg = M <= 32 ? 2 : 4;
+  *ncg = M <= 32 ? 2 : M <= 64 ? 4 : 8;
   return q64_slot(s);
 }
 
@@ -497,9 +500,11 @@ static int launch_norm_stage(float* x, const float* w, int K, float eps, void* x
   else {
     static const hipError_t c2 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     static const hipError_t c4 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    TGA_HIP(c2); TGA_HIP(c4);
+    static const hipError_t c8 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    TGA_HIP(c2); TGA_HIP(c4); TGA_HIP(c8);
     if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
-    else q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    else if (ncg == 4) q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    else q64_norm_stage_kernel<T, 8><<<dim3(128), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
     TGA_LAUNCH_CHECK();
     return 0;
   }
@@ -508,7 +513,7 @@ static int launch_norm_stage(float* x, const float* w, int K, float eps, void* x
 // buffer of a consumer of format fmt in the multiplying layout (tga_qgemm64_staging's, or the caller's).  part != nullptr: the rows are first completed in place with
 // the partial tiles of a deferred linear (ks splits, row pitch np).  -1: outside the range.
 int tga_qgemm64_norm_stage(int fmt, float* x, const float* w, int K, float eps, void* xn_out, void* staged, int M, int ncg, const float* part, int ks, int np, hipStream_t s) {
-  if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)xn_out | (uintptr_t)staged | (uintptr_t)part) & 15) != 0 || K % 256 != 0 || K > Q64_MAX_K || M < 1 || M > 16 * ncg || (ncg != 2 && ncg != 4)) return -1;
+  if ((((uintptr_t)x | (uintptr_t)w | (uintptr_t)xn_out | (uintptr_t)staged | (uintptr_t)part) & 15) != 0 || K % 256 != 0 || K > Q64_MAX_K || M < 1 || M > 16 * ncg || (ncg != 2 && ncg != 4 && ncg != 8)) return -1;
   if (part && (ks < 1 || np < K || np % 4 != 0)) return -1;
   switch (fmt) {
     case F_Q4_0P: return launch_norm_stage<F_Q4_0P>(x, w, K, eps, xn_out, staged, M, ncg, part, ks, np, s);

@@ -365,7 +365,7 @@ struct AttnIn { int n_splits, head_dim; const int* touch_pos; const void* k; con
 static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const float* norm_w, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream);
-// the 64-column kernel's format for a weight of this type with rows of K values, -1: none (block pairs need an even number of blocks; K in steps of 256)
+// the prefill kernel's format for a weight of this type with rows of K values, -1: none (block pairs need an even number of blocks; K in steps of 256)
 static int q64_fmt_of(int ggml_type, int64_t K) {
   if (K <= 0 || K % 256 != 0) return -1;
   switch (ggml_type) {
@@ -374,7 +374,7 @@ static int q64_fmt_of(int ggml_type, int64_t K) {
   }
   return -1;
 }
-// the arguments of the 17 .. 64 row GEMM (qgemm64.hip) for a call whose pointers and epilogue have been checked; false: a format or alignment it does not take
+// the arguments of the 17 .. 128 row GEMM (qgemm64.hip) for a call whose pointers and epilogue have been checked; false: a format or alignment it does not take
 static bool q64_args(int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n, const void* x, int x_dtype, int y_dtype, int64_t K,
                      int epilogue, const void* const* resid, QArgs& q, int& fmt64) {
   bool pair64 = K > 0 && (K / 32) % 2 == 0;
@@ -409,11 +409,11 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
                               const void* x, int x_dtype, int y_dtype, int M, int64_t K,
                               int epilogue, const void* const* resid, int y_stage_type, int64_t y_stage_K, void* stream) {
   TGA_REQUIRE(nseg >= 1 && nseg <= QG_MAX_SEG, "tga_qlinear_multi: nseg=%d out of range 1..%d", nseg, QG_MAX_SEG);
-  TGA_REQUIRE(M >= 1 && M <= 64, "tga_qlinear: M=%d out of range 1..64", M);
-  // 17 .. 64 rows (prefill steps): one pass over the weights on the 64-column kernel where it applies (qgemm64.hip), else blocks of sixteen rows (every block
+  TGA_REQUIRE(M >= 1 && M <= 128, "tga_qlinear: M=%d out of range 1..128", M);
+  // 17 .. 128 rows (prefill steps): one pass over the weights on the prefill kernel where it applies (qgemm64.hip), else blocks of sixteen rows (every block
   // after the first finds the weights in the Infinity Cache)
   if (M > 16) {
-    // x_dtype TGA_F16_STAGED: x holds the rows in the layout the 64-column kernel multiplies from (written by tga_rmsnorm_rows_stage, by a SwiGLU launch with
+    // x_dtype TGA_F16_STAGED: x holds the rows in the layout the prefill kernel multiplies from (written by tga_rmsnorm_rows_stage, by a SwiGLU launch with
     // y_stage_type, or by tga_attention_prefill_chunk_staged); y_stage_type (SwiGLU): the fp16 rows are written in that layout for a consumer of that type
     const bool xst = x_dtype == TGA_F16_STAGED;
     TGA_REQUIRE(!comb && !norm_w && (x_dtype == TGA_F16 || x_dtype == TGA_F32 || xst) && x && (epilogue != 1 || resid) && epilogue >= 0 && epilogue <= 2,
@@ -433,7 +433,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
         if (rc >= 0) return rc;
       }
     }
-    TGA_REQUIRE(!xst && !y_stage_type, "tga_qlinear: rows in the multiplying layout are outside the 64-column kernel's range here (tga_rows_staged_plan says which linears take them)");
+    TGA_REQUIRE(!xst && !y_stage_type, "tga_qlinear: rows in the multiplying layout are outside the prefill kernel's range here (tga_rows_staged_plan says which linears take them)");
     return qlinear_row_blocks(16, ggml_type, nseg, w, y, n, x, x_dtype, y_dtype, M, K, epilogue, resid, stream);
   }
   TGA_REQUIRE(x_dtype == TGA_F16 || x_dtype == TGA_F32 || x_dtype == TGA_F16_STAGED, "tga_qlinear: x_dtype must be TGA_F16, TGA_F32 or TGA_F16_STAGED");
@@ -627,7 +627,7 @@ extern "C" int tga_rmsnorm_qlinear_mixed(const float* norm_weight, float norm_ep
 extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps, int ggml_type, int nseg, const void* const* w, void* const* y, const int64_t* n,
                                         const float* x, void* xn_scratch_f16, int y_dtype, int M, int64_t K, int epilogue, const void* const* resid, void* stream) {
   TGA_REQUIRE(norm_weight && x && xn_scratch_f16, "tga_rmsnorm_qlinear_rows: null pointer");
-  TGA_REQUIRE(M >= 1 && M <= 64 && K > 0 && K <= (1 << 24), "tga_rmsnorm_qlinear_rows: M=%d (1..64), K=%lld", M, (long long)K);
+  TGA_REQUIRE(M >= 1 && M <= 128 && K > 0 && K <= (1 << 24), "tga_rmsnorm_qlinear_rows: M=%d (1..128), K=%lld", M, (long long)K);
   // up to eight rows: beyond, what every workgroup reads and normalises again (M float32 rows) costs more than the norm's own launch (8B-arch prefill in
   // chunks of sixteen: 208 ms folded against 195 ms; chunks of eight 320 against 328, of four 562 against 610)
   if (M >= 2 && M <= 8 && ((uintptr_t)norm_weight & 15) == 0) {
@@ -636,7 +636,7 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
   }
   if (M > 16 && nseg >= 1 && nseg <= QG_MAX_SEG && w && y && n && (y_dtype == TGA_F16 || y_dtype == TGA_F32) && epilogue >= 0 && epilogue <= 2 && (epilogue != 1 || (resid && y_dtype == TGA_F32)) &&
       (epilogue != 2 || (nseg == 2 && n[0] == n[1]))) {
-    // 17 .. 64 rows on the 64-column kernel: the norm's launch writes the rows in the layout that kernel multiplies from as well (no staging launch)
+    // 17 .. 128 rows on the prefill kernel: the norm's launch writes the rows in the layout that kernel multiplies from as well (no staging launch)
     bool ok = true;
     for (int i = 0; i < nseg; i++) ok = ok && n[i] > 0 && w[i] && (y[i] || (epilogue == 2 && i == 1)) && (epilogue != 1 || resid[i]);
     QArgs q; int fmt64, ncg = 0;
@@ -658,28 +658,28 @@ extern "C" int tga_rmsnorm_qlinear_rows(const float* norm_weight, float norm_eps
   return qlinear_multi_impl(nullptr, nullptr, nullptr, 0.f, ggml_type, nseg, w, y, n, xn_scratch_f16, TGA_F16, y_dtype, M, K, epilogue, resid, 0, 0, stream);
 }
 
-// ---- a prefill step of 17 .. 64 rows with the rows handed from launch to launch in the layout the 64-column kernel multiplies from, and the split-K sums of the
+// ---- a prefill step of 17 .. 128 rows with the rows handed from launch to launch in the layout the prefill kernel multiplies from, and the split-K sums of the
 // residual linears completed by the norm launch behind them (llm.BatchedTransformer's step for chunks of more than sixteen positions)
 
 // Whether a linear of this type with rows of K values takes M activation rows in the multiplying layout: *ncg = column groups of sixteen rows (2 or 4; the buffer holds
 // 16 ncg x K fp16 values), 0 = no.
 extern "C" int tga_rows_staged_plan(int ggml_type, int64_t K, int M, int* ncg) {
   TGA_REQUIRE(ncg, "tga_rows_staged_plan: null pointer");
-  *ncg = (M >= 17 && M <= 64 && K <= 32768 && q64_fmt_of(ggml_type, K) >= 0) ? (M <= 32 ? 2 : 4) : 0;
+  *ncg = (M >= 17 && M <= 128 && K <= 32768 && q64_fmt_of(ggml_type, K) >= 0) ? (M <= 32 ? 2 : M <= 64 ? 4 : 8) : 0;
   return 0;
 }
 
 // y = y + x W^T for one matrix (attn_output, ffn_down: the residual adds of model.py:149-150) over rows in the multiplying layout.  When the kernel splits K, the sum over
-// the splits is NOT taken: *partials / *ks / *np describe the partial tiles (in the stream's workspace, valid until the next call of 17 .. 64 rows on this stream) and y is
+// the splits is NOT taken: *partials / *ks / *np describe the partial tiles (in the stream's workspace, valid until the next call of 17 .. 128 rows on this stream) and y is
 // untouched - tga_rmsnorm_rows_stage (or tga_rows_add_partials) completes it.  *ks = 0: nothing is pending, y is complete.
 extern "C" int tga_qlinear_rows_deferred(int ggml_type, const void* w, int64_t N, int64_t K, const void* x_staged, int M, float* y, const float** partials, int* ks, int* np, void* stream) {
   TGA_REQUIRE(w && x_staged && y && partials && ks && np && N > 0, "tga_qlinear_rows_deferred: null pointer or no rows");
   const void* wv[1] = {w}; void* yv[1] = {y}; const void* rv[1] = {y}; const int64_t nv[1] = {N};
   QArgs q; int fmt64;
-  TGA_REQUIRE(q64_args(ggml_type, 1, wv, yv, nv, x_staged, TGA_F16, TGA_F32, K, 1, rv, q, fmt64), "tga_qlinear_rows_deferred: type %d with K=%lld is outside the 64-column kernel's range", ggml_type, (long long)K);
+  TGA_REQUIRE(q64_args(ggml_type, 1, wv, yv, nv, x_staged, TGA_F16, TGA_F32, K, 1, rv, q, fmt64), "tga_qlinear_rows_deferred: type %d with K=%lld is outside the prefill kernel's range", ggml_type, (long long)K);
   Q64Opt o = {true, x_staged, true, nullptr, 0, 0};
   const int rc = tga_qgemm64_dispatch(fmt64, q, M, o, (hipStream_t)stream);
-  TGA_REQUIRE(rc >= 0, "tga_qlinear_rows_deferred: M=%d, N=%lld, K=%lld outside the 64-column kernel's range", M, (long long)N, (long long)K);
+  TGA_REQUIRE(rc >= 0, "tga_qlinear_rows_deferred: M=%d, N=%lld, K=%lld outside the prefill kernel's range", M, (long long)N, (long long)K);
   *partials = o.part; *ks = o.ks; *np = o.np;
   return rc;
 }
@@ -687,17 +687,17 @@ extern "C" int tga_qlinear_rows_deferred(int ggml_type, const void* w, int64_t N
 // RMSNorm of `rows` float32 rows (nn.RMSNorm, tinygrad/nn/__init__.py:296-304) written as fp16 in the multiplying layout of a consumer of consumer_type (and, when
 // xn_out is given, as plain fp16 rows).  partials != NULL: every row is first completed in place with the partial tiles a tga_qlinear_rows_deferred call left.
 extern "C" int tga_rmsnorm_rows_stage(float* x, const float* partials, int ks, int np, const float* weight, float eps, int rows, int dim, int consumer_type, void* xn_out_f16, void* staged_out, void* stream) {
-  TGA_REQUIRE(x && weight && staged_out && rows >= 17 && rows <= 64, "tga_rmsnorm_rows_stage: null pointer or rows=%d outside 17..64", rows);
+  TGA_REQUIRE(x && weight && staged_out && rows >= 17 && rows <= 128, "tga_rmsnorm_rows_stage: null pointer or rows=%d outside 17..128", rows);
   const int fmt = q64_fmt_of(consumer_type, dim);
   TGA_REQUIRE(fmt >= 0, "tga_rmsnorm_rows_stage: no multiplying layout for type %d with K=%d", consumer_type, dim);
-  const int rc = tga_qgemm64_norm_stage(fmt, x, weight, dim, eps, xn_out_f16, staged_out, rows, rows <= 32 ? 2 : 4, partials, ks, np, (hipStream_t)stream);
+  const int rc = tga_qgemm64_norm_stage(fmt, x, weight, dim, eps, xn_out_f16, staged_out, rows, rows <= 32 ? 2 : rows <= 64 ? 4 : 8, partials, ks, np, (hipStream_t)stream);
   TGA_REQUIRE(rc >= 0, "tga_rmsnorm_rows_stage: pointers must be 16-byte aligned, dim a multiple of 256 up to 32768");
   return rc;
 }
 
 // x += the sum of the partial tiles a tga_qlinear_rows_deferred call left (what its own reduce launch would have done): rows x dim float32
 extern "C" int tga_rows_add_partials(float* x, const float* partials, int ks, int np, int rows, int dim, void* stream) {
-  TGA_REQUIRE(x && partials && ks >= 1 && np >= dim && np % 4 == 0 && rows >= 1 && rows <= 64 && dim > 0, "tga_rows_add_partials: null pointer or ks=%d np=%d rows=%d dim=%d", ks, np, rows, dim);
+  TGA_REQUIRE(x && partials && ks >= 1 && np >= dim && np % 4 == 0 && rows >= 1 && rows <= 128 && dim > 0, "tga_rows_add_partials: null pointer or ks=%d np=%d rows=%d dim=%d", ks, np, rows, dim);
   return tga_qgemm64_add_partials(x, partials, ks, np, rows, dim, (hipStream_t)stream);
 }
 

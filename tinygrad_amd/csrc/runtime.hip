@@ -25,7 +25,7 @@ int tga_init(int device) {
   TGA_HIP(hipGetDeviceProperties(&p, device));
   TGA_REQUIRE(strncmp(p.gcnArchName, "gfx950", 6) == 0, "tga_init: kernels are built for gfx950 only, device is %s", p.gcnArchName);
   if (const int rc = tga_route_scratch_setup(device)) return rc;   // device address of the static workspace of tga_moe_route_static on this GPU
-  return tga_qgemm64_setup(device);                          // workspace of the 17 .. 64 row GEMM (staged activations, split-K partial tiles)
+  return tga_qgemm64_setup(device);                          // workspace of the 17 .. 128 row GEMM (staged activations, split-K partial tiles)
 }
 
 int tga_device_name(char* buf, size_t len) {
@@ -69,7 +69,7 @@ int tga_sync(void) { TGA_HIP(hipDeviceSynchronize()); return 0; }
 
 int tga_stream_create(void** stream) { TGA_HIP(hipStreamCreate((hipStream_t*)stream)); return 0; }   // default priority only
 int tga_stream_destroy(void* stream) {
-  // waits for the stream's work first: the workspace slot of the 17 .. 64 row GEMM that the stream holds may then pass to another stream at once
+  // waits for the stream's work first: the workspace slot of the 17 .. 128 row GEMM that the stream holds may then pass to another stream at once
   TGA_HIP(hipStreamSynchronize((hipStream_t)stream));
   tga_qgemm64_release((hipStream_t)stream);
   TGA_HIP(hipStreamDestroy((hipStream_t)stream));

@@ -374,7 +374,7 @@ class Transformer:
     self._cached_tokens, self._last_input, self.prefill_steps = [], None, 0   # tokens whose K / V rows the cache holds (KV-prefix reuse, model.py:455-462)
     self.replay = "cmdlist"                                          # how a captured step is replayed: "cmdlist" (plain launches in capture order) or "graph" (hipGraphLaunch)
     self._state_dict, self._chunker, self._tail_chunkers = state_dict, None, {}   # (references to the weight buffers: the chunked prefill builds its linears over the same bytes)
-    self.prefill_chunk = 64                                          # prompt positions per prefill step, 2..64 (the reference's chunks hold 32, model.py:464; MoE models: at most 16); 1: token by token
+    self.prefill_chunk = 128                                         # prompt positions per prefill step, 2..128 (the reference's chunks hold 32, model.py:464; MoE models: at most 16); 1: token by token
 
   def check_state(self):
     """Raises when a kernel of the last steps refused its input (state.error: bit 0 = a token id outside the vocabulary reached the embedding
@@ -515,14 +515,14 @@ class Transformer:
     self._cached_tokens = self._cached_tokens[:start]                   # the rows from here on are about to be overwritten: if a step below raises, they are not claimed
     B = self.prefill_chunk if on_block is None else 1
     if B > 16 and self.config.num_experts: B = 16                       # (MoE blocks keep steps of sixteen positions: longer ones are not measured there)
-    # Whole chunks as small-batch steps (model.py:476-481) of the largest size that the prompt holds (the chosen one, else 32, 16, 8 or 4 positions).  Dense models: what
+    # Whole chunks as small-batch steps (model.py:476-481) of the largest size that the prompt holds (the chosen one, else 64, 32, 16, 8 or 4 positions).  Dense models: what
     # they leave is ONE more chunk that ends at the last position and computes some positions again - every row of a step depends on the cache and on its own token
     # only, so the same values are written again - instead of a ladder of smaller steps and up to three single ones (seven steps, a tenth of a 1023-position prefill).
     # MoE models keep the ladder (one step each of 8 and / or 4 positions, then single ones).
     overlap = not self.config.num_experts
-    for b in [B] + [t for t in (32, 16, 8, 4) if t < B]:
+    for b in [B] + [t for t in (64, 32, 16, 8, 4) if t < B]:
       total = len(tokens) - 1 - start
-      if not 2 <= b <= 64 or total < b: continue
+      if not 2 <= b <= 128 or total < b: continue
       if b == B:
         if self._chunker is None or self._chunker.batch != B: self._chunker = BatchedTransformer(self.config, self._state_dict, B, max_new=1, chunk_of=self)
         chunker = self._chunker
@@ -585,7 +585,7 @@ class BatchedTransformer:
   def __init__(self, config: TransformerConfig, state_dict: dict, batch: int, max_new: int = 1024, chunk_of: "Transformer | None" = None):
     """chunk_of: the rows are `batch` consecutive prompt positions of that Transformer's sequence instead of `batch` sequences (chunked prefill,
     model.py:464, 476-481): its KV caches and rotation table are used, the attention is causal inside the chunk, no token is sampled."""
-    if not 1 <= batch <= (16 if chunk_of is None else 64): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..16")
+    if not 1 <= batch <= (16 if chunk_of is None else 128): raise ValueError(f"batch of {batch} sequences is outside the decode range 1..16")
     self.config, self.batch, self.max_new = config, batch, max_new
     # (no reference back to the Transformer: a cycle would leave its buffers to the cycle collector, which may free them in the middle of a stream capture)
     self.chunked, self._owner_stream = chunk_of is not None, (chunk_of.stream if chunk_of is not None else None)
@@ -649,17 +649,17 @@ class BatchedTransformer:
     self._graphs, self._steps_done = {}, 0
     self.replay = "cmdlist"                                          # as Transformer.replay
     self.expert_path = os.environ.get("TGA_EXPERT_PATH", "jobs")      # "jobs": one GEMV per (sequence, slot); "grouped": one small-batch GEMM per selected expert
-    # Prefill steps of 17 .. 64 positions of a dense model: the rows pass from launch to launch in the layout the 64-column GEMM multiplies from (norm -> q/k/v and gate/up,
+    # Prefill steps of 17 .. 128 positions of a dense model: the rows pass from launch to launch in the layout the prefill GEMM multiplies from (norm -> q/k/v and gate/up,
     # attention -> attn_output, SwiGLU -> ffn_down: no staging launches) and the split-K sums of attn_output / ffn_down are completed by the norm launch behind them
     self.rows64 = 0
-    if self.chunked and 17 <= B <= 64 and not c.num_experts and os.environ.get("TGA_ROWS64", "1") == "1":
+    if self.chunked and 17 <= B <= 128 and not c.num_experts and os.environ.get("TGA_ROWS64", "1") == "1":
       def ncg_of(l):
         n = ctypes.c_int(0); rt.check(rt.lib().tga_rows_staged_plan(l.ggml_type, l.in_features, B, ctypes.byref(n))); return n.value
       ok = all("bias" not in b and not b["moe"] and b["ffn_gate"].ggml_type == b["ffn_up"].ggml_type
                and all(ncg_of(b[nm]) for nm in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"))
                and all(b[nm].out_features % 16 == 0 for nm in ("attn_q", "attn_k", "attn_v")) for b in self.blk)
       if ok and c.dim % 256 == 0 and c.hidden_dim % 256 == 0 and nq % 256 == 0:
-        self.rows64 = 2 if B <= 32 else 4                              # column groups of sixteen rows in the layout
+        self.rows64 = 2 if B <= 32 else 4 if B <= 64 else 8             # column groups of sixteen rows in the layout
         R = 16 * self.rows64
         self.xn_st, self.attn_st, self.act_st = Buffer((R, c.dim), f16).zero_(), Buffer((R, nq), f16).zero_(), Buffer((R, c.hidden_dim), f16).zero_()
 
@@ -753,7 +753,7 @@ class BatchedTransformer:
                                     self.out_tokens.ptr, self.max_new, st))
 
   def _blocks_rows64(self, done):
-    """The blocks of a prefill step of 17 .. 64 rows (see rows64 in __init__): per block norm (+ the pending split-K sums of the linear before it) -> q/k/v -> attention ->
+    """The blocks of a prefill step of 17 .. 128 rows (see rows64 in __init__): per block norm (+ the pending split-K sums of the linear before it) -> q/k/v -> attention ->
     attn_output (sums deferred) -> norm -> gate/up + SwiGLU -> ffn_down (sums deferred); what the last block leaves pending is added at the end."""
     c, B, L, st = self.config, self.batch, rt.lib(), self.stream.handle
     VP2, I2 = ctypes.c_void_p * 2, ctypes.c_int64 * 2

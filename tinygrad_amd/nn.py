@@ -24,7 +24,7 @@ class QuantLinear:
     """x: (..., in_features) float16 or float32 with at most 8 rows (up to 16 for prefill chunks).  Returns (rows, out_features); the caller may pass `out`."""
     assert x.shape[-1] == self.in_features, f"{x.shape} vs in_features {self.in_features}"
     m = int(np.prod(x.shape[:-1], dtype=np.int64)) if len(x.shape) > 1 else 1
-    assert 1 <= m <= 64, f"batch of {m} rows is outside the range 1..64"
+    assert 1 <= m <= 128, f"batch of {m} rows is outside the range 1..128"
     if out is None: out = Buffer((*x.shape[:-1], self.out_features), out_dtype or x.dtype)
     assert out.nbytes == m * self.out_features * out.dtype.itemsize
     rt.check(rt.lib().tga_qlinear(self.ggml_type, self.blocks.ptr, x.ptr, rt.dtype_code(x.dtype), out.ptr, rt.dtype_code(out.dtype),
