@@ -17,8 +17,8 @@ HBM_PEAK_GBS = 8000.0
 # `python -m tinygrad_amd.benchmarks --traffic`, each scaled by what the same counter reads for a 1 GiB copy kernel (x2.0000 and x1.0000):
 # 66 509 824 B fetched + 71 680 B written.  A recorded figure (profiles/qgemv1_gate_up_hbm_traffic.md), not re-measured by this run.
 GATE_UP_TRAFFIC_BYTES = 66581504
-GATE_UP_ROCPROF_AVG_US = 15.11    # rocprofv3 --kernel-trace --stats average of the same kernel over every call of an eagerly launched run (profiles/decode_llama3_8b_q4_0_kernel_stats.md)
-GATE_UP_ROCPROF_B2B_US = 14.51    # the same trace, only the passes that issue the 32 launches back to back (the region the HIP events below bracket)
+GATE_UP_ROCPROF_AVG_US = 15.17    # rocprofv3 --kernel-trace --stats average of the same kernel over every call of an eagerly launched run (profiles/decode_llama3_8b_q4_0_kernel_stats.md)
+GATE_UP_ROCPROF_B2B_US = 14.40    # the same trace, only the passes that issue the 32 launches back to back (the region the HIP events below bracket)
 PARITY_TOL = 1e-3
 
 def _host_layer(model, i):
