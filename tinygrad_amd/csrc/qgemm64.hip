@@ -71,16 +71,16 @@ __global__ __launch_bounds__(256) void q64_stage_kernel(const QArgs args, const 
 // part != nullptr: the row is first completed in place as x + the sum of the partial tiles a deferred linear left (ks splits of [64][np] float32, in the order of K:
 // what q64_reduce_kernel would have written).
 template <int T_, int NCG>
-__global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__ x, const float* __restrict__ w, const int K, const float eps,
+__global__ __launch_bounds__(1024) void q64_norm_stage_kernel(float* __restrict__ x, const float* __restrict__ w, const int K, const float eps,
                                                              _Float16* __restrict__ xn_out, u32x4* __restrict__ xs, const int M,
                                                              const float* __restrict__ part, const int ks, const int np) {
   using F = Fmt<T_>;
   extern __shared__ u32x4 lds[];                          // the normalised fp16 row
-  __shared__ float red[4];
-  const int m = blockIdx.x, tid = threadIdx.x, nu = K >> 6;
+  __shared__ float red[16];
+  const int m = blockIdx.x, tid = threadIdx.x, nu = K >> 6, nth = blockDim.x;      // 256 or 1024 threads: with one 16-byte piece of the row per thread the partial tiles of all splits are requested in one round trip
   auto dst_of = [&](int u) { return xs + (size_t)(u >> 2) * (F::XV * NCG * 64) + (m >> 4) * 64 + (u & 3) * 16 + (m & 15); };
   if (m >= M) {
-    for (int u = tid; u < nu; u += 256) {
+    for (int u = tid; u < nu; u += nth) {
       u32x4* dst = dst_of(u);
 #pragma unroll
       for (int v = 0; v < F::XV; v++) dst[v * NCG * 64] = u32x4{0u, 0u, 0u, 0u};
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__
   const f32x4* wr = (const f32x4*)w;
   const int n4 = K >> 2;
   float s = 0.f;
-  for (int i = tid; i < n4; i += 256) {
+  for (int i = tid; i < n4; i += nth) {
     f32x4 v = xr[i];
     if (part) {                                           // (the same thread reads this piece again below: its own store, in program order)
       for (int k0 = 0; k0 < ks; k0 += 8) {                // eight splits requested together, added in the order of K
@@ -108,10 +108,12 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__
   s = wave_sum(s);
   if ((tid & 63) == 0) red[tid >> 6] = s;
   __syncthreads();
-  const float scale = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)K + eps);
+  float tot = 0.f;
+  for (int j = 0; j < (nth >> 6); j++) tot += red[j];
+  const float scale = 1.0f / sqrtf(tot / (float)K + eps);
   uint32_t* row32 = (uint32_t*)lds;
   uint32_t* out32 = (uint32_t*)(xn_out + (size_t)m * K);
-  for (int i = tid; i < n4; i += 256) {
+  for (int i = tid; i < n4; i += nth) {
     const f32x4 v = xr[i], g = wr[i];
     const uint32_t lo = f2h_bits((v.x * scale) * g.x) | (f2h_bits((v.y * scale) * g.y) << 16), hi = f2h_bits((v.z * scale) * g.z) | (f2h_bits((v.w * scale) * g.w) << 16);
     row32[2 * i] = lo; row32[2 * i + 1] = hi;
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(256) void q64_norm_stage_kernel(float* __restrict__
   __syncthreads();
   QArgs q = {};
   q.x = (const void*)lds; q.x_f32 = 0; q.K = K;
-  for (int u = tid; u < nu; u += 256) {
+  for (int u = tid; u < nu; u += nth) {
     uint32_t nx[F::UW / 2];
     stage_fetch<T_>(q, 0, u, nx);
     u32x4 xv[F::XV]; float cs[F::NG];
@@ -502,9 +504,11 @@ static int launch_norm_stage(float* x, const float* w, int K, float eps, void* x
     static const hipError_t c4 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     static const hipError_t c8 = hipFuncSetAttribute((const void*)q64_norm_stage_kernel<T, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
     TGA_HIP(c2); TGA_HIP(c4); TGA_HIP(c8);
-    if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
-    else if (ncg == 4) q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
-    else q64_norm_stage_kernel<T, 8><<<dim3(128), dim3(256), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    static const int env_nth = getenv("TGA_NS_THREADS") ? atoi(getenv("TGA_NS_THREADS")) : 0;
+    const int nth = env_nth == 256 || env_nth == 1024 ? env_nth : (K >= 4096 ? 1024 : 256);
+    if (ncg == 2) q64_norm_stage_kernel<T, 2><<<dim3(32), dim3(nth), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    else if (ncg == 4) q64_norm_stage_kernel<T, 4><<<dim3(64), dim3(nth), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
+    else q64_norm_stage_kernel<T, 8><<<dim3(128), dim3(nth), (size_t)K * 2, s>>>(x, w, K, eps, (_Float16*)xn_out, (u32x4*)staged, M, part, ks, np);
     TGA_LAUNCH_CHECK();
     return 0;
   }
