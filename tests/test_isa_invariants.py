@@ -1,4 +1,4 @@
-"""Guards for the inline-assembly loads of csrc/qgemm_dma.hip (CPU only: the file is compiled to gfx950 assembly and read as text).
+"""Guards for the inline-assembly loads of csrc/qgemm_dma.hip and csrc/qgemm_wp.hip (CPU only: the files are compiled to gfx950 assembly and read as text).
 
 The kernel requests activations with `global_load_dwordx4` written as inline assembly and waits for them with a hand-counted `s_waitcnt vmcnt(n)`, so
 that weight pieces issued behind them stay in flight.  The compiler takes the destination registers for valid as soon as the request is issued: if it
@@ -9,7 +9,7 @@ import os, pathlib, re, subprocess, tempfile
 import pytest
 from tinygrad_amd import build as tb
 
-SRC = tb.CSRC / "qgemm_dma.hip"
+SOURCES = {"qgemm_dma.hip": (r"^(_Z16qgemm_dma_kernelI\w+EEv5QArgsii):", 19), "qgemm_wp.hip": (r"^(_Z15qgemm_wp_kernelI\w+EEv5QArgsii):", 12)}
 
 def _regs(line: str) -> set:
   out, code = set(), line.split(";")[0]
@@ -17,19 +17,20 @@ def _regs(line: str) -> set:
   for m in re.finditer(r"\bv(\d+)\b", code): out.add(int(m.group(1)))
   return out
 
-@pytest.fixture(scope="module")
-def kernels():
+@pytest.fixture(scope="module", params=sorted(SOURCES))
+def kernels(request):
   try: hipcc = tb._hipcc()
   except RuntimeError: pytest.skip("hipcc not found")
+  pattern, at_least = SOURCES[request.param]
   with tempfile.TemporaryDirectory() as d:
-    out = pathlib.Path(d) / "qgemm_dma.s"
-    r = subprocess.run([hipcc, *tb.HIPCC_FLAGS, "--cuda-device-only", "-S", str(SRC), "-o", str(out)], capture_output=True, text=True)
+    out = pathlib.Path(d) / (request.param + ".s")
+    r = subprocess.run([hipcc, *tb.HIPCC_FLAGS, "--cuda-device-only", "-S", str(tb.CSRC / request.param), "-o", str(out)], capture_output=True, text=True)
     if r.returncode != 0: pytest.fail(f"hipcc -S failed:\n{r.stderr[-2000:]}")
     text = out.read_text()
   ks = {}
-  for name in re.findall(r"^(_Z16qgemm_dma_kernelI\w+EEv5QArgsii):", text, re.M):
+  for name in re.findall(pattern, text, re.M):
     ks[name] = text[text.index("\n" + name + ":"):text.index(".set " + name + ".uses_flat_scratch")].split("\n")
-  assert len(ks) >= 19, sorted(ks)
+  assert len(ks) >= at_least, sorted(ks)
   return text, ks
 
 def test_no_scratch(kernels):
@@ -46,12 +47,17 @@ def _touches_in_flight(L):
   analysis); an instruction that names a register in flight - other than a request that overwrites it - is a finding.  Returns the findings as (line number, text)."""
   ins = []                                                                     # (line index, text) of instructions; labels -> index of the next instruction
   labels = {}
+  in_asm, has_marks = False, any(l.strip().startswith(";;#ASMSTART") for l in L)   # (hand-made listings carry no ASMSTART / ASMEND: every request counts there)
   for i, l in enumerate(L):
     m = re.match(r"(\.LBB\d+_\d+):", l)
     if m: labels[m.group(1)] = len(ins); continue
+    if l.strip().startswith(";;#ASMSTART"): in_asm = True; continue
+    if l.strip().startswith(";;#ASMEND"): in_asm = False; continue
     if l.strip() == "; landed": ins.append((i, "; landed")); continue
     t = l.split(";")[0].strip()
     if not l.startswith("\t") or not t or t.startswith("."): continue
+    # a 16-byte load that the compiler wrote (it places that load's wait itself) is an ordinary instruction here, not a request
+    if has_marks and not in_asm and t.startswith("global_load_dwordx4"): t = "compiler_" + t
     ins.append((i, t))
   n = len(ins)
   succ = [[] for _ in range(n)]
@@ -97,3 +103,27 @@ def test_the_check_itself():
   assert [t for _, t in _touches_in_flight(branch)] == ["v_add_u32_e32 v6, v1, v2"]
   loop = [".LBB0_1:", "\tv_mov_b32_e32 v9, v4", "\t; landed", "\tds_write_b128 v1, v[4:7]", "\tglobal_load_dwordx4 v[4:7], v[2:3], off", "\ts_cbranch_scc1 .LBB0_1", "\t; landed", "\ts_endpgm"]
   assert [t for _, t in _touches_in_flight(loop)] == ["v_mov_b32_e32 v9, v4"]
+
+def test_wave_private_loop_keeps_its_ring_in_flight(kernels):
+  """qgemm_wp.hip counts its direct-to-LDS pieces by hand; a compiler-placed `s_waitcnt vmcnt(0)` inside the row-group loop (it puts one in front of an LDS atomic
+  builtin, for instance, because it cannot tell the counters from the rings) would empty the ring once per group.  Inside the loop of the SwiGLU
+  instantiations every vector-memory wait must be one of the source's own (between ASMSTART / ASMEND); the others also hold the residual load of the
+  summing wave, which the compiler waits for."""
+  _, ks = kernels
+  names = [n for n in ks if "qgemm_wp_kernel" in n]
+  if not names: pytest.skip("not the wave-private source")
+  checked = 0
+  for name in names:
+    m = re.match(r"_Z15qgemm_wp_kernelILi\d+ELb([01])ELb([01])E", name)
+    if m.group(2) == "0": continue                                           # (plain, residual, q / k / v)
+    L = ks[name]
+    start = max(i for i, l in enumerate(L) if "This Loop Header: Depth=1" in l)
+    inside_asm, bad = False, []
+    for i in range(start, len(L)):
+      t = L[i].strip()
+      if t.startswith(";;#ASMSTART"): inside_asm = True
+      elif t.startswith(";;#ASMEND"): inside_asm = False
+      elif t.startswith("s_waitcnt") and "vmcnt" in t and not inside_asm and i < len(L) - 6: bad.append((i, t))
+    assert not bad, (name, bad)
+    checked += 1
+  assert checked >= 4

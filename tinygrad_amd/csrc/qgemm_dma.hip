@@ -20,139 +20,7 @@
 // whole 128-byte lines (eight loads of 1 KB, two rows each: a lane-per-unit read would touch 64 lines per instruction and use 16 bytes of each),
 // issued in front of the weight pieces of the stage after (loads return in issue order: the wait that lets the weights of later stages stay in
 // flight then covers them), and turns them into the operand layout through a wave-private piece of LDS.
-#include "qfmt.h"
-#include <type_traits>
-
-typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
-typedef float v4f32 __attribute__((ext_vector_type(4)));
-
-#define QD_NW 8                       // waves per workgroup
-#define QD_LDS_CU (160 * 1024)
-#define QD_MAX_NB 3
-
-// slot_bytes(su): bytes of su units of one row; PAD: 16-byte pieces between the rows of a slot in LDS (the pitch spreads sixteen rows over the banks);
-// from_lds(row, u): unit u of a slot's row.
-// Geometry of a slot whose rows are whole 16-byte pieces at 16-byte aligned offsets: pieces(su) per row, the second slot of a stage second_off(su) bytes
-// behind the first, stage_stride(su) bytes of a row per stage, the slot's first unit skew(su, half) bytes into the staged row.
-template <class D> struct DmaPlain {
-  static constexpr int pieces(int su) { return D::slot_bytes(su) / 16; }
-  static constexpr int second_off(int su) { return D::slot_bytes(su); }
-  static constexpr int stage_stride(int su) { return 2 * D::slot_bytes(su); }
-  static constexpr int skew(int, int) { return 0; }
-};
-template <int T> struct DmaFmt;
-template <> struct DmaFmt<F_Q4_0P> : DmaPlain<DmaFmt<F_Q4_0P>> {
-  static constexpr int PAD = 1;
-  static constexpr int slot_bytes(int su) { return su * 36; }
-  static __device__ __forceinline__ Fmt<F_Q4_0P>::Raw from_lds(const char* row, int u) {
-    const uint32_t* p = (const uint32_t*)(row + 36 * u);
-    Fmt<F_Q4_0P>::Raw r;
-    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = p[8];
-    return r;
-  }
-};
-template <> struct DmaFmt<F_Q8_0P> : DmaPlain<DmaFmt<F_Q8_0P>> {
-  static constexpr int PAD = 1;
-  static constexpr int slot_bytes(int su) { return su * 68; }
-  static __device__ __forceinline__ Fmt<F_Q8_0P>::Raw from_lds(const char* row, int u) {
-    const uint32_t* p = (const uint32_t*)(row + 68 * u);
-    Fmt<F_Q8_0P>::Raw r;
-    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]}; r.c = u32x4{p[8], p[9], p[10], p[11]}; r.d = u32x4{p[12], p[13], p[14], p[15]}; r.e = p[16];
-    return r;
-  }
-};
-
-// fp16 weights (model.py:376 keeps dense tensors as fp16): a unit is 64 consecutive weights = eight aligned pieces, nothing to decode
-template <> struct DmaFmt<GGML_F16> : DmaPlain<DmaFmt<GGML_F16>> {
-  static constexpr int PAD = 1;
-  static constexpr int slot_bytes(int su) { return su * 128; }
-  static __device__ __forceinline__ Fmt<GGML_F16>::Raw from_lds(const char* row, int u) {
-    const u32x4* p = (const u32x4*)(row + 128 * u);
-    Fmt<GGML_F16>::Raw r;
-#pragma unroll
-    for (int i = 0; i < 8; i++) r.q[i] = p[i];
-    return r;
-  }
-};
-// Q6_K (gguf.py:68-72): four units = one superblock of 210 bytes, so a slot is 32 units = 8 superblocks = 105 pieces and a wave's step of four units is one
-// superblock; superblocks are 2-byte aligned in the slot's row: every 16-byte piece is read as its enclosing aligned dwords and funnel-shifted (by 0 or 16 bits,
-// the same for the whole wave), as Fmt<GGML_Q6_K>::load does from global memory.
-__device__ __forceinline__ u32x4 lds16_a2(const char* p, uint32_t& tail_dword, uint32_t& sh) {
-  const uint32_t a = (uint32_t)(uintptr_t)p; sh = (a & 2u) * 8u;
-  const uint32_t* q = (const uint32_t*)(p - (a & 3u));
-  const uint32_t v0 = q[0], v1 = q[1], v2 = q[2], v3 = q[3], e = q[4];
-  tail_dword = e;
-  return u32x4{__builtin_amdgcn_alignbit(v1, v0, sh), __builtin_amdgcn_alignbit(v2, v1, sh), __builtin_amdgcn_alignbit(v3, v2, sh), __builtin_amdgcn_alignbit(e, v3, sh)};
-}
-template <> struct DmaFmt<GGML_Q6_K> {
-  static constexpr int PAD = 2;                          // pitches of 107 and 55 pieces = 428 and 220 dwords = 44 and 28 mod 64: sixteen rows on sixteen different bank quads
-  // Slots of 16 units (K beyond 4096, an even number of slots): 4 superblocks = 840 bytes start 8 bytes off a 16-byte boundary in every second slot.  A stage
-  // (1680 bytes of a row) is fetched as two windows of 53 aligned pieces, [0, 848) and [832, 1680): the second slot's units start 8 bytes into its window.
-  static constexpr int pieces(int su) { return su == 32 ? 105 : 53; }
-  static constexpr int second_off(int su) { return su == 32 ? 1680 : 832; }
-  static constexpr int stage_stride(int su) { return su / 4 * 210 * 2; }
-  static constexpr int skew(int su, int half) { return su == 32 ? 0 : 8 * half; }
-  static __device__ __forceinline__ Fmt<GGML_Q6_K>::Raw from_lds(const char* row, int u) {
-    const char* p = row + 210 * (u >> 2); const int h = (u >> 1) & 1, g = u & 1;
-    uint32_t tail, sh;
-    Fmt<GGML_Q6_K>::Raw r;
-    r.a = lds16_a2(p + 64 * h + 16 * g, tail, sh); r.b = lds16_a2(p + 64 * h + 32 + 16 * g, tail, sh); r.h = lds16_a2(p + 128 + 32 * h + 16 * g, tail, sh);
-    const u32x4 sc = lds16_a2(p + 192, tail, sh);          // sc[0..15]; the tail dword holds d (bytes 208, 209)
-    r.sc0 = h ? sc.z : sc.x; r.sc1 = h ? sc.w : sc.y;
-    r.d = (uint32_t)g | (__builtin_amdgcn_alignbit(0u, tail, sh) << 16);
-    return r;
-  }
-};
-
-// Q4_K / Q5_K (gguf.py:57-67): four units = one superblock of 144 / 176 bytes = 9 / 11 aligned pieces; a wave's step of four units is one superblock per row
-// (lane group g: sub-block pair g), every read is an aligned 16-byte piece.
-template <bool FIVE> struct DmaFmtK45 : DmaPlain<DmaFmtK45<FIVE>> {
-  using F = FmtK45<FIVE>;
-  static constexpr int PAD = 1;                          // pitches of 37 / 73 (Q4_K) and 45 / 89 (Q5_K) pieces: sixteen rows on sixteen different bank quads
-  static constexpr int slot_bytes(int su) { return su / 4 * F::BB; }
-  static __device__ __forceinline__ typename F::Raw from_lds(const char* row, int u) {
-    const char* b = row + F::BB * (u >> 2); const int p = u & 3;
-    typename F::Raw r;
-    r.hdr = *(const u32x4*)b; r.q0 = *(const u32x4*)(b + F::QS + 32 * p); r.q1 = *(const u32x4*)(b + F::QS + 32 * p + 16);
-    if constexpr (FIVE) { r.h0 = *(const u32x4*)(b + 16); r.h1 = *(const u32x4*)(b + 32); }
-    r.p = (uint32_t)p;
-    return r;
-  }
-};
-template <> struct DmaFmt<GGML_Q4_K> : DmaFmtK45<false> {};
-template <> struct DmaFmt<GGML_Q5_K> : DmaFmtK45<true> {};
-
-// Q4_1 / Q5_0 / Q5_1 block pairs (gguf.py:47-55): units of 40 / 44 / 48 bytes at 4-byte aligned offsets of the slot's row; 16 units are 40 / 44 / 48 pieces
-// (pitches of 41 / 45 / 49 pieces = 36 / 52 / 4 mod 64 dwords: sixteen rows on sixteen different bank quads)
-template <int KIND> struct DmaFmtL : DmaPlain<DmaFmtL<KIND>> {
-  using F = FmtL<KIND>;
-  static constexpr int PAD = 1;
-  static constexpr int slot_bytes(int su) { return su * F::BB; }
-  static __device__ __forceinline__ typename F::Raw from_lds(const char* row, int u) {
-    const uint32_t* p = (const uint32_t*)(row + F::BB * u);
-    typename F::Raw r;
-    r.a = u32x4{p[0], p[1], p[2], p[3]}; r.b = u32x4{p[4], p[5], p[6], p[7]};
-#pragma unroll
-    for (int i = 0; i < F::ND - 8; i++) r.t[i] = p[8 + i];
-    return r;
-  }
-};
-template <> struct DmaFmt<GGML_Q4_1> : DmaFmtL<0> {};
-template <> struct DmaFmt<GGML_Q5_0> : DmaFmtL<1> {};
-template <> struct DmaFmt<GGML_Q5_1> : DmaFmtL<2> {};
-
-// at most n vector-memory operations of this wave still outstanding (n is the same for the whole wave).  Behind it, the registers of inline-assembly
-// requests are passed through an empty asm statement with the comment "; landed": no use of them can move in front of the wait, and the comment marks
-// the place in the generated assembly for tests/test_isa_invariants.py
-__device__ __forceinline__ void qd_wait_vm(int n) {
-  switch (n) {
-#define QD_W(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
-    QD_W(1) QD_W(2) QD_W(3) QD_W(4) QD_W(5) QD_W(6) QD_W(7) QD_W(8) QD_W(9) QD_W(10) QD_W(11) QD_W(12) QD_W(13) QD_W(14) QD_W(15) QD_W(16)
-    QD_W(17) QD_W(18) QD_W(19) QD_W(20) QD_W(21) QD_W(22) QD_W(23) QD_W(24)
-#undef QD_W
-    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-  }
-}
+#include "qdma_fmt.h"
 
 // SW: silu(gate) * up (dense SwiGLU, tinygrad/llm/model.py:137) over the two matrices w[0] / w[1]: a row group is eight rows of the gate matrix followed
 // by the same eight rows of the up matrix, so the partial tiles of both meet in one reduction and the product is formed before the store.
@@ -589,12 +457,23 @@ static int launch_qd(QArgs a, int M, hipStream_t s) {
 // 16 rows at a 16-byte aligned address (8 rows for the SwiGLU pair);
 // Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 block pairs: K = 1024, 2048, 3072 or 4096 (larger multiples of 1024 for one matrix); Q4_K / Q5_K: K = 2048 or 4096 (Q5_K: and 1024, 3072), larger
 // multiples of 1024 for one matrix; Q6_K: one matrix, K a multiple of 2048; fp16 weights: K <= 4096, no SwiGLU pair.
+int tga_qgemm_wp_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm_wp.hip: the same call on wave-private rings (Q8_0, K = 2048 / 4096), -1 outside its range
+// what both kernels ask of a call: 2 <= M <= 16, every matrix whole row groups at a 16-byte aligned address, float32 rows where a norm folds in
+static bool qd_call_ok(const QArgs& a, int M) {
+  if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return false;
+  if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return false;      // the folded norm: float32 rows that the workgroup's operands cover whole
+  if (((uintptr_t)a.x & 15) != 0) return false;
+  if (a.epilogue == 2) return a.w[1] && a.n[0] % 8 == 0 && a.n[0] > 0 && (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) == 0;   // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
+  for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return false;
+  return true;
+}
+// the wave-private kernel or nothing (two rows of a large Q8_0 matrix: there the barrier kernel is slower than the single-row kernel's two-row walk, this one is not)
+int tga_qgemm_wp_checked_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) { return qd_call_ok(a, M) ? tga_qgemm_wp_dispatch(fmt, a, M, s) : -1; }
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   if (fmt != F_Q4_0P && fmt != F_Q8_0P && fmt != GGML_Q6_K && fmt != GGML_F16 && fmt != GGML_Q4_K && fmt != GGML_Q5_K && fmt != GGML_Q4_1 && fmt != GGML_Q5_0 && fmt != GGML_Q5_1) return -1;
-  if (M < 2 || M > 16 || a.nseg < 1 || a.nseg > 3 || a.epilogue > 2 || a.sel || a.x_staged || a.y_stage_fmt) return -1;
-  if (a.norm_w && (!a.x_f32 || a.K > 4096 || ((uintptr_t)a.norm_w & 15) != 0)) return -1;      // the folded norm: float32 rows that the workgroup's operands cover whole
-  if (a.epilogue == 2) {                                              // silu(gate) * up: two matrices of equal shape, eight rows of each per row group
-    if (!a.w[1] || a.n[0] % 8 != 0 || a.n[0] <= 0 || (((uintptr_t)a.w[0] | (uintptr_t)a.w[1]) & 15) != 0 || ((uintptr_t)a.x & 15) != 0) return -1;
+  if (!qd_call_ok(a, M)) return -1;
+  if (const int rc = tga_qgemm_wp_dispatch(fmt, a, M, s); rc >= 0) return rc;
+  if (a.epilogue == 2) {
     switch (fmt) {
       case F_Q4_0P: return launch_qd<F_Q4_0P>(a, M, s);
       case F_Q8_0P: return launch_qd<F_Q8_0P>(a, M, s);
@@ -606,8 +485,6 @@ int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
     }
     return -1;
   }
-  for (int i = 0; i < a.nseg; i++) if (a.n[i] % 16 != 0 || a.n[i] <= 0 || ((uintptr_t)a.w[i] & 15) != 0) return -1;
-  if (((uintptr_t)a.x & 15) != 0) return -1;
   switch (fmt) {
     case F_Q4_0P: return launch_qd<F_Q4_0P>(a, M, s);
     case F_Q8_0P: return launch_qd<F_Q8_0P>(a, M, s);

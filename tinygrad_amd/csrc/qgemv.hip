@@ -318,6 +318,7 @@ static int launch_qgemv_m(const QArgs& a, int M, hipStream_t s) {
 int tga_qgemv1_dispatch(int fmt, const QArgs& a, hipStream_t s);   // qgemv1.hip
 int tga_qgemm_mfma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm.hip
 int tga_qgemm_dma_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);    // qgemm_dma.hip
+int tga_qgemm_wp_checked_dispatch(int fmt, const QArgs& a, int M, hipStream_t s);   // qgemm_dma.hip / qgemm_wp.hip
 int tga_qgemv1_multi_dispatch(int fmt, const QArgs& a, int M, hipStream_t s); // qgemv1_multi.hip
 struct Q64Opt { bool prestaged; const void* xs_ext; bool defer; float* part; int ks, np; };   // qgemm64.hip
 int tga_qgemm64_dispatch(int fmt, const QArgs& a, int M, Q64Opt& o, hipStream_t s);            // qgemm64.hip
@@ -514,6 +515,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     // (Q4_0 4096 x 4096: 7.4 us against 9.1 us on the LDS-staged dot2 kernel, which takes the rest)
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
     if (fmt == F_Q8_0P && a.K > 4096) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }   // (Q8_0 4096 x 14336: streamed activations 17.3 us, the walk 18.7)
+    if (fmt == F_Q8_0P && a.K <= 4096) { const int rc = tga_qgemm_wp_checked_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }   // (Q8_0 14336 x 4096: wave-private rings 15.8 us, the walk 17.0)
     if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     const int fmt2 = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt2 >= 0 && a.ntot * (long long)a.K < (1ll << 25)) { const int rc = tga_qgemm_dma_dispatch(fmt2, a, M, s); if (rc >= 0) return rc; }
