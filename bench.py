@@ -229,6 +229,11 @@ def main():
   prompt = [int(t) for t in rng.integers(0, c.vocab_size, size=args.prefill)]
   ug = not args.no_graph
   model.prefill(prompt, ug)                                    # fills positions 0..prefill-2; the last prompt token is the first decode input
+  rt.synchronize()
+  tp = time.perf_counter()
+  model.prefill(prompt, ug, reuse_cache=False)                 # the same prompt once more, now with every step kind recorded: the prefill rate (extra/benchmark_llm.py reports it beside the decode rate)
+  rt.synchronize()
+  prefill_s = time.perf_counter() - tp
   for _ in range(args.warmup): model.decode_step(ug)
   rt.synchronize()
   t0 = time.perf_counter()
@@ -326,6 +331,8 @@ def main():
                                "(profiles/decode_llama3_8b_q4_0_kernel_stats.md), neither re-measured by this run",
                      "share_of_block_time": round(dom["avg_us"] / per_block, 3),
                      "per_op_kernels": {k: v for k, v in kern.items() if k != "gate_up"}}
+  out["prefill"] = {"positions": args.prefill - 1, "ms": round(prefill_s * 1e3, 2), "positions_per_s": round((args.prefill - 1) / prefill_s, 1), "positions_per_step": int(model.prefill_chunk),
+                    "what": "the prompt prefilled once more before the timed decode steps (recorded steps replayed; one pass over the weights per step of positions_per_step rows), host wall clock; not part of `value`"}
   if parity is not None: out["parity"] = parity
   if not args.no_cpu:
     from oracle import cref
