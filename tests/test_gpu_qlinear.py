@@ -531,22 +531,24 @@ def test_sixteen_and_more_rows_segments_residual_and_swiglu(gpu, m):
     a, b = refs[1], ol.linear_f64(x.astype(np.float32), ol.weight_f32(g[1].blocks.numpy(), ns[1], k, t))
     assert ol.rel_err(out.numpy(), a / (1 + np.exp(-a)) * b) <= TOL, (t, k)
 
-@pytest.mark.parametrize("k,m,f32", [(4096, 2, False), (4096, 3, True), (2048, 5, False), (4096, 8, True), (2048, 9, True), (4096, 13, False), (4096, 16, True), (2048, 16, False)])
-def test_q8_0_small_batch_on_wave_private_rings(gpu, k, m, f32):
-  """The Q8_0 small-batch kernel whose waves stream their own slices of K (qgemm_wp.hip: K = 2048 / 4096, 2 .. 16 rows): q / k / v in one launch, the residual
-  epilogue in place, silu(gate) * up, and a matrix of 14336 rows (three or four row groups per workgroup, so the rings wrap and both tile sets are reused),
-  fp16 and float32 activations, against the float64 anchor; twice, to see that a launch leaves nothing behind that the next one reads."""
+@pytest.mark.parametrize("t,k,m,f32", [(8, 4096, 2, False), (8, 4096, 3, True), (8, 2048, 5, False), (8, 4096, 8, True), (8, 2048, 9, True), (8, 4096, 13, False), (8, 4096, 16, True), (8, 2048, 16, False),
+                                       (1, 2048, 2, False), (1, 2048, 4, True), (1, 2048, 8, False), (1, 2048, 11, True), (1, 2048, 16, False)])
+def test_small_batch_on_wave_private_rings(gpu, t, k, m, f32):
+  """The small-batch kernel whose waves stream their own slices of K (qgemm_wp.hip: Q8_0 at K = 2048 / 4096 and fp16 weights at K = 2048, 2 .. 16 rows): q / k / v in
+  one launch, the residual epilogue in place, silu(gate) * up (Q8_0), and a matrix of 14336 rows (three or four row groups per workgroup, so the rings wrap and both
+  tile sets are reused), fp16 and float32 activations, against the float64 anchor; twice, to see that a launch leaves nothing behind that the next one reads."""
   from tinygrad_amd.nn import QuantLinear, qlinear_multi
-  t = 8
   rng = np.random.default_rng(88 + k + m)
   ns = [1024, 256, 256]
-  ws = [synth.random_blocks(rng, t, n, k) for n in ns]
+  mkw = lambda n: synth.random_blocks(rng, t, n, k) if t != 1 else (rng.standard_normal((n, k)) * 0.02).astype(np.float16).view(np.uint8).reshape(-1)
+  wf32 = lambda w, n: ol.weight_f32(w, n, k, t) if t != 1 else w.view(np.float16).reshape(n, k).astype(np.float32)
+  ws = [mkw(n) for n in ns]
   x = synth.activations(rng, m, k, np.float32 if f32 else np.float16)
   xf = x.astype(np.float32) if f32 else x.astype(np.float32)
   h = xf.astype(np.float16).astype(np.float32)                          # the kernel rounds float32 rows to fp16 operands
   layers = [QuantLinear(gpu.Buffer.from_numpy(w), t, n, k) for w, n in zip(ws, ns)]
   xb = gpu.Buffer.from_numpy(x)
-  refs = [ol.linear_f64(h, ol.weight_f32(w, n, k, t)) for w, n in zip(ws, ns)]
+  refs = [ol.linear_f64(h, wf32(w, n)) for w, n in zip(ws, ns)]
   for rep in range(2):
     outs = [gpu.Buffer((m, n), np.float32) for n in ns]
     for o in outs: gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))
@@ -556,6 +558,7 @@ def test_q8_0_small_batch_on_wave_private_rings(gpu, k, m, f32):
     rb = [gpu.Buffer.from_numpy(r) for r in res]
     qlinear_multi(layers[:1], xb, rb[:1], epilogue=1, resid=rb[:1])
     assert ol.rel_err(rb[0].numpy(), res[0] + refs[0]) <= TOL, (k, m, rep)
+    if t != 8: continue                                                 # (fp16 weights: no SwiGLU pair on this kernel)
     g = [layers[1], layers[2]]
     out = gpu.Buffer((m, ns[1]), np.float32)
     qlinear_multi(g, xb, [out], epilogue=2)
@@ -563,11 +566,11 @@ def test_q8_0_small_batch_on_wave_private_rings(gpu, k, m, f32):
     out16 = gpu.Buffer((m, ns[1]), np.float16)
     qlinear_multi(g, xb, [out16], epilogue=2)
     assert ol.rel_err(out16.numpy().astype(np.float32), refs[1] / (1 + np.exp(-refs[1])) * refs[2]) <= 2 * TOL, (k, m, rep)
-  if k == 4096 and m in (8, 16):
+  if (t, k) in ((8, 4096), (1, 2048)) and m in (8, 16):
     n = 14336
-    w = synth.random_blocks(rng, t, n, k)
+    w = mkw(n)
     lin = QuantLinear(gpu.Buffer.from_numpy(w), t, n, k)
-    ref = ol.linear_f64(h, ol.weight_f32(w, n, k, t))
+    ref = ol.linear_f64(h, wf32(w, n))
     for rep in range(2):
       o = gpu.Buffer((m, n), np.float16)
       gpu.check(gpu.lib().tga_memset(o.ptr, 0xFF, o.nbytes, None))

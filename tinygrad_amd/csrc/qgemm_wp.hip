@@ -1,4 +1,4 @@
-// Small-batch GEMM over Q8_0 block pairs (2 <= M <= 16 activation rows, K = 2048 or 4096) with the weights streamed into LDS by direct-to-LDS loads into rings
+// Small-batch GEMM over Q8_0 block pairs (K = 2048 or 4096) and fp16 weights (K = 2048), 2 <= M <= 16 activation rows, with the weights streamed into LDS by direct-to-LDS loads into rings
 // that belong to ONE WAVE each: the same call sites and arithmetic as qgemm_dma.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177,
 // tinygrad/mixin/op.py:367-392; a unit is decoded once into fp16 weights - the reference's fp16 weight cast, tinygrad/llm/model.py:376 - and
 // v_mfma_f32_16x16x32_f16 multiplies it with all activation rows), without a workgroup barrier in the loop.
@@ -317,13 +317,15 @@ static int launch_wp(QArgs a, int M, hipStream_t s) {
 }
 
 // Called by tga_qgemm_dma_dispatch with a call it has checked (2 <= M <= 16, matrices of whole row groups at 16-byte aligned addresses, float32 rows where a norm
-// folds in).  Returns -1 outside this kernel's range.  Q8_0 only: the kernel template takes every format whose rows split into eight aligned runs, and in
-// isolated launches it is 3 - 20 % faster for all of them except the large Q4_0 / Q4_K matrices, but in a replayed batched decode step only the Q8_0 model gained
-// (8B-arch at B = 4 / 8: 2.81 -> 2.68 / 3.21 -> 3.03 ms per step; the Q4_K_M mix unchanged, Q4_0 3 % slower), so the others stay on qgemm_dma.hip.
+// folds in).  Returns -1 outside this kernel's range.  Q8_0 and fp16 weights only - the formats with the most bytes per decoded weight: the kernel template takes
+// every format whose rows split into eight aligned runs, and in isolated launches it is 3 - 20 % faster for all of them except the large Q4_0 / Q4_K matrices, but in a
+// replayed batched decode step only these two gained (8B-arch Q8_0 model at B = 4 / 8: 2.81 -> 2.68 / 3.21 -> 3.03 ms per step; OLMoE-arch, fp16 dense weights, at
+// B = 2 / 4 / 8: +4 / +4 / +3 % tokens per second; the Q4_K_M mix unchanged, Q4_0 3 % slower), so the others stay on qgemm_dma.hip.
 int tga_qgemm_wp_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   static const bool off = getenv("TGA_WP") && atoi(getenv("TGA_WP")) == 0;      // (for A / B runs against the barrier kernel)
-  if (off || fmt != F_Q8_0P) return -1;
+  if (off || (fmt != F_Q8_0P && fmt != GGML_F16)) return -1;
+  if (fmt == GGML_F16 && (a.epilogue == 2 || a.K != 2048)) return -1;  // (fp16 rows of 4096 values: a ring of two groups does not fit)
   for (int i = 0; i < (a.epilogue == 2 ? 1 : a.nseg); i++)          // four rows of a column leave as one vector store
     if (((uintptr_t)a.y[i] & 15) != 0 || (a.epilogue == 1 && ((uintptr_t)a.resid[i] & 15) != 0)) return -1;
-  return launch_wp<F_Q8_0P>(a, M, s);
+  return fmt == GGML_F16 ? launch_wp<GGML_F16>(a, M, s) : launch_wp<F_Q8_0P>(a, M, s);
 }
