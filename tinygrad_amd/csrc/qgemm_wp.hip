@@ -300,7 +300,8 @@ template <int T, int UPW>
 static int launch_wp_u(const QArgs& a, int M, hipStream_t s) {
   // three groups in flight per wave where the ring holds them, else two
   int rc;
-  if (a.epilogue == 2) { rc = launch_wp_k<T, false, true, UPW, 3>(a, M, s); return rc >= 0 ? rc : launch_wp_k<T, false, true, UPW, 2>(a, M, s); }
+  if constexpr (T != GGML_F16) { if (a.epilogue == 2) { rc = launch_wp_k<T, false, true, UPW, 3>(a, M, s); return rc >= 0 ? rc : launch_wp_k<T, false, true, UPW, 2>(a, M, s); } }
+  if (a.epilogue == 2) return -1;
   if (a.nseg > 1) { rc = launch_wp_k<T, true, false, UPW, 3>(a, M, s); return rc >= 0 ? rc : launch_wp_k<T, true, false, UPW, 2>(a, M, s); }
   rc = launch_wp_k<T, false, false, UPW, 3>(a, M, s); return rc >= 0 ? rc : launch_wp_k<T, false, false, UPW, 2>(a, M, s);
 }
@@ -311,7 +312,7 @@ static int launch_wp(QArgs a, int M, hipStream_t s) {
   a.nu = a.K / F::UW;
   a.row_bytes = (long long)(a.K / F::BW) * F::BB;
   if (a.K % F::UW != 0 || a.row_bytes % 16 != 0) return -1;
-  if (a.nu == 64) return launch_wp_u<T, 8>(a, M, s);
+  if constexpr (T != GGML_F16) { if (a.nu == 64) return launch_wp_u<T, 8>(a, M, s); }       // (fp16 rows of 4096 values: a ring of two groups does not fit, and its operands would spill)
   if (a.nu == 32) return launch_wp_u<T, 4>(a, M, s);
   return -1;
 }
