@@ -516,6 +516,7 @@ static int qlinear_multi_impl(const CombineIn* comb, const AttnIn* attn, const f
     const int fmt = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type == GGML_Q6_K ? GGML_Q6_K : -1;
     if (fmt == F_Q8_0P && a.K > 4096) { const int rc = tga_qgemm_dma_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }   // (Q8_0 4096 x 14336: streamed activations 17.3 us, the walk 18.7)
     if (fmt == F_Q8_0P && a.K <= 4096) { const int rc = tga_qgemm_wp_checked_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }   // (Q8_0 14336 x 4096: wave-private rings 15.8 us, the walk 17.0)
+    if (ggml_type == GGML_F16) { const int rc = tga_qgemm_wp_checked_dispatch(GGML_F16, a, M, s); if (rc >= 0) return rc; }          // (fp16 50304 x 2048 lm-head: 41 us against 55 on the LDS-staged kernel)
     if (fmt >= 0) { const int rc = tga_qgemv1_multi_dispatch(fmt, a, M, s); if (rc >= 0) return rc; }
     const int fmt2 = ggml_type == GGML_Q4_0 ? (pair ? F_Q4_0P : -1) : ggml_type == GGML_Q8_0 ? (pair ? F_Q8_0P : -1) : ggml_type;
     if (fmt2 >= 0 && a.ntot * (long long)a.K < (1ll << 25)) { const int rc = tga_qgemm_dma_dispatch(fmt2, a, M, s); if (rc >= 0) return rc; }
