@@ -347,7 +347,13 @@ __global__ __launch_bounds__(256) void q64_reduce_kernel(const QArgs a, const in
   const int m = (int)(idx / q); long long row = 4 * (idx - (long long)m * q);
   if (m >= M) return;
   v4f32 v = *(const v4f32*)(part + (size_t)m * np + row);
-  for (int k = 1; k < ks; k++) { const v4f32 t = *(const v4f32*)(part + ((size_t)k * Q64_COLS + m) * np + row); v += t; }
+  for (int k0 = 1; k0 < ks; k0 += 8) {                   // eight splits requested together (one round trip), added in the order of K
+    v4f32 t[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) t[k] = *(const v4f32*)(part + ((size_t)(k0 + k < ks ? k0 + k : ks - 1) * Q64_COLS + m) * np + row);
+#pragma unroll
+    for (int k = 0; k < 8; k++) if (k0 + k < ks) v += t[k];
+  }
   int sg = 0; long long nrows = a.n[0];
   if (a.nseg > 1 && row >= a.n[0]) { row -= a.n[0]; sg = 1; nrows = a.n[1]; if (a.nseg > 2 && row >= a.n[1]) { row -= a.n[1]; sg = 2; nrows = a.n[2]; } }
   void* yb = sg == 0 ? a.y[0] : sg == 1 ? a.y[1] : a.y[2];
