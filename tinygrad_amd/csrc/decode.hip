@@ -143,6 +143,7 @@ struct AttnArgs {
   // chunk 1 = the launch that only rotates and appends every row's key / value, chunk 2 = the launch that attends from the cache alone
   // (the rows of the chunk were appended by the launch before; a row sees the positions up to its own).  0: decode.
   int chunk, pos_step;
+  int split_shift;                                     // log2 of the positions per split partial that the merge launch sums (6: splits of 64; the matrix-core chunk launch may cover several tiles per partial)
 };
 __device__ __forceinline__ AttnArgs attn_args_of_sequence(AttnArgs a, int z) {
   a.q += z * a.q_bs; a.k += z * a.kv_bs; a.v += z * a.kv_bs; a.cache_k += z * a.cache_bs; a.cache_v += z * a.cache_bs; a.part += z * a.part_bs;
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 }
 
 // Chunked prefill, the attending launch on the matrix cores (chunk rows z = 0, 1, ... are consecutive positions of one sequence; the launch before has rotated
-// and appended every row's key / value).  Workgroup = (kv head, split of 64 cached positions, tile of 16 chunk rows): the per-row workgroups of
+// and appended every row's key / value).  Workgroup = (kv head, split of 64 TS cached positions walked in tiles of 64, tile of 16 chunk rows): the per-row workgroups of
 // attn_decode_kernel read every 32 KB K / V tile once per row and query-head group - 64 rows x 8 kv heads x 16 splits = 268 MB of L2 reads per layer at a
 // context of 1024 - here a tile is read once per sixteen rows.  Wave w serves query head w of the group (w + 4, ... for larger groups):
 //   S^T = K Q^T   v_mfma_f32_16x16x32_f16, A = lane (g, r): 8 values 32 j + 8 g .. of cached key 16 t + r (16-byte loads straight from the cache), B = lane (g, c):
@@ -427,7 +428,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const AttnArgs args) {
 //                 transposed with its keys in that order, so that the A operand is one 16-byte LDS read
 // The partial (float32 weighted V sums, max, sum) goes where attn_decode_kernel writes it; attn_merge_kernel finishes.  Deviation from the float32 products of
 // the per-row kernel: the probabilities are rounded to fp16 (2^-11 relative, fp32 accumulation).
-template <int HD8>
+// TS consecutive 64-key tiles per workgroup (one split partial of 64 TS positions): the rotated queries are formed once and the softmax partial runs over
+// the tiles with a running maximum (the sums and the weighted V sums are rescaled when it grows), so TS times fewer partials are written here and read by the merge
+// launch, and the queries are read and rotated TS times less often.  HPW: query heads per wave (the group has at most 4 HPW heads).
+template <int HD8, int TS, int HPW>
 __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, const int rows) {
   typedef _Float16 v8f16 __attribute__((ext_vector_type(8)));
   typedef float v4f32 __attribute__((ext_vector_type(4)));
@@ -439,113 +443,144 @@ __global__ __launch_bounds__(256) void attn_chunk_mfma_kernel(const AttnArgs a, 
   const int group = a.n_heads / a.n_kv;
   const int row = 16 * rz + c < rows ? 16 * rz + c : rows - 1;             // this lane's chunk row (a tile that the chunk ends in repeats the last row, stored by nobody)
   const bool row_ok = 16 * rz + c < rows;
-  // ---- loads that do not depend on the position: the V tile (lane = key, pieces 4 wave .. 4 wave + 3 of HD8), the K operands, the first head's query
-  const int key0 = split * 64;
+  // ---- loads that do not depend on the position: the V tile (lane = key, pieces 4 wave .. 4 wave + 3 of HD8) and the K operands of the first tile
   u32x4 vv[HD8 / 4];
-  {
-    const int kr = key0 + lane < a.max_ctx ? key0 + lane : a.max_ctx - 1;
-    const _Float16* vb = a.cache_v + ((size_t)kvh * a.max_ctx + kr) * HD;
-#pragma unroll
-    for (int i = 0; i < HD8 / 4; i++) vv[i] = *(const u32x4*)(vb + 8 * ((HD8 / 4) * wave + i));
-  }
   u32x4 kt[4][NJ];
+  auto load_tile = [&](int key0) __attribute__((always_inline)) {
+    {
+      const int kr = key0 + lane < a.max_ctx ? key0 + lane : a.max_ctx - 1;
+      const _Float16* vb = a.cache_v + ((size_t)kvh * a.max_ctx + kr) * HD;
 #pragma unroll
-  for (int t = 0; t < 4; t++) {
-    const int kr = key0 + 16 * t + c < a.max_ctx ? key0 + 16 * t + c : a.max_ctx - 1;   // (rows beyond the cache are masked below: they lie beyond every position)
-    const _Float16* kb = a.cache_k + ((size_t)kvh * a.max_ctx + kr) * HD + 8 * g;
+      for (int i = 0; i < HD8 / 4; i++) vv[i] = *(const u32x4*)(vb + 8 * ((HD8 / 4) * wave + i));
+    }
 #pragma unroll
-    for (int j = 0; j < NJ; j++) kt[t][j] = *(const u32x4*)(kb + 32 * j);
-  }
+    for (int t = 0; t < 4; t++) {
+      const int kr = key0 + 16 * t + c < a.max_ctx ? key0 + 16 * t + c : a.max_ctx - 1;   // (rows beyond the cache are masked below: they lie beyond every position)
+      const _Float16* kb = a.cache_k + ((size_t)kvh * a.max_ctx + kr) * HD + 8 * g;
+#pragma unroll
+      for (int j = 0; j < NJ; j++) kt[t][j] = *(const u32x4*)(kb + 32 * j);
+    }
+  };
+  const int key_first = split * 64 * TS;
+  load_tile(key_first);
   const int pos0 = a.st->pos;
   const int last = pos0 + (16 * rz + 15 < rows ? 16 * rz + 15 : rows - 1);   // the last position of this row tile
   if (pos0 < 0 || last >= a.max_ctx) return;             // (refused by the appending launch: state.error)
-  if (key0 > last) return;                               // nothing of this split is visible to the tile
+  if (key_first > last) return;                          // nothing of this split is visible to the tile
   const int pos = pos0 + row;
-  // ---- the V tile transposed: key j of the split goes to slot 32 (j / 32) + 8 ((j % 16) / 4) + 4 ((j % 32) / 16) + j % 4 of every dimension's row
-  {
-    const int j = lane, slot = (j & 32) + 8 * ((j & 15) >> 2) + 4 * ((j >> 4) & 1) + (j & 3);
+  // ---- the rotated queries of this wave's heads (row, head): the lane's values 32 j + 8 g + e; the partner of a low value is the value half further, in the same
+  // lane (j + NJ / 2); as TWO fp16 operands, the rounded value and what the rounding left over, so that the scores see the float32 queries
+  u32x4 qb[HPW][NJ], qr[HPW][NJ];
+  auto form_queries = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < HD8 / 4; i++) {
-      const int d0 = 8 * ((HD8 / 4) * wave + i);
-      const uint32_t w[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
+  for (int hw = 0; hw < HPW; hw++) {
+    const int hh = wave + 4 * hw < group ? wave + 4 * hw : group - 1;
+    const int head = kvh * group + hh;
+    const float* qrow = a.q + (size_t)row * a.q_bs + (size_t)head * HD;
+    const float* rr = a.rope + (size_t)pos * HD;
 #pragma unroll
-      for (int e = 0; e < 8; e++) vts[(d0 + e) * VP + slot] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    for (int j = 0; j < NJ / 2; j++) {
+      float lo[8], hi[8];
+#pragma unroll
+      for (int e4 = 0; e4 < 8; e4 += 4) {
+        const int i = 32 * j + 8 * g + e4;
+        const f32x4 x1 = *(const f32x4*)(qrow + i), x2 = *(const f32x4*)(qrow + half + i), cs = *(const f32x4*)(rr + i), sn = *(const f32x4*)(rr + half + i);
+        lo[e4] = rope_lo(x1.x, x2.x, cs.x, sn.x); lo[e4 + 1] = rope_lo(x1.y, x2.y, cs.y, sn.y); lo[e4 + 2] = rope_lo(x1.z, x2.z, cs.z, sn.z); lo[e4 + 3] = rope_lo(x1.w, x2.w, cs.w, sn.w);
+        hi[e4] = rope_hi(x1.x, x2.x, cs.x, sn.x); hi[e4 + 1] = rope_hi(x1.y, x2.y, cs.y, sn.y); hi[e4 + 2] = rope_hi(x1.z, x2.z, cs.z, sn.z); hi[e4 + 3] = rope_hi(x1.w, x2.w, cs.w, sn.w);
+      }
+      qb[hw][j] = pack8_f16(lo); qb[hw][j + NJ / 2] = pack8_f16(hi);
+      float lr[8], hr[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) { lr[e] = lo[e] - (float)(_Float16)lo[e]; hr[e] = hi[e] - (float)(_Float16)hi[e]; }
+      qr[hw][j] = pack8_f16(lr); qr[hw][j + NJ / 2] = pack8_f16(hr);
     }
   }
-  __syncthreads();
-  for (int hh = wave; hh < group; hh += 4) {
-    const int head = kvh * group + hh;
-    // the rotated query of (row, head): the lane's values 32 j + 8 g + e; the partner of a low value is the value half further, in the same lane (j + NJ / 2)
-    u32x4 qb[NJ], qr[NJ];
+  };
+  float M[HPW], L[HPW];
+  v4f32 O[HPW][NH];
+#pragma unroll
+  for (int hw = 0; hw < HPW; hw++) {
+    M[hw] = -INFINITY; L[hw] = 0.f;
+#pragma unroll
+    for (int h = 0; h < NH; h++) O[hw][h] = v4f32{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int tt = 0; tt < TS; tt++) {
+    const int key0 = key_first + 64 * tt;
+    if (key0 > last) break;                              // (the same for the whole workgroup)
+    const bool final = tt + 1 == TS || key0 + 64 > last;  // the last tile of this split that the row tile sees: its weighted sums go straight to the partial
+    if (tt > 0) { __syncthreads(); load_tile(key0); }    // every wave is done with the V tile in LDS before it is replaced
+    // ---- the V tile transposed: key j of the tile goes to slot 32 (j / 32) + 8 ((j % 16) / 4) + 4 ((j % 32) / 16) + j % 4 of every dimension's row
     {
-      const float* qrow = a.q + (size_t)row * a.q_bs + (size_t)head * HD;
-      const float* rr = a.rope + (size_t)pos * HD;
+      const int j = lane, slot = (j & 32) + 8 * ((j & 15) >> 2) + 4 * ((j >> 4) & 1) + (j & 3);
 #pragma unroll
-      for (int j = 0; j < NJ / 2; j++) {
-        float lo[8], hi[8];
+      for (int i = 0; i < HD8 / 4; i++) {
+        const int d0 = 8 * ((HD8 / 4) * wave + i);
+        const uint32_t w[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
 #pragma unroll
-        for (int e4 = 0; e4 < 8; e4 += 4) {
-          const int i = 32 * j + 8 * g + e4;
-          const f32x4 x1 = *(const f32x4*)(qrow + i), x2 = *(const f32x4*)(qrow + half + i), cs = *(const f32x4*)(rr + i), sn = *(const f32x4*)(rr + half + i);
-          lo[e4] = rope_lo(x1.x, x2.x, cs.x, sn.x); lo[e4 + 1] = rope_lo(x1.y, x2.y, cs.y, sn.y); lo[e4 + 2] = rope_lo(x1.z, x2.z, cs.z, sn.z); lo[e4 + 3] = rope_lo(x1.w, x2.w, cs.w, sn.w);
-          hi[e4] = rope_hi(x1.x, x2.x, cs.x, sn.x); hi[e4 + 1] = rope_hi(x1.y, x2.y, cs.y, sn.y); hi[e4 + 2] = rope_hi(x1.z, x2.z, cs.z, sn.z); hi[e4 + 3] = rope_hi(x1.w, x2.w, cs.w, sn.w);
+        for (int e = 0; e < 8; e++) vts[(d0 + e) * VP + slot] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+      }
+    }
+    __syncthreads();
+    if (tt == 0) form_queries();                        // (behind the first tile's V transposition: the query and rotation rows arrive while it runs)
+#pragma unroll
+    for (int hw = 0; hw < HPW; hw++) {
+      if (wave + 4 * hw >= group) break;
+      // scores of the 64 keys x 16 rows
+      v4f32 sc[4];
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        sc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qr[hw][j]), sc[t], 0, 0, 0);
+          sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qb[hw][j]), sc[t], 0, 0, 0);
         }
-        qb[j] = pack8_f16(lo); qb[j + NJ / 2] = pack8_f16(hi);
-        float lr[8], hr[8];                               // what the fp16 rounding left over: a second operand, so that the scores see the float32 queries
-#pragma unroll
-        for (int e = 0; e < 8; e++) { lr[e] = lo[e] - (float)(_Float16)lo[e]; hr[e] = hi[e] - (float)(_Float16)hi[e]; }
-        qr[j] = pack8_f16(lr); qr[j + NJ / 2] = pack8_f16(hr);
       }
-    }
-    // scores of the 64 keys x 16 rows
-    v4f32 sc[4];
+      float m = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-      sc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
+      for (int t = 0; t < 4; t++) {
 #pragma unroll
-      for (int j = 0; j < NJ; j++) {
-        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qr[j]), sc[t], 0, 0, 0);
-        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, kt[t][j]), __builtin_bit_cast(v8f16, qb[j]), sc[t], 0, 0, 0);
+        for (int i = 0; i < 4; i++) {
+          const float sv = key0 + 16 * t + 4 * g + i <= pos ? sc[t][i] * a.scale : -INFINITY;
+          sc[t][i] = sv; m = fmaxf(m, sv);
+        }
       }
-    }
-    float m = -INFINITY;
+      m = fmaxf(m, __shfl_xor(m, 16, 64)); m = fmaxf(m, __shfl_xor(m, 32, 64));
+      const float mn = fmaxf(M[hw], m);                  // the running maximum of the row (still -inf: the row lies before everything seen so far)
+      const bool seen = mn != -INFINITY;
+      const float alpha = M[hw] != -INFINITY ? __expf(M[hw] - mn) : 0.f;
+      float l = 0.f;
+      float pr[4][4];
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
+      for (int t = 0; t < 4; t++) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const float sv = key0 + 16 * t + 4 * g + i <= pos ? sc[t][i] * a.scale : -INFINITY;
-        sc[t][i] = sv; m = fmaxf(m, sv);
+        for (int i = 0; i < 4; i++) { const float pj = seen ? __expf(sc[t][i] - mn) : 0.f; pr[t][i] = pj; l += pj; }
       }
-    }
-    m = fmaxf(m, __shfl_xor(m, 16, 64)); m = fmaxf(m, __shfl_xor(m, 32, 64));
-    const bool seen = m != -INFINITY;                    // (false: the row lies before this split)
-    float l = 0.f;
-    float pr[4][4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) { const float pj = seen ? __expf(sc[t][i] - m) : 0.f; pr[t][i] = pj; l += pj; }
-    }
-    l += __shfl_xor(l, 16, 64); l += __shfl_xor(l, 32, 64);
-    u32x4 pb[2];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-      const float e8[8] = {pr[2 * u][0], pr[2 * u][1], pr[2 * u][2], pr[2 * u][3], pr[2 * u + 1][0], pr[2 * u + 1][1], pr[2 * u + 1][2], pr[2 * u + 1][3]};
-      pb[u] = pack8_f16(e8);
-    }
-    // weighted V sums: dimension tile h, lane (g, c) ends with dimensions 16 h + 4 g + i of row c
-    float* po = a.part + (size_t)row * a.part_bs + ((size_t)head * a.nsplit + split) * (HD + 2);
-#pragma unroll
-    for (int h = 0; h < NH; h++) {
-      v4f32 o = {0.f, 0.f, 0.f, 0.f};
+      l += __shfl_xor(l, 16, 64); l += __shfl_xor(l, 32, 64);
+      L[hw] = L[hw] * alpha + l; M[hw] = mn;
+      u32x4 pb[2];
 #pragma unroll
       for (int u = 0; u < 2; u++) {
-        const u32x4 va = *(const u32x4*)(vts + (16 * h + c) * VP + 32 * u + 8 * g);
-        o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, va), __builtin_bit_cast(v8f16, pb[u]), o, 0, 0, 0);
+        const float e8[8] = {pr[2 * u][0], pr[2 * u][1], pr[2 * u][2], pr[2 * u][3], pr[2 * u + 1][0], pr[2 * u + 1][1], pr[2 * u + 1][2], pr[2 * u + 1][3]};
+        pb[u] = pack8_f16(e8);
       }
-      if (row_ok && seen) { float* pd = po + 16 * h + 4 * g; pd[0] = o[0]; pd[1] = o[1]; pd[2] = o[2]; pd[3] = o[3]; }
+      // weighted V sums: dimension tile h, lane (g, c) ends with dimensions 16 h + 4 g + i of row c
+      float* po = a.part + (size_t)row * a.part_bs + ((size_t)(kvh * group + wave + 4 * hw) * a.nsplit + split) * (HD + 2);
+#pragma unroll
+      for (int h = 0; h < NH; h++) {
+        v4f32 o = tt == 0 ? v4f32{0.f, 0.f, 0.f, 0.f} : O[hw][h] * alpha;   // (the first tile starts the sums: nothing to rescale)
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+          const u32x4 va = *(const u32x4*)(vts + (16 * h + c) * VP + 32 * u + 8 * g);
+          o = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8f16, va), __builtin_bit_cast(v8f16, pb[u]), o, 0, 0, 0);
+        }
+        if (final) { if (row_ok && seen) { float* pd = po + 16 * h + 4 * g; pd[0] = o[0]; pd[1] = o[1]; pd[2] = o[2]; pd[3] = o[3]; } }   // (the stores leave while the next products run)
+        else O[hw][h] = o;
+      }
+      if (final && row_ok && seen && g == 0) { po[HD] = M[hw]; po[HD + 1] = L[hw]; }
     }
-    if (row_ok && seen && g == 0) { po[HD] = m; po[HD + 1] = l; }
+    if (final) break;
   }
 }
 
@@ -727,7 +762,7 @@ __global__ __launch_bounds__(HD) void attn_merge_kernel(const AttnArgs args) {
   float v[FB];
 #pragma unroll
   for (int j = 0; j < FB; j++) v[j] = ph[(size_t)(j < nsp ? j : nsp - 1) * (HD + 2) + d];
-  const int pos = a.st->pos + blockIdx.y * a.pos_step, ns = (pos >> 6) + 1;
+  const int pos = a.st->pos + blockIdx.y * a.pos_step, ns = (pos >> a.split_shift) + 1;
   if (pos >= a.max_ctx || pos < 0) return;              // refused by the split launch (state.error): the output row keeps its contents
   float m = -INFINITY, l = 0.f;
   if (nsp <= HD) {
@@ -997,7 +1032,7 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
   a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps; a.norm_per_head = norm_per_head;
   a.q_bs = (long long)n_heads * head_dim; a.kv_bs = (long long)n_kv_heads * head_dim; a.cache_bs = (long long)n_kv_heads * max_ctx * head_dim;
   a.part_bs = (long long)n_heads * a.nsplit * (head_dim + 2); a.out_bs = (long long)n_heads * head_dim;
-  a.chunk = 0; a.pos_step = 0;
+  a.chunk = 0; a.pos_step = 0; a.split_shift = 6;
   if (chunk) { a.cache_bs = 0; a.pos_step = 1; }
   if (stage_type) { a.stage_fmt = decode_staged_fmt(stage_type, (long long)n_heads * head_dim, &a.stage_nu); TGA_REQUIRE(a.stage_fmt >= 0, "tga_attention_decode: no staged layout for type %d", stage_type); }
   if (stage_type && chunk) {                            // the rows of a prefill step for the 17 .. 128 row GEMM
@@ -1012,12 +1047,23 @@ static int attention_launch(int chunk, int batch, const float* q, const float* k
     if (norm == 0) attn_decode_kernel<HD8, 0><<<grid, 256, 0, s>>>(a); else if (norm == 1) attn_decode_kernel<HD8, 1><<<grid, 256, 0, s>>>(a); \
     else if (norm == 2) attn_decode_kernel<HD8, 2><<<grid, 256, 0, s>>>(a); else attn_decode_kernel<HD8, 3><<<grid, 256, 0, s>>>(a); } while (0)
   static const bool chunk_mfma_off = getenv("TGA_ATTN_CHUNK") && !strcmp(getenv("TGA_ATTN_CHUNK"), "rows");
-  const bool chunk_mfma = chunk && batch > 8 && norm == 0 && (head_dim == 64 || head_dim == 128) && !chunk_mfma_off;   // chunks of more than eight rows attend on the matrix cores
+  const bool chunk_mfma = chunk && batch > 8 && norm == 0 && (head_dim == 64 || head_dim == 128) && n_heads / n_kv_heads <= 8 && !chunk_mfma_off;   // chunks of more than eight rows attend on the matrix cores
   for (int pass = chunk ? 1 : 0; pass <= (chunk ? 2 : 0); pass++) {   // chunked prefill: append every row, then attend from the cache
     a.chunk = pass;
     if (pass == 2 && chunk_mfma) {
+      // TS tiles of 64 keys per split partial: fewer and larger partials for the merge launch (its arguments follow)
+      static const int env_ts = getenv("TGA_ATTN_CHUNK_TILES") ? atoi(getenv("TGA_ATTN_CHUNK_TILES")) : 0;
+      const int group = n_heads / n_kv_heads;
+      const int ts = env_ts == 1 ? 1 : 2;                                  // (four tiles per partial leave a context of 1024 with one workgroup per CU: 21 us against 17)
+      a.split_shift = ts == 2 ? 7 : 6;
+      a.nsplit = (a.nsplit + ts - 1) / ts;
+      a.part_bs = (long long)n_heads * a.nsplit * (head_dim + 2);
       const dim3 cgrid(n_kv_heads, a.nsplit, (batch + 15) / 16);
-      if (head_dim == 64) attn_chunk_mfma_kernel<8><<<cgrid, 256, 0, s>>>(a, batch); else attn_chunk_mfma_kernel<16><<<cgrid, 256, 0, s>>>(a, batch);
+#define TGA_CHUNK_T(HD8, TS) do { if (group <= 4) attn_chunk_mfma_kernel<HD8, TS, 1><<<cgrid, 256, 0, s>>>(a, batch); else attn_chunk_mfma_kernel<HD8, TS, 2><<<cgrid, 256, 0, s>>>(a, batch); } while (0)
+#define TGA_CHUNK(HD8) do { if (ts == 2) TGA_CHUNK_T(HD8, 2); else TGA_CHUNK_T(HD8, 1); } while (0)
+      if (head_dim == 64) TGA_CHUNK(8); else TGA_CHUNK(16);
+#undef TGA_CHUNK
+#undef TGA_CHUNK_T
       TGA_LAUNCH_CHECK();
       break;
     }
@@ -1069,7 +1115,7 @@ static int attention_decode_split(const float* q, const float* k, const float* v
   TGA_REQUIRE(it > 0, "tga_attention_decode_split: max_ctx=%d outside 1..2048 (tga_attention_split_plan reports 0 splits)", max_ctx);
   AttnArgs a = {};
   a.q = q; a.k = k; a.v = v; a.cache_k = (_Float16*)cache_k; a.cache_v = (_Float16*)cache_v; a.part = partials; a.st = (DecodeState*)state;
-  a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = ns;
+  a.n_heads = n_heads; a.n_kv = n_kv_heads; a.hd = head_dim; a.max_ctx = max_ctx; a.nsplit = ns; a.split_shift = 6;
   a.rope = rope_table; a.scale = 1.0f / sqrtf((float)head_dim);
   a.q_norm = q_norm_weight; a.k_norm = k_norm_weight; a.norm_eps = norm_eps;
   const int norm = q_norm_weight ? (norm_per_head ? 2 : 1) : 0;
