@@ -1,16 +1,18 @@
-// Small-batch GEMM over Q8_0 block pairs (K = 2048 or 4096) and fp16 weights (K = 2048), 2 <= M <= 16 activation rows, with the weights streamed into LDS by direct-to-LDS loads into rings
+// Small-batch GEMM over Q4_0 / Q8_0 / Q4_1 / Q5_0 / Q5_1 block pairs, Q4_K / Q5_K superblocks (K = 2048 or 4096) and fp16 weights (K = 2048), 2 <= M <= 16 activation rows, with the weights streamed into LDS by direct-to-LDS loads into rings
 // that belong to ONE WAVE each: the same call sites and arithmetic as qgemm_dma.hip (x.linear(W.T) over a lazily dequantized weight: tinygrad/nn/__init__.py:177,
 // tinygrad/mixin/op.py:367-392; a unit is decoded once into fp16 weights - the reference's fp16 weight cast, tinygrad/llm/model.py:376 - and
 // v_mfma_f32_16x16x32_f16 multiplies it with all activation rows), without a workgroup barrier in the loop.
 //
 // Why.  In qgemm_dma.hip the eight waves of a workgroup request a stage's pieces together and meet at one barrier per stage, so all of them wait, read LDS, decode
 // and multiply in the same phase at the same time: a stage costs the sum of its phases.  Here wave w of the workgroup owns units [w UPW, (w + 1) UPW) of every row
-// (UPW = 4 or 8: an eighth of K), i.e. bytes [w S, (w + 1) S) of each of the 16 rows of a row group (S = 272 or 544 for Q8_0); it requests them itself (16-byte
+// (UPW = 4 or 8: an eighth of K), i.e. bytes [w S, (w + 1) S) of each of the 16 rows of a row group (S = 144 .. 544); it requests them itself (16-byte
 // pieces, 64 per instruction), waits for them with its own counter, reads them back in the MFMA operand layout and requests the next group into the freed ring
 // position - nobody else touches its ring, so no barrier orders it, and the waves of a CU drift into different phases by themselves.  Measured: bare streaming of
-// that pattern (requests and LDS reads only) moves 14336 x 4096 of Q8_0 bytes in 12.2 us; the kernel takes 16.7 us at eight rows where the barrier kernel takes
-// 18.4 (4096 x 4096: 8.0 against 9.05), and an 8B-architecture Q8_0 model decodes 4 / 8 sequences in lockstep 5 / 6 % faster.  Per-wave clock stamps put the rest
-// in the decode's VALU work and a 1.7 - 3 us prologue (the second wave of a SIMD forms its activation operands behind the first).
+// that pattern (requests and LDS reads only) moves 14336 x 4096 of Q4_0 / Q8_0 bytes in 7.2 / 12.2 us; the kernel at eight rows: Q8_0 16.0 us where the barrier
+// kernel takes 18.4 (4096 x 4096: 7.6 against 9.05), Q4_0 13.4 against 13.3 (6.55 against 7.2), the K-quants and 5-bit pairs 3 - 20 % less on 4096 x 4096 and
+// -8 .. +4 % on 14336 x 4096.  Replayed batched decode of 8B-architecture models, B = 4 / 8 / 16: Q8_0 -5 / -6 % per step, Q4_0 -2 / -1.2 / -0.6 %, the Q4_K_M mix
+// -1.1 / -0.9 / -2 %; OLMoE-architecture (fp16 dense weights) +4 / +3 / +1.5 % tokens per second.  Per-wave clock stamps put what is left in the decode's VALU work
+// (the 4- to 6-bit formats: 2.3 operations per weight) and a 1.7 - 3 us prologue (the second wave of a SIMD forms its activation operands behind the first).
 // The eight partial 16 x 16 tiles of a row group meet in LDS once per group: every wave stores its tile and counts itself in with an LDS operation; wave j % 8
 // waits (bounded) for the eight counts of group j, sums the tiles in wave order and stores the rows - the role rotates, so that the wave that arrives last is not
 // the one that falls further behind.  Two tile sets alternate; a wave that is two groups ahead waits (bounded) until the set it wants has been summed.  Both waits
@@ -318,15 +320,23 @@ static int launch_wp(QArgs a, int M, hipStream_t s) {
 }
 
 // Called by tga_qgemm_dma_dispatch with a call it has checked (2 <= M <= 16, matrices of whole row groups at 16-byte aligned addresses, float32 rows where a norm
-// folds in).  Returns -1 outside this kernel's range.  Q8_0 and fp16 weights only - the formats with the most bytes per decoded weight: the kernel template takes
-// every format whose rows split into eight aligned runs, and in isolated launches it is 3 - 20 % faster for all of them except the large Q4_0 / Q4_K matrices, but in a
-// replayed batched decode step only these two gained (8B-arch Q8_0 model at B = 4 / 8: 2.81 -> 2.68 / 3.21 -> 3.03 ms per step; OLMoE-arch, fp16 dense weights, at
-// B = 2 / 4 / 8: +4 / +4 / +3 % tokens per second; the Q4_K_M mix unchanged, Q4_0 3 % slower), so the others stay on qgemm_dma.hip.
+// folds in).  Returns -1 outside this kernel's range (K other than 2048 / 4096, Q6_K and the formats that are not block pairs, a ring that does not fit LDS,
+// outputs that are not 16-byte aligned).
 int tga_qgemm_wp_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   static const bool off = getenv("TGA_WP") && atoi(getenv("TGA_WP")) == 0;      // (for A / B runs against the barrier kernel)
-  if (off || (fmt != F_Q8_0P && fmt != GGML_F16)) return -1;
+  if (off) return -1;
   if (fmt == GGML_F16 && (a.epilogue == 2 || a.K != 2048)) return -1;  // (fp16 rows of 4096 values: a ring of two groups does not fit)
   for (int i = 0; i < (a.epilogue == 2 ? 1 : a.nseg); i++)          // four rows of a column leave as one vector store
     if (((uintptr_t)a.y[i] & 15) != 0 || (a.epilogue == 1 && ((uintptr_t)a.resid[i] & 15) != 0)) return -1;
-  return fmt == GGML_F16 ? launch_wp<GGML_F16>(a, M, s) : launch_wp<F_Q8_0P>(a, M, s);
+  switch (fmt) {
+    case F_Q4_0P: return launch_wp<F_Q4_0P>(a, M, s);
+    case F_Q8_0P: return launch_wp<F_Q8_0P>(a, M, s);
+    case GGML_Q4_K: return launch_wp<GGML_Q4_K>(a, M, s);
+    case GGML_Q5_K: return launch_wp<GGML_Q5_K>(a, M, s);
+    case GGML_Q4_1: return launch_wp<GGML_Q4_1>(a, M, s);
+    case GGML_Q5_0: return launch_wp<GGML_Q5_0>(a, M, s);
+    case GGML_Q5_1: return launch_wp<GGML_Q5_1>(a, M, s);
+    case GGML_F16: return launch_wp<GGML_F16>(a, M, s);
+  }
+  return -1;
 }
