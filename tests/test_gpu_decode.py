@@ -197,14 +197,14 @@ def test_attention_prefill_chunk_kernel_vs_numpy(gpu):
     np.testing.assert_array_equal(tokb.numpy(), prompt[np.minimum(pos0 + B + np.arange(B), ctx - 1)])
   assert ol.rel_err(ck.numpy().astype(np.float32), rk.astype(np.float32)) < 2e-3
 
-@pytest.mark.parametrize("H,KV,hd,B", [(8, 2, 128, 16), (8, 2, 128, 37), (4, 4, 64, 64), (16, 2, 64, 24), (8, 8, 128, 17), (8, 1, 128, 9), (8, 2, 128, 128), (4, 4, 64, 100)])
-def test_attention_prefill_chunk_on_the_matrix_cores_vs_numpy(gpu, H, KV, hd, B):
-  """tga_attention_prefill_chunk for more than eight rows without q / k norm (the launch that attends multiplies on the matrix cores: workgroup per kv head, 64-position
-  split and tile of sixteen rows, wave per query head of the group): steps of B consecutive positions over one cache up to position 150 and beyond two split
-  boundaries, groups of 1, 4 and 8 query heads per kv head (8: two passes of the four waves), row counts that end inside a tile; every row against numpy attention over the
+@pytest.mark.parametrize("H,KV,hd,B,ctx", [(8, 2, 128, 16, 256), (8, 2, 128, 37, 256), (4, 4, 64, 64, 256), (16, 2, 64, 24, 256), (8, 8, 128, 17, 256), (8, 1, 128, 9, 256), (8, 2, 128, 128, 256),
+                                           (4, 4, 64, 100, 256), (8, 2, 128, 16, 192), (8, 2, 64, 37, 320)])
+def test_attention_prefill_chunk_on_the_matrix_cores_vs_numpy(gpu, H, KV, hd, B, ctx):
+  """tga_attention_prefill_chunk for more than eight rows without q / k norm (the launch that attends multiplies on the matrix cores: workgroup per kv head, split of two
+  64-position tiles walked with a running maximum, and tile of sixteen rows, wave per query head of the group): steps of B consecutive positions over one cache up to
+  position 150 and beyond two split boundaries, caches of an odd number of tiles (192, 320 positions: the last split's second tile lies beyond the cache), groups of 1, 4 and 8 query heads per kv head (8: two passes of the four waves), row counts that end inside a tile; every row against numpy attention over the
   positions up to its own.  The rotated queries and the probabilities are rounded to fp16 there: the bar is the linears' 1e-3."""
   from tinygrad_amd.llm import precompute_freqs_cis
-  ctx = 256
   rng = np.random.default_rng(1000 * H + 10 * KV + B)
   rope = precompute_freqs_cis(hd, ctx, 10000.0)
   ck, cv = gpu.Buffer((KV, ctx, hd), np.float16).zero_(), gpu.Buffer((KV, ctx, hd), np.float16).zero_()
@@ -217,7 +217,7 @@ def test_attention_prefill_chunk_on_the_matrix_cores_vs_numpy(gpu, H, KV, hd, B)
   stb = gpu.Buffer.from_numpy(np.zeros(16, np.int32))
   rk, rv = np.zeros((KV, ctx, hd), np.float16), np.zeros((KV, ctx, hd), np.float16)
   worst, pos0 = 0.0, 0
-  while pos0 + B <= 150 + B and pos0 + B < ctx:
+  while pos0 + B <= (150 if ctx == 256 else ctx) + B and pos0 + B < ctx:
     q, k, v = (rng.standard_normal((B, n)).astype(np.float32) * 1.5 for n in (H * hd, KV * hd, KV * hd))
     qb, kb, vb = (gpu.Buffer.from_numpy(t) for t in (q, k, v))
     gpu.check(gpu.lib().tga_attention_prefill_chunk(B, qb.ptr, kb.ptr, vb.ptr, None, None, 0.0, 0, ck.ptr, cv.ptr, part.ptr, stb.ptr, H, KV, hd, ctx, ropeb.ptr,
