@@ -325,7 +325,10 @@ static int launch_wp(QArgs a, int M, hipStream_t s) {
 int tga_qgemm_wp_dispatch(int fmt, const QArgs& a, int M, hipStream_t s) {
   static const bool off = getenv("TGA_WP") && atoi(getenv("TGA_WP")) == 0;      // (for A / B runs against the barrier kernel)
   if (off) return -1;
+  static const int skip = getenv("TGA_WP_SKIP") ? atoi(getenv("TGA_WP_SKIP")) : 0;   // (A / B: 1 plain, 2 several matrices, 4 SwiGLU pair stay on the barrier kernel)
+  if (skip & (a.epilogue == 2 ? 4 : a.nseg > 1 ? 2 : 1)) return -1;
   if (fmt == GGML_F16 && (a.epilogue == 2 || a.K != 2048)) return -1;  // (fp16 rows of 4096 values: a ring of two groups does not fit)
+  if (fmt == F_Q4_0P && a.epilogue == 2) return -1;                    // (the Q4_0 SwiGLU pair: the barrier kernel is 0.8 % of a batched 8B step ahead from eight rows on, equal below)
   for (int i = 0; i < (a.epilogue == 2 ? 1 : a.nseg); i++)          // four rows of a column leave as one vector store
     if (((uintptr_t)a.y[i] & 15) != 0 || (a.epilogue == 1 && ((uintptr_t)a.resid[i] & 15) != 0)) return -1;
   switch (fmt) {
